@@ -1,0 +1,418 @@
+// extern "C" boundary of libflare_hip.so: host-side validation, planning and dispatch.
+// No exception crosses this file; every error is a status code plus a thread-local text.
+#include "../../include/flare_hip.h"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "common.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int esize(int dtype) { return dtype == FLARE_DT_F32 ? 4 : 2; }
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+bool strides_mult8(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0; }
+
+// ---- mixer ----------------------------------------------------------------------------
+struct MixerPlan {
+    bool mfma;
+    int n_splits, n_parts, tokens_per_split;
+    size_t off_m, off_l, off_acc, off_z, total;
+};
+
+int check_mixer_desc(const FlareMixerDesc* d)
+{
+    if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
+    if (d->B < 1 || d->H < 1 || d->N < 1 || d->M < 1 || d->D < 1)
+        return fail(FLARE_EINVAL, "B,H,N,M,D must be >= 1 (got %d,%d,%d,%d,%d)", d->B, d->H, d->N, d->M, d->D);
+    if (d->dtype < FLARE_DT_F32 || d->dtype > FLARE_DT_F16) return fail(FLARE_EINVAL, "unknown dtype %d", d->dtype);
+    if (!(d->scale > 0.f)) return fail(FLARE_EINVAL, "scale must be > 0 (got %g)", (double)d->scale);
+    if (d->D > 128) return fail(FLARE_EUNSUPPORTED, "head dim D=%d > 128 is not supported", d->D);
+    if (d->H > 65535 || d->B > 65535) return fail(FLARE_EUNSUPPORTED, "B and H must be <= 65535");
+    if (d->n_splits < 0) return fail(FLARE_EINVAL, "n_splits must be >= 0");
+    const int64_t* ss[4] = {d->q_stride, d->k_stride, d->v_stride, d->y_stride};
+    const char* nm[4] = {"q", "k", "v", "y"};
+    for (int t = 0; t < 4; ++t) {
+        if (ss[t][2] < d->D) return fail(FLARE_EINVAL, "%s row stride %lld < D=%d (rows overlap)", nm[t], (long long)ss[t][2], d->D);
+        if (ss[t][0] < 0 || ss[t][1] < 0) return fail(FLARE_EINVAL, "%s has a negative stride", nm[t]);
+    }
+    return FLARE_OK;
+}
+
+bool mixer_ptrs_ok_for_mfma(const FlareMixerDesc* d, const void* q, const void* k, const void* v, const void* y)
+{
+    if (q && !aligned16(q)) return false;
+    if (k && !aligned16(k)) return false;
+    if (v && !aligned16(v)) return false;
+    if (y && !aligned16(y)) return false;
+    return strides_mult8(d->q_stride) && strides_mult8(d->k_stride) && strides_mult8(d->v_stride) &&
+           strides_mult8(d->y_stride);
+}
+
+// The plan depends on the descriptor only (never on pointer values) so that the workspace
+// query and the launch always agree.  Misaligned pointers demote to the generic kernels,
+// whose partial count (4 per workgroup) is covered by sizing for the larger of the two.
+MixerPlan plan_mixer(const FlareMixerDesc* d, bool want_mfma)
+{
+    MixerPlan p;
+    p.mfma = want_mfma;
+    const int unit = p.mfma ? flare::mfma_gather_tokens_per_iter() : 32;
+    const int mblk = p.mfma ? ((d->M % 256 == 0) ? d->M / 256 : (d->M % 128 == 0) ? d->M / 128 : d->M / 64)
+                            : (d->M + 63) / 64;
+    int s = d->n_splits;
+    if (s <= 0) {
+        const int64_t target = 1024;  // ~4 workgroups per CU on 256 CUs
+        int64_t per = (int64_t)d->B * d->H * mblk;
+        s = (int)((target + per - 1) / per);
+        if (s < 1) s = 1;
+    }
+    int64_t tps = ((int64_t)d->N + s - 1) / s;
+    tps = ((tps + unit - 1) / unit) * unit;
+    const int min_tokens = p.mfma ? 4 * unit : 8 * unit;  // keep the split overhead small
+    if (tps < min_tokens) tps = min_tokens;
+    p.tokens_per_split = (int)tps;
+    p.n_splits = (int)(((int64_t)d->N + tps - 1) / tps);
+    p.n_parts = p.mfma ? p.n_splits : p.n_splits * flare::gather_generic_parts_per_wg();
+    const size_t bh = (size_t)d->B * d->H;
+    const size_t rows = bh * p.n_parts * d->M;
+    p.off_m = 0;
+    p.off_l = p.off_m + rows * 4;
+    p.off_acc = p.off_l + rows * 4;
+    p.off_z = p.off_acc + rows * d->D * 4;
+    p.off_z = (p.off_z + 255) & ~(size_t)255;
+    p.total = p.off_z + bh * d->M * d->D * 4;
+    return p;
+}
+
+bool desc_wants_mfma(const FlareMixerDesc* d)
+{
+    return !(d->flags & FLARE_FLAG_FORCE_GENERIC) && flare::mfma_mixer_supported(d->dtype, d->M, d->D) &&
+           strides_mult8(d->q_stride) && strides_mult8(d->k_stride) && strides_mult8(d->v_stride) &&
+           strides_mult8(d->y_stride);
+}
+
+size_t mixer_ws_bytes(const FlareMixerDesc* d)
+{
+    size_t a = plan_mixer(d, false).total;
+    if (desc_wants_mfma(d)) {
+        size_t b = plan_mixer(d, true).total;
+        if (b > a) a = b;
+    }
+    return a;
+}
+
+void fill_mixer_args(flare::MixerArgs& a, const FlareMixerDesc* d, const MixerPlan& p, void* ws)
+{
+    memset(&a, 0, sizeof(a));
+    a.B = d->B; a.H = d->H; a.N = d->N; a.M = d->M; a.D = d->D;
+    a.n_splits = p.n_splits; a.n_parts = p.n_parts; a.tokens_per_split = p.tokens_per_split;
+    a.scale_log2 = d->scale * flare::kLog2e;
+    for (int i = 0; i < 3; ++i) {
+        a.qs[i] = d->q_stride[i]; a.ks[i] = d->k_stride[i]; a.vs[i] = d->v_stride[i]; a.ys[i] = d->y_stride[i];
+    }
+    if (ws) {
+        char* w = static_cast<char*>(ws);
+        a.part_m = reinterpret_cast<float*>(w + p.off_m);
+        a.part_l = reinterpret_cast<float*>(w + p.off_l);
+        a.part_acc = reinterpret_cast<float*>(w + p.off_acc);
+    }
+}
+
+int hip_status(hipError_t e, const char* what)
+{
+    if (e == hipSuccess) return FLARE_OK;
+    return fail(FLARE_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+int do_gather(const FlareMixerDesc* d, const void* q, const void* k, const void* v, const uint8_t* mask,
+              float* z, float* lse, void* ws, size_t ws_bytes, hipStream_t st)
+{
+    if (!ws) return fail(FLARE_EWORKSPACE, "workspace is NULL");
+    if (!aligned16(ws)) return fail(FLARE_EINVAL, "workspace must be 16-byte aligned");
+    const size_t need = mixer_ws_bytes(d);
+    if (ws_bytes < need) return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", ws_bytes, need);
+    const bool mfma = desc_wants_mfma(d) && mixer_ptrs_ok_for_mfma(d, q, k, v, nullptr);
+    const MixerPlan p = plan_mixer(d, mfma);
+    flare::MixerArgs a;
+    fill_mixer_args(a, d, p, ws);
+    a.q = q; a.k = k; a.v = v; a.mask = mask; a.z = z; a.lse = lse;
+    hipError_t e = mfma ? flare::launch_gather_mfma(a, d->dtype, st) : flare::launch_gather_generic(a, d->dtype, st);
+    if (e != hipSuccess) return hip_status(e, "gather launch");
+    return hip_status(flare::launch_gather_merge(a, st), "gather merge launch");
+}
+
+int do_scatter(const FlareMixerDesc* d, const void* q, const void* k, const float* z, const uint8_t* mask,
+               void* y, hipStream_t st)
+{
+    const bool mfma = desc_wants_mfma(d) && mixer_ptrs_ok_for_mfma(d, q, k, nullptr, y);
+    const MixerPlan p = plan_mixer(d, mfma);
+    flare::MixerArgs a;
+    fill_mixer_args(a, d, p, nullptr);
+    a.q = q; a.k = k; a.y = y; a.mask = mask; a.z = const_cast<float*>(z);
+    hipError_t e = mfma ? flare::launch_scatter_mfma(a, d->dtype, st) : flare::launch_scatter_generic(a, d->dtype, st);
+    return hip_status(e, "scatter launch");
+}
+
+// ---- causal ---------------------------------------------------------------------------
+int check_causal_desc(const FlareCausalDesc* d)
+{
+    if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
+    if (d->B < 1 || d->H < 1 || d->N < 1 || d->M < 1 || d->D < 1)
+        return fail(FLARE_EINVAL, "B,H,N,M,D must be >= 1 (got %d,%d,%d,%d,%d)", d->B, d->H, d->N, d->M, d->D);
+    if (d->dtype < FLARE_DT_F32 || d->dtype > FLARE_DT_F16) return fail(FLARE_EINVAL, "unknown dtype %d", d->dtype);
+    if (!(d->scale > 0.f)) return fail(FLARE_EINVAL, "scale must be > 0 (got %g)", (double)d->scale);
+    if (d->D > 128) return fail(FLARE_EUNSUPPORTED, "head dim D=%d > 128 is not supported", d->D);
+    if (d->chunk < 0) return fail(FLARE_EINVAL, "chunk must be >= 0");
+    if (flare::causal_lds_bytes(d->M, d->D, false) > 160 * 1024)
+        return fail(FLARE_EUNSUPPORTED, "state M*D=%d*%d does not fit the 160 KB LDS", d->M, d->D);
+    if ((int64_t)d->B * d->H > 2147483647LL / 4) return fail(FLARE_EUNSUPPORTED, "B*H too large");
+    const int64_t* ss[4] = {d->q_stride, d->k_stride, d->v_stride, d->y_stride};
+    const char* nm[4] = {"q", "k", "v", "y"};
+    for (int t = 0; t < 4; ++t)
+        if (ss[t][2] < d->D) return fail(FLARE_EINVAL, "%s row stride %lld < D=%d", nm[t], (long long)ss[t][2], d->D);
+    return FLARE_OK;
+}
+
+void fill_causal_args(flare::CausalArgs& a, const FlareCausalDesc* d)
+{
+    memset(&a, 0, sizeof(a));
+    a.B = d->B; a.H = d->H; a.N = d->N; a.M = d->M; a.D = d->D;
+    a.chunk = d->chunk > 0 ? d->chunk : 256;
+    a.scale = d->scale;
+    for (int i = 0; i < 3; ++i) {
+        a.qs[i] = d->q_stride[i]; a.ks[i] = d->k_stride[i]; a.vs[i] = d->v_stride[i]; a.ys[i] = d->y_stride[i];
+    }
+}
+
+// ---- triple ---------------------------------------------------------------------------
+int check_triple_desc(const FlareTripleDesc* d)
+{
+    if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
+    if (d->B < 1 || d->H < 1 || d->N < 1 || d->Dq < 1 || d->Dv < 1)
+        return fail(FLARE_EINVAL, "B,H,N,Dq,Dv must be >= 1");
+    if (d->dtype < FLARE_DT_F32 || d->dtype > FLARE_DT_F16) return fail(FLARE_EINVAL, "unknown dtype %d", d->dtype);
+    if (d->Dq > 64 || d->Dv > 64) return fail(FLARE_EUNSUPPORTED, "Dq=%d, Dv=%d: at most 64 supported", d->Dq, d->Dv);
+    if (d->feature_map < 0 || d->feature_map > 1) return fail(FLARE_EINVAL, "feature_map must be 0 or 1");
+    if (d->n_splits < 0) return fail(FLARE_EINVAL, "n_splits must be >= 0");
+    if (d->H > 65535 || d->B > 65535) return fail(FLARE_EUNSUPPORTED, "B and H must be <= 65535");
+    return FLARE_OK;
+}
+
+struct TriplePlan { int n_splits, tokens_per_split; size_t per_split, off_kk, total; };
+
+TriplePlan plan_triple(const FlareTripleDesc* d)
+{
+    TriplePlan p;
+    int s = d->n_splits;
+    if (s <= 0) {
+        const int64_t per = (int64_t)d->B * d->H;
+        s = (int)((1024 + per - 1) / per);
+        if (s < 1) s = 1;
+    }
+    int64_t tps = ((int64_t)d->N + s - 1) / s;
+    if (tps < 64) tps = 64;
+    p.tokens_per_split = (int)tps;
+    p.n_splits = (int)(((int64_t)d->N + tps - 1) / tps);
+    p.per_split = (size_t)d->Dq * d->Dv * d->Dq + (size_t)d->Dq * d->Dq;
+    const size_t bh = (size_t)d->B * d->H;
+    p.off_kk = bh * p.n_splits * p.per_split * 4;
+    p.off_kk = (p.off_kk + 255) & ~(size_t)255;
+    p.total = p.off_kk + bh * d->Dq * d->Dq * 4;
+    return p;
+}
+
+void fill_triple_args(flare::TripleArgs& a, const FlareTripleDesc* d, const TriplePlan& p)
+{
+    memset(&a, 0, sizeof(a));
+    a.B = d->B; a.H = d->H; a.N = d->N; a.Dq = d->Dq; a.Dv = d->Dv;
+    a.feature_map = d->feature_map; a.normalize = d->normalize;
+    a.n_splits = p.n_splits; a.tokens_per_split = p.tokens_per_split;
+    for (int i = 0; i < 3; ++i) {
+        a.q1s[i] = d->q1_stride[i]; a.q2s[i] = d->q2_stride[i]; a.k1s[i] = d->k1_stride[i];
+        a.k2s[i] = d->k2_stride[i]; a.vs[i] = d->v_stride[i]; a.os[i] = d->o_stride[i];
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int flare_abi_version(void) { return FLARE_ABI_VERSION; }
+
+const char* flare_last_error_string(void) { return g_err; }
+
+const char* flare_mixer_kernel_name(const FlareMixerDesc* desc)
+{
+    if (check_mixer_desc(desc) != FLARE_OK) return nullptr;
+    if (!desc_wants_mfma(desc)) return "generic";
+    return desc->dtype == FLARE_DT_BF16 ? "mfma_bf16" : "mfma_f16";
+}
+
+int flare_mixer_workspace_bytes(const FlareMixerDesc* desc, size_t* bytes)
+{
+    if (!bytes) return fail(FLARE_EINVAL, "bytes is NULL");
+    int rc = check_mixer_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    *bytes = mixer_ws_bytes(desc);
+    return FLARE_OK;
+}
+
+int flare_gather_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
+                     const uint8_t* key_mask, float* z, float* lse, void* workspace,
+                     size_t workspace_bytes, void* stream)
+{
+    int rc = check_mixer_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !v || !z) return fail(FLARE_EINVAL, "q, k, v and z must not be NULL");
+    return do_gather(desc, q, k, v, key_mask, z, lse, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+int flare_scatter_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const float* z,
+                      const uint8_t* key_mask, void* y, void* stream)
+{
+    int rc = check_mixer_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !z || !y) return fail(FLARE_EINVAL, "q, k, z and y must not be NULL");
+    return do_scatter(desc, q, k, z, key_mask, y, static_cast<hipStream_t>(stream));
+}
+
+int flare_mixer_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
+                    const uint8_t* key_mask, void* y, float* z_out, void* workspace,
+                    size_t workspace_bytes, void* stream)
+{
+    int rc = check_mixer_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !v || !y) return fail(FLARE_EINVAL, "q, k, v and y must not be NULL");
+    if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
+    float* z = z_out;
+    if (!z) {
+        // z lives at the tail of the workspace; the offset is the same for both plans' maximum
+        const size_t need = mixer_ws_bytes(desc);
+        if (workspace_bytes < need)
+            return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, need);
+        const size_t zbytes = (size_t)desc->B * desc->H * desc->M * desc->D * 4;
+        z = reinterpret_cast<float*>(static_cast<char*>(workspace) + (need - zbytes));
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    rc = do_gather(desc, q, k, v, key_mask, z, nullptr, workspace, workspace_bytes, st);
+    if (rc != FLARE_OK) return rc;
+    return do_scatter(desc, q, k, z, key_mask, y, st);
+}
+
+int flare_causal_workspace_bytes(const FlareCausalDesc* desc, size_t* bytes)
+{
+    if (!bytes) return fail(FLARE_EINVAL, "bytes is NULL");
+    int rc = check_causal_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    *bytes = 0;
+    return FLARE_OK;
+}
+
+int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const void* k, const void* v,
+                             void* y, float* mu, float* den, float* num, void* workspace,
+                             size_t workspace_bytes, void* stream)
+{
+    (void)workspace; (void)workspace_bytes;
+    int rc = check_causal_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !v || !y || !mu || !den || !num)
+        return fail(FLARE_EINVAL, "q, k, v, y, mu, den, num must not be NULL");
+    flare::CausalArgs a;
+    fill_causal_args(a, desc);
+    a.q = q; a.k = k; a.v = v; a.y = y; a.mu = mu; a.den = den; a.num = num;
+    return hip_status(flare::launch_causal_prefill(a, desc->dtype, static_cast<hipStream_t>(stream)),
+                      "causal prefill launch");
+}
+
+int flare_causal_decode_fwd(const FlareCausalDesc* desc, const void* q, const void* k, const void* v,
+                            void* y, float* mu, float* den, float* num, void* stream)
+{
+    int rc = check_causal_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !v || !y || !mu || !den || !num)
+        return fail(FLARE_EINVAL, "q, k, v, y, mu, den, num must not be NULL");
+    flare::CausalArgs a;
+    fill_causal_args(a, desc);
+    a.q = q; a.k = k; a.v = v; a.y = y; a.mu = mu; a.den = den; a.num = num;
+    return hip_status(flare::launch_causal_decode(a, desc->dtype, static_cast<hipStream_t>(stream)),
+                      "causal decode launch");
+}
+
+int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes)
+{
+    if (!bytes) return fail(FLARE_EINVAL, "bytes is NULL");
+    int rc = check_triple_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    *bytes = plan_triple(desc).total;
+    return FLARE_OK;
+}
+
+int flare_triple_state_fwd(const FlareTripleDesc* desc, const void* k1, const void* k2, const void* v,
+                           float* state, float* kk_state, void* workspace, size_t workspace_bytes,
+                           void* stream)
+{
+    int rc = check_triple_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!k1 || !k2 || !v || !state) return fail(FLARE_EINVAL, "k1, k2, v and state must not be NULL");
+    if (desc->normalize && !kk_state) return fail(FLARE_EINVAL, "kk_state is required when normalize != 0");
+    if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
+    const TriplePlan p = plan_triple(desc);
+    if (workspace_bytes < p.total)
+        return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, p.total);
+    flare::TripleArgs a;
+    fill_triple_args(a, desc, p);
+    a.k1 = k1; a.k2 = k2; a.v = v; a.state = state; a.kk = kk_state;
+    a.part = static_cast<float*>(workspace);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = flare::launch_triple_state(a, desc->dtype, st);
+    if (e != hipSuccess) return hip_status(e, "triple state launch");
+    return hip_status(flare::launch_triple_merge(a, st), "triple merge launch");
+}
+
+int flare_triple_out_fwd(const FlareTripleDesc* desc, const void* q1, const void* q2, const float* state,
+                         const float* kk_state, void* out, void* stream)
+{
+    int rc = check_triple_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q1 || !q2 || !state || !out) return fail(FLARE_EINVAL, "q1, q2, state and out must not be NULL");
+    if (desc->normalize && !kk_state) return fail(FLARE_EINVAL, "kk_state is required when normalize != 0");
+    const TriplePlan p = plan_triple(desc);
+    flare::TripleArgs a;
+    fill_triple_args(a, desc, p);
+    a.q1 = q1; a.q2 = q2; a.out = out; a.state = const_cast<float*>(state); a.kk = const_cast<float*>(kk_state);
+    return hip_status(flare::launch_triple_out(a, desc->dtype, static_cast<hipStream_t>(stream)), "triple out launch");
+}
+
+int flare_triple_fwd(const FlareTripleDesc* desc, const void* q1, const void* q2, const void* k1,
+                     const void* k2, const void* v, float* state, void* out, void* workspace,
+                     size_t workspace_bytes, void* stream)
+{
+    int rc = check_triple_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q1 || !q2 || !k1 || !k2 || !v || !state || !out)
+        return fail(FLARE_EINVAL, "q1, q2, k1, k2, v, state and out must not be NULL");
+    if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
+    const TriplePlan p = plan_triple(desc);
+    if (workspace_bytes < p.total)
+        return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, p.total);
+    float* kk = reinterpret_cast<float*>(static_cast<char*>(workspace) + p.off_kk);
+    rc = flare_triple_state_fwd(desc, k1, k2, v, state, kk, workspace, workspace_bytes, stream);
+    if (rc != FLARE_OK) return rc;
+    return flare_triple_out_fwd(desc, q1, q2, state, kk, out, stream);
+}
+
+}  // extern "C"

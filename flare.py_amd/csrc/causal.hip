@@ -1,0 +1,217 @@
+// Causal FLARE: chunked prefill and recurrent decode, fp32 arithmetic, state resident in LDS.
+//
+// Definition (the reference names causal FLARE in README.md:60 but holds no code for it;
+// the chunk structure follows lra/models/triton/causal_linear.py:81-137 with the plain sum
+// replaced by the online-softmax triple):
+//   sigma[t,m] = s <q_m, k_t>
+//   z_t[m]     = sum_{tau<=t} softmax over tau<=t of sigma[.,m] applied to v
+//   y_t        = sum_m softmax_m(sigma[t,.])_m z_t[m]
+// State per (b,h): mu[M] (max), den[M], num[M,D], with z_t = num/den.
+//
+// One workgroup owns one (b,h) and walks its tokens in blocks of TB tokens; the state never
+// leaves LDS between blocks, so N decode steps (TB = 1) cost one launch.
+// Within a block the per-latent reference maximum is the block maximum, so a score that
+// jumps by more than ~2^120 inside one block of 16 tokens would underflow the earlier
+// denominators; prefill uses TB = 16 to keep that exposure small.
+#include "common.hpp"
+
+namespace flare {
+
+namespace {
+
+constexpr int kThreads = 256;
+
+struct CausalLds {
+    int q, U, sg, gg, ks, vs, As, mu, den, al, rmax, rinv, total;  // offsets in floats
+};
+
+__host__ __device__ inline CausalLds causal_lds_layout(int M, int D, int TB)
+{
+    CausalLds L;
+    int o = 0;
+    L.q = o;    o += M * (D + 1);
+    L.U = o;    o += M * D;
+    L.sg = o;   o += TB * (M + 1);
+    L.gg = o;   o += TB * (M + 1);
+    L.ks = o;   o += TB * D;
+    L.vs = o;   o += TB * D;
+    L.As = o;   o += TB * TB;
+    L.mu = o;   o += M;
+    L.den = o;  o += M;
+    L.al = o;   o += M;
+    L.rmax = o; o += TB;
+    L.rinv = o; o += TB;
+    L.total = o;
+    return L;
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+template <typename T, int TB>
+__global__ __launch_bounds__(kThreads) void causal_generic_kernel(CausalArgs a)
+{
+    extern __shared__ float sm[];
+    const int M = a.M, D = a.D, N = a.N;
+    const CausalLds L = causal_lds_layout(M, D, TB);
+    float* qs = sm + L.q;   float* U = sm + L.U;   float* sg = sm + L.sg; float* gg = sm + L.gg;
+    float* ks = sm + L.ks;  float* vs = sm + L.vs; float* As = sm + L.As;
+    float* mu_s = sm + L.mu; float* den_s = sm + L.den; float* al_s = sm + L.al;
+    float* rmax = sm + L.rmax; float* rinv = sm + L.rinv;
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H;
+    const T* q = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
+    const T* k = (const T*)a.k + b * a.ks[0] + h * a.ks[1];
+    const T* v = (const T*)a.v + b * a.vs[0] + h * a.vs[1];
+    T* y = (T*)a.y + b * a.ys[0] + h * a.ys[1];
+    float* mu_g = a.mu + (int64_t)bh * M;
+    float* den_g = a.den + (int64_t)bh * M;
+    float* num_g = a.num + (int64_t)bh * M * D;
+    const float sl2 = a.scale * kLog2e;
+
+    for (int idx = tid; idx < M * D; idx += kThreads) {
+        const int m = idx / D, d = idx - m * D;
+        qs[m * (D + 1) + d] = to_f32(q[(int64_t)m * a.qs[2] + d]) * sl2;
+        U[idx] = num_g[idx];
+    }
+    for (int m = tid; m < M; m += kThreads) {
+        const float mu = mu_g[m];
+        mu_s[m] = mu <= kNegBig ? kNegBig : mu * kLog2e;
+        den_s[m] = den_g[m];
+    }
+
+    for (int n0 = 0; n0 < N; n0 += TB) {
+        const int tb = min(TB, N - n0);
+        __syncthreads();
+        for (int idx = tid; idx < tb * D; idx += kThreads) {
+            const int t = idx / D, d = idx - t * D;
+            ks[idx] = to_f32(k[(int64_t)(n0 + t) * a.ks[2] + d]);
+            vs[idx] = to_f32(v[(int64_t)(n0 + t) * a.vs[2] + d]);
+        }
+        __syncthreads();
+        // scores (log2 units)
+        for (int idx = tid; idx < tb * M; idx += kThreads) {
+            const int t = idx / M, m = idx - t * M;
+            float s = 0.f;
+            for (int d = 0; d < D; ++d) s = fmaf(ks[t * D + d], qs[m * (D + 1) + d], s);
+            sg[t * (M + 1) + m] = s;
+        }
+        __syncthreads();
+        // softmax statistics over the latents of each token
+        for (int t = wave; t < tb; t += kThreads / 64) {
+            float mx = kNegBig;
+            for (int m = lane; m < M; m += 64) mx = fmaxf(mx, sg[t * (M + 1) + m]);
+            mx = wave_max(mx);
+            float sum = 0.f;
+            for (int m = lane; m < M; m += 64) sum += fast_exp2(sg[t * (M + 1) + m] - mx);
+            sum = wave_sum(sum);
+            if (lane == 0) { rmax[t] = mx; rinv[t] = 1.f / sum; }
+        }
+        __syncthreads();
+        // per latent: block maximum, running denominator, G = w / den, P in place of sigma
+        for (int m = tid; m < M; m += kThreads) {
+            const float mp = mu_s[m];
+            float mc = mp;
+            for (int t = 0; t < tb; ++t) mc = fmaxf(mc, sg[t * (M + 1) + m]);
+            const float al = fast_exp2(mp - mc);
+            float dc = al * den_s[m];
+            for (int t = 0; t < tb; ++t) {
+                const float s = sg[t * (M + 1) + m];
+                const float p = fast_exp2(s - mc);
+                dc += p;
+                const float w = fast_exp2(s - rmax[t]) * rinv[t];
+                gg[t * (M + 1) + m] = w / dc;
+                sg[t * (M + 1) + m] = p;
+            }
+            mu_s[m] = mc; den_s[m] = dc; al_s[m] = al;
+        }
+        __syncthreads();
+        // A[t][tau] = sum_m G[t,m] P[tau,m] for tau <= t
+        if (TB > 1) {
+            for (int idx = tid; idx < tb * tb; idx += kThreads) {
+                const int t = idx / tb, tau = idx - t * tb;
+                float acc = 0.f;
+                if (tau <= t)
+                    for (int m = 0; m < M; ++m) acc = fmaf(gg[t * (M + 1) + m], sg[tau * (M + 1) + m], acc);
+                As[t * TB + tau] = acc;
+            }
+            __syncthreads();
+        }
+        // y[t,d] = sum_m G[t,m] alpha[m] U[m,d] + sum_{tau<=t} A[t,tau] v[tau,d]
+        for (int idx = tid; idx < tb * D; idx += kThreads) {
+            const int t = idx / D, d = idx - t * D;
+            float acc = 0.f;
+            for (int m = 0; m < M; ++m) acc = fmaf(gg[t * (M + 1) + m] * al_s[m], U[m * D + d], acc);
+            if (TB > 1) {
+                for (int tau = 0; tau <= t; ++tau) acc = fmaf(As[t * TB + tau], vs[tau * D + d], acc);
+            } else {
+                // single token: A[0][0] = sum_m G[0,m] P[0,m]
+                float a00 = 0.f;
+                for (int m = 0; m < M; ++m) a00 = fmaf(gg[m], sg[m], a00);
+                acc = fmaf(a00, vs[d], acc);
+            }
+            y[(int64_t)(n0 + t) * a.ys[2] + d] = from_f32<T>(acc);
+        }
+        __syncthreads();
+        // U[m,d] = alpha[m] U[m,d] + sum_t P[t,m] v[t,d]
+        for (int idx = tid; idx < M * D; idx += kThreads) {
+            const int m = idx / D, d = idx - m * D;
+            float u = al_s[m] * U[idx];
+            for (int t = 0; t < tb; ++t) u = fmaf(sg[t * (M + 1) + m], vs[t * D + d], u);
+            U[idx] = u;
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < M * D; idx += kThreads) num_g[idx] = U[idx];
+    for (int m = tid; m < M; m += kThreads) {
+        mu_g[m] = mu_s[m] <= kNegBig ? -INFINITY : mu_s[m] * kLn2;
+        den_g[m] = den_s[m];
+    }
+}
+
+template <typename T, int TB>
+hipError_t launch_tb(const CausalArgs& a, hipStream_t st)
+{
+    const CausalLds L = causal_lds_layout(a.M, a.D, TB);
+    const size_t lds = (size_t)L.total * sizeof(float);
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    auto kern = causal_generic_kernel<T, TB>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3(a.B * a.H), dim3(kThreads), lds, st, a);
+    return hipGetLastError();
+}
+
+template <int TB>
+hipError_t launch_dt(const CausalArgs& a, int dtype, hipStream_t st)
+{
+    switch (dtype) {
+        case 0: return launch_tb<float, TB>(a, st);
+        case 1: return launch_tb<bf16_t, TB>(a, st);
+        default: return launch_tb<f16_t, TB>(a, st);
+    }
+}
+
+}  // namespace
+
+size_t causal_lds_bytes(int M, int D, bool decode)
+{
+    return (size_t)causal_lds_layout(M, D, decode ? 1 : 16).total * sizeof(float);
+}
+
+hipError_t launch_causal_prefill(const CausalArgs& a, int dtype, hipStream_t st) { return launch_dt<16>(a, dtype, st); }
+hipError_t launch_causal_decode(const CausalArgs& a, int dtype, hipStream_t st) { return launch_dt<1>(a, dtype, st); }
+
+}  // namespace flare

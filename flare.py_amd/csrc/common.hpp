@@ -1,0 +1,92 @@
+// Shared device helpers and launch-argument structs for the gfx950 FLARE kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace flare {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2   = 0.6931471805599453f;
+constexpr float kNegBig = -1.0e30f;  // "minus infinity" that stays finite under subtraction
+
+// ---- element types -------------------------------------------------------------------
+struct bf16_t { uint16_t x; };
+typedef _Float16 f16_t;
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float(uint32_t(v.x) << 16); }
+__device__ __forceinline__ float to_f32(f16_t v) { return float(v); }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return uint16_t((u >> 16) | 0x40u);  // quiet NaN
+    u += 0x7fffu + ((u >> 16) & 1u);                                          // RNE
+    return uint16_t(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return bf16_t{f32_to_bf16_bits(v)}; }
+template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float v) { return f16_t(v); }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---- kernel argument blocks (host fills them; passed by value) -------------------------
+struct MixerArgs {
+    const void* q; const void* k; const void* v; void* y;
+    const uint8_t* mask;      // [B,N] or null
+    float* z;                 // [B,H,M,D] fp32
+    float* lse;               // [B,H,M] or null (natural log)
+    float* part_m;            // [B,H,P,M]   per-partial running max (log2 units)
+    float* part_l;            // [B,H,P,M]   per-partial sum
+    float* part_acc;          // [B,H,P,M,D] per-partial numerator
+    int B, H, N, M, D;
+    int n_splits;             // workgroups along N
+    int n_parts;              // partials per (b,h): n_splits * partials-per-workgroup
+    int tokens_per_split;
+    float scale_log2;         // scale * log2(e)
+    int64_t qs[3], ks[3], vs[3], ys[3];
+};
+
+struct CausalArgs {
+    const void* q; const void* k; const void* v; void* y;
+    float* mu; float* den; float* num;   // state, natural-log units for mu
+    int B, H, N, M, D;
+    int chunk;
+    float scale;
+    int64_t qs[3], ks[3], vs[3], ys[3];
+};
+
+struct TripleArgs {
+    const void* q1; const void* q2; const void* k1; const void* k2; const void* v; void* out;
+    float* state;      // [B,H,Dq,Dv,Dq]
+    float* kk;         // [B,H,Dq,Dq] normaliser state or null
+    float* part;       // [B,H,S,Dq*Dv*Dq (+Dq*Dq)] split partials
+    int B, H, N, Dq, Dv;
+    int feature_map, normalize;
+    int n_splits, tokens_per_split;
+    int64_t q1s[3], q2s[3], k1s[3], k2s[3], vs[3], os[3];
+};
+
+// ---- launchers implemented in the .hip files -------------------------------------------
+hipError_t launch_gather_generic(const MixerArgs& a, int dtype, hipStream_t st);
+hipError_t launch_gather_merge(const MixerArgs& a, hipStream_t st);
+hipError_t launch_scatter_generic(const MixerArgs& a, int dtype, hipStream_t st);
+int        gather_generic_parts_per_wg();
+
+bool       mfma_mixer_supported(int dtype, int M, int D);
+int        mfma_gather_tokens_per_iter();
+hipError_t launch_gather_mfma(const MixerArgs& a, int dtype, hipStream_t st);
+hipError_t launch_scatter_mfma(const MixerArgs& a, int dtype, hipStream_t st);
+
+size_t     causal_lds_bytes(int M, int D, bool decode);
+hipError_t launch_causal_prefill(const CausalArgs& a, int dtype, hipStream_t st);
+hipError_t launch_causal_decode(const CausalArgs& a, int dtype, hipStream_t st);
+
+hipError_t launch_triple_state(const TripleArgs& a, int dtype, hipStream_t st);
+hipError_t launch_triple_merge(const TripleArgs& a, hipStream_t st);
+hipError_t launch_triple_out(const TripleArgs& a, int dtype, hipStream_t st);
+
+}  // namespace flare

@@ -1,0 +1,598 @@
+// MFMA (v_mfma_f32_16x16x32_{bf16,f16}) FLARE mixer kernels for gfx950, wave64.
+//
+// Operand conventions of the 16x16x32 MFMA used throughout (c16 = lane % 16, g = lane / 16):
+//   A (16 x 32): lane holds row c16,    k-slots 8g .. 8g+7
+//   B (32 x 16): lane holds column c16, k-slots 8g .. 8g+7
+//   D (16 x 16): lane holds column c16, rows 4g .. 4g+3 (one per accumulator register)
+// A contraction may visit its k index in any order as long as A and B agree, so the
+// accumulator of a score tile (rows 4g+r) is fed straight back as the B operand of the
+// second product: two score tiles give the 8 k-slots of one lane, no cross-lane traffic.
+//
+// Scores are produced in log2 units: scale*log2(e) is folded into the latent queries when
+// they are converted to MFMA operands, and the softmax shift enters as the accumulator
+// input (C = -shift), so the steady state per score is exp2 + pack + dot2 only.  The
+// shift is lazy: it is only required to stay within 2^kLazyLog2 of the running maximum,
+// which is checked from the per-tile sums; a tile that violates it (and every ragged or
+// masked tile) goes through an exact path that recomputes the maximum and rescales.
+//
+//   gather : z = softmax_n(s q k^T) v   split over N, partial (shift, sum, numerator)
+//   scatter: y = softmax_m(s k q^T) z   token parallel, Q and Z^T resident in LDS
+#include "common.hpp"
+
+namespace flare {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr float kLazyLimit = 1024.f;  // 2^10: largest per-tile partial sum the lazy shift accepts
+
+template <typename T> struct Mma;
+
+template <> struct Mma<bf16_t> {
+    static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        bf16x2 v = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float sum2(uint32_t pk, float acc)
+    {
+        const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), ones, acc, false);
+    }
+};
+
+template <> struct Mma<f16_t> {
+    static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        f16x2 v = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float sum2(uint32_t pk, float acc)
+    {
+        const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pk), ones, acc, false);
+    }
+};
+
+template <typename T> __device__ __forceinline__ uint16_t elem_bits(float v);
+template <> __device__ __forceinline__ uint16_t elem_bits<bf16_t>(float v) { return f32_to_bf16_bits(v); }
+template <> __device__ __forceinline__ uint16_t elem_bits<f16_t>(float v)
+{
+    _Float16 hv = (_Float16)v;
+    return __builtin_bit_cast(uint16_t, hv);
+}
+template <typename T> __device__ __forceinline__ float bits_elem(uint16_t b);
+template <> __device__ __forceinline__ float bits_elem<bf16_t>(uint16_t b) { return __uint_as_float(uint32_t(b) << 16); }
+template <> __device__ __forceinline__ float bits_elem<f16_t>(uint16_t b) { return float(__builtin_bit_cast(_Float16, b)); }
+
+__device__ __forceinline__ u32x4 zero4() { return u32x4{0u, 0u, 0u, 0u}; }
+
+// 8 elements (16 bytes) from global memory
+__device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+
+// multiply 8 packed elements by f (fp32) and repack
+template <typename T> __device__ __forceinline__ u32x4 scale8(u32x4 v, float f)
+{
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float lo = bits_elem<T>(uint16_t(v[i] & 0xffffu)) * f;
+        const float hi = bits_elem<T>(uint16_t(v[i] >> 16)) * f;
+        o[i] = uint32_t(elem_bits<T>(lo)) | (uint32_t(elem_bits<T>(hi)) << 16);
+    }
+    return o;
+}
+
+__device__ __forceinline__ float xg_max(float v)  // max over the 4 lane groups of a column
+{
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+__device__ __forceinline__ float xg_sum(float v)
+{
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+
+// =====================================================================================
+// gather
+// =====================================================================================
+constexpr int kGTile = 64;            // tokens per barrier step (2 k-steps of 32)
+constexpr int kGVtStride = kGTile + 8;  // elements per V^T row in LDS (pad: conflict-free b128 reads)
+
+// One workgroup = 4 waves, 64*CT latents (wave w owns 16*CT of them), one token range.
+template <typename T, int D, int CT>
+__global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
+{
+    constexpr int KD = (D + 31) / 32;   // k-steps over d for the score product
+    constexpr int RT = D / 16;          // 16-row tiles of z^T
+    constexpr int CH = D / 8;           // 16-byte chunks per row
+    constexpr int MB = 64 * CT;
+    using M_ = Mma<T>;
+
+    __shared__ __attribute__((aligned(16))) uint16_t vt[2][D][kGVtStride];
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int mblocks = a.M / MB;
+    const int split = blockIdx.x / mblocks, mb = blockIdx.x % mblocks;
+    const int h = blockIdx.y, b = blockIdx.z;
+
+    const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
+    const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
+    const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
+    const uint8_t* mask = a.mask ? a.mask + (int64_t)b * a.N : nullptr;
+    const int m_base = mb * MB + w * 16 * CT;
+
+    // latent operands (B of the score product), log2-scaled
+    u32x4 qb[CT][KD];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const int ch = kd * 4 + g;
+            qb[ct][kd] = ch < CH ? scale8<T>(load16(q + (int64_t)(m_base + ct * 16 + c16) * a.qs[2] + ch * 8),
+                                             a.scale_log2)
+                                 : zero4();
+        }
+
+    float shift[CT], lsum[CT];
+    f32x4 zacc[RT][CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        shift[ct] = kNegBig;
+        lsum[ct] = 0.f;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int n_begin = split * a.tokens_per_split;
+    const int n_end = min(a.N, n_begin + a.tokens_per_split);
+
+    // V staging: 16-byte chunk c of the tile = (token c / CH, chunk c % CH)
+    constexpr int VCH = kGTile * CH;              // chunks per tile
+    constexpr int VPT = (VCH + 255) / 256;        // chunks per thread
+    u32x4 ka[4][KD], kn[4][KD], vr[VPT];
+
+    auto load_k = [&](int n0, u32x4 (&dst)[4][KD]) {
+#pragma unroll
+        for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                const int n = n0 + sub * 16 + c16, ch = kd * 4 + g;
+                dst[sub][kd] = (n < n_end && ch < CH) ? load16(k + (int64_t)n * a.ks[2] + ch * 8) : zero4();
+            }
+    };
+    auto load_v = [&](int n0) {
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int c = tid + i * 256;
+            const int j = c / CH, ch = c % CH;
+            vr[i] = (c < VCH && n0 + j < n_end) ? load16(v + (int64_t)(n0 + j) * a.vs[2] + ch * 8) : zero4();
+        }
+    };
+    auto store_v = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int c = tid + i * 256;
+            if (c < VCH) {
+                const int j = c / CH, ch = c % CH;
+                // token j = ks*32 + t*16 + 4*gg + e  ->  column ks*32 + gg*8 + t*4 + e
+                const int pos = (j & 32) | (((j >> 2) & 3) << 3) | (((j >> 4) & 1) << 2) | (j & 3);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    vt[buf][ch * 8 + 2 * e][pos] = uint16_t(vr[i][e] & 0xffffu);
+                    vt[buf][ch * 8 + 2 * e + 1][pos] = uint16_t(vr[i][e] >> 16);
+                }
+            }
+        }
+    };
+
+    if (n_begin < n_end) {
+        load_k(n_begin, ka);
+        load_v(n_begin);
+    }
+
+    int it = 0;
+    for (int n0 = n_begin; n0 < n_end; n0 += kGTile, ++it) {
+        const int buf = it & 1;
+        store_v(buf);
+        if (n0 + kGTile < n_end) {
+            load_k(n0 + kGTile, kn);
+            load_v(n0 + kGTile);
+        }
+        __syncthreads();
+
+        const bool exact_tile = (n0 + kGTile > n_end) || (mask != nullptr);
+
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            uint32_t pk[CT][4];
+            float tsum[CT];
+            bool bad = exact_tile;
+            if (!exact_tile) {
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    const float nc = -shift[ct];
+                    f32x4 s0 = {nc, nc, nc, nc}, s1 = {nc, nc, nc, nc};
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) {
+                        s0 = M_::mma(ka[2 * ks][kd], qb[ct][kd], s0);
+                        s1 = M_::mma(ka[2 * ks + 1][kd], qb[ct][kd], s1);
+                    }
+                    pk[ct][0] = M_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1]));
+                    pk[ct][1] = M_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3]));
+                    pk[ct][2] = M_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1]));
+                    pk[ct][3] = M_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]));
+                    float t = M_::sum2(pk[ct][0], 0.f);
+                    t = M_::sum2(pk[ct][1], t);
+                    t = M_::sum2(pk[ct][2], t);
+                    t = M_::sum2(pk[ct][3], t);
+                    tsum[ct] = t;
+                    bad = bad || !(t < kLazyLimit);
+                }
+            }
+            if (__any(bad)) {
+                // exact path: true tile maximum, rescale of the running partial, validity
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) {
+                        s0 = M_::mma(ka[2 * ks][kd], qb[ct][kd], s0);
+                        s1 = M_::mma(ka[2 * ks + 1][kd], qb[ct][kd], s1);
+                    }
+                    float sc[8];
+                    bool ok[8];
+                    float mx = kNegBig;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int n = n0 + ks * 32 + (e >> 2) * 16 + 4 * g + (e & 3);
+                        ok[e] = n < n_end && (mask == nullptr || mask[n] != 0);
+                        sc[e] = e < 4 ? s0[e] : s1[e - 4];
+                        if (ok[e]) mx = fmaxf(mx, sc[e]);
+                    }
+                    mx = xg_max(mx);
+                    const float nc = fmaxf(shift[ct], mx);
+                    const float al = fast_exp2(shift[ct] - nc);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] *= al;
+                    lsum[ct] *= al;
+                    shift[ct] = nc;
+                    float p[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) p[e] = ok[e] ? fast_exp2(sc[e] - nc) : 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) pk[ct][e] = M_::pack2(p[2 * e], p[2 * e + 1]);
+                    float t = M_::sum2(pk[ct][0], 0.f);
+                    t = M_::sum2(pk[ct][1], t);
+                    t = M_::sum2(pk[ct][2], t);
+                    t = M_::sum2(pk[ct][3], t);
+                    tsum[ct] = t;
+                }
+            }
+            u32x4 va[RT];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+                va[rt] = *reinterpret_cast<const u32x4*>(&vt[buf][rt * 16 + c16][ks * 32 + g * 8]);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const u32x4 pb = {pk[ct][0], pk[ct][1], pk[ct][2], pk[ct][3]};
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = M_::mma(va[rt], pb, zacc[rt][ct]);
+                lsum[ct] += tsum[ct];
+            }
+        }
+
+        if (n0 + kGTile < n_end) {
+#pragma unroll
+            for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) ka[sub][kd] = kn[sub][kd];
+        }
+    }
+
+    // partial for this split: shift (log2 units), sum, numerator
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const float l = xg_sum(lsum[ct]);
+        const int m = m_base + ct * 16 + c16;
+        const int64_t row = (((int64_t)b * a.H + h) * a.n_parts + split) * a.M + m;
+        if (g == 0) {
+            a.part_m[row] = shift[ct];
+            a.part_l[row] = l;
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+            *reinterpret_cast<f32x4*>(a.part_acc + row * D + rt * 16 + 4 * g) = zacc[rt][ct];
+    }
+}
+
+// =====================================================================================
+// scatter
+// =====================================================================================
+constexpr int kSTW = 4;             // 16-token column tiles per wave iteration
+constexpr int kSTokWave = 16 * kSTW;
+
+// One workgroup = 4 independent waves sharing Q and Z^T operands in LDS; wave w walks the
+// workgroup's token range in steps of 64 tokens.  No barrier after the set-up.
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int tokens_per_wg)
+{
+    constexpr int KD = (D + 31) / 32;
+    constexpr int RT = D / 16;
+    constexpr int CH = D / 8;
+    using M_ = Mma<T>;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    // qa[mt][ch][c16]  : 16 bytes each, latent m = 16 mt + c16, d = 8 ch .. 8 ch + 7
+    // zt[ks][rt][lane] : 16 bytes each, row d = (D/4) (c16/4) + 4 rt + c16 % 4,
+    //                    slots e<4 -> m = 32 ks + 4 g + e, e>=4 -> m = 32 ks + 16 + 4 g + e - 4
+    u32x4* qa = reinterpret_cast<u32x4*>(smem);
+    u32x4* zt = qa + (size_t)a.M * CH;
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int M = a.M, MT = M / 16, KS = M / 32;
+
+    const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
+    const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
+    uint16_t* y = (uint16_t*)a.y + b * a.ys[0] + h * a.ys[1];
+    const float* z = a.z + ((int64_t)b * a.H + h) * M * D;
+    const uint8_t* mask = a.mask ? a.mask + (int64_t)b * a.N : nullptr;
+
+    for (int idx = tid; idx < M * CH; idx += 256) {
+        const int m = idx / CH, ch = idx % CH;
+        qa[((m >> 4) * CH + ch) * 16 + (m & 15)] =
+            scale8<T>(load16(q + (int64_t)m * a.qs[2] + ch * 8), a.scale_log2);
+    }
+    for (int idx = tid; idx < KS * RT * 64; idx += 256) {
+        const int ln = idx & 63, rt = (idx >> 6) % RT, ks = idx / (64 * RT);
+        const int cc = ln & 15, gg = ln >> 4;
+        const int d = (D / 4) * (cc >> 2) + 4 * rt + (cc & 3);
+        u32x4 o;
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+            const int e = 2 * e2;
+            const int m0 = 32 * ks + (e >> 2) * 16 + 4 * gg + (e & 3);
+            o[e2] = uint32_t(elem_bits<T>(z[(int64_t)m0 * D + d])) |
+                    (uint32_t(elem_bits<T>(z[(int64_t)(m0 + 1) * D + d])) << 16);
+        }
+        zt[idx] = o;
+    }
+    __syncthreads();
+
+    const int wg_n0 = blockIdx.x * tokens_per_wg;
+    const int wg_n1 = min(a.N, wg_n0 + tokens_per_wg);
+
+    u32x4 kb[kSTW][KD], kn[kSTW][KD];
+    auto load_k = [&](int t0, u32x4 (&dst)[kSTW][KD]) {
+#pragma unroll
+        for (int tw = 0; tw < kSTW; ++tw)
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                const int n = t0 + tw * 16 + c16, ch = kd * 4 + g;
+                dst[tw][kd] = (n < wg_n1 && ch < CH) ? load16(k + (int64_t)n * a.ks[2] + ch * 8) : zero4();
+            }
+    };
+
+    int t0 = wg_n0 + w * kSTokWave;
+    if (t0 < wg_n1) load_k(t0, kb);
+
+    for (; t0 < wg_n1; t0 += 4 * kSTokWave) {
+        const int tnext = t0 + 4 * kSTokWave;
+        if (tnext < wg_n1) load_k(tnext, kn);
+
+        f32x4 yacc[kSTW][RT];
+        float shift[kSTW], lsum[kSTW];
+#pragma unroll
+        for (int tw = 0; tw < kSTW; ++tw) {
+            shift[tw] = kNegBig;
+            lsum[tw] = 0.f;
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+
+        for (int ks = 0; ks < KS; ++ks) {
+            u32x4 q0[KD], q1[KD], za[RT];
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                const int ch = kd * 4 + g;
+                q0[kd] = ch < CH ? qa[((2 * ks) * CH + ch) * 16 + c16] : zero4();
+                q1[kd] = ch < CH ? qa[((2 * ks + 1) * CH + ch) * 16 + c16] : zero4();
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) za[rt] = zt[(ks * RT + rt) * 64 + lane];
+
+            uint32_t pk[kSTW][4];
+            float tsum[kSTW];
+            bool bad = (ks == 0);
+            if (ks != 0) {
+#pragma unroll
+                for (int tw = 0; tw < kSTW; ++tw) {
+                    const float nc = -shift[tw];
+                    f32x4 s0 = {nc, nc, nc, nc}, s1 = {nc, nc, nc, nc};
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) {
+                        s0 = M_::mma(q0[kd], kb[tw][kd], s0);
+                        s1 = M_::mma(q1[kd], kb[tw][kd], s1);
+                    }
+                    pk[tw][0] = M_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1]));
+                    pk[tw][1] = M_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3]));
+                    pk[tw][2] = M_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1]));
+                    pk[tw][3] = M_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]));
+                    float t = M_::sum2(pk[tw][0], 0.f);
+                    t = M_::sum2(pk[tw][1], t);
+                    t = M_::sum2(pk[tw][2], t);
+                    t = M_::sum2(pk[tw][3], t);
+                    tsum[tw] = t;
+                    bad = bad || !(t < kLazyLimit);
+                }
+            }
+            if (__any(bad)) {
+#pragma unroll
+                for (int tw = 0; tw < kSTW; ++tw) {
+                    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) {
+                        s0 = M_::mma(q0[kd], kb[tw][kd], s0);
+                        s1 = M_::mma(q1[kd], kb[tw][kd], s1);
+                    }
+                    float mx = fmaxf(fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])),
+                                     fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
+                    mx = xg_max(mx);
+                    const float nc = fmaxf(shift[tw], mx);
+                    const float al = fast_exp2(shift[tw] - nc);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] *= al;
+                    lsum[tw] *= al;
+                    shift[tw] = nc;
+                    pk[tw][0] = M_::pack2(fast_exp2(s0[0] - nc), fast_exp2(s0[1] - nc));
+                    pk[tw][1] = M_::pack2(fast_exp2(s0[2] - nc), fast_exp2(s0[3] - nc));
+                    pk[tw][2] = M_::pack2(fast_exp2(s1[0] - nc), fast_exp2(s1[1] - nc));
+                    pk[tw][3] = M_::pack2(fast_exp2(s1[2] - nc), fast_exp2(s1[3] - nc));
+                    float t = M_::sum2(pk[tw][0], 0.f);
+                    t = M_::sum2(pk[tw][1], t);
+                    t = M_::sum2(pk[tw][2], t);
+                    t = M_::sum2(pk[tw][3], t);
+                    tsum[tw] = t;
+                }
+            }
+#pragma unroll
+            for (int tw = 0; tw < kSTW; ++tw) {
+                const u32x4 pb = {pk[tw][0], pk[tw][1], pk[tw][2], pk[tw][3]};
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = M_::mma(za[rt], pb, yacc[tw][rt]);
+                lsum[tw] += tsum[tw];
+            }
+        }
+
+        // normalise and store: lane (token c16, group g) owns d = (D/4) g .. (D/4) g + D/4 - 1
+#pragma unroll
+        for (int tw = 0; tw < kSTW; ++tw) {
+            const int n = t0 + tw * 16 + c16;
+            const float l = xg_sum(lsum[tw]);
+            const bool on = n < wg_n1 && (mask == nullptr || mask[n] != 0);
+            const float inv = on ? 1.f / l : 0.f;
+            if (n < wg_n1) {
+                uint16_t* yr = y + (int64_t)n * a.ys[2] + (D / 4) * g;
+                uint32_t o[2 * RT];
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    o[2 * rt] = M_::pack2(yacc[tw][rt][0] * inv, yacc[tw][rt][1] * inv);
+                    o[2 * rt + 1] = M_::pack2(yacc[tw][rt][2] * inv, yacc[tw][rt][3] * inv);
+                }
+                if constexpr (RT == 1) {
+                    *reinterpret_cast<uint2*>(yr) = make_uint2(o[0], o[1]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < RT / 2; ++i)
+                        *reinterpret_cast<u32x4*>(yr + 8 * i) = u32x4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+                }
+            }
+        }
+
+        if (tnext < wg_n1) {
+#pragma unroll
+            for (int tw = 0; tw < kSTW; ++tw)
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) kb[tw][kd] = kn[tw][kd];
+        }
+    }
+}
+
+constexpr size_t kScatterLdsMax = 150 * 1024;
+
+template <typename T, int D>
+hipError_t gather_launch_ct(const MixerArgs& a, hipStream_t st)
+{
+    const int MB = (a.M % 256 == 0) ? 256 : (a.M % 128 == 0) ? 128 : 64;
+    dim3 grid(a.n_splits * (a.M / MB), a.H, a.B);
+    if (MB == 256)      hipLaunchKernelGGL((gather_mfma_kernel<T, D, 4>), grid, dim3(256), 0, st, a);
+    else if (MB == 128) hipLaunchKernelGGL((gather_mfma_kernel<T, D, 2>), grid, dim3(256), 0, st, a);
+    else                hipLaunchKernelGGL((gather_mfma_kernel<T, D, 1>), grid, dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t gather_launch_d(const MixerArgs& a, hipStream_t st)
+{
+    switch (a.D) {
+        case 16: return gather_launch_ct<T, 16>(a, st);
+        case 32: return gather_launch_ct<T, 32>(a, st);
+        case 64: return gather_launch_ct<T, 64>(a, st);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+template <typename T, int D>
+hipError_t scatter_launch(const MixerArgs& a, hipStream_t st)
+{
+    const size_t lds = (size_t)a.M * D * 2 * 2;
+    auto kern = scatter_mfma_kernel<T, D>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    // tokens per workgroup: aim at ~4 workgroups per CU over the whole grid, multiple of 256
+    const int64_t total = (int64_t)a.B * a.H * a.N;
+    int64_t tpw = (total + 1023) / 1024;
+    tpw = ((tpw + 255) / 256) * 256;
+    if (tpw < 256) tpw = 256;
+    if (tpw > 16384) tpw = 16384;
+    dim3 grid((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, a, (int)tpw);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t scatter_launch_d(const MixerArgs& a, hipStream_t st)
+{
+    switch (a.D) {
+        case 16: return scatter_launch<T, 16>(a, st);
+        case 32: return scatter_launch<T, 32>(a, st);
+        case 64: return scatter_launch<T, 64>(a, st);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+bool mfma_mixer_supported(int dtype, int M, int D)
+{
+    if (dtype != 1 && dtype != 2) return false;
+    if (D != 16 && D != 32 && D != 64) return false;
+    if (M < 64 || M % 64 != 0) return false;
+    if ((size_t)M * D * 4 > kScatterLdsMax) return false;
+    return true;
+}
+
+int mfma_gather_tokens_per_iter() { return kGTile; }
+
+hipError_t launch_gather_mfma(const MixerArgs& a, int dtype, hipStream_t st)
+{
+    return dtype == 1 ? gather_launch_d<bf16_t>(a, st) : gather_launch_d<f16_t>(a, st);
+}
+
+hipError_t launch_scatter_mfma(const MixerArgs& a, int dtype, hipStream_t st)
+{
+    return dtype == 1 ? scatter_launch_d<bf16_t>(a, st) : scatter_launch_d<f16_t>(a, st);
+}
+
+}  // namespace flare

@@ -1,0 +1,372 @@
+"""Functional API of the MI355X FLARE engine.
+
+Mirrors the reference's operator interface (paths relative to the reference tree):
+  flare_multihead_mixer(q, k, v)          README.md:39-52
+  TripleAttentionFunction.apply(...)      lra/models/triton/triple.py:27-121 -> (STATE, O)
+and adds the entry points the causal path needs (flare_causal_prefill / _decode).
+
+Every function here launches HIP kernels from libflare_hip.so through ctypes.  torch is
+used for device memory, streams and autograd plumbing only; there is no PyTorch or CPU
+implementation behind these calls, and a missing library raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import FlareCausalDesc, FlareMixerDesc, FlareTripleDesc
+
+_DTYPES = {torch.float32: _lib.DT_F32, torch.bfloat16: _lib.DT_BF16, torch.float16: _lib.DT_F16}
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}; expected float32, bfloat16 or float16") from None
+
+
+def _require_cuda(*ts: torch.Tensor):
+    dev = ts[0].device
+    for t in ts:
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                "FLARE HIP kernels need tensors on a HIP device ('cuda'); got "
+                f"{t.device}. There is no CPU implementation in this package.")
+        if t.device != dev:
+            raise RuntimeError("all tensors must live on the same device")
+
+
+def _rows_last_contig(t: torch.Tensor) -> torch.Tensor:
+    """[B,H,N,D] tensor usable without a copy iff its innermost stride is 1."""
+    if t.stride(-1) != 1 and t.size(-1) != 1:
+        return t.contiguous()
+    return t
+
+
+def _s3(t: torch.Tensor):
+    """(b, h, row) element strides of a 4-d tensor."""
+    return _lib.I3(t.stride(0), t.stride(1), t.stride(2))
+
+
+def _q4(q: torch.Tensor, B: int) -> torch.Tensor:
+    """Latent queries as a [B?,H,M,D] view; a 3-d q is shared over the batch (stride 0)."""
+    if q.dim() == 3:
+        q = q.unsqueeze(0).expand(B, -1, -1, -1)
+    elif q.dim() != 4:
+        raise ValueError(f"q must be [H,M,D] or [B,H,M,D], got shape {tuple(q.shape)}")
+    if q.stride(-1) != 1 and q.size(-1) != 1:
+        q = q.contiguous()
+    return q
+
+
+def _stream_ptr(dev) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _mixer_desc(q4, k, v, y, scale, n_splits, force_generic) -> FlareMixerDesc:
+    B, H, N, D = k.shape
+    d = FlareMixerDesc()
+    d.B, d.H, d.N, d.M, d.D = B, H, N, q4.shape[2], D
+    d.dtype = _dtype_code(k)
+    d.scale = float(scale)
+    d.n_splits = int(n_splits)
+    d.flags = _lib.FLAG_FORCE_GENERIC if force_generic else 0
+    d.q_stride = _s3(q4)
+    d.k_stride = _s3(k)
+    d.v_stride = _s3(v if v is not None else k)
+    d.y_stride = _s3(y if y is not None else k)
+    return d
+
+
+def _check_mixer_shapes(q4, k, v):
+    if k.dim() != 4:
+        raise ValueError(f"k must be [B,H,N,D], got {tuple(k.shape)}")
+    if v is not None and v.shape != k.shape:
+        raise ValueError(f"v {tuple(v.shape)} must match k {tuple(k.shape)}")
+    B, H, N, D = k.shape
+    if q4.shape[0] != B or q4.shape[1] != H or q4.shape[3] != D:
+        raise ValueError(f"q {tuple(q4.shape)} does not match k {tuple(k.shape)}")
+
+
+def _mask_u8(key_mask, B, N, device):
+    if key_mask is None:
+        return None
+    if key_mask.shape != (B, N):
+        raise ValueError(f"key_mask must be [B,N]=({B},{N}), got {tuple(key_mask.shape)}")
+    return key_mask.to(device=device, dtype=torch.uint8).contiguous()
+
+
+def mixer_kernel_name(q, k, v=None, scale=1.0, force_generic=False) -> str:
+    """Which kernel family the dispatcher picks for these operands (no launch)."""
+    q4 = _q4(q, k.shape[0])
+    d = _mixer_desc(q4, k, v, None, scale, 0, force_generic)
+    name = _lib.load().flare_mixer_kernel_name(C.byref(d))
+    if name is None:
+        raise ValueError(_lib.last_error())
+    return name.decode()
+
+
+def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic):
+    _require_cuda(q, k, v)
+    lib = _lib.load()
+    if q.dtype != k.dtype:
+        q = q.to(k.dtype)
+    if v.dtype != k.dtype:
+        raise TypeError("k and v must share a dtype")
+    k, v = _rows_last_contig(k), _rows_last_contig(v)
+    q4 = _q4(q, k.shape[0])
+    _check_mixer_shapes(q4, k, v)
+    B, H, N, D = k.shape
+    M = q4.shape[2]
+    y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    z = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
+    mask = _mask_u8(key_mask, B, N, k.device)
+    d = _mixer_desc(q4, k, v, y, scale, n_splits, force_generic)
+    need = C.c_size_t(0)
+    _lib.check(lib.flare_mixer_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_workspace_bytes")
+    ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
+    with torch.cuda.device(k.device):
+        rc = lib.flare_mixer_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(mask), _ptr(y), _ptr(z),
+                                 _ptr(ws), ws.numel(), C.c_void_p(_stream_ptr(k.device)))
+    _lib.check(rc, "flare_mixer_fwd")
+    return y, z
+
+
+def _mixer_torch_grad(q, k, v, scale, key_mask, gy):
+    """Backward by recomputation in plain torch ops on the device the inputs live on.
+    The HIP backward kernels are not built yet; the forward never takes this path."""
+    with torch.enable_grad():
+        q_, k_, v_ = (t.detach().float().requires_grad_(True) for t in (q, k, v))
+        qe = q_ if q_.dim() == 4 else q_.unsqueeze(0)
+        s = scale * (qe @ k_.transpose(-2, -1))
+        if key_mask is not None:
+            keep = key_mask.to(torch.bool)[:, None, None, :]
+            s_enc = s.masked_fill(~keep, float("-inf"))
+        else:
+            s_enc = s
+        z = torch.softmax(s_enc, dim=-1) @ v_
+        y = torch.softmax(s.transpose(-2, -1), dim=-1) @ z
+        if key_mask is not None:
+            y = y * key_mask.to(y.dtype)[:, None, :, None]
+        gq, gk, gv = torch.autograd.grad(y, (q_, k_, v_), gy.float())
+    return gq.to(q.dtype), gk.to(k.dtype), gv.to(v.dtype)
+
+
+class _MixerFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, scale, key_mask, n_splits, force_generic):
+        y, z = _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic)
+        ctx.save_for_backward(q, k, v)
+        ctx.scale, ctx.key_mask = scale, key_mask
+        ctx.mark_non_differentiable(z)
+        return y, z
+
+    @staticmethod
+    def backward(ctx, gy, _gz):
+        q, k, v = ctx.saved_tensors
+        gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy)
+        return gq, gk, gv, None, None, None, None
+
+
+def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: bool = False,
+                          n_splits: int = 0, force_generic: bool = False):
+    """FLARE gather-scatter mixer (README.md:39-52 of the reference).
+
+    q: [H,M,D] latent queries (or [B,H,M,D]); k, v: [B,H,N,D]; returns y [B,H,N,D] with
+      z = softmax_n(scale q k^T) v ;  y = softmax_m(scale k q^T) z
+    key_mask ([B,N], nonzero = token present) removes padded tokens from the gather and
+    zeroes their output rows (lra/models/backends.py:603-606,615-622).
+    k and v may be strided views (e.g. 'b n (h d) -> b h n d') as long as D is contiguous.
+    """
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+        y, z = _MixerFn.apply(q, k, v, float(scale), key_mask, n_splits, force_generic)
+    else:
+        y, z = _mixer_forward(q, k, v, float(scale), key_mask, n_splits, force_generic)
+    return (y, z) if return_z else y
+
+
+def flare_gather(q, k, v, scale: float = 1.0, key_mask=None, n_splits: int = 0,
+                 force_generic: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """z [B,H,M,D] fp32 = softmax_n(scale q k^T) v and lse [B,H,M] (natural log)."""
+    _require_cuda(q, k, v)
+    lib = _lib.load()
+    if q.dtype != k.dtype:
+        q = q.to(k.dtype)
+    k, v = _rows_last_contig(k), _rows_last_contig(v)
+    q4 = _q4(q, k.shape[0])
+    _check_mixer_shapes(q4, k, v)
+    B, H, N, D = k.shape
+    M = q4.shape[2]
+    z = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
+    lse = torch.empty((B, H, M), dtype=torch.float32, device=k.device)
+    mask = _mask_u8(key_mask, B, N, k.device)
+    d = _mixer_desc(q4, k, v, None, scale, n_splits, force_generic)
+    need = C.c_size_t(0)
+    _lib.check(lib.flare_mixer_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_workspace_bytes")
+    ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
+    with torch.cuda.device(k.device):
+        rc = lib.flare_gather_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(mask), _ptr(z), _ptr(lse),
+                                  _ptr(ws), ws.numel(), C.c_void_p(_stream_ptr(k.device)))
+    _lib.check(rc, "flare_gather_fwd")
+    return z, lse
+
+
+def flare_scatter(q, k, z, scale: float = 1.0, key_mask=None, force_generic: bool = False) -> torch.Tensor:
+    """y [B,H,N,D] = softmax_m(scale k q^T) z with z [B,H,M,D] fp32."""
+    _require_cuda(q, k, z)
+    lib = _lib.load()
+    if q.dtype != k.dtype:
+        q = q.to(k.dtype)
+    k = _rows_last_contig(k)
+    q4 = _q4(q, k.shape[0])
+    _check_mixer_shapes(q4, k, None)
+    B, H, N, D = k.shape
+    M = q4.shape[2]
+    if z.shape != (B, H, M, D):
+        raise ValueError(f"z must be [B,H,M,D]=({B},{H},{M},{D}), got {tuple(z.shape)}")
+    z = z.to(torch.float32).contiguous()
+    y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    mask = _mask_u8(key_mask, B, N, k.device)
+    d = _mixer_desc(q4, k, None, y, scale, 0, force_generic)
+    with torch.cuda.device(k.device):
+        rc = lib.flare_scatter_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(z), _ptr(mask), _ptr(y),
+                                   C.c_void_p(_stream_ptr(k.device)))
+    _lib.check(rc, "flare_scatter_fwd")
+    return y
+
+
+# --------------------------------------------------------------------------------------
+# causal FLARE
+# --------------------------------------------------------------------------------------
+def causal_fresh_state(B, H, M, D, device):
+    """(mu, den, num) of an empty prefix: mu = -inf, den = 0, num = 0 (fp32)."""
+    mu = torch.full((B, H, M), float("-inf"), dtype=torch.float32, device=device)
+    den = torch.zeros((B, H, M), dtype=torch.float32, device=device)
+    num = torch.zeros((B, H, M, D), dtype=torch.float32, device=device)
+    return mu, den, num
+
+
+def _causal_call(entry, q, k, v, scale, chunk, state):
+    _require_cuda(q, k, v)
+    lib = _lib.load()
+    if q.dtype != k.dtype:
+        q = q.to(k.dtype)
+    if v.dtype != k.dtype or v.shape != k.shape or k.dim() != 4:
+        raise ValueError("k and v must be [B,H,N,D] tensors of one dtype")
+    k, v = _rows_last_contig(k), _rows_last_contig(v)
+    B, H, N, D = k.shape
+    q4 = _q4(q, B)
+    _check_mixer_shapes(q4, k, v)
+    M = q4.shape[2]
+    if state is None:
+        mu, den, num = causal_fresh_state(B, H, M, D, k.device)
+    else:
+        mu, den, num = (s.to(device=k.device, dtype=torch.float32).contiguous().clone() for s in state)
+        if mu.shape != (B, H, M) or den.shape != (B, H, M) or num.shape != (B, H, M, D):
+            raise ValueError("state must be (mu[B,H,M], den[B,H,M], num[B,H,M,D])")
+    y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    d = FlareCausalDesc()
+    d.B, d.H, d.N, d.M, d.D = B, H, N, M, D
+    d.dtype = _dtype_code(k)
+    d.scale = float(scale)
+    d.chunk = int(chunk)
+    d.q_stride, d.k_stride, d.v_stride, d.y_stride = _s3(q4), _s3(k), _s3(v), _s3(y)
+    st = C.c_void_p(_stream_ptr(k.device))
+    with torch.cuda.device(k.device):
+        if entry == "prefill":
+            need = C.c_size_t(0)
+            _lib.check(lib.flare_causal_workspace_bytes(C.byref(d), C.byref(need)), "flare_causal_workspace_bytes")
+            ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
+            rc = lib.flare_causal_prefill_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(y), _ptr(mu),
+                                              _ptr(den), _ptr(num), _ptr(ws), ws.numel(), st)
+        else:
+            rc = lib.flare_causal_decode_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(y), _ptr(mu),
+                                             _ptr(den), _ptr(num), st)
+    _lib.check(rc, f"flare_causal_{entry}_fwd")
+    return y, (mu, den, num)
+
+
+def flare_causal_prefill(q, k, v, scale: float = 1.0, chunk: int = 256, state=None):
+    """Causal FLARE over N tokens: y_t uses keys/values of tokens <= t only.
+    Returns (y [B,H,N,D], state) where state = (mu, den, num) continues the recurrence."""
+    return _causal_call("prefill", q, k, v, scale, chunk, state)
+
+
+def flare_causal_decode(q, k, v, state, scale: float = 1.0):
+    """n recurrent single-token steps in one launch; k, v are [B,H,n,D]."""
+    return _causal_call("decode", q, k, v, scale, 0, state)
+
+
+def flare_causal_decode_step(q, k_t, v_t, state, scale: float = 1.0):
+    """One token: k_t, v_t are [B,H,D] or [B,H,1,D]."""
+    squeeze = k_t.dim() == 3
+    if squeeze:
+        k_t, v_t = k_t.unsqueeze(2), v_t.unsqueeze(2)
+    y, st = _causal_call("decode", q, k_t, v_t, scale, 0, state)
+    return (y.squeeze(2) if squeeze else y), st
+
+
+# --------------------------------------------------------------------------------------
+# triple attention
+# --------------------------------------------------------------------------------------
+def _triple_forward(q1, q2, k1, k2, v, feature_map: bool, normalize: bool, n_splits: int = 0):
+    _require_cuda(q1, q2, k1, k2, v)
+    lib = _lib.load()
+    if not (q1.shape == q2.shape == k1.shape == k2.shape):
+        raise ValueError("q1, q2, k1, k2 must share one shape [B,H,N,Dq]")
+    if v.shape[:-1] != q1.shape[:-1] or q1.dim() != 4:
+        raise ValueError("v must be [B,H,N,Dv] with the same B,H,N as q1")
+    if not (q1.dtype == q2.dtype == k1.dtype == k2.dtype == v.dtype):
+        raise TypeError("all five inputs must share a dtype")
+    q1, q2, k1, k2, v = (_rows_last_contig(t) for t in (q1, q2, k1, k2, v))
+    B, H, N, Dq = q1.shape
+    Dv = v.shape[-1]
+    state = torch.empty((B, H, Dq, Dv, Dq), dtype=torch.float32, device=q1.device)
+    out = torch.empty((B, H, N, Dv), dtype=q1.dtype, device=q1.device)
+    d = FlareTripleDesc()
+    d.B, d.H, d.N, d.Dq, d.Dv = B, H, N, Dq, Dv
+    d.dtype = _dtype_code(q1)
+    d.feature_map = 1 if feature_map else 0
+    d.normalize = 1 if normalize else 0
+    d.n_splits = int(n_splits)
+    d.q1_stride, d.q2_stride, d.k1_stride, d.k2_stride = _s3(q1), _s3(q2), _s3(k1), _s3(k2)
+    d.v_stride, d.o_stride = _s3(v), _s3(out)
+    need = C.c_size_t(0)
+    _lib.check(lib.flare_triple_workspace_bytes(C.byref(d), C.byref(need)), "flare_triple_workspace_bytes")
+    ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=q1.device)
+    with torch.cuda.device(q1.device):
+        rc = lib.flare_triple_fwd(C.byref(d), _ptr(q1), _ptr(q2), _ptr(k1), _ptr(k2), _ptr(v), _ptr(state),
+                                  _ptr(out), _ptr(ws), ws.numel(), C.c_void_p(_stream_ptr(q1.device)))
+    _lib.check(rc, "flare_triple_fwd")
+    return state, out
+
+
+def triple_attention(q1, q2, k1, k2, v, normalize: bool = False, feature_map: Optional[str] = None,
+                     n_splits: int = 0):
+    """Third-order linear attention (lra/models/backends.py:1285-1292 of the reference).
+
+    Returns (state [B,H,Dq,Dv,Dq] fp32, out [B,H,N,Dv]).  feature_map=None expects inputs that
+    already went through the kernel map (as TripleAttention.forward does at backends.py:1258);
+    feature_map='elu' applies elu(x)+1 to q1,q2,k1,k2 inside the kernels.
+    normalize=True divides out by the matching normaliser (same contraction with v == 1).
+    """
+    if feature_map not in (None, "identity", "elu"):
+        raise ValueError("feature_map must be None, 'identity' or 'elu'")
+    return _triple_forward(q1, q2, k1, k2, v, feature_map == "elu", normalize, n_splits)
+
+
+class TripleAttentionFunction:
+    """Call-compatible stand-in for lra/models/triton/triple.py:27 `TripleAttentionFunction`:
+    `TripleAttentionFunction.apply(Q1, Q2, K1, K2, V) -> (STATE, O)`.  Forward only."""
+
+    @staticmethod
+    def apply(Q1, Q2, K1, K2, V):
+        return _triple_forward(Q1, Q2, K1, K2, V, False, False)

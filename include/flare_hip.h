@@ -1,0 +1,172 @@
+/*
+ * flare_hip.h — C-ABI of libflare_hip.so, the MI355X (gfx950) FLARE attention engine.
+ *
+ * Plain pointers and sizes only; no torch types.  Every device pointer is owned by the
+ * caller (inputs, outputs and the workspace).  The library allocates no device memory,
+ * keeps no mutable global state, launches asynchronously on the hipStream_t handed in
+ * (passed as void*) and never synchronises the device.  All entry points return an int
+ * status (0 = OK, negative = error); the text of the last error on the calling thread is
+ * available from flare_last_error_string().  Shapes, dtypes, strides, alignment and the
+ * workspace size are validated on the host BEFORE anything is launched.
+ *
+ * Reference interfaces each entry point replaces (paths relative to the reference tree):
+ *   flare_mixer_fwd            README.md:39-52 (flare_multihead_mixer),
+ *                              pdebench/models/flare.py:136-138, lra/models/backends.py:603-606
+ *   flare_gather_fwd           first F.scaled_dot_product_attention(q, k, v) of the above
+ *   flare_scatter_fwd          second F.scaled_dot_product_attention(k, q, z) of the above
+ *   flare_causal_prefill_fwd   causal restriction of the mixer (README.md:60 names it; the
+ *   flare_causal_decode_fwd    reference holds no code for it) following the 3-phase chunk
+ *                              scheme of lra/models/triton/causal_linear.py:81-137 and the
+ *                              token recurrence of causal_linear.py:317-336
+ *   flare_triple_fwd           TripleAttentionFunction.apply lra/models/triton/triple.py:29-121
+ *                              == TripleAttention.attn_einsum lra/models/backends.py:1285-1292
+ */
+#ifndef FLARE_HIP_H
+#define FLARE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FLARE_ABI_VERSION 1
+
+/* status codes */
+#define FLARE_OK            0
+#define FLARE_EINVAL       (-1)  /* null pointer, bad shape / stride / alignment            */
+#define FLARE_EUNSUPPORTED (-2)  /* valid request that no kernel covers (e.g. D > 128)      */
+#define FLARE_EWORKSPACE   (-3)  /* workspace missing or smaller than *_workspace_bytes()   */
+#define FLARE_EHIP         (-4)  /* a HIP runtime call failed (launch error)                */
+
+/* element types of q / k / v / y */
+#define FLARE_DT_F32  0
+#define FLARE_DT_BF16 1
+#define FLARE_DT_F16  2
+
+/* FlareMixerDesc.flags */
+#define FLARE_FLAG_FORCE_GENERIC 1  /* skip the MFMA kernels, use the fp32-FMA kernels */
+
+/*
+ * Mixer problem description.  Logical shapes:
+ *   q [B?,H,M,D]   latent queries; q_stride[0] == 0 means one set shared by every batch
+ *   k [B,H,N,D]    keys           v [B,H,N,D] values        y [B,H,N,D] output
+ *   z [B,H,M,D]    latent summary, ALWAYS fp32 and contiguous
+ * Strides are in ELEMENTS for dims (b, h, row); the innermost (D) stride must be 1, so
+ * the [B,N,H*D] views produced by 'b n (h d) -> b h n d' are consumed without a copy.
+ * Softmax and all accumulation are fp32 whatever the element type.
+ */
+typedef struct FlareMixerDesc {
+    int32_t B, H, N, M, D;
+    int32_t dtype;        /* FLARE_DT_* of q, k, v, y                                  */
+    float   scale;        /* softmax scale s: scores are s * <q_m, k_n>                */
+    int32_t n_splits;     /* gather split-N factor; 0 = choose automatically           */
+    int32_t flags;        /* FLARE_FLAG_*                                              */
+    int32_t reserved;
+    int64_t q_stride[3];
+    int64_t k_stride[3];
+    int64_t v_stride[3];
+    int64_t y_stride[3];
+} FlareMixerDesc;
+
+/*
+ * Causal FLARE.  Recurrent state per (b,h): mu[M] running max of s*<q_m,k_t>, den[M]
+ * softmax denominator relative to mu, num[M,D] numerator relative to mu; all fp32,
+ * contiguous [B,H,M], [B,H,M], [B,H,M,D].  A fresh state is mu=-inf (any value <= -1e30),
+ * den=0, num=0.  For token t:
+ *   sigma_m = s*<q_m,k_t>; mu' = max(mu, sigma); a = exp(mu-mu'); p = exp(sigma-mu');
+ *   den = a*den + p; num = a*num + p (x) v_t; y_t = sum_m softmax_m(sigma)_m * num_m/den_m
+ * k, v, y are [B,H,N,D] with the same stride convention as the mixer.
+ */
+typedef struct FlareCausalDesc {
+    int32_t B, H, N, M, D;
+    int32_t dtype;
+    float   scale;
+    int32_t chunk;        /* prefill chunk length (tokens); 0 = default 256            */
+    int32_t flags;
+    int32_t reserved;
+    int64_t q_stride[3];
+    int64_t k_stride[3];
+    int64_t v_stride[3];
+    int64_t y_stride[3];
+} FlareCausalDesc;
+
+/*
+ * Triple (third-order) linear attention.  q1,q2,k1,k2 [B,H,N,Dq], v [B,H,N,Dv],
+ *   state[b,h,i,j,k] = (1/N) sum_n f(k1)[n,i] v[n,j] f(k2)[n,k]      fp32 [B,H,Dq,Dv,Dq]
+ *   out[b,h,n,j]     = sum_{i,k} f(q1)[n,i] state[i,j,k] f(q2)[n,k]  [B,H,N,Dv]
+ * f = identity (feature_map 0) or elu(x)+1 (feature_map 1).  With normalize != 0 the
+ * output is divided by the same contraction evaluated with v == 1.
+ * All five inputs and out share one stride triple layout (b, h, n), innermost stride 1.
+ */
+typedef struct FlareTripleDesc {
+    int32_t B, H, N, Dq, Dv;
+    int32_t dtype;
+    int32_t feature_map;  /* 0 identity, 1 elu+1 applied to q1,q2,k1,k2 inside the kernel */
+    int32_t normalize;    /* 0 reference-exact (no denominator), 1 divide by normaliser  */
+    int32_t n_splits;     /* state split-N factor; 0 = automatic                         */
+    int32_t flags;
+    int64_t q1_stride[3], q2_stride[3], k1_stride[3], k2_stride[3], v_stride[3], o_stride[3];
+} FlareTripleDesc;
+
+int         flare_abi_version(void);
+const char* flare_last_error_string(void);
+
+/* Name of the kernel family the dispatcher would pick for this problem
+ * ("mfma_bf16", "mfma_f16", "generic"); NULL + error on an invalid descriptor. */
+const char* flare_mixer_kernel_name(const FlareMixerDesc* desc);
+
+/* Bytes of device workspace flare_gather_fwd / flare_mixer_fwd need for this problem. */
+int flare_mixer_workspace_bytes(const FlareMixerDesc* desc, size_t* bytes);
+
+/* z[B,H,M,D] (fp32) = softmax_n(s q k^T) v.  lse (fp32 [B,H,M], natural log of the softmax
+ * normaliser) may be NULL.  key_mask (uint8 [B,N], 1 = token present) may be NULL; a
+ * latent whose every key is masked gets z = 0. */
+int flare_gather_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
+                     const uint8_t* key_mask, float* z, float* lse,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* y[B,H,N,D] = softmax_m(s k q^T) z.  Rows of masked tokens are written as 0. */
+int flare_scatter_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const float* z,
+                      const uint8_t* key_mask, void* y, void* stream);
+
+/* gather + merge + scatter on one stream.  z_out (fp32 [B,H,M,D]) may be NULL, in which
+ * case z lives in the workspace. */
+int flare_mixer_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
+                    const uint8_t* key_mask, void* y, float* z_out,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+int flare_causal_workspace_bytes(const FlareCausalDesc* desc, size_t* bytes);
+
+/* Chunked prefill over N tokens; state (mu, den, num) is read, advanced and written back. */
+int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const void* k,
+                             const void* v, void* y, float* mu, float* den, float* num,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/* N recurrent single-token steps in ONE launch (desc->N = number of steps; k, v, y hold
+ * the steps along their n axis); the state stays on chip between steps. */
+int flare_causal_decode_fwd(const FlareCausalDesc* desc, const void* q, const void* k,
+                            const void* v, void* y, float* mu, float* den, float* num,
+                            void* stream);
+
+int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes);
+
+/* state only (split-N partial sums + fixed-order merge; no atomics). */
+int flare_triple_state_fwd(const FlareTripleDesc* desc, const void* k1, const void* k2,
+                           const void* v, float* state, float* kk_state,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
+/* out from a given state.  kk_state (fp32 [B,H,Dq,Dq]) is only read when normalize != 0. */
+int flare_triple_out_fwd(const FlareTripleDesc* desc, const void* q1, const void* q2,
+                         const float* state, const float* kk_state, void* out, void* stream);
+
+/* state + out.  The workspace also holds kk_state when normalize != 0. */
+int flare_triple_fwd(const FlareTripleDesc* desc, const void* q1, const void* q2,
+                     const void* k1, const void* k2, const void* v, float* state, void* out,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLARE_HIP_H */

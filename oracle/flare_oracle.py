@@ -1,0 +1,219 @@
+"""CPU oracle for the FLARE hot path — TEST INFRASTRUCTURE, not product code.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this
+module.  Nothing under the product package imports it, and the product never falls back
+to it: when the HIP library is missing the product raises.
+
+Every function restates, in plain torch on the CPU, the arithmetic of one reference
+function (paths relative to the reference tree):
+
+  mixer_sdpa            README.md:39-52; pdebench/models/flare.py:136-138 (fused branch)
+  mixer_explicit        pdebench/models/flare.py:142-150 (spelled-out branch; note that the
+                        reference omits attn_scale there, this restatement applies it so
+                        that it equals the fused branch for every scale)
+  mixer_masked_explicit lra/models/backends.py:603-606,615-622 (key mask for the gather;
+                        the scatter mask hits whole query rows, for which torch's result
+                        is backend dependent — this oracle defines those rows as 0)
+  triple_einsum         lra/models/backends.py:1285-1292 == lra/models/triton/triple.py:846-860
+  elu_plus_one          lra/models/kernels.py:23-24
+  causal_*              the reference has NO code for causal FLARE (README.md:60 links a blog
+                        post).  The definition adopted is the causal restriction of the
+                        mixer: z_t = softmax over tokens <= t, y_t = softmax_m(k_t q_m) z_t.
+                        causal_recurrent follows the token recurrence shape of
+                        lra/models/triton/causal_linear.py:317-336; causal_bruteforce applies
+                        mixer_explicit to every prefix and keeps the last row.
+
+Pinning status (what each function is checked against in tests/test_oracle.py):
+  mixer_sdpa / mixer_explicit : each other (independent code paths: torch's SDPA kernel vs
+      explicit softmax), the C restatement oracle/flare_oracle.c, closed forms (q=0 => mean,
+      N=1 => y=v, M=1 => rows equal z_0, convex-hull bounds, shift invariance,
+      permutation equivariance) and a pure-Python-float brute force.  The reference's own
+      tests hold no golden values for this path, so none are used.
+  causal_recurrent            : causal_bruteforce, last-row == non-causal mixer, chunk
+      independence; C restatement.
+  triple_einsum               : hand cases (N=1, D=1), pure-Python loops, linearity in v,
+      (k1,q1)<->(k2,q2) symmetry; C restatement.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+NEG_INF = float("-inf")
+
+
+# --------------------------------------------------------------------------------------
+# mixer
+# --------------------------------------------------------------------------------------
+def mixer_sdpa(q, k, v, scale=1.0):
+    """y = SDPA(k, q, SDPA(q, k, v)) on the torch MATH backend (README.md:49-50)."""
+    from torch.nn.attention import SDPBackend, sdpa_kernel
+
+    B = k.shape[0]
+    qe = q.unsqueeze(0).expand(B, -1, -1, -1) if q.dim() == 3 else q
+    with sdpa_kernel(SDPBackend.MATH):
+        z = F.scaled_dot_product_attention(qe, k, v, scale=scale)
+        y = F.scaled_dot_product_attention(k, qe, z, scale=scale)
+    return y, z
+
+
+def gather_explicit(q, k, v, scale=1.0, key_mask=None, dtype=torch.float64):
+    """z = softmax_n(s q k^T) v, plus lse = log sum_n exp(s q k^T)."""
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    if q.dim() == 3:
+        q = q.unsqueeze(0)
+    scores = scale * (q @ k.transpose(-2, -1))  # [B,H,M,N]
+    if key_mask is not None:
+        keep = key_mask.to(torch.bool)[:, None, None, :]
+        scores = scores.masked_fill(~keep, NEG_INF)
+    lse = torch.logsumexp(scores, dim=-1)
+    w = torch.exp(scores - lse.unsqueeze(-1))
+    w = torch.nan_to_num(w, nan=0.0)  # latents whose every key is masked: z = 0
+    z = w @ v
+    return z, lse
+
+
+def scatter_explicit(q, k, z, scale=1.0, key_mask=None, dtype=torch.float64):
+    """y = softmax_m(s k q^T) z; rows of masked tokens are 0."""
+    q, k, z = q.to(dtype), k.to(dtype), z.to(dtype)
+    if q.dim() == 3:
+        q = q.unsqueeze(0)
+    scores = scale * (k @ q.transpose(-2, -1))  # [B,H,N,M]
+    y = torch.softmax(scores, dim=-1) @ z
+    if key_mask is not None:
+        y = y * key_mask.to(dtype)[:, None, :, None]
+    return y
+
+
+def mixer_explicit(q, k, v, scale=1.0, key_mask=None, dtype=torch.float64):
+    z, _ = gather_explicit(q, k, v, scale, key_mask, dtype)
+    y = scatter_explicit(q, k, z, scale, key_mask, dtype)
+    return y, z
+
+
+def mixer_bruteforce_py(q, k, v, scale=1.0):
+    """Pure-Python-float loops; tiny shapes only.  q [H,M,D], k,v [B,H,N,D] as nested lists
+    or tensors.  Returns y as a nested list [B][H][N][D]."""
+    q = q.tolist() if hasattr(q, "tolist") else q
+    k = k.tolist() if hasattr(k, "tolist") else k
+    v = v.tolist() if hasattr(v, "tolist") else v
+    B, H, N, D, M = len(k), len(k[0]), len(k[0][0]), len(k[0][0][0]), len(q[0])
+    out = []
+    for b in range(B):
+        ob = []
+        for h in range(H):
+            s = [[scale * sum(q[h][m][d] * k[b][h][n][d] for d in range(D)) for n in range(N)]
+                 for m in range(M)]
+            z = []
+            for m in range(M):
+                mx = max(s[m])
+                e = [math.exp(x - mx) for x in s[m]]
+                tot = sum(e)
+                z.append([sum(e[n] * v[b][h][n][d] for n in range(N)) / tot for d in range(D)])
+            rows = []
+            for n in range(N):
+                col = [s[m][n] for m in range(M)]
+                mx = max(col)
+                e = [math.exp(x - mx) for x in col]
+                tot = sum(e)
+                rows.append([sum(e[m] * z[m][d] for m in range(M)) / tot for d in range(D)])
+            ob.append(rows)
+        out.append(ob)
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# causal FLARE
+# --------------------------------------------------------------------------------------
+def causal_fresh_state(B, H, M, D, dtype=torch.float64):
+    mu = torch.full((B, H, M), NEG_INF, dtype=dtype)
+    den = torch.zeros((B, H, M), dtype=dtype)
+    num = torch.zeros((B, H, M, D), dtype=dtype)
+    return mu, den, num
+
+
+def causal_recurrent(q, k, v, scale=1.0, state=None, dtype=torch.float64):
+    """Token-by-token recurrence.  Returns (y [B,H,N,D], (mu, den, num))."""
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    B, H, N, D = k.shape
+    M = q.shape[-2]
+    if state is None:
+        mu, den, num = causal_fresh_state(B, H, M, D, dtype)
+    else:
+        mu, den, num = (s.to(dtype).clone() for s in state)
+        mu = torch.where(mu <= -1e30, torch.full_like(mu, NEG_INF), mu)
+    y = torch.empty(B, H, N, D, dtype=dtype)
+    for t in range(N):
+        sigma = scale * torch.einsum("hmd,bhd->bhm", q, k[:, :, t])
+        mu_new = torch.maximum(mu, sigma)
+        a = torch.exp(mu - mu_new)
+        a = torch.nan_to_num(a, nan=0.0)  # (-inf) - (-inf) on the first token
+        p = torch.exp(sigma - mu_new)
+        den = a * den + p
+        num = a.unsqueeze(-1) * num + p.unsqueeze(-1) * v[:, :, t].unsqueeze(-2)
+        mu = mu_new
+        w = torch.softmax(sigma, dim=-1)
+        y[:, :, t] = torch.einsum("bhm,bhmd->bhd", w, num / den.unsqueeze(-1))
+    return y, (mu, den, num)
+
+
+def causal_bruteforce(q, k, v, scale=1.0, dtype=torch.float64):
+    """Row t of the non-causal mixer applied to the prefix [0..t]; O(N^2 M)."""
+    B, H, N, D = k.shape
+    y = torch.empty(B, H, N, D, dtype=dtype)
+    for t in range(N):
+        yt, _ = mixer_explicit(q, k[:, :, : t + 1], v[:, :, : t + 1], scale, dtype=dtype)
+        y[:, :, t] = yt[:, :, t]
+    return y
+
+
+def causal_state_invariants(mu, den, num):
+    """The shift-invariant content of a state: z = num/den and lse = mu + log den."""
+    return num / den.unsqueeze(-1), mu + torch.log(den)
+
+
+# --------------------------------------------------------------------------------------
+# triple attention
+# --------------------------------------------------------------------------------------
+def elu_plus_one(x):
+    return F.elu(x) + 1.0
+
+
+def triple_einsum(q1, q2, k1, k2, v, feature_map=False, normalize=False, dtype=torch.float32):
+    """state = einsum(k1, v, k2)/N, out = einsum(q1, state, q2) (backends.py:1288-1291).
+
+    The reference divides each of k1, k2, v by N**(1/3) in fp32; the product of the three
+    factors is the 1/N used here (triple.py:368 applies 1/N in one piece as well)."""
+    out_dtype = q1.dtype
+    q1, q2, k1, k2, v = (t.to(dtype) for t in (q1, q2, k1, k2, v))
+    if feature_map:
+        q1, q2, k1, k2 = (elu_plus_one(t) for t in (q1, q2, k1, k2))
+    N = q1.shape[-2]
+    state = torch.einsum("bhni,bhnj,bhnk->bhijk", k1, v, k2) / N
+    out = torch.einsum("bhni,bhijk,bhnk->bhnj", q1, state, q2)
+    if normalize:
+        kk = torch.einsum("bhni,bhnk->bhik", k1, k2) / N
+        den = torch.einsum("bhni,bhik,bhnk->bhn", q1, kk, q2)
+        out = out / den.unsqueeze(-1)
+    return state, out.to(out_dtype) if dtype == torch.float32 else out
+
+
+def triple_reference_scaling(q1, q2, k1, k2, v):
+    """Literal restatement of backends.py:1288-1291 including the three N**(1/3) divisions
+    (used to show that the single 1/N of triple_einsum is the same thing)."""
+    N = q1.size(-2)
+    k1, k2, v = [t.to(torch.float32) / (N ** (1 / 3)) for t in (k1, k2, v)]
+    state = torch.einsum("bhni,bhnj,bhnk->bhijk", k1, v, k2)
+    out = torch.einsum("bhni,bhijk,bhnk->bhnj", q1.to(torch.float32), state, q2.to(torch.float32))
+    return state, out.to(q1.dtype)
+
+
+# --------------------------------------------------------------------------------------
+# helpers shared by tests and bench
+# --------------------------------------------------------------------------------------
+def rel_l2(a, b):
+    a = a.detach().to(torch.float64).cpu()
+    b = b.detach().to(torch.float64).cpu()
+    return float((a - b).norm() / b.norm().clamp_min(1e-300))

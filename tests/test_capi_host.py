@@ -1,0 +1,122 @@
+"""Host-side checks of the C-ABI that need no GPU: the library loads, exports every symbol
+include/flare_hip.h declares, and rejects bad requests before anything is launched."""
+import ctypes as C
+import os
+import re
+
+import pytest
+import torch
+
+import flare_py_amd as F
+from flare_py_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _mixer_desc(B=1, H=2, N=128, M=64, D=32, dtype=_lib.DT_BF16, scale=1.0):
+    d = _lib.FlareMixerDesc()
+    d.B, d.H, d.N, d.M, d.D, d.dtype, d.scale = B, H, N, M, D, dtype, scale
+    d.q_stride = _lib.I3(0, M * D, D)
+    d.k_stride = d.v_stride = d.y_stride = _lib.I3(H * N * D, N * D, D)
+    return d
+
+
+def test_header_symbols_all_exported():
+    text = open(os.path.join(ROOT, "include", "flare_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    declared = set(re.findall(r"\b(flare_[a-z_]+)\s*\(", text))
+    assert declared, "no declarations parsed"
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in flare_hip.h but not exported"
+    assert declared == set(_lib.SYMBOLS), "ctypes binding and header disagree"
+    assert lib.flare_abi_version() == 1
+
+
+def test_struct_sizes_match_header_layout():
+    assert C.sizeof(_lib.FlareMixerDesc) == 10 * 4 + 4 * 24
+    assert C.sizeof(_lib.FlareCausalDesc) == 10 * 4 + 4 * 24
+    assert C.sizeof(_lib.FlareTripleDesc) == 10 * 4 + 6 * 24
+
+
+def test_workspace_query_and_kernel_choice():
+    lib = _lib.load()
+    n = C.c_size_t(0)
+    d = _mixer_desc()
+    assert lib.flare_mixer_workspace_bytes(C.byref(d), C.byref(n)) == 0 and n.value > 0
+    assert lib.flare_mixer_kernel_name(C.byref(d)) == b"mfma_bf16"
+    d.flags = _lib.FLAG_FORCE_GENERIC
+    assert lib.flare_mixer_kernel_name(C.byref(d)) == b"generic"
+    assert lib.flare_mixer_kernel_name(C.byref(_mixer_desc(dtype=_lib.DT_F32))) == b"generic"
+    assert lib.flare_mixer_kernel_name(C.byref(_mixer_desc(M=16, D=8))) == b"generic"
+    assert lib.flare_mixer_kernel_name(C.byref(_mixer_desc(dtype=_lib.DT_F16))) == b"mfma_f16"
+
+
+@pytest.mark.parametrize("field,value,code", [
+    ("N", 0, _lib.FLARE_EINVAL), ("M", -1, _lib.FLARE_EINVAL), ("D", 256, _lib.FLARE_EUNSUPPORTED),
+    ("dtype", 7, _lib.FLARE_EINVAL), ("scale", 0.0, _lib.FLARE_EINVAL), ("n_splits", -2, _lib.FLARE_EINVAL),
+])
+def test_bad_descriptor_rejected(field, value, code):
+    lib = _lib.load()
+    d = _mixer_desc()
+    setattr(d, field, value)
+    n = C.c_size_t(0)
+    assert lib.flare_mixer_workspace_bytes(C.byref(d), C.byref(n)) == code
+    assert _lib.last_error() != ""
+
+
+def test_null_pointers_and_workspace_rejected_before_launch():
+    lib = _lib.load()
+    d = _mixer_desc()
+    one = C.c_void_p(16)  # never dereferenced: validation fails first
+    assert lib.flare_mixer_fwd(C.byref(d), None, one, one, None, one, None, one, 1 << 30, None) == _lib.FLARE_EINVAL
+    assert lib.flare_mixer_fwd(C.byref(d), one, one, one, None, one, None, None, 0, None) == _lib.FLARE_EWORKSPACE
+    assert lib.flare_mixer_fwd(C.byref(d), one, one, one, None, one, None, one, 8, None) == _lib.FLARE_EWORKSPACE
+    assert "needed" in _lib.last_error()
+    assert lib.flare_gather_fwd(C.byref(d), one, one, one, None, None, None, one, 1 << 30, None) == _lib.FLARE_EINVAL
+    assert lib.flare_scatter_fwd(C.byref(d), one, one, None, None, one, None) == _lib.FLARE_EINVAL
+    d.k_stride = _lib.I3(0, 0, 3)  # row stride < D
+    assert lib.flare_scatter_fwd(C.byref(d), one, one, one, None, one, None) == _lib.FLARE_EINVAL
+    assert lib.flare_mixer_workspace_bytes(None, C.byref(C.c_size_t(0))) == _lib.FLARE_EINVAL
+
+
+def test_causal_and_triple_validation():
+    lib = _lib.load()
+    one = C.c_void_p(16)
+    c = _lib.FlareCausalDesc()
+    c.B, c.H, c.N, c.M, c.D, c.dtype, c.scale = 1, 1, 8, 16, 16, 0, 1.0
+    c.q_stride = _lib.I3(0, 256, 16)
+    c.k_stride = c.v_stride = c.y_stride = _lib.I3(128, 128, 16)
+    assert lib.flare_causal_prefill_fwd(C.byref(c), one, one, one, one, None, one, one, None, 0, None) == _lib.FLARE_EINVAL
+    c.M, c.D = 4096, 128
+    n = C.c_size_t(0)
+    assert lib.flare_causal_workspace_bytes(C.byref(c), C.byref(n)) == _lib.FLARE_EUNSUPPORTED
+    t = _lib.FlareTripleDesc()
+    t.B, t.H, t.N, t.Dq, t.Dv, t.dtype = 1, 1, 64, 16, 16, 1
+    assert lib.flare_triple_workspace_bytes(C.byref(t), C.byref(n)) == 0 and n.value > 0
+    assert lib.flare_triple_fwd(C.byref(t), one, one, one, one, one, one, one, one, 4, None) == _lib.FLARE_EWORKSPACE
+    t.Dq = 128
+    assert lib.flare_triple_workspace_bytes(C.byref(t), C.byref(n)) == _lib.FLARE_EUNSUPPORTED
+    t.Dq, t.feature_map = 16, 5
+    assert lib.flare_triple_workspace_bytes(C.byref(t), C.byref(n)) == _lib.FLARE_EINVAL
+
+
+def test_python_api_fails_loudly_on_cpu_tensors():
+    q = torch.randn(2, 4, 8)
+    k = torch.randn(1, 2, 16, 8)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        F.flare_multihead_mixer(q, k, k)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        F.triple_attention(k, k, k, k, k)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        F.flare_causal_prefill(q, k, k)
+
+
+def test_status_to_exception_mapping():
+    _lib.load().flare_mixer_workspace_bytes(None, None)
+    with pytest.raises(ValueError):
+        _lib.check(_lib.FLARE_EINVAL, "x")
+    with pytest.raises(NotImplementedError):
+        _lib.check(_lib.FLARE_EUNSUPPORTED, "x")
+    with pytest.raises(RuntimeError):
+        _lib.check(_lib.FLARE_EHIP, "x")

@@ -1,0 +1,223 @@
+"""Pins the CPU oracle (oracle/flare_oracle.py and oracle/flare_oracle.c) WITHOUT the product.
+
+The reference's tests hold no golden values for this path, so the oracle is pinned by
+independent restatements against each other (torch SDPA kernel / explicit softmax / plain C /
+pure-Python floats) and by what the mathematics fixes (closed forms and invariants chosen so
+that a dropped scale, a softmax over the wrong axis, a transposed operand or a wrong index
+fails at least one of them).
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import flare_oracle as O
+
+
+def _rand(B=2, H=3, N=37, M=5, D=4, seed=0, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(H, M, D, generator=g, dtype=dtype) * D ** -0.5
+    k = torch.randn(B, H, N, D, generator=g, dtype=dtype)
+    v = torch.randn(B, H, N, D, generator=g, dtype=dtype)
+    return q, k, v
+
+
+# ---------------------------------------------------------------- mixer
+@pytest.mark.parametrize("scale", [1.0, 0.37])
+def test_mixer_sdpa_vs_explicit_vs_c(scale):
+    q, k, v = _rand(dtype=torch.float32)
+    y1, z1 = O.mixer_sdpa(q, k, v, scale)
+    y2, z2 = O.mixer_explicit(q, k, v, scale)
+    y3, z3 = c_oracle.mixer(q, k, v, scale)
+    assert O.rel_l2(y1, y2) < 2e-6 and O.rel_l2(z1, z2) < 2e-6
+    assert O.rel_l2(y3, y2) < 2e-7 and O.rel_l2(z3, z2) < 2e-7
+
+
+def test_mixer_bruteforce_python_floats():
+    q, k, v = _rand(B=1, H=2, N=6, M=3, D=2)
+    y, _ = O.mixer_explicit(q, k, v, 0.8)
+    yb = torch.tensor(O.mixer_bruteforce_py(q, k, v, 0.8), dtype=torch.float64)
+    assert O.rel_l2(y, yb) < 1e-13
+
+
+def test_mixer_cfg1_shape_sdpa_vs_explicit():
+    # BASELINE config 1: q[8,64,16]~N(0,1/D), k,v[1,8,4096,16]~N(0,1), scale 1, fp32
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(8, 64, 16, generator=g) * 16 ** -0.5
+    k = torch.randn(1, 8, 4096, 16, generator=g)
+    v = torch.randn(1, 8, 4096, 16, generator=g)
+    y1, _ = O.mixer_sdpa(q, k, v, 1.0)
+    y2, _ = O.mixer_explicit(q, k, v, 1.0)
+    assert O.rel_l2(y1, y2) < 1e-5
+
+
+def test_mixer_zero_q_gives_mean():
+    q, k, v = _rand()
+    y, z = O.mixer_explicit(torch.zeros_like(q), k, v)
+    mean = v.mean(dim=2, keepdim=True)
+    assert torch.allclose(z, mean.expand_as(z), atol=1e-12)
+    assert torch.allclose(y, mean.expand_as(y), atol=1e-12)
+
+
+def test_mixer_single_token_and_single_latent():
+    q, k, v = _rand(N=1)
+    y, _ = O.mixer_explicit(q, k, v)
+    assert torch.allclose(y, v, atol=1e-12)          # N=1: every softmax weight is 1
+    q, k, v = _rand(M=1)
+    y, z = O.mixer_explicit(q, k, v)
+    assert torch.allclose(y, z.expand_as(y), atol=1e-12)  # M=1: every token receives z_0
+
+
+def test_mixer_convex_hull_and_constant_v():
+    q, k, v = _rand()
+    y, z = O.mixer_explicit(q, k, v, 2.0)
+    lo, hi = v.amin(dim=2, keepdim=True), v.amax(dim=2, keepdim=True)
+    assert (y >= lo - 1e-12).all() and (y <= hi + 1e-12).all()
+    c = torch.full_like(v, 3.25)
+    y, _ = O.mixer_explicit(q, k, c, 2.0)
+    assert torch.allclose(y, c, atol=1e-12)
+
+
+def test_mixer_permutation_equivariance_and_axis():
+    q, k, v = _rand()
+    perm = torch.randperm(k.shape[2], generator=torch.Generator().manual_seed(1))
+    y, z = O.mixer_explicit(q, k, v)
+    yp, zp = O.mixer_explicit(q, k[:, :, perm], v[:, :, perm])
+    assert torch.allclose(zp, z, atol=1e-12)               # gather is permutation invariant
+    assert torch.allclose(yp, y[:, :, perm], atol=1e-12)   # scatter is equivariant
+    # a softmax over the wrong axis would break this: duplicating every token leaves z, y unchanged
+    y2, z2 = O.mixer_explicit(q, torch.cat([k, k], 2), torch.cat([v, v], 2))
+    assert torch.allclose(z2, z, atol=1e-12) and torch.allclose(y2[:, :, : k.shape[2]], y, atol=1e-12)
+
+
+def test_mixer_scale_is_applied_to_both_softmaxes():
+    q, k, v = _rand()
+    y1, z1 = O.mixer_explicit(q, k, v, 0.5)
+    y2, z2 = O.mixer_explicit(0.5 * q, k, v, 1.0)
+    assert torch.allclose(y1, y2, atol=1e-12) and torch.allclose(z1, z2, atol=1e-12)
+
+
+def test_mixer_two_token_closed_form():
+    # H=B=M=D=1, N=2: z = sigmoid(q(k0-k1)) v0 + (1-sigmoid) v1 ; y_n = z
+    q = torch.tensor([[[0.7]]], dtype=torch.float64)
+    k = torch.tensor([[[[1.0], [-2.0]]]], dtype=torch.float64)
+    v = torch.tensor([[[[3.0], [5.0]]]], dtype=torch.float64)
+    y, z = O.mixer_explicit(q, k, v)
+    w0 = 1.0 / (1.0 + math.exp(-0.7 * 3.0))
+    assert abs(float(z) - (w0 * 3.0 + (1 - w0) * 5.0)) < 1e-12
+    assert torch.allclose(y, z.expand_as(y))
+
+
+def test_masked_mixer_equals_dropping_tokens():
+    q, k, v = _rand(B=2, N=11)
+    mask = torch.ones(2, 11, dtype=torch.bool)
+    mask[0, 7:] = False
+    mask[1, 3:] = False
+    y, z = O.mixer_explicit(q, k, v, key_mask=mask)
+    yc, zc = c_oracle.mixer(q, k, v, key_mask=mask)
+    assert O.rel_l2(yc, y) < 1e-6 and O.rel_l2(zc, z) < 1e-6
+    for b, n in ((0, 7), (1, 3)):
+        yb, zb = O.mixer_explicit(q, k[b : b + 1, :, :n], v[b : b + 1, :, :n])
+        assert torch.allclose(z[b], zb[0], atol=1e-12)
+        assert torch.allclose(y[b, :, :n], yb[0], atol=1e-12)
+        assert (y[b, :, n:] == 0).all()
+
+
+def test_gather_lse():
+    q, k, v = _rand()
+    _, lse = O.gather_explicit(q, k, v, 1.3)
+    s = 1.3 * torch.einsum("hmd,bhnd->bhmn", q, k)
+    assert torch.allclose(lse, torch.log(torch.exp(s).sum(-1)), atol=1e-12)
+
+
+# ---------------------------------------------------------------- causal
+def test_causal_recurrent_vs_bruteforce_vs_c():
+    q, k, v = _rand(B=1, H=2, N=19, M=4, D=3)
+    y, st = O.causal_recurrent(q, k, v, 0.9)
+    yb = O.causal_bruteforce(q, k, v, 0.9)
+    yc, stc = c_oracle.causal(q, k, v, 0.9)
+    assert O.rel_l2(y, yb) < 1e-12
+    assert O.rel_l2(yc, yb) < 1e-6
+    z, lse = O.causal_state_invariants(*st)
+    zc, lsec = O.causal_state_invariants(*stc)
+    assert O.rel_l2(zc, z) < 1e-6 and O.rel_l2(lsec, lse) < 1e-6
+
+
+def test_causal_last_row_is_noncausal_and_state_is_gather():
+    q, k, v = _rand(B=1, H=2, N=23, M=4, D=3)
+    y, st = O.causal_recurrent(q, k, v)
+    yn, zn = O.mixer_explicit(q, k, v)
+    assert torch.allclose(y[:, :, -1], yn[:, :, -1], atol=1e-12)
+    z, lse = O.causal_state_invariants(*st)
+    _, lse_n = O.gather_explicit(q, k, v)
+    assert torch.allclose(z, zn, atol=1e-12) and torch.allclose(lse, lse_n, atol=1e-12)
+
+
+def test_causal_continuation_and_first_token():
+    q, k, v = _rand(B=2, H=2, N=17, M=3, D=2)
+    y, st = O.causal_recurrent(q, k, v)
+    y1, s1 = O.causal_recurrent(q, k[:, :, :9], v[:, :, :9])
+    y2, s2 = O.causal_recurrent(q, k[:, :, 9:], v[:, :, 9:], state=s1)
+    assert torch.allclose(torch.cat([y1, y2], 2), y, atol=1e-12)
+    assert torch.allclose(y[:, :, 0], v[:, :, 0], atol=1e-12)   # first token sees only itself
+
+
+# ---------------------------------------------------------------- triple
+def _rand5(B=2, H=2, N=13, Dq=3, Dv=4, seed=0, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda d: torch.randn(B, H, N, d, generator=g, dtype=dtype)
+    return mk(Dq), mk(Dq), mk(Dq), mk(Dq), mk(Dv)
+
+
+def test_triple_python_loops_and_c():
+    q1, q2, k1, k2, v = _rand5(B=1, H=1, N=5, Dq=2, Dv=3)
+    st, out = O.triple_einsum(q1, q2, k1, k2, v, dtype=torch.float64)
+    N = 5
+    for i in range(2):
+        for j in range(3):
+            for kk in range(2):
+                ref = sum(float(k1[0, 0, n, i] * v[0, 0, n, j] * k2[0, 0, n, kk]) for n in range(N)) / N
+                assert abs(float(st[0, 0, i, j, kk]) - ref) < 1e-12
+    for n in range(N):
+        for j in range(3):
+            ref = sum(float(q1[0, 0, n, i] * st[0, 0, i, j, kk] * q2[0, 0, n, kk]) for i in range(2) for kk in range(2))
+            assert abs(float(out[0, 0, n, j]) - ref) < 1e-12
+    stc, outc = c_oracle.triple(q1, q2, k1, k2, v)
+    assert O.rel_l2(stc, st) < 1e-6 and O.rel_l2(outc, out) < 1e-6
+
+
+def test_triple_matches_reference_scaling_and_feature_map():
+    q1, q2, k1, k2, v = _rand5(dtype=torch.float32)
+    st, out = O.triple_einsum(q1, q2, k1, k2, v)
+    st2, out2 = O.triple_reference_scaling(q1, q2, k1, k2, v)   # three N^(1/3) divisions
+    assert O.rel_l2(st, st2) < 1e-6 and O.rel_l2(out, out2) < 1e-6
+    stf, outf = O.triple_einsum(q1, q2, k1, k2, v, feature_map=True)
+    f = O.elu_plus_one
+    stg, outg = O.triple_einsum(f(q1), f(q2), f(k1), f(k2), v)
+    assert O.rel_l2(stf, stg) < 1e-7 and O.rel_l2(outf, outg) < 1e-7
+    stc, outc = c_oracle.triple(q1, q2, k1, k2, v, feature_map=True, normalize=True)
+    stn, outn = O.triple_einsum(q1, q2, k1, k2, v, feature_map=True, normalize=True)
+    assert O.rel_l2(stc, stn) < 1e-5 and O.rel_l2(outc, outn) < 1e-4
+    x = torch.tensor([-2.0, -0.5, 0.0, 0.5, 3.0])
+    assert torch.allclose(f(x), torch.where(x > 0, x + 1, torch.exp(x)))
+
+
+def test_triple_invariants():
+    q1, q2, k1, k2, v = _rand5()
+    st, out = O.triple_einsum(q1, q2, k1, k2, v, dtype=torch.float64)
+    # swapping (k1,q1) <-> (k2,q2) transposes the state in (i,k) and keeps the output
+    st2, out2 = O.triple_einsum(q2, q1, k2, k1, v, dtype=torch.float64)
+    assert torch.allclose(st2, st.transpose(2, 4), atol=1e-12) and torch.allclose(out2, out, atol=1e-12)
+    # linear in v
+    _, o3 = O.triple_einsum(q1, q2, k1, k2, 2.5 * v, dtype=torch.float64)
+    assert torch.allclose(o3, 2.5 * out, atol=1e-12)
+    # normalised, positive features, constant v  =>  constant output
+    c = torch.full_like(v, 1.75)
+    _, on = O.triple_einsum(q1, q2, k1, k2, c, feature_map=True, normalize=True, dtype=torch.float64)
+    assert torch.allclose(on, c, atol=1e-12)
+    # N = 1: state is the outer product, out = <q1,k1><q2,k2> v
+    a = _rand5(N=1)
+    st1, o1 = O.triple_einsum(*a, dtype=torch.float64)
+    ref = (a[0] * a[2]).sum(-1, keepdim=True) * (a[1] * a[3]).sum(-1, keepdim=True) * a[4]
+    assert torch.allclose(o1, ref, atol=1e-12)
