@@ -75,7 +75,8 @@ MixerPlan plan_mixer(const FlareMixerDesc* d, bool want_mfma)
                             : (d->M + 63) / 64;
     int s = d->n_splits;
     if (s <= 0) {
-        const int64_t target = 1024;  // ~4 workgroups per CU on 256 CUs
+        // one full round of resident workgroups (MFMA kernels) or ~4 per CU (generic)
+        const int64_t target = p.mfma ? flare::mfma_gather_resident_slots(d->dtype, d->M, d->D) : 1024;
         int64_t per = (int64_t)d->B * d->H * mblk;
         s = (int)((target + per - 1) / per);
         if (s < 1) s = 1;

@@ -78,6 +78,7 @@ int        gather_generic_parts_per_wg();
 
 bool       mfma_mixer_supported(int dtype, int M, int D);
 int        mfma_gather_tokens_per_iter();
+int        mfma_gather_resident_slots(int dtype, int M, int D);
 hipError_t launch_gather_mfma(const MixerArgs& a, int dtype, hipStream_t st);
 hipError_t launch_scatter_mfma(const MixerArgs& a, int dtype, hipStream_t st);
 

@@ -154,10 +154,12 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
         }
 
     float shift[CT], lsum[CT];
+    f32x4 negc[CT];   // -shift, broadcast: the accumulator input of the score product
     f32x4 zacc[RT][CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         shift[ct] = kNegBig;
+        negc[ct] = f32x4{-kNegBig, -kNegBig, -kNegBig, -kNegBig};
         lsum[ct] = 0.f;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -230,8 +232,7 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
             if (!exact_tile) {
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
-                    const float nc = -shift[ct];
-                    f32x4 s0 = {nc, nc, nc, nc}, s1 = {nc, nc, nc, nc};
+                    f32x4 s0 = negc[ct], s1 = negc[ct];
 #pragma unroll
                     for (int kd = 0; kd < KD; ++kd) {
                         s0 = M_::mma(ka[2 * ks][kd], qb[ct][kd], s0);
@@ -249,8 +250,11 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                     bad = bad || !(t < kLazyLimit);
                 }
             }
-            if (__any(bad)) {
-                // exact path: true tile maximum, rescale of the running partial, validity
+            if (__builtin_expect(__any(bad), 0)) {
+                // exact path: true tile maximum, rescale of the running partial, validity.
+                // The empty asm keeps the compiler from speculating this block into the
+                // steady-state loop.
+                asm volatile("; exact path" ::: "memory");
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
                     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -276,6 +280,7 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                     for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] *= al;
                     lsum[ct] *= al;
                     shift[ct] = nc;
+                    negc[ct] = f32x4{-nc, -nc, -nc, -nc};
                     float p[8];
 #pragma unroll
                     for (int e = 0; e < 8; ++e) p[e] = ok[e] ? fast_exp2(sc[e] - nc) : 0.f;
@@ -400,11 +405,12 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
         const int tnext = t0 + 4 * kSTokWave;
         if (tnext < wg_n1) load_k(tnext, kn);
 
-        f32x4 yacc[kSTW][RT];
+        f32x4 yacc[kSTW][RT], negc[kSTW];
         float shift[kSTW], lsum[kSTW];
 #pragma unroll
         for (int tw = 0; tw < kSTW; ++tw) {
             shift[tw] = kNegBig;
+            negc[tw] = f32x4{-kNegBig, -kNegBig, -kNegBig, -kNegBig};
             lsum[tw] = 0.f;
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -427,8 +433,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
             if (ks != 0) {
 #pragma unroll
                 for (int tw = 0; tw < kSTW; ++tw) {
-                    const float nc = -shift[tw];
-                    f32x4 s0 = {nc, nc, nc, nc}, s1 = {nc, nc, nc, nc};
+                    f32x4 s0 = negc[tw], s1 = negc[tw];
 #pragma unroll
                     for (int kd = 0; kd < KD; ++kd) {
                         s0 = M_::mma(q0[kd], kb[tw][kd], s0);
@@ -446,7 +451,8 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                     bad = bad || !(t < kLazyLimit);
                 }
             }
-            if (__any(bad)) {
+            if (__builtin_expect(__any(bad), 0)) {
+                asm volatile("; exact path" ::: "memory");
 #pragma unroll
                 for (int tw = 0; tw < kSTW; ++tw) {
                     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -464,6 +470,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                     for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] *= al;
                     lsum[tw] *= al;
                     shift[tw] = nc;
+                    negc[tw] = f32x4{-nc, -nc, -nc, -nc};
                     pk[tw][0] = M_::pack2(fast_exp2(s0[0] - nc), fast_exp2(s0[1] - nc));
                     pk[tw][1] = M_::pack2(fast_exp2(s0[2] - nc), fast_exp2(s0[3] - nc));
                     pk[tw][2] = M_::pack2(fast_exp2(s1[0] - nc), fast_exp2(s1[1] - nc));
@@ -520,6 +527,50 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
 
 constexpr size_t kScatterLdsMax = 150 * 1024;
 
+// Workgroups of `kern` the current device holds at once (CUs x occupancy).  Grids are sized
+// to a whole multiple of this so that no partially filled last round is left over.
+// Falls back to 2 per CU on 256 CUs when no device can be queried (host-only planning).
+int resident_slots(const void* kern, size_t dyn_lds)
+{
+    struct Entry { const void* k; size_t lds; int dev; int slots; };
+    static Entry cache[64];
+    static int ncache = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return 512; }
+    for (int i = 0; i < ncache; ++i)
+        if (cache[i].k == kern && cache[i].lds == dyn_lds && cache[i].dev == dev) return cache[i].slots;
+    int occ = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, 256, dyn_lds) != hipSuccess || occ < 1) {
+        (void)hipGetLastError();
+        return 512;
+    }
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
+        (void)hipGetLastError();
+        return 512;
+    }
+    const int slots = occ * cus;
+    if (ncache < 64) cache[ncache++] = Entry{kern, dyn_lds, dev, slots};
+    return slots;
+}
+
+template <typename T, int D>
+const void* gather_kernel_ptr(int M)
+{
+    if (M % 256 == 0) return reinterpret_cast<const void*>(gather_mfma_kernel<T, D, 4>);
+    if (M % 128 == 0) return reinterpret_cast<const void*>(gather_mfma_kernel<T, D, 2>);
+    return reinterpret_cast<const void*>(gather_mfma_kernel<T, D, 1>);
+}
+
+template <typename T>
+const void* gather_kernel_ptr_d(int M, int D)
+{
+    switch (D) {
+        case 16: return gather_kernel_ptr<T, 16>(M);
+        case 32: return gather_kernel_ptr<T, 32>(M);
+        default: return gather_kernel_ptr<T, 64>(M);
+    }
+}
+
 template <typename T, int D>
 hipError_t gather_launch_ct(const MixerArgs& a, hipStream_t st)
 {
@@ -550,12 +601,13 @@ hipError_t scatter_launch(const MixerArgs& a, hipStream_t st)
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    // tokens per workgroup: aim at ~4 workgroups per CU over the whole grid, multiple of 256
-    const int64_t total = (int64_t)a.B * a.H * a.N;
-    int64_t tpw = (total + 1023) / 1024;
+    // tokens per workgroup (multiple of 256): one full round of resident workgroups when the
+    // problem is large enough, so that every CU finishes at the same time
+    const int slots = resident_slots(reinterpret_cast<const void*>(kern), lds);
+    const int64_t per_bh = (slots + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H);   // workgroups per (b,h)
+    int64_t tpw = (a.N + per_bh - 1) / per_bh;
     tpw = ((tpw + 255) / 256) * 256;
-    if (tpw < 256) tpw = 256;
-    if (tpw > 16384) tpw = 16384;
+    if (tpw < 1024) tpw = 1024;
     dim3 grid((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, a, (int)tpw);
     return hipGetLastError();
@@ -584,6 +636,12 @@ bool mfma_mixer_supported(int dtype, int M, int D)
 }
 
 int mfma_gather_tokens_per_iter() { return kGTile; }
+
+int mfma_gather_resident_slots(int dtype, int M, int D)
+{
+    const void* k = dtype == 1 ? gather_kernel_ptr_d<bf16_t>(M, D) : gather_kernel_ptr_d<f16_t>(M, D);
+    return resident_slots(k, 0);
+}
 
 hipError_t launch_gather_mfma(const MixerArgs& a, int dtype, hipStream_t st)
 {

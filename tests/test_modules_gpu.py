@@ -1,0 +1,103 @@
+"""FLARE modules on the HIP path: the reference's four contract tests
+(tests/pdebench/test_pdebench_model_contracts.py:23-132) plus value parity against the same modules
+evaluated with the CPU oracle mixer."""
+import pytest
+import torch
+
+import flare_py_amd as F
+from flare_py_amd import FLAREBlock, FLAREModel, functional, lra_modules, modules
+from oracle import flare_oracle as O
+
+pytestmark = pytest.mark.gpu
+KW = dict(in_dim=4, out_dim=3, channel_dim=32, num_blocks=2, num_heads=4, num_latents=16)
+
+
+def oracle_forward(model, x, monkeypatch, key_mask_aware=False):
+    """Run `model` on the CPU with the mixer swapped for the oracle (same weights)."""
+    def mix(q, k, v, scale=1.0, key_mask=None, **kw):
+        y, _ = O.mixer_explicit(q, k, v, scale, key_mask, dtype=torch.float64)
+        return y.to(k.dtype)
+    import copy
+    cpu = copy.deepcopy(model).cpu()
+    monkeypatch.setattr(modules, "flare_multihead_mixer", mix)
+    monkeypatch.setattr(lra_modules, "flare_multihead_mixer", mix)
+    with torch.no_grad():
+        out = cpu(x.cpu()) if not key_mask_aware else None
+    return out, cpu
+
+
+@pytest.mark.parametrize("B,N", [(1, 16), (2, 32), (2, 64)])
+def test_model_contracts_on_hip(dev, B, N, monkeypatch):
+    torch.manual_seed(0)
+    m = FLAREModel(**KW).to(dev).eval()
+    x = torch.randn(B, N, 4, device=dev)
+    with torch.no_grad():
+        y1, y2 = m(x), m(x)
+    assert y1.shape == (B, N, 3) and torch.isfinite(y1).all()       # smoke + shape matrix
+    assert torch.allclose(y1, y2, atol=1e-6)                         # determinism in eval
+    m2 = FLAREModel(**KW).to(dev).eval()
+    m2.load_state_dict(m.state_dict(), strict=True)                  # state_dict round trip
+    with torch.no_grad():
+        assert torch.allclose(m2(x), y1, atol=1e-6)
+    yr, _ = oracle_forward(m, x, monkeypatch)
+    assert O.rel_l2(y1, yr) <= 1e-5
+
+
+def test_block_bf16_cfg2_geometry_reduced(dev, monkeypatch):
+    # BASELINE config 2 geometry (C=128, H=8, D=16, M=128, bf16) on a reduced cloud: B=2, N=4096
+    torch.manual_seed(0)
+    blk = FLAREBlock(channel_dim=128, num_heads=8, num_latents=128).to(dev).eval()
+    for p in blk.parameters():
+        if p.dim() == 2 and p.shape[0] == p.shape[1]:
+            torch.nn.init.xavier_uniform_(p)
+    x = torch.randn(2, 4096, 128, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y, scores = blk(x)
+    assert scores is None and y.shape == x.shape
+    # oracle: same block in fp32 on the CPU with the oracle mixer
+    (yr, _), _ = oracle_forward(blk, x, monkeypatch)
+    assert O.rel_l2(y, yr) <= 2e-2
+    k = blk.att.k_proj(blk.norm1(x)).bfloat16().view(2, 4096, 8, 16).permute(0, 2, 1, 3)
+    assert functional.mixer_kernel_name(blk.att.latent_q.view(8, 128, 16).bfloat16(), k) == "mfma_bf16"
+
+
+def test_scores_branch_equals_mixer_branch(dev):
+    torch.manual_seed(1)
+    m = FLAREModel(**KW).to(dev).eval()
+    x = torch.randn(2, 48, 4, device=dev)
+    with torch.no_grad():
+        y = m(x)
+        ys, scores = m(x, return_scores=True)
+    assert O.rel_l2(y, ys) <= 1e-5 and len(scores) == 2
+
+
+def test_lra_block_with_padding_mask(dev, monkeypatch):
+    torch.manual_seed(2)
+    blk = lra_modules.FLAREBlock(channel_dim=64, num_heads=4, num_latents=16, kv_proj_hidden_dim=64,
+                                 ffn_hidden_dim=64).to(dev).eval()
+    x = torch.randn(3, 40, 64, device=dev)
+    mask = torch.ones(3, 40, dtype=torch.bool, device=dev)
+    mask[0, 25:] = False
+    mask[2, 5:] = False
+    with torch.no_grad():
+        y = blk(x, attention_mask=mask)
+    _, cpu = oracle_forward(blk, x, monkeypatch, key_mask_aware=True)
+    with torch.no_grad():
+        yr = cpu(x.cpu(), attention_mask=mask.cpu())
+    assert O.rel_l2(y, yr) <= 1e-5
+    # padded tokens do not influence real ones
+    x2 = x.clone()
+    x2[0, 25:] = 7.0
+    with torch.no_grad():
+        y2 = blk(x2, attention_mask=mask)
+    assert torch.allclose(y2[0, :25], y[0, :25], atol=1e-5)
+
+
+def test_training_step_runs(dev):
+    torch.manual_seed(3)
+    m = FLAREModel(**KW).to(dev).train()
+    x = torch.randn(2, 32, 4, device=dev)
+    loss = m(x).square().mean()
+    loss.backward()
+    g = m.blocks[0].att.latent_q.grad
+    assert g is not None and torch.isfinite(g).all() and float(g.abs().sum()) > 0

@@ -1,0 +1,73 @@
+"""GPU parity of the triple (third-order) linear attention kernels vs the einsum oracle
+(lra/models/backends.py:1285-1292 of the reference).  Tolerance: relative L2 <= 1e-5 for fp32,
+<= 2e-2 for bf16/f16 (the reference's own check is allclose(rtol=atol=1e-3) on half inputs,
+lra/models/triton/triple.py:1130), against the oracle on the same rounded inputs."""
+import pytest
+import torch
+
+import flare_py_amd as F
+from oracle import c_oracle
+from oracle import flare_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+
+def make(B, H, N, Dq, Dv, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda d: (torch.randn(B, H, N, d, generator=g) * Dq ** -0.5).to(dtype)
+    return mk(Dq), mk(Dq), mk(Dq), mk(Dq), mk(Dv)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1, 1), (2, 2, 13, 3, 4), (1, 2, 500, 16, 16), (1, 2, 300, 32, 32),
+                                   (1, 1, 130, 64, 64), (2, 1, 1000, 16, 24), (1, 1, 77, 20, 5)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_reference_exact_mode(dev, shape, dtype):
+    a = make(*shape, dtype)
+    st, out = F.triple_attention(*[t.to(dev) for t in a])
+    sr, orf = O.triple_einsum(*[t.float() for t in a], dtype=torch.float64)
+    assert O.rel_l2(st, sr) <= max(TOL[dtype] * 0.1, 1e-5)   # state is fp32 accumulate of exact products
+    assert O.rel_l2(out, orf) <= TOL[dtype]
+    assert st.dtype == torch.float32 and out.dtype == dtype
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feature_map_and_normaliser(dev, dtype):
+    a = make(2, 2, 700, 16, 16, dtype, seed=1)
+    st, out = F.triple_attention(*[t.to(dev) for t in a], normalize=True, feature_map="elu")
+    sr, orf = O.triple_einsum(*[t.float() for t in a], feature_map=True, normalize=True, dtype=torch.float64)
+    assert O.rel_l2(st, sr) <= 1e-5 and O.rel_l2(out, orf) <= TOL[dtype]
+    sc, oc = c_oracle.triple(*[t.float() for t in a], feature_map=True, normalize=True)
+    assert O.rel_l2(out, oc) <= TOL[dtype]
+    # positive features, constant v, normalised  =>  constant output
+    c = torch.full_like(a[4], 0.75)
+    _, oc = F.triple_attention(*[t.to(dev) for t in a[:4]], c.to(dev), normalize=True, feature_map="elu")
+    assert torch.allclose(oc.float().cpu(), c.float(), atol=1e-2 if dtype != torch.float32 else 1e-5)
+
+
+def test_function_apply_signature_and_split_stability(dev):
+    a = [t.to(dev) for t in make(1, 2, 5000, 16, 16, torch.float32, seed=2)]
+    st, out = F.TripleAttentionFunction.apply(*a)
+    st2, out2 = F.TripleAttentionFunction.apply(*a)
+    assert torch.equal(st, st2) and torch.equal(out, out2)      # no atomics: bit-stable
+    for s in (1, 3, 16):
+        sts, outs = F.triple_attention(*a, n_splits=s)
+        assert O.rel_l2(sts, st) <= 2e-6 and O.rel_l2(outs, out) <= 2e-6
+
+
+def test_strided_heads_view(dev):
+    B, H, N, D = 2, 4, 300, 16
+    g = torch.Generator().manual_seed(3)
+    xs = [torch.randn(B, N, H * D, generator=g).to(dev) * 0.25 for _ in range(5)]
+    views = [x.view(B, N, H, D).permute(0, 2, 1, 3) for x in xs]
+    st, out = F.triple_attention(*views)
+    sr, orf = O.triple_einsum(*[t.cpu() for t in views], dtype=torch.float64)
+    assert O.rel_l2(st, sr) <= 1e-5 and O.rel_l2(out, orf) <= 1e-5
+
+
+def test_cfg5_shape(dev):
+    # BASELINE config 5: B=4,H=8,N=16384,D=16, bf16 in / fp32 state, elu+1 features, normalised
+    a = make(4, 8, 16384, 16, 16, torch.bfloat16)
+    st, out = F.triple_attention(*[t.to(dev) for t in a], normalize=True, feature_map="elu")
+    sr, orf = O.triple_einsum(*[t.float() for t in a], feature_map=True, normalize=True)
+    assert O.rel_l2(st, sr) <= 1e-4 and O.rel_l2(out, orf) <= 2e-2
