@@ -88,7 +88,8 @@ __global__ __launch_bounds__(kGatherThreads) void gather_generic_kernel(MixerArg
 }
 
 // Fixed-order merge of the split-N partials: bit-stable for a given n_parts.
-// One thread per (b,h,m,d).
+// One thread per (b,h,m,d); partials are visited in batches of 8 so that the loads of a batch
+// are all in flight before the first is consumed.
 __global__ __launch_bounds__(256) void gather_merge_kernel(MixerArgs a)
 {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -99,16 +100,44 @@ __global__ __launch_bounds__(256) void gather_merge_kernel(MixerArgs a)
     const int m = r % a.M;
     const int64_t bh = r / a.M;
     const int P = a.n_parts;
-    const int64_t base = bh * P * a.M + m;
+    const float* __restrict__ pm = a.part_m + bh * P * a.M + m;
+    const float* __restrict__ pl = a.part_l + bh * P * a.M + m;
+    const float* __restrict__ pa = a.part_acc + (bh * P * a.M + m) * a.D + d;
+    const int64_t sm = a.M, sa = (int64_t)a.M * a.D;
+    constexpr int U = 8;
 
     float mx = kNegBig;
-    for (int p = 0; p < P; ++p) mx = fmaxf(mx, a.part_m[base + (int64_t)p * a.M]);
+    int p = 0;
+    for (; p + U <= P; p += U) {
+        float t[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) t[u] = pm[(p + u) * sm];
+#pragma unroll
+        for (int u = 0; u < U; ++u) mx = fmaxf(mx, t[u]);
+    }
+    for (; p < P; ++p) mx = fmaxf(mx, pm[p * sm]);
+
     float l = 0.f, acc = 0.f;
-    for (int p = 0; p < P; ++p) {
-        const int64_t row = base + (int64_t)p * a.M;
-        const float w = fast_exp2(a.part_m[row] - mx);
-        l = fmaf(a.part_l[row], w, l);
-        acc = fmaf(a.part_acc[row * a.D + d], w, acc);
+    p = 0;
+    for (; p + U <= P; p += U) {
+        float tm[U], tl[U], ta[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            tm[u] = pm[(p + u) * sm];
+            tl[u] = pl[(p + u) * sm];
+            ta[u] = pa[(p + u) * sa];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const float w = fast_exp2(tm[u] - mx);
+            l = fmaf(tl[u], w, l);
+            acc = fmaf(ta[u], w, acc);
+        }
+    }
+    for (; p < P; ++p) {
+        const float w = fast_exp2(pm[p * sm] - mx);
+        l = fmaf(pl[p * sm], w, l);
+        acc = fmaf(pa[p * sa], w, acc);
     }
     a.z[idx] = l > 0.f ? acc / l : 0.f;
     if (a.lse && d == 0) a.lse[r] = l > 0.f ? (mx + __log2f(l)) * kLn2 : -INFINITY;

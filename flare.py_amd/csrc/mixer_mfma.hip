@@ -17,6 +17,8 @@
 //
 //   gather : z = softmax_n(s q k^T) v   split over N, partial (shift, sum, numerator)
 //   scatter: y = softmax_m(s k q^T) z   token parallel, Q and Z^T resident in LDS
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace flare {
@@ -31,6 +33,9 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr float kLazyLimit = 1024.f;  // 2^10: largest per-tile partial sum the lazy shift accepts
+// range of an unshifted softmax denominator that proves no exponential overflowed or lost
+// the terms that matter to underflow (2^-60 .. 2^120)
+constexpr float kLMin = 8.6736174e-19f, kLMax = 1.329228e36f;
 
 template <typename T> struct Mma;
 
@@ -45,11 +50,12 @@ template <> struct Mma<bf16_t> {
         bf16x2 v = {(__bf16)lo, (__bf16)hi};
         return __builtin_bit_cast(uint32_t, v);
     }
-    static __device__ __forceinline__ float sum2(uint32_t pk, float acc)
+    static constexpr uint32_t kOnes2 = 0x3f803f80u;   // two bf16 ones
+    static __device__ __forceinline__ float dot2(uint32_t x, uint32_t y, float acc)
     {
-        const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), ones, acc, false);
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, x), __builtin_bit_cast(bf16x2, y), acc, false);
     }
+    static __device__ __forceinline__ float sum2(uint32_t pk, float acc) { return dot2(pk, kOnes2, acc); }
 };
 
 template <> struct Mma<f16_t> {
@@ -63,11 +69,12 @@ template <> struct Mma<f16_t> {
         f16x2 v = {(_Float16)lo, (_Float16)hi};
         return __builtin_bit_cast(uint32_t, v);
     }
-    static __device__ __forceinline__ float sum2(uint32_t pk, float acc)
+    static constexpr uint32_t kOnes2 = 0x3c003c00u;   // two f16 ones
+    static __device__ __forceinline__ float dot2(uint32_t x, uint32_t y, float acc)
     {
-        const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, pk), ones, acc, false);
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, x), __builtin_bit_cast(f16x2, y), acc, false);
     }
+    static __device__ __forceinline__ float sum2(uint32_t pk, float acc) { return dot2(pk, kOnes2, acc); }
 };
 
 template <typename T> __device__ __forceinline__ uint16_t elem_bits(float v);
@@ -82,6 +89,26 @@ template <> __device__ __forceinline__ float bits_elem<bf16_t>(uint16_t b) { ret
 template <> __device__ __forceinline__ float bits_elem<f16_t>(uint16_t b) { return float(__builtin_bit_cast(_Float16, b)); }
 
 __device__ __forceinline__ u32x4 zero4() { return u32x4{0u, 0u, 0u, 0u}; }
+
+#ifndef FLARE_EXPERIMENT
+#define FLARE_EXPERIMENT 0
+#endif
+__device__ __forceinline__ float xexp2(float x)
+{
+#if FLARE_EXPERIMENT == 1 || FLARE_EXPERIMENT == 6
+    return x * 1.0001f;
+#else
+    return fast_exp2(x);
+#endif
+}
+template <typename M_> __device__ __forceinline__ uint32_t xpack2(float lo, float hi)
+{
+#if FLARE_EXPERIMENT == 3
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+#else
+    return M_::pack2(lo, hi);
+#endif
+}
 
 // 8 elements (16 bytes) from global memory
 __device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
@@ -112,13 +139,38 @@ __device__ __forceinline__ float xg_sum(float v)
     return v;
 }
 
+// Scheduling hint: N groups of (1 matrix instruction, 2-3 vector/transcendental instructions).
+template <int N> __device__ __forceinline__ void interleave_mfma_valu()
+{
+    if constexpr (N > 0) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x402, (N & 1) ? 3 : 2, 0);
+        interleave_mfma_valu<N - 1>();
+    }
+}
+
 // =====================================================================================
 // gather
 // =====================================================================================
-constexpr int kGTile = 64;            // tokens per barrier step (2 k-steps of 32)
-constexpr int kGVtStride = kGTile + 8;  // elements per V^T row in LDS (pad: conflict-free b128 reads)
+constexpr int kGTile = 64;            // tokens per barrier step (k-steps of 32)
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// LDS transpose read: the 16 lanes of a group each name 8 bytes (4 elements) of a row-major
+// tile; lane i of the group receives element i of the four rows named by lane quads 0..3.
+__device__ __forceinline__ uint2 lds_read_tr16(const void* lds_addr)
+{
+    typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
+    const s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)lds_addr);
+    return __builtin_bit_cast(uint2, r);
+}
 
 // One workgroup = 4 waves, 64*CT latents (wave w owns 16*CT of them), one token range.
+// K and V tiles of 64 tokens are staged row-major in LDS (double buffered, one barrier per
+// tile).  The score product reads K rows as its A operand; the value product needs V^T and
+// gets it from the LDS transpose read.  The optimistic pass uses no softmax shift (see the
+// scatter kernel); its denominators, produced by a row of ones in the value product, are
+// validated at the end and a workgroup that fails repeats its range with a running maximum.
 template <typename T, int D, int CT>
 __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
 {
@@ -126,9 +178,13 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
     constexpr int RT = D / 16;          // 16-row tiles of z^T
     constexpr int CH = D / 8;           // 16-byte chunks per row
     constexpr int MB = 64 * CT;
+    constexpr int ROWB = D * 2;         // bytes per token row
+    constexpr int TILEB = kGTile * ROWB;
     using M_ = Mma<T>;
 
-    __shared__ __attribute__((aligned(16))) uint16_t vt[2][D][kGVtStride];
+    __shared__ __attribute__((aligned(16))) uint8_t kt[2][TILEB];
+    __shared__ __attribute__((aligned(16))) uint8_t vt[2][TILEB];
+    __shared__ int wg_flag[4];
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
     const int mblocks = a.M / MB;
@@ -152,181 +208,217 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                                              a.scale_log2)
                                  : zero4();
         }
-
-    float shift[CT], lsum[CT];
-    f32x4 negc[CT];   // -shift, broadcast: the accumulator input of the score product
-    f32x4 zacc[RT][CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        shift[ct] = kNegBig;
-        negc[ct] = f32x4{-kNegBig, -kNegBig, -kNegBig, -kNegBig};
-        lsum[ct] = 0.f;
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
+    const u32x4 ones8 = {M_::kOnes2, M_::kOnes2, M_::kOnes2, M_::kOnes2};
 
     const int n_begin = split * a.tokens_per_split;
     const int n_end = min(a.N, n_begin + a.tokens_per_split);
 
-    // V staging: 16-byte chunk c of the tile = (token c / CH, chunk c % CH)
-    constexpr int VCH = kGTile * CH;              // chunks per tile
-    constexpr int VPT = (VCH + 255) / 256;        // chunks per thread
-    u32x4 ka[4][KD], kn[4][KD], vr[VPT];
+    // staging: 16-byte chunk c of a tile = (token c / CH, chunk c % CH); rows beyond n_end are
+    // clamped to the last valid row (their probabilities are forced to 0 below)
+    constexpr int TCH = kGTile * CH;
+    constexpr int CPT = (TCH + 255) / 256;
+    // K chunks are XOR-swizzled by (token / 4) so that the 16 rows an A-operand read touches
+    // fall into distinct banks; V rows swap their 32-byte halves on odd (token / 4) for the
+    // transpose read
+    auto k_slot = [](int tok, int ch) { return tok * ROWB + ((ch ^ ((tok >> 2) & (CH - 1))) << 4); };
+    auto v_slot = [](int tok, int ch) { return tok * ROWB + ((CH >= 4 ? (ch ^ (((tok >> 2) & 1) << 1)) : ch) << 4); };
 
-    auto load_k = [&](int n0, u32x4 (&dst)[4][KD]) {
+    // two register sets: tiles are fetched two iterations before they are consumed
+    u32x4 kr[2][CPT], vr[2][CPT];
+    auto load_tile = [&](auto set_tag, int n0) {
+        constexpr int S = decltype(set_tag)::value;
 #pragma unroll
-        for (int sub = 0; sub < 4; ++sub)
-#pragma unroll
-            for (int kd = 0; kd < KD; ++kd) {
-                const int n = n0 + sub * 16 + c16, ch = kd * 4 + g;
-                dst[sub][kd] = (n < n_end && ch < CH) ? load16(k + (int64_t)n * a.ks[2] + ch * 8) : zero4();
-            }
-    };
-    auto load_v = [&](int n0) {
-#pragma unroll
-        for (int i = 0; i < VPT; ++i) {
+        for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * 256;
-            const int j = c / CH, ch = c % CH;
-            vr[i] = (c < VCH && n0 + j < n_end) ? load16(v + (int64_t)(n0 + j) * a.vs[2] + ch * 8) : zero4();
+            if (c < TCH) {
+                const int n = min(n0 + c / CH, n_end - 1), ch = c % CH;
+                kr[S][i] = load16(k + (int64_t)n * a.ks[2] + ch * 8);
+                vr[S][i] = load16(v + (int64_t)n * a.vs[2] + ch * 8);
+            }
         }
     };
-    auto store_v = [&](int buf) {
+    auto store_tile = [&](auto set_tag) {   // register set S always feeds LDS buffer S
+        constexpr int S = decltype(set_tag)::value;
 #pragma unroll
-        for (int i = 0; i < VPT; ++i) {
+        for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * 256;
-            if (c < VCH) {
-                const int j = c / CH, ch = c % CH;
-                // token j = ks*32 + t*16 + 4*gg + e  ->  column ks*32 + gg*8 + t*4 + e
-                const int pos = (j & 32) | (((j >> 2) & 3) << 3) | (((j >> 4) & 1) << 2) | (j & 3);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    vt[buf][ch * 8 + 2 * e][pos] = uint16_t(vr[i][e] & 0xffffu);
-                    vt[buf][ch * 8 + 2 * e + 1][pos] = uint16_t(vr[i][e] >> 16);
-                }
+            if (c < TCH) {
+                const int tok = c / CH, ch = c % CH;
+                *reinterpret_cast<u32x4*>(&kt[S][k_slot(tok, ch)]) = kr[S][i];
+                *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = vr[S][i];
             }
         }
     };
+    using Set0 = std::integral_constant<int, 0>;
+    using Set1 = std::integral_constant<int, 1>;
 
-    if (n_begin < n_end) {
-        load_k(n_begin, ka);
-        load_v(n_begin);
-    }
+    float shift[CT];
+    f32x4 zacc[RT][CT], lacc[CT];
 
-    int it = 0;
-    for (int n0 = n_begin; n0 < n_end; n0 += kGTile, ++it) {
-        const int buf = it & 1;
-        store_v(buf);
-        if (n0 + kGTile < n_end) {
-            load_k(n0 + kGTile, kn);
-            load_v(n0 + kGTile);
+    // one pass over the token range; EXACT keeps a running maximum per latent
+    auto run = [&](auto exact_tag) {
+        constexpr bool EXACT = decltype(exact_tag)::value;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            shift[ct] = EXACT ? kNegBig : 0.f;
+            lacc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-        __syncthreads();
-
-        const bool exact_tile = (n0 + kGTile > n_end) || (mask != nullptr);
-
+        // tile i lives in LDS buffer i & 1; it is written there one iteration before its use from
+        // the register set of the same parity, which was loaded two iterations before
+        auto process = [&](int n0, int buf) {
+            const bool ragged = (n0 + kGTile > n_end) || (mask != nullptr);
+            auto tile = [&](auto ragged_tag) {
+                constexpr bool RAGGED = decltype(ragged_tag)::value;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            uint32_t pk[CT][4];
-            float tsum[CT];
-            bool bad = exact_tile;
-            if (!exact_tile) {
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct) {
-                    f32x4 s0 = negc[ct], s1 = negc[ct];
-#pragma unroll
+                for (int ks = 0; ks < kGTile / 32; ++ks) {
+                    // operands: two 16-token K sub-tiles (A of the score product), V^T (A of the value product)
+                    u32x4 ka0[KD], ka1[KD], va[RT];
+    #pragma unroll
                     for (int kd = 0; kd < KD; ++kd) {
-                        s0 = M_::mma(ka[2 * ks][kd], qb[ct][kd], s0);
-                        s1 = M_::mma(ka[2 * ks + 1][kd], qb[ct][kd], s1);
+                        const int ch = kd * 4 + g;
+                        const int t0 = ks * 32 + c16, t1 = t0 + 16;
+                        ka0[kd] = ch < CH ? *reinterpret_cast<const u32x4*>(&kt[buf][k_slot(t0, ch)]) : zero4();
+                        ka1[kd] = ch < CH ? *reinterpret_cast<const u32x4*>(&kt[buf][k_slot(t1, ch)]) : zero4();
                     }
-                    pk[ct][0] = M_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1]));
-                    pk[ct][1] = M_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3]));
-                    pk[ct][2] = M_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1]));
-                    pk[ct][3] = M_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]));
-                    float t = M_::sum2(pk[ct][0], 0.f);
-                    t = M_::sum2(pk[ct][1], t);
-                    t = M_::sum2(pk[ct][2], t);
-                    t = M_::sum2(pk[ct][3], t);
-                    tsum[ct] = t;
-                    bad = bad || !(t < kLazyLimit);
+    #pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) {
+                        // lane (c16, g): rows 4g + (c16 >> 2) of each sub-tile, 8 bytes at d = 16 rt + 4 (c16 & 3)
+                        const int r0 = ks * 32 + 4 * g + (c16 >> 2), r1 = r0 + 16;
+                        const int ch = 2 * rt + ((c16 & 3) >> 1), sub = (c16 & 1) << 3;
+                        const uint2 lo = lds_read_tr16(&vt[buf][v_slot(r0, ch) + sub]);
+                        const uint2 hi = lds_read_tr16(&vt[buf][v_slot(r1, ch) + sub]);
+                        va[rt] = u32x4{lo.x, lo.y, hi.x, hi.y};
+                    }
+    #pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) {
+                        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+    #pragma unroll
+                        for (int kd = 0; kd < KD; ++kd) {
+                            s0 = M_::mma(ka0[kd], qb[ct][kd], s0);
+                            s1 = M_::mma(ka1[kd], qb[ct][kd], s1);
+                        }
+                        float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+                        bool ok[8];
+                        if (EXACT || RAGGED) {
+    #pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                const int n = n0 + ks * 32 + (e >> 2) * 16 + 4 * g + (e & 3);
+                                ok[e] = !RAGGED || (n < n_end && (mask == nullptr || mask[n] != 0));
+                            }
+                        }
+                        if (EXACT) {
+                            float mx = kNegBig;
+    #pragma unroll
+                            for (int e = 0; e < 8; ++e)
+                                if (ok[e]) mx = fmaxf(mx, sc[e]);
+                            mx = xg_max(mx);
+                            const float nc = fmaxf(shift[ct], mx);
+                            const float al = fast_exp2(shift[ct] - nc);
+    #pragma unroll
+                            for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] *= al;
+                            lacc[ct] *= al;
+                            shift[ct] = nc;
+    #pragma unroll
+                            for (int e = 0; e < 8; ++e) sc[e] -= nc;
+                        }
+                        float p[8];
+    #pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            p[e] = xexp2(sc[e]);
+                            if (EXACT || RAGGED) p[e] = ok[e] ? p[e] : 0.f;
+                        }
+                        const u32x4 pb = {xpack2<M_>(p[0], p[1]), xpack2<M_>(p[2], p[3]),
+                                          xpack2<M_>(p[4], p[5]), xpack2<M_>(p[6], p[7])};
+    #pragma unroll
+                        for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = M_::mma(va[rt], pb, zacc[rt][ct]);
+                        lacc[ct] = M_::mma(ones8, pb, lacc[ct]);   // row of ones: the softmax denominator
+                    }
                 }
-            }
-            if (__builtin_expect(__any(bad), 0)) {
-                // exact path: true tile maximum, rescale of the running partial, validity.
-                // The empty asm keeps the compiler from speculating this block into the
-                // steady-state loop.
-                asm volatile("; exact path" ::: "memory");
+    };
+            if (ragged) tile(std::true_type{});
+            else        tile(std::false_type{});
+        };
+        auto iter = [&](int n0, auto par) {
+            constexpr int P = decltype(par)::value;
+            using Other = std::integral_constant<int, 1 - P>;
+#if FLARE_EXPERIMENT == 7
+            // loads only: fold the staged registers into an accumulator, no LDS, no barrier
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct) {
-                    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int kd = 0; kd < KD; ++kd) {
-                        s0 = M_::mma(ka[2 * ks][kd], qb[ct][kd], s0);
-                        s1 = M_::mma(ka[2 * ks + 1][kd], qb[ct][kd], s1);
-                    }
-                    float sc[8];
-                    bool ok[8];
-                    float mx = kNegBig;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int n = n0 + ks * 32 + (e >> 2) * 16 + 4 * g + (e & 3);
-                        ok[e] = n < n_end && (mask == nullptr || mask[n] != 0);
-                        sc[e] = e < 4 ? s0[e] : s1[e - 4];
-                        if (ok[e]) mx = fmaxf(mx, sc[e]);
-                    }
-                    mx = xg_max(mx);
-                    const float nc = fmaxf(shift[ct], mx);
-                    const float al = fast_exp2(shift[ct] - nc);
-#pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] *= al;
-                    lsum[ct] *= al;
-                    shift[ct] = nc;
-                    negc[ct] = f32x4{-nc, -nc, -nc, -nc};
-                    float p[8];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) p[e] = ok[e] ? fast_exp2(sc[e] - nc) : 0.f;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) pk[ct][e] = M_::pack2(p[2 * e], p[2 * e + 1]);
-                    float t = M_::sum2(pk[ct][0], 0.f);
-                    t = M_::sum2(pk[ct][1], t);
-                    t = M_::sum2(pk[ct][2], t);
-                    t = M_::sum2(pk[ct][3], t);
-                    tsum[ct] = t;
-                }
-            }
-            u32x4 va[RT];
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-                va[rt] = *reinterpret_cast<const u32x4*>(&vt[buf][rt * 16 + c16][ks * 32 + g * 8]);
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) {
-                const u32x4 pb = {pk[ct][0], pk[ct][1], pk[ct][2], pk[ct][3]};
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = M_::mma(va[rt], pb, zacc[rt][ct]);
-                lsum[ct] += tsum[ct];
-            }
+            for (int i = 0; i < CPT; ++i)
+                lacc[0] += __builtin_bit_cast(f32x4, kr[1 - P][i]) + __builtin_bit_cast(f32x4, vr[1 - P][i]);
+            if (n0 + 3 * kGTile < n_end) load_tile(Other{}, n0 + 3 * kGTile);
+#elif FLARE_EXPERIMENT == 8
+            // loads + LDS stores + barrier, no LDS reads / compute
+            __syncthreads();
+            if (n0 + kGTile < n_end) store_tile(Other{});
+            if (n0 + 3 * kGTile < n_end) load_tile(Other{}, n0 + 3 * kGTile);
+#else
+            __syncthreads();
+            if (n0 + kGTile < n_end) store_tile(Other{});
+            if (n0 + 3 * kGTile < n_end) load_tile(Other{}, n0 + 3 * kGTile);
+            process(n0, P);
+#endif
+        };
+        if (n_begin < n_end) {
+            load_tile(Set0{}, n_begin);
+            if (n_begin + kGTile < n_end) load_tile(Set1{}, n_begin + kGTile);
+            store_tile(Set0{});
+            if (n_begin + 2 * kGTile < n_end) load_tile(Set0{}, n_begin + 2 * kGTile);
         }
-
-        if (n0 + kGTile < n_end) {
-#pragma unroll
-            for (int sub = 0; sub < 4; ++sub)
-#pragma unroll
-                for (int kd = 0; kd < KD; ++kd) ka[sub][kd] = kn[sub][kd];
+        for (int n0 = n_begin; n0 < n_end; n0 += 2 * kGTile) {
+            iter(n0, Set0{});
+            if (n0 + kGTile < n_end) iter(n0 + kGTile, Set1{});
         }
-    }
+    };
 
-    // partial for this split: shift (log2 units), sum, numerator
+    run(std::false_type{});
+    // validate: every denominator of this wave inside the safe range, numerators finite
+    bool bad = false;
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
-        const float l = xg_sum(lsum[ct]);
+        const float l = lacc[ct][0];
+        bad = bad || !(l <= kLMax) || (n_begin < n_end && mask == nullptr && !(l >= kLMin));
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) bad = bad || !(fabsf(zacc[rt][ct][r]) <= 3.0e38f);
+    }
+#if FLARE_EXPERIMENT != 0
+    bad = false;
+#endif
+    if (mask != nullptr) {
+        // with a key mask an all-masked range legitimately gives l = 0; small l cannot be told
+        // apart from underflow cheaply, so masked problems always take the exact pass
+        bad = true;
+    }
+    const int anybad = __any(bad);
+    __syncthreads();
+    if (lane == 0) wg_flag[w] = anybad;
+    __syncthreads();
+    if (wg_flag[0] | wg_flag[1] | wg_flag[2] | wg_flag[3]) {
+        asm volatile("; exact pass" ::: "memory");
+        run(std::true_type{});
+    }
+
+    // partial for this split: shift (log2 units), sum, numerator, renormalised so that the
+    // sum has exponent 0 (keeps the merge free of overflow whatever the pass left behind)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const float l = lacc[ct][0];
+        int e = 0;
+        if (l > 0.f) (void)frexpf(l, &e);
+        const float sc = l > 0.f ? ldexpf(1.f, -e) : 0.f;
         const int m = m_base + ct * 16 + c16;
         const int64_t row = (((int64_t)b * a.H + h) * a.n_parts + split) * a.M + m;
         if (g == 0) {
-            a.part_m[row] = shift[ct];
-            a.part_l[row] = l;
+            a.part_m[row] = l > 0.f ? shift[ct] + (float)e : kNegBig;
+            a.part_l[row] = l * sc;
         }
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-            *reinterpret_cast<f32x4*>(a.part_acc + row * D + rt * 16 + 4 * g) = zacc[rt][ct];
+            *reinterpret_cast<f32x4*>(a.part_acc + row * D + rt * 16 + 4 * g) = zacc[rt][ct] * sc;
     }
 }
 
@@ -346,6 +438,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
     constexpr int CH = D / 8;
     using M_ = Mma<T>;
 
+    __shared__ float red[4];
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     // qa[mt][ch][c16]  : 16 bytes each, latent m = 16 mt + c16, d = 8 ch .. 8 ch + 7
     // zt[ks][rt][lane] : 16 bytes each, row d = (D/4) (c16/4) + 4 rt + c16 % 4,
@@ -398,6 +491,8 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
             }
     };
 
+    const u32x4 ones8 = {M_::kOnes2, M_::kOnes2, M_::kOnes2, M_::kOnes2};
+
     int t0 = wg_n0 + w * kSTokWave;
     if (t0 < wg_n1) load_k(t0, kb);
 
@@ -405,54 +500,100 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
         const int tnext = t0 + 4 * kSTokWave;
         if (tnext < wg_n1) load_k(tnext, kn);
 
-        f32x4 yacc[kSTW][RT], negc[kSTW];
-        float shift[kSTW], lsum[kSTW];
+        f32x4 yacc[kSTW][RT];
+        float lrow[kSTW];       // softmax denominators, complete for the lane's token
+        bool redo = false;
+        {
+            // Optimistic pass: no softmax shift at all.  fp32 and bf16 share an 8-bit exponent, so
+            // exp2(score) is exact enough whenever the scores of a token stay inside (-60, 120);
+            // that is validated afterwards on the denominators, and only a token tile that
+            // fails goes through the exact (running maximum) path below.
+            f32x4 yl[kSTW];
 #pragma unroll
-        for (int tw = 0; tw < kSTW; ++tw) {
-            shift[tw] = kNegBig;
-            negc[tw] = f32x4{-kNegBig, -kNegBig, -kNegBig, -kNegBig};
-            lsum[tw] = 0.f;
+            for (int tw = 0; tw < kSTW; ++tw) {
+                yl[tw] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-
-        for (int ks = 0; ks < KS; ++ks) {
-            u32x4 q0[KD], q1[KD], za[RT];
-#pragma unroll
-            for (int kd = 0; kd < KD; ++kd) {
-                const int ch = kd * 4 + g;
-                q0[kd] = ch < CH ? qa[((2 * ks) * CH + ch) * 16 + c16] : zero4();
-                q1[kd] = ch < CH ? qa[((2 * ks + 1) * CH + ch) * 16 + c16] : zero4();
+                for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
+            // operands of latent step ks live in registers one step ahead of their use
+            u32x4 q0[KD], q1[KD], za[RT];
+            auto load_ops = [&](int ks, u32x4 (&o0)[KD], u32x4 (&o1)[KD], u32x4 (&oz)[RT]) {
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) za[rt] = zt[(ks * RT + rt) * 64 + lane];
-
-            uint32_t pk[kSTW][4];
-            float tsum[kSTW];
-            bool bad = (ks == 0);
-            if (ks != 0) {
+                for (int kd = 0; kd < KD; ++kd) {
+                    const int ch = kd * 4 + g;
+                    o0[kd] = ch < CH ? qa[((2 * ks) * CH + ch) * 16 + c16] : zero4();
+                    o1[kd] = ch < CH ? qa[((2 * ks + 1) * CH + ch) * 16 + c16] : zero4();
+                }
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) oz[rt] = zt[(ks * RT + rt) * 64 + lane];
+            };
+            // one latent step (32 latents) for the wave's 4 column tiles
+            auto step = [&](const u32x4 (&o0)[KD], const u32x4 (&o1)[KD], const u32x4 (&oz)[RT]) {
 #pragma unroll
                 for (int tw = 0; tw < kSTW; ++tw) {
-                    f32x4 s0 = negc[tw], s1 = negc[tw];
+                    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#if FLARE_EXPERIMENT == 5 || FLARE_EXPERIMENT == 6
+                    s0 = __builtin_bit_cast(f32x4, o0[0]) + __builtin_bit_cast(f32x4, kb[tw][0]);
+                    s1 = __builtin_bit_cast(f32x4, o1[0]) + __builtin_bit_cast(f32x4, kb[tw][0]);
+#else
 #pragma unroll
                     for (int kd = 0; kd < KD; ++kd) {
-                        s0 = M_::mma(q0[kd], kb[tw][kd], s0);
-                        s1 = M_::mma(q1[kd], kb[tw][kd], s1);
+                        s0 = M_::mma(o0[kd], kb[tw][kd], s0);
+                        s1 = M_::mma(o1[kd], kb[tw][kd], s1);
                     }
-                    pk[tw][0] = M_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1]));
-                    pk[tw][1] = M_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3]));
-                    pk[tw][2] = M_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1]));
-                    pk[tw][3] = M_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]));
-                    float t = M_::sum2(pk[tw][0], 0.f);
-                    t = M_::sum2(pk[tw][1], t);
-                    t = M_::sum2(pk[tw][2], t);
-                    t = M_::sum2(pk[tw][3], t);
-                    tsum[tw] = t;
-                    bad = bad || !(t < kLazyLimit);
+#endif
+                    const u32x4 pb = {xpack2<M_>(xexp2(s0[0]), xexp2(s0[1])),
+                                      xpack2<M_>(xexp2(s0[2]), xexp2(s0[3])),
+                                      xpack2<M_>(xexp2(s1[0]), xexp2(s1[1])),
+                                      xpack2<M_>(xexp2(s1[2]), xexp2(s1[3]))};
+#if FLARE_EXPERIMENT == 2 || FLARE_EXPERIMENT == 6
+                    yl[tw] += __builtin_bit_cast(f32x4, pb);
+#else
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = M_::mma(oz[rt], pb, yacc[tw][rt]);
+                    yl[tw] = M_::mma(ones8, pb, yl[tw]);   // row of ones: the softmax denominator
+#endif
                 }
+            };
+            // two operand sets, each loaded from LDS one step before it is used (KS is even or 1
+            // step is peeled: M is a multiple of 64, so KS is always even)
+            u32x4 q0b[KD], q1b[KD], zab[RT];
+            load_ops(0, q0, q1, za);
+            for (int ks = 0; ks < KS; ks += 2) {
+                load_ops(ks + 1, q0b, q1b, zab);
+                step(q0, q1, za);
+                load_ops(ks + 2 < KS ? ks + 2 : ks, q0, q1, za);
+                step(q0b, q1b, zab);
             }
-            if (__builtin_expect(__any(bad), 0)) {
-                asm volatile("; exact path" ::: "memory");
+#pragma unroll
+            for (int tw = 0; tw < kSTW; ++tw) {
+                lrow[tw] = yl[tw][0];
+#if FLARE_EXPERIMENT == 0
+                redo = redo || !(lrow[tw] >= kLMin && lrow[tw] <= kLMax);
+#endif
+            }
+        }
+        if (__builtin_expect(__any(redo), 0)) {
+            // exact path: online maximum with rescaling
+            asm volatile("; exact path" ::: "memory");
+            float shift[kSTW], lsum[kSTW];
+#pragma unroll
+            for (int tw = 0; tw < kSTW; ++tw) {
+                shift[tw] = kNegBig;
+                lsum[tw] = 0.f;
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+            for (int ks = 0; ks < KS; ++ks) {
+                u32x4 q0[KD], q1[KD], za[RT];
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) {
+                    const int ch = kd * 4 + g;
+                    q0[kd] = ch < CH ? qa[((2 * ks) * CH + ch) * 16 + c16] : zero4();
+                    q1[kd] = ch < CH ? qa[((2 * ks + 1) * CH + ch) * 16 + c16] : zero4();
+                }
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) za[rt] = zt[(ks * RT + rt) * 64 + lane];
 #pragma unroll
                 for (int tw = 0; tw < kSTW; ++tw) {
                     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -470,34 +611,29 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                     for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] *= al;
                     lsum[tw] *= al;
                     shift[tw] = nc;
-                    negc[tw] = f32x4{-nc, -nc, -nc, -nc};
-                    pk[tw][0] = M_::pack2(fast_exp2(s0[0] - nc), fast_exp2(s0[1] - nc));
-                    pk[tw][1] = M_::pack2(fast_exp2(s0[2] - nc), fast_exp2(s0[3] - nc));
-                    pk[tw][2] = M_::pack2(fast_exp2(s1[0] - nc), fast_exp2(s1[1] - nc));
-                    pk[tw][3] = M_::pack2(fast_exp2(s1[2] - nc), fast_exp2(s1[3] - nc));
-                    float t = M_::sum2(pk[tw][0], 0.f);
-                    t = M_::sum2(pk[tw][1], t);
-                    t = M_::sum2(pk[tw][2], t);
-                    t = M_::sum2(pk[tw][3], t);
-                    tsum[tw] = t;
+                    const u32x4 pb = {M_::pack2(fast_exp2(s0[0] - nc), fast_exp2(s0[1] - nc)),
+                                      M_::pack2(fast_exp2(s0[2] - nc), fast_exp2(s0[3] - nc)),
+                                      M_::pack2(fast_exp2(s1[0] - nc), fast_exp2(s1[1] - nc)),
+                                      M_::pack2(fast_exp2(s1[2] - nc), fast_exp2(s1[3] - nc))};
+                    float t = M_::sum2(pb[0], 0.f);
+                    t = M_::sum2(pb[1], t);
+                    t = M_::sum2(pb[2], t);
+                    t = M_::sum2(pb[3], t);
+                    lsum[tw] += t;
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = M_::mma(za[rt], pb, yacc[tw][rt]);
                 }
             }
 #pragma unroll
-            for (int tw = 0; tw < kSTW; ++tw) {
-                const u32x4 pb = {pk[tw][0], pk[tw][1], pk[tw][2], pk[tw][3]};
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = M_::mma(za[rt], pb, yacc[tw][rt]);
-                lsum[tw] += tsum[tw];
-            }
+            for (int tw = 0; tw < kSTW; ++tw) lrow[tw] = xg_sum(lsum[tw]);
         }
 
         // normalise and store: lane (token c16, group g) owns d = (D/4) g .. (D/4) g + D/4 - 1
 #pragma unroll
         for (int tw = 0; tw < kSTW; ++tw) {
             const int n = t0 + tw * 16 + c16;
-            const float l = xg_sum(lsum[tw]);
             const bool on = n < wg_n1 && (mask == nullptr || mask[n] != 0);
-            const float inv = on ? 1.f / l : 0.f;
+            const float inv = on ? 1.f / lrow[tw] : 0.f;
             if (n < wg_n1) {
                 uint16_t* yr = y + (int64_t)n * a.ys[2] + (D / 4) * g;
                 uint32_t o[2 * RT];
