@@ -188,6 +188,13 @@ int check_causal_desc(const FlareCausalDesc* d)
     return FLARE_OK;
 }
 
+bool causal_wants_mfma(const FlareCausalDesc* d)
+{
+    return !(d->flags & FLARE_FLAG_FORCE_GENERIC) && flare::causal_mfma_supported(d->dtype, d->M, d->D) &&
+           strides_mult8(d->q_stride) && strides_mult8(d->k_stride) && strides_mult8(d->v_stride) &&
+           strides_mult8(d->y_stride);
+}
+
 void fill_causal_args(flare::CausalArgs& a, const FlareCausalDesc* d)
 {
     memset(&a, 0, sizeof(a));
@@ -319,7 +326,7 @@ int flare_causal_workspace_bytes(const FlareCausalDesc* desc, size_t* bytes)
     if (!bytes) return fail(FLARE_EINVAL, "bytes is NULL");
     int rc = check_causal_desc(desc);
     if (rc != FLARE_OK) return rc;
-    *bytes = 0;
+    *bytes = causal_wants_mfma(desc) ? (size_t)desc->B * desc->H * sizeof(int) : 0;
     return FLARE_OK;
 }
 
@@ -327,7 +334,6 @@ int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const v
                              void* y, float* mu, float* den, float* num, void* workspace,
                              size_t workspace_bytes, void* stream)
 {
-    (void)workspace; (void)workspace_bytes;
     int rc = check_causal_desc(desc);
     if (rc != FLARE_OK) return rc;
     if (!q || !k || !v || !y || !mu || !den || !num)
@@ -335,8 +341,19 @@ int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const v
     flare::CausalArgs a;
     fill_causal_args(a, desc);
     a.q = q; a.k = k; a.v = v; a.y = y; a.mu = mu; a.den = den; a.num = num;
-    return hip_status(flare::launch_causal_prefill(a, desc->dtype, static_cast<hipStream_t>(stream)),
-                      "causal prefill launch");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (causal_wants_mfma(desc) && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y)) {
+        // matrix-core kernel without a running maximum; it marks the (b,h) it could not validate
+        // and the fp32 kernel, launched right behind it, redoes exactly those
+        const size_t need = (size_t)desc->B * desc->H * sizeof(int);
+        if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
+        if (workspace_bytes < need)
+            return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, need);
+        a.flags = static_cast<int*>(workspace);
+        hipError_t e = flare::launch_causal_prefill_mfma(a, desc->dtype, st);
+        if (e != hipSuccess) return hip_status(e, "causal prefill (mfma) launch");
+    }
+    return hip_status(flare::launch_causal_prefill(a, desc->dtype, st), "causal prefill launch");
 }
 
 int flare_causal_decode_fwd(const FlareCausalDesc* desc, const void* q, const void* k, const void* v,

@@ -10,9 +10,9 @@
 //
 // One workgroup owns one (b,h) and walks its tokens in blocks of TB tokens; the state never
 // leaves LDS between blocks, so N decode steps (TB = 1) cost one launch.
-// Within a block the per-latent reference maximum is the block maximum, so a score that
-// jumps by more than ~2^120 inside one block of 16 tokens would underflow the earlier
-// denominators; prefill uses TB = 16 to keep that exposure small.
+// Inside a block every token keeps its own per-latent running maximum (the intra-block weights
+// are exp2(sigma[tau,m] - mc_t[m]) with tau <= t, so no exponent is ever positive), which makes the
+// kernel exact for arbitrary score jumps at the price of TB*TB*M/2 extra exponentials per block.
 #include "common.hpp"
 
 namespace flare {
@@ -22,7 +22,7 @@ namespace {
 constexpr int kThreads = 256;
 
 struct CausalLds {
-    int q, U, sg, gg, ks, vs, As, mu, den, al, rmax, rinv, total;  // offsets in floats
+    int q, U, sg, gg, mct, cf, ks, vs, As, mu, den, al, rmax, rinv, total;  // offsets in floats
 };
 
 __host__ __device__ inline CausalLds causal_lds_layout(int M, int D, int TB)
@@ -33,6 +33,8 @@ __host__ __device__ inline CausalLds causal_lds_layout(int M, int D, int TB)
     L.U = o;    o += M * D;
     L.sg = o;   o += TB * (M + 1);
     L.gg = o;   o += TB * (M + 1);
+    L.mct = o;  o += TB * (M + 1);
+    L.cf = o;   o += TB * (M + 1);
     L.ks = o;   o += TB * D;
     L.vs = o;   o += TB * D;
     L.As = o;   o += TB * TB;
@@ -65,12 +67,14 @@ __global__ __launch_bounds__(kThreads) void causal_generic_kernel(CausalArgs a)
     const int M = a.M, D = a.D, N = a.N;
     const CausalLds L = causal_lds_layout(M, D, TB);
     float* qs = sm + L.q;   float* U = sm + L.U;   float* sg = sm + L.sg; float* gg = sm + L.gg;
+    float* mct = sm + L.mct; float* cf = sm + L.cf;
     float* ks = sm + L.ks;  float* vs = sm + L.vs; float* As = sm + L.As;
     float* mu_s = sm + L.mu; float* den_s = sm + L.den; float* al_s = sm + L.al;
     float* rmax = sm + L.rmax; float* rinv = sm + L.rinv;
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H;
+    if (a.flags != nullptr && a.flags[bh] == 0) return;   // fallback launch: only marked (b,h) are redone
     const T* q = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
     const T* k = (const T*)a.k + b * a.ks[0] + h * a.ks[1];
     const T* v = (const T*)a.v + b * a.vs[0] + h * a.vs[1];
@@ -119,49 +123,57 @@ __global__ __launch_bounds__(kThreads) void causal_generic_kernel(CausalArgs a)
             if (lane == 0) { rmax[t] = mx; rinv[t] = 1.f / sum; }
         }
         __syncthreads();
-        // per latent: block maximum, running denominator, G = w / den, P in place of sigma
+        // per latent, token by token: running maximum mc_t, denominator relative to it,
+        // G = w / den_t and the coefficient of the carried-in state exp2(mu - mc_t) G
         for (int m = tid; m < M; m += kThreads) {
             const float mp = mu_s[m];
-            float mc = mp;
-            for (int t = 0; t < tb; ++t) mc = fmaxf(mc, sg[t * (M + 1) + m]);
-            const float al = fast_exp2(mp - mc);
-            float dc = al * den_s[m];
+            float mc = mp, dc = den_s[m];
             for (int t = 0; t < tb; ++t) {
                 const float s = sg[t * (M + 1) + m];
-                const float p = fast_exp2(s - mc);
-                dc += p;
+                const float mn = fmaxf(mc, s);
+                dc = dc * fast_exp2(mc - mn) + fast_exp2(s - mn);
+                mc = mn;
                 const float w = fast_exp2(s - rmax[t]) * rinv[t];
-                gg[t * (M + 1) + m] = w / dc;
-                sg[t * (M + 1) + m] = p;
+                const float gv = w / dc;
+                gg[t * (M + 1) + m] = gv;
+                mct[t * (M + 1) + m] = mc;
+                cf[t * (M + 1) + m] = gv * fast_exp2(mp - mc);
             }
-            mu_s[m] = mc; den_s[m] = dc; al_s[m] = al;
+            mu_s[m] = mc; den_s[m] = dc; al_s[m] = fast_exp2(mp - mc);
         }
         __syncthreads();
-        // A[t][tau] = sum_m G[t,m] P[tau,m] for tau <= t
+        // A[t][tau] = sum_m G[t,m] exp2(sigma[tau,m] - mc_t[m]) for tau <= t (every exponent <= 0)
         if (TB > 1) {
             for (int idx = tid; idx < tb * tb; idx += kThreads) {
                 const int t = idx / tb, tau = idx - t * tb;
                 float acc = 0.f;
                 if (tau <= t)
-                    for (int m = 0; m < M; ++m) acc = fmaf(gg[t * (M + 1) + m], sg[tau * (M + 1) + m], acc);
+                    for (int m = 0; m < M; ++m)
+                        acc = fmaf(gg[t * (M + 1) + m], fast_exp2(sg[tau * (M + 1) + m] - mct[t * (M + 1) + m]), acc);
                 As[t * TB + tau] = acc;
             }
             __syncthreads();
         }
-        // y[t,d] = sum_m G[t,m] alpha[m] U[m,d] + sum_{tau<=t} A[t,tau] v[tau,d]
+        // y[t,d] = sum_m cf[t,m] U[m,d] + sum_{tau<=t} A[t,tau] v[tau,d]
         for (int idx = tid; idx < tb * D; idx += kThreads) {
             const int t = idx / D, d = idx - t * D;
             float acc = 0.f;
-            for (int m = 0; m < M; ++m) acc = fmaf(gg[t * (M + 1) + m] * al_s[m], U[m * D + d], acc);
+            for (int m = 0; m < M; ++m) acc = fmaf(cf[t * (M + 1) + m], U[m * D + d], acc);
             if (TB > 1) {
                 for (int tau = 0; tau <= t; ++tau) acc = fmaf(As[t * TB + tau], vs[tau * D + d], acc);
             } else {
-                // single token: A[0][0] = sum_m G[0,m] P[0,m]
+                // single token: A[0][0] = sum_m G[0,m] exp2(sigma[0,m] - mc_0[m])
                 float a00 = 0.f;
-                for (int m = 0; m < M; ++m) a00 = fmaf(gg[m], sg[m], a00);
+                for (int m = 0; m < M; ++m) a00 = fmaf(gg[m], fast_exp2(sg[m] - mct[m]), a00);
                 acc = fmaf(a00, vs[d], acc);
             }
             y[(int64_t)(n0 + t) * a.ys[2] + d] = from_f32<T>(acc);
+        }
+        __syncthreads();
+        // probabilities relative to the end-of-block maximum, in place of the scores
+        for (int idx = tid; idx < tb * M; idx += kThreads) {
+            const int t = idx / M, m = idx - t * M;
+            sg[t * (M + 1) + m] = fast_exp2(sg[t * (M + 1) + m] - mu_s[m]);
         }
         __syncthreads();
         // U[m,d] = alpha[m] U[m,d] + sum_t P[t,m] v[t,d]

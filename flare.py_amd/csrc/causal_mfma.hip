@@ -1,0 +1,343 @@
+// Causal FLARE chunked prefill on the matrix cores (bf16 / f16, D in {32, 64}, M in {128, 256}).
+//
+// Same definition and state as causal.hip:  z_t = gather over tokens <= t,  y_t = scatter of z_t.
+// One workgroup (4 waves) owns one (b,h) and walks its tokens in blocks of 16; wave w owns
+// MW = M/4 latents (their scores, running denominators and state rows), so the only cross-wave
+// step is the sum over latents of the 16 x D output tile, done through LDS with one barrier per
+// block.  Per block and wave, with P = exp2(score - mu0) for the wave's latents (mu0 = the shift
+// of the incoming state, 0 for a fresh one; no running maximum):
+//   dcum[t,m] = den[m] + sum_{tau<=t} P[tau,m]          (MFMA with a lower-triangular ones matrix)
+//   G[t,m]    = P[t,m] / dcum[t,m]
+//   Y[t,:]   += G[t,:] U  +  tril(G P^T)[t,:] V          (U = state numerator [m,d])
+//   r[t]     += sum_m P[t,m]                             (MFMA against ones)
+//   U[m,:]   += P[:,m]^T V ;  den[m] += sum_tau P[tau,m]
+// and finally y_t = (sum over waves of Y[t,:]) / (sum over waves of r[t]).
+// A 16x16 accumulator tile (lane = column c16, registers = rows 4g..4g+3) is reused directly as the
+// A or B operand of a 16x16x16 MFMA whose contraction runs over those rows; operands that need the
+// other orientation (tokens in lanes, latents in registers) go through a wave-private LDS tile and
+// the transpose read.  Working without a running maximum is validated (finite outputs, softmax
+// sums and denominators inside 2^-60..2^120); a (b,h) that fails leaves its state untouched and
+// raises a flag, and the fp32 kernel of causal.hip, launched right after, redoes exactly those.
+#include "common.hpp"
+
+namespace flare {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr float kLMin = 8.6736174e-19f, kLMax = 1.329228e36f;   // 2^-60, 2^120
+
+template <typename T> struct Mm;
+template <> struct Mm<bf16_t> {
+    static constexpr uint32_t kOnes2 = 0x3f803f80u;
+    static __device__ __forceinline__ f32x4 mma32(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 mma16(uint2 a, uint2 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        bf16x2 v = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float unpack(uint16_t b) { return __uint_as_float(uint32_t(b) << 16); }
+};
+template <> struct Mm<f16_t> {
+    static constexpr uint32_t kOnes2 = 0x3c003c00u;
+    static __device__ __forceinline__ f32x4 mma32(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4 mma16(uint2 a, uint2 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        f16x2 v = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float unpack(uint16_t b) { return float(__builtin_bit_cast(_Float16, b)); }
+};
+
+__device__ __forceinline__ uint2 tr16(const void* lds_addr)
+{
+    typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
+    return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)lds_addr));
+}
+
+constexpr int kTB = 16;   // tokens per block
+
+template <typename T, int D, int KM>
+__global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a)
+{
+    constexpr int KD = D / 32;          // k-steps over d of the score product
+    constexpr int DT = D / 16;          // 16-column tiles of d
+    constexpr int CT = 2 * KM;          // 16-latent column tiles per wave
+    constexpr int MW = 32 * KM;         // latents per wave
+    constexpr int M = 4 * MW;
+    constexpr int YS = D + 4;           // padded row stride (floats) of the output partials
+    using M_ = Mm<T>;
+
+    __shared__ __attribute__((aligned(16))) uint16_t vs[2][kTB][D];       // V block, row-major
+    __shared__ __attribute__((aligned(16))) uint16_t pt[4][MW][kTB];      // P^T per wave  [latent][token]
+    __shared__ __attribute__((aligned(16))) uint16_t gt[4][MW][kTB];      // G^T per wave
+    __shared__ __attribute__((aligned(16))) float yp[2][4][kTB][YS];      // output partials per wave
+    __shared__ float rp[2][4][kTB];                                       // softmax-sum partials per wave
+    __shared__ int bad_flag;
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H;
+    const int N = a.N;
+    const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
+    const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
+    const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
+    uint16_t* y = (uint16_t*)a.y + b * a.ys[0] + h * a.ys[1];
+    float* mu_g = a.mu + (int64_t)bh * M;
+    float* den_g = a.den + (int64_t)bh * M;
+    float* num_g = a.num + (int64_t)bh * M * D;
+    const float sl2 = a.scale * kLog2e;
+    const int m0 = w * MW;
+
+    if (tid == 0) bad_flag = 0;
+
+    // latent operands (B of the score product), log2-scaled; shift and denominators per column
+    u32x4 qb[CT][KD];
+    f32x4 negmu[CT], den[CT];
+    float mu0[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int m = m0 + ct * 16 + c16;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const u32x4 raw = *reinterpret_cast<const u32x4*>(q + (int64_t)m * a.qs[2] + kd * 32 + g * 8);
+            u32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                o[i] = M_::pack2(M_::unpack(uint16_t(raw[i] & 0xffffu)) * sl2, M_::unpack(uint16_t(raw[i] >> 16)) * sl2);
+            qb[ct][kd] = o;
+        }
+        const float mu = mu_g[m];
+        mu0[ct] = mu <= kNegBig ? 0.f : mu * kLog2e;
+        negmu[ct] = f32x4{-mu0[ct], -mu0[ct], -mu0[ct], -mu0[ct]};
+        const float d0 = mu <= kNegBig ? 0.f : den_g[m];
+        den[ct] = f32x4{d0, d0, d0, d0};
+    }
+    // state numerator U[m, d]: tile (mt, dt) holds rows m0 + 16 mt + 4g + r, column 16 dt + c16
+    f32x4 U[CT][DT];
+#pragma unroll
+    for (int mt = 0; mt < CT; ++mt)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = m0 + mt * 16 + 4 * g + r;
+                U[mt][dt][r] = mu_g[m] <= kNegBig ? 0.f : num_g[(int64_t)m * D + dt * 16 + c16];
+            }
+
+    // constant operands: lower-triangular ones L[t = c16][tau = 4g + e] and all ones
+    uint2 ltri, ones4 = make_uint2(M_::kOnes2, M_::kOnes2);
+    {
+        const uint32_t one = M_::kOnes2 & 0xffffu;
+        uint32_t e[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) e[i] = (4 * g + i <= c16) ? one : 0u;
+        ltri = make_uint2(e[0] | (e[1] << 16), e[2] | (e[3] << 16));
+    }
+    const u32x4 ones8 = {M_::kOnes2, M_::kOnes2, M_::kOnes2, M_::kOnes2};
+
+    // block staging: K as A operand straight from global memory, V through LDS (threads < 2 D)
+    u32x4 ka[KD], kn[KD], vr;
+    auto load_block = [&](int n0, u32x4 (&kd_)[KD]) {
+        const int n = min(n0 + c16, N - 1);
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) kd_[kd] = *reinterpret_cast<const u32x4*>(k + (int64_t)n * a.ks[2] + kd * 32 + g * 8);
+        if (tid < 2 * D) {
+            const int tok = tid / (D / 8), ch = tid % (D / 8);
+            vr = *reinterpret_cast<const u32x4*>(v + (int64_t)min(n0 + tok, N - 1) * a.vs[2] + ch * 8);
+        }
+    };
+    auto store_v = [&](int buf) {
+        if (tid < 2 * D) {
+            const int tok = tid / (D / 8), ch = tid % (D / 8);
+            *reinterpret_cast<u32x4*>(&vs[buf][tok][ch * 8]) = vr;
+        }
+    };
+
+    bool bad = false;
+    load_block(0, ka);
+    store_v(0);
+    if (kTB < N) load_block(kTB, kn);
+    __syncthreads();
+
+    int it = 0;
+    for (int n0 = 0; n0 < N; n0 += kTB, ++it) {
+        const int buf = it & 1;
+        const int tb = min(kTB, N - n0);
+
+        // scores and probabilities of the wave's latents: rows tau = 4g + r, column m = c16
+        float p[CT][4];
+        uint2 ppk[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            f32x4 s = negmu[ct];
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) s = M_::mma32(ka[kd], qb[ct][kd], s);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) p[ct][r] = (4 * g + r < tb) ? fast_exp2(s[r]) : 0.f;
+            ppk[ct] = make_uint2(M_::pack2(p[ct][0], p[ct][1]), M_::pack2(p[ct][2], p[ct][3]));
+        }
+        // running denominators: dcum = den + L P ; den += 1 P ; G = P / dcum
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            const f32x4 dc = M_::mma16(ltri, ppk[ct], den[ct]);
+            den[ct] = M_::mma16(ones4, ppk[ct], den[ct]);
+            float gv[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) gv[r] = p[ct][r] > 0.f ? p[ct][r] * __builtin_amdgcn_rcpf(dc[r]) : 0.f;
+            const uint2 gpk = make_uint2(M_::pack2(gv[0], gv[1]), M_::pack2(gv[2], gv[3]));
+            *reinterpret_cast<uint2*>(&pt[w][ct * 16 + c16][4 * g]) = ppk[ct];
+            *reinterpret_cast<uint2*>(&gt[w][ct * 16 + c16][4 * g]) = gpk;
+        }
+        // operands with tokens in lanes and latents in k-slots (e < 4: tile 2 km, e >= 4: tile 2 km + 1)
+        u32x4 pop[KM], gop[KM];
+#pragma unroll
+        for (int km = 0; km < KM; ++km) {
+            const int r0 = km * 32 + 4 * g + (c16 >> 2), r1 = r0 + 16, piece = (c16 & 3) * 4;
+            const uint2 p0 = tr16(&pt[w][r0][piece]), p1 = tr16(&pt[w][r1][piece]);
+            const uint2 g0 = tr16(&gt[w][r0][piece]), g1 = tr16(&gt[w][r1][piece]);
+            pop[km] = u32x4{p0.x, p0.y, p1.x, p1.y};
+            gop[km] = u32x4{g0.x, g0.y, g1.x, g1.y};
+        }
+        // V operand (k-slots = tokens 4g..4g+3, lane = column d)
+        uint2 vop[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vop[dt] = tr16(&vs[buf][4 * g + (c16 >> 2)][dt * 16 + (c16 & 3) * 4]);
+
+        // intra-block matrix AccT[tau, t] = sum_m P[tau,m] G[t,m], masked to tau <= t, and r[t]
+        f32x4 acct = {0.f, 0.f, 0.f, 0.f}, rsum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int km = 0; km < KM; ++km) {
+            acct = M_::mma32(pop[km], gop[km], acct);
+            rsum = M_::mma32(pop[km], ones8, rsum);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acct[r] = (4 * g + r <= c16) ? acct[r] : 0.f;
+        const uint2 aop = make_uint2(M_::pack2(acct[0], acct[1]), M_::pack2(acct[2], acct[3]));
+
+        // output partial over the wave's latents, then the state update
+        f32x4 yacc[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int km = 0; km < KM; ++km) {
+                const f32x4 u0 = U[2 * km][dt], u1 = U[2 * km + 1][dt];
+                const u32x4 ub = {M_::pack2(u0[0], u0[1]), M_::pack2(u0[2], u0[3]),
+                                  M_::pack2(u1[0], u1[1]), M_::pack2(u1[2], u1[3])};
+                acc = M_::mma32(gop[km], ub, acc);
+            }
+            yacc[dt] = M_::mma16(aop, vop[dt], acc);
+        }
+#pragma unroll
+        for (int mt = 0; mt < CT; ++mt)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) U[mt][dt] = M_::mma16(ppk[mt], vop[dt], U[mt][dt]);
+
+        // partials to LDS (rows t = 4g + r, column d = 16 dt + c16)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) yp[buf][w][4 * g + r][dt * 16 + c16] = yacc[dt][r];
+        if (c16 == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) rp[buf][w][4 * g + r] = rsum[r];
+        }
+
+        // stage the next block
+        if (n0 + kTB < N) {
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) ka[kd] = kn[kd];
+            store_v(buf ^ 1);
+            if (n0 + 2 * kTB < N) load_block(n0 + 2 * kTB, kn);
+        }
+        __syncthreads();
+
+        // y[t, :] = sum_w Y_w[t, :] / sum_w r_w[t]; thread = (token, 4 consecutive d)
+        for (int idx = tid; idx < kTB * (D / 4); idx += 256) {
+            const int t = idx / (D / 4), d4 = (idx % (D / 4)) * 4;
+            const f32x4 s = *reinterpret_cast<const f32x4*>(&yp[buf][0][t][d4]) + *reinterpret_cast<const f32x4*>(&yp[buf][1][t][d4]) +
+                            *reinterpret_cast<const f32x4*>(&yp[buf][2][t][d4]) + *reinterpret_cast<const f32x4*>(&yp[buf][3][t][d4]);
+            const float r = rp[buf][0][t] + rp[buf][1][t] + rp[buf][2][t] + rp[buf][3][t];
+            if (t < tb) {
+                const float inv = 1.f / r;
+                const f32x4 o = s * inv;
+                bad = bad || !(r >= kLMin && r <= kLMax) || !(fabsf(o[0]) + fabsf(o[1]) + fabsf(o[2]) + fabsf(o[3]) <= 3.0e38f);
+                *reinterpret_cast<uint2*>(y + (int64_t)(n0 + t) * a.ys[2] + d4) =
+                    make_uint2(M_::pack2(o[0], o[1]), M_::pack2(o[2], o[3]));
+            }
+        }
+    }
+
+    // validate the final denominators, then publish the state (or the redo flag)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) bad = bad || !(den[ct][0] >= kLMin && den[ct][0] <= kLMax);
+    if (__any(bad) && lane == 0) bad_flag = 1;
+    __syncthreads();
+    if (bad_flag) {
+        if (tid == 0) a.flags[bh] = 1;
+        return;
+    }
+    if (tid == 0) a.flags[bh] = 0;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int m = m0 + ct * 16 + c16;
+        if (g == 0) {
+            mu_g[m] = mu0[ct] * kLn2;
+            den_g[m] = den[ct][0];
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) num_g[(int64_t)(m0 + ct * 16 + 4 * g + r) * D + dt * 16 + c16] = U[ct][dt][r];
+    }
+}
+
+template <typename T>
+hipError_t launch_t(const CausalArgs& a, hipStream_t st)
+{
+    dim3 grid(a.B * a.H), block(256);
+    if (a.D == 64 && a.M == 128)      hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 1>), grid, block, 0, st, a);
+    else if (a.D == 64 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 2>), grid, block, 0, st, a);
+    else if (a.D == 32 && a.M == 128) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 1>), grid, block, 0, st, a);
+    else if (a.D == 32 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 2>), grid, block, 0, st, a);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool causal_mfma_supported(int dtype, int M, int D)
+{
+    // the fp32 kernel must be able to redo any (b,h), so its LDS limit applies here too
+    return (dtype == 1 || dtype == 2) && (D == 32 || D == 64) && (M == 128 || M == 256) &&
+           causal_lds_bytes(M, D, false) <= 160 * 1024;
+}
+
+hipError_t launch_causal_prefill_mfma(const CausalArgs& a, int dtype, hipStream_t st)
+{
+    return dtype == 1 ? launch_t<bf16_t>(a, st) : launch_t<f16_t>(a, st);
+}
+
+}  // namespace flare

@@ -53,6 +53,7 @@ struct MixerArgs {
 struct CausalArgs {
     const void* q; const void* k; const void* v; void* y;
     float* mu; float* den; float* num;   // state, natural-log units for mu
+    int* flags;                          // [B*H] or null: per-(b,h) "redo with the fp32 kernel" marks
     int B, H, N, M, D;
     int chunk;
     float scale;
@@ -85,6 +86,8 @@ hipError_t launch_scatter_mfma(const MixerArgs& a, int dtype, hipStream_t st);
 size_t     causal_lds_bytes(int M, int D, bool decode);
 hipError_t launch_causal_prefill(const CausalArgs& a, int dtype, hipStream_t st);
 hipError_t launch_causal_decode(const CausalArgs& a, int dtype, hipStream_t st);
+bool       causal_mfma_supported(int dtype, int M, int D);
+hipError_t launch_causal_prefill_mfma(const CausalArgs& a, int dtype, hipStream_t st);
 
 hipError_t launch_triple_state(const TripleArgs& a, int dtype, hipStream_t st);
 hipError_t launch_triple_merge(const TripleArgs& a, hipStream_t st);

@@ -117,3 +117,42 @@ def test_cfg4_shape_reduced_length(dev):
     assert O.rel_l2(y1, yr[:, :, :NP]) <= 2e-2
     assert O.rel_l2(y2, yr[:, :, NP:]) <= 2e-2
     state_close(st, tuple(s.double() for s in str_), 2e-2)
+
+
+# ---- matrix-core prefill kernel (bf16/f16, M in {128,256}, D in {32,64}) ------------------------
+@pytest.mark.parametrize("shape", [(1, 2, 333, 128, 32), (1, 1, 100, 256, 32), (2, 1, 64, 128, 64), (1, 3, 1000, 128, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_prefill_shapes(dev, shape, dtype):
+    q, k, v = make(*shape, dtype)
+    y, st = F.flare_causal_prefill(q.to(dev), k.to(dev), v.to(dev))
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float(), dtype=torch.float32)
+    assert O.rel_l2(y, yr) <= 2e-2
+    state_close(st, tuple(s.double() for s in str_), 2e-2)
+
+
+def test_mfma_prefill_continuation_and_decode(dev):
+    # state handed from one matrix-core prefill to the next and on to the recurrent decode
+    q, k, v = make(1, 2, 700, 128, 64, torch.bfloat16, seed=6)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    y1, st = F.flare_causal_prefill(qd, kd[:, :, :300], vd[:, :, :300])
+    y2, st = F.flare_causal_prefill(qd, kd[:, :, 300:650], vd[:, :, 300:650], state=st)
+    y3, st = F.flare_causal_decode(qd, kd[:, :, 650:], vd[:, :, 650:], st)
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float(), dtype=torch.float32)
+    assert O.rel_l2(torch.cat([y1, y2, y3], 2), yr) <= 2e-2
+    state_close(st, tuple(s.double() for s in str_), 2e-2)
+
+
+def test_mfma_prefill_out_of_window_scores_fall_back(dev):
+    # scores far outside the window in which the matrix-core kernel may skip the running maximum:
+    # it must flag those (b,h) and the fp32 kernel must redo them; one head stays in the window.
+    q, k, v = make(1, 2, 200, 128, 64, torch.bfloat16, seed=7, std=1.0)
+    k[:, 0] *= 8.0                      # head 0: |score| up to several hundred
+    k[:, 1] *= 0.05                     # head 1: tame
+    s = torch.einsum("hmd,bhnd->bhmn", q.float(), k.float())
+    assert float(s[:, 0].abs().max()) > 150 and float(s[:, 1].abs().max()) < 20
+    y, st = F.flare_causal_prefill(q.to(dev), k.to(dev), v.to(dev))
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float())
+    assert torch.isfinite(y.float()).all()
+    assert O.rel_l2(y[:, 0], yr[:, 0]) <= 1e-5 * 1e3   # fp32 kernel on bf16 outputs: bf16 output rounding only
+    assert O.rel_l2(y[:, 1], yr[:, 1]) <= 2e-2
+    state_close(st, str_, 2e-2)
