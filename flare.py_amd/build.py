@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libflare_hip.so")
-SOURCES = ["capi.hip", "mixer_generic.hip", "mixer_mfma.hip", "causal.hip", "causal_mfma.hip", "triple.hip"]
+SOURCES = ["capi.hip", "mixer_generic.hip", "mixer_mfma.hip", "causal.hip", "causal_mfma.hip", "triple.hip", "triple_mfma.hip"]
 # packed-fp32 instruction selection is switched off for every device translation unit
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-math-errno", "-ffp-contract=fast",
@@ -26,7 +26,7 @@ def hipcc() -> str:
     return exe
 
 
-def build(verbose: bool = True, jobs: int = 6) -> str:
+def build(verbose: bool = True, jobs: int = 7) -> str:
     cc = hipcc()
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)

@@ -220,11 +220,22 @@ int check_triple_desc(const FlareTripleDesc* d)
     return FLARE_OK;
 }
 
-struct TriplePlan { int n_splits, tokens_per_split; size_t per_split, off_kk, total; };
+struct TriplePlan { bool mfma; int n_splits, n_parts, tokens_per_split; size_t per_split, off_kk, total; };
+
+bool strides_mult4(const int64_t* s) { return s[0] % 4 == 0 && s[1] % 4 == 0 && s[2] % 4 == 0; }
+bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
+
+bool triple_wants_mfma(const FlareTripleDesc* d)
+{
+    return !(d->flags & FLARE_FLAG_FORCE_GENERIC) && flare::triple_mfma_supported(d->dtype, d->Dq, d->Dv) &&
+           strides_mult4(d->q1_stride) && strides_mult4(d->q2_stride) && strides_mult4(d->k1_stride) &&
+           strides_mult4(d->k2_stride) && strides_mult4(d->v_stride);
+}
 
 TriplePlan plan_triple(const FlareTripleDesc* d)
 {
     TriplePlan p;
+    p.mfma = triple_wants_mfma(d);
     int s = d->n_splits;
     if (s <= 0) {
         const int64_t per = (int64_t)d->B * d->H;
@@ -232,12 +243,13 @@ TriplePlan plan_triple(const FlareTripleDesc* d)
         if (s < 1) s = 1;
     }
     int64_t tps = ((int64_t)d->N + s - 1) / s;
-    if (tps < 64) tps = 64;
+    tps = ((tps + 63) / 64) * 64;
     p.tokens_per_split = (int)tps;
     p.n_splits = (int)(((int64_t)d->N + tps - 1) / tps);
+    p.n_parts = p.n_splits;
     p.per_split = (size_t)d->Dq * d->Dv * d->Dq + (size_t)d->Dq * d->Dq;
     const size_t bh = (size_t)d->B * d->H;
-    p.off_kk = bh * p.n_splits * p.per_split * 4;
+    p.off_kk = bh * p.n_parts * p.per_split * 4;
     p.off_kk = (p.off_kk + 255) & ~(size_t)255;
     p.total = p.off_kk + bh * d->Dq * d->Dq * 4;
     return p;
@@ -248,7 +260,7 @@ void fill_triple_args(flare::TripleArgs& a, const FlareTripleDesc* d, const Trip
     memset(&a, 0, sizeof(a));
     a.B = d->B; a.H = d->H; a.N = d->N; a.Dq = d->Dq; a.Dv = d->Dv;
     a.feature_map = d->feature_map; a.normalize = d->normalize;
-    a.n_splits = p.n_splits; a.tokens_per_split = p.tokens_per_split;
+    a.n_splits = p.n_splits; a.tokens_per_split = p.tokens_per_split; a.n_parts = p.n_splits;
     for (int i = 0; i < 3; ++i) {
         a.q1s[i] = d->q1_stride[i]; a.q2s[i] = d->q2_stride[i]; a.k1s[i] = d->k1_stride[i];
         a.k2s[i] = d->k2_stride[i]; a.vs[i] = d->v_stride[i]; a.os[i] = d->o_stride[i];
@@ -396,7 +408,9 @@ int flare_triple_state_fwd(const FlareTripleDesc* desc, const void* k1, const vo
     a.k1 = k1; a.k2 = k2; a.v = v; a.state = state; a.kk = kk_state;
     a.part = static_cast<float*>(workspace);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    hipError_t e = flare::launch_triple_state(a, desc->dtype, st);
+    const bool mfma = p.mfma && aligned8(k1) && aligned8(k2) && aligned8(v);
+    if (mfma) a.n_parts = p.n_parts;
+    hipError_t e = mfma ? flare::launch_triple_state_mfma(a, desc->dtype, st) : flare::launch_triple_state(a, desc->dtype, st);
     if (e != hipSuccess) return hip_status(e, "triple state launch");
     return hip_status(flare::launch_triple_merge(a, st), "triple merge launch");
 }
@@ -412,7 +426,10 @@ int flare_triple_out_fwd(const FlareTripleDesc* desc, const void* q1, const void
     flare::TripleArgs a;
     fill_triple_args(a, desc, p);
     a.q1 = q1; a.q2 = q2; a.out = out; a.state = const_cast<float*>(state); a.kk = const_cast<float*>(kk_state);
-    return hip_status(flare::launch_triple_out(a, desc->dtype, static_cast<hipStream_t>(stream)), "triple out launch");
+    const bool mfma = p.mfma && aligned8(q1) && aligned8(q2);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return hip_status(mfma ? flare::launch_triple_out_mfma(a, desc->dtype, st) : flare::launch_triple_out(a, desc->dtype, st),
+                      "triple out launch");
 }
 
 int flare_triple_fwd(const FlareTripleDesc* desc, const void* q1, const void* q2, const void* k1,

@@ -68,6 +68,7 @@ struct TripleArgs {
     int B, H, N, Dq, Dv;
     int feature_map, normalize;
     int n_splits, tokens_per_split;
+    int n_parts;       // partials per (b,h) in `part`
     int64_t q1s[3], q2s[3], k1s[3], k2s[3], vs[3], os[3];
 };
 
@@ -92,5 +93,8 @@ hipError_t launch_causal_prefill_mfma(const CausalArgs& a, int dtype, hipStream_
 hipError_t launch_triple_state(const TripleArgs& a, int dtype, hipStream_t st);
 hipError_t launch_triple_merge(const TripleArgs& a, hipStream_t st);
 hipError_t launch_triple_out(const TripleArgs& a, int dtype, hipStream_t st);
+bool       triple_mfma_supported(int dtype, int Dq, int Dv);
+hipError_t launch_triple_state_mfma(const TripleArgs& a, int dtype, hipStream_t st);
+hipError_t launch_triple_out_mfma(const TripleArgs& a, int dtype, hipStream_t st);
 
 }  // namespace flare

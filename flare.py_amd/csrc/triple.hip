@@ -82,7 +82,7 @@ __global__ __launch_bounds__(kThreads) void triple_state_kernel(TripleArgs a, in
     }
     if (live) {
         const size_t per = (size_t)Dq * Dv * Dq + (size_t)Dq * Dq;
-        float* part = a.part + (((size_t)b * a.H + h) * a.n_splits + split) * per;
+        float* part = a.part + (((size_t)b * a.H + h) * a.n_parts + split) * per;
         for (int k = 0; k < Dq; ++k) part[((size_t)i * Dv + j) * Dq + k] = acc[k];
         if (j == 0)
             for (int k = 0; k < Dq; ++k) part[(size_t)Dq * Dv * Dq + (size_t)i * Dq + k] = kk[k];
@@ -96,9 +96,9 @@ __global__ __launch_bounds__(kThreads) void triple_merge_kernel(TripleArgs a)
     const size_t idx = (size_t)blockIdx.x * kThreads + threadIdx.x;
     if (idx >= total) return;
     const size_t bh = idx / per, e = idx - bh * per;
-    const float* p = a.part + bh * a.n_splits * per + e;
+    const float* p = a.part + bh * a.n_parts * per + e;
     float s = 0.f;
-    for (int sp = 0; sp < a.n_splits; ++sp) s += p[(size_t)sp * per];
+    for (int sp = 0; sp < a.n_parts; ++sp) s += p[(size_t)sp * per];
     s *= 1.0f / (float)a.N;
     if (e < ns) a.state[bh * ns + e] = s;
     else if (a.kk) a.kk[bh * nk + (e - ns)] = s;
