@@ -342,9 +342,9 @@ int flare_causal_workspace_bytes(const FlareCausalDesc* desc, size_t* bytes)
     return FLARE_OK;
 }
 
-int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const void* k, const void* v,
-                             void* y, float* mu, float* den, float* num, void* workspace,
-                             size_t workspace_bytes, void* stream)
+namespace {
+int causal_run(const FlareCausalDesc* desc, bool decode, const void* q, const void* k, const void* v, void* y,
+               float* mu, float* den, float* num, void* workspace, size_t workspace_bytes, void* stream)
 {
     int rc = check_causal_desc(desc);
     if (rc != FLARE_OK) return rc;
@@ -362,24 +362,26 @@ int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const v
         if (workspace_bytes < need)
             return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, need);
         a.flags = static_cast<int*>(workspace);
-        hipError_t e = flare::launch_causal_prefill_mfma(a, desc->dtype, st);
-        if (e != hipSuccess) return hip_status(e, "causal prefill (mfma) launch");
+        hipError_t e = flare::launch_causal_mfma(a, desc->dtype, decode ? 1 : 16, st);
+        if (e != hipSuccess) return hip_status(e, "causal (mfma) launch");
     }
-    return hip_status(flare::launch_causal_prefill(a, desc->dtype, st), "causal prefill launch");
+    hipError_t e = decode ? flare::launch_causal_decode(a, desc->dtype, st) : flare::launch_causal_prefill(a, desc->dtype, st);
+    return hip_status(e, decode ? "causal decode launch" : "causal prefill launch");
+}
+}  // namespace
+
+int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const void* k, const void* v,
+                             void* y, float* mu, float* den, float* num, void* workspace,
+                             size_t workspace_bytes, void* stream)
+{
+    return causal_run(desc, false, q, k, v, y, mu, den, num, workspace, workspace_bytes, stream);
 }
 
 int flare_causal_decode_fwd(const FlareCausalDesc* desc, const void* q, const void* k, const void* v,
-                            void* y, float* mu, float* den, float* num, void* stream)
+                            void* y, float* mu, float* den, float* num, void* workspace,
+                            size_t workspace_bytes, void* stream)
 {
-    int rc = check_causal_desc(desc);
-    if (rc != FLARE_OK) return rc;
-    if (!q || !k || !v || !y || !mu || !den || !num)
-        return fail(FLARE_EINVAL, "q, k, v, y, mu, den, num must not be NULL");
-    flare::CausalArgs a;
-    fill_causal_args(a, desc);
-    a.q = q; a.k = k; a.v = v; a.y = y; a.mu = mu; a.den = den; a.num = num;
-    return hip_status(flare::launch_causal_decode(a, desc->dtype, static_cast<hipStream_t>(stream)),
-                      "causal decode launch");
+    return causal_run(desc, true, q, k, v, y, mu, den, num, workspace, workspace_bytes, stream);
 }
 
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes)

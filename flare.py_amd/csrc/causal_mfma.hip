@@ -80,7 +80,7 @@ __device__ __forceinline__ uint2 tr16(const void* lds_addr)
 constexpr int kTB = 16;   // tokens per block
 
 template <typename T, int D, int KM>
-__global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a)
+__global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step)
 {
     constexpr int KD = D / 32;          // k-steps over d of the score product
     constexpr int DT = D / 16;          // 16-column tiles of d
@@ -178,13 +178,14 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a)
     bool bad = false;
     load_block(0, ka);
     store_v(0);
-    if (kTB < N) load_block(kTB, kn);
+    if (step < N) load_block(step, kn);
     __syncthreads();
 
     int it = 0;
-    for (int n0 = 0; n0 < N; n0 += kTB, ++it) {
+    // step = 16: chunked prefill; step = 1: recurrent decode, one token per block (rows >= tb are masked)
+    for (int n0 = 0; n0 < N; n0 += step, ++it) {
         const int buf = it & 1;
-        const int tb = min(kTB, N - n0);
+        const int tb = min(step, N - n0);
 
         // scores and probabilities of the wave's latents: rows tau = 4g + r, column m = c16
         float p[CT][4];
@@ -266,11 +267,11 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a)
         }
 
         // stage the next block
-        if (n0 + kTB < N) {
+        if (n0 + step < N) {
 #pragma unroll
             for (int kd = 0; kd < KD; ++kd) ka[kd] = kn[kd];
             store_v(buf ^ 1);
-            if (n0 + 2 * kTB < N) load_block(n0 + 2 * kTB, kn);
+            if (n0 + 2 * step < N) load_block(n0 + 2 * step, kn);
         }
         __syncthreads();
 
@@ -315,13 +316,13 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a)
 }
 
 template <typename T>
-hipError_t launch_t(const CausalArgs& a, hipStream_t st)
+hipError_t launch_t(const CausalArgs& a, int step, hipStream_t st)
 {
     dim3 grid(a.B * a.H), block(256);
-    if (a.D == 64 && a.M == 128)      hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 1>), grid, block, 0, st, a);
-    else if (a.D == 64 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 2>), grid, block, 0, st, a);
-    else if (a.D == 32 && a.M == 128) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 1>), grid, block, 0, st, a);
-    else if (a.D == 32 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 2>), grid, block, 0, st, a);
+    if (a.D == 64 && a.M == 128)      hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 1>), grid, block, 0, st, a, step);
+    else if (a.D == 64 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 2>), grid, block, 0, st, a, step);
+    else if (a.D == 32 && a.M == 128) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 1>), grid, block, 0, st, a, step);
+    else if (a.D == 32 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 2>), grid, block, 0, st, a, step);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }
@@ -335,9 +336,9 @@ bool causal_mfma_supported(int dtype, int M, int D)
            causal_lds_bytes(M, D, false) <= 160 * 1024;
 }
 
-hipError_t launch_causal_prefill_mfma(const CausalArgs& a, int dtype, hipStream_t st)
+hipError_t launch_causal_mfma(const CausalArgs& a, int dtype, int step, hipStream_t st)
 {
-    return dtype == 1 ? launch_t<bf16_t>(a, st) : launch_t<f16_t>(a, st);
+    return dtype == 1 ? launch_t<bf16_t>(a, step, st) : launch_t<f16_t>(a, step, st);
 }
 
 }  // namespace flare

@@ -88,7 +88,7 @@ size_t     causal_lds_bytes(int M, int D, bool decode);
 hipError_t launch_causal_prefill(const CausalArgs& a, int dtype, hipStream_t st);
 hipError_t launch_causal_decode(const CausalArgs& a, int dtype, hipStream_t st);
 bool       causal_mfma_supported(int dtype, int M, int D);
-hipError_t launch_causal_prefill_mfma(const CausalArgs& a, int dtype, hipStream_t st);
+hipError_t launch_causal_mfma(const CausalArgs& a, int dtype, int step, hipStream_t st);   // step 16 prefill, 1 decode
 
 hipError_t launch_triple_state(const TripleArgs& a, int dtype, hipStream_t st);
 hipError_t launch_triple_merge(const TripleArgs& a, hipStream_t st);

@@ -281,15 +281,12 @@ def _causal_call(entry, q, k, v, scale, chunk, state):
     d.q_stride, d.k_stride, d.v_stride, d.y_stride = _s3(q4), _s3(k), _s3(v), _s3(y)
     st = C.c_void_p(_stream_ptr(k.device))
     with torch.cuda.device(k.device):
-        if entry == "prefill":
-            need = C.c_size_t(0)
-            _lib.check(lib.flare_causal_workspace_bytes(C.byref(d), C.byref(need)), "flare_causal_workspace_bytes")
-            ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
-            rc = lib.flare_causal_prefill_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(y), _ptr(mu),
-                                              _ptr(den), _ptr(num), _ptr(ws), ws.numel(), st)
-        else:
-            rc = lib.flare_causal_decode_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(y), _ptr(mu),
-                                             _ptr(den), _ptr(num), st)
+        need = C.c_size_t(0)
+        _lib.check(lib.flare_causal_workspace_bytes(C.byref(d), C.byref(need)), "flare_causal_workspace_bytes")
+        ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
+        fn = lib.flare_causal_prefill_fwd if entry == "prefill" else lib.flare_causal_decode_fwd
+        rc = fn(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(y), _ptr(mu), _ptr(den), _ptr(num), _ptr(ws),
+                ws.numel(), st)
     _lib.check(rc, f"flare_causal_{entry}_fwd")
     return y, (mu, den, num)
 

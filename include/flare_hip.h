@@ -145,10 +145,11 @@ int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const v
                              void* workspace, size_t workspace_bytes, void* stream);
 
 /* N recurrent single-token steps in ONE launch (desc->N = number of steps; k, v, y hold
- * the steps along their n axis); the state stays on chip between steps. */
+ * the steps along their n axis); the state stays on chip between steps.  The workspace is
+ * the one flare_causal_workspace_bytes() reports (it may be NULL when that is 0). */
 int flare_causal_decode_fwd(const FlareCausalDesc* desc, const void* q, const void* k,
                             const void* v, void* y, float* mu, float* den, float* num,
-                            void* stream);
+                            void* workspace, size_t workspace_bytes, void* stream);
 
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes);
 
