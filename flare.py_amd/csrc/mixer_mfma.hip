@@ -9,11 +9,12 @@
 // second product: two score tiles give the 8 k-slots of one lane, no cross-lane traffic.
 //
 // Scores are produced in log2 units: scale*log2(e) is folded into the latent queries when
-// they are converted to MFMA operands, and the softmax shift enters as the accumulator
-// input (C = -shift), so the steady state per score is exp2 + pack + dot2 only.  The
-// shift is lazy: it is only required to stay within 2^kLazyLog2 of the running maximum,
-// which is checked from the per-tile sums; a tile that violates it (and every ragged or
-// masked tile) goes through an exact path that recomputes the maximum and rescales.
+// they are converted to MFMA operands, so the steady state per score is exp2 + pack.
+// The optimistic pass uses NO softmax shift: fp32 and bf16/f16-as-accumulated share enough exponent
+// range that exp2(score) is safe while the scores of a row stay inside (-60, +120); the
+// denominators come out of the second product as a row of ones in its A operand and are
+// validated after the pass (2^-60 <= l <= 2^120).  What fails validation (and, in the gather,
+// every masked problem) is recomputed through an exact path with a running maximum.
 //
 //   gather : z = softmax_n(s q k^T) v   split over N, partial (shift, sum, numerator)
 //   scatter: y = softmax_m(s k q^T) z   token parallel, Q and Z^T resident in LDS
@@ -32,7 +33,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr float kLazyLimit = 1024.f;  // 2^10: largest per-tile partial sum the lazy shift accepts
 // range of an unshifted softmax denominator that proves no exponential overflowed or lost
 // the terms that matter to underflow (2^-60 .. 2^120)
 constexpr float kLMin = 8.6736174e-19f, kLMax = 1.329228e36f;
@@ -90,28 +90,14 @@ template <> __device__ __forceinline__ float bits_elem<f16_t>(uint16_t b) { retu
 
 __device__ __forceinline__ u32x4 zero4() { return u32x4{0u, 0u, 0u, 0u}; }
 
-#ifndef FLARE_EXPERIMENT
-#define FLARE_EXPERIMENT 0
-#endif
-__device__ __forceinline__ float xexp2(float x)
-{
-#if FLARE_EXPERIMENT == 1 || FLARE_EXPERIMENT == 6
-    return x * 1.0001f;
-#else
-    return fast_exp2(x);
-#endif
-}
-template <typename M_> __device__ __forceinline__ uint32_t xpack2(float lo, float hi)
-{
-#if FLARE_EXPERIMENT == 3
-    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
-#else
-    return M_::pack2(lo, hi);
-#endif
-}
 
 // 8 elements (16 bytes) from global memory
 __device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+// same, for data that is read once: does not displace reusable lines in the caches
+__device__ __forceinline__ u32x4 load16_stream(const void* p)
+{
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
 
 // multiply 8 packed elements by f (fp32) and repack
 template <typename T> __device__ __forceinline__ u32x4 scale8(u32x4 v, float f)
@@ -137,16 +123,6 @@ __device__ __forceinline__ float xg_sum(float v)
     v += __shfl_xor(v, 16);
     v += __shfl_xor(v, 32);
     return v;
-}
-
-// Scheduling hint: N groups of (1 matrix instruction, 2-3 vector/transcendental instructions).
-template <int N> __device__ __forceinline__ void interleave_mfma_valu()
-{
-    if constexpr (N > 0) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x402, (N & 1) ? 3 : 2, 0);
-        interleave_mfma_valu<N - 1>();
-    }
 }
 
 // =====================================================================================
@@ -232,8 +208,8 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
             const int c = tid + i * 256;
             if (c < TCH) {
                 const int n = min(n0 + c / CH, n_end - 1), ch = c % CH;
-                kr[S][i] = load16(k + (int64_t)n * a.ks[2] + ch * 8);
-                vr[S][i] = load16(v + (int64_t)n * a.vs[2] + ch * 8);
+                kr[S][i] = load16_stream(k + (int64_t)n * a.ks[2] + ch * 8);
+                vr[S][i] = load16_stream(v + (int64_t)n * a.vs[2] + ch * 8);
             }
         }
     };
@@ -326,11 +302,11 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                         float p[8];
     #pragma unroll
                         for (int e = 0; e < 8; ++e) {
-                            p[e] = xexp2(sc[e]);
+                            p[e] = fast_exp2(sc[e]);
                             if (EXACT || RAGGED) p[e] = ok[e] ? p[e] : 0.f;
                         }
-                        const u32x4 pb = {xpack2<M_>(p[0], p[1]), xpack2<M_>(p[2], p[3]),
-                                          xpack2<M_>(p[4], p[5]), xpack2<M_>(p[6], p[7])};
+                        const u32x4 pb = {M_::pack2(p[0], p[1]), M_::pack2(p[2], p[3]),
+                                          M_::pack2(p[4], p[5]), M_::pack2(p[6], p[7])};
     #pragma unroll
                         for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = M_::mma(va[rt], pb, zacc[rt][ct]);
                         lacc[ct] = M_::mma(ones8, pb, lacc[ct]);   // row of ones: the softmax denominator
@@ -343,23 +319,10 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
         auto iter = [&](int n0, auto par) {
             constexpr int P = decltype(par)::value;
             using Other = std::integral_constant<int, 1 - P>;
-#if FLARE_EXPERIMENT == 7
-            // loads only: fold the staged registers into an accumulator, no LDS, no barrier
-#pragma unroll
-            for (int i = 0; i < CPT; ++i)
-                lacc[0] += __builtin_bit_cast(f32x4, kr[1 - P][i]) + __builtin_bit_cast(f32x4, vr[1 - P][i]);
-            if (n0 + 3 * kGTile < n_end) load_tile(Other{}, n0 + 3 * kGTile);
-#elif FLARE_EXPERIMENT == 8
-            // loads + LDS stores + barrier, no LDS reads / compute
-            __syncthreads();
-            if (n0 + kGTile < n_end) store_tile(Other{});
-            if (n0 + 3 * kGTile < n_end) load_tile(Other{}, n0 + 3 * kGTile);
-#else
             __syncthreads();
             if (n0 + kGTile < n_end) store_tile(Other{});
             if (n0 + 3 * kGTile < n_end) load_tile(Other{}, n0 + 3 * kGTile);
             process(n0, P);
-#endif
         };
         if (n_begin < n_end) {
             load_tile(Set0{}, n_begin);
@@ -385,9 +348,6 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
 #pragma unroll
             for (int r = 0; r < 4; ++r) bad = bad || !(fabsf(zacc[rt][ct][r]) <= 3.0e38f);
     }
-#if FLARE_EXPERIMENT != 0
-    bad = false;
-#endif
     if (mask != nullptr) {
         // with a key mask an all-masked range legitimately gives l = 0; small l cannot be told
         // apart from underflow cheaply, so masked problems always take the exact pass
@@ -487,7 +447,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
 #pragma unroll
             for (int kd = 0; kd < KD; ++kd) {
                 const int n = t0 + tw * 16 + c16, ch = kd * 4 + g;
-                dst[tw][kd] = (n < wg_n1 && ch < CH) ? load16(k + (int64_t)n * a.ks[2] + ch * 8) : zero4();
+                dst[tw][kd] = (n < wg_n1 && ch < CH) ? load16_stream(k + (int64_t)n * a.ks[2] + ch * 8) : zero4();
             }
     };
 
@@ -532,27 +492,18 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
 #pragma unroll
                 for (int tw = 0; tw < kSTW; ++tw) {
                     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#if FLARE_EXPERIMENT == 5 || FLARE_EXPERIMENT == 6
-                    s0 = __builtin_bit_cast(f32x4, o0[0]) + __builtin_bit_cast(f32x4, kb[tw][0]);
-                    s1 = __builtin_bit_cast(f32x4, o1[0]) + __builtin_bit_cast(f32x4, kb[tw][0]);
-#else
 #pragma unroll
                     for (int kd = 0; kd < KD; ++kd) {
                         s0 = M_::mma(o0[kd], kb[tw][kd], s0);
                         s1 = M_::mma(o1[kd], kb[tw][kd], s1);
                     }
-#endif
-                    const u32x4 pb = {xpack2<M_>(xexp2(s0[0]), xexp2(s0[1])),
-                                      xpack2<M_>(xexp2(s0[2]), xexp2(s0[3])),
-                                      xpack2<M_>(xexp2(s1[0]), xexp2(s1[1])),
-                                      xpack2<M_>(xexp2(s1[2]), xexp2(s1[3]))};
-#if FLARE_EXPERIMENT == 2 || FLARE_EXPERIMENT == 6
-                    yl[tw] += __builtin_bit_cast(f32x4, pb);
-#else
+                    const u32x4 pb = {M_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])),
+                                      M_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
+                                      M_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])),
+                                      M_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]))};
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = M_::mma(oz[rt], pb, yacc[tw][rt]);
                     yl[tw] = M_::mma(ones8, pb, yl[tw]);   // row of ones: the softmax denominator
-#endif
                 }
             };
             // two operand sets, each loaded from LDS one step before it is used (KS is even or 1
@@ -568,9 +519,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
 #pragma unroll
             for (int tw = 0; tw < kSTW; ++tw) {
                 lrow[tw] = yl[tw][0];
-#if FLARE_EXPERIMENT == 0
                 redo = redo || !(lrow[tw] >= kLMin && lrow[tw] <= kLMax);
-#endif
             }
         }
         if (__builtin_expect(__any(redo), 0)) {
@@ -646,8 +595,10 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                     *reinterpret_cast<uint2*>(yr) = make_uint2(o[0], o[1]);
                 } else {
 #pragma unroll
-                    for (int i = 0; i < RT / 2; ++i)
-                        *reinterpret_cast<u32x4*>(yr + 8 * i) = u32x4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+                    for (int i = 0; i < RT / 2; ++i) {
+                        const u32x4 ov = {o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+                        __builtin_nontemporal_store(ov, reinterpret_cast<u32x4*>(yr + 8 * i));   // written once, never re-read here
+                    }
                 }
             }
         }
@@ -666,7 +617,7 @@ constexpr size_t kScatterLdsMax = 150 * 1024;
 // Workgroups of `kern` the current device holds at once (CUs x occupancy).  Grids are sized
 // to a whole multiple of this so that no partially filled last round is left over.
 // Falls back to 2 per CU on 256 CUs when no device can be queried (host-only planning).
-int resident_slots(const void* kern, size_t dyn_lds)
+int resident_slots(const void* kern, size_t dyn_lds, int block_threads = 256)
 {
     struct Entry { const void* k; size_t lds; int dev; int slots; };
     static Entry cache[64];
@@ -676,7 +627,7 @@ int resident_slots(const void* kern, size_t dyn_lds)
     for (int i = 0; i < ncache; ++i)
         if (cache[i].k == kern && cache[i].lds == dyn_lds && cache[i].dev == dev) return cache[i].slots;
     int occ = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, 256, dyn_lds) != hipSuccess || occ < 1) {
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, block_threads, dyn_lds) != hipSuccess || occ < 1) {
         (void)hipGetLastError();
         return 512;
     }
