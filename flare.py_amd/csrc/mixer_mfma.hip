@@ -112,6 +112,17 @@ template <typename T> __device__ __forceinline__ u32x4 scale8(u32x4 v, float f)
     return o;
 }
 
+// 8 packed elements of type T as 8 packed bf16 (identity for bf16)
+template <typename T> __device__ __forceinline__ u32x4 to_bf16x8(u32x4 v)
+{
+    if constexpr (std::is_same<T, bf16_t>::value) return v;
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        o[i] = Mma<bf16_t>::pack2(bits_elem<T>(uint16_t(v[i] & 0xffffu)), bits_elem<T>(uint16_t(v[i] >> 16)));
+    return o;
+}
+
 __device__ __forceinline__ float xg_max(float v)  // max over the 4 lane groups of a column
 {
     v = fmaxf(v, __shfl_xor(v, 16));
@@ -156,7 +167,8 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
     constexpr int MB = 64 * CT;
     constexpr int ROWB = D * 2;         // bytes per token row
     constexpr int TILEB = kGTile * ROWB;
-    using M_ = Mma<T>;
+    using M_ = Mma<T>;          // score product, in the element type of q and k
+    using P_ = Mma<bf16_t>;     // value product: probabilities (and the values they meet) are always bf16
 
     __shared__ __attribute__((aligned(16))) uint8_t kt[2][TILEB];
     __shared__ __attribute__((aligned(16))) uint8_t vt[2][TILEB];
@@ -184,7 +196,7 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                                              a.scale_log2)
                                  : zero4();
         }
-    const u32x4 ones8 = {M_::kOnes2, M_::kOnes2, M_::kOnes2, M_::kOnes2};
+    const u32x4 ones8 = {P_::kOnes2, P_::kOnes2, P_::kOnes2, P_::kOnes2};
 
     const int n_begin = split * a.tokens_per_split;
     const int n_end = min(a.N, n_begin + a.tokens_per_split);
@@ -221,7 +233,7 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
             if (c < TCH) {
                 const int tok = c / CH, ch = c % CH;
                 *reinterpret_cast<u32x4*>(&kt[S][k_slot(tok, ch)]) = kr[S][i];
-                *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = vr[S][i];
+                *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = to_bf16x8<T>(vr[S][i]);
             }
         }
     };
@@ -305,11 +317,11 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                             p[e] = fast_exp2(sc[e]);
                             if (EXACT || RAGGED) p[e] = ok[e] ? p[e] : 0.f;
                         }
-                        const u32x4 pb = {M_::pack2(p[0], p[1]), M_::pack2(p[2], p[3]),
-                                          M_::pack2(p[4], p[5]), M_::pack2(p[6], p[7])};
+                        const u32x4 pb = {P_::pack2(p[0], p[1]), P_::pack2(p[2], p[3]),
+                                          P_::pack2(p[4], p[5]), P_::pack2(p[6], p[7])};
     #pragma unroll
-                        for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = M_::mma(va[rt], pb, zacc[rt][ct]);
-                        lacc[ct] = M_::mma(ones8, pb, lacc[ct]);   // row of ones: the softmax denominator
+                        for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = P_::mma(va[rt], pb, zacc[rt][ct]);
+                        lacc[ct] = P_::mma(ones8, pb, lacc[ct]);   // row of ones: the softmax denominator
                     }
                 }
     };
@@ -396,7 +408,8 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
     constexpr int KD = (D + 31) / 32;
     constexpr int RT = D / 16;
     constexpr int CH = D / 8;
-    using M_ = Mma<T>;
+    using M_ = Mma<T>;          // score product, in the element type of q and k
+    using P_ = Mma<bf16_t>;     // value product: probabilities (and the values they meet) are always bf16
 
     __shared__ float red[4];
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -430,8 +443,8 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
         for (int e2 = 0; e2 < 4; ++e2) {
             const int e = 2 * e2;
             const int m0 = 32 * ks + (e >> 2) * 16 + 4 * gg + (e & 3);
-            o[e2] = uint32_t(elem_bits<T>(z[(int64_t)m0 * D + d])) |
-                    (uint32_t(elem_bits<T>(z[(int64_t)(m0 + 1) * D + d])) << 16);
+            o[e2] = uint32_t(elem_bits<bf16_t>(z[(int64_t)m0 * D + d])) |
+                    (uint32_t(elem_bits<bf16_t>(z[(int64_t)(m0 + 1) * D + d])) << 16);
         }
         zt[idx] = o;
     }
@@ -451,7 +464,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
             }
     };
 
-    const u32x4 ones8 = {M_::kOnes2, M_::kOnes2, M_::kOnes2, M_::kOnes2};
+    const u32x4 ones8 = {P_::kOnes2, P_::kOnes2, P_::kOnes2, P_::kOnes2};
 
     int t0 = wg_n0 + w * kSTokWave;
     if (t0 < wg_n1) load_k(t0, kb);
@@ -497,13 +510,13 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                         s0 = M_::mma(o0[kd], kb[tw][kd], s0);
                         s1 = M_::mma(o1[kd], kb[tw][kd], s1);
                     }
-                    const u32x4 pb = {M_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])),
-                                      M_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
-                                      M_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])),
-                                      M_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]))};
+                    const u32x4 pb = {P_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])),
+                                      P_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
+                                      P_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])),
+                                      P_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]))};
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = M_::mma(oz[rt], pb, yacc[tw][rt]);
-                    yl[tw] = M_::mma(ones8, pb, yl[tw]);   // row of ones: the softmax denominator
+                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = P_::mma(oz[rt], pb, yacc[tw][rt]);
+                    yl[tw] = P_::mma(ones8, pb, yl[tw]);   // row of ones: the softmax denominator
                 }
             };
             // two operand sets, each loaded from LDS one step before it is used (KS is even or 1
@@ -560,17 +573,17 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                     for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] *= al;
                     lsum[tw] *= al;
                     shift[tw] = nc;
-                    const u32x4 pb = {M_::pack2(fast_exp2(s0[0] - nc), fast_exp2(s0[1] - nc)),
-                                      M_::pack2(fast_exp2(s0[2] - nc), fast_exp2(s0[3] - nc)),
-                                      M_::pack2(fast_exp2(s1[0] - nc), fast_exp2(s1[1] - nc)),
-                                      M_::pack2(fast_exp2(s1[2] - nc), fast_exp2(s1[3] - nc))};
-                    float t = M_::sum2(pb[0], 0.f);
-                    t = M_::sum2(pb[1], t);
-                    t = M_::sum2(pb[2], t);
-                    t = M_::sum2(pb[3], t);
+                    const u32x4 pb = {P_::pack2(fast_exp2(s0[0] - nc), fast_exp2(s0[1] - nc)),
+                                      P_::pack2(fast_exp2(s0[2] - nc), fast_exp2(s0[3] - nc)),
+                                      P_::pack2(fast_exp2(s1[0] - nc), fast_exp2(s1[1] - nc)),
+                                      P_::pack2(fast_exp2(s1[2] - nc), fast_exp2(s1[3] - nc))};
+                    float t = P_::sum2(pb[0], 0.f);
+                    t = P_::sum2(pb[1], t);
+                    t = P_::sum2(pb[2], t);
+                    t = P_::sum2(pb[3], t);
                     lsum[tw] += t;
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = M_::mma(za[rt], pb, yacc[tw][rt]);
+                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = P_::mma(za[rt], pb, yacc[tw][rt]);
                 }
             }
 #pragma unroll

@@ -156,3 +156,16 @@ def test_mfma_prefill_out_of_window_scores_fall_back(dev):
     assert O.rel_l2(y[:, 0], yr[:, 0]) <= 1e-5 * 1e3   # fp32 kernel on bf16 outputs: bf16 output rounding only
     assert O.rel_l2(y[:, 1], yr[:, 1]) <= 2e-2
     state_close(st, str_, 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("offset", [-16.0, 14.0])
+def test_mfma_prefill_constant_score_offset(dev, dtype, offset):
+    # every score carries the same constant; all softmaxes of the recurrence are invariant to it
+    q, k, v = make(1, 2, 300, 128, 32, dtype)
+    q[..., 0] = 4.0
+    k[..., 0] = offset / 4.0
+    y, st = F.flare_causal_prefill(q.to(dev), k.to(dev), v.to(dev))
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float(), 1.0)
+    assert O.rel_l2(y, yr) <= TOL[dtype]
+    state_close(st, str_, TOL[dtype])

@@ -215,3 +215,17 @@ def test_autograd_plumbing(dev):
     yr.square().sum().backward()
     for a, b in ((q, qr), (k, kr), (v, vr)):
         assert O.rel_l2(a.grad, b.grad) < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("offset", [-16.0, 14.0])
+def test_constant_score_offset(dev, dtype, offset):
+    # One feature column makes every score carry the same constant (in natural-log units).  Both
+    # softmaxes are invariant to it, so the oracle result is that of the remaining columns; the
+    # kernels must not lose precision to it whatever the element type (f16 probabilities of
+    # e^-16 would be subnormal, of e^14 infinite).
+    q, k, v = make(1, 2, 3000, 128, 32, dtype)
+    q[..., 0] = 4.0
+    k[..., 0] = offset / 4.0
+    assert F.mixer_kernel_name(q, k, v).startswith("mfma")
+    check(dev, q, k, v)
