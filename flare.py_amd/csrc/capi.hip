@@ -195,6 +195,42 @@ bool causal_wants_mfma(const FlareCausalDesc* d)
            strides_mult8(d->y_stride);
 }
 
+// Matrix-core prefill plan: the token axis is cut into segments that run in parallel (local
+// states first, then the recurrence of each segment from the summed states before it).
+struct CausalPlan { bool mfma; int n_segs, seg_len; size_t off_den, off_num, total; };
+
+CausalPlan plan_causal(const FlareCausalDesc* d)
+{
+    CausalPlan p{};
+    p.mfma = causal_wants_mfma(d);
+    p.n_segs = 1;
+    p.seg_len = d->N;
+    if (!p.mfma) return p;
+    const int64_t BH = (int64_t)d->B * d->H;
+    int64_t seg_len;
+    if (d->chunk > 0) {
+        seg_len = ((int64_t)d->chunk + 15) / 16 * 16;
+    } else {
+        // two workgroups per compute unit (what the kernel's LDS footprint allows on 256 CUs),
+        // segments of at least 256 tokens
+        const int64_t want = std::max<int64_t>(1, (512 + BH - 1) / BH);
+        seg_len = std::max<int64_t>(256, ((d->N + want - 1) / want + 15) / 16 * 16);
+    }
+    int64_t n_segs = (d->N + seg_len - 1) / seg_len;
+    if (n_segs > 64) {
+        seg_len = ((d->N + 63) / 64 + 15) / 16 * 16;
+        n_segs = (d->N + seg_len - 1) / seg_len;
+    }
+    if (n_segs > 1) {
+        p.n_segs = (int)n_segs;
+        p.seg_len = (int)seg_len;
+    }
+    p.off_den = ((size_t)BH * sizeof(int) + 255) / 256 * 256;
+    p.off_num = p.off_den + (p.n_segs > 1 ? (size_t)BH * p.n_segs * d->M * sizeof(float) : 0);
+    p.total = p.off_num + (p.n_segs > 1 ? (size_t)BH * p.n_segs * d->M * d->D * sizeof(float) : 0);
+    return p;
+}
+
 void fill_causal_args(flare::CausalArgs& a, const FlareCausalDesc* d)
 {
     memset(&a, 0, sizeof(a));
@@ -338,7 +374,8 @@ int flare_causal_workspace_bytes(const FlareCausalDesc* desc, size_t* bytes)
     if (!bytes) return fail(FLARE_EINVAL, "bytes is NULL");
     int rc = check_causal_desc(desc);
     if (rc != FLARE_OK) return rc;
-    *bytes = causal_wants_mfma(desc) ? (size_t)desc->B * desc->H * sizeof(int) : 0;
+    const CausalPlan p = plan_causal(desc);
+    *bytes = p.mfma ? p.total : 0;
     return FLARE_OK;
 }
 
@@ -357,11 +394,16 @@ int causal_run(const FlareCausalDesc* desc, bool decode, const void* q, const vo
     if (causal_wants_mfma(desc) && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y)) {
         // matrix-core kernel without a running maximum; it marks the (b,h) it could not validate
         // and the fp32 kernel, launched right behind it, redoes exactly those
-        const size_t need = (size_t)desc->B * desc->H * sizeof(int);
+        const CausalPlan p = plan_causal(desc);
         if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
-        if (workspace_bytes < need)
-            return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, need);
+        if (workspace_bytes < p.total)
+            return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, p.total);
+        if (!aligned16(workspace)) return fail(FLARE_EINVAL, "workspace must be 16-byte aligned");
         a.flags = static_cast<int*>(workspace);
+        a.n_segs = decode ? 1 : p.n_segs;          // decode steps are sequential by nature
+        a.seg_len = decode ? desc->N : p.seg_len;
+        a.seg_den = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p.off_den);
+        a.seg_num = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p.off_num);
         hipError_t e = flare::launch_causal_mfma(a, desc->dtype, decode ? 1 : 16, st);
         if (e != hipSuccess) return hip_status(e, "causal (mfma) launch");
     }

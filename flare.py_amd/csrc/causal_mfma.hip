@@ -81,7 +81,11 @@ __device__ __forceinline__ uint2 tr16(const void* lds_addr)
 
 constexpr int kTB = 16;   // tokens per block
 
-template <typename T, int D, int KM>
+// STATE_ONLY = false: the full recurrence over the workgroup's token segment, from the incoming
+// state plus the local states of all earlier segments (summed in segment order).  A single
+// segment writes the state back itself; with several, the last one stages it in the workspace.
+// STATE_ONLY = true: only the segment's local denominators and numerators (first phase).
+template <typename T, int D, int KM, bool STATE_ONLY>
 __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step)
 {
     constexpr int KD = D / 32;          // k-steps over d of the score product
@@ -101,8 +105,11 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step
     __shared__ int bad_flag;
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
-    const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H;
-    const int N = a.N;
+    const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H, seg = blockIdx.y;
+    const int n_lo = seg * a.seg_len, N = min(a.N, n_lo + a.seg_len);   // this segment: tokens n_lo .. N-1
+    const bool single = a.n_segs == 1;
+    float* seg_den = a.seg_den + ((int64_t)bh * a.n_segs + seg) * M;
+    float* seg_num = a.seg_num + ((int64_t)bh * a.n_segs + seg) * M * D;
     const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
     const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
     const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
@@ -134,7 +141,9 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step
         const float mu = mu_g[m];
         mu0[ct] = mu <= kNegBig ? 0.f : mu * kLog2e;
         negmu[ct] = f32x4{-mu0[ct], -mu0[ct], -mu0[ct], -mu0[ct]};
-        const float d0 = mu <= kNegBig ? 0.f : den_g[m];
+        float d0 = (STATE_ONLY || mu <= kNegBig) ? 0.f : den_g[m];
+        if (!STATE_ONLY)
+            for (int s = 0; s < seg; ++s) d0 += a.seg_den[((int64_t)bh * a.n_segs + s) * M + m];
         den[ct] = f32x4{d0, d0, d0, d0};
     }
     // state numerator U[m, d]: tile (mt, dt) holds rows m0 + 16 mt + 4g + r, column 16 dt + c16
@@ -146,7 +155,11 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = m0 + mt * 16 + 4 * g + r;
-                U[mt][dt][r] = mu_g[m] <= kNegBig ? 0.f : num_g[(int64_t)m * D + dt * 16 + c16];
+                float u = (STATE_ONLY || mu_g[m] <= kNegBig) ? 0.f : num_g[(int64_t)m * D + dt * 16 + c16];
+                if (!STATE_ONLY)
+                    for (int s = 0; s < seg; ++s)
+                        u += a.seg_num[(((int64_t)bh * a.n_segs + s) * M + m) * D + dt * 16 + c16];
+                U[mt][dt][r] = u;
             }
 
     // constant operands: lower-triangular ones L[t = c16][tau = 4g + e] and all ones
@@ -185,14 +198,14 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step
     };
 
     bool bad = false;
-    load_block(0, ka);
+    load_block(n_lo, ka);
     store_v(0);
-    if (step < N) load_block(step, kn);
+    if (n_lo + step < N) load_block(n_lo + step, kn);
     __syncthreads();
 
     int it = 0;
     // step = 16: chunked prefill; step = 1: recurrent decode, one token per block (rows >= tb are masked)
-    for (int n0 = 0; n0 < N; n0 += step, ++it) {
+    for (int n0 = n_lo; n0 < N; n0 += step, ++it) {
         const int buf = it & 1;
         const int tb = min(step, N - n0);
 
@@ -207,6 +220,25 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step
 #pragma unroll
             for (int r = 0; r < 4; ++r) p[ct][r] = (4 * g + r < tb) ? fast_exp2(s[r]) : 0.f;
             ppk[ct] = make_uint2(P_::pack2(p[ct][0], p[ct][1]), P_::pack2(p[ct][2], p[ct][3]));
+        }
+        if constexpr (STATE_ONLY) {
+            uint2 vop[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vop[dt] = tr16(&vs[buf][4 * g + (c16 >> 2)][dt * 16 + (c16 & 3) * 4]);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                den[ct] = P_::mma16(ones4, ppk[ct], den[ct]);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) U[ct][dt] = P_::mma16(ppk[ct], vop[dt], U[ct][dt]);
+            }
+            if (n0 + step < N) {
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) ka[kd] = kn[kd];
+                store_v(buf ^ 1);
+                if (n0 + 2 * step < N) load_block(n0 + 2 * step, kn);
+            }
+            __syncthreads();
+            continue;
         }
         // running denominators: dcum = den + L P ; den += 1 P ; G = P / dcum
 #pragma unroll
@@ -300,39 +332,99 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step
         }
     }
 
-    // validate the final denominators, then publish the state (or the redo flag)
+    if constexpr (STATE_ONLY) {
+        // local state of the segment, relative to the shift of the incoming state; whatever
+        // overflowed or vanished here is caught by the checks of the segments that use it
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) bad = bad || !(den[ct][0] >= kLMin && den[ct][0] <= kLMax);
+        for (int ct = 0; ct < CT; ++ct) {
+            if (g == 0) seg_den[m0 + ct * 16 + c16] = den[ct][0];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) seg_num[(int64_t)(m0 + ct * 16 + 4 * g + r) * D + dt * 16 + c16] = U[ct][dt][r];
+        }
+        return;
+    }
+
+    // validate the final denominators, then publish the state (or the redo flag).  With several
+    // segments the flags were cleared beforehand and are only ever raised; the last segment
+    // stages the state in its workspace slot and a commit kernel copies it once every segment
+    // of the (b,h) has passed.
+    const bool last = seg == a.n_segs - 1;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) bad = bad || (last && !(den[ct][0] >= kLMin && den[ct][0] <= kLMax));
     if (__any(bad) && lane == 0) bad_flag = 1;
     __syncthreads();
     if (bad_flag) {
         if (tid == 0) a.flags[bh] = 1;
         return;
     }
-    if (tid == 0) a.flags[bh] = 0;
+    if (single && tid == 0) a.flags[bh] = 0;
+    if (!last) return;
+    float* den_o = single ? den_g : seg_den;
+    float* num_o = single ? num_g : seg_num;
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         const int m = m0 + ct * 16 + c16;
         if (g == 0) {
-            mu_g[m] = mu0[ct] * kLn2;
-            den_g[m] = den[ct][0];
+            if (single) mu_g[m] = mu0[ct] * kLn2;
+            den_o[m] = den[ct][0];
         }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) num_g[(int64_t)(m0 + ct * 16 + 4 * g + r) * D + dt * 16 + c16] = U[ct][dt][r];
+            for (int r = 0; r < 4; ++r) num_o[(int64_t)(m0 + ct * 16 + 4 * g + r) * D + dt * 16 + c16] = U[ct][dt][r];
     }
+}
+
+// Clears the per-(b,h) redo flags (a kernel rather than a memset so that callers may capture
+// the call in a graph).
+__global__ void causal_clear_flags_kernel(int* flags, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) flags[i] = 0;
+}
+
+// Copies the state staged by the last segment into (mu, den, num) for every (b,h) whose
+// segments all passed validation; a fresh state's shift becomes 0.
+__global__ __launch_bounds__(256) void causal_commit_kernel(CausalArgs a)
+{
+    const int bh = blockIdx.x;
+    if (a.flags[bh] != 0) return;
+    const int M = a.M, D = a.D;
+    const float* sd = a.seg_den + ((int64_t)bh * a.n_segs + a.n_segs - 1) * M;
+    const float* sn = a.seg_num + ((int64_t)bh * a.n_segs + a.n_segs - 1) * M * D;
+    for (int i = threadIdx.x; i < M; i += 256) {
+        const float mu = a.mu[(int64_t)bh * M + i];
+        a.mu[(int64_t)bh * M + i] = mu <= kNegBig ? 0.f : mu;
+        a.den[(int64_t)bh * M + i] = sd[i];
+    }
+    for (int i = threadIdx.x; i < M * D; i += 256) a.num[(int64_t)bh * M * D + i] = sn[i];
+}
+
+template <typename T, bool STATE_ONLY>
+hipError_t launch_phase(const CausalArgs& a, int step, dim3 grid, hipStream_t st)
+{
+    dim3 block(256);
+    if (a.D == 64 && a.M == 128)      hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 1, STATE_ONLY>), grid, block, 0, st, a, step);
+    else if (a.D == 64 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 2, STATE_ONLY>), grid, block, 0, st, a, step);
+    else if (a.D == 32 && a.M == 128) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 1, STATE_ONLY>), grid, block, 0, st, a, step);
+    else if (a.D == 32 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 2, STATE_ONLY>), grid, block, 0, st, a, step);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
 }
 
 template <typename T>
 hipError_t launch_t(const CausalArgs& a, int step, hipStream_t st)
 {
-    dim3 grid(a.B * a.H), block(256);
-    if (a.D == 64 && a.M == 128)      hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 1>), grid, block, 0, st, a, step);
-    else if (a.D == 64 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 2>), grid, block, 0, st, a, step);
-    else if (a.D == 32 && a.M == 128) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 1>), grid, block, 0, st, a, step);
-    else if (a.D == 32 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 2>), grid, block, 0, st, a, step);
-    else return hipErrorInvalidValue;
+    const int BH = a.B * a.H;
+    if (a.n_segs == 1) return launch_phase<T, false>(a, step, dim3(BH, 1), st);
+    hipLaunchKernelGGL(causal_clear_flags_kernel, dim3((BH + 255) / 256), dim3(256), 0, st, a.flags, BH);
+    hipError_t e = launch_phase<T, true>(a, step, dim3(BH, a.n_segs - 1), st);
+    if (e != hipSuccess) return e;
+    e = launch_phase<T, false>(a, step, dim3(BH, a.n_segs), st);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(causal_commit_kernel, dim3(BH), dim3(256), 0, st, a);
     return hipGetLastError();
 }
 

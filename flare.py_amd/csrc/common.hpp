@@ -54,6 +54,8 @@ struct CausalArgs {
     const void* q; const void* k; const void* v; void* y;
     float* mu; float* den; float* num;   // state, natural-log units for mu
     int* flags;                          // [B*H] or null: per-(b,h) "redo with the fp32 kernel" marks
+    float* seg_den; float* seg_num;      // [B*H, n_segs, M] and [B*H, n_segs, M, D]: per-segment states (matrix-core prefill)
+    int n_segs, seg_len;                 // token segments processed in parallel; seg_len is a multiple of 16
     int B, H, N, M, D;
     int chunk;
     float scale;

@@ -291,9 +291,11 @@ def _causal_call(entry, q, k, v, scale, chunk, state):
     return y, (mu, den, num)
 
 
-def flare_causal_prefill(q, k, v, scale: float = 1.0, chunk: int = 256, state=None):
+def flare_causal_prefill(q, k, v, scale: float = 1.0, chunk: int = 0, state=None):
     """Causal FLARE over N tokens: y_t uses keys/values of tokens <= t only.
-    Returns (y [B,H,N,D], state) where state = (mu, den, num) continues the recurrence."""
+    Returns (y [B,H,N,D], state) where state = (mu, den, num) continues the recurrence.
+    `chunk` is the length of the token segments the matrix-core path runs in parallel
+    (0 = chosen from B*H and N); the result depends on it only through rounding."""
     return _causal_call("prefill", q, k, v, scale, chunk, state)
 
 

@@ -169,3 +169,40 @@ def test_mfma_prefill_constant_score_offset(dev, dtype, offset):
     yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float(), 1.0)
     assert O.rel_l2(y, yr) <= TOL[dtype]
     state_close(st, str_, TOL[dtype])
+
+
+def test_mfma_prefill_segment_length_independence(dev):
+    # the matrix-core prefill cuts the tokens into segments that run in parallel; any segment
+    # length (one segment, ragged last segment, many short segments) gives the same result, with
+    # and without an incoming state
+    q, k, v = make(2, 2, 1000, 128, 64, torch.bfloat16, seed=9)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float())
+    _, st0 = F.flare_causal_prefill(qd, kd[:, :, :200], vd[:, :, :200], chunk=1000)
+    for chunk in (0, 16, 48, 256, 400, 1000):
+        y, st = F.flare_causal_prefill(qd, kd, vd, chunk=chunk)
+        y2, st2 = F.flare_causal_prefill(qd, kd, vd, chunk=chunk)
+        assert torch.equal(y, y2) and all(torch.equal(a, b) for a, b in zip(st, st2))   # bit-stable
+        assert O.rel_l2(y, yr) <= 2e-2, chunk
+        state_close(st, str_, 2e-2)
+        yc, stc = F.flare_causal_prefill(qd, kd[:, :, 200:], vd[:, :, 200:], chunk=chunk, state=st0)
+        assert O.rel_l2(yc, yr[:, :, 200:]) <= 2e-2, chunk
+        state_close(stc, str_, 2e-2)
+
+
+def test_mfma_prefill_fallback_from_a_middle_segment(dev):
+    # only the tokens of one middle segment leave the window: the whole (b,h) must be redone by the
+    # fp32 kernel FROM THE INCOMING STATE (which the matrix-core pass must not have touched)
+    q, k, v = make(1, 2, 640, 128, 64, torch.bfloat16, seed=11, std=1.0)
+    k[:, 1] *= 0.05
+    k[:, 0, :256] *= 0.05
+    k[:, 0, 256:384] *= 8.0
+    k[:, 0, 384:] *= 0.05
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    _, st0 = F.flare_causal_prefill(qd, kd[:, :, :100], vd[:, :, :100])
+    y, st = F.flare_causal_prefill(qd, kd[:, :, 100:], vd[:, :, 100:], chunk=128, state=st0)
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float())
+    assert torch.isfinite(y.float()).all()
+    assert O.rel_l2(y[:, 0], yr[:, 0, 100:]) <= 1e-2
+    assert O.rel_l2(y[:, 1], yr[:, 1, 100:]) <= 2e-2
+    state_close(st, str_, 2e-2)
