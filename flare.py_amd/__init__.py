@@ -6,7 +6,9 @@ importable as `flare_py_amd` (a symlink at the repository root).
 """
 from . import _lib
 from .functional import (
+    CausalLinear,
     TripleAttentionFunction,
+    causal_linear_attention,
     causal_fresh_state,
     flare_causal_decode,
     flare_causal_decode_step,
@@ -20,7 +22,7 @@ from .functional import (
 from .modules import FLARE, FLAREBlock, FLAREModel, FinalLayer, ResidualMLP
 
 __all__ = [
-    "FLARE", "FLAREBlock", "FLAREModel", "FinalLayer", "ResidualMLP", "TripleAttentionFunction",
+    "CausalLinear", "causal_linear_attention", "FLARE", "FLAREBlock", "FLAREModel", "FinalLayer", "ResidualMLP", "TripleAttentionFunction",
     "causal_fresh_state", "flare_causal_decode", "flare_causal_decode_step", "flare_causal_prefill",
     "flare_gather", "flare_multihead_mixer", "flare_scatter", "mixer_kernel_name", "triple_attention",
 ]

@@ -38,6 +38,14 @@ class FlareCausalDesc(C.Structure):
     ]
 
 
+class FlareCausalLinearDesc(C.Structure):
+    _fields_ = [
+        ("B", C.c_int32), ("H", C.c_int32), ("N", C.c_int32), ("Dk", C.c_int32), ("Dv", C.c_int32),
+        ("dtype", C.c_int32), ("n_segs", C.c_int32), ("flags", C.c_int32),
+        ("q_stride", I3), ("k_stride", I3), ("v_stride", I3), ("y_stride", I3),
+    ]
+
+
 class FlareTripleDesc(C.Structure):
     _fields_ = [
         ("B", C.c_int32), ("H", C.c_int32), ("N", C.c_int32), ("Dq", C.c_int32), ("Dv", C.c_int32),
@@ -61,6 +69,8 @@ SYMBOLS = {
     "flare_causal_workspace_bytes": (C.c_int, [C.POINTER(FlareCausalDesc), C.POINTER(_SZ)]),
     "flare_causal_prefill_fwd": (C.c_int, [C.POINTER(FlareCausalDesc), _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_causal_decode_fwd": (C.c_int, [C.POINTER(FlareCausalDesc), _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "flare_causal_linear_workspace_bytes": (C.c_int, [C.POINTER(FlareCausalLinearDesc), C.POINTER(_SZ)]),
+    "flare_causal_linear_fwd": (C.c_int, [C.POINTER(FlareCausalLinearDesc), _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_triple_workspace_bytes": (C.c_int, [C.POINTER(FlareTripleDesc), C.POINTER(_SZ)]),
     "flare_triple_state_fwd": (C.c_int, [C.POINTER(FlareTripleDesc), _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_triple_out_fwd": (C.c_int, [C.POINTER(FlareTripleDesc), _P, _P, _P, _P, _P, _P]),

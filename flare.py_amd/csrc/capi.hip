@@ -242,6 +242,42 @@ void fill_causal_args(flare::CausalArgs& a, const FlareCausalDesc* d)
     }
 }
 
+// ---- causal linear --------------------------------------------------------------------
+int check_causal_linear_desc(const FlareCausalLinearDesc* d)
+{
+    if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
+    if (d->B < 1 || d->H < 1 || d->N < 1 || d->Dk < 1 || d->Dv < 1)
+        return fail(FLARE_EINVAL, "B,H,N,Dk,Dv must be >= 1 (got %d,%d,%d,%d,%d)", d->B, d->H, d->N, d->Dk, d->Dv);
+    if (d->dtype < FLARE_DT_F32 || d->dtype > FLARE_DT_F16) return fail(FLARE_EINVAL, "unknown dtype %d", d->dtype);
+    if (d->Dk > 128 || d->Dv > 128) return fail(FLARE_EUNSUPPORTED, "Dk=%d, Dv=%d: at most 128 supported", d->Dk, d->Dv);
+    if (d->n_segs < 0) return fail(FLARE_EINVAL, "n_segs must be >= 0");
+    if ((int64_t)d->B * d->H > 65535) return fail(FLARE_EUNSUPPORTED, "B*H must be <= 65535");
+    const int64_t* ss[4] = {d->q_stride, d->k_stride, d->v_stride, d->y_stride};
+    const int w[4] = {d->Dk, d->Dk, d->Dv, d->Dv};
+    const char* nm[4] = {"q", "k", "v", "y"};
+    for (int t = 0; t < 4; ++t)
+        if (ss[t][2] < w[t]) return fail(FLARE_EINVAL, "%s row stride %lld < row width %d", nm[t], (long long)ss[t][2], w[t]);
+    return FLARE_OK;
+}
+
+struct CausalLinearPlan { int n_segs, seg_len; size_t total; };
+
+CausalLinearPlan plan_causal_linear(const FlareCausalLinearDesc* d)
+{
+    const int tile = flare::causal_linear_tile();
+    const int64_t BH = (int64_t)d->B * d->H;
+    const int64_t tiles = ((int64_t)d->N + tile - 1) / tile;
+    // automatic: about four workgroups per compute unit (256 CUs), never more segments than tiles
+    int64_t want = d->n_segs > 0 ? d->n_segs : std::max<int64_t>(1, (1024 + BH - 1) / BH);
+    want = std::min<int64_t>(std::min<int64_t>(want, tiles), 4096);
+    const int64_t tiles_per_seg = (tiles + want - 1) / want;
+    CausalLinearPlan p;
+    p.seg_len = (int)(tiles_per_seg * tile);
+    p.n_segs = (int)((tiles + tiles_per_seg - 1) / tiles_per_seg);
+    p.total = (size_t)BH * p.n_segs * d->Dk * d->Dv * sizeof(float);
+    return p;
+}
+
 // ---- triple ---------------------------------------------------------------------------
 int check_triple_desc(const FlareTripleDesc* d)
 {
@@ -424,6 +460,39 @@ int flare_causal_decode_fwd(const FlareCausalDesc* desc, const void* q, const vo
                             size_t workspace_bytes, void* stream)
 {
     return causal_run(desc, true, q, k, v, y, mu, den, num, workspace, workspace_bytes, stream);
+}
+
+int flare_causal_linear_workspace_bytes(const FlareCausalLinearDesc* desc, size_t* bytes)
+{
+    if (!bytes) return fail(FLARE_EINVAL, "bytes is NULL");
+    int rc = check_causal_linear_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    *bytes = plan_causal_linear(desc).total;
+    return FLARE_OK;
+}
+
+int flare_causal_linear_fwd(const FlareCausalLinearDesc* desc, const void* q, const void* k, const void* v,
+                            void* y, void* workspace, size_t workspace_bytes, void* stream)
+{
+    int rc = check_causal_linear_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !v || !y) return fail(FLARE_EINVAL, "q, k, v, y must not be NULL");
+    const CausalLinearPlan p = plan_causal_linear(desc);
+    if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
+    if (workspace_bytes < p.total)
+        return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, p.total);
+    if (reinterpret_cast<uintptr_t>(workspace) % 4) return fail(FLARE_EINVAL, "workspace must be 4-byte aligned");
+    flare::CausalLinearArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = q; a.k = k; a.v = v; a.y = y;
+    a.states = static_cast<float*>(workspace);
+    a.B = desc->B; a.H = desc->H; a.N = desc->N; a.Dk = desc->Dk; a.Dv = desc->Dv;
+    a.n_segs = p.n_segs; a.seg_len = p.seg_len;
+    a.inv_n = 1.0f / (float)desc->N;
+    for (int i = 0; i < 3; ++i) {
+        a.qs[i] = desc->q_stride[i]; a.ks[i] = desc->k_stride[i]; a.vs[i] = desc->v_stride[i]; a.ys[i] = desc->y_stride[i];
+    }
+    return hip_status(flare::launch_causal_linear(a, desc->dtype, static_cast<hipStream_t>(stream)), "causal linear launch");
 }
 
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes)

@@ -74,6 +74,15 @@ struct TripleArgs {
     int64_t q1s[3], q2s[3], k1s[3], k2s[3], vs[3], os[3];
 };
 
+struct CausalLinearArgs {
+    const void* q; const void* k; const void* v; void* y;
+    float* states;     // [B*H, n_segs, Dk, Dv] segment states (workspace)
+    int B, H, N, Dk, Dv;
+    int n_segs, seg_len;   // seg_len is a multiple of the 64-token tile
+    float inv_n;           // 1 / N
+    int64_t qs[3], ks[3], vs[3], ys[3];
+};
+
 // ---- launchers implemented in the .hip files -------------------------------------------
 hipError_t launch_gather_generic(const MixerArgs& a, int dtype, hipStream_t st);
 hipError_t launch_gather_merge(const MixerArgs& a, hipStream_t st);
@@ -91,6 +100,9 @@ hipError_t launch_causal_prefill(const CausalArgs& a, int dtype, hipStream_t st)
 hipError_t launch_causal_decode(const CausalArgs& a, int dtype, hipStream_t st);
 bool       causal_mfma_supported(int dtype, int M, int D);
 hipError_t launch_causal_mfma(const CausalArgs& a, int dtype, int step, hipStream_t st);   // step 16 prefill, 1 decode
+
+int        causal_linear_tile();
+hipError_t launch_causal_linear(const CausalLinearArgs& a, int dtype, hipStream_t st);
 
 hipError_t launch_triple_state(const TripleArgs& a, int dtype, hipStream_t st);
 hipError_t launch_triple_merge(const TripleArgs& a, hipStream_t st);

@@ -314,6 +314,85 @@ def flare_causal_decode_step(q, k_t, v_t, state, scale: float = 1.0):
 
 
 # --------------------------------------------------------------------------------------
+# causal linear attention
+# --------------------------------------------------------------------------------------
+def _causal_linear_forward(q, k, v, n_segs: int = 0):
+    _require_cuda(q, k, v)
+    lib = _lib.load()
+    if q.dim() != 4 or q.shape != k.shape:
+        raise ValueError(f"Q, K must have the same shape [B,H,N,Dk]. Got Q.shape={tuple(q.shape)}, K.shape={tuple(k.shape)}")
+    B, H, N, Dk = q.shape
+    if v.dim() != 4 or v.shape[:3] != (B, H, N):
+        raise ValueError(f"V must have shape ({B}, {H}, {N}, Dv). Got V.shape={tuple(v.shape)}")
+    if not (q.dtype == k.dtype == v.dtype):
+        raise ValueError("Q, K, V must share one dtype")
+    Dv = v.shape[-1]
+    q, k, v = _rows_last_contig(q), _rows_last_contig(k), _rows_last_contig(v)
+    y = torch.empty((B, H, N, Dv), dtype=q.dtype, device=q.device)
+    d = _lib.FlareCausalLinearDesc()
+    d.B, d.H, d.N, d.Dk, d.Dv = B, H, N, Dk, Dv
+    d.dtype = _dtype_code(q)
+    d.n_segs = int(n_segs)
+    d.q_stride, d.k_stride, d.v_stride, d.y_stride = _s3(q), _s3(k), _s3(v), _s3(y)
+    with torch.cuda.device(q.device):
+        need = C.c_size_t(0)
+        _lib.check(lib.flare_causal_linear_workspace_bytes(C.byref(d), C.byref(need)),
+                   "flare_causal_linear_workspace_bytes")
+        ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=q.device)
+        rc = lib.flare_causal_linear_fwd(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(y), _ptr(ws), ws.numel(),
+                                         C.c_void_p(_stream_ptr(q.device)))
+    _lib.check(rc, "flare_causal_linear_fwd")
+    return y
+
+
+def _causal_linear_torch(q, k, v):
+    # differentiable restatement used for the backward pass only: tril(Q K^T) V / N per 128-token
+    # chunk plus the running state, in fp32
+    B, H, N, Dk = q.shape
+    qf, kf, vf = q.float(), k.float(), v.float()
+    S = qf.new_zeros(B, H, Dk, v.shape[-1])
+    out = []
+    for n0 in range(0, N, 128):
+        qc, kc, vc = qf[:, :, n0:n0 + 128], kf[:, :, n0:n0 + 128], vf[:, :, n0:n0 + 128]
+        a = torch.tril(qc @ kc.mT)
+        out.append(qc @ S + a @ vc)
+        S = S + kc.mT @ vc
+    return (torch.cat(out, 2) / N).to(q.dtype)
+
+
+class _CausalLinearFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v):
+        ctx.save_for_backward(q, k, v)
+        return _causal_linear_forward(q, k, v)
+
+    @staticmethod
+    def backward(ctx, gy):
+        q, k, v = ctx.saved_tensors
+        with torch.enable_grad():
+            qq, kk, vv = (t.detach().requires_grad_(True) for t in (q, k, v))
+            y = _causal_linear_torch(qq, kk, vv)
+            return torch.autograd.grad(y, (qq, kk, vv), gy)
+
+
+def causal_linear_attention(q, k, v, n_segs: int = 0):
+    """y_t = (1/N) sum_{tau<=t} <q_t,k_tau> v_tau for q,k [B,H,N,Dk], v [B,H,N,Dv] -> [B,H,N,Dv]
+    (lra/models/triton/causal_linear.py:317-336).  n_segs = token segments run in parallel (0 = auto)."""
+    if n_segs == 0 and torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+        return _CausalLinearFn.apply(q, k, v)
+    return _causal_linear_forward(q, k, v, n_segs)
+
+
+class CausalLinear:
+    """Call-compatible stand-in for lra/models/triton/causal_linear.py:23 `CausalLinear`:
+    `CausalLinear.apply(Q, K, V) -> Y`.  The HIP kernels need no N % 64 == 0."""
+
+    @staticmethod
+    def apply(Q, K, V):
+        return causal_linear_attention(Q, K, V)
+
+
+# --------------------------------------------------------------------------------------
 # triple attention
 # --------------------------------------------------------------------------------------
 def _triple_forward(q1, q2, k1, k2, v, feature_map: bool, normalize: bool, n_splits: int = 0):

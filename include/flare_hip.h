@@ -18,6 +18,8 @@
  *   flare_causal_decode_fwd    reference holds no code for it) following the 3-phase chunk
  *                              scheme of lra/models/triton/causal_linear.py:81-137 and the
  *                              token recurrence of causal_linear.py:317-336
+ *   flare_causal_linear_fwd    CausalLinear.apply lra/models/triton/causal_linear.py:23-145
+ *                              == linear_causal_reference causal_linear.py:317-336
  *   flare_triple_fwd           TripleAttentionFunction.apply lra/models/triton/triple.py:29-121
  *                              == TripleAttention.attn_einsum lra/models/backends.py:1285-1292
  */
@@ -110,6 +112,19 @@ typedef struct FlareTripleDesc {
     int64_t q1_stride[3], q2_stride[3], k1_stride[3], k2_stride[3], v_stride[3], o_stride[3];
 } FlareTripleDesc;
 
+/*
+ * Causal linear attention.  q, k [B,H,N,Dk], v, y [B,H,N,Dv] (Dk, Dv <= 128):
+ *   y_t = (1/N) sum_{tau <= t} <q_t, k_tau> v_tau
+ * (k and v each carry the reference's N^-1/2).  fp32 arithmetic whatever the element type.
+ */
+typedef struct FlareCausalLinearDesc {
+    int32_t B, H, N, Dk, Dv;
+    int32_t dtype;
+    int32_t n_segs;       /* token segments processed in parallel; 0 = automatic          */
+    int32_t flags;
+    int64_t q_stride[3], k_stride[3], v_stride[3], y_stride[3];
+} FlareCausalLinearDesc;
+
 int         flare_abi_version(void);
 const char* flare_last_error_string(void);
 
@@ -150,6 +165,13 @@ int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const v
 int flare_causal_decode_fwd(const FlareCausalDesc* desc, const void* q, const void* k,
                             const void* v, void* y, float* mu, float* den, float* num,
                             void* workspace, size_t workspace_bytes, void* stream);
+
+int flare_causal_linear_workspace_bytes(const FlareCausalLinearDesc* desc, size_t* bytes);
+
+/* Segment states, exclusive prefix over the segments, then the outputs; sums in a fixed order. */
+int flare_causal_linear_fwd(const FlareCausalLinearDesc* desc, const void* q, const void* k,
+                            const void* v, void* y, void* workspace, size_t workspace_bytes,
+                            void* stream);
 
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes);
 

@@ -23,6 +23,9 @@ function (paths relative to the reference tree):
                         lra/models/triton/causal_linear.py:317-336; causal_bruteforce applies
                         mixer_explicit to every prefix and keeps the last row.
 
+  causal_linear_*       lra/models/triton/causal_linear.py:317-336 (token recurrence, k and v
+                        each scaled by N^-1/2) and :338-389 (chunked form)
+
 Pinning status (what each function is checked against in tests/test_oracle.py):
   mixer_sdpa / mixer_explicit : each other (independent code paths: torch's SDPA kernel vs
       explicit softmax), the C restatement oracle/flare_oracle.c, closed forms (q=0 => mean,
@@ -33,6 +36,8 @@ Pinning status (what each function is checked against in tests/test_oracle.py):
       independence; C restatement.
   triple_einsum               : hand cases (N=1, D=1), pure-Python loops, linearity in v,
       (k1,q1)<->(k2,q2) symmetry; C restatement.
+  causal_linear_recurrent     : the closed form tril(Q K^T) V / N, the chunked form for several
+      chunk sizes, a pure-Python-float brute force, last row == non-causal linear attention.
 """
 from __future__ import annotations
 
@@ -172,6 +177,60 @@ def causal_bruteforce(q, k, v, scale=1.0, dtype=torch.float64):
 def causal_state_invariants(mu, den, num):
     """The shift-invariant content of a state: z = num/den and lse = mu + log den."""
     return num / den.unsqueeze(-1), mu + torch.log(den)
+
+
+# --------------------------------------------------------------------------------------
+# causal linear attention
+# --------------------------------------------------------------------------------------
+def causal_linear_recurrent(q, k, v, dtype=torch.float64):
+    """Token recurrence of lra/models/triton/causal_linear.py:317-336:
+    S += (v_t N^-1/2)(k_t N^-1/2)^T ;  y_t = S q_t."""
+    B, H, N, Dk = k.shape
+    Dv = v.shape[-1]
+    scale = N ** -0.5
+    q, k, v = q.to(dtype), k.to(dtype) * scale, v.to(dtype) * scale
+    S = torch.zeros(B, H, Dv, Dk, dtype=dtype)
+    y = torch.zeros(B, H, N, Dv, dtype=dtype)
+    for t in range(N):
+        S = S + v[:, :, t, :, None] * k[:, :, t, None, :]
+        y[:, :, t] = (S @ q[:, :, t, :, None])[..., 0]
+    return y
+
+
+def causal_linear_closed_form(q, k, v, dtype=torch.float64):
+    """y = tril(Q K^T) V / N  (the definition the recurrence unrolls to)."""
+    N = k.shape[2]
+    a = torch.tril(q.to(dtype) @ k.to(dtype).mT)
+    return a @ v.to(dtype) / N
+
+
+def causal_linear_chunked(q, k, v, chunk=128, dtype=torch.float64):
+    """Chunked form of lra/models/triton/causal_linear.py:338-389: exclusive prefix of the
+    per-chunk states for the inter-chunk term, masked Q K^T for the intra-chunk term."""
+    B, H, N, Dk = k.shape
+    scale = N ** -0.5
+    q, k, v = q.to(dtype), k.to(dtype) * scale, v.to(dtype) * scale
+    out = []
+    S = torch.zeros(B, H, Dk, v.shape[-1], dtype=dtype)
+    for n0 in range(0, N, chunk):
+        qc, kc, vc = q[:, :, n0:n0 + chunk], k[:, :, n0:n0 + chunk], v[:, :, n0:n0 + chunk]
+        out.append(qc @ S + torch.tril(qc @ kc.mT) @ vc)
+        S = S + kc.mT @ vc
+    return torch.cat(out, 2)
+
+
+def causal_linear_bruteforce_py(q, k, v):
+    """Pure-Python floats, one (b,h): q,k [N][Dk], v [N][Dv] nested lists."""
+    N = len(k)
+    y = []
+    for t in range(N):
+        row = [0.0] * len(v[0])
+        for tau in range(t + 1):
+            s = sum(a * b for a, b in zip(q[t], k[tau]))
+            for j in range(len(row)):
+                row[j] += s * v[tau][j] / N
+        y.append(row)
+    return y
 
 
 # --------------------------------------------------------------------------------------

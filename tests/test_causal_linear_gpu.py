@@ -1,0 +1,79 @@
+"""GPU parity of causal linear attention (CausalLinear.apply) vs the CPU oracle.
+
+The oracle is the token recurrence of lra/models/triton/causal_linear.py:317-336, pinned in
+tests/test_oracle.py by the closed form tril(QK^T)V/N.  Tolerances: 1e-5 (fp32) and 2e-2 (bf16/f16)
+relative L2 on the same rounded inputs (the reference's own self-test uses allclose 1e-5 / 1e-3,
+causal_linear.py:455-457).
+"""
+import pytest
+import torch
+
+import flare_py_amd as F
+from oracle import flare_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2, torch.float16: 2e-2}
+
+
+def make(B, H, N, Dk, Dv, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(B, H, N, Dk, generator=g).to(dtype), torch.randn(B, H, N, Dk, generator=g).to(dtype),
+            torch.randn(B, H, N, Dv, generator=g).to(dtype))
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1, 1), (2, 3, 37, 5, 3), (1, 2, 64, 16, 16), (1, 2, 65, 16, 8),
+                                   (2, 2, 300, 24, 40), (1, 2, 1000, 128, 128), (1, 1, 513, 100, 7)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_shapes_vs_recurrence(dev, shape, dtype):
+    q, k, v = make(*shape, dtype)
+    y = F.CausalLinear.apply(q.to(dev), k.to(dev), v.to(dev))
+    yr = O.causal_linear_closed_form(q, k, v)
+    assert y.dtype == dtype and y.shape == v.shape
+    assert O.rel_l2(y, yr) <= TOL[dtype]
+
+
+def test_reference_selftest_shape_fp32(dev):
+    # the shape of the reference's own test: B=1, H=8, N=2048, Dk=128, Dv=32, fp32 (causal_linear.py:650)
+    q, k, v = make(1, 8, 2048, 128, 32, torch.float32, seed=1)
+    y = F.CausalLinear.apply(q.to(dev), k.to(dev), v.to(dev))
+    yr = O.causal_linear_recurrent(q[:, :2], k[:, :2], v[:, :2])      # token loop on two heads
+    assert O.rel_l2(y[:, :2], yr) <= 1e-5
+    assert O.rel_l2(y, O.causal_linear_closed_form(q, k, v)) <= 1e-5
+    assert torch.allclose(y.cpu().double(), O.causal_linear_closed_form(q, k, v), atol=1e-5, rtol=1e-5)
+
+
+def test_segment_count_independence_and_determinism(dev):
+    q, k, v = make(1, 2, 1500, 32, 32, torch.float32, seed=2)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    yr = O.causal_linear_closed_form(q, k, v)
+    for s in (1, 2, 5, 24, 1000):
+        y = F.causal_linear_attention(qd, kd, vd, n_segs=s)
+        assert torch.equal(y, F.causal_linear_attention(qd, kd, vd, n_segs=s))
+        assert O.rel_l2(y, yr) <= 1e-5, s
+
+
+def test_last_row_is_noncausal_linear_attention_and_strided_views(dev):
+    B, H, N, D = 2, 4, 200, 16
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3, B, N, H * D, generator=g).to(dev)
+    q, k, v = (t.view(B, N, H, D).permute(0, 2, 1, 3) for t in x)     # 'b n (h d) -> b h n d' views, no copy
+    y = F.causal_linear_attention(q, k, v)
+    full = q[:, :, -1:].double() @ (k.double().mT @ v.double()) / N
+    assert O.rel_l2(y[:, :, -1:], full.cpu()) <= 1e-5
+    assert O.rel_l2(y, O.causal_linear_closed_form(q.cpu(), k.cpu(), v.cpu())) <= 1e-5
+
+
+def test_errors_and_autograd_plumbing(dev):
+    q, k, v = make(1, 1, 32, 8, 8, torch.float32)
+    with pytest.raises(ValueError):
+        F.CausalLinear.apply(q.to(dev), k[:, :, :16].to(dev), v.to(dev))
+    with pytest.raises(NotImplementedError):
+        F.CausalLinear.apply(torch.zeros(1, 1, 8, 200, device=dev), torch.zeros(1, 1, 8, 200, device=dev),
+                             torch.zeros(1, 1, 8, 4, device=dev))
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    y = F.CausalLinear.apply(qd, kd, vd)
+    y.square().sum().backward()
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    O.causal_linear_closed_form(qr, kr, vr).square().sum().backward()
+    for a, b in ((qd, qr), (kd, kr), (vd, vr)):
+        assert O.rel_l2(a.grad, b.grad) <= 1e-4

@@ -221,3 +221,25 @@ def test_triple_invariants():
     st1, o1 = O.triple_einsum(*a, dtype=torch.float64)
     ref = (a[0] * a[2]).sum(-1, keepdim=True) * (a[1] * a[3]).sum(-1, keepdim=True) * a[4]
     assert torch.allclose(o1, ref, atol=1e-12)
+
+
+# ---- causal linear attention ------------------------------------------------------------
+def test_causal_linear_oracle_is_pinned():
+    g = torch.Generator().manual_seed(3)
+    q, k = torch.randn(2, 2, 70, 6, generator=g, dtype=torch.float64), torch.randn(2, 2, 70, 6, generator=g, dtype=torch.float64)
+    v = torch.randn(2, 2, 70, 5, generator=g, dtype=torch.float64)
+    yr = O.causal_linear_recurrent(q, k, v)
+    assert O.rel_l2(yr, O.causal_linear_closed_form(q, k, v)) < 1e-12
+    for c in (1, 7, 64, 70, 128):
+        assert O.rel_l2(O.causal_linear_chunked(q, k, v, chunk=c), yr) < 1e-12
+    # last token sees every key: equals non-causal linear attention  Q (K^T V) / N
+    full = q[:, :, -1:] @ (k.mT @ v) / 70
+    assert O.rel_l2(yr[:, :, -1:], full) < 1e-12
+    # pure-Python floats on one (b,h)
+    bp = O.causal_linear_bruteforce_py(q[0, 1, :9].tolist(), k[0, 1, :9].tolist(), v[0, 1, :9].tolist())
+    y9 = O.causal_linear_recurrent(q[:1, 1:2, :9], k[:1, 1:2, :9], v[:1, 1:2, :9])
+    assert O.rel_l2(torch.tensor(bp, dtype=torch.float64), y9[0, 0]) < 1e-12
+    # a hand case: N=2, Dk=Dv=1: y0 = q0 k0 v0 / 2, y1 = q1 (k0 v0 + k1 v1) / 2
+    q2 = torch.tensor([[[[2.0], [3.0]]]]); k2 = torch.tensor([[[[5.0], [7.0]]]]); v2 = torch.tensor([[[[11.0], [13.0]]]])
+    y2 = O.causal_linear_recurrent(q2, k2, v2)
+    assert torch.allclose(y2.flatten(), torch.tensor([2 * 5 * 11 / 2, 3 * (5 * 11 + 7 * 13) / 2], dtype=torch.float64))
