@@ -1,13 +1,18 @@
 #!/usr/bin/env python3
 """Benchmark of the FLARE mixer forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block]
 
 One step = one forward of the mixer (split-N gather, merge, scatter) over the headline workload
 B=1, H=8, N=1,048,576, M=256, D=32, bf16 in / fp32 accumulate, inputs resident in HBM.
 Prints ONE JSON line: tokens/s, the roofline of the dominant kernel (measured with HIP events
 on the launch stream), and the CPU baseline (torch SDPA, MATH backend, fp32) timed on this
 machine's host cores on a bounded sample of the same workload.
+
+--workload selects one of the other configurations instead (same JSON shape, one line): causal =
+causal FLARE prefill of 8192 tokens + 256 decode steps at B=8,H=16,M=128,D=64; triple = triple
+attention at B=4,H=8,N=16384,D=16 (elu+1, normalised); block = one FLAREBlock forward at
+B=4,N=65536,C=128,H=8,M=128 under bf16 autocast (torch layers around the HIP mixer).
 """
 from __future__ import annotations
 
@@ -75,6 +80,126 @@ def cpu_baseline(q, k, v, n_sample):
     return torch.cat(outs, dim=1), dt
 
 
+def wall_ms(fn, steps, warmup):
+    """Wall-clock ms per call between device synchronisations."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def base_record(args, metric, value, unit, ms_step, workload, extra_cfg=None):
+    cfg = {"workload": workload, "seed": 0}
+    cfg.update(extra_cfg or {})
+    return {"metric": metric, "value": round(value, 1), "unit": unit, "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic", "config": cfg}
+
+
+def bench_causal(args, F, dev):
+    """BASELINE config 4: prefill of 8192 tokens, then 256 recurrent decode steps."""
+    from oracle import flare_oracle as O
+
+    B, H, D, M, NP, ND = 8, 16, 64, 128, 8192, 256
+    g = torch.Generator(device=dev).manual_seed(0)
+    std = D ** -0.25                      # "N(0, 1/sqrt(D))" read as variance 1/sqrt(D)
+    q = (torch.randn(H, M, D, generator=g, device=dev) * std).bfloat16()
+    k = (torch.randn(B, H, NP + ND, D, generator=g, device=dev) * std).bfloat16()
+    v = (torch.randn(B, H, NP + ND, D, generator=g, device=dev) * std).bfloat16()
+    kp, vp, kd, vd = (t.contiguous() for t in (k[:, :, :NP], v[:, :, :NP], k[:, :, NP:], v[:, :, NP:]))
+    _, st = F.flare_causal_prefill(q, kp, vp)
+    ms_step = wall_ms(lambda: F.flare_causal_decode(q, kd, vd, F.flare_causal_prefill(q, kp, vp)[1]),
+                      args.steps, args.warmup)
+    ms_prefill = time_events(lambda: F.flare_causal_prefill(q, kp, vp), args.steps, 2)
+    ms_decode = time_events(lambda: F.flare_causal_decode(q, kd, vd, st), args.steps, 2)
+    bytes_prefill = 3 * B * H * NP * D * 2      # K, V read, Y written
+    achieved = bytes_prefill / (ms_prefill * 1e-3) / 1e9
+    out = base_record(args, "causal FLARE prefill+decode tokens/sec at B=8,H=16,N=8192+256,M=128,D=64 bf16",
+                      B * (NP + ND) / (ms_step * 1e-3), "tokens/s", ms_step,
+                      "causal FLARE: prefill 8192 tokens then 256 decode steps, B=8,H=16,M=128,D=64 (BASELINE config 4)",
+                      {"input_std": "D^-1/4 (variance 1/sqrt(D))"})
+    out["roofline"] = {"bound": "hbm", "kernel": "causal_mfma_kernel (prefill)", "achieved": round(achieved, 1),
+                       "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                       "traffic": None, "algorithmic_bytes": bytes_prefill, "ms_prefill": round(ms_prefill, 4),
+                       "ms_decode_256_steps": round(ms_decode, 4), "us_per_decode_step": round(ms_decode / ND * 1e3, 3)}
+    if not args.no_cpu:
+        # the recurrence of the oracle on the first batch element (all heads) over the whole prompt
+        ns = NP
+        qc, kc, vc = q.float().cpu(), kp[:1].float().cpu(), vp[:1].float().cpu()
+        t0 = time.perf_counter()
+        yr, _ = O.causal_recurrent(qc, kc, vc, dtype=torch.float32)
+        dt = time.perf_counter() - t0
+        yg, _ = F.flare_causal_prefill(q, kp[:1].contiguous(), vp[:1].contiguous())
+        out["cpu_baseline"] = {"value": round(B * ns / (dt * B), 1), "unit": "tokens/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": f"token recurrence (torch, fp32) on batch element 0 of {B}, all {H} heads, "
+                               f"{ns} prompt tokens, {dt:.2f} s; value scaled to the {B} batch elements"}
+        out["rel_l2_vs_cpu_on_sample"] = O.rel_l2(yg, yr)
+    return out
+
+
+def bench_triple(args, F, dev):
+    """BASELINE config 5: triple attention, elu+1 feature map, normalised."""
+    from oracle import flare_oracle as O
+
+    B, H, N, D = 4, 8, 16384, 16
+    g = torch.Generator(device=dev).manual_seed(0)
+    a = [(torch.randn(B, H, N, D, generator=g, device=dev) * 0.25).bfloat16() for _ in range(5)]
+    step = lambda: F.triple_attention(*a, normalize=True, feature_map="elu")
+    ms_step = wall_ms(step, args.steps, args.warmup)
+    ms_ev = time_events(step, args.steps, 2)
+    nbytes = 6 * B * H * N * D * 2
+    achieved = nbytes / (ms_ev * 1e-3) / 1e9
+    out = base_record(args, "triple attention tokens/sec at B=4,H=8,N=16384,D=16 bf16", B * N / (ms_step * 1e-3),
+                      "tokens/s", ms_step, "triple attention, elu+1, normalised, B=4,H=8,N=16384,D=16 (BASELINE config 5)")
+    out["roofline"] = {"bound": "hbm", "kernel": "triple_state_mfma_kernel + triple_out_mfma_kernel",
+                       "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                       "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "algorithmic_bytes": nbytes,
+                       "ms_events": round(ms_ev, 4)}
+    if not args.no_cpu:
+        c = [t.float().cpu() for t in a]
+        t0 = time.perf_counter()
+        _, o_ref = O.triple_einsum(*c, feature_map=True, normalize=True)
+        dt = time.perf_counter() - t0
+        _, o = step()
+        out["cpu_baseline"] = {"value": round(B * N / dt, 1), "unit": "tokens/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"einsum restatement (torch, fp32) of the whole workload, {dt:.2f} s"}
+        out["rel_l2_vs_cpu_on_sample"] = O.rel_l2(o, o_ref)
+    return out
+
+
+def bench_block(args, F, dev):
+    """BASELINE config 2: one FLAREBlock forward (LayerNorm, k/v ResidualMLPs, HIP mixer, out_proj, FFN)."""
+    torch.manual_seed(0)
+    blk = F.FLAREBlock(channel_dim=128, num_heads=8, num_latents=128).to(dev).eval()
+    for m in blk.modules():
+        if isinstance(m, torch.nn.Linear):
+            torch.nn.init.xavier_uniform_(m.weight)
+            torch.nn.init.zeros_(m.bias)
+    x = torch.randn(4, 65536, 128, device=dev)
+    def step():
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+            return blk(x)
+    ms_step = wall_ms(step, args.steps, args.warmup)
+    kk = torch.randn(4, 65536, 128, device=dev).bfloat16().view(4, 65536, 8, 16).permute(0, 2, 1, 3)
+    qq = (torch.randn(8, 128, 16, device=dev) * 0.25).bfloat16()
+    ms_mixer = time_events(lambda: F.flare_multihead_mixer(qq, kk, kk), args.steps, 2)
+    nbytes = 4 * 4 * 8 * 65536 * 16 * 2
+    out = base_record(args, "FLAREBlock forward tokens/sec at B=4,N=65536,C=128,H=8,M=128 bf16",
+                      4 * 65536 / (ms_step * 1e-3), "tokens/s", ms_step,
+                      "FLAREBlock forward, bf16 autocast, B=4,N=65536,C=128,H=8,D=16,M=128 (BASELINE config 2)")
+    achieved = nbytes / (ms_mixer * 1e-3) / 1e9
+    out["roofline"] = {"bound": "hbm", "kernel": "mixer (gather + merge + scatter) inside the block",
+                       "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                       "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "algorithmic_bytes": nbytes,
+                       "ms_mixer": round(ms_mixer, 4), "ms_block": round(ms_step, 4)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -82,6 +207,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-sample", type=int, default=1048576, help="tokens of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block"], default="mixer",
+                    help="mixer = the headline configuration (default); the others are BASELINE configs 4, 5, 2")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this build has no multi-GPU path (run with --gpus 1)",
@@ -94,6 +221,10 @@ def main():
     import flare_py_amd as F
 
     dev = torch.device("cuda:0")
+    if args.workload != "mixer":
+        fn = {"causal": bench_causal, "triple": bench_triple, "block": bench_block}[args.workload]
+        print(json.dumps(fn(args, F, dev)))
+        return
     B, H, N, M, D = 1, 8, 1 << 20, 256, 32
     dtype = torch.bfloat16
     q, k, v = make_inputs(B, H, N, M, D, dtype, dev)
