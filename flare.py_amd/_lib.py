@@ -46,6 +46,16 @@ class FlareCausalLinearDesc(C.Structure):
     ]
 
 
+class FlareMlpDesc(C.Structure):
+    _fields_ = [
+        ("T", C.c_int64), ("C", C.c_int32), ("L", C.c_int32), ("w_dtype", C.c_int32),
+        ("x_dtype", C.c_int32), ("res_dtype", C.c_int32), ("y_dtype", C.c_int32),
+        ("norm", C.c_int32), ("eps", C.c_float), ("act", C.c_int32),
+        ("act_mask", C.c_uint32), ("add_mask", C.c_uint32), ("flags", C.c_int32),
+        ("x_stride", C.c_int64), ("res_stride", C.c_int64), ("y_stride", C.c_int64),
+    ]
+
+
 class FlareTripleDesc(C.Structure):
     _fields_ = [
         ("B", C.c_int32), ("H", C.c_int32), ("N", C.c_int32), ("Dq", C.c_int32), ("Dv", C.c_int32),
@@ -71,6 +81,7 @@ SYMBOLS = {
     "flare_causal_decode_fwd": (C.c_int, [C.POINTER(FlareCausalDesc), _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_causal_linear_workspace_bytes": (C.c_int, [C.POINTER(FlareCausalLinearDesc), C.POINTER(_SZ)]),
     "flare_causal_linear_fwd": (C.c_int, [C.POINTER(FlareCausalLinearDesc), _P, _P, _P, _P, _P, _SZ, _P]),
+    "flare_mlp_fwd": (C.c_int, [C.POINTER(FlareMlpDesc), _P, _P, _P, _P, _P, _P, _P, _P]),
     "flare_triple_workspace_bytes": (C.c_int, [C.POINTER(FlareTripleDesc), C.POINTER(_SZ)]),
     "flare_triple_state_fwd": (C.c_int, [C.POINTER(FlareTripleDesc), _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_triple_out_fwd": (C.c_int, [C.POINTER(FlareTripleDesc), _P, _P, _P, _P, _P, _P]),

@@ -495,6 +495,38 @@ int flare_causal_linear_fwd(const FlareCausalLinearDesc* desc, const void* q, co
     return hip_status(flare::launch_causal_linear(a, desc->dtype, static_cast<hipStream_t>(stream)), "causal linear launch");
 }
 
+int flare_mlp_fwd(const FlareMlpDesc* d, const void* x, const void* w, const float* bias, const float* gamma,
+                  const float* beta, const void* res, void* y, void* stream)
+{
+    if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
+    if (d->T < 1 || d->L < 1 || d->L > 16) return fail(FLARE_EINVAL, "T >= 1 and 1 <= L <= 16 required (got %lld, %d)", (long long)d->T, d->L);
+    if (d->w_dtype != FLARE_DT_BF16 && d->w_dtype != FLARE_DT_F16) return fail(FLARE_EINVAL, "w_dtype must be bf16 or f16");
+    const int dts[3] = {d->x_dtype, d->res_dtype, d->y_dtype};
+    for (int i = 0; i < 3; ++i)
+        if (dts[i] < FLARE_DT_F32 || dts[i] > FLARE_DT_F16) return fail(FLARE_EINVAL, "unknown dtype %d", dts[i]);
+    if (d->norm < FLARE_NORM_NONE || d->norm > FLARE_NORM_RMS) return fail(FLARE_EINVAL, "unknown norm %d", d->norm);
+    if (d->act < FLARE_ACT_GELU_TANH || d->act > FLARE_ACT_SILU) return fail(FLARE_EINVAL, "unknown activation %d", d->act);
+    if (!flare::mlp_mfma_supported(d->w_dtype, d->C)) return fail(FLARE_EUNSUPPORTED, "C=%d: only 32, 64 and 128 are supported", d->C);
+    if (!x || !w || !y) return fail(FLARE_EINVAL, "x, w, y must not be NULL");
+    if (d->norm != FLARE_NORM_NONE && !gamma) return fail(FLARE_EINVAL, "gamma must not be NULL when a norm is requested");
+    if (d->norm != FLARE_NORM_NONE && !(d->eps >= 0.f)) return fail(FLARE_EINVAL, "eps must be >= 0");
+    if (d->x_stride < d->C || d->y_stride < d->C || (res && d->res_stride < d->C))
+        return fail(FLARE_EINVAL, "row strides must be >= C");
+    // every lane moves 4 consecutive elements at a time
+    if (d->x_stride % 4 || d->y_stride % 4 || (res && d->res_stride % 4)) return fail(FLARE_EINVAL, "row strides must be multiples of 4");
+    if (!aligned16(x) || !aligned16(y) || !aligned16(w) || (res && !aligned16(res)) || (bias && !aligned16(bias)) ||
+        (gamma && !aligned16(gamma)) || (beta && !aligned16(beta)))
+        return fail(FLARE_EINVAL, "x, w, bias, gamma, beta, res, y must be 16-byte aligned");
+    flare::MlpArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = x; a.res = res; a.y = y; a.w = static_cast<const uint16_t*>(w); a.bias = bias; a.gamma = gamma; a.beta = beta;
+    a.T = d->T; a.C = d->C; a.L = d->L;
+    a.x_dtype = d->x_dtype; a.res_dtype = d->res_dtype; a.y_dtype = d->y_dtype;
+    a.norm = d->norm; a.eps = d->eps; a.act = d->act; a.act_mask = d->act_mask; a.add_mask = d->add_mask;
+    a.xs = d->x_stride; a.rs = d->res_stride; a.ys = d->y_stride;
+    return hip_status(flare::launch_mlp_mfma(a, d->w_dtype, static_cast<hipStream_t>(stream)), "mlp launch");
+}
+
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes)
 {
     if (!bytes) return fail(FLARE_EINVAL, "bytes is NULL");

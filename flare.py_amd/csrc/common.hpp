@@ -83,6 +83,21 @@ struct CausalLinearArgs {
     int64_t qs[3], ks[3], vs[3], ys[3];
 };
 
+struct MlpArgs {
+    const void* x; const void* res; void* y;   // [T,C] rows; res may be null
+    const uint16_t* w;                          // [L,C,C] 16-bit weights, row-major [out][in]
+    const float* bias;                          // [L,C] or null
+    const float* gamma; const float* beta;      // [C] norm parameters (beta may be null)
+    int64_t T;
+    int C, L;
+    int x_dtype, res_dtype, y_dtype;            // 0 f32, 1 bf16, 2 f16
+    int norm;                                   // 0 none, 1 LayerNorm, 2 RMSNorm
+    float eps;
+    int act;                                    // 0 tanh-GELU, 1 SiLU
+    uint32_t act_mask, add_mask;                // bit l: layer l applies the activation / adds to the stream
+    int64_t xs, rs, ys;                         // row strides in elements
+};
+
 // ---- launchers implemented in the .hip files -------------------------------------------
 hipError_t launch_gather_generic(const MixerArgs& a, int dtype, hipStream_t st);
 hipError_t launch_gather_merge(const MixerArgs& a, hipStream_t st);
@@ -100,6 +115,9 @@ hipError_t launch_causal_prefill(const CausalArgs& a, int dtype, hipStream_t st)
 hipError_t launch_causal_decode(const CausalArgs& a, int dtype, hipStream_t st);
 bool       causal_mfma_supported(int dtype, int M, int D);
 hipError_t launch_causal_mfma(const CausalArgs& a, int dtype, int step, hipStream_t st);   // step 16 prefill, 1 decode
+
+bool       mlp_mfma_supported(int w_dtype, int C);
+hipError_t launch_mlp_mfma(const MlpArgs& a, int w_dtype, hipStream_t st);
 
 int        causal_linear_tile();
 hipError_t launch_causal_linear(const CausalLinearArgs& a, int dtype, hipStream_t st);

@@ -1,0 +1,279 @@
+// Fused token-wise MLP stack on the matrix cores (bf16 / f16 weights, C in {32, 64, 128}).
+//
+// One launch evaluates, per token, what pdebench/models/flare.py of the reference spells as
+// separate torch layers: an optional LayerNorm / RMSNorm (FLAREBlock.forward :204-215), a chain of
+// C x C Linear layers each optionally followed by the activation and optionally added to the
+// running stream (ResidualMLP.forward :45-59; a single Linear is the chain of length one), and an
+// optional outer residual.  Layer l:  t = W_l s + b_l;  t = act(t) if bit l of act_mask;
+// s = s + t if bit l of add_mask else t.   Output = res + s  (res may be absent).
+//
+// Layout.  The product is taken transposed, S'^T = W S^T, with v_mfma_f32_16x16x32: A = W tile
+// (lane = output row, 8 consecutive input features per lane), B = S^T (lane = token c16, k-slots =
+// input features), D: lane = token, registers = 4 output rows.  Output row j of tile ft is given
+// the feature (C/4) (j/4) + 4 ft + j%4, so lane (c16, g) of every tile holds features
+// (C/4) g + 4 ft + r: over all tiles one CONTIGUOUS quarter row of its token.  Therefore
+//   * x, res and y are read / written as contiguous C/4-element runs per lane,
+//   * the accumulators of one layer, packed to 16 bits in place, ARE the B operands of the next
+//     layer (k-slot e of step ks in lane g = feature (C/4) g + 8 ks + e): the stream never leaves
+//     the registers between layers, in fp32 for the residual path,
+//   * the A operand of step ks is the 16 contiguous bytes W[row][(C/4) g + 8 ks ..].
+// Weights are staged per layer into LDS (double buffered, one barrier per layer) and shared by
+// the 4 waves of a workgroup, each of which owns 16*TW tokens per pass.
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace flare {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mm;
+template <> struct Mm<bf16_t> {
+    static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        bf16x2 v = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+};
+template <> struct Mm<f16_t> {
+    static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        f16x2 v = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+};
+
+// four consecutive elements of a row of element type dt (0 f32, 1 bf16, 2 f16) as fp32
+__device__ __forceinline__ f32x4 load4(const void* base, int64_t elem, int dt)
+{
+    if (dt == 0) return *reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + elem);
+    const uint2 r = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + elem);
+    if (dt == 1)
+        return f32x4{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
+                     __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u)};
+    const f16x2 lo = __builtin_bit_cast(f16x2, r.x), hi = __builtin_bit_cast(f16x2, r.y);
+    return f32x4{(float)lo[0], (float)lo[1], (float)hi[0], (float)hi[1]};
+}
+
+__device__ __forceinline__ void store4(void* base, int64_t elem, int dt, f32x4 v)
+{
+    if (dt == 0) {
+        *reinterpret_cast<f32x4*>(static_cast<float*>(base) + elem) = v;
+    } else if (dt == 1) {
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(base) + elem) =
+            make_uint2(Mm<bf16_t>::pack2(v[0], v[1]), Mm<bf16_t>::pack2(v[2], v[3]));
+    } else {
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(base) + elem) =
+            make_uint2(Mm<f16_t>::pack2(v[0], v[1]), Mm<f16_t>::pack2(v[2], v[3]));
+    }
+}
+
+__device__ __forceinline__ float xg_sum(float v)   // sum over the 4 lane groups that share a token
+{
+    v += __shfl_xor(v, 16);
+    v += __shfl_xor(v, 32);
+    return v;
+}
+
+// tanh-GELU (torch's approximate='tanh') = x * sigmoid(2 u), u = sqrt(2/pi) (x + 0.044715 x^3)
+__device__ __forceinline__ float gelu_tanh(float x)
+{
+    const float t = x * (2.3022081f + 0.10294324f * x * x);      // 2 u log2(e)
+    return x * __builtin_amdgcn_rcpf(1.f + fast_exp2(-t));
+}
+__device__ __forceinline__ float silu(float x)
+{
+    return x * __builtin_amdgcn_rcpf(1.f + fast_exp2(-kLog2e * x));
+}
+
+template <typename T, int C, int TW>
+__global__ __launch_bounds__(256, 2) void mlp_mfma_kernel(MlpArgs a)
+{
+    constexpr int FT = C / 16;        // feature tiles of the stream
+    constexpr int KS = C / 32;        // k-steps of one layer
+    constexpr int Q4 = C / 4;         // features per lane
+    constexpr int RS = C * 2 + 16;    // LDS row stride in bytes (padded: conflict-free 16-byte reads)
+    constexpr int WBUF = C * RS;
+    constexpr int TOKW = 16 * TW;     // tokens per wave and pass
+    using M_ = Mm<T>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int arow = Q4 * (c16 >> 2) + (c16 & 3);   // + 4 ft: the W row this lane supplies to tile ft
+
+    auto stage = [&](int layer, int buf) {
+        const uint16_t* wl = a.w + (size_t)layer * C * C;
+        for (int c = tid; c < C * C / 8; c += 256) {
+            const int row = c / (C / 8), ch = c % (C / 8);
+            *reinterpret_cast<u32x4*>(smem + buf * WBUF + row * RS + ch * 16) =
+                *reinterpret_cast<const u32x4*>(wl + row * C + ch * 8);
+        }
+    };
+
+    int lcount = 0;   // layers done by this workgroup: its parity names the LDS buffer in use
+    stage(0, 0);
+    __syncthreads();
+
+    const int64_t nblk = ((int64_t)a.T + 4 * TOKW - 1) / (4 * TOKW);
+    for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
+        int64_t tok[TW];
+        bool live[TW];
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw) {
+            const int64_t t = blk * (4 * TOKW) + w * TOKW + tw * 16 + c16;
+            live[tw] = t < a.T;
+            tok[tw] = live[tw] ? t : a.T - 1;
+        }
+
+        // the stream: lane (c16, g) holds features Q4 g + 4 ft + r of token c16 of each tile
+        f32x4 xs[FT][TW];
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) xs[ft][tw] = load4(a.x, tok[tw] * a.xs + Q4 * g + 4 * ft, a.x_dtype);
+
+        if (a.norm != 0) {
+#pragma unroll
+            for (int tw = 0; tw < TW; ++tw) {
+                float mean = 0.f;
+                if (a.norm == 1) {
+                    float s = 0.f;
+#pragma unroll
+                    for (int ft = 0; ft < FT; ++ft) s += xs[ft][tw][0] + xs[ft][tw][1] + xs[ft][tw][2] + xs[ft][tw][3];
+                    mean = xg_sum(s) * (1.f / C);
+                }
+                float ss = 0.f;
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float d = xs[ft][tw][r] - mean;
+                        ss = fmaf(d, d, ss);
+                    }
+                const float rstd = rsqrtf(xg_sum(ss) * (1.f / C) + a.eps);
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft) {
+                    const f32x4 gm = *reinterpret_cast<const f32x4*>(a.gamma + Q4 * g + 4 * ft);
+                    f32x4 bt = {0.f, 0.f, 0.f, 0.f};
+                    if (a.beta) bt = *reinterpret_cast<const f32x4*>(a.beta + Q4 * g + 4 * ft);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) xs[ft][tw][r] = (xs[ft][tw][r] - mean) * rstd * gm[r] + bt[r];
+                }
+            }
+        }
+
+        for (int l = 0; l < a.L; ++l, ++lcount) {
+            const int buf = lcount & 1;
+            // weights of the layer after this one (layer 0 of the next pass after the last)
+            stage(l + 1 < a.L ? l + 1 : 0, buf ^ 1);
+
+            // B operands: the stream, packed
+            u32x4 xb[KS][TW];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int tw = 0; tw < TW; ++tw) {
+                    const f32x4 lo = xs[2 * ks][tw], hi = xs[2 * ks + 1][tw];
+                    xb[ks][tw] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]),
+                                       M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
+                }
+
+            const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
+            const uint8_t* wb = smem + buf * WBUF + arow * RS + (Q4 * g) * 2;
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                const f32x4 bias = a.bias ? *reinterpret_cast<const f32x4*>(a.bias + (size_t)l * C + Q4 * g + 4 * ft)
+                                          : f32x4{0.f, 0.f, 0.f, 0.f};
+                f32x4 acc[TW];
+#pragma unroll
+                for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    const u32x4 wa = *reinterpret_cast<const u32x4*>(wb + (4 * ft) * RS + ks * 16);
+#pragma unroll
+                    for (int tw = 0; tw < TW; ++tw) acc[tw] = M_::mma(wa, xb[ks][tw], acc[tw]);
+                }
+#pragma unroll
+                for (int tw = 0; tw < TW; ++tw) {
+                    f32x4 t = acc[tw];
+                    if (act) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) t[r] = a.act == 0 ? gelu_tanh(t[r]) : silu(t[r]);
+                    }
+                    // tile ft of the stream is not an input of this layer any more once xb is packed
+                    xs[ft][tw] = add ? xs[ft][tw] + t : t;
+                }
+            }
+            __syncthreads();
+        }
+
+#pragma unroll
+        for (int tw = 0; tw < TW; ++tw) {
+            if (!live[tw]) continue;
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                f32x4 o = xs[ft][tw];
+                if (a.res) o += load4(a.res, tok[tw] * a.rs + Q4 * g + 4 * ft, a.res_dtype);
+                store4(a.y, tok[tw] * a.ys + Q4 * g + 4 * ft, a.y_dtype, o);
+            }
+        }
+    }
+}
+
+template <typename T, int C, int TW>
+hipError_t launch_ct(const MlpArgs& a, hipStream_t st)
+{
+    auto kern = mlp_mfma_kernel<T, C, TW>;
+    const size_t lds = 2 * (size_t)C * (C * 2 + 16);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    int occ = 0, cus = 0, dev = 0;
+    int slots = 512;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern), 256, lds) == hipSuccess && occ > 0 &&
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
+        slots = occ * cus;
+    else
+        (void)hipGetLastError();
+    const int64_t nblk = ((int64_t)a.T + 64 * TW - 1) / (64 * TW);
+    const unsigned grid = (unsigned)(nblk < slots ? nblk : slots);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_t(const MlpArgs& a, hipStream_t st)
+{
+    switch (a.C) {
+        case 32:  return launch_ct<T, 32, 4>(a, st);
+        case 64:  return launch_ct<T, 64, 4>(a, st);
+        case 128: return launch_ct<T, 128, 2>(a, st);
+        default:  return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+bool mlp_mfma_supported(int w_dtype, int C) { return (w_dtype == 1 || w_dtype == 2) && (C == 32 || C == 64 || C == 128); }
+
+hipError_t launch_mlp_mfma(const MlpArgs& a, int w_dtype, hipStream_t st)
+{
+    return w_dtype == 1 ? launch_t<bf16_t>(a, st) : launch_t<f16_t>(a, st);
+}
+
+}  // namespace flare

@@ -114,7 +114,14 @@ def mixer_kernel_name(q, k, v=None, scale=1.0, force_generic=False) -> str:
     return name.decode()
 
 
-def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic):
+def _autocast_dtype(t):
+    """The dtype torch.autocast would run scaled_dot_product_attention in on t's device, or None."""
+    if t.device.type == "cuda" and torch.is_autocast_enabled("cuda"):
+        return torch.get_autocast_dtype("cuda")
+    return None
+
+
+def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major=False):
     _require_cuda(q, k, v)
     lib = _lib.load()
     if q.dtype != k.dtype:
@@ -126,7 +133,10 @@ def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic):
     _check_mixer_shapes(q4, k, v)
     B, H, N, D = k.shape
     M = q4.shape[2]
-    y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    if token_major:   # memory order [B,N,H,D]: the head merge 'b h n d -> b n (h d)' is then a free view
+        y = torch.empty((B, N, H, D), dtype=k.dtype, device=k.device).permute(0, 2, 1, 3)
+    else:
+        y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
     z = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
     mask = _mask_u8(key_mask, B, N, k.device)
     d = _mixer_desc(q4, k, v, y, scale, n_splits, force_generic)
@@ -162,8 +172,8 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy):
 
 class _MixerFn(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, scale, key_mask, n_splits, force_generic):
-        y, z = _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic)
+    def forward(ctx, q, k, v, scale, key_mask, n_splits, force_generic, token_major):
+        y, z = _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major)
         ctx.save_for_backward(q, k, v)
         ctx.scale, ctx.key_mask = scale, key_mask
         ctx.mark_non_differentiable(z)
@@ -173,11 +183,11 @@ class _MixerFn(torch.autograd.Function):
     def backward(ctx, gy, _gz):
         q, k, v = ctx.saved_tensors
         gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy)
-        return gq, gk, gv, None, None, None, None
+        return gq, gk, gv, None, None, None, None, None
 
 
 def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: bool = False,
-                          n_splits: int = 0, force_generic: bool = False):
+                          n_splits: int = 0, force_generic: bool = False, token_major_out: bool = False):
     """FLARE gather-scatter mixer (README.md:39-52 of the reference).
 
     q: [H,M,D] latent queries (or [B,H,M,D]); k, v: [B,H,N,D]; returns y [B,H,N,D] with
@@ -185,11 +195,17 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
     key_mask ([B,N], nonzero = token present) removes padded tokens from the gather and
     zeroes their output rows (lra/models/backends.py:603-606,615-622).
     k and v may be strided views (e.g. 'b n (h d) -> b h n d') as long as D is contiguous.
+    Under torch.autocast the operands are cast to the autocast dtype, as torch does for the
+    scaled_dot_product_attention calls this replaces.  token_major_out=True lays y out as
+    [B,N,H,D] in memory (returned as its [B,H,N,D] view) so that merging the heads is free.
     """
+    ac = _autocast_dtype(k)
+    if ac is not None:
+        q, k, v = (t if t.dtype == ac else t.to(ac) for t in (q, k, v))
     if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
-        y, z = _MixerFn.apply(q, k, v, float(scale), key_mask, n_splits, force_generic)
+        y, z = _MixerFn.apply(q, k, v, float(scale), key_mask, n_splits, force_generic, token_major_out)
     else:
-        y, z = _mixer_forward(q, k, v, float(scale), key_mask, n_splits, force_generic)
+        y, z = _mixer_forward(q, k, v, float(scale), key_mask, n_splits, force_generic, token_major_out)
     return (y, z) if return_z else y
 
 

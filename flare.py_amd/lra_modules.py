@@ -53,7 +53,7 @@ class FLARE(nn.Module):
         v = self.v_proj(x).view(B, N, self.num_heads, self.head_dim).permute(0, 2, 1, 3)
         if self.rope is not None:
             k = self.rope(k)
-        y = flare_multihead_mixer(q, k, v, scale=self.attn_scale, key_mask=attention_mask)
+        y = flare_multihead_mixer(q, k, v, scale=self.attn_scale, key_mask=attention_mask, token_major_out=True)
         y = self.out_proj(y.permute(0, 2, 1, 3).reshape(B, N, C))
         return F.dropout(y, p=self.proj_drop_p if self.training else 0.0)
 

@@ -5,6 +5,11 @@ Drop-in counterparts of pdebench/models/flare.py of the reference (ResidualMLP :
 the reference loads with strict=True.  The projections, norms and MLPs are ordinary torch
 layers (hipBLASLt GEMMs); the mixer is the HIP engine (`functional.flare_multihead_mixer`),
 which reads k and v as strided [B,N,H*D] views, so no head-split copy is made.
+
+Inference fast path: when no gradient is needed and the Linear layers may run in bf16/f16
+(autocast, or 16-bit weights) and channel_dim is 32, 64 or 128, FLAREBlock runs as four fused HIP
+launches around the mixer (norm1 + k_proj, norm1 + v_proj, out_proj + residual, norm2 + FFN +
+residual; see fused.py) instead of ~70 torch kernels.  Training and fp32 use the torch layers.
 """
 from __future__ import annotations
 
@@ -12,6 +17,7 @@ import torch
 from torch import nn
 from torch.nn import functional as F
 
+from . import fused
 from .functional import flare_multihead_mixer
 
 __all__ = ["ResidualMLP", "FLARE", "FLAREBlock", "FinalLayer", "FLAREModel"]
@@ -97,9 +103,31 @@ class FLARE(nn.Module):
         B, N, _ = t.shape
         return t.view(B, N, self.num_heads, self.head_dim).permute(0, 2, 1, 3)  # [B,H,N,D] view, no copy
 
-    def forward(self, x, return_scores: bool = False):
+    def _fusable(self, x, return_scores):
+        """The 16-bit dtype for the fused projections, or None."""
+        if return_scores:
+            return None
+        cds = {fused.compute_dtype(x, m) for m in (self.k_proj, self.v_proj, self.out_proj)}
+        return cds.pop() if len(cds) == 1 else None
+
+    def forward(self, x, return_scores: bool = False, _norm=None, _res=None):
+        """(y, scores).  _norm / _res are FLAREBlock's pre-norm and residual, folded into the fused
+        launches when the fast path applies: then y = _res + out_proj(mixer(.. _norm(x) ..))."""
         B, N, C = x.shape
         q = self.latent_q.view(self.num_heads, self.num_latents, self.head_dim)
+        cd = self._fusable(x, return_scores)
+        if cd is not None:
+            k = self._heads(fused.fused_mlp(x, self.k_proj, cd, norm=_norm, out_dtype=cd))
+            v = self._heads(fused.fused_mlp(x, self.v_proj, cd, norm=_norm, out_dtype=cd))
+            if self.qk_norm:
+                q = self.q_norm(q)
+                k = self.k_norm(k)
+            y = flare_multihead_mixer(q, k, v, scale=self.attn_scale, token_major_out=True)
+            y = y.permute(0, 2, 1, 3).reshape(B, N, C)
+            out_dtype = _res.dtype if _res is not None else x.dtype
+            return fused.fused_mlp(y, self.out_proj, cd, res=_res, out_dtype=out_dtype), None
+        if _norm is not None:
+            x = _norm(x)
         k = self._heads(self.k_proj(x))
         v = self._heads(self.v_proj(x))
         if self.qk_norm:
@@ -107,7 +135,7 @@ class FLARE(nn.Module):
             k = self.k_norm(k)
 
         if not return_scores:
-            y = flare_multihead_mixer(q, k, v, scale=self.attn_scale)
+            y = flare_multihead_mixer(q, k, v, scale=self.attn_scale, token_major_out=True)
             scores = None
         else:
             # Diagnostic branch: materialises the [B,H,M,N] score matrix, exactly as the
@@ -117,7 +145,8 @@ class FLARE(nn.Module):
             y = F.softmax(scores.transpose(-2, -1), dim=-1) @ z
 
         y = y.permute(0, 2, 1, 3).reshape(B, N, C)
-        return self.out_proj(y), scores
+        y = self.out_proj(y)
+        return (y if _res is None else _res + y), scores
 
 
 class FLAREBlock(nn.Module):
@@ -138,9 +167,12 @@ class FLAREBlock(nn.Module):
                                num_layers=num_layers_ffn, act=act, input_residual=True, output_residual=True)
 
     def forward(self, x, return_scores: bool = False):
-        a, scores = self.att(self.norm1(x), return_scores=return_scores)
-        x = x + a
-        x = x + self.mlp(self.norm2(x))
+        x, scores = self.att(x, return_scores=return_scores, _norm=self.norm1, _res=x)
+        cd = fused.compute_dtype(x, self.mlp)
+        if cd is not None:
+            x = fused.fused_mlp(x, self.mlp, cd, norm=self.norm2, res=x)
+        else:
+            x = x + self.mlp(self.norm2(x))
         return x, scores
 
 

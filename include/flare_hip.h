@@ -20,6 +20,9 @@
  *                              token recurrence of causal_linear.py:317-336
  *   flare_causal_linear_fwd    CausalLinear.apply lra/models/triton/causal_linear.py:23-145
  *                              == linear_causal_reference causal_linear.py:317-336
+ *   flare_mlp_fwd              ResidualMLP.forward pdebench/models/flare.py:45-59 (and lra/models/
+ *                              backends.py:504-539), with the norm and residual around it of
+ *                              FLAREBlock.forward flare.py:204-215; a chain of one layer is nn.Linear
  *   flare_triple_fwd           TripleAttentionFunction.apply lra/models/triton/triple.py:29-121
  *                              == TripleAttention.attn_einsum lra/models/backends.py:1285-1292
  */
@@ -125,6 +128,33 @@ typedef struct FlareCausalLinearDesc {
     int64_t q_stride[3], k_stride[3], v_stride[3], y_stride[3];
 } FlareCausalLinearDesc;
 
+/*
+ * Fused token-wise MLP stack:  s = norm(x);  for l < L: t = W_l s + b_l; t = act(t) if bit l of
+ * act_mask; s = s + t if bit l of add_mask else t;  y = res + s.
+ * x, res, y: [T, C] rows (row strides in elements, rows contiguous); w: [L, C, C] row-major
+ * [out][in] in w_dtype (bf16 or f16, the type the products run in); bias [L, C], gamma, beta [C]
+ * fp32.  ResidualMLP(C, C, C, n layers, input_residual, output_residual) is L = n + 2 with
+ * act_mask = all but the last layer, add_mask = all layers (minus the first / last when the
+ * matching flag is off).  C must be 32, 64 or 128.
+ */
+#define FLARE_NORM_NONE  0
+#define FLARE_NORM_LAYER 1   /* (x - mean) * rsqrt(var + eps) * gamma + beta */
+#define FLARE_NORM_RMS   2   /* x * rsqrt(mean(x^2) + eps) * gamma           */
+#define FLARE_ACT_GELU_TANH 0
+#define FLARE_ACT_SILU      1
+typedef struct FlareMlpDesc {
+    int64_t  T;
+    int32_t  C, L;                        /* 1 <= L <= 16                                  */
+    int32_t  w_dtype;                     /* FLARE_DT_BF16 or FLARE_DT_F16                 */
+    int32_t  x_dtype, res_dtype, y_dtype; /* FLARE_DT_*                                    */
+    int32_t  norm;                        /* FLARE_NORM_*                                  */
+    float    eps;
+    int32_t  act;                         /* FLARE_ACT_*                                   */
+    uint32_t act_mask, add_mask;
+    int32_t  flags;
+    int64_t  x_stride, res_stride, y_stride;
+} FlareMlpDesc;
+
 int         flare_abi_version(void);
 const char* flare_last_error_string(void);
 
@@ -172,6 +202,11 @@ int flare_causal_linear_workspace_bytes(const FlareCausalLinearDesc* desc, size_
 int flare_causal_linear_fwd(const FlareCausalLinearDesc* desc, const void* q, const void* k,
                             const void* v, void* y, void* workspace, size_t workspace_bytes,
                             void* stream);
+
+/* bias, gamma (when norm == NONE), beta and res may be NULL.  y may alias res or x only row by
+ * row at equal strides (every row is read completely before it is written). */
+int flare_mlp_fwd(const FlareMlpDesc* desc, const void* x, const void* w, const float* bias,
+                  const float* gamma, const float* beta, const void* res, void* y, void* stream);
 
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes);
 

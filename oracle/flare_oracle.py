@@ -23,6 +23,8 @@ function (paths relative to the reference tree):
                         lra/models/triton/causal_linear.py:317-336; causal_bruteforce applies
                         mixer_explicit to every prefix and keeps the last row.
 
+  residual_mlp          pdebench/models/flare.py:45-59 (ResidualMLP.forward) with the pre-norm and
+                        outer residual of FLAREBlock.forward :204-215
   causal_linear_*       lra/models/triton/causal_linear.py:317-336 (token recurrence, k and v
                         each scaled by N^-1/2) and :338-389 (chunked form)
 
@@ -36,6 +38,9 @@ Pinning status (what each function is checked against in tests/test_oracle.py):
       independence; C restatement.
   triple_einsum               : hand cases (N=1, D=1), pure-Python loops, linearity in v,
       (k1,q1)<->(k2,q2) symmetry; C restatement.
+  residual_mlp                : torch's own nn.Linear / nn.GELU(approximate='tanh') / nn.SiLU /
+      nn.LayerNorm / nn.RMSNorm modules carrying the same weights, and the erf-free closed form of
+      tanh-GELU at a few points.
   causal_linear_recurrent     : the closed form tril(Q K^T) V / N, the chunked form for several
       chunk sizes, a pure-Python-float brute force, last row == non-causal linear attention.
 """
@@ -177,6 +182,48 @@ def causal_bruteforce(q, k, v, scale=1.0, dtype=torch.float64):
 def causal_state_invariants(mu, den, num):
     """The shift-invariant content of a state: z = num/den and lse = mu + log den."""
     return num / den.unsqueeze(-1), mu + torch.log(den)
+
+
+# --------------------------------------------------------------------------------------
+# token-wise MLP stack (ResidualMLP, norm, residual)
+# --------------------------------------------------------------------------------------
+def gelu_tanh(x):
+    return 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x ** 3)))
+
+
+def residual_mlp(x, weights, biases, act="gelu", input_residual=True, output_residual=True,
+                 norm=None, gamma=None, beta=None, eps=1e-5, res=None, dtype=torch.float64):
+    """res + ResidualMLP(norm(x)) following pdebench/models/flare.py:45-59: fc1 -> act,
+    (+ input if input_residual), n x (x + act(fc x)), fc2 (+ x if output_residual).  A single
+    weight is the num_layers == -1 case (one Linear, residual iff both flags).
+    norm: None | 'layer' | 'rms'."""
+    f = gelu_tanh if act == "gelu" else (lambda t: t * torch.sigmoid(t))
+    x = x.to(dtype)
+    ws = [w.to(dtype) for w in weights]
+    bs = [None if b is None else b.to(dtype) for b in biases]
+    lin = lambda t, i: t @ ws[i].T + (0 if bs[i] is None else bs[i])
+    if norm == "layer":
+        mu = x.mean(-1, keepdim=True)
+        var = ((x - mu) ** 2).mean(-1, keepdim=True)
+        x = (x - mu) / torch.sqrt(var + eps)
+    elif norm == "rms":
+        x = x / torch.sqrt((x ** 2).mean(-1, keepdim=True) + eps)
+    if norm is not None:
+        if gamma is not None:
+            x = x * gamma.to(dtype)
+        if beta is not None:
+            x = x + beta.to(dtype)
+    if len(ws) == 1:
+        h = lin(x, 0)
+        out = x + h if (input_residual and output_residual) else h
+    else:
+        h = f(lin(x, 0))
+        x = x + h if input_residual else h
+        for i in range(1, len(ws) - 1):
+            x = x + f(lin(x, i))
+        h = lin(x, len(ws) - 1)
+        out = x + h if output_residual else h
+    return out if res is None else res.to(dtype) + out
 
 
 # --------------------------------------------------------------------------------------

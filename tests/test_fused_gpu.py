@@ -1,0 +1,145 @@
+"""GPU parity of the fused token-wise MLP launches (flare_mlp_fwd) and of the fused FLAREBlock path.
+
+Oracle: oracle.flare_oracle.residual_mlp (restatement of pdebench/models/flare.py:45-59, 204-215),
+evaluated in fp64 on the SAME weights rounded to the compute type, so weight rounding is not charged
+to the kernel.  Tolerance 2e-2 relative L2 (the 16-bit bar): the stream is rounded to 16 bits once
+per layer as a matrix-core operand, accumulation and the residual path are fp32.
+"""
+import pytest
+import torch
+from torch import nn
+
+import flare_py_amd as F
+from flare_py_amd import fused
+from oracle import flare_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def make_mlp(C, n, ir, orr, act, dev, seed=0):
+    torch.manual_seed(seed)
+    m = F.ResidualMLP(C, C, C, num_layers=n, act=act, input_residual=ir, output_residual=orr)
+    for l in m.modules():
+        if isinstance(l, nn.Linear):
+            nn.init.normal_(l.weight, 0.0, C ** -0.5)
+            nn.init.normal_(l.bias, 0.0, 0.2)
+    return m.to(dev)
+
+
+def oracle_of(m, x, cd, norm=None, res=None):
+    layers, _, _, act = fused._layers_of(m)
+    ws = [l.weight.detach().to(cd).double().cpu() for l in layers]
+    bs = [l.bias.detach().double().cpu() for l in layers]
+    ir = getattr(m, "input_residual", getattr(m, "residual", False))
+    orr = getattr(m, "output_residual", getattr(m, "residual", False))
+    kind = gamma = beta = None
+    eps = 1e-5
+    if isinstance(norm, nn.LayerNorm):
+        kind, gamma, beta, eps = "layer", norm.weight.detach().cpu(), norm.bias.detach().cpu(), norm.eps
+    elif isinstance(norm, nn.RMSNorm):
+        kind, gamma, eps = "rms", norm.weight.detach().cpu(), norm.eps
+    return O.residual_mlp(x.double().cpu(), ws, bs, "gelu" if act == 0 else "silu", ir, orr, kind, gamma, beta, eps,
+                          None if res is None else res.double().cpu())
+
+
+@pytest.mark.parametrize("C", [32, 64, 128])
+@pytest.mark.parametrize("n,ir,orr,act", [(3, True, True, "gelu"), (0, False, True, "silu"), (1, True, False, "gelu"),
+                                          (-1, True, True, "gelu"), (6, True, True, "silu")])
+def test_mlp_stack_vs_oracle(dev, C, n, ir, orr, act):
+    m = make_mlp(C, n, ir, orr, act, dev)
+    x = torch.randn(3, 333, C, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        cd = fused.compute_dtype(x, m)
+        assert cd == torch.bfloat16
+        y = fused.fused_mlp(x, m, cd)
+    assert y.dtype == torch.float32 and y.shape == x.shape
+    assert O.rel_l2(y, oracle_of(m, x, cd)) <= 2e-2
+
+
+@pytest.mark.parametrize("norm_kind", ["layer", "rms"])
+@pytest.mark.parametrize("xdt,odt,cd", [(torch.float32, torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.bfloat16, torch.bfloat16),
+                                        (torch.float32, torch.float32, torch.float16), (torch.float16, torch.float16, torch.float16)])
+def test_norm_residual_dtypes_and_ragged_rows(dev, norm_kind, xdt, odt, cd):
+    C = 128
+    m = make_mlp(C, 3, True, True, "gelu", dev, seed=1)
+    norm = (nn.LayerNorm(C) if norm_kind == "layer" else nn.RMSNorm(C, eps=1e-6)).to(dev)
+    nn.init.normal_(norm.weight, 1.0, 0.3)
+    if norm_kind == "layer":
+        nn.init.normal_(norm.bias, 0.0, 0.3)
+    for T in (1, 17, 129, 1000):
+        x = (torch.randn(T, C, device=dev) * 2 + 0.5).to(xdt)
+        with torch.no_grad():
+            y = fused.fused_mlp(x, m, cd, norm=norm, res=x, out_dtype=odt)
+        assert y.dtype == odt
+        assert O.rel_l2(y, oracle_of(m, x, cd, norm, x)) <= 2e-2, T
+
+
+def test_single_linear_with_residual_and_strided_rows(dev):
+    C = 64
+    lin = nn.Linear(C, C).to(dev)
+    big = torch.randn(500, 2 * C, device=dev)
+    x = big[:, :C]                                   # row stride 2C: consumed without a copy
+    res = torch.randn(500, C, device=dev)
+    with torch.no_grad():
+        y = fused.fused_mlp(x, lin, torch.bfloat16, res=res)
+    ref = res.double().cpu() + x.double().cpu() @ lin.weight.detach().bfloat16().double().cpu().T + lin.bias.detach().double().cpu()
+    assert O.rel_l2(y, ref) <= 2e-2
+
+
+def test_fast_path_conditions(dev):
+    m = make_mlp(128, 3, True, True, "gelu", dev)
+    x = torch.randn(4, 128, device=dev)
+    assert fused.compute_dtype(x, m) is None                                  # grad enabled
+    with torch.no_grad():
+        assert fused.compute_dtype(x, m) is None                              # fp32 weights, no autocast
+        assert fused.compute_dtype(x.cpu(), m) is None
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            assert fused.compute_dtype(x, m) == torch.bfloat16
+            assert fused.compute_dtype(torch.randn(4, 48, device=dev), make_mlp(48, 1, True, True, "gelu", dev)) is None
+        assert fused.compute_dtype(x.half(), m.half()) == torch.float16
+    from flare_py_amd import _lib
+    d = _lib.FlareMlpDesc()
+    d.T, d.C, d.L, d.w_dtype = 4, 48, 1, 1
+    with pytest.raises(NotImplementedError):
+        _lib.check(_lib.load().flare_mlp_fwd(d, None, None, None, None, None, None, None, None), "flare_mlp_fwd")
+
+
+@pytest.mark.parametrize("C,H,M", [(128, 8, 128), (64, 4, 64)])
+@pytest.mark.parametrize("rms", [False, True])
+def test_block_fused_path_vs_torch_layers(dev, C, H, M, rms, monkeypatch):
+    torch.manual_seed(3)
+    blk = F.FLAREBlock(channel_dim=C, num_heads=H, num_latents=M, rmsnorm=rms).to(dev).eval()
+    for l in blk.modules():
+        if isinstance(l, nn.Linear):
+            nn.init.xavier_uniform_(l.weight)
+            nn.init.normal_(l.bias, 0.0, 0.1)
+    x = torch.randn(2, 3000, C, device=dev)
+    calls = []
+    real = fused.fused_mlp
+    monkeypatch.setattr(fused, "fused_mlp", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    with torch.no_grad():
+        ref, _ = blk(x)                                   # fp32 torch layers + fp32 HIP mixer
+        assert not calls
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y, _ = blk(x)                                 # four fused launches + bf16 HIP mixer
+    assert len(calls) == 4
+    assert y.dtype == torch.float32
+    assert O.rel_l2(y, ref) <= 2e-2
+    # gradients still flow through the torch layers when they are needed
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        yt, _ = blk(x[:, :256])
+    assert len(calls) == 4 and yt.requires_grad
+
+
+def test_model_fused_path_vs_fp32(dev):
+    torch.manual_seed(4)
+    model = F.FLAREModel(in_dim=3, out_dim=2, channel_dim=64, num_blocks=2, num_heads=4, num_latents=64).to(dev).eval()
+    for l in model.modules():
+        if isinstance(l, nn.Linear):
+            nn.init.xavier_uniform_(l.weight)
+    x = torch.randn(2, 2000, 3, device=dev)
+    with torch.no_grad():
+        ref = model(x)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = model(x)
+    assert O.rel_l2(y, ref) <= 3e-2

@@ -243,3 +243,42 @@ def test_causal_linear_oracle_is_pinned():
     q2 = torch.tensor([[[[2.0], [3.0]]]]); k2 = torch.tensor([[[[5.0], [7.0]]]]); v2 = torch.tensor([[[[11.0], [13.0]]]])
     y2 = O.causal_linear_recurrent(q2, k2, v2)
     assert torch.allclose(y2.flatten(), torch.tensor([2 * 5 * 11 / 2, 3 * (5 * 11 + 7 * 13) / 2], dtype=torch.float64))
+
+
+# ---- token-wise MLP stack -----------------------------------------------------------------
+def test_residual_mlp_oracle_matches_torch_layers():
+    from torch import nn
+    torch.manual_seed(0)
+    C = 12
+    for n, ir, orr, act, norm in [(3, True, True, "gelu", "layer"), (0, False, True, "silu", "rms"),
+                                  (1, True, False, "gelu", None), (-1, True, True, "gelu", "layer")]:
+        lins = [nn.Linear(C, C).double() for _ in range(n + 2 if n >= 0 else 1)]
+        a = nn.GELU(approximate="tanh") if act == "gelu" else nn.SiLU()
+        nm = {"layer": nn.LayerNorm(C).double(), "rms": nn.RMSNorm(C, eps=1e-6).double(), None: nn.Identity()}[norm]
+        if norm is not None:
+            nn.init.normal_(nm.weight, 1.0, 0.3)
+            if norm == "layer":
+                nn.init.normal_(nm.bias, 0.0, 0.3)
+        x = torch.randn(5, 7, C, dtype=torch.float64)
+        with torch.no_grad():
+            s = nm(x)
+            if n == -1:
+                h = lins[0](s)
+                ref = s + h if (ir and orr) else h
+            else:
+                h = a(lins[0](s))
+                s = s + h if ir else h
+                for l in lins[1:-1]:
+                    s = s + a(l(s))
+                h = lins[-1](s)
+                ref = s + h if orr else h
+            ref = x + ref
+        got = O.residual_mlp(x, [l.weight.detach() for l in lins], [l.bias.detach() for l in lins], act, ir, orr,
+                             norm, None if norm is None else nm.weight.detach(),
+                             nm.bias.detach() if norm == "layer" else None, 1e-5 if norm == "layer" else 1e-6, res=x)
+        assert O.rel_l2(got, ref) < 1e-12, (n, ir, orr, act, norm)
+    # tanh-GELU known values: gelu(0) = 0, gelu(x) - gelu(-x) = x, gelu(1) = 0.841192 (tanh form)
+    t = torch.tensor([0.0, 1.0, -1.0, 3.0, -3.0], dtype=torch.float64)
+    gv = O.gelu_tanh(t)
+    assert gv[0] == 0 and abs(float(gv[1]) - 0.8411919906082768) < 1e-12
+    assert torch.allclose(gv[1] - gv[2], t[1]) and torch.allclose(gv[3] - gv[4], t[3])
