@@ -9,16 +9,20 @@
 //
 // Layout.  The product is taken transposed, S'^T = W S^T, with v_mfma_f32_16x16x32: A = W tile
 // (lane = output row, 8 consecutive input features per lane), B = S^T (lane = token c16, k-slots =
-// input features), D: lane = token, registers = 4 output rows.  Output row j of tile ft is given
-// the feature (C/4) (j/4) + 4 ft + j%4, so lane (c16, g) of every tile holds features
-// (C/4) g + 4 ft + r: over all tiles one CONTIGUOUS quarter row of its token.  Therefore
-//   * x, res and y are read / written as contiguous C/4-element runs per lane,
+// input features), D: lane = token, registers = 4 output rows.  Lane (c16, g) of stream tile ft
+// holds features 16 ft + 4 g + r (r = 0..3) of token c16.  Therefore
+//   * x, res and y move as 4-element runs per lane; the 4 lanes of a token cover 16 consecutive
+//     features per instruction (64 contiguous bytes of fp32 per row),
 //   * the accumulators of one layer, packed to 16 bits in place, ARE the B operands of the next
-//     layer (k-slot e of step ks in lane g = feature (C/4) g + 8 ks + e): the stream never leaves
-//     the registers between layers, in fp32 for the residual path,
-//   * the A operand of step ks is the 16 contiguous bytes W[row][(C/4) g + 8 ks ..].
-// Weights are staged per layer into LDS (double buffered, one barrier per layer) and shared by
-// the 4 waves of a workgroup, each of which owns 16*TW tokens per pass.
+//     layer: a contraction may visit its index in any order, so k-slot e of step ks in lane g is
+//     simply feature 32 ks + 16 (e/4) + 4 g + e%4, and the stream never leaves the registers
+//     between layers (fp32 on the residual path),
+//   * the weights are staged into LDS with their columns in that slot order, so the A operand of
+//     step ks is one 16-byte read at column position 32 ks + 8 g.
+// Weights live in LDS, shared by the WAVES waves of a workgroup, each of which owns 16*TW tokens
+// per pass.  When all L layers fit they are staged once and the token loop has no barrier at all;
+// otherwise two slots form a ring: the next layer's weights are fetched into registers before the
+// products of the current layer and written to the free slot after them (one barrier per layer).
 #include <type_traits>
 
 #include "common.hpp"
@@ -101,12 +105,13 @@ __device__ __forceinline__ float silu(float x)
     return x * __builtin_amdgcn_rcpf(1.f + fast_exp2(-kLog2e * x));
 }
 
-template <typename T, int C, int TW>
-__global__ __launch_bounds__(256, 2) void mlp_mfma_kernel(MlpArgs a)
+template <typename T, int C, int TW, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kernel(MlpArgs a, int resident)
 {
+    constexpr int NT = 64 * WAVES;
+    constexpr int NCH = (C * C / 8 + NT - 1) / NT;   // 16-byte weight chunks per thread and layer
     constexpr int FT = C / 16;        // feature tiles of the stream
     constexpr int KS = C / 32;        // k-steps of one layer
-    constexpr int Q4 = C / 4;         // features per lane
     constexpr int RS = C * 2 + 16;    // LDS row stride in bytes (padded: conflict-free 16-byte reads)
     constexpr int WBUF = C * RS;
     constexpr int TOKW = 16 * TW;     // tokens per wave and pass
@@ -114,38 +119,61 @@ __global__ __launch_bounds__(256, 2) void mlp_mfma_kernel(MlpArgs a)
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
-    const int arow = Q4 * (c16 >> 2) + (c16 & 3);   // + 4 ft: the W row this lane supplies to tile ft
 
-    auto stage = [&](int layer, int buf) {
+    u32x4 wreg[NCH];
+    auto fetch = [&](int layer) {
         const uint16_t* wl = a.w + (size_t)layer * C * C;
-        for (int c = tid; c < C * C / 8; c += 256) {
-            const int row = c / (C / 8), ch = c % (C / 8);
-            *reinterpret_cast<u32x4*>(smem + buf * WBUF + row * RS + ch * 16) =
-                *reinterpret_cast<const u32x4*>(wl + row * C + ch * 8);
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + i * NT;
+            if (c < C * C / 8) wreg[i] = *reinterpret_cast<const u32x4*>(wl + (c / (C / 8)) * C + (c % (C / 8)) * 8);
+        }
+    };
+    auto put = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + i * NT;
+            if (c < C * C / 8) {
+                const int row = c / (C / 8), ch = c % (C / 8);
+                // features 8 ch .. 8 ch + 3 belong to k-step ch / 4, half (ch % 4) / 2, lane group 2 (ch % 2);
+                // features 8 ch + 4 .. + 7 to the next lane group.  Position = 32 ks + 8 g + 4 half.
+                const int pos = 32 * (ch >> 2) + 16 * (ch & 1) + 4 * ((ch & 3) >> 1);
+                uint8_t* dst = smem + slot * WBUF + row * RS + pos * 2;
+                *reinterpret_cast<uint2*>(dst) = make_uint2(wreg[i][0], wreg[i][1]);
+                *reinterpret_cast<uint2*>(dst + 16) = make_uint2(wreg[i][2], wreg[i][3]);
+            }
         }
     };
 
-    int lcount = 0;   // layers done by this workgroup: its parity names the LDS buffer in use
-    stage(0, 0);
+    int lcount = 0;   // ring mode: layers done by this workgroup; its parity names the slot in use
+    if (resident) {
+        for (int l = 0; l < a.L; ++l) {
+            fetch(l);
+            put(l);
+        }
+    } else {
+        fetch(0);
+        put(0);
+    }
     __syncthreads();
 
-    const int64_t nblk = ((int64_t)a.T + 4 * TOKW - 1) / (4 * TOKW);
+    const int64_t nblk = ((int64_t)a.T + WAVES * TOKW - 1) / (WAVES * TOKW);
     for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
         int64_t tok[TW];
         bool live[TW];
 #pragma unroll
         for (int tw = 0; tw < TW; ++tw) {
-            const int64_t t = blk * (4 * TOKW) + w * TOKW + tw * 16 + c16;
+            const int64_t t = blk * (WAVES * TOKW) + w * TOKW + tw * 16 + c16;
             live[tw] = t < a.T;
             tok[tw] = live[tw] ? t : a.T - 1;
         }
 
-        // the stream: lane (c16, g) holds features Q4 g + 4 ft + r of token c16 of each tile
+        // the stream: lane (c16, g) holds features 16 ft + 4 g + r of token c16 of each tile
         f32x4 xs[FT][TW];
 #pragma unroll
         for (int tw = 0; tw < TW; ++tw)
 #pragma unroll
-            for (int ft = 0; ft < FT; ++ft) xs[ft][tw] = load4(a.x, tok[tw] * a.xs + Q4 * g + 4 * ft, a.x_dtype);
+            for (int ft = 0; ft < FT; ++ft) xs[ft][tw] = load4(a.x, tok[tw] * a.xs + 16 * ft + 4 * g, a.x_dtype);
 
         if (a.norm != 0) {
 #pragma unroll
@@ -168,9 +196,9 @@ __global__ __launch_bounds__(256, 2) void mlp_mfma_kernel(MlpArgs a)
                 const float rstd = rsqrtf(xg_sum(ss) * (1.f / C) + a.eps);
 #pragma unroll
                 for (int ft = 0; ft < FT; ++ft) {
-                    const f32x4 gm = *reinterpret_cast<const f32x4*>(a.gamma + Q4 * g + 4 * ft);
+                    const f32x4 gm = *reinterpret_cast<const f32x4*>(a.gamma + 16 * ft + 4 * g);
                     f32x4 bt = {0.f, 0.f, 0.f, 0.f};
-                    if (a.beta) bt = *reinterpret_cast<const f32x4*>(a.beta + Q4 * g + 4 * ft);
+                    if (a.beta) bt = *reinterpret_cast<const f32x4*>(a.beta + 16 * ft + 4 * g);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) xs[ft][tw][r] = (xs[ft][tw][r] - mean) * rstd * gm[r] + bt[r];
                 }
@@ -178,9 +206,9 @@ __global__ __launch_bounds__(256, 2) void mlp_mfma_kernel(MlpArgs a)
         }
 
         for (int l = 0; l < a.L; ++l, ++lcount) {
-            const int buf = lcount & 1;
-            // weights of the layer after this one (layer 0 of the next pass after the last)
-            stage(l + 1 < a.L ? l + 1 : 0, buf ^ 1);
+            const int slot = resident ? l : (lcount & 1);
+            // ring: fetch the weights of the layer after this one (layer 0 of the next pass after the last)
+            if (!resident) fetch(l + 1 < a.L ? l + 1 : 0);
 
             // B operands: the stream, packed
             u32x4 xb[KS][TW];
@@ -194,17 +222,17 @@ __global__ __launch_bounds__(256, 2) void mlp_mfma_kernel(MlpArgs a)
                 }
 
             const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
-            const uint8_t* wb = smem + buf * WBUF + arow * RS + (Q4 * g) * 2;
+            const uint8_t* wb = smem + slot * WBUF + c16 * RS + g * 16;
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
-                const f32x4 bias = a.bias ? *reinterpret_cast<const f32x4*>(a.bias + (size_t)l * C + Q4 * g + 4 * ft)
+                const f32x4 bias = a.bias ? *reinterpret_cast<const f32x4*>(a.bias + (size_t)l * C + 16 * ft + 4 * g)
                                           : f32x4{0.f, 0.f, 0.f, 0.f};
                 f32x4 acc[TW];
 #pragma unroll
                 for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    const u32x4 wa = *reinterpret_cast<const u32x4*>(wb + (4 * ft) * RS + ks * 16);
+                    const u32x4 wa = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + ks * 64);
 #pragma unroll
                     for (int tw = 0; tw < TW; ++tw) acc[tw] = M_::mma(wa, xb[ks][tw], acc[tw]);
                 }
@@ -219,7 +247,10 @@ __global__ __launch_bounds__(256, 2) void mlp_mfma_kernel(MlpArgs a)
                     xs[ft][tw] = add ? xs[ft][tw] + t : t;
                 }
             }
-            __syncthreads();
+            if (!resident) {
+                put(slot ^ 1);      // nobody reads that slot during this layer
+                __syncthreads();
+            }
         }
 
 #pragma unroll
@@ -228,31 +259,36 @@ __global__ __launch_bounds__(256, 2) void mlp_mfma_kernel(MlpArgs a)
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
                 f32x4 o = xs[ft][tw];
-                if (a.res) o += load4(a.res, tok[tw] * a.rs + Q4 * g + 4 * ft, a.res_dtype);
-                store4(a.y, tok[tw] * a.ys + Q4 * g + 4 * ft, a.y_dtype, o);
+                if (a.res) o += load4(a.res, tok[tw] * a.rs + 16 * ft + 4 * g, a.res_dtype);
+                store4(a.y, tok[tw] * a.ys + 16 * ft + 4 * g, a.y_dtype, o);
             }
         }
     }
 }
 
-template <typename T, int C, int TW>
+constexpr size_t kMlpLdsMax = 156 * 1024;
+
+template <typename T, int C, int TW, int WAVES>
 hipError_t launch_ct(const MlpArgs& a, hipStream_t st)
 {
-    auto kern = mlp_mfma_kernel<T, C, TW>;
-    const size_t lds = 2 * (size_t)C * (C * 2 + 16);
+    auto kern = mlp_mfma_kernel<T, C, TW, WAVES>;
+    const size_t wbuf = (size_t)C * (C * 2 + 16);
+    const int resident = (size_t)a.L * wbuf <= kMlpLdsMax ? 1 : 0;
+    const size_t lds = (resident ? (size_t)a.L : 2) * wbuf;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     int occ = 0, cus = 0, dev = 0;
     int slots = 512;
     if (hipGetDevice(&dev) == hipSuccess &&
-        hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern), 256, lds) == hipSuccess && occ > 0 &&
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern), 64 * WAVES, lds) == hipSuccess && occ > 0 &&
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
         slots = occ * cus;
     else
         (void)hipGetLastError();
-    const int64_t nblk = ((int64_t)a.T + 64 * TW - 1) / (64 * TW);
+    const int64_t per = 16 * TW * WAVES;
+    const int64_t nblk = ((int64_t)a.T + per - 1) / per;
     const unsigned grid = (unsigned)(nblk < slots ? nblk : slots);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES), lds, st, a, resident);
     return hipGetLastError();
 }
 
@@ -260,9 +296,9 @@ template <typename T>
 hipError_t launch_t(const MlpArgs& a, hipStream_t st)
 {
     switch (a.C) {
-        case 32:  return launch_ct<T, 32, 4>(a, st);
-        case 64:  return launch_ct<T, 64, 4>(a, st);
-        case 128: return launch_ct<T, 128, 2>(a, st);
+        case 32:  return launch_ct<T, 32, 4, 4>(a, st);
+        case 64:  return launch_ct<T, 64, 4, 4>(a, st);
+        case 128: return launch_ct<T, 128, 2, 8>(a, st);
         default:  return hipErrorInvalidValue;
     }
 }
