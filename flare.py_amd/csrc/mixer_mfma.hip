@@ -402,7 +402,12 @@ constexpr int kSTokWave = 16 * kSTW;
 
 // One workgroup = 4 independent waves sharing Q and Z^T operands in LDS; wave w walks the
 // workgroup's token range in steps of 64 tokens.  No barrier after the set-up.
-template <typename T, int D>
+// KSC = M / 32 fixed at compile time (the latent loop is then fully unrolled, operands renamed
+// instead of copied, accumulators started from a literal zero) or 0 for any M at run time.
+// Inside a latent step the 4 token tiles are software pipelined: the scores of tile t+1 are
+// issued before the exponentials of tile t, and the value product of tile t-1 after them, so
+// that no instruction waits on the matrix-core result just issued.
+template <typename T, int D, int KSC>
 __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int tokens_per_wg)
 {
     constexpr int KD = (D + 31) / 32;
@@ -411,7 +416,6 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
     using M_ = Mma<T>;          // score product, in the element type of q and k
     using P_ = Mma<bf16_t>;     // value product: probabilities (and the values they meet) are always bf16
 
-    __shared__ float red[4];
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     // qa[mt][ch][c16]  : 16 bytes each, latent m = 16 mt + c16, d = 8 ch .. 8 ch + 7
     // zt[ks][rt][lane] : 16 bytes each, row d = (D/4) (c16/4) + 4 rt + c16 % 4,
@@ -421,7 +425,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
     const int h = blockIdx.y, b = blockIdx.z;
-    const int M = a.M, MT = M / 16, KS = M / 32;
+    const int M = KSC ? 32 * KSC : a.M, KS = M / 32;
 
     const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
     const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
@@ -452,8 +456,9 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
 
     const int wg_n0 = blockIdx.x * tokens_per_wg;
     const int wg_n1 = min(a.N, wg_n0 + tokens_per_wg);
+    const u32x4 ones8 = {P_::kOnes2, P_::kOnes2, P_::kOnes2, P_::kOnes2};
+    const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
 
-    u32x4 kb[kSTW][KD], kn[kSTW][KD];
     auto load_k = [&](int t0, u32x4 (&dst)[kSTW][KD]) {
 #pragma unroll
         for (int tw = 0; tw < kSTW; ++tw)
@@ -463,16 +468,25 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                 dst[tw][kd] = (n < wg_n1 && ch < CH) ? load16_stream(k + (int64_t)n * a.ks[2] + ch * 8) : zero4();
             }
     };
+    auto load_ops = [&](int ks, u32x4 (&o0)[KD], u32x4 (&o1)[KD], u32x4 (&oz)[RT]) {
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const int ch = kd * 4 + g;
+            o0[kd] = ch < CH ? qa[((2 * ks) * CH + ch) * 16 + c16] : zero4();
+            o1[kd] = ch < CH ? qa[((2 * ks + 1) * CH + ch) * 16 + c16] : zero4();
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) oz[rt] = zt[(ks * RT + rt) * 64 + lane];
+    };
+    auto scores = [&](const u32x4 (&o)[KD], const u32x4 (&kk)[KD]) {
+        f32x4 s = zf;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) s = M_::mma(o[kd], kk[kd], s);
+        return s;
+    };
 
-    const u32x4 ones8 = {P_::kOnes2, P_::kOnes2, P_::kOnes2, P_::kOnes2};
-
-    int t0 = wg_n0 + w * kSTokWave;
-    if (t0 < wg_n1) load_k(t0, kb);
-
-    for (; t0 < wg_n1; t0 += 4 * kSTokWave) {
-        const int tnext = t0 + 4 * kSTokWave;
-        if (tnext < wg_n1) load_k(tnext, kn);
-
+    // one 64-token tile of this wave: kb = its K rows as B operands
+    auto tile64 = [&](const u32x4 (&kb)[kSTW][KD], int t0) {
         f32x4 yacc[kSTW][RT];
         float lrow[kSTW];       // softmax denominators, complete for the lane's token
         bool redo = false;
@@ -482,52 +496,60 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
             // that is validated afterwards on the denominators, and only a token tile that
             // fails goes through the exact (running maximum) path below.
             f32x4 yl[kSTW];
+            u32x4 q0[KD], q1[KD], za[RT], q0n[KD], q1n[KD], zan[RT];
+            // one latent step (32 latents) for the wave's 4 column tiles, pipelined over the tiles
+            auto step = [&](bool first) {
+                auto pv = [&](int tw, u32x4 pb) {
 #pragma unroll
-            for (int tw = 0; tw < kSTW; ++tw) {
-                yl[tw] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
-            }
-            // operands of latent step ks live in registers one step ahead of their use
-            u32x4 q0[KD], q1[KD], za[RT];
-            auto load_ops = [&](int ks, u32x4 (&o0)[KD], u32x4 (&o1)[KD], u32x4 (&oz)[RT]) {
-#pragma unroll
-                for (int kd = 0; kd < KD; ++kd) {
-                    const int ch = kd * 4 + g;
-                    o0[kd] = ch < CH ? qa[((2 * ks) * CH + ch) * 16 + c16] : zero4();
-                    o1[kd] = ch < CH ? qa[((2 * ks + 1) * CH + ch) * 16 + c16] : zero4();
-                }
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt) oz[rt] = zt[(ks * RT + rt) * 64 + lane];
-            };
-            // one latent step (32 latents) for the wave's 4 column tiles
-            auto step = [&](const u32x4 (&o0)[KD], const u32x4 (&o1)[KD], const u32x4 (&oz)[RT]) {
+                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = P_::mma(za[rt], pb, first ? zf : yacc[tw][rt]);
+                    yl[tw] = P_::mma(ones8, pb, first ? zf : yl[tw]);   // row of ones: the softmax denominator
+                };
+                f32x4 s0 = scores(q0, kb[0]), s1 = scores(q1, kb[0]);
+                u32x4 pbp = zero4();
 #pragma unroll
                 for (int tw = 0; tw < kSTW; ++tw) {
-                    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int kd = 0; kd < KD; ++kd) {
-                        s0 = M_::mma(o0[kd], kb[tw][kd], s0);
-                        s1 = M_::mma(o1[kd], kb[tw][kd], s1);
+                    f32x4 n0 = zf, n1 = zf;
+                    if (tw + 1 < kSTW) {
+                        n0 = scores(q0, kb[tw + 1]);
+                        n1 = scores(q1, kb[tw + 1]);
                     }
                     const u32x4 pb = {P_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])),
                                       P_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
                                       P_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])),
                                       P_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]))};
-#pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = P_::mma(oz[rt], pb, yacc[tw][rt]);
-                    yl[tw] = P_::mma(ones8, pb, yl[tw]);   // row of ones: the softmax denominator
+                    if (tw > 0) pv(tw - 1, pbp);
+                    s0 = n0;
+                    s1 = n1;
+                    pbp = pb;
+                    __builtin_amdgcn_sched_barrier(0);
                 }
+                pv(kSTW - 1, pbp);
             };
-            // two operand sets, each loaded from LDS one step before it is used (KS is even or 1
-            // step is peeled: M is a multiple of 64, so KS is always even)
-            u32x4 q0b[KD], q1b[KD], zab[RT];
+            auto advance = [&](int ks) {   // operands of step ks become current, those of ks + 1 are fetched
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) {
+                    q0[kd] = q0n[kd];
+                    q1[kd] = q1n[kd];
+                }
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) za[rt] = zan[rt];
+                if (ks + 1 < KS) load_ops(ks + 1, q0n, q1n, zan);
+            };
             load_ops(0, q0, q1, za);
-            for (int ks = 0; ks < KS; ks += 2) {
-                load_ops(ks + 1, q0b, q1b, zab);
-                step(q0, q1, za);
-                load_ops(ks + 2 < KS ? ks + 2 : ks, q0, q1, za);
-                step(q0b, q1b, zab);
+            if (KS > 1) load_ops(1, q0n, q1n, zan);
+            step(true);
+            if constexpr (KSC > 0) {
+#pragma unroll
+                for (int ks = 1; ks < KSC; ++ks) {
+                    advance(ks);
+                    step(false);
+                }
+            } else {
+#pragma unroll 1
+                for (int ks = 1; ks < KS; ++ks) {
+                    advance(ks);
+                    step(false);
+                }
             }
 #pragma unroll
             for (int tw = 0; tw < kSTW; ++tw) {
@@ -544,26 +566,15 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                 shift[tw] = kNegBig;
                 lsum[tw] = 0.f;
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+                for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = zf;
             }
+#pragma unroll 1
             for (int ks = 0; ks < KS; ++ks) {
                 u32x4 q0[KD], q1[KD], za[RT];
-#pragma unroll
-                for (int kd = 0; kd < KD; ++kd) {
-                    const int ch = kd * 4 + g;
-                    q0[kd] = ch < CH ? qa[((2 * ks) * CH + ch) * 16 + c16] : zero4();
-                    q1[kd] = ch < CH ? qa[((2 * ks + 1) * CH + ch) * 16 + c16] : zero4();
-                }
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt) za[rt] = zt[(ks * RT + rt) * 64 + lane];
+                load_ops(ks, q0, q1, za);
 #pragma unroll
                 for (int tw = 0; tw < kSTW; ++tw) {
-                    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int kd = 0; kd < KD; ++kd) {
-                        s0 = M_::mma(q0[kd], kb[tw][kd], s0);
-                        s1 = M_::mma(q1[kd], kb[tw][kd], s1);
-                    }
+                    const f32x4 s0 = scores(q0, kb[tw]), s1 = scores(q1, kb[tw]);
                     float mx = fmaxf(fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])),
                                      fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
                     mx = xg_max(mx);
@@ -591,13 +602,15 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
         }
 
         // normalise and store: lane (token c16, group g) owns d = (D/4) g .. (D/4) g + D/4 - 1
+        const bool full = t0 + kSTokWave <= wg_n1 && mask == nullptr;   // wave-uniform: no per-row tests
+        uint16_t* yr0 = y + (int64_t)(t0 + c16) * a.ys[2] + (D / 4) * g;
 #pragma unroll
         for (int tw = 0; tw < kSTW; ++tw) {
             const int n = t0 + tw * 16 + c16;
-            const bool on = n < wg_n1 && (mask == nullptr || mask[n] != 0);
+            const bool on = full || (n < wg_n1 && (mask == nullptr || mask[n] != 0));
             const float inv = on ? 1.f / lrow[tw] : 0.f;
-            if (n < wg_n1) {
-                uint16_t* yr = y + (int64_t)n * a.ys[2] + (D / 4) * g;
+            if (full || n < wg_n1) {
+                uint16_t* yr = yr0 + (int64_t)tw * 16 * a.ys[2];
                 uint32_t o[2 * RT];
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
@@ -615,12 +628,19 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                 }
             }
         }
+    };
 
-        if (tnext < wg_n1) {
-#pragma unroll
-            for (int tw = 0; tw < kSTW; ++tw)
-#pragma unroll
-                for (int kd = 0; kd < KD; ++kd) kb[tw][kd] = kn[tw][kd];
+    // two K register sets alternate, each fetched one tile before its use
+    u32x4 ka[kSTW][KD], kc[kSTW][KD];
+    constexpr int kStride = 4 * kSTokWave;
+    int t0 = wg_n0 + w * kSTokWave;
+    if (t0 < wg_n1) load_k(t0, ka);
+    for (; t0 < wg_n1; t0 += 2 * kStride) {
+        if (t0 + kStride < wg_n1) load_k(t0 + kStride, kc);
+        tile64(ka, t0);
+        if (t0 + kStride < wg_n1) {
+            if (t0 + 2 * kStride < wg_n1) load_k(t0 + 2 * kStride, ka);
+            tile64(kc, t0 + kStride);
         }
     }
 }
@@ -697,7 +717,17 @@ template <typename T, int D>
 hipError_t scatter_launch(const MixerArgs& a, hipStream_t st)
 {
     const size_t lds = (size_t)a.M * D * 2 * 2;
-    auto kern = scatter_mfma_kernel<T, D>;
+    // the latent loop is unrolled at compile time for the usual latent counts at D <= 32
+    auto kern = scatter_mfma_kernel<T, D, 0>;
+    if constexpr (D <= 32) {
+        switch (a.M) {
+            case 64:  kern = scatter_mfma_kernel<T, D, 2>; break;
+            case 128: kern = scatter_mfma_kernel<T, D, 4>; break;
+            case 256: kern = scatter_mfma_kernel<T, D, 8>; break;
+            case 512: kern = scatter_mfma_kernel<T, D, 16>; break;
+            default: break;
+        }
+    }
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
