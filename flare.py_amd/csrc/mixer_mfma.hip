@@ -279,6 +279,42 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                         const uint2 hi = lds_read_tr16(&vt[buf][v_slot(r1, ch) + sub]);
                         va[rt] = u32x4{lo.x, lo.y, hi.x, hi.y};
                     }
+                    if constexpr (!EXACT && !RAGGED) {
+                        // steady state: latent tiles software pipelined (scores of tile ct+1 issued before
+                        // the exponentials of tile ct, value product of tile ct-1 after them)
+                        auto sc2 = [&](int ct, f32x4& s0, f32x4& s1) {
+                            s0 = f32x4{0.f, 0.f, 0.f, 0.f};
+                            s1 = s0;
+    #pragma unroll
+                            for (int kd = 0; kd < KD; ++kd) {
+                                s0 = M_::mma(ka0[kd], qb[ct][kd], s0);
+                                s1 = M_::mma(ka1[kd], qb[ct][kd], s1);
+                            }
+                        };
+                        auto pv = [&](int ct, u32x4 pb) {
+    #pragma unroll
+                            for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = P_::mma(va[rt], pb, zacc[rt][ct]);
+                            lacc[ct] = P_::mma(ones8, pb, lacc[ct]);   // row of ones: the softmax denominator
+                        };
+                        f32x4 s0, s1;
+                        sc2(0, s0, s1);
+                        u32x4 pbp = zero4();
+    #pragma unroll
+                        for (int ct = 0; ct < CT; ++ct) {
+                            f32x4 n0 = s0, n1 = s1;
+                            if (ct + 1 < CT) sc2(ct + 1, n0, n1);
+                            const u32x4 pb = {P_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])),
+                                              P_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
+                                              P_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])),
+                                              P_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]))};
+                            if (ct > 0) pv(ct - 1, pbp);
+                            s0 = n0;
+                            s1 = n1;
+                            pbp = pb;
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                        pv(CT - 1, pbp);
+                    } else
     #pragma unroll
                     for (int ct = 0; ct < CT; ++ct) {
                         f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
