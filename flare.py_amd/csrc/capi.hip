@@ -310,8 +310,9 @@ TriplePlan plan_triple(const FlareTripleDesc* d)
     p.mfma = triple_wants_mfma(d);
     int s = d->n_splits;
     if (s <= 0) {
+        // about two workgroups per compute unit: more splits only add partials to write and merge
         const int64_t per = (int64_t)d->B * d->H;
-        s = (int)((1024 + per - 1) / per);
+        s = (int)((512 + per - 1) / per);
         if (s < 1) s = 1;
     }
     int64_t tps = ((int64_t)d->N + s - 1) / s;

@@ -214,11 +214,19 @@ __global__ __launch_bounds__(256) void triple_out_mfma_kernel(TripleArgs a, int 
 
     const int wg_n0 = blockIdx.x * tokens_per_wg;
     const int wg_n1 = min(a.N, wg_n0 + tokens_per_wg);
-    for (int n0 = wg_n0 + w * 16; n0 < wg_n1; n0 += 64) {
+    // the features of the next tile are fetched while the current one is being worked on
+    auto fetch = [&](int n0, uint2& f1, uint2& f2) {
         const int n = n0 + tok;
         const bool live = n < wg_n1;
-        *reinterpret_cast<uint2*>(&q1s[w][tok][piece]) = load_feat4<T>(q1 + (int64_t)n * a.q1s[2] + piece, live, a.feature_map);
-        *reinterpret_cast<uint2*>(&q2s[w][tok][piece]) = load_feat4<T>(q2 + (int64_t)n * a.q2s[2] + piece, live, a.feature_map);
+        f1 = load_feat4<T>(q1 + (int64_t)n * a.q1s[2] + piece, live, a.feature_map);
+        f2 = load_feat4<T>(q2 + (int64_t)n * a.q2s[2] + piece, live, a.feature_map);
+    };
+    uint2 f1 = make_uint2(0u, 0u), f2 = f1;
+    if (wg_n0 + w * 16 < wg_n1) fetch(wg_n0 + w * 16, f1, f2);
+    for (int n0 = wg_n0 + w * 16; n0 < wg_n1; n0 += 64) {
+        *reinterpret_cast<uint2*>(&q1s[w][tok][piece]) = f1;
+        *reinterpret_cast<uint2*>(&q2s[w][tok][piece]) = f2;
+        if (n0 + 64 < wg_n1) fetch(n0 + 64, f1, f2);
 
         // A operand: row = token c16, k-slots i = 4g..4g+3
         const uint2 q1a = *reinterpret_cast<const uint2*>(&q1s[w][c16][4 * g]);
