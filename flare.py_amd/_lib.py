@@ -75,6 +75,9 @@ SYMBOLS = {
     "flare_mixer_workspace_bytes": (C.c_int, [C.POINTER(FlareMixerDesc), C.POINTER(_SZ)]),
     "flare_gather_fwd": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_scatter_fwd": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P]),
+    "flare_scatter_fwd_lse": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, _P]),
+    "flare_mixer_bwd_workspace_bytes": (C.c_int, [C.POINTER(FlareMixerDesc), C.POINTER(_SZ)]),
+    "flare_mixer_bwd": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, _P, _P, C.POINTER(C.c_int64), _P, _P, _P, _P, _SZ, _P]),
     "flare_mixer_fwd": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_causal_workspace_bytes": (C.c_int, [C.POINTER(FlareCausalDesc), C.POINTER(_SZ)]),
     "flare_causal_prefill_fwd": (C.c_int, [C.POINTER(FlareCausalDesc), _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),

@@ -157,13 +157,13 @@ int do_gather(const FlareMixerDesc* d, const void* q, const void* k, const void*
 }
 
 int do_scatter(const FlareMixerDesc* d, const void* q, const void* k, const float* z, const uint8_t* mask,
-               void* y, hipStream_t st)
+               void* y, hipStream_t st, float* lse_tok = nullptr)
 {
     const bool mfma = desc_wants_mfma(d) && mixer_ptrs_ok_for_mfma(d, q, k, nullptr, y);
     const MixerPlan p = plan_mixer(d, mfma);
     flare::MixerArgs a;
     fill_mixer_args(a, d, p, nullptr);
-    a.q = q; a.k = k; a.y = y; a.mask = mask; a.z = const_cast<float*>(z);
+    a.q = q; a.k = k; a.y = y; a.mask = mask; a.z = const_cast<float*>(z); a.lse_tok = lse_tok;
     hipError_t e = mfma ? flare::launch_scatter_mfma(a, d->dtype, st) : flare::launch_scatter_generic(a, d->dtype, st);
     return hip_status(e, "scatter launch");
 }
@@ -381,6 +381,97 @@ int flare_scatter_fwd(const FlareMixerDesc* desc, const void* q, const void* k, 
     if (rc != FLARE_OK) return rc;
     if (!q || !k || !z || !y) return fail(FLARE_EINVAL, "q, k, z and y must not be NULL");
     return do_scatter(desc, q, k, z, key_mask, y, static_cast<hipStream_t>(stream));
+}
+
+int flare_scatter_fwd_lse(const FlareMixerDesc* desc, const void* q, const void* k, const float* z,
+                          const uint8_t* key_mask, void* y, float* lse_tok, void* stream)
+{
+    int rc = check_mixer_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !z || !y) return fail(FLARE_EINVAL, "q, k, z, y must not be NULL");
+    return do_scatter(desc, q, k, z, key_mask, y, static_cast<hipStream_t>(stream), lse_tok);
+}
+
+namespace {
+struct BwdPlan { int n_splits, tokens_per_split; size_t off_dz, off_dl, off_part, total; };
+
+BwdPlan plan_bwd(const FlareMixerDesc* d)
+{
+    BwdPlan p;
+    const int64_t bh = (int64_t)d->B * d->H;
+    const int mblocks = d->M % 256 == 0 ? d->M / 256 : d->M % 128 == 0 ? d->M / 128 : d->M / 64;
+    // about two workgroups per compute unit over the latent-side grids, token ranges of 64 k tokens
+    int64_t s = std::max<int64_t>(1, 512 / (bh * mblocks));
+    int64_t tps = ((int64_t)d->N + s - 1) / s;
+    tps = (tps + 63) / 64 * 64;
+    p.tokens_per_split = (int)tps;
+    p.n_splits = (int)(((int64_t)d->N + tps - 1) / tps);
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    p.off_dz = up((size_t)bh * d->N * 4);
+    p.off_dl = p.off_dz + up((size_t)bh * d->M * d->D * 4);
+    p.off_part = p.off_dl + up((size_t)bh * d->M * 4);
+    p.total = p.off_part + (size_t)bh * p.n_splits * d->M * d->D * 4;
+    return p;
+}
+
+int check_bwd(const FlareMixerDesc* d)
+{
+    int rc = check_mixer_desc(d);
+    if (rc != FLARE_OK) return rc;
+    if (!flare::mixer_bwd_supported(d->dtype, d->M, d->D))
+        return fail(FLARE_EUNSUPPORTED, "mixer backward covers bf16/f16, D in {16,32,64}, M %% 64 == 0, 5*M*D*2 + 8*M <= 150 KB of LDS "
+                                        "(got dtype %d, M=%d, D=%d)", d->dtype, d->M, d->D);
+    if (!strides_mult8(d->q_stride) || !strides_mult8(d->k_stride) || !strides_mult8(d->v_stride) || !strides_mult8(d->y_stride))
+        return fail(FLARE_EUNSUPPORTED, "mixer backward needs strides that are multiples of 8 elements");
+    return FLARE_OK;
+}
+}  // namespace
+
+int flare_mixer_bwd_workspace_bytes(const FlareMixerDesc* desc, size_t* bytes)
+{
+    if (!bytes) return fail(FLARE_EINVAL, "bytes is NULL");
+    int rc = check_bwd(desc);
+    if (rc != FLARE_OK) return rc;
+    *bytes = plan_bwd(desc).total;
+    return FLARE_OK;
+}
+
+int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v, const void* y,
+                    const float* z, const float* lse_lat, const float* lse_tok, const void* dy,
+                    const int64_t dy_stride[3], float* dq, void* dk, void* dv,
+                    void* workspace, size_t workspace_bytes, void* stream)
+{
+    int rc = check_bwd(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !v || !y || !z || !lse_lat || !lse_tok || !dy || !dy_stride || !dq || !dk || !dv)
+        return fail(FLARE_EINVAL, "q, k, v, y, z, lse_lat, lse_tok, dy, dy_stride, dq, dk, dv must not be NULL");
+    if (!strides_mult8(dy_stride) || dy_stride[2] < desc->D) return fail(FLARE_EINVAL, "dy strides must be multiples of 8 and its rows >= D");
+    const void* ptrs[7] = {q, k, v, y, dy, dk, dv};
+    for (const void* p : ptrs)
+        if (!aligned16(p)) return fail(FLARE_EINVAL, "q, k, v, y, dy, dk, dv must be 16-byte aligned");
+    const BwdPlan p = plan_bwd(desc);
+    if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
+    if (workspace_bytes < p.total) return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, p.total);
+    if (!aligned16(workspace)) return fail(FLARE_EINVAL, "workspace must be 16-byte aligned");
+    flare::MixerBwdArgs a;
+    memset(&a, 0, sizeof(a));
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    a.q = q; a.k = k; a.v = v; a.y = y; a.dy = dy; a.z = z; a.lse_lat = lse_lat; a.lse_tok = lse_tok;
+    a.delta_tok = reinterpret_cast<float*>(ws);
+    a.dz = reinterpret_cast<float*>(ws + p.off_dz);
+    a.delta_lat = reinterpret_cast<float*>(ws + p.off_dl);
+    a.part = reinterpret_cast<float*>(ws + p.off_part);
+    a.dq = dq; a.dk = dk; a.dv = dv;
+    a.B = desc->B; a.H = desc->H; a.N = desc->N; a.M = desc->M; a.D = desc->D;
+    a.n_splits = p.n_splits; a.tokens_per_split = p.tokens_per_split;
+    a.scale = desc->scale; a.scale_log2 = desc->scale * 1.4426950408889634f;
+    const int64_t nd = (int64_t)desc->N * desc->D;
+    for (int i = 0; i < 3; ++i) {
+        a.qs[i] = desc->q_stride[i]; a.ks[i] = desc->k_stride[i]; a.vs[i] = desc->v_stride[i];
+        a.ys[i] = desc->y_stride[i]; a.dys[i] = dy_stride[i];
+    }
+    a.dks[0] = a.dvs[0] = (int64_t)desc->H * nd; a.dks[1] = a.dvs[1] = nd; a.dks[2] = a.dvs[2] = desc->D;
+    return hip_status(flare::launch_mixer_bwd(a, desc->dtype, static_cast<hipStream_t>(stream)), "mixer backward launch");
 }
 
 int flare_mixer_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,

@@ -39,6 +39,7 @@ struct MixerArgs {
     const uint8_t* mask;      // [B,N] or null
     float* z;                 // [B,H,M,D] fp32
     float* lse;               // [B,H,M] or null (natural log)
+    float* lse_tok;           // [B,H,N] or null: natural log of each token's softmax sum over the latents (scatter)
     float* part_m;            // [B,H,P,M]   per-partial running max (log2 units)
     float* part_l;            // [B,H,P,M]   per-partial sum
     float* part_acc;          // [B,H,P,M,D] per-partial numerator
@@ -72,6 +73,23 @@ struct TripleArgs {
     int n_splits, tokens_per_split;
     int n_parts;       // partials per (b,h) in `part`
     int64_t q1s[3], q2s[3], k1s[3], k2s[3], vs[3], os[3];
+};
+
+struct MixerBwdArgs {
+    const void* q; const void* k; const void* v; const void* y; const void* dy;
+    const float* z;          // [B,H,M,D] forward latent summary
+    const float* lse_lat;    // [B,H,M] natural log of the gather's softmax sums
+    const float* lse_tok;    // [B,H,N] natural log of the scatter's softmax sums
+    float* delta_tok;        // [B,H,N]   <dy_n, y_n>               (workspace)
+    float* dz;               // [B,H,M,D] gradient of z             (workspace)
+    float* delta_lat;        // [B,H,M]   <dz_m, z_m>               (workspace)
+    float* part;             // [B,H,P,M,D] split-N partial sums    (workspace)
+    float* dq;               // [B,H,M,D] fp32
+    void* dk; void* dv;      // [B,H,N,D] element type
+    int B, H, N, M, D;
+    int n_splits, tokens_per_split;
+    float scale, scale_log2;
+    int64_t qs[3], ks[3], vs[3], ys[3], dys[3], dks[3], dvs[3];
 };
 
 struct CausalLinearArgs {
@@ -115,6 +133,10 @@ hipError_t launch_causal_prefill(const CausalArgs& a, int dtype, hipStream_t st)
 hipError_t launch_causal_decode(const CausalArgs& a, int dtype, hipStream_t st);
 bool       causal_mfma_supported(int dtype, int M, int D);
 hipError_t launch_causal_mfma(const CausalArgs& a, int dtype, int step, hipStream_t st);   // step 16 prefill, 1 decode
+
+size_t     mixer_bwd_lds_bytes(int M, int D);
+bool       mixer_bwd_supported(int dtype, int M, int D);
+hipError_t launch_mixer_bwd(const MixerBwdArgs& a, int dtype, hipStream_t st);
 
 bool       mlp_mfma_supported(int w_dtype, int C);
 hipError_t launch_mlp_mfma(const MlpArgs& a, int w_dtype, hipStream_t st);

@@ -1,0 +1,580 @@
+// Backward of the FLARE mixer on the matrix cores (bf16 / f16, no key mask).
+//
+// Forward (README.md:39-52 of the reference):  S[m,n] = s <q_m,k_n>,  z_m = sum_n A[m,n] v_n with
+// A = softmax over n,  y_n = sum_m Bt[n,m] z_m with Bt = softmax over m.  With L_m, rho_n the two
+// log-sum-exps saved by the forward:  A[m,n] = exp(S - L_m) <= 1,  Bt[n,m] = exp(S - rho_n) <= 1.
+// Given dy:
+//   delta_n = <dy_n, y_n>                          (bwd_delta_kernel)
+//   dz_m    = sum_n Bt[n,m] dy_n                   (bwd_lat_kernel, MODE 0; split over N + merge)
+//   Delta_m = <dz_m, z_m>                          (merge)
+//   dS[m,n] = A (<dz_m,v_n> - Delta_m) + Bt (<dy_n,z_m> - delta_n)
+//   dv_n    = sum_m A[m,n] dz_m ;  dk_n = s sum_m dS[m,n] q_m      (bwd_tok_kernel, token parallel)
+//   dq_m    = s sum_n dS[m,n] k_n                  (bwd_lat_kernel, MODE 1; split over N + merge)
+// Both exponentials are bounded by 1, so no running maximum is needed anywhere.  The two kernel
+// shapes are those of the forward: "latent side" = the gather's (K/V/dY tiles of 64 tokens in LDS,
+// lane = latent, contraction over tokens), "token side" = the scatter's (latent operands in LDS,
+// lane = token, contraction over latents).  Score-like products <.,.> run on v_mfma_f32_16x16x32
+// exactly like the scores; their fp32 tiles line up element by element with the score tile, so dS
+// is assembled in registers and, packed to bf16, is the B operand of the last product.
+// q and k meet in the element type; every other product runs in bf16 (f16 tiles are converted while
+// they are staged), because dz, Delta and dS have no useful bound in f16.
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace flare {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mb;
+template <> struct Mb<bf16_t> {
+    static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        bf16x2 v = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float unpack(uint16_t b) { return __uint_as_float(uint32_t(b) << 16); }
+};
+template <> struct Mb<f16_t> {
+    static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        f16x2 v = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float unpack(uint16_t b) { return float(__builtin_bit_cast(_Float16, b)); }
+};
+using Pb = Mb<bf16_t>;
+
+__device__ __forceinline__ u32x4 zero4() { return u32x4{0u, 0u, 0u, 0u}; }
+__device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+
+// 8 packed elements of type T scaled by f, repacked in T
+template <typename T> __device__ __forceinline__ u32x4 scale8(u32x4 v, float f)
+{
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        o[i] = Mb<T>::pack2(Mb<T>::unpack(uint16_t(v[i] & 0xffffu)) * f, Mb<T>::unpack(uint16_t(v[i] >> 16)) * f);
+    return o;
+}
+// 8 packed elements of type T scaled by f, as packed bf16
+template <typename T> __device__ __forceinline__ u32x4 to_bf16x8(u32x4 v, float f = 1.f)
+{
+    if (std::is_same<T, bf16_t>::value && f == 1.f) return v;
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        o[i] = Pb::pack2(Mb<T>::unpack(uint16_t(v[i] & 0xffffu)) * f, Mb<T>::unpack(uint16_t(v[i] >> 16)) * f);
+    return o;
+}
+// 8 consecutive fp32 values as packed bf16
+__device__ __forceinline__ u32x4 pack8(const float* p)
+{
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+    return u32x4{Pb::pack2(a[0], a[1]), Pb::pack2(a[2], a[3]), Pb::pack2(b[0], b[1]), Pb::pack2(b[2], b[3])};
+}
+__device__ __forceinline__ u32x4 pack8(const float (&v)[8])
+{
+    return u32x4{Pb::pack2(v[0], v[1]), Pb::pack2(v[2], v[3]), Pb::pack2(v[4], v[5]), Pb::pack2(v[6], v[7])};
+}
+
+__device__ __forceinline__ uint2 lds_read_tr16(const void* lds_addr)
+{
+    typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
+    return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)lds_addr));
+}
+
+// ---- delta_n = <dy_n, y_n> -----------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void bwd_delta_kernel(MixerBwdArgs a)
+{
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t total = (int64_t)a.B * a.H * a.N;
+    if (idx >= total) return;
+    const int n = idx % a.N;
+    const int64_t bh = idx / a.N;
+    const int h = bh % a.H, b = bh / a.H;
+    const uint16_t* y = (const uint16_t*)a.y + b * a.ys[0] + h * a.ys[1] + (int64_t)n * a.ys[2];
+    const uint16_t* dy = (const uint16_t*)a.dy + b * a.dys[0] + h * a.dys[1] + (int64_t)n * a.dys[2];
+    float s = 0.f;
+    for (int d = 0; d < a.D; d += 8) {
+        const u32x4 u = load16(y + d), w = load16(dy + d);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            s = fmaf(Mb<T>::unpack(uint16_t(u[i] & 0xffffu)), Mb<T>::unpack(uint16_t(w[i] & 0xffffu)), s);
+            s = fmaf(Mb<T>::unpack(uint16_t(u[i] >> 16)), Mb<T>::unpack(uint16_t(w[i] >> 16)), s);
+        }
+    }
+    a.delta_tok[idx] = s;
+}
+
+// ---- latent side ---------------------------------------------------------------------------
+constexpr int kBTile = 64;   // tokens per LDS tile
+
+// One workgroup = 4 waves x (16 CT latents) x one token range.  MODE 0: dz partial; MODE 1: dq partial.
+template <typename T, int D, int CT, int MODE>
+__global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
+{
+    constexpr int KD = (D + 31) / 32, RT = D / 16, CH = D / 8, MB = 64 * CT, ROWB = D * 2, TILEB = kBTile * ROWB;
+    constexpr int NT = MODE == 0 ? 2 : 4;          // staged tiles: K rows, dY^T | K rows, K^T, V rows, dY rows
+    using M_ = Mb<T>;
+    __shared__ __attribute__((aligned(16))) uint8_t tl[2][NT][TILEB];
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int mblocks = a.M / MB;
+    const int split = blockIdx.x / mblocks, mb = blockIdx.x % mblocks;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int64_t bh = (int64_t)b * a.H + h;
+    const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
+    const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
+    const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
+    const uint16_t* dy = (const uint16_t*)a.dy + b * a.dys[0] + h * a.dys[1];
+    const float* rho = a.lse_tok + bh * a.N;
+    const float* dlt = a.delta_tok + bh * a.N;
+    const int m_base = mb * MB + w * 16 * CT;
+
+    // latent operands (B of the score-like products) and per-latent scalars
+    u32x4 qb[CT][KD], dzb[CT][KD], zb[CT][KD];
+    float l2m[CT], dm[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int m = m_base + ct * 16 + c16;
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) {
+            const int ch = kd * 4 + g;
+            qb[ct][kd] = ch < CH ? scale8<T>(load16(q + (int64_t)m * a.qs[2] + ch * 8), a.scale_log2) : zero4();
+            if (MODE == 1) {
+                dzb[ct][kd] = ch < CH ? pack8(a.dz + (bh * a.M + m) * D + ch * 8) : zero4();
+                zb[ct][kd] = ch < CH ? pack8(a.z + (bh * a.M + m) * D + ch * 8) : zero4();
+            }
+        }
+        if (MODE == 1) {
+            l2m[ct] = a.lse_lat[bh * a.M + m] * kLog2e;
+            dm[ct] = a.delta_lat[bh * a.M + m];
+        }
+    }
+
+    const int n_begin = split * a.tokens_per_split;
+    const int n_end = min(a.N, n_begin + a.tokens_per_split);
+
+    constexpr int TCH = kBTile * CH;
+    constexpr int CPT = (TCH + 255) / 256;
+    auto k_slot = [](int tok, int ch) { return tok * ROWB + ((ch ^ ((tok >> 2) & (CH - 1))) << 4); };
+    auto v_slot = [](int tok, int ch) { return tok * ROWB + ((CH >= 4 ? (ch ^ (((tok >> 2) & 1) << 1)) : ch) << 4); };
+
+    u32x4 kr[CPT], vr[CPT], yr[CPT];
+    auto load_tile = [&](int n0) {
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int c = tid + i * 256;
+            if (c < TCH) {
+                const int n = min(n0 + c / CH, n_end - 1), ch = c % CH;
+                kr[i] = load16(k + (int64_t)n * a.ks[2] + ch * 8);
+                yr[i] = load16(dy + (int64_t)n * a.dys[2] + ch * 8);
+                if (MODE == 1) vr[i] = load16(v + (int64_t)n * a.vs[2] + ch * 8);
+            }
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < CPT; ++i) {
+            const int c = tid + i * 256;
+            if (c < TCH) {
+                const int tok = c / CH, ch = c % CH;
+                *reinterpret_cast<u32x4*>(&tl[buf][0][k_slot(tok, ch)]) = kr[i];
+                if (MODE == 0) {
+                    *reinterpret_cast<u32x4*>(&tl[buf][1][v_slot(tok, ch)]) = to_bf16x8<T>(yr[i]);
+                } else {
+                    *reinterpret_cast<u32x4*>(&tl[buf][1][v_slot(tok, ch)]) = to_bf16x8<T>(kr[i]);
+                    *reinterpret_cast<u32x4*>(&tl[buf][2][k_slot(tok, ch)]) = to_bf16x8<T>(vr[i]);
+                    *reinterpret_cast<u32x4*>(&tl[buf][3][k_slot(tok, ch)]) = to_bf16x8<T>(yr[i]);
+                }
+            }
+        }
+    };
+
+    f32x4 acc[RT][CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) acc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
+
+    auto process = [&](int n0, int buf) {
+#pragma unroll
+        for (int ks = 0; ks < kBTile / 32; ++ks) {
+            u32x4 ka0[KD], ka1[KD], va0[KD], va1[KD], ya0[KD], ya1[KD], tr[RT];
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                const int ch = kd * 4 + g, t0 = ks * 32 + c16, t1 = t0 + 16;
+                ka0[kd] = ch < CH ? *reinterpret_cast<const u32x4*>(&tl[buf][0][k_slot(t0, ch)]) : zero4();
+                ka1[kd] = ch < CH ? *reinterpret_cast<const u32x4*>(&tl[buf][0][k_slot(t1, ch)]) : zero4();
+                if (MODE == 1) {
+                    va0[kd] = ch < CH ? *reinterpret_cast<const u32x4*>(&tl[buf][2][k_slot(t0, ch)]) : zero4();
+                    va1[kd] = ch < CH ? *reinterpret_cast<const u32x4*>(&tl[buf][2][k_slot(t1, ch)]) : zero4();
+                    ya0[kd] = ch < CH ? *reinterpret_cast<const u32x4*>(&tl[buf][3][k_slot(t0, ch)]) : zero4();
+                    ya1[kd] = ch < CH ? *reinterpret_cast<const u32x4*>(&tl[buf][3][k_slot(t1, ch)]) : zero4();
+                }
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                // transposed tile (dY^T or K^T): rows d, k-slots = the 8 tokens of this lane group
+                const int r0 = ks * 32 + 4 * g + (c16 >> 2), r1 = r0 + 16;
+                const int ch = 2 * rt + ((c16 & 3) >> 1), sub = (c16 & 1) << 3;
+                const uint2 lo = lds_read_tr16(&tl[buf][1][v_slot(r0, ch) + sub]);
+                const uint2 hi = lds_read_tr16(&tl[buf][1][v_slot(r1, ch) + sub]);
+                tr[rt] = u32x4{lo.x, lo.y, hi.x, hi.y};
+            }
+            // per-token scalars of the 8 tokens (rows) this lane holds: e < 4 -> 4g+e, else 16+4g+e-4
+            float r2[8], de[8];
+            bool ok[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int n = n0 + ks * 32 + (e >> 2) * 16 + 4 * g + (e & 3);
+                ok[e] = n < n_end;
+                const int nc = ok[e] ? n : n_end - 1;
+                r2[e] = rho[nc] * kLog2e;
+                de[e] = MODE == 1 ? dlt[nc] : 0.f;
+            }
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                f32x4 s0 = zf, s1 = zf;
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) {
+                    s0 = M_::mma(ka0[kd], qb[ct][kd], s0);
+                    s1 = M_::mma(ka1[kd], qb[ct][kd], s1);
+                }
+                const float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+                float o[8];
+                if (MODE == 0) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) o[e] = ok[e] ? fast_exp2(sc[e] - r2[e]) : 0.f;
+                } else {
+                    f32x4 g10 = zf, g11 = zf, g20 = zf, g21 = zf;
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) {
+                        g10 = Pb::mma(va0[kd], dzb[ct][kd], g10);
+                        g11 = Pb::mma(va1[kd], dzb[ct][kd], g11);
+                        g20 = Pb::mma(ya0[kd], zb[ct][kd], g20);
+                        g21 = Pb::mma(ya1[kd], zb[ct][kd], g21);
+                    }
+                    const float g1[8] = {g10[0], g10[1], g10[2], g10[3], g11[0], g11[1], g11[2], g11[3]};
+                    const float g2[8] = {g20[0], g20[1], g20[2], g20[3], g21[0], g21[1], g21[2], g21[3]};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float av = fast_exp2(sc[e] - l2m[ct]), bv = fast_exp2(sc[e] - r2[e]);
+                        const float ds = av * (g1[e] - dm[ct]) + bv * (g2[e] - de[e]);
+                        o[e] = ok[e] ? ds : 0.f;
+                    }
+                }
+                const u32x4 ob = pack8(o);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) acc[rt][ct] = Pb::mma(tr[rt], ob, acc[rt][ct]);
+            }
+        }
+    };
+
+    if (n_begin < n_end) {
+        load_tile(n_begin);
+        store_tile(0);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int n0 = n_begin; n0 < n_end; n0 += kBTile, buf ^= 1) {
+        const bool more = n0 + kBTile < n_end;
+        if (more) load_tile(n0 + kBTile);
+        process(n0, buf);
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int m = m_base + ct * 16 + c16;
+        const int64_t row = ((int64_t)bh * a.n_splits + split) * a.M + m;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) *reinterpret_cast<f32x4*>(a.part + row * D + rt * 16 + 4 * g) = acc[rt][ct];
+    }
+}
+
+// MODE 0: dz = sum of partials, Delta_m = <dz_m, z_m>;  MODE 1: dq = scale * sum of partials.
+// One thread per (b,h,m); the partials are summed in split order (bit-stable).
+template <int MODE>
+__global__ __launch_bounds__(256) void bwd_merge_kernel(MixerBwdArgs a)
+{
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;   // (b*H + h)*M + m
+    if (r >= (int64_t)a.B * a.H * a.M) return;
+    const int m = r % a.M;
+    const int64_t bh = r / a.M;
+    const float* p0 = a.part + (bh * a.n_splits * a.M + m) * a.D;
+    const int64_t sp = (int64_t)a.M * a.D;
+    float delta = 0.f;
+    for (int d = 0; d < a.D; d += 4) {
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < a.n_splits; ++p) s += *reinterpret_cast<const f32x4*>(p0 + p * sp + d);
+        if (MODE == 0) {
+            *reinterpret_cast<f32x4*>(a.dz + r * a.D + d) = s;
+            const f32x4 zz = *reinterpret_cast<const f32x4*>(a.z + r * a.D + d);
+            delta += s[0] * zz[0] + s[1] * zz[1] + s[2] * zz[2] + s[3] * zz[3];
+        } else {
+            *reinterpret_cast<f32x4*>(a.dq + r * a.D + d) = s * a.scale;
+        }
+    }
+    if (MODE == 0) a.delta_lat[r] = delta;
+}
+
+// ---- token side ----------------------------------------------------------------------------
+constexpr int kBTW = 2;   // 16-token column tiles per wave iteration
+
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void bwd_tok_kernel(MixerBwdArgs a, int tokens_per_wg)
+{
+    constexpr int KD = (D + 31) / 32, RT = D / 16, CH = D / 8;
+    using M_ = Mb<T>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int M = a.M, KS = M / 32;
+    // A-operand layout [mt][ch][c16] for q (scaled, log2 units), dz, z;  PV-operand layout
+    // [ks][rt][lane] for dz^T and (scale q)^T;  per-latent scalars
+    u32x4* qa = reinterpret_cast<u32x4*>(smem);
+    u32x4* dza = qa + (size_t)M * CH;
+    u32x4* zza = dza + (size_t)M * CH;
+    u32x4* dzt = zza + (size_t)M * CH;
+    u32x4* qt = dzt + (size_t)M * CH;
+    float* l2 = reinterpret_cast<float*>(qt + (size_t)M * CH);
+    float* dl = l2 + M;
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int64_t bh = (int64_t)b * a.H + h;
+    const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
+    const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
+    const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
+    const uint16_t* dy = (const uint16_t*)a.dy + b * a.dys[0] + h * a.dys[1];
+    uint16_t* dk = (uint16_t*)a.dk + b * a.dks[0] + h * a.dks[1];
+    uint16_t* dv = (uint16_t*)a.dv + b * a.dvs[0] + h * a.dvs[1];
+    const float* z = a.z + bh * M * D;
+    const float* dz = a.dz + bh * M * D;
+    const float* rho = a.lse_tok + bh * a.N;
+    const float* dlt = a.delta_tok + bh * a.N;
+
+    for (int idx = tid; idx < M * CH; idx += 256) {
+        const int m = idx / CH, ch = idx % CH;
+        const int slot = ((m >> 4) * CH + ch) * 16 + (m & 15);
+        qa[slot] = scale8<T>(load16(q + (int64_t)m * a.qs[2] + ch * 8), a.scale_log2);
+        dza[slot] = pack8(dz + (int64_t)m * D + ch * 8);
+        zza[slot] = pack8(z + (int64_t)m * D + ch * 8);
+    }
+    for (int idx = tid; idx < KS * RT * 64; idx += 256) {
+        const int ln = idx & 63, rt = (idx >> 6) % RT, ks = idx / (64 * RT);
+        const int cc = ln & 15, gg = ln >> 4;
+        const int d = (D / 4) * (cc >> 2) + 4 * rt + (cc & 3);
+        u32x4 o1, o2;
+#pragma unroll
+        for (int e2 = 0; e2 < 4; ++e2) {
+            const int e = 2 * e2;
+            const int m0 = 32 * ks + (e >> 2) * 16 + 4 * gg + (e & 3);
+            o1[e2] = Pb::pack2(dz[(int64_t)m0 * D + d], dz[(int64_t)(m0 + 1) * D + d]);
+            o2[e2] = Pb::pack2(M_::unpack(q[(int64_t)m0 * a.qs[2] + d]) * a.scale, M_::unpack(q[(int64_t)(m0 + 1) * a.qs[2] + d]) * a.scale);
+        }
+        dzt[idx] = o1;
+        qt[idx] = o2;
+    }
+    for (int m = tid; m < M; m += 256) {
+        l2[m] = a.lse_lat[bh * M + m] * kLog2e;
+        dl[m] = a.delta_lat[bh * M + m];
+    }
+    __syncthreads();
+
+    const int wg_n0 = blockIdx.x * tokens_per_wg;
+    const int wg_n1 = min(a.N, wg_n0 + tokens_per_wg);
+    const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
+
+    for (int t0 = wg_n0 + w * 16 * kBTW; t0 < wg_n1; t0 += 4 * 16 * kBTW) {
+        u32x4 kb[kBTW][KD], vb[kBTW][KD], yb[kBTW][KD];
+        float r2[kBTW], de[kBTW];
+#pragma unroll
+        for (int tw = 0; tw < kBTW; ++tw) {
+            const int n = t0 + tw * 16 + c16;
+            const bool live = n < wg_n1;
+            const int nc = live ? n : wg_n1 - 1;
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                const int ch = kd * 4 + g;
+                const bool in = live && ch < CH;
+                kb[tw][kd] = in ? load16(k + (int64_t)n * a.ks[2] + ch * 8) : zero4();
+                vb[tw][kd] = in ? to_bf16x8<T>(load16(v + (int64_t)n * a.vs[2] + ch * 8)) : zero4();
+                yb[tw][kd] = in ? to_bf16x8<T>(load16(dy + (int64_t)n * a.dys[2] + ch * 8)) : zero4();
+            }
+            r2[tw] = rho[nc] * kLog2e;
+            de[tw] = dlt[nc];
+        }
+        f32x4 adk[kBTW][RT], adv[kBTW][RT];
+#pragma unroll
+        for (int tw = 0; tw < kBTW; ++tw)
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) adk[tw][rt] = adv[tw][rt] = zf;
+
+        for (int ks = 0; ks < KS; ++ks) {
+            u32x4 q0[KD], q1[KD], d0[KD], d1[KD], z0[KD], z1[KD], odz[RT], oq[RT];
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) {
+                const int ch = kd * 4 + g;
+                const int s0 = ((2 * ks) * CH + ch) * 16 + c16, s1 = ((2 * ks + 1) * CH + ch) * 16 + c16;
+                q0[kd] = ch < CH ? qa[s0] : zero4();
+                q1[kd] = ch < CH ? qa[s1] : zero4();
+                d0[kd] = ch < CH ? dza[s0] : zero4();
+                d1[kd] = ch < CH ? dza[s1] : zero4();
+                z0[kd] = ch < CH ? zza[s0] : zero4();
+                z1[kd] = ch < CH ? zza[s1] : zero4();
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                odz[rt] = dzt[(ks * RT + rt) * 64 + lane];
+                oq[rt] = qt[(ks * RT + rt) * 64 + lane];
+            }
+            // per-latent scalars of the 8 latents (rows) this lane holds
+            const f32x4 la = *reinterpret_cast<const f32x4*>(l2 + 32 * ks + 4 * g), lb = *reinterpret_cast<const f32x4*>(l2 + 32 * ks + 16 + 4 * g);
+            const f32x4 da = *reinterpret_cast<const f32x4*>(dl + 32 * ks + 4 * g), db = *reinterpret_cast<const f32x4*>(dl + 32 * ks + 16 + 4 * g);
+            const float lm[8] = {la[0], la[1], la[2], la[3], lb[0], lb[1], lb[2], lb[3]};
+            const float dm[8] = {da[0], da[1], da[2], da[3], db[0], db[1], db[2], db[3]};
+#pragma unroll
+            for (int tw = 0; tw < kBTW; ++tw) {
+                f32x4 s0 = zf, s1 = zf, g10 = zf, g11 = zf, g20 = zf, g21 = zf;
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) {
+                    s0 = M_::mma(q0[kd], kb[tw][kd], s0);
+                    s1 = M_::mma(q1[kd], kb[tw][kd], s1);
+                    g10 = Pb::mma(d0[kd], vb[tw][kd], g10);
+                    g11 = Pb::mma(d1[kd], vb[tw][kd], g11);
+                    g20 = Pb::mma(z0[kd], yb[tw][kd], g20);
+                    g21 = Pb::mma(z1[kd], yb[tw][kd], g21);
+                }
+                const float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+                const float g1[8] = {g10[0], g10[1], g10[2], g10[3], g11[0], g11[1], g11[2], g11[3]};
+                const float g2[8] = {g20[0], g20[1], g20[2], g20[3], g21[0], g21[1], g21[2], g21[3]};
+                float av[8], ds[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    av[e] = fast_exp2(sc[e] - lm[e]);
+                    const float bv = fast_exp2(sc[e] - r2[tw]);
+                    ds[e] = av[e] * (g1[e] - dm[e]) + bv * (g2[e] - de[tw]);
+                }
+                const u32x4 pa = pack8(av), pd = pack8(ds);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    adv[tw][rt] = Pb::mma(odz[rt], pa, adv[tw][rt]);
+                    adk[tw][rt] = Pb::mma(oq[rt], pd, adk[tw][rt]);
+                }
+            }
+        }
+
+        // lane (token c16, group g) owns d = (D/4) g .. (D/4) g + D/4 - 1 of both gradients
+#pragma unroll
+        for (int tw = 0; tw < kBTW; ++tw) {
+            const int n = t0 + tw * 16 + c16;
+            if (n >= wg_n1) continue;
+            auto put = [&](uint16_t* base, int64_t stride, const f32x4 (&acc)[RT]) {
+                uint16_t* p = base + (int64_t)n * stride + (D / 4) * g;
+                uint32_t o[2 * RT];
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    o[2 * rt] = M_::pack2(acc[rt][0], acc[rt][1]);
+                    o[2 * rt + 1] = M_::pack2(acc[rt][2], acc[rt][3]);
+                }
+                if constexpr (RT == 1) {
+                    *reinterpret_cast<uint2*>(p) = make_uint2(o[0], o[1]);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < RT / 2; ++i)
+                        *reinterpret_cast<u32x4*>(p + 8 * i) = u32x4{o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+                }
+            };
+            put(dk, a.dks[2], adk[tw]);
+            put(dv, a.dvs[2], adv[tw]);
+        }
+    }
+}
+
+template <typename T, int D, int MODE>
+hipError_t lat_launch(const MixerBwdArgs& a, hipStream_t st)
+{
+    // 4 latent tiles per wave need too many registers at D = 64 in the dq pass
+    if (a.M % 256 == 0 && !(D == 64 && MODE == 1)) {
+        hipLaunchKernelGGL((bwd_lat_kernel<T, D, 4, MODE>), dim3(a.n_splits * (a.M / 256), a.H, a.B), dim3(256), 0, st, a);
+    } else if (a.M % 128 == 0) {
+        hipLaunchKernelGGL((bwd_lat_kernel<T, D, 2, MODE>), dim3(a.n_splits * (a.M / 128), a.H, a.B), dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((bwd_lat_kernel<T, D, 1, MODE>), dim3(a.n_splits * (a.M / 64), a.H, a.B), dim3(256), 0, st, a);
+    }
+    return hipGetLastError();
+}
+
+template <typename T, int D>
+hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
+{
+    const int64_t tok = (int64_t)a.B * a.H * a.N, lat = (int64_t)a.B * a.H * a.M;
+    hipLaunchKernelGGL(bwd_delta_kernel<T>, dim3((unsigned)((tok + 255) / 256)), dim3(256), 0, st, a);
+    hipError_t e = lat_launch<T, D, 0>(a, st);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(bwd_merge_kernel<0>, dim3((unsigned)((lat + 255) / 256)), dim3(256), 0, st, a);
+    {
+        auto kern = bwd_tok_kernel<T, D>;
+        const size_t lds = mixer_bwd_lds_bytes(a.M, D);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        // about two workgroups per compute unit, ranges a multiple of 128 tokens
+        const int64_t per_bh = (512 + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H);
+        int64_t tpw = (a.N + per_bh - 1) / per_bh;
+        tpw = ((tpw + 127) / 128) * 128;
+        if (tpw < 512) tpw = 512;
+        hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(256), lds, st, a, (int)tpw);
+    }
+    e = lat_launch<T, D, 1>(a, st);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(bwd_merge_kernel<1>, dim3((unsigned)((lat + 255) / 256)), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t bwd_d(const MixerBwdArgs& a, hipStream_t st)
+{
+    switch (a.D) {
+        case 16: return bwd_all<T, 16>(a, st);
+        case 32: return bwd_all<T, 32>(a, st);
+        case 64: return bwd_all<T, 64>(a, st);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+size_t mixer_bwd_lds_bytes(int M, int D) { return (size_t)M * D * 2 * 5 + (size_t)M * 8; }
+
+bool mixer_bwd_supported(int dtype, int M, int D)
+{
+    return (dtype == 1 || dtype == 2) && (D == 16 || D == 32 || D == 64) && M >= 64 && M % 64 == 0 &&
+           mixer_bwd_lds_bytes(M, D) <= 150 * 1024;
+}
+
+hipError_t launch_mixer_bwd(const MixerBwdArgs& a, int dtype, hipStream_t st)
+{
+    return dtype == 1 ? bwd_d<bf16_t>(a, st) : bwd_d<f16_t>(a, st);
+}
+
+}  // namespace flare

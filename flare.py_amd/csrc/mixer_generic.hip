@@ -201,6 +201,7 @@ __global__ __launch_bounds__(kScatterThreads) void scatter_generic_kernel(MixerA
     if (live) {
         const bool on = a.mask ? a.mask[(int64_t)b * a.N + n] != 0 : true;
         const float inv = on ? 1.f / l : 0.f;
+        if (a.lse_tok) a.lse_tok[((int64_t)b * a.H + h) * a.N + n] = (mx + __log2f(l)) * kLn2;
         T* y = (T*)a.y + b * a.ys[0] + h * a.ys[1] + (int64_t)n * a.ys[2];
 #pragma unroll
         for (int d = 0; d < DMAX; ++d)

@@ -525,7 +525,10 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
     auto tile64 = [&](const u32x4 (&kb)[kSTW][KD], int t0) {
         f32x4 yacc[kSTW][RT];
         float lrow[kSTW];       // softmax denominators, complete for the lane's token
+        float lshift[kSTW];     // log2 shift the denominators are relative to (0 in the optimistic pass)
         bool redo = false;
+#pragma unroll
+        for (int tw = 0; tw < kSTW; ++tw) lshift[tw] = 0.f;
         {
             // Optimistic pass: no softmax shift at all.  fp32 and bf16 share an 8-bit exponent, so
             // exp2(score) is exact enough whenever the scores of a token stay inside (-60, 120);
@@ -634,7 +637,10 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                 }
             }
 #pragma unroll
-            for (int tw = 0; tw < kSTW; ++tw) lrow[tw] = xg_sum(lsum[tw]);
+            for (int tw = 0; tw < kSTW; ++tw) {
+                lrow[tw] = xg_sum(lsum[tw]);
+                lshift[tw] = shift[tw];
+            }
         }
 
         // normalise and store: lane (token c16, group g) owns d = (D/4) g .. (D/4) g + D/4 - 1
@@ -645,6 +651,8 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
             const int n = t0 + tw * 16 + c16;
             const bool on = full || (n < wg_n1 && (mask == nullptr || mask[n] != 0));
             const float inv = on ? 1.f / lrow[tw] : 0.f;
+            if (a.lse_tok && g == 0 && (full || n < wg_n1))
+                a.lse_tok[((int64_t)b * a.H + h) * a.N + n] = (lshift[tw] + __log2f(lrow[tw])) * kLn2;
             if (full || n < wg_n1) {
                 uint16_t* yr = yr0 + (int64_t)tw * 16 * a.ys[2];
                 uint32_t o[2 * RT];

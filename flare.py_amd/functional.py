@@ -121,7 +121,8 @@ def _autocast_dtype(t):
     return None
 
 
-def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major=False):
+def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major=False, want_lse=False):
+    """y, z (and with want_lse the two log-sum-exps the HIP backward needs)."""
     _require_cuda(q, k, v)
     lib = _lib.load()
     if q.dtype != k.dtype:
@@ -143,16 +144,66 @@ def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_majo
     need = C.c_size_t(0)
     _lib.check(lib.flare_mixer_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_workspace_bytes")
     ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
+    st = C.c_void_p(_stream_ptr(k.device))
+    if want_lse:
+        lse_lat = torch.empty((B, H, M), dtype=torch.float32, device=k.device)
+        lse_tok = torch.empty((B, H, N), dtype=torch.float32, device=k.device)
+        with torch.cuda.device(k.device):
+            rc = lib.flare_gather_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(mask), _ptr(z), _ptr(lse_lat),
+                                      _ptr(ws), ws.numel(), st)
+            _lib.check(rc, "flare_gather_fwd")
+            rc = lib.flare_scatter_fwd_lse(C.byref(d), _ptr(q4), _ptr(k), _ptr(z), _ptr(mask), _ptr(y), _ptr(lse_tok), st)
+        _lib.check(rc, "flare_scatter_fwd_lse")
+        return y, z, lse_lat, lse_tok
     with torch.cuda.device(k.device):
         rc = lib.flare_mixer_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(mask), _ptr(y), _ptr(z),
-                                 _ptr(ws), ws.numel(), C.c_void_p(_stream_ptr(k.device)))
+                                 _ptr(ws), ws.numel(), st)
     _lib.check(rc, "flare_mixer_fwd")
     return y, z
 
 
+def _hip_backward_ok(q, k, v, key_mask, force_generic) -> bool:
+    """True when flare_mixer_bwd covers this problem (16-bit types, no mask, supported M, D, strides)."""
+    if key_mask is not None or force_generic or k.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    if q.dtype != k.dtype or v.dtype != k.dtype or k.device.type != "cuda":
+        return False
+    k, v = _rows_last_contig(k), _rows_last_contig(v)
+    q4 = _q4(q, k.shape[0])
+    d = _mixer_desc(q4, k, v, None, 1.0, 0, False)
+    need = C.c_size_t(0)
+    return _lib.load().flare_mixer_bwd_workspace_bytes(C.byref(d), C.byref(need)) == _lib.FLARE_OK
+
+
+def _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy):
+    """dq, dk, dv from the HIP backward kernels (flare_mixer_bwd)."""
+    lib = _lib.load()
+    k, v = _rows_last_contig(k), _rows_last_contig(v)
+    B, H, N, D = k.shape
+    q4 = _q4(q, B)
+    M = q4.shape[2]
+    gy = gy.to(k.dtype)
+    if gy.stride(-1) != 1 or any(s % 8 for s in gy.stride()[:3]) or gy.data_ptr() % 16:
+        gy = gy.contiguous()
+    d = _mixer_desc(q4, k, v, y, scale, 0, False)
+    dq = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
+    dk = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    dv = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    need = C.c_size_t(0)
+    _lib.check(lib.flare_mixer_bwd_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_bwd_workspace_bytes")
+    ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
+    with torch.cuda.device(k.device):
+        rc = lib.flare_mixer_bwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(y), _ptr(z), _ptr(lse_lat), _ptr(lse_tok),
+                                 _ptr(gy), _s3(gy), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(),
+                                 C.c_void_p(_stream_ptr(k.device)))
+    _lib.check(rc, "flare_mixer_bwd")
+    gq = dq.sum(0) if q.dim() == 3 else dq
+    return gq.to(q.dtype), dk, dv
+
+
 def _mixer_torch_grad(q, k, v, scale, key_mask, gy):
-    """Backward by recomputation in plain torch ops on the device the inputs live on.
-    The HIP backward kernels are not built yet; the forward never takes this path."""
+    """Backward by recomputation in plain torch ops on the device the inputs live on: used for what
+    the HIP backward does not cover (fp32, key masks, unusual shapes).  The forward never takes this path."""
     with torch.enable_grad():
         q_, k_, v_ = (t.detach().float().requires_grad_(True) for t in (q, k, v))
         qe = q_ if q_.dim() == 4 else q_.unsqueeze(0)
@@ -173,16 +224,25 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy):
 class _MixerFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, scale, key_mask, n_splits, force_generic, token_major):
-        y, z = _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major)
-        ctx.save_for_backward(q, k, v)
         ctx.scale, ctx.key_mask = scale, key_mask
+        ctx.hip = _hip_backward_ok(q, k, v, key_mask, force_generic)
+        if ctx.hip:
+            y, z, lse_lat, lse_tok = _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major, True)
+            ctx.save_for_backward(q, k, v, y, z, lse_lat, lse_tok)
+        else:
+            y, z = _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major)
+            ctx.save_for_backward(q, k, v)
         ctx.mark_non_differentiable(z)
         return y, z
 
     @staticmethod
     def backward(ctx, gy, _gz):
-        q, k, v = ctx.saved_tensors
-        gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy)
+        if ctx.hip:
+            q, k, v, y, z, lse_lat, lse_tok = ctx.saved_tensors
+            gq, gk, gv = _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, ctx.scale, gy)
+        else:
+            q, k, v = ctx.saved_tensors
+            gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy)
         return gq, gk, gv, None, None, None, None, None
 
 

@@ -14,6 +14,9 @@
  *                              pdebench/models/flare.py:136-138, lra/models/backends.py:603-606
  *   flare_gather_fwd           first F.scaled_dot_product_attention(q, k, v) of the above
  *   flare_scatter_fwd          second F.scaled_dot_product_attention(k, q, z) of the above
+ *   flare_scatter_fwd_lse      the same, also returning each token's log-sum-exp over the latents
+ *   flare_mixer_bwd            gradient of flare_multihead_mixer (torch autograd through the two SDPA
+ *                              calls upstream; ablation/time_memory_bwd.py:460-478 times fwd+bwd)
  *   flare_causal_prefill_fwd   causal restriction of the mixer (README.md:60 names it; the
  *   flare_causal_decode_fwd    reference holds no code for it) following the 3-phase chunk
  *                              scheme of lra/models/triton/causal_linear.py:81-137 and the
@@ -175,6 +178,22 @@ int flare_gather_fwd(const FlareMixerDesc* desc, const void* q, const void* k, c
 /* y[B,H,N,D] = softmax_m(s k q^T) z.  Rows of masked tokens are written as 0. */
 int flare_scatter_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const float* z,
                       const uint8_t* key_mask, void* y, void* stream);
+
+/* flare_scatter_fwd plus lse_tok (fp32 [B,H,N], may be NULL): natural log of sum_m exp(s <k_n,q_m>),
+ * which the backward pass needs. */
+int flare_scatter_fwd_lse(const FlareMixerDesc* desc, const void* q, const void* k, const float* z,
+                          const uint8_t* key_mask, void* y, float* lse_tok, void* stream);
+
+/* Backward of the mixer (no key mask; bf16 / f16; the shapes flare_mixer_bwd_workspace_bytes accepts).
+ * Inputs: q, k, v as in the forward; y and z its outputs; lse_lat = lse of flare_gather_fwd;
+ * lse_tok of flare_scatter_fwd_lse; dy [B,H,N,D] with strides dy_stride.
+ * Outputs: dq fp32 [B,H,M,D] contiguous (per batch element: sum over b when q is shared);
+ * dk, dv [B,H,N,D] contiguous in the element type. */
+int flare_mixer_bwd_workspace_bytes(const FlareMixerDesc* desc, size_t* bytes);
+int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v, const void* y,
+                    const float* z, const float* lse_lat, const float* lse_tok, const void* dy,
+                    const int64_t dy_stride[3], float* dq, void* dk, void* dv,
+                    void* workspace, size_t workspace_bytes, void* stream);
 
 /* gather + merge + scatter on one stream.  z_out (fp32 [B,H,M,D]) may be NULL, in which
  * case z lives in the workspace. */
