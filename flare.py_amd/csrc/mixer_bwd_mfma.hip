@@ -135,6 +135,7 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
     constexpr int NT = MODE == 0 ? 2 : 4;          // staged tiles: K rows, dY^T | K rows, K^T, V rows, dY rows
     using M_ = Mb<T>;
     __shared__ __attribute__((aligned(16))) uint8_t tl[2][NT][TILEB];
+    __shared__ __attribute__((aligned(16))) float tsc[2][2][kBTile];   // per-token scalars of a tile: rho * log2(e), delta
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
     const int mblocks = a.M / MB;
@@ -179,7 +180,13 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
     auto v_slot = [](int tok, int ch) { return tok * ROWB + ((CH >= 4 ? (ch ^ (((tok >> 2) & 1) << 1)) : ch) << 4); };
 
     u32x4 kr[CPT], vr[CPT], yr[CPT];
+    float rr = 0.f, dd = 0.f;
     auto load_tile = [&](int n0) {
+        if (tid < kBTile) {
+            const int n = min(n0 + tid, n_end - 1);
+            rr = rho[n] * kLog2e;
+            if (MODE == 1) dd = dlt[n];
+        }
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * 256;
@@ -192,6 +199,10 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
         }
     };
     auto store_tile = [&](int buf) {
+        if (tid < kBTile) {
+            tsc[buf][0][tid] = rr;
+            tsc[buf][1][tid] = dd;
+        }
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * 256;
@@ -244,13 +255,17 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
             // per-token scalars of the 8 tokens (rows) this lane holds: e < 4 -> 4g+e, else 16+4g+e-4
             float r2[8], de[8];
             bool ok[8];
+            {
+                const int tb = ks * 32 + 4 * g;
+                const f32x4 ra = *reinterpret_cast<const f32x4*>(&tsc[buf][0][tb]), rb = *reinterpret_cast<const f32x4*>(&tsc[buf][0][tb + 16]);
+                const f32x4 da = *reinterpret_cast<const f32x4*>(&tsc[buf][1][tb]), db = *reinterpret_cast<const f32x4*>(&tsc[buf][1][tb + 16]);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int n = n0 + ks * 32 + (e >> 2) * 16 + 4 * g + (e & 3);
-                ok[e] = n < n_end;
-                const int nc = ok[e] ? n : n_end - 1;
-                r2[e] = rho[nc] * kLog2e;
-                de[e] = MODE == 1 ? dlt[nc] : 0.f;
+                for (int e = 0; e < 4; ++e) {
+                    r2[e] = ra[e]; r2[e + 4] = rb[e];
+                    de[e] = da[e]; de[e + 4] = db[e];
+                    ok[e] = n0 + tb + e < n_end;
+                    ok[e + 4] = n0 + tb + 16 + e < n_end;
+                }
             }
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
@@ -340,12 +355,12 @@ __global__ __launch_bounds__(256) void bwd_merge_kernel(MixerBwdArgs a)
 }
 
 // ---- token side ----------------------------------------------------------------------------
-constexpr int kBTW = 2;   // 16-token column tiles per wave iteration
 
 template <typename T, int D>
 __global__ __launch_bounds__(256, 2) void bwd_tok_kernel(MixerBwdArgs a, int tokens_per_wg)
 {
     constexpr int KD = (D + 31) / 32, RT = D / 16, CH = D / 8;
+    constexpr int kBTW = D <= 32 ? 4 : 2;   // 16-token column tiles per wave iteration (registers allow 2 at D = 64)
     using M_ = Mb<T>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int M = a.M, KS = M / 32;
@@ -541,7 +556,7 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
         // about two workgroups per compute unit, ranges a multiple of 128 tokens
         const int64_t per_bh = (512 + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H);
         int64_t tpw = (a.N + per_bh - 1) / per_bh;
-        tpw = ((tpw + 127) / 128) * 128;
+        tpw = ((tpw + 255) / 256) * 256;
         if (tpw < 512) tpw = 512;
         hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(256), lds, st, a, (int)tpw);
     }
