@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FLARE mixer forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block|train]
 
 One step = one forward of the mixer (split-N gather, merge, scatter) over the headline workload
 B=1, H=8, N=1,048,576, M=256, D=32, bf16 in / fp32 accumulate, inputs resident in HBM.
@@ -12,7 +12,8 @@ machine's host cores on a bounded sample of the same workload.
 --workload selects one of the other configurations instead (same JSON shape, one line): causal =
 causal FLARE prefill of 8192 tokens + 256 decode steps at B=8,H=16,M=128,D=64; triple = triple
 attention at B=4,H=8,N=16384,D=16 (elu+1, normalised); block = one FLAREBlock forward at
-B=4,N=65536,C=128,H=8,M=128 under bf16 autocast (torch layers around the HIP mixer).
+B=4,N=65536,C=128,H=8,M=128 under bf16 autocast (fused HIP launches around the HIP mixer); train =
+the headline configuration with the backward pass (HIP kernels both ways).
 """
 from __future__ import annotations
 
@@ -172,6 +173,31 @@ def bench_triple(args, F, dev):
     return out
 
 
+def bench_train(args, F, dev):
+    """Headline configuration, forward + backward of the mixer (HIP kernels both ways)."""
+    B, H, N, M, D = 1, 8, 1 << 20, 256, 32
+    q, k, v = make_inputs(B, H, N, M, D, torch.bfloat16, dev)
+    gy = torch.randn_like(k)
+    qd, kd, vd = (t.detach().requires_grad_(True) for t in (q, k, v))
+
+    def step():
+        F.flare_multihead_mixer(qd, kd, vd).backward(gy)
+        qd.grad = kd.grad = vd.grad = None
+
+    ms_step = wall_ms(step, args.steps, args.warmup)
+    ms_fwd = time_events(lambda: F.flare_multihead_mixer(q, k, v), args.steps, 2)
+    flops = 8 * B * H * N * M * D * 3.75          # forward 4 products of 2*N*M*D, backward 11
+    nbytes = B * H * N * D * 2 * (4 + 9)          # forward K,V,K,Y; backward y,dy | K,dY | K,V,dY,dK,dV | K,V,dY
+    t_roof = max(nbytes / (HBM_PEAK_GBPS * 1e9), flops / (MFMA_BF16_PEAK_TFLOPS * 1e12))
+    out = base_record(args, "FLARE mixer forward+backward tokens/sec at N=1M,M=256,D=32 bf16", B * N / (ms_step * 1e-3),
+                      "tokens/s", ms_step, "FLARE mixer forward + backward B=1,H=8,N=1048576,M=256,D=32 (BASELINE config 3 with gradients)")
+    out["roofline"] = {"bound": "mfma", "kernel": "forward + backward kernels together", "achieved": round(flops / (ms_step * 1e-3) / 1e12, 1),
+                       "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / (ms_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                       "traffic": None, "algorithmic_flops": flops, "algorithmic_bytes": nbytes,
+                       "frac_of_roofline_time": round(t_roof * 1e3 / ms_step, 4), "ms_forward_only": round(ms_fwd, 4)}
+    return out
+
+
 def bench_block(args, F, dev):
     """BASELINE config 2: one FLAREBlock forward (LayerNorm, k/v ResidualMLPs, HIP mixer, out_proj, FFN)."""
     torch.manual_seed(0)
@@ -207,7 +233,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-sample", type=int, default=1048576, help="tokens of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block"], default="mixer",
+    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train"], default="mixer",
                     help="mixer = the headline configuration (default); the others are BASELINE configs 4, 5, 2")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -222,7 +248,7 @@ def main():
 
     dev = torch.device("cuda:0")
     if args.workload != "mixer":
-        fn = {"causal": bench_causal, "triple": bench_triple, "block": bench_block}[args.workload]
+        fn = {"causal": bench_causal, "triple": bench_triple, "block": bench_block, "train": bench_train}[args.workload]
         print(json.dumps(fn(args, F, dev)))
         return
     B, H, N, M, D = 1, 8, 1 << 20, 256, 32
