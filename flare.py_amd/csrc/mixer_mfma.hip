@@ -18,6 +18,7 @@
 //
 //   gather : z = softmax_n(s q k^T) v   split over N, partial (shift, sum, numerator)
 //   scatter: y = softmax_m(s k q^T) z   token parallel, Q and Z^T resident in LDS
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
@@ -699,6 +700,8 @@ int resident_slots(const void* kern, size_t dyn_lds, int block_threads = 256)
     struct Entry { const void* k; size_t lds; int dev; int slots; };
     static Entry cache[64];
     static int ncache = 0;
+    static std::mutex mu;     // the cache is the only mutable state of the library: guard it
+    std::lock_guard<std::mutex> lock(mu);
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return 512; }
     for (int i = 0; i < ncache; ++i)

@@ -120,3 +120,38 @@ def test_status_to_exception_mapping():
         _lib.check(_lib.FLARE_EUNSUPPORTED, "x")
     with pytest.raises(RuntimeError):
         _lib.check(_lib.FLARE_EHIP, "x")
+
+
+def test_new_struct_sizes_and_entry_point_validation():
+    assert C.sizeof(_lib.FlareCausalLinearDesc) == 8 * 4 + 4 * 24
+    assert C.sizeof(_lib.FlareMlpDesc) == 8 + 12 * 4 + 3 * 8
+    lib = _lib.load()
+    # fused MLP: argument checks happen before anything is launched
+    m = _lib.FlareMlpDesc()
+    m.T, m.C, m.L, m.w_dtype = 16, 128, 2, _lib.DT_BF16
+    m.x_stride = m.y_stride = 128
+    assert lib.flare_mlp_fwd(m, None, None, None, None, None, None, None, None) == _lib.FLARE_EINVAL
+    assert "must not be NULL" in _lib.last_error()
+    m.C = 48
+    assert lib.flare_mlp_fwd(m, None, None, None, None, None, None, None, None) == _lib.FLARE_EUNSUPPORTED
+    m.C, m.L = 128, 0
+    assert lib.flare_mlp_fwd(m, None, None, None, None, None, None, None, None) == _lib.FLARE_EINVAL
+    m.L, m.w_dtype = 2, _lib.DT_F32
+    assert lib.flare_mlp_fwd(m, None, None, None, None, None, None, None, None) == _lib.FLARE_EINVAL
+    # causal linear attention
+    c = _lib.FlareCausalLinearDesc()
+    c.B, c.H, c.N, c.Dk, c.Dv, c.dtype = 1, 2, 100, 32, 16, _lib.DT_F32
+    c.q_stride = c.k_stride = _lib.I3(6400, 3200, 32)
+    c.v_stride = c.y_stride = _lib.I3(3200, 1600, 16)
+    need = C.c_size_t(0)
+    assert lib.flare_causal_linear_workspace_bytes(c, C.byref(need)) == _lib.FLARE_OK and need.value > 0
+    assert lib.flare_causal_linear_fwd(c, None, None, None, None, None, 0, None) == _lib.FLARE_EINVAL
+    c.Dk = 200
+    assert lib.flare_causal_linear_workspace_bytes(c, C.byref(need)) == _lib.FLARE_EUNSUPPORTED
+    # mixer backward: supported shapes only, workspace checked
+    d = _mixer_desc(M=128, D=32)
+    assert lib.flare_mixer_bwd_workspace_bytes(d, C.byref(need)) == _lib.FLARE_OK and need.value > 0
+    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(dtype=_lib.DT_F32), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
+    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=256, D=64), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
+    assert lib.flare_mixer_bwd(d, *([None] * 8), None, None, None, None, None, 0, None) == _lib.FLARE_EINVAL
+    assert lib.flare_scatter_fwd_lse(d, None, None, None, None, None, None, None) == _lib.FLARE_EINVAL
