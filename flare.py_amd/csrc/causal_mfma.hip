@@ -197,6 +197,91 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step
         }
     };
 
+    if constexpr (STATE_ONLY) {
+        // Local state of the segment.  A 16-token block is too little work here to cover the memory
+        // latency of its own prefetch, so this phase walks 64-token tiles: K as four A operands per
+        // lane, V through a 64-row LDS tile, the next tile in flight while the current is used.
+        __shared__ __attribute__((aligned(16))) uint16_t v64[2][64][D];
+        constexpr int VPT = (64 * (D / 8) + 255) / 256;     // 16-byte V chunks per thread and tile
+        u32x4 k4[4][KD], k4n[4][KD], vreg[VPT];
+        auto load64 = [&](int n0, u32x4 (&kk)[4][KD]) {
+#pragma unroll
+            for (int sb = 0; sb < 4; ++sb) {
+                const int n = min(n0 + sb * 16 + c16, N - 1);
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) kk[sb][kd] = *reinterpret_cast<const u32x4*>(k + (int64_t)n * a.ks[2] + kd * 32 + g * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                const int c = tid + i * 256, tok = c / (D / 8), ch = c % (D / 8);
+                if (c < 64 * (D / 8)) vreg[i] = *reinterpret_cast<const u32x4*>(v + (int64_t)min(n0 + tok, N - 1) * a.vs[2] + ch * 8);
+            }
+        };
+        auto store64 = [&](int buf) {
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                const int c = tid + i * 256, tok = c / (D / 8), ch = c % (D / 8);
+                if (c < 64 * (D / 8)) {
+                    u32x4 o = vreg[i];
+                    if constexpr (!std::is_same<T, bf16_t>::value) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            o[j] = P_::pack2(M_::unpack(uint16_t(vreg[i][j] & 0xffffu)), M_::unpack(uint16_t(vreg[i][j] >> 16)));
+                    }
+                    *reinterpret_cast<u32x4*>(&v64[buf][tok][ch * 8]) = o;
+                }
+            }
+        };
+        load64(n_lo, k4);
+        store64(0);
+        if (n_lo + 64 < N) load64(n_lo + 64, k4n);
+        __syncthreads();
+        int it = 0;
+        for (int n0 = n_lo; n0 < N; n0 += 64, ++it) {
+            const int buf = it & 1;
+#pragma unroll
+            for (int sb = 0; sb < 4; ++sb) {
+                const int tb = N - (n0 + sb * 16);   // rows >= tb are beyond the segment
+                uint2 vop[DT];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) vop[dt] = tr16(&v64[buf][sb * 16 + 4 * g + (c16 >> 2)][dt * 16 + (c16 & 3) * 4]);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    f32x4 s = negmu[ct];
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) s = M_::mma32(k4[sb][kd], qb[ct][kd], s);
+                    float p[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) p[r] = (4 * g + r < tb) ? fast_exp2(s[r]) : 0.f;
+                    const uint2 ppk = make_uint2(P_::pack2(p[0], p[1]), P_::pack2(p[2], p[3]));
+                    den[ct] = P_::mma16(ones4, ppk, den[ct]);
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) U[ct][dt] = P_::mma16(ppk, vop[dt], U[ct][dt]);
+                }
+            }
+            if (n0 + 64 < N) {
+#pragma unroll
+                for (int sb = 0; sb < 4; ++sb)
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) k4[sb][kd] = k4n[sb][kd];
+                store64(buf ^ 1);
+                if (n0 + 128 < N) load64(n0 + 128, k4n);
+            }
+            __syncthreads();
+        }
+        // local state of the segment, relative to the shift of the incoming state; whatever
+        // overflowed or vanished here is caught by the checks of the segments that use it
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            if (g == 0) seg_den[m0 + ct * 16 + c16] = den[ct][0];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) seg_num[(int64_t)(m0 + ct * 16 + 4 * g + r) * D + dt * 16 + c16] = U[ct][dt][r];
+        }
+        return;
+    }
+
     bool bad = false;
     load_block(n_lo, ka);
     store_v(0);
@@ -220,25 +305,6 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step
 #pragma unroll
             for (int r = 0; r < 4; ++r) p[ct][r] = (4 * g + r < tb) ? fast_exp2(s[r]) : 0.f;
             ppk[ct] = make_uint2(P_::pack2(p[ct][0], p[ct][1]), P_::pack2(p[ct][2], p[ct][3]));
-        }
-        if constexpr (STATE_ONLY) {
-            uint2 vop[DT];
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vop[dt] = tr16(&vs[buf][4 * g + (c16 >> 2)][dt * 16 + (c16 & 3) * 4]);
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) {
-                den[ct] = P_::mma16(ones4, ppk[ct], den[ct]);
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) U[ct][dt] = P_::mma16(ppk[ct], vop[dt], U[ct][dt]);
-            }
-            if (n0 + step < N) {
-#pragma unroll
-                for (int kd = 0; kd < KD; ++kd) ka[kd] = kn[kd];
-                store_v(buf ^ 1);
-                if (n0 + 2 * step < N) load_block(n0 + 2 * step, kn);
-            }
-            __syncthreads();
-            continue;
         }
         // running denominators: dcum = den + L P ; den += 1 P ; G = P / dcum
 #pragma unroll
@@ -330,20 +396,6 @@ __global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step
                     make_uint2(M_::pack2(o[0], o[1]), M_::pack2(o[2], o[3]));
             }
         }
-    }
-
-    if constexpr (STATE_ONLY) {
-        // local state of the segment, relative to the shift of the incoming state; whatever
-        // overflowed or vanished here is caught by the checks of the segments that use it
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            if (g == 0) seg_den[m0 + ct * 16 + c16] = den[ct][0];
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) seg_num[(int64_t)(m0 + ct * 16 + 4 * g + r) * D + dt * 16 + c16] = U[ct][dt][r];
-        }
-        return;
     }
 
     // validate the final denominators, then publish the state (or the redo flag).  With several
