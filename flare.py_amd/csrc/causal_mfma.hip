@@ -75,8 +75,13 @@ template <> struct Mm<f16_t> {
 
 __device__ __forceinline__ uint2 tr16(const void* lds_addr)
 {
+    // The pointer reaches the intrinsic through an integer cast, so the compiler may not see that it
+    // aliases the ordinary stores that fill the tile: keep it from moving either across the read.
     typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
-    return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)lds_addr));
+    asm volatile("" ::: "memory");
+    const s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)lds_addr);
+    asm volatile("" ::: "memory");
+    return __builtin_bit_cast(uint2, r);
 }
 
 constexpr int kTB = 16;   // tokens per block
@@ -86,7 +91,7 @@ constexpr int kTB = 16;   // tokens per block
 // segment writes the state back itself; with several, the last one stages it in the workspace.
 // STATE_ONLY = true: only the segment's local denominators and numerators (first phase).
 template <typename T, int D, int KM, bool STATE_ONLY>
-__global__ __launch_bounds__(256) void causal_mfma_kernel(CausalArgs a, int step)
+__global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int step)
 {
     constexpr int KD = D / 32;          // k-steps over d of the score product
     constexpr int DT = D / 16;          // 16-column tiles of d

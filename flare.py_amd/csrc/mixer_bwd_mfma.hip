@@ -96,8 +96,13 @@ __device__ __forceinline__ u32x4 pack8(const float (&v)[8])
 
 __device__ __forceinline__ uint2 lds_read_tr16(const void* lds_addr)
 {
+    // The pointer reaches the intrinsic through an integer cast, so the compiler may not see that it
+    // aliases the ordinary stores that fill the tile: keep it from moving either across the read.
     typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
-    return __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)lds_addr));
+    asm volatile("" ::: "memory");
+    const s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)lds_addr);
+    asm volatile("" ::: "memory");
+    return __builtin_bit_cast(uint2, r);
 }
 
 // ---- delta_n = <dy_n, y_n> -----------------------------------------------------------------

@@ -148,8 +148,12 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 // tile; lane i of the group receives element i of the four rows named by lane quads 0..3.
 __device__ __forceinline__ uint2 lds_read_tr16(const void* lds_addr)
 {
+    // The pointer reaches the intrinsic through an integer cast, so the compiler may not see that it
+    // aliases the ordinary stores that fill the tile: keep it from moving either across the read.
     typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
+    asm volatile("" ::: "memory");
     const s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)lds_addr);
+    asm volatile("" ::: "memory");
     return __builtin_bit_cast(uint2, r);
 }
 
