@@ -503,6 +503,93 @@ def _triple_forward(q1, q2, k1, k2, v, feature_map: bool, normalize: bool, n_spl
     return state, out
 
 
+def _triple_desc(a, b, vlike, out):
+    B, H, N, Dq = a.shape
+    d = FlareTripleDesc()
+    d.B, d.H, d.N, d.Dq, d.Dv = B, H, N, Dq, vlike.shape[-1]
+    d.dtype = _dtype_code(a)
+    d.q1_stride = d.k1_stride = _s3(a)
+    d.q2_stride = d.k2_stride = _s3(b)
+    d.v_stride = _s3(vlike)
+    d.o_stride = _s3(out if out is not None else vlike)
+    return d
+
+
+def _triple_state(k1, k2, v):
+    """state [B,H,Dq,Dv,Dq] fp32 = (1/N) sum_n k1[n,i] v[n,j] k2[n,k]  (flare_triple_state_fwd)."""
+    lib = _lib.load()
+    k1, k2, v = (_rows_last_contig(t) for t in (k1, k2, v))
+    B, H, N, Dq = k1.shape
+    state = torch.empty((B, H, Dq, v.shape[-1], Dq), dtype=torch.float32, device=k1.device)
+    d = _triple_desc(k1, k2, v, None)
+    need = C.c_size_t(0)
+    _lib.check(lib.flare_triple_workspace_bytes(C.byref(d), C.byref(need)), "flare_triple_workspace_bytes")
+    ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k1.device)
+    with torch.cuda.device(k1.device):
+        rc = lib.flare_triple_state_fwd(C.byref(d), _ptr(k1), _ptr(k2), _ptr(v), _ptr(state), None, _ptr(ws), ws.numel(),
+                                        C.c_void_p(_stream_ptr(k1.device)))
+    _lib.check(rc, "flare_triple_state_fwd")
+    return state
+
+
+def _triple_out(q1, q2, state):
+    """out [B,H,N,Dv] = sum_{i,k} q1[n,i] state[i,j,k] q2[n,k]  (flare_triple_out_fwd)."""
+    lib = _lib.load()
+    q1, q2 = _rows_last_contig(q1), _rows_last_contig(q2)
+    state = state.to(torch.float32).contiguous()
+    B, H, N, Dq = q1.shape
+    out = torch.empty((B, H, N, state.shape[3]), dtype=q1.dtype, device=q1.device)
+    d = _triple_desc(q1, q2, out, out)
+    with torch.cuda.device(q1.device):
+        rc = lib.flare_triple_out_fwd(C.byref(d), _ptr(q1), _ptr(q2), _ptr(state), None, _ptr(out),
+                                      C.c_void_p(_stream_ptr(q1.device)))
+    _lib.check(rc, "flare_triple_out_fwd")
+    return out
+
+
+class _TripleFn(torch.autograd.Function):
+    """(STATE, O) = triple attention with the gradients of lra/models/triton/triple.py:124-135.  Every
+    gradient is again a state or an output contraction, so for Dq == Dv the backward runs on the
+    same two HIP kernels with permuted states; otherwise it is the reference's einsum formulas."""
+
+    @staticmethod
+    def forward(ctx, q1, q2, k1, k2, v):
+        state, out = _triple_forward(q1, q2, k1, k2, v, False, False)
+        ctx.save_for_backward(q1, q2, k1, k2, v, state)
+        return state, out
+
+    @staticmethod
+    def backward(ctx, dstate, dout):
+        q1, q2, k1, k2, v, state = ctx.saved_tensors
+        N = q1.shape[2]
+        dt = q1.dtype
+        if dout is None:
+            dout = torch.zeros_like(v)
+        if q1.shape[-1] == v.shape[-1]:
+            do = dout.to(dt)
+            dq1 = _triple_out(do, q2, state.permute(0, 1, 3, 2, 4))        # sum_{j,k} dO[n,j] S[i,j,k] q2[n,k]
+            dq2 = _triple_out(q1, do, state.permute(0, 1, 2, 4, 3))        # sum_{i,j} q1[n,i] S[i,j,k] dO[n,j]
+            ds = _triple_state(q1, q2, do) * float(N)                      # sum_n q1[n,i] dO[n,j] q2[n,k]
+            if dstate is not None:
+                ds = ds + dstate.float()
+            ds = ds / N
+            dk1 = _triple_out(v, k2, ds.permute(0, 1, 3, 2, 4))
+            dk2 = _triple_out(k1, v, ds.permute(0, 1, 2, 4, 3))
+            dv = _triple_out(k1, k2, ds)
+            return dq1, dq2, dk1, dk2, dv
+        f = lambda t: t.float()
+        do = f(dout)
+        dq1 = torch.einsum("bhnj,bhijk,bhnk->bhni", do, state, f(q2))
+        dq2 = torch.einsum("bhnj,bhni,bhijk->bhnk", do, f(q1), state)
+        ds = torch.einsum("bhnj,bhni,bhnk->bhijk", do, f(q1), f(q2))
+        if dstate is not None:
+            ds = ds + dstate.float()
+        dk1 = torch.einsum("bhijk,bhnj,bhnk->bhni", ds, f(v), f(k2)) / N
+        dk2 = torch.einsum("bhijk,bhni,bhnj->bhnk", ds, f(k1), f(v)) / N
+        dv = torch.einsum("bhijk,bhni,bhnk->bhnj", ds, f(k1), f(k2)) / N
+        return dq1.to(dt), dq2.to(dt), dk1.to(dt), dk2.to(dt), dv.to(dt)
+
+
 def triple_attention(q1, q2, k1, k2, v, normalize: bool = False, feature_map: Optional[str] = None,
                      n_splits: int = 0):
     """Third-order linear attention (lra/models/backends.py:1285-1292 of the reference).
@@ -514,13 +601,19 @@ def triple_attention(q1, q2, k1, k2, v, normalize: bool = False, feature_map: Op
     """
     if feature_map not in (None, "identity", "elu"):
         raise ValueError("feature_map must be None, 'identity' or 'elu'")
+    needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q1, q2, k1, k2, v))
+    if needs_grad:
+        if normalize or feature_map == "elu":
+            raise NotImplementedError("gradients of triple_attention are available for feature_map=None, "
+                                      "normalize=False (apply the feature map in torch, as the reference does)")
+        return _TripleFn.apply(q1, q2, k1, k2, v)
     return _triple_forward(q1, q2, k1, k2, v, feature_map == "elu", normalize, n_splits)
 
 
 class TripleAttentionFunction:
     """Call-compatible stand-in for lra/models/triton/triple.py:27 `TripleAttentionFunction`:
-    `TripleAttentionFunction.apply(Q1, Q2, K1, K2, V) -> (STATE, O)`.  Forward only."""
+    `TripleAttentionFunction.apply(Q1, Q2, K1, K2, V) -> (STATE, O)`, differentiable like the original."""
 
     @staticmethod
     def apply(Q1, Q2, K1, K2, V):
-        return _triple_forward(Q1, Q2, K1, K2, V, False, False)
+        return triple_attention(Q1, Q2, K1, K2, V)

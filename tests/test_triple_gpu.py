@@ -72,3 +72,22 @@ def test_cfg5_shape(dev):
     st, out = F.triple_attention(*[t.to(dev) for t in a], normalize=True, feature_map="elu")
     sr, orf = O.triple_einsum(*[t.float() for t in a], feature_map=True, normalize=True)
     assert O.rel_l2(st, sr) <= 1e-2 and O.rel_l2(out, orf) <= 2e-2
+
+
+@pytest.mark.parametrize("dtype,D,Dv,tol", [(torch.float32, 16, 16, 1e-4), (torch.bfloat16, 16, 16, 3e-2), (torch.float32, 8, 12, 1e-4)])
+def test_backward_matches_autograd_of_the_einsum_oracle(dev, dtype, D, Dv, tol):
+    # gradients of lra/models/triton/triple.py:124-135, including a gradient flowing into STATE
+    g = torch.Generator().manual_seed(11)
+    B, H, N = 1, 2, 300
+    ins = [(torch.randn(B, H, N, D, generator=g) * 0.5).to(dtype) for _ in range(4)] + [torch.randn(B, H, N, Dv, generator=g).to(dtype)]
+    gs = torch.randn(B, H, D, Dv, D, generator=g)
+    go = torch.randn(B, H, N, Dv, generator=g).to(dtype)
+    dins = [t.to(dev).requires_grad_(True) for t in ins]
+    st, out = F.TripleAttentionFunction.apply(*dins)
+    (st * gs.to(dev)).sum().add((out.float() * go.to(dev).float()).sum()).backward()
+    rins = [t.double().requires_grad_(True) for t in ins]
+    sr, orf = O.triple_einsum(*rins, dtype=torch.float64)
+    ((sr * gs.double()).sum() + (orf * go.double()).sum()).backward()
+    for name, a, b in zip(("dq1", "dq2", "dk1", "dk2", "dv"), dins, rins):
+        err = O.rel_l2(a.grad, b.grad)
+        assert err <= tol, f"{name}: {err:.3e}"
