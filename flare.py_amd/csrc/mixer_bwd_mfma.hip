@@ -361,9 +361,14 @@ __global__ __launch_bounds__(256) void bwd_merge_kernel(MixerBwdArgs a)
 
 // ---- token side ----------------------------------------------------------------------------
 
+// The five latent-side operand sets fill most of a CU's LDS at the usual sizes (82 KB at M = 256,
+// D = 32), so only one workgroup fits: it has 8 waves, two per SIMD, all reading the same operands.
+constexpr int kTokWaves = 8;
+
 template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void bwd_tok_kernel(MixerBwdArgs a, int tokens_per_wg)
+__global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs a, int tokens_per_wg)
 {
+    constexpr int NTH = 64 * kTokWaves;
     constexpr int KD = (D + 31) / 32, RT = D / 16, CH = D / 8;
     constexpr int kBTW = D <= 32 ? 4 : 2;   // 16-token column tiles per wave iteration (registers allow 2 at D = 64)
     using M_ = Mb<T>;
@@ -393,14 +398,14 @@ __global__ __launch_bounds__(256, 2) void bwd_tok_kernel(MixerBwdArgs a, int tok
     const float* rho = a.lse_tok + bh * a.N;
     const float* dlt = a.delta_tok + bh * a.N;
 
-    for (int idx = tid; idx < M * CH; idx += 256) {
+    for (int idx = tid; idx < M * CH; idx += NTH) {
         const int m = idx / CH, ch = idx % CH;
         const int slot = ((m >> 4) * CH + ch) * 16 + (m & 15);
         qa[slot] = scale8<T>(load16(q + (int64_t)m * a.qs[2] + ch * 8), a.scale_log2);
         dza[slot] = pack8(dz + (int64_t)m * D + ch * 8);
         zza[slot] = pack8(z + (int64_t)m * D + ch * 8);
     }
-    for (int idx = tid; idx < KS * RT * 64; idx += 256) {
+    for (int idx = tid; idx < KS * RT * 64; idx += NTH) {
         const int ln = idx & 63, rt = (idx >> 6) % RT, ks = idx / (64 * RT);
         const int cc = ln & 15, gg = ln >> 4;
         const int d = (D / 4) * (cc >> 2) + 4 * rt + (cc & 3);
@@ -415,7 +420,7 @@ __global__ __launch_bounds__(256, 2) void bwd_tok_kernel(MixerBwdArgs a, int tok
         dzt[idx] = o1;
         qt[idx] = o2;
     }
-    for (int m = tid; m < M; m += 256) {
+    for (int m = tid; m < M; m += NTH) {
         l2[m] = a.lse_lat[bh * M + m] * kLog2e;
         dl[m] = a.delta_lat[bh * M + m];
     }
@@ -425,7 +430,7 @@ __global__ __launch_bounds__(256, 2) void bwd_tok_kernel(MixerBwdArgs a, int tok
     const int wg_n1 = min(a.N, wg_n0 + tokens_per_wg);
     const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
 
-    for (int t0 = wg_n0 + w * 16 * kBTW; t0 < wg_n1; t0 += 4 * 16 * kBTW) {
+    for (int t0 = wg_n0 + w * 16 * kBTW; t0 < wg_n1; t0 += kTokWaves * 16 * kBTW) {
         u32x4 kb[kBTW][KD], vb[kBTW][KD], yb[kBTW][KD];
         float r2[kBTW], de[kBTW];
 #pragma unroll
@@ -558,12 +563,11 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
         const size_t lds = mixer_bwd_lds_bytes(a.M, D);
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        // about two workgroups per compute unit, ranges a multiple of 128 tokens
-        const int64_t per_bh = (512 + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H);
+        // one workgroup per compute unit (256 CUs), ranges a multiple of its 512-token pass
+        const int64_t per_bh = (256 + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H);
         int64_t tpw = (a.N + per_bh - 1) / per_bh;
-        tpw = ((tpw + 255) / 256) * 256;
-        if (tpw < 512) tpw = 512;
-        hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(256), lds, st, a, (int)tpw);
+        tpw = ((tpw + 511) / 512) * 512;
+        hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(64 * kTokWaves), lds, st, a, (int)tpw);
     }
     e = lat_launch<T, D, 1>(a, st);
     if (e != hipSuccess) return e;
