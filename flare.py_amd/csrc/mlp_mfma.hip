@@ -112,8 +112,10 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
     constexpr int NCH = (C * C / 8 + NT - 1) / NT;   // 16-byte weight chunks per thread and layer
     constexpr int FT = C / 16;        // feature tiles of the stream
     constexpr int KS = C / 32;        // k-steps of one layer
-    constexpr int RS = C * 2 + 16;    // LDS row stride in bytes (padded: conflict-free 16-byte reads)
-    constexpr int WBUF = C * RS;
+    constexpr int RS = C * 2;         // LDS row stride in bytes; no padding: the 16-byte chunks of a row are
+    constexpr int WBUF = C * RS;      // XOR-swizzled with the row number so that 16 rows read 16 different bank groups
+    constexpr int CPR = C / 8;        // 16-byte chunks per row
+    constexpr int SWS = CPR == 16 ? 0 : CPR == 8 ? 1 : 2;   // swizzle key of row r: ((r & 15) >> SWS), below CPR
     constexpr int TOKW = 16 * TW;     // tokens per wave and pass
     using M_ = Mm<T>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -137,13 +139,19 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
                 const int row = c / (C / 8), ch = c % (C / 8);
                 // features 8 ch .. 8 ch + 3 belong to k-step ch / 4, half (ch % 4) / 2, lane group 2 (ch % 2);
                 // features 8 ch + 4 .. + 7 to the next lane group.  Position = 32 ks + 8 g + 4 half.
-                const int pos = 32 * (ch >> 2) + 16 * (ch & 1) + 4 * ((ch & 3) >> 1);
-                uint8_t* dst = smem + slot * WBUF + row * RS + pos * 2;
-                *reinterpret_cast<uint2*>(dst) = make_uint2(wreg[i][0], wreg[i][1]);
-                *reinterpret_cast<uint2*>(dst + 16) = make_uint2(wreg[i][2], wreg[i][3]);
+                // In 16-byte chunks: chunk 4 ks + 2 (ch % 2) and the one after it, 8-byte half (ch % 4) / 2.
+                const int chunk = 4 * (ch >> 2) + 2 * (ch & 1), half = (ch & 3) >> 1;
+                const int key = (row & 15) >> SWS;
+                uint8_t* dst = smem + slot * WBUF + row * RS + half * 8;
+                *reinterpret_cast<uint2*>(dst + ((chunk ^ key) << 4)) = make_uint2(wreg[i][0], wreg[i][1]);
+                *reinterpret_cast<uint2*>(dst + (((chunk + 1) ^ key) << 4)) = make_uint2(wreg[i][2], wreg[i][3]);
             }
         }
     };
+
+    int woff[KS];     // byte offset of this lane's chunk of k-step ks inside its weight row (swizzled)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) woff[ks] = ((4 * ks + g) ^ (c16 >> SWS)) << 4;
 
     int lcount = 0;   // ring mode: layers done by this workgroup; its parity names the slot in use
     if (resident) {
@@ -222,7 +230,7 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
                 }
 
             const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
-            const uint8_t* wb = smem + slot * WBUF + c16 * RS + g * 16;
+            const uint8_t* wb = smem + slot * WBUF + c16 * RS;
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
                 const f32x4 bias = a.bias ? *reinterpret_cast<const f32x4*>(a.bias + (size_t)l * C + 16 * ft + 4 * g)
@@ -232,7 +240,7 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
                 for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    const u32x4 wa = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + ks * 64);
+                    const u32x4 wa = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]);
 #pragma unroll
                     for (int tw = 0; tw < TW; ++tw) acc[tw] = M_::mma(wa, xb[ks][tw], acc[tw]);
                 }
@@ -266,16 +274,22 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
     }
 }
 
-constexpr size_t kMlpLdsMax = 156 * 1024;
+constexpr size_t kMlpLdsMax = 160 * 1024;   // all of a CU's LDS: five layers of 128 channels stay resident
 
 template <typename T, int C, int TW, int WAVES>
 hipError_t launch_ct(const MlpArgs& a, hipStream_t st)
 {
     auto kern = mlp_mfma_kernel<T, C, TW, WAVES>;
-    const size_t wbuf = (size_t)C * (C * 2 + 16);
-    const int resident = (size_t)a.L * wbuf <= kMlpLdsMax ? 1 : 0;
-    const size_t lds = (resident ? (size_t)a.L : 2) * wbuf;
+    const size_t wbuf = (size_t)C * C * 2;
+    int resident = (size_t)a.L * wbuf <= kMlpLdsMax ? 1 : 0;
+    size_t lds = (resident ? (size_t)a.L : 2) * wbuf;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess && resident) {      // the device grants less LDS than the layers need: stream them instead
+        (void)hipGetLastError();
+        resident = 0;
+        lds = 2 * wbuf;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    }
     if (e != hipSuccess) return e;
     int occ = 0, cus = 0, dev = 0;
     int slots = 512;
