@@ -4,12 +4,15 @@
 // A = softmax over n,  y_n = sum_m Bt[n,m] z_m with Bt = softmax over m.  With L_m, rho_n the two
 // log-sum-exps saved by the forward:  A[m,n] = exp(S - L_m) <= 1,  Bt[n,m] = exp(S - rho_n) <= 1.
 // Given dy:
-//   delta_n = <dy_n, y_n>                          (bwd_delta_kernel)
+//   delta_n = <dy_n, y_n>                          (bwd_lat_kernel, MODE 0, beside the tiles it stages)
 //   dz_m    = sum_n Bt[n,m] dy_n                   (bwd_lat_kernel, MODE 0; split over N + merge)
 //   Delta_m = <dz_m, z_m>                          (merge)
 //   dS[m,n] = A (<dz_m,v_n> - Delta_m) + Bt (<dy_n,z_m> - delta_n)
 //   dv_n    = sum_m A[m,n] dz_m ;  dk_n = s sum_m dS[m,n] q_m      (bwd_tok_kernel, token parallel)
 //   dq_m    = s sum_n dS[m,n] k_n                  (bwd_lat_kernel, MODE 1; split over N + merge)
+// The additive terms (-L_m, -rho_n, -Delta_m, -delta_n) enter as the initial accumulator of the
+// matrix product they belong to wherever the tile layout gives them for free (a row vector of the
+// tile), instead of one subtraction per element.
 // Both exponentials are bounded by 1, so no running maximum is needed anywhere.  The two kernel
 // shapes are those of the forward: "latent side" = the gather's (K/V/dY tiles of 64 tokens in LDS,
 // lane = latent, contraction over tokens), "token side" = the scatter's (latent operands in LDS,
@@ -105,28 +108,17 @@ __device__ __forceinline__ uint2 lds_read_tr16(const void* lds_addr)
     return __builtin_bit_cast(uint2, r);
 }
 
-// ---- delta_n = <dy_n, y_n> -----------------------------------------------------------------
+// <u, w> of eight 16-bit elements
 template <typename T>
-__global__ __launch_bounds__(256) void bwd_delta_kernel(MixerBwdArgs a)
+__device__ __forceinline__ float dot8(u32x4 u, u32x4 w)
 {
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t total = (int64_t)a.B * a.H * a.N;
-    if (idx >= total) return;
-    const int n = idx % a.N;
-    const int64_t bh = idx / a.N;
-    const int h = bh % a.H, b = bh / a.H;
-    const uint16_t* y = (const uint16_t*)a.y + b * a.ys[0] + h * a.ys[1] + (int64_t)n * a.ys[2];
-    const uint16_t* dy = (const uint16_t*)a.dy + b * a.dys[0] + h * a.dys[1] + (int64_t)n * a.dys[2];
     float s = 0.f;
-    for (int d = 0; d < a.D; d += 8) {
-        const u32x4 u = load16(y + d), w = load16(dy + d);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            s = fmaf(Mb<T>::unpack(uint16_t(u[i] & 0xffffu)), Mb<T>::unpack(uint16_t(w[i] & 0xffffu)), s);
-            s = fmaf(Mb<T>::unpack(uint16_t(u[i] >> 16)), Mb<T>::unpack(uint16_t(w[i] >> 16)), s);
-        }
+    for (int i = 0; i < 4; ++i) {
+        s = fmaf(Mb<T>::unpack(uint16_t(u[i] & 0xffffu)), Mb<T>::unpack(uint16_t(w[i] & 0xffffu)), s);
+        s = fmaf(Mb<T>::unpack(uint16_t(u[i] >> 16)), Mb<T>::unpack(uint16_t(w[i] >> 16)), s);
     }
-    a.delta_tok[idx] = s;
+    return s;
 }
 
 // ---- latent side ---------------------------------------------------------------------------
@@ -140,7 +132,7 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
     constexpr int NT = MODE == 0 ? 2 : 4;          // staged tiles: K rows, dY^T | K rows, K^T, V rows, dY rows
     using M_ = Mb<T>;
     __shared__ __attribute__((aligned(16))) uint8_t tl[2][NT][TILEB];
-    __shared__ __attribute__((aligned(16))) float tsc[2][2][kBTile];   // per-token scalars of a tile: rho * log2(e), delta
+    __shared__ __attribute__((aligned(16))) float tsc[2][2][kBTile];   // per-token scalars of a tile: -rho * log2(e), -delta
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
     const int mblocks = a.M / MB;
@@ -151,13 +143,23 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
     const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
     const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
     const uint16_t* dy = (const uint16_t*)a.dy + b * a.dys[0] + h * a.dys[1];
+    const uint16_t* yv = (const uint16_t*)a.y + b * a.ys[0] + h * a.ys[1];
     const float* rho = a.lse_tok + bh * a.N;
-    const float* dlt = a.delta_tok + bh * a.N;
+    float* dlt = a.delta_tok + bh * a.N;
     const int m_base = mb * MB + w * 16 * CT;
+    // The dz pass also produces delta_n = <dy_n, y_n> for the later passes: its first latent block
+    // reads the rows of y next to those of dy, which it stages anyway.
+    const bool make_delta = MODE == 0 && mb == 0;
 
     // latent operands (B of the score-like products) and per-latent scalars
     u32x4 qb[CT][KD], dzb[CT][KD], zb[CT][KD];
+    // The additive terms of the score-like products (-L_m, -rho_n, -Delta_m, -delta_n) are not
+    // subtracted element by element: they are the initial accumulator of the matrix product.  A
+    // per-token term is a row vector of the tile (free); a per-latent term needs four registers
+    // holding the same value, which the register budget allows up to D = 32.
+    constexpr bool kFoldLat = MODE == 1 && D <= 32;
     float l2m[CT], dm[CT];
+    f32x4 nl4[kFoldLat ? CT : 1], nd4[kFoldLat ? CT : 1];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         const int m = m_base + ct * 16 + c16;
@@ -173,6 +175,10 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
         if (MODE == 1) {
             l2m[ct] = a.lse_lat[bh * a.M + m] * kLog2e;
             dm[ct] = a.delta_lat[bh * a.M + m];
+            if constexpr (kFoldLat) {
+                nl4[ct] = f32x4{-l2m[ct], -l2m[ct], -l2m[ct], -l2m[ct]};
+                nd4[ct] = f32x4{-dm[ct], -dm[ct], -dm[ct], -dm[ct]};
+            }
         }
     }
 
@@ -186,11 +192,13 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
 
     u32x4 kr[CPT], vr[CPT], yr[CPT];
     float rr = 0.f, dd = 0.f;
+    int ln0 = 0;       // first token of the tile held in kr/vr/yr
     auto load_tile = [&](int n0) {
+        ln0 = n0;
         if (tid < kBTile) {
             const int n = min(n0 + tid, n_end - 1);
-            rr = rho[n] * kLog2e;
-            if (MODE == 1) dd = dlt[n];
+            rr = -rho[n] * kLog2e;          // negated: they start the accumulators of the products below
+            if (MODE == 1) dd = -dlt[n];
         }
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
@@ -200,6 +208,7 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
                 kr[i] = load16(k + (int64_t)n * a.ks[2] + ch * 8);
                 yr[i] = load16(dy + (int64_t)n * a.dys[2] + ch * 8);
                 if (MODE == 1) vr[i] = load16(v + (int64_t)n * a.vs[2] + ch * 8);
+                if (MODE == 0 && make_delta) vr[i] = load16(yv + (int64_t)n * a.ys[2] + ch * 8);
             }
         }
     };
@@ -216,6 +225,12 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
                 *reinterpret_cast<u32x4*>(&tl[buf][0][k_slot(tok, ch)]) = kr[i];
                 if (MODE == 0) {
                     *reinterpret_cast<u32x4*>(&tl[buf][1][v_slot(tok, ch)]) = to_bf16x8<T>(yr[i]);
+                    if (make_delta) {      // uniform over the workgroup; the CH lanes of a token are neighbours
+                        float pd = dot8<T>(yr[i], vr[i]);
+#pragma unroll
+                        for (int o = 1; o < CH; o <<= 1) pd += __shfl_xor(pd, o);
+                        if (ch == 0 && ln0 + tok < n_end) dlt[ln0 + tok] = pd;
+                    }
                 } else {
                     *reinterpret_cast<u32x4*>(&tl[buf][1][v_slot(tok, ch)]) = to_bf16x8<T>(kr[i]);
                     *reinterpret_cast<u32x4*>(&tl[buf][2][k_slot(tok, ch)]) = to_bf16x8<T>(vr[i]);
@@ -233,6 +248,7 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
     const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
 
     auto process = [&](int n0, int buf) {
+        const bool full = n0 + kBTile <= n_end;
 #pragma unroll
         for (int ks = 0; ks < kBTile / 32; ++ks) {
             u32x4 ka0[KD], ka1[KD], va0[KD], va1[KD], ya0[KD], ya1[KD], tr[RT];
@@ -257,50 +273,62 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
                 const uint2 hi = lds_read_tr16(&tl[buf][1][v_slot(r1, ch) + sub]);
                 tr[rt] = u32x4{lo.x, lo.y, hi.x, hi.y};
             }
-            // per-token scalars of the 8 tokens (rows) this lane holds: e < 4 -> 4g+e, else 16+4g+e-4
-            float r2[8], de[8];
-            bool ok[8];
-            {
-                const int tb = ks * 32 + 4 * g;
-                const f32x4 ra = *reinterpret_cast<const f32x4*>(&tsc[buf][0][tb]), rb = *reinterpret_cast<const f32x4*>(&tsc[buf][0][tb + 16]);
-                const f32x4 da = *reinterpret_cast<const f32x4*>(&tsc[buf][1][tb]), db = *reinterpret_cast<const f32x4*>(&tsc[buf][1][tb + 16]);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    r2[e] = ra[e]; r2[e + 4] = rb[e];
-                    de[e] = da[e]; de[e + 4] = db[e];
-                    ok[e] = n0 + tb + e < n_end;
-                    ok[e + 4] = n0 + tb + 16 + e < n_end;
-                }
+            // negated per-token scalars of the 8 tokens (rows) this lane holds: 4g .. 4g+3 and 16+4g .. 16+4g+3
+            const int tb = ks * 32 + 4 * g;
+            const f32x4 ra = *reinterpret_cast<const f32x4*>(&tsc[buf][0][tb]), rb = *reinterpret_cast<const f32x4*>(&tsc[buf][0][tb + 16]);
+            f32x4 da = zf, db = zf;
+            if (MODE == 1) {
+                da = *reinterpret_cast<const f32x4*>(&tsc[buf][1][tb]);
+                db = *reinterpret_cast<const f32x4*>(&tsc[buf][1][tb + 16]);
             }
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                f32x4 s0 = zf, s1 = zf;
+                // S - rho_n: the token scatter's exponent
+                constexpr bool kFoldTok = MODE == 0 || kFoldLat;
+                f32x4 b0 = kFoldTok ? ra : zf, b1 = kFoldTok ? rb : zf;
 #pragma unroll
                 for (int kd = 0; kd < KD; ++kd) {
-                    s0 = M_::mma(ka0[kd], qb[ct][kd], s0);
-                    s1 = M_::mma(ka1[kd], qb[ct][kd], s1);
+                    b0 = M_::mma(ka0[kd], qb[ct][kd], b0);
+                    b1 = M_::mma(ka1[kd], qb[ct][kd], b1);
                 }
-                const float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
                 float o[8];
                 if (MODE == 0) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) o[e] = ok[e] ? fast_exp2(sc[e] - r2[e]) : 0.f;
+                    for (int e = 0; e < 4; ++e) {
+                        o[e] = fast_exp2(b0[e]);
+                        o[e + 4] = fast_exp2(b1[e]);
+                    }
                 } else {
-                    f32x4 g10 = zf, g11 = zf, g20 = zf, g21 = zf;
+                    // S - L_m (the latent gather's exponent), <dz_m, v_n> - Delta_m and <dy_n, z_m> - delta_n
+                    f32x4 a0 = kFoldLat ? nl4[kFoldLat ? ct : 0] : zf, a1 = a0;
+                    f32x4 g10 = kFoldLat ? nd4[kFoldLat ? ct : 0] : zf, g11 = g10, g20 = kFoldLat ? da : zf, g21 = kFoldLat ? db : zf;
 #pragma unroll
                     for (int kd = 0; kd < KD; ++kd) {
+                        if constexpr (kFoldLat) {
+                            a0 = M_::mma(ka0[kd], qb[ct][kd], a0);
+                            a1 = M_::mma(ka1[kd], qb[ct][kd], a1);
+                        }
                         g10 = Pb::mma(va0[kd], dzb[ct][kd], g10);
                         g11 = Pb::mma(va1[kd], dzb[ct][kd], g11);
                         g20 = Pb::mma(ya0[kd], zb[ct][kd], g20);
                         g21 = Pb::mma(ya1[kd], zb[ct][kd], g21);
                     }
-                    const float g1[8] = {g10[0], g10[1], g10[2], g10[3], g11[0], g11[1], g11[2], g11[3]};
-                    const float g2[8] = {g20[0], g20[1], g20[2], g20[3], g21[0], g21[1], g21[2], g21[3]};
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float av = fast_exp2(sc[e] - l2m[ct]), bv = fast_exp2(sc[e] - r2[e]);
-                        const float ds = av * (g1[e] - dm[ct]) + bv * (g2[e] - de[e]);
-                        o[e] = ok[e] ? ds : 0.f;
+                    for (int e = 0; e < 4; ++e) {
+                        if constexpr (kFoldLat) {
+                            o[e] = fast_exp2(a0[e]) * g10[e] + fast_exp2(b0[e]) * g20[e];
+                            o[e + 4] = fast_exp2(a1[e]) * g11[e] + fast_exp2(b1[e]) * g21[e];
+                        } else {    // plain products; every term is applied element by element
+                            o[e] = fast_exp2(b0[e] - l2m[ct]) * (g10[e] - dm[ct]) + fast_exp2(b0[e] + ra[e]) * (g20[e] + da[e]);
+                            o[e + 4] = fast_exp2(b1[e] - l2m[ct]) * (g11[e] - dm[ct]) + fast_exp2(b1[e] + rb[e]) * (g21[e] + db[e]);
+                        }
+                    }
+                }
+                if (!full) {       // rows past the end of the token range (clamped copies of the last token)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (n0 + tb + e >= n_end) o[e] = 0.f;
+                        if (n0 + tb + 16 + e >= n_end) o[e + 4] = 0.f;
                     }
                 }
                 const u32x4 ob = pack8(o);
@@ -334,29 +362,33 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
 }
 
 // MODE 0: dz = sum of partials, Delta_m = <dz_m, z_m>;  MODE 1: dq = scale * sum of partials.
-// One thread per (b,h,m); the partials are summed in split order (bit-stable).
+// One thread per (b,h,m) and four channels; the partials are summed in split order (bit-stable).
 template <int MODE>
 __global__ __launch_bounds__(256) void bwd_merge_kernel(MixerBwdArgs a)
 {
-    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;   // (b*H + h)*M + m
-    if (r >= (int64_t)a.B * a.H * a.M) return;
+    const int dq4 = a.D / 4;                                       // threads per row: 4, 8 or 16
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t rows = (int64_t)a.B * a.H * a.M;
+    const bool live = t < rows * dq4;
+    const int64_t r = live ? t / dq4 : rows - 1;                   // (b*H + h)*M + m
+    const int d = (int)(t % dq4) * 4;
     const int m = r % a.M;
     const int64_t bh = r / a.M;
-    const float* p0 = a.part + (bh * a.n_splits * a.M + m) * a.D;
+    const float* p0 = a.part + (bh * a.n_splits * a.M + m) * a.D + d;
     const int64_t sp = (int64_t)a.M * a.D;
-    float delta = 0.f;
-    for (int d = 0; d < a.D; d += 4) {
-        f32x4 s = {0.f, 0.f, 0.f, 0.f};
-        for (int p = 0; p < a.n_splits; ++p) s += *reinterpret_cast<const f32x4*>(p0 + p * sp + d);
-        if (MODE == 0) {
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    for (int p = 0; p < a.n_splits; ++p) s += *reinterpret_cast<const f32x4*>(p0 + p * sp);
+    if (MODE == 0) {
+        const f32x4 zz = *reinterpret_cast<const f32x4*>(a.z + r * a.D + d);
+        float delta = s[0] * zz[0] + s[1] * zz[1] + s[2] * zz[2] + s[3] * zz[3];
+        for (int o = 1; o < dq4; o <<= 1) delta += __shfl_xor(delta, o);   // the threads of a row are neighbours
+        if (live) {
             *reinterpret_cast<f32x4*>(a.dz + r * a.D + d) = s;
-            const f32x4 zz = *reinterpret_cast<const f32x4*>(a.z + r * a.D + d);
-            delta += s[0] * zz[0] + s[1] * zz[1] + s[2] * zz[2] + s[3] * zz[3];
-        } else {
-            *reinterpret_cast<f32x4*>(a.dq + r * a.D + d) = s * a.scale;
+            if (d == 0) a.delta_lat[r] = delta;
         }
+    } else if (live) {
+        *reinterpret_cast<f32x4*>(a.dq + r * a.D + d) = s * a.scale;
     }
-    if (MODE == 0) a.delta_lat[r] = delta;
 }
 
 // ---- token side ----------------------------------------------------------------------------
@@ -421,8 +453,8 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
         qt[idx] = o2;
     }
     for (int m = tid; m < M; m += NTH) {
-        l2[m] = a.lse_lat[bh * M + m] * kLog2e;
-        dl[m] = a.delta_lat[bh * M + m];
+        l2[m] = -a.lse_lat[bh * M + m] * kLog2e;     // negated: they start the accumulators below
+        dl[m] = -a.delta_lat[bh * M + m];
     }
     __syncthreads();
 
@@ -473,16 +505,17 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
                 odz[rt] = dzt[(ks * RT + rt) * 64 + lane];
                 oq[rt] = qt[(ks * RT + rt) * 64 + lane];
             }
-            // per-latent scalars of the 8 latents (rows) this lane holds
+            // negated per-latent scalars of the 8 latents (rows) this lane holds: -L_m log2(e) and -Delta_m
+            // start the accumulators of S and <dz, v>, so neither is subtracted element by element
             const f32x4 la = *reinterpret_cast<const f32x4*>(l2 + 32 * ks + 4 * g), lb = *reinterpret_cast<const f32x4*>(l2 + 32 * ks + 16 + 4 * g);
             const f32x4 da = *reinterpret_cast<const f32x4*>(dl + 32 * ks + 4 * g), db = *reinterpret_cast<const f32x4*>(dl + 32 * ks + 16 + 4 * g);
-            const float lm[8] = {la[0], la[1], la[2], la[3], lb[0], lb[1], lb[2], lb[3]};
-            const float dm[8] = {da[0], da[1], da[2], da[3], db[0], db[1], db[2], db[3]};
 #pragma unroll
             for (int tw = 0; tw < kBTW; ++tw) {
-                f32x4 s0 = zf, s1 = zf, g10 = zf, g11 = zf, g20 = zf, g21 = zf;
+                f32x4 a0 = la, a1 = lb, s0 = zf, s1 = zf, g10 = da, g11 = db, g20 = zf, g21 = zf;
 #pragma unroll
                 for (int kd = 0; kd < KD; ++kd) {
+                    a0 = M_::mma(q0[kd], kb[tw][kd], a0);
+                    a1 = M_::mma(q1[kd], kb[tw][kd], a1);
                     s0 = M_::mma(q0[kd], kb[tw][kd], s0);
                     s1 = M_::mma(q1[kd], kb[tw][kd], s1);
                     g10 = Pb::mma(d0[kd], vb[tw][kd], g10);
@@ -490,15 +523,13 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
                     g20 = Pb::mma(z0[kd], yb[tw][kd], g20);
                     g21 = Pb::mma(z1[kd], yb[tw][kd], g21);
                 }
-                const float sc[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-                const float g1[8] = {g10[0], g10[1], g10[2], g10[3], g11[0], g11[1], g11[2], g11[3]};
-                const float g2[8] = {g20[0], g20[1], g20[2], g20[3], g21[0], g21[1], g21[2], g21[3]};
                 float av[8], ds[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    av[e] = fast_exp2(sc[e] - lm[e]);
-                    const float bv = fast_exp2(sc[e] - r2[tw]);
-                    ds[e] = av[e] * (g1[e] - dm[e]) + bv * (g2[e] - de[tw]);
+                for (int e = 0; e < 4; ++e) {
+                    av[e] = fast_exp2(a0[e]);
+                    av[e + 4] = fast_exp2(a1[e]);
+                    ds[e] = av[e] * g10[e] + fast_exp2(s0[e] - r2[tw]) * (g20[e] - de[tw]);
+                    ds[e + 4] = av[e + 4] * g11[e] + fast_exp2(s1[e] - r2[tw]) * (g21[e] - de[tw]);
                 }
                 const u32x4 pa = pack8(av), pd = pack8(ds);
 #pragma unroll
@@ -553,11 +584,10 @@ hipError_t lat_launch(const MixerBwdArgs& a, hipStream_t st)
 template <typename T, int D>
 hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
 {
-    const int64_t tok = (int64_t)a.B * a.H * a.N, lat = (int64_t)a.B * a.H * a.M;
-    hipLaunchKernelGGL(bwd_delta_kernel<T>, dim3((unsigned)((tok + 255) / 256)), dim3(256), 0, st, a);
+    const int64_t lat = (int64_t)a.B * a.H * a.M;
     hipError_t e = lat_launch<T, D, 0>(a, st);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(bwd_merge_kernel<0>, dim3((unsigned)((lat + 255) / 256)), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(bwd_merge_kernel<0>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a);
     {
         auto kern = bwd_tok_kernel<T, D>;
         const size_t lds = mixer_bwd_lds_bytes(a.M, D);
@@ -571,7 +601,7 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
     }
     e = lat_launch<T, D, 1>(a, st);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(bwd_merge_kernel<1>, dim3((unsigned)((lat + 255) / 256)), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(bwd_merge_kernel<1>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a);
     return hipGetLastError();
 }
 
