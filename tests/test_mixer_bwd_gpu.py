@@ -32,7 +32,7 @@ def oracle_grads(q, k, v, gy, scale):
 
 
 @pytest.mark.parametrize("shape", [(1, 2, 777, 64, 32), (2, 2, 1000, 128, 16), (1, 1, 300, 256, 32), (1, 2, 500, 128, 64),
-                                   (2, 1, 2500, 256, 32), (1, 8, 4100, 64, 16)])
+                                   (2, 1, 2500, 256, 32), (1, 8, 4100, 64, 16), (1, 2, 900, 512, 16), (1, 1, 70001, 256, 32)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_backward_vs_autograd_oracle(dev, shape, dtype):
     q, k, v, gy = make(*shape, dtype)

@@ -92,3 +92,29 @@ def test_lra_block_keys():
     assert "att.k_proj.fcs.2.weight" in keys and "att.out_proj.bias" in keys and "mlp.fc2.bias" in keys
     blk2 = FLAREBlock(channel_dim=64, num_heads=4, num_latents=16)
     assert set(keys) == set(blk2.state_dict().keys())
+
+
+def test_triple_block_keys_and_feature_maps():
+    # construction order of backends.py:1222-1241, 1316-1328 fixes the state_dict key order
+    blk = lra_modules.TripleBlock(64, 4, kernel="hadamard", qk_dim_ratio=0.5)
+    keys = list(blk.state_dict().keys())
+    assert keys[:6] == ["norm1.weight", "norm1.bias", "norm2.weight", "norm2.bias", "att.out_proj.weight", "att.out_proj.bias"]
+    assert keys[6:16] == [f"att.{p}_proj.fc.{w}" for p in ("q1", "q2", "k1", "k2", "v") for w in ("weight", "bias")]
+    assert keys[16:20] == ["att.kernel.layer1.weight", "att.kernel.layer1.bias", "att.kernel.layer2.weight", "att.kernel.layer2.bias"]
+    assert keys[20:] == ["att.norm.weight", "att.norm.bias", "mlp.fc1.weight", "mlp.fc1.bias", "mlp.fc2.weight", "mlp.fc2.bias"]
+    assert blk.att.kernel.layer1.weight.shape == (8, 16)
+    x = torch.linspace(-3, 3, 24).view(2, 3, 4)
+    k = lra_modules.make_kernel
+    assert torch.allclose(k("elu", 4)(x), torch.where(x > 0, x + 1, x.exp()))
+    assert torch.allclose(k("relu_squared", 4)(x), x.clamp_min(0) ** 2)
+    assert torch.allclose(k("silu", 4)(x), x * torch.sigmoid(x) + 0.5)
+    assert torch.allclose(k("exp", 4)(100 * x).max(), torch.tensor(30.0).exp())
+    assert torch.allclose(k("elu_norm", 4)(x), k("elu", 4)(x / x.norm(dim=-1, keepdim=True)))
+    assert k("identity", 4)(x) is x
+    hh = k("hedgehog", 4)
+    y = hh(x)
+    assert y.shape == (2, 3, 8) and torch.allclose(y.sum(-1), torch.ones(2, 3))
+    assert torch.allclose(y, torch.cat([2 * x, -2 * x], -1).softmax(-1))     # identity-initialised
+    assert k("swiglu", 4, 6)(x).shape == (2, 3, 6)
+    with pytest.raises(NotImplementedError):
+        k("nope", 4)

@@ -2,6 +2,8 @@
 (tests/pdebench/test_pdebench_model_contracts.py:23-132) plus value parity against the same modules
 evaluated with the CPU oracle mixer."""
 import pytest
+import copy
+
 import torch
 
 import flare_py_amd as F
@@ -101,3 +103,64 @@ def test_training_step_runs(dev):
     loss.backward()
     g = m.blocks[0].att.latent_q.grad
     assert g is not None and torch.isfinite(g).all() and float(g.abs().sum()) > 0
+
+
+def _triple_block_expected(blk, x, mask=None):
+    """TripleBlock.forward of the reference (backends.py:1244-1292, 1329-1332) in fp64 torch on the CPU."""
+    blk = copy.deepcopy(blk).cpu().double()
+    att, x = blk.att, x.cpu().double()
+    h = blk.norm1(x)
+    B, N, C = h.shape
+    heads = lambda t: t.view(B, N, att.num_heads, att.head_dim).permute(0, 2, 1, 3)
+    q1, q2, k1, k2, v = (heads(p(h)) for p in (att.q1_proj, att.q2_proj, att.k1_proj, att.k2_proj, att.v_proj))
+    q1, q2, k1, k2 = (att.kernel(t) for t in (q1, q2, k1, k2))
+    if att.norm_q:
+        q1, q2 = (t / (t.norm(dim=-1, keepdim=True) + 1e-6) for t in (q1, q2))
+    if att.norm_k:
+        k1, k2 = (t / (t.norm(dim=-1, keepdim=True) + 1e-6) for t in (k1, k2))
+    if mask is not None:
+        m = mask.cpu().double().view(B, 1, N, 1)
+        q1, q2, k1, k2, v = (t * m for t in (q1, q2, k1, k2, v))
+    _, out = O.triple_einsum(q1, q2, k1, k2, v, dtype=torch.float64)
+    out = att.out_proj(att.norm(out.permute(0, 2, 1, 3).reshape(B, N, C)))
+    x = x + out
+    return x + blk.mlp(blk.norm2(x))
+
+
+@pytest.mark.parametrize("kernel,kw", [("identity", {}), ("elu", {}), ("elu", {"norm_q": True, "norm_k": True}),
+                                       ("hadamard", {"qk_dim_ratio": 2.0}), ("relu_squared", {"num_layers_kv_proj": 1, "act": "silu"})])
+def test_triple_block_matches_reference_forward(dev, kernel, kw):
+    torch.manual_seed(5)
+    blk = lra_modules.TripleBlock(64, 4, kernel=kernel, num_layers_ffn=1, **kw).to(dev).eval()
+    x = torch.randn(2, 150, 64, device=dev)
+    mask = torch.ones(2, 150, device=dev)
+    mask[1, 90:] = 0
+    with torch.no_grad():
+        y = blk(x)
+        ym = blk(x, attention_mask=mask)
+    assert O.rel_l2(y, _triple_block_expected(blk, x)) <= 2e-5
+    assert O.rel_l2(ym, _triple_block_expected(blk, x, mask)) <= 2e-5
+
+
+def test_triple_block_trains(dev):
+    torch.manual_seed(6)
+    blk = lra_modules.TripleBlock(64, 4, kernel="elu").to(dev).train()
+    x = torch.randn(2, 64, 64, device=dev)
+    blk(x).square().mean().backward()
+    g = blk.att.k1_proj.fc.weight.grad
+    assert g is not None and torch.isfinite(g).all() and float(g.abs().sum()) > 0
+    # the same loss through the fp64 CPU restatement
+    ref = copy.deepcopy(blk).cpu().double()
+    for p_ in ref.parameters():
+        p_.grad = None
+    att, xd = ref.att, x.cpu().double()
+    h = ref.norm1(xd)
+    B, N, C = h.shape
+    heads = lambda t: t.view(B, N, att.num_heads, att.head_dim).permute(0, 2, 1, 3)
+    q1, q2, k1, k2, v = (heads(p_(h)) for p_ in (att.q1_proj, att.q2_proj, att.k1_proj, att.k2_proj, att.v_proj))
+    q1, q2, k1, k2 = (att.kernel(t) for t in (q1, q2, k1, k2))
+    _, out = O.triple_einsum(q1, q2, k1, k2, v, dtype=torch.float64)
+    y = xd + att.out_proj(att.norm(out.permute(0, 2, 1, 3).reshape(B, N, C)))
+    y = y + ref.mlp(ref.norm2(y))
+    y.square().mean().backward()
+    assert O.rel_l2(g, att.k1_proj.fc.weight.grad) <= 1e-3
