@@ -308,11 +308,12 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                         for (int ct = 0; ct < CT; ++ct) {
                             f32x4 n0 = s0, n1 = s1;
                             if (ct + 1 < CT) sc2(ct + 1, n0, n1);
+                            if (ct > 0) pv(ct - 1, pbp);
+                            __builtin_amdgcn_sched_barrier(0);     // matrix products first: the exponentials run under them
                             const u32x4 pb = {P_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])),
                                               P_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
                                               P_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])),
                                               P_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]))};
-                            if (ct > 0) pv(ct - 1, pbp);
                             s0 = n0;
                             s1 = n1;
                             pbp = pb;
@@ -557,11 +558,12 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                         n0 = scores(q0, kb[tw + 1]);
                         n1 = scores(q1, kb[tw + 1]);
                     }
+                    if (tw > 0) pv(tw - 1, pbp);
+                    __builtin_amdgcn_sched_barrier(0);     // matrix products first: the exponentials run under them
                     const u32x4 pb = {P_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])),
                                       P_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
                                       P_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])),
                                       P_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]))};
-                    if (tw > 0) pv(tw - 1, pbp);
                     s0 = n0;
                     s1 = n1;
                     pbp = pb;
