@@ -94,15 +94,15 @@ __device__ __forceinline__ float xg_sum(float v)   // sum over the 4 lane groups
     return v;
 }
 
-// tanh-GELU (torch's approximate='tanh') = x * sigmoid(2 u), u = sqrt(2/pi) (x + 0.044715 x^3)
-__device__ __forceinline__ float gelu_tanh(float x)
+// tanh-GELU (torch's approximate='tanh') = x * sigmoid(2 u), u = sqrt(2/pi) (x + 0.044715 x^3); the gate is the sigmoid
+__device__ __forceinline__ float gelu_gate(float x)
 {
     const float t = x * (2.3022081f + 0.10294324f * x * x);      // 2 u log2(e)
-    return x * __builtin_amdgcn_rcpf(1.f + fast_exp2(-t));
+    return __builtin_amdgcn_rcpf(1.f + fast_exp2(-t));
 }
-__device__ __forceinline__ float silu(float x)
+__device__ __forceinline__ float silu_gate(float x)
 {
-    return x * __builtin_amdgcn_rcpf(1.f + fast_exp2(-kLog2e * x));
+    return __builtin_amdgcn_rcpf(1.f + fast_exp2(-kLog2e * x));
 }
 
 template <typename T, int C, int TW, int WAVES>
@@ -231,29 +231,50 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
 
             const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
             const uint8_t* wb = smem + slot * WBUF + c16 * RS;
+            // One layer for the wave's tokens.  ACT: 0 none, 1 tanh-GELU, 2 SiLU; ADD: the result is added to
+            // the stream.  Both are compile-time here (the caller branches once per layer, uniformly), so the
+            // epilogue has no selects and the last multiply of the activation fuses with the residual add.
+            auto layer = [&](auto act_c, auto add_c) {
+                constexpr int ACT = decltype(act_c)::value;
+                constexpr bool ADD = decltype(add_c)::value;
 #pragma unroll
-            for (int ft = 0; ft < FT; ++ft) {
-                const f32x4 bias = a.bias ? *reinterpret_cast<const f32x4*>(a.bias + (size_t)l * C + 16 * ft + 4 * g)
-                                          : f32x4{0.f, 0.f, 0.f, 0.f};
-                f32x4 acc[TW];
+                for (int ft = 0; ft < FT; ++ft) {
+                    const f32x4 bias = a.bias ? *reinterpret_cast<const f32x4*>(a.bias + (size_t)l * C + 16 * ft + 4 * g)
+                                              : f32x4{0.f, 0.f, 0.f, 0.f};
+                    f32x4 acc[TW];
 #pragma unroll
-                for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
+                    for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    const u32x4 wa = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]);
+                    for (int ks = 0; ks < KS; ++ks) {
+                        const u32x4 wa = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]);
 #pragma unroll
-                    for (int tw = 0; tw < TW; ++tw) acc[tw] = M_::mma(wa, xb[ks][tw], acc[tw]);
-                }
-#pragma unroll
-                for (int tw = 0; tw < TW; ++tw) {
-                    f32x4 t = acc[tw];
-                    if (act) {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) t[r] = a.act == 0 ? gelu_tanh(t[r]) : silu(t[r]);
+                        for (int tw = 0; tw < TW; ++tw) acc[tw] = M_::mma(wa, xb[ks][tw], acc[tw]);
                     }
                     // tile ft of the stream is not an input of this layer any more once xb is packed
-                    xs[ft][tw] = add ? xs[ft][tw] + t : t;
+#pragma unroll
+                    for (int tw = 0; tw < TW; ++tw) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const float t = acc[tw][r];
+                            if constexpr (ACT == 0) {
+                                xs[ft][tw][r] = ADD ? xs[ft][tw][r] + t : t;
+                            } else {
+                                const float gate = ACT == 1 ? gelu_gate(t) : silu_gate(t);     // act(t) = t * gate
+                                xs[ft][tw][r] = ADD ? fmaf(t, gate, xs[ft][tw][r]) : t * gate;
+                            }
+                        }
+                    }
                 }
+            };
+            using I0 = std::integral_constant<int, 0>;
+            using I1 = std::integral_constant<int, 1>;
+            using I2 = std::integral_constant<int, 2>;
+            if (!act) {
+                if (add) layer(I0{}, std::true_type{}); else layer(I0{}, std::false_type{});
+            } else if (a.act == 0) {
+                if (add) layer(I1{}, std::true_type{}); else layer(I1{}, std::false_type{});
+            } else {
+                if (add) layer(I2{}, std::true_type{}); else layer(I2{}, std::false_type{});
             }
             if (!resident) {
                 put(slot ^ 1);      // nobody reads that slot during this layer
