@@ -123,7 +123,7 @@ def bench_causal(args, F, dev):
                       B * (NP + ND) / (ms_step * 1e-3), "tokens/s", ms_step,
                       "causal FLARE: prefill 8192 tokens then 256 decode steps, B=8,H=16,M=128,D=64 (BASELINE config 4)",
                       {"input_std": "D^-1/4 (variance 1/sqrt(D))"})
-    out["roofline"] = {"bound": "hbm", "kernel": "causal_mfma_kernel (prefill)", "achieved": round(achieved, 1),
+    out["roofline"] = {"bound": "hbm", "kernel": "causal prefill (causal_mfma_kernel<state only> + causal_chunk_kernel)", "achieved": round(achieved, 1),
                        "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                        "traffic": None, "algorithmic_bytes": bytes_prefill, "ms_prefill": round(ms_prefill, 4),
                        "ms_decode_256_steps": round(ms_decode, 4), "us_per_decode_step": round(ms_decode / ND * 1e3, 3)}

@@ -85,6 +85,7 @@ __device__ __forceinline__ uint2 tr16(const void* lds_addr)
 }
 
 constexpr int kTB = 16;   // tokens per block
+constexpr int kVPad = 16; // elements of padding per V row in LDS (row stride D*2 + 32 bytes)
 
 // STATE_ONLY = false: the full recurrence over the workgroup's token segment, from the incoming
 // state plus the local states of all earlier segments (summed in segment order).  A single
@@ -102,7 +103,7 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
     using M_ = Mm<T>;         // score product and output, in the element type of q, k, y
     using P_ = Mm<bf16_t>;    // every other product: probabilities, weights, state and values as bf16
 
-    __shared__ __attribute__((aligned(16))) uint16_t vs[2][kTB][D];       // V block, row-major
+    __shared__ __attribute__((aligned(16))) uint16_t vs[2][kTB][D + kVPad];   // V block, row-major; rows padded: the transpose reads of 8 rows hit 8 bank groups
     __shared__ __attribute__((aligned(16))) uint16_t pt[4][MW][kTB];      // P^T per wave  [latent][token]
     __shared__ __attribute__((aligned(16))) uint16_t gt[4][MW][kTB];      // G^T per wave
     __shared__ __attribute__((aligned(16))) float yp[2][4][kTB][YS];      // output partials per wave
@@ -206,7 +207,7 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
         // Local state of the segment.  A 16-token block is too little work here to cover the memory
         // latency of its own prefetch, so this phase walks 64-token tiles: K as four A operands per
         // lane, V through a 64-row LDS tile, the next tile in flight while the current is used.
-        __shared__ __attribute__((aligned(16))) uint16_t v64[2][64][D];
+        __shared__ __attribute__((aligned(16))) uint16_t v64[2][64][D + kVPad];
         constexpr int VPT = (64 * (D / 8) + 255) / 256;     // 16-byte V chunks per thread and tile
         u32x4 k4[4][KD], k4n[4][KD], vreg[VPT];
         auto load64 = [&](int n0, u32x4 (&kk)[4][KD]) {
@@ -434,6 +435,326 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
     }
 }
 
+// ---- 64-token chunks, tokens split across the waves (M = 128) ---------------------------------
+// The full recurrence again, organised the other way round: a chunk of 64 tokens per step, wave w
+// owning tokens 16w..16w+15 of the chunk for everything on the token side (all 128 latents: scores,
+// P, running denominators, G, the output rows) and latents 32w..32w+31 for the state update.  The
+// output rows need no sum across waves any more, and one chunk costs two barriers instead of four
+// blocks with a dependent chain and a barrier each.  Per chunk, P = exp2(score - mu0) as above:
+//   cs_w[m]   = sum over the wave's tokens of P                      (published with P^T in LDS)
+//   dcum[t,m] = den[m] + sum_{w' < w} cs_w'[m] + (L P_w)[t,m]
+//   G = P / dcum;   Y_w = G U0 + sum_{w' <= w} tril?(G P_w'^T) V_w'    (tril on the diagonal tile only)
+//   U[own m] += sum_w' P_w'[:, m]^T V_w';   den += sum_w' cs_w'
+// U0 = the state at the start of the chunk, published by its owners as bf16 B operands in LDS.
+constexpr int kChunk = 64;
+
+template <int D> constexpr size_t causal_chunk_lds()
+{
+    // q operands, V chunk, P^T and G^T of the four waves, U0 operands, column sums
+    return (size_t)8 * (D / 32) * 64 * 16 + (size_t)kChunk * (D + kVPad) * 2 + 2 * (size_t)4 * 128 * 16 * 2 +
+           (size_t)4 * (D / 16) * 64 * 16 + (size_t)4 * 128 * 4;
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
+{
+    constexpr int M = 128, KD = D / 32, DT = D / 16, CTA = M / 16, KS = M / 32, MT = 2;
+    constexpr int VPT = (kChunk * (D / 8) + 255) / 256;     // 16-byte V pieces per thread and chunk
+    constexpr int VS = D + kVPad;                           // V row stride in LDS (elements)
+    using M_ = Mm<T>;
+    using P_ = Mm<bf16_t>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    u32x4* qs = reinterpret_cast<u32x4*>(smem);                                   // [CTA][KD][64]
+    uint16_t* vs = reinterpret_cast<uint16_t*>(qs + CTA * KD * 64);               // [64][VS], VS = D + padding
+    uint16_t* pt = vs + kChunk * VS;                                              // [4][M][16]
+    uint16_t* gt = pt + 4 * M * 16;                                               // [4][M][16]
+    u32x4* u0s = reinterpret_cast<u32x4*>(gt + 4 * M * 16);                       // [KS][DT][64]
+    float* cs = reinterpret_cast<float*>(u0s + KS * DT * 64);                     // [4][M]
+    __shared__ int bad_flag;
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H, seg = blockIdx.y;
+    const int n_lo = seg * a.seg_len, N = min(a.N, n_lo + a.seg_len);
+    const bool single = a.n_segs == 1;
+    float* seg_den = a.seg_den + ((int64_t)bh * a.n_segs + seg) * M;
+    float* seg_num = a.seg_num + ((int64_t)bh * a.n_segs + seg) * M * D;
+    const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
+    const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
+    const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
+    uint16_t* y = (uint16_t*)a.y + b * a.ys[0] + h * a.ys[1];
+    float* mu_g = a.mu + (int64_t)bh * M;
+    float* den_g = a.den + (int64_t)bh * M;
+    float* num_g = a.num + (int64_t)bh * M * D;
+    const float sl2 = a.scale * kLog2e;
+    const int m0 = w * 32;
+    uint16_t* ptw = pt + w * M * 16;      // this wave's P^T  [latent][token]
+    uint16_t* gtw = gt + w * M * 16;      // this wave's G^T, later its output transposition tiles
+
+    if (tid == 0) bad_flag = 0;
+
+    // q as B operands of the score product (log2-scaled), for every latent tile
+    for (int idx = tid; idx < CTA * KD * 64; idx += 256) {
+        const int ln = idx & 63, kd = (idx >> 6) % KD, ct = idx / (64 * KD);
+        const int m = ct * 16 + (ln & 15);
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(q + (int64_t)m * a.qs[2] + kd * 32 + (ln >> 4) * 8);
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            o[i] = M_::pack2(M_::unpack(uint16_t(raw[i] & 0xffffu)) * sl2, M_::unpack(uint16_t(raw[i] >> 16)) * sl2);
+        qs[idx] = o;
+    }
+    // shift and running denominators of every latent (column c16 of tile ct), replicated in the waves
+    float mu0[CTA], den0[CTA];
+#pragma unroll
+    for (int ct = 0; ct < CTA; ++ct) {
+        const int m = ct * 16 + c16;
+        const float mu = mu_g[m];
+        mu0[ct] = mu <= kNegBig ? 0.f : mu * kLog2e;
+        float d0 = mu <= kNegBig ? 0.f : den_g[m];
+        for (int s = 0; s < seg; ++s) d0 += a.seg_den[((int64_t)bh * a.n_segs + s) * M + m];
+        den0[ct] = d0;
+    }
+    // state numerator of the wave's own latents: tile (mt, dt) holds rows m0 + 16 mt + 4g + r, column 16 dt + c16
+    f32x4 U[MT][DT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = m0 + mt * 16 + 4 * g + r;
+                float u = mu_g[m] <= kNegBig ? 0.f : num_g[(int64_t)m * D + dt * 16 + c16];
+                for (int s = 0; s < seg; ++s)
+                    u += a.seg_num[(((int64_t)bh * a.n_segs + s) * M + m) * D + dt * 16 + c16];
+                U[mt][dt][r] = u;
+            }
+
+    uint2 ltri, ones4 = make_uint2(P_::kOnes2, P_::kOnes2);
+    {
+        const uint32_t one = P_::kOnes2 & 0xffffu;
+        uint32_t e[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) e[i] = (4 * g + i <= c16) ? one : 0u;
+        ltri = make_uint2(e[0] | (e[1] << 16), e[2] | (e[3] << 16));
+    }
+    const u32x4 ones8 = {P_::kOnes2, P_::kOnes2, P_::kOnes2, P_::kOnes2};
+    const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
+
+    u32x4 ka[KD], kn[KD], vr[VPT];
+    auto load_chunk = [&](int n0, u32x4 (&kk)[KD]) {
+        const int n = min(n0 + 16 * w + c16, N - 1);
+#pragma unroll
+        for (int kd = 0; kd < KD; ++kd) kk[kd] = *reinterpret_cast<const u32x4*>(k + (int64_t)n * a.ks[2] + kd * 32 + g * 8);
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int c = tid + i * 256, tok = c / (D / 8), ch = c % (D / 8);
+            if (c < kChunk * (D / 8)) vr[i] = *reinterpret_cast<const u32x4*>(v + (int64_t)min(n0 + tok, N - 1) * a.vs[2] + ch * 8);
+        }
+    };
+    auto store_v = [&]() {
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int c = tid + i * 256, tok = c / (D / 8), ch = c % (D / 8);
+            if (c < kChunk * (D / 8)) {
+                u32x4 o = vr[i];
+                if constexpr (!std::is_same<T, bf16_t>::value) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        o[j] = P_::pack2(M_::unpack(uint16_t(vr[i][j] & 0xffffu)), M_::unpack(uint16_t(vr[i][j] >> 16)));
+                }
+                *reinterpret_cast<u32x4*>(vs + tok * VS + ch * 8) = o;
+            }
+        }
+    };
+    // the state of the wave's latents as B operands (k-slots = its 32 latents, lane = column d)
+    auto publish_u = [&]() {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const f32x4 u0 = U[0][dt], u1 = U[1][dt];
+            u0s[(w * DT + dt) * 64 + lane] = u32x4{P_::pack2(u0[0], u0[1]), P_::pack2(u0[2], u0[3]),
+                                                   P_::pack2(u1[0], u1[1]), P_::pack2(u1[2], u1[3])};
+        }
+    };
+    // operand with tokens in lanes and latents in k-slots from a [latent][token] tile (k-step ks = 32 latents)
+    auto tr_op = [&](const uint16_t* tile, int ks) {
+        const int r0 = ks * 32 + 4 * g + (c16 >> 2), piece = (c16 & 3) * 4;
+        const uint2 lo = tr16(tile + r0 * 16 + piece), hi = tr16(tile + (r0 + 16) * 16 + piece);
+        return u32x4{lo.x, lo.y, hi.x, hi.y};
+    };
+
+    bool bad = false;
+    load_chunk(n_lo, ka);
+    store_v();
+    publish_u();
+    if (n_lo + kChunk < N) load_chunk(n_lo + kChunk, kn);
+    __syncthreads();                                        // q operands
+
+    for (int n0 = n_lo; n0 < N; n0 += kChunk) {
+        const int tbase = n0 + 16 * w;
+        const int tbw = min(16, max(0, N - tbase));        // valid tokens of this wave in the chunk
+
+        // ---- token side, part 1: scores, P, column sums; publish P^T ----
+        // (staged over the eight latent tiles: every LDS read before the first LDS write, so that the reads
+        // can be issued together instead of one tile's round trip after the other)
+        float p[CTA][4];
+        uint2 ppk[CTA];
+        {
+            f32x4 sc[CTA];
+#pragma unroll
+            for (int ct = 0; ct < CTA; ++ct) {
+                f32x4 s = zf;
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) s = M_::mma32(ka[kd], qs[(ct * KD + kd) * 64 + lane], s);
+                sc[ct] = s;
+            }
+#pragma unroll
+            for (int ct = 0; ct < CTA; ++ct) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) p[ct][r] = (4 * g + r < tbw) ? fast_exp2(sc[ct][r] - mu0[ct]) : 0.f;
+                ppk[ct] = make_uint2(P_::pack2(p[ct][0], p[ct][1]), P_::pack2(p[ct][2], p[ct][3]));
+            }
+            f32x4 csv[CTA];
+#pragma unroll
+            for (int ct = 0; ct < CTA; ++ct) csv[ct] = P_::mma16(ones4, ppk[ct], zf);
+#pragma unroll
+            for (int ct = 0; ct < CTA; ++ct) {
+                if (g == 0) cs[w * M + ct * 16 + c16] = csv[ct][0];
+                *reinterpret_cast<uint2*>(ptw + (ct * 16 + c16) * 16 + 4 * g) = ppk[ct];
+            }
+        }
+        __syncthreads();                                    // P^T, cs, V chunk, U0 operands visible
+
+        // ---- token side, part 2: running denominators, G ----
+#pragma unroll
+        for (int ct = 0; ct < CTA; ++ct) {
+            const int m = ct * 16 + c16;
+            const float c0 = cs[m], c1 = cs[M + m], c2 = cs[2 * M + m], c3 = cs[3 * M + m];
+            float base = den0[ct];
+            if (w > 0) base += c0;
+            if (w > 1) base += c1;
+            if (w > 2) base += c2;
+            den0[ct] = den0[ct] + c0 + c1 + c2 + c3;        // same order in every wave
+            const f32x4 dc = P_::mma16(ltri, ppk[ct], zf);
+            float gv[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) gv[r] = p[ct][r] > 0.f ? p[ct][r] * __builtin_amdgcn_rcpf(dc[r] + base) : 0.f;
+            *reinterpret_cast<uint2*>(gtw + (ct * 16 + c16) * 16 + 4 * g) = make_uint2(P_::pack2(gv[0], gv[1]), P_::pack2(gv[2], gv[3]));
+        }
+        u32x4 gop[KS], pop[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            gop[ks] = tr_op(gtw, ks);
+            pop[ks] = tr_op(ptw, ks);
+        }
+        // softmax sums over the latents of the wave's tokens (rows t = 4g + r, equal in every column)
+        f32x4 rsum = zf;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) rsum = P_::mma32(pop[ks], ones8, rsum);
+
+        // ---- outputs: G U0, then the chunk's own tokens up to and including this wave's ----
+        f32x4 yacc[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            f32x4 acc = zf;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) acc = P_::mma32(gop[ks], u0s[(ks * DT + dt) * 64 + lane], acc);
+            yacc[dt] = acc;
+        }
+        for (int wp = 0; wp <= w; ++wp) {
+            f32x4 acct = zf;      // [tau of wave wp, t of this wave] = sum_m P[tau,m] G[t,m]
+            if (wp == w) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) acct = P_::mma32(pop[ks], gop[ks], acct);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acct[r] = (4 * g + r <= c16) ? acct[r] : 0.f;
+            } else {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) acct = P_::mma32(tr_op(pt + wp * M * 16, ks), gop[ks], acct);
+            }
+            const uint2 aop = make_uint2(P_::pack2(acct[0], acct[1]), P_::pack2(acct[2], acct[3]));
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const uint2 vop = tr16(vs + (wp * 16 + 4 * g + (c16 >> 2)) * VS + dt * 16 + (c16 & 3) * 4);
+                yacc[dt] = P_::mma16(aop, vop, yacc[dt]);
+            }
+        }
+        // y rows / softmax sums, transposed through the wave's (now free) G^T region: lane (g, c16) ends
+        // up with y[token c16][16 dt + 4g .. 4g + 3]
+        {
+            float inv[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                inv[r] = 1.f / rsum[r];
+                if (4 * g + r < tbw) bad = bad || !(rsum[r] >= kLMin && rsum[r] <= kLMax);
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                float o[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    o[r] = yacc[dt][r] * inv[r];
+                    if (4 * g + r < tbw) bad = bad || !(fabsf(o[r]) <= 3.0e38f);
+                }
+                *reinterpret_cast<uint2*>(gtw + (dt * 16 + c16) * 16 + 4 * g) = make_uint2(M_::pack2(o[0], o[1]), M_::pack2(o[2], o[3]));
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                const uint2 o = tr16(gtw + (dt * 16 + 4 * g + (c16 >> 2)) * 16 + (c16 & 3) * 4);
+                if (c16 < tbw) *reinterpret_cast<uint2*>(y + (int64_t)(tbase + c16) * a.ys[2] + dt * 16 + 4 * g) = o;
+            }
+        }
+
+        // ---- state update of the wave's own latents over all 64 tokens ----
+#pragma unroll
+        for (int wp = 0; wp < 4; ++wp) {
+            uint2 vop[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vop[dt] = tr16(vs + (wp * 16 + 4 * g + (c16 >> 2)) * VS + dt * 16 + (c16 & 3) * 4);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const uint2 pa = *reinterpret_cast<const uint2*>(pt + wp * M * 16 + (m0 + mt * 16 + c16) * 16 + 4 * g);
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) U[mt][dt] = P_::mma16(pa, vop[dt], U[mt][dt]);
+            }
+        }
+
+        __syncthreads();                                    // everyone is done with V, U0, P^T of this chunk
+        if (n0 + kChunk < N) {
+#pragma unroll
+            for (int kd = 0; kd < KD; ++kd) ka[kd] = kn[kd];
+            store_v();
+            publish_u();
+            if (n0 + 2 * kChunk < N) load_chunk(n0 + 2 * kChunk, kn);
+        }
+    }
+
+    const bool last = seg == a.n_segs - 1;
+#pragma unroll
+    for (int ct = 0; ct < CTA; ++ct) bad = bad || (last && !(den0[ct] >= kLMin && den0[ct] <= kLMax));
+    if (__any(bad) && lane == 0) bad_flag = 1;
+    __syncthreads();
+    if (bad_flag) {
+        if (tid == 0) a.flags[bh] = 1;
+        return;
+    }
+    if (single && tid == 0) a.flags[bh] = 0;
+    if (!last) return;
+    float* den_o = single ? den_g : seg_den;
+    float* num_o = single ? num_g : seg_num;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int ct = 2 * w + mt, m = ct * 16 + c16;
+        if (g == 0) {
+            if (single) mu_g[m] = mu0[ct] * kLn2;
+            den_o[m] = den0[ct];
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) num_o[(int64_t)(m0 + mt * 16 + 4 * g + r) * D + dt * 16 + c16] = U[mt][dt][r];
+    }
+}
+
 // Clears the per-(b,h) redo flags (a kernel rather than a memset so that callers may capture
 // the call in a graph).
 __global__ void causal_clear_flags_kernel(int* flags, int n)
@@ -471,15 +792,34 @@ hipError_t launch_phase(const CausalArgs& a, int step, dim3 grid, hipStream_t st
     return hipGetLastError();
 }
 
+template <typename T, int D>
+hipError_t launch_chunk_d(const CausalArgs& a, dim3 grid, hipStream_t st)
+{
+    auto kern = causal_chunk_kernel<T, D>;
+    constexpr size_t lds = causal_chunk_lds<D>();
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, a);
+    return hipGetLastError();
+}
+
+// The recurrence phase: 64-token chunks for the prefill at M = 128, 16-token (or 1-token) blocks otherwise.
+template <typename T>
+hipError_t launch_recurrence(const CausalArgs& a, int step, dim3 grid, hipStream_t st)
+{
+    if (step == kTB && a.M == 128) return a.D == 64 ? launch_chunk_d<T, 64>(a, grid, st) : launch_chunk_d<T, 32>(a, grid, st);
+    return launch_phase<T, false>(a, step, grid, st);
+}
+
 template <typename T>
 hipError_t launch_t(const CausalArgs& a, int step, hipStream_t st)
 {
     const int BH = a.B * a.H;
-    if (a.n_segs == 1) return launch_phase<T, false>(a, step, dim3(BH, 1), st);
+    if (a.n_segs == 1) return launch_recurrence<T>(a, step, dim3(BH, 1), st);
     hipLaunchKernelGGL(causal_clear_flags_kernel, dim3((BH + 255) / 256), dim3(256), 0, st, a.flags, BH);
     hipError_t e = launch_phase<T, true>(a, step, dim3(BH, a.n_segs - 1), st);
     if (e != hipSuccess) return e;
-    e = launch_phase<T, false>(a, step, dim3(BH, a.n_segs), st);
+    e = launch_recurrence<T>(a, step, dim3(BH, a.n_segs), st);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(causal_commit_kernel, dim3(BH), dim3(256), 0, st, a);
     return hipGetLastError();
