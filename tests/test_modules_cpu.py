@@ -118,3 +118,32 @@ def test_triple_block_keys_and_feature_maps():
     assert k("swiglu", 4, 6)(x).shape == (2, 3, 6)
     with pytest.raises(NotImplementedError):
         k("nope", 4)
+
+
+def test_reference_trainer_snapshot_loads(tmp_path):
+    """A snapshot in the layout of mlutils/trainer.py:382-432 (DDP-prefixed names, EMA shadow, optimiser state)
+    loads with the non-executing loader; names and values arrive unchanged."""
+    from flare_py_amd.checkpoint import load_reference_checkpoint, read_snapshot
+    torch.manual_seed(0)
+    src = FLAREModel(in_dim=3, out_dim=2, channel_dim=32, num_blocks=2, num_heads=4, num_latents=8)
+    opt = torch.optim.AdamW(src.parameters(), lr=1e-3)
+    for p_ in src.parameters():      # (no forward on the CPU: the mixer has no CPU path)
+        p_.grad = torch.ones_like(p_)
+    opt.step()
+    ema = {k: v.detach() * 0.5 for k, v in src.named_parameters()}
+    snap = {"model_state": {"module." + k: v for k, v in src.state_dict().items()},
+            "ema_shadow": {"module." + k: v for k, v in ema.items()},
+            "step": 7, "epoch": 1, "opt_state": opt.state_dict(), "schedule_state": None,
+            "train_loss_per_batch": [0.5, 0.25], "memory_utilization": None}
+    path = str(tmp_path / "model.pt")
+    torch.save(snap, path)
+    dst = FLAREModel(in_dim=3, out_dim=2, channel_dim=32, num_blocks=2, num_heads=4, num_latents=8)
+    out = load_reference_checkpoint(dst, path)
+    assert out["step"] == 7 and read_snapshot(path)["epoch"] == 1
+    for (ka, a), (kb, b) in zip(src.state_dict().items(), dst.state_dict().items()):
+        assert ka == kb and torch.equal(a, b)
+    load_reference_checkpoint(dst, path, use_ema=True)
+    assert torch.equal(dst.blocks[0].att.latent_q, src.blocks[0].att.latent_q * 0.5)
+    torch.save({"weights": 1}, path)
+    with pytest.raises(ValueError):
+        read_snapshot(path)
