@@ -103,7 +103,8 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
     using M_ = Mm<T>;         // score product and output, in the element type of q, k, y
     using P_ = Mm<bf16_t>;    // every other product: probabilities, weights, state and values as bf16
 
-    __shared__ __attribute__((aligned(16))) uint16_t vs[2][kTB][D + kVPad];   // V block, row-major; rows padded: the transpose reads of 8 rows hit 8 bank groups
+    // V block, row-major; rows padded so that the transpose reads of 8 rows hit 8 different bank groups
+    __shared__ __attribute__((aligned(16))) uint16_t vs[2][kTB][D + kVPad];
     __shared__ __attribute__((aligned(16))) uint16_t pt[4][MW][kTB];      // P^T per wave  [latent][token]
     __shared__ __attribute__((aligned(16))) uint16_t gt[4][MW][kTB];      // G^T per wave
     __shared__ __attribute__((aligned(16))) float yp[2][4][kTB][YS];      // output partials per wave

@@ -125,6 +125,8 @@ int        gather_generic_parts_per_wg();
 bool       mfma_mixer_supported(int dtype, int M, int D);
 int        mfma_gather_tokens_per_iter();
 int        mfma_gather_resident_slots(int dtype, int M, int D);
+// workgroups of `kern` resident on the current device at once (CUs x occupancy), cached per kernel, LDS size and device
+int        resident_slots(const void* kern, size_t dyn_lds, int block_threads = 256);
 hipError_t launch_gather_mfma(const MixerArgs& a, int dtype, hipStream_t st);
 hipError_t launch_scatter_mfma(const MixerArgs& a, int dtype, hipStream_t st);
 

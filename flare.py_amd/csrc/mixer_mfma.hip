@@ -698,34 +698,6 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
 
 constexpr size_t kScatterLdsMax = 150 * 1024;
 
-// Workgroups of `kern` the current device holds at once (CUs x occupancy).  Grids are sized
-// to a whole multiple of this so that no partially filled last round is left over.
-// Falls back to 2 per CU on 256 CUs when no device can be queried (host-only planning).
-int resident_slots(const void* kern, size_t dyn_lds, int block_threads = 256)
-{
-    struct Entry { const void* k; size_t lds; int dev; int slots; };
-    static Entry cache[64];
-    static int ncache = 0;
-    static std::mutex mu;     // the cache is the only mutable state of the library: guard it
-    std::lock_guard<std::mutex> lock(mu);
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return 512; }
-    for (int i = 0; i < ncache; ++i)
-        if (cache[i].k == kern && cache[i].lds == dyn_lds && cache[i].dev == dev) return cache[i].slots;
-    int occ = 0, cus = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, block_threads, dyn_lds) != hipSuccess || occ < 1) {
-        (void)hipGetLastError();
-        return 512;
-    }
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
-        (void)hipGetLastError();
-        return 512;
-    }
-    const int slots = occ * cus;
-    if (ncache < 64) cache[ncache++] = Entry{kern, dyn_lds, dev, slots};
-    return slots;
-}
-
 template <typename T, int D>
 const void* gather_kernel_ptr(int M)
 {
@@ -808,6 +780,34 @@ hipError_t scatter_launch_d(const MixerArgs& a, hipStream_t st)
 }
 
 }  // namespace
+
+// Workgroups of `kern` the current device holds at once (CUs x occupancy).  Grids are sized
+// to a whole multiple of this so that no partially filled last round is left over.
+// Falls back to 2 per CU on 256 CUs when no device can be queried (host-only planning).
+int resident_slots(const void* kern, size_t dyn_lds, int block_threads)
+{
+    struct Entry { const void* k; size_t lds; int dev; int slots; };
+    static Entry cache[64];
+    static int ncache = 0;
+    static std::mutex mu;     // the cache is the only mutable state of the library: guard it
+    std::lock_guard<std::mutex> lock(mu);
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return 512; }
+    for (int i = 0; i < ncache; ++i)
+        if (cache[i].k == kern && cache[i].lds == dyn_lds && cache[i].dev == dev) return cache[i].slots;
+    int occ = 0, cus = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, block_threads, dyn_lds) != hipSuccess || occ < 1) {
+        (void)hipGetLastError();
+        return 512;
+    }
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
+        (void)hipGetLastError();
+        return 512;
+    }
+    const int slots = occ * cus;
+    if (ncache < 64) cache[ncache++] = Entry{kern, dyn_lds, dev, slots};
+    return slots;
+}
 
 bool mfma_mixer_supported(int dtype, int M, int D)
 {

@@ -312,14 +312,7 @@ hipError_t launch_ct(const MlpArgs& a, hipStream_t st)
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     }
     if (e != hipSuccess) return e;
-    int occ = 0, cus = 0, dev = 0;
-    int slots = 512;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void*>(kern), 64 * WAVES, lds) == hipSuccess && occ > 0 &&
-        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
-        slots = occ * cus;
-    else
-        (void)hipGetLastError();
+    const int slots = resident_slots(reinterpret_cast<const void*>(kern), lds, 64 * WAVES);
     const int64_t per = 16 * TW * WAVES;
     const int64_t nblk = ((int64_t)a.T + per - 1) / per;
     const unsigned grid = (unsigned)(nblk < slots ? nblk : slots);

@@ -3,8 +3,9 @@
  *
  * Plain pointers and sizes only; no torch types.  Every device pointer is owned by the
  * caller (inputs, outputs and the workspace).  The library allocates no device memory,
- * keeps no mutable global state beyond a mutex-guarded cache of occupancy queries, launches asynchronously on the hipStream_t handed in
- * (passed as void*) and never synchronises the device.  All entry points return an int
+ * keeps no mutable global state beyond a mutex-guarded cache of occupancy queries,
+ * launches asynchronously on the hipStream_t handed in (passed as void*) and never
+ * synchronises the device.  All entry points return an int
  * status (0 = OK, negative = error); the text of the last error on the calling thread is
  * available from flare_last_error_string().  Shapes, dtypes, strides, alignment and the
  * workspace size are validated on the host BEFORE anything is launched.
