@@ -269,9 +269,7 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
     return (y, z) if return_z else y
 
 
-def flare_gather(q, k, v, scale: float = 1.0, key_mask=None, n_splits: int = 0,
-                 force_generic: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
-    """z [B,H,M,D] fp32 = softmax_n(scale q k^T) v and lse [B,H,M] (natural log)."""
+def _gather_forward(q, k, v, scale, key_mask, n_splits, force_generic):
     _require_cuda(q, k, v)
     lib = _lib.load()
     if q.dtype != k.dtype:
@@ -295,8 +293,7 @@ def flare_gather(q, k, v, scale: float = 1.0, key_mask=None, n_splits: int = 0,
     return z, lse
 
 
-def flare_scatter(q, k, z, scale: float = 1.0, key_mask=None, force_generic: bool = False) -> torch.Tensor:
-    """y [B,H,N,D] = softmax_m(scale k q^T) z with z [B,H,M,D] fp32."""
+def _scatter_forward(q, k, z, scale, key_mask, force_generic):
     _require_cuda(q, k, z)
     lib = _lib.load()
     if q.dtype != k.dtype:
@@ -317,6 +314,72 @@ def flare_scatter(q, k, z, scale: float = 1.0, key_mask=None, force_generic: boo
                                    C.c_void_p(_stream_ptr(k.device)))
     _lib.check(rc, "flare_scatter_fwd")
     return y
+
+
+def _half_torch_grad(which, q, k, x, scale, key_mask, g):
+    """Gradients of one half of the mixer by recomputation in plain torch ops on the device (the forward
+    never takes this path): which='gather' -> z = softmax_n(s q k^T) x with x = v; which='scatter' ->
+    y = softmax_m(s k q^T) x with x = z.  Materialises the [B,H,M,N] scores in fp32."""
+    with torch.enable_grad():
+        q_, k_, x_ = (t.detach().float().requires_grad_(True) for t in (q, k, x))
+        qe = q_ if q_.dim() == 4 else q_.unsqueeze(0)
+        s = scale * (qe @ k_.transpose(-2, -1))
+        if which == "gather":
+            if key_mask is not None:
+                s = s.masked_fill(~key_mask.to(torch.bool)[:, None, None, :], float("-inf"))
+            out = torch.softmax(s, dim=-1) @ x_
+        else:
+            out = torch.softmax(s.transpose(-2, -1), dim=-1) @ x_
+            if key_mask is not None:
+                out = out * key_mask.to(out.dtype)[:, None, :, None]
+        gq, gk, gx = torch.autograd.grad(out, (q_, k_, x_), g.float())
+    return gq.to(q.dtype), gk.to(k.dtype), gx.to(x.dtype)
+
+
+class _GatherFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, scale, key_mask, n_splits, force_generic):
+        ctx.scale, ctx.key_mask = scale, key_mask
+        ctx.save_for_backward(q, k, v)
+        z, lse = _gather_forward(q, k, v, scale, key_mask, n_splits, force_generic)
+        ctx.mark_non_differentiable(lse)
+        return z, lse
+
+    @staticmethod
+    def backward(ctx, gz, _glse):
+        q, k, v = ctx.saved_tensors
+        return (*_half_torch_grad("gather", q, k, v, ctx.scale, ctx.key_mask, gz), None, None, None, None)
+
+
+class _ScatterFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, z, scale, key_mask, force_generic):
+        ctx.scale, ctx.key_mask = scale, key_mask
+        ctx.save_for_backward(q, k, z)
+        return _scatter_forward(q, k, z, scale, key_mask, force_generic)
+
+    @staticmethod
+    def backward(ctx, gy):
+        q, k, z = ctx.saved_tensors
+        return (*_half_torch_grad("scatter", q, k, z, ctx.scale, ctx.key_mask, gy), None, None, None)
+
+
+def flare_gather(q, k, v, scale: float = 1.0, key_mask=None, n_splits: int = 0,
+                 force_generic: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """z [B,H,M,D] fp32 = softmax_n(scale q k^T) v and lse [B,H,M] (natural log).
+    Differentiable in q, k, v (the backward recomputes the scores with torch ops: for models that put
+    layers between the two halves; the whole mixer has its own HIP backward)."""
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+        return _GatherFn.apply(q, k, v, float(scale), key_mask, n_splits, force_generic)
+    return _gather_forward(q, k, v, float(scale), key_mask, n_splits, force_generic)
+
+
+def flare_scatter(q, k, z, scale: float = 1.0, key_mask=None, force_generic: bool = False) -> torch.Tensor:
+    """y [B,H,N,D] = softmax_m(scale k q^T) z with z [B,H,M,D] (computed from its fp32 copy).
+    Differentiable in q, k, z like flare_gather."""
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, z)):
+        return _ScatterFn.apply(q, k, z, float(scale), key_mask, force_generic)
+    return _scatter_forward(q, k, z, float(scale), key_mask, force_generic)
 
 
 # --------------------------------------------------------------------------------------

@@ -164,3 +164,56 @@ def test_triple_block_trains(dev):
     y = y + ref.mlp(ref.norm2(y))
     y.square().mean().backward()
     assert O.rel_l2(g, att.k1_proj.fc.weight.grad) <= 1e-3
+
+
+def _bigflare_expected(model, x):
+    """BigFLAREModel.forward (pdebench/models/flare_ablations.py:96-131, 176-186, 297-311) in fp64 torch on the CPU,
+    the two softmax products written out as in the reference's explicit branch (:116-125)."""
+    m = copy.deepcopy(model).cpu().double()
+    x = m.in_proj(x.detach().cpu().double())
+    for blk in m.blocks:
+        att = blk.att
+        h = blk.ln1(x)
+        B, N, C = h.shape
+        if att.shared_latents:
+            q = att.latent_q.view(1, att.num_latents, att.head_dim).expand(att.num_heads, -1, -1)
+        else:
+            q = att.latent_q.view(att.num_heads, att.num_latents, att.head_dim)
+        k = att.k_proj(h).view(B, N, att.num_heads, att.head_dim).permute(0, 2, 1, 3)
+        v = att.v_proj(h).view(B, N, att.num_heads, att.head_dim).permute(0, 2, 1, 3)
+        scores = q.unsqueeze(0) @ k.transpose(-2, -1)
+        z = torch.softmax(scores, dim=-1) @ v
+        z = att.apply_latent_blocks(z)
+        y = torch.softmax(scores.transpose(-2, -1), dim=-1) @ z
+        x = x + att.out_proj(y.permute(0, 2, 1, 3).reshape(B, N, C))
+        x = x + blk.mlp(blk.ln2(x))
+    return m, m.out_proj(x)
+
+
+@pytest.mark.parametrize("kw", [dict(num_latent_blocks=1), dict(shared_latents=True), dict()])
+def test_bigflare_ablation_model(dev, kw):
+    from flare_py_amd.ablations import BigFLAREModel
+    torch.manual_seed(7)
+    model = BigFLAREModel(in_dim=3, out_dim=2, channel_dim=32, num_blocks=2, num_latents=16, num_heads=4, **kw).to(dev)
+    with torch.no_grad():       # the reference's N(0, 0.02) weights make every block nearly the identity: widen them
+        for p_ in model.parameters():
+            if p_.dim() == 2:
+                p_.mul_(8.0)
+    keys = list(model.state_dict().keys())
+    assert keys[0] == "in_proj.fc1.weight" and "blocks.0.att.latent_q" in keys and "out_proj.ln.weight" in keys
+    assert ("blocks.0.att.latent_blocks.0.att.qkv_proj.weight" in keys) == (kw.get("num_latent_blocks", 0) > 0)
+    assert model.blocks[0].att.latent_q.shape == ((8, 16) if kw.get("shared_latents") else (32, 16))
+    x = torch.randn(2, 200, 3, device=dev)
+    y = model(x)
+    ref, yr = _bigflare_expected(model, x)
+    assert O.rel_l2(y, yr) <= 2e-5
+    if not kw.get("num_latent_blocks"):
+        ys, scores = model(x, return_scores=True)
+        assert len(scores) == 2 and scores[0].shape == (2, 4, 16, 200) and torch.equal(ys, y)
+    # one training step: gradients through gather -> latent blocks -> scatter against fp64 autograd
+    y.square().mean().backward()
+    yr.square().mean().backward()
+    g, gr = model.blocks[0].att.latent_q.grad, ref.blocks[0].att.latent_q.grad
+    assert O.rel_l2(g, gr) <= 1e-3
+    g, gr = model.blocks[0].att.k_proj.fc1.weight.grad, ref.blocks[0].att.k_proj.fc1.weight.grad
+    assert O.rel_l2(g, gr) <= 1e-3
