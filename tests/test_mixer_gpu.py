@@ -229,3 +229,54 @@ def test_constant_score_offset(dev, dtype, offset):
     k[..., 0] = offset / 4.0
     assert F.mixer_kernel_name(q, k, v).startswith("mfma")
     check(dev, q, k, v)
+
+
+def test_offsets_beyond_2_31_elements(dev):
+    """k, v, y of exactly 2^31 elements each: the last (batch, head) slice sits beyond what 32-bit element
+    offsets reach.  Heads are independent, so that slice computed alone (small offsets) must give the same rows."""
+    B, H, N, M, D = 4, 8, 1 << 21, 64, 32
+    g = torch.Generator(device=dev).manual_seed(3)
+    q = (torch.randn(H, M, D, device=dev, generator=g) * D ** -0.5).bfloat16()
+    k = torch.randn(B, H, N, D, device=dev, generator=g, dtype=torch.bfloat16)
+    v = torch.randn(B, H, N, D, device=dev, generator=g, dtype=torch.bfloat16)
+    assert k.numel() == 1 << 31
+    y = F.flare_multihead_mixer(q, k, v)
+    ks, vs = k[B - 1:, H - 1:].clone(), v[B - 1:, H - 1:].clone()
+    ys = F.flare_multihead_mixer(q[H - 1:], ks, vs)
+    assert O.rel_l2(y[B - 1:, H - 1:], ys) <= 2e-3        # same kernels, another split of N: rounding only
+    # and against the oracle on the first tokens of that slice: y_n needs z of the whole slice, from the small call
+    _, z = F.flare_multihead_mixer(q[H - 1:], ks, vs, return_z=True)
+    n = 4096
+    s = (ks[0, 0, :n].float() @ q[H - 1].float().T)
+    yr = torch.softmax(s, dim=-1) @ z[0, 0]
+    assert O.rel_l2(y[B - 1, H - 1, :n], yr) <= TOL[torch.bfloat16]
+    assert y.amax() <= v.amax() and y.amin() >= v.amin()    # every output is a convex combination of rows of v
+
+
+def test_graph_capture_and_replay(dev):
+    """The mixer and the causal prefill (whose flags are cleared by a kernel, not a memset) captured in a HIP
+    graph: every replay, with eager work in between, reproduces the eager result bit for bit."""
+    q, k, v = (t.to(dev) for t in make(2, 4, 5000, 128, 32, torch.bfloat16, seed=9))
+    y_eager = F.flare_multihead_mixer(q, k, v)
+    qc = (torch.randn(4, 128, 32, device=dev) * 0.3).bfloat16()
+    yc_eager, st_eager = F.flare_causal_prefill(qc, k, v)
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(2):      # warm the allocator on the side stream
+            F.flare_multihead_mixer(q, k, v)
+            F.flare_causal_prefill(qc, k, v)
+    torch.cuda.current_stream().wait_stream(s)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y_g = F.flare_multihead_mixer(q, k, v)
+        yc_g, st_g = F.flare_causal_prefill(qc, k, v)
+    for i in range(3):
+        y_g.zero_(); yc_g.zero_()
+        (k.float().sum() + i).item()          # eager work and a synchronisation between the replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_g, y_eager), f"mixer replay {i}"
+        assert torch.equal(yc_g, yc_eager), f"causal replay {i}"
+        assert all(torch.equal(a, b) for a, b in zip(st_g, st_eager))
