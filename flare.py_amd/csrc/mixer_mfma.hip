@@ -502,6 +502,14 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
     const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
 
     auto load_k = [&](int t0, u32x4 (&dst)[kSTW][KD]) {
+        if (CH == 4 * KD && t0 + kSTokWave <= wg_n1) {      // wave-uniform: whole tile in range, no per-lane tests
+            const uint16_t* kr = k + (int64_t)(t0 + c16) * a.ks[2] + g * 8;
+#pragma unroll
+            for (int tw = 0; tw < kSTW; ++tw)
+#pragma unroll
+                for (int kd = 0; kd < KD; ++kd) dst[tw][kd] = load16_stream(kr + (int64_t)tw * 16 * a.ks[2] + kd * 32);
+            return;
+        }
 #pragma unroll
         for (int tw = 0; tw < kSTW; ++tw)
 #pragma unroll
@@ -653,32 +661,41 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
         // normalise and store: lane (token c16, group g) owns d = (D/4) g .. (D/4) g + D/4 - 1
         const bool full = t0 + kSTokWave <= wg_n1 && mask == nullptr;   // wave-uniform: no per-row tests
         uint16_t* yr0 = y + (int64_t)(t0 + c16) * a.ys[2] + (D / 4) * g;
+        auto emit = [&](auto full_c) {
+            constexpr bool FULL = decltype(full_c)::value;
 #pragma unroll
-        for (int tw = 0; tw < kSTW; ++tw) {
-            const int n = t0 + tw * 16 + c16;
-            const bool on = full || (n < wg_n1 && (mask == nullptr || mask[n] != 0));
-            const float inv = on ? 1.f / lrow[tw] : 0.f;
-            if (a.lse_tok && g == 0 && (full || n < wg_n1))
-                a.lse_tok[((int64_t)b * a.H + h) * a.N + n] = (lshift[tw] + __log2f(lrow[tw])) * kLn2;
-            if (full || n < wg_n1) {
-                uint16_t* yr = yr0 + (int64_t)tw * 16 * a.ys[2];
-                uint32_t o[2 * RT];
+            for (int tw = 0; tw < kSTW; ++tw) {
+                const int n = t0 + tw * 16 + c16;
+                const bool in = FULL || n < wg_n1;
+                const bool on = FULL || (in && (mask == nullptr || mask[n] != 0));
+                const float inv = on ? __builtin_amdgcn_rcpf(lrow[tw]) : 0.f;
+                if (in) {
+                    uint16_t* yr = yr0 + (int64_t)tw * 16 * a.ys[2];
+                    uint32_t o[2 * RT];
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt) {
-                    o[2 * rt] = M_::pack2(yacc[tw][rt][0] * inv, yacc[tw][rt][1] * inv);
-                    o[2 * rt + 1] = M_::pack2(yacc[tw][rt][2] * inv, yacc[tw][rt][3] * inv);
-                }
-                if constexpr (RT == 1) {
-                    *reinterpret_cast<uint2*>(yr) = make_uint2(o[0], o[1]);
-                } else {
+                    for (int rt = 0; rt < RT; ++rt) {
+                        o[2 * rt] = M_::pack2(yacc[tw][rt][0] * inv, yacc[tw][rt][1] * inv);
+                        o[2 * rt + 1] = M_::pack2(yacc[tw][rt][2] * inv, yacc[tw][rt][3] * inv);
+                    }
+                    if constexpr (RT == 1) {
+                        *reinterpret_cast<uint2*>(yr) = make_uint2(o[0], o[1]);
+                    } else {
 #pragma unroll
-                    for (int i = 0; i < RT / 2; ++i) {
-                        const u32x4 ov = {o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
-                        __builtin_nontemporal_store(ov, reinterpret_cast<u32x4*>(yr + 8 * i));   // written once, never re-read here
+                        for (int i = 0; i < RT / 2; ++i) {
+                            const u32x4 ov = {o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]};
+                            __builtin_nontemporal_store(ov, reinterpret_cast<u32x4*>(yr + 8 * i));   // written once, never re-read here
+                        }
                     }
                 }
             }
-        }
+            if (a.lse_tok) {        // log-sum-exp of the token's scores, for the backward pass
+                float* lo = a.lse_tok + ((int64_t)b * a.H + h) * a.N + t0 + c16;
+#pragma unroll
+                for (int tw = 0; tw < kSTW; ++tw)
+                    if (g == 0 && (FULL || t0 + tw * 16 + c16 < wg_n1)) lo[tw * 16] = (lshift[tw] + __log2f(lrow[tw])) * kLn2;
+            }
+        };
+        if (full) emit(std::true_type{}); else emit(std::false_type{});
     };
 
     // two K register sets alternate, each fetched one tile before its use
