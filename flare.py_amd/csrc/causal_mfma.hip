@@ -7,9 +7,12 @@
 // block.  Per block and wave, with P = exp2(score - mu0) for the wave's latents (mu0 = the shift
 // of the incoming state, 0 for a fresh one; no running maximum):
 //   dcum[t,m] = den[m] + sum_{tau<=t} P[tau,m]          (MFMA with a lower-triangular ones matrix)
-//   G[t,m]    = P[t,m] / dcum[t,m]
+//   W[t,m]    = P[t,m] f[m],  f[m] = exp2(mu0[m] - max_m mu0)     (the token's softmax weight over the latents:
+//                                                                   one shift for all latents; f = 1 unless
+//                                                                   the state carries per-latent shifts)
+//   G[t,m]    = W[t,m] / dcum[t,m]
 //   Y[t,:]   += G[t,:] U  +  tril(G P^T)[t,:] V          (U = state numerator [m,d])
-//   r[t]     += sum_m P[t,m]                             (MFMA against ones)
+//   r[t]     += sum_m W[t,m]                             (MFMA against the factors f)
 //   U[m,:]   += P[:,m]^T V ;  den[m] += sum_tau P[tau,m]
 // and finally y_t = (sum over waves of Y[t,:]) / (sum over waves of r[t]).
 // A 16x16 accumulator tile (lane = column c16, registers = rows 4g..4g+3) is reused directly as the
@@ -82,6 +85,23 @@ __device__ __forceinline__ uint2 tr16(const void* lds_addr)
     const s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)lds_addr);
     asm volatile("" ::: "memory");
     return __builtin_bit_cast(uint2, r);
+}
+
+// The state's numerators and denominators are relative to a shift mu0[m] per latent, which cancels in
+// z = U/den.  The softmax over the latents of one token's scores needs ONE shift for all latents
+// instead: its weights are exp2(score - cref) = P[t,m] * exp2(mu0[m] - cref) with
+// cref = max_m mu0[m].  For a state this kernel produced itself mu0 is the same for every latent and
+// the factor is exactly 1; a state that comes from the fp32 kernel carries per-latent running maxima.
+__device__ __forceinline__ float common_shift(const float* mu_g, int M, int lane)
+{
+    float mx = kNegBig;
+    for (int m = lane; m < M; m += 64) {
+        const float mu = mu_g[m];
+        mx = fmaxf(mx, mu <= kNegBig ? 0.f : mu * kLog2e);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    return mx;
 }
 
 constexpr int kTB = 16;   // tokens per block
@@ -178,7 +198,23 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
         for (int i = 0; i < 4; ++i) e[i] = (4 * g + i <= c16) ? one : 0u;
         ltri = make_uint2(e[0] | (e[1] << 16), e[2] | (e[3] << 16));
     }
-    const u32x4 ones8 = {P_::kOnes2, P_::kOnes2, P_::kOnes2, P_::kOnes2};
+    // weights of the softmax over latents: fw[ct] = exp2(mu0 - cref) per column, and the same factors as a B
+    // operand (k-slots = the wave's latents 32 km + 4g + e / 32 km + 16 + 4g + e - 4) for the row sums
+    const float cref = common_shift(mu_g, M, lane);
+    float fw[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) fw[ct] = fast_exp2(mu0[ct] - cref);
+    u32x4 fop[KM];
+#pragma unroll
+    for (int km = 0; km < KM; ++km) {
+        float f8[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float mu = mu_g[m0 + km * 32 + (e >> 2) * 16 + 4 * g + (e & 3)];
+            f8[e] = fast_exp2((mu <= kNegBig ? 0.f : mu * kLog2e) - cref);
+        }
+        fop[km] = u32x4{P_::pack2(f8[0], f8[1]), P_::pack2(f8[2], f8[3]), P_::pack2(f8[4], f8[5]), P_::pack2(f8[6], f8[7])};
+    }
 
     // block staging: K as A operand straight from global memory, V through LDS (threads < 2 D)
     u32x4 ka[KD], kn[KD], vr;
@@ -320,7 +356,7 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
             den[ct] = P_::mma16(ones4, ppk[ct], den[ct]);
             float gv[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) gv[r] = p[ct][r] > 0.f ? p[ct][r] * __builtin_amdgcn_rcpf(dc[r]) : 0.f;
+            for (int r = 0; r < 4; ++r) gv[r] = p[ct][r] > 0.f ? p[ct][r] * fw[ct] * __builtin_amdgcn_rcpf(dc[r]) : 0.f;
             const uint2 gpk = make_uint2(P_::pack2(gv[0], gv[1]), P_::pack2(gv[2], gv[3]));
             *reinterpret_cast<uint2*>(&pt[w][ct * 16 + c16][4 * g]) = ppk[ct];
             *reinterpret_cast<uint2*>(&gt[w][ct * 16 + c16][4 * g]) = gpk;
@@ -345,7 +381,7 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
 #pragma unroll
         for (int km = 0; km < KM; ++km) {
             acct = P_::mma32(pop[km], gop[km], acct);
-            rsum = P_::mma32(pop[km], ones8, rsum);
+            rsum = P_::mma32(pop[km], fop[km], rsum);
         }
 #pragma unroll
         for (int r = 0; r < 4; ++r) acct[r] = (4 * g + r <= c16) ? acct[r] : 0.f;
@@ -453,7 +489,7 @@ template <int D> constexpr size_t causal_chunk_lds()
 {
     // q operands, V chunk, P^T and G^T of the four waves, U0 operands, column sums
     return (size_t)8 * (D / 32) * 64 * 16 + (size_t)kChunk * (D + kVPad) * 2 + 2 * (size_t)4 * 128 * 16 * 2 +
-           (size_t)4 * (D / 16) * 64 * 16 + (size_t)4 * 128 * 4;
+           (size_t)4 * (D / 16) * 64 * 16 + (size_t)4 * 128 * 4 + (size_t)4 * 4 * 16;
 }
 
 template <typename T, int D>
@@ -471,6 +507,7 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     uint16_t* gt = pt + 4 * M * 16;                                               // [4][M][16]
     u32x4* u0s = reinterpret_cast<u32x4*>(gt + 4 * M * 16);                       // [KS][DT][64]
     float* cs = reinterpret_cast<float*>(u0s + KS * DT * 64);                     // [4][M]
+    u32x4* fops = reinterpret_cast<u32x4*>(cs + 4 * M);                           // [KS][4]: weight factors as B operands
     __shared__ int bad_flag;
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
@@ -503,6 +540,19 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
         for (int i = 0; i < 4; ++i)
             o[i] = M_::pack2(M_::unpack(uint16_t(raw[i] & 0xffffu)) * sl2, M_::unpack(uint16_t(raw[i] >> 16)) * sl2);
         qs[idx] = o;
+    }
+    // factors exp2(mu0 - cref) of the softmax over latents as B operands: k-step ks, lane group gg hold the
+    // latents 32 ks + 4 gg + e (e < 4) and 32 ks + 16 + 4 gg + e - 4
+    const float cref = common_shift(mu_g, M, lane);
+    if (tid < KS * 4) {
+        const int ks = tid >> 2, gg = tid & 3;
+        float f8[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float mu = mu_g[ks * 32 + (e >> 2) * 16 + 4 * gg + (e & 3)];
+            f8[e] = fast_exp2((mu <= kNegBig ? 0.f : mu * kLog2e) - cref);
+        }
+        fops[tid] = u32x4{P_::pack2(f8[0], f8[1]), P_::pack2(f8[2], f8[3]), P_::pack2(f8[4], f8[5]), P_::pack2(f8[6], f8[7])};
     }
     // shift and running denominators of every latent (column c16 of tile ct), replicated in the waves
     float mu0[CTA], den0[CTA];
@@ -538,7 +588,6 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
         for (int i = 0; i < 4; ++i) e[i] = (4 * g + i <= c16) ? one : 0u;
         ltri = make_uint2(e[0] | (e[1] << 16), e[2] | (e[3] << 16));
     }
-    const u32x4 ones8 = {P_::kOnes2, P_::kOnes2, P_::kOnes2, P_::kOnes2};
     const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
 
     u32x4 ka[KD], kn[KD], vr[VPT];
@@ -613,6 +662,10 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) p[ct][r] = (4 * g + r < tbw) ? fast_exp2(sc[ct][r] - mu0[ct]) : 0.f;
                 ppk[ct] = make_uint2(P_::pack2(p[ct][0], p[ct][1]), P_::pack2(p[ct][2], p[ct][3]));
+                // from here on p holds the token's softmax weight exp2(score - cref) = P * exp2(mu0 - cref)
+                const float fw = fast_exp2(mu0[ct] - cref);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) p[ct][r] *= fw;
             }
             f32x4 csv[CTA];
 #pragma unroll
@@ -650,7 +703,7 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
         // softmax sums over the latents of the wave's tokens (rows t = 4g + r, equal in every column)
         f32x4 rsum = zf;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) rsum = P_::mma32(pop[ks], ones8, rsum);
+        for (int ks = 0; ks < KS; ++ks) rsum = P_::mma32(pop[ks], fops[ks * 4 + g], rsum);
 
         // ---- outputs: G U0, then the chunk's own tokens up to and including this wave's ----
         f32x4 yacc[DT];

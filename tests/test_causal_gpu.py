@@ -206,3 +206,35 @@ def test_mfma_prefill_fallback_from_a_middle_segment(dev):
     assert O.rel_l2(y[:, 0], yr[:, 0, 100:]) <= 1e-2
     assert O.rel_l2(y[:, 1], yr[:, 1, 100:]) <= 2e-2
     state_close(st, str_, 2e-2)
+
+
+@pytest.mark.parametrize("M,D", [(128, 64), (256, 32)])
+def test_mfma_continues_a_state_with_per_latent_shifts(dev, M, D):
+    """The fp32 kernel leaves a running maximum PER LATENT in the state (mu differs from latent to latent by
+    several units here).  The matrix-core kernels keep those shifts for the state but must weigh the latents of
+    one token against each other with ONE common shift: prefill (64-token chunks at M = 128, 16-token blocks at
+    M = 256) and decode, continued from such a state, against one long pass of the oracle."""
+    N1, N2, ND = 300, 200, 9
+    q, k, v = make(1, 2, N1 + N2 + ND, M, D, torch.bfloat16, seed=11, std=0.8)
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float())
+    _, st = F.flare_causal_prefill(q.float().to(dev), k[:, :, :N1].float().to(dev), v[:, :, :N1].float().to(dev))
+    assert float((st[0].amax(-1) - st[0].amin(-1)).min()) > 2.0      # the shifts really differ
+    y2, st2 = F.flare_causal_prefill(q.to(dev), k[:, :, N1:N1 + N2].to(dev), v[:, :, N1:N1 + N2].to(dev), state=st)
+    assert O.rel_l2(y2, yr[:, :, N1:N1 + N2]) <= TOL[torch.bfloat16]
+    y3, st3 = F.flare_causal_decode(q.to(dev), k[:, :, N1 + N2:].to(dev), v[:, :, N1 + N2:].to(dev), st2)
+    assert O.rel_l2(y3, yr[:, :, N1 + N2:]) <= TOL[torch.bfloat16]
+    state_close(st3, str_, TOL[torch.bfloat16])
+
+
+def test_mfma_continues_after_a_fallback(dev):
+    """A (b,h) the matrix-core kernel could not validate is redone by the fp32 kernel, which leaves per-latent
+    shifts in its state; the next call starts from that state on the matrix cores again."""
+    q, k, v = make(1, 2, 264, 128, 64, torch.bfloat16, seed=7, std=1.0)
+    k[:, 0, :200] *= 8.0                # head 0 leaves the window during the first call only
+    k[:, 0, 200:] *= 0.05
+    k[:, 1] *= 0.05
+    yr, _ = O.causal_recurrent(q.float(), k.float(), v.float())
+    _, st = F.flare_causal_prefill(q.to(dev), k[:, :, :200].to(dev), v[:, :, :200].to(dev))
+    y, _ = F.flare_causal_prefill(q.to(dev), k[:, :, 200:].to(dev), v[:, :, 200:].to(dev), state=st)
+    assert torch.isfinite(y.float()).all()
+    assert O.rel_l2(y, yr[:, :, 200:]) <= TOL[torch.bfloat16]
