@@ -217,3 +217,34 @@ def test_bigflare_ablation_model(dev, kw):
     assert O.rel_l2(g, gr) <= 1e-3
     g, gr = model.blocks[0].att.k_proj.fc1.weight.grad, ref.blocks[0].att.k_proj.fc1.weight.grad
     assert O.rel_l2(g, gr) <= 1e-3
+
+
+def test_autocast_training_step_gradients(dev, monkeypatch):
+    """One bf16-autocast training step of FLAREModel: the mixer runs forward and backward on the HIP kernels
+    (token-major output, strided gradient, fp32 latent parameter cast per call); gradients against the same model
+    in fp64 on the CPU with the oracle mixer.  Tolerance: bf16 arithmetic through two blocks."""
+    torch.manual_seed(8)
+    m = FLAREModel(in_dim=4, out_dim=3, channel_dim=64, num_blocks=2, num_heads=4, num_latents=64).to(dev).train()
+    with torch.no_grad():
+        for p_ in m.parameters():
+            if p_.dim() == 2:
+                p_.mul_(6.0)
+    x = torch.randn(2, 700, 4, device=dev)
+    tgt = torch.randn(2, 700, 3, device=dev)
+    assert functional._hip_backward_ok(torch.empty(4, 64, 16, device=dev, dtype=torch.bfloat16),
+                                       torch.empty(2, 4, 700, 16, device=dev, dtype=torch.bfloat16),
+                                       torch.empty(2, 4, 700, 16, device=dev, dtype=torch.bfloat16), None, False)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        loss = (m(x).float() - tgt).square().mean()
+    loss.backward()
+    _, cpu = oracle_forward(m, x, monkeypatch)
+    cpu = cpu.double()
+    for p_ in cpu.parameters():
+        p_.grad = None
+    loss_r = (cpu(x.cpu().double()) - tgt.cpu().double()).square().mean()
+    loss_r.backward()
+    assert abs(float(loss.detach()) - float(loss_r.detach())) <= 3e-2 * abs(float(loss_r.detach()))
+    got = dict(m.named_parameters())
+    for name, pr in cpu.named_parameters():
+        if name in ("blocks.0.att.latent_q", "blocks.1.att.k_proj.fc1.weight", "blocks.0.att.v_proj.fc2.weight", "in_proj.fc1.weight"):
+            assert O.rel_l2(got[name].grad, pr.grad) <= 6e-2, name
