@@ -280,3 +280,23 @@ def test_graph_capture_and_replay(dev):
         assert torch.equal(y_g, y_eager), f"mixer replay {i}"
         assert torch.equal(yc_g, yc_eager), f"causal replay {i}"
         assert all(torch.equal(a, b) for a, b in zip(st_g, st_eager))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_localized_large_scores_mix_fast_and_exact_paths(dev, dtype):
+    """A short burst of tokens with scores far outside the window in which the kernels may skip the running
+    maximum: only the token splits / tiles that contain the burst take the exact path, the rest stays on the fast
+    one, and the merge has to combine partials with and without a shift."""
+    B, H, N, M, D = 1, 2, 40000, 128, 32
+    q, k, v = make(B, H, N, M, D, dtype, seed=21, qstd=1.0)
+    k[:, :, 17000:17100] *= 6.0
+    s = torch.einsum("hmd,bhnd->bhmn", q.float(), k.float())
+    assert float(s[:, :, :, 17000:17100].abs().max()) > 130 and float(s[:, :, :, :17000].abs().max()) < 60
+    y, _ = check(dev, q, k, v)
+    # and the gradients on the same inputs (both exponentials of the backward are bounded by construction)
+    gy = torch.randn(B, H, N, D, generator=torch.Generator().manual_seed(1)).to(dtype)
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    F.flare_multihead_mixer(qd, kd, vd).backward(gy.to(dev))
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    O.mixer_explicit(qr, kr, vr, 1.0)[0].backward(gy.double())
+    assert O.rel_l2(qd.grad, qr.grad) <= 3e-2 and O.rel_l2(kd.grad, kr.grad) <= 3e-2 and O.rel_l2(vd.grad, vr.grad) <= 3e-2
