@@ -489,7 +489,7 @@ template <int D> constexpr size_t causal_chunk_lds()
 {
     // q operands, V chunk, P^T and G^T of the four waves, U0 operands, column sums
     return (size_t)8 * (D / 32) * 64 * 16 + (size_t)kChunk * (D + kVPad) * 2 + 2 * (size_t)4 * 128 * 16 * 2 +
-           (size_t)4 * (D / 16) * 64 * 16 + (size_t)4 * 128 * 4 + (size_t)4 * 4 * 16;
+           (size_t)4 * (D / 16) * 64 * 16 + (size_t)4 * 128 * 4 + (size_t)4 * 4 * 16 + (size_t)2 * 128 * 4;
 }
 
 template <typename T, int D>
@@ -508,6 +508,8 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     u32x4* u0s = reinterpret_cast<u32x4*>(gt + 4 * M * 16);                       // [KS][DT][64]
     float* cs = reinterpret_cast<float*>(u0s + KS * DT * 64);                     // [4][M]
     u32x4* fops = reinterpret_cast<u32x4*>(cs + 4 * M);                           // [KS][4]: weight factors as B operands
+    float* mu0s = reinterpret_cast<float*>(fops + KS * 4);                        // [M] shift of each latent (log2 units)
+    float* fws = mu0s + M;                                                        // [M] weight factor exp2(mu0 - cref)
     __shared__ int bad_flag;
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
@@ -554,13 +556,19 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
         }
         fops[tid] = u32x4{P_::pack2(f8[0], f8[1]), P_::pack2(f8[2], f8[3]), P_::pack2(f8[4], f8[5]), P_::pack2(f8[6], f8[7])};
     }
-    // shift and running denominators of every latent (column c16 of tile ct), replicated in the waves
-    float mu0[CTA], den0[CTA];
+    // per-latent shift and weight factor: small tables in LDS (registers are short in this kernel)
+    if (tid < M) {
+        const float mu = mu_g[tid];
+        const float m2 = mu <= kNegBig ? 0.f : mu * kLog2e;
+        mu0s[tid] = m2;
+        fws[tid] = fast_exp2(m2 - cref);
+    }
+    // running denominators of every latent (column c16 of tile ct), replicated in the waves
+    float den0[CTA];
 #pragma unroll
     for (int ct = 0; ct < CTA; ++ct) {
         const int m = ct * 16 + c16;
         const float mu = mu_g[m];
-        mu0[ct] = mu <= kNegBig ? 0.f : mu * kLog2e;
         float d0 = mu <= kNegBig ? 0.f : den_g[m];
         for (int s = 0; s < seg; ++s) d0 += a.seg_den[((int64_t)bh * a.n_segs + s) * M + m];
         den0[ct] = d0;
@@ -659,13 +667,10 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
             }
 #pragma unroll
             for (int ct = 0; ct < CTA; ++ct) {
+                const float mu0 = mu0s[ct * 16 + c16];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) p[ct][r] = (4 * g + r < tbw) ? fast_exp2(sc[ct][r] - mu0[ct]) : 0.f;
+                for (int r = 0; r < 4; ++r) p[ct][r] = (4 * g + r < tbw) ? fast_exp2(sc[ct][r] - mu0) : 0.f;
                 ppk[ct] = make_uint2(P_::pack2(p[ct][0], p[ct][1]), P_::pack2(p[ct][2], p[ct][3]));
-                // from here on p holds the token's softmax weight exp2(score - cref) = P * exp2(mu0 - cref)
-                const float fw = fast_exp2(mu0[ct] - cref);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) p[ct][r] *= fw;
             }
             f32x4 csv[CTA];
 #pragma unroll
@@ -690,8 +695,9 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
             den0[ct] = den0[ct] + c0 + c1 + c2 + c3;        // same order in every wave
             const f32x4 dc = P_::mma16(ltri, ppk[ct], zf);
             float gv[4];
+            const float fw = fws[m];      // the token's softmax weight over the latents is P * exp2(mu0 - cref)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) gv[r] = p[ct][r] > 0.f ? p[ct][r] * __builtin_amdgcn_rcpf(dc[r] + base) : 0.f;
+            for (int r = 0; r < 4; ++r) gv[r] = p[ct][r] > 0.f ? p[ct][r] * fw * __builtin_amdgcn_rcpf(dc[r] + base) : 0.f;
             *reinterpret_cast<uint2*>(gtw + (ct * 16 + c16) * 16 + 4 * g) = make_uint2(P_::pack2(gv[0], gv[1]), P_::pack2(gv[2], gv[3]));
         }
         u32x4 gop[KS], pop[KS];
@@ -799,7 +805,7 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     for (int mt = 0; mt < MT; ++mt) {
         const int ct = 2 * w + mt, m = ct * 16 + c16;
         if (g == 0) {
-            if (single) mu_g[m] = mu0[ct] * kLn2;
+            if (single) mu_g[m] = mu0s[m] * kLn2;
             den_o[m] = den0[ct];
         }
 #pragma unroll
