@@ -896,6 +896,7 @@ bool causal_mfma_supported(int dtype, int M, int D)
 
 hipError_t launch_causal_mfma(const CausalArgs& a, int dtype, int step, hipStream_t st)
 {
+    if (step == 1) return launch_causal_decode_steps(a, dtype, st);      // a decode step has no matrix shape
     return dtype == 1 ? launch_t<bf16_t>(a, step, st) : launch_t<f16_t>(a, step, st);
 }
 

@@ -135,6 +135,7 @@ hipError_t launch_causal_prefill(const CausalArgs& a, int dtype, hipStream_t st)
 hipError_t launch_causal_decode(const CausalArgs& a, int dtype, hipStream_t st);
 bool       causal_mfma_supported(int dtype, int M, int D);
 hipError_t launch_causal_mfma(const CausalArgs& a, int dtype, int step, hipStream_t st);   // step 16 prefill, 1 decode
+hipError_t launch_causal_decode_steps(const CausalArgs& a, int dtype, hipStream_t st);      // N one-token steps, same shapes as above
 
 size_t     mixer_bwd_lds_bytes(int M, int D);
 bool       mixer_bwd_supported(int dtype, int M, int D);
