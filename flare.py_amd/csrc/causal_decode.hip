@@ -29,20 +29,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr float kLMin = 8.6736174e-19f, kLMax = 1.329228e36f;   // 2^-60, 2^120
 constexpr int kDecWaves = 8;
 
-// x + (x of lane ^ 16) and x + (x of lane ^ 32) with the row / half swaps of gfx950 (vector ALU, no LDS crossbar):
-// swapping a register with its own copy leaves one of the pair holding the partner's value in every lane.
-typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ float sum_xor16(float x)
-{
-    const u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-__device__ __forceinline__ float sum_xor32(float x)
-{
-    const u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-
 template <typename T> struct Dt;
 template <> struct Dt<bf16_t> {
     static __device__ __forceinline__ float dot2(uint32_t x, uint32_t y, float acc)

@@ -33,6 +33,31 @@ template <> __device__ __forceinline__ f16_t from_f32<f16_t>(float v) { return f
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// The value of lane ^ 16 / lane ^ 32 with the row / half swaps of gfx950 (vector ALU, no LDS crossbar):
+// swapping a register with its own copy leaves, in every lane, the lane's own value in one register of the
+// pair and its partner's in the other.
+typedef unsigned flare_u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ float sum_xor16(float x)
+{
+    const flare_u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float sum_xor32(float x)
+{
+    const flare_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float max_xor16(float x)
+{
+    const flare_u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float max_xor32(float x)
+{
+    const flare_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 // ---- kernel argument blocks (host fills them; passed by value) -------------------------
 struct MixerArgs {
     const void* q; const void* k; const void* v; void* y;

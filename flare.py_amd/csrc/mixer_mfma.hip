@@ -126,14 +126,14 @@ template <typename T> __device__ __forceinline__ u32x4 to_bf16x8(u32x4 v)
 
 __device__ __forceinline__ float xg_max(float v)  // max over the 4 lane groups of a column
 {
-    v = fmaxf(v, __shfl_xor(v, 16));
-    v = fmaxf(v, __shfl_xor(v, 32));
+    v = max_xor16(v);
+    v = max_xor32(v);
     return v;
 }
 __device__ __forceinline__ float xg_sum(float v)
 {
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
+    v = sum_xor16(v);
+    v = sum_xor32(v);
     return v;
 }
 

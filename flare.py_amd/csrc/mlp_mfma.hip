@@ -89,8 +89,8 @@ __device__ __forceinline__ void store4(void* base, int64_t elem, int dt, f32x4 v
 
 __device__ __forceinline__ float xg_sum(float v)   // sum over the 4 lane groups that share a token
 {
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
+    v = sum_xor16(v);
+    v = sum_xor32(v);
     return v;
 }
 
