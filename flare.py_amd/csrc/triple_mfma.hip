@@ -79,6 +79,20 @@ __device__ __forceinline__ uint2 load_feat4(const uint16_t* p, bool live, int fm
                       Tm<T>::pack2(featf(Tm<T>::lo(raw.y), fm), featf(Tm<T>::hi(raw.y), fm)));
 }
 
+// Sum over the 16 lanes of a row with DPP operands (vector ALU only): pairs, quads, half rows, the row.
+template <int CTRL> __device__ __forceinline__ float dpp_of(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row16_sum(float x)
+{
+    x += dpp_of<0xB1>(x);      // quad_perm [1,0,3,2]
+    x += dpp_of<0x4E>(x);      // quad_perm [2,3,0,1]
+    x += dpp_of<0x141>(x);     // row_half_mirror
+    x += dpp_of<0x140>(x);     // row_mirror
+    return x;
+}
+
 constexpr int kD = 16;
 
 // grid (n_splits, H, B); wave w of a workgroup takes the 16-token tiles w, w+4, ... of the split.
@@ -89,6 +103,7 @@ __global__ __launch_bounds__(256) void triple_state_mfma_kernel(TripleArgs a)
     __shared__ __attribute__((aligned(16))) uint16_t k1s[4][16][kD];
     __shared__ __attribute__((aligned(16))) uint16_t k2s[4][16][kD];
     __shared__ __attribute__((aligned(16))) uint16_t vs[4][16][kD];
+    __shared__ __attribute__((aligned(16))) float k2f[4][16][kD];      // f(k2) of the tile in fp32, for the scalar factors
     __shared__ __attribute__((aligned(16))) float red[kD + 1][64][4];
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
@@ -124,7 +139,9 @@ __global__ __launch_bounds__(256) void triple_state_mfma_kernel(TripleArgs a)
         const bool live = n0 + tok < n_end;
         fetch(n0 + 64, x1, x2, xv);
         *reinterpret_cast<uint2*>(&k1s[w][tok][piece]) = feat4(c1, live);
-        *reinterpret_cast<uint2*>(&k2s[w][tok][piece]) = feat4(c2, live);
+        const uint2 f2 = feat4(c2, live);
+        *reinterpret_cast<uint2*>(&k2s[w][tok][piece]) = f2;
+        *reinterpret_cast<f32x4*>(&k2f[w][tok][piece]) = f32x4{M_::lo(f2.x), M_::hi(f2.x), M_::lo(f2.y), M_::hi(f2.y)};
         *reinterpret_cast<uint2*>(&vs[w][tok][piece]) = live ? cv : make_uint2(0u, 0u);
         c1 = x1; c2 = x2; cv = xv;
 
@@ -136,19 +153,15 @@ __global__ __launch_bounds__(256) void triple_state_mfma_kernel(TripleArgs a)
         kk = M_::mma16(k1t, k2t, kk);
         const float a0 = M_::lo(k1t.x), a1 = M_::hi(k1t.x), a2 = M_::lo(k1t.y), a3 = M_::hi(k1t.y);
         // f(k2) rows of the lane's four tokens
-        u32x4 r[4][2];
+        f32x4 r[4][4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            r[e][0] = *reinterpret_cast<const u32x4*>(&k2s[w][4 * g + e][0]);
-            r[e][1] = *reinterpret_cast<const u32x4*>(&k2s[w][4 * g + e][8]);
-        }
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) r[e][c] = *reinterpret_cast<const f32x4*>(&k2f[w][4 * g + e][4 * c]);
 #pragma unroll
         for (int k = 0; k < kD; ++k) {
-            const int wd = (k >> 1) & 3, hf = k >> 3;
-            float c[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) c[e] = (k & 1) ? M_::hi(r[e][hf][wd]) : M_::lo(r[e][hf][wd]);
-            const uint2 ak = make_uint2(M_::pack2(a0 * c[0], a1 * c[1]), M_::pack2(a2 * c[2], a3 * c[3]));
+            const int kc = k >> 2, ke = k & 3;
+            const uint2 ak = make_uint2(M_::pack2(a0 * r[0][kc][ke], a1 * r[1][kc][ke]), M_::pack2(a2 * r[2][kc][ke], a3 * r[3][kc][ke]));
             S[k] = M_::mma16(ak, vt, S[k]);
         }
     }
@@ -186,7 +199,7 @@ __global__ __launch_bounds__(256) void triple_out_mfma_kernel(TripleArgs a, int 
 {
     using M_ = Tm<T>;
     __shared__ __attribute__((aligned(16))) uint16_t q1s[4][16][kD];
-    __shared__ __attribute__((aligned(16))) uint16_t q2s[4][16][kD];
+    __shared__ __attribute__((aligned(16))) float q2f[4][16][kD];     // f(q2) of the tile in fp32: multiplied as it is
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
     const int h = blockIdx.y, b = blockIdx.z;
@@ -230,39 +243,28 @@ __global__ __launch_bounds__(256) void triple_out_mfma_kernel(TripleArgs a, int 
     if (wg_n0 + w * 16 < wg_n1) fetch(wg_n0 + w * 16, f1, f2);
     for (int n0 = wg_n0 + w * 16; n0 < wg_n1; n0 += 64) {
         *reinterpret_cast<uint2*>(&q1s[w][tok][piece]) = f1;
-        *reinterpret_cast<uint2*>(&q2s[w][tok][piece]) = f2;
+        *reinterpret_cast<f32x4*>(&q2f[w][tok][piece]) = f32x4{M_::lo(f2.x), M_::hi(f2.x), M_::lo(f2.y), M_::hi(f2.y)};
         if (n0 + 64 < wg_n1) fetch(n0 + 64, f1, f2);
 
         // A operand: row = token c16, k-slots i = 4g..4g+3
         const uint2 q1a = *reinterpret_cast<const uint2*>(&q1s[w][c16][4 * g]);
-        u32x4 r[4][2];
+        f32x4 r[4][4];       // f(q2)[n = 4g + e][k = 4 c .. 4 c + 3]
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            r[e][0] = *reinterpret_cast<const u32x4*>(&q2s[w][4 * g + e][0]);
-            r[e][1] = *reinterpret_cast<const u32x4*>(&q2s[w][4 * g + e][8]);
-        }
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) r[e][c] = *reinterpret_cast<const f32x4*>(&q2f[w][4 * g + e][4 * c]);
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};   // out[n = 4g + r][j = c16]
 #pragma unroll
         for (int k = 0; k < kD; ++k) {
-            const int wd = (k >> 1) & 3, hf = k >> 3;
             const f32x4 t = M_::mma16(q1a, sk[k], f32x4{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float c = (k & 1) ? M_::hi(r[e][hf][wd]) : M_::lo(r[e][hf][wd]);
-                acc[e] = fmaf(t[e], c, acc[e]);
-            }
+            for (int e = 0; e < 4; ++e) acc[e] = fmaf(t[e], r[e][k >> 2][k & 3], acc[e]);
         }
         if (a.normalize) {
             // den[n] = sum_k' (f(q1)[n,:] kk[:,k']) f(q2)[n,k'] : k' runs over the 16 lanes of a row group
             const f32x4 wv = M_::mma16(q1a, kkb, f32x4{0.f, 0.f, 0.f, 0.f});
-            const uint2 q2t = tr16(&q2s[w][4 * g + (c16 >> 2)][(c16 & 3) * 4]);   // f(q2)[n = 4g+e][k' = c16]
-            float dn[4] = {wv[0] * M_::lo(q2t.x), wv[1] * M_::hi(q2t.x), wv[2] * M_::lo(q2t.y), wv[3] * M_::hi(q2t.y)};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-#pragma unroll
-                for (int o = 8; o > 0; o >>= 1) dn[e] += __shfl_xor(dn[e], o);
-                acc[e] = acc[e] / dn[e];
-            }
+            for (int e = 0; e < 4; ++e) acc[e] = acc[e] / row16_sum(wv[e] * q2f[w][4 * g + e][c16]);
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
