@@ -219,7 +219,6 @@ hipError_t launch_t(const CausalArgs& a, hipStream_t st)
     dim3 grid(a.B * a.H), block(64 * kDecWaves);
     if (a.M == 128 && a.D == 64)      hipLaunchKernelGGL((causal_decode_kernel<T, 64, 16>), grid, block, 0, st, a);
     else if (a.M == 128 && a.D == 32) hipLaunchKernelGGL((causal_decode_kernel<T, 32, 16>), grid, block, 0, st, a);
-    else if (a.M == 256 && a.D == 64) hipLaunchKernelGGL((causal_decode_kernel<T, 64, 32>), grid, block, 0, st, a);
     else if (a.M == 256 && a.D == 32) hipLaunchKernelGGL((causal_decode_kernel<T, 32, 32>), grid, block, 0, st, a);
     else return hipErrorInvalidValue;
     return hipGetLastError();

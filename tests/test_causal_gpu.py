@@ -238,3 +238,17 @@ def test_mfma_continues_after_a_fallback(dev):
     y, _ = F.flare_causal_prefill(q.to(dev), k[:, :, 200:].to(dev), v[:, :, 200:].to(dev), state=st)
     assert torch.isfinite(y.float()).all()
     assert O.rel_l2(y, yr[:, :, 200:]) <= TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("M,D", [(128, 64), (128, 32), (256, 32)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_decode_kernel_shapes(dev, M, D, dtype):
+    """Every instantiation of the one-launch decode kernel: 37 steps from a fresh state and 21 more from the state
+    they leave, against the oracle's recurrence; the state at the end against the oracle's."""
+    q, k, v = make(2, 3, 58, M, D, dtype, seed=5)
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float())
+    st = F.causal_fresh_state(2, 3, M, D, dev)
+    y1, st = F.flare_causal_decode(q.to(dev), k[:, :, :37].to(dev), v[:, :, :37].to(dev), st)
+    y2, st = F.flare_causal_decode(q.to(dev), k[:, :, 37:].to(dev), v[:, :, 37:].to(dev), st)
+    assert O.rel_l2(torch.cat([y1, y2], 2), yr) <= TOL[dtype]
+    state_close(st, str_, TOL[dtype])
