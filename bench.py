@@ -7,7 +7,9 @@ One step = one forward of the mixer (split-N gather, merge, scatter) over the he
 B=1, H=8, N=1,048,576, M=256, D=32, bf16 in / fp32 accumulate, inputs resident in HBM.
 Prints ONE JSON line: tokens/s, the roofline of the dominant kernel (measured with HIP events
 on the launch stream), and the CPU baseline (torch SDPA, MATH backend, fp32) timed on this
-machine's host cores on a bounded sample of the same workload.
+machine's host cores on a bounded sample of the same workload.  Before the W warm-up steps the step is
+called until at least 40 untimed calls have been made in all: a freshly started process runs its first ~30 ms
+of GPU work about 7 % slower than the steady state.
 
 --workload selects one of the other configurations instead (same JSON shape, one line): causal =
 causal FLARE prefill of 8192 tokens + 256 decode steps at B=8,H=16,M=128,D=64; triple = triple
@@ -81,9 +83,12 @@ def cpu_baseline(q, k, v, n_sample):
     return torch.cat(outs, dim=1), dt
 
 
+SETTLE_STEPS = 40   # untimed calls before the warm-up proper: the device needs ~30 ms of work to reach its steady clocks
+
+
 def wall_ms(fn, steps, warmup):
     """Wall-clock ms per call between device synchronisations."""
-    for _ in range(warmup):
+    for _ in range(max(0, SETTLE_STEPS - warmup) + warmup):
         fn()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -258,7 +263,7 @@ def main():
 
     # ---- whole step, wall clock between device synchronisations -------------------------
     step = lambda: F.flare_multihead_mixer(q, k, v)
-    for _ in range(args.warmup):
+    for _ in range(max(0, SETTLE_STEPS - args.warmup) + args.warmup):   # at least SETTLE_STEPS untimed calls in all
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
