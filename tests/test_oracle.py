@@ -282,3 +282,62 @@ def test_residual_mlp_oracle_matches_torch_layers():
     gv = O.gelu_tanh(t)
     assert gv[0] == 0 and abs(float(gv[1]) - 0.8411919906082768) < 1e-12
     assert torch.allclose(gv[1] - gv[2], t[1]) and torch.allclose(gv[3] - gv[4], t[3])
+
+
+# ---------------------------------------------------------------- frozen known answers
+def _golden():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "vectors.json")) as f:
+        return json.load(f)
+
+
+def _t(x, dtype=torch.float64):
+    return torch.tensor(x, dtype=dtype)
+
+
+def test_golden_vectors_pin_both_oracles():
+    """tests/golden/vectors.json holds outputs of pure-Python-float loops over the definitions
+    (tests/golden/make_vectors.py).  The torch oracle (fp64) and the C oracle (fp32) must reproduce them."""
+    g = _golden()
+    m = g["mixer"]
+    q, k, v = _t(m["q"]), _t(m["k"]).unsqueeze(0), _t(m["v"]).unsqueeze(0)
+    assert O.rel_l2(O.mixer_explicit(q, k, v, m["scale"])[0][0], _t(m["y"])) < 1e-12
+    assert O.rel_l2(O.mixer_sdpa(q.float(), k.float(), v.float(), m["scale"])[0][0], _t(m["y"])) < 2e-6
+    assert O.rel_l2(c_oracle.mixer(q, k, v, m["scale"])[0][0], _t(m["y"])) < 2e-6
+    c = g["causal"]
+    q, k, v = _t(c["q"]), _t(c["k"]).unsqueeze(0), _t(c["v"]).unsqueeze(0)
+    assert O.rel_l2(O.causal_recurrent(q, k, v, c["scale"])[0][0], _t(c["y"])) < 1e-12
+    assert O.rel_l2(O.causal_bruteforce(q, k, v, c["scale"])[0], _t(c["y"])) < 1e-12
+    assert O.rel_l2(c_oracle.causal(q, k, v, c["scale"])[0][0], _t(c["y"])) < 2e-6
+    t = g["triple"]
+    a = [_t(t[n]).unsqueeze(0) for n in ("q1", "q2", "k1", "k2", "v")]
+    st, out = O.triple_einsum(*a, dtype=torch.float64)
+    assert O.rel_l2(st[0], _t(t["state"])) < 1e-12 and O.rel_l2(out[0], _t(t["out"])) < 1e-12
+    st, out = O.triple_reference_scaling(*[x.float() for x in a])
+    assert O.rel_l2(st[0], _t(t["state"])) < 2e-6 and O.rel_l2(out[0], _t(t["out"])) < 2e-6
+    st, out = c_oracle.triple(*a)
+    assert O.rel_l2(st[0], _t(t["state"])) < 2e-6 and O.rel_l2(out[0], _t(t["out"])) < 2e-6
+    cl = g["causal_linear"]
+    q, k, v = _t(cl["q"]).unsqueeze(0), _t(cl["k"]).unsqueeze(0), _t(cl["v"]).unsqueeze(0)
+    assert O.rel_l2(O.causal_linear_recurrent(q, k, v)[0], _t(cl["y"])) < 1e-12
+    assert O.rel_l2(O.causal_linear_chunked(q, k, v, chunk=4)[0], _t(cl["y"])) < 1e-12
+
+
+def test_golden_vectors_are_reproducible(tmp_path):
+    """The committed fixture is what its generator writes (plain Python floats: platform independent up to libm's exp)."""
+    import importlib.util
+    import json
+    import os
+    here = os.path.join(os.path.dirname(__file__), "golden")
+    spec = importlib.util.spec_from_file_location("make_vectors", os.path.join(here, "make_vectors.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    mod.HERE = str(tmp_path)
+    mod.main()
+    new = json.load(open(tmp_path / "vectors.json"))
+    old = _golden()
+    for key in old:
+        for name, val in old[key].items():
+            a, b = torch.tensor(val, dtype=torch.float64), torch.tensor(new[key][name], dtype=torch.float64)
+            assert torch.allclose(a, b, rtol=1e-13, atol=1e-15), (key, name)
