@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(HERE, "libflare_hip.so")
 FLARE_OK, FLARE_EINVAL, FLARE_EUNSUPPORTED, FLARE_EWORKSPACE, FLARE_EHIP = 0, -1, -2, -3, -4
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 FLAG_FORCE_GENERIC = 1
+MLP_EXPAND = 1
 ABI_VERSION = 1
 
 I3 = C.c_int64 * 3
@@ -85,6 +86,8 @@ SYMBOLS = {
     "flare_causal_linear_workspace_bytes": (C.c_int, [C.POINTER(FlareCausalLinearDesc), C.POINTER(_SZ)]),
     "flare_causal_linear_fwd": (C.c_int, [C.POINTER(FlareCausalLinearDesc), _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_mlp_fwd": (C.c_int, [C.POINTER(FlareMlpDesc), _P, _P, _P, _P, _P, _P, _P, _P]),
+    "flare_mlp_io_fwd": (C.c_int, [C.POINTER(FlareMlpDesc), C.c_int32, C.c_int32, _P, _P, C.c_int32,
+                                   _P, _P, _P, _P, _P, _P, _P, _P]),
     "flare_triple_workspace_bytes": (C.c_int, [C.POINTER(FlareTripleDesc), C.POINTER(_SZ)]),
     "flare_triple_state_fwd": (C.c_int, [C.POINTER(FlareTripleDesc), _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_triple_out_fwd": (C.c_int, [C.POINTER(FlareTripleDesc), _P, _P, _P, _P, _P, _P]),

@@ -587,8 +587,9 @@ int flare_causal_linear_fwd(const FlareCausalLinearDesc* desc, const void* q, co
     return hip_status(flare::launch_causal_linear(a, desc->dtype, static_cast<hipStream_t>(stream)), "causal linear launch");
 }
 
-int flare_mlp_fwd(const FlareMlpDesc* d, const void* x, const void* w, const float* bias, const float* gamma,
-                  const float* beta, const void* res, void* y, void* stream)
+static int mlp_fwd_impl(const FlareMlpDesc* d, int in_dim, int in_act, const float* w_in, const float* b_in, int out_dim,
+                        const void* x, const void* w, const float* bias, const float* gamma, const float* beta,
+                        const void* res, void* y, void* stream)
 {
     if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
     if (d->T < 1 || d->L < 1 || d->L > 16) return fail(FLARE_EINVAL, "T >= 1 and 1 <= L <= 16 required (got %lld, %d)", (long long)d->T, d->L);
@@ -602,21 +603,52 @@ int flare_mlp_fwd(const FlareMlpDesc* d, const void* x, const void* w, const flo
     if (!x || !w || !y) return fail(FLARE_EINVAL, "x, w, y must not be NULL");
     if (d->norm != FLARE_NORM_NONE && !gamma) return fail(FLARE_EINVAL, "gamma must not be NULL when a norm is requested");
     if (d->norm != FLARE_NORM_NONE && !(d->eps >= 0.f)) return fail(FLARE_EINVAL, "eps must be >= 0");
-    if (d->x_stride < d->C || d->y_stride < d->C || (res && d->res_stride < d->C))
-        return fail(FLARE_EINVAL, "row strides must be >= C");
-    // every lane moves 4 consecutive elements at a time
-    if (d->x_stride % 4 || d->y_stride % 4 || (res && d->res_stride % 4)) return fail(FLARE_EINVAL, "row strides must be multiples of 4");
-    if (!aligned16(x) || !aligned16(y) || !aligned16(w) || (res && !aligned16(res)) || (bias && !aligned16(bias)) ||
-        (gamma && !aligned16(gamma)) || (beta && !aligned16(beta)))
-        return fail(FLARE_EINVAL, "x, w, bias, gamma, beta, res, y must be 16-byte aligned");
+    if (in_dim < 0 || in_dim > 4 || out_dim < 0 || out_dim > 4) return fail(FLARE_EINVAL, "in_dim and out_dim must be in [0, 4] (got %d, %d)", in_dim, out_dim);
+    if ((in_dim || out_dim) && (d->flags & FLARE_MLP_EXPAND)) return fail(FLARE_EINVAL, "FLARE_MLP_EXPAND cannot be combined with in_dim / out_dim");
+    if (in_dim) {
+        if (!w_in || !b_in || !aligned16(w_in) || !aligned16(b_in)) return fail(FLARE_EINVAL, "w_in and b_in must be 16-byte aligned and not NULL when in_dim > 0");
+        if (d->norm != FLARE_NORM_NONE) return fail(FLARE_EINVAL, "no norm in front of a lifting first layer");
+        if (d->x_stride < in_dim) return fail(FLARE_EINVAL, "x_stride must be >= in_dim");
+    } else {
+        // every lane moves 4 consecutive elements at a time
+        if (d->x_stride < d->C || d->x_stride % 4 || !aligned16(x)) return fail(FLARE_EINVAL, "x: row stride >= C, a multiple of 4, base 16-byte aligned");
+    }
+    if (out_dim) {
+        if (res) return fail(FLARE_EINVAL, "res must be NULL when out_dim > 0");
+        if (d->y_stride < out_dim) return fail(FLARE_EINVAL, "y_stride must be >= out_dim");
+    } else {
+        if (d->y_stride < d->C || d->y_stride % 4 || !aligned16(y)) return fail(FLARE_EINVAL, "y: row stride >= C, a multiple of 4, base 16-byte aligned");
+    }
+    if (res && (d->res_stride < d->C || d->res_stride % 4 || !aligned16(res))) return fail(FLARE_EINVAL, "res: row stride >= C, a multiple of 4, base 16-byte aligned");
+    if (!aligned16(w) || (bias && !aligned16(bias)) || (gamma && !aligned16(gamma)) || (beta && !aligned16(beta)))
+        return fail(FLARE_EINVAL, "w, bias, gamma, beta must be 16-byte aligned");
     flare::MlpArgs a;
     memset(&a, 0, sizeof(a));
     a.x = x; a.res = res; a.y = y; a.w = static_cast<const uint16_t*>(w); a.bias = bias; a.gamma = gamma; a.beta = beta;
     a.T = d->T; a.C = d->C; a.L = d->L;
     a.x_dtype = d->x_dtype; a.res_dtype = d->res_dtype; a.y_dtype = d->y_dtype;
     a.norm = d->norm; a.eps = d->eps; a.act = d->act; a.act_mask = d->act_mask; a.add_mask = d->add_mask;
+    a.expand = (d->flags & FLARE_MLP_EXPAND) ? 1 : 0;
+    if (a.expand) {
+        if (d->L % 2) return fail(FLARE_EINVAL, "FLARE_MLP_EXPAND needs an even number of weight tiles (got L=%d)", d->L);
+        a.act_mask = (d->act_mask & 1u) ? 0x55555555u : 0u;      // the activation follows every first product
+    }
+    a.in_dim = in_dim; a.in_act = in_act ? 1 : 0; a.w_in = w_in; a.b_in = b_in; a.out_dim = out_dim;
     a.xs = d->x_stride; a.rs = d->res_stride; a.ys = d->y_stride;
     return hip_status(flare::launch_mlp_mfma(a, d->w_dtype, static_cast<hipStream_t>(stream)), "mlp launch");
+}
+
+int flare_mlp_fwd(const FlareMlpDesc* d, const void* x, const void* w, const float* bias, const float* gamma,
+                  const float* beta, const void* res, void* y, void* stream)
+{
+    return mlp_fwd_impl(d, 0, 0, nullptr, nullptr, 0, x, w, bias, gamma, beta, res, y, stream);
+}
+
+int flare_mlp_io_fwd(const FlareMlpDesc* d, int32_t in_dim, int32_t in_act, const float* w_in, const float* b_in,
+                     int32_t out_dim, const void* x, const void* w, const float* bias, const float* gamma,
+                     const float* beta, const void* res, void* y, void* stream)
+{
+    return mlp_fwd_impl(d, in_dim, in_act, w_in, b_in, out_dim, x, w, bias, gamma, beta, res, y, stream);
 }
 
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes)

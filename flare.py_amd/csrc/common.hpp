@@ -138,6 +138,12 @@ struct MlpArgs {
     float eps;
     int act;                                    // 0 tanh-GELU, 1 SiLU
     uint32_t act_mask, add_mask;                // bit l: layer l applies the activation / adds to the stream
+    int expand;                                 // 1: L = 2E tiles of the two-layer MLP with hidden width E*C (see mlp_mfma.hip)
+    int in_dim;                                 // > 0: x rows have in_dim <= 4 features and a first layer w_in lifts them to C
+    const float* w_in;                          // [C][4] fp32 rows of the lifting layer (columns >= in_dim are zero), b_in [C]
+    const float* b_in;
+    int in_act;                                 // the lifting layer is followed by the activation
+    int out_dim;                                // > 0: only features [0, out_dim <= 4) of the result are stored, y rows are out_dim wide
     int64_t xs, rs, ys;                         // row strides in elements
 };
 

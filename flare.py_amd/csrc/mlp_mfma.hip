@@ -6,6 +6,14 @@
 // running stream (ResidualMLP.forward :45-59; a single Linear is the chain of length one), and an
 // optional outer residual.  Layer l:  t = W_l s + b_l;  t = act(t) if bit l of act_mask;
 // s = s + t if bit l of add_mask else t.   Output = res + s  (res may be absent).
+// Expanding mode (a.expand): the two-layer MLP with hidden width E*C, y = W2 act(W1 n + b1) + b2, as E pairs of
+// C x C tiles: h_j = act(W1[j] n + b1[j]) from the packed input n, then s += W2[:, j] h_j, the hidden chunk h_j
+// never leaving the registers (tiles come as L = 2E "layers": W1[0], W2[:,0], W1[1], W2[:,1], ...).
+// Lifting mode (a.in_dim > 0): the rows of x have only in_dim <= 4 features (coordinates and a field value, say)
+// and a first layer C x in_dim, evaluated with in_dim multiply-adds per output on the vector ALU, produces the
+// stream that the C x C chain continues from (ResidualMLP(in_dim, C, C, ...), the models' input projection).
+// Projecting mode (a.out_dim > 0): the last tile has only out_dim <= 4 real rows (the rest are zero) and only those
+// outputs are stored, y rows being out_dim wide (ResidualMLP(C, C, out_dim, ...), the models' output projection).
 //
 // Layout.  The product is taken transposed, S'^T = W S^T, with v_mfma_f32_16x16x32: A = W tile
 // (lane = output row, 8 consecutive input features per lane), B = S^T (lane = token c16, k-slots =
@@ -105,7 +113,8 @@ __device__ __forceinline__ float silu_gate(float x)
     return __builtin_amdgcn_rcpf(1.f + fast_exp2(-kLog2e * x));
 }
 
-template <typename T, int C, int TW, int WAVES>
+// MODE: 0 the C x C chain, 1 the expanding two-layer MLP, 2 the chain with a narrow first input and/or last output
+template <typename T, int C, int TW, int WAVES, int MODE>
 __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kernel(MlpArgs a, int resident)
 {
     constexpr int NT = 64 * WAVES;
@@ -178,10 +187,44 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
 
         // the stream: lane (c16, g) holds features 16 ft + 4 g + r of token c16 of each tile
         f32x4 xs[FT][TW];
+        if (MODE == 2 && a.in_dim > 0) {
+            // lifting layer: s[f] = act(b_in[f] + sum_i w_in[f][i] x[i]) from the token's few input features
+            float xin[TW][4];
 #pragma unroll
-        for (int tw = 0; tw < TW; ++tw)
+            for (int tw = 0; tw < TW; ++tw)
 #pragma unroll
-            for (int ft = 0; ft < FT; ++ft) xs[ft][tw] = load4(a.x, tok[tw] * a.xs + 16 * ft + 4 * g, a.x_dtype);
+                for (int i = 0; i < 4; ++i) {
+                    float v = 0.f;
+                    if (i < a.in_dim) {
+                        const int64_t e = tok[tw] * a.xs + i;
+                        v = a.x_dtype == 0 ? static_cast<const float*>(a.x)[e]
+                          : a.x_dtype == 1 ? __uint_as_float(uint32_t(static_cast<const uint16_t*>(a.x)[e]) << 16)
+                                           : (float)static_cast<const _Float16*>(a.x)[e];
+                    }
+                    xin[tw][i] = v;
+                }
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                const f32x4 b4 = *reinterpret_cast<const f32x4*>(a.b_in + 16 * ft + 4 * g);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const f32x4 wr = *reinterpret_cast<const f32x4*>(a.w_in + (16 * ft + 4 * g + r) * 4);
+#pragma unroll
+                    for (int tw = 0; tw < TW; ++tw) {
+                        float t = b4[r];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) t = fmaf(wr[i], xin[tw][i], t);
+                        if (a.in_act) t *= a.act == 0 ? gelu_gate(t) : silu_gate(t);
+                        xs[ft][tw][r] = t;
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft) xs[ft][tw] = load4(a.x, tok[tw] * a.xs + 16 * ft + 4 * g, a.x_dtype);
+        }
 
         if (a.norm != 0) {
 #pragma unroll
@@ -213,6 +256,85 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
             }
         }
 
+        if constexpr (MODE == 1) {
+            // n = the (normalised) input, packed once; the stream restarts at zero and collects the second products
+            u32x4 xb0[KS][TW], hb[KS][TW];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int tw = 0; tw < TW; ++tw) {
+                    const f32x4 lo = xs[2 * ks][tw], hi = xs[2 * ks + 1][tw];
+                    xb0[ks][tw] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]),
+                                        M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
+                    hb[ks][tw] = xb0[ks][tw];
+                }
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+                for (int tw = 0; tw < TW; ++tw) xs[ft][tw] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int l = 0; l < a.L; ++l, ++lcount) {
+                const int slot = resident ? l : (lcount & 1);
+                if (!resident) fetch(l + 1 < a.L ? l + 1 : 0);
+                const uint8_t* wb = smem + slot * WBUF + c16 * RS;
+                const float* bl = a.bias ? a.bias + (size_t)l * C + 4 * g : nullptr;
+                if (!(l & 1)) {
+                    // h = act(W1[j] n + b1[j]): tile ft of h is half (ft & 1) of k-step ft / 2 of the next product
+                    auto first = [&](auto act_c) {
+                        constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+                        for (int ft = 0; ft < FT; ++ft) {
+                            const f32x4 bias = bl ? *reinterpret_cast<const f32x4*>(bl + 16 * ft) : f32x4{0.f, 0.f, 0.f, 0.f};
+                            f32x4 acc[TW];
+#pragma unroll
+                            for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
+#pragma unroll
+                            for (int ks = 0; ks < KS; ++ks) {
+                                const u32x4 wa = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]);
+#pragma unroll
+                                for (int tw = 0; tw < TW; ++tw) acc[tw] = M_::mma(wa, xb0[ks][tw], acc[tw]);
+                            }
+#pragma unroll
+                            for (int tw = 0; tw < TW; ++tw) {
+                                float t[4];
+#pragma unroll
+                                for (int r = 0; r < 4; ++r)
+                                    t[r] = ACT == 0 ? acc[tw][r] : acc[tw][r] * (ACT == 1 ? gelu_gate(acc[tw][r]) : silu_gate(acc[tw][r]));
+                                hb[ft >> 1][tw][2 * (ft & 1)] = M_::pack2(t[0], t[1]);
+                                hb[ft >> 1][tw][2 * (ft & 1) + 1] = M_::pack2(t[2], t[3]);
+                            }
+                        }
+                    };
+                    if (!((a.act_mask >> l) & 1u)) first(std::integral_constant<int, 0>{});
+                    else if (a.act == 0) first(std::integral_constant<int, 1>{});
+                    else first(std::integral_constant<int, 2>{});
+                } else {
+                    // s += W2[:, j] h (+ the bias row of this tile: b2 on the first pair, zeros after it)
+#pragma unroll
+                    for (int ft = 0; ft < FT; ++ft) {
+                        f32x4 acc[TW];
+#pragma unroll
+                        for (int tw = 0; tw < TW; ++tw) acc[tw] = xs[ft][tw];
+                        if (bl && l == 1) {
+                            const f32x4 bias = *reinterpret_cast<const f32x4*>(bl + 16 * ft);
+#pragma unroll
+                            for (int tw = 0; tw < TW; ++tw) acc[tw] += bias;
+                        }
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks) {
+                            const u32x4 wa = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]);
+#pragma unroll
+                            for (int tw = 0; tw < TW; ++tw) acc[tw] = M_::mma(wa, hb[ks][tw], acc[tw]);
+                        }
+#pragma unroll
+                        for (int tw = 0; tw < TW; ++tw) xs[ft][tw] = acc[tw];
+                    }
+                }
+                if (!resident) {
+                    put(slot ^ 1);
+                    __syncthreads();
+                }
+            }
+        } else
         for (int l = 0; l < a.L; ++l, ++lcount) {
             const int slot = resident ? l : (lcount & 1);
             // ring: fetch the weights of the layer after this one (layer 0 of the next pass after the last)
@@ -285,6 +407,18 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
 #pragma unroll
         for (int tw = 0; tw < TW; ++tw) {
             if (!live[tw]) continue;
+            if (MODE == 2 && a.out_dim > 0) {
+                // projecting last layer: only its first out_dim <= 4 rows are real, lane g == 0 holds them
+                if (g == 0)
+                    for (int r = 0; r < a.out_dim; ++r) {
+                        const int64_t e = tok[tw] * a.ys + r;
+                        const float o = xs[0][tw][r];
+                        if (a.y_dtype == 0) static_cast<float*>(a.y)[e] = o;
+                        else if (a.y_dtype == 1) static_cast<uint16_t*>(a.y)[e] = (uint16_t)Mm<bf16_t>::pack2(o, 0.f);
+                        else static_cast<_Float16*>(a.y)[e] = (_Float16)o;
+                    }
+                continue;
+            }
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
                 f32x4 o = xs[ft][tw];
@@ -297,10 +431,10 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
 
 constexpr size_t kMlpLdsMax = 160 * 1024;   // all of a CU's LDS: five layers of 128 channels stay resident
 
-template <typename T, int C, int TW, int WAVES>
-hipError_t launch_ct(const MlpArgs& a, hipStream_t st)
+template <typename T, int C, int TW, int WAVES, int MODE>
+hipError_t launch_cte(const MlpArgs& a, hipStream_t st)
 {
-    auto kern = mlp_mfma_kernel<T, C, TW, WAVES>;
+    auto kern = mlp_mfma_kernel<T, C, TW, WAVES, MODE>;
     const size_t wbuf = (size_t)C * C * 2;
     int resident = (size_t)a.L * wbuf <= kMlpLdsMax ? 1 : 0;
     size_t lds = (resident ? (size_t)a.L : 2) * wbuf;
@@ -318,6 +452,14 @@ hipError_t launch_ct(const MlpArgs& a, hipStream_t st)
     const unsigned grid = (unsigned)(nblk < slots ? nblk : slots);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES), lds, st, a, resident);
     return hipGetLastError();
+}
+
+template <typename T, int C, int TW, int WAVES>
+hipError_t launch_ct(const MlpArgs& a, hipStream_t st)
+{
+    if (a.expand) return launch_cte<T, C, TW, WAVES, 1>(a, st);
+    if (a.in_dim > 0 || a.out_dim > 0) return launch_cte<T, C, TW, WAVES, 2>(a, st);
+    return launch_cte<T, C, TW, WAVES, 0>(a, st);
 }
 
 template <typename T>

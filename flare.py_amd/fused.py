@@ -6,6 +6,12 @@ between layers, what the reference runs as separate torch layers:
     res + ResidualMLP(norm(x))         pdebench/models/flare.py:45-59 and 204-215
     res + Linear(x)                    (out_proj, flare.py:156)
 
+    ResidualMLP(in_dim <= 4, C, C)     (the models' in_proj, flare.py:137-140: the narrow first layer runs on
+    ResidualMLP(C, C, out_dim <= 4)     the vector ALU; of out_proj's last layer only the real rows are stored)
+
+A ResidualMLP with num_layers == 0 and a hidden width of E*C (2 <= E <= 8; the "4x expansion" feed-forward
+block) runs in the same launch as E pairs of C x C tiles, the hidden activations never leaving the registers.
+
 It is used by the modules only when no gradient is needed and the products may run in bf16/f16
 (torch.autocast is on, or the weights already are bf16/f16) — the conditions under which torch
 itself would run these Linear layers in that type.  Everything else stays with the torch layers.
@@ -46,6 +52,33 @@ def _layers_of(mod):
     return layers, act_mask, add_mask, act
 
 
+def _expand_factor(mod, Cdim):
+    """E when mod is the two-layer MLP C -> E*C -> C (ResidualMLP with num_layers == 0 and no residual that
+    applies), else 0."""
+    if getattr(mod, "num_layers", None) != 0 or mod.input_residual or mod.output_residual:
+        return 0
+    f1, f2 = mod.fc1, mod.fc2
+    hid = f1.out_features
+    if f1.in_features != Cdim or f2.out_features != Cdim or f2.in_features != hid or hid % Cdim or hid == Cdim:
+        return 0
+    E = hid // Cdim
+    return E if 2 <= E <= 8 else 0
+
+
+def _io_dims(mod, layers):
+    """(C, in_dim, out_dim) of a stack that is C x C except for a narrow (<= 4) first input and/or last output
+    (0 = that end is C wide), or None."""
+    if len(layers) < 2:
+        return None
+    Cdim = layers[0].out_features
+    if any(l.in_features != Cdim or l.out_features != Cdim for l in layers[1:-1]) or layers[-1].in_features != Cdim:
+        return None
+    i, o = layers[0].in_features, layers[-1].out_features
+    if not ((i == Cdim or i <= 4) and (o == Cdim or o <= 4)):
+        return None
+    return Cdim, (0 if i == Cdim else i), (0 if o == Cdim else o)
+
+
 def compute_dtype(x, mod):
     """The 16-bit type the fused kernel may run this module in, or None (then torch runs it)."""
     if torch.is_grad_enabled() or x.device.type != "cuda":
@@ -54,11 +87,18 @@ def compute_dtype(x, mod):
     if info is None:
         return None
     layers = info[0]
-    Cdim = x.shape[-1]
-    if Cdim not in _SUPPORTED_C or len(layers) > 16:
+    if len(layers) > 16:
         return None
-    if any(l.in_features != Cdim or l.out_features != Cdim for l in layers):
-        return None
+    io = _io_dims(mod, layers)
+    if io is not None and (io[1] or io[2]):
+        if io[0] not in _SUPPORTED_C or x.shape[-1] != layers[0].in_features:
+            return None
+    else:
+        Cdim = x.shape[-1]
+        if Cdim not in _SUPPORTED_C:
+            return None
+        if not _expand_factor(mod, Cdim) and any(l.in_features != Cdim or l.out_features != Cdim for l in layers):
+            return None
     if x.dtype not in (torch.float32, torch.bfloat16, torch.float16) or x.stride(-1) != 1:
         return None
     ac = _autocast_dtype(x)
@@ -83,23 +123,84 @@ def _packed(mod, layers, cd):
     return w, b
 
 
-def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None):
-    """y = res + mod(norm(x)) in one HIP launch.  x: [..., C]; mod: ResidualMLP or nn.Linear; cd: the
-    dtype from compute_dtype(); norm: nn.LayerNorm / nn.RMSNorm / None; res: [..., C] or None."""
+def _packed_expand(mod, E, cd):
+    """Tiles W1[0:C], W2[:,0:C], W1[C:2C], W2[:,C:2C], ... as [2E,C,C] and bias rows b1[0:C], b2, b1[C:2C], 0, ...
+    (the layout FLARE_MLP_EXPAND asks for), cached on the module."""
+    f1, f2 = mod.fc1, mod.fc2
+    key = ("expand", cd, tuple((l.weight.data_ptr(), l.weight._version, None if l.bias is None else l.bias._version)
+                               for l in (f1, f2)))
+    cache = getattr(mod, "_flare_packed", None)
+    if cache is not None and cache[0] == key:
+        return cache[1], cache[2]
+    Cdim = f1.in_features
+    w1 = f1.weight.detach().to(cd).view(E, Cdim, Cdim)                       # [j][hidden row in chunk][in]
+    w2 = f2.weight.detach().to(cd).view(Cdim, E, Cdim).permute(1, 0, 2)      # [j][out][hidden col in chunk]
+    w = torch.stack([w1, w2], dim=1).reshape(2 * E, Cdim, Cdim).contiguous()
+    b = torch.zeros(2 * E, Cdim, dtype=torch.float32, device=w.device)
+    if f1.bias is not None:
+        b[0::2] = f1.bias.detach().float().view(E, Cdim)
+    if f2.bias is not None:
+        b[1] = f2.bias.detach().float()
+    mod._flare_packed = (key, w, b)
+    return w, b
+
+
+def _packed_io(mod, layers, cd, Cdim, in_dim, out_dim):
+    """Tiles of a stack with a narrow first and/or last layer: (w [L,C,C], b [L,C], w_in [C,4] fp32, b_in [C]),
+    the narrow last layer zero-padded to C rows; cached on the module."""
+    key = ("io", cd, tuple((l.weight.data_ptr(), l.weight._version, None if l.bias is None else l.bias._version) for l in layers))
+    cache = getattr(mod, "_flare_packed", None)
+    if cache is not None and cache[0] == key:
+        return cache[1:]
+    dev = layers[0].weight.device
+    tiles = layers[1:] if in_dim else layers
+    w = torch.zeros(len(tiles), Cdim, Cdim, dtype=cd, device=dev)
+    b = torch.zeros(len(tiles), Cdim, dtype=torch.float32, device=dev)
+    for i, l in enumerate(tiles):
+        w[i, :l.out_features] = l.weight.detach().to(cd)
+        if l.bias is not None:
+            b[i, :l.out_features] = l.bias.detach().float()
+    w_in = b_in = None
+    if in_dim:
+        w_in = torch.zeros(Cdim, 4, dtype=torch.float32, device=dev)
+        w_in[:, :in_dim] = layers[0].weight.detach().float()
+        b_in = (layers[0].bias.detach().float().contiguous() if layers[0].bias is not None
+                else torch.zeros(Cdim, dtype=torch.float32, device=dev))
+    mod._flare_packed = (key, w, b, w_in, b_in)
+    return w, b, w_in, b_in
+
+
+def _fused_mlp_io(x, mod, cd, io, info, norm, out_dtype):
     lib = _lib.load()
-    layers, act_mask, add_mask, act = _layers_of(mod)
-    Cdim = x.shape[-1]
-    w, b = _packed(mod, layers, cd)
-    x2 = x.reshape(-1, Cdim)
-    if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 16:
+    layers, act_mask, add_mask, act = info
+    Cdim, in_dim, out_dim = io
+    w, b, w_in, b_in = _packed_io(mod, layers, cd, Cdim, in_dim, out_dim)
+    in_act = act_mask & 1
+    if in_dim:                       # the first layer is not one of the tiles
+        act_mask >>= 1
+        add_mask >>= 1
+    xw = x.shape[-1]
+    x2 = x.reshape(-1, xw)
+    if x2.stride(-1) != 1 or (not in_dim and (x2.stride(0) % 4 or x2.data_ptr() % 16)):
         x2 = x2.contiguous()
     out_dtype = x.dtype if out_dtype is None else out_dtype
-    y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    yw = out_dim if out_dim else Cdim
+    y = torch.empty(*x.shape[:-1], yw, dtype=out_dtype, device=x.device)
     d = _lib.FlareMlpDesc()
-    d.T, d.C, d.L = x2.shape[0], Cdim, len(layers)
+    d.T, d.C, d.L = x2.shape[0], Cdim, w.shape[0]
     d.w_dtype, d.x_dtype, d.y_dtype = _dtype_code(w), _dtype_code(x2), _dtype_code(y)
     d.act, d.act_mask, d.add_mask = act, act_mask, add_mask
-    d.x_stride, d.y_stride = x2.stride(0), Cdim
+    d.x_stride, d.y_stride = x2.stride(0), yw
+    gamma, beta = _norm_args(d, norm, x, Cdim)
+    with torch.cuda.device(x.device):
+        rc = lib.flare_mlp_io_fwd(C.byref(d), in_dim, in_act, _ptr(w_in), _ptr(b_in), out_dim, _ptr(x2), _ptr(w), _ptr(b),
+                                  _ptr(gamma), _ptr(beta), None, _ptr(y), C.c_void_p(_stream_ptr(x.device)))
+    _lib.check(rc, "flare_mlp_io_fwd")
+    return y
+
+
+def _norm_args(d, norm, x, Cdim):
+    """Fill the descriptor's norm fields; returns (gamma, beta) fp32 tensors or None."""
     gamma = beta = None
     if norm is not None and not isinstance(norm, nn.Identity):
         if isinstance(norm, nn.LayerNorm):
@@ -112,6 +213,38 @@ def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None):
             raise TypeError(f"unsupported norm {type(norm).__name__}")
         gamma = (norm.weight.detach().float().contiguous() if getattr(norm, "weight", None) is not None
                  else torch.ones(Cdim, dtype=torch.float32, device=x.device))
+    return gamma, beta
+
+
+def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None):
+    """y = res + mod(norm(x)) in one HIP launch.  x: [..., C]; mod: ResidualMLP or nn.Linear; cd: the
+    dtype from compute_dtype(); norm: nn.LayerNorm / nn.RMSNorm / None; res: [..., C] or None."""
+    lib = _lib.load()
+    info = _layers_of(mod)
+    layers, act_mask, add_mask, act = info
+    io = _io_dims(mod, layers)
+    if io is not None and (io[1] or io[2]):
+        y = _fused_mlp_io(x, mod, cd, io, info, norm, out_dtype)
+        return y if res is None else res + y
+    Cdim = x.shape[-1]
+    E = _expand_factor(mod, Cdim)
+    if E:
+        w, b = _packed_expand(mod, E, cd)
+        act_mask, add_mask = 1, 0
+    else:
+        w, b = _packed(mod, layers, cd)
+    x2 = x.reshape(-1, Cdim)
+    if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    out_dtype = x.dtype if out_dtype is None else out_dtype
+    y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    d = _lib.FlareMlpDesc()
+    d.T, d.C, d.L = x2.shape[0], Cdim, w.shape[0]
+    d.flags = _lib.MLP_EXPAND if E else 0
+    d.w_dtype, d.x_dtype, d.y_dtype = _dtype_code(w), _dtype_code(x2), _dtype_code(y)
+    d.act, d.act_mask, d.add_mask = act, act_mask, add_mask
+    d.x_stride, d.y_stride = x2.stride(0), Cdim
+    gamma, beta = _norm_args(d, norm, x, Cdim)
     r2 = None
     if res is not None:
         r2 = res.reshape(-1, Cdim)

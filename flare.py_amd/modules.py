@@ -186,6 +186,9 @@ class FinalLayer(nn.Module):
                                input_residual=True, output_residual=False)
 
     def forward(self, x):
+        cd = fused.compute_dtype(x, self.mlp)
+        if cd is not None:
+            return fused.fused_mlp(x, self.mlp, cd, norm=self.ln)
         return self.mlp(self.ln(x))
 
 
@@ -232,10 +235,12 @@ class FLAREModel(nn.Module):
 
     def forward(self, x, return_scores: bool = False):
         scores = []
-        x = self.in_proj(x)
+        cd = fused.compute_dtype(x, self.in_proj)
+        x = fused.fused_mlp(x, self.in_proj, cd) if cd is not None else self.in_proj(x)
         for block in self.blocks:
             x, s = block(x, return_scores=return_scores)
             if return_scores:
                 scores.append(s)
-        x = self.out_proj(x)
+        cd = fused.compute_dtype(x, self.out_proj[1])
+        x = fused.fused_mlp(x, self.out_proj[1], cd, norm=self.out_proj[0]) if cd is not None else self.out_proj(x)
         return (x, scores) if return_scores else x

@@ -140,7 +140,13 @@ typedef struct FlareCausalLinearDesc {
  * fp32.  ResidualMLP(C, C, C, n layers, input_residual, output_residual) is L = n + 2 with
  * act_mask = all but the last layer, add_mask = all layers (minus the first / last when the
  * matching flag is off).  C must be 32, 64 or 128.
+ * With FLARE_MLP_EXPAND in flags the launch evaluates the two-layer MLP with hidden width E*C,
+ * y = res + W2 act(W1 norm(x) + b1) + b2 (ResidualMLP(C, E*C, C, num_layers = 0), the "4x expansion"
+ * feed-forward block), from L = 2E tiles of C x C weights in the order W1[0:C,:], W2[:,0:C],
+ * W1[C:2C,:], W2[:,C:2C], ... and bias rows b1[0:C], b2, b1[C:2C], 0, ...; act_mask bit 0 says
+ * whether the activation is applied, add_mask is ignored.
  */
+#define FLARE_MLP_EXPAND 1
 #define FLARE_NORM_NONE  0
 #define FLARE_NORM_LAYER 1   /* (x - mean) * rsqrt(var + eps) * gamma + beta */
 #define FLARE_NORM_RMS   2   /* x * rsqrt(mean(x^2) + eps) * gamma           */
@@ -227,6 +233,19 @@ int flare_causal_linear_fwd(const FlareCausalLinearDesc* desc, const void* q, co
  * row at equal strides (every row is read completely before it is written). */
 int flare_mlp_fwd(const FlareMlpDesc* desc, const void* x, const void* w, const float* bias,
                   const float* gamma, const float* beta, const void* res, void* y, void* stream);
+
+/* The same stack between a narrow input and/or a narrow output (the models' in_proj and out_proj,
+ * pdebench/models/flare.py:137-160: ResidualMLP(in_dim, C, C, ...) and ResidualMLP(C, C, out_dim, ...)).
+ * in_dim > 0: x rows hold in_dim <= 4 features (x_stride >= in_dim, any alignment of the element
+ *   type) and a first layer t = w_in x + b_in (w_in fp32 [C][4], columns >= in_dim zero; b_in fp32
+ *   [C]; followed by the activation when in_act != 0) produces the stream the L tiles continue
+ *   from; norm must be FLARE_NORM_NONE.  in_dim == 0: x rows are C wide as in flare_mlp_fwd.
+ * out_dim > 0: only outputs [0, out_dim <= 4) of the last tile are stored (its other rows should be
+ *   zero), y rows are out_dim wide (y_stride >= out_dim) and res must be NULL.  out_dim == 0: C wide.
+ * FLARE_MLP_EXPAND is not accepted here. */
+int flare_mlp_io_fwd(const FlareMlpDesc* desc, int32_t in_dim, int32_t in_act, const float* w_in,
+                     const float* b_in, int32_t out_dim, const void* x, const void* w, const float* bias,
+                     const float* gamma, const float* beta, const void* res, void* y, void* stream);
 
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes);
 

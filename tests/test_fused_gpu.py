@@ -143,3 +143,133 @@ def test_model_fused_path_vs_fp32(dev):
         with torch.autocast("cuda", dtype=torch.bfloat16):
             y = model(x)
     assert O.rel_l2(y, ref) <= 3e-2
+
+
+@pytest.mark.parametrize("C,E", [(32, 2), (64, 4), (128, 4), (128, 2)])
+@pytest.mark.parametrize("act,cd", [("gelu", torch.bfloat16), ("silu", torch.float16)])
+def test_expanding_two_layer_mlp(dev, C, E, act, cd):
+    """The feed-forward block with a hidden width of E*C (ResidualMLP(C, E*C, C, num_layers=0)): one launch, E pairs of
+    C x C tiles, against the oracle on the same rounded weights; with norm and outer residual, ragged row counts."""
+    torch.manual_seed(4)
+    m = F.ResidualMLP(C, E * C, C, num_layers=0, act=act, input_residual=True, output_residual=True)
+    for l in (m.fc1, m.fc2):
+        nn.init.normal_(l.weight, 0.0, l.in_features ** -0.5)
+        nn.init.normal_(l.bias, 0.0, 0.2)
+    m = m.to(dev)
+    assert not m.input_residual and not m.output_residual
+    norm = nn.LayerNorm(C).to(dev)
+    nn.init.normal_(norm.weight, 1.0, 0.3)
+    nn.init.normal_(norm.bias, 0.0, 0.3)
+    for T in (5, 300, 2049):
+        x = torch.randn(T, C, device=dev) * 1.5
+        with torch.no_grad(), torch.autocast("cuda", dtype=cd):
+            assert fused.compute_dtype(x, m) == cd
+            y = fused.fused_mlp(x, m, cd, norm=norm, res=x)
+            y0 = fused.fused_mlp(x, m, cd)
+        assert O.rel_l2(y, oracle_of(m, x, cd, norm, x)) <= 2e-2, T
+        assert O.rel_l2(y0, oracle_of(m, x, cd)) <= 2e-2, T
+
+
+def test_block_with_4x_feed_forward(dev):
+    """BASELINE config 2's block shape (pre-norm, H=8 heads of D=16, M=128 latents, feed-forward with 4x expansion) at
+    reduced length: the fused path against the block's own torch layers in fp32."""
+    torch.manual_seed(5)
+    blk = F.FLAREBlock(channel_dim=128, num_heads=8, num_latents=128, ffn_mlp_ratio=4.0, num_layers_ffn=0).to(dev).eval()
+    for mod in blk.modules():
+        if isinstance(mod, nn.Linear):
+            nn.init.xavier_uniform_(mod.weight)
+    x = torch.randn(2, 3000, 128, device=dev)
+    with torch.no_grad():
+        ref = blk(x)[0]
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            assert fused.compute_dtype(x, blk.mlp) == torch.bfloat16
+            y = blk(x)[0]
+    assert O.rel_l2(y, ref) <= 2e-2
+
+
+def _narrow_mlp(i, h, o, n, ir, orr, act, dev, seed):
+    torch.manual_seed(seed)
+    m = F.ResidualMLP(i, h, o, num_layers=n, act=act, input_residual=ir, output_residual=orr)
+    for l in m.modules():
+        if isinstance(l, nn.Linear):
+            nn.init.normal_(l.weight, 0.0, l.in_features ** -0.5)
+            nn.init.normal_(l.bias, 0.0, 0.2)
+    return m.to(dev)
+
+
+def _narrow_oracle(m, x, cd, norm=None):
+    """fp64 oracle on the weights as the kernel holds them: the narrow first layer in fp32, the tiles in cd."""
+    layers, _, _, act = fused._layers_of(m)
+    C = layers[0].out_features
+    ws = [(l.weight.detach() if l.in_features <= 4 and C > 4 else l.weight.detach().to(cd)).double().cpu() for l in layers]
+    bs = [l.bias.detach().double().cpu() for l in layers]
+    kind = gamma = beta = None
+    eps = 1e-5
+    if isinstance(norm, nn.LayerNorm):
+        kind, gamma, beta, eps = "layer", norm.weight.detach().cpu(), norm.bias.detach().cpu(), norm.eps
+    return O.residual_mlp(x.double().cpu(), ws, bs, "gelu" if act == 0 else "silu", m.input_residual, m.output_residual,
+                          kind, gamma, beta, eps)
+
+
+@pytest.mark.parametrize("C", [32, 64, 128])
+@pytest.mark.parametrize("in_dim,n,act,xdt", [(3, 2, "gelu", torch.float32), (1, 0, "silu", torch.float32),
+                                              (4, 3, "gelu", torch.bfloat16), (2, 1, "silu", torch.float16)])
+def test_lifting_first_layer_vs_oracle(dev, C, in_dim, n, act, xdt):
+    """ResidualMLP(in_dim <= 4, C, C): the model's in_proj (pdebench/models/flare.py:137-140) in one launch."""
+    m = _narrow_mlp(in_dim, C, C, n, False, True, act, dev, seed=C + in_dim)
+    x = torch.randn(2, 777, in_dim, device=dev).to(xdt)
+    cdt = torch.float16 if xdt == torch.float16 else torch.bfloat16
+    with torch.no_grad(), torch.autocast("cuda", dtype=cdt):
+        cd = fused.compute_dtype(x, m)
+        assert cd == cdt
+        y = fused.fused_mlp(x, m, cd, out_dtype=torch.float32)
+    assert y.shape == (2, 777, C) and y.dtype == torch.float32
+    assert O.rel_l2(y, _narrow_oracle(m, x, cd)) <= 2e-2
+
+
+@pytest.mark.parametrize("C", [32, 64, 128])
+@pytest.mark.parametrize("out_dim,n,ln,odt", [(1, 2, True, torch.float32), (4, 0, False, torch.bfloat16), (3, 1, True, torch.float16)])
+def test_projecting_last_layer_vs_oracle(dev, C, out_dim, n, ln, odt):
+    """norm + ResidualMLP(C, C, out_dim <= 4): the model's out_proj (pdebench/models/flare.py:141-147)."""
+    m = _narrow_mlp(C, C, out_dim, n, True, False, "gelu", dev, seed=C + out_dim)
+    norm = nn.LayerNorm(C).to(dev) if ln else None
+    if ln:
+        nn.init.normal_(norm.weight, 1.0, 0.2)
+        nn.init.normal_(norm.bias, 0.0, 0.2)
+    x = torch.randn(3, 501, C, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        cd = fused.compute_dtype(x, m)
+        assert cd == torch.bfloat16
+        y = fused.fused_mlp(x, m, cd, norm=norm, out_dtype=odt)
+    assert y.shape == (3, 501, out_dim) and y.dtype == odt
+    assert O.rel_l2(y, _narrow_oracle(m, x, cd, norm)) <= 2e-2
+
+
+def test_narrow_both_ends_and_torch_fallbacks(dev):
+    """in_dim and out_dim narrow at once; widths the kernel does not take stay with the torch layers."""
+    m = _narrow_mlp(2, 64, 3, 2, False, False, "gelu", dev, seed=9)
+    x = torch.randn(1000, 2, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        cd = fused.compute_dtype(x, m)
+        assert cd == torch.bfloat16
+        y = fused.fused_mlp(x, m, cd)
+        assert fused.compute_dtype(torch.randn(10, 5, device=dev), _narrow_mlp(5, 64, 64, 1, False, True, "gelu", dev, 1)) is None
+        assert fused.compute_dtype(torch.randn(10, 3, device=dev), _narrow_mlp(3, 48, 48, 1, False, True, "gelu", dev, 1)) is None
+        assert fused.compute_dtype(torch.randn(10, 64, device=dev), _narrow_mlp(64, 64, 8, 1, True, False, "gelu", dev, 1)) is None
+    assert y.shape == (1000, 3)
+    assert O.rel_l2(y, _narrow_oracle(m, x, cd)) <= 2e-2
+
+
+def test_model_launch_count_with_fused_ends(dev):
+    """The whole model forward under autocast is in_proj + per block (k, v, mixer x3, out, ffn) + out_proj launches:
+    no torch Linear runs (each would show as an addmm / mm kernel in the profiler)."""
+    torch.manual_seed(5)
+    model = F.FLAREModel(in_dim=3, out_dim=1, channel_dim=64, num_blocks=2, num_heads=4, num_latents=64).to(dev).eval()
+    x = torch.randn(2, 1500, 3, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        model(x)
+        with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CPU]) as prof:
+            y = model(x)
+    names = {e.name for e in prof.events()}
+    assert not any(n in names for n in ("aten::linear", "aten::addmm", "aten::mm", "aten::layer_norm")), names
+    assert y.shape == (2, 1500, 1)
