@@ -138,6 +138,21 @@ def test_new_struct_sizes_and_entry_point_validation():
     assert lib.flare_mlp_fwd(m, None, None, None, None, None, None, None, None) == _lib.FLARE_EINVAL
     m.L, m.w_dtype = 2, _lib.DT_F32
     assert lib.flare_mlp_fwd(m, None, None, None, None, None, None, None, None) == _lib.FLARE_EINVAL
+    # narrow first / last layers: widths above 4, a norm in front of a lifting layer, expand mode and a
+    # residual next to a narrow output are refused (fake non-NULL pointers: nothing is dereferenced before the checks)
+    m.w_dtype = _lib.DT_BF16
+    fake = C.c_void_p(4096)
+    io = lambda i, o, res=None: lib.flare_mlp_io_fwd(m, i, 1, fake, fake, o, fake, fake, None, fake, None, res, fake, None)
+    assert io(5, 0) == _lib.FLARE_EINVAL and "in_dim and out_dim" in _lib.last_error()
+    assert io(0, 7) == _lib.FLARE_EINVAL
+    m.norm = 1
+    assert io(3, 0) == _lib.FLARE_EINVAL and "norm" in _lib.last_error()
+    m.norm, m.flags = 0, _lib.MLP_EXPAND
+    assert io(3, 0) == _lib.FLARE_EINVAL and "EXPAND" in _lib.last_error()
+    m.flags = 0
+    assert io(0, 2, fake) == _lib.FLARE_EINVAL and "res must be NULL" in _lib.last_error()
+    m.x_stride = 2
+    assert io(3, 0) == _lib.FLARE_EINVAL and "x_stride" in _lib.last_error()
     # causal linear attention
     c = _lib.FlareCausalLinearDesc()
     c.B, c.H, c.N, c.Dk, c.Dv, c.dtype = 1, 2, 100, 32, 16, _lib.DT_F32
