@@ -252,3 +252,32 @@ def test_decode_kernel_shapes(dev, M, D, dtype):
     y2, st = F.flare_causal_decode(q.to(dev), k[:, :, 37:].to(dev), v[:, :, 37:].to(dev), st)
     assert O.rel_l2(torch.cat([y1, y2], 2), yr) <= TOL[dtype]
     state_close(st, str_, TOL[dtype])
+
+
+def test_cfg4_full_size_properties(dev):
+    """BASELINE config 4 at its full size (B=8, H=16, D=64, M=128, bf16; 8192 prefill tokens in chunks of 256, then 256
+    decode steps), through properties that need no full-size CPU run: decode after prefill = one longer prefill;
+    the final state = the non-causal gather over all tokens; the last output row = the non-causal mixer's;
+    and one (b, h) pair against the fp64 token recurrence over the whole length."""
+    B, H, D, M, NP, ND = 8, 16, 64, 128, 8192, 256
+    q, k, v = make(B, H, NP + ND, M, D, torch.bfloat16, seed=4)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    y1, st = F.flare_causal_prefill(qd, kd[:, :, :NP], vd[:, :, :NP], chunk=256)
+    y2, st = F.flare_causal_decode(qd, kd[:, :, NP:], vd[:, :, NP:], st)
+    yl, stl = F.flare_causal_prefill(qd, kd, vd, chunk=256)
+    assert torch.isfinite(y1).all() and torch.isfinite(y2).all()
+    assert O.rel_l2(y1, yl[:, :, :NP]) <= 1e-6                    # same kernel, same chunks
+    assert O.rel_l2(y2, yl[:, :, NP:]) <= 2e-2
+    z, lse = O.causal_state_invariants(*(t.double() for t in st))
+    zl, lsel = O.causal_state_invariants(*(t.double() for t in stl))
+    assert O.rel_l2(z, zl) <= 2e-2 and float((lse - lsel).abs().max()) <= 0.2
+    zg, lseg = F.flare_gather(qd, kd, vd)
+    assert O.rel_l2(z, zg.double()) <= 2e-2 and float((lse - lseg.double()).abs().max()) <= 0.2
+    yn = F.flare_multihead_mixer(qd, kd, vd)
+    assert O.rel_l2(y2[:, :, -1], yn[:, :, -1]) <= 2e-2
+    b, h = 5, 11
+    yr, str_ = O.causal_recurrent(q[h:h + 1].float(), k[b:b + 1, h:h + 1].float(), v[b:b + 1, h:h + 1].float(), dtype=torch.float64)
+    assert O.rel_l2(y1[b, h], yr[0, 0, :NP]) <= 2e-2
+    assert O.rel_l2(y2[b, h], yr[0, 0, NP:]) <= 2e-2
+    zr, lser = O.causal_state_invariants(*str_)
+    assert O.rel_l2(z[b, h].cpu(), zr[0, 0]) <= 2e-2 and float((lse[b, h].cpu() - lser[0, 0]).abs().max()) <= 0.2

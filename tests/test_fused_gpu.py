@@ -273,3 +273,28 @@ def test_model_launch_count_with_fused_ends(dev):
     names = {e.name for e in prof.events()}
     assert not any(n in names for n in ("aten::linear", "aten::addmm", "aten::mm", "aten::layer_norm")), names
     assert y.shape == (2, 1500, 1)
+
+
+def test_cfg2_full_size_fused_vs_fp32_layers(dev):
+    """BASELINE config 2 at its full size (B=4 clouds of 65,536 points, 2 coordinates + 1 field; lift MLP to 128;
+    block with H=8, D=16, M=128 and a 4x GELU MLP; Xavier weights): the fused bf16 path against the same modules run
+    as fp32 torch layers around the fp32 HIP mixer, and 64 sampled tokens of the lift against the fp64 oracle."""
+    torch.manual_seed(0)
+    lift = F.ResidualMLP(3, 128, 128, num_layers=2, input_residual=False, output_residual=True).to(dev).eval()
+    blk = F.FLAREBlock(channel_dim=128, num_heads=8, num_latents=128, num_layers_ffn=0, ffn_mlp_ratio=4.0).to(dev).eval()
+    for l in [*lift.modules(), *blk.modules()]:
+        if isinstance(l, nn.Linear):
+            nn.init.xavier_uniform_(l.weight)
+            nn.init.zeros_(l.bias)
+    pts = torch.cat([torch.rand(4, 65536, 2, device=dev), torch.randn(4, 65536, 1, device=dev)], dim=-1)
+    with torch.no_grad():
+        ref = blk(lift(pts))[0]
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            cd = fused.compute_dtype(pts, lift)
+            assert cd == torch.bfloat16 and fused.compute_dtype(ref, blk.mlp) == torch.bfloat16
+            h = fused.fused_mlp(pts, lift, cd)
+            y = blk(h)[0]
+    assert y.shape == (4, 65536, 128) and torch.isfinite(y).all()
+    assert O.rel_l2(y, ref) <= 2e-2
+    idx = torch.randint(0, 65536, (64,), device=dev)
+    assert O.rel_l2(h[2, idx], _narrow_oracle(lift, pts[2, idx], cd)) <= 2e-2
