@@ -27,6 +27,10 @@ function (paths relative to the reference tree):
                         outer residual of FLAREBlock.forward :204-215
   causal_linear_*       lra/models/triton/causal_linear.py:317-336 (token recurrence, k and v
                         each scaled by N^-1/2) and :338-389 (chunked form)
+  flare_layer / flare_block / flare_model
+                        pdebench/models/flare.py:122-156 (FLARE.forward), :204-215 (FLAREBlock.forward),
+                        :337-349 (FLAREModel.forward) as functions of a state_dict with the reference's
+                        key names; composed of mixer_explicit and residual_mlp only
 
 Pinning status (what each function is checked against in tests/test_oracle.py):
   mixer_sdpa / mixer_explicit : each other (independent code paths: torch's SDPA kernel vs
@@ -41,6 +45,9 @@ Pinning status (what each function is checked against in tests/test_oracle.py):
   residual_mlp                : torch's own nn.Linear / nn.GELU(approximate='tanh') / nn.SiLU /
       nn.LayerNorm / nn.RMSNorm modules carrying the same weights, and the erf-free closed form of
       tanh-GELU at a few points.
+  flare_layer / flare_block / flare_model : compositions of the pinned functions above; the composition
+      itself (norm and residual placement, head split 'b n (h d) -> b h n d', latent_q.view(H, M, D)) against
+      torch.nn modules assembled in the test from nn.Linear / nn.LayerNorm and F.scaled_dot_product_attention.
   causal_linear_recurrent     : the closed form tril(Q K^T) V / N, the chunked form for several
       chunk sizes, a pure-Python-float brute force, last row == non-causal linear attention.
 """
@@ -224,6 +231,83 @@ def residual_mlp(x, weights, biases, act="gelu", input_residual=True, output_res
         h = lin(x, len(ws) - 1)
         out = x + h if output_residual else h
     return out if res is None else res.to(dtype) + out
+
+
+# --------------------------------------------------------------------------------------
+# FLARE layer, block and model as functions of a state_dict (reference key names)
+# --------------------------------------------------------------------------------------
+def _mlp_params(sd, prefix):
+    """Weights and biases of the ResidualMLP stored under `prefix` (fc1, fcs.i, fc2; or the single fc)."""
+    if prefix + "fc.weight" in sd:
+        return [sd[prefix + "fc.weight"]], [sd.get(prefix + "fc.bias")]
+    names = ["fc1"]
+    i = 0
+    while f"{prefix}fcs.{i}.weight" in sd:
+        names.append(f"fcs.{i}")
+        i += 1
+    names.append("fc2")
+    return [sd[prefix + n + ".weight"] for n in names], [sd.get(prefix + n + ".bias") for n in names]
+
+
+def _mlp(sd, prefix, x, act, input_residual, output_residual):
+    """ResidualMLP (flare.py:24-59): a residual flag only takes effect when the widths match."""
+    ws, bs = _mlp_params(sd, prefix)
+    if len(ws) > 1:
+        input_residual = input_residual and ws[0].shape[1] == ws[0].shape[0]
+        output_residual = output_residual and ws[-1].shape[1] == ws[-1].shape[0]
+    else:
+        input_residual = output_residual = input_residual and output_residual and ws[0].shape[0] == ws[0].shape[1]
+    return residual_mlp(x, ws, bs, act, input_residual, output_residual)
+
+
+def _norm(sd, prefix, x, rmsnorm, eps):
+    """nn.LayerNorm (eps 1e-5) or nn.RMSNorm (eps=None: machine epsilon of the input type) over the last axis."""
+    x = x.double()
+    w = sd[prefix + "weight"].double()
+    if rmsnorm:
+        e = torch.finfo(torch.float32).eps if eps is None else eps
+        return x / torch.sqrt((x ** 2).mean(-1, keepdim=True) + e) * w
+    e = 1e-5 if eps is None else eps
+    mu = x.mean(-1, keepdim=True)
+    var = ((x - mu) ** 2).mean(-1, keepdim=True)
+    return (x - mu) / torch.sqrt(var + e) * w + sd[prefix + "bias"].double()
+
+
+def flare_layer(sd, prefix, x, num_heads, act="gelu", attn_scale=1.0, qk_norm=False, rmsnorm=False):
+    """FLARE.forward (flare.py:122-156): k, v = MLPs of x split into heads, q = latent_q.view(H, M, D),
+    y = out_proj(merge heads(mixer(q, k, v)))."""
+    B, N, Cdim = x.shape
+    H = num_heads
+    D = Cdim // H
+    q = sd[prefix + "latent_q"].double().reshape(H, -1, D)                       # view(H, M, D) of the [C, M] parameter
+    k = _mlp(sd, prefix + "k_proj.", x, act, True, True).reshape(B, N, H, D).permute(0, 2, 1, 3)
+    v = _mlp(sd, prefix + "v_proj.", x, act, True, True).reshape(B, N, H, D).permute(0, 2, 1, 3)
+    if qk_norm:
+        q = _norm(sd, prefix + "q_norm.", q, rmsnorm, None)
+        k = _norm(sd, prefix + "k_norm.", k, rmsnorm, None)
+    y, _ = mixer_explicit(q, k, v, attn_scale, dtype=torch.float64)
+    y = y.permute(0, 2, 1, 3).reshape(B, N, Cdim)
+    return y @ sd[prefix + "out_proj.weight"].double().T + sd[prefix + "out_proj.bias"].double()
+
+
+def flare_block(sd, prefix, x, num_heads, act="gelu", attn_scale=1.0, qk_norm=False, rmsnorm=False):
+    """FLAREBlock.forward (flare.py:204-215): x += att(norm1(x)); x += mlp(norm2(x))."""
+    x = x.double()
+    x = x + flare_layer(sd, prefix + "att.", _norm(sd, prefix + "norm1.", x, rmsnorm, None), num_heads, act,
+                        attn_scale, qk_norm, rmsnorm)
+    return x + _mlp(sd, prefix + "mlp.", _norm(sd, prefix + "norm2.", x, rmsnorm, None), act, True, True)
+
+
+def flare_model(sd, x, num_heads, num_blocks, act="gelu", attn_scale=1.0, qk_norm=False, rmsnorm=False,
+                out_proj_norm=True):
+    """FLAREModel.forward (flare.py:337-349; layers built at :274-318): in_proj (output residual only), the blocks,
+    then norm + out MLP (input residual only)."""
+    x = _mlp(sd, "in_proj.", x.double(), act, False, True)
+    for b in range(num_blocks):
+        x = flare_block(sd, f"blocks.{b}.", x, num_heads, act, attn_scale, qk_norm, rmsnorm)
+    if out_proj_norm:
+        x = _norm(sd, "out_proj.0.", x, rmsnorm, None)
+    return _mlp(sd, "out_proj.1.", x, act, True, False)
 
 
 # --------------------------------------------------------------------------------------

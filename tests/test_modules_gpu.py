@@ -248,3 +248,36 @@ def test_autocast_training_step_gradients(dev, monkeypatch):
     for name, pr in cpu.named_parameters():
         if name in ("blocks.0.att.latent_q", "blocks.1.att.k_proj.fc1.weight", "blocks.0.att.v_proj.fc2.weight", "in_proj.fc1.weight"):
             assert O.rel_l2(got[name].grad, pr.grad) <= 6e-2, name
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(rmsnorm=True, qk_norm=True, act="silu"), dict(attn_scale=0.5, num_layers_ffn=0, ffn_mlp_ratio=2.0),
+                                dict(num_layers_k_proj=-1, num_layers_v_proj=0, out_proj_norm=False)])
+def test_model_on_hip_against_state_dict_oracle(dev, kw):
+    """FLAREModel on the HIP mixer path (fp32) against oracle.flare_model, which knows the model only through
+    its state_dict under the reference's key names (pdebench/models/flare.py:251-349)."""
+    torch.manual_seed(2)
+    m = FLAREModel(in_dim=3, out_dim=2, channel_dim=32, num_blocks=2, num_heads=4, num_latents=16, **kw).to(dev).eval()
+    for p_ in m.parameters():
+        torch.nn.init.normal_(p_, 0.0, 0.3) if p_.dim() > 1 else torch.nn.init.normal_(p_, 0.3, 0.3)
+    x = torch.randn(2, 200, 3, device=dev)
+    with torch.no_grad():
+        y = m(x)
+    sd = {k: v.cpu() for k, v in m.state_dict().items()}
+    ref = O.flare_model(sd, x.cpu(), 4, 2, act=kw.get("act", "gelu"), attn_scale=kw.get("attn_scale", 1.0),
+                        qk_norm=kw.get("qk_norm", False), rmsnorm=kw.get("rmsnorm", False),
+                        out_proj_norm=kw.get("out_proj_norm", True))
+    assert O.rel_l2(y, ref) <= 1e-5
+
+
+def test_block_bf16_fused_against_state_dict_oracle(dev):
+    """The fused bf16 inference path of one block (C=128, H=8, M=128) against oracle.flare_block in fp64."""
+    torch.manual_seed(3)
+    blk = FLAREBlock(channel_dim=128, num_heads=8, num_latents=128).to(dev).eval()
+    for p_ in blk.parameters():
+        if p_.dim() == 2 and p_.shape[0] == p_.shape[1]:
+            torch.nn.init.xavier_uniform_(p_)
+    x = torch.randn(2, 1024, 128, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y, _ = blk(x)
+    ref = O.flare_block({k: v.cpu() for k, v in blk.state_dict().items()}, "", x.cpu(), 8)
+    assert O.rel_l2(y, ref) <= 2e-2

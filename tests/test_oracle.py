@@ -341,3 +341,84 @@ def test_golden_vectors_are_reproducible(tmp_path):
         for name, val in old[key].items():
             a, b = torch.tensor(val, dtype=torch.float64), torch.tensor(new[key][name], dtype=torch.float64)
             assert torch.allclose(a, b, rtol=1e-13, atol=1e-15), (key, name)
+
+
+# ---- layer / block / model compositions ------------------------------------------------------------
+class _TorchBlock(torch.nn.Module):
+    """Pre-norm block assembled from torch's own layers and SDPA, for pinning flare_block's composition:
+    x += out(merge(SDPA(k, q, SDPA(q, k, v)))) with k, v = MLP(norm1 x); x += MLP(norm2 x)."""
+
+    def __init__(self, C, H, M, n):
+        super().__init__()
+        nn = torch.nn
+        mk = lambda: nn.ModuleList(nn.Linear(C, C) for _ in range(n + 2))
+        self.H, self.M, self.n1, self.n2 = H, M, nn.LayerNorm(C), nn.LayerNorm(C)
+        self.kp, self.vp, self.ff, self.out = mk(), mk(), mk(), nn.Linear(C, C)
+        self.lq = nn.Parameter(torch.randn(C, M) * 0.3)
+        self.act = nn.GELU(approximate="tanh")
+
+    def mlp(self, ls, x):
+        x = x + self.act(ls[0](x))
+        for l in ls[1:-1]:
+            x = x + self.act(l(x))
+        return x + ls[-1](x)
+
+    def forward(self, x):
+        B, N, C = x.shape
+        h = self.n1(x)
+        split = lambda t: t.view(B, N, self.H, C // self.H).transpose(1, 2)
+        k, v = split(self.mlp(self.kp, h)), split(self.mlp(self.vp, h))
+        q = self.lq.view(self.H, self.M, C // self.H).unsqueeze(0).expand(B, -1, -1, -1)
+        sdpa = torch.nn.functional.scaled_dot_product_attention
+        z = sdpa(q, k, v, scale=1.0)
+        y = sdpa(k, q, z, scale=1.0)
+        x = x + self.out(y.transpose(1, 2).reshape(B, N, C))
+        return x + self.mlp(self.ff, self.n2(x))
+
+    def reference_keys(self):
+        """The same parameters under the state_dict names of pdebench/models/flare.py."""
+        sd = {"norm1.weight": self.n1.weight, "norm1.bias": self.n1.bias, "norm2.weight": self.n2.weight,
+              "norm2.bias": self.n2.bias, "att.latent_q": self.lq, "att.out_proj.weight": self.out.weight,
+              "att.out_proj.bias": self.out.bias}
+        for name, ls in (("att.k_proj.", self.kp), ("att.v_proj.", self.vp), ("mlp.", self.ff)):
+            keys = ["fc1"] + [f"fcs.{i}" for i in range(len(ls) - 2)] + ["fc2"]
+            for kname, l in zip(keys, ls):
+                sd[name + kname + ".weight"], sd[name + kname + ".bias"] = l.weight, l.bias
+        return {k: v.detach() for k, v in sd.items()}
+
+
+@pytest.mark.parametrize("C,H,M,n", [(32, 4, 8, 1), (48, 3, 5, 0), (16, 2, 16, 3)])
+def test_block_composition_against_torch_layers(C, H, M, n):
+    torch.manual_seed(C + n)
+    blk = _TorchBlock(C, H, M, n).double()
+    for p_ in blk.parameters():
+        if p_.dim() == 1:
+            torch.nn.init.normal_(p_, 0.5, 0.3)
+    x = torch.randn(2, 37, C, dtype=torch.float64)
+    with torch.no_grad():
+        ref = blk(x)
+    got = O.flare_block(blk.reference_keys(), "", x, H)
+    assert O.rel_l2(got, ref) <= 1e-12
+    # a dropped residual, a swapped norm or a transposed head split must show
+    sd = blk.reference_keys()
+    sd["norm1.weight"], sd["norm2.weight"] = sd["norm2.weight"], sd["norm1.weight"]
+    assert O.rel_l2(O.flare_block(sd, "", x, H), ref) > 1e-3
+
+
+def test_product_modules_scores_branch_against_model_oracle():
+    """The product's modules on the CPU (their spelled-out return_scores branch needs no HIP kernel) against the
+    state_dict oracle: key names, flag handling and layer order of FLAREModel agree with flare.py:251-349."""
+    import flare_py_amd as FA
+    for kw in (dict(), dict(rmsnorm=True, qk_norm=True, act="silu"), dict(num_layers_ffn=0, ffn_mlp_ratio=2.0, num_layers_k_proj=-1),
+               dict(out_proj_norm=False, num_layers_in_out_proj=0)):
+        torch.manual_seed(1)
+        m = FA.FLAREModel(in_dim=3, out_dim=2, channel_dim=32, num_blocks=2, num_heads=4, num_latents=8, **kw).eval()
+        for p_ in m.parameters():
+            torch.nn.init.normal_(p_, 0.0, 0.3) if p_.dim() > 1 else torch.nn.init.normal_(p_, 0.3, 0.3)
+        x = torch.randn(2, 19, 3)
+        with torch.no_grad():
+            y, scores = m(x, return_scores=True)
+        assert len(scores) == 2 and scores[0].shape == (2, 4, 8, 19)
+        ref = O.flare_model(m.state_dict(), x, 4, 2, act=kw.get("act", "gelu") or "gelu", qk_norm=kw.get("qk_norm", False),
+                            rmsnorm=kw.get("rmsnorm", False), out_proj_norm=kw.get("out_proj_norm", True))
+        assert O.rel_l2(y, ref) <= 1e-5, kw
