@@ -21,7 +21,33 @@ from torch.nn import functional as F
 from .functional import flare_multihead_mixer, triple_attention
 from .modules import ResidualMLP, _norm
 
-__all__ = ["FLARE", "FLAREBlock", "TripleAttention", "TripleBlock", "make_kernel"]
+__all__ = ["FLARE", "FLAREBlock", "TripleAttention", "TripleBlock", "make_kernel", "RotaryPositionalEmbeddings"]
+
+
+class RotaryPositionalEmbeddings(nn.Module):
+    """The rotary embedding the sequence models hand to their blocks as `rope` (lra/models/embeddings.py:103-147;
+    built at lra/models/wrapper.py:87-88 with D = head_dim), applied to k only (backends.py:600-601).
+
+    Position p turns channel j by the angle p * base^(-(j // 2) / (D / 2)):  out = x * cos + r * sin, where the
+    partner r is the reference's own arrangement: its first half holds the negated odd channels
+    (-x[1], -x[3], ...) and its second half the even channels (x[0], x[2], ...) -- not the interleaved pairing
+    of the usual rotary embedding.  Checkpoints trained with the reference depend on it, so it is kept.
+    Buffers C, S [max_length, D] are not part of the state_dict (as in the reference)."""
+
+    def __init__(self, D: int, max_length: int, base: int = 10_000):
+        super().__init__()
+        assert D % 2 == 0
+        self.D, self.N, self.base = D, max_length, float(base)
+        rate = self.base ** (-(torch.arange(D, dtype=torch.float32) // 2) / (D // 2))      # [D], equal in pairs
+        angle = torch.arange(max_length, dtype=torch.float32)[:, None] * rate[None, :]     # [N, D]
+        self.register_buffer("C", torch.cos(angle), persistent=False)
+        self.register_buffer("S", torch.sin(angle), persistent=False)
+
+    def forward(self, x: torch.Tensor):
+        N, D = x.shape[-2], x.shape[-1]
+        assert D == self.D and N <= self.N
+        partner = torch.cat([-x[..., 1::2], x[..., 0::2]], dim=-1)
+        return x * self.C[:N].to(x.dtype) + partner * self.S[:N].to(x.dtype)
 
 
 class FLARE(nn.Module):

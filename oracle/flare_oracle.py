@@ -27,6 +27,7 @@ function (paths relative to the reference tree):
                         outer residual of FLAREBlock.forward :204-215
   causal_linear_*       lra/models/triton/causal_linear.py:317-336 (token recurrence, k and v
                         each scaled by N^-1/2) and :338-389 (chunked form)
+  rope_reference        lra/models/embeddings.py:103-147 (rotary embedding applied to k, backends.py:600-601)
   flare_layer / flare_block / flare_model
                         pdebench/models/flare.py:122-156 (FLARE.forward), :204-215 (FLAREBlock.forward),
                         :337-349 (FLAREModel.forward) as functions of a state_dict with the reference's
@@ -48,6 +49,8 @@ Pinning status (what each function is checked against in tests/test_oracle.py):
   flare_layer / flare_block / flare_model : compositions of the pinned functions above; the composition
       itself (norm and residual placement, head split 'b n (h d) -> b h n d', latent_q.view(H, M, D)) against
       torch.nn modules assembled in the test from nn.Linear / nn.LayerNorm and F.scaled_dot_product_attention.
+  rope_reference              : position 0 is the identity; D = 2 is the plane rotation by p radians; a D = 4
+      vector worked out by hand from the text of embeddings.py:136-147; linearity in x.
   causal_linear_recurrent     : the closed form tril(Q K^T) V / N, the chunked form for several
       chunk sizes, a pure-Python-float brute force, last row == non-causal linear attention.
 """
@@ -234,6 +237,25 @@ def residual_mlp(x, weights, biases, act="gelu", input_residual=True, output_res
 
 
 # --------------------------------------------------------------------------------------
+# rotary embedding of the sequence models
+# --------------------------------------------------------------------------------------
+def rope_reference(x, base=10000.0):
+    """lra/models/embeddings.py:103-147 element by element: for position p and channel j of x [..., N, D],
+    out[p, j] = x[p, j] cos(p w_j) + r[p, j] sin(p w_j) with w_j = base^(-(j // 2) / (D / 2)) and the partner
+    r[j] = -x[2 j + 1] for j < D/2, x[2 (j - D/2)] for j >= D/2 (the reference concatenates the negated odd
+    channels and the even channels; it does not interleave them)."""
+    x = x.double()
+    N, D = x.shape[-2], x.shape[-1]
+    out = torch.empty_like(x)
+    for j in range(D):
+        w = base ** (-(j // 2) / (D // 2))
+        ang = torch.arange(N, dtype=torch.float64) * w
+        r = -x[..., 2 * j + 1] if j < D // 2 else x[..., 2 * (j - D // 2)]
+        out[..., j] = x[..., j] * torch.cos(ang) + r * torch.sin(ang)
+    return out
+
+
+# --------------------------------------------------------------------------------------
 # FLARE layer, block and model as functions of a state_dict (reference key names)
 # --------------------------------------------------------------------------------------
 def _mlp_params(sd, prefix):
@@ -273,9 +295,11 @@ def _norm(sd, prefix, x, rmsnorm, eps):
     return (x - mu) / torch.sqrt(var + e) * w + sd[prefix + "bias"].double()
 
 
-def flare_layer(sd, prefix, x, num_heads, act="gelu", attn_scale=1.0, qk_norm=False, rmsnorm=False):
+def flare_layer(sd, prefix, x, num_heads, act="gelu", attn_scale=1.0, qk_norm=False, rmsnorm=False, key_mask=None,
+                rope=None):
     """FLARE.forward (flare.py:122-156): k, v = MLPs of x split into heads, q = latent_q.view(H, M, D),
-    y = out_proj(merge heads(mixer(q, k, v)))."""
+    y = out_proj(merge heads(mixer(q, k, v))).  key_mask [B,N] (True = real token) and rope (a function of k)
+    give the sequence variant lra/models/backends.py:588-622: padded keys are left out of the gather, rope turns k only."""
     B, N, Cdim = x.shape
     H = num_heads
     D = Cdim // H
@@ -285,16 +309,20 @@ def flare_layer(sd, prefix, x, num_heads, act="gelu", attn_scale=1.0, qk_norm=Fa
     if qk_norm:
         q = _norm(sd, prefix + "q_norm.", q, rmsnorm, None)
         k = _norm(sd, prefix + "k_norm.", k, rmsnorm, None)
-    y, _ = mixer_explicit(q, k, v, attn_scale, dtype=torch.float64)
+    if rope is not None:
+        k = rope(k)
+    y, _ = mixer_explicit(q, k, v, attn_scale, key_mask, dtype=torch.float64)
     y = y.permute(0, 2, 1, 3).reshape(B, N, Cdim)
     return y @ sd[prefix + "out_proj.weight"].double().T + sd[prefix + "out_proj.bias"].double()
 
 
-def flare_block(sd, prefix, x, num_heads, act="gelu", attn_scale=1.0, qk_norm=False, rmsnorm=False):
-    """FLAREBlock.forward (flare.py:204-215): x += att(norm1(x)); x += mlp(norm2(x))."""
+def flare_block(sd, prefix, x, num_heads, act="gelu", attn_scale=1.0, qk_norm=False, rmsnorm=False, key_mask=None,
+                rope=None):
+    """FLAREBlock.forward (flare.py:204-215; lra/models/backends.py:665-672 with attention_mask):
+    x += att(norm1(x)); x += mlp(norm2(x))."""
     x = x.double()
     x = x + flare_layer(sd, prefix + "att.", _norm(sd, prefix + "norm1.", x, rmsnorm, None), num_heads, act,
-                        attn_scale, qk_norm, rmsnorm)
+                        attn_scale, qk_norm, rmsnorm, key_mask, rope)
     return x + _mlp(sd, prefix + "mlp.", _norm(sd, prefix + "norm2.", x, rmsnorm, None), act, True, True)
 
 

@@ -147,3 +147,18 @@ def test_reference_trainer_snapshot_loads(tmp_path):
     torch.save({"weights": 1}, path)
     with pytest.raises(ValueError):
         read_snapshot(path)
+
+
+def test_rotary_embedding_module_against_oracle():
+    """RotaryPositionalEmbeddings (lra/models/embeddings.py:103-147): values, strided head views, and buffers that
+    stay out of the state_dict."""
+    from flare_py_amd.lra_modules import RotaryPositionalEmbeddings
+    from oracle import flare_oracle as O
+    rope = RotaryPositionalEmbeddings(16, 64)
+    assert list(rope.state_dict().keys()) == [] and rope.C.shape == (64, 16)
+    x = torch.randn(2, 50, 4 * 16)
+    k = x.view(2, 50, 4, 16).permute(0, 2, 1, 3)                     # the view the block hands over
+    assert O.rel_l2(rope(k), O.rope_reference(k)) <= 1e-6
+    assert O.rel_l2(rope(k.bfloat16()).float(), O.rope_reference(k.bfloat16().float())) <= 2e-2
+    with pytest.raises(AssertionError):
+        rope(torch.randn(1, 1, 65, 16))

@@ -87,6 +87,10 @@ def test_lra_block_with_padding_mask(dev, monkeypatch):
     with torch.no_grad():
         yr = cpu(x.cpu(), attention_mask=mask.cpu())
     assert O.rel_l2(y, yr) <= 1e-5
+    # and against the state_dict oracle (rows of padded tokens are backend dependent in torch: compare real tokens)
+    yo = O.flare_block({k_: v_.cpu() for k_, v_ in blk.state_dict().items()}, "", x.cpu(), 4, key_mask=mask.cpu())
+    keep = mask.cpu()
+    assert O.rel_l2(y.cpu()[keep], yo[keep]) <= 1e-5
     # padded tokens do not influence real ones
     x2 = x.clone()
     x2[0, 25:] = 7.0
@@ -281,3 +285,26 @@ def test_block_bf16_fused_against_state_dict_oracle(dev):
         y, _ = blk(x)
     ref = O.flare_block({k: v.cpu() for k, v in blk.state_dict().items()}, "", x.cpu(), 8)
     assert O.rel_l2(y, ref) <= 2e-2
+
+
+def test_lra_block_with_rope_and_mask_against_oracle(dev):
+    """The sequence block with the rotary embedding on k and a padding mask (lra/models/backends.py:588-622)."""
+    torch.manual_seed(5)
+    rope = lra_modules.RotaryPositionalEmbeddings(16, 128)
+    blk = lra_modules.FLAREBlock(channel_dim=64, num_heads=4, num_latents=16, kv_proj_hidden_dim=64, ffn_hidden_dim=64,
+                                 rope=rope).to(dev).eval()
+    for p_ in blk.parameters():
+        torch.nn.init.normal_(p_, 0.0, 0.3) if p_.dim() > 1 else torch.nn.init.normal_(p_, 0.3, 0.3)
+    x = torch.randn(2, 100, 64, device=dev)
+    mask = torch.ones(2, 100, dtype=torch.bool, device=dev)
+    mask[1, 60:] = False
+    with torch.no_grad():
+        y = blk(x, attention_mask=mask)
+        y_nomask = blk(x)
+    assert not any(k_.startswith("att.rope") for k_ in blk.state_dict())          # buffers are not persistent
+    sd = {k_: v_.cpu() for k_, v_ in blk.state_dict().items()}
+    yo = O.flare_block(sd, "", x.cpu(), 4, key_mask=mask.cpu(), rope=O.rope_reference)
+    keep = mask.cpu()
+    assert O.rel_l2(y.cpu()[keep], yo[keep]) <= 1e-5
+    assert O.rel_l2(y_nomask, O.flare_block(sd, "", x.cpu(), 4, rope=O.rope_reference)) <= 1e-5
+    assert O.rel_l2(y_nomask, O.flare_block(sd, "", x.cpu(), 4)) > 1e-3             # the rotation matters

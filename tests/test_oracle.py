@@ -422,3 +422,28 @@ def test_product_modules_scores_branch_against_model_oracle():
         ref = O.flare_model(m.state_dict(), x, 4, 2, act=kw.get("act", "gelu") or "gelu", qk_norm=kw.get("qk_norm", False),
                             rmsnorm=kw.get("rmsnorm", False), out_proj_norm=kw.get("out_proj_norm", True))
         assert O.rel_l2(y, ref) <= 1e-5, kw
+
+
+def test_rope_reference_hand_cases():
+    # position 0: identity
+    x = torch.randn(2, 3, 1, 8, dtype=torch.float64)
+    assert torch.equal(O.rope_reference(x), x)
+    # D = 2: the plane rotation by p radians
+    x = torch.randn(5, 2, dtype=torch.float64)
+    got = O.rope_reference(x)
+    for p_ in range(5):
+        c, s_ = math.cos(p_), math.sin(p_)
+        assert abs(float(got[p_, 0]) - (float(x[p_, 0]) * c - float(x[p_, 1]) * s_)) < 1e-12
+        assert abs(float(got[p_, 1]) - (float(x[p_, 1]) * c + float(x[p_, 0]) * s_)) < 1e-12
+    # D = 4 by hand from lra/models/embeddings.py:136-147: rates (1, 1, b, b), b = base^-1/2; partner (-a1, -a3, a0, a2)
+    a = [0.3, -1.1, 0.7, 2.0]
+    x = torch.tensor([a, a, a], dtype=torch.float64)
+    got = O.rope_reference(x, base=100.0)
+    b = 100.0 ** -0.5
+    for p_ in range(3):
+        want = [a[0] * math.cos(p_) - a[1] * math.sin(p_), a[1] * math.cos(p_) - a[3] * math.sin(p_),
+                a[2] * math.cos(p_ * b) + a[0] * math.sin(p_ * b), a[3] * math.cos(p_ * b) + a[2] * math.sin(p_ * b)]
+        assert max(abs(float(got[p_, j]) - want[j]) for j in range(4)) < 1e-12
+    # linear in x
+    u, v = torch.randn(7, 6, dtype=torch.float64), torch.randn(7, 6, dtype=torch.float64)
+    assert O.rel_l2(O.rope_reference(2.0 * u - v), 2.0 * O.rope_reference(u) - O.rope_reference(v)) < 1e-14
