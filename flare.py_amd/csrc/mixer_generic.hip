@@ -205,7 +205,7 @@ __global__ __launch_bounds__(kScatterThreads) void scatter_generic_kernel(MixerA
         T* y = (T*)a.y + b * a.ys[0] + h * a.ys[1] + (int64_t)n * a.ys[2];
 #pragma unroll
         for (int d = 0; d < DMAX; ++d)
-            if (d < D) y[d] = from_f32<T>(acc[d] * inv);
+            if (d < D) y[d] = from_f32<T>(on ? acc[d] * inv : 0.f);      // a padded row is 0 whatever its key row held
     }
 }
 

@@ -14,7 +14,7 @@
 // range that exp2(score) is safe while the scores of a row stay inside (-60, +120); the
 // denominators come out of the second product as a row of ones in its A operand and are
 // validated after the pass (2^-60 <= l <= 2^120).  What fails validation (and, in the gather,
-// every masked problem) is recomputed through an exact path with a running maximum.
+// a masked range whose real tokens underflow) is recomputed through an exact path with a running maximum.
 //
 //   gather : z = softmax_n(s q k^T) v   split over N, partial (shift, sum, numerator)
 //   scatter: y = softmax_m(s k q^T) z   token parallel, Q and Z^T resident in LDS
@@ -177,6 +177,7 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
 
     __shared__ __attribute__((aligned(16))) uint8_t kt[2][TILEB];
     __shared__ __attribute__((aligned(16))) uint8_t vt[2][TILEB];
+    __shared__ __attribute__((aligned(16))) uint16_t mt[2][kGTile];   // per token: bf16 1 (real) or 0 (masked / past the range)
     __shared__ int wg_flag[4];
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
@@ -216,17 +217,21 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
     auto k_slot = [](int tok, int ch) { return tok * ROWB + ((ch ^ ((tok >> 2) & (CH - 1))) << 4); };
     auto v_slot = [](int tok, int ch) { return tok * ROWB + ((CH >= 4 ? (ch ^ (((tok >> 2) & 1) << 1)) : ch) << 4); };
 
-    // two register sets: tiles are fetched two iterations before they are consumed
+    // two register sets: tiles are fetched two iterations before they are consumed.  A token that is masked or
+    // lies past the range keeps a (finite) K row but gets a zero V row and a zero in the tile's row of "ones":
+    // whatever its probability, it adds nothing to the numerators or the denominators.
     u32x4 kr[2][CPT], vr[2][CPT];
+    bool live[2][CPT];
     auto load_tile = [&](auto set_tag, int n0) {
         constexpr int S = decltype(set_tag)::value;
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * 256;
             if (c < TCH) {
-                const int n = min(n0 + c / CH, n_end - 1), ch = c % CH;
+                const int nn = n0 + c / CH, n = min(nn, n_end - 1), ch = c % CH;
                 kr[S][i] = load16_stream(k + (int64_t)n * a.ks[2] + ch * 8);
                 vr[S][i] = load16_stream(v + (int64_t)n * a.vs[2] + ch * 8);
+                live[S][i] = nn < n_end && (mask == nullptr || mask[n] != 0);
             }
         }
     };
@@ -238,7 +243,8 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
             if (c < TCH) {
                 const int tok = c / CH, ch = c % CH;
                 *reinterpret_cast<u32x4*>(&kt[S][k_slot(tok, ch)]) = kr[S][i];
-                *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = to_bf16x8<T>(vr[S][i]);
+                *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = live[S][i] ? to_bf16x8<T>(vr[S][i]) : zero4();
+                if (ch == 0) mt[S][tok] = live[S][i] ? uint16_t(P_::kOnes2 & 0xffffu) : uint16_t(0);
             }
         }
     };
@@ -284,9 +290,16 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                         const uint2 hi = lds_read_tr16(&vt[buf][v_slot(r1, ch) + sub]);
                         va[rt] = u32x4{lo.x, lo.y, hi.x, hi.y};
                     }
-                    if constexpr (!EXACT && !RAGGED) {
+                    if constexpr (!EXACT) {
                         // steady state: latent tiles software pipelined (scores of tile ct+1 issued before
-                        // the exponentials of tile ct, value product of tile ct-1 after them)
+                        // the exponentials of tile ct, value product of tile ct-1 after them).  The row of ones is
+                        // the tile's live-token row when the tile is ragged or masked.
+                        u32x4 ones_a = ones8;
+                        if constexpr (RAGGED) {
+                            const uint2 lo = *reinterpret_cast<const uint2*>(&mt[buf][ks * 32 + 4 * g]);
+                            const uint2 hi = *reinterpret_cast<const uint2*>(&mt[buf][ks * 32 + 16 + 4 * g]);
+                            ones_a = u32x4{lo.x, lo.y, hi.x, hi.y};
+                        }
                         auto sc2 = [&](int ct, f32x4& s0, f32x4& s1) {
                             s0 = f32x4{0.f, 0.f, 0.f, 0.f};
                             s1 = s0;
@@ -299,7 +312,7 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                         auto pv = [&](int ct, u32x4 pb) {
     #pragma unroll
                             for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = P_::mma(va[rt], pb, zacc[rt][ct]);
-                            lacc[ct] = P_::mma(ones8, pb, lacc[ct]);   // row of ones: the softmax denominator
+                            lacc[ct] = P_::mma(ones_a, pb, lacc[ct]);   // row of ones: the softmax denominator
                         };
                         f32x4 s0, s1;
                         sc2(0, s0, s1);
@@ -390,28 +403,35 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
         }
     };
 
-    run(std::false_type{});
-    // validate: every denominator of this wave inside the safe range, numerators finite
-    bool bad = false;
+    // validate: every denominator of this wave inside the safe range, numerators finite.  With a key mask a
+    // range without a single real token legitimately gives l = 0: the lower bound applies only when the
+    // range holds one (counted here; the mask and the range are uniform over the workgroup).
+    bool exact;
+    {
+        run(std::false_type{});
+        int has_valid = n_begin < n_end;
+        if (mask != nullptr) {
+            int any = 0;
+            for (int n = n_begin + tid; n < n_end; n += 256) any |= mask[n];
+            has_valid = __syncthreads_or(any);
+        }
+        bool bad = false;
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        const float l = lacc[ct][0];
-        bad = bad || !(l <= kLMax) || (n_begin < n_end && mask == nullptr && !(l >= kLMin));
+        for (int ct = 0; ct < CT; ++ct) {
+            const float l = lacc[ct][0];
+            bad = bad || !(l <= kLMax) || (has_valid && !(l >= kLMin));
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+            for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) bad = bad || !(fabsf(zacc[rt][ct][r]) <= 3.0e38f);
+                for (int r = 0; r < 4; ++r) bad = bad || !(fabsf(zacc[rt][ct][r]) <= 3.0e38f);
+        }
+        const int anybad = __any(bad);
+        __syncthreads();
+        if (lane == 0) wg_flag[w] = anybad;
+        __syncthreads();
+        exact = (wg_flag[0] | wg_flag[1] | wg_flag[2] | wg_flag[3]) != 0;
     }
-    if (mask != nullptr) {
-        // with a key mask an all-masked range legitimately gives l = 0; small l cannot be told
-        // apart from underflow cheaply, so masked problems always take the exact pass
-        bad = true;
-    }
-    const int anybad = __any(bad);
-    __syncthreads();
-    if (lane == 0) wg_flag[w] = anybad;
-    __syncthreads();
-    if (wg_flag[0] | wg_flag[1] | wg_flag[2] | wg_flag[3]) {
+    if (exact) {
         asm volatile("; exact pass" ::: "memory");
         run(std::true_type{});
     }
@@ -674,8 +694,10 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                     uint32_t o[2 * RT];
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt) {
-                        o[2 * rt] = M_::pack2(yacc[tw][rt][0] * inv, yacc[tw][rt][1] * inv);
-                        o[2 * rt + 1] = M_::pack2(yacc[tw][rt][2] * inv, yacc[tw][rt][3] * inv);
+                        f32x4 yv = yacc[tw][rt] * inv;
+                        if (!FULL && !on) yv = f32x4{0.f, 0.f, 0.f, 0.f};      // a padded row is 0 whatever its key row held
+                        o[2 * rt] = M_::pack2(yv[0], yv[1]);
+                        o[2 * rt + 1] = M_::pack2(yv[2], yv[3]);
                     }
                     if constexpr (RT == 1) {
                         *reinterpret_cast<uint2*>(yr) = make_uint2(o[0], o[1]);

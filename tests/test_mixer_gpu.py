@@ -116,6 +116,30 @@ def test_key_mask(dev, dtype, fg):
     assert (y.cpu()[~mask[:, None, :, None].expand_as(y)] == 0).all()
 
 
+@pytest.mark.parametrize("fg", [False, True])
+@pytest.mark.parametrize("garbage", [0.0, 300.0, float("nan")])
+def test_key_mask_over_many_splits_and_padding_garbage(dev, garbage, fg):
+    """A long masked batch: whole split ranges without a real token (their zero denominators are legitimate), ranges
+    that end in padding, and padded rows holding values that overflow the unshifted exponentials or are NaN
+    (the kernel then repeats the range exactly; padding must never reach the result)."""
+    q, k, v = make(3, 2, 8192, 128, 32, torch.bfloat16, seed=11)
+    mask = torch.ones(3, 8192, dtype=torch.bool)
+    mask[1, 100:] = False
+    mask[2, 5000:] = False
+    mask[2, 17:4000:5] = False
+    kk, vv = k.clone(), v.clone()
+    if garbage != 0.0:
+        kk[~mask[:, None, :, None].expand_as(k)] = garbage
+        vv[~mask[:, None, :, None].expand_as(v)] = garbage
+    y, z = F.flare_multihead_mixer(q.to(dev), kk.to(dev), vv.to(dev), key_mask=mask.to(dev), return_z=True,
+                                   force_generic=fg)
+    yr, zr = O.mixer_explicit(q.float(), k.float(), v.float(), 1.0, mask)
+    keep = mask[:, None, :, None].expand_as(yr)
+    assert torch.isfinite(z).all() and O.rel_l2(z, zr) <= 2e-2
+    assert O.rel_l2(y.float().cpu()[keep], yr[keep]) <= 2e-2
+    assert (y.cpu()[~keep] == 0).all()
+
+
 def test_fully_masked_batch_gives_zero(dev):
     q, k, v = make(2, 1, 130, 64, 32, torch.bfloat16)
     mask = torch.ones(2, 130, dtype=torch.bool)
