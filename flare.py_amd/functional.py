@@ -163,8 +163,9 @@ def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_majo
 
 
 def _hip_backward_ok(q, k, v, key_mask, force_generic) -> bool:
-    """True when flare_mixer_bwd covers this problem (16-bit types, no mask, supported M, D, strides)."""
-    if key_mask is not None or force_generic or k.dtype not in (torch.bfloat16, torch.float16):
+    """True when flare_mixer_bwd covers this problem (16-bit types, supported M, D, strides; a key mask is
+    handled around the kernels, see _MixerFn.backward)."""
+    if force_generic or k.dtype not in (torch.bfloat16, torch.float16):
         return False
     if q.dtype != k.dtype or v.dtype != k.dtype or k.device.type != "cuda":
         return False
@@ -203,7 +204,7 @@ def _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy):
 
 def _mixer_torch_grad(q, k, v, scale, key_mask, gy):
     """Backward by recomputation in plain torch ops on the device the inputs live on: used for what
-    the HIP backward does not cover (fp32, key masks, unusual shapes).  The forward never takes this path."""
+    the HIP backward does not cover (fp32, unusual shapes).  The forward never takes this path."""
     with torch.enable_grad():
         q_, k_, v_ = (t.detach().float().requires_grad_(True) for t in (q, k, v))
         qe = q_ if q_.dim() == 4 else q_.unsqueeze(0)
@@ -239,7 +240,21 @@ class _MixerFn(torch.autograd.Function):
     def backward(ctx, gy, _gz):
         if ctx.hip:
             q, k, v, y, z, lse_lat, lse_tok = ctx.saved_tensors
+            km = ctx.key_mask
+            if km is not None:
+                # A padded token takes no part in either softmax.  The kernels need no mask for that: with its k, v
+                # and dy rows zeroed it adds nothing to dq or dz, with its log-sum-exp set far above any score its
+                # scatter weights vanish, and its own dk, dv rows are cleared afterwards.  A batch element without
+                # a single real token has lse_lat = -inf; the same treatment turns its gather weights into 0.
+                keep = km.to(torch.bool)
+                m4 = keep[:, None, :, None]
+                zero = torch.zeros((), dtype=k.dtype, device=k.device)
+                k, v, gy = torch.where(m4, k, zero), torch.where(m4, v, zero), torch.where(m4, gy.to(k.dtype), zero)
+                lse_tok = torch.where(keep[:, None, :], lse_tok, lse_tok.new_tensor(1e30))
+                lse_lat = torch.where(torch.isfinite(lse_lat), lse_lat, lse_lat.new_tensor(1e30))
             gq, gk, gv = _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, ctx.scale, gy)
+            if km is not None:
+                gk, gv = torch.where(m4, gk, zero), torch.where(m4, gv, zero)
         else:
             q, k, v = ctx.saved_tensors
             gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy)

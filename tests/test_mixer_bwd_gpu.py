@@ -74,13 +74,12 @@ def test_backward_is_deterministic_and_matches_torch_recompute(dev):
 
 
 def test_fallbacks_keep_working(dev):
-    # fp32 and masked problems differentiate through the torch recomputation
+    # fp32 problems and shapes the kernels do not take differentiate through the torch recomputation
     q, k, v, gy = make(1, 2, 200, 64, 16, torch.float32, seed=7)
     qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
     assert not FN._hip_backward_ok(qd, kd, vd, None, False)
     big = [t.to(dev).bfloat16() for t in make(1, 1, 64, 256, 64, torch.float32)[:3]]
     assert not FN._hip_backward_ok(*big, None, False)                      # latent operands would not fit the LDS
-    assert not FN._hip_backward_ok(qd.bfloat16(), kd.bfloat16(), vd.bfloat16(), torch.ones(1, 200, device=dev), False)
     F.flare_multihead_mixer(qd, kd, vd).backward(gy.to(dev))
     gq, gk, gv = oracle_grads(q, k, v, gy, 1.0)
     assert O.rel_l2(qd.grad, gq) <= 1e-4 and O.rel_l2(kd.grad, gk) <= 1e-4 and O.rel_l2(vd.grad, gv) <= 1e-4
@@ -94,3 +93,33 @@ def test_lse_outputs(dev):
     assert float((lse_tok.cpu().double() - torch.logsumexp(s, -2)).abs().max()) <= 2e-2
     yg, zg, _, lt = FN._mixer_forward(q.to(dev), k.to(dev), v.to(dev), 0.7, None, 0, True, False, True)   # fp32-FMA kernels
     assert float((lt - lse_tok).abs().max()) <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_masked_backward_vs_autograd_oracle(dev, dtype):
+    """Key mask (lra/models/backends.py:603-622) through the HIP backward: holes, a padded tail, a batch element with a
+    single real token and one with none; padded rows hold NaN in k, v and dy and must not reach any gradient."""
+    B, H, N, M, D = 4, 2, 1500, 128, 32
+    q, k, v, gy = make(B, H, N, M, D, dtype, seed=13)
+    mask = torch.ones(B, N, dtype=torch.bool)
+    mask[0, 900:] = False
+    mask[0, 5:700:7] = False
+    mask[1, 1:] = False
+    mask[2] = False
+    m4 = mask[:, None, :, None]
+    nan = torch.full((), float("nan"), dtype=dtype)
+    qd = q.to(dev).requires_grad_(True)
+    kd, vd = (torch.where(m4, t, nan).to(dev).requires_grad_(True) for t in (k, v))
+    assert FN._hip_backward_ok(qd, kd, vd, mask.to(dev), False)
+    y = F.flare_multihead_mixer(qd, kd, vd, scale=0.9, key_mask=mask.to(dev))
+    y.backward(torch.where(m4, gy, nan).to(dev))
+    real = [0, 1, 3]                   # the oracle differentiates the batch elements that hold tokens; the empty one adds 0
+    qr = q.double().requires_grad_(True)
+    kr, vr = (t[real].double().requires_grad_(True) for t in (k, v))
+    yr, _ = O.mixer_explicit(qr, kr, vr, 0.9, mask[real])
+    yr.backward((gy.double() * m4)[real])
+    assert torch.isfinite(qd.grad).all() and torch.isfinite(kd.grad).all() and torch.isfinite(vd.grad).all()
+    for name, got, ref in (("dq", qd.grad, qr.grad), ("dk", kd.grad[real], kr.grad), ("dv", vd.grad[real], vr.grad)):
+        err = O.rel_l2(got, ref)
+        assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
+    assert (kd.grad.cpu()[~m4.expand_as(k)] == 0).all() and (vd.grad.cpu()[~m4.expand_as(v)] == 0).all()
