@@ -106,6 +106,9 @@ def _mask_u8(key_mask, B, N, device):
 
 def mixer_kernel_name(q, k, v=None, scale=1.0, force_generic=False) -> str:
     """Which kernel family the dispatcher picks for these operands (no launch)."""
+    pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype else 0
+    if pad:                                 # what flare_multihead_mixer hands to the library for a narrow head
+        q, k, v = _pad_last(q, pad), _pad_last(k, pad), None
     q4 = _q4(q, k.shape[0])
     d = _mixer_desc(q4, k, v, None, scale, 0, force_generic)
     name = _lib.load().flare_mixer_kernel_name(C.byref(d))
@@ -261,6 +264,20 @@ class _MixerFn(torch.autograd.Function):
         return gq, gk, gv, None, None, None, None, None
 
 
+def _narrow_head_pad(q, k, force_generic) -> int:
+    """Columns of zeros to append to a head dim below 16 so that the matrix-core kernels (D in {16, 32, 64}) take
+    the problem, or 0.  Zero columns change neither the scores q.k nor the first D output columns; the reference's
+    default model has D = channel_dim / num_heads = 8, which the fp32-FMA kernels would serve 5-15x slower."""
+    D = k.shape[-1]
+    if force_generic or D >= 16 or k.dtype not in (torch.bfloat16, torch.float16) or k.device.type != "cuda":
+        return 0
+    return 16 - D if q.shape[-2] % 64 == 0 else 0
+
+
+def _pad_last(t, n):
+    return torch.nn.functional.pad(t, (0, n))
+
+
 def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: bool = False,
                           n_splits: int = 0, force_generic: bool = False, token_major_out: bool = False):
     """FLARE gather-scatter mixer (README.md:39-52 of the reference).
@@ -277,10 +294,16 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
     ac = _autocast_dtype(k)
     if ac is not None:
         q, k, v = (t if t.dtype == ac else t.to(ac) for t in (q, k, v))
+    D = k.shape[-1]
+    pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype == v.dtype else 0
+    if pad:
+        q, k, v = _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad)
     if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
         y, z = _MixerFn.apply(q, k, v, float(scale), key_mask, n_splits, force_generic, token_major_out)
     else:
         y, z = _mixer_forward(q, k, v, float(scale), key_mask, n_splits, force_generic, token_major_out)
+    if pad:
+        y, z = y[..., :D], z[..., :D]
     return (y, z) if return_z else y
 
 
@@ -384,17 +407,29 @@ def flare_gather(q, k, v, scale: float = 1.0, key_mask=None, n_splits: int = 0,
     """z [B,H,M,D] fp32 = softmax_n(scale q k^T) v and lse [B,H,M] (natural log).
     Differentiable in q, k, v (the backward recomputes the scores with torch ops: for models that put
     layers between the two halves; the whole mixer has its own HIP backward)."""
+    D = k.shape[-1]
+    pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype == v.dtype else 0
+    if pad:
+        q, k, v = _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad)
     if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
-        return _GatherFn.apply(q, k, v, float(scale), key_mask, n_splits, force_generic)
-    return _gather_forward(q, k, v, float(scale), key_mask, n_splits, force_generic)
+        z, lse = _GatherFn.apply(q, k, v, float(scale), key_mask, n_splits, force_generic)
+    else:
+        z, lse = _gather_forward(q, k, v, float(scale), key_mask, n_splits, force_generic)
+    return (z[..., :D] if pad else z), lse
 
 
 def flare_scatter(q, k, z, scale: float = 1.0, key_mask=None, force_generic: bool = False) -> torch.Tensor:
     """y [B,H,N,D] = softmax_m(scale k q^T) z with z [B,H,M,D] (computed from its fp32 copy).
     Differentiable in q, k, z like flare_gather."""
+    D = k.shape[-1]
+    pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype else 0
+    if pad:
+        q, k, z = _pad_last(q, pad), _pad_last(k, pad), _pad_last(z, pad)
     if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, z)):
-        return _ScatterFn.apply(q, k, z, float(scale), key_mask, force_generic)
-    return _scatter_forward(q, k, z, float(scale), key_mask, force_generic)
+        y = _ScatterFn.apply(q, k, z, float(scale), key_mask, force_generic)
+    else:
+        y = _scatter_forward(q, k, z, float(scale), key_mask, force_generic)
+    return y[..., :D] if pad else y
 
 
 # --------------------------------------------------------------------------------------

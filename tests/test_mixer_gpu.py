@@ -324,3 +324,29 @@ def test_localized_large_scores_mix_fast_and_exact_paths(dev, dtype):
     qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
     O.mixer_explicit(qr, kr, vr, 1.0)[0].backward(gy.double())
     assert O.rel_l2(qd.grad, qr.grad) <= 3e-2 and O.rel_l2(kd.grad, kr.grad) <= 3e-2 and O.rel_l2(vd.grad, vr.grad) <= 3e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(2, 8, 3000, 64, 8), (1, 4, 1111, 256, 8), (1, 2, 500, 128, 4)])
+def test_narrow_heads_run_on_the_matrix_core_kernels(dev, shape, dtype):
+    """Head dims below 16 (the reference's default model has channel_dim 64 / 8 heads = 8, pdebench/__main__.py:1122-1123)
+    are zero-padded to 16: same scores, same outputs, matrix-core kernels."""
+    B, H, N, M, D = shape
+    q, k, v = make(B, H, N, M, D, dtype, seed=21)
+    x = torch.stack([k, v]).permute(0, 1, 3, 2, 4).reshape(2, B, N, H * D).contiguous().to(dev)
+    kd, vd = (t.view(B, N, H, D).permute(0, 2, 1, 3) for t in x)                # the views the modules hand over
+    assert F.mixer_kernel_name(q.to(dev), kd, vd) == ("mfma_bf16" if dtype == torch.bfloat16 else "mfma_f16")
+    mask = torch.ones(B, N, dtype=torch.bool)
+    mask[0, N // 2:] = False
+    for km in (None, mask):
+        y, z = F.flare_multihead_mixer(q.to(dev), kd, vd, scale=0.7, key_mask=None if km is None else km.to(dev), return_z=True)
+        yr, zr = O.mixer_explicit(q.float(), k.float(), v.float(), 0.7, km)
+        assert y.shape == (B, H, N, D) and z.shape == (B, H, M, D)
+        assert O.rel_l2(y, yr) <= 2e-2 and O.rel_l2(z, zr) <= 2e-2
+    # the two halves separately, and the fp32 kernels on request
+    zg, _ = F.flare_gather(q.to(dev), kd, vd, scale=0.7)
+    yg = F.flare_scatter(q.to(dev), kd, zg, scale=0.7)
+    yr, zr = O.mixer_explicit(q.float(), k.float(), v.float(), 0.7)
+    assert zg.shape == zr.shape and O.rel_l2(zg, zr) <= 2e-2 and O.rel_l2(yg, yr) <= 2e-2
+    assert F.mixer_kernel_name(q.to(dev), kd, vd, force_generic=True) == "generic"
+    assert O.rel_l2(F.flare_multihead_mixer(q.to(dev), kd, vd, scale=0.7, force_generic=True), yr) <= 2e-2

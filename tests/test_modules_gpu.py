@@ -308,3 +308,25 @@ def test_lra_block_with_rope_and_mask_against_oracle(dev):
     assert O.rel_l2(y.cpu()[keep], yo[keep]) <= 1e-5
     assert O.rel_l2(y_nomask, O.flare_block(sd, "", x.cpu(), 4, rope=O.rope_reference)) <= 1e-5
     assert O.rel_l2(y_nomask, O.flare_block(sd, "", x.cpu(), 4)) > 1e-3             # the rotation matters
+
+
+def test_default_model_geometry_uses_matrix_core_mixer(dev, monkeypatch):
+    """The reference's default model (channel_dim 64, 8 heads: head dim 8; pdebench/__main__.py:1122-1143 with 64
+    latents) under bf16 autocast: the mixer runs on the matrix-core kernels and the model matches the oracle."""
+    torch.manual_seed(6)
+    m = FLAREModel(in_dim=3, out_dim=1, channel_dim=64, num_blocks=2, num_heads=8, num_latents=64).to(dev).eval()
+    for l in m.modules():
+        if isinstance(l, torch.nn.Linear):
+            torch.nn.init.xavier_uniform_(l.weight)
+    names = []
+    real = functional._mixer_forward
+    def spy(q, k, v, *a, **kw):
+        names.append((k.shape[-1], functional.mixer_kernel_name(q, k, v)))
+        return real(q, k, v, *a, **kw)
+    monkeypatch.setattr(functional, "_mixer_forward", spy)
+    x = torch.randn(2, 3000, 3, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y = m(x)
+    assert names == [(16, "mfma_bf16")] * 2
+    ref = O.flare_model({k_: v_.cpu() for k_, v_ in m.state_dict().items()}, x.cpu(), 8, 2)
+    assert O.rel_l2(y, ref) <= 2e-2
