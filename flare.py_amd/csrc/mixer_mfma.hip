@@ -217,13 +217,14 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
     auto k_slot = [](int tok, int ch) { return tok * ROWB + ((ch ^ ((tok >> 2) & (CH - 1))) << 4); };
     auto v_slot = [](int tok, int ch) { return tok * ROWB + ((CH >= 4 ? (ch ^ (((tok >> 2) & 1) << 1)) : ch) << 4); };
 
-    // two register sets: tiles are fetched two iterations before they are consumed.  A token that is masked or
-    // lies past the range keeps a (finite) K row but gets a zero V row and a zero in the tile's row of "ones":
-    // whatever its probability, it adds nothing to the numerators or the denominators.
+    // two register sets: tiles are fetched two iterations before they are consumed.  With a key mask (MASKED) a
+    // token that is padded or lies past the range keeps a (finite) K row but gets a zero V row and a zero in the
+    // tile's row of "ones": whatever its probability, it adds nothing to the numerators or the denominators.
     u32x4 kr[2][CPT], vr[2][CPT];
     bool live[2][CPT];
-    auto load_tile = [&](auto set_tag, int n0) {
+    auto load_tile = [&](auto set_tag, int n0, auto masked_tag) {
         constexpr int S = decltype(set_tag)::value;
+        constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * 256;
@@ -231,20 +232,25 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                 const int nn = n0 + c / CH, n = min(nn, n_end - 1), ch = c % CH;
                 kr[S][i] = load16_stream(k + (int64_t)n * a.ks[2] + ch * 8);
                 vr[S][i] = load16_stream(v + (int64_t)n * a.vs[2] + ch * 8);
-                live[S][i] = nn < n_end && (mask == nullptr || mask[n] != 0);
+                if constexpr (MASKED) live[S][i] = nn < n_end && mask[n] != 0;
             }
         }
     };
-    auto store_tile = [&](auto set_tag) {   // register set S always feeds LDS buffer S
+    auto store_tile = [&](auto set_tag, auto masked_tag) {   // register set S always feeds LDS buffer S
         constexpr int S = decltype(set_tag)::value;
+        constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * 256;
             if (c < TCH) {
                 const int tok = c / CH, ch = c % CH;
                 *reinterpret_cast<u32x4*>(&kt[S][k_slot(tok, ch)]) = kr[S][i];
-                *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = live[S][i] ? to_bf16x8<T>(vr[S][i]) : zero4();
-                if (ch == 0) mt[S][tok] = live[S][i] ? uint16_t(P_::kOnes2 & 0xffffu) : uint16_t(0);
+                if constexpr (MASKED) {
+                    *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = live[S][i] ? to_bf16x8<T>(vr[S][i]) : zero4();
+                    if (ch == 0) mt[S][tok] = live[S][i] ? uint16_t(P_::kOnes2 & 0xffffu) : uint16_t(0);
+                } else {
+                    *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = to_bf16x8<T>(vr[S][i]);
+                }
             }
         }
     };
@@ -255,8 +261,10 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
     f32x4 zacc[RT][CT], lacc[CT];
 
     // one pass over the token range; EXACT keeps a running maximum per latent
-    auto run = [&](auto exact_tag) {
+    // MASKED: the problem has a key mask (decided once per launch, so the unmasked instance carries none of it)
+    auto run = [&](auto exact_tag, auto masked_tag) {
         constexpr bool EXACT = decltype(exact_tag)::value;
+        constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             shift[ct] = EXACT ? kNegBig : 0.f;
@@ -267,9 +275,23 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
         // tile i lives in LDS buffer i & 1; it is written there one iteration before its use from
         // the register set of the same parity, which was loaded two iterations before
         auto process = [&](int n0, int buf) {
-            const bool ragged = (n0 + kGTile > n_end) || (mask != nullptr);
+            const bool ragged = MASKED || (n0 + kGTile > n_end);
             auto tile = [&](auto ragged_tag) {
                 constexpr bool RAGGED = decltype(ragged_tag)::value;
+                // the optimistic pass of a masked problem runs every tile through the pipelined loop with the tile's
+                // live-token row as its row of "ones", read once per tile: lane (c16, g) meets tokens 4g..4g+3 of
+                // both 16-token sub-tiles of a k-step.  Without a mask only the one ragged tile at the end of a range
+                // leaves the pipelined loop (element-wise selects below).
+                constexpr bool PIPELINED = !EXACT && (MASKED || !RAGGED);
+                u32x4 ones_t[kGTile / 32];
+                if constexpr (PIPELINED && MASKED) {
+#pragma unroll
+                    for (int ks = 0; ks < kGTile / 32; ++ks) {
+                        const uint2 lo = *reinterpret_cast<const uint2*>(&mt[buf][ks * 32 + 4 * g]);
+                        const uint2 hi = *reinterpret_cast<const uint2*>(&mt[buf][ks * 32 + 16 + 4 * g]);
+                        ones_t[ks] = u32x4{lo.x, lo.y, hi.x, hi.y};
+                    }
+                }
 #pragma unroll
                 for (int ks = 0; ks < kGTile / 32; ++ks) {
                     // operands: two 16-token K sub-tiles (A of the score product), V^T (A of the value product)
@@ -290,16 +312,11 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                         const uint2 hi = lds_read_tr16(&vt[buf][v_slot(r1, ch) + sub]);
                         va[rt] = u32x4{lo.x, lo.y, hi.x, hi.y};
                     }
-                    if constexpr (!EXACT) {
+                    if constexpr (PIPELINED) {
                         // steady state: latent tiles software pipelined (scores of tile ct+1 issued before
-                        // the exponentials of tile ct, value product of tile ct-1 after them).  The row of ones is
-                        // the tile's live-token row when the tile is ragged or masked.
+                        // the exponentials of tile ct, value product of tile ct-1 after them)
                         u32x4 ones_a = ones8;
-                        if constexpr (RAGGED) {
-                            const uint2 lo = *reinterpret_cast<const uint2*>(&mt[buf][ks * 32 + 4 * g]);
-                            const uint2 hi = *reinterpret_cast<const uint2*>(&mt[buf][ks * 32 + 16 + 4 * g]);
-                            ones_a = u32x4{lo.x, lo.y, hi.x, hi.y};
-                        }
+                        if constexpr (MASKED) ones_a = ones_t[ks];
                         auto sc2 = [&](int ct, f32x4& s0, f32x4& s1) {
                             s0 = f32x4{0.f, 0.f, 0.f, 0.f};
                             s1 = s0;
@@ -387,15 +404,15 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
             constexpr int P = decltype(par)::value;
             using Other = std::integral_constant<int, 1 - P>;
             __syncthreads();
-            if (n0 + kGTile < n_end) store_tile(Other{});
-            if (n0 + 3 * kGTile < n_end) load_tile(Other{}, n0 + 3 * kGTile);
+            if (n0 + kGTile < n_end) store_tile(Other{}, masked_tag);
+            if (n0 + 3 * kGTile < n_end) load_tile(Other{}, n0 + 3 * kGTile, masked_tag);
             process(n0, P);
         };
         if (n_begin < n_end) {
-            load_tile(Set0{}, n_begin);
-            if (n_begin + kGTile < n_end) load_tile(Set1{}, n_begin + kGTile);
-            store_tile(Set0{});
-            if (n_begin + 2 * kGTile < n_end) load_tile(Set0{}, n_begin + 2 * kGTile);
+            load_tile(Set0{}, n_begin, masked_tag);
+            if (n_begin + kGTile < n_end) load_tile(Set1{}, n_begin + kGTile, masked_tag);
+            store_tile(Set0{}, masked_tag);
+            if (n_begin + 2 * kGTile < n_end) load_tile(Set0{}, n_begin + 2 * kGTile, masked_tag);
         }
         for (int n0 = n_begin; n0 < n_end; n0 += 2 * kGTile) {
             iter(n0, Set0{});
@@ -408,12 +425,14 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
     // range holds one (counted here; the mask and the range are uniform over the workgroup).
     bool exact;
     {
-        run(std::false_type{});
         int has_valid = n_begin < n_end;
         if (mask != nullptr) {
+            run(std::false_type{}, std::true_type{});
             int any = 0;
             for (int n = n_begin + tid; n < n_end; n += 256) any |= mask[n];
             has_valid = __syncthreads_or(any);
+        } else {
+            run(std::false_type{}, std::false_type{});
         }
         bool bad = false;
 #pragma unroll
@@ -433,7 +452,8 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
     }
     if (exact) {
         asm volatile("; exact pass" ::: "memory");
-        run(std::true_type{});
+        if (mask != nullptr) run(std::true_type{}, std::true_type{});
+        else                 run(std::true_type{}, std::false_type{});
     }
 
     // partial for this split: shift (log2 units), sum, numerator, renormalised so that the
