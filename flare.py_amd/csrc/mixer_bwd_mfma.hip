@@ -512,6 +512,7 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
 #pragma unroll
             for (int tw = 0; tw < kBTW; ++tw) {
                 f32x4 a0 = la, a1 = lb, s0 = zf, s1 = zf, g10 = da, g11 = db, g20 = zf, g21 = zf;
+                __builtin_amdgcn_s_setprio(1);      // matrix-product issue goes first, the other waves' vector work fills in behind
 #pragma unroll
                 for (int kd = 0; kd < KD; ++kd) {
                     a0 = M_::mma(q0[kd], kb[tw][kd], a0);
@@ -523,6 +524,7 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
                     g20 = Pb::mma(z0[kd], yb[tw][kd], g20);
                     g21 = Pb::mma(z1[kd], yb[tw][kd], g21);
                 }
+                __builtin_amdgcn_s_setprio(0);
                 float av[8], ds[8];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {

@@ -336,10 +336,14 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                         u32x4 pbp = zero4();
     #pragma unroll
                         for (int ct = 0; ct < CT; ++ct) {
+                            // waves that are issuing matrix products go first: the other waves' exponentials fill in behind them
+                            __builtin_amdgcn_s_setprio(1);
                             f32x4 n0 = s0, n1 = s1;
                             if (ct + 1 < CT) sc2(ct + 1, n0, n1);
                             if (ct > 0) pv(ct - 1, pbp);
                             __builtin_amdgcn_sched_barrier(0);     // matrix products first: the exponentials run under them
+                            __builtin_amdgcn_s_setprio(0);
+                            __builtin_amdgcn_sched_barrier(0);
                             const u32x4 pb = {P_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])),
                                               P_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
                                               P_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])),
@@ -601,6 +605,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                 u32x4 pbp = zero4();
 #pragma unroll
                 for (int tw = 0; tw < kSTW; ++tw) {
+                    __builtin_amdgcn_s_setprio(1);      // as in the gather: matrix-product issue takes precedence
                     f32x4 n0 = zf, n1 = zf;
                     if (tw + 1 < kSTW) {
                         n0 = scores(q0, kb[tw + 1]);
@@ -608,6 +613,8 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                     }
                     if (tw > 0) pv(tw - 1, pbp);
                     __builtin_amdgcn_sched_barrier(0);     // matrix products first: the exponentials run under them
+                    __builtin_amdgcn_s_setprio(0);
+                    __builtin_amdgcn_sched_barrier(0);
                     const u32x4 pb = {P_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])),
                                       P_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
                                       P_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])),
