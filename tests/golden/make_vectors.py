@@ -2,8 +2,9 @@
 """Writes tests/golden/vectors.json: small seeded inputs and the outputs the pure-Python brute-force
 restatements give for them (oracle.flare_oracle.mixer_bruteforce_py and the loops below, plain Python
 floats, no tensor library arithmetic).  The reference is not involved: these are frozen known answers of
-the DEFINITIONS (README.md:39-52, lra/models/backends.py:1285-1292, lra/models/triton/causal_linear.py:317-336
-of the reference, and the causal restriction of the first), against which the torch oracle, the C oracle and
+the DEFINITIONS (README.md:39-52, lra/models/backends.py:1285-1292, lra/models/triton/causal_linear.py:317-336,
+pdebench/models/flare.py:45-59 and 204-215, lra/models/embeddings.py:136-147 of the reference, and the causal
+restriction of the first), against which the torch oracle, the C oracle and
 the HIP kernels are all checked, so that none of them can drift unnoticed.
 
     python tests/golden/make_vectors.py        # rewrites vectors.json (deterministic)
@@ -91,6 +92,41 @@ def causal_linear(q, k, v):
     return out
 
 
+def mlp_stack(x, ws, bs, gamma, beta, eps, res):
+    """res + ResidualMLP(LayerNorm(x)) for rows x [T][C] (pdebench/models/flare.py:45-59 inside :204-215), all widths
+    equal so that both residual flags act: s = n + gelu(W0 n + b0); s += gelu(Wi s + bi) for the hidden layers;
+    s += W_last s + b_last; tanh-GELU."""
+    def gelu(t):
+        return 0.5 * t * (1.0 + math.tanh(math.sqrt(2.0 / math.pi) * (t + 0.044715 * t ** 3)))
+    def lin(w, b, s):
+        return [sum(w[o][i] * s[i] for i in range(len(s))) + b[o] for o in range(len(w))]
+    out = []
+    for t in range(len(x)):
+        C = len(x[t])
+        mu = sum(x[t]) / C
+        var = sum((a - mu) ** 2 for a in x[t]) / C
+        n = [(x[t][c] - mu) / math.sqrt(var + eps) * gamma[c] + beta[c] for c in range(C)]
+        h = lin(ws[0], bs[0], n)
+        s = [n[c] + gelu(h[c]) for c in range(C)]
+        for l in range(1, len(ws) - 1):
+            h = lin(ws[l], bs[l], s)
+            s = [s[c] + gelu(h[c]) for c in range(C)]
+        h = lin(ws[-1], bs[-1], s)
+        out.append([res[t][c] + s[c] + h[c] for c in range(C)])
+    return out
+
+
+def rope(x, base):
+    """lra/models/embeddings.py:136-147 for x [N][D]: rates base^-(j//2)/(D/2); partner = (-odd channels, even channels)."""
+    out = []
+    for p, row in enumerate(x):
+        D = len(row)
+        partner = [-row[2 * j + 1] for j in range(D // 2)] + [row[2 * j] for j in range(D // 2)]
+        ang = [p * base ** (-(j // 2) / (D // 2)) for j in range(D)]
+        out.append([row[j] * math.cos(ang[j]) + partner[j] * math.sin(ang[j]) for j in range(D)])
+    return out
+
+
 def main():
     rng = random.Random(20240521)
     vec = {}
@@ -104,6 +140,16 @@ def main():
     vec["triple"] = {"q1": q1, "q2": q2, "k1": k1, "k2": k2, "v": v, "state": st, "out": o}
     q, k, v = rnd(rng, 1, 10, 4), rnd(rng, 1, 10, 4), rnd(rng, 1, 10, 3)
     vec["causal_linear"] = {"q": q, "k": k, "v": v, "y": causal_linear(q, k, v)}
+    # drawn after everything above, so that the earlier vectors keep their values
+    C = 32
+    ws = [rnd(rng, C, C, std=C ** -0.5) for _ in range(3)]
+    bs = [rnd(rng, C, std=0.2) for _ in range(3)]
+    gamma, beta = [1.0 + g_ for g_ in rnd(rng, C, std=0.2)], rnd(rng, C, std=0.2)
+    x, res = rnd(rng, 3, C, std=1.5), rnd(rng, 3, C)
+    vec["mlp_stack"] = {"x": x, "w": ws, "b": bs, "gamma": gamma, "beta": beta, "eps": 1e-5, "res": res,
+                        "y": mlp_stack(x, ws, bs, gamma, beta, 1e-5, res)}
+    x = rnd(rng, 6, 8)
+    vec["rope"] = {"base": 50.0, "x": x, "y": rope(x, 50.0)}
     with open(os.path.join(HERE, "vectors.json"), "w") as f:
         json.dump(vec, f, separators=(",", ":"))
     print("wrote", os.path.join(HERE, "vectors.json"))

@@ -1,6 +1,6 @@
 """The HIP kernels (fp32, through the C-ABI) against the frozen known answers in tests/golden/vectors.json, which
 come from pure-Python-float loops over the definitions (tests/golden/make_vectors.py).  Tolerance: the fp32 bar,
-relative L2 <= 1e-5."""
+relative L2 <= 1e-5; the fused MLP launch computes in bf16 / f16 and is held to the 16-bit bar, 2e-2."""
 import json
 import os
 
@@ -52,3 +52,27 @@ def test_causal_linear(dev, g):
     c = g["causal_linear"]
     y = F.causal_linear_attention(_t(c["q"], dev).unsqueeze(0), _t(c["k"], dev).unsqueeze(0), _t(c["v"], dev).unsqueeze(0))
     assert O.rel_l2(y[0], torch.tensor(c["y"], dtype=torch.float64)) <= 1e-5
+
+
+@pytest.mark.parametrize("cd", [torch.bfloat16, torch.float16])
+def test_fused_mlp_stack(dev, g, cd):
+    """res + ResidualMLP(LayerNorm(x)) in one launch (flare_mlp_fwd) against the plain-Python known answer."""
+    from torch import nn
+    from flare_py_amd import fused
+    ms = g["mlp_stack"]
+    Cdim = len(ms["gamma"])
+    mlp = F.ResidualMLP(Cdim, Cdim, Cdim, num_layers=len(ms["w"]) - 2, input_residual=True, output_residual=True).to(dev)
+    norm = nn.LayerNorm(Cdim, eps=ms["eps"]).to(dev)
+    with torch.no_grad():
+        for lin, w, b in zip([mlp.fc1, *mlp.fcs, mlp.fc2], ms["w"], ms["b"]):
+            lin.weight.copy_(_t(w, dev))
+            lin.bias.copy_(_t(b, dev))
+        norm.weight.copy_(_t(ms["gamma"], dev))
+        norm.bias.copy_(_t(ms["beta"], dev))
+        x, res = _t(ms["x"], dev), _t(ms["res"], dev)
+        ref = torch.tensor(ms["y"], dtype=torch.float64)
+        assert O.rel_l2(res + mlp(norm(x)), ref) <= 1e-5                      # the module itself, fp32 torch layers
+        with torch.autocast("cuda", dtype=cd):
+            assert fused.compute_dtype(x, mlp) == cd
+            y = fused.fused_mlp(x, mlp, cd, norm=norm, res=res)
+    assert O.rel_l2(y, ref) <= 2e-2

@@ -322,6 +322,14 @@ def test_golden_vectors_pin_both_oracles():
     q, k, v = _t(cl["q"]).unsqueeze(0), _t(cl["k"]).unsqueeze(0), _t(cl["v"]).unsqueeze(0)
     assert O.rel_l2(O.causal_linear_recurrent(q, k, v)[0], _t(cl["y"])) < 1e-12
     assert O.rel_l2(O.causal_linear_chunked(q, k, v, chunk=4)[0], _t(cl["y"])) < 1e-12
+    ms = g["mlp_stack"]
+    y = O.residual_mlp(_t(ms["x"]), [_t(w) for w in ms["w"]], [_t(b) for b in ms["b"]], "gelu", True, True, "layer",
+                       _t(ms["gamma"]), _t(ms["beta"]), ms["eps"], _t(ms["res"]))
+    assert O.rel_l2(y, _t(ms["y"])) < 1e-12
+    rp = g["rope"]
+    assert O.rel_l2(O.rope_reference(_t(rp["x"]), rp["base"]), _t(rp["y"])) < 1e-12
+    from flare_py_amd.lra_modules import RotaryPositionalEmbeddings
+    assert O.rel_l2(RotaryPositionalEmbeddings(8, 16, base=rp["base"])(_t(rp["x"], torch.float32)[None, None])[0, 0], _t(rp["y"])) < 1e-6
 
 
 def test_golden_vectors_are_reproducible(tmp_path):
