@@ -604,20 +604,25 @@ static int mlp_fwd_impl(const FlareMlpDesc* d, int in_dim, int in_act, const flo
     if (d->norm != FLARE_NORM_NONE && !gamma) return fail(FLARE_EINVAL, "gamma must not be NULL when a norm is requested");
     if (d->norm != FLARE_NORM_NONE && !(d->eps >= 0.f)) return fail(FLARE_EINVAL, "eps must be >= 0");
     if (in_dim < 0 || in_dim > 4 || out_dim < 0 || out_dim > 4) return fail(FLARE_EINVAL, "in_dim and out_dim must be in [0, 4] (got %d, %d)", in_dim, out_dim);
-    if ((in_dim || out_dim) && (d->flags & FLARE_MLP_EXPAND)) return fail(FLARE_EINVAL, "FLARE_MLP_EXPAND cannot be combined with in_dim / out_dim");
+    const int x_head = 4 * ((d->flags >> 8) & 15), y_head = 4 * ((d->flags >> 12) & 15);
+    if ((in_dim || out_dim || x_head || y_head) && (d->flags & FLARE_MLP_EXPAND))
+        return fail(FLARE_EINVAL, "FLARE_MLP_EXPAND cannot be combined with in_dim / out_dim / head-padded rows");
+    if ((x_head || y_head) && (x_head > 8 || y_head > 8 || in_dim || out_dim))
+        return fail(FLARE_EINVAL, "head-padded rows need a head dim of 4 or 8 and cannot be combined with in_dim / out_dim");
+    const int64_t x_width = x_head ? 16 * (int64_t)(d->C / x_head) : d->C, y_width = y_head ? 16 * (int64_t)(d->C / y_head) : d->C;
     if (in_dim) {
         if (!w_in || !b_in || !aligned16(w_in) || !aligned16(b_in)) return fail(FLARE_EINVAL, "w_in and b_in must be 16-byte aligned and not NULL when in_dim > 0");
         if (d->norm != FLARE_NORM_NONE) return fail(FLARE_EINVAL, "no norm in front of a lifting first layer");
         if (d->x_stride < in_dim) return fail(FLARE_EINVAL, "x_stride must be >= in_dim");
     } else {
         // every lane moves 4 consecutive elements at a time
-        if (d->x_stride < d->C || d->x_stride % 4 || !aligned16(x)) return fail(FLARE_EINVAL, "x: row stride >= C, a multiple of 4, base 16-byte aligned");
+        if (d->x_stride < x_width || d->x_stride % 4 || !aligned16(x)) return fail(FLARE_EINVAL, "x: row stride >= the row width, a multiple of 4, base 16-byte aligned");
     }
     if (out_dim) {
         if (res) return fail(FLARE_EINVAL, "res must be NULL when out_dim > 0");
         if (d->y_stride < out_dim) return fail(FLARE_EINVAL, "y_stride must be >= out_dim");
     } else {
-        if (d->y_stride < d->C || d->y_stride % 4 || !aligned16(y)) return fail(FLARE_EINVAL, "y: row stride >= C, a multiple of 4, base 16-byte aligned");
+        if (d->y_stride < y_width || d->y_stride % 4 || !aligned16(y)) return fail(FLARE_EINVAL, "y: row stride >= the row width, a multiple of 4, base 16-byte aligned");
     }
     if (res && (d->res_stride < d->C || d->res_stride % 4 || !aligned16(res))) return fail(FLARE_EINVAL, "res: row stride >= C, a multiple of 4, base 16-byte aligned");
     if (!aligned16(w) || (bias && !aligned16(bias)) || (gamma && !aligned16(gamma)) || (beta && !aligned16(beta)))
@@ -634,6 +639,7 @@ static int mlp_fwd_impl(const FlareMlpDesc* d, int in_dim, int in_act, const flo
         a.act_mask = (d->act_mask & 1u) ? 0x55555555u : 0u;      // the activation follows every first product
     }
     a.in_dim = in_dim; a.in_act = in_act ? 1 : 0; a.w_in = w_in; a.b_in = b_in; a.out_dim = out_dim;
+    a.x_head = x_head; a.y_head = y_head;
     a.xs = d->x_stride; a.rs = d->res_stride; a.ys = d->y_stride;
     return hip_status(flare::launch_mlp_mfma(a, d->w_dtype, static_cast<hipStream_t>(stream)), "mlp launch");
 }

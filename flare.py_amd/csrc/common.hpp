@@ -144,6 +144,7 @@ struct MlpArgs {
     const float* b_in;
     int in_act;                                 // the lifting layer is followed by the activation
     int out_dim;                                // > 0: only features [0, out_dim <= 4) of the result are stored, y rows are out_dim wide
+    int x_head, y_head;                         // > 0: rows of x / y hold heads of x_head / y_head (4 or 8) channels, each padded to 16 columns
     int64_t xs, rs, ys;                         // row strides in elements
 };
 

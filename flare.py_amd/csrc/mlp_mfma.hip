@@ -14,6 +14,9 @@
 // stream that the C x C chain continues from (ResidualMLP(in_dim, C, C, ...), the models' input projection).
 // Projecting mode (a.out_dim > 0): the last tile has only out_dim <= 4 real rows (the rest are zero) and only those
 // outputs are stored, y rows being out_dim wide (ResidualMLP(C, C, out_dim, ...), the models' output projection).
+// Head-padded rows (a.x_head / a.y_head > 0, an instance of their own): the C channels of a row are H heads of fewer
+// than 16 channels and each head occupies 16 columns, the layout the mixer's matrix-core kernels read and write
+// for narrow heads -- the projections write it and the output projection reads it, so nothing is copied between.
 //
 // Layout.  The product is taken transposed, S'^T = W S^T, with v_mfma_f32_16x16x32: A = W tile
 // (lane = output row, 8 consecutive input features per lane), B = S^T (lane = token c16, k-slots =
@@ -113,7 +116,8 @@ __device__ __forceinline__ float silu_gate(float x)
     return __builtin_amdgcn_rcpf(1.f + fast_exp2(-kLog2e * x));
 }
 
-// MODE: 0 the C x C chain, 1 the expanding two-layer MLP, 2 the chain with a narrow first input and/or last output
+// MODE: 0 the C x C chain, 1 the expanding two-layer MLP, 2 the chain with a narrow first input and/or last output,
+// 3 the chain with head-padded rows on either end
 template <typename T, int C, int TW, int WAVES, int MODE>
 __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kernel(MlpArgs a, int resident)
 {
@@ -219,6 +223,14 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
                     }
                 }
             }
+        } else if (MODE == 3 && a.x_head > 0) {
+            // head-padded rows: channel f = 16 ft + 4 g of the row sits at column 16 (f / x_head) + f % x_head,
+            // which is ft * 32 + 8 g - 4 (g & 1) for heads of 8 and ft * 64 + 16 g for heads of 4
+            const int cf = a.x_head == 8 ? 32 : 64, c0 = a.x_head == 8 ? 8 * g - 4 * (g & 1) : 16 * g;
+#pragma unroll
+            for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft) xs[ft][tw] = load4(a.x, tok[tw] * a.xs + ft * cf + c0, a.x_dtype);
         } else {
 #pragma unroll
             for (int tw = 0; tw < TW; ++tw)
@@ -419,6 +431,22 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
                     }
                 continue;
             }
+            if (MODE == 3 && a.y_head > 0) {
+                // head-padded rows (columns as for x above): each head's channels, then zeros up to 16 columns,
+                // written by the lane that holds the head's last four channels
+                const int cf = a.y_head == 8 ? 32 : 64, c0 = a.y_head == 8 ? 8 * g - 4 * (g & 1) : 16 * g;
+                const int nz = a.y_head == 8 ? ((g & 1) ? 2 : 0) : 3;        // groups of 4 zero columns behind this lane's channels
+                const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft) {
+                    f32x4 o = xs[ft][tw];
+                    if (a.res) o += load4(a.res, tok[tw] * a.rs + 16 * ft + 4 * g, a.res_dtype);
+                    const int64_t col = tok[tw] * a.ys + ft * cf + c0;
+                    store4(a.y, col, a.y_dtype, o);
+                    for (int z = 1; z <= nz; ++z) store4(a.y, col + 4 * z, a.y_dtype, zero);
+                }
+                continue;
+            }
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
                 f32x4 o = xs[ft][tw];
@@ -459,6 +487,7 @@ hipError_t launch_ct(const MlpArgs& a, hipStream_t st)
 {
     if (a.expand) return launch_cte<T, C, TW, WAVES, 1>(a, st);
     if (a.in_dim > 0 || a.out_dim > 0) return launch_cte<T, C, TW, WAVES, 2>(a, st);
+    if (a.x_head > 0 || a.y_head > 0) return launch_cte<T, C, TW, WAVES, 3>(a, st);
     return launch_cte<T, C, TW, WAVES, 0>(a, st);
 }
 

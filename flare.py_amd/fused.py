@@ -216,9 +216,11 @@ def _norm_args(d, norm, x, Cdim):
     return gamma, beta
 
 
-def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None):
+def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None, x_head=0, y_head=0):
     """y = res + mod(norm(x)) in one HIP launch.  x: [..., C]; mod: ResidualMLP or nn.Linear; cd: the
-    dtype from compute_dtype(); norm: nn.LayerNorm / nn.RMSNorm / None; res: [..., C] or None."""
+    dtype from compute_dtype(); norm: nn.LayerNorm / nn.RMSNorm / None; res: [..., C] or None.
+    x_head / y_head (4 or 8): x is / y comes back head-padded, [..., (C / head) * 16] with every head's channels
+    followed by zeros up to 16 columns -- the layout the mixer reads and writes for head dims below 16."""
     lib = _lib.load()
     info = _layers_of(mod)
     layers, act_mask, add_mask, act = info
@@ -226,24 +228,29 @@ def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None):
     if io is not None and (io[1] or io[2]):
         y = _fused_mlp_io(x, mod, cd, io, info, norm, out_dtype)
         return y if res is None else res + y
-    Cdim = x.shape[-1]
+    Cdim = layers[0].in_features
+    if x.shape[-1] != (Cdim // x_head * 16 if x_head else Cdim):
+        raise ValueError(f"x rows are {x.shape[-1]} wide, expected {Cdim // x_head * 16 if x_head else Cdim}")
     E = _expand_factor(mod, Cdim)
     if E:
+        if x_head or y_head:
+            raise ValueError("head-padded rows are not available for the expanding two-layer MLP")
         w, b = _packed_expand(mod, E, cd)
         act_mask, add_mask = 1, 0
     else:
         w, b = _packed(mod, layers, cd)
-    x2 = x.reshape(-1, Cdim)
+    x2 = x.reshape(-1, x.shape[-1])
     if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 16:
         x2 = x2.contiguous()
     out_dtype = x.dtype if out_dtype is None else out_dtype
-    y = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    ywidth = Cdim // y_head * 16 if y_head else Cdim
+    y = torch.empty(*x.shape[:-1], ywidth, dtype=out_dtype, device=x.device)
     d = _lib.FlareMlpDesc()
     d.T, d.C, d.L = x2.shape[0], Cdim, w.shape[0]
-    d.flags = _lib.MLP_EXPAND if E else 0
+    d.flags = (_lib.MLP_EXPAND if E else 0) | ((x_head // 4) << 8) | ((y_head // 4) << 12)
     d.w_dtype, d.x_dtype, d.y_dtype = _dtype_code(w), _dtype_code(x2), _dtype_code(y)
     d.act, d.act_mask, d.add_mask = act, act_mask, add_mask
-    d.x_stride, d.y_stride = x2.stride(0), Cdim
+    d.x_stride, d.y_stride = x2.stride(0), ywidth
     gamma, beta = _norm_args(d, norm, x, Cdim)
     r2 = None
     if res is not None:

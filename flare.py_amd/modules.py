@@ -116,6 +116,18 @@ class FLARE(nn.Module):
         B, N, C = x.shape
         q = self.latent_q.view(self.num_heads, self.num_latents, self.head_dim)
         cd = self._fusable(x, return_scores)
+        D = self.head_dim
+        if cd is not None and D in (4, 8) and self.num_latents % 64 == 0 and not self.qk_norm:
+            # narrow heads: the projections write k, v head-padded to 16 columns, which is what the mixer's
+            # matrix-core kernels take, and the output projection reads the mixer's padded rows: no copies between
+            H = self.num_heads
+            k = fused.fused_mlp(x, self.k_proj, cd, norm=_norm, out_dtype=cd, y_head=D).view(B, N, H, 16).permute(0, 2, 1, 3)
+            v = fused.fused_mlp(x, self.v_proj, cd, norm=_norm, out_dtype=cd, y_head=D).view(B, N, H, 16).permute(0, 2, 1, 3)
+            q16 = torch.nn.functional.pad(q, (0, 16 - D))
+            y = flare_multihead_mixer(q16, k, v, scale=self.attn_scale, token_major_out=True)
+            y = y.permute(0, 2, 1, 3).reshape(B, N, H * 16)          # a view: the kernel laid y out as [B,N,H,16]
+            out_dtype = _res.dtype if _res is not None else x.dtype
+            return fused.fused_mlp(y, self.out_proj, cd, res=_res, out_dtype=out_dtype, x_head=D), None
         if cd is not None:
             k = self._heads(fused.fused_mlp(x, self.k_proj, cd, norm=_norm, out_dtype=cd))
             v = self._heads(fused.fused_mlp(x, self.v_proj, cd, norm=_norm, out_dtype=cd))

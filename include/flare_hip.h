@@ -244,7 +244,13 @@ int flare_mlp_fwd(const FlareMlpDesc* desc, const void* x, const void* w, const 
  *   from; norm must be FLARE_NORM_NONE.  in_dim == 0: x rows are C wide as in flare_mlp_fwd.
  * out_dim > 0: only outputs [0, out_dim <= 4) of the last tile are stored (its other rows should be
  *   zero), y rows are out_dim wide (y_stride >= out_dim) and res must be NULL.  out_dim == 0: C wide.
+ * Head-padded rows: FLARE_MLP_X_HEAD(h) / FLARE_MLP_Y_HEAD(h) in desc->flags (h = 4 or 8) say that
+ *   the C channels of an x / y row are C/h heads of h channels and that each head occupies 16 columns of the row
+ *   (channel f at column 16 (f / h) + f % h; x_stride / y_stride >= 16 C / h; stored pad columns are zeros).  This
+ *   is the [B, N, H, 16] layout the mixer uses for head dims below 16.  Not combinable with in_dim / out_dim.  flare_mlp_fwd accepts these two flags as well.
  * FLARE_MLP_EXPAND is not accepted here. */
+#define FLARE_MLP_X_HEAD(h) (((h) / 4) << 8)
+#define FLARE_MLP_Y_HEAD(h) (((h) / 4) << 12)
 int flare_mlp_io_fwd(const FlareMlpDesc* desc, int32_t in_dim, int32_t in_act, const float* w_in,
                      const float* b_in, int32_t out_dim, const void* x, const void* w, const float* bias,
                      const float* gamma, const float* beta, const void* res, void* y, void* stream);

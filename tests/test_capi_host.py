@@ -153,6 +153,14 @@ def test_new_struct_sizes_and_entry_point_validation():
     assert io(0, 2, fake) == _lib.FLARE_EINVAL and "res must be NULL" in _lib.last_error()
     m.x_stride = 2
     assert io(3, 0) == _lib.FLARE_EINVAL and "x_stride" in _lib.last_error()
+    # head-padded rows: head dims 4 and 8 only, not next to in_dim / out_dim, and rows wide enough for the padding
+    m.x_stride = 128
+    m.flags = (12 // 4) << 8
+    assert lib.flare_mlp_fwd(m, fake, fake, None, fake, None, None, fake, None) == _lib.FLARE_EINVAL and "head dim" in _lib.last_error()
+    m.flags = (8 // 4) << 12
+    assert io(3, 0) == _lib.FLARE_EINVAL and "head dim" in _lib.last_error()
+    assert lib.flare_mlp_fwd(m, fake, fake, None, fake, None, None, fake, None) == _lib.FLARE_EINVAL and "row width" in _lib.last_error()
+    m.flags = 0
     # causal linear attention
     c = _lib.FlareCausalLinearDesc()
     c.B, c.H, c.N, c.Dk, c.Dv, c.dtype = 1, 2, 100, 32, 16, _lib.DT_F32

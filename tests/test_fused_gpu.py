@@ -298,3 +298,30 @@ def test_cfg2_full_size_fused_vs_fp32_layers(dev):
     assert O.rel_l2(y, ref) <= 2e-2
     idx = torch.randint(0, 65536, (64,), device=dev)
     assert O.rel_l2(h[2, idx], _narrow_oracle(lift, pts[2, idx], cd)) <= 2e-2
+
+
+@pytest.mark.parametrize("C,hd", [(64, 8), (32, 4), (128, 8), (32, 8)])
+def test_head_padded_rows(dev, C, hd):
+    """Rows whose heads of hd < 16 channels are padded to 16 columns (the layout the mixer takes for narrow heads):
+    written by one launch (pad columns are zeros), read back by another, against the oracle on plain rows."""
+    H = C // hd
+    m = make_mlp(C, 2, True, True, "gelu", dev, seed=C + hd)
+    norm = nn.LayerNorm(C).to(dev)
+    x = torch.randn(2, 301, C, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        cd = fused.compute_dtype(x, m)
+        yp = fused.fused_mlp(x, m, cd, norm=norm, out_dtype=cd, y_head=hd)
+        y = fused.fused_mlp(x, m, cd, norm=norm, out_dtype=cd)
+    assert yp.shape == (2, 301, H * 16)
+    yp4 = yp.view(2, 301, H, 16)
+    assert torch.equal(yp4[..., :hd].reshape(2, 301, C), y) and (yp4[..., hd:] == 0).all()
+    assert O.rel_l2(y, oracle_of(m, x, cd, norm)) <= 2e-2
+    # reading padded rows: a single Linear with a residual, fed the padded tensor
+    lin = nn.Linear(C, C).to(dev)
+    res = torch.randn(2, 301, C, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        out_p = fused.fused_mlp(yp, lin, cd, res=res, out_dtype=torch.float32, x_head=hd)
+        out = fused.fused_mlp(y, lin, cd, res=res, out_dtype=torch.float32)
+    assert torch.equal(out_p, out)
+    with pytest.raises(ValueError):
+        fused.fused_mlp(y, lin, cd, x_head=hd)                    # plain rows where padded ones are announced
