@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
     __shared__ int wg_flag[4];
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
-    const int mblocks = a.M / MB;
+    const int mblocks = (a.M + MB - 1) / MB;      // M % 64 == 32: the last block's waves 2, 3 own no latent and only help stage
     const int split = blockIdx.x / mblocks, mb = blockIdx.x % mblocks;
     const int h = blockIdx.y, b = blockIdx.z;
 
@@ -198,9 +198,9 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd) {
             const int ch = kd * 4 + g;
-            qb[ct][kd] = ch < CH ? scale8<T>(load16(q + (int64_t)(m_base + ct * 16 + c16) * a.qs[2] + ch * 8),
-                                             a.scale_log2)
-                                 : zero4();
+            qb[ct][kd] = ch < CH && m_base + ct * 16 < a.M
+                             ? scale8<T>(load16(q + (int64_t)(m_base + ct * 16 + c16) * a.qs[2] + ch * 8), a.scale_log2)
+                             : zero4();
         }
     const u32x4 ones8 = {P_::kOnes2, P_::kOnes2, P_::kOnes2, P_::kOnes2};
 
@@ -469,6 +469,7 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
         if (l > 0.f) (void)frexpf(l, &e);
         const float sc = l > 0.f ? ldexpf(1.f, -e) : 0.f;
         const int m = m_base + ct * 16 + c16;
+        if (m >= a.M) continue;
         const int64_t row = (((int64_t)b * a.H + h) * a.n_parts + split) * a.M + m;
         if (g == 0) {
             a.part_m[row] = l > 0.f ? shift[ct] + (float)e : kNegBig;
@@ -786,7 +787,7 @@ template <typename T, int D>
 hipError_t gather_launch_ct(const MixerArgs& a, hipStream_t st)
 {
     const int MB = (a.M % 256 == 0) ? 256 : (a.M % 128 == 0) ? 128 : 64;
-    dim3 grid(a.n_splits * (a.M / MB), a.H, a.B);
+    dim3 grid(a.n_splits * ((a.M + MB - 1) / MB), a.H, a.B);
     if (MB == 256)      hipLaunchKernelGGL((gather_mfma_kernel<T, D, 4>), grid, dim3(256), 0, st, a);
     else if (MB == 128) hipLaunchKernelGGL((gather_mfma_kernel<T, D, 2>), grid, dim3(256), 0, st, a);
     else                hipLaunchKernelGGL((gather_mfma_kernel<T, D, 1>), grid, dim3(256), 0, st, a);
@@ -879,7 +880,7 @@ bool mfma_mixer_supported(int dtype, int M, int D)
 {
     if (dtype != 1 && dtype != 2) return false;
     if (D != 16 && D != 32 && D != 64) return false;
-    if (M < 64 || M % 64 != 0) return false;
+    if (M < 32 || M % 32 != 0) return false;      // the scatter walks the latents 32 at a time, the gather pads its last block
     if ((size_t)M * D * 4 > kScatterLdsMax) return false;
     return true;
 }

@@ -271,7 +271,7 @@ def _narrow_head_pad(q, k, force_generic) -> int:
     D = k.shape[-1]
     if force_generic or D >= 16 or k.dtype not in (torch.bfloat16, torch.float16) or k.device.type != "cuda":
         return 0
-    return 16 - D if q.shape[-2] % 64 == 0 else 0
+    return 16 - D if q.shape[-2] % 32 == 0 else 0
 
 
 def _pad_last(t, n):

@@ -350,3 +350,24 @@ def test_narrow_heads_run_on_the_matrix_core_kernels(dev, shape, dtype):
     assert zg.shape == zr.shape and O.rel_l2(zg, zr) <= 2e-2 and O.rel_l2(yg, yr) <= 2e-2
     assert F.mixer_kernel_name(q.to(dev), kd, vd, force_generic=True) == "generic"
     assert O.rel_l2(F.flare_multihead_mixer(q.to(dev), kd, vd, scale=0.7, force_generic=True), yr) <= 2e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(2, 2, 3000, 32, 32), (1, 3, 1500, 96, 16), (1, 2, 700, 160, 64), (2, 4, 2000, 32, 8)])
+def test_latent_counts_that_are_odd_multiples_of_32(dev, shape, dtype):
+    """M = 32 is the FLARE layer's own default (pdebench/models/flare.py:68): the gather pads its last 64-latent block
+    with waves that own no latent, the scatter walks the latents 32 at a time."""
+    B, H, N, M, D = shape
+    q, k, v = make(B, H, N, M, D, dtype, seed=31)
+    assert F.mixer_kernel_name(q.to(dev), k.to(dev), v.to(dev)).startswith("mfma")
+    mask = torch.ones(B, N, dtype=torch.bool)
+    mask[0, N // 3:] = False
+    for km in (None, mask):
+        y, z = F.flare_multihead_mixer(q.to(dev), k.to(dev), v.to(dev), scale=0.9, key_mask=None if km is None else km.to(dev),
+                                       return_z=True)
+        yr, zr = O.mixer_explicit(q.float(), k.float(), v.float(), 0.9, km)
+        assert z.shape == zr.shape and O.rel_l2(z, zr) <= 2e-2 and O.rel_l2(y, yr) <= 2e-2
+    # gradients for these latent counts come from the torch recomputation (the HIP backward wants M % 64 == 0)
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    F.flare_multihead_mixer(qd, kd, vd, scale=0.9).sum().backward()
+    assert torch.isfinite(qd.grad).all() and torch.isfinite(kd.grad).all() and torch.isfinite(vd.grad).all()
