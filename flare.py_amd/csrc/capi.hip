@@ -399,7 +399,7 @@ BwdPlan plan_bwd(const FlareMixerDesc* d)
 {
     BwdPlan p;
     const int64_t bh = (int64_t)d->B * d->H;
-    const int mblocks = d->M % 256 == 0 ? d->M / 256 : d->M % 128 == 0 ? d->M / 128 : d->M / 64;
+    const int mblocks = d->M % 256 == 0 ? d->M / 256 : d->M % 128 == 0 ? d->M / 128 : (d->M + 63) / 64;
     // about two workgroups per compute unit over the latent-side grids, token ranges of 64 k tokens
     int64_t s = std::max<int64_t>(1, 512 / (bh * mblocks));
     int64_t tps = ((int64_t)d->N + s - 1) / s;
@@ -419,7 +419,7 @@ int check_bwd(const FlareMixerDesc* d)
     int rc = check_mixer_desc(d);
     if (rc != FLARE_OK) return rc;
     if (!flare::mixer_bwd_supported(d->dtype, d->M, d->D))
-        return fail(FLARE_EUNSUPPORTED, "mixer backward covers bf16/f16, D in {16,32,64}, M %% 64 == 0, 5*M*D*2 + 8*M <= 150 KB of LDS "
+        return fail(FLARE_EUNSUPPORTED, "mixer backward covers bf16/f16, D in {16,32,64}, M %% 32 == 0, 5*M*D*2 + 8*M <= 150 KB of LDS "
                                         "(got dtype %d, M=%d, D=%d)", d->dtype, d->M, d->D);
     if (!strides_mult8(d->q_stride) || !strides_mult8(d->k_stride) || !strides_mult8(d->v_stride) || !strides_mult8(d->y_stride))
         return fail(FLARE_EUNSUPPORTED, "mixer backward needs strides that are multiples of 8 elements");

@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
     __shared__ __attribute__((aligned(16))) float tsc[2][2][kBTile];   // per-token scalars of a tile: -rho * log2(e), -delta
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
-    const int mblocks = a.M / MB;
+    const int mblocks = (a.M + MB - 1) / MB;     // M % 64 == 32: waves 2, 3 of the last block own no latent, they only help stage
     const int split = blockIdx.x / mblocks, mb = blockIdx.x % mblocks;
     const int h = blockIdx.y, b = blockIdx.z;
     const int64_t bh = (int64_t)b * a.H + h;
@@ -163,18 +163,20 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         const int m = m_base + ct * 16 + c16;
+        const bool own = m_base + ct * 16 < a.M;       // uniform over the wave
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd) {
             const int ch = kd * 4 + g;
-            qb[ct][kd] = ch < CH ? scale8<T>(load16(q + (int64_t)m * a.qs[2] + ch * 8), a.scale_log2) : zero4();
+            const bool in = own && ch < CH;
+            qb[ct][kd] = in ? scale8<T>(load16(q + (int64_t)m * a.qs[2] + ch * 8), a.scale_log2) : zero4();
             if (MODE == 1) {
-                dzb[ct][kd] = ch < CH ? pack8(a.dz + (bh * a.M + m) * D + ch * 8) : zero4();
-                zb[ct][kd] = ch < CH ? pack8(a.z + (bh * a.M + m) * D + ch * 8) : zero4();
+                dzb[ct][kd] = in ? pack8(a.dz + (bh * a.M + m) * D + ch * 8) : zero4();
+                zb[ct][kd] = in ? pack8(a.z + (bh * a.M + m) * D + ch * 8) : zero4();
             }
         }
         if (MODE == 1) {
-            l2m[ct] = a.lse_lat[bh * a.M + m] * kLog2e;
-            dm[ct] = a.delta_lat[bh * a.M + m];
+            l2m[ct] = own ? a.lse_lat[bh * a.M + m] * kLog2e : 0.f;
+            dm[ct] = own ? a.delta_lat[bh * a.M + m] : 0.f;
             if constexpr (kFoldLat) {
                 nl4[ct] = f32x4{-l2m[ct], -l2m[ct], -l2m[ct], -l2m[ct]};
                 nd4[ct] = f32x4{-dm[ct], -dm[ct], -dm[ct], -dm[ct]};
@@ -355,6 +357,7 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         const int m = m_base + ct * 16 + c16;
+        if (m >= a.M) continue;
         const int64_t row = ((int64_t)bh * a.n_splits + split) * a.M + m;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) *reinterpret_cast<f32x4*>(a.part + row * D + rt * 16 + 4 * g) = acc[rt][ct];
@@ -578,7 +581,7 @@ hipError_t lat_launch(const MixerBwdArgs& a, hipStream_t st)
     } else if (a.M % 128 == 0) {
         hipLaunchKernelGGL((bwd_lat_kernel<T, D, 2, MODE>), dim3(a.n_splits * (a.M / 128), a.H, a.B), dim3(256), 0, st, a);
     } else {
-        hipLaunchKernelGGL((bwd_lat_kernel<T, D, 1, MODE>), dim3(a.n_splits * (a.M / 64), a.H, a.B), dim3(256), 0, st, a);
+        hipLaunchKernelGGL((bwd_lat_kernel<T, D, 1, MODE>), dim3(a.n_splits * ((a.M + 63) / 64), a.H, a.B), dim3(256), 0, st, a);
     }
     return hipGetLastError();
 }
@@ -624,7 +627,7 @@ size_t mixer_bwd_lds_bytes(int M, int D) { return (size_t)M * D * 2 * 5 + (size_
 
 bool mixer_bwd_supported(int dtype, int M, int D)
 {
-    return (dtype == 1 || dtype == 2) && (D == 16 || D == 32 || D == 64) && M >= 64 && M % 64 == 0 &&
+    return (dtype == 1 || dtype == 2) && (D == 16 || D == 32 || D == 64) && M >= 32 && M % 32 == 0 &&
            mixer_bwd_lds_bytes(M, D) <= 150 * 1024;
 }
 
