@@ -20,9 +20,10 @@ from .functional import (
     triple_attention,
 )
 from .modules import FLARE, FLAREBlock, FLAREModel, FinalLayer, ResidualMLP
+from .serving import GraphedForward
 
 __all__ = [
     "CausalLinear", "causal_linear_attention", "FLARE", "FLAREBlock", "FLAREModel", "FinalLayer", "ResidualMLP", "TripleAttentionFunction",
     "causal_fresh_state", "flare_causal_decode", "flare_causal_decode_step", "flare_causal_prefill",
-    "flare_gather", "flare_multihead_mixer", "flare_scatter", "mixer_kernel_name", "triple_attention",
+    "flare_gather", "flare_multihead_mixer", "flare_scatter", "mixer_kernel_name", "triple_attention", "GraphedForward",
 ]

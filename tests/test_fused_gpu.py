@@ -325,3 +325,55 @@ def test_head_padded_rows(dev, C, hd):
     assert torch.equal(out_p, out)
     with pytest.raises(ValueError):
         fused.fused_mlp(y, lin, cd, x_head=hd)                    # plain rows where padded ones are announced
+
+
+def test_block_forward_replays_from_a_hip_graph(dev):
+    """A serving loop captures the fused block forward (7 launches, no host round trips) once and replays it: every
+    replay, with new input written into the static buffer and eager work in between, must equal the eager result."""
+    torch.manual_seed(8)
+    blk = F.FLAREBlock(channel_dim=64, num_heads=8, num_latents=64).to(dev).eval()        # head dim 8: padded-row path
+    blk2 = F.FLAREBlock(channel_dim=128, num_heads=8, num_latents=128, num_layers_ffn=0, ffn_mlp_ratio=4.0).to(dev).eval()
+    for b, C in ((blk, 64), (blk2, 128)):
+        static_x = torch.randn(2, 4096, C, device=dev)
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+            s = torch.cuda.Stream()
+            s.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(s):
+                for _ in range(3):
+                    b(static_x)                                  # warm-up: weight packing, kernel attributes
+            torch.cuda.current_stream().wait_stream(s)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_y = b(static_x)[0]
+            for i in range(3):
+                x = torch.randn(2, 4096, C, device=dev) * (1.0 + i)
+                eager = b(x)[0]
+                static_x.copy_(x)
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(static_y, eager), i
+
+
+def test_graphed_forward_helper(dev):
+    """serving.GraphedForward: one capture per input shape, replays equal the eager forward, reset() recaptures."""
+    torch.manual_seed(9)
+    model = F.FLAREModel(in_dim=3, out_dim=2, channel_dim=64, num_blocks=2, num_heads=8, num_latents=64).to(dev).eval()
+    fwd = F.GraphedForward(model, autocast_dtype=torch.bfloat16)
+    for shape in ((1, 2000, 3), (2, 777, 3), (1, 2000, 3)):
+        for i in range(2):
+            x = torch.randn(*shape, device=dev) * (1 + i)
+            with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+                eager = model(x)
+            assert torch.equal(fwd(x), eager)
+    assert len(fwd._graphs) == 2
+    with torch.no_grad():
+        model.out_proj[1].fc2.bias.add_(1.0)
+    fwd.reset()
+    x = torch.randn(1, 2000, 3, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        assert torch.equal(fwd(x), model(x))
+    with pytest.raises(ValueError):
+        fwd(torch.randn(1, 10, 3))
+    model.train()
+    with pytest.raises(RuntimeError):
+        fwd(torch.randn(1, 11, 3, device=dev))
