@@ -241,13 +241,13 @@ __global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kerne
         if (a.norm != 0) {
 #pragma unroll
             for (int tw = 0; tw < TW; ++tw) {
-                float mean = 0.f;
-                if (a.norm == 1) {
-                    float s = 0.f;
+                // the row sum is taken for both norms and dropped for RMSNorm: straight-line code (with the sum
+                // under a branch, the one-token-tile instances of this kernel came out wrong for RMSNorm)
+                float s = 0.f;
 #pragma unroll
-                    for (int ft = 0; ft < FT; ++ft) s += xs[ft][tw][0] + xs[ft][tw][1] + xs[ft][tw][2] + xs[ft][tw][3];
-                    mean = xg_sum(s) * (1.f / C);
-                }
+                for (int ft = 0; ft < FT; ++ft) s += xs[ft][tw][0] + xs[ft][tw][1] + xs[ft][tw][2] + xs[ft][tw][3];
+                const float rowmean = xg_sum(s) * (1.f / C);
+                const float mean = a.norm == 1 ? rowmean : 0.f;
                 float ss = 0.f;
 #pragma unroll
                 for (int ft = 0; ft < FT; ++ft)
@@ -494,10 +494,14 @@ hipError_t launch_ct(const MlpArgs& a, hipStream_t st)
 template <typename T>
 hipError_t launch_t(const MlpArgs& a, hipStream_t st)
 {
+    // Few tokens: workgroups of 16 tokens per wave instead of 64 (32 at C = 128), four times as many of them.
+    // Each one then re-reads its weight operands from LDS for every product, which costs throughput that a
+    // launch too small to fill the chip does not need, and the layers' latency chain gets 4x (2x) shorter.
+    const bool few = a.T < 32768;
     switch (a.C) {
-        case 32:  return launch_ct<T, 32, 4, 4>(a, st);
-        case 64:  return launch_ct<T, 64, 4, 4>(a, st);
-        case 128: return launch_ct<T, 128, 2, 8>(a, st);
+        case 32:  return few ? launch_ct<T, 32, 1, 4>(a, st) : launch_ct<T, 32, 4, 4>(a, st);
+        case 64:  return few ? launch_ct<T, 64, 1, 4>(a, st) : launch_ct<T, 64, 4, 4>(a, st);
+        case 128: return few ? launch_ct<T, 128, 1, 8>(a, st) : launch_ct<T, 128, 2, 8>(a, st);
         default:  return hipErrorInvalidValue;
     }
 }

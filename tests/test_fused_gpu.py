@@ -377,3 +377,41 @@ def test_graphed_forward_helper(dev):
     model.train()
     with pytest.raises(RuntimeError):
         fwd(torch.randn(1, 11, 3, device=dev))
+
+
+@pytest.mark.parametrize("C", [32, 64, 128])
+def test_many_token_instances_of_every_mode(dev, C):
+    """Launches of fewer than 32768 tokens take kernel instances with one 16-token tile per wave; this test feeds the
+    many-token instances (4 tiles per wave, 2 at C = 128) of every mode: chain with both norms, expanding MLP,
+    narrow ends, head-padded rows."""
+    T = 40000
+    x = torch.randn(T, C, device=dev) * 1.5 + 0.3
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        for kind in ("layer", "rms", None):
+            m = make_mlp(C, 2, True, True, "gelu" if kind != "rms" else "silu", dev, seed=C)
+            norm = None if kind is None else (nn.LayerNorm(C) if kind == "layer" else nn.RMSNorm(C, eps=1e-6)).to(dev)
+            if norm is not None:
+                nn.init.normal_(norm.weight, 1.0, 0.3)
+            y = fused.fused_mlp(x, m, torch.bfloat16, norm=norm, res=x)
+            assert O.rel_l2(y, oracle_of(m, x, torch.bfloat16, norm, x)) <= 2e-2, kind
+        # expanding two-layer MLP
+        torch.manual_seed(C)
+        e = F.ResidualMLP(C, 4 * C, C, num_layers=0, act="gelu", input_residual=True, output_residual=True).to(dev)
+        assert fused.compute_dtype(x, e) == torch.bfloat16
+        ye = fused.fused_mlp(x, e, torch.bfloat16)
+        w1, w2 = e.fc1.weight.bfloat16().double().cpu(), e.fc2.weight.bfloat16().double().cpu()
+        h = O.gelu_tanh(x.double().cpu() @ w1.T + e.fc1.bias.double().cpu())
+        assert O.rel_l2(ye, h @ w2.T + e.fc2.bias.double().cpu()) <= 2e-2
+        # narrow ends
+        lift = _narrow_mlp(3, C, C, 1, False, True, "gelu", dev, seed=C)
+        pts = torch.randn(T, 3, device=dev)
+        assert O.rel_l2(fused.fused_mlp(pts, lift, torch.bfloat16), _narrow_oracle(lift, pts, torch.bfloat16)) <= 2e-2
+        proj = _narrow_mlp(C, C, 2, 1, True, False, "gelu", dev, seed=C + 1)
+        assert O.rel_l2(fused.fused_mlp(x, proj, torch.bfloat16), _narrow_oracle(proj, x, torch.bfloat16)) <= 2e-2
+        # head-padded rows out and back in
+        m = make_mlp(C, 1, True, True, "gelu", dev, seed=C + 2)
+        yp = fused.fused_mlp(x, m, torch.bfloat16, out_dtype=torch.bfloat16, y_head=8)
+        y = fused.fused_mlp(x, m, torch.bfloat16, out_dtype=torch.bfloat16)
+        assert torch.equal(yp.view(T, C // 8, 16)[..., :8].reshape(T, C), y) and (yp.view(T, C // 8, 16)[..., 8:] == 0).all()
+        lin = nn.Linear(C, C).to(dev)
+        assert torch.equal(fused.fused_mlp(yp, lin, torch.bfloat16, x_head=8), fused.fused_mlp(y, lin, torch.bfloat16))
