@@ -103,6 +103,18 @@ class FLARE(nn.Module):
         B, N, _ = t.shape
         return t.view(B, N, self.num_heads, self.head_dim).permute(0, 2, 1, 3)  # [B,H,N,D] view, no copy
 
+    def _cached_q(self, cd, pad):
+        """latent_q as [H, M, D + pad] in the compute dtype for the inference fast path, rebuilt when the parameter
+        changes (saves a cast, a fill and a copy per call, which is most of a small launch-bound forward)."""
+        key = (self.latent_q._version, self.latent_q.data_ptr(), cd, pad)
+        c = getattr(self, "_q_cache", None)
+        if c is None or c[0] != key:
+            q = self.latent_q.detach().view(self.num_heads, self.num_latents, self.head_dim).to(cd)
+            if pad:
+                q = torch.nn.functional.pad(q, (0, pad))
+            c = self._q_cache = (key, q.contiguous())
+        return c[1]
+
     def _fusable(self, x, return_scores):
         """The 16-bit dtype for the fused projections, or None."""
         if return_scores:
@@ -123,8 +135,7 @@ class FLARE(nn.Module):
             H = self.num_heads
             k = fused.fused_mlp(x, self.k_proj, cd, norm=_norm, out_dtype=cd, y_head=D).view(B, N, H, 16).permute(0, 2, 1, 3)
             v = fused.fused_mlp(x, self.v_proj, cd, norm=_norm, out_dtype=cd, y_head=D).view(B, N, H, 16).permute(0, 2, 1, 3)
-            q16 = torch.nn.functional.pad(q, (0, 16 - D))
-            y = flare_multihead_mixer(q16, k, v, scale=self.attn_scale, token_major_out=True)
+            y = flare_multihead_mixer(self._cached_q(cd, 16 - D), k, v, scale=self.attn_scale, token_major_out=True)
             y = y.permute(0, 2, 1, 3).reshape(B, N, H * 16)          # a view: the kernel laid y out as [B,N,H,16]
             out_dtype = _res.dtype if _res is not None else x.dtype
             return fused.fused_mlp(y, self.out_proj, cd, res=_res, out_dtype=out_dtype, x_head=D), None
@@ -134,6 +145,8 @@ class FLARE(nn.Module):
             if self.qk_norm:
                 q = self.q_norm(q)
                 k = self.k_norm(k)
+            else:
+                q = self._cached_q(cd, 0)
             y = flare_multihead_mixer(q, k, v, scale=self.attn_scale, token_major_out=True)
             y = y.permute(0, 2, 1, 3).reshape(B, N, C)
             out_dtype = _res.dtype if _res is not None else x.dtype

@@ -415,3 +415,26 @@ def test_many_token_instances_of_every_mode(dev, C):
         assert torch.equal(yp.view(T, C // 8, 16)[..., :8].reshape(T, C), y) and (yp.view(T, C // 8, 16)[..., 8:] == 0).all()
         lin = nn.Linear(C, C).to(dev)
         assert torch.equal(fused.fused_mlp(yp, lin, torch.bfloat16, x_head=8), fused.fused_mlp(y, lin, torch.bfloat16))
+
+
+@pytest.mark.parametrize("C,H", [(64, 8), (64, 4)])
+def test_cached_operands_follow_parameter_updates(dev, C, H):
+    """The fast path caches 16-bit copies of the weights and of latent_q on the modules; an in-place update of a
+    parameter (an optimiser step, load_state_dict) must show in the next forward."""
+    import copy
+    torch.manual_seed(10)
+    blk = F.FLAREBlock(channel_dim=C, num_heads=H, num_latents=64).to(dev).eval()
+    x = torch.randn(1, 1000, C, device=dev)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y0 = blk(x)[0]
+        blk.att.latent_q.mul_(3.0)
+        blk.mlp.fc1.weight.add_(0.05)
+        blk.att.out_proj.bias.add_(0.5)
+        y1 = blk(x)[0]
+        fresh = copy.deepcopy(blk)
+        for mod in fresh.modules():
+            for name in ("_q_cache", "_flare_packed"):
+                if hasattr(mod, name):
+                    delattr(mod, name)
+        y2 = fresh(x)[0]
+    assert not torch.equal(y0, y1) and torch.equal(y1, y2)
