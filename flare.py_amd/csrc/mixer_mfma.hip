@@ -829,7 +829,7 @@ hipError_t scatter_launch(const MixerArgs& a, hipStream_t st)
     const int64_t per_bh = (slots + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H);   // workgroups per (b,h)
     int64_t tpw = (a.N + per_bh - 1) / per_bh;
     tpw = ((tpw + 255) / 256) * 256;
-    if (tpw < 1024) tpw = 1024;
+    if (tpw < 256) tpw = 256;       // one 64-token pass per wave: a launch this small is bound by latency, not by the operand set-up
     dim3 grid((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, a, (int)tpw);
     return hipGetLastError();

@@ -2,7 +2,7 @@
 
 A FLARE model forward on the inference fast path is a fixed sequence of HIP launches (7 per block) with no host
 round trip, so on small point clouds its cost is the launches themselves: an 8-block model at N = 4096 takes
-1.50 ms eagerly and 0.42 ms replayed from a HIP graph.  `GraphedForward` captures that sequence once per input
+1.48 ms eagerly and 0.38 ms replayed from a HIP graph.  `GraphedForward` captures that sequence once per input
 shape and replays it; there is no tracing compiler behind it and nothing is specialised beyond the shapes.
 
     fwd = GraphedForward(model, autocast_dtype=torch.bfloat16)
