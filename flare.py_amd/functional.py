@@ -63,8 +63,33 @@ def _q4(q: torch.Tensor, B: int) -> torch.Tensor:
     return q
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(dev) -> int:
+    """The HIP stream torch would launch on for this device (every launch of the library goes there)."""
+    if _raw_stream is not None:          # the same handle without building a torch.cuda.Stream object per call
+        idx = dev.index if isinstance(dev, torch.device) else dev
+        return _raw_stream(torch.cuda.current_device() if idx is None else idx)
     return torch.cuda.current_stream(dev).cuda_stream
+
+
+class _NoGuard:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def _on_device(dev):
+    """Context that makes dev the current HIP device for a launch; free when it already is."""
+    if dev.index is None or dev.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(dev)
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -151,14 +176,14 @@ def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_majo
     if want_lse:
         lse_lat = torch.empty((B, H, M), dtype=torch.float32, device=k.device)
         lse_tok = torch.empty((B, H, N), dtype=torch.float32, device=k.device)
-        with torch.cuda.device(k.device):
+        with _on_device(k.device):
             rc = lib.flare_gather_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(mask), _ptr(z), _ptr(lse_lat),
                                       _ptr(ws), ws.numel(), st)
             _lib.check(rc, "flare_gather_fwd")
             rc = lib.flare_scatter_fwd_lse(C.byref(d), _ptr(q4), _ptr(k), _ptr(z), _ptr(mask), _ptr(y), _ptr(lse_tok), st)
         _lib.check(rc, "flare_scatter_fwd_lse")
         return y, z, lse_lat, lse_tok
-    with torch.cuda.device(k.device):
+    with _on_device(k.device):
         rc = lib.flare_mixer_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(mask), _ptr(y), _ptr(z),
                                  _ptr(ws), ws.numel(), st)
     _lib.check(rc, "flare_mixer_fwd")
@@ -196,7 +221,7 @@ def _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy):
     need = C.c_size_t(0)
     _lib.check(lib.flare_mixer_bwd_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_bwd_workspace_bytes")
     ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
-    with torch.cuda.device(k.device):
+    with _on_device(k.device):
         rc = lib.flare_mixer_bwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(y), _ptr(z), _ptr(lse_lat), _ptr(lse_tok),
                                  _ptr(gy), _s3(gy), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws.numel(),
                                  C.c_void_p(_stream_ptr(k.device)))
@@ -324,7 +349,7 @@ def _gather_forward(q, k, v, scale, key_mask, n_splits, force_generic):
     need = C.c_size_t(0)
     _lib.check(lib.flare_mixer_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_workspace_bytes")
     ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
-    with torch.cuda.device(k.device):
+    with _on_device(k.device):
         rc = lib.flare_gather_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(mask), _ptr(z), _ptr(lse),
                                   _ptr(ws), ws.numel(), C.c_void_p(_stream_ptr(k.device)))
     _lib.check(rc, "flare_gather_fwd")
@@ -347,7 +372,7 @@ def _scatter_forward(q, k, z, scale, key_mask, force_generic):
     y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
     mask = _mask_u8(key_mask, B, N, k.device)
     d = _mixer_desc(q4, k, None, y, scale, 0, force_generic)
-    with torch.cuda.device(k.device):
+    with _on_device(k.device):
         rc = lib.flare_scatter_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(z), _ptr(mask), _ptr(y),
                                    C.c_void_p(_stream_ptr(k.device)))
     _lib.check(rc, "flare_scatter_fwd")
@@ -469,7 +494,7 @@ def _causal_call(entry, q, k, v, scale, chunk, state):
     d.chunk = int(chunk)
     d.q_stride, d.k_stride, d.v_stride, d.y_stride = _s3(q4), _s3(k), _s3(v), _s3(y)
     st = C.c_void_p(_stream_ptr(k.device))
-    with torch.cuda.device(k.device):
+    with _on_device(k.device):
         need = C.c_size_t(0)
         _lib.check(lib.flare_causal_workspace_bytes(C.byref(d), C.byref(need)), "flare_causal_workspace_bytes")
         ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
@@ -523,7 +548,7 @@ def _causal_linear_forward(q, k, v, n_segs: int = 0):
     d.dtype = _dtype_code(q)
     d.n_segs = int(n_segs)
     d.q_stride, d.k_stride, d.v_stride, d.y_stride = _s3(q), _s3(k), _s3(v), _s3(y)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         need = C.c_size_t(0)
         _lib.check(lib.flare_causal_linear_workspace_bytes(C.byref(d), C.byref(need)),
                    "flare_causal_linear_workspace_bytes")
@@ -609,7 +634,7 @@ def _triple_forward(q1, q2, k1, k2, v, feature_map: bool, normalize: bool, n_spl
     need = C.c_size_t(0)
     _lib.check(lib.flare_triple_workspace_bytes(C.byref(d), C.byref(need)), "flare_triple_workspace_bytes")
     ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=q1.device)
-    with torch.cuda.device(q1.device):
+    with _on_device(q1.device):
         rc = lib.flare_triple_fwd(C.byref(d), _ptr(q1), _ptr(q2), _ptr(k1), _ptr(k2), _ptr(v), _ptr(state),
                                   _ptr(out), _ptr(ws), ws.numel(), C.c_void_p(_stream_ptr(q1.device)))
     _lib.check(rc, "flare_triple_fwd")
@@ -638,7 +663,7 @@ def _triple_state(k1, k2, v):
     need = C.c_size_t(0)
     _lib.check(lib.flare_triple_workspace_bytes(C.byref(d), C.byref(need)), "flare_triple_workspace_bytes")
     ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k1.device)
-    with torch.cuda.device(k1.device):
+    with _on_device(k1.device):
         rc = lib.flare_triple_state_fwd(C.byref(d), _ptr(k1), _ptr(k2), _ptr(v), _ptr(state), None, _ptr(ws), ws.numel(),
                                         C.c_void_p(_stream_ptr(k1.device)))
     _lib.check(rc, "flare_triple_state_fwd")
@@ -653,7 +678,7 @@ def _triple_out(q1, q2, state):
     B, H, N, Dq = q1.shape
     out = torch.empty((B, H, N, state.shape[3]), dtype=q1.dtype, device=q1.device)
     d = _triple_desc(q1, q2, out, out)
-    with torch.cuda.device(q1.device):
+    with _on_device(q1.device):
         rc = lib.flare_triple_out_fwd(C.byref(d), _ptr(q1), _ptr(q2), _ptr(state), None, _ptr(out),
                                       C.c_void_p(_stream_ptr(q1.device)))
     _lib.check(rc, "flare_triple_out_fwd")

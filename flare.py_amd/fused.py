@@ -25,14 +25,24 @@ import torch
 from torch import nn
 
 from . import _lib
-from .functional import _autocast_dtype, _dtype_code, _ptr, _stream_ptr
+from .functional import _autocast_dtype, _dtype_code, _on_device, _ptr, _stream_ptr
 
 _SUPPORTED_C = (32, 64, 128)
 _ACTS = {"gelu": 0, "silu": 1}
 
 
 def _layers_of(mod):
-    """(linear layers, act_mask, add_mask, act code) of a ResidualMLP or nn.Linear, or None."""
+    """(linear layers, act_mask, add_mask, act code) of a ResidualMLP or nn.Linear, or None.  The structure of a
+    module does not change after construction: the answer is kept on the module."""
+    cached = mod.__dict__.get("_flare_layers")
+    if cached is not None:
+        return cached[0]
+    info = _layers_of_uncached(mod)
+    mod.__dict__["_flare_layers"] = (info,)
+    return info
+
+
+def _layers_of_uncached(mod):
     if isinstance(mod, nn.Linear):
         return [mod], 0, 0, 0
     if getattr(mod, "num_layers", None) is None:
@@ -192,7 +202,7 @@ def _fused_mlp_io(x, mod, cd, io, info, norm, out_dtype):
     d.act, d.act_mask, d.add_mask = act, act_mask, add_mask
     d.x_stride, d.y_stride = x2.stride(0), yw
     gamma, beta = _norm_args(d, norm, x, Cdim)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.flare_mlp_io_fwd(C.byref(d), in_dim, in_act, _ptr(w_in), _ptr(b_in), out_dim, _ptr(x2), _ptr(w), _ptr(b),
                                   _ptr(gamma), _ptr(beta), None, _ptr(y), C.c_void_p(_stream_ptr(x.device)))
     _lib.check(rc, "flare_mlp_io_fwd")
@@ -258,7 +268,7 @@ def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None, x_head=0, y_head=
         if r2.stride(-1) != 1 or r2.stride(0) % 4 or r2.data_ptr() % 16:
             r2 = r2.contiguous()
         d.res_dtype, d.res_stride = _dtype_code(r2), r2.stride(0)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         rc = lib.flare_mlp_fwd(C.byref(d), _ptr(x2), _ptr(w), _ptr(b), _ptr(gamma), _ptr(beta), _ptr(r2), _ptr(y),
                                C.c_void_p(_stream_ptr(x.device)))
     _lib.check(rc, "flare_mlp_fwd")
