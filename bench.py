@@ -253,6 +253,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--cpu-sample", type=int, default=1048576, help="tokens of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-torch-sdpa", action="store_true", help="skip timing torch's own SDPA formulation on the GPU")
     ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train"], default="mixer",
                     help="mixer = the headline configuration (default); the others are BASELINE configs 4, 5, 2")
     args = ap.parse_args()
@@ -326,6 +327,27 @@ def main():
                    "kernel": kernel, "scale": 1.0, "seed": 0},
         "roofline": roofline,
     }
+
+    # ---- the reference's formulation on this GPU: y = SDPA(k, q, SDPA(q, k, v)) through torch's own fused
+    # attention (README.md:49-50 of the reference; torch library kernels, no reference code involved) ----
+    if not args.no_torch_sdpa:
+        try:
+            import torch.nn.functional as TF
+            qe = q.unsqueeze(0).expand(B, -1, -1, -1)
+            def sdpa_step():
+                z = TF.scaled_dot_product_attention(qe, k, v, scale=1.0)
+                return TF.scaled_dot_product_attention(k, qe, z, scale=1.0)
+            y_t = sdpa_step()
+            ms_t = time_events(sdpa_step, 5, 2)
+            y_h = step()
+            out["torch_sdpa_same_gpu"] = {
+                "ms_per_step": round(ms_t, 3), "speedup": round(ms_t / ms_step, 1),
+                "rel_l2_hip_vs_torch": float((y_h.float() - y_t.float()).norm() / y_t.float().norm()),
+                "what": "two torch scaled_dot_product_attention calls in bf16 on the same device and inputs",
+            }
+            del y_t, y_h
+        except Exception as e:      # a backend that refuses the shape must not cost the bench line
+            out["torch_sdpa_same_gpu"] = {"error": f"{type(e).__name__}: {str(e)[:160]}"}
 
     # ---- CPU baseline on a bounded sample + parity of the HIP path on the same sample ----
     if not args.no_cpu:
