@@ -7,14 +7,16 @@ One step = one forward of the mixer (split-N gather, merge, scatter) over the he
 B=1, H=8, N=1,048,576, M=256, D=32, bf16 in / fp32 accumulate, inputs resident in HBM.
 Prints ONE JSON line: tokens/s, the roofline of the dominant kernel (measured with HIP events
 on the launch stream), and the CPU baseline (torch SDPA, MATH backend, fp32) timed on this
-machine's host cores on a bounded sample of the same workload.  Before the W warm-up steps the step is
+machine's host cores on a bounded sample of the same workload; `torch_sdpa_same_gpu` is the same forward written as
+two torch scaled_dot_product_attention calls (the formulation of the reference) timed on this GPU for orientation.
+Before the W warm-up steps the step is
 called until at least 40 untimed calls have been made in all: a freshly started process runs its first ~30 ms
 of GPU work about 7 % slower than the steady state.
 
 --workload selects one of the other configurations instead (same JSON shape, one line): causal =
 causal FLARE prefill of 8192 tokens + 256 decode steps at B=8,H=16,M=128,D=64; triple = triple
-attention at B=4,H=8,N=16384,D=16 (elu+1, normalised); block = one FLAREBlock forward at
-B=4,N=65536,C=128,H=8,M=128 under bf16 autocast (fused HIP launches around the HIP mixer); train =
+attention at B=4,H=8,N=16384,D=16 (elu+1, normalised); block = lift MLP 3 -> 128 and one FLAREBlock forward with a
+4x GELU MLP at B=4,N=65536,C=128,H=8,M=128 under bf16 autocast (fused HIP launches around the HIP mixer); train =
 the headline configuration with the backward pass (HIP kernels both ways).
 """
 from __future__ import annotations
