@@ -202,6 +202,28 @@ def bench_train(args, F, dev):
                        "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / (ms_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                        "traffic": None, "algorithmic_flops": flops, "algorithmic_bytes": nbytes,
                        "frac_of_roofline_time": round(t_roof * 1e3 / ms_step, 4), "ms_forward_only": round(ms_fwd, 4)}
+    # the reference's formulation with autograd through torch's fused attention, same device and inputs
+    try:
+        import torch.nn.functional as TF
+
+        def sdpa_step():
+            qe = qd.unsqueeze(0).expand(B, -1, -1, -1)
+            z = TF.scaled_dot_product_attention(qe, kd, vd, scale=1.0)
+            TF.scaled_dot_product_attention(kd, qe, z, scale=1.0).backward(gy)
+            grads = (qd.grad, kd.grad, vd.grad)
+            qd.grad = kd.grad = vd.grad = None
+            return grads
+
+        ref = sdpa_step()
+        ms_t = time_events(sdpa_step, 3, 1)
+        F.flare_multihead_mixer(qd, kd, vd).backward(gy)
+        rel = [float((a.float() - b.float()).norm() / b.float().norm()) for a, b in zip((qd.grad, kd.grad, vd.grad), ref)]
+        qd.grad = kd.grad = vd.grad = None
+        out["torch_sdpa_same_gpu"] = {"ms_per_step": round(ms_t, 2), "speedup": round(ms_t / ms_step, 1),
+                                      "rel_l2_hip_vs_torch_dq_dk_dv": [round(r, 5) for r in rel],
+                                      "what": "forward + backward through two torch scaled_dot_product_attention calls, bf16"}
+    except Exception as e:
+        out["torch_sdpa_same_gpu"] = {"error": f"{type(e).__name__}: {str(e)[:160]}"}
     return out
 
 
