@@ -36,6 +36,10 @@ HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 
+class _Skip(Exception):
+    """--no-torch-sdpa: leave out the legs that time torch's own formulation on the GPU."""
+
+
 def make_inputs(B, H, N, M, D, dtype, device, seed=0):
     g = torch.Generator(device="cpu").manual_seed(seed)
     q = (torch.randn(H, M, D, generator=g) * D ** -0.5).to(dtype)
@@ -167,6 +171,24 @@ def bench_triple(args, F, dev):
                        "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                        "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "algorithmic_bytes": nbytes,
                        "ms_events": round(ms_ev, 4)}
+    # the reference's einsum formulation (lra/models/backends.py:1288-1291: state, then output; k1, k2, v carry
+    # N^-1/3 each) through torch on the same device, elu+1 features applied first, without the normaliser
+    try:
+        if args.no_torch_sdpa:
+            raise _Skip()
+        def einsum_step():
+            q1, q2, k1, k2 = (torch.nn.functional.elu(t) + 1 for t in a[:4])
+            sc = N ** (-1.0 / 3.0)
+            state = torch.einsum("bhni,bhnj,bhnk->bhijk", k1.float() * sc, a[4].float() * sc, k2.float() * sc)
+            return torch.einsum("bhni,bhijk,bhnk->bhnj", q1.float(), state, q2.float()).to(a[4].dtype)
+        einsum_step()
+        ms_t = time_events(einsum_step, 5, 2)
+        out["torch_einsum_same_gpu"] = {"ms_per_step": round(ms_t, 3), "speedup": round(ms_t / ms_step, 1),
+                                        "what": "elu+1 and the two einsums of the reference in torch on the same device (no normaliser)"}
+    except _Skip:
+        pass
+    except Exception as e:
+        out["torch_einsum_same_gpu"] = {"error": f"{type(e).__name__}: {str(e)[:160]}"}
     if not args.no_cpu:
         c = [t.float().cpu() for t in a]
         t0 = time.perf_counter()
@@ -204,6 +226,8 @@ def bench_train(args, F, dev):
                        "frac_of_roofline_time": round(t_roof * 1e3 / ms_step, 4), "ms_forward_only": round(ms_fwd, 4)}
     # the reference's formulation with autograd through torch's fused attention, same device and inputs
     try:
+        if args.no_torch_sdpa:
+            raise _Skip()
         import torch.nn.functional as TF
 
         def sdpa_step():
@@ -222,6 +246,8 @@ def bench_train(args, F, dev):
         out["torch_sdpa_same_gpu"] = {"ms_per_step": round(ms_t, 2), "speedup": round(ms_t / ms_step, 1),
                                       "rel_l2_hip_vs_torch_dq_dk_dv": [round(r, 5) for r in rel],
                                       "what": "forward + backward through two torch scaled_dot_product_attention calls, bf16"}
+    except _Skip:
+        pass
     except Exception as e:
         out["torch_sdpa_same_gpu"] = {"error": f"{type(e).__name__}: {str(e)[:160]}"}
     return out
@@ -267,6 +293,36 @@ def bench_block(args, F, dev):
                        "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "algorithmic_bytes": nbytes,
                        "ms_mixer": round(ms_mixer, 4), "ms_block": round(ms_step, 4)}
     out["ms_block_default_ffn_no_lift"] = round(ms_default, 4)
+    # the same modules the way the reference runs them on this device: torch Linear / LayerNorm layers under the
+    # same autocast, the mixer as two torch scaled_dot_product_attention calls (pdebench/models/flare.py:122-156)
+    try:
+        if args.no_torch_sdpa:
+            raise _Skip()
+        import torch.nn.functional as TF
+        from flare_py_amd import modules as Mod
+
+        def sdpa_mixer(q_, k_, v_, scale=1.0, **kw):
+            qe = q_.unsqueeze(0).expand(k_.size(0), -1, -1, -1)
+            return TF.scaled_dot_product_attention(k_, qe, TF.scaled_dot_product_attention(qe, k_, v_, scale=scale), scale=scale)
+
+        real_cd, real_mix = fused.compute_dtype, Mod.flare_multihead_mixer
+        fused.compute_dtype, Mod.flare_multihead_mixer = (lambda *a, **k: None), sdpa_mixer
+        try:
+            def torch_step():
+                with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+                    return blk(lift(pts))
+            y_t = torch_step()[0]
+            ms_t = time_events(torch_step, 10, 3)
+        finally:
+            fused.compute_dtype, Mod.flare_multihead_mixer = real_cd, real_mix
+        y_h = step()[0]
+        out["torch_layers_same_gpu"] = {"ms_per_step": round(ms_t, 3), "speedup": round(ms_t / ms_step, 1),
+                                        "rel_l2_hip_vs_torch": float((y_h.float() - y_t.float()).norm() / y_t.float().norm()),
+                                        "what": "the same lift MLP and block as torch layers with two fused SDPA calls, same autocast"}
+    except _Skip:
+        pass
+    except Exception as e:
+        out["torch_layers_same_gpu"] = {"error": f"{type(e).__name__}: {str(e)[:160]}"}
     return out
 
 
@@ -277,7 +333,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--cpu-sample", type=int, default=1048576, help="tokens of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-torch-sdpa", action="store_true", help="skip timing torch's own SDPA formulation on the GPU")
+    ap.add_argument("--no-torch-sdpa", action="store_true", help="skip the legs that time torch's own formulation (fused SDPA, einsum, torch layers) on the GPU")
     ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train"], default="mixer",
                     help="mixer = the headline configuration (default); the others are BASELINE configs 4, 5, 2")
     args = ap.parse_args()
