@@ -71,7 +71,7 @@ MixerPlan plan_mixer(const FlareMixerDesc* d, bool want_mfma)
     MixerPlan p;
     p.mfma = want_mfma;
     const int unit = p.mfma ? flare::mfma_gather_tokens_per_iter() : 32;
-    const int mblk = p.mfma ? ((d->M % 256 == 0) ? d->M / 256 : (d->M % 128 == 0) ? d->M / 128 : (d->M + 63) / 64)
+    const int mblk = p.mfma ? ((d->M % 256 == 0 && d->D <= 32) ? d->M / 256 : (d->M % 128 == 0) ? d->M / 128 : (d->M + 63) / 64)
                             : (d->M + 63) / 64;
     int s = d->n_splits;
     if (s <= 0) {

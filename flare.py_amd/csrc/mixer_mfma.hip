@@ -484,8 +484,9 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
 // =====================================================================================
 // scatter
 // =====================================================================================
-constexpr int kSTW = 4;             // 16-token column tiles per wave iteration
-constexpr int kSTokWave = 16 * kSTW;
+// 16-token column tiles per wave iteration: 4, and 2 at D = 64, where the accumulators and K operands of 4
+// tiles do not fit the register file (84 registers spilled, and twice the time per score)
+constexpr int scatter_tiles(int D) { return D <= 32 ? 4 : 2; }
 
 // One workgroup = 4 independent waves sharing Q and Z^T operands in LDS; wave w walks the
 // workgroup's token range in steps of 64 tokens.  No barrier after the set-up.
@@ -500,6 +501,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
     constexpr int KD = (D + 31) / 32;
     constexpr int RT = D / 16;
     constexpr int CH = D / 8;
+    constexpr int kSTW = scatter_tiles(D), kSTokWave = 16 * kSTW;
     using M_ = Mma<T>;          // score product, in the element type of q and k
     using P_ = Mma<bf16_t>;     // value product: probabilities (and the values they meet) are always bf16
 
@@ -768,7 +770,9 @@ constexpr size_t kScatterLdsMax = 150 * 1024;
 template <typename T, int D>
 const void* gather_kernel_ptr(int M)
 {
-    if (M % 256 == 0) return reinterpret_cast<const void*>(gather_mfma_kernel<T, D, 4>);
+    if constexpr (D <= 32) {
+        if (M % 256 == 0) return reinterpret_cast<const void*>(gather_mfma_kernel<T, D, 4>);
+    }
     if (M % 128 == 0) return reinterpret_cast<const void*>(gather_mfma_kernel<T, D, 2>);
     return reinterpret_cast<const void*>(gather_mfma_kernel<T, D, 1>);
 }
@@ -786,11 +790,17 @@ const void* gather_kernel_ptr_d(int M, int D)
 template <typename T, int D>
 hipError_t gather_launch_ct(const MixerArgs& a, hipStream_t st)
 {
-    const int MB = (a.M % 256 == 0) ? 256 : (a.M % 128 == 0) ? 128 : 64;
+    // 64 latents per wave only up to D = 32: at D = 64 that instance spills 445 registers
+    const int MB = (a.M % 256 == 0 && D <= 32) ? 256 : (a.M % 128 == 0) ? 128 : 64;
     dim3 grid(a.n_splits * ((a.M + MB - 1) / MB), a.H, a.B);
-    if (MB == 256)      hipLaunchKernelGGL((gather_mfma_kernel<T, D, 4>), grid, dim3(256), 0, st, a);
-    else if (MB == 128) hipLaunchKernelGGL((gather_mfma_kernel<T, D, 2>), grid, dim3(256), 0, st, a);
-    else                hipLaunchKernelGGL((gather_mfma_kernel<T, D, 1>), grid, dim3(256), 0, st, a);
+    if constexpr (D <= 32) {
+        if (MB == 256) {
+            hipLaunchKernelGGL((gather_mfma_kernel<T, D, 4>), grid, dim3(256), 0, st, a);
+            return hipGetLastError();
+        }
+    }
+    if (MB == 128) hipLaunchKernelGGL((gather_mfma_kernel<T, D, 2>), grid, dim3(256), 0, st, a);
+    else           hipLaunchKernelGGL((gather_mfma_kernel<T, D, 1>), grid, dim3(256), 0, st, a);
     return hipGetLastError();
 }
 
