@@ -419,7 +419,7 @@ int check_bwd(const FlareMixerDesc* d)
     int rc = check_mixer_desc(d);
     if (rc != FLARE_OK) return rc;
     if (!flare::mixer_bwd_supported(d->dtype, d->M, d->D))
-        return fail(FLARE_EUNSUPPORTED, "mixer backward covers bf16/f16, D in {16,32,64}, M %% 32 == 0, 5*M*D*2 + 8*M <= 150 KB of LDS "
+        return fail(FLARE_EUNSUPPORTED, "mixer backward covers bf16/f16, D in {16,32,64}, M %% 32 == 0, M*D <= 65536 "
                                         "(got dtype %d, M=%d, D=%d)", d->dtype, d->M, d->D);
     if (!strides_mult8(d->q_stride) || !strides_mult8(d->k_stride) || !strides_mult8(d->v_stride) || !strides_mult8(d->y_stride))
         return fail(FLARE_EUNSUPPORTED, "mixer backward needs strides that are multiples of 8 elements");

@@ -115,6 +115,7 @@ struct MixerBwdArgs {
     int n_splits, tokens_per_split;
     float scale, scale_log2;
     int64_t qs[3], ks[3], vs[3], ys[3], dys[3], dks[3], dvs[3];
+    int m0, mc, accumulate;  // token-side kernel only: latents [m0, m0 + mc) of the M (mc = 0: all), added to dk, dv when accumulate
 };
 
 struct CausalLinearArgs {
@@ -170,6 +171,7 @@ hipError_t launch_causal_mfma(const CausalArgs& a, int dtype, int step, hipStrea
 hipError_t launch_causal_decode_steps(const CausalArgs& a, int dtype, hipStream_t st);      // N one-token steps, same shapes as above
 
 size_t     mixer_bwd_lds_bytes(int M, int D);
+int        mixer_bwd_tok_chunks(int M, int D);
 bool       mixer_bwd_supported(int dtype, int M, int D);
 hipError_t launch_mixer_bwd(const MixerBwdArgs& a, int dtype, hipStream_t st);
 

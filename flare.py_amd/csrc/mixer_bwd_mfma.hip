@@ -408,7 +408,9 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
     constexpr int kBTW = D <= 32 ? 4 : 2;   // 16-token column tiles per wave iteration (registers allow 2 at D = 64)
     using M_ = Mb<T>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    const int M = a.M, KS = M / 32;
+    // M here is the chunk of latents this launch covers: when the five operand sets of all latents exceed the LDS,
+    // the launch is repeated over chunks and every launch after the first adds to dk, dv
+    const int M = a.mc > 0 ? a.mc : a.M, KS = M / 32;
     // A-operand layout [mt][ch][c16] for q (scaled, log2 units), dz, z;  PV-operand layout
     // [ks][rt][lane] for dz^T and (scale q)^T;  per-latent scalars
     u32x4* qa = reinterpret_cast<u32x4*>(smem);
@@ -416,20 +418,22 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
     u32x4* zza = dza + (size_t)M * CH;
     u32x4* dzt = zza + (size_t)M * CH;
     u32x4* qt = dzt + (size_t)M * CH;
-    float* l2 = reinterpret_cast<float*>(qt + (size_t)M * CH);
-    float* dl = l2 + M;
+    // the per-latent scalars (log-sum-exp, Delta) stay in global memory: the five operand sets may then take all
+    // 160 KB of LDS (M = 256 at D = 64, M = 512 at D = 32)
+    const float* lse_lat = a.lse_lat + ((int64_t)blockIdx.z * a.H + blockIdx.y) * a.M + a.m0;
+    const float* delta_lat = a.delta_lat + ((int64_t)blockIdx.z * a.H + blockIdx.y) * a.M + a.m0;
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
     const int h = blockIdx.y, b = blockIdx.z;
     const int64_t bh = (int64_t)b * a.H + h;
-    const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
+    const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1] + (int64_t)a.m0 * a.qs[2];
     const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
     const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
     const uint16_t* dy = (const uint16_t*)a.dy + b * a.dys[0] + h * a.dys[1];
     uint16_t* dk = (uint16_t*)a.dk + b * a.dks[0] + h * a.dks[1];
     uint16_t* dv = (uint16_t*)a.dv + b * a.dvs[0] + h * a.dvs[1];
-    const float* z = a.z + bh * M * D;
-    const float* dz = a.dz + bh * M * D;
+    const float* z = a.z + (bh * a.M + a.m0) * D;
+    const float* dz = a.dz + (bh * a.M + a.m0) * D;
     const float* rho = a.lse_tok + bh * a.N;
     const float* dlt = a.delta_tok + bh * a.N;
 
@@ -454,10 +458,6 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
         }
         dzt[idx] = o1;
         qt[idx] = o2;
-    }
-    for (int m = tid; m < M; m += NTH) {
-        l2[m] = -a.lse_lat[bh * M + m] * kLog2e;     // negated: they start the accumulators below
-        dl[m] = -a.delta_lat[bh * M + m];
     }
     __syncthreads();
 
@@ -510,8 +510,10 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
             }
             // negated per-latent scalars of the 8 latents (rows) this lane holds: -L_m log2(e) and -Delta_m
             // start the accumulators of S and <dz, v>, so neither is subtracted element by element
-            const f32x4 la = *reinterpret_cast<const f32x4*>(l2 + 32 * ks + 4 * g), lb = *reinterpret_cast<const f32x4*>(l2 + 32 * ks + 16 + 4 * g);
-            const f32x4 da = *reinterpret_cast<const f32x4*>(dl + 32 * ks + 4 * g), db = *reinterpret_cast<const f32x4*>(dl + 32 * ks + 16 + 4 * g);
+            const f32x4 la = *reinterpret_cast<const f32x4*>(lse_lat + 32 * ks + 4 * g) * -kLog2e;
+            const f32x4 lb = *reinterpret_cast<const f32x4*>(lse_lat + 32 * ks + 16 + 4 * g) * -kLog2e;
+            const f32x4 da = -*reinterpret_cast<const f32x4*>(delta_lat + 32 * ks + 4 * g);
+            const f32x4 db = -*reinterpret_cast<const f32x4*>(delta_lat + 32 * ks + 16 + 4 * g);
 #pragma unroll
             for (int tw = 0; tw < kBTW; ++tw) {
                 f32x4 a0 = la, a1 = lb, s0 = zf, s1 = zf, g10 = da, g11 = db, g20 = zf, g21 = zf;
@@ -555,8 +557,16 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
                 uint32_t o[2 * RT];
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                    o[2 * rt] = M_::pack2(acc[rt][0], acc[rt][1]);
-                    o[2 * rt + 1] = M_::pack2(acc[rt][2], acc[rt][3]);
+                    f32x4 t = acc[rt];
+                    if (a.accumulate) {       // a later chunk of latents: add to what the earlier launches stored
+                        const uint2 old = *reinterpret_cast<const uint2*>(p + 4 * rt);
+                        t[0] += M_::unpack(uint16_t(old.x & 0xffffu));
+                        t[1] += M_::unpack(uint16_t(old.x >> 16));
+                        t[2] += M_::unpack(uint16_t(old.y & 0xffffu));
+                        t[3] += M_::unpack(uint16_t(old.y >> 16));
+                    }
+                    o[2 * rt] = M_::pack2(t[0], t[1]);
+                    o[2 * rt + 1] = M_::pack2(t[2], t[3]);
                 }
                 if constexpr (RT == 1) {
                     *reinterpret_cast<uint2*>(p) = make_uint2(o[0], o[1]);
@@ -595,14 +605,24 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
     hipLaunchKernelGGL(bwd_merge_kernel<0>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a);
     {
         auto kern = bwd_tok_kernel<T, D>;
-        const size_t lds = mixer_bwd_lds_bytes(a.M, D);
+        // the latents are covered in 1, 2 or 4 launches, each with the operand sets of its chunk in LDS
+        const int chunks = mixer_bwd_tok_chunks(a.M, D);
+        if (chunks == 0) return hipErrorInvalidValue;
+        const int mc = a.M / chunks;
+        const size_t lds = mixer_bwd_lds_bytes(mc, D);
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         // one workgroup per compute unit (256 CUs), ranges a multiple of its 512-token pass
         const int64_t per_bh = (256 + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H);
         int64_t tpw = (a.N + per_bh - 1) / per_bh;
         tpw = ((tpw + 511) / 512) * 512;
-        hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(64 * kTokWaves), lds, st, a, (int)tpw);
+        for (int c = 0; c < chunks; ++c) {
+            MixerBwdArgs ac = a;
+            ac.m0 = c * mc;
+            ac.mc = mc;
+            ac.accumulate = c > 0;
+            hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(64 * kTokWaves), lds, st, ac, (int)tpw);
+        }
     }
     e = lat_launch<T, D, 1>(a, st);
     if (e != hipSuccess) return e;
@@ -623,12 +643,21 @@ hipError_t bwd_d(const MixerBwdArgs& a, hipStream_t st)
 
 }  // namespace
 
-size_t mixer_bwd_lds_bytes(int M, int D) { return (size_t)M * D * 2 * 5 + (size_t)M * 8; }
+size_t mixer_bwd_lds_bytes(int M, int D) { return (size_t)M * D * 2 * 5; }
+
+// Launches of the token-side kernel needed to cover M latents (each takes a chunk that is a multiple of 32 and whose
+// five operand sets fit the 160 KB of LDS), or 0 when even four do not do.
+int mixer_bwd_tok_chunks(int M, int D)
+{
+    for (int c = 1; c <= 4; c *= 2)
+        if (M % (32 * c) == 0 && mixer_bwd_lds_bytes(M / c, D) <= 160 * 1024) return c;
+    return 0;
+}
 
 bool mixer_bwd_supported(int dtype, int M, int D)
 {
     return (dtype == 1 || dtype == 2) && (D == 16 || D == 32 || D == 64) && M >= 32 && M % 32 == 0 &&
-           mixer_bwd_lds_bytes(M, D) <= 150 * 1024;
+           mixer_bwd_tok_chunks(M, D) > 0;
 }
 
 hipError_t launch_mixer_bwd(const MixerBwdArgs& a, int dtype, hipStream_t st)

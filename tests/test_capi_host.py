@@ -175,6 +175,9 @@ def test_new_struct_sizes_and_entry_point_validation():
     d = _mixer_desc(M=128, D=32)
     assert lib.flare_mixer_bwd_workspace_bytes(d, C.byref(need)) == _lib.FLARE_OK and need.value > 0
     assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(dtype=_lib.DT_F32), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
-    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=256, D=64), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
+    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=256, D=64), C.byref(need)) == _lib.FLARE_OK      # one LDS-full exactly
+    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=1024, D=64), C.byref(need)) == _lib.FLARE_OK     # four chunks of latents
+    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=2048, D=64), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
+    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=48, D=32), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
     assert lib.flare_mixer_bwd(d, *([None] * 8), None, None, None, None, None, 0, None) == _lib.FLARE_EINVAL
     assert lib.flare_scatter_fwd_lse(d, None, None, None, None, None, None, None) == _lib.FLARE_EINVAL

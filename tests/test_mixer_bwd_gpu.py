@@ -78,8 +78,8 @@ def test_fallbacks_keep_working(dev):
     q, k, v, gy = make(1, 2, 200, 64, 16, torch.float32, seed=7)
     qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
     assert not FN._hip_backward_ok(qd, kd, vd, None, False)
-    big = [t.to(dev).bfloat16() for t in make(1, 1, 64, 256, 64, torch.float32)[:3]]
-    assert not FN._hip_backward_ok(*big, None, False)                      # latent operands would not fit the LDS
+    big = [t.to(dev).bfloat16() for t in make(1, 1, 64, 2048, 64, torch.float32)[:3]]
+    assert not FN._hip_backward_ok(*big, None, False)                      # more latents than four chunks of LDS hold
     F.flare_multihead_mixer(qd, kd, vd).backward(gy.to(dev))
     gq, gk, gv = oracle_grads(q, k, v, gy, 1.0)
     assert O.rel_l2(qd.grad, gq) <= 1e-4 and O.rel_l2(kd.grad, gk) <= 1e-4 and O.rel_l2(vd.grad, gv) <= 1e-4
@@ -135,5 +135,19 @@ def test_narrow_head_backward(dev):
     gq, gk, gv = oracle_grads(q, k, v, gy, 1.1)
     for name, got, ref in (("dq", qd.grad, gq), ("dk", kd.grad, gk), ("dv", vd.grad, gv)):
         assert got.shape == ref.shape
+        err = O.rel_l2(got, ref)
+        assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
+
+
+@pytest.mark.parametrize("shape", [(1, 2, 1500, 256, 64), (1, 1, 1200, 512, 32), (1, 1, 900, 512, 64), (1, 1, 700, 1024, 32)])
+def test_backward_with_latents_in_chunks(dev, shape):
+    """M * D beyond one LDS-full of operand sets (160 KB = M * D of 16384): the token-side kernel runs once per chunk
+    of latents and adds to dk, dv; at exactly 16384 everything is resident with the per-latent scalars read from global."""
+    q, k, v, gy = make(*shape, torch.bfloat16, seed=19)
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    assert FN._hip_backward_ok(qd, kd, vd, None, False)
+    F.flare_multihead_mixer(qd, kd, vd, scale=0.8).backward(gy.to(dev))
+    gq, gk, gv = oracle_grads(q, k, v, gy, 0.8)
+    for name, got, ref in (("dq", qd.grad, gq), ("dk", kd.grad, gk), ("dv", vd.grad, gv)):
         err = O.rel_l2(got, ref)
         assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
