@@ -26,7 +26,9 @@ def test_reference_exact_mode(dev, shape, dtype):
     a = make(*shape, dtype)
     st, out = F.triple_attention(*[t.to(dev) for t in a])
     sr, orf = O.triple_einsum(*[t.float() for t in a], dtype=torch.float64)
-    assert O.rel_l2(st, sr) <= max(TOL[dtype] * 0.1, 1e-5)   # state is fp32 accumulate of exact products
+    # state: fp32 accumulation; the 16-bit kernels round each product k1[n,i] k2[n,k] to the element type once before
+    # the matrix product (half an ulp, 2^-9 for bf16: with a single token nothing averages it out)
+    assert O.rel_l2(st, sr) <= (1e-5 if dtype == torch.float32 else 4e-3)
     assert O.rel_l2(out, orf) <= TOL[dtype]
     assert st.dtype == torch.float32 and out.dtype == dtype
 
@@ -74,7 +76,8 @@ def test_cfg5_shape(dev):
     assert O.rel_l2(st, sr) <= 1e-2 and O.rel_l2(out, orf) <= 2e-2
 
 
-@pytest.mark.parametrize("dtype,D,Dv,tol", [(torch.float32, 16, 16, 1e-4), (torch.bfloat16, 16, 16, 3e-2), (torch.float32, 8, 12, 1e-4)])
+@pytest.mark.parametrize("dtype,D,Dv,tol", [(torch.float32, 16, 16, 1e-4), (torch.bfloat16, 16, 16, 3e-2), (torch.float32, 8, 12, 1e-4),
+                                            (torch.bfloat16, 32, 32, 3e-2)])
 def test_backward_matches_autograd_of_the_einsum_oracle(dev, dtype, D, Dv, tol):
     # gradients of lra/models/triton/triple.py:124-135, including a gradient flowing into STATE
     g = torch.Generator().manual_seed(11)
@@ -91,3 +94,19 @@ def test_backward_matches_autograd_of_the_einsum_oracle(dev, dtype, D, Dv, tol):
     for name, a, b in zip(("dq1", "dq2", "dk1", "dk2", "dv"), dins, rins):
         err = O.rel_l2(a.grad, b.grad)
         assert err <= tol, f"{name}: {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("Dq,Dv", [(32, 32), (16, 32), (32, 16), (64, 64), (48, 32), (8, 8), (20, 24), (4, 40)])
+def test_head_dims_in_blocks_of_16(dev, Dq, Dv, dtype):
+    """Head dims other than 16 run as launches of the 16 x 16 x 16 matrix-core kernels over index blocks, zero-padded to
+    a multiple of 16 where needed (the reference's Triton path takes any D >= 16 with D % 4 == 0,
+    lra/models/triton/triple.py:69-70; its einsum path any D)."""
+    a = make(2, 2, 900, Dq, Dv, dtype, seed=Dq + Dv)
+    st, out = F.triple_attention(*[t.to(dev) for t in a], normalize=True, feature_map="elu")
+    sr, orf = O.triple_einsum(*[t.float() for t in a], feature_map=True, normalize=True, dtype=torch.float64)
+    assert st.shape == (2, 2, Dq, Dv, Dq) and out.shape == (2, 2, 900, Dv) and out.dtype == dtype
+    assert O.rel_l2(st, sr) <= 1e-2 and O.rel_l2(out, orf) <= 2e-2
+    c = torch.full_like(a[4], -0.5)                       # constant v, normalised => constant output
+    _, oc = F.triple_attention(*[t.to(dev) for t in a[:4]], c.to(dev), normalize=True, feature_map="elu")
+    assert torch.allclose(oc.float().cpu(), c.float(), atol=1e-2)
