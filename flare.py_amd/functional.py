@@ -470,6 +470,20 @@ def causal_fresh_state(B, H, M, D, device):
 
 def _causal_call(entry, q, k, v, scale, chunk, state):
     _require_cuda(q, k, v)
+    D = k.shape[-1]
+    if (k.dtype in (torch.bfloat16, torch.float16) and D < 32 and q.shape[-2] in (128, 256) and q.shape[-1] == D
+            and v.shape == k.shape):
+        # the matrix-core causal kernels take D = 32 and 64: a narrower head gets zero columns (scores and the first
+        # D columns of every output and of the state's numerators are unchanged) instead of the fp32 kernel
+        pad = 32 - D
+        if state is not None:
+            state = (state[0], state[1], _pad_last(state[2], pad))
+        y, (mu, den, num) = _causal_call_launch(entry, _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad), scale, chunk, state)
+        return y[..., :D], (mu, den, num[..., :D].contiguous())
+    return _causal_call_launch(entry, q, k, v, scale, chunk, state)
+
+
+def _causal_call_launch(entry, q, k, v, scale, chunk, state):
     lib = _lib.load()
     if q.dtype != k.dtype:
         q = q.to(k.dtype)

@@ -281,3 +281,18 @@ def test_cfg4_full_size_properties(dev):
     assert O.rel_l2(y2[b, h], yr[0, 0, NP:]) <= 2e-2
     zr, lser = O.causal_state_invariants(*str_)
     assert O.rel_l2(z[b, h].cpu(), zr[0, 0]) <= 2e-2 and float((lse[b, h].cpu() - lser[0, 0]).abs().max()) <= 0.2
+
+
+@pytest.mark.parametrize("M,D", [(128, 16), (256, 8)])
+def test_narrow_heads_on_the_matrix_core_path(dev, M, D):
+    """D below 32 is zero-padded to 32 around the matrix-core kernels: prefill, a second prefill from the returned
+    state, then decode, against the recurrence; the state comes back with its own D columns."""
+    q, k, v = make(2, 2, 900, M, D, torch.bfloat16, seed=12)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    y1, st = F.flare_causal_prefill(qd, kd[:, :, :400], vd[:, :, :400])
+    assert st[2].shape == (2, 2, M, D)
+    y2, st = F.flare_causal_prefill(qd, kd[:, :, 400:850], vd[:, :, 400:850], state=st)
+    y3, st = F.flare_causal_decode(qd, kd[:, :, 850:], vd[:, :, 850:], st)
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float(), dtype=torch.float32)
+    assert O.rel_l2(torch.cat([y1, y2, y3], 2), yr) <= 2e-2
+    state_close(st, tuple(s.double() for s in str_), 2e-2)
