@@ -290,13 +290,14 @@ class _MixerFn(torch.autograd.Function):
 
 
 def _narrow_head_pad(q, k, force_generic) -> int:
-    """Columns of zeros to append to a head dim below 16 so that the matrix-core kernels (D in {16, 32, 64}) take
-    the problem, or 0.  Zero columns change neither the scores q.k nor the first D output columns; the reference's
-    default model has D = channel_dim / num_heads = 8, which the fp32-FMA kernels would serve 5-15x slower."""
+    """Columns of zeros to append to a head dim so that the matrix-core kernels (D in {16, 32, 64}) take the problem,
+    or 0.  Zero columns change neither the scores q.k nor the first D output columns; the reference's default model
+    has D = channel_dim / num_heads = 8, which the fp32-FMA kernels would serve 5-15x slower."""
     D = k.shape[-1]
-    if force_generic or D >= 16 or k.dtype not in (torch.bfloat16, torch.float16) or k.device.type != "cuda":
+    if force_generic or D > 64 or k.dtype not in (torch.bfloat16, torch.float16) or k.device.type != "cuda":
         return 0
-    return 16 - D if q.shape[-2] % 32 == 0 else 0
+    target = 16 if D <= 16 else 32 if D <= 32 else 64
+    return target - D if q.shape[-2] % 32 == 0 else 0
 
 
 def _pad_last(t, n):

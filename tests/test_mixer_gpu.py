@@ -327,10 +327,10 @@ def test_localized_large_scores_mix_fast_and_exact_paths(dev, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("shape", [(2, 8, 3000, 64, 8), (1, 4, 1111, 256, 8), (1, 2, 500, 128, 4)])
+@pytest.mark.parametrize("shape", [(2, 8, 3000, 64, 8), (1, 4, 1111, 256, 8), (1, 2, 500, 128, 4), (1, 2, 900, 64, 24), (1, 2, 700, 128, 40), (1, 3, 800, 32, 10)])
 def test_narrow_heads_run_on_the_matrix_core_kernels(dev, shape, dtype):
-    """Head dims below 16 (the reference's default model has channel_dim 64 / 8 heads = 8, pdebench/__main__.py:1122-1123)
-    are zero-padded to 16: same scores, same outputs, matrix-core kernels."""
+    """Head dims other than 16, 32, 64 (the reference's default model has channel_dim 64 / 8 heads = 8,
+    pdebench/__main__.py:1122-1123) are zero-padded to the next of them: same scores, same outputs, matrix-core kernels."""
     B, H, N, M, D = shape
     q, k, v = make(B, H, N, M, D, dtype, seed=21)
     x = torch.stack([k, v]).permute(0, 1, 3, 2, 4).reshape(2, B, N, H * D).contiguous().to(dev)
