@@ -131,6 +131,12 @@ def _mask_u8(key_mask, B, N, device):
 
 def mixer_kernel_name(q, k, v=None, scale=1.0, force_generic=False) -> str:
     """Which kernel family the dispatcher picks for these operands (no launch)."""
+    M, D = q.shape[-2], k.shape[-1]
+    if (M % 32 != 0 and not force_generic and q.dtype == k.dtype and D < 64 and k.dtype in (torch.bfloat16, torch.float16)
+            and k.device.type == "cuda"):           # dead latents and a wider head, see _mixer_odd_latents
+        Dp = 16 if D < 16 else 32 if D < 32 else 64
+        q = q.new_zeros(*q.shape[:-2], -(-M // 32) * 32, Dp)
+        k, v = _pad_last(k, Dp - D), None
     pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype else 0
     if pad:                                 # what flare_multihead_mixer hands to the library for a narrow head
         q, k, v = _pad_last(q, pad), _pad_last(k, pad), None
@@ -321,6 +327,9 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
     if ac is not None:
         q, k, v = (t if t.dtype == ac else t.to(ac) for t in (q, k, v))
     D = k.shape[-1]
+    if (q.shape[-2] % 32 != 0 and not force_generic and q.dtype == k.dtype == v.dtype and D < 64
+            and k.dtype in (torch.bfloat16, torch.float16) and k.device.type == "cuda"):
+        return _mixer_odd_latents(q, k, v, float(scale), key_mask, return_z, n_splits, token_major_out)
     pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype == v.dtype else 0
     if pad:
         q, k, v = _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad)
@@ -331,6 +340,32 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
     if pad:
         y, z = y[..., :D], z[..., :D]
     return (y, z) if return_z else y
+
+
+def _mixer_odd_latents(q, k, v, scale, key_mask, return_z, n_splits, token_major_out):
+    """A latent count that is not a multiple of 32 on the matrix-core kernels: the latents are filled up with dead
+    ones.  In the gather a dead latent is a zero query whose row of z is never used.  In the scatter it must get no
+    weight: k receives one extra column of ones and the dead queries hold -16384 there (the real ones 0), which takes
+    their scores out of every token's softmax.  The extra column rides in the zero padding of the head dim (D grows to
+    the next of 16, 32, 64 that leaves room for it).  Gradients come from the two halves' torch recomputation."""
+    M, D = q.shape[-2], k.shape[-1]
+    Mp = -(-M // 32) * 32
+    Dp = 16 if D < 16 else 32 if D < 32 else 64
+    qz = _pad_last(q, Dp - D)
+    dead = qz.new_zeros(*qz.shape[:-2], Mp - M, Dp)
+    q_gather = torch.cat([qz, dead], dim=-2)
+    dead_s = dead.clone()
+    dead_s[..., D] = -16384.0
+    q_scatter = torch.cat([qz, dead_s], dim=-2)
+    kp = _pad_last(k, Dp - D).clone() if Dp - D else k
+    kp[..., D] = 1.0
+    vp = _pad_last(v, Dp - D)
+    z, _ = flare_gather(q_gather, kp, vp, scale, key_mask, n_splits)
+    y = flare_scatter(q_scatter, kp, z, scale, key_mask)
+    y = y[..., :D]
+    if token_major_out:
+        y = y.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    return (y, z[..., :M, :D]) if return_z else y
 
 
 def _gather_forward(q, k, v, scale, key_mask, n_splits, force_generic):

@@ -397,3 +397,35 @@ def test_against_torch_fused_attention_on_the_device(dev, dtype):
         # and about as close to the fp64 oracle as torch is (for f16 inputs the HIP kernels still carry the
         # probabilities in bf16, whose exponent range the unshifted softmax needs: 3e-3 there)
         assert O.rel_l2(y, yr) <= max(O.rel_l2(yt, yr) * 1.5 + 1e-3, 3e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(2, 2, 2000, 48, 16), (1, 3, 1500, 100, 32), (1, 2, 900, 20, 8), (1, 2, 700, 7, 24)])
+def test_latent_counts_that_are_not_multiples_of_32(dev, shape, dtype):
+    """Dead latents fill M up to a multiple of 32 (zero queries in the gather, a -16384 score offset in the scatter):
+    forward against the oracle with and without a mask, gradients against fp64 autograd, strongly negative scores."""
+    B, H, N, M, D = shape
+    q, k, v = make(B, H, N, M, D, dtype, seed=51)
+    assert F.mixer_kernel_name(q.to(dev), k.to(dev), v.to(dev)).startswith("mfma")
+    mask = torch.ones(B, N, dtype=torch.bool)
+    mask[0, N // 2:] = False
+    for km in (None, mask):
+        y, z = F.flare_multihead_mixer(q.to(dev), k.to(dev), v.to(dev), scale=0.8, key_mask=None if km is None else km.to(dev), return_z=True)
+        yr, zr = O.mixer_explicit(q.float(), k.float(), v.float(), 0.8, km)
+        assert y.shape == yr.shape and z.shape == zr.shape
+        assert O.rel_l2(z, zr) <= 2e-2 and O.rel_l2(y, yr) <= 2e-2
+    # every real score far below the dead latents' gather score of 0: the dead ones must still get no weight
+    k2 = (k.float() * 0.05).to(dtype)
+    q2 = (q.float() - 3.0).to(dtype) if D >= 16 else q
+    y2 = F.flare_multihead_mixer(q2.to(dev), (k2.float().abs()).to(dtype).to(dev), v.to(dev), scale=4.0)
+    yr2, _ = O.mixer_explicit(q2.float(), k2.float().abs().to(dtype).float(), v.float(), 4.0)
+    assert O.rel_l2(y2, yr2) <= 2e-2
+    gy = torch.randn(B, H, N, D, generator=torch.Generator().manual_seed(52)).to(dtype)
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    F.flare_multihead_mixer(qd, kd, vd, scale=0.8).backward(gy.to(dev))
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    O.mixer_explicit(qr, kr, vr, 0.8)[0].backward(gy.double())
+    for name, got, ref in (("dq", qd.grad, qr.grad), ("dk", kd.grad, kr.grad), ("dv", vd.grad, vr.grad)):
+        assert got.shape == ref.shape
+        err = O.rel_l2(got, ref)
+        assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
