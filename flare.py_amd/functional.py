@@ -504,9 +504,29 @@ def causal_fresh_state(B, H, M, D, device):
     return mu, den, num
 
 
+#: decode calls of at least this many tokens also take the replicated-latent route below (a shorter decode is
+#: launch-bound, and the fp32 step kernel reads a state half the size or less)
+CAUSAL_REPLICATE_DECODE_MIN_TOKENS = 32
+
+
 def _causal_call(entry, q, k, v, scale, chunk, state):
     _require_cuda(q, k, v)
     D = k.shape[-1]
+    M = q.shape[-2]
+    if (k.dtype in (torch.bfloat16, torch.float16) and M < 128 and 128 % M == 0 and (D <= 32 or D == 64)
+            and q.shape[-1] == D and v.shape == k.shape and k.dim() == 4
+            and (entry == "prefill" or k.shape[2] >= CAUSAL_REPLICATE_DECODE_MIN_TOKENS)):
+        # The matrix-core causal kernels take 128 or 256 latents.  r copies of every latent leave y unchanged: each
+        # copy carries the same running state z_m(t), and the softmax over the r*M copies gives each 1/r of the
+        # weight latent m had.  So a power-of-two latent count below 128 is tiled up to 128 (state in and out
+        # likewise) instead of taking the fp32 kernel.
+        r = 128 // M
+        qr = q.repeat(*([1] * (q.dim() - 2)), r, 1)
+        if state is not None:
+            mu, den, num = state
+            state = (mu.repeat(1, 1, r), den.repeat(1, 1, r), num.repeat(1, 1, r, 1))
+        y, (mu, den, num) = _causal_call(entry, qr, k, v, scale, chunk, state)
+        return y, (mu[..., :M].contiguous(), den[..., :M].contiguous(), num[..., :M, :].contiguous())
     if (k.dtype in (torch.bfloat16, torch.float16) and D < 32 and q.shape[-2] in (128, 256) and q.shape[-1] == D
             and v.shape == k.shape):
         # the matrix-core causal kernels take D = 32 and 64: a narrower head gets zero columns (scores and the first

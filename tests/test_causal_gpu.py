@@ -296,3 +296,25 @@ def test_narrow_heads_on_the_matrix_core_path(dev, M, D):
     yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float(), dtype=torch.float32)
     assert O.rel_l2(torch.cat([y1, y2, y3], 2), yr) <= 2e-2
     state_close(st, tuple(s.double() for s in str_), 2e-2)
+
+
+@pytest.mark.parametrize("M,D", [(64, 32), (64, 8), (32, 64), (16, 16)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_power_of_two_latent_counts_below_128(dev, M, D, dtype):
+    """Fewer than 128 latents run on the matrix-core kernels as 128 // M copies of every latent (the copies share
+    the softmax weight of the one they stand for): prefill, a continued prefill, a long decode (same route) and
+    single steps (fp32 step kernel) against the recurrence; the state comes back with M latents, and matches
+    what the fp32 kernels give for the same call."""
+    q, k, v = make(2, 2, 700, M, D, dtype, seed=21)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    y1, st = F.flare_causal_prefill(qd, kd[:, :, :300], vd[:, :, :300])
+    assert st[0].shape == (2, 2, M) and st[2].shape == (2, 2, M, D)
+    y2, st = F.flare_causal_prefill(qd, kd[:, :, 300:640], vd[:, :, 300:640], state=st)
+    y3, st = F.flare_causal_decode(qd, kd[:, :, 640:698], vd[:, :, 640:698], st)
+    ys = []
+    for t in (698, 699):
+        yt, st = F.flare_causal_decode_step(qd, kd[:, :, t], vd[:, :, t], st)
+        ys.append(yt.unsqueeze(2))
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float(), dtype=torch.float32)
+    assert O.rel_l2(torch.cat([y1, y2, y3] + ys, 2), yr) <= 2e-2
+    state_close(st, tuple(s.double() for s in str_), 2e-2)
