@@ -12,6 +12,7 @@ implementation behind these calls, and a missing library raises.
 from __future__ import annotations
 
 import ctypes as C
+import math
 from typing import Optional, Tuple
 
 import torch
@@ -131,6 +132,9 @@ def _mask_u8(key_mask, B, N, device):
 
 def mixer_kernel_name(q, k, v=None, scale=1.0, force_generic=False) -> str:
     """Which kernel family the dispatcher picks for these operands (no launch)."""
+    r = _latent_copies(q, k, force_generic)
+    if r > 1:                               # copies of every latent, see flare_multihead_mixer
+        q = q.repeat(*([1] * (q.dim() - 2)), r, 1)
     M, D = q.shape[-2], k.shape[-1]
     if (M % 32 != 0 and not force_generic and q.dtype == k.dtype and D < 64 and k.dtype in (torch.bfloat16, torch.float16)
             and k.device.type == "cuda"):           # dead latents and a wider head, see _mixer_odd_latents
@@ -327,6 +331,14 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
     if ac is not None:
         q, k, v = (t if t.dtype == ac else t.to(ac) for t in (q, k, v))
     D = k.shape[-1]
+    r = _latent_copies(q, k, force_generic)
+    if r > 1 and q.dtype == v.dtype:
+        # r copies of every latent: each copy gathers the same row of z and the softmax over the r*M copies gives each
+        # 1/r of the weight latent m had, so y is unchanged; autograd sums the copies' gradients through repeat()
+        M = q.shape[-2]
+        out = flare_multihead_mixer(q.repeat(*([1] * (q.dim() - 2)), r, 1), k, v, scale, key_mask, return_z, n_splits,
+                                    force_generic, token_major_out)
+        return (out[0], out[1][..., :M, :]) if return_z else out
     if (q.shape[-2] % 32 != 0 and not force_generic and q.dtype == k.dtype == v.dtype and D < 64
             and k.dtype in (torch.bfloat16, torch.float16) and k.device.type == "cuda"):
         return _mixer_odd_latents(q, k, v, float(scale), key_mask, return_z, n_splits, token_major_out)
@@ -340,6 +352,16 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
     if pad:
         y, z = y[..., :D], z[..., :D]
     return (y, z) if return_z else y
+
+
+def _latent_copies(q, k, force_generic) -> int:
+    """How many copies of every latent bring a 16-bit problem's latent count to a multiple of 32 (what the matrix-core
+    kernels and the HIP backward take): 2 or 4 for multiples of 8, else 1 (other counts get dead latents instead)."""
+    M, D = q.shape[-2], k.shape[-1]
+    if (M % 32 == 0 or M % 8 != 0 or force_generic or D > 64 or q.dtype != k.dtype
+            or k.dtype not in (torch.bfloat16, torch.float16) or k.device.type != "cuda"):
+        return 1
+    return 32 // math.gcd(M, 32)
 
 
 def _mixer_odd_latents(q, k, v, scale, key_mask, return_z, n_splits, token_major_out):

@@ -429,3 +429,34 @@ def test_latent_counts_that_are_not_multiples_of_32(dev, shape, dtype):
         assert got.shape == ref.shape
         err = O.rel_l2(got, ref)
         assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(1, 2, 800, 16, 32), (1, 2, 600, 8, 64), (2, 1, 900, 48, 64), (1, 2, 500, 24, 8), (1, 1, 700, 80, 16)])
+def test_latent_counts_that_are_multiples_of_8(dev, shape, dtype):
+    """A latent count that is a multiple of 8 but not of 32 runs as 2 or 4 copies of every latent on the matrix-core
+    kernels, forward and backward (the copies share each latent's softmax weight, autograd sums their gradients):
+    y and z against the oracle with and without a mask, gradients against fp64 autograd."""
+    from flare_py_amd import functional as fn
+    B, H, N, M, D = shape
+    q, k, v = make(B, H, N, M, D, dtype, seed=61)
+    assert F.mixer_kernel_name(q.to(dev), k.to(dev), v.to(dev)).startswith("mfma")
+    r = fn._latent_copies(q.to(dev), k.to(dev), False)
+    assert r in (2, 4) and (r * M) % 32 == 0
+    assert fn._hip_backward_ok(q.to(dev).repeat(1, r, 1), k.to(dev), v.to(dev), None, False) or D < 16
+    mask = torch.ones(B, N, dtype=torch.bool)
+    mask[0, N // 3:] = False
+    for km in (None, mask):
+        y, z = F.flare_multihead_mixer(q.to(dev), k.to(dev), v.to(dev), scale=0.8, key_mask=None if km is None else km.to(dev), return_z=True)
+        yr, zr = O.mixer_explicit(q.float(), k.float(), v.float(), 0.8, km)
+        assert y.shape == yr.shape and z.shape == zr.shape
+        assert O.rel_l2(z, zr) <= 2e-2 and O.rel_l2(y, yr) <= 2e-2
+    gy = torch.randn(B, H, N, D, generator=torch.Generator().manual_seed(62)).to(dtype)
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    F.flare_multihead_mixer(qd, kd, vd, scale=0.8).backward(gy.to(dev))
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    O.mixer_explicit(qr, kr, vr, 0.8)[0].backward(gy.double())
+    for name, got, ref in (("dq", qd.grad, qr.grad), ("dk", kd.grad, kr.grad), ("dv", vd.grad, vr.grad)):
+        assert got.shape == ref.shape
+        err = O.rel_l2(got, ref)
+        assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
