@@ -535,7 +535,7 @@ def _causal_call(entry, q, k, v, scale, chunk, state):
     _require_cuda(q, k, v)
     D = k.shape[-1]
     M = q.shape[-2]
-    if (k.dtype in (torch.bfloat16, torch.float16) and M < 128 and 128 % M == 0 and (D <= 32 or D == 64)
+    if (k.dtype in (torch.bfloat16, torch.float16) and M < 128 and 128 % M == 0 and D <= 64
             and q.shape[-1] == D and v.shape == k.shape and k.dim() == 4
             and (entry == "prefill" or k.shape[2] >= CAUSAL_REPLICATE_DECODE_MIN_TOKENS)):
         # The matrix-core causal kernels take 128 or 256 latents.  r copies of every latent leave y unchanged: each
@@ -549,11 +549,11 @@ def _causal_call(entry, q, k, v, scale, chunk, state):
             state = (mu.repeat(1, 1, r), den.repeat(1, 1, r), num.repeat(1, 1, r, 1))
         y, (mu, den, num) = _causal_call(entry, qr, k, v, scale, chunk, state)
         return y, (mu[..., :M].contiguous(), den[..., :M].contiguous(), num[..., :M, :].contiguous())
-    if (k.dtype in (torch.bfloat16, torch.float16) and D < 32 and q.shape[-2] in (128, 256) and q.shape[-1] == D
-            and v.shape == k.shape):
-        # the matrix-core causal kernels take D = 32 and 64: a narrower head gets zero columns (scores and the first
-        # D columns of every output and of the state's numerators are unchanged) instead of the fp32 kernel
-        pad = 32 - D
+    if (k.dtype in (torch.bfloat16, torch.float16) and (D < 32 and M in (128, 256) or 32 < D < 64 and M == 128)
+            and q.shape[-1] == D and v.shape == k.shape):
+        # the matrix-core causal kernels take D = 32 and 64: any other head up to 64 gets zero columns (scores and the
+        # first D columns of every output and of the state's numerators are unchanged) instead of the fp32 kernel
+        pad = (32 if D < 32 else 64) - D
         if state is not None:
             state = (state[0], state[1], _pad_last(state[2], pad))
         y, (mu, den, num) = _causal_call_launch(entry, _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad), scale, chunk, state)

@@ -283,9 +283,9 @@ def test_cfg4_full_size_properties(dev):
     assert O.rel_l2(z[b, h].cpu(), zr[0, 0]) <= 2e-2 and float((lse[b, h].cpu() - lser[0, 0]).abs().max()) <= 0.2
 
 
-@pytest.mark.parametrize("M,D", [(128, 16), (256, 8)])
+@pytest.mark.parametrize("M,D", [(128, 16), (256, 8), (128, 48)])
 def test_narrow_heads_on_the_matrix_core_path(dev, M, D):
-    """D below 32 is zero-padded to 32 around the matrix-core kernels: prefill, a second prefill from the returned
+    """D below 32 is zero-padded to 32, D between 32 and 64 to 64 (128 latents: 256 x 64 does not fit the kernels' LDS), around the matrix-core kernels: prefill, a second prefill from the returned
     state, then decode, against the recurrence; the state comes back with its own D columns."""
     q, k, v = make(2, 2, 900, M, D, torch.bfloat16, seed=12)
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
@@ -298,7 +298,7 @@ def test_narrow_heads_on_the_matrix_core_path(dev, M, D):
     state_close(st, tuple(s.double() for s in str_), 2e-2)
 
 
-@pytest.mark.parametrize("M,D", [(64, 32), (64, 8), (32, 64), (16, 16)])
+@pytest.mark.parametrize("M,D", [(64, 32), (64, 8), (32, 64), (16, 16), (64, 40)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_power_of_two_latent_counts_below_128(dev, M, D, dtype):
     """Fewer than 128 latents run on the matrix-core kernels as 128 // M copies of every latent (the copies share
