@@ -526,6 +526,41 @@ def causal_fresh_state(B, H, M, D, device):
     return mu, den, num
 
 
+def _scatter_lse(q, k, scale):
+    """ln sum_m exp(scale <k_n, q_m>) per token, [B,H,N] fp32, from flare_scatter_fwd_lse (its y goes to a scratch
+    tensor): the weight a group of latents carries in a softmax over several groups."""
+    lib = _lib.load()
+    k = _rows_last_contig(k)
+    B, H, N, D = k.shape
+    q4 = _q4(q.to(k.dtype), B)
+    M = q4.shape[2]
+    y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    z = torch.zeros((B, H, M, D), dtype=torch.float32, device=k.device)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=k.device)
+    d = _mixer_desc(q4, k, k, y, scale, 0, False)
+    with _on_device(k.device):
+        rc = lib.flare_scatter_fwd_lse(C.byref(d), _ptr(q4), _ptr(k), _ptr(z), None, _ptr(y), _ptr(lse),
+                                       C.c_void_p(_stream_ptr(k.device)))
+    _lib.check(rc, "flare_scatter_fwd_lse")
+    return lse
+
+
+def _causal_latent_groups(M, D):
+    """Sizes of the latent groups a 16-bit causal problem is run in when the matrix-core kernels do not take its M
+    in one piece: 256 (heads up to 32) or 128 latents, then powers of two down to 32 for the rest.  [] when M is not
+    a multiple of 32 or D is above 64; a single entry when no split is needed."""
+    if M % 32 != 0 or D > 64 or M <= 128 and M & (M - 1) == 0:
+        return [M] if M % 32 == 0 and D <= 64 else []
+    big = 256 if D <= 32 else 128
+    sizes = [big] * (M // big)
+    rest = M % big
+    for p in (128, 64, 32):
+        if rest >= p:
+            sizes.append(p)
+            rest -= p
+    return sizes
+
+
 #: decode calls of at least this many tokens also take the replicated-latent route below (a shorter decode is
 #: launch-bound, and the fp32 step kernel reads a state half the size or less)
 CAUSAL_REPLICATE_DECODE_MIN_TOKENS = 32
@@ -549,6 +584,25 @@ def _causal_call(entry, q, k, v, scale, chunk, state):
             state = (mu.repeat(1, 1, r), den.repeat(1, 1, r), num.repeat(1, 1, r, 1))
         y, (mu, den, num) = _causal_call(entry, qr, k, v, scale, chunk, state)
         return y, (mu[..., :M].contiguous(), den[..., :M].contiguous(), num[..., :M, :].contiguous())
+    groups = _causal_latent_groups(M, D) if k.dtype in (torch.bfloat16, torch.float16) else []
+    if len(groups) > 1 and q.shape[-1] == D and v.shape == k.shape and k.dim() == 4:
+        # A latent count the matrix-core kernels do not take in one piece (256 latents with a head above 32 exceed a
+        # workgroup's LDS; 96, 192, 384, 512 ... have no kernel instance).  The softmax over the latents splits: each
+        # group of latents is a causal problem of its own whose y_g is normalised within the group, and
+        # y = sum_g w_g y_g with w_g = S_g / sum_g' S_g', S_g(t) = sum over the group of exp(scale <k_t, q_m>);
+        # the state is per latent and is cut and joined along M.
+        ys, sts, lses, m0 = [], [], [], 0
+        for g in groups:
+            sl = slice(m0, m0 + g)
+            m0 += g
+            st_g = None if state is None else (state[0][..., sl], state[1][..., sl], state[2][..., sl, :])
+            y_g, st_g = _causal_call(entry, q[..., sl, :], k, v, scale, chunk, st_g)
+            ys.append(y_g.float())
+            sts.append(st_g)
+            lses.append(_scatter_lse(q[..., sl, :], k, scale))
+        w = torch.softmax(torch.stack(lses), dim=0).unsqueeze(-1)
+        y = (w * torch.stack(ys)).sum(0).to(k.dtype)
+        return y, tuple(torch.cat(parts, dim=2) for parts in zip(*sts))
     if (k.dtype in (torch.bfloat16, torch.float16) and (D < 32 and M in (128, 256) or 32 < D < 64 and M == 128)
             and q.shape[-1] == D and v.shape == k.shape):
         # the matrix-core causal kernels take D = 32 and 64: any other head up to 64 gets zero columns (scores and the

@@ -318,3 +318,37 @@ def test_power_of_two_latent_counts_below_128(dev, M, D, dtype):
     yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float(), dtype=torch.float32)
     assert O.rel_l2(torch.cat([y1, y2, y3] + ys, 2), yr) <= 2e-2
     state_close(st, tuple(s.double() for s in str_), 2e-2)
+
+
+@pytest.mark.parametrize("M,D", [(256, 64), (256, 48), (96, 32), (192, 64), (512, 32), (224, 16), (384, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_latent_counts_run_in_groups(dev, M, D, dtype):
+    """Latent counts the matrix-core kernels do not take in one piece (256 with D above 32, 96, 192, 224, 384, 512)
+    run as causal problems over groups of latents, joined per token by the groups' softmax weights: prefill,
+    continued prefill, long decode and single steps against the recurrence, with the later latents' scores scaled
+    so that the groups' weights differ by orders of magnitude on part of the tokens."""
+    from flare_py_amd import functional as fn
+    assert len(fn._causal_latent_groups(M, D)) > 1 and sum(fn._causal_latent_groups(M, D)) == M
+    q, k, v = make(1, 2, 600, M, D, dtype, seed=31)
+    q[:, M // 2:] = (q[:, M // 2:].float() * 1.5).to(dtype)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    y1, st = F.flare_causal_prefill(qd, kd[:, :, :250], vd[:, :, :250])
+    assert st[0].shape == (1, 2, M) and st[2].shape == (1, 2, M, D)
+    y2, st = F.flare_causal_prefill(qd, kd[:, :, 250:540], vd[:, :, 250:540], state=st)
+    y3, st = F.flare_causal_decode(qd, kd[:, :, 540:598], vd[:, :, 540:598], st)
+    ys = []
+    for t in (598, 599):
+        yt, st = F.flare_causal_decode_step(qd, kd[:, :, t], vd[:, :, t], st)
+        ys.append(yt.unsqueeze(2))
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float(), dtype=torch.float32)
+    assert O.rel_l2(torch.cat([y1, y2, y3] + ys, 2), yr) <= 2e-2
+    state_close(st, tuple(s.double() for s in str_), 2e-2)
+
+
+def test_latent_group_sizes():
+    from flare_py_amd import functional as fn
+    assert fn._causal_latent_groups(128, 64) == [128] and fn._causal_latent_groups(256, 32) == [256]
+    assert fn._causal_latent_groups(64, 8) == [64] and fn._causal_latent_groups(48, 32) == []
+    assert fn._causal_latent_groups(256, 33) == [128, 128] and fn._causal_latent_groups(224, 16) == [128, 64, 32]
+    assert fn._causal_latent_groups(768, 32) == [256, 256, 256] and fn._causal_latent_groups(160, 64) == [128, 32]
+    assert fn._causal_latent_groups(128, 65) == []
