@@ -17,6 +17,7 @@ DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 FLAG_FORCE_GENERIC = 1
 MLP_EXPAND = 1
 ABI_VERSION = 1
+STATIC_SCRATCH_BYTES = 64 << 20
 
 I3 = C.c_int64 * 3
 
@@ -80,6 +81,7 @@ SYMBOLS = {
     "flare_mixer_bwd_workspace_bytes": (C.c_int, [C.POINTER(FlareMixerDesc), C.POINTER(_SZ)]),
     "flare_mixer_bwd": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, _P, _P, C.POINTER(C.c_int64), _P, _P, _P, _P, _SZ, _P]),
     "flare_mixer_fwd": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "flare_mixer_fwd_static": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P]),
     "flare_causal_workspace_bytes": (C.c_int, [C.POINTER(FlareCausalDesc), C.POINTER(_SZ)]),
     "flare_causal_prefill_fwd": (C.c_int, [C.POINTER(FlareCausalDesc), _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_causal_decode_fwd": (C.c_int, [C.POINTER(FlareCausalDesc), _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),

@@ -5,8 +5,13 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "common.hpp"
+
+// Scratch memory of flare_mixer_fwd_static: one array per device, held until the process ends.  Its name is
+// only a host-side handle; the device address is looked up once per device (static_scratch below).
+static __device__ __align__(256) unsigned char scratch[FLARE_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -495,6 +500,47 @@ int flare_mixer_fwd(const FlareMixerDesc* desc, const void* q, const void* k, co
     rc = do_gather(desc, q, k, v, key_mask, z, nullptr, workspace, workspace_bytes, st);
     if (rc != FLARE_OK) return rc;
     return do_scatter(desc, q, k, z, key_mask, y, st);
+}
+
+namespace {
+// Device address of `scratch` on the current device, looked up on the first call there and kept.
+int static_scratch(void** out)
+{
+    constexpr int kMaxDevices = 64;
+    static void* ptrs[kMaxDevices] = {};
+    static std::mutex mu;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_status(e, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(FLARE_EUNSUPPORTED, "device index %d outside [0, %d)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_status(e, "hipGetSymbolAddress(scratch)");
+        if (!p) return fail(FLARE_EHIP, "hipGetSymbolAddress(scratch) returned a null address");
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return FLARE_OK;
+}
+}  // namespace
+
+int flare_mixer_fwd_static(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
+                           const uint8_t* key_mask, void* y, void* stream)
+{
+    int rc = check_mixer_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !v || !y) return fail(FLARE_EINVAL, "q, k, v and y must not be NULL");
+    const size_t need = mixer_ws_bytes(desc);
+    if (need > (size_t)FLARE_STATIC_SCRATCH_BYTES)
+        return fail(FLARE_EWORKSPACE, "problem needs %zu bytes of scratch, the static buffer holds %zu: use flare_mixer_fwd with a caller-owned workspace",
+                    need, (size_t)FLARE_STATIC_SCRATCH_BYTES);
+    void* ws = nullptr;
+    rc = static_scratch(&ws);
+    if (rc != FLARE_OK) return rc;
+    // every partial row and every row of z that is read is written first by this call's own kernels: nothing to clear
+    return flare_mixer_fwd(desc, q, k, v, key_mask, y, nullptr, ws, (size_t)FLARE_STATIC_SCRATCH_BYTES, stream);
 }
 
 int flare_causal_workspace_bytes(const FlareCausalDesc* desc, size_t* bytes)

@@ -18,6 +18,7 @@
  *   flare_scatter_fwd_lse      the same, also returning each token's log-sum-exp over the latents
  *   flare_mixer_bwd            gradient of flare_multihead_mixer (torch autograd through the two SDPA
  *                              calls upstream; ablation/time_memory_bwd.py:460-478 times fwd+bwd)
+ *   flare_mixer_fwd_static     (no counterpart upstream: flare_mixer_fwd without a caller workspace)
  *   flare_causal_prefill_fwd   causal restriction of the mixer (README.md:60 names it; the
  *   flare_causal_decode_fwd    reference holds no code for it) following the 3-phase chunk
  *                              scheme of lra/models/triton/causal_linear.py:81-137 and the
@@ -92,7 +93,9 @@ typedef struct FlareCausalDesc {
     int32_t B, H, N, M, D;
     int32_t dtype;
     float   scale;
-    int32_t chunk;        /* prefill chunk length (tokens); 0 = default 256            */
+    int32_t chunk;        /* prefill segment length in tokens (rounded up to 16); 0 = automatic: the
+                             token axis is cut so that about two workgroups per compute unit run,
+                             segments of at least 256 tokens, at most 64 segments              */
     int32_t flags;
     int32_t reserved;
     int64_t q_stride[3];
@@ -209,6 +212,17 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
 int flare_mixer_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
                     const uint8_t* key_mask, void* y, float* z_out,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* flare_mixer_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The split
+ * partials and z live in a buffer of FLARE_STATIC_SCRATCH_BYTES that is part of the library's code object
+ * (one copy per GPU, held until the process ends); the call allocates and frees nothing.  A problem whose
+ * flare_mixer_workspace_bytes() exceeds that size is rejected with FLARE_EWORKSPACE before anything is
+ * launched.  All calls on one GPU share the buffer: calls that overlap in time on the same GPU (different
+ * streams or threads) race and must be serialised by the caller.  Results are those of flare_mixer_fwd. */
+#define FLARE_STATIC_SCRATCH_BYTES (64u << 20)
+int flare_mixer_fwd_static(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
+                           const uint8_t* key_mask, void* y, void* stream);
 
 int flare_causal_workspace_bytes(const FlareCausalDesc* desc, size_t* bytes);
 
