@@ -15,6 +15,8 @@ LIB_PATH = os.path.join(HERE, "libflare_hip.so")
 FLARE_OK, FLARE_EINVAL, FLARE_EUNSUPPORTED, FLARE_EWORKSPACE, FLARE_EHIP = 0, -1, -2, -3, -4
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 FLAG_FORCE_GENERIC = 1
+FLAG_MFMA16 = 2
+FLAG_GATHER32 = 4
 MLP_EXPAND = 1
 ABI_VERSION = 1
 STATIC_SCRATCH_BYTES = 64 << 20

@@ -81,7 +81,7 @@ MixerPlan plan_mixer(const FlareMixerDesc* d, bool want_mfma)
     int s = d->n_splits;
     if (s <= 0) {
         // one full round of resident workgroups (MFMA kernels) or ~4 per CU (generic)
-        const int64_t target = p.mfma ? flare::mfma_gather_resident_slots(d->dtype, d->M, d->D) : 1024;
+        const int64_t target = p.mfma ? flare::mfma_gather_resident_slots(d->dtype, d->M, d->D) : 4 * flare::device_cus();
         int64_t per = (int64_t)d->B * d->H * mblk;
         s = (int)((target + per - 1) / per);
         if (s < 1) s = 1;
@@ -127,6 +127,8 @@ void fill_mixer_args(flare::MixerArgs& a, const FlareMixerDesc* d, const MixerPl
     a.B = d->B; a.H = d->H; a.N = d->N; a.M = d->M; a.D = d->D;
     a.n_splits = p.n_splits; a.n_parts = p.n_parts; a.tokens_per_split = p.tokens_per_split;
     a.scale_log2 = d->scale * flare::kLog2e;
+    a.no_mfma32 = (d->flags & FLARE_FLAG_MFMA16) ? 1 : 0;
+    a.gather32 = (d->flags & FLARE_FLAG_GATHER32) ? 1 : 0;
     for (int i = 0; i < 3; ++i) {
         a.qs[i] = d->q_stride[i]; a.ks[i] = d->k_stride[i]; a.vs[i] = d->v_stride[i]; a.ys[i] = d->y_stride[i];
     }
@@ -216,9 +218,8 @@ CausalPlan plan_causal(const FlareCausalDesc* d)
     if (d->chunk > 0) {
         seg_len = ((int64_t)d->chunk + 15) / 16 * 16;
     } else {
-        // two workgroups per compute unit (what the kernel's LDS footprint allows on 256 CUs),
-        // segments of at least 256 tokens
-        const int64_t want = std::max<int64_t>(1, (512 + BH - 1) / BH);
+        // two workgroups per compute unit (what the kernel's LDS footprint allows), segments of at least 256 tokens
+        const int64_t want = std::max<int64_t>(1, (2 * flare::device_cus() + BH - 1) / BH);
         seg_len = std::max<int64_t>(256, ((d->N + want - 1) / want + 15) / 16 * 16);
     }
     int64_t n_segs = (d->N + seg_len - 1) / seg_len;
@@ -272,8 +273,8 @@ CausalLinearPlan plan_causal_linear(const FlareCausalLinearDesc* d)
     const int tile = flare::causal_linear_tile();
     const int64_t BH = (int64_t)d->B * d->H;
     const int64_t tiles = ((int64_t)d->N + tile - 1) / tile;
-    // automatic: about four workgroups per compute unit (256 CUs), never more segments than tiles
-    int64_t want = d->n_segs > 0 ? d->n_segs : std::max<int64_t>(1, (1024 + BH - 1) / BH);
+    // automatic: about four workgroups per compute unit, never more segments than tiles
+    int64_t want = d->n_segs > 0 ? d->n_segs : std::max<int64_t>(1, (4 * flare::device_cus() + BH - 1) / BH);
     want = std::min<int64_t>(std::min<int64_t>(want, tiles), 4096);
     const int64_t tiles_per_seg = (tiles + want - 1) / want;
     CausalLinearPlan p;
@@ -317,7 +318,7 @@ TriplePlan plan_triple(const FlareTripleDesc* d)
     if (s <= 0) {
         // about two workgroups per compute unit: more splits only add partials to write and merge
         const int64_t per = (int64_t)d->B * d->H;
-        s = (int)((512 + per - 1) / per);
+        s = (int)((2 * flare::device_cus() + per - 1) / per);
         if (s < 1) s = 1;
     }
     int64_t tps = ((int64_t)d->N + s - 1) / s;
@@ -406,7 +407,7 @@ BwdPlan plan_bwd(const FlareMixerDesc* d)
     const int64_t bh = (int64_t)d->B * d->H;
     const int mblocks = d->M % 256 == 0 ? d->M / 256 : d->M % 128 == 0 ? d->M / 128 : (d->M + 63) / 64;
     // about two workgroups per compute unit over the latent-side grids, token ranges of 64 k tokens
-    int64_t s = std::max<int64_t>(1, 512 / (bh * mblocks));
+    int64_t s = std::max<int64_t>(1, 2 * flare::device_cus() / (bh * mblocks));
     int64_t tps = ((int64_t)d->N + s - 1) / s;
     tps = (tps + 63) / 64 * 64;
     p.tokens_per_split = (int)tps;

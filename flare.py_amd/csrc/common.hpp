@@ -73,6 +73,8 @@ struct MixerArgs {
     int n_parts;              // partials per (b,h): n_splits * partials-per-workgroup
     int tokens_per_split;
     float scale_log2;         // scale * log2(e)
+    int no_mfma32;            // 1: keep the 16x16x32 kernels where the 32x32x16 ones would run
+    int gather32;             // 1: the gather may take the 32x32x16 kernel too
     int64_t qs[3], ks[3], vs[3], ys[3];
 };
 
@@ -160,8 +162,15 @@ int        mfma_gather_tokens_per_iter();
 int        mfma_gather_resident_slots(int dtype, int M, int D);
 // workgroups of `kern` resident on the current device at once (CUs x occupancy), cached per kernel, LDS size and device
 int        resident_slots(const void* kern, size_t dyn_lds, int block_threads = 256);
+int        device_cus();
 hipError_t launch_gather_mfma(const MixerArgs& a, int dtype, hipStream_t st);
 hipError_t launch_scatter_mfma(const MixerArgs& a, int dtype, hipStream_t st);
+// 32x32x16 instances (bf16, D = 32), chosen inside the two launchers above
+bool       mfma32_gather_supported(int dtype, int M, int D, bool masked);
+bool       mfma32_scatter_supported(int dtype, int M, int D, bool masked);
+int        mfma32_gather_resident_slots();
+hipError_t launch_gather_mfma32(const MixerArgs& a, hipStream_t st);
+hipError_t launch_scatter_mfma32(const MixerArgs& a, hipStream_t st);
 
 size_t     causal_lds_bytes(int M, int D, bool decode);
 hipError_t launch_causal_prefill(const CausalArgs& a, int dtype, hipStream_t st);

@@ -612,8 +612,8 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
         const size_t lds = mixer_bwd_lds_bytes(mc, D);
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        // one workgroup per compute unit (256 CUs), ranges a multiple of its 512-token pass
-        const int64_t per_bh = (256 + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H);
+        // one workgroup per compute unit, ranges a multiple of its 512-token pass
+        const int64_t per_bh = (device_cus() + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H);
         int64_t tpw = (a.N + per_bh - 1) / per_bh;
         tpw = ((tpw + 511) / 512) * 512;
         for (int c = 0; c < chunks; ++c) {

@@ -886,6 +886,23 @@ int resident_slots(const void* kern, size_t dyn_lds, int block_threads)
     return slots;
 }
 
+// Compute units of the current device (256 when no device can be queried: host-only planning).
+int device_cus()
+{
+    static int cached[64];
+    static std::mutex mu;
+    std::lock_guard<std::mutex> lock(mu);
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return 256; }
+    if (dev >= 0 && dev < 64 && cached[dev] > 0) return cached[dev];
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    if (dev >= 0 && dev < 64) cached[dev] = cus;
+    return cus;
+}
+
 bool mfma_mixer_supported(int dtype, int M, int D)
 {
     if (dtype != 1 && dtype != 2) return false;
@@ -905,11 +922,13 @@ int mfma_gather_resident_slots(int dtype, int M, int D)
 
 hipError_t launch_gather_mfma(const MixerArgs& a, int dtype, hipStream_t st)
 {
+    if (!a.no_mfma32 && a.gather32 && mfma32_gather_supported(dtype, a.M, a.D, a.mask != nullptr)) return launch_gather_mfma32(a, st);
     return dtype == 1 ? gather_launch_d<bf16_t>(a, st) : gather_launch_d<f16_t>(a, st);
 }
 
 hipError_t launch_scatter_mfma(const MixerArgs& a, int dtype, hipStream_t st)
 {
+    if (!a.no_mfma32 && mfma32_scatter_supported(dtype, a.M, a.D, a.mask != nullptr)) return launch_scatter_mfma32(a, st);
     return dtype == 1 ? scatter_launch_d<bf16_t>(a, st) : scatter_launch_d<f16_t>(a, st);
 }
 

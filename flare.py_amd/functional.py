@@ -97,6 +97,29 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else C.c_void_p(t.data_ptr())
 
 
+_extra_mixer_flags = 0
+
+
+class mixer_flags:
+    """Context manager that ORs FLARE_FLAG_* bits into every mixer descriptor built inside it (e.g.
+    ``_lib.FLAG_MFMA16`` to time or test the 16x16x32 kernels where the 32x32x16 scatter would run,
+    ``_lib.FLAG_GATHER32`` to run the gather on 32x32x16 products as well)."""
+
+    def __init__(self, flags: int):
+        self.flags = int(flags)
+
+    def __enter__(self):
+        global _extra_mixer_flags
+        self.saved = _extra_mixer_flags
+        _extra_mixer_flags |= self.flags
+        return self
+
+    def __exit__(self, *exc):
+        global _extra_mixer_flags
+        _extra_mixer_flags = self.saved
+        return False
+
+
 def _mixer_desc(q4, k, v, y, scale, n_splits, force_generic) -> FlareMixerDesc:
     B, H, N, D = k.shape
     d = FlareMixerDesc()
@@ -104,7 +127,7 @@ def _mixer_desc(q4, k, v, y, scale, n_splits, force_generic) -> FlareMixerDesc:
     d.dtype = _dtype_code(k)
     d.scale = float(scale)
     d.n_splits = int(n_splits)
-    d.flags = _lib.FLAG_FORCE_GENERIC if force_generic else 0
+    d.flags = (_lib.FLAG_FORCE_GENERIC if force_generic else 0) | _extra_mixer_flags
     d.q_stride = _s3(q4)
     d.k_stride = _s3(k)
     d.v_stride = _s3(v if v is not None else k)

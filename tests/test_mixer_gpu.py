@@ -460,3 +460,103 @@ def test_latent_counts_that_are_multiples_of_8(dev, shape, dtype):
         assert got.shape == ref.shape
         err = O.rel_l2(got, ref)
         assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
+
+
+# ---- 32x32x16 kernels (bf16, D = 32, no key mask): scatter at M in {64, 128, 256, 512} (default), gather at
+# M % 256 == 0 (behind FLAG_GATHER32) ----
+@pytest.mark.parametrize("shape", [
+    (1, 1, 1, 256, 32), (1, 2, 5, 256, 32), (1, 2, 31, 256, 32), (1, 2, 33, 256, 32), (2, 2, 127, 256, 32),
+    (1, 2, 129, 256, 32), (1, 3, 1000, 256, 32), (2, 2, 4096 + 17, 256, 32), (1, 2, 3000, 512, 32),
+    (1, 2, 20000, 256, 32), (1, 2, 777, 64, 32), (1, 2, 1999, 128, 32),
+])
+def test_mfma32_shapes_and_ragged_ends(dev, shape):
+    from flare_py_amd import _lib
+    from flare_py_amd import functional as FN
+    q, k, v = make(*shape, torch.bfloat16, seed=3)
+    y, z = check(dev, q, k, v)                  # default: 32x32x16 scatter
+    with FN.mixer_flags(_lib.FLAG_GATHER32):    # 32x32x16 gather as well
+        y32, z32 = check(dev, q, k, v)
+    assert O.rel_l2(y32, y) < 1e-2
+    with FN.mixer_flags(_lib.FLAG_MFMA16):      # the 16x16x32 kernels on the same problem
+        y16, z16 = check(dev, q, k, v)
+    assert O.rel_l2(z, z16) < 5e-3 and O.rel_l2(y, y16) < 1e-2
+
+
+@pytest.mark.parametrize("n_splits", [1, 3, 7, 64])
+def test_mfma32_split_invariance_and_determinism(dev, n_splits):
+    from flare_py_amd import _lib
+    from flare_py_amd import functional as FN
+    q, k, v = make(1, 2, 9000, 256, 32, torch.bfloat16, seed=5)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    with FN.mixer_flags(_lib.FLAG_GATHER32):
+        y, z = F.flare_multihead_mixer(qd, kd, vd, return_z=True, n_splits=n_splits)
+        y2, z2 = F.flare_multihead_mixer(qd, kd, vd, return_z=True, n_splits=n_splits)
+    assert torch.equal(y, y2) and torch.equal(z, z2)
+    yr, zr = O.mixer_explicit(q.float(), k.float(), v.float(), 1.0)
+    assert O.rel_l2(z, zr) <= 2e-2 and O.rel_l2(y, yr) <= 2e-2
+
+
+def test_mfma32_large_scores_take_the_exact_paths(dev):
+    # scores far outside the unshifted window in both directions, along N and along M
+    B, H, N, M, D = 1, 2, 3000, 256, 32
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn(H, M, D, generator=g) * torch.linspace(0.2, 2.0, M)[None, :, None]
+    k = torch.randn(B, H, N, D, generator=g) * torch.linspace(0.2, 3.0, N)[None, None, :, None]
+    v = torch.randn(B, H, N, D, generator=g)
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    s = torch.einsum("hmd,bhnd->bhmn", q.float(), k.float())
+    assert float(s.max()) > 100.0
+    from flare_py_amd import _lib
+    from flare_py_amd import functional as FN
+    check(dev, q, k, v, tol=3e-2)
+    with FN.mixer_flags(_lib.FLAG_GATHER32):
+        check(dev, q, k, v, tol=3e-2)
+        check(dev, q, k, v, n_splits=4, tol=3e-2)
+
+
+@pytest.mark.parametrize("offset", [-30.0, 60.0])
+def test_mfma32_constant_score_offset_stays_on_the_fast_path(dev, offset):
+    # a constant added to every score (one extra head-dim pair) moves all exponentials by e^offset and cancels in
+    # both softmaxes: inside the unshifted window the result must not change
+    q, k, v = make(1, 2, 2000, 256, 32, torch.bfloat16, seed=9)
+    q2, k2 = q.clone(), k.clone()
+    q2[..., 0] = 1.0
+    k2[..., 0] = offset
+    q0, k0 = q.clone(), k.clone()
+    q0[..., 0] = 0.0
+    k0[..., 0] = 0.0
+    from flare_py_amd import _lib
+    from flare_py_amd import functional as FN
+    for flags in (0, _lib.FLAG_GATHER32):
+        with FN.mixer_flags(flags):
+            y0, _ = check(dev, q0, k0, v)
+            y1, _ = check(dev, q2, k2, v)
+        assert O.rel_l2(y1, y0) < 1e-2
+
+
+def test_mfma32_strided_views_per_batch_q_mask_and_lse(dev):
+    B, H, N, M, D = 2, 4, 1500, 256, 32
+    g = torch.Generator().manual_seed(11)
+    kk = torch.randn(B, N, H * D, generator=g).bfloat16()
+    vv = torch.randn(B, N, H * D, generator=g).bfloat16()
+    q = (torch.randn(B, H, M, D, generator=g) * D ** -0.5).bfloat16()      # one latent set per batch element
+    k = kk.view(B, N, H, D).permute(0, 2, 1, 3)
+    v = vv.view(B, N, H, D).permute(0, 2, 1, 3)
+    y = F.flare_multihead_mixer(q.to(dev), k.to(dev), v.to(dev))
+    yr, _ = O.mixer_explicit(q.float(), k.float(), v.float(), 1.0)
+    assert O.rel_l2(y, yr) <= 2e-2
+    # key mask: both halves keep the 16x16x32 kernels, padded rows come out as zeros
+    mask = torch.ones(B, N, dtype=torch.bool)
+    mask[0, 1000:] = False
+    mask[1, ::3] = False
+    ym = F.flare_multihead_mixer(q.to(dev), k.to(dev), v.to(dev), key_mask=mask.to(dev))
+    yr, _ = O.mixer_explicit(q.float(), k.float(), v.float(), 1.0, mask)
+    assert O.rel_l2(ym, yr) <= 2e-2
+    assert (ym.cpu()[0, :, 1000:] == 0).all()
+    # token log-sum-exp of the scatter (the backward needs it)
+    z, lse = F.flare_gather(q.to(dev), k.to(dev), v.to(dev))
+    sc = torch.einsum("bhnd,bhmd->bhnm", k.float(), q.float())
+    want = torch.logsumexp(sc, dim=-1)
+    from flare_py_amd import functional as FN
+    out = FN._mixer_forward(q.to(dev), k.to(dev), v.to(dev), 1.0, None, 0, False, False, True)
+    assert float((out[3].cpu() - want).abs().max()) < 3e-2
