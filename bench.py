@@ -89,6 +89,36 @@ def cpu_baseline(q, k, v, n_sample):
     return torch.cat(outs, dim=1), dt
 
 
+def sustained_clock_mhz(fn, dev, ms_step, probe_ms=8.0):
+    """Shader clock the device holds while `fn` runs back to back: a one-wave probe kernel on a second stream
+    (default priority) brackets `probe_ms` of the constant 100 MHz counter with the shader-cycle counter while
+    the main stream is kept busy with `fn`."""
+    from flare_py_amd import _lib
+
+    lib = _lib.load()
+    side = torch.cuda.Stream(device=dev)
+    out = torch.zeros(2, dtype=torch.int64, device=dev)
+    for _ in range(20):
+        fn()
+    _lib.check(lib.flare_clock_probe(float(probe_ms), out.data_ptr(), side.cuda_stream), "flare_clock_probe")
+    for _ in range(int(1.5 * probe_ms / max(ms_step, 1e-3)) + 4):
+        fn()
+    torch.cuda.synchronize()
+    cyc, ticks = (int(x) for x in out.tolist())
+    return 100.0 * cyc / max(ticks, 1)
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 SETTLE_STEPS = 40   # untimed calls before the warm-up proper: the device needs ~30 ms of work to reach its steady clocks
 
 
@@ -146,7 +176,7 @@ def bench_causal(args, F, dev):
         yr, _ = O.causal_recurrent(qc, kc, vc, dtype=torch.float32)
         dt = time.perf_counter() - t0
         yg, _ = F.flare_causal_prefill(q, kp[:1].contiguous(), vp[:1].contiguous())
-        out["cpu_baseline"] = {"value": round(B * ns / (dt * B), 1), "unit": "tokens/s", "cores": torch.get_num_threads(),
+        out["cpu_baseline"] = {"value": round(B * ns / (dt * B), 1), "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(),
                                "kind": "port", "sample": f"token recurrence (torch, fp32) on batch element 0 of {B}, all {H} heads, "
                                f"{ns} prompt tokens, {dt:.2f} s; value scaled to the {B} batch elements"}
         out["rel_l2_vs_cpu_on_sample"] = O.rel_l2(yg, yr)
@@ -196,7 +226,7 @@ def bench_triple(args, F, dev):
         dt = time.perf_counter() - t0
         _, o = step()
         out["cpu_baseline"] = {"value": round(B * N / dt, 1), "unit": "tokens/s",
-                               "cores": torch.get_num_threads(), "kind": "port",
+                               "cores": torch.get_num_threads(), "cpu": cpu_model(), "kind": "port",
                                "sample": f"einsum restatement (torch, fp32) of the whole workload, {dt:.2f} s"}
         out["rel_l2_vs_cpu_on_sample"] = O.rel_l2(o, o_ref)
     return out
@@ -368,11 +398,21 @@ def main():
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
     tokens_per_s = B * N / (ms_step * 1e-3)
+    # spread: the same loop again in five blocks, each between synchronisations (not part of `value`)
+    blocks = []
+    for _ in range(5):
+        nb = max(1, args.steps // 5)
+        t1 = time.perf_counter()
+        for _ in range(nb):
+            step()
+        torch.cuda.synchronize()
+        blocks.append((time.perf_counter() - t1) * 1e3 / nb)
+    blocks.sort()
 
     # ---- per-kernel durations (HIP events on the launch stream) --------------------------
     z, _ = F.flare_gather(q, k, v)
-    ms_gather = time_events(lambda: F.flare_gather(q, k, v), args.steps, 2)       # split-N kernel + merge
-    ms_scatter = time_events(lambda: F.flare_scatter(q, k, z), args.steps, 2)
+    ms_gather = time_events(lambda: F.flare_gather(q, k, v), args.steps, 10)      # split-N kernel + merge
+    ms_scatter = time_events(lambda: F.flare_scatter(q, k, z), args.steps, 10)
     esz = 2
     bytes_gather = 2 * B * H * N * D * esz          # K and V read once
     bytes_scatter = 2 * B * H * N * D * esz         # K read, Y written
@@ -387,6 +427,10 @@ def main():
     achieved = bytes_dom / (ms_dom * 1e-3) / 1e9
     t_hbm = 4 * B * H * N * D * esz / (HBM_PEAK_GBPS * 1e9)
     t_mfma = 2 * flops_phase / (MFMA_BF16_PEAK_TFLOPS * 1e12)
+    clock_mhz = sustained_clock_mhz(step, dev, ms_step)
+    # the published matrix-core peak is quoted at the 2400 MHz peak engine clock; under this kernel's load the
+    # device sustains clock_mhz, which scales what the matrix cores can deliver
+    mfma_sustained = MFMA_BF16_PEAK_TFLOPS * clock_mhz / 2400.0
     roofline = {
         "bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic_measured[dom],
@@ -395,6 +439,10 @@ def main():
         "mixer_frac_of_roofline": round(max(t_hbm, t_mfma) * 1e3 / ms_step, 4),
         "mixer_tflops": round(2 * flops_phase / (ms_step * 1e-3) / 1e12, 1),
         "mfma_peak_tflops": MFMA_BF16_PEAK_TFLOPS,
+        "sustained_clock_mhz": round(clock_mhz, 0),
+        "mfma_tflops_at_sustained_clock": round(mfma_sustained, 1),
+        "mixer_frac_of_mfma_at_sustained_clock": round(2 * flops_phase / (ms_step * 1e-3) / 1e12 / mfma_sustained, 4),
+        "ms_per_step_blocks_min_median_max": [round(blocks[0], 4), round(blocks[2], 4), round(blocks[-1], 4)],
         "copy_GBps_measured": round(copy_bandwidth(dev), 1),
     }
 
@@ -436,7 +484,7 @@ def main():
         y_gpu = F.flare_multihead_mixer(q, k[:, :, :ns], v[:, :, :ns]).float().cpu()
         rel = float((y_gpu.double() - y_cpu.double()).norm() / y_cpu.double().norm())
         out["cpu_baseline"] = {
-            "value": round(B * ns / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "value": round(B * ns / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(), "kind": "port",
             "sample": f"first {ns} tokens of the same seeded workload, all {H} heads, torch SDPA MATH backend fp32, "
                       f"{dt:.2f} s",
         }

@@ -15,6 +15,19 @@ static __device__ __align__(256) unsigned char scratch[FLARE_STATIC_SCRATCH_BYTE
 
 namespace {
 
+// One wave: shader cycles and 100 MHz ticks that pass while it sleeps for `ticks` of the 100 MHz counter.
+// The loop is bounded by that counter, which never stops, so the wave always exits.
+__global__ void clock_probe_kernel(long long* out, long long ticks)
+{
+    const long long r0 = wall_clock64(), c0 = clock64();
+    while (wall_clock64() - r0 < ticks) __builtin_amdgcn_s_sleep(64);
+    const long long c1 = clock64(), r1 = wall_clock64();
+    if (threadIdx.x == 0) {
+        out[0] = c1 - c0;
+        out[1] = r1 - r0;
+    }
+}
+
 thread_local char g_err[512] = "";
 
 int fail(int code, const char* fmt, ...)
@@ -542,6 +555,16 @@ int flare_mixer_fwd_static(const FlareMixerDesc* desc, const void* q, const void
     if (rc != FLARE_OK) return rc;
     // every partial row and every row of z that is read is written first by this call's own kernels: nothing to clear
     return flare_mixer_fwd(desc, q, k, v, key_mask, y, nullptr, ws, (size_t)FLARE_STATIC_SCRATCH_BYTES, stream);
+}
+
+int flare_clock_probe(double milliseconds, int64_t* out, void* stream)
+{
+    if (!out) return fail(FLARE_EINVAL, "out must not be NULL");
+    if (!(milliseconds > 0.0) || milliseconds > 100.0) return fail(FLARE_EINVAL, "milliseconds must be in (0, 100]");
+    hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                       reinterpret_cast<long long*>(out), (long long)(milliseconds * 1.0e5));
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? FLARE_OK : fail(FLARE_EHIP, "clock probe launch: %s", hipGetErrorString(e));
 }
 
 int flare_causal_workspace_bytes(const FlareCausalDesc* desc, size_t* bytes)

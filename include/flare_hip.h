@@ -19,6 +19,7 @@
  *   flare_mixer_bwd            gradient of flare_multihead_mixer (torch autograd through the two SDPA
  *                              calls upstream; ablation/time_memory_bwd.py:460-478 times fwd+bwd)
  *   flare_mixer_fwd_static     (no counterpart upstream: flare_mixer_fwd without a caller workspace)
+ *   flare_clock_probe          (no counterpart upstream: measurement aid, sustained shader clock)
  *   flare_causal_prefill_fwd   causal restriction of the mixer (README.md:60 names it; the
  *   flare_causal_decode_fwd    reference holds no code for it) following the 3-phase chunk
  *                              scheme of lra/models/triton/causal_linear.py:81-137 and the
@@ -225,6 +226,14 @@ int flare_mixer_fwd(const FlareMixerDesc* desc, const void* q, const void* k, co
 #define FLARE_STATIC_SCRATCH_BYTES (64u << 20)
 int flare_mixer_fwd_static(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
                            const uint8_t* key_mask, void* y, void* stream);
+
+/* Diagnostic with no counterpart in the reference: one wave that reads the shader-clock counter and the
+ * constant 100 MHz counter, sleeps for about `milliseconds` (at most 100) and reads both again.
+ * out[0] = shader cycles, out[1] = 100 MHz ticks (device memory, two int64).  Launched on a second stream
+ * beside the kernels under test it gives the clock the device actually sustains under their load, which is
+ * what the matrix-core peak has to be scaled by (the device lowers its clock when matrix cores, vector units
+ * and HBM all draw power). */
+int flare_clock_probe(double milliseconds, int64_t* out, void* stream);
 
 int flare_causal_workspace_bytes(const FlareCausalDesc* desc, size_t* bytes);
 
