@@ -10,6 +10,7 @@ from .functional import (
     TripleAttentionFunction,
     causal_linear_attention,
     causal_fresh_state,
+    causal_workspace,
     flare_causal_decode,
     flare_causal_decode_step,
     flare_causal_prefill,
@@ -24,6 +25,6 @@ from .serving import GraphedForward
 
 __all__ = [
     "CausalLinear", "causal_linear_attention", "FLARE", "FLAREBlock", "FLAREModel", "FinalLayer", "ResidualMLP", "TripleAttentionFunction",
-    "causal_fresh_state", "flare_causal_decode", "flare_causal_decode_step", "flare_causal_prefill",
+    "causal_fresh_state", "causal_workspace", "flare_causal_decode", "flare_causal_decode_step", "flare_causal_prefill",
     "flare_gather", "flare_multihead_mixer", "flare_scatter", "mixer_kernel_name", "triple_attention", "GraphedForward",
 ]

@@ -88,6 +88,9 @@ SYMBOLS = {
     "flare_causal_workspace_bytes": (C.c_int, [C.POINTER(FlareCausalDesc), C.POINTER(_SZ)]),
     "flare_causal_prefill_fwd": (C.c_int, [C.POINTER(FlareCausalDesc), _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_causal_decode_fwd": (C.c_int, [C.POINTER(FlareCausalDesc), _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "flare_causal_prefill_fwd_lse": (C.c_int, [C.POINTER(FlareCausalDesc), _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "flare_causal_decode_fwd_lse": (C.c_int, [C.POINTER(FlareCausalDesc), _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "flare_causal_join": (C.c_int, [C.c_int32, C.c_int32, C.c_int64, C.c_int32, C.POINTER(_P), C.POINTER(_P), _P, _P]),
     "flare_causal_linear_workspace_bytes": (C.c_int, [C.POINTER(FlareCausalLinearDesc), C.POINTER(_SZ)]),
     "flare_causal_linear_fwd": (C.c_int, [C.POINTER(FlareCausalLinearDesc), _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_mlp_fwd": (C.c_int, [C.POINTER(FlareMlpDesc), _P, _P, _P, _P, _P, _P, _P, _P]),

@@ -13,6 +13,8 @@
 // only a host-side handle; the device address is looked up once per device (static_scratch below).
 static __device__ __align__(256) unsigned char scratch[FLARE_STATIC_SCRATCH_BYTES];
 
+static_assert(FLARE_JOIN_MAX_GROUPS == flare::kJoinMaxGroups, "header and kernel argument block disagree");
+
 namespace {
 
 // One wave: shader cycles and 100 MHz ticks that pass while it sleeps for `ticks` of the 100 MHz counter.
@@ -579,7 +581,7 @@ int flare_causal_workspace_bytes(const FlareCausalDesc* desc, size_t* bytes)
 
 namespace {
 int causal_run(const FlareCausalDesc* desc, bool decode, const void* q, const void* k, const void* v, void* y,
-               float* mu, float* den, float* num, void* workspace, size_t workspace_bytes, void* stream)
+               float* lse_tok, float* mu, float* den, float* num, void* workspace, size_t workspace_bytes, void* stream)
 {
     int rc = check_causal_desc(desc);
     if (rc != FLARE_OK) return rc;
@@ -587,7 +589,7 @@ int causal_run(const FlareCausalDesc* desc, bool decode, const void* q, const vo
         return fail(FLARE_EINVAL, "q, k, v, y, mu, den, num must not be NULL");
     flare::CausalArgs a;
     fill_causal_args(a, desc);
-    a.q = q; a.k = k; a.v = v; a.y = y; a.mu = mu; a.den = den; a.num = num;
+    a.q = q; a.k = k; a.v = v; a.y = y; a.mu = mu; a.den = den; a.num = num; a.lse = lse_tok;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (causal_wants_mfma(desc) && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y)) {
         // matrix-core kernel without a running maximum; it marks the (b,h) it could not validate
@@ -614,14 +616,52 @@ int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const v
                              void* y, float* mu, float* den, float* num, void* workspace,
                              size_t workspace_bytes, void* stream)
 {
-    return causal_run(desc, false, q, k, v, y, mu, den, num, workspace, workspace_bytes, stream);
+    return causal_run(desc, false, q, k, v, y, nullptr, mu, den, num, workspace, workspace_bytes, stream);
+}
+
+int flare_causal_prefill_fwd_lse(const FlareCausalDesc* desc, const void* q, const void* k, const void* v,
+                                 void* y, float* lse_tok, float* mu, float* den, float* num, void* workspace,
+                                 size_t workspace_bytes, void* stream)
+{
+    if (!lse_tok) return fail(FLARE_EINVAL, "lse_tok must not be NULL");
+    return causal_run(desc, false, q, k, v, y, lse_tok, mu, den, num, workspace, workspace_bytes, stream);
 }
 
 int flare_causal_decode_fwd(const FlareCausalDesc* desc, const void* q, const void* k, const void* v,
                             void* y, float* mu, float* den, float* num, void* workspace,
                             size_t workspace_bytes, void* stream)
 {
-    return causal_run(desc, true, q, k, v, y, mu, den, num, workspace, workspace_bytes, stream);
+    return causal_run(desc, true, q, k, v, y, nullptr, mu, den, num, workspace, workspace_bytes, stream);
+}
+
+int flare_causal_decode_fwd_lse(const FlareCausalDesc* desc, const void* q, const void* k, const void* v,
+                                void* y, float* lse_tok, float* mu, float* den, float* num, void* workspace,
+                                size_t workspace_bytes, void* stream)
+{
+    if (!lse_tok) return fail(FLARE_EINVAL, "lse_tok must not be NULL");
+    return causal_run(desc, true, q, k, v, y, lse_tok, mu, den, num, workspace, workspace_bytes, stream);
+}
+
+int flare_causal_join(int32_t dtype, int32_t n_groups, int64_t rows, int32_t D, const void* const* y_groups,
+                      const float* const* lse_groups, void* y, void* stream)
+{
+    if (dtype < FLARE_DT_F32 || dtype > FLARE_DT_F16) return fail(FLARE_EINVAL, "unknown dtype %d", dtype);
+    if (n_groups < 1 || n_groups > FLARE_JOIN_MAX_GROUPS)
+        return fail(FLARE_EINVAL, "n_groups must be in 1..%d (got %d)", FLARE_JOIN_MAX_GROUPS, n_groups);
+    if (rows < 0 || D < 1 || D > 128 || D % 8 != 0) return fail(FLARE_EINVAL, "rows must be >= 0, D a multiple of 8 up to 128");
+    if (!y_groups || !lse_groups || !y) return fail(FLARE_EINVAL, "y_groups, lse_groups, y must not be NULL");
+    flare::CausalJoinArgs a;
+    memset(&a, 0, sizeof(a));
+    for (int g = 0; g < n_groups; ++g) {
+        if (!y_groups[g] || !lse_groups[g]) return fail(FLARE_EINVAL, "group %d has a NULL pointer", g);
+        if (!aligned16(y_groups[g])) return fail(FLARE_EINVAL, "group outputs must be 16-byte aligned");
+        a.yg[g] = y_groups[g];
+        a.lse[g] = lse_groups[g];
+    }
+    if (!aligned16(y)) return fail(FLARE_EINVAL, "y must be 16-byte aligned");
+    a.y = y; a.n_groups = n_groups; a.rows = rows; a.D = D;
+    if (rows == 0) return FLARE_OK;
+    return hip_status(flare::launch_causal_join(a, dtype, static_cast<hipStream_t>(stream)), "causal join launch");
 }
 
 int flare_causal_linear_workspace_bytes(const FlareCausalLinearDesc* desc, size_t* bytes)

@@ -120,7 +120,11 @@ __global__ __launch_bounds__(kThreads) void causal_generic_kernel(CausalArgs a)
             float sum = 0.f;
             for (int m = lane; m < M; m += 64) sum += fast_exp2(sg[t * (M + 1) + m] - mx);
             sum = wave_sum(sum);
-            if (lane == 0) { rmax[t] = mx; rinv[t] = 1.f / sum; }
+            if (lane == 0) {
+                rmax[t] = mx;
+                rinv[t] = 1.f / sum;
+                if (a.lse) a.lse[(int64_t)bh * N + n0 + t] = (mx + __log2f(sum)) * kLn2;
+            }
         }
         __syncthreads();
         // per latent, token by token: running maximum mc_t, denominator relative to it,
@@ -216,7 +220,47 @@ hipError_t launch_dt(const CausalArgs& a, int dtype, hipStream_t st)
     }
 }
 
+// Joins latent groups that ran as causal problems of their own: y[r,:] = sum_g w_g y_g[r,:] with
+// w_g = exp(lse_g[r]) / sum_g' exp(lse_g'[r]).  One thread per 8 consecutive elements of a row (16 bytes of a
+// 16-bit type), fp32 arithmetic, groups visited in order (bit-stable).
+template <typename T>
+__global__ __launch_bounds__(256) void causal_join_kernel(CausalJoinArgs a)
+{
+    const int per_row = a.D / 8;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= a.rows * per_row) return;
+    const int64_t r = idx / per_row;
+    const int c = (int)(idx - r * per_row) * 8;
+    float mx = -INFINITY;
+    for (int g = 0; g < a.n_groups; ++g) mx = fmaxf(mx, a.lse[g][r]);
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float sum = 0.f;
+    for (int g = 0; g < a.n_groups; ++g) {
+        const float w = __expf(a.lse[g][r] - mx);
+        sum += w;
+        const T* src = (const T*)a.yg[g] + r * a.D + c;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = fmaf(w, to_f32(src[e]), acc[e]);
+    }
+    const float inv = 1.f / sum;
+    T* dst = (T*)a.y + r * a.D + c;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dst[e] = from_f32<T>(acc[e] * inv);
+}
+
 }  // namespace
+
+hipError_t launch_causal_join(const CausalJoinArgs& a, int dtype, hipStream_t st)
+{
+    const int64_t threads = a.rows * (a.D / 8);
+    dim3 grid((unsigned)((threads + 255) / 256));
+    switch (dtype) {
+        case 0: hipLaunchKernelGGL(causal_join_kernel<float>, grid, dim3(256), 0, st, a); break;
+        case 1: hipLaunchKernelGGL(causal_join_kernel<bf16_t>, grid, dim3(256), 0, st, a); break;
+        default: hipLaunchKernelGGL(causal_join_kernel<f16_t>, grid, dim3(256), 0, st, a); break;
+    }
+    return hipGetLastError();
+}
 
 size_t causal_lds_bytes(int M, int D, bool decode)
 {

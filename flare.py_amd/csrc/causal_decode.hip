@@ -193,6 +193,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void causal_decode_kernel(CausalArg
                 const float o = ys * __builtin_amdgcn_rcpf(r);
                 bad = bad || !(r >= kLMin && r <= kLMax) || !(fabsf(o) <= 3.0e38f);
                 y[(int64_t)n * a.ys[2] + lane] = E::bits(o);
+                if (a.lse && lane == 0) a.lse[(int64_t)bh * N + n] = (cref + __log2f(r)) * kLn2;
             }
         }
     }

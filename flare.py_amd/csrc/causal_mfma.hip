@@ -437,6 +437,7 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
                 bad = bad || !(r >= kLMin && r <= kLMax) || !(fabsf(o[0]) + fabsf(o[1]) + fabsf(o[2]) + fabsf(o[3]) <= 3.0e38f);
                 *reinterpret_cast<uint2*>(y + (int64_t)(n0 + t) * a.ys[2] + d4) =
                     make_uint2(M_::pack2(o[0], o[1]), M_::pack2(o[2], o[3]));
+                if (a.lse && d4 == 0) a.lse[(int64_t)bh * a.N + n0 + t] = (cref + __log2f(r)) * kLn2;
             }
         }
     }
@@ -745,7 +746,10 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 inv[r] = 1.f / rsum[r];
-                if (4 * g + r < tbw) bad = bad || !(rsum[r] >= kLMin && rsum[r] <= kLMax);
+                if (4 * g + r < tbw) {
+                    bad = bad || !(rsum[r] >= kLMin && rsum[r] <= kLMax);
+                    if (a.lse && c16 == 0) a.lse[(int64_t)bh * a.N + tbase + 4 * g + r] = (cref + __log2f(rsum[r])) * kLn2;
+                }
             }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {

@@ -81,6 +81,7 @@ struct MixerArgs {
 struct CausalArgs {
     const void* q; const void* k; const void* v; void* y;
     float* mu; float* den; float* num;   // state, natural-log units for mu
+    float* lse;                          // [B,H,N] or null: natural log of each token's softmax sum over the latents
     int* flags;                          // [B*H] or null: per-(b,h) "redo with the fp32 kernel" marks
     float* seg_den; float* seg_num;      // [B*H, n_segs, M] and [B*H, n_segs, M, D]: per-segment states (matrix-core prefill)
     int n_segs, seg_len;                 // token segments processed in parallel; seg_len is a multiple of 16
@@ -88,6 +89,15 @@ struct CausalArgs {
     int chunk;
     float scale;
     int64_t qs[3], ks[3], vs[3], ys[3];
+};
+
+constexpr int kJoinMaxGroups = 16;
+struct CausalJoinArgs {
+    const void* yg[kJoinMaxGroups];      // per group: outputs [rows, D], contiguous, normalised within the group
+    const float* lse[kJoinMaxGroups];    // per group: [rows] natural log of the group's softmax sum
+    void* y;                             // [rows, D]
+    int n_groups, D;
+    int64_t rows;
 };
 
 struct TripleArgs {
@@ -173,6 +183,7 @@ hipError_t launch_gather_mfma32(const MixerArgs& a, hipStream_t st);
 hipError_t launch_scatter_mfma32(const MixerArgs& a, hipStream_t st);
 
 size_t     causal_lds_bytes(int M, int D, bool decode);
+hipError_t launch_causal_join(const CausalJoinArgs& a, int dtype, hipStream_t st);
 hipError_t launch_causal_prefill(const CausalArgs& a, int dtype, hipStream_t st);
 hipError_t launch_causal_decode(const CausalArgs& a, int dtype, hipStream_t st);
 bool       causal_mfma_supported(int dtype, int M, int D);

@@ -160,7 +160,8 @@ def mixer_kernel_name(q, k, v=None, scale=1.0, force_generic=False) -> str:
         q = q.repeat(*([1] * (q.dim() - 2)), r, 1)
     M, D = q.shape[-2], k.shape[-1]
     if (M % 32 != 0 and not force_generic and q.dtype == k.dtype and D < 64 and k.dtype in (torch.bfloat16, torch.float16)
-            and k.device.type == "cuda"):           # dead latents and a wider head, see _mixer_odd_latents
+            and k.device.type == "cuda" and _dead_latent_bias(float(scale), k.dtype) is not None):
+        # dead latents and a wider head, see _mixer_odd_latents
         Dp = 16 if D < 16 else 32 if D < 32 else 64
         q = q.new_zeros(*q.shape[:-2], -(-M // 32) * 32, Dp)
         k, v = _pad_last(k, Dp - D), None
@@ -232,6 +233,8 @@ def _hip_backward_ok(q, k, v, key_mask, force_generic) -> bool:
         return False
     k, v = _rows_last_contig(k), _rows_last_contig(v)
     q4 = _q4(q, k.shape[0])
+    if any(t.data_ptr() % 16 for t in (q4, k, v)):      # the kernels read 16-byte chunks: a view that starts off
+        return False                                    # that grid differentiates through the torch recomputation
     d = _mixer_desc(q4, k, v, None, 1.0, 0, False)
     need = C.c_size_t(0)
     return _lib.load().flare_mixer_bwd_workspace_bytes(C.byref(d), C.byref(need)) == _lib.FLARE_OK
@@ -363,12 +366,21 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
                                     force_generic, token_major_out)
         return (out[0], out[1][..., :M, :]) if return_z else out
     if (q.shape[-2] % 32 != 0 and not force_generic and q.dtype == k.dtype == v.dtype and D < 64
-            and k.dtype in (torch.bfloat16, torch.float16) and k.device.type == "cuda"):
+            and k.dtype in (torch.bfloat16, torch.float16) and k.device.type == "cuda"
+            and _dead_latent_bias(float(scale), k.dtype) is not None):
         return _mixer_odd_latents(q, k, v, float(scale), key_mask, return_z, n_splits, token_major_out)
     pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype == v.dtype else 0
     if pad:
         q, k, v = _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad)
-    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+    needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
+    if needs_grad and return_z:
+        # z is handed out and may enter a loss of its own: take the two differentiable halves, so that gradients
+        # reach q, k, v through z as well as through y (the fused function below treats z as an internal value)
+        z, _ = flare_gather(q, k, v, scale, key_mask, n_splits, force_generic)
+        y = flare_scatter(q, k, z, scale, key_mask, force_generic)
+        if token_major_out:
+            y = y.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    elif needs_grad:
         y, z = _MixerFn.apply(q, k, v, float(scale), key_mask, n_splits, force_generic, token_major_out)
     else:
         y, z = _mixer_forward(q, k, v, float(scale), key_mask, n_splits, force_generic, token_major_out)
@@ -387,10 +399,22 @@ def _latent_copies(q, k, force_generic) -> int:
     return 32 // math.gcd(M, 32)
 
 
+def _dead_latent_bias(scale: float, dtype):
+    """The entry a dead latent's query holds in the column of ones (see _mixer_odd_latents): its score is
+    scale * bias, which has to sit at least 200 below any real score's neighbourhood whatever the scale is.
+    None when the element type cannot hold such a value (f16 with a scale below about 200 / 60000)."""
+    if not scale > 0.0:
+        return None
+    need = max(16384.0, 256.0 / scale)        # 256 rather than 200: room for the rounding to the element type
+    limit = 60000.0 if dtype == torch.float16 else 1.0e30
+    return -need if need <= limit else None
+
+
 def _mixer_odd_latents(q, k, v, scale, key_mask, return_z, n_splits, token_major_out):
     """A latent count that is not a multiple of 32 on the matrix-core kernels: the latents are filled up with dead
     ones.  In the gather a dead latent is a zero query whose row of z is never used.  In the scatter it must get no
-    weight: k receives one extra column of ones and the dead queries hold -16384 there (the real ones 0), which takes
+    weight: k receives one extra column of ones and the dead queries hold a large negative number there (the real
+    ones 0; -16384, or -256 / scale when the scale is small, so that scale * bias stays below -200), which takes
     their scores out of every token's softmax.  The extra column rides in the zero padding of the head dim (D grows to
     the next of 16, 32, 64 that leaves room for it).  Gradients come from the two halves' torch recomputation."""
     M, D = q.shape[-2], k.shape[-1]
@@ -400,7 +424,7 @@ def _mixer_odd_latents(q, k, v, scale, key_mask, return_z, n_splits, token_major
     dead = qz.new_zeros(*qz.shape[:-2], Mp - M, Dp)
     q_gather = torch.cat([qz, dead], dim=-2)
     dead_s = dead.clone()
-    dead_s[..., D] = -16384.0
+    dead_s[..., D] = _dead_latent_bias(scale, k.dtype)
     q_scatter = torch.cat([qz, dead_s], dim=-2)
     kp = _pad_last(k, Dp - D).clone() if Dp - D else k
     kp[..., D] = 1.0
@@ -549,25 +573,6 @@ def causal_fresh_state(B, H, M, D, device):
     return mu, den, num
 
 
-def _scatter_lse(q, k, scale):
-    """ln sum_m exp(scale <k_n, q_m>) per token, [B,H,N] fp32, from flare_scatter_fwd_lse (its y goes to a scratch
-    tensor): the weight a group of latents carries in a softmax over several groups."""
-    lib = _lib.load()
-    k = _rows_last_contig(k)
-    B, H, N, D = k.shape
-    q4 = _q4(q.to(k.dtype), B)
-    M = q4.shape[2]
-    y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
-    z = torch.zeros((B, H, M, D), dtype=torch.float32, device=k.device)
-    lse = torch.empty((B, H, N), dtype=torch.float32, device=k.device)
-    d = _mixer_desc(q4, k, k, y, scale, 0, False)
-    with _on_device(k.device):
-        rc = lib.flare_scatter_fwd_lse(C.byref(d), _ptr(q4), _ptr(k), _ptr(z), None, _ptr(y), _ptr(lse),
-                                       C.c_void_p(_stream_ptr(k.device)))
-    _lib.check(rc, "flare_scatter_fwd_lse")
-    return lse
-
-
 def _causal_latent_groups(M, D):
     """Sizes of the latent groups a 16-bit causal problem is run in when the matrix-core kernels do not take its M
     in one piece: 256 (heads up to 32) or 128 latents, then powers of two down to 32 for the rest.  [] when M is not
@@ -589,7 +594,27 @@ def _causal_latent_groups(M, D):
 CAUSAL_REPLICATE_DECODE_MIN_TOKENS = 32
 
 
-def _causal_call(entry, q, k, v, scale, chunk, state):
+def _causal_join(ys, lses):
+    """y = sum_g softmax_g(lse_g) y_g in one launch (flare_causal_join)."""
+    lib = _lib.load()
+    if ys[0].shape[-1] % 8 != 0 or len(ys) > 16:      # rows the join kernel's 16-byte accesses do not fit
+        w = torch.softmax(torch.stack(lses), dim=0).unsqueeze(-1)
+        return (w * torch.stack([t.float() for t in ys])).sum(0).to(ys[0].dtype)
+    ys = [t.contiguous() for t in ys]
+    lses = [t.contiguous() for t in lses]
+    y = torch.empty_like(ys[0])
+    G = len(ys)
+    yp = (C.c_void_p * G)(*[t.data_ptr() for t in ys])
+    lp = (C.c_void_p * G)(*[t.data_ptr() for t in lses])
+    rows = y.numel() // y.shape[-1]
+    with _on_device(y.device):
+        rc = lib.flare_causal_join(_dtype_code(y), G, rows, y.shape[-1], yp, lp, _ptr(y), C.c_void_p(_stream_ptr(y.device)))
+    _lib.check(rc, "flare_causal_join")
+    return y
+
+
+def _causal_call(entry, q, k, v, scale, chunk, state, want_lse=False, inplace=False, workspace=None, out=None):
+    """(y, state) or, with want_lse, (y, state, lse) where lse [B,H,N] is each token's log-sum-exp over the latents."""
     _require_cuda(q, k, v)
     D = k.shape[-1]
     M = q.shape[-2]
@@ -600,13 +625,18 @@ def _causal_call(entry, q, k, v, scale, chunk, state):
         # copy carries the same running state z_m(t), and the softmax over the r*M copies gives each 1/r of the
         # weight latent m had.  So a power-of-two latent count below 128 is tiled up to 128 (state in and out
         # likewise) instead of taking the fp32 kernel.
+        if inplace:
+            raise ValueError("inplace=True needs a latent count the kernels take as it is (this one runs as copies)")
         r = 128 // M
         qr = q.repeat(*([1] * (q.dim() - 2)), r, 1)
         if state is not None:
             mu, den, num = state
             state = (mu.repeat(1, 1, r), den.repeat(1, 1, r), num.repeat(1, 1, r, 1))
-        y, (mu, den, num) = _causal_call(entry, qr, k, v, scale, chunk, state)
-        return y, (mu[..., :M].contiguous(), den[..., :M].contiguous(), num[..., :M, :].contiguous())
+        res = _causal_call(entry, qr, k, v, scale, chunk, state, want_lse=want_lse)
+        mu, den, num = res[1]
+        st = (mu[..., :M].contiguous(), den[..., :M].contiguous(), num[..., :M, :].contiguous())
+        # the r copies of every latent multiply each token's softmax sum by r
+        return (res[0], st, res[2] - math.log(r)) if want_lse else (res[0], st)
     groups = _causal_latent_groups(M, D) if k.dtype in (torch.bfloat16, torch.float16) else []
     if len(groups) > 1 and q.shape[-1] == D and v.shape == k.shape and k.dim() == 4:
         # A latent count the matrix-core kernels do not take in one piece (256 latents with a head above 32 exceed a
@@ -614,31 +644,56 @@ def _causal_call(entry, q, k, v, scale, chunk, state):
         # group of latents is a causal problem of its own whose y_g is normalised within the group, and
         # y = sum_g w_g y_g with w_g = S_g / sum_g' S_g', S_g(t) = sum over the group of exp(scale <k_t, q_m>);
         # the state is per latent and is cut and joined along M.
+        if inplace:
+            raise ValueError("inplace=True needs a latent count the kernels take in one piece (this one runs in groups)")
         ys, sts, lses, m0 = [], [], [], 0
         for g in groups:
             sl = slice(m0, m0 + g)
             m0 += g
             st_g = None if state is None else (state[0][..., sl], state[1][..., sl], state[2][..., sl, :])
-            y_g, st_g = _causal_call(entry, q[..., sl, :], k, v, scale, chunk, st_g)
-            ys.append(y_g.float())
+            y_g, st_g, lse_g = _causal_call(entry, q[..., sl, :], k, v, scale, chunk, st_g, want_lse=True)
+            ys.append(y_g)
             sts.append(st_g)
-            lses.append(_scatter_lse(q[..., sl, :], k, scale))
-        w = torch.softmax(torch.stack(lses), dim=0).unsqueeze(-1)
-        y = (w * torch.stack(ys)).sum(0).to(k.dtype)
-        return y, tuple(torch.cat(parts, dim=2) for parts in zip(*sts))
+            lses.append(lse_g)
+        y = _causal_join(ys, lses)
+        st = tuple(torch.cat(parts, dim=2) for parts in zip(*sts))
+        if want_lse:
+            return y, st, torch.logsumexp(torch.stack(lses), dim=0)
+        return y, st
     if (k.dtype in (torch.bfloat16, torch.float16) and (D < 32 and M in (128, 256) or 32 < D < 64 and M == 128)
             and q.shape[-1] == D and v.shape == k.shape):
         # the matrix-core causal kernels take D = 32 and 64: any other head up to 64 gets zero columns (scores and the
         # first D columns of every output and of the state's numerators are unchanged) instead of the fp32 kernel
+        if inplace:
+            raise ValueError("inplace=True needs a head dim the kernels take as it is (this one is zero-padded)")
         pad = (32 if D < 32 else 64) - D
         if state is not None:
             state = (state[0], state[1], _pad_last(state[2], pad))
-        y, (mu, den, num) = _causal_call_launch(entry, _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad), scale, chunk, state)
-        return y[..., :D], (mu, den, num[..., :D].contiguous())
-    return _causal_call_launch(entry, q, k, v, scale, chunk, state)
+        res = _causal_call_launch(entry, _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad), scale, chunk, state, want_lse)
+        mu, den, num = res[1]
+        st = (mu, den, num[..., :D].contiguous())
+        return (res[0][..., :D], st, res[2]) if want_lse else (res[0][..., :D], st)
+    return _causal_call_launch(entry, q, k, v, scale, chunk, state, want_lse, inplace, workspace, out)
 
 
-def _causal_call_launch(entry, q, k, v, scale, chunk, state):
+def causal_workspace(q, k) -> torch.Tensor:
+    """A workspace for flare_causal_* calls on operands of these shapes (for callers that reuse one across calls,
+    e.g. a decode loop with inplace=True)."""
+    B, H, N, D = k.shape
+    y = torch.empty(0, dtype=k.dtype, device=k.device)
+    d = FlareCausalDesc()
+    d.B, d.H, d.N, d.M, d.D = B, H, N, q.shape[-2], D
+    d.dtype = _dtype_code(k)
+    d.scale = 1.0
+    q4 = _q4(q, B)
+    d.q_stride, d.k_stride, d.v_stride = _s3(q4), _s3(k), _s3(k)
+    d.y_stride = _lib.I3(H * N * D, N * D, D)
+    need = C.c_size_t(0)
+    _lib.check(_lib.load().flare_causal_workspace_bytes(C.byref(d), C.byref(need)), "flare_causal_workspace_bytes")
+    return torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
+
+
+def _causal_call_launch(entry, q, k, v, scale, chunk, state, want_lse=False, inplace=False, workspace=None, out=None):
     lib = _lib.load()
     if q.dtype != k.dtype:
         q = q.to(k.dtype)
@@ -651,11 +706,22 @@ def _causal_call_launch(entry, q, k, v, scale, chunk, state):
     M = q4.shape[2]
     if state is None:
         mu, den, num = causal_fresh_state(B, H, M, D, k.device)
+    elif inplace:
+        mu, den, num = state
+        for s_ in (mu, den, num):
+            if s_.dtype != torch.float32 or s_.device != k.device or not s_.is_contiguous():
+                raise ValueError("inplace=True advances the given state tensors: they must be contiguous fp32 tensors on k's device")
     else:
         mu, den, num = (s.to(device=k.device, dtype=torch.float32).contiguous().clone() for s in state)
-        if mu.shape != (B, H, M) or den.shape != (B, H, M) or num.shape != (B, H, M, D):
-            raise ValueError("state must be (mu[B,H,M], den[B,H,M], num[B,H,M,D])")
-    y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    if mu.shape != (B, H, M) or den.shape != (B, H, M) or num.shape != (B, H, M, D):
+        raise ValueError("state must be (mu[B,H,M], den[B,H,M], num[B,H,M,D])")
+    if out is None:
+        y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    else:
+        y = out
+        if y.shape != (B, H, N, D) or y.dtype != k.dtype or y.device != k.device or y.stride(-1) != 1:
+            raise ValueError("out must be a [B,H,N,D] tensor of k's dtype and device with contiguous rows")
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=k.device) if want_lse else None
     d = FlareCausalDesc()
     d.B, d.H, d.N, d.M, d.D = B, H, N, M, D
     d.dtype = _dtype_code(k)
@@ -664,14 +730,22 @@ def _causal_call_launch(entry, q, k, v, scale, chunk, state):
     d.q_stride, d.k_stride, d.v_stride, d.y_stride = _s3(q4), _s3(k), _s3(v), _s3(y)
     st = C.c_void_p(_stream_ptr(k.device))
     with _on_device(k.device):
-        need = C.c_size_t(0)
-        _lib.check(lib.flare_causal_workspace_bytes(C.byref(d), C.byref(need)), "flare_causal_workspace_bytes")
-        ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
-        fn = lib.flare_causal_prefill_fwd if entry == "prefill" else lib.flare_causal_decode_fwd
-        rc = fn(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(y), _ptr(mu), _ptr(den), _ptr(num), _ptr(ws),
-                ws.numel(), st)
+        if workspace is None:
+            need = C.c_size_t(0)
+            _lib.check(lib.flare_causal_workspace_bytes(C.byref(d), C.byref(need)), "flare_causal_workspace_bytes")
+            ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
+        else:
+            ws = workspace          # the library checks its size and alignment
+        if want_lse:
+            fn = lib.flare_causal_prefill_fwd_lse if entry == "prefill" else lib.flare_causal_decode_fwd_lse
+            rc = fn(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(y), _ptr(lse), _ptr(mu), _ptr(den), _ptr(num), _ptr(ws),
+                    ws.numel(), st)
+        else:
+            fn = lib.flare_causal_prefill_fwd if entry == "prefill" else lib.flare_causal_decode_fwd
+            rc = fn(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(y), _ptr(mu), _ptr(den), _ptr(num), _ptr(ws),
+                    ws.numel(), st)
     _lib.check(rc, f"flare_causal_{entry}_fwd")
-    return y, (mu, den, num)
+    return (y, (mu, den, num), lse) if want_lse else (y, (mu, den, num))
 
 
 def flare_causal_prefill(q, k, v, scale: float = 1.0, chunk: int = 0, state=None):
@@ -682,17 +756,23 @@ def flare_causal_prefill(q, k, v, scale: float = 1.0, chunk: int = 0, state=None
     return _causal_call("prefill", q, k, v, scale, chunk, state)
 
 
-def flare_causal_decode(q, k, v, state, scale: float = 1.0):
-    """n recurrent single-token steps in one launch; k, v are [B,H,n,D]."""
-    return _causal_call("decode", q, k, v, scale, 0, state)
+def flare_causal_decode(q, k, v, state, scale: float = 1.0, inplace: bool = False, workspace=None, out=None):
+    """n recurrent single-token steps in one launch; k, v are [B,H,n,D].
+
+    By default the incoming state is left as it was and a new one is returned.  inplace=True advances the given
+    state tensors themselves (contiguous fp32 on the device; returned again), `workspace` (from causal_workspace)
+    and `out` ([B,H,n,D]) let a decode loop reuse its buffers, so that a step allocates nothing and can be
+    captured in a HIP graph.  In-place calls need a shape the kernels take directly (M in {128, 256} with
+    D in {32, 64} for 16-bit inputs, or anything the fp32 kernel takes)."""
+    return _causal_call("decode", q, k, v, scale, 0, state, inplace=inplace, workspace=workspace, out=out)
 
 
-def flare_causal_decode_step(q, k_t, v_t, state, scale: float = 1.0):
-    """One token: k_t, v_t are [B,H,D] or [B,H,1,D]."""
+def flare_causal_decode_step(q, k_t, v_t, state, scale: float = 1.0, inplace: bool = False, workspace=None, out=None):
+    """One token: k_t, v_t are [B,H,D] or [B,H,1,D] (out, if given, [B,H,1,D]).  See flare_causal_decode."""
     squeeze = k_t.dim() == 3
     if squeeze:
         k_t, v_t = k_t.unsqueeze(2), v_t.unsqueeze(2)
-    y, st = _causal_call("decode", q, k_t, v_t, scale, 0, state)
+    y, st = _causal_call("decode", q, k_t, v_t, scale, 0, state, inplace=inplace, workspace=workspace, out=out)
     return (y.squeeze(2) if squeeze else y), st
 
 

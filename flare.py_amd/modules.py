@@ -129,7 +129,11 @@ class FLARE(nn.Module):
         q = self.latent_q.view(self.num_heads, self.num_latents, self.head_dim)
         cd = self._fusable(x, return_scores)
         D = self.head_dim
-        if cd is not None and D in (4, 8) and self.num_latents % 32 == 0 and not self.qk_norm:
+        narrow = (cd is not None and D in (4, 8) and self.num_latents % 32 == 0 and not self.qk_norm
+                  # head-padded rows exist for the chain of square layers only: an expanding two-layer k/v projection
+                  # takes the generic fused branch below, where the mixer pads the heads itself
+                  and not fused._expand_factor(self.k_proj, C) and not fused._expand_factor(self.v_proj, C))
+        if narrow:
             # narrow heads: the projections write k, v head-padded to 16 columns, which is what the mixer's
             # matrix-core kernels take, and the output projection reads the mixer's padded rows: no copies between
             H = self.num_heads

@@ -9,8 +9,12 @@ shape and replays it; there is no tracing compiler behind it and nothing is spec
     y = fwd(x)            # first call with a new shape: warm-up + capture; later calls: copy in, replay
 
 The returned tensor is the graph's static output buffer: it is overwritten by the next call with the same shape
-(clone it to keep it).  The weights are read at replay time, but the 16-bit copies the fused launches use are
-packed when the graph is captured: call `reset()` after changing parameters.
+(clone it to keep it).  A captured graph reads the 16-bit operand copies that the fused launches cache on the
+modules (packed weights, the cast latent queries).  Every graph keeps those tensors alive, so an eager forward
+that rebuilds a module's cache (another compute dtype, an optimizer step, `load_state_dict`) can never free
+memory a graph still reads; and every call compares the versions and addresses of the module's parameters and
+buffers with those seen at capture and captures again when any of them changed, so a replay never computes
+with operands packed from old weights.
 """
 from __future__ import annotations
 
@@ -37,6 +41,22 @@ class GraphedForward:
             return contextlib.nullcontext()
         return torch.autocast("cuda", dtype=self.autocast_dtype)
 
+    def _param_key(self):
+        """Versions and addresses of everything the forward reads: an in-place update bumps the version, a
+        replaced tensor changes the address."""
+        return tuple((t.data_ptr(), t._version) for t in list(self.module.parameters()) + list(self.module.buffers()))
+
+    def _cached_operands(self):
+        """The operand caches the fused launches left on the modules during warm-up (their tensors' addresses are
+        baked into the graph)."""
+        keep = []
+        for m in self.module.modules():
+            for name in ("_flare_packed", "_q_cache"):
+                c = getattr(m, name, None)
+                if c is not None:
+                    keep.append(c)
+        return keep
+
     def _capture(self, x):
         static_x = x.clone()
         with torch.no_grad(), self._context():
@@ -49,18 +69,20 @@ class GraphedForward:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 static_y = self.module(static_x)
-        return graph, static_x, static_y
+        return graph, static_x, static_y, self._param_key(), self._cached_operands()
 
     def __call__(self, x: torch.Tensor):
         if x.device.type != "cuda":
             raise ValueError("GraphedForward replays HIP graphs: the input must live on a HIP device")
         key = (tuple(x.shape), x.dtype, x.device.index)
         entry = self._graphs.get(key)
+        if entry is not None and entry[3] != self._param_key():
+            entry = None                      # parameters changed since the capture: its packed operands are stale
         if entry is None:
             if self.module.training:
                 raise RuntimeError("GraphedForward captures inference forwards: call module.eval() first")
             entry = self._graphs[key] = self._capture(x)
-        graph, static_x, static_y = entry
+        graph, static_x, static_y = entry[:3]
         static_x.copy_(x)
         graph.replay()
         return static_y

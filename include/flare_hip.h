@@ -24,6 +24,9 @@
  *   flare_causal_decode_fwd    reference holds no code for it) following the 3-phase chunk
  *                              scheme of lra/models/triton/causal_linear.py:81-137 and the
  *                              token recurrence of causal_linear.py:317-336
+ *   flare_causal_*_fwd_lse     the same with each token's log-sum-exp over the latents; flare_causal_join
+ *                              combines latent groups with it (softmax over all latents = softmax over the
+ *                              groups' sums times the softmax within each group)
  *   flare_causal_linear_fwd    CausalLinear.apply lra/models/triton/causal_linear.py:23-145
  *                              == linear_causal_reference causal_linear.py:317-336
  *   flare_mlp_fwd              ResidualMLP.forward pdebench/models/flare.py:45-59 (and lra/models/
@@ -248,6 +251,22 @@ int flare_causal_prefill_fwd(const FlareCausalDesc* desc, const void* q, const v
 int flare_causal_decode_fwd(const FlareCausalDesc* desc, const void* q, const void* k,
                             const void* v, void* y, float* mu, float* den, float* num,
                             void* workspace, size_t workspace_bytes, void* stream);
+
+/* The same two entry points, also returning each token's log-sum-exp over the latents, lse_tok [B,H,N]
+ * (natural log, contiguous): what joins latent groups that run as causal problems of their own. */
+int flare_causal_prefill_fwd_lse(const FlareCausalDesc* desc, const void* q, const void* k,
+                                 const void* v, void* y, float* lse_tok, float* mu, float* den, float* num,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+int flare_causal_decode_fwd_lse(const FlareCausalDesc* desc, const void* q, const void* k,
+                                const void* v, void* y, float* lse_tok, float* mu, float* den, float* num,
+                                void* workspace, size_t workspace_bytes, void* stream);
+
+/* Join of latent groups: y[r,:] = sum_g softmax_g(lse_groups[g][r]) * y_groups[g][r,:] over rows = B*H*N rows of
+ * D elements (all contiguous, element type dtype, D a multiple of 8, at most FLARE_JOIN_MAX_GROUPS groups).
+ * The softmax over all M latents of a token splits over groups of latents this way. */
+#define FLARE_JOIN_MAX_GROUPS 16
+int flare_causal_join(int32_t dtype, int32_t n_groups, int64_t rows, int32_t D, const void* const* y_groups,
+                      const float* const* lse_groups, void* y, void* stream);
 
 int flare_causal_linear_workspace_bytes(const FlareCausalLinearDesc* desc, size_t* bytes);
 

@@ -352,3 +352,112 @@ def test_latent_group_sizes():
     assert fn._causal_latent_groups(256, 33) == [128, 128] and fn._causal_latent_groups(224, 16) == [128, 64, 32]
     assert fn._causal_latent_groups(768, 32) == [256, 256, 256] and fn._causal_latent_groups(160, 64) == [128, 32]
     assert fn._causal_latent_groups(128, 65) == []
+
+
+# ---- per-token log-sum-exp over the latents (what joins latent groups), from every kernel that writes y ----
+@pytest.mark.parametrize("shape,dtype,chunk", [
+    ((1, 2, 300, 128, 64), torch.bfloat16, 0),       # 64-token chunk kernel
+    ((1, 2, 1200, 128, 32), torch.float16, 256),     # the same in several segments
+    ((1, 1, 200, 256, 32), torch.bfloat16, 0),       # 16-token block kernel
+    ((2, 1, 90, 24, 8), torch.float32, 0),           # fp32 kernel
+    ((1, 2, 150, 64, 32), torch.bfloat16, 0),        # copies of every latent
+    ((1, 2, 100, 128, 16), torch.bfloat16, 0),       # zero-padded head
+])
+def test_token_lse_of_prefill_and_decode(dev, shape, dtype, chunk):
+    from flare_py_amd import functional as FN
+    B, H, N, M, D = shape
+    q, k, v = make(*shape, dtype, seed=41)
+    scale = 0.9
+    want = torch.logsumexp(scale * torch.einsum("bhnd,hmd->bhnm", k.double(), q.double()), dim=-1)
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    y, st, lse = FN._causal_call("prefill", q.to(dev), k.to(dev), v.to(dev), scale, chunk, None, want_lse=True)
+    assert lse.shape == (B, H, N) and float((lse.double().cpu() - want).abs().max()) <= tol
+    y0, _ = F.flare_causal_prefill(q.to(dev), k.to(dev), v.to(dev), scale=scale, chunk=chunk)
+    assert torch.equal(y, y0)                        # asking for the sums changes nothing else
+    # decode: the last 40 tokens as steps after a prefill of the rest
+    n0 = N - 40
+    _, st = F.flare_causal_prefill(q.to(dev), k[:, :, :n0].contiguous().to(dev), v[:, :, :n0].contiguous().to(dev), scale=scale)
+    _, _, lse_d = FN._causal_call("decode", q.to(dev), k[:, :, n0:].contiguous().to(dev), v[:, :, n0:].contiguous().to(dev),
+                                  scale, 0, st, want_lse=True)
+    assert float((lse_d.double().cpu() - want[:, :, n0:]).abs().max()) <= tol
+
+
+def test_group_join_kernel(dev):
+    from flare_py_amd import functional as FN
+    g = torch.Generator().manual_seed(43)
+    ys = [torch.randn(2, 3, 50, 32, generator=g).bfloat16() for _ in range(3)]
+    lses = [torch.randn(2, 3, 50, generator=g) * 3 for _ in range(3)]
+    got = FN._causal_join([t.to(dev) for t in ys], [t.to(dev) for t in lses])
+    w = torch.softmax(torch.stack(lses).double(), dim=0).unsqueeze(-1)
+    want = (w * torch.stack([t.double() for t in ys])).sum(0)
+    assert got.dtype == torch.bfloat16 and O.rel_l2(got, want) <= 5e-3
+    assert torch.equal(got, FN._causal_join([t.to(dev) for t in ys], [t.to(dev) for t in lses]))
+
+
+# ---- decoding token by token: state advanced in place, buffers reused, nothing allocated per step ----
+def test_single_step_calls_equal_one_launch_bit_for_bit(dev):
+    B, H, M, D, NP, ND = 2, 4, 128, 64, 512, 256           # config 4's M, D and step count
+    q, k, v = make(B, H, NP + ND, M, D, torch.bfloat16, seed=45)
+    qd = q.to(dev)
+    kp, vp = k[:, :, :NP].contiguous().to(dev), v[:, :, :NP].contiguous().to(dev)
+    kd, vd = k[:, :, NP:].contiguous().to(dev), v[:, :, NP:].contiguous().to(dev)
+    _, st0 = F.flare_causal_prefill(qd, kp, vp)
+    y_all, st_all = F.flare_causal_decode(qd, kd, vd, st0)                 # 256 steps in one launch
+    st = tuple(s.clone() for s in st0)
+    ws = F.causal_workspace(qd, kd[:, :, :1])
+    y_steps = torch.empty_like(y_all)
+    ptrs = [s.data_ptr() for s in st]
+    for t in range(ND):
+        _, st_t = F.flare_causal_decode_step(qd, kd[:, :, t:t + 1], vd[:, :, t:t + 1], st, inplace=True, workspace=ws,
+                                             out=y_steps[:, :, t:t + 1])
+        assert [s.data_ptr() for s in st_t] == ptrs        # the same tensors, advanced
+    assert torch.equal(y_steps, y_all)
+    for a, b in zip(st, st_all):
+        assert torch.equal(a, b)
+    # the incoming state of a call without inplace is left as it was
+    before = tuple(s.clone() for s in st0)
+    F.flare_causal_decode(qd, kd[:, :, :3], vd[:, :, :3], st0)
+    for a, b in zip(st0, before):
+        assert torch.equal(a, b)
+    with pytest.raises(ValueError):
+        q192 = torch.cat([qd, qd[:, :64]], dim=1)                  # 192 latents run as groups: no in-place form
+        F.flare_causal_decode_step(q192, kd[:, :, :1], vd[:, :, :1], F.causal_fresh_state(B, H, 192, D, dev), inplace=True)
+
+
+def test_decode_steps_replay_from_a_hip_graph(dev):
+    """256 in-place single-token steps captured once in a HIP graph: every replay (with eager work in between) must
+    reproduce the eager 256-step launch from the same starting state."""
+    B, H, M, D, NP, ND = 2, 4, 128, 64, 256, 256
+    q, k, v = make(B, H, NP + ND, M, D, torch.bfloat16, seed=47)
+    qd = q.to(dev)
+    kp, vp = k[:, :, :NP].contiguous().to(dev), v[:, :, :NP].contiguous().to(dev)
+    kd, vd = k[:, :, NP:].contiguous().to(dev), v[:, :, NP:].contiguous().to(dev)
+    _, st0 = F.flare_causal_prefill(qd, kp, vp)
+    y_all, st_all = F.flare_causal_decode(qd, kd, vd, st0)
+    st = tuple(s.clone() for s in st0)
+    ws = F.causal_workspace(qd, kd[:, :, :1])
+    y_steps = torch.empty_like(y_all)
+
+    def steps():
+        for t in range(ND):
+            F.flare_causal_decode_step(qd, kd[:, :, t:t + 1], vd[:, :, t:t + 1], st, inplace=True, workspace=ws,
+                                       out=y_steps[:, :, t:t + 1])
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        steps()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        steps()
+    for rep in range(3):
+        for a, b in zip(st, st0):
+            a.copy_(b)
+        y_steps.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_steps, y_all), rep
+        for a, b in zip(st, st_all):
+            assert torch.equal(a, b)
+        F.flare_causal_prefill(qd, kp, vp)               # eager work between replays

@@ -131,6 +131,28 @@ def test_block_fused_path_vs_torch_layers(dev, C, H, M, rms, monkeypatch):
     assert len(calls) == 4 and yt.requires_grad
 
 
+def test_narrow_heads_with_expanding_kv_projection(dev):
+    """D = 8 heads (the reference's default geometry) with the two-layer expanding k / v projections
+    (num_layers_*_proj = 0, ratio 2): no head-padded rows exist for that MLP form, so the layer must take the
+    generic fused branch (the mixer pads the heads) instead of raising, and match its own fp32 layers."""
+    torch.manual_seed(13)
+    att = F.FLARE(64, 8, 32, num_layers_k_proj=0, k_proj_mlp_ratio=2.0, num_layers_v_proj=0, v_proj_mlp_ratio=2.0).to(dev).eval()
+    blk = F.FLAREBlock(64, 8, 32, num_layers_k_proj=0, k_proj_mlp_ratio=2.0).to(dev).eval()
+    x = torch.randn(2, 1500, 64, device=dev)
+    for mod in (att, blk):
+        with torch.no_grad():
+            ref = mod(x)[0]
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                y = mod(x)[0]
+        assert O.rel_l2(y, ref) <= 2e-2
+    # against the state-dict restatement of the layer (fp64, same weights)
+    sd = {k: v.detach().double().cpu() for k, v in att.state_dict().items()}
+    want = O.flare_layer(sd, "", x.double().cpu(), num_heads=8)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        got = att(x)[0]
+    assert O.rel_l2(got, want) <= 2e-2
+
+
 def test_model_fused_path_vs_fp32(dev):
     torch.manual_seed(4)
     model = F.FLAREModel(in_dim=3, out_dim=2, channel_dim=64, num_blocks=2, num_heads=4, num_latents=64).to(dev).eval()
@@ -372,6 +394,21 @@ def test_graphed_forward_helper(dev):
     x = torch.randn(1, 2000, 3, device=dev)
     with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
         assert torch.equal(fwd(x), model(x))
+    # a parameter update without reset(): the next call notices and captures again
+    with torch.no_grad():
+        for p in model.parameters():
+            p.mul_(1.01)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        assert torch.equal(fwd(x), model(x))
+    # an eager forward in another compute dtype rebuilds the modules' operand caches; the graph keeps the ones it
+    # was captured with alive, so its replay still equals the bf16 eager result
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        want = model(x).clone()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        model(x)
+    junk = [torch.full((1 << 20,), float("nan"), device=dev) for _ in range(8)]     # recycle whatever was freed
+    assert torch.equal(fwd(x), want)
+    del junk
     with pytest.raises(ValueError):
         fwd(torch.randn(1, 10, 3))
     model.train()

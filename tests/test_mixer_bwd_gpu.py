@@ -151,3 +151,40 @@ def test_backward_with_latents_in_chunks(dev, shape):
     for name, got, ref in (("dq", qd.grad, gq), ("dk", kd.grad, gk), ("dv", vd.grad, gv)):
         err = O.rel_l2(got, ref)
         assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
+
+
+def test_z_handed_out_under_autograd_carries_gradients(dev):
+    """flare_multihead_mixer(..., return_z=True) with gradients required: a loss that uses z as well as y must
+    reach q, k, v through both (autograd of the explicit-softmax oracle in fp64 is the reference)."""
+    q, k, v, gy = make(2, 2, 600, 64, 32, torch.bfloat16, seed=21)
+    gz = torch.randn(2, 2, 64, 32, generator=torch.Generator().manual_seed(22))
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    y, z = F.flare_multihead_mixer(qd, kd, vd, scale=0.7, return_z=True)
+    assert z.requires_grad
+    ((y.float() * gy.to(dev).float()).sum() + (z * gz.to(dev)).sum()).backward()
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    yr, zr = O.mixer_explicit(qr, kr, vr, 0.7)
+    ((yr * gy.double()).sum() + (zr * gz.double()).sum()).backward()
+    for name, got, ref in (("dq", qd.grad, qr.grad), ("dk", kd.grad, kr.grad), ("dv", vd.grad, vr.grad)):
+        err = O.rel_l2(got, ref)
+        assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
+
+
+def test_backward_of_a_view_off_the_16_byte_grid(dev):
+    """k, v views whose first element is not 16-byte aligned: the HIP backward does not take them, the gradients
+    must come from the torch recomputation instead of an error."""
+    q, k, v, gy = make(1, 2, 400, 64, 32, torch.bfloat16, seed=23)
+    kb = torch.zeros(k.numel() + 4, dtype=k.dtype)
+    vb = torch.zeros(v.numel() + 4, dtype=v.dtype)
+    kb[4:] = k.reshape(-1)
+    vb[4:] = v.reshape(-1)
+    kd = kb.to(dev)[4:].view_as(k).requires_grad_(True)        # starts 8 bytes into the allocation
+    vd = vb.to(dev)[4:].view_as(v).requires_grad_(True)
+    assert kd.data_ptr() % 16 != 0
+    assert not FN._hip_backward_ok(q.to(dev), kd, vd, None, False)
+    qd = q.to(dev).requires_grad_(True)
+    F.flare_multihead_mixer(qd, kd, vd, scale=0.9).backward(gy.to(dev))
+    want = oracle_grads(q, k, v, gy, 0.9)
+    for name, got, ref in zip(("dq", "dk", "dv"), (qd.grad, kd.grad, vd.grad), want):
+        err = O.rel_l2(got, ref)
+        assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"

@@ -560,3 +560,17 @@ def test_mfma32_strided_views_per_batch_q_mask_and_lse(dev):
     from flare_py_amd import functional as FN
     out = FN._mixer_forward(q.to(dev), k.to(dev), v.to(dev), 1.0, None, 0, False, False, True)
     assert float((out[3].cpu() - want).abs().max()) < 3e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("scale", [1e-4, 3e-3, 1.0, 40.0])
+def test_dead_latents_get_no_weight_at_any_scale(dev, dtype, scale):
+    """M = 20 runs with 12 dead latents whose scores are scale * bias: the bias follows the scale, and where the
+    element type cannot hold it (f16 with a tiny scale) the fp32-FMA kernels take the problem."""
+    from flare_py_amd import functional as FN
+    q, k, v = make(1, 2, 700, 20, 16, dtype, seed=31)
+    bias = FN._dead_latent_bias(scale, dtype)
+    assert bias is None or scale * bias <= -200.0
+    if dtype == torch.float16 and scale == 1e-4:
+        assert bias is None and F.mixer_kernel_name(q.to(dev), k.to(dev), v.to(dev), scale=scale) == "generic"
+    check(dev, q, k, v, scale=scale)
