@@ -168,6 +168,33 @@ def bench_causal(args, F, dev):
                        "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                        "traffic": None, "algorithmic_bytes": bytes_prefill, "ms_prefill": round(ms_prefill, 4),
                        "ms_decode_256_steps": round(ms_decode, 4), "us_per_decode_step": round(ms_decode / ND * 1e3, 3)}
+    # ---- decoding token by token: 256 separate single-step calls on a state advanced in place (workspace and
+    # output reused), timed eagerly and as one HIP graph of the same 256 calls replayed ----
+    st_live = tuple(s.clone() for s in st)
+    ws = F.causal_workspace(q, kd[:, :, :1])
+    y_steps = torch.empty_like(kd)
+
+    def token_steps():
+        for t in range(ND):
+            F.flare_causal_decode_step(q, kd[:, :, t:t + 1], vd[:, :, t:t + 1], st_live, inplace=True, workspace=ws,
+                                       out=y_steps[:, :, t:t + 1])
+
+    ms_tok = time_events(token_steps, max(2, args.steps // 10), 2)
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        token_steps()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        token_steps()
+    ms_tok_graph = time_events(graph.replay, max(2, args.steps // 5), 2)
+    out["roofline"]["us_per_decode_step_separate_calls"] = round(ms_tok / ND * 1e3, 3)
+    out["roofline"]["us_per_decode_step_graph_replay"] = round(ms_tok_graph / ND * 1e3, 3)
+    # a latent count that runs as two groups of 128 joined by their softmax sums (256 latents with D = 64)
+    q2 = torch.cat([q, q.flip(1)], dim=1)
+    ms_prefill_256 = time_events(lambda: F.flare_causal_prefill(q2, kp, vp), max(2, args.steps // 5), 2)
+    out["roofline"]["ms_prefill_M256_two_groups"] = round(ms_prefill_256, 4)
     if not args.no_cpu:
         # the recurrence of the oracle on the first batch element (all heads) over the whole prompt
         ns = NP
@@ -317,11 +344,31 @@ def bench_block(args, F, dev):
     out = base_record(args, "FLAREBlock forward tokens/sec at B=4,N=65536,C=128,H=8,M=128 bf16",
                       4 * 65536 / (ms_step * 1e-3), "tokens/s", ms_step,
                       "lift MLP 3->128 + FLAREBlock forward with 4x GELU MLP, bf16 autocast, B=4,N=65536,C=128,H=8,D=16,M=128 (BASELINE config 2)")
-    achieved = nbytes / (ms_mixer * 1e-3) / 1e9
-    out["roofline"] = {"bound": "hbm", "kernel": "mixer (gather + merge + scatter) inside the block",
+    # Whole step: bytes every launch of the fused sequence has to move per token (C = 128; the stream x is fp32, k, v
+    # and the mixer's y are bf16) and the flops of its Linear layers and of the mixer; weights are read once.
+    T, Cw = 4 * 65536, 128
+    per_token = {
+        "lift (3 fp32 in, x out)": 3 * 4 + Cw * 4,
+        "norm1 + k_proj (x in, k out)": Cw * 4 + Cw * 2,
+        "norm1 + v_proj (x in, v out)": Cw * 4 + Cw * 2,
+        "mixer (k twice, v, y)": 4 * Cw * 2,
+        "out_proj + residual (y, x in, x out)": Cw * 2 + Cw * 4 + Cw * 4,
+        "norm2 + 4x MLP + residual (x in, x out)": Cw * 4 + Cw * 4,
+    }
+    bytes_step = T * sum(per_token.values())
+    flops_token = 2 * (3 * Cw + 3 * Cw * Cw) + 2 * 2 * 5 * Cw * Cw + 8 * 128 * 16 * 8 + 2 * Cw * Cw + 2 * 2 * Cw * 4 * Cw
+    flops_step = T * flops_token
+    t_hbm, t_mfma = bytes_step / (HBM_PEAK_GBPS * 1e9), flops_step / (MFMA_BF16_PEAK_TFLOPS * 1e12)
+    achieved = bytes_step / (ms_step * 1e-3) / 1e9
+    out["roofline"] = {"bound": "hbm" if t_hbm >= t_mfma else "mfma",
+                       "kernel": "whole step: lift + block, 6 fused launches + mixer; mlp_mfma_kernel is about 70 % of it",
                        "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                       "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "algorithmic_bytes": nbytes,
-                       "ms_mixer": round(ms_mixer, 4), "ms_block": round(ms_step, 4)}
+                       "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "algorithmic_bytes": bytes_step,
+                       "algorithmic_flops": flops_step, "ms_at_hbm_peak": round(t_hbm * 1e3, 4),
+                       "ms_at_mfma_peak": round(t_mfma * 1e3, 4), "step_tflops": round(flops_step / (ms_step * 1e-3) / 1e12, 1),
+                       "bytes_per_token_by_launch": per_token,
+                       "ms_mixer": round(ms_mixer, 4), "mixer_GBps": round(nbytes / (ms_mixer * 1e-3) / 1e9, 1),
+                       "ms_block": round(ms_step, 4)}
     out["ms_block_default_ffn_no_lift"] = round(ms_default, 4)
     # the same modules the way the reference runs them on this device: torch Linear / LayerNorm layers under the
     # same autocast, the mixer as two torch scaled_dot_product_attention calls (pdebench/models/flare.py:122-156)

@@ -266,24 +266,80 @@ def _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy):
     return gq.to(q.dtype), dk, dv
 
 
+#: elements of one [B,H,M,T] fp32 temporary of the tiled gradients below (64 MiB); about six such temporaries are
+#: alive at a time, whatever N is
+GRAD_TILE_ELEMS = 1 << 24
+
+
+def _grad_tile(B, H, M, N) -> int:
+    return int(min(N, max(256, GRAD_TILE_ELEMS // max(1, B * H * M))))
+
+
+def _gather_stats_tiled(qe, k, v, scale, keep, T):
+    """Log-sum-exp L [B,H,M] and z [B,H,M,D] of the gather by an online softmax over token tiles of T (fp32).
+    A latent row without a single real token gets L = +inf (so that exp(s - L) = 0 below) and z = 0."""
+    B, H, N, D = k.shape
+    M = qe.shape[2]
+    dev = k.device
+    m_run = torch.full((B, H, M), float("-inf"), device=dev)
+    l_run = torch.zeros((B, H, M), device=dev)
+    acc = torch.zeros((B, H, M, D), device=dev) if v is not None else None
+    m_safe = torch.zeros((B, H, M), device=dev)
+    for n0 in range(0, N, T):
+        s = scale * (qe @ k[:, :, n0:n0 + T].float().mT)
+        if keep is not None:
+            s = s.masked_fill(~keep[:, None, None, n0:n0 + T], float("-inf"))
+        m_new = torch.maximum(m_run, s.amax(-1))
+        m_safe = torch.where(torch.isfinite(m_new), m_new, torch.zeros_like(m_new))
+        p = torch.exp(s - m_safe[..., None])
+        alpha = torch.exp(m_run - m_safe)
+        l_run = l_run * alpha + p.sum(-1)
+        if acc is not None:
+            acc = acc * alpha[..., None] + p @ v[:, :, n0:n0 + T].float()
+        m_run = m_new
+    some = l_run > 0
+    L = torch.where(some, m_safe + torch.log(l_run.clamp_min(1e-37)), torch.full_like(l_run, float("inf")))
+    z = None if acc is None else torch.where(some[..., None], acc / l_run.clamp_min(1e-37)[..., None], torch.zeros_like(acc))
+    return L, z
+
+
 def _mixer_torch_grad(q, k, v, scale, key_mask, gy):
-    """Backward by recomputation in plain torch ops on the device the inputs live on: used for what
-    the HIP backward does not cover (fp32, unusual shapes).  The forward never takes this path."""
-    with torch.enable_grad():
-        q_, k_, v_ = (t.detach().float().requires_grad_(True) for t in (q, k, v))
-        qe = q_ if q_.dim() == 4 else q_.unsqueeze(0)
-        s = scale * (qe @ k_.transpose(-2, -1))
-        if key_mask is not None:
-            keep = key_mask.to(torch.bool)[:, None, None, :]
-            s_enc = s.masked_fill(~keep, float("-inf"))
-        else:
-            s_enc = s
-        z = torch.softmax(s_enc, dim=-1) @ v_
-        y = torch.softmax(s.transpose(-2, -1), dim=-1) @ z
-        if key_mask is not None:
-            y = y * key_mask.to(y.dtype)[:, None, :, None]
-        gq, gk, gv = torch.autograd.grad(y, (q_, k_, v_), gy.float())
-    return gq.to(q.dtype), gk.to(k.dtype), gv.to(v.dtype)
+    """dq, dk, dv of the mixer by recomputation in plain torch ops on the device: used for what the HIP backward
+    does not cover (fp32, unusual shapes); the forward never takes this path.  The scores are recomputed in token
+    tiles of [B,H,M,T] (GRAD_TILE_ELEMS), never as the whole [B,H,M,N] matrix, with the formulas of the HIP
+    backward: A = exp(S - L_m), B = exp(S - rho_n), dz = B dy, Delta = <dz,z>, delta = <dy,y>,
+    dS = A (dz v^T - Delta) + B (z dy^T - delta), dv = A^T dz, dk = s dS^T q, dq = s dS k."""
+    B, H, N, D = k.shape
+    qe = (q if q.dim() == 4 else q.unsqueeze(0)).float()
+    M = qe.shape[2]
+    keep = None if key_mask is None else key_mask.to(torch.bool)
+    T = _grad_tile(B, H, M, N)
+    gy = gy if keep is None else gy * keep[:, None, :, None].to(gy.dtype)
+    L, z = _gather_stats_tiled(qe, k, v, scale, keep, T)
+    dz = torch.zeros_like(z)
+    for n0 in range(0, N, T):
+        s = scale * (qe @ k[:, :, n0:n0 + T].float().mT)
+        Bt = torch.softmax(s, dim=2)
+        dz += Bt @ gy[:, :, n0:n0 + T].float()
+    Delta = (dz * z).sum(-1)
+    gq = torch.zeros((B, H, M, D), device=k.device)
+    gk = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    gv = torch.empty((B, H, N, D), dtype=v.dtype, device=k.device)
+    for n0 in range(0, N, T):
+        kt, vt, gyt = k[:, :, n0:n0 + T].float(), v[:, :, n0:n0 + T].float(), gy[:, :, n0:n0 + T].float()
+        s = scale * (qe @ kt.mT)
+        Bt = torch.softmax(s, dim=2)
+        if keep is not None:
+            s = s.masked_fill(~keep[:, None, None, n0:n0 + T], float("-inf"))
+        A = torch.exp(s - L[..., None])
+        delta = (gyt * (Bt.mT @ z)).sum(-1)
+        dS = A * (dz @ vt.mT - Delta[..., None]) + Bt * (z @ gyt.mT - delta[:, :, None, :])
+        gv[:, :, n0:n0 + T] = (A.mT @ dz).to(gv.dtype)
+        gk[:, :, n0:n0 + T] = (scale * (dS.mT @ qe)).to(gk.dtype)
+        gq += scale * (dS @ kt)
+    if q.dim() == 3:
+        gq = gq.sum(0)
+    return gq.to(q.dtype), gk, gv
 
 
 class _MixerFn(torch.autograd.Function):
@@ -486,22 +542,46 @@ def _scatter_forward(q, k, z, scale, key_mask, force_generic):
 
 def _half_torch_grad(which, q, k, x, scale, key_mask, g):
     """Gradients of one half of the mixer by recomputation in plain torch ops on the device (the forward
-    never takes this path): which='gather' -> z = softmax_n(s q k^T) x with x = v; which='scatter' ->
-    y = softmax_m(s k q^T) x with x = z.  Materialises the [B,H,M,N] scores in fp32."""
-    with torch.enable_grad():
-        q_, k_, x_ = (t.detach().float().requires_grad_(True) for t in (q, k, x))
-        qe = q_ if q_.dim() == 4 else q_.unsqueeze(0)
-        s = scale * (qe @ k_.transpose(-2, -1))
-        if which == "gather":
-            if key_mask is not None:
-                s = s.masked_fill(~key_mask.to(torch.bool)[:, None, None, :], float("-inf"))
-            out = torch.softmax(s, dim=-1) @ x_
-        else:
-            out = torch.softmax(s.transpose(-2, -1), dim=-1) @ x_
-            if key_mask is not None:
-                out = out * key_mask.to(out.dtype)[:, None, :, None]
-        gq, gk, gx = torch.autograd.grad(out, (q_, k_, x_), g.float())
-    return gq.to(q.dtype), gk.to(k.dtype), gx.to(x.dtype)
+    never takes this path), in token tiles like _mixer_torch_grad: which='gather' -> z = softmax_n(s q k^T) x with
+    x = v and g = dz; which='scatter' -> y = softmax_m(s k q^T) x with x = z and g = dy."""
+    B, H, N, D = k.shape
+    qe = (q if q.dim() == 4 else q.unsqueeze(0)).float()
+    M = qe.shape[2]
+    keep = None if key_mask is None else key_mask.to(torch.bool)
+    T = _grad_tile(B, H, M, N)
+    gq = torch.zeros((B, H, M, D), device=k.device)
+    gk = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    if which == "gather":
+        L, z = _gather_stats_tiled(qe, k, x, scale, keep, T)
+        dz = g.float()
+        Delta = (dz * z).sum(-1)
+        gx = torch.empty((B, H, N, D), dtype=x.dtype, device=k.device)
+        for n0 in range(0, N, T):
+            kt, vt = k[:, :, n0:n0 + T].float(), x[:, :, n0:n0 + T].float()
+            s = scale * (qe @ kt.mT)
+            if keep is not None:
+                s = s.masked_fill(~keep[:, None, None, n0:n0 + T], float("-inf"))
+            A = torch.exp(s - L[..., None])
+            dS = A * (dz @ vt.mT - Delta[..., None])
+            gx[:, :, n0:n0 + T] = (A.mT @ dz).to(gx.dtype)
+            gk[:, :, n0:n0 + T] = (scale * (dS.mT @ qe)).to(gk.dtype)
+            gq += scale * (dS @ kt)
+    else:
+        z = x.float()
+        gy = g if keep is None else g * keep[:, None, :, None].to(g.dtype)
+        gz = torch.zeros((B, H, M, D), device=k.device)
+        for n0 in range(0, N, T):
+            kt, gyt = k[:, :, n0:n0 + T].float(), gy[:, :, n0:n0 + T].float()
+            Bt = torch.softmax(scale * (qe @ kt.mT), dim=2)
+            delta = (gyt * (Bt.mT @ z)).sum(-1)
+            dS = Bt * (z @ gyt.mT - delta[:, :, None, :])
+            gz += Bt @ gyt
+            gk[:, :, n0:n0 + T] = (scale * (dS.mT @ qe)).to(gk.dtype)
+            gq += scale * (dS @ kt)
+        gx = gz.to(x.dtype)
+    if q.dim() == 3:
+        gq = gq.sum(0)
+    return gq.to(q.dtype), gk, gx
 
 
 class _GatherFn(torch.autograd.Function):
@@ -705,7 +785,11 @@ def _causal_call_launch(entry, q, k, v, scale, chunk, state, want_lse=False, inp
     _check_mixer_shapes(q4, k, v)
     M = q4.shape[2]
     if state is None:
-        mu, den, num = causal_fresh_state(B, H, M, D, k.device)
+        # fresh: mu = -inf marks every latent as empty, and no kernel reads the sums of an empty latent, so den and
+        # num need no fill (every element of the returned state is written by the call)
+        mu = torch.full((B, H, M), float("-inf"), dtype=torch.float32, device=k.device)
+        den = torch.empty((B, H, M), dtype=torch.float32, device=k.device)
+        num = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
     elif inplace:
         mu, den, num = state
         for s_ in (mu, den, num):

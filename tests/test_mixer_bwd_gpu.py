@@ -188,3 +188,29 @@ def test_backward_of_a_view_off_the_16_byte_grid(dev):
     for name, got, ref in zip(("dq", "dk", "dv"), (qd.grad, kd.grad, vd.grad), want):
         err = O.rel_l2(got, ref)
         assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
+
+
+def test_fp32_backward_at_262144_tokens_stays_inside_a_memory_bound(dev):
+    """fp32 inputs differentiate through the token-tiled recomputation: at N = 262,144, M = 256 it must never hold
+    the [B,H,M,N] scores (268 MB per copy here; the old recomputation kept about eight of them) — peak extra
+    memory is bounded by a few [B,H,M,T] tiles of 64 MiB — and match fp64 autograd of the explicit formulas,
+    evaluated on the device, to 1e-4."""
+    B, H, N, M, D = 1, 1, 262144, 256, 32
+    g = torch.Generator().manual_seed(51)
+    q = (torch.randn(H, M, D, generator=g) * D ** -0.5).to(dev)
+    k, v, gy = (torch.randn(B, H, N, D, generator=g).to(dev) for _ in range(3))
+    qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    base = torch.cuda.memory_allocated()
+    F.flare_multihead_mixer(qd, kd, vd, scale=0.9).backward(gy)
+    torch.cuda.synchronize()
+    extra = torch.cuda.max_memory_allocated() - base
+    assert extra < 900 * 2 ** 20, f"{extra / 2 ** 20:.0f} MiB"        # y, grads, workspace (~140 MiB) + tiles (~450 MiB)
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    s = 0.9 * (qr.unsqueeze(0) @ kr.mT)
+    y = torch.softmax(s.mT, -1) @ (torch.softmax(s, -1) @ vr)
+    y.backward(gy.double())
+    for name, got, ref in (("dq", qd.grad, qr.grad), ("dk", kd.grad, kr.grad), ("dv", vd.grad, vr.grad)):
+        err = float((got.double() - ref).norm() / ref.norm())
+        assert err <= 1e-4, f"{name} rel-L2 {err:.3e}"
