@@ -542,6 +542,36 @@ int static_scratch(void** out)
 }
 }  // namespace
 
+int flare_mixer_fwd_dropout(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
+                            const uint8_t* key_mask, float dropout_p, uint64_t seed, void* y, float* z_out,
+                            void* workspace, size_t workspace_bytes, void* stream)
+{
+    int rc = check_mixer_desc(desc);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !v || !y) return fail(FLARE_EINVAL, "q, k, v, y must not be NULL");
+    if (!(dropout_p >= 0.f) || !(dropout_p < 1.f)) return fail(FLARE_EINVAL, "dropout_p must be in [0, 1) (got %g)", (double)dropout_p);
+    if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
+    if (!aligned16(workspace)) return fail(FLARE_EINVAL, "workspace must be 16-byte aligned");
+    const size_t need = mixer_ws_bytes(desc);
+    if (workspace_bytes < need) return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, need);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // the fp32-FMA kernels carry the dropout; the plan is the generic one whatever the shape
+    const MixerPlan p = plan_mixer(desc, false);
+    flare::MixerArgs a;
+    fill_mixer_args(a, desc, p, workspace);
+    float* z = z_out ? z_out : reinterpret_cast<float*>(static_cast<char*>(workspace) + p.off_z);
+    a.q = q; a.k = k; a.v = v; a.y = y; a.mask = key_mask; a.z = z;
+    a.drop_thr = (uint32_t)((double)dropout_p * 16777216.0);
+    a.drop_rs = 1.0f / (1.0f - dropout_p);
+    a.seed_lo = (uint32_t)(seed & 0xffffffffu);
+    a.seed_hi = (uint32_t)(seed >> 32);
+    hipError_t e = flare::launch_gather_generic(a, desc->dtype, st);
+    if (e != hipSuccess) return hip_status(e, "gather launch");
+    e = flare::launch_gather_merge(a, st);
+    if (e != hipSuccess) return hip_status(e, "gather merge launch");
+    return hip_status(flare::launch_scatter_generic(a, desc->dtype, st), "scatter launch");
+}
+
 int flare_mixer_fwd_static(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
                            const uint8_t* key_mask, void* y, void* stream)
 {

@@ -58,6 +58,20 @@ __device__ __forceinline__ float max_xor32(float x)
     return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
+// Counter-based keep/drop decision of attention dropout: a 24-bit hash of (seed, phase, b*H + h, latent, token);
+// phase 0 = gather weights, 1 = scatter weights.  The backward recomputes it from the same inputs.
+__host__ __device__ __forceinline__ uint32_t lowbias32(uint32_t x)
+{
+    x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+    return x;
+}
+__host__ __device__ __forceinline__ uint32_t dropout_hash24(uint32_t seed_lo, uint32_t seed_hi, uint32_t phase, uint32_t bh,
+                                                            uint32_t m, uint32_t n)
+{
+    const uint32_t x = seed_lo + n * 0x9E3779B1u + m * 0x85EBCA77u + bh * 0xC2B2AE3Du + phase * 0x27D4EB2Fu;
+    return lowbias32(lowbias32(x) ^ seed_hi) >> 8;
+}
+
 // ---- kernel argument blocks (host fills them; passed by value) -------------------------
 struct MixerArgs {
     const void* q; const void* k; const void* v; void* y;
@@ -75,6 +89,10 @@ struct MixerArgs {
     float scale_log2;         // scale * log2(e)
     int no_mfma32;            // 1: keep the 16x16x32 kernels where the 32x32x16 ones would run
     int gather32;             // 1: the gather may take the 32x32x16 kernel too
+    // attention dropout (fp32-FMA kernels only): an entry of the softmax weights is kept when its hash is >= drop_thr
+    // (24-bit compare) and then scaled by drop_rs = 1 / (1 - p); drop_thr == 0 switches it off
+    uint32_t drop_thr, seed_lo, seed_hi;
+    float drop_rs;
     int64_t qs[3], ks[3], vs[3], ys[3];
 };
 

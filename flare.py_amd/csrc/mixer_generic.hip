@@ -47,6 +47,7 @@ __global__ __launch_bounds__(kGatherThreads) void gather_generic_kernel(MixerArg
         acc[d] = 0.f;
     }
     float mx = kNegBig, l = 0.f;
+    const uint32_t bh = (uint32_t)(b * a.H + h);
 
     const int n_begin = split * a.tokens_per_split;
     const int n_end = min(a.N, n_begin + a.tokens_per_split);
@@ -71,9 +72,13 @@ __global__ __launch_bounds__(kGatherThreads) void gather_generic_kernel(MixerArg
             const float al = fast_exp2(mx - mn);
             const float p = fast_exp2(s - mn);
             l = l * al + p;
+            // dropout acts on the normalised weight: the denominator keeps every term, the numerator the kept ones
+            float pv = p;
+            if (a.drop_thr != 0)
+                pv = dropout_hash24(a.seed_lo, a.seed_hi, 0u, bh, (uint32_t)m, (uint32_t)(n0 + j)) >= a.drop_thr ? p * a.drop_rs : 0.f;
 #pragma unroll
             for (int d = 0; d < DMAX; ++d)
-                if (d < D) acc[d] = fmaf(acc[d], al, p * vs[j][d]);
+                if (d < D) acc[d] = fmaf(acc[d], al, pv * vs[j][d]);
             mx = mn;
         }
     }
@@ -191,9 +196,13 @@ __global__ __launch_bounds__(kScatterThreads) void scatter_generic_kernel(MixerA
             const float al = fast_exp2(mx - mn);
             const float p = fast_exp2(s - mn);
             l = l * al + p;
+            float pv = p;
+            if (a.drop_thr != 0)
+                pv = dropout_hash24(a.seed_lo, a.seed_hi, 1u, (uint32_t)(b * a.H + h), (uint32_t)(m0 + j), (uint32_t)n) >= a.drop_thr
+                         ? p * a.drop_rs : 0.f;
 #pragma unroll
             for (int d = 0; d < DMAX; ++d)
-                if (d < D) acc[d] = fmaf(acc[d], al, p * zs[j][d]);
+                if (d < D) acc[d] = fmaf(acc[d], al, pv * zs[j][d]);
             mx = mn;
         }
     }

@@ -275,7 +275,30 @@ def _grad_tile(B, H, M, N) -> int:
     return int(min(N, max(256, GRAD_TILE_ELEMS // max(1, B * H * M))))
 
 
-def _gather_stats_tiled(qe, k, v, scale, keep, T):
+_M32 = 0xFFFFFFFF
+
+
+def _lowbias32(x):
+    x = x ^ (x >> 16)
+    x = (x * 0x7FEB352D) & _M32
+    x = x ^ (x >> 15)
+    x = (x * 0x846CA68B) & _M32
+    return x ^ (x >> 16)
+
+
+def _dropout_keep(seed: int, phase: int, B, H, M, n0, n1, p: float, device):
+    """The keep mask [B,H,M,n1-n0] of attention dropout, bit for bit the decision the kernels take
+    (dropout_hash24 in csrc/common.hpp): 32-bit wrap-around arithmetic carried out in int64."""
+    thr = int(p * 16777216.0)
+    bh = torch.arange(B * H, device=device, dtype=torch.int64).view(B, H, 1, 1)
+    m = torch.arange(M, device=device, dtype=torch.int64).view(1, 1, M, 1)
+    n = torch.arange(n0, n1, device=device, dtype=torch.int64).view(1, 1, 1, -1)
+    x = ((seed & _M32) + n * 0x9E3779B1 + m * 0x85EBCA77 + bh * 0xC2B2AE3D + phase * 0x27D4EB2F) & _M32
+    x = _lowbias32(_lowbias32(x) ^ ((seed >> 32) & _M32))
+    return (x >> 8) >= thr
+
+
+def _gather_stats_tiled(qe, k, v, scale, keep, T, drop=None):
     """Log-sum-exp L [B,H,M] and z [B,H,M,D] of the gather by an online softmax over token tiles of T (fp32).
     A latent row without a single real token gets L = +inf (so that exp(s - L) = 0 below) and z = 0."""
     B, H, N, D = k.shape
@@ -295,6 +318,8 @@ def _gather_stats_tiled(qe, k, v, scale, keep, T):
         alpha = torch.exp(m_run - m_safe)
         l_run = l_run * alpha + p.sum(-1)
         if acc is not None:
+            if drop is not None:     # the numerator keeps the surviving weights (scaled), the denominator all of them
+                p = p * _dropout_keep(drop[1], 0, B, H, M, n0, min(N, n0 + T), drop[0], dev) / (1.0 - drop[0])
             acc = acc * alpha[..., None] + p @ v[:, :, n0:n0 + T].float()
         m_run = m_new
     some = l_run > 0
@@ -303,23 +328,29 @@ def _gather_stats_tiled(qe, k, v, scale, keep, T):
     return L, z
 
 
-def _mixer_torch_grad(q, k, v, scale, key_mask, gy):
+def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None):
     """dq, dk, dv of the mixer by recomputation in plain torch ops on the device: used for what the HIP backward
     does not cover (fp32, unusual shapes); the forward never takes this path.  The scores are recomputed in token
     tiles of [B,H,M,T] (GRAD_TILE_ELEMS), never as the whole [B,H,M,N] matrix, with the formulas of the HIP
     backward: A = exp(S - L_m), B = exp(S - rho_n), dz = B dy, Delta = <dz,z>, delta = <dy,y>,
-    dS = A (dz v^T - Delta) + B (z dy^T - delta), dv = A^T dz, dk = s dS^T q, dq = s dS k."""
+    dS = A (dz v^T - Delta) + B (z dy^T - delta), dv = A^T dz, dk = s dS^T q, dq = s dS k.
+    drop = (p, seed): attention dropout as the forward kernels applied it; with keep masks K1, K2 (recomputed from
+    the seed) and r = 1 / (1 - p) the weights that met v and z were A K1 r and B K2 r, so
+    dz = (B K2 r) dy, dS = A (K1 r dz v^T - Delta) + B (K2 r z dy^T - delta), dv = (A K1 r)^T dz."""
     B, H, N, D = k.shape
     qe = (q if q.dim() == 4 else q.unsqueeze(0)).float()
     M = qe.shape[2]
     keep = None if key_mask is None else key_mask.to(torch.bool)
     T = _grad_tile(B, H, M, N)
     gy = gy if keep is None else gy * keep[:, None, :, None].to(gy.dtype)
-    L, z = _gather_stats_tiled(qe, k, v, scale, keep, T)
+    L, z = _gather_stats_tiled(qe, k, v, scale, keep, T, drop)
+    rs = 1.0 if drop is None else 1.0 / (1.0 - drop[0])
     dz = torch.zeros_like(z)
     for n0 in range(0, N, T):
         s = scale * (qe @ k[:, :, n0:n0 + T].float().mT)
         Bt = torch.softmax(s, dim=2)
+        if drop is not None:
+            Bt = Bt * _dropout_keep(drop[1], 1, B, H, M, n0, min(N, n0 + T), drop[0], k.device) * rs
         dz += Bt @ gy[:, :, n0:n0 + T].float()
     Delta = (dz * z).sum(-1)
     gq = torch.zeros((B, H, M, D), device=k.device)
@@ -332,8 +363,16 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy):
         if keep is not None:
             s = s.masked_fill(~keep[:, None, None, n0:n0 + T], float("-inf"))
         A = torch.exp(s - L[..., None])
-        delta = (gyt * (Bt.mT @ z)).sum(-1)
-        dS = A * (dz @ vt.mT - Delta[..., None]) + Bt * (z @ gyt.mT - delta[:, :, None, :])
+        if drop is None:
+            delta = (gyt * (Bt.mT @ z)).sum(-1)
+            dS = A * (dz @ vt.mT - Delta[..., None]) + Bt * (z @ gyt.mT - delta[:, :, None, :])
+        else:
+            n1 = min(N, n0 + T)
+            K1 = _dropout_keep(drop[1], 0, B, H, M, n0, n1, drop[0], k.device) * rs
+            K2 = _dropout_keep(drop[1], 1, B, H, M, n0, n1, drop[0], k.device) * rs
+            delta = (gyt * ((Bt * K2).mT @ z)).sum(-1)
+            dS = A * (K1 * (dz @ vt.mT) - Delta[..., None]) + Bt * (K2 * (z @ gyt.mT) - delta[:, :, None, :])
+            A = A * K1
         gv[:, :, n0:n0 + T] = (A.mT @ dz).to(gv.dtype)
         gk[:, :, n0:n0 + T] = (scale * (dS.mT @ qe)).to(gk.dtype)
         gq += scale * (dS @ kt)
@@ -381,6 +420,52 @@ class _MixerFn(torch.autograd.Function):
         return gq, gk, gv, None, None, None, None, None
 
 
+def _mixer_forward_dropout(q, k, v, scale, key_mask, p, seed, token_major):
+    """y, z of the mixer with attention dropout (flare_mixer_fwd_dropout: fp32-FMA kernels)."""
+    _require_cuda(q, k, v)
+    lib = _lib.load()
+    if q.dtype != k.dtype:
+        q = q.to(k.dtype)
+    if v.dtype != k.dtype:
+        raise TypeError("k and v must share a dtype")
+    k, v = _rows_last_contig(k), _rows_last_contig(v)
+    q4 = _q4(q, k.shape[0])
+    _check_mixer_shapes(q4, k, v)
+    B, H, N, D = k.shape
+    M = q4.shape[2]
+    if token_major:
+        y = torch.empty((B, N, H, D), dtype=k.dtype, device=k.device).permute(0, 2, 1, 3)
+    else:
+        y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    z = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
+    mask = _mask_u8(key_mask, B, N, k.device)
+    d = _mixer_desc(q4, k, v, y, scale, 0, True)
+    need = C.c_size_t(0)
+    _lib.check(lib.flare_mixer_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_workspace_bytes")
+    ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
+    with _on_device(k.device):
+        rc = lib.flare_mixer_fwd_dropout(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(mask), float(p), int(seed), _ptr(y), _ptr(z),
+                                         _ptr(ws), ws.numel(), C.c_void_p(_stream_ptr(k.device)))
+    _lib.check(rc, "flare_mixer_fwd_dropout")
+    return y, z
+
+
+class _MixerDropoutFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, scale, key_mask, p, seed, token_major):
+        ctx.scale, ctx.key_mask, ctx.drop = scale, key_mask, (p, seed)
+        ctx.save_for_backward(q, k, v)
+        y, z = _mixer_forward_dropout(q, k, v, scale, key_mask, p, seed, token_major)
+        ctx.mark_non_differentiable(z)
+        return y, z
+
+    @staticmethod
+    def backward(ctx, gy, _gz):
+        q, k, v = ctx.saved_tensors
+        gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy, ctx.drop)
+        return gq, gk, gv, None, None, None, None, None
+
+
 def _narrow_head_pad(q, k, force_generic) -> int:
     """Columns of zeros to append to a head dim so that the matrix-core kernels (D in {16, 32, 64}) take the problem,
     or 0.  Zero columns change neither the scores q.k nor the first D output columns; the reference's default model
@@ -397,7 +482,8 @@ def _pad_last(t, n):
 
 
 def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: bool = False,
-                          n_splits: int = 0, force_generic: bool = False, token_major_out: bool = False):
+                          n_splits: int = 0, force_generic: bool = False, token_major_out: bool = False,
+                          dropout_p: float = 0.0, dropout_seed: Optional[int] = None):
     """FLARE gather-scatter mixer (README.md:39-52 of the reference).
 
     q: [H,M,D] latent queries (or [B,H,M,D]); k, v: [B,H,N,D]; returns y [B,H,N,D] with
@@ -408,10 +494,22 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
     Under torch.autocast the operands are cast to the autocast dtype, as torch does for the
     scaled_dot_product_attention calls this replaces.  token_major_out=True lays y out as
     [B,N,H,D] in memory (returned as its [B,H,N,D] view) so that merging the heads is free.
+    dropout_p > 0 drops entries of both softmaxes' weights the way torch's scaled_dot_product_attention does
+    in training (lra/models/backends.py:592,605-606); the mask is a function of dropout_seed (drawn from torch's
+    default generator when None), so the backward recomputes it.  That path runs on the fp32-FMA kernels.
     """
     ac = _autocast_dtype(k)
     if ac is not None:
         q, k, v = (t if t.dtype == ac else t.to(ac) for t in (q, k, v))
+    if dropout_p > 0.0:
+        if not dropout_p < 1.0:
+            raise ValueError("dropout_p must be in [0, 1)")
+        seed = int(torch.randint(0, 2 ** 62, (), dtype=torch.int64)) if dropout_seed is None else int(dropout_seed)
+        if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+            y, z = _MixerDropoutFn.apply(q, k, v, float(scale), key_mask, float(dropout_p), seed, token_major_out)
+        else:
+            y, z = _mixer_forward_dropout(q, k, v, float(scale), key_mask, float(dropout_p), seed, token_major_out)
+        return (y, z) if return_z else y
     D = k.shape[-1]
     r = _latent_copies(q, k, force_generic)
     if r > 1 and q.dtype == v.dtype:

@@ -4,8 +4,9 @@ reference): same state_dict keys and constructor arguments; `forward(x, attentio
 Mask semantics: attention_mask [B,N], nonzero = real token.  Padded tokens are left out of
 the gather softmax; their own output rows are written as 0 (torch's fused attention leaves
 fully masked query rows backend dependent; 0 is the value that does not poison mean pooling).
-Attention dropout inside the softmax is not implemented in the kernels: attn_drop > 0 in
-training mode raises.
+Attention dropout (attn_drop > 0 in training mode) acts on both softmaxes' weights, as the
+reference's two scaled_dot_product_attention calls do (backends.py:592,605-606); it runs on the
+fp32-FMA kernels with a counter-based mask that the backward recomputes.
 
 Also here: the third-order linear-attention block of the same file (`TripleAttention`,
 `TripleBlock`, backends.py:1195-1331) and the feature maps it selects by name
@@ -77,14 +78,14 @@ class FLARE(nn.Module):
 
     def forward(self, x, attention_mask=None):
         B, N, C = x.shape
-        if self.training and self.attn_drop_p > 0.0:
-            raise NotImplementedError("attention dropout is not implemented in the FLARE HIP kernels")
+        drop = self.attn_drop_p if self.training else 0.0       # on both softmaxes, as backends.py:592,605-606
         q = self.latent_q.view(self.num_heads, self.num_latents, self.head_dim)
         k = self.k_proj(x).view(B, N, self.num_heads, self.head_dim).permute(0, 2, 1, 3)
         v = self.v_proj(x).view(B, N, self.num_heads, self.head_dim).permute(0, 2, 1, 3)
         if self.rope is not None:
             k = self.rope(k)
-        y = flare_multihead_mixer(q, k, v, scale=self.attn_scale, key_mask=attention_mask, token_major_out=True)
+        y = flare_multihead_mixer(q, k, v, scale=self.attn_scale, key_mask=attention_mask, token_major_out=True,
+                                  dropout_p=drop)
         y = self.out_proj(y.permute(0, 2, 1, 3).reshape(B, N, C))
         return F.dropout(y, p=self.proj_drop_p if self.training else 0.0)
 

@@ -18,6 +18,7 @@
  *   flare_scatter_fwd_lse      the same, also returning each token's log-sum-exp over the latents
  *   flare_mixer_bwd            gradient of flare_multihead_mixer (torch autograd through the two SDPA
  *                              calls upstream; ablation/time_memory_bwd.py:460-478 times fwd+bwd)
+ *   flare_mixer_fwd_dropout    the same two calls with dropout_p > 0 (lra/models/backends.py:592,605-606)
  *   flare_mixer_fwd_static     (no counterpart upstream: flare_mixer_fwd without a caller workspace)
  *   flare_clock_probe          (no counterpart upstream: measurement aid, sustained shader clock)
  *   flare_causal_prefill_fwd   causal restriction of the mixer (README.md:60 names it; the
@@ -218,6 +219,17 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
 int flare_mixer_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
                     const uint8_t* key_mask, void* y, float* z_out,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* The mixer with attention dropout on both softmaxes, as torch's scaled_dot_product_attention applies it in
+ * training (lra/models/backends.py:592,605-606: dropout_p on both calls): every normalised weight is kept with
+ * probability 1 - dropout_p and then divided by it, independently in the gather and in the scatter.  The decision
+ * for the weight of (batch, head, latent, token) is a counter-based hash of those indices, the phase and `seed`
+ * (no state, nothing stored): the same call repeats the same mask and a backward pass can recompute it.  Runs on
+ * the fp32-FMA kernels for every element type; dropout_p = 0 gives flare_mixer_fwd's result on those kernels.
+ * Workspace as flare_mixer_workspace_bytes(). */
+int flare_mixer_fwd_dropout(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
+                            const uint8_t* key_mask, float dropout_p, uint64_t seed, void* y, float* z_out,
+                            void* workspace, size_t workspace_bytes, void* stream);
 
 /* flare_mixer_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The split

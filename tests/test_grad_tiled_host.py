@@ -65,3 +65,21 @@ def test_batch_element_without_tokens_gets_zero_gradients():
     gq, gk, gv = FN._mixer_torch_grad(q, k, v, 1.0, mask, gy)
     assert torch.isfinite(gq).all() and torch.isfinite(gk).all() and torch.isfinite(gv).all()
     assert float(gk[1].abs().max()) == 0.0 and float(gv[1].abs().max()) == 0.0
+
+
+def test_dropout_hash_restatement_matches_plain_python():
+    """_dropout_keep (int64 tensors) against the same 32-bit hash written with Python integers."""
+    def low(x):
+        x ^= x >> 16; x = (x * 0x7FEB352D) & 0xFFFFFFFF; x ^= x >> 15; x = (x * 0x846CA68B) & 0xFFFFFFFF; x ^= x >> 16
+        return x
+    seed, phase, p = 0x123456789ABCDEF, 1, 0.3
+    B, H, M, n0, n1 = 2, 3, 5, 40, 47
+    got = FN._dropout_keep(seed, phase, B, H, M, n0, n1, p, "cpu")
+    thr = int(p * 16777216.0)
+    for b in range(B):
+        for h in range(H):
+            for m in range(M):
+                for n in range(n0, n1):
+                    x = ((seed & 0xFFFFFFFF) + n * 0x9E3779B1 + m * 0x85EBCA77 + (b * H + h) * 0xC2B2AE3D + phase * 0x27D4EB2F) & 0xFFFFFFFF
+                    keep = (low(low(x) ^ (seed >> 32)) >> 8) >= thr
+                    assert bool(got[b, h, m, n - n0]) == keep
