@@ -825,6 +825,7 @@ int flare_triple_state_fwd(const FlareTripleDesc* desc, const void* k1, const vo
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool mfma = p.mfma && aligned8(k1) && aligned8(k2) && aligned8(v);
     if (mfma) a.n_parts = p.n_parts;
+    a.diag_parts = mfma ? 1 : 0;
     hipError_t e = mfma ? flare::launch_triple_state_mfma(a, desc->dtype, st) : flare::launch_triple_state(a, desc->dtype, st);
     if (e != hipSuccess) return hip_status(e, "triple state launch");
     return hip_status(flare::launch_triple_merge(a, st), "triple merge launch");
@@ -841,7 +842,7 @@ int flare_triple_out_fwd(const FlareTripleDesc* desc, const void* q1, const void
     flare::TripleArgs a;
     fill_triple_args(a, desc, p);
     a.q1 = q1; a.q2 = q2; a.out = out; a.state = const_cast<float*>(state); a.kk = const_cast<float*>(kk_state);
-    const bool mfma = p.mfma && aligned8(q1) && aligned8(q2);
+    const bool mfma = p.mfma && aligned8(q1) && aligned8(q2) && aligned8(out) && strides_mult4(desc->o_stride);
     hipStream_t st = static_cast<hipStream_t>(stream);
     return hip_status(mfma ? flare::launch_triple_out_mfma(a, desc->dtype, st) : flare::launch_triple_out(a, desc->dtype, st),
                       "triple out launch");

@@ -125,6 +125,7 @@ struct TripleArgs {
     float* part;       // [B,H,S,Dq*Dv*Dq (+Dq*Dq)] split partials
     int B, H, N, Dq, Dv;
     int feature_map, normalize;
+    int diag_parts;    // 1: partials in the matrix-core kernel's accumulator order [step][lane][register] (16^3 only)
     int n_splits, tokens_per_split;
     int n_parts;       // partials per (b,h) in `part`
     int64_t q1s[3], q2s[3], k1s[3], k2s[3], vs[3], os[3];

@@ -100,8 +100,16 @@ __global__ __launch_bounds__(kThreads) void triple_merge_kernel(TripleArgs a)
     float s = 0.f;
     for (int sp = 0; sp < a.n_parts; ++sp) s += p[(size_t)sp * per];
     s *= 1.0f / (float)a.N;
-    if (e < ns) a.state[bh * ns + e] = s;
-    else if (a.kk) a.kk[bh * nk + (e - ns)] = s;
+    size_t o = e < ns ? e : e - ns;
+    if (a.diag_parts) {
+        // element (step r, lane = 16 g + c16, register rr) of the matrix-core kernel's accumulators holds
+        // state[i = 4g + rr][j = c16][k = (i - r) mod 16]; its normaliser tile holds kk[i = 4g + rr][k' = c16]
+        const int r = (int)(o >> 8), lane = (int)(o >> 2) & 63, rr = (int)o & 3;
+        const int i = 4 * (lane >> 4) + rr, c16 = lane & 15;
+        o = e < ns ? ((size_t)i * 16 + c16) * 16 + ((i - r) & 15) : (size_t)i * 16 + c16;
+    }
+    if (e < ns) a.state[bh * ns + o] = s;
+    else if (a.kk) a.kk[bh * nk + o] = s;
 }
 
 constexpr int kOutLdsFloats = 8192;

@@ -5,11 +5,13 @@
 // For a fixed k both contractions are 16x16x16 products:
 //   state[:, :, k] += A_k^T V     with A_k[n,i] = f(k1)[n,i] f(k2)[n,k]           (contraction over 16 tokens)
 //   T_k[n,:]        = f(q1)[n,:] state[:, :, k] ;  out[n,:] += T_k[n,:] f(q2)[n,k] (contraction over i)
-// so a wave walks 16-token tiles with v_mfma_f32_16x16x16.  Tiles are staged (feature map applied,
-// rounded to the element type) in a wave-private LDS tile; operands that need tokens in the
-// k-slots come from the LDS transpose read.  No barrier in the token loop and no atomics: a
-// workgroup sums its four waves in a fixed order and writes one split partial; the fixed-order
-// merge of triple.hip sums the partials.
+// so a wave walks 16-token tiles with v_mfma_f32_16x16x16.  The state kernel stages its tiles (feature map
+// applied, rounded to the element type) in a wave-private LDS tile and takes them with tokens in the k-slots
+// through the LDS transpose read; the output kernel reads f(q1) straight from global memory as a B operand.
+// No barrier in the token loops and no atomics: a workgroup sums its four waves in a fixed order and writes one
+// split partial; the fixed-order merge of triple.hip sums the partials.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace flare {
@@ -68,15 +70,15 @@ __device__ __forceinline__ float featf(float x, int fm)
     return x > 0.f ? x + 1.f : __expf(x);
 }
 
-// 4 elements (8 bytes) -> feature map -> repacked; `live` = false gives zeros
+// 4 elements (8 bytes, already in registers) -> feature map -> repacked; `live` = false gives zeros
 template <typename T>
-__device__ __forceinline__ uint2 load_feat4(const uint16_t* p, bool live, int fm)
+__device__ __forceinline__ uint2 feat4_of(uint2 raw, bool live, int fm)
 {
-    if (!live) return make_uint2(0u, 0u);
-    const uint2 raw = *reinterpret_cast<const uint2*>(p);
-    if (!fm) return raw;
-    return make_uint2(Tm<T>::pack2(featf(Tm<T>::lo(raw.x), fm), featf(Tm<T>::hi(raw.x), fm)),
-                      Tm<T>::pack2(featf(Tm<T>::lo(raw.y), fm), featf(Tm<T>::hi(raw.y), fm)));
+    uint2 f = raw;
+    if (fm)
+        f = make_uint2(Tm<T>::pack2(featf(Tm<T>::lo(raw.x), fm), featf(Tm<T>::hi(raw.x), fm)),
+                       Tm<T>::pack2(featf(Tm<T>::lo(raw.y), fm), featf(Tm<T>::hi(raw.y), fm)));
+    return make_uint2(live ? f.x : 0u, live ? f.y : 0u);
 }
 
 // Sum over the 16 lanes of a row with DPP operands (vector ALU only): pairs, quads, half rows, the row.
@@ -95,16 +97,38 @@ __device__ __forceinline__ float row16_sum(float x)
 
 constexpr int kD = 16;
 
+// x * (the value y has in lane (c - R) mod 16 of the same 16-lane row): one vector instruction with a DPP row
+// rotate on its first operand.  y must have been written at least two instructions earlier (the DPP read of a
+// freshly written register needs two wait states, which callers provide by computing all factors up front).
+template <int R> __device__ __forceinline__ float mul_row_ror(float x, float y)
+{
+    if constexpr (R == 0) {
+        return x * y;
+    } else {
+        float d;
+        asm("v_mul_f32_dpp %0, %1, %2 row_ror:%3 row_mask:0xf bank_mask:0xf" : "=v"(d) : "v"(y), "v"(x), "i"(R));
+        return d;
+    }
+}
+
+constexpr size_t kStateRedBytes = 4 * (kD + 1) * 64 * 4 * sizeof(float);
+
 // grid (n_splits, H, B); wave w of a workgroup takes the 16-token tiles w, w+4, ... of the split.
+//
+// Per tile the wave stages f(k1), f(k2), v (rounded to the element type) in its own LDS tile and takes all three
+// with tokens in the k-slots (transpose read: lane = feature c16, slots = tokens 4g..4g+3).  The state is
+// accumulated along "diagonals": step r multiplies the lane's f(k1)[n, i = c16] by f(k2)[n, (c16 - r) mod 16],
+// which is the value its neighbour r lanes down the row holds (a DPP rotate inside the multiply: no LDS read,
+// no broadcast), so S[r][i][j] = state[i][j][(i - r) mod 16].  The four waves meet once, at the end.
 template <typename T>
-__global__ __launch_bounds__(256) void triple_state_mfma_kernel(TripleArgs a)
+__global__ __launch_bounds__(256, 2) void triple_state_mfma_kernel(TripleArgs a)
 {
     using M_ = Tm<T>;
     __shared__ __attribute__((aligned(16))) uint16_t k1s[4][16][kD];
     __shared__ __attribute__((aligned(16))) uint16_t k2s[4][16][kD];
     __shared__ __attribute__((aligned(16))) uint16_t vs[4][16][kD];
-    __shared__ __attribute__((aligned(16))) float k2f[4][16][kD];      // f(k2) of the tile in fp32, for the scalar factors
-    __shared__ __attribute__((aligned(16))) float red[kD + 1][64][4];
+    extern __shared__ __attribute__((aligned(16))) uint8_t triple_red[];      // kStateRedBytes: where the waves meet
+    float (*red)[kD + 1][64][4] = reinterpret_cast<float (*)[kD + 1][64][4]>(triple_red);
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
     const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -119,87 +143,106 @@ __global__ __launch_bounds__(256) void triple_state_mfma_kernel(TripleArgs a)
 #pragma unroll
     for (int k = 0; k < kD; ++k) S[k] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // raw 8-byte pieces of the next tile are fetched while the current one is processed
+    // Raw 8-byte pieces of the tiles two ahead are fetched while the current one is processed.  The loads are
+    // unconditional (rows past the end repeat the last row and are zeroed when staged): with no branch around a
+    // memory instruction the compiler's waits count exactly what is in flight instead of draining everything.
     auto fetch = [&](int n0, uint2& r1, uint2& r2, uint2& rv) {
-        const int n = n0 + tok;
-        const bool live = n < n_end;
-        r1 = live ? *reinterpret_cast<const uint2*>(k1 + (int64_t)n * a.k1s[2] + piece) : make_uint2(0u, 0u);
-        r2 = live ? *reinterpret_cast<const uint2*>(k2 + (int64_t)n * a.k2s[2] + piece) : make_uint2(0u, 0u);
-        rv = live ? *reinterpret_cast<const uint2*>(v + (int64_t)n * a.vs[2] + piece) : make_uint2(0u, 0u);
+        const int n = min(n0 + tok, n_end - 1);
+        r1 = *reinterpret_cast<const uint2*>(k1 + (int64_t)n * a.k1s[2] + piece);
+        r2 = *reinterpret_cast<const uint2*>(k2 + (int64_t)n * a.k2s[2] + piece);
+        rv = *reinterpret_cast<const uint2*>(v + (int64_t)n * a.vs[2] + piece);
     };
     auto feat4 = [&](uint2 raw, bool live) {
-        if (!live) return make_uint2(0u, 0u);
-        if (!a.feature_map) return raw;
-        return make_uint2(M_::pack2(featf(M_::lo(raw.x), 1), featf(M_::hi(raw.x), 1)),
-                          M_::pack2(featf(M_::lo(raw.y), 1), featf(M_::hi(raw.y), 1)));
+        uint2 f = raw;
+        if (a.feature_map)
+            f = make_uint2(M_::pack2(featf(M_::lo(raw.x), 1), featf(M_::hi(raw.x), 1)),
+                           M_::pack2(featf(M_::lo(raw.y), 1), featf(M_::hi(raw.y), 1)));
+        return make_uint2(live ? f.x : 0u, live ? f.y : 0u);
     };
-    uint2 c1, c2, cv, x1, x2, xv;
-    fetch(n_begin + w * 16, c1, c2, cv);
-    for (int n0 = n_begin + w * 16; n0 < n_end; n0 += 64) {
+    auto step = [&](auto r_c, const float (&k1f)[4], const float (&k2f)[4], uint2 vt) {
+        constexpr int R = decltype(r_c)::value;
+        const uint2 ak = make_uint2(M_::pack2(mul_row_ror<R>(k1f[0], k2f[0]), mul_row_ror<R>(k1f[1], k2f[1])),
+                                    M_::pack2(mul_row_ror<R>(k1f[2], k2f[2]), mul_row_ror<R>(k1f[3], k2f[3])));
+        S[R] = M_::mma16(ak, vt, S[R]);
+    };
+    // one tile: stage (c1, c2, cv), then the seventeen products
+    auto tile = [&](int n0, uint2 c1, uint2 c2, uint2 cv) {
         const bool live = n0 + tok < n_end;
-        fetch(n0 + 64, x1, x2, xv);
         *reinterpret_cast<uint2*>(&k1s[w][tok][piece]) = feat4(c1, live);
-        const uint2 f2 = feat4(c2, live);
-        *reinterpret_cast<uint2*>(&k2s[w][tok][piece]) = f2;
-        *reinterpret_cast<f32x4*>(&k2f[w][tok][piece]) = f32x4{M_::lo(f2.x), M_::hi(f2.x), M_::lo(f2.y), M_::hi(f2.y)};
-        *reinterpret_cast<uint2*>(&vs[w][tok][piece]) = live ? cv : make_uint2(0u, 0u);
-        c1 = x1; c2 = x2; cv = xv;
-
+        *reinterpret_cast<uint2*>(&k2s[w][tok][piece]) = feat4(c2, live);
+        *reinterpret_cast<uint2*>(&vs[w][tok][piece]) = make_uint2(live ? cv.x : 0u, live ? cv.y : 0u);
         // tokens 4g..4g+3 in the k-slots, lane = feature index c16
         const int tr_row = 4 * g + (c16 >> 2), tr_col = (c16 & 3) * 4;
         const uint2 k1t = tr16(&k1s[w][tr_row][tr_col]);
         const uint2 k2t = tr16(&k2s[w][tr_row][tr_col]);
         const uint2 vt = tr16(&vs[w][tr_row][tr_col]);
         kk = M_::mma16(k1t, k2t, kk);
-        const float a0 = M_::lo(k1t.x), a1 = M_::hi(k1t.x), a2 = M_::lo(k1t.y), a3 = M_::hi(k1t.y);
-        // f(k2) rows of the lane's four tokens
-        f32x4 r[4][4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) r[e][c] = *reinterpret_cast<const f32x4*>(&k2f[w][4 * g + e][4 * c]);
-#pragma unroll
-        for (int k = 0; k < kD; ++k) {
-            const int kc = k >> 2, ke = k & 3;
-            const uint2 ak = make_uint2(M_::pack2(a0 * r[0][kc][ke], a1 * r[1][kc][ke]), M_::pack2(a2 * r[2][kc][ke], a3 * r[3][kc][ke]));
-            S[k] = M_::mma16(ak, vt, S[k]);
+        const float k1f[4] = {M_::lo(k1t.x), M_::hi(k1t.x), M_::lo(k1t.y), M_::hi(k1t.y)};
+        const float k2f[4] = {M_::lo(k2t.x), M_::hi(k2t.x), M_::lo(k2t.y), M_::hi(k2t.y)};
+        step(std::integral_constant<int, 0>{}, k1f, k2f, vt);   step(std::integral_constant<int, 1>{}, k1f, k2f, vt);
+        step(std::integral_constant<int, 2>{}, k1f, k2f, vt);   step(std::integral_constant<int, 3>{}, k1f, k2f, vt);
+        step(std::integral_constant<int, 4>{}, k1f, k2f, vt);   step(std::integral_constant<int, 5>{}, k1f, k2f, vt);
+        step(std::integral_constant<int, 6>{}, k1f, k2f, vt);   step(std::integral_constant<int, 7>{}, k1f, k2f, vt);
+        step(std::integral_constant<int, 8>{}, k1f, k2f, vt);   step(std::integral_constant<int, 9>{}, k1f, k2f, vt);
+        step(std::integral_constant<int, 10>{}, k1f, k2f, vt);  step(std::integral_constant<int, 11>{}, k1f, k2f, vt);
+        step(std::integral_constant<int, 12>{}, k1f, k2f, vt);  step(std::integral_constant<int, 13>{}, k1f, k2f, vt);
+        step(std::integral_constant<int, 14>{}, k1f, k2f, vt);  step(std::integral_constant<int, 15>{}, k1f, k2f, vt);
+    };
+    // three register sets take turns: a set is refilled with the tile three ahead as soon as its tile is staged,
+    // so no register is copied from one set to another (a copy would have to wait for the load it copies)
+    uint2 a1, a2, av, b1, b2, bv, c1, c2, cv;
+    int n0 = n_begin + w * 16;
+    if (n0 < n_end) {
+        fetch(n0, a1, a2, av);
+        fetch(n0 + 64, b1, b2, bv);
+        fetch(n0 + 128, c1, c2, cv);
+        for (;; n0 += 192) {
+            { const uint2 t1 = a1, t2 = a2, tv = av; fetch(n0 + 192, a1, a2, av); tile(n0, t1, t2, tv); }
+            if (n0 + 64 >= n_end) break;
+            { const uint2 t1 = b1, t2 = b2, tv = bv; fetch(n0 + 256, b1, b2, bv); tile(n0 + 64, t1, t2, tv); }
+            if (n0 + 128 >= n_end) break;
+            { const uint2 t1 = c1, t2 = c2, tv = cv; fetch(n0 + 320, c1, c2, cv); tile(n0 + 128, t1, t2, tv); }
+            if (n0 + 192 >= n_end) break;
         }
     }
 
-    // fixed-order sum of the four waves' accumulators through LDS (wave 1, 2, 3 into wave 0),
-    // then one partial per workgroup
-    for (int src = 1; src < 4; ++src) {
-        __syncthreads();
-        if (w == src) {
+    // the four waves' accumulators meet in LDS once; wave w then sums steps 4w..4w+3 (and wave 0 the normaliser
+    // state) over the waves in a fixed order and writes its share of the workgroup's partial
 #pragma unroll
-            for (int k = 0; k < kD; ++k) *reinterpret_cast<f32x4*>(&red[k][lane][0]) = S[k];
-            *reinterpret_cast<f32x4*>(&red[kD][lane][0]) = kk;
-        }
-        __syncthreads();
-        if (w == 0) {
-#pragma unroll
-            for (int k = 0; k < kD; ++k) S[k] += *reinterpret_cast<const f32x4*>(&red[k][lane][0]);
-            kk += *reinterpret_cast<const f32x4*>(&red[kD][lane][0]);
-        }
-    }
-    if (w != 0) return;
+    for (int k = 0; k < kD; ++k) *reinterpret_cast<f32x4*>(&red[w][k][lane][0]) = S[k];
+    *reinterpret_cast<f32x4*>(&red[w][kD][lane][0]) = kk;
+    __syncthreads();
     const size_t per = (size_t)kD * kD * kD + (size_t)kD * kD;
     float* part = a.part + (((size_t)b * a.H + h) * a.n_parts + split) * per;
+    // The partial keeps the accumulators' own order, [step r][lane][register rr] (and the normaliser tile behind
+    // them), so that every store is 16 contiguous bytes per lane; the merge kernel puts the sums into [i][j][k].
 #pragma unroll
-    for (int k = 0; k < kD; ++k)
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) part[((size_t)(4 * g + rr) * kD + c16) * kD + k] = S[k][rr];   // [i][j][k]
-#pragma unroll
-    for (int rr = 0; rr < 4; ++rr) part[(size_t)kD * kD * kD + (size_t)(4 * g + rr) * kD + c16] = kk[rr];   // [i][k']
+    for (int rr4 = 0; rr4 < 4; ++rr4) {
+        const int r = 4 * w + rr4;
+        const f32x4 t = *reinterpret_cast<const f32x4*>(&red[0][r][lane][0]) + *reinterpret_cast<const f32x4*>(&red[1][r][lane][0]) +
+                        *reinterpret_cast<const f32x4*>(&red[2][r][lane][0]) + *reinterpret_cast<const f32x4*>(&red[3][r][lane][0]);
+        *reinterpret_cast<f32x4*>(part + ((size_t)r * 64 + lane) * 4) = t;
+    }
+    if (w == 0) {
+        const f32x4 t = *reinterpret_cast<const f32x4*>(&red[0][kD][lane][0]) + *reinterpret_cast<const f32x4*>(&red[1][kD][lane][0]) +
+                        *reinterpret_cast<const f32x4*>(&red[2][kD][lane][0]) + *reinterpret_cast<const f32x4*>(&red[3][kD][lane][0]);
+        *reinterpret_cast<f32x4*>(part + ((size_t)kD * 64 + lane) * 4) = t;
+    }
 }
 
 // grid (ceil(N / tokens_per_wg), H, B); each wave walks 16-token tiles of the workgroup's range.
+//
+// The products are taken transposed, T_k^T[j, n] = sum_i state[i,j,k] f(q1)[n,i]: the state slices are the A
+// operands (row j = c16, slots i = 4g..4g+3, set up once), f(q1) rows are the B operands straight from global
+// memory (lane = token c16, slots i = 4g..4g+3: 8 contiguous bytes of the token's row), and the result has the
+// token in the lane, so the factor f(q2)[n,k] is a per-lane scalar.  Only f(q2) passes through (wave-private) LDS,
+// to hand every lane its token's sixteen features.
 template <typename T>
 __global__ __launch_bounds__(256) void triple_out_mfma_kernel(TripleArgs a, int tokens_per_wg)
 {
     using M_ = Tm<T>;
-    __shared__ __attribute__((aligned(16))) uint16_t q1s[4][16][kD];
-    __shared__ __attribute__((aligned(16))) float q2f[4][16][kD];     // f(q2) of the tile in fp32: multiplied as it is
+    constexpr int QS = kD + 4;                                          // row stride of the f(q2) tile in floats
+    __shared__ __attribute__((aligned(16))) float q2f[4][16][QS];
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
     const int h = blockIdx.y, b = blockIdx.z;
@@ -210,7 +253,7 @@ __global__ __launch_bounds__(256) void triple_out_mfma_kernel(TripleArgs a, int 
     const float* state = a.state + bh * kD * kD * kD;
     const int tok = lane >> 2, piece = (lane & 3) * 4;
 
-    // B operands: sk[k] = state[i = 4g..4g+3][j = c16][k], kkb = kk[i = 4g..4g+3][k' = c16]
+    // A operands: sk[k] = state[i = 4g..4g+3][j = c16][k], kkb = kk[i = 4g..4g+3][k' = c16]
     uint2 sk[kD], kkb = make_uint2(0u, 0u);
     {
         float sv[4][kD];
@@ -232,44 +275,60 @@ __global__ __launch_bounds__(256) void triple_out_mfma_kernel(TripleArgs a, int 
 
     const int wg_n0 = blockIdx.x * tokens_per_wg;
     const int wg_n1 = min(a.N, wg_n0 + tokens_per_wg);
-    // the features of the next tile are fetched while the current one is being worked on
-    auto fetch = [&](int n0, uint2& f1, uint2& f2) {
-        const int n = n0 + tok;
-        const bool live = n < wg_n1;
-        f1 = load_feat4<T>(q1 + (int64_t)n * a.q1s[2] + piece, live, a.feature_map);
-        f2 = load_feat4<T>(q2 + (int64_t)n * a.q2s[2] + piece, live, a.feature_map);
+    // Raw pieces of the tiles two ahead are fetched while the current one is being worked on: q1 as this lane's B
+    // operand (token c16, features 4g..4g+3), q2 as the lane's share of the tile (token tok, features piece..).
+    // Unconditional loads (rows past the end repeat the last row): no branch around a memory instruction, so the
+    // compiler's waits count what is in flight.
+    auto fetch = [&](int n0, uint2& r1, uint2& r2) {
+        r1 = *reinterpret_cast<const uint2*>(q1 + (int64_t)min(n0 + c16, wg_n1 - 1) * a.q1s[2] + 4 * g);
+        r2 = *reinterpret_cast<const uint2*>(q2 + (int64_t)min(n0 + tok, wg_n1 - 1) * a.q2s[2] + piece);
     };
-    uint2 f1 = make_uint2(0u, 0u), f2 = f1;
-    if (wg_n0 + w * 16 < wg_n1) fetch(wg_n0 + w * 16, f1, f2);
-    for (int n0 = wg_n0 + w * 16; n0 < wg_n1; n0 += 64) {
-        *reinterpret_cast<uint2*>(&q1s[w][tok][piece]) = f1;
+    auto tile = [&](int n0, uint2 r1, uint2 r2) {
+        const uint2 f2 = feat4_of<T>(r2, n0 + tok < wg_n1, a.feature_map);
         *reinterpret_cast<f32x4*>(&q2f[w][tok][piece]) = f32x4{M_::lo(f2.x), M_::hi(f2.x), M_::lo(f2.y), M_::hi(f2.y)};
-        if (n0 + 64 < wg_n1) fetch(n0 + 64, f1, f2);
-
-        // A operand: row = token c16, k-slots i = 4g..4g+3
-        const uint2 q1a = *reinterpret_cast<const uint2*>(&q1s[w][c16][4 * g]);
-        f32x4 r[4][4];       // f(q2)[n = 4g + e][k = 4 c .. 4 c + 3]
+        const uint2 q1b = feat4_of<T>(r1, n0 + c16 < wg_n1, a.feature_map);
+        // the sixteen f(q2) of the lane's token (the tile is private to the wave: reads follow its writes in program order)
+        float r[kD];
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) r[e][c] = *reinterpret_cast<const f32x4*>(&q2f[w][4 * g + e][4 * c]);
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};   // out[n = 4g + r][j = c16]
+        for (int c = 0; c < 4; ++c) {
+            const f32x4 t = *reinterpret_cast<const f32x4*>(&q2f[w][c16][4 * c]);
+            r[4 * c] = t[0]; r[4 * c + 1] = t[1]; r[4 * c + 2] = t[2]; r[4 * c + 3] = t[3];
+        }
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};   // out[n = c16][j = 4g + e]
 #pragma unroll
         for (int k = 0; k < kD; ++k) {
-            const f32x4 t = M_::mma16(q1a, sk[k], f32x4{0.f, 0.f, 0.f, 0.f});
+            const f32x4 t = M_::mma16(sk[k], q1b, f32x4{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] = fmaf(t[e], r[e][k >> 2][k & 3], acc[e]);
+            for (int e = 0; e < 4; ++e) acc[e] = fmaf(t[e], r[k], acc[e]);
         }
         if (a.normalize) {
-            // den[n] = sum_k' (f(q1)[n,:] kk[:,k']) f(q2)[n,k'] : k' runs over the 16 lanes of a row group
-            const f32x4 wv = M_::mma16(q1a, kkb, f32x4{0.f, 0.f, 0.f, 0.f});
+            // den[n] = sum_k' (sum_i kk[i,k'] f(q1)[n,i]) f(q2)[n,k']: the lane holds k' = 4g..4g+3 of its token
+            const f32x4 wv = M_::mma16(kkb, q1b, f32x4{0.f, 0.f, 0.f, 0.f});
+            const f32x4 rq = *reinterpret_cast<const f32x4*>(&q2f[w][c16][4 * g]);
+            float den = wv[0] * rq[0] + wv[1] * rq[1] + wv[2] * rq[2] + wv[3] * rq[3];
+            den = sum_xor32(sum_xor16(den));
+            const float inv = 1.f / den;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] = acc[e] / row16_sum(wv[e] * q2f[w][4 * g + e][c16]);
+            for (int e = 0; e < 4; ++e) acc[e] *= inv;
         }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int nn = n0 + 4 * g + e;
-            if (nn < wg_n1) out[(int64_t)nn * a.os[2] + c16] = uint16_t(M_::pack2(acc[e], 0.f) & 0xffffu);
+        if (n0 + c16 < wg_n1)
+            *reinterpret_cast<uint2*>(out + (int64_t)(n0 + c16) * a.os[2] + 4 * g) =
+                make_uint2(M_::pack2(acc[0], acc[1]), M_::pack2(acc[2], acc[3]));
+    };
+    // three register sets take turns, each refilled with the tile three ahead once its own has been taken
+    uint2 a1, a2, b1, b2, c1, c2;
+    int n0 = wg_n0 + w * 16;
+    if (n0 < wg_n1) {
+        fetch(n0, a1, a2);
+        fetch(n0 + 64, b1, b2);
+        fetch(n0 + 128, c1, c2);
+        for (;; n0 += 192) {
+            { const uint2 t1 = a1, t2 = a2; fetch(n0 + 192, a1, a2); tile(n0, t1, t2); }
+            if (n0 + 64 >= wg_n1) break;
+            { const uint2 t1 = b1, t2 = b2; fetch(n0 + 256, b1, b2); tile(n0 + 64, t1, t2); }
+            if (n0 + 128 >= wg_n1) break;
+            { const uint2 t1 = c1, t2 = c2; fetch(n0 + 320, c1, c2); tile(n0 + 128, t1, t2); }
+            if (n0 + 192 >= wg_n1) break;
         }
     }
 }
@@ -281,8 +340,10 @@ bool triple_mfma_supported(int dtype, int Dq, int Dv) { return (dtype == 1 || dt
 hipError_t launch_triple_state_mfma(const TripleArgs& a, int dtype, hipStream_t st)
 {
     dim3 grid(a.n_splits, a.H, a.B);
-    if (dtype == 1) hipLaunchKernelGGL(triple_state_mfma_kernel<bf16_t>, grid, dim3(256), 0, st, a);
-    else            hipLaunchKernelGGL(triple_state_mfma_kernel<f16_t>, grid, dim3(256), 0, st, a);
+    auto kern = dtype == 1 ? triple_state_mfma_kernel<bf16_t> : triple_state_mfma_kernel<f16_t>;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStateRedBytes);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, grid, dim3(256), kStateRedBytes, st, a);
     return hipGetLastError();
 }
 
