@@ -565,14 +565,13 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
         fws[tid] = fast_exp2(m2 - cref);
     }
     // running denominators of every latent (column c16 of tile ct), replicated in the waves
+    // (the earlier segments' local states are added segment by segment, in segment order: every load of one
+    // segment's contribution is issued before the first is consumed, instead of one round trip per element)
     float den0[CTA];
 #pragma unroll
     for (int ct = 0; ct < CTA; ++ct) {
         const int m = ct * 16 + c16;
-        const float mu = mu_g[m];
-        float d0 = mu <= kNegBig ? 0.f : den_g[m];
-        for (int s = 0; s < seg; ++s) d0 += a.seg_den[((int64_t)bh * a.n_segs + s) * M + m];
-        den0[ct] = d0;
+        den0[ct] = mu_g[m] <= kNegBig ? 0.f : den_g[m];
     }
     // state numerator of the wave's own latents: tile (mt, dt) holds rows m0 + 16 mt + 4g + r, column 16 dt + c16
     f32x4 U[MT][DT];
@@ -583,11 +582,28 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = m0 + mt * 16 + 4 * g + r;
-                float u = mu_g[m] <= kNegBig ? 0.f : num_g[(int64_t)m * D + dt * 16 + c16];
-                for (int s = 0; s < seg; ++s)
-                    u += a.seg_num[(((int64_t)bh * a.n_segs + s) * M + m) * D + dt * 16 + c16];
-                U[mt][dt][r] = u;
+                U[mt][dt][r] = mu_g[m] <= kNegBig ? 0.f : num_g[(int64_t)m * D + dt * 16 + c16];
             }
+    for (int s = 0; s < seg; ++s) {
+        const float* sd = a.seg_den + ((int64_t)bh * a.n_segs + s) * M;
+        const float* sn = a.seg_num + ((int64_t)bh * a.n_segs + s) * M * D;
+        float td[CTA];
+        f32x4 tu[MT][DT];
+#pragma unroll
+        for (int ct = 0; ct < CTA; ++ct) td[ct] = sd[ct * 16 + c16];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) tu[mt][dt][r] = sn[(int64_t)(m0 + mt * 16 + 4 * g + r) * D + dt * 16 + c16];
+#pragma unroll
+        for (int ct = 0; ct < CTA; ++ct) den0[ct] += td[ct];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) U[mt][dt] += tu[mt][dt];
+    }
 
     uint2 ltri, ones4 = make_uint2(P_::kOnes2, P_::kOnes2);
     {
@@ -599,7 +615,10 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     }
     const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
 
+    static_assert(kChunk * (D / 8) == VPT * 256, "every thread stages the same number of V pieces");
     u32x4 ka[KD], kn[KD], vr[VPT];
+    // K rows of the wave's 16 tokens and the thread's V pieces of a chunk; rows past the end of the segment repeat
+    // its last row (their probabilities are zeroed where they are used).  No branch: see the main loop.
     auto load_chunk = [&](int n0, u32x4 (&kk)[KD]) {
         const int n = min(n0 + 16 * w + c16, N - 1);
 #pragma unroll
@@ -607,22 +626,20 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             const int c = tid + i * 256, tok = c / (D / 8), ch = c % (D / 8);
-            if (c < kChunk * (D / 8)) vr[i] = *reinterpret_cast<const u32x4*>(v + (int64_t)min(n0 + tok, N - 1) * a.vs[2] + ch * 8);
+            vr[i] = *reinterpret_cast<const u32x4*>(v + (int64_t)min(n0 + tok, N - 1) * a.vs[2] + ch * 8);
         }
     };
     auto store_v = [&]() {
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             const int c = tid + i * 256, tok = c / (D / 8), ch = c % (D / 8);
-            if (c < kChunk * (D / 8)) {
-                u32x4 o = vr[i];
-                if constexpr (!std::is_same<T, bf16_t>::value) {
+            u32x4 o = vr[i];
+            if constexpr (!std::is_same<T, bf16_t>::value) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        o[j] = P_::pack2(M_::unpack(uint16_t(vr[i][j] & 0xffffu)), M_::unpack(uint16_t(vr[i][j] >> 16)));
-                }
-                *reinterpret_cast<u32x4*>(vs + tok * VS + ch * 8) = o;
+                for (int j = 0; j < 4; ++j)
+                    o[j] = P_::pack2(M_::unpack(uint16_t(vr[i][j] & 0xffffu)), M_::unpack(uint16_t(vr[i][j] >> 16)));
             }
+            *reinterpret_cast<u32x4*>(vs + tok * VS + ch * 8) = o;
         }
     };
     // the state of the wave's latents as B operands (k-slots = its 32 latents, lane = column d)
@@ -645,12 +662,16 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     load_chunk(n_lo, ka);
     store_v();
     publish_u();
-    if (n_lo + kChunk < N) load_chunk(n_lo + kChunk, kn);
     __syncthreads();                                        // q operands
 
     for (int n0 = n_lo; n0 < N; n0 += kChunk) {
         const int tbase = n0 + 16 * w;
         const int tbw = min(16, max(0, N - tbase));        // valid tokens of this wave in the chunk
+        // The next chunk's K rows and V pieces are requested here, a whole chunk before they are handed over at the
+        // bottom of the iteration (past the end of the segment the last rows are fetched again and never used).
+        // Unconditional, so that the compiler's wait at the hand-over counts what is in flight instead of draining
+        // whatever was issued last.
+        load_chunk(n0 + kChunk, kn);
 
         // ---- token side, part 1: scores, P, column sums; publish P^T ----
         // (staged over the eight latent tiles: every LDS read before the first LDS write, so that the reads
@@ -788,7 +809,6 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
             for (int kd = 0; kd < KD; ++kd) ka[kd] = kn[kd];
             store_v();
             publish_u();
-            if (n0 + 2 * kChunk < N) load_chunk(n0 + 2 * kChunk, kn);
         }
     }
 
