@@ -331,8 +331,10 @@ TriplePlan plan_triple(const FlareTripleDesc* d)
     p.mfma = triple_wants_mfma(d);
     int s = d->n_splits;
     if (s <= 0) {
-        // about two workgroups per compute unit: more splits only add partials to write and merge
-        const int64_t per = (int64_t)d->B * d->H;
+        // about two workgroups per compute unit: more splits only add partials to write and merge (the matrix-core
+        // state kernel runs one workgroup per split and 16 x 16 x 16 block of the state)
+        const int64_t nb = p.mfma ? (int64_t)(d->Dq / 16) * (d->Dv / 16) * (d->Dq / 16) : 1;
+        const int64_t per = (int64_t)d->B * d->H * nb;
         s = (int)((2 * flare::device_cus() + per - 1) / per);
         if (s < 1) s = 1;
     }
@@ -341,7 +343,9 @@ TriplePlan plan_triple(const FlareTripleDesc* d)
     p.tokens_per_split = (int)tps;
     p.n_splits = (int)(((int64_t)d->N + tps - 1) / tps);
     p.n_parts = p.n_splits;
-    p.per_split = (size_t)d->Dq * d->Dv * d->Dq + (size_t)d->Dq * d->Dq;
+    // sized for whichever kernel family ends up running (misaligned pointers demote to the fp32 kernels)
+    p.per_split = flare::triple_partial_floats(d->Dq, d->Dv, false);
+    if (p.mfma) p.per_split = std::max(p.per_split, flare::triple_partial_floats(d->Dq, d->Dv, true));
     const size_t bh = (size_t)d->B * d->H;
     p.off_kk = bh * p.n_parts * p.per_split * 4;
     p.off_kk = (p.off_kk + 255) & ~(size_t)255;

@@ -125,11 +125,18 @@ struct TripleArgs {
     float* part;       // [B,H,S,Dq*Dv*Dq (+Dq*Dq)] split partials
     int B, H, N, Dq, Dv;
     int feature_map, normalize;
-    int diag_parts;    // 1: partials in the matrix-core kernel's accumulator order [step][lane][register] (16^3 only)
+    int diag_parts;    // 1: partials from the matrix-core kernel: blocks of 16^3 in accumulator order [step][lane][register]
     int n_splits, tokens_per_split;
     int n_parts;       // partials per (b,h) in `part`
     int64_t q1s[3], q2s[3], k1s[3], k2s[3], vs[3], os[3];
 };
+
+// Floats of one split partial of the triple state: [Dq][Dv][Dq] + [Dq][Dq] from the fp32 kernels, or one
+// (16^3 + 16^2)-float tile per 16 x 16 x 16 block from the matrix-core kernels.
+__host__ __device__ inline size_t triple_partial_floats(int Dq, int Dv, bool diag)
+{
+    return diag ? (size_t)(Dq / 16) * (Dv / 16) * (Dq / 16) * 4352 : (size_t)Dq * Dv * Dq + (size_t)Dq * Dq;
+}
 
 struct MixerBwdArgs {
     const void* q; const void* k; const void* v; const void* y; const void* dy;

@@ -91,7 +91,8 @@ __global__ __launch_bounds__(kThreads) void triple_state_kernel(TripleArgs a, in
 
 __global__ __launch_bounds__(kThreads) void triple_merge_kernel(TripleArgs a)
 {
-    const size_t ns = (size_t)a.Dq * a.Dv * a.Dq, nk = (size_t)a.Dq * a.Dq, per = ns + nk;
+    const size_t ns = (size_t)a.Dq * a.Dv * a.Dq, nk = (size_t)a.Dq * a.Dq;
+    const size_t per = triple_partial_floats(a.Dq, a.Dv, a.diag_parts != 0);
     const size_t total = (size_t)a.B * a.H * per;
     const size_t idx = (size_t)blockIdx.x * kThreads + threadIdx.x;
     if (idx >= total) return;
@@ -100,16 +101,25 @@ __global__ __launch_bounds__(kThreads) void triple_merge_kernel(TripleArgs a)
     float s = 0.f;
     for (int sp = 0; sp < a.n_parts; ++sp) s += p[(size_t)sp * per];
     s *= 1.0f / (float)a.N;
-    size_t o = e < ns ? e : e - ns;
-    if (a.diag_parts) {
-        // element (step r, lane = 16 g + c16, register rr) of the matrix-core kernel's accumulators holds
-        // state[i = 4g + rr][j = c16][k = (i - r) mod 16]; its normaliser tile holds kk[i = 4g + rr][k' = c16]
-        const int r = (int)(o >> 8), lane = (int)(o >> 2) & 63, rr = (int)o & 3;
-        const int i = 4 * (lane >> 4) + rr, c16 = lane & 15;
-        o = e < ns ? ((size_t)i * 16 + c16) * 16 + ((i - r) & 15) : (size_t)i * 16 + c16;
+    if (!a.diag_parts) {
+        if (e < ns) a.state[bh * ns + e] = s;
+        else if (a.kk) a.kk[bh * nk + (e - ns)] = s;
+        return;
     }
-    if (e < ns) a.state[bh * ns + o] = s;
-    else if (a.kk) a.kk[bh * nk + o] = s;
+    // Matrix-core partials: one 16 x 16 x 16 block after the other, each in the kernel's accumulator order.  Element
+    // (step r, lane = 16 g + c16, register rr) of a block holds state[i = 4g + rr][j = c16][k = (i - r) mod 16] of
+    // the block; the tile behind the sixteen steps holds the block's kk[i = 4g + rr][k' = c16] (the same for every
+    // column block jb: taken from jb = 0).
+    const int nbq = a.Dq >> 4, nbv = a.Dv >> 4;
+    const int blk = (int)(e / 4352), o = (int)(e % 4352);
+    const int ib = blk / (nbv * nbq), jb = (blk / nbq) % nbv, kb = blk % nbq;
+    const int r = o >> 8, lane = (o >> 2) & 63, rr = o & 3;
+    const int i = 4 * (lane >> 4) + rr, c16 = lane & 15;
+    if (o < 4096) {
+        a.state[bh * ns + ((size_t)(16 * ib + i) * a.Dv + 16 * jb + c16) * a.Dq + 16 * kb + ((i - r) & 15)] = s;
+    } else if (a.kk && jb == 0) {
+        a.kk[bh * nk + (size_t)(16 * ib + i) * a.Dq + 16 * kb + c16] = s;
+    }
 }
 
 constexpr int kOutLdsFloats = 8192;
@@ -229,7 +239,7 @@ hipError_t launch_triple_state(const TripleArgs& a, int dtype, hipStream_t st)
 
 hipError_t launch_triple_merge(const TripleArgs& a, hipStream_t st)
 {
-    const size_t per = (size_t)a.Dq * a.Dv * a.Dq + (size_t)a.Dq * a.Dq;
+    const size_t per = triple_partial_floats(a.Dq, a.Dv, a.diag_parts != 0);
     const size_t total = (size_t)a.B * a.H * per;
     hipLaunchKernelGGL(triple_merge_kernel, dim3((unsigned)((total + kThreads - 1) / kThreads)), dim3(kThreads), 0, st, a);
     return hipGetLastError();

@@ -1,4 +1,5 @@
-// Triple (third-order) linear attention on the matrix cores: bf16 / f16, Dq = Dv = 16.
+// Triple (third-order) linear attention on the matrix cores: bf16 / f16, head dims that are multiples of 16 up to 64
+// (both contractions are sums over blocks of 16 indices; the text below describes one 16 x 16 x 16 block).
 //
 //   state[i,j,k] = (1/N) sum_n f(k1)[n,i] v[n,j] f(k2)[n,k]      (lra/models/backends.py:1289 of the reference)
 //   out[n,j]     = sum_{i,k} f(q1)[n,i] state[i,j,k] f(q2)[n,k]  (backends.py:1290)
@@ -98,8 +99,8 @@ __device__ __forceinline__ float row16_sum(float x)
 constexpr int kD = 16;
 
 // x * (the value y has in lane (c - R) mod 16 of the same 16-lane row): one vector instruction with a DPP row
-// rotate on its first operand.  y must have been written at least two instructions earlier (the DPP read of a
-// freshly written register needs two wait states, which callers provide by computing all factors up front).
+// rotate on its first operand.  The DPP read of a freshly written register needs two wait states that the compiler
+// does not insert for assembly it cannot see into: the caller provides them (see the state kernel's tile).
 template <int R> __device__ __forceinline__ float mul_row_ror(float x, float y)
 {
     if constexpr (R == 0) {
@@ -113,7 +114,8 @@ template <int R> __device__ __forceinline__ float mul_row_ror(float x, float y)
 
 constexpr size_t kStateRedBytes = 4 * (kD + 1) * 64 * 4 * sizeof(float);
 
-// grid (n_splits, H, B); wave w of a workgroup takes the 16-token tiles w, w+4, ... of the split.
+// grid (n_splits * blocks, H, B), blocks = (Dq/16)^2 (Dv/16) blocks of 16 x 16 x 16 state entries (one for head dims
+// of 16); wave w of a workgroup takes the 16-token tiles w, w+4, ... of the split.
 //
 // Per tile the wave stages f(k1), f(k2), v (rounded to the element type) in its own LDS tile and takes all three
 // with tokens in the k-slots (transpose read: lane = feature c16, slots = tokens 4g..4g+3).  The state is
@@ -131,10 +133,13 @@ __global__ __launch_bounds__(256, 2) void triple_state_mfma_kernel(TripleArgs a)
     float (*red)[kD + 1][64][4] = reinterpret_cast<float (*)[kD + 1][64][4]>(triple_red);
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
-    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const uint16_t* k1 = (const uint16_t*)a.k1 + b * a.k1s[0] + h * a.k1s[1];
-    const uint16_t* k2 = (const uint16_t*)a.k2 + b * a.k2s[0] + h * a.k2s[1];
-    const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
+    // the workgroup's 16 x 16 x 16 block of the state: rows i of block ib, columns j of block jb, slices k of block kb
+    const int nbq = a.Dq >> 4, nbv = a.Dv >> 4, NB = nbq * nbv * nbq;
+    const int split = blockIdx.x / NB, blk = blockIdx.x % NB, h = blockIdx.y, b = blockIdx.z;
+    const int ib = blk / (nbv * nbq), jb = (blk / nbq) % nbv, kb = blk % nbq;
+    const uint16_t* k1 = (const uint16_t*)a.k1 + b * a.k1s[0] + h * a.k1s[1] + 16 * ib;
+    const uint16_t* k2 = (const uint16_t*)a.k2 + b * a.k2s[0] + h * a.k2s[1] + 16 * kb;
+    const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1] + 16 * jb;
     const int n_begin = split * a.tokens_per_split;
     const int n_end = min(a.N, n_begin + a.tokens_per_split);
     const int tok = lane >> 2, piece = (lane & 3) * 4;   // staging: lane = (token, 4 elements)
@@ -178,7 +183,11 @@ __global__ __launch_bounds__(256, 2) void triple_state_mfma_kernel(TripleArgs a)
         const uint2 vt = tr16(&vs[w][tr_row][tr_col]);
         kk = M_::mma16(k1t, k2t, kk);
         const float k1f[4] = {M_::lo(k1t.x), M_::hi(k1t.x), M_::lo(k1t.y), M_::hi(k1t.y)};
-        const float k2f[4] = {M_::lo(k2t.x), M_::hi(k2t.x), M_::lo(k2t.y), M_::hi(k2t.y)};
+        float k2f[4] = {M_::lo(k2t.x), M_::hi(k2t.x), M_::lo(k2t.y), M_::hi(k2t.y)};
+        // The DPP reads of k2f below sit in assembly the compiler does not look into, so it cannot place the two wait
+        // states a DPP read needs after the instruction that wrote the register: this statement "rewrites" the four
+        // factors (nothing may move across it) and spends those wait states once per tile.
+        asm volatile("s_nop 1" : "+v"(k2f[0]), "+v"(k2f[1]), "+v"(k2f[2]), "+v"(k2f[3]));
         step(std::integral_constant<int, 0>{}, k1f, k2f, vt);   step(std::integral_constant<int, 1>{}, k1f, k2f, vt);
         step(std::integral_constant<int, 2>{}, k1f, k2f, vt);   step(std::integral_constant<int, 3>{}, k1f, k2f, vt);
         step(std::integral_constant<int, 4>{}, k1f, k2f, vt);   step(std::integral_constant<int, 5>{}, k1f, k2f, vt);
@@ -213,7 +222,7 @@ __global__ __launch_bounds__(256, 2) void triple_state_mfma_kernel(TripleArgs a)
     *reinterpret_cast<f32x4*>(&red[w][kD][lane][0]) = kk;
     __syncthreads();
     const size_t per = (size_t)kD * kD * kD + (size_t)kD * kD;
-    float* part = a.part + (((size_t)b * a.H + h) * a.n_parts + split) * per;
+    float* part = a.part + ((((size_t)b * a.H + h) * a.n_parts + split) * NB + blk) * per;
     // The partial keeps the accumulators' own order, [step r][lane][register rr] (and the normaliser tile behind
     // them), so that every store is 16 contiguous bytes per lane; the merge kernel puts the sums into [i][j][k].
 #pragma unroll
@@ -333,13 +342,119 @@ __global__ __launch_bounds__(256) void triple_out_mfma_kernel(TripleArgs a, int 
     }
 }
 
+// Head dims that are larger multiples of 16 (up to 64).  grid (ceil(N / tokens_per_wg) * Dv/16, H, B): a workgroup
+// produces 16 output columns (block jb) for its token range.  The contraction over (i, k) runs over (Dq/16)^2 pairs
+// of index blocks; their state slices sit in LDS as A operands (built once per workgroup), f(q1) pieces come
+// straight from global memory as B operands, and f(q2) of the wave's tile passes through a wave-private LDS tile
+// that hands every lane its token's features.
+template <typename T>
+__global__ __launch_bounds__(256) void triple_out_blocks_kernel(TripleArgs a, int tokens_per_wg)
+{
+    using M_ = Tm<T>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t triple_out_lds[];
+    const int Dq = a.Dq, Dv = a.Dv, nbq = Dq >> 4, nbv = Dv >> 4, NP = nbq * nbq, QS = Dq + 4;
+    uint2* skt = reinterpret_cast<uint2*>(triple_out_lds);                 // [pair][k][lane]
+    uint2* kkt = skt + (size_t)NP * kD * 64;                                // [pair][lane]
+    float* q2f = reinterpret_cast<float*>(kkt + (size_t)NP * 64);           // [wave][16][QS]
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int jb = blockIdx.x % nbv, wgx = blockIdx.x / nbv, h = blockIdx.y, b = blockIdx.z;
+    const size_t bh = (size_t)b * a.H + h;
+    const uint16_t* q1 = (const uint16_t*)a.q1 + b * a.q1s[0] + h * a.q1s[1];
+    const uint16_t* q2 = (const uint16_t*)a.q2 + b * a.q2s[0] + h * a.q2s[1];
+    uint16_t* out = (uint16_t*)a.out + b * a.os[0] + h * a.os[1] + 16 * jb;
+    const float* state = a.state + bh * Dq * Dv * Dq;
+    const float* kkp = a.kk + bh * Dq * Dq;
+    float* q2w = q2f + (size_t)w * 16 * QS;
+
+    // operand tables: entry (pair = ib nbq + kb, k, lane) = state[16 ib + 4g + e][16 jb + c16][16 kb + k], e = 0..3
+    for (int idx = tid; idx < NP * kD * 64; idx += 256) {
+        const int ln = idx & 63, k = (idx >> 6) & 15, pair = idx >> 10;
+        const int ibb = pair / nbq, kbb = pair % nbq, gg = ln >> 4, cc = ln & 15;
+        const float* s0 = state + ((size_t)(16 * ibb + 4 * gg) * Dv + 16 * jb + cc) * Dq + 16 * kbb + k;
+        const size_t rs = (size_t)Dv * Dq;
+        skt[idx] = make_uint2(M_::pack2(s0[0], s0[rs]), M_::pack2(s0[2 * rs], s0[3 * rs]));
+    }
+    if (a.normalize)
+        for (int idx = tid; idx < NP * 64; idx += 256) {
+            const int ln = idx & 63, pair = idx >> 6;
+            const int ibb = pair / nbq, kbb = pair % nbq, gg = ln >> 4, cc = ln & 15;
+            const float* s0 = kkp + (size_t)(16 * ibb + 4 * gg) * Dq + 16 * kbb + cc;
+            kkt[idx] = make_uint2(M_::pack2(s0[0], s0[Dq]), M_::pack2(s0[2 * Dq], s0[3 * Dq]));
+        }
+    __syncthreads();
+
+    const int wg_n0 = wgx * tokens_per_wg;
+    const int wg_n1 = min(a.N, wg_n0 + tokens_per_wg);
+    const int tok = lane >> 2, piece = (lane & 3) * 4;
+    for (int n0 = wg_n0 + w * 16; n0 < wg_n1; n0 += 64) {
+        // raw pieces of the tile: q1 as B operands (token c16, features 16 ib + 4g..), q2 as the lane's share of the tile
+        uint2 r1[4], r2[4];
+        const uint16_t* q1r = q1 + (int64_t)min(n0 + c16, wg_n1 - 1) * a.q1s[2] + 4 * g;
+        const uint16_t* q2r = q2 + (int64_t)min(n0 + tok, wg_n1 - 1) * a.q2s[2] + piece;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (i < nbq) {
+                r1[i] = *reinterpret_cast<const uint2*>(q1r + 16 * i);
+                r2[i] = *reinterpret_cast<const uint2*>(q2r + 16 * i);
+            }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (i < nbq) {
+                const uint2 f2 = feat4_of<T>(r2[i], n0 + tok < wg_n1, a.feature_map);
+                *reinterpret_cast<f32x4*>(q2w + tok * QS + 16 * i + piece) = f32x4{M_::lo(f2.x), M_::hi(f2.x), M_::lo(f2.y), M_::hi(f2.y)};
+            }
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};   // out[n = c16][j = 16 jb + 4g + e]
+        float den = 0.f;
+        for (int ibb = 0; ibb < nbq; ++ibb) {
+            uint2 raw = r1[0];
+#pragma unroll
+            for (int i = 1; i < 4; ++i) raw = ibb == i ? r1[i] : raw;
+            const uint2 q1b = feat4_of<T>(raw, n0 + c16 < wg_n1, a.feature_map);
+            for (int kbb = 0; kbb < nbq; ++kbb) {
+                const int pair = ibb * nbq + kbb;
+                float r[kD];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const f32x4 t = *reinterpret_cast<const f32x4*>(q2w + c16 * QS + 16 * kbb + 4 * c);
+                    r[4 * c] = t[0]; r[4 * c + 1] = t[1]; r[4 * c + 2] = t[2]; r[4 * c + 3] = t[3];
+                }
+                const uint2* sk = skt + (size_t)pair * kD * 64 + lane;
+#pragma unroll
+                for (int k = 0; k < kD; ++k) {
+                    const f32x4 t = M_::mma16(sk[k * 64], q1b, f32x4{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[e] = fmaf(t[e], r[k], acc[e]);
+                }
+                if (a.normalize) {
+                    const f32x4 wv = M_::mma16(kkt[pair * 64 + lane], q1b, f32x4{0.f, 0.f, 0.f, 0.f});
+                    const f32x4 rq = *reinterpret_cast<const f32x4*>(q2w + c16 * QS + 16 * kbb + 4 * g);
+                    den += wv[0] * rq[0] + wv[1] * rq[1] + wv[2] * rq[2] + wv[3] * rq[3];
+                }
+            }
+        }
+        if (a.normalize) {
+            const float inv = 1.f / sum_xor32(sum_xor16(den));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] *= inv;
+        }
+        if (n0 + c16 < wg_n1)
+            *reinterpret_cast<uint2*>(out + (int64_t)(n0 + c16) * a.os[2] + 4 * g) =
+                make_uint2(M_::pack2(acc[0], acc[1]), M_::pack2(acc[2], acc[3]));
+    }
+}
+
 }  // namespace
 
-bool triple_mfma_supported(int dtype, int Dq, int Dv) { return (dtype == 1 || dtype == 2) && Dq == 16 && Dv == 16; }
+// 16-bit inputs, both head dims multiples of 16 up to 64
+bool triple_mfma_supported(int dtype, int Dq, int Dv)
+{
+    return (dtype == 1 || dtype == 2) && Dq % 16 == 0 && Dv % 16 == 0 && Dq >= 16 && Dv >= 16 && Dq <= 64 && Dv <= 64;
+}
 
 hipError_t launch_triple_state_mfma(const TripleArgs& a, int dtype, hipStream_t st)
 {
-    dim3 grid(a.n_splits, a.H, a.B);
+    dim3 grid(a.n_splits * (a.Dq / 16) * (a.Dv / 16) * (a.Dq / 16), a.H, a.B);
     auto kern = dtype == 1 ? triple_state_mfma_kernel<bf16_t> : triple_state_mfma_kernel<f16_t>;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStateRedBytes);
     if (e != hipSuccess) return e;
@@ -354,6 +469,18 @@ hipError_t launch_triple_out_mfma(const TripleArgs& a, int dtype, hipStream_t st
     int64_t tpw = (a.N + per_bh - 1) / per_bh;
     tpw = ((tpw + 63) / 64) * 64;
     if (tpw < 256) tpw = 256;
+    if (a.Dq > 16 || a.Dv > 16) {
+        const int nbq = a.Dq / 16, nbv = a.Dv / 16;
+        // the operand tables are rebuilt by every workgroup: longer token ranges than for 16 x 16
+        if (tpw < 1024) tpw = 1024;
+        const size_t lds = (size_t)nbq * nbq * (kD + 1) * 64 * sizeof(uint2) + (size_t)4 * 16 * (a.Dq + 4) * sizeof(float);
+        auto kern = dtype == 1 ? triple_out_blocks_kernel<bf16_t> : triple_out_blocks_kernel<f16_t>;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        dim3 grid((unsigned)((a.N + tpw - 1) / tpw) * nbv, a.H, a.B);
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, a, (int)tpw);
+        return hipGetLastError();
+    }
     dim3 grid((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B);
     if (dtype == 1) hipLaunchKernelGGL(triple_out_mfma_kernel<bf16_t>, grid, dim3(256), 0, st, a, (int)tpw);
     else            hipLaunchKernelGGL(triple_out_mfma_kernel<f16_t>, grid, dim3(256), 0, st, a, (int)tpw);

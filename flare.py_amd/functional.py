@@ -1053,23 +1053,17 @@ def _triple_forward(q1, q2, k1, k2, v, feature_map: bool, normalize: bool, n_spl
     B, H, N, Dq = q1.shape
     Dv = v.shape[-1]
     Dqp, Dvp = -(-Dq // 16) * 16, -(-Dv // 16) * 16
-    if (Dq, Dv) != (16, 16) and n_splits == 0:
-        if q1.dtype in (torch.bfloat16, torch.float16) and max(Dqp, Dvp) <= 64:
-            # Any head dims up to 64 on the 16 x 16 x 16 matrix-core kernels: features first (elu + 1, rounded to the
-            # element type as the kernels do when they stage a tile), then zero columns up to a multiple of 16 (they add
-            # nothing to either contraction), then one launch per block of indices.
-            if feature_map:
-                q1, q2, k1, k2 = ((torch.nn.functional.elu(t.float()) + 1.0).to(t.dtype) for t in (q1, q2, k1, k2))
-            if Dqp != Dq:
-                q1, q2, k1, k2 = (_pad_last(t, Dqp - Dq) for t in (q1, q2, k1, k2))
-            vp = _pad_last(v, Dvp - Dv) if Dvp != Dv else v
-            state = _triple_state(k1, k2, vp)
-            num = _triple_out(q1, q2, state, torch.float32)
-            if normalize:           # the same contraction with v = 1 (one block column of ones)
-                ones = torch.ones((B, H, N, 16), dtype=v.dtype, device=v.device)
-                den = _triple_out(q1, q2, _triple_state(k1, k2, ones), torch.float32)[..., :1]
-                num = num / den
-            return state[:, :, :Dq, :Dv, :Dq].contiguous(), num[..., :Dv].to(q1.dtype)
+    if (Dqp, Dvp) != (Dq, Dv) and q1.dtype in (torch.bfloat16, torch.float16) and max(Dqp, Dvp) <= 64:
+        # The matrix-core kernels take head dims that are multiples of 16 (up to 64).  Any other head dim up to 64:
+        # features first (elu + 1, rounded to the element type as the kernels do when they stage a tile), then zero
+        # columns up to the next multiple of 16 (they add nothing to either contraction, nor to the normaliser).
+        if feature_map:
+            q1, q2, k1, k2 = ((torch.nn.functional.elu(t.float()) + 1.0).to(t.dtype) for t in (q1, q2, k1, k2))
+        if Dqp != Dq:
+            q1, q2, k1, k2 = (_pad_last(t, Dqp - Dq) for t in (q1, q2, k1, k2))
+        vp = _pad_last(v, Dvp - Dv) if Dvp != Dv else v
+        state, out = _triple_forward(q1, q2, k1, k2, vp, False, normalize, n_splits)
+        return state[:, :, :Dq, :Dv, :Dq].contiguous(), out[..., :Dv].contiguous()
     state = torch.empty((B, H, Dq, Dv, Dq), dtype=torch.float32, device=q1.device)
     out = torch.empty((B, H, N, Dv), dtype=q1.dtype, device=q1.device)
     d = FlareTripleDesc()
@@ -1134,41 +1128,15 @@ def _triple_out_launch(q1, q2, state):
     return out
 
 
-def _in_blocks_of_16(Dq, Dv, t) -> bool:
-    """The matrix-core triple kernels are 16 x 16 x 16.  Both contractions are sums over index blocks, so head dims
-    that are larger multiples of 16 run as (Dq/16)^2 (Dv/16) launches of those kernels on 16-column slices (views,
-    no copies of the inputs) instead of one launch of the fp32-FMA kernels: 9.2 -> about 1 ms at Dq = Dv = 32."""
-    return (t.dtype in (torch.bfloat16, torch.float16) and t.device.type == "cuda" and Dq % 16 == 0 and Dv % 16 == 0
-            and max(Dq, Dv) > 16 and max(Dq, Dv) <= 64)          # 16 x 16 itself is the plain launch
-
-
 def _triple_state(k1, k2, v):
     """state [B,H,Dq,Dv,Dq] fp32 = (1/N) sum_n k1[n,i] v[n,j] k2[n,k]."""
-    Dq, Dv = k1.shape[-1], v.shape[-1]
-    if not _in_blocks_of_16(Dq, Dv, k1):
-        return _triple_state_launch(k1, k2, v)
-    B, H = k1.shape[:2]
-    state = torch.empty((B, H, Dq, Dv, Dq), dtype=torch.float32, device=k1.device)
-    for i in range(0, Dq, 16):
-        for j in range(0, Dv, 16):
-            for k in range(0, Dq, 16):
-                state[:, :, i:i + 16, j:j + 16, k:k + 16] = _triple_state_launch(k1[..., i:i + 16], k2[..., k:k + 16], v[..., j:j + 16])
-    return state
+    return _triple_state_launch(k1, k2, v)
 
 
 def _triple_out(q1, q2, state, out_dtype=None):
-    """out [B,H,N,Dv] = sum_{i,k} q1[n,i] state[i,j,k] q2[n,k]; out_dtype=torch.float32 keeps the block sums unrounded."""
-    Dq, Dv = q1.shape[-1], state.shape[3]
-    if not _in_blocks_of_16(Dq, Dv, q1):
-        out = _triple_out_launch(q1, q2, state)
-        return out if out_dtype is None else out.to(out_dtype)
-    B, H, N = q1.shape[:3]
-    out = torch.zeros((B, H, N, Dv), dtype=torch.float32, device=q1.device)
-    for j in range(0, Dv, 16):
-        for i in range(0, Dq, 16):
-            for k in range(0, Dq, 16):
-                out[..., j:j + 16] += _triple_out_launch(q1[..., i:i + 16], q2[..., k:k + 16], state[:, :, i:i + 16, j:j + 16, k:k + 16])
-    return out.to(q1.dtype if out_dtype is None else out_dtype)
+    """out [B,H,N,Dv] = sum_{i,k} q1[n,i] state[i,j,k] q2[n,k]."""
+    out = _triple_out_launch(q1, q2, state)
+    return out if out_dtype is None else out.to(out_dtype)
 
 
 class _TripleFn(torch.autograd.Function):

@@ -99,9 +99,10 @@ def test_backward_matches_autograd_of_the_einsum_oracle(dev, dtype, D, Dv, tol):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("Dq,Dv", [(32, 32), (16, 32), (32, 16), (64, 64), (48, 32), (8, 8), (20, 24), (4, 40)])
 def test_head_dims_in_blocks_of_16(dev, Dq, Dv, dtype):
-    """Head dims other than 16 run as launches of the 16 x 16 x 16 matrix-core kernels over index blocks, zero-padded to
-    a multiple of 16 where needed (the reference's Triton path takes any D >= 16 with D % 4 == 0,
-    lra/models/triton/triple.py:69-70; its einsum path any D)."""
+    """Head dims that are larger multiples of 16 run on the matrix-core kernels block by block inside one launch (state:
+    one workgroup per 16 x 16 x 16 block and split; output: the (i, k) block pairs looped over LDS-resident operands);
+    other head dims are zero-padded to a multiple of 16 first (the reference's Triton path takes any D >= 16 with
+    D % 4 == 0, lra/models/triton/triple.py:69-70; its einsum path any D)."""
     a = make(2, 2, 900, Dq, Dv, dtype, seed=Dq + Dv)
     st, out = F.triple_attention(*[t.to(dev) for t in a], normalize=True, feature_map="elu")
     sr, orf = O.triple_einsum(*[t.float() for t in a], feature_map=True, normalize=True, dtype=torch.float64)
@@ -110,3 +111,17 @@ def test_head_dims_in_blocks_of_16(dev, Dq, Dv, dtype):
     c = torch.full_like(a[4], -0.5)                       # constant v, normalised => constant output
     _, oc = F.triple_attention(*[t.to(dev) for t in a[:4]], c.to(dev), normalize=True, feature_map="elu")
     assert torch.allclose(oc.float().cpu(), c.float(), atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 5e-3), (torch.float16, 1e-3)])
+@pytest.mark.parametrize("D", [16, 32, 64])
+def test_state_is_tight_for_any_number_of_tiles_per_wave(dev, dtype, tol, D):
+    """The state kernel's waves walk 1, 2, 4 ... tiles depending on the split count; its per-tile factors are read
+    through DPP row rotates, whose wait states the kernel provides itself.  The state must stay at rounding level
+    (products rounded once to the element type: about 3e-3 in bf16, 4e-4 in f16) for every split count."""
+    a = make(2, 2, 900, D, D, dtype, seed=3 * D)
+    sr, orf = O.triple_einsum(*[t.float() for t in a], feature_map=True, normalize=True, dtype=torch.float64)
+    for ns in (0, 1, 2, 4, 8):
+        st, out = F.triple_attention(*[t.to(dev) for t in a], normalize=True, feature_map="elu", n_splits=ns)
+        assert O.rel_l2(st, sr) <= tol, (ns, O.rel_l2(st, sr))
+        assert O.rel_l2(out, orf) <= TOL[dtype]
