@@ -667,6 +667,11 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     for (int n0 = n_lo; n0 < N; n0 += kChunk) {
         const int tbase = n0 + 16 * w;
         const int tbw = min(16, max(0, N - tbase));        // valid tokens of this wave in the chunk
+        // Tokens past the end of the segment (only its last chunk can have any) get probability 0 through the initial
+        // value of their score accumulators: one quad per chunk, shared by the eight latent tiles.
+        f32x4 absent;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) absent[r] = (4 * g + r < tbw) ? 0.f : -1.0e30f;
         // The next chunk's K rows and V pieces are requested here, a whole chunk before they are handed over at the
         // bottom of the iteration (past the end of the segment the last rows are fetched again and never used).
         // Unconditional, so that the compiler's wait at the hand-over counts what is in flight instead of draining
@@ -682,7 +687,7 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
             f32x4 sc[CTA];
 #pragma unroll
             for (int ct = 0; ct < CTA; ++ct) {
-                f32x4 s = zf;
+                f32x4 s = absent;
 #pragma unroll
                 for (int kd = 0; kd < KD; ++kd) s = M_::mma32(ka[kd], qs[(ct * KD + kd) * 64 + lane], s);
                 sc[ct] = s;
@@ -691,7 +696,7 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
             for (int ct = 0; ct < CTA; ++ct) {
                 const float mu0 = mu0s[ct * 16 + c16];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) p[ct][r] = (4 * g + r < tbw) ? fast_exp2(sc[ct][r] - mu0) : 0.f;
+                for (int r = 0; r < 4; ++r) p[ct][r] = fast_exp2(sc[ct][r] - mu0);
                 ppk[ct] = make_uint2(P_::pack2(p[ct][0], p[ct][1]), P_::pack2(p[ct][2], p[ct][3]));
             }
             f32x4 csv[CTA];
@@ -719,7 +724,8 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
             float gv[4];
             const float fw = fws[m];      // the token's softmax weight over the latents is P * exp2(mu0 - cref)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) gv[r] = p[ct][r] > 0.f ? p[ct][r] * fw * __builtin_amdgcn_rcpf(dc[r] + base) : 0.f;
+            for (int r = 0; r < 4; ++r)      // dcum >= the element's own P: clamped away from 0 it gives G = 0 where P = 0
+                gv[r] = p[ct][r] * fw * __builtin_amdgcn_rcpf(fmaxf(dc[r] + base, 1.17549435e-38f));
             *reinterpret_cast<uint2*>(gtw + (ct * 16 + c16) * 16 + 4 * g) = make_uint2(P_::pack2(gv[0], gv[1]), P_::pack2(gv[2], gv[3]));
         }
         u32x4 gop[KS], pop[KS];
@@ -766,7 +772,7 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
             float inv[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                inv[r] = 1.f / rsum[r];
+                inv[r] = __builtin_amdgcn_rcpf(rsum[r]);
                 if (4 * g + r < tbw) {
                     bad = bad || !(rsum[r] >= kLMin && rsum[r] <= kLMax);
                     if (a.lse && c16 == 0) a.lse[(int64_t)bh * a.N + tbase + 4 * g + r] = (cref + __log2f(rsum[r])) * kLn2;
