@@ -74,7 +74,29 @@ __global__ __launch_bounds__(kThreads) void causal_generic_kernel(CausalArgs a)
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H;
-    if (a.flags != nullptr && a.flags[bh] == 0) return;   // fallback launch: only marked (b,h) are redone
+    if (a.flags != nullptr && a.flags[bh] == 0) {
+        // Launched behind the matrix-core kernels: only marked (b,h) are redone.  For the others a prefill in several
+        // segments has staged its final state in the last segment's workspace slot; it becomes (mu, den, num) here,
+        // once every segment is known to have passed (a fresh state's shift becomes 0).
+        if (a.n_segs > 1) {
+            const int M = a.M, D = a.D;
+            const float* sd = a.seg_den + ((int64_t)bh * a.n_segs + a.n_segs - 1) * M;
+            const float* sn = a.seg_num + ((int64_t)bh * a.n_segs + a.n_segs - 1) * M * D;
+            float* num = a.num + (int64_t)bh * M * D;
+            for (int i = tid; i < M; i += kThreads) {
+                const float mu = a.mu[(int64_t)bh * M + i];
+                a.mu[(int64_t)bh * M + i] = mu <= kNegBig ? 0.f : mu;
+                a.den[(int64_t)bh * M + i] = sd[i];
+            }
+            if (((reinterpret_cast<uintptr_t>(num) | reinterpret_cast<uintptr_t>(sn)) & 15) == 0 && (M * D) % 4 == 0) {
+                for (int i = tid; i < M * D / 4; i += kThreads)
+                    reinterpret_cast<float4*>(num)[i] = reinterpret_cast<const float4*>(sn)[i];
+            } else {
+                for (int i = tid; i < M * D; i += kThreads) num[i] = sn[i];
+            }
+        }
+        return;
+    }
     const T* q = (const T*)a.q + b * a.qs[0] + h * a.qs[1];
     const T* k = (const T*)a.k + b * a.ks[0] + h * a.ks[1];
     const T* v = (const T*)a.v + b * a.vs[0] + h * a.vs[1];

@@ -241,50 +241,59 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
     };
 
     if constexpr (STATE_ONLY) {
+        // The first phase never raises a flag, and the recurrence phase starts after it has finished: its first
+        // segment clears the (b,h)'s redo flag (by a kernel, so that a caller may capture the call in a graph).
+        if (seg == 0 && tid == 0) a.flags[bh] = 0;
         // Local state of the segment.  A 16-token block is too little work here to cover the memory
         // latency of its own prefetch, so this phase walks 64-token tiles: K as four A operands per
-        // lane, V through a 64-row LDS tile, the next tile in flight while the current is used.
+        // lane, V through a 64-row LDS tile.  Three register sets take turns, each refilled with the tile
+        // three ahead as soon as its own has been used: loads are unconditional (rows past the end of
+        // the segment repeat its last row) and never copied between registers, so that every wait counts
+        // exactly what is in flight.
         __shared__ __attribute__((aligned(16))) uint16_t v64[2][64][D + kVPad];
-        constexpr int VPT = (64 * (D / 8) + 255) / 256;     // 16-byte V chunks per thread and tile
-        u32x4 k4[4][KD], k4n[4][KD], vreg[VPT];
-        auto load64 = [&](int n0, u32x4 (&kk)[4][KD]) {
+        constexpr int VPT = 64 * (D / 8) / 256;     // 16-byte V chunks per thread and tile
+        static_assert(64 * (D / 8) == VPT * 256, "every thread stages the same number of V chunks");
+        struct Tile { u32x4 k[4][KD]; u32x4 v[VPT]; };
+        auto fetch = [&](int n0, Tile& t) {
 #pragma unroll
             for (int sb = 0; sb < 4; ++sb) {
                 const int n = min(n0 + sb * 16 + c16, N - 1);
 #pragma unroll
-                for (int kd = 0; kd < KD; ++kd) kk[sb][kd] = *reinterpret_cast<const u32x4*>(k + (int64_t)n * a.ks[2] + kd * 32 + g * 8);
+                for (int kd = 0; kd < KD; ++kd) t.k[sb][kd] = *reinterpret_cast<const u32x4*>(k + (int64_t)n * a.ks[2] + kd * 32 + g * 8);
             }
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
                 const int c = tid + i * 256, tok = c / (D / 8), ch = c % (D / 8);
-                if (c < 64 * (D / 8)) vreg[i] = *reinterpret_cast<const u32x4*>(v + (int64_t)min(n0 + tok, N - 1) * a.vs[2] + ch * 8);
+                t.v[i] = *reinterpret_cast<const u32x4*>(v + (int64_t)min(n0 + tok, N - 1) * a.vs[2] + ch * 8);
             }
         };
-        auto store64 = [&](int buf) {
+        // V rows of absent tokens are staged as zeros (their probabilities then add nothing to the numerators)
+        auto stage = [&](int n0, int buf, const Tile& t) {
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
                 const int c = tid + i * 256, tok = c / (D / 8), ch = c % (D / 8);
-                if (c < 64 * (D / 8)) {
-                    u32x4 o = vreg[i];
-                    if constexpr (!std::is_same<T, bf16_t>::value) {
+                u32x4 o = t.v[i];
+                if constexpr (!std::is_same<T, bf16_t>::value) {
 #pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            o[j] = P_::pack2(M_::unpack(uint16_t(vreg[i][j] & 0xffffu)), M_::unpack(uint16_t(vreg[i][j] >> 16)));
-                    }
-                    *reinterpret_cast<u32x4*>(&v64[buf][tok][ch * 8]) = o;
+                    for (int j = 0; j < 4; ++j)
+                        o[j] = P_::pack2(M_::unpack(uint16_t(t.v[i][j] & 0xffffu)), M_::unpack(uint16_t(t.v[i][j] >> 16)));
                 }
+                if (n0 + tok >= N) o = u32x4{0u, 0u, 0u, 0u};
+                *reinterpret_cast<u32x4*>(&v64[buf][tok][ch * 8]) = o;
             }
         };
-        load64(n_lo, k4);
-        store64(0);
-        if (n_lo + 64 < N) load64(n_lo + 64, k4n);
-        __syncthreads();
-        int it = 0;
-        for (int n0 = n_lo; n0 < N; n0 += 64, ++it) {
-            const int buf = it & 1;
+        // the tile's contribution; the denominators count live tokens only (the A operand of their product
+        // holds ones in the k-slots of live tokens)
+        auto work = [&](int n0, int buf, const Tile& t) {
 #pragma unroll
             for (int sb = 0; sb < 4; ++sb) {
-                const int tb = N - (n0 + sb * 16);   // rows >= tb are beyond the segment
+                const int tb = N - (n0 + sb * 16);   // tokens >= tb of this block are beyond the segment
+                uint2 live4 = ones4;
+                if (tb < 16) {
+                    const uint32_t one = P_::kOnes2 & 0xffffu;
+                    live4 = make_uint2((4 * g + 0 < tb ? one : 0u) | (4 * g + 1 < tb ? one << 16 : 0u),
+                                       (4 * g + 2 < tb ? one : 0u) | (4 * g + 3 < tb ? one << 16 : 0u));
+                }
                 uint2 vop[DT];
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) vop[dt] = tr16(&v64[buf][sb * 16 + 4 * g + (c16 >> 2)][dt * 16 + (c16 & 3) * 4]);
@@ -292,25 +301,39 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
                 for (int ct = 0; ct < CT; ++ct) {
                     f32x4 s = negmu[ct];
 #pragma unroll
-                    for (int kd = 0; kd < KD; ++kd) s = M_::mma32(k4[sb][kd], qb[ct][kd], s);
-                    float p[4];
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) p[r] = (4 * g + r < tb) ? fast_exp2(s[r]) : 0.f;
-                    const uint2 ppk = make_uint2(P_::pack2(p[0], p[1]), P_::pack2(p[2], p[3]));
-                    den[ct] = P_::mma16(ones4, ppk, den[ct]);
+                    for (int kd = 0; kd < KD; ++kd) s = M_::mma32(t.k[sb][kd], qb[ct][kd], s);
+                    const uint2 ppk = make_uint2(P_::pack2(fast_exp2(s[0]), fast_exp2(s[1])), P_::pack2(fast_exp2(s[2]), fast_exp2(s[3])));
+                    den[ct] = P_::mma16(live4, ppk, den[ct]);
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) U[ct][dt] = P_::mma16(ppk, vop[dt], U[ct][dt]);
                 }
             }
-            if (n0 + 64 < N) {
-#pragma unroll
-                for (int sb = 0; sb < 4; ++sb)
-#pragma unroll
-                    for (int kd = 0; kd < KD; ++kd) k4[sb][kd] = k4n[sb][kd];
-                store64(buf ^ 1);
-                if (n0 + 128 < N) load64(n0 + 128, k4n);
-            }
+        };
+        Tile ta, tb_, tc;
+        fetch(n_lo, ta);
+        fetch(n_lo + 64, tb_);
+        fetch(n_lo + 128, tc);
+        stage(n_lo, 0, ta);
+        __syncthreads();
+        int buf = 0;
+        for (int n0 = n_lo;; n0 += 192) {
+            // tile n0 (K in ta, V staged in v64[buf]); the next tile's V goes into the other buffer meanwhile
+            work(n0, buf, ta);
+            fetch(n0 + 192, ta);
+            if (n0 + 64 >= N) break;
+            stage(n0 + 64, buf ^ 1, tb_);
             __syncthreads();
+            work(n0 + 64, buf ^ 1, tb_);
+            fetch(n0 + 256, tb_);
+            if (n0 + 128 >= N) break;
+            stage(n0 + 128, buf, tc);
+            __syncthreads();
+            work(n0 + 128, buf, tc);
+            fetch(n0 + 320, tc);
+            if (n0 + 192 >= N) break;
+            stage(n0 + 192, buf ^ 1, ta);
+            __syncthreads();
+            buf ^= 1;
         }
         // local state of the segment, relative to the shift of the incoming state; whatever
         // overflowed or vanished here is caught by the checks of the segments that use it
@@ -845,37 +868,11 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     }
 }
 
-// Clears the per-(b,h) redo flags (a kernel rather than a memset so that callers may capture
-// the call in a graph).
-__global__ void causal_clear_flags_kernel(int* flags, int n)
-{
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) flags[i] = 0;
-}
-
-// Copies the state staged by the last segment into (mu, den, num) for every (b,h) whose
-// segments all passed validation; a fresh state's shift becomes 0.
-__global__ __launch_bounds__(256) void causal_commit_kernel(CausalArgs a)
-{
-    const int bh = blockIdx.x;
-    if (a.flags[bh] != 0) return;
-    const int M = a.M, D = a.D;
-    const float* sd = a.seg_den + ((int64_t)bh * a.n_segs + a.n_segs - 1) * M;
-    const float* sn = a.seg_num + ((int64_t)bh * a.n_segs + a.n_segs - 1) * M * D;
-    for (int i = threadIdx.x; i < M; i += 256) {
-        const float mu = a.mu[(int64_t)bh * M + i];
-        a.mu[(int64_t)bh * M + i] = mu <= kNegBig ? 0.f : mu;
-        a.den[(int64_t)bh * M + i] = sd[i];
-    }
-    for (int i = threadIdx.x; i < M * D; i += 256) a.num[(int64_t)bh * M * D + i] = sn[i];
-}
-
 template <typename T, bool STATE_ONLY>
 hipError_t launch_phase(const CausalArgs& a, int step, dim3 grid, hipStream_t st)
 {
     dim3 block(256);
     if (a.D == 64 && a.M == 128)      hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 1, STATE_ONLY>), grid, block, 0, st, a, step);
-    else if (a.D == 64 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 64, 2, STATE_ONLY>), grid, block, 0, st, a, step);
     else if (a.D == 32 && a.M == 128) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 1, STATE_ONLY>), grid, block, 0, st, a, step);
     else if (a.D == 32 && a.M == 256) hipLaunchKernelGGL((causal_mfma_kernel<T, 32, 2, STATE_ONLY>), grid, block, 0, st, a, step);
     else return hipErrorInvalidValue;
@@ -906,13 +903,12 @@ hipError_t launch_t(const CausalArgs& a, int step, hipStream_t st)
 {
     const int BH = a.B * a.H;
     if (a.n_segs == 1) return launch_recurrence<T>(a, step, dim3(BH, 1), st);
-    hipLaunchKernelGGL(causal_clear_flags_kernel, dim3((BH + 255) / 256), dim3(256), 0, st, a.flags, BH);
+    // the first phase also clears the redo flags and segment counters
     hipError_t e = launch_phase<T, true>(a, step, dim3(BH, a.n_segs - 1), st);
     if (e != hipSuccess) return e;
-    e = launch_recurrence<T>(a, step, dim3(BH, a.n_segs), st);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(causal_commit_kernel, dim3(BH), dim3(256), 0, st, a);
-    return hipGetLastError();
+    // The last segment has staged the final state in the workspace; the fp32 kernel launched behind this one copies
+    // it into (mu, den, num) for every (b,h) whose flag stayed clear and redoes the others from their incoming state.
+    return launch_recurrence<T>(a, step, dim3(BH, a.n_segs), st);
 }
 
 }  // namespace
