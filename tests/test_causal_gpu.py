@@ -254,19 +254,22 @@ def test_decode_kernel_shapes(dev, M, D, dtype):
     state_close(st, str_, TOL[dtype])
 
 
-def test_cfg4_full_size_properties(dev):
-    """BASELINE config 4 at its full size (B=8, H=16, D=64, M=128, bf16; 8192 prefill tokens in chunks of 256, then 256
+@pytest.mark.parametrize("chunk", [256, 0])
+def test_cfg4_full_size_properties(dev, chunk):
+    """BASELINE config 4 at its full size (B=8, H=16, D=64, M=128, bf16; 8192 prefill tokens in chunks of 256 as the
+    config words it, and in the segments the library chooses itself (chunk=0: what bench.py times), then 256
     decode steps), through properties that need no full-size CPU run: decode after prefill = one longer prefill;
     the final state = the non-causal gather over all tokens; the last output row = the non-causal mixer's;
     and one (b, h) pair against the fp64 token recurrence over the whole length."""
     B, H, D, M, NP, ND = 8, 16, 64, 128, 8192, 256
     q, k, v = make(B, H, NP + ND, M, D, torch.bfloat16, seed=4)
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
-    y1, st = F.flare_causal_prefill(qd, kd[:, :, :NP], vd[:, :, :NP], chunk=256)
+    y1, st = F.flare_causal_prefill(qd, kd[:, :, :NP], vd[:, :, :NP], chunk=chunk)
     y2, st = F.flare_causal_decode(qd, kd[:, :, NP:], vd[:, :, NP:], st)
-    yl, stl = F.flare_causal_prefill(qd, kd, vd, chunk=256)
+    yl, stl = F.flare_causal_prefill(qd, kd, vd, chunk=chunk)
     assert torch.isfinite(y1).all() and torch.isfinite(y2).all()
-    assert O.rel_l2(y1, yl[:, :, :NP]) <= 1e-6                    # same kernel, same chunks
+    # chunks of 256: same kernel, same segment boundaries; the library's own plan cuts the longer call elsewhere
+    assert O.rel_l2(y1, yl[:, :, :NP]) <= (1e-6 if chunk else 2e-2)
     assert O.rel_l2(y2, yl[:, :, NP:]) <= 2e-2
     z, lse = O.causal_state_invariants(*(t.double() for t in st))
     zl, lsel = O.causal_state_invariants(*(t.double() for t in stl))
