@@ -418,7 +418,7 @@ int flare_scatter_fwd_lse(const FlareMixerDesc* desc, const void* q, const void*
 }
 
 namespace {
-struct BwdPlan { int n_splits, tokens_per_split; size_t off_dz, off_dl, off_part, total; };
+struct BwdPlan { int n_splits, tokens_per_split; size_t off_dz, off_dl, off_rm, off_part, total; };
 
 BwdPlan plan_bwd(const FlareMixerDesc* d)
 {
@@ -434,7 +434,8 @@ BwdPlan plan_bwd(const FlareMixerDesc* d)
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     p.off_dz = up((size_t)bh * d->N * 4);
     p.off_dl = p.off_dz + up((size_t)bh * d->M * d->D * 4);
-    p.off_part = p.off_dl + up((size_t)bh * d->M * 4);
+    p.off_rm = p.off_dl + up((size_t)bh * d->M * 4);
+    p.off_part = p.off_rm + up((size_t)bh * p.n_splits * 4);
     p.total = p.off_part + (size_t)bh * p.n_splits * d->M * d->D * 4;
     return p;
 }
@@ -485,6 +486,7 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
     a.delta_tok = reinterpret_cast<float*>(ws);
     a.dz = reinterpret_cast<float*>(ws + p.off_dz);
     a.delta_lat = reinterpret_cast<float*>(ws + p.off_dl);
+    a.rho_min = reinterpret_cast<float*>(ws + p.off_rm);
     a.part = reinterpret_cast<float*>(ws + p.off_part);
     a.dq = dq; a.dk = dk; a.dv = dv;
     a.B = desc->B; a.H = desc->H; a.N = desc->N; a.M = desc->M; a.D = desc->D;

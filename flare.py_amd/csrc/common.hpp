@@ -147,6 +147,7 @@ struct MixerBwdArgs {
     float* dz;               // [B,H,M,D] gradient of z             (workspace)
     float* delta_lat;        // [B,H,M]   <dz_m, z_m>               (workspace)
     float* part;             // [B,H,P,M,D] split-N partial sums    (workspace)
+    float* rho_min;          // [B,H,P]   smallest token log-sum-exp of each split, log2 units   (workspace)
     float* dq;               // [B,H,M,D] fp32
     void* dk; void* dv;      // [B,H,N,D] element type
     int B, H, N, M, D;
@@ -154,6 +155,7 @@ struct MixerBwdArgs {
     float scale, scale_log2;
     int64_t qs[3], ks[3], vs[3], ys[3], dys[3], dks[3], dvs[3];
     int m0, mc, accumulate;  // token-side kernel only: latents [m0, m0 + mc) of the M (mc = 0: all), added to dk, dv when accumulate
+    int scal_lds;            // token-side kernel only: per-latent scalars are tabled in LDS behind the operand sets
 };
 
 struct CausalLinearArgs {

@@ -21,6 +21,17 @@
 // is assembled in registers and, packed to bf16, is the B operand of the last product.
 // q and k meet in the element type; every other product runs in bf16 (f16 tiles are converted while
 // they are staged), because dz, Delta and dS have no useful bound in f16.
+//
+// One exponential per score instead of two.  Both weights come from the same score, so
+//   Bt[n,m] = A[m,n] * eL[m] * eR[n],   eL[m] = exp2(L2_m - Lmax2) <= 1,   eR[n] = exp2(Lmax2 - rho2_n)
+// (log2 units, Lmax2 = the largest L2_m of the (b,h)).  The kernels that need both weights fold eR into the rows of
+// dy and into delta_n when they load a token tile, and eL into a per-latent factor, and evaluate
+//   dS = A * (<dz_m,v_n> - Delta_m + eL[m] * (<z_m, eR dy_n> - eR delta_n)).
+// That is exact unless A underflows where Bt still matters or eR overflows, which needs log-sum-exps more than
+// kFactorSpan apart: the dz pass records the smallest rho2_n of every split, and a (b,h) whose Lmax2 exceeds the
+// smallest rho2_n by more than kFactorSpan takes the two-exponential form for all its tiles.
+// (Padded tokens and empty batch elements carry log-sum-exps of 1e30: the former are ignored by the minimum and
+// get eR = 0, the latter send their (b,h) to the two-exponential form.)
 #include <type_traits>
 
 #include "common.hpp"
@@ -96,6 +107,36 @@ __device__ __forceinline__ u32x4 pack8(const float (&v)[8])
 {
     return u32x4{Pb::pack2(v[0], v[1]), Pb::pack2(v[2], v[3]), Pb::pack2(v[4], v[5]), Pb::pack2(v[6], v[7])};
 }
+// 8 consecutive fp32 values times f as packed bf16
+__device__ __forceinline__ u32x4 pack8(const float* p, float f)
+{
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p) * f, b = *reinterpret_cast<const f32x4*>(p + 4) * f;
+    return u32x4{Pb::pack2(a[0], a[1]), Pb::pack2(a[2], a[3]), Pb::pack2(b[0], b[1]), Pb::pack2(b[2], b[3])};
+}
+
+// Largest distance (log2 units) between the latents' largest log-sum-exp and a token's for which the token
+// scatter's weights are formed from the gather's (see the head of this file): exp2(64) and the 2^-62 that is
+// left of a weight whose partner underflowed are both far inside what fp32 and bf16 hold.
+constexpr float kFactorSpan = 64.f;
+
+__device__ __forceinline__ float wave_max(float x)
+{
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) x = fmaxf(x, __shfl_xor(x, o));
+    return x;
+}
+
+// Whether the (b,h) may use the one-exponential form, and its Lmax2.  Every wave computes the same answer.
+__device__ __forceinline__ bool factor_plan(const MixerBwdArgs& a, int64_t bh, int lane, float& lmax2)
+{
+    float lm = -3.0e38f, rm = -3.0e38f;
+    for (int m = lane; m < a.M; m += 64) lm = fmaxf(lm, a.lse_lat[bh * a.M + m]);
+    for (int p = lane; p < a.n_splits; p += 64) rm = fmaxf(rm, -a.rho_min[bh * a.n_splits + p]);
+    lmax2 = wave_max(lm) * kLog2e;
+    // An empty batch element (its latents carry 1e30) takes the other form: differences of such magnitudes are
+    // rounding noise far above the range of exp2.
+    return lmax2 <= 1.0e6f && lmax2 + wave_max(rm) <= kFactorSpan;
+}
 
 __device__ __forceinline__ uint2 lds_read_tr16(const void* lds_addr)
 {
@@ -151,8 +192,13 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
     // reads the rows of y next to those of dy, which it stages anyway.
     const bool make_delta = MODE == 0 && mb == 0;
 
+    // the dq pass forms the token scatter's weights from the gather's where the (b,h) allows it
+    float lmax2 = 0.f;
+    const bool fast = MODE == 1 && factor_plan(a, bh, lane, lmax2);
+
     // latent operands (B of the score-like products) and per-latent scalars
     u32x4 qb[CT][KD], dzb[CT][KD], zb[CT][KD];
+    float nel[CT];                                  // -eL[m] of the lane's latent (one-exponential form)
     // The additive terms of the score-like products (-L_m, -rho_n, -Delta_m, -delta_n) are not
     // subtracted element by element: they are the initial accumulator of the matrix product.  A
     // per-token term is a row vector of the tile (free); a per-latent term needs four registers
@@ -164,6 +210,9 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
     for (int ct = 0; ct < CT; ++ct) {
         const int m = m_base + ct * 16 + c16;
         const bool own = m_base + ct * 16 < a.M;       // uniform over the wave
+        // eL[m]: the rows of z carry it in the one-exponential form (1 otherwise)
+        const float el = (MODE == 1 && fast && own) ? fast_exp2(a.lse_lat[bh * a.M + m] * kLog2e - lmax2) : 1.f;
+        nel[ct] = -el;
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd) {
             const int ch = kd * 4 + g;
@@ -171,7 +220,7 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
             qb[ct][kd] = in ? scale8<T>(load16(q + (int64_t)m * a.qs[2] + ch * 8), a.scale_log2) : zero4();
             if (MODE == 1) {
                 dzb[ct][kd] = in ? pack8(a.dz + (bh * a.M + m) * D + ch * 8) : zero4();
-                zb[ct][kd] = in ? pack8(a.z + (bh * a.M + m) * D + ch * 8) : zero4();
+                zb[ct][kd] = in ? pack8(a.z + (bh * a.M + m) * D + ch * 8, el) : zero4();
             }
         }
         if (MODE == 1) {
@@ -193,20 +242,25 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
     auto v_slot = [](int tok, int ch) { return tok * ROWB + ((CH >= 4 ? (ch ^ (((tok >> 2) & 1) << 1)) : ch) << 4); };
 
     u32x4 kr[CPT], vr[CPT], yr[CPT];
+    float ysc[CPT];    // eR of the token a staged dy chunk belongs to (one-exponential form)
     float rr = 0.f, dd = 0.f;
+    float rr_max = -3.0e38f;   // MODE 0: -(smallest rho2_n) over the tokens this thread has loaded
     int ln0 = 0;       // first token of the tile held in kr/vr/yr
     auto load_tile = [&](int n0) {
         ln0 = n0;
         if (tid < kBTile) {
             const int n = min(n0 + tid, n_end - 1);
             rr = -rho[n] * kLog2e;          // negated: they start the accumulators of the products below
-            if (MODE == 1) dd = -dlt[n];
+            if (MODE == 0) rr_max = fmaxf(rr_max, rr);
+            if (MODE == 1) dd = fast ? dlt[n] * fast_exp2(lmax2 + rr) : -dlt[n];     // eR delta_n | -delta_n
         }
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * 256;
+            ysc[i] = 1.f;
             if (c < TCH) {
                 const int n = min(n0 + c / CH, n_end - 1), ch = c % CH;
+                if (MODE == 1 && fast) ysc[i] = fast_exp2(lmax2 - rho[n] * kLog2e);
                 kr[i] = load16(k + (int64_t)n * a.ks[2] + ch * 8);
                 yr[i] = load16(dy + (int64_t)n * a.dys[2] + ch * 8);
                 if (MODE == 1) vr[i] = load16(v + (int64_t)n * a.vs[2] + ch * 8);
@@ -236,7 +290,7 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
                 } else {
                     *reinterpret_cast<u32x4*>(&tl[buf][1][v_slot(tok, ch)]) = to_bf16x8<T>(kr[i]);
                     *reinterpret_cast<u32x4*>(&tl[buf][2][k_slot(tok, ch)]) = to_bf16x8<T>(vr[i]);
-                    *reinterpret_cast<u32x4*>(&tl[buf][3][k_slot(tok, ch)]) = to_bf16x8<T>(yr[i]);
+                    *reinterpret_cast<u32x4*>(&tl[buf][3][k_slot(tok, ch)]) = to_bf16x8<T>(yr[i], ysc[i]);
                 }
             }
         }
@@ -249,7 +303,8 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
         for (int rt = 0; rt < RT; ++rt) acc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
     const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
 
-    auto process = [&](int n0, int buf) {
+    auto process = [&](auto fast_c, int n0, int buf) {
+        constexpr bool FAST = decltype(fast_c)::value;      // one-exponential form (dq pass only)
         const bool full = n0 + kBTile <= n_end;
 #pragma unroll
         for (int ks = 0; ks < kBTile / 32; ++ks) {
@@ -285,6 +340,45 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
             }
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
+                float o[8];
+                if constexpr (FAST) {
+                    // A = exp2(S - L_m);  g = <dz_m,v_n> - Delta_m + <eL z_m, eR dy_n>;  dS = A (g - eL[m] eR delta_n)
+                    f32x4 a0 = kFoldLat ? nl4[kFoldLat ? ct : 0] : zf, a1 = a0;
+                    f32x4 g0 = kFoldLat ? nd4[kFoldLat ? ct : 0] : zf, g1 = g0;
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) {
+                        a0 = M_::mma(ka0[kd], qb[ct][kd], a0);
+                        a1 = M_::mma(ka1[kd], qb[ct][kd], a1);
+                        g0 = Pb::mma(va0[kd], dzb[ct][kd], g0);
+                        g1 = Pb::mma(va1[kd], dzb[ct][kd], g1);
+                    }
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) {
+                        g0 = Pb::mma(ya0[kd], zb[ct][kd], g0);
+                        g1 = Pb::mma(ya1[kd], zb[ct][kd], g1);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if constexpr (kFoldLat) {
+                            o[e] = fast_exp2(a0[e]) * fmaf(nel[ct], da[e], g0[e]);
+                            o[e + 4] = fast_exp2(a1[e]) * fmaf(nel[ct], db[e], g1[e]);
+                        } else {
+                            o[e] = fast_exp2(a0[e] - l2m[ct]) * (fmaf(nel[ct], da[e], g0[e]) - dm[ct]);
+                            o[e + 4] = fast_exp2(a1[e] - l2m[ct]) * (fmaf(nel[ct], db[e], g1[e]) - dm[ct]);
+                        }
+                    }
+                    if (!full) {       // rows past the end of the token range (clamped copies of the last token)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (n0 + tb + e >= n_end) o[e] = 0.f;
+                            if (n0 + tb + 16 + e >= n_end) o[e + 4] = 0.f;
+                        }
+                    }
+                    const u32x4 obf = pack8(o);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) acc[rt][ct] = Pb::mma(tr[rt], obf, acc[rt][ct]);
+                    continue;
+                }
                 // S - rho_n: the token scatter's exponent
                 constexpr bool kFoldTok = MODE == 0 || kFoldLat;
                 f32x4 b0 = kFoldTok ? ra : zf, b1 = kFoldTok ? rb : zf;
@@ -293,7 +387,6 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
                     b0 = M_::mma(ka0[kd], qb[ct][kd], b0);
                     b1 = M_::mma(ka1[kd], qb[ct][kd], b1);
                 }
-                float o[8];
                 if (MODE == 0) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -345,13 +438,27 @@ __global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
         store_tile(0);
     }
     __syncthreads();
-    int buf = 0;
-    for (int n0 = n_begin; n0 < n_end; n0 += kBTile, buf ^= 1) {
-        const bool more = n0 + kBTile < n_end;
-        if (more) load_tile(n0 + kBTile);
-        process(n0, buf);
-        if (more) store_tile(buf ^ 1);
-        __syncthreads();
+    auto walk = [&](auto fast_c) {
+        int buf = 0;
+        for (int n0 = n_begin; n0 < n_end; n0 += kBTile, buf ^= 1) {
+            const bool more = n0 + kBTile < n_end;
+            if (more) load_tile(n0 + kBTile);
+            process(fast_c, n0, buf);
+            if (more) store_tile(buf ^ 1);
+            __syncthreads();
+        }
+    };
+    if constexpr (MODE == 1) {
+        if (fast) walk(std::true_type{});
+        else walk(std::false_type{});
+    } else {
+        walk(std::false_type{});
+    }
+
+    if (make_delta) {
+        // the smallest token log-sum-exp of this split (log2 units), for the passes that follow
+        const float rm = wave_max(rr_max);      // wave 0 = the threads that read the tokens' scalars
+        if (tid == 0) a.rho_min[bh * a.n_splits + split] = -rm;
     }
 
 #pragma unroll
@@ -418,8 +525,10 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
     u32x4* zza = dza + (size_t)M * CH;
     u32x4* dzt = zza + (size_t)M * CH;
     u32x4* qt = dzt + (size_t)M * CH;
-    // the per-latent scalars (log-sum-exp, Delta) stay in global memory: the five operand sets may then take all
-    // 160 KB of LDS (M = 256 at D = 64, M = 512 at D = 32)
+    // The per-latent scalars (-L2_m, -Delta_m, -eL[m]) sit behind the operand sets when the LDS has room for them
+    // (a.scal_lds); when the five operand sets take all 160 KB (M = 256 at D = 64, M = 512 at D = 32) they are read
+    // from global memory at every latent step.
+    float* sc_l = reinterpret_cast<float*>(qt + (size_t)M * CH);     // [3][M] when a.scal_lds
     const float* lse_lat = a.lse_lat + ((int64_t)blockIdx.z * a.H + blockIdx.y) * a.M + a.m0;
     const float* delta_lat = a.delta_lat + ((int64_t)blockIdx.z * a.H + blockIdx.y) * a.M + a.m0;
 
@@ -437,12 +546,23 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
     const float* rho = a.lse_tok + bh * a.N;
     const float* dlt = a.delta_tok + bh * a.N;
 
+    float lmax2 = 0.f;
+    const bool fast = factor_plan(a, (int64_t)blockIdx.z * a.H + blockIdx.y, threadIdx.x & 63, lmax2);
+    if (a.scal_lds) {
+        for (int m = threadIdx.x; m < M; m += NTH) {
+            const float l2 = lse_lat[m] * kLog2e;
+            sc_l[m] = -l2;
+            sc_l[M + m] = -delta_lat[m];
+            sc_l[2 * M + m] = -fast_exp2(l2 - lmax2);
+        }
+    }
     for (int idx = tid; idx < M * CH; idx += NTH) {
         const int m = idx / CH, ch = idx % CH;
         const int slot = ((m >> 4) * CH + ch) * 16 + (m & 15);
         qa[slot] = scale8<T>(load16(q + (int64_t)m * a.qs[2] + ch * 8), a.scale_log2);
         dza[slot] = pack8(dz + (int64_t)m * D + ch * 8);
-        zza[slot] = pack8(z + (int64_t)m * D + ch * 8);
+        // the rows of z carry eL[m] in the one-exponential form
+        zza[slot] = pack8(z + (int64_t)m * D + ch * 8, fast ? fast_exp2(lse_lat[m] * kLog2e - lmax2) : 1.f);
     }
     for (int idx = tid; idx < KS * RT * 64; idx += NTH) {
         const int ln = idx & 63, rt = (idx >> 6) % RT, ks = idx / (64 * RT);
@@ -465,24 +585,29 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
     const int wg_n1 = min(a.N, wg_n0 + tokens_per_wg);
     const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
 
+    // FAST = the one-exponential form (head of this file): the rows of dy and delta_n carry eR[n], the element-wise
+    // part applies eL[m]; otherwise both exponentials are taken.
+    auto walk = [&](auto fast_c, const float lmax2) {
+    constexpr bool FAST = decltype(fast_c)::value;
     for (int t0 = wg_n0 + w * 16 * kBTW; t0 < wg_n1; t0 += kTokWaves * 16 * kBTW) {
         u32x4 kb[kBTW][KD], vb[kBTW][KD], yb[kBTW][KD];
-        float r2[kBTW], de[kBTW];
+        float r2[kBTW], de[kBTW];      // FAST: r2 is unused, de = eR delta_n
 #pragma unroll
         for (int tw = 0; tw < kBTW; ++tw) {
             const int n = t0 + tw * 16 + c16;
             const bool live = n < wg_n1;
             const int nc = live ? n : wg_n1 - 1;
+            r2[tw] = rho[nc] * kLog2e;
+            const float er = FAST ? fast_exp2(lmax2 - r2[tw]) : 1.f;
+            de[tw] = dlt[nc] * er;
 #pragma unroll
             for (int kd = 0; kd < KD; ++kd) {
                 const int ch = kd * 4 + g;
                 const bool in = live && ch < CH;
                 kb[tw][kd] = in ? load16(k + (int64_t)n * a.ks[2] + ch * 8) : zero4();
                 vb[tw][kd] = in ? to_bf16x8<T>(load16(v + (int64_t)n * a.vs[2] + ch * 8)) : zero4();
-                yb[tw][kd] = in ? to_bf16x8<T>(load16(dy + (int64_t)n * a.dys[2] + ch * 8)) : zero4();
+                yb[tw][kd] = in ? to_bf16x8<T>(load16(dy + (int64_t)n * a.dys[2] + ch * 8), er) : zero4();
             }
-            r2[tw] = rho[nc] * kLog2e;
-            de[tw] = dlt[nc];
         }
         f32x4 adk[kBTW][RT], adv[kBTW][RT];
 #pragma unroll
@@ -510,10 +635,83 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
             }
             // negated per-latent scalars of the 8 latents (rows) this lane holds: -L_m log2(e) and -Delta_m
             // start the accumulators of S and <dz, v>, so neither is subtracted element by element
-            const f32x4 la = *reinterpret_cast<const f32x4*>(lse_lat + 32 * ks + 4 * g) * -kLog2e;
-            const f32x4 lb = *reinterpret_cast<const f32x4*>(lse_lat + 32 * ks + 16 + 4 * g) * -kLog2e;
-            const f32x4 da = -*reinterpret_cast<const f32x4*>(delta_lat + 32 * ks + 4 * g);
-            const f32x4 db = -*reinterpret_cast<const f32x4*>(delta_lat + 32 * ks + 16 + 4 * g);
+            f32x4 la, lb, da, db, nea = zf, neb = zf;      // -L2_m, -Delta_m, -eL[m] of the 8 latents (rows) this lane holds
+            if (a.scal_lds) {
+                const float* t = sc_l + 32 * ks + 4 * g;
+                la = *reinterpret_cast<const f32x4*>(t);            lb = *reinterpret_cast<const f32x4*>(t + 16);
+                da = *reinterpret_cast<const f32x4*>(t + M);        db = *reinterpret_cast<const f32x4*>(t + M + 16);
+                if (FAST) {
+                    nea = *reinterpret_cast<const f32x4*>(t + 2 * M);
+                    neb = *reinterpret_cast<const f32x4*>(t + 2 * M + 16);
+                }
+            } else {
+                la = *reinterpret_cast<const f32x4*>(lse_lat + 32 * ks + 4 * g) * -kLog2e;
+                lb = *reinterpret_cast<const f32x4*>(lse_lat + 32 * ks + 16 + 4 * g) * -kLog2e;
+                da = -*reinterpret_cast<const f32x4*>(delta_lat + 32 * ks + 4 * g);
+                db = -*reinterpret_cast<const f32x4*>(delta_lat + 32 * ks + 16 + 4 * g);
+                if (FAST) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        nea[e] = -fast_exp2(-la[e] - lmax2);
+                        neb[e] = -fast_exp2(-lb[e] - lmax2);
+                    }
+                }
+            }
+            if constexpr (FAST) {
+                // The rows of z carry eL[m] (staged that way when the (b,h) takes this form), so
+                //   g = <dz_m,v_n> - Delta_m + <eL z_m, eR dy_n>   is one accumulator chain,   dS = A (g - eL[m] eR delta_n).
+                // Software pipeline over the wave's tiles: the score-like products of tile tw + 1 and the gradient
+                // products of tile tw - 1 are issued ahead of the exponentials of tile tw, which run under them.
+                auto front = [&](int tw, f32x4& a0, f32x4& a1, f32x4& g0, f32x4& g1) {
+                    a0 = la; a1 = lb; g0 = da; g1 = db;
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) {
+                        a0 = M_::mma(q0[kd], kb[tw][kd], a0);
+                        a1 = M_::mma(q1[kd], kb[tw][kd], a1);
+                        g0 = Pb::mma(d0[kd], vb[tw][kd], g0);
+                        g1 = Pb::mma(d1[kd], vb[tw][kd], g1);
+                    }
+#pragma unroll
+                    for (int kd = 0; kd < KD; ++kd) {
+                        g0 = Pb::mma(z0[kd], yb[tw][kd], g0);
+                        g1 = Pb::mma(z1[kd], yb[tw][kd], g1);
+                    }
+                };
+                auto back = [&](int tw, u32x4 pa, u32x4 pd) {
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) {
+                        adv[tw][rt] = Pb::mma(odz[rt], pa, adv[tw][rt]);
+                        adk[tw][rt] = Pb::mma(oq[rt], pd, adk[tw][rt]);
+                    }
+                };
+                f32x4 a0, a1, g0, g1;
+                front(0, a0, a1, g0, g1);
+                u32x4 pap = zero4(), pdp = zero4();
+#pragma unroll
+                for (int tw = 0; tw < kBTW; ++tw) {
+                    __builtin_amdgcn_s_setprio(1);      // matrix-product issue goes first, the other waves' vector work fills in behind
+                    f32x4 na0 = zf, na1 = zf, ng0 = zf, ng1 = zf;
+                    if (tw + 1 < kBTW) front(tw + 1, na0, na1, ng0, ng1);
+                    if (tw > 0) back(tw - 1, pap, pdp);
+                    __builtin_amdgcn_sched_barrier(0);
+                    __builtin_amdgcn_s_setprio(0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    float av[8], ds[8];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        av[e] = fast_exp2(a0[e]);
+                        av[e + 4] = fast_exp2(a1[e]);
+                        ds[e] = av[e] * fmaf(nea[e], de[tw], g0[e]);
+                        ds[e + 4] = av[e + 4] * fmaf(neb[e], de[tw], g1[e]);
+                    }
+                    pap = pack8(av);
+                    pdp = pack8(ds);
+                    a0 = na0; a1 = na1; g0 = ng0; g1 = ng1;
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                back(kBTW - 1, pap, pdp);
+                continue;
+            }
 #pragma unroll
             for (int tw = 0; tw < kBTW; ++tw) {
                 f32x4 a0 = la, a1 = lb, s0 = zf, s1 = zf, g10 = da, g11 = db, g20 = zf, g21 = zf;
@@ -580,6 +778,9 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
             put(dv, a.dvs[2], adv[tw]);
         }
     }
+    };
+    if (fast) walk(std::true_type{}, lmax2);
+    else walk(std::false_type{}, 0.f);
 }
 
 template <typename T, int D, int MODE>
@@ -609,7 +810,9 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
         const int chunks = mixer_bwd_tok_chunks(a.M, D);
         if (chunks == 0) return hipErrorInvalidValue;
         const int mc = a.M / chunks;
-        const size_t lds = mixer_bwd_lds_bytes(mc, D);
+        // per-latent scalar tables behind the operand sets where the LDS has room
+        const bool scal_lds = mixer_bwd_lds_bytes(mc, D) + (size_t)3 * mc * sizeof(float) <= 160 * 1024;
+        const size_t lds = mixer_bwd_lds_bytes(mc, D) + (scal_lds ? (size_t)3 * mc * sizeof(float) : 0);
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         // one workgroup per compute unit, ranges a multiple of its 512-token pass
@@ -621,6 +824,7 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
             ac.m0 = c * mc;
             ac.mc = mc;
             ac.accumulate = c > 0;
+            ac.scal_lds = scal_lds ? 1 : 0;
             hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(64 * kTokWaves), lds, st, ac, (int)tpw);
         }
     }
