@@ -95,6 +95,33 @@ def test_lse_outputs(dev):
     assert float((lt - lse_tok).abs().max()) <= 2e-2
 
 
+@pytest.mark.parametrize("a", [3.0, 5.0, 6.75])
+def test_backward_with_log_sum_exps_far_apart(dev, a):
+    """The kernels form the token scatter's weights from the gather's (one exponential per score) only while the
+    latents' largest log-sum-exp and the tokens' smallest are at most 2^64 apart, and take both exponentials
+    otherwise.  Half of the tokens score +a^2 with every latent, the other half -a^2: a = 3 stays inside that span,
+    a = 5 leaves it, and at a = 6.75 the gather's weights of the second half underflow in fp32 while their own
+    softmax over the latents still decides their gradients."""
+    B, H, N, M, D = 1, 2, 600, 64, 32
+    q, k, v, gy = make(B, H, N, M, D, torch.bfloat16, seed=31)
+    q[..., 0] = a
+    k[..., 0] = a
+    k[:, :, ::2, 0] = -a
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    assert FN._hip_backward_ok(qd, kd, vd, None, False)
+    F.flare_multihead_mixer(qd, kd, vd).backward(gy.to(dev))
+    gq, gk, gv = oracle_grads(q, k, v, gy, 1.0)
+    for name, got, ref in (("dq", qd.grad, gq), ("dk", kd.grad, gk), ("dv", vd.grad, gv)):
+        assert torch.isfinite(got).all()
+        err = O.rel_l2(got, ref)
+        assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
+    # The tokens of the low half on their own: their gradients are small next to the others' and must still be right.
+    # They are differences <dy_n, z_m - y_n> of latent rows that are nearly equal here (every latent sees the same
+    # dominant tokens) and enter the matrix cores rounded to bf16, hence the wider bar.
+    err = O.rel_l2(kd.grad[:, :, ::2], gk[:, :, ::2])
+    assert err <= 6e-2, f"dk of the low-scoring tokens rel-L2 {err:.3e}"
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_masked_backward_vs_autograd_oracle(dev, dtype):
     """Key mask (lra/models/backends.py:603-622) through the HIP backward: holes, a padded tail, a batch element with a
