@@ -505,14 +505,15 @@ __global__ __launch_bounds__(256) void bwd_merge_kernel(MixerBwdArgs a)
 
 // The five latent-side operand sets fill most of a CU's LDS at the usual sizes (82 KB at M = 256,
 // D = 32), so only one workgroup fits: it has 8 waves, two per SIMD, all reading the same operands.
-constexpr int kTokWaves = 8;
+template <int D> constexpr int kTokWaves = D <= 32 ? 12 : 8;
+template <int D> constexpr int kTokTiles = 2;      // 16-token column tiles per wave iteration
 
 template <typename T, int D>
-__global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs a, int tokens_per_wg)
+__global__ __launch_bounds__(64 * kTokWaves<D>, 1) void bwd_tok_kernel(MixerBwdArgs a, int tokens_per_wg)
 {
-    constexpr int NTH = 64 * kTokWaves;
+    constexpr int NTH = 64 * kTokWaves<D>;
     constexpr int KD = (D + 31) / 32, RT = D / 16, CH = D / 8;
-    constexpr int kBTW = D <= 32 ? 4 : 2;   // 16-token column tiles per wave iteration (registers allow 2 at D = 64)
+    constexpr int kBTW = kTokTiles<D>;
     using M_ = Mb<T>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     // M here is the chunk of latents this launch covers: when the five operand sets of all latents exceed the LDS,
@@ -589,7 +590,7 @@ __global__ __launch_bounds__(64 * kTokWaves, 1) void bwd_tok_kernel(MixerBwdArgs
     // part applies eL[m]; otherwise both exponentials are taken.
     auto walk = [&](auto fast_c, const float lmax2) {
     constexpr bool FAST = decltype(fast_c)::value;
-    for (int t0 = wg_n0 + w * 16 * kBTW; t0 < wg_n1; t0 += kTokWaves * 16 * kBTW) {
+    for (int t0 = wg_n0 + w * 16 * kBTW; t0 < wg_n1; t0 += kTokWaves<D> * 16 * kBTW) {
         u32x4 kb[kBTW][KD], vb[kBTW][KD], yb[kBTW][KD];
         float r2[kBTW], de[kBTW];      // FAST: r2 is unused, de = eR delta_n
 #pragma unroll
@@ -818,14 +819,15 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
         // one workgroup per compute unit, ranges a multiple of its 512-token pass
         const int64_t per_bh = (device_cus() + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H);
         int64_t tpw = (a.N + per_bh - 1) / per_bh;
-        tpw = ((tpw + 511) / 512) * 512;
+        constexpr int pass = kTokWaves<D> * 16 * kTokTiles<D>;
+        tpw = ((tpw + pass - 1) / pass) * pass;
         for (int c = 0; c < chunks; ++c) {
             MixerBwdArgs ac = a;
             ac.m0 = c * mc;
             ac.mc = mc;
             ac.accumulate = c > 0;
             ac.scal_lds = scal_lds ? 1 : 0;
-            hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(64 * kTokWaves), lds, st, ac, (int)tpw);
+            hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(64 * kTokWaves<D>), lds, st, ac, (int)tpw);
         }
     }
     e = lat_launch<T, D, 1>(a, st);
