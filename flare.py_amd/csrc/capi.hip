@@ -418,25 +418,30 @@ int flare_scatter_fwd_lse(const FlareMixerDesc* desc, const void* q, const void*
 }
 
 namespace {
-struct BwdPlan { int n_splits, tokens_per_split; size_t off_dz, off_dl, off_rm, off_part, total; };
+struct BwdPlan { int n_splits, tokens_per_split, n_splits0, tokens_per_split0; size_t off_dz, off_dl, off_rm, off_part, total; };
 
 BwdPlan plan_bwd(const FlareMixerDesc* d)
 {
     BwdPlan p;
     const int64_t bh = (int64_t)d->B * d->H;
     const int mblocks = d->M % 256 == 0 ? d->M / 256 : d->M % 128 == 0 ? d->M / 128 : (d->M + 63) / 64;
-    // about two workgroups per compute unit over the latent-side grids, token ranges of 64 k tokens
-    int64_t s = std::max<int64_t>(1, 2 * flare::device_cus() / (bh * mblocks));
-    int64_t tps = ((int64_t)d->N + s - 1) / s;
-    tps = (tps + 63) / 64 * 64;
-    p.tokens_per_split = (int)tps;
-    p.n_splits = (int)(((int64_t)d->N + tps - 1) / tps);
+    // About two workgroups per compute unit over the latent-side grids, which is what the registers of the dq pass
+    // allow; the dz pass needs fewer (up to D = 32) and gets three, with its own split of the token axis.
+    auto split = [&](int per_cu, int& n_splits, int& tokens_per_split) {
+        int64_t s = std::max<int64_t>(1, per_cu * flare::device_cus() / (bh * mblocks));
+        int64_t tps = ((int64_t)d->N + s - 1) / s;
+        tps = (tps + 63) / 64 * 64;
+        tokens_per_split = (int)tps;
+        n_splits = (int)(((int64_t)d->N + tps - 1) / tps);
+    };
+    split(2, p.n_splits, p.tokens_per_split);
+    split(d->D <= 32 ? 3 : 2, p.n_splits0, p.tokens_per_split0);
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     p.off_dz = up((size_t)bh * d->N * 4);
     p.off_dl = p.off_dz + up((size_t)bh * d->M * d->D * 4);
     p.off_rm = p.off_dl + up((size_t)bh * d->M * 4);
-    p.off_part = p.off_rm + up((size_t)bh * p.n_splits * 4);
-    p.total = p.off_part + (size_t)bh * p.n_splits * d->M * d->D * 4;
+    p.off_part = p.off_rm + up((size_t)bh * p.n_splits0 * 4);
+    p.total = p.off_part + (size_t)bh * std::max(p.n_splits, p.n_splits0) * d->M * d->D * 4;
     return p;
 }
 
@@ -491,6 +496,7 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
     a.dq = dq; a.dk = dk; a.dv = dv;
     a.B = desc->B; a.H = desc->H; a.N = desc->N; a.M = desc->M; a.D = desc->D;
     a.n_splits = p.n_splits; a.tokens_per_split = p.tokens_per_split;
+    a.n_splits0 = p.n_splits0; a.tokens_per_split0 = p.tokens_per_split0;
     a.scale = desc->scale; a.scale_log2 = desc->scale * 1.4426950408889634f;
     const int64_t nd = (int64_t)desc->N * desc->D;
     for (int i = 0; i < 3; ++i) {

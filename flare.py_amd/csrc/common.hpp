@@ -151,7 +151,8 @@ struct MixerBwdArgs {
     float* dq;               // [B,H,M,D] fp32
     void* dk; void* dv;      // [B,H,N,D] element type
     int B, H, N, M, D;
-    int n_splits, tokens_per_split;
+    int n_splits, tokens_per_split;      // split of the token axis a latent-side launch works in
+    int n_splits0, tokens_per_split0;    // the dz pass's own split (rho_min has one entry per such split)
     float scale, scale_log2;
     int64_t qs[3], ks[3], vs[3], ys[3], dys[3], dks[3], dvs[3];
     int m0, mc, accumulate;  // token-side kernel only: latents [m0, m0 + mc) of the M (mc = 0: all), added to dk, dv when accumulate

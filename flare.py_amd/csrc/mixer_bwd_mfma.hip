@@ -131,7 +131,7 @@ __device__ __forceinline__ bool factor_plan(const MixerBwdArgs& a, int64_t bh, i
 {
     float lm = -3.0e38f, rm = -3.0e38f;
     for (int m = lane; m < a.M; m += 64) lm = fmaxf(lm, a.lse_lat[bh * a.M + m]);
-    for (int p = lane; p < a.n_splits; p += 64) rm = fmaxf(rm, -a.rho_min[bh * a.n_splits + p]);
+    for (int p = lane; p < a.n_splits0; p += 64) rm = fmaxf(rm, -a.rho_min[bh * a.n_splits0 + p]);
     lmax2 = wave_max(lm) * kLog2e;
     // An empty batch element (its latents carry 1e30) takes the other form: differences of such magnitudes are
     // rounding noise far above the range of exp2.
@@ -802,9 +802,12 @@ template <typename T, int D>
 hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
 {
     const int64_t lat = (int64_t)a.B * a.H * a.M;
-    hipError_t e = lat_launch<T, D, 0>(a, st);
+    MixerBwdArgs a0 = a;          // the dz pass and its merge work in the dz pass's own split of the token axis
+    a0.n_splits = a.n_splits0;
+    a0.tokens_per_split = a.tokens_per_split0;
+    hipError_t e = lat_launch<T, D, 0>(a0, st);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(bwd_merge_kernel<0>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(bwd_merge_kernel<0>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a0);
     {
         auto kern = bwd_tok_kernel<T, D>;
         // the latents are covered in 1, 2 or 4 launches, each with the operand sets of its chunk in LDS
