@@ -487,6 +487,7 @@ __global__ __launch_bounds__(256) void bwd_merge_kernel(MixerBwdArgs a)
     const float* p0 = a.part + (bh * a.n_splits * a.M + m) * a.D + d;
     const int64_t sp = (int64_t)a.M * a.D;
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8      // eight loads in flight; the additions keep the split order
     for (int p = 0; p < a.n_splits; ++p) s += *reinterpret_cast<const f32x4*>(p0 + p * sp);
     if (MODE == 0) {
         const f32x4 zz = *reinterpret_cast<const f32x4*>(a.z + r * a.D + d);
