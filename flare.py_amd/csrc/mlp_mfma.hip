@@ -119,7 +119,7 @@ __device__ __forceinline__ float silu_gate(float x)
 // MODE: 0 the C x C chain, 1 the expanding two-layer MLP, 2 the chain with a narrow first input and/or last output,
 // 3 the chain with head-padded rows on either end
 template <typename T, int C, int TW, int WAVES, int MODE>
-__global__ __launch_bounds__(64 * WAVES, 512 / (64 * WAVES)) void mlp_mfma_kernel(MlpArgs a, int resident)
+__global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * WAVES) : 1)) void mlp_mfma_kernel(MlpArgs a, int resident)
 {
     constexpr int NT = 64 * WAVES;
     constexpr int NCH = (C * C / 8 + NT - 1) / NT;   // 16-byte weight chunks per thread and layer
@@ -500,7 +500,7 @@ hipError_t launch_t(const MlpArgs& a, hipStream_t st)
     const bool few = a.T < 32768;
     switch (a.C) {
         case 32:  return few ? launch_ct<T, 32, 1, 4>(a, st) : launch_ct<T, 32, 4, 4>(a, st);
-        case 64:  return few ? launch_ct<T, 64, 1, 4>(a, st) : launch_ct<T, 64, 4, 4>(a, st);
+        case 64:  return few ? launch_ct<T, 64, 1, 4>(a, st) : launch_ct<T, 64, 2, 4>(a, st);
         case 128: return few ? launch_ct<T, 128, 1, 8>(a, st) : launch_ct<T, 128, 2, 8>(a, st);
         default:  return hipErrorInvalidValue;
     }
