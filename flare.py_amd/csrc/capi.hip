@@ -809,6 +809,55 @@ int flare_mlp_io_fwd(const FlareMlpDesc* d, int32_t in_dim, int32_t in_act, cons
     return mlp_fwd_impl(d, in_dim, in_act, w_in, b_in, out_dim, x, w, bias, gamma, beta, res, y, stream);
 }
 
+int flare_mlp_bwd_partial_rows(const FlareMlpDesc* d, int32_t* rows)
+{
+    if (!d || !rows) return fail(FLARE_EINVAL, "descriptor and rows must not be NULL");
+    if (d->T < 1) return fail(FLARE_EINVAL, "T >= 1 required");
+    *rows = flare::mlp_bwd_partial_rows(d->T);
+    return FLARE_OK;
+}
+
+int flare_mlp_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const void* w_img, const void* wt_img,
+                  const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* a_in,
+                  void* g_out, void* dn, float* stats, float* gb_part, void* stream)
+{
+    if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
+    if (d->T < 1 || d->L < 1) return fail(FLARE_EINVAL, "T >= 1 and L >= 1 required (got %lld, %d)", (long long)d->T, d->L);
+    if (d->w_dtype != FLARE_DT_BF16 && d->w_dtype != FLARE_DT_F16) return fail(FLARE_EINVAL, "w_dtype must be bf16 or f16");
+    if (d->x_dtype < FLARE_DT_F32 || d->x_dtype > FLARE_DT_F16 || d->y_dtype < FLARE_DT_F32 || d->y_dtype > FLARE_DT_F16)
+        return fail(FLARE_EINVAL, "unknown dtype");
+    if (d->norm < FLARE_NORM_NONE || d->norm > FLARE_NORM_RMS) return fail(FLARE_EINVAL, "unknown norm %d", d->norm);
+    if (d->act < FLARE_ACT_GELU_TANH || d->act > FLARE_ACT_SILU) return fail(FLARE_EINVAL, "unknown activation %d", d->act);
+    if (!flare::mlp_mfma_supported(d->w_dtype, d->C)) return fail(FLARE_EUNSUPPORTED, "C=%d: only 32, 64 and 128 are supported", d->C);
+    if (d->L > flare::mlp_bwd_max_layers(d->C))
+        return fail(FLARE_EUNSUPPORTED, "the backward keeps every layer's slopes in registers: at most %d layers at C=%d (got %d)",
+                    flare::mlp_bwd_max_layers(d->C), d->C, d->L);
+    if (d->flags != 0) return fail(FLARE_EUNSUPPORTED, "the backward covers the chain of C x C layers only (flags must be 0)");
+    if (!x || !dy || !w_img || !wt_img || !dx || !a_in || !g_out) return fail(FLARE_EINVAL, "x, dy, w_img, wt_img, dx, a_in, g_out must not be NULL");
+    if (d->norm != FLARE_NORM_NONE && (!gamma || !dn || !stats || !gb_part))
+        return fail(FLARE_EINVAL, "gamma, dn, stats and gb_part must not be NULL when a norm is requested");
+    if (d->norm != FLARE_NORM_NONE && !(d->eps >= 0.f)) return fail(FLARE_EINVAL, "eps must be >= 0");
+    if (d->x_stride < d->C || d->x_stride % 4 || !aligned16(x)) return fail(FLARE_EINVAL, "x: row stride >= C, a multiple of 4, base 16-byte aligned");
+    if (d->y_stride < d->C || d->y_stride % 4 || !aligned16(dy)) return fail(FLARE_EINVAL, "dy: row stride (y_stride) >= C, a multiple of 4, base 16-byte aligned");
+    if (!aligned16(dx) || !aligned16(a_in) || !aligned16(g_out) || !aligned16(w_img) || !aligned16(wt_img) ||
+        (bias && !aligned16(bias)) || (gamma && !aligned16(gamma)) || (beta && !aligned16(beta)) || (dn && !aligned16(dn)) ||
+        (stats && !aligned16(stats)))
+        return fail(FLARE_EINVAL, "every buffer must be 16-byte aligned");
+    flare::MlpBwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = x; a.dy = dy; a.dx = dx;
+    a.w = static_cast<const uint16_t*>(w_img); a.wt = static_cast<const uint16_t*>(wt_img);
+    a.bias = bias; a.gamma = gamma; a.beta = beta;
+    a.a_in = static_cast<uint16_t*>(a_in); a.g_out = static_cast<uint16_t*>(g_out);
+    a.dn = static_cast<uint16_t*>(dn); a.stats = stats; a.gb_part = gb_part;
+    a.T = d->T; a.C = d->C; a.L = d->L;
+    a.x_dtype = d->x_dtype; a.dy_dtype = d->y_dtype; a.dx_dtype = d->x_dtype;
+    a.norm = d->norm; a.eps = d->eps; a.act = d->act; a.act_mask = d->act_mask; a.add_mask = d->add_mask;
+    a.add_dy = add_dy ? 1 : 0;
+    a.xs = d->x_stride; a.dys = d->y_stride; a.dxs = d->C;
+    return hip_status(flare::launch_mlp_bwd(a, d->w_dtype, static_cast<hipStream_t>(stream)), "mlp backward launch");
+}
+
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes)
 {
     if (!bytes) return fail(FLARE_EINVAL, "bytes is NULL");

@@ -190,6 +190,28 @@ struct MlpArgs {
     int64_t xs, rs, ys;                         // row strides in elements
 };
 
+// backward of the fused MLP chain (mlp_bwd_mfma.hip)
+struct MlpBwdArgs {
+    const void* x; const void* dy; void* dx;    // [T,C] rows: the forward's input, the gradient of its output, the gradient of x
+    const uint16_t* w; const uint16_t* wt;      // [L,C,C] 16-bit weights [out][in] and their transposes [in][out]
+    const float* bias;                          // [L,C] or null
+    const float* gamma; const float* beta;      // [C] norm parameters (beta may be null)
+    uint16_t* a_in;                             // [L,T,C] out: the input s_l of every layer, in the weights' type
+    uint16_t* g_out;                            // [L,T,C] out: dt_l, the gradient at every layer's product, same type
+    uint16_t* dn;                               // [T,C] out (norm != 0): ds_0, the gradient at the norm's output, same type
+    float* stats;                               // [T,2] out (norm != 0): mean and 1/std of every token
+    float* gb_part;                             // [rows,2,C] out (norm != 0): partial sums of dgamma, dbeta over token ranges
+    int64_t T;
+    int C, L;
+    int x_dtype, dy_dtype, dx_dtype;            // 0 f32, 1 bf16, 2 f16
+    int norm;                                   // 0 none, 1 LayerNorm, 2 RMSNorm
+    float eps;
+    int act;                                    // 0 tanh-GELU, 1 SiLU
+    uint32_t act_mask, add_mask;
+    int add_dy;                                 // the forward's residual input was x itself: dx also receives dy
+    int64_t xs, dys, dxs;                       // row strides in elements
+};
+
 // ---- launchers implemented in the .hip files -------------------------------------------
 hipError_t launch_gather_generic(const MixerArgs& a, int dtype, hipStream_t st);
 hipError_t launch_gather_merge(const MixerArgs& a, hipStream_t st);
@@ -226,6 +248,9 @@ hipError_t launch_mixer_bwd(const MixerBwdArgs& a, int dtype, hipStream_t st);
 
 bool       mlp_mfma_supported(int w_dtype, int C);
 hipError_t launch_mlp_mfma(const MlpArgs& a, int w_dtype, hipStream_t st);
+int        mlp_bwd_max_layers(int C);
+int        mlp_bwd_partial_rows(int64_t T);
+hipError_t launch_mlp_bwd(const MlpBwdArgs& a, int w_dtype, hipStream_t st);
 
 int        causal_linear_tile();
 hipError_t launch_causal_linear(const CausalLinearArgs& a, int dtype, hipStream_t st);

@@ -1,0 +1,447 @@
+// Backward of the fused token-wise MLP stack of mlp_mfma.hip (the chain of C x C layers; bf16 / f16 weights,
+// C in {32, 64, 128}): what torch autograd does for  y = res + ResidualMLP(norm(x))  of
+// pdebench/models/flare.py:45-59 and 204-215, in one token-parallel launch plus a few library products.
+//
+// Forward, per token:  s_0 = norm(x);  layer l:  t_l = W_l s_l + b_l,  u_l = act(t_l) if bit l of act_mask else t_l,
+// s_{l+1} = s_l + u_l if bit l of add_mask else u_l;  y = res + s_L.
+// Backward, given dy:  ds_L = dy;  for l = L-1 .. 0:  dt_l = ds_{l+1} * act'(t_l),
+// ds_l = (ds_{l+1} if add) + W_l^T dt_l;  then the norm's backward gives dx.  Parameter gradients:
+//   dW_l = sum_t dt_l s_l^T,   db_l = sum_t dt_l,   dgamma = sum_t ds_0 * xhat,   dbeta = sum_t ds_0.
+//
+// The kernel recomputes the forward for its 16-token tile (same layout as mlp_mfma.hip: the product is taken
+// transposed, lane = token, the accumulators of one layer packed to 16 bits are the B operands of the next), keeps
+// act'(t_l) of every layer packed to 16 bits in registers, and walks the chain back with the TRANSPOSED weights in
+// the place of the weights (ds_l^T = W_l^T dt_l^T is the same product shape).  What a reduction over all tokens
+// needs leaves the kernel as 16-bit rows: s_l (the input of every layer) and dt_l, from which the caller forms
+// dW_l = dt_l^T s_l and db_l with library products; for the norm's parameters the kernel leaves ds_0 as 16-bit rows
+// and every token's (mean, 1/std), and mlp_norm_grads_kernel sums dgamma, dbeta over token ranges into one partial
+// row per workgroup (summed by the caller in a fixed order: no atomics).
+// Weights move through LDS: all 2 L tiles resident when they fit, else a two-slot ring in the order
+// W_0 .. W_{L-1}, W_{L-1}^T .. W_0^T with one barrier per layer; they arrive as LDS images and are loaded straight
+// into their slots.
+#include <algorithm>
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace flare {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct Mw;
+template <> struct Mw<bf16_t> {
+    static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        bf16x2 v = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float lo(uint32_t p) { return __uint_as_float(p << 16); }
+    static __device__ __forceinline__ float hi(uint32_t p) { return __uint_as_float(p & 0xffff0000u); }
+};
+template <> struct Mw<f16_t> {
+    static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        f16x2 v = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ float lo(uint32_t p) { return (float)__builtin_bit_cast(f16x2, p)[0]; }
+    static __device__ __forceinline__ float hi(uint32_t p) { return (float)__builtin_bit_cast(f16x2, p)[1]; }
+};
+
+// four consecutive elements of a row of element type dt (0 f32, 1 bf16, 2 f16) as fp32
+__device__ __forceinline__ f32x4 ld4(const void* base, int64_t elem, int dt)
+{
+    if (dt == 0) return *reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + elem);
+    const uint2 r = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + elem);
+    if (dt == 1)
+        return f32x4{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
+                     __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u)};
+    const f16x2 lo = __builtin_bit_cast(f16x2, r.x), hi = __builtin_bit_cast(f16x2, r.y);
+    return f32x4{(float)lo[0], (float)lo[1], (float)hi[0], (float)hi[1]};
+}
+
+__device__ __forceinline__ void st4(void* base, int64_t elem, int dt, f32x4 v)
+{
+    if (dt == 0) {
+        *reinterpret_cast<f32x4*>(static_cast<float*>(base) + elem) = v;
+    } else if (dt == 1) {
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(base) + elem) =
+            make_uint2(Mw<bf16_t>::pack2(v[0], v[1]), Mw<bf16_t>::pack2(v[2], v[3]));
+    } else {
+        *reinterpret_cast<uint2*>(static_cast<uint16_t*>(base) + elem) =
+            make_uint2(Mw<f16_t>::pack2(v[0], v[1]), Mw<f16_t>::pack2(v[2], v[3]));
+    }
+}
+
+__device__ __forceinline__ float tok_sum(float v)   // sum over the 4 lane groups that share a token
+{
+    v = sum_xor16(v);
+    v = sum_xor32(v);
+    return v;
+}
+
+// act(t) = t * gate and its derivative.  tanh-GELU: gate = sigmoid(2u), 2u = t (1.5957691 + 0.0713548 t^2), so
+// act' = gate (1 + t (1 - gate) (1.5957691 + 0.2140645 t^2));  SiLU: gate = sigmoid(t), act' = gate (1 + t (1 - gate)).
+template <int ACT>
+__device__ __forceinline__ void act_and_slope(float t, float& value, float& slope)
+{
+    if (ACT == 1) {
+        const float t2 = t * t;
+        const float gate = __builtin_amdgcn_rcpf(1.f + fast_exp2(-t * (2.3022081f + 0.10294324f * t2)));
+        value = t * gate;
+        slope = gate * fmaf(t * (1.f - gate), fmaf(0.2140645f, t2, 1.5957691f), 1.f);
+    } else {
+        const float gate = __builtin_amdgcn_rcpf(1.f + fast_exp2(-kLog2e * t));
+        value = t * gate;
+        slope = gate * fmaf(t, 1.f - gate, 1.f);
+    }
+}
+
+// LMAX: the layers are unrolled up to this count (their saved slopes live in registers), a.L <= LMAX.
+template <typename T, int C, int WAVES, int LMAX>
+__global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, int resident)
+{
+    constexpr int NT = 64 * WAVES;
+    constexpr int NCH = (C * C / 8 + NT - 1) / NT;   // 16-byte weight chunks per thread and tile
+    constexpr int FT = C / 16;        // feature tiles of the stream
+    constexpr int KS = C / 32;        // k-steps of one layer
+    constexpr int RS = C * 2;         // LDS row stride in bytes (16-byte chunks XOR-swizzled with the row number)
+    constexpr int WBUF = C * RS;
+    constexpr int CPR = C / 8;
+    constexpr int SWS = CPR == 16 ? 0 : CPR == 8 ? 1 : 2;
+    using M_ = Mw<T>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int L = a.L;
+
+    // Weight tile of ring step q: W_q for q < L (forward), W_{2L-1-q}^T after that (backward).  The caller hands
+    // the tiles over as LDS images (the 16-bit elements already in the order the A-operand reads expect, see
+    // mlp_weight_image in the host code), so a tile goes from global memory straight into its slot, 16 bytes per
+    // lane, with no registers and no LDS stores in between.
+    auto stage = [&](int q, int slot) {
+        const uint16_t* img = q < L ? a.w + (size_t)q * C * C : a.wt + (size_t)(2 * L - 1 - q) * C * C;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c0 = i * NT + w * 64;           // first 16-byte chunk of this wave's share (uniform over the wave)
+            if (c0 < C * C / 8)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(img + (size_t)(c0 + lane) * 8),
+                                                 (__attribute__((address_space(3))) void*)(smem + slot * WBUF + c0 * 16), 16, 0, 0);
+        }
+    };
+    auto staged = [&]() {       // the workgroup's loads have landed and are visible to all its waves
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    };
+    int woff[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) woff[ks] = ((4 * ks + g) ^ (c16 >> SWS)) << 4;
+
+    int qcount = 0;      // ring mode: steps done by this workgroup; its parity names the slot in use
+    if (resident) {
+        for (int q = 0; q < 2 * L; ++q) stage(q, q);
+    } else {
+        stage(0, 0);
+    }
+    staged();
+
+    // one product of a layer: out tile ft = init + (weight tile of the current ring slot) x (packed operand)
+    auto ring_step_begin = [&](int q) -> const uint8_t* {
+        const int slot = resident ? q : (qcount & 1);
+        // ring: the next step's tile goes into the other slot, which nobody has read since the last barrier
+        if (!resident) stage(q + 1 < 2 * L ? q + 1 : 0, slot ^ 1);
+        return smem + slot * WBUF + c16 * RS;
+    };
+    auto ring_step_end = [&]() {
+        if (!resident) staged();
+        ++qcount;
+    };
+
+    const int64_t nblk = ((int64_t)a.T + WAVES * 16 - 1) / (WAVES * 16);
+    for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
+        const int64_t t = blk * (WAVES * 16) + w * 16 + c16;
+        const bool live = t < a.T;
+        const int64_t tok = live ? t : a.T - 1;
+
+        // ---- forward, recomputed: the stream, the inputs of every layer, the slopes of every activation ----
+        f32x4 xs[FT];
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft) xs[ft] = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+        float mean = 0.f, rstd = 1.f;
+        if (a.norm != 0) {
+            float s = 0.f;
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) s += xs[ft][0] + xs[ft][1] + xs[ft][2] + xs[ft][3];
+            const float rowmean = tok_sum(s) * (1.f / C);
+            mean = a.norm == 1 ? rowmean : 0.f;
+            float ss = 0.f;
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float d = xs[ft][r] - mean;
+                    ss = fmaf(d, d, ss);
+                }
+            rstd = rsqrtf(tok_sum(ss) * (1.f / C) + a.eps);
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                const f32x4 gm = *reinterpret_cast<const f32x4*>(a.gamma + 16 * ft + 4 * g);
+                f32x4 bt = {0.f, 0.f, 0.f, 0.f};
+                if (a.beta) bt = *reinterpret_cast<const f32x4*>(a.beta + 16 * ft + 4 * g);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) xs[ft][r] = (xs[ft][r] - mean) * rstd * gm[r] + bt[r];
+            }
+        }
+
+        uint32_t slope[LMAX][FT][2];      // act'(t_l), packed to 16 bits (layers without activation: unused)
+#pragma unroll
+        for (int l = 0; l < LMAX; ++l) {
+            if (l >= L) break;
+            const uint8_t* wb = ring_step_begin(l);
+            u32x4 xb[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const f32x4 lo = xs[2 * ks], hi = xs[2 * ks + 1];
+                xb[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
+            }
+            if (live) {       // s_l, the input of layer l, as a 16-bit row (for dW_l)
+                uint16_t* row = a.a_in + ((size_t)l * a.T + tok) * C + 4 * g;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    *reinterpret_cast<uint2*>(row + 32 * ks) = make_uint2(xb[ks][0], xb[ks][1]);
+                    *reinterpret_cast<uint2*>(row + 32 * ks + 16) = make_uint2(xb[ks][2], xb[ks][3]);
+                }
+            }
+            const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
+            auto layer = [&](auto act_c, auto add_c) {
+                constexpr int ACT = decltype(act_c)::value;
+                constexpr bool ADD = decltype(add_c)::value;
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft) {
+                    f32x4 acc = a.bias ? *reinterpret_cast<const f32x4*>(a.bias + (size_t)l * C + 16 * ft + 4 * g)
+                                       : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks)
+                        acc = M_::mma(*reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]), xb[ks], acc);
+                    float sl[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float u = acc[r];
+                        sl[r] = 1.f;
+                        if constexpr (ACT != 0) act_and_slope<ACT>(acc[r], u, sl[r]);
+                        xs[ft][r] = ADD ? xs[ft][r] + u : u;
+                    }
+                    slope[l][ft][0] = M_::pack2(sl[0], sl[1]);
+                    slope[l][ft][1] = M_::pack2(sl[2], sl[3]);
+                    // two feature tiles at a time: without a fence the scheduler lifts the operand reads of all
+                    // tiles to the front and the slopes of five layers no longer fit beside them
+                    if (C == 128 && (ft & 1)) __builtin_amdgcn_sched_barrier(0);
+                }
+            };
+            using I0 = std::integral_constant<int, 0>;
+            using I1 = std::integral_constant<int, 1>;
+            using I2 = std::integral_constant<int, 2>;
+            if (!act) {
+                if (add) layer(I0{}, std::true_type{}); else layer(I0{}, std::false_type{});
+            } else if (a.act == 0) {
+                if (add) layer(I1{}, std::true_type{}); else layer(I1{}, std::false_type{});
+            } else {
+                if (add) layer(I2{}, std::true_type{}); else layer(I2{}, std::false_type{});
+            }
+            ring_step_end();
+        }
+
+        // ---- backward through the chain: xs becomes ds ----
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft) {
+            xs[ft] = ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
+            if (!live) xs[ft] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int l = LMAX - 1; l >= 0; --l) {
+            if (l >= L) continue;
+            const uint8_t* wb = ring_step_begin(2 * L - 1 - l);
+            const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
+            // dt_l = ds_{l+1} * act'(t_l), packed: the B operands of this product and the rows kept for dW_l, db_l
+            u32x4 db[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                f32x4 lo = xs[2 * ks], hi = xs[2 * ks + 1];
+                if (act) {
+                    const uint32_t* s0 = slope[l][2 * ks];
+                    const uint32_t* s1 = slope[l][2 * ks + 1];
+                    lo[0] *= M_::lo(s0[0]); lo[1] *= M_::hi(s0[0]); lo[2] *= M_::lo(s0[1]); lo[3] *= M_::hi(s0[1]);
+                    hi[0] *= M_::lo(s1[0]); hi[1] *= M_::hi(s1[0]); hi[2] *= M_::lo(s1[1]); hi[3] *= M_::hi(s1[1]);
+                }
+                db[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
+            }
+            if (live) {
+                uint16_t* row = a.g_out + ((size_t)l * a.T + tok) * C + 4 * g;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    *reinterpret_cast<uint2*>(row + 32 * ks) = make_uint2(db[ks][0], db[ks][1]);
+                    *reinterpret_cast<uint2*>(row + 32 * ks + 16) = make_uint2(db[ks][2], db[ks][3]);
+                }
+            }
+            // ds_l = (ds_{l+1} if the layer added to the stream) + W_l^T dt_l
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                f32x4 acc = add ? xs[ft] : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks)
+                    acc = M_::mma(*reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]), db[ks], acc);
+                xs[ft] = acc;
+                if (C == 128 && (ft & 1)) __builtin_amdgcn_sched_barrier(0);
+            }
+            ring_step_end();
+        }
+
+        // ---- the norm's backward, dx ----
+        if (a.norm != 0) {
+            // ds_0 and the token's statistics go out for dgamma, dbeta; xhat is taken again from x (the row is still
+            // in cache) rather than kept in registers;  g = ds_0 * gamma
+            if (live) {
+                uint16_t* row = a.dn + (size_t)tok * C + 4 * g;
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft)
+                    *reinterpret_cast<uint2*>(row + 16 * ft) = make_uint2(M_::pack2(xs[ft][0], xs[ft][1]), M_::pack2(xs[ft][2], xs[ft][3]));
+                if (lane < 16) *reinterpret_cast<float2*>(a.stats + 2 * tok) = make_float2(mean, rstd);
+            }
+            float m1 = 0.f, m2 = 0.f;
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                const f32x4 xr = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+                const f32x4 gm = *reinterpret_cast<const f32x4*>(a.gamma + 16 * ft + 4 * g);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    xs[ft][r] *= gm[r];
+                    m1 += xs[ft][r];
+                    m2 = fmaf(xs[ft][r], (xr[r] - mean) * rstd, m2);
+                }
+            }
+            m1 = a.norm == 1 ? tok_sum(m1) * (1.f / C) : 0.f;
+            m2 = tok_sum(m2) * (1.f / C);
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                const f32x4 xr = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) xs[ft][r] = rstd * (xs[ft][r] - m1 - (xr[r] - mean) * rstd * m2);
+            }
+        }
+        if (live) {
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                f32x4 o = xs[ft];
+                if (a.add_dy) o += ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
+                st4(a.dx, tok * a.dxs + 16 * ft + 4 * g, a.dx_dtype, o);
+            }
+        }
+    }
+}
+
+// dgamma[c] = sum_t ds_0[t,c] xhat[t,c],  dbeta[c] = sum_t ds_0[t,c]  over the workgroup's token range: thread = channel
+// (C <= 128 of the 128 threads), rows read coalesced, one partial row pair per workgroup.
+template <typename T>
+__global__ __launch_bounds__(128) void mlp_norm_grads_kernel(MlpBwdArgs a, int64_t tokens_per_wg)
+{
+    using M_ = Mw<T>;
+    const int c = threadIdx.x;
+    const int64_t t0 = (int64_t)blockIdx.x * tokens_per_wg, t1 = t0 + tokens_per_wg < a.T ? t0 + tokens_per_wg : a.T;
+    float gs = 0.f, bs = 0.f;
+    if (c < a.C) {
+        for (int64_t t = t0; t < t1; ++t) {
+            const float2 st = *reinterpret_cast<const float2*>(a.stats + 2 * t);
+            const int64_t e = t * a.xs + c;
+            const float xv = a.x_dtype == 0 ? static_cast<const float*>(a.x)[e]
+                           : a.x_dtype == 1 ? __uint_as_float(uint32_t(static_cast<const uint16_t*>(a.x)[e]) << 16)
+                                            : (float)static_cast<const _Float16*>(a.x)[e];
+            const uint32_t raw = a.dn[(size_t)t * a.C + c];
+            const float dv = M_::lo(raw);
+            gs = fmaf(dv, (xv - st.x) * st.y, gs);
+            bs += dv;
+        }
+        a.gb_part[((size_t)blockIdx.x * 2 + 0) * a.C + c] = gs;
+        a.gb_part[((size_t)blockIdx.x * 2 + 1) * a.C + c] = bs;
+    }
+}
+
+template <typename T, int C, int WAVES, int LMAX>
+hipError_t launch_l(const MlpBwdArgs& a, hipStream_t st)
+{
+    auto kern = mlp_bwd_kernel<T, C, WAVES, LMAX>;
+    const size_t wbuf = (size_t)C * C * 2;
+    int resident = (size_t)2 * a.L * wbuf <= 160 * 1024 ? 1 : 0;
+    size_t lds = (resident ? (size_t)2 * a.L : 2) * wbuf;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess && resident) {
+        (void)hipGetLastError();
+        resident = 0;
+        lds = 2 * wbuf;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    }
+    if (e != hipSuccess) return e;
+    const int64_t nblk = (a.T + WAVES * 16 - 1) / (WAVES * 16);
+    const int64_t cus = device_cus();
+    hipLaunchKernelGGL(kern, dim3((unsigned)(nblk < cus ? nblk : cus)), dim3(64 * WAVES), lds, st, a, resident);
+    e = hipGetLastError();
+    if (e != hipSuccess || a.norm == 0) return e;
+    const int rows = mlp_bwd_partial_rows(a.T);
+    const int64_t tpw = (a.T + rows - 1) / rows;
+    hipLaunchKernelGGL(mlp_norm_grads_kernel<T>, dim3(rows), dim3(128), 0, st, a, tpw);
+    return hipGetLastError();
+}
+
+template <typename T, int C, int WAVES>
+hipError_t launch_c(const MlpBwdArgs& a, hipStream_t st)
+{
+    if (a.L <= 1) return launch_l<T, C, WAVES, 1>(a, st);
+    if (a.L <= 5) return launch_l<T, C, WAVES, 5>(a, st);
+    if (a.L <= mlp_bwd_max_layers(C)) return launch_l<T, C, WAVES, (C == 128 ? 5 : 8)>(a, st);
+    return hipErrorInvalidValue;
+}
+
+template <typename T>
+hipError_t launch_t(const MlpBwdArgs& a, hipStream_t st)
+{
+    switch (a.C) {
+        case 32:  return launch_c<T, 32, 4>(a, st);
+        case 64:  return launch_c<T, 64, 4>(a, st);
+        case 128: return launch_c<T, 128, 8>(a, st);
+        default:  return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+// layers whose activation slopes fit the registers of one lane
+int mlp_bwd_max_layers(int C) { return C == 128 ? 5 : 8; }
+
+// partial rows of dgamma, dbeta a launch writes (one per workgroup of the reduction over tokens: token ranges of at
+// least 256 tokens, at most two workgroups per compute unit)
+int mlp_bwd_partial_rows(int64_t T)
+{
+    const int64_t want = (T + 255) / 256, cap = 2 * (int64_t)device_cus();
+    return (int)(want < cap ? (want < 1 ? 1 : want) : cap);
+}
+
+hipError_t launch_mlp_bwd(const MlpBwdArgs& a, int w_dtype, hipStream_t st)
+{
+    return w_dtype == 1 ? launch_t<bf16_t>(a, st) : launch_t<f16_t>(a, st);
+}
+
+}  // namespace flare

@@ -1,4 +1,4 @@
-"""Fused inference path for the token-wise layers around the mixer (HIP kernel flare_mlp_fwd).
+"""Fused path for the token-wise layers around the mixer (HIP kernels flare_mlp_fwd / flare_mlp_bwd).
 
 `fused_mlp(x, mlp, norm=..., res=...)` evaluates, in ONE launch and without leaving the chip
 between layers, what the reference runs as separate torch layers:
@@ -12,10 +12,16 @@ between layers, what the reference runs as separate torch layers:
 A ResidualMLP with num_layers == 0 and a hidden width of E*C (2 <= E <= 8; the "4x expansion" feed-forward
 block) runs in the same launch as E pairs of C x C tiles, the hidden activations never leaving the registers.
 
-It is used by the modules only when no gradient is needed and the products may run in bf16/f16
-(torch.autocast is on, or the weights already are bf16/f16) — the conditions under which torch
-itself would run these Linear layers in that type.  Everything else stays with the torch layers.
-The 16-bit copies of the weights are cached per module and rebuilt when a parameter changes.
+It is used by the modules only when the products may run in bf16/f16 (torch.autocast is on, or the
+weights already are bf16/f16) — the conditions under which torch itself would run these Linear layers
+in that type.  Everything else stays with the torch layers.  The 16-bit copies of the weights are
+cached per module and rebuilt when a parameter changes.
+
+With gradients enabled the chain of C x C layers (the k/v projections, the feed-forward block and the output
+projection of a FLAREBlock at the reference's default ratios) runs through `_FusedMlpFn`: the same forward
+launch, and a backward that recomputes the chain per token tile in one launch (flare_mlp_bwd) and forms the
+parameter gradients from the rows it leaves with two batched library products.  The narrow-end, expanding and
+head-padded variants have no backward and stay with the torch layers while gradients are enabled.
 """
 from __future__ import annotations
 
@@ -89,9 +95,13 @@ def _io_dims(mod, layers):
     return Cdim, (0 if i == Cdim else i), (0 if o == Cdim else o)
 
 
+_BWD_MAX_LAYERS = {32: 8, 64: 8, 128: 5}      # the backward keeps every layer's slopes in registers
+
+
 def compute_dtype(x, mod):
-    """The 16-bit type the fused kernel may run this module in, or None (then torch runs it)."""
-    if torch.is_grad_enabled() or x.device.type != "cuda":
+    """The 16-bit type the fused kernels may run this module in, or None (then torch runs it).  With gradients
+    enabled only the chain of C x C layers qualifies (the shapes flare_mlp_bwd differentiates)."""
+    if x.device.type != "cuda":
         return None
     info = _layers_of(mod)
     if info is None:
@@ -99,6 +109,12 @@ def compute_dtype(x, mod):
     layers = info[0]
     if len(layers) > 16:
         return None
+    if torch.is_grad_enabled():
+        Cdim = x.shape[-1]
+        if Cdim not in _SUPPORTED_C or len(layers) > _BWD_MAX_LAYERS[Cdim]:
+            return None
+        if any(l.in_features != Cdim or l.out_features != Cdim for l in layers):
+            return None
     io = _io_dims(mod, layers)
     if io is not None and (io[1] or io[2]):
         if io[0] not in _SUPPORTED_C or x.shape[-1] != layers[0].in_features:
@@ -230,7 +246,16 @@ def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None, x_head=0, y_head=
     """y = res + mod(norm(x)) in one HIP launch.  x: [..., C]; mod: ResidualMLP or nn.Linear; cd: the
     dtype from compute_dtype(); norm: nn.LayerNorm / nn.RMSNorm / None; res: [..., C] or None.
     x_head / y_head (4 or 8): x is / y comes back head-padded, [..., (C / head) * 16] with every head's channels
-    followed by zeros up to 16 columns -- the layout the mixer reads and writes for head dims below 16."""
+    followed by zeros up to 16 columns -- the layout the mixer reads and writes for head dims below 16.
+    With gradients enabled the call is differentiable (chain of C x C layers only, see compute_dtype)."""
+    if torch.is_grad_enabled():
+        if x_head or y_head:
+            raise ValueError("head-padded rows have no backward: call under torch.no_grad()")
+        return _fused_mlp_train(x, mod, cd, norm, res, out_dtype)
+    return _fused_mlp_fwd(x, mod, cd, norm, res, out_dtype, x_head, y_head)
+
+
+def _fused_mlp_fwd(x, mod, cd, norm=None, res=None, out_dtype=None, x_head=0, y_head=0):
     lib = _lib.load()
     info = _layers_of(mod)
     layers, act_mask, add_mask, act = info
@@ -273,3 +298,134 @@ def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None, x_head=0, y_head=
                                C.c_void_p(_stream_ptr(x.device)))
     _lib.check(rc, "flare_mlp_fwd")
     return y
+
+
+# --------------------------------------------------------------------------------------
+# training: forward launch + flare_mlp_bwd
+# --------------------------------------------------------------------------------------
+_IMG_INDEX = {}
+
+
+def _image_index(Cdim, device):
+    """For every 16-bit position of a weight tile's LDS image, the row-major element that sits there (the inverse of
+    the formula in include/flare_hip.h): element (row, col) of the tile is the A operand of output row `row`, and
+    the kernels read 8 consecutive k-slots per lane."""
+    key = (Cdim, str(device))
+    idx = _IMG_INDEX.get(key)
+    if idx is None:
+        sws = {128: 0, 64: 1, 32: 2}[Cdim]
+        row = torch.arange(Cdim).view(-1, 1).expand(Cdim, Cdim)
+        col = torch.arange(Cdim).view(1, -1).expand(Cdim, Cdim)
+        ch, j = col // 8, col % 8
+        chunk = 4 * (ch // 4) + 2 * (ch % 2) + j // 4
+        pos = row * Cdim + 8 * (chunk ^ ((row % 16) >> sws)) + 4 * ((ch % 4) // 2) + j % 4
+        idx = torch.empty(Cdim * Cdim, dtype=torch.long)
+        idx[pos.reshape(-1)] = torch.arange(Cdim * Cdim)
+        idx = _IMG_INDEX[key] = idx.to(device)
+    return idx
+
+
+def mlp_weight_image(w):
+    """[L,C,C] weights ([out][in] per tile) -> the LDS images flare_mlp_bwd loads straight into its weight slots."""
+    L, Cdim, _ = w.shape
+    return w.reshape(L, Cdim * Cdim)[:, _image_index(Cdim, w.device)].contiguous()
+
+
+def _packed_train(mod, layers, cd):
+    """(w [L,C,C] for the forward launch, images of the weights and of their transposes for the backward, fp32 biases
+    [L,C]), cached on the module until a parameter changes."""
+    key = ("train", cd, tuple((l.weight.data_ptr(), l.weight._version, None if l.bias is None else l.bias._version) for l in layers))
+    cache = mod.__dict__.get("_flare_packed_train")
+    if cache is not None and cache[0] == key:
+        return cache[1:]
+    w, b = _packed(mod, layers, cd)
+    w_img = mlp_weight_image(w)
+    wt_img = mlp_weight_image(w.transpose(1, 2).contiguous())
+    mod.__dict__["_flare_packed_train"] = (key, w, b, w_img, wt_img)
+    return w, b, w_img, wt_img
+
+
+class _FusedMlpFn(torch.autograd.Function):
+    """y = res + chain(norm(x)); parameters are passed as inputs so that autograd routes their gradients:
+    (x, res, gamma, beta, w_0 .. w_{L-1}, b_0 .. b_{L-1}) with None where a tensor does not exist."""
+
+    @staticmethod
+    def forward(ctx, mod, cd, norm, out_dtype, x, res, gamma, beta, *wb):
+        with torch.no_grad():
+            y = _fused_mlp_fwd(x, mod, cd, norm=norm, res=res, out_dtype=out_dtype)
+        ctx.mod, ctx.cd, ctx.norm = mod, cd, norm
+        ctx.res_is_x = (res is not None and res.data_ptr() == x.data_ptr() and res.shape == x.shape
+                        and res.stride() == x.stride() and res.dtype == x.dtype)
+        ctx.has_res = res is not None
+        ctx.n_wb = len(wb)
+        ctx.save_for_backward(x)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        (x,) = ctx.saved_tensors
+        mod, cd, norm = ctx.mod, ctx.cd, ctx.norm
+        lib = _lib.load()
+        layers, act_mask, add_mask, act = _layers_of(mod)
+        L = len(layers)
+        Cdim = x.shape[-1]
+        _, b, w_img, wt_img = _packed_train(mod, layers, cd)
+        x2 = x.reshape(-1, Cdim)
+        if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 16:
+            x2 = x2.contiguous()
+        dy2 = dy.reshape(-1, Cdim)
+        if dy2.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+            dy2 = dy2.float()
+        if dy2.stride(-1) != 1 or dy2.stride(0) % 4 or dy2.data_ptr() % 16:
+            dy2 = dy2.contiguous()
+        T = x2.shape[0]
+        dev = x.device
+        d = _lib.FlareMlpDesc()
+        d.T, d.C, d.L = T, Cdim, L
+        d.w_dtype, d.x_dtype, d.y_dtype = _dtype_code(w_img), _dtype_code(x2), _dtype_code(dy2)
+        d.act, d.act_mask, d.add_mask = act, act_mask, add_mask
+        d.x_stride, d.y_stride = x2.stride(0), dy2.stride(0)
+        gamma, beta = _norm_args(d, norm, x, Cdim)
+        dx = torch.empty(T, Cdim, dtype=x2.dtype, device=dev)
+        a_in = torch.empty(L, T, Cdim, dtype=cd, device=dev)
+        g_out = torch.empty(L, T, Cdim, dtype=cd, device=dev)
+        dn = stats = gb = None
+        if d.norm:
+            rows = C.c_int32(0)
+            _lib.check(lib.flare_mlp_bwd_partial_rows(C.byref(d), C.byref(rows)), "flare_mlp_bwd_partial_rows")
+            dn = torch.empty(T, Cdim, dtype=cd, device=dev)
+            stats = torch.empty(T, 2, dtype=torch.float32, device=dev)
+            gb = torch.empty(rows.value, 2, Cdim, dtype=torch.float32, device=dev)
+        with _on_device(dev):
+            rc = lib.flare_mlp_bwd(C.byref(d), _ptr(x2), _ptr(dy2), _ptr(w_img), _ptr(wt_img), _ptr(b), _ptr(gamma), _ptr(beta),
+                                   1 if ctx.res_is_x else 0, _ptr(dx), _ptr(a_in), _ptr(g_out), _ptr(dn), _ptr(stats), _ptr(gb),
+                                   C.c_void_p(_stream_ptr(dev)))
+        _lib.check(rc, "flare_mlp_bwd")
+        # parameter gradients: two batched products over the rows the kernel left (16-bit products with fp32
+        # accumulation, as torch runs a Linear's backward under autocast), sums in a fixed order
+        dW = torch.bmm(g_out.transpose(1, 2), a_in)                      # [L, out, in]
+        db = g_out.sum(dim=1, dtype=torch.float32)                       # [L, C]
+        need = ctx.needs_input_grad            # (mod, cd, norm, out_dtype, x, res, gamma, beta, *wb)
+        grads = [None, None, None, None]
+        grads.append(dx.view(x.shape) if need[4] else None)
+        grads.append(None if (not ctx.has_res or ctx.res_is_x or not need[5]) else dy)
+        if d.norm:
+            gsum = gb.sum(0)
+            grads.append(gsum[0].to(norm.weight.dtype) if need[6] else None)
+            grads.append(gsum[1].to(norm.bias.dtype) if (need[7] and getattr(norm, "bias", None) is not None) else None)
+        else:
+            grads += [None, None]
+        for i, l in enumerate(layers):
+            grads.append(dW[i].to(l.weight.dtype) if need[8 + i] else None)
+        for i, l in enumerate(layers):
+            grads.append(db[i].to(l.bias.dtype) if (l.bias is not None and need[8 + L + i]) else None)
+        return tuple(grads)
+
+
+def _fused_mlp_train(x, mod, cd, norm, res, out_dtype):
+    layers = _layers_of(mod)[0]
+    has_norm = norm is not None and not isinstance(norm, nn.Identity)
+    gamma = getattr(norm, "weight", None) if has_norm else None
+    beta = getattr(norm, "bias", None) if has_norm else None
+    wb = [l.weight for l in layers] + [l.bias for l in layers]
+    return _FusedMlpFn.apply(mod, cd, norm if has_norm else None, out_dtype, x, res, gamma, beta, *wb)

@@ -129,7 +129,8 @@ class FLARE(nn.Module):
         q = self.latent_q.view(self.num_heads, self.num_latents, self.head_dim)
         cd = self._fusable(x, return_scores)
         D = self.head_dim
-        narrow = (cd is not None and D in (4, 8) and self.num_latents % 32 == 0 and not self.qk_norm
+        # (head-padded rows have no backward: with gradients enabled the generic fused branch pads inside the mixer)
+        narrow = (cd is not None and not torch.is_grad_enabled() and D in (4, 8) and self.num_latents % 32 == 0 and not self.qk_norm
                   # head-padded rows exist for the chain of square layers only: an expanding two-layer k/v projection
                   # takes the generic fused branch below, where the mixer pads the heads itself
                   and not fused._expand_factor(self.k_proj, C) and not fused._expand_factor(self.v_proj, C))
@@ -149,8 +150,9 @@ class FLARE(nn.Module):
             if self.qk_norm:
                 q = self.q_norm(q)
                 k = self.k_norm(k)
-            else:
+            elif not torch.is_grad_enabled():
                 q = self._cached_q(cd, 0)
+            # (with gradients enabled q stays the parameter's view: the mixer casts it itself and differentiates it)
             y = flare_multihead_mixer(q, k, v, scale=self.attn_scale, token_major_out=True)
             y = y.permute(0, 2, 1, 3).reshape(B, N, C)
             out_dtype = _res.dtype if _res is not None else x.dtype

@@ -311,6 +311,28 @@ int flare_mlp_io_fwd(const FlareMlpDesc* desc, int32_t in_dim, int32_t in_act, c
                      const float* b_in, int32_t out_dim, const void* x, const void* w, const float* bias,
                      const float* gamma, const float* beta, const void* res, void* y, void* stream);
 
+/* Backward of flare_mlp_fwd for the chain of C x C layers (desc->flags == 0; at most 8 layers, 5 at C = 128): what
+ * torch autograd computes for  y = res + ResidualMLP(norm(x))  (pdebench/models/flare.py:45-59, 204-215) when
+ * the reference trains a block.  One token-parallel launch recomputes the forward and walks the chain back;
+ * reductions over all tokens are left to the caller as library products:
+ *   dx      [T,C]   contiguous, x's dtype: gradient of x (plus dy when add_dy != 0: the forward's res was x itself;
+ *                   otherwise the gradient of res is dy)
+ *   a_in    [L,T,C] the input of every layer and
+ *   g_out   [L,T,C] the gradient at every layer's product, both in the weights' type:
+ *                   dW_l = g_out[l]^T a_in[l],  db_l = column sums of g_out[l]
+ *   dn      [T,C]   (norm only) gradient at the norm's output, weights' type;  stats [T,2] fp32 mean and 1/std
+ *   gb_part [rows,2,C] fp32 (norm only; rows from flare_mlp_bwd_partial_rows): dgamma = sum over rows of
+ *                   gb_part[:,0,:], dbeta = sum of gb_part[:,1,:] (fixed order: no atomics)
+ * dy has desc->y_dtype and row stride desc->y_stride.  w_img, wt_img [L,C,C]: the weights and their transposes as
+ * the kernel's LDS images: element (row, col) of a tile sits at 16-bit position
+ *   row * C + 8 * (((4 * (ch / 4) + 2 * (ch % 2) + (j / 4)) ^ key)) + 4 * ((ch % 4) / 2) + j % 4,
+ *   ch = col / 8, j = col % 8, key = (row % 16) >> (C == 128 ? 0 : C == 64 ? 1 : 2)
+ * (flare.py_amd/fused.py::mlp_weight_image builds them). */
+int flare_mlp_bwd_partial_rows(const FlareMlpDesc* desc, int32_t* rows);
+int flare_mlp_bwd(const FlareMlpDesc* desc, const void* x, const void* dy, const void* w_img, const void* wt_img,
+                  const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* a_in,
+                  void* g_out, void* dn, float* stats, float* gb_part, void* stream);
+
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes);
 
 /* state only (split-N partial sums + fixed-order merge; no atomics). */
