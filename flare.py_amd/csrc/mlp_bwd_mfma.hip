@@ -354,29 +354,65 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
     }
 }
 
-// dgamma[c] = sum_t ds_0[t,c] xhat[t,c],  dbeta[c] = sum_t ds_0[t,c]  over the workgroup's token range: thread = channel
-// (C <= 128 of the 128 threads), rows read coalesced, one partial row pair per workgroup.
+// dgamma[c] = sum_t ds_0[t,c] xhat[t,c],  dbeta[c] = sum_t ds_0[t,c]  over the workgroup's token range.  Thread =
+// (channel pair, token lane): 256 threads cover C / 2 channel pairs x 512 / C token lanes, every lane walks its
+// tokens four at a time (all loads of a group in flight together), the lanes meet in LDS at the end.  Rows are read
+// coalesced (4 bytes of ds_0 and 8 bytes of x per thread); one partial row pair per workgroup.
 template <typename T>
-__global__ __launch_bounds__(128) void mlp_norm_grads_kernel(MlpBwdArgs a, int64_t tokens_per_wg)
+__global__ __launch_bounds__(256) void mlp_norm_grads_kernel(MlpBwdArgs a, int64_t tokens_per_wg)
 {
     using M_ = Mw<T>;
-    const int c = threadIdx.x;
+    __shared__ float red[2][256][2];
+    const int pairs = a.C / 2, lanes = 256 / pairs;             // 16 x 16, 32 x 8 or 64 x 4
+    const int cp = threadIdx.x % pairs, tl = threadIdx.x / pairs;
     const int64_t t0 = (int64_t)blockIdx.x * tokens_per_wg, t1 = t0 + tokens_per_wg < a.T ? t0 + tokens_per_wg : a.T;
-    float gs = 0.f, bs = 0.f;
-    if (c < a.C) {
-        for (int64_t t = t0; t < t1; ++t) {
-            const float2 st = *reinterpret_cast<const float2*>(a.stats + 2 * t);
-            const int64_t e = t * a.xs + c;
-            const float xv = a.x_dtype == 0 ? static_cast<const float*>(a.x)[e]
-                           : a.x_dtype == 1 ? __uint_as_float(uint32_t(static_cast<const uint16_t*>(a.x)[e]) << 16)
-                                            : (float)static_cast<const _Float16*>(a.x)[e];
-            const uint32_t raw = a.dn[(size_t)t * a.C + c];
-            const float dv = M_::lo(raw);
-            gs = fmaf(dv, (xv - st.x) * st.y, gs);
-            bs += dv;
+    float gs0 = 0.f, gs1 = 0.f, bs0 = 0.f, bs1 = 0.f;
+    auto xval = [&](int64_t t, float& x0, float& x1) {
+        const int64_t e = t * a.xs + 2 * cp;
+        if (a.x_dtype == 0) {
+            const float2 v = *reinterpret_cast<const float2*>(static_cast<const float*>(a.x) + e);
+            x0 = v.x; x1 = v.y;
+        } else {
+            const uint32_t v = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.x) + e);
+            if (a.x_dtype == 1) { x0 = __uint_as_float(v << 16); x1 = __uint_as_float(v & 0xffff0000u); }
+            else { x0 = Mw<f16_t>::lo(v); x1 = Mw<f16_t>::hi(v); }
         }
-        a.gb_part[((size_t)blockIdx.x * 2 + 0) * a.C + c] = gs;
-        a.gb_part[((size_t)blockIdx.x * 2 + 1) * a.C + c] = bs;
+    };
+    for (int64_t t = t0 + tl; t < t1; t += 4 * lanes) {
+        float x0[4], x1[4];
+        float2 st[4];
+        uint32_t dv[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t tt = t + u * lanes < t1 ? t + u * lanes : t1 - 1;
+            st[u] = *reinterpret_cast<const float2*>(a.stats + 2 * tt);
+            xval(tt, x0[u], x1[u]);
+            dv[u] = *reinterpret_cast<const uint32_t*>(a.dn + (size_t)tt * a.C + 2 * cp);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (t + u * lanes >= t1) continue;
+            const float d0 = M_::lo(dv[u]), d1 = M_::hi(dv[u]);
+            gs0 = fmaf(d0, (x0[u] - st[u].x) * st[u].y, gs0);
+            gs1 = fmaf(d1, (x1[u] - st[u].x) * st[u].y, gs1);
+            bs0 += d0;
+            bs1 += d1;
+        }
+    }
+    red[0][threadIdx.x][0] = gs0; red[0][threadIdx.x][1] = gs1;
+    red[1][threadIdx.x][0] = bs0; red[1][threadIdx.x][1] = bs1;
+    __syncthreads();
+    if (threadIdx.x < pairs) {
+        float s[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+        for (int l = 0; l < lanes; ++l)
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                s[k][0] += red[k][l * pairs + cp][0];
+                s[k][1] += red[k][l * pairs + cp][1];
+            }
+#pragma unroll
+        for (int k = 0; k < 2; ++k)
+            *reinterpret_cast<float2*>(a.gb_part + ((size_t)blockIdx.x * 2 + k) * a.C + 2 * cp) = make_float2(s[k][0], s[k][1]);
     }
 }
 
@@ -402,7 +438,7 @@ hipError_t launch_l(const MlpBwdArgs& a, hipStream_t st)
     if (e != hipSuccess || a.norm == 0) return e;
     const int rows = mlp_bwd_partial_rows(a.T);
     const int64_t tpw = (a.T + rows - 1) / rows;
-    hipLaunchKernelGGL(mlp_norm_grads_kernel<T>, dim3(rows), dim3(128), 0, st, a, tpw);
+    hipLaunchKernelGGL(mlp_norm_grads_kernel<T>, dim3(rows), dim3(256), 0, st, a, tpw);
     return hipGetLastError();
 }
 
@@ -432,10 +468,10 @@ hipError_t launch_t(const MlpBwdArgs& a, hipStream_t st)
 int mlp_bwd_max_layers(int C) { return C == 128 ? 5 : 8; }
 
 // partial rows of dgamma, dbeta a launch writes (one per workgroup of the reduction over tokens: token ranges of at
-// least 256 tokens, at most two workgroups per compute unit)
+// least 256 tokens, at most four workgroups per compute unit)
 int mlp_bwd_partial_rows(int64_t T)
 {
-    const int64_t want = (T + 255) / 256, cap = 2 * (int64_t)device_cus();
+    const int64_t want = (T + 255) / 256, cap = 4 * (int64_t)device_cus();
     return (int)(want < cap ? (want < 1 ? 1 : want) : cap);
 }
 

@@ -345,6 +345,26 @@ def _packed_train(mod, layers, cd):
     return w, b, w_img, wt_img
 
 
+_DW_CHUNK = 4096      # tokens per partial product of the weight gradients
+
+
+def _weight_grads(g_out, a_in):
+    """dW[l] = g_out[l]^T a_in[l] over T tokens, [L, C, C] fp32.  The contraction is as long as the token axis and the
+    result is tiny, so it is split into chunks of _DW_CHUNK tokens that run as one batched product (the library then
+    has L * T / chunk independent problems instead of L with nothing to parallelise), and the partial results are
+    summed in fp32 in a fixed order."""
+    L, T, Cdim = g_out.shape
+    n = T // _DW_CHUNK
+    parts = []
+    if n > 0:
+        gm = g_out[:, :n * _DW_CHUNK].reshape(L * n, _DW_CHUNK, Cdim)
+        am = a_in[:, :n * _DW_CHUNK].reshape(L * n, _DW_CHUNK, Cdim)
+        parts.append(torch.bmm(gm.transpose(1, 2), am).view(L, n, Cdim, Cdim).sum(dim=1, dtype=torch.float32))
+    if n * _DW_CHUNK < T:
+        parts.append(torch.bmm(g_out[:, n * _DW_CHUNK:].transpose(1, 2), a_in[:, n * _DW_CHUNK:]).float())
+    return parts[0] if len(parts) == 1 else parts[0] + parts[1]
+
+
 class _FusedMlpFn(torch.autograd.Function):
     """y = res + chain(norm(x)); parameters are passed as inputs so that autograd routes their gradients:
     (x, res, gamma, beta, w_0 .. w_{L-1}, b_0 .. b_{L-1}) with None where a tensor does not exist."""
@@ -403,7 +423,7 @@ class _FusedMlpFn(torch.autograd.Function):
         _lib.check(rc, "flare_mlp_bwd")
         # parameter gradients: two batched products over the rows the kernel left (16-bit products with fp32
         # accumulation, as torch runs a Linear's backward under autocast), sums in a fixed order
-        dW = torch.bmm(g_out.transpose(1, 2), a_in)                      # [L, out, in]
+        dW = _weight_grads(g_out, a_in)                                  # [L, out, in] fp32
         db = g_out.sum(dim=1, dtype=torch.float32)                       # [L, C]
         need = ctx.needs_input_grad            # (mod, cd, norm, out_dtype, x, res, gamma, beta, *wb)
         grads = [None, None, None, None]
