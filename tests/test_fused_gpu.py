@@ -125,10 +125,11 @@ def test_block_fused_path_vs_torch_layers(dev, C, H, M, rms, monkeypatch):
     assert len(calls) == 4
     assert y.dtype == torch.float32
     assert O.rel_l2(y, ref) <= 2e-2
-    # gradients still flow through the torch layers when they are needed
+    # with gradients enabled the same four launches run behind autograd (tests/test_fused_train_gpu.py holds their
+    # backward to the torch layers)
     with torch.autocast("cuda", dtype=torch.bfloat16):
         yt, _ = blk(x[:, :256])
-    assert len(calls) == 4 and yt.requires_grad
+    assert len(calls) == 8 and yt.requires_grad
 
 
 def test_narrow_heads_with_expanding_kv_projection(dev):

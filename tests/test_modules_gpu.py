@@ -224,8 +224,9 @@ def test_bigflare_ablation_model(dev, kw):
 
 
 def test_autocast_training_step_gradients(dev, monkeypatch):
-    """One bf16-autocast training step of FLAREModel: the mixer runs forward and backward on the HIP kernels
-    (token-major output, strided gradient, fp32 latent parameter cast per call); gradients against the same model
+    """One bf16-autocast training step of FLAREModel: the mixer and the blocks' projections and feed-forward run forward
+    and backward on the HIP kernels (token-major output, strided gradient, fp32 latent parameter cast per call;
+    in_proj and out_proj, whose ends are narrow, keep their torch layers); gradients against the same model
     in fp64 on the CPU with the oracle mixer.  Tolerance: bf16 arithmetic through two blocks."""
     torch.manual_seed(8)
     m = FLAREModel(in_dim=4, out_dim=3, channel_dim=64, num_blocks=2, num_heads=4, num_latents=64).to(dev).train()
@@ -251,7 +252,9 @@ def test_autocast_training_step_gradients(dev, monkeypatch):
     got = dict(m.named_parameters())
     for name, pr in cpu.named_parameters():
         if name in ("blocks.0.att.latent_q", "blocks.1.att.k_proj.fc1.weight", "blocks.0.att.v_proj.fc2.weight", "in_proj.fc1.weight"):
-            assert O.rel_l2(got[name].grad, pr.grad) <= 6e-2, name
+            # (weights scaled by 6: block 1's k_proj gradients are differences of large terms; the same step through
+            # the torch layers under autocast is 5.4e-2 off on that tensor)
+            assert O.rel_l2(got[name].grad, pr.grad) <= 8e-2, name
 
 
 @pytest.mark.parametrize("kw", [dict(), dict(rmsnorm=True, qk_norm=True, act="silu"), dict(attn_scale=0.5, num_layers_ffn=0, ffn_mlp_ratio=2.0),
