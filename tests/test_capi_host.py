@@ -181,3 +181,87 @@ def test_new_struct_sizes_and_entry_point_validation():
     assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=48, D=32), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
     assert lib.flare_mixer_bwd(d, *([None] * 8), None, None, None, None, None, 0, None) == _lib.FLARE_EINVAL
     assert lib.flare_scatter_fwd_lse(d, None, None, None, None, None, None, None) == _lib.FLARE_EINVAL
+
+
+@pytest.mark.parametrize("Cdim", [32, 64, 128])
+def test_mlp_weight_image_follows_the_header_formula(Cdim):
+    """fused.mlp_weight_image against include/flare_hip.h's position formula, element by element in plain loops:
+    the image is a permutation inside each row, and a 16-byte piece holds four columns of one 8-column block and the
+    same four of the block two further on."""
+    from flare_py_amd import fused
+    shift = {128: 0, 64: 1, 32: 2}[Cdim]
+    w = torch.arange(2 * Cdim * Cdim, dtype=torch.float32).view(2, Cdim, Cdim)
+    img = fused.mlp_weight_image(w).view(2, Cdim * Cdim)
+    seen = set()
+    for row in range(Cdim):
+        for col in range(Cdim):
+            ch, j = col // 8, col % 8
+            key = (row % 16) >> shift
+            pos = row * Cdim + 8 * ((4 * (ch // 4) + 2 * (ch % 2) + j // 4) ^ key) + 4 * ((ch % 4) // 2) + j % 4
+            assert pos // Cdim == row and pos not in seen
+            seen.add(pos)
+            for l in range(2):
+                assert img[l, pos] == w[l, row, col]
+    assert len(seen) == Cdim * Cdim
+    piece = img[0].view(Cdim, Cdim // 8, 8)[5].long() - 5 * Cdim          # columns held by row 5's pieces
+    for p in piece:
+        lo, hi = p[:4].tolist(), p[4:].tolist()
+        assert lo == list(range(lo[0], lo[0] + 4)) and lo[0] % 4 == 0
+        assert hi == [c + 16 for c in lo]
+
+
+def test_mlp_bwd_validation():
+    lib = _lib.load()
+    m = _lib.FlareMlpDesc()
+    m.T, m.C, m.L = 64, 128, 2
+    m.x_dtype = m.y_dtype = m.w_dtype = _lib.DT_BF16
+    m.norm, m.act, m.eps = 1, 0, 1e-5      # layer norm, tanh gelu
+    m.x_stride = m.y_stride = 128
+    fake = C.c_void_p(4096)
+    odd = C.c_void_p(4100)
+    ff = fake
+    rows = C.c_int32(0)
+    assert lib.flare_mlp_bwd_partial_rows(m, C.byref(rows)) == _lib.FLARE_OK and rows.value == 1
+    m.T = 1 << 20
+    assert lib.flare_mlp_bwd_partial_rows(m, C.byref(rows)) == _lib.FLARE_OK and 1 <= rows.value <= 4096
+    big = rows.value
+    m.T = 1 << 22
+    assert lib.flare_mlp_bwd_partial_rows(m, C.byref(rows)) == _lib.FLARE_OK and rows.value == big     # capped by the CU count
+    assert lib.flare_mlp_bwd_partial_rows(m, None) == _lib.FLARE_EINVAL
+    m.T = 64
+
+    def call(x=fake, dy=fake, gamma=ff, dn=fake, stats=ff, gb=ff):
+        return lib.flare_mlp_bwd(m, x, dy, fake, fake, ff, gamma, ff, 0, fake, fake, fake, dn, stats, gb, None)
+
+    assert lib.flare_mlp_bwd(None, *([None] * 7), 0, *([None] * 7)) == _lib.FLARE_EINVAL
+    assert call(x=None) == _lib.FLARE_EINVAL and "must not be NULL" in _lib.last_error()
+    assert call(gamma=None) == _lib.FLARE_EINVAL and "norm" in _lib.last_error()
+    assert call(gb=None) == _lib.FLARE_EINVAL and "norm" in _lib.last_error()
+    assert call(x=odd) == _lib.FLARE_EINVAL and "16-byte" in _lib.last_error()
+    assert call(dn=odd) == _lib.FLARE_EINVAL and "16-byte" in _lib.last_error()
+    m.L = 6
+    assert call() == _lib.FLARE_EUNSUPPORTED and "at most 5 layers" in _lib.last_error()
+    m.C = 64
+    m.x_stride = 62
+    assert call() == _lib.FLARE_EINVAL and "row stride" in _lib.last_error()
+    m.x_stride = 64
+    m.y_stride = 66
+    assert call() == _lib.FLARE_EINVAL and "y_stride" in _lib.last_error()
+    m.y_stride = 64
+    m.L = 9
+    assert call() == _lib.FLARE_EUNSUPPORTED and "at most 8 layers" in _lib.last_error()
+    m.L = 2
+    m.C = 48
+    assert call() == _lib.FLARE_EUNSUPPORTED and "32, 64 and 128" in _lib.last_error()
+    m.C = 128
+    m.x_stride = m.y_stride = 128
+    m.flags = _lib.MLP_EXPAND
+    assert call() == _lib.FLARE_EUNSUPPORTED and "flags must be 0" in _lib.last_error()
+    m.flags = 0
+    m.w_dtype = _lib.DT_F32
+    assert call() == _lib.FLARE_EINVAL and "w_dtype" in _lib.last_error()
+    m.w_dtype = _lib.DT_BF16
+    m.act = 7
+    assert call() == _lib.FLARE_EINVAL and "activation" in _lib.last_error()
+    m.act, m.eps = 0, -1.0
+    assert call() == _lib.FLARE_EINVAL and "eps" in _lib.last_error()
