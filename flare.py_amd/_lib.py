@@ -98,7 +98,7 @@ SYMBOLS = {
     "flare_mlp_io_fwd": (C.c_int, [C.POINTER(FlareMlpDesc), C.c_int32, C.c_int32, _P, _P, C.c_int32,
                                    _P, _P, _P, _P, _P, _P, _P, _P]),
     "flare_mlp_bwd_partial_rows": (C.c_int, [C.POINTER(FlareMlpDesc), C.POINTER(C.c_int32)]),
-    "flare_mlp_bwd": (C.c_int, [C.POINTER(FlareMlpDesc), _P, _P, _P, _P, _P, _P, _P, C.c_int32, _P, _P, _P, _P, _P, _P, _P]),
+    "flare_mlp_bwd": (C.c_int, [C.POINTER(FlareMlpDesc), _P, _P, _P, _P, _P, _P, _P, C.c_int32, _P, _P, _P, _P, _P, _P, _P, _P]),
     "flare_triple_workspace_bytes": (C.c_int, [C.POINTER(FlareTripleDesc), C.POINTER(_SZ)]),
     "flare_triple_state_fwd": (C.c_int, [C.POINTER(FlareTripleDesc), _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_triple_out_fwd": (C.c_int, [C.POINTER(FlareTripleDesc), _P, _P, _P, _P, _P, _P]),

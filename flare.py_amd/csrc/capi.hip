@@ -819,7 +819,7 @@ int flare_mlp_bwd_partial_rows(const FlareMlpDesc* d, int32_t* rows)
 
 int flare_mlp_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const void* w_img, const void* wt_img,
                   const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* a_in,
-                  void* g_out, void* dn, float* stats, float* gb_part, void* stream)
+                  void* g_out, void* dn, float* stats, float* gb_part, float* db_part, void* stream)
 {
     if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
     if (d->T < 1 || d->L < 1) return fail(FLARE_EINVAL, "T >= 1 and L >= 1 required (got %lld, %d)", (long long)d->T, d->L);
@@ -849,7 +849,7 @@ int flare_mlp_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const vo
     a.w = static_cast<const uint16_t*>(w_img); a.wt = static_cast<const uint16_t*>(wt_img);
     a.bias = bias; a.gamma = gamma; a.beta = beta;
     a.a_in = static_cast<uint16_t*>(a_in); a.g_out = static_cast<uint16_t*>(g_out);
-    a.dn = static_cast<uint16_t*>(dn); a.stats = stats; a.gb_part = gb_part;
+    a.dn = static_cast<uint16_t*>(dn); a.stats = stats; a.gb_part = gb_part; a.db_part = db_part;
     a.T = d->T; a.C = d->C; a.L = d->L;
     a.x_dtype = d->x_dtype; a.dy_dtype = d->y_dtype; a.dx_dtype = d->x_dtype;
     a.norm = d->norm; a.eps = d->eps; a.act = d->act; a.act_mask = d->act_mask; a.add_mask = d->add_mask;

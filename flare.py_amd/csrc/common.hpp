@@ -201,6 +201,7 @@ struct MlpBwdArgs {
     uint16_t* dn;                               // [T,C] out (norm != 0): ds_0, the gradient at the norm's output, same type
     float* stats;                               // [T,2] out (norm != 0): mean and 1/std of every token
     float* gb_part;                             // [rows,2,C] out (norm != 0): partial sums of dgamma, dbeta over token ranges
+    float* db_part;                             // [rows,L,C] out or null: partial column sums of g_out (the bias gradients)
     int64_t T;
     int C, L;
     int x_dtype, dy_dtype, dx_dtype;            // 0 f32, 1 bf16, 2 f16

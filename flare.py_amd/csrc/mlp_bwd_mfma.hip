@@ -416,6 +416,47 @@ __global__ __launch_bounds__(256) void mlp_norm_grads_kernel(MlpBwdArgs a, int64
     }
 }
 
+// db_l[c] = sum_t g_out[l,t,c] over the workgroup's token range (blockIdx.y = layer).  Thread = (piece of eight
+// channels, token lane): 256 threads cover C / 8 pieces x 2048 / C token lanes, 16 bytes per load, four tokens per
+// lane in flight; the lanes meet in LDS.  One partial row per workgroup and layer.
+template <typename T>
+__global__ __launch_bounds__(256) void mlp_bias_grads_kernel(MlpBwdArgs a, int64_t tokens_per_wg)
+{
+    using M_ = Mw<T>;
+    __shared__ float red[256][8];
+    const int pieces = a.C / 8, lanes = 256 / pieces;           // 4 x 64, 8 x 32 or 16 x 16
+    const int pc = threadIdx.x % pieces, tl = threadIdx.x / pieces, l = blockIdx.y;
+    const int64_t t0 = (int64_t)blockIdx.x * tokens_per_wg, t1 = t0 + tokens_per_wg < a.T ? t0 + tokens_per_wg : a.T;
+    const uint16_t* g = a.g_out + (size_t)l * a.T * a.C + 8 * pc;
+    float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int64_t t = t0 + tl; t < t1; t += 4 * lanes) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t tt = t + u * lanes < t1 ? t + u * lanes : t1 - 1;
+            v[u] = *reinterpret_cast<const u32x4*>(g + (size_t)tt * a.C);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            if (t + u * lanes >= t1) continue;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                s[2 * k] += M_::lo(v[u][k]);
+                s[2 * k + 1] += M_::hi(v[u][k]);
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) red[threadIdx.x][k] = s[k];
+    __syncthreads();
+    if ((int)threadIdx.x < a.C) {
+        const int c = threadIdx.x;
+        float r = 0.f;
+        for (int q = 0; q < lanes; ++q) r += red[q * pieces + c / 8][c % 8];
+        a.db_part[((size_t)blockIdx.x * a.L + l) * a.C + c] = r;
+    }
+}
+
 template <typename T, int C, int WAVES, int LMAX>
 hipError_t launch_l(const MlpBwdArgs& a, hipStream_t st)
 {
@@ -435,9 +476,14 @@ hipError_t launch_l(const MlpBwdArgs& a, hipStream_t st)
     const int64_t cus = device_cus();
     hipLaunchKernelGGL(kern, dim3((unsigned)(nblk < cus ? nblk : cus)), dim3(64 * WAVES), lds, st, a, resident);
     e = hipGetLastError();
-    if (e != hipSuccess || a.norm == 0) return e;
+    if (e != hipSuccess) return e;
     const int rows = mlp_bwd_partial_rows(a.T);
     const int64_t tpw = (a.T + rows - 1) / rows;
+    if (a.db_part) {
+        hipLaunchKernelGGL(mlp_bias_grads_kernel<T>, dim3(rows, a.L), dim3(256), 0, st, a, tpw);
+        e = hipGetLastError();
+    }
+    if (e != hipSuccess || a.norm == 0) return e;
     hipLaunchKernelGGL(mlp_norm_grads_kernel<T>, dim3(rows), dim3(256), 0, st, a, tpw);
     return hipGetLastError();
 }

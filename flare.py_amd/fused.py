@@ -409,22 +409,26 @@ class _FusedMlpFn(torch.autograd.Function):
         dx = torch.empty(T, Cdim, dtype=x2.dtype, device=dev)
         a_in = torch.empty(L, T, Cdim, dtype=cd, device=dev)
         g_out = torch.empty(L, T, Cdim, dtype=cd, device=dev)
-        dn = stats = gb = None
+        dn = stats = gb = dbp = None
+        any_bias = any(l.bias is not None for l in layers)
+        rows = C.c_int32(0)
+        _lib.check(lib.flare_mlp_bwd_partial_rows(C.byref(d), C.byref(rows)), "flare_mlp_bwd_partial_rows")
+        if any_bias:
+            dbp = torch.empty(rows.value, L, Cdim, dtype=torch.float32, device=dev)
         if d.norm:
-            rows = C.c_int32(0)
-            _lib.check(lib.flare_mlp_bwd_partial_rows(C.byref(d), C.byref(rows)), "flare_mlp_bwd_partial_rows")
             dn = torch.empty(T, Cdim, dtype=cd, device=dev)
             stats = torch.empty(T, 2, dtype=torch.float32, device=dev)
             gb = torch.empty(rows.value, 2, Cdim, dtype=torch.float32, device=dev)
         with _on_device(dev):
             rc = lib.flare_mlp_bwd(C.byref(d), _ptr(x2), _ptr(dy2), _ptr(w_img), _ptr(wt_img), _ptr(b), _ptr(gamma), _ptr(beta),
                                    1 if ctx.res_is_x else 0, _ptr(dx), _ptr(a_in), _ptr(g_out), _ptr(dn), _ptr(stats), _ptr(gb),
-                                   C.c_void_p(_stream_ptr(dev)))
+                                   _ptr(dbp), C.c_void_p(_stream_ptr(dev)))
         _lib.check(rc, "flare_mlp_bwd")
-        # parameter gradients: two batched products over the rows the kernel left (16-bit products with fp32
-        # accumulation, as torch runs a Linear's backward under autocast), sums in a fixed order
+        # weight gradients: batched products over the rows the kernel left (16-bit products with fp32 accumulation,
+        # as torch runs a Linear's backward under autocast); bias and norm gradients: the kernels' partial rows,
+        # summed in a fixed order
         dW = _weight_grads(g_out, a_in)                                  # [L, out, in] fp32
-        db = g_out.sum(dim=1, dtype=torch.float32)                       # [L, C]
+        db = dbp.sum(0) if any_bias else None                            # [L, C]
         need = ctx.needs_input_grad            # (mod, cd, norm, out_dtype, x, res, gamma, beta, *wb)
         grads = [None, None, None, None]
         grads.append(dx.view(x.shape) if need[4] else None)

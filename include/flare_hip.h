@@ -323,6 +323,7 @@ int flare_mlp_io_fwd(const FlareMlpDesc* desc, int32_t in_dim, int32_t in_act, c
  *   dn      [T,C]   (norm only) gradient at the norm's output, weights' type;  stats [T,2] fp32 mean and 1/std
  *   gb_part [rows,2,C] fp32 (norm only; rows from flare_mlp_bwd_partial_rows): dgamma = sum over rows of
  *                   gb_part[:,0,:], dbeta = sum of gb_part[:,1,:] (fixed order: no atomics)
+ *   db_part [rows,L,C] fp32 or NULL (same rows): db_l = sum over rows of db_part[:,l,:]; NULL skips that launch
  * dy has desc->y_dtype and row stride desc->y_stride.  w_img, wt_img [L,C,C]: the weights and their transposes as
  * the kernel's LDS images: element (row, col) of a tile sits at 16-bit position
  *   row * C + 8 * (((4 * (ch / 4) + 2 * (ch % 2) + (j / 4)) ^ key)) + 4 * ((ch % 4) / 2) + j % 4,
@@ -331,7 +332,7 @@ int flare_mlp_io_fwd(const FlareMlpDesc* desc, int32_t in_dim, int32_t in_act, c
 int flare_mlp_bwd_partial_rows(const FlareMlpDesc* desc, int32_t* rows);
 int flare_mlp_bwd(const FlareMlpDesc* desc, const void* x, const void* dy, const void* w_img, const void* wt_img,
                   const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* a_in,
-                  void* g_out, void* dn, float* stats, float* gb_part, void* stream);
+                  void* g_out, void* dn, float* stats, float* gb_part, float* db_part, void* stream);
 
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes);
 

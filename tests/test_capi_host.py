@@ -231,9 +231,9 @@ def test_mlp_bwd_validation():
     m.T = 64
 
     def call(x=fake, dy=fake, gamma=ff, dn=fake, stats=ff, gb=ff):
-        return lib.flare_mlp_bwd(m, x, dy, fake, fake, ff, gamma, ff, 0, fake, fake, fake, dn, stats, gb, None)
+        return lib.flare_mlp_bwd(m, x, dy, fake, fake, ff, gamma, ff, 0, fake, fake, fake, dn, stats, gb, None, None)
 
-    assert lib.flare_mlp_bwd(None, *([None] * 7), 0, *([None] * 7)) == _lib.FLARE_EINVAL
+    assert lib.flare_mlp_bwd(None, *([None] * 7), 0, *([None] * 8)) == _lib.FLARE_EINVAL
     assert call(x=None) == _lib.FLARE_EINVAL and "must not be NULL" in _lib.last_error()
     assert call(gamma=None) == _lib.FLARE_EINVAL and "norm" in _lib.last_error()
     assert call(gb=None) == _lib.FLARE_EINVAL and "norm" in _lib.last_error()
