@@ -95,6 +95,18 @@ __device__ __forceinline__ float tok_sum(float v)   // sum over the 4 lane group
     return v;
 }
 
+// A packed operand quad {lo01, lo23, hi01, hi23} holds channels 4g..4g+3 of two feature tiles 16 channels apart.
+// Lanes 16 apart (g and g ^ 1) exchange halves, after which every lane holds eight consecutive channels: those
+// starting at row_col(g) = 0, 16, 8, 24 for g = 0..3.  A token's row then leaves as 16-byte pieces, 64 contiguous
+// bytes per store instruction, instead of 8-byte pieces that cover 32.  All lanes of the wave must be active.
+__device__ __forceinline__ u32x4 row_piece(u32x4 q)
+{
+    const auto r0 = __builtin_amdgcn_permlane16_swap(q[0], q[2], false, false);
+    const auto r1 = __builtin_amdgcn_permlane16_swap(q[1], q[3], false, false);
+    return u32x4{r0[0], r1[0], r0[1], r1[1]};
+}
+__device__ __forceinline__ int row_col(int g) { return (g & 1) ? 12 + 4 * g : 4 * g; }
+
 // act(t) = t * gate and its derivative.  tanh-GELU: gate = sigmoid(2u), 2u = t (1.5957691 + 0.0713548 t^2), so
 // act' = gate (1 + t (1 - gate) (1.5957691 + 0.2140645 t^2));  SiLU: gate = sigmoid(t), act' = gate (1 + t (1 - gate)).
 template <int ACT>
@@ -127,20 +139,39 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
     using M_ = Mw<T>;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
-    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    // bias rows of every layer, then gamma and beta, as fp32 in LDS: read from there the values cost no vector-memory
+    // slot (a global load in the middle of a step would queue behind the weight tile requested at its start)
+    __shared__ __attribute__((aligned(16))) float pvec[(LMAX + 2) * C];
+
+    const int tid = threadIdx.x, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);       // the wave number, known to be uniform
     const int L = a.L;
+    for (int i = tid; i < (LMAX + 2) * C; i += NT) {
+        const int row = i / C, c = i % C;
+        float v = 0.f;
+        if (row < LMAX) { if (a.bias && row < L) v = a.bias[(size_t)row * C + c]; }
+        else if (row == LMAX) { if (a.norm != 0) v = a.gamma[c]; }
+        else if (a.norm != 0 && a.beta) v = a.beta[c];
+        pvec[i] = v;
+    }
 
     // Weight tile of ring step q: W_q for q < L (forward), W_{2L-1-q}^T after that (backward).  The caller hands
     // the tiles over as LDS images (the 16-bit elements already in the order the A-operand reads expect, see
     // mlp_weight_image in the host code), so a tile goes from global memory straight into its slot, 16 bytes per
     // lane, with no registers and no LDS stores in between.
     auto stage = [&](int q, int slot) {
-        const uint16_t* img = q < L ? a.w + (size_t)q * C * C : a.wt + (size_t)(2 * L - 1 - q) * C * C;
+        const uint8_t* img = reinterpret_cast<const uint8_t*>(q < L ? a.w + (size_t)q * C * C : a.wt + (size_t)(2 * L - 1 - q) * C * C);
+        // The lane's byte offset passes through an empty asm statement so that the 64-bit address of each (tile,
+        // chunk) is formed here, with one add, and not ahead of the token loop: kept across the loop those addresses
+        // would be 8 * L * NCH registers that end up in scratch memory, and each reload from there waits for every
+        // vector-memory operation in flight, the previous chunk's load included.
+        uint32_t loff = lane * 16;
+        asm volatile("" : "+v"(loff));
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             const int c0 = i * NT + w * 64;           // first 16-byte chunk of this wave's share (uniform over the wave)
-            if (c0 < C * C / 8)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(img + (size_t)(c0 + lane) * 8),
+            if ((C * C / 8) % NT == 0 || c0 < C * C / 8)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(img + (size_t)c0 * 16 + loff),
                                                  (__attribute__((address_space(3))) void*)(smem + slot * WBUF + c0 * 16), 16, 0, 0);
         }
     };
@@ -200,9 +231,8 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
             rstd = rsqrtf(tok_sum(ss) * (1.f / C) + a.eps);
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
-                const f32x4 gm = *reinterpret_cast<const f32x4*>(a.gamma + 16 * ft + 4 * g);
-                f32x4 bt = {0.f, 0.f, 0.f, 0.f};
-                if (a.beta) bt = *reinterpret_cast<const f32x4*>(a.beta + 16 * ft + 4 * g);
+                const f32x4 gm = *reinterpret_cast<const f32x4*>(pvec + LMAX * C + 16 * ft + 4 * g);
+                const f32x4 bt = *reinterpret_cast<const f32x4*>(pvec + (LMAX + 1) * C + 16 * ft + 4 * g);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) xs[ft][r] = (xs[ft][r] - mean) * rstd * gm[r] + bt[r];
             }
@@ -219,12 +249,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
                 const f32x4 lo = xs[2 * ks], hi = xs[2 * ks + 1];
                 xb[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
             }
-            if (live) {       // s_l, the input of layer l, as a 16-bit row (for dW_l)
-                uint16_t* row = a.a_in + ((size_t)l * a.T + tok) * C + 4 * g;
+            {                 // s_l, the input of layer l, as a 16-bit row (for dW_l)
+                u32x4 piece[KS];
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    *reinterpret_cast<uint2*>(row + 32 * ks) = make_uint2(xb[ks][0], xb[ks][1]);
-                    *reinterpret_cast<uint2*>(row + 32 * ks + 16) = make_uint2(xb[ks][2], xb[ks][3]);
+                for (int ks = 0; ks < KS; ++ks) piece[ks] = row_piece(xb[ks]);
+                if (live) {
+                    uint16_t* row = a.a_in + ((size_t)l * a.T + tok) * C + row_col(g);
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<u32x4*>(row + 32 * ks) = piece[ks];
                 }
             }
             const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
@@ -233,8 +265,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
                 constexpr bool ADD = decltype(add_c)::value;
 #pragma unroll
                 for (int ft = 0; ft < FT; ++ft) {
-                    f32x4 acc = a.bias ? *reinterpret_cast<const f32x4*>(a.bias + (size_t)l * C + 16 * ft + 4 * g)
-                                       : f32x4{0.f, 0.f, 0.f, 0.f};
+                    f32x4 acc = *reinterpret_cast<const f32x4*>(pvec + l * C + 16 * ft + 4 * g);
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks)
                         acc = M_::mma(*reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]), xb[ks], acc);
@@ -290,12 +321,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
                 }
                 db[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
             }
-            if (live) {
-                uint16_t* row = a.g_out + ((size_t)l * a.T + tok) * C + 4 * g;
+            {
+                u32x4 piece[KS];
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    *reinterpret_cast<uint2*>(row + 32 * ks) = make_uint2(db[ks][0], db[ks][1]);
-                    *reinterpret_cast<uint2*>(row + 32 * ks + 16) = make_uint2(db[ks][2], db[ks][3]);
+                for (int ks = 0; ks < KS; ++ks) piece[ks] = row_piece(db[ks]);
+                if (live) {
+                    uint16_t* row = a.g_out + ((size_t)l * a.T + tok) * C + row_col(g);
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<u32x4*>(row + 32 * ks) = piece[ks];
                 }
             }
             // ds_l = (ds_{l+1} if the layer added to the stream) + W_l^T dt_l
@@ -315,18 +348,23 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
         if (a.norm != 0) {
             // ds_0 and the token's statistics go out for dgamma, dbeta; xhat is taken again from x (the row is still
             // in cache) rather than kept in registers;  g = ds_0 * gamma
-            if (live) {
-                uint16_t* row = a.dn + (size_t)tok * C + 4 * g;
+            u32x4 piece[KS];
 #pragma unroll
-                for (int ft = 0; ft < FT; ++ft)
-                    *reinterpret_cast<uint2*>(row + 16 * ft) = make_uint2(M_::pack2(xs[ft][0], xs[ft][1]), M_::pack2(xs[ft][2], xs[ft][3]));
+            for (int ks = 0; ks < KS; ++ks) {
+                const f32x4 lo = xs[2 * ks], hi = xs[2 * ks + 1];
+                piece[ks] = row_piece(u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])});
+            }
+            if (live) {
+                uint16_t* row = a.dn + (size_t)tok * C + row_col(g);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<u32x4*>(row + 32 * ks) = piece[ks];
                 if (lane < 16) *reinterpret_cast<float2*>(a.stats + 2 * tok) = make_float2(mean, rstd);
             }
             float m1 = 0.f, m2 = 0.f;
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
                 const f32x4 xr = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
-                const f32x4 gm = *reinterpret_cast<const f32x4*>(a.gamma + 16 * ft + 4 * g);
+                const f32x4 gm = *reinterpret_cast<const f32x4*>(pvec + LMAX * C + 16 * ft + 4 * g);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     xs[ft][r] *= gm[r];
@@ -462,7 +500,8 @@ hipError_t launch_l(const MlpBwdArgs& a, hipStream_t st)
 {
     auto kern = mlp_bwd_kernel<T, C, WAVES, LMAX>;
     const size_t wbuf = (size_t)C * C * 2;
-    int resident = (size_t)2 * a.L * wbuf <= 160 * 1024 ? 1 : 0;
+    const size_t fixed = (size_t)(LMAX + 2) * C * sizeof(float);       // the kernel's own LDS array of parameter vectors
+    int resident = (size_t)2 * a.L * wbuf + fixed <= 160 * 1024 ? 1 : 0;
     size_t lds = (resident ? (size_t)2 * a.L : 2) * wbuf;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess && resident) {
