@@ -527,12 +527,14 @@ hipError_t launch_l(const MlpBwdArgs& a, hipStream_t st)
     return hipGetLastError();
 }
 
-template <typename T, int C, int WAVES>
+// One workgroup per compute unit; its wave count is what the registers of the instance allow (two waves per SIMD
+// up to 256 registers, three up to 168, four up to 128).
+template <typename T, int C>
 hipError_t launch_c(const MlpBwdArgs& a, hipStream_t st)
 {
-    if (a.L <= 1) return launch_l<T, C, WAVES, 1>(a, st);
-    if (a.L <= 5) return launch_l<T, C, WAVES, 5>(a, st);
-    if (a.L <= mlp_bwd_max_layers(C)) return launch_l<T, C, WAVES, (C == 128 ? 5 : 8)>(a, st);
+    if (a.L <= 1) return launch_l<T, C, (C == 128 ? 12 : 16), 1>(a, st);
+    if (a.L <= 5) return launch_l<T, C, (C == 128 ? 8 : C == 64 ? 12 : 16), 5>(a, st);
+    if (a.L <= mlp_bwd_max_layers(C)) return launch_l<T, C, (C == 128 ? 8 : C == 64 ? 12 : 16), (C == 128 ? 5 : 8)>(a, st);
     return hipErrorInvalidValue;
 }
 
@@ -540,9 +542,9 @@ template <typename T>
 hipError_t launch_t(const MlpBwdArgs& a, hipStream_t st)
 {
     switch (a.C) {
-        case 32:  return launch_c<T, 32, 4>(a, st);
-        case 64:  return launch_c<T, 64, 4>(a, st);
-        case 128: return launch_c<T, 128, 8>(a, st);
+        case 32:  return launch_c<T, 32>(a, st);
+        case 64:  return launch_c<T, 64>(a, st);
+        case 128: return launch_c<T, 128>(a, st);
         default:  return hipErrorInvalidValue;
     }
 }
