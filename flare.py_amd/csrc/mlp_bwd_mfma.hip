@@ -183,6 +183,41 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) woff[ks] = ((4 * ks + g) ^ (c16 >> SWS)) << 4;
 
+    // A [T,C] 16-bit row array receives the wave's 16 tokens from packed operand quads.  After row_piece a token's
+    // four lanes hold 64 contiguous bytes per k-step; the two half-rows of 8 lanes then trade pieces of neighbouring
+    // k-steps (one rotate by 8 within each 16 lanes), so that one store instruction completes 128-byte lines: the
+    // first for tokens 0-7 of the tile, the second for tokens 8-15.
+    auto store_rows = [&](uint16_t* base, const u32x4* q, int64_t t, int64_t n_tok) {
+        u32x4 piece[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) piece[ks] = row_piece(q[ks]);
+        const int rc = row_col(g);
+        if constexpr (KS == 1) {
+            if (t < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)t * C + rc) = piece[0];
+        } else {
+            const bool low = c16 < 8;
+#pragma unroll
+            for (int kp = 0; kp < KS; kp += 2) {
+                u32x4 send, recv;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    send[r] = low ? piece[kp + 1][r] : piece[kp][r];
+                    recv[r] = __builtin_amdgcn_update_dpp(send[r], send[r], 0x128, 0xf, 0xf, false);     // row_ror:8
+                }
+                u32x4 va, vb;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    va[r] = low ? piece[kp][r] : recv[r];
+                    vb[r] = low ? recv[r] : piece[kp + 1][r];
+                }
+                const int64_t ta = low ? t : t - 8, tb = low ? t + 8 : t;
+                const int col = 32 * (low ? kp : kp + 1) + rc;
+                if (ta < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)ta * C + col) = va;
+                if (tb < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)tb * C + col) = vb;
+            }
+        }
+    };
+
     int qcount = 0;      // ring mode: steps done by this workgroup; its parity names the slot in use
     if (resident) {
         for (int q = 0; q < 2 * L; ++q) stage(q, q);
@@ -249,16 +284,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
                 const f32x4 lo = xs[2 * ks], hi = xs[2 * ks + 1];
                 xb[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
             }
-            {                 // s_l, the input of layer l, as a 16-bit row (for dW_l)
-                u32x4 piece[KS];
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) piece[ks] = row_piece(xb[ks]);
-                if (live) {
-                    uint16_t* row = a.a_in + ((size_t)l * a.T + tok) * C + row_col(g);
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<u32x4*>(row + 32 * ks) = piece[ks];
-                }
-            }
+            store_rows(a.a_in + (size_t)l * a.T * C, xb, t, a.T);      // s_l, the input of layer l, as a 16-bit row (for dW_l)
             const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
             auto layer = [&](auto act_c, auto add_c) {
                 constexpr int ACT = decltype(act_c)::value;
@@ -321,16 +347,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
                 }
                 db[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
             }
-            {
-                u32x4 piece[KS];
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) piece[ks] = row_piece(db[ks]);
-                if (live) {
-                    uint16_t* row = a.g_out + ((size_t)l * a.T + tok) * C + row_col(g);
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<u32x4*>(row + 32 * ks) = piece[ks];
-                }
-            }
+            store_rows(a.g_out + (size_t)l * a.T * C, db, t, a.T);
             // ds_l = (ds_{l+1} if the layer added to the stream) + W_l^T dt_l
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
@@ -348,18 +365,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
         if (a.norm != 0) {
             // ds_0 and the token's statistics go out for dgamma, dbeta; xhat is taken again from x (the row is still
             // in cache) rather than kept in registers;  g = ds_0 * gamma
-            u32x4 piece[KS];
+            u32x4 dq[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 const f32x4 lo = xs[2 * ks], hi = xs[2 * ks + 1];
-                piece[ks] = row_piece(u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])});
+                dq[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
             }
-            if (live) {
-                uint16_t* row = a.dn + (size_t)tok * C + row_col(g);
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) *reinterpret_cast<u32x4*>(row + 32 * ks) = piece[ks];
-                if (lane < 16) *reinterpret_cast<float2*>(a.stats + 2 * tok) = make_float2(mean, rstd);
-            }
+            store_rows(a.dn, dq, t, a.T);
+            if (live && lane < 16) *reinterpret_cast<float2*>(a.stats + 2 * tok) = make_float2(mean, rstd);
             float m1 = 0.f, m2 = 0.f;
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
@@ -534,7 +547,7 @@ hipError_t launch_c(const MlpBwdArgs& a, hipStream_t st)
 {
     if (a.L <= 1) return launch_l<T, C, (C == 128 ? 12 : 16), 1>(a, st);
     if (a.L <= 5) return launch_l<T, C, (C == 128 ? 8 : C == 64 ? 12 : 16), 5>(a, st);
-    if (a.L <= mlp_bwd_max_layers(C)) return launch_l<T, C, (C == 128 ? 8 : C == 64 ? 12 : 16), (C == 128 ? 5 : 8)>(a, st);
+    if (a.L <= mlp_bwd_max_layers(C)) return launch_l<T, C, (C == 32 ? 16 : 8), (C == 128 ? 5 : 8)>(a, st);
     return hipErrorInvalidValue;
 }
 
