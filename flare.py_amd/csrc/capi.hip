@@ -504,6 +504,8 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
         a.ys[i] = desc->y_stride[i]; a.dys[i] = dy_stride[i];
     }
     a.dks[0] = a.dvs[0] = (int64_t)desc->H * nd; a.dks[1] = a.dvs[1] = nd; a.dks[2] = a.dvs[2] = desc->D;
+    if (desc->flags & FLARE_FLAG_GRAD_LIKE_KV)
+        for (int i = 0; i < 3; ++i) { a.dks[i] = desc->k_stride[i]; a.dvs[i] = desc->v_stride[i]; }
     return hip_status(flare::launch_mixer_bwd(a, desc->dtype, static_cast<hipStream_t>(stream)), "mixer backward launch");
 }
 

@@ -252,8 +252,16 @@ def _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy):
         gy = gy.contiguous()
     d = _mixer_desc(q4, k, v, y, scale, 0, False)
     dq = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
-    dk = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
-    dv = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+    # k and v that are token-major views ([B,N,H,D] storage, as a projection's output is) get their gradients in the
+    # same layout: the projection's backward then reads them as [B*N, H*D] rows without a copy
+    like_kv = all(t.stride() == (N * H * D, D, H * D, 1) for t in (k, v)) and H > 1
+    if like_kv:
+        d.flags |= _lib.FLAG_GRAD_LIKE_KV
+        dk = torch.empty((B, N, H, D), dtype=k.dtype, device=k.device).permute(0, 2, 1, 3)
+        dv = torch.empty((B, N, H, D), dtype=k.dtype, device=k.device).permute(0, 2, 1, 3)
+    else:
+        dk = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
+        dv = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
     need = C.c_size_t(0)
     _lib.check(lib.flare_mixer_bwd_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_bwd_workspace_bytes")
     ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)

@@ -63,6 +63,7 @@ extern "C" {
 /* FlareMixerDesc.flags */
 #define FLARE_FLAG_FORCE_GENERIC 1  /* skip the MFMA kernels, use the fp32-FMA kernels */
 #define FLARE_FLAG_MFMA16        2  /* keep the 16x16x32 MFMA kernels where the 32x32x16 scatter (bf16, D = 32, no key mask) would run */
+#define FLARE_FLAG_GRAD_LIKE_KV  8  /* flare_mixer_bwd: dk has k's strides and dv has v's (default: both [B,H,N,D] contiguous) */
 #define FLARE_FLAG_GATHER32      4  /* also run the gather on 32x32x16 products (bf16, D = 32, M % 256 == 0, no key mask); measured slower than the 16x16x32 gather at the headline shape, kept for comparison */
 
 /*
@@ -207,7 +208,8 @@ int flare_scatter_fwd_lse(const FlareMixerDesc* desc, const void* q, const void*
  * Inputs: q, k, v as in the forward; y and z its outputs; lse_lat = lse of flare_gather_fwd;
  * lse_tok of flare_scatter_fwd_lse; dy [B,H,N,D] with strides dy_stride.
  * Outputs: dq fp32 [B,H,M,D] contiguous (per batch element: sum over b when q is shared);
- * dk, dv [B,H,N,D] contiguous in the element type. */
+ * dk, dv [B,H,N,D] in the element type: contiguous, or with FLARE_FLAG_GRAD_LIKE_KV laid out as k and v are (a
+ * projection that produced k token-major then takes dk back without a copy). */
 int flare_mixer_bwd_workspace_bytes(const FlareMixerDesc* desc, size_t* bytes);
 int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v, const void* y,
                     const float* z, const float* lse_lat, const float* lse_tok, const void* dy,

@@ -241,3 +241,27 @@ def test_fp32_backward_at_262144_tokens_stays_inside_a_memory_bound(dev):
     for name, got, ref in (("dq", qd.grad, qr.grad), ("dk", kd.grad, kr.grad), ("dv", vd.grad, vr.grad)):
         err = float((got.double() - ref).norm() / ref.norm())
         assert err <= 1e-4, f"{name} rel-L2 {err:.3e}"
+
+
+def test_gradients_in_the_layout_of_token_major_inputs():
+    """k and v that are views of [B,N,H,D] storage (a projection's output) get dk, dv in that layout
+    (FLARE_FLAG_GRAD_LIKE_KV): same numbers as for head-major copies, and the [B,N,H*D] view of the gradient is
+    contiguous."""
+    torch.manual_seed(5)
+    B, H, N, M, D = 2, 4, 1500, 64, 32
+    dev = torch.device("cuda:0")
+    q = (torch.randn(H, M, D, device=dev) * 0.3).bfloat16().requires_grad_(True)
+    kt = torch.randn(B, N, H, D, device=dev).bfloat16().requires_grad_(True)
+    vt = torch.randn(B, N, H, D, device=dev).bfloat16().requires_grad_(True)
+    gy = torch.randn(B, H, N, D, device=dev).bfloat16()
+    y = F.flare_multihead_mixer(q, kt.permute(0, 2, 1, 3), vt.permute(0, 2, 1, 3))
+    y.backward(gy)
+    got = (q.grad.clone(), kt.grad.clone(), vt.grad.clone())
+    assert kt.grad.is_contiguous() and vt.grad.is_contiguous()
+    q.grad = None
+    kh = kt.detach().permute(0, 2, 1, 3).contiguous().requires_grad_(True)
+    vh = vt.detach().permute(0, 2, 1, 3).contiguous().requires_grad_(True)
+    F.flare_multihead_mixer(q, kh, vh).backward(gy)
+    assert torch.equal(got[0], q.grad)
+    assert torch.equal(got[1], kh.grad.permute(0, 2, 1, 3))
+    assert torch.equal(got[2], vh.grad.permute(0, 2, 1, 3))
