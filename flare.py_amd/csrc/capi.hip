@@ -821,7 +821,7 @@ int flare_mlp_bwd_partial_rows(const FlareMlpDesc* d, int32_t* rows)
 
 int flare_mlp_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const void* w_img, const void* wt_img,
                   const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* a_in,
-                  void* g_out, void* dn, float* stats, float* gb_part, float* db_part, void* stream)
+                  void* g_out, void* dn, float* stats, float* gb_part, float* gb, void* stream)
 {
     if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
     if (d->T < 1 || d->L < 1) return fail(FLARE_EINVAL, "T >= 1 and L >= 1 required (got %lld, %d)", (long long)d->T, d->L);
@@ -851,13 +851,50 @@ int flare_mlp_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const vo
     a.w = static_cast<const uint16_t*>(w_img); a.wt = static_cast<const uint16_t*>(wt_img);
     a.bias = bias; a.gamma = gamma; a.beta = beta;
     a.a_in = static_cast<uint16_t*>(a_in); a.g_out = static_cast<uint16_t*>(g_out);
-    a.dn = static_cast<uint16_t*>(dn); a.stats = stats; a.gb_part = gb_part; a.db_part = db_part;
+    a.dn = static_cast<uint16_t*>(dn); a.stats = stats; a.gb_part = gb_part; a.gb = gb;
     a.T = d->T; a.C = d->C; a.L = d->L;
     a.x_dtype = d->x_dtype; a.dy_dtype = d->y_dtype; a.dx_dtype = d->x_dtype;
     a.norm = d->norm; a.eps = d->eps; a.act = d->act; a.act_mask = d->act_mask; a.add_mask = d->add_mask;
     a.add_dy = add_dy ? 1 : 0;
     a.xs = d->x_stride; a.dys = d->y_stride; a.dxs = d->C;
     return hip_status(flare::launch_mlp_bwd(a, d->w_dtype, static_cast<hipStream_t>(stream)), "mlp backward launch");
+}
+
+static int check_wgrad_desc(const FlareMlpDesc* d)
+{
+    if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
+    if (d->T < 1 || d->L < 1) return fail(FLARE_EINVAL, "T >= 1 and L >= 1 required (got %lld, %d)", (long long)d->T, d->L);
+    if (d->w_dtype != FLARE_DT_BF16 && d->w_dtype != FLARE_DT_F16) return fail(FLARE_EINVAL, "w_dtype must be bf16 or f16");
+    if (!flare::mlp_mfma_supported(d->w_dtype, d->C)) return fail(FLARE_EUNSUPPORTED, "C=%d: only 32, 64 and 128 are supported", d->C);
+    if (d->L > 65535) return fail(FLARE_EUNSUPPORTED, "at most 65535 layers");
+    return FLARE_OK;
+}
+
+int flare_mlp_wgrad_partials(const FlareMlpDesc* d, int32_t* parts)
+{
+    if (!parts) return fail(FLARE_EINVAL, "parts is NULL");
+    int rc = check_wgrad_desc(d);
+    if (rc != FLARE_OK) return rc;
+    *parts = flare::mlp_wgrad_partials(d->T, d->C, d->L);
+    return FLARE_OK;
+}
+
+int flare_mlp_wgrad(const FlareMlpDesc* d, const void* a_in, const void* g_out, float* dw_part, float* db_part,
+                    float* dw, float* db, void* stream)
+{
+    int rc = check_wgrad_desc(d);
+    if (rc != FLARE_OK) return rc;
+    if (!a_in || !g_out || !dw_part) return fail(FLARE_EINVAL, "a_in, g_out and dw_part must not be NULL");
+    if (!aligned16(a_in) || !aligned16(g_out) || !aligned16(dw_part) || (db_part && !aligned16(db_part)) ||
+        (dw && !aligned16(dw)) || (db && !aligned16(db)))
+        return fail(FLARE_EINVAL, "every buffer must be 16-byte aligned");
+    if (db && !db_part) return fail(FLARE_EINVAL, "db needs db_part");
+    flare::MlpWgradArgs a;
+    memset(&a, 0, sizeof(a));
+    a.a_in = static_cast<const uint16_t*>(a_in); a.g_out = static_cast<const uint16_t*>(g_out);
+    a.dw_part = dw_part; a.db_part = db_part; a.dw = dw; a.db = db;
+    a.T = d->T; a.C = d->C; a.L = d->L;
+    return hip_status(flare::launch_mlp_wgrad(a, d->w_dtype, static_cast<hipStream_t>(stream)), "mlp weight-gradient launch");
 }
 
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes)

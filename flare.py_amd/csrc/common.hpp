@@ -201,7 +201,7 @@ struct MlpBwdArgs {
     uint16_t* dn;                               // [T,C] out (norm != 0): ds_0, the gradient at the norm's output, same type
     float* stats;                               // [T,2] out (norm != 0): mean and 1/std of every token
     float* gb_part;                             // [rows,2,C] out (norm != 0): partial sums of dgamma, dbeta over token ranges
-    float* db_part;                             // [rows,L,C] out or null: partial column sums of g_out (the bias gradients)
+    float* gb;                                  // [2,C] out or null (norm != 0): the partial rows summed in index order
     int64_t T;
     int C, L;
     int x_dtype, dy_dtype, dx_dtype;            // 0 f32, 1 bf16, 2 f16
@@ -211,6 +211,18 @@ struct MlpBwdArgs {
     uint32_t act_mask, add_mask;
     int add_dy;                                 // the forward's residual input was x itself: dx also receives dy
     int64_t xs, dys, dxs;                       // row strides in elements
+};
+
+// Arguments of the weight-gradient kernel (mlp_wgrad_mfma.hip): the rows launch_mlp_bwd leaves, reduced over tokens.
+struct MlpWgradArgs {
+    const uint16_t* a_in;                       // [L,T,C] the input of every layer (16-bit)
+    const uint16_t* g_out;                      // [L,T,C] the gradient at every layer's product (16-bit)
+    float* dw_part;                             // [parts,L,C,C] out: partial dW_l[out][in] per token range
+    float* db_part;                             // [parts,L,C] out or null: partial db_l
+    float* dw; float* db;                       // [L,C,C], [L,C] out or null: the partials summed in index order
+    int64_t T;
+    int C, L;
+    int64_t tokens_per_wg;                      // set by the launcher
 };
 
 // ---- launchers implemented in the .hip files -------------------------------------------
@@ -252,6 +264,9 @@ hipError_t launch_mlp_mfma(const MlpArgs& a, int w_dtype, hipStream_t st);
 int        mlp_bwd_max_layers(int C);
 int        mlp_bwd_partial_rows(int64_t T);
 hipError_t launch_mlp_bwd(const MlpBwdArgs& a, int w_dtype, hipStream_t st);
+int64_t    mlp_wgrad_tokens_per_wg(int64_t T, int C, int L);
+int        mlp_wgrad_partials(int64_t T, int C, int L);
+hipError_t launch_mlp_wgrad(const MlpWgradArgs& a, int w_dtype, hipStream_t st);
 
 int        causal_linear_tile();
 hipError_t launch_causal_linear(const CausalLinearArgs& a, int dtype, hipStream_t st);

@@ -1,6 +1,6 @@
 // Backward of the fused token-wise MLP stack of mlp_mfma.hip (the chain of C x C layers; bf16 / f16 weights,
 // C in {32, 64, 128}): what torch autograd does for  y = res + ResidualMLP(norm(x))  of
-// pdebench/models/flare.py:45-59 and 204-215, in one token-parallel launch plus a few library products.
+// pdebench/models/flare.py:45-59 and 204-215, in one token-parallel launch plus reductions over tokens for the parameters.
 //
 // Forward, per token:  s_0 = norm(x);  layer l:  t_l = W_l s_l + b_l,  u_l = act(t_l) if bit l of act_mask else t_l,
 // s_{l+1} = s_l + u_l if bit l of add_mask else u_l;  y = res + s_L.
@@ -13,9 +13,9 @@
 // act'(t_l) of every layer packed to 16 bits in registers, and walks the chain back with the TRANSPOSED weights in
 // the place of the weights (ds_l^T = W_l^T dt_l^T is the same product shape).  What a reduction over all tokens
 // needs leaves the kernel as 16-bit rows: s_l (the input of every layer) and dt_l, from which the caller forms
-// dW_l = dt_l^T s_l and db_l with library products; for the norm's parameters the kernel leaves ds_0 as 16-bit rows
-// and every token's (mean, 1/std), and mlp_norm_grads_kernel sums dgamma, dbeta over token ranges into one partial
-// row per workgroup (summed by the caller in a fixed order: no atomics).
+// dW_l = dt_l^T s_l and db_l are formed in one pass by mlp_wgrad_mfma.hip; for the norm's parameters the kernel
+// leaves ds_0 as 16-bit rows and every token's (mean, 1/std), and mlp_norm_grads_kernel sums dgamma, dbeta over token
+// ranges into one partial row per workgroup (summed in a fixed order by a last small launch: no atomics).
 // Weights move through LDS: all 2 L tiles resident when they fit, else a two-slot ring in the order
 // W_0 .. W_{L-1}, W_{L-1}^T .. W_0^T with one barrier per layer; they arrive as LDS images and are loaded straight
 // into their slots.
@@ -406,105 +406,76 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
 }
 
 // dgamma[c] = sum_t ds_0[t,c] xhat[t,c],  dbeta[c] = sum_t ds_0[t,c]  over the workgroup's token range.  Thread =
-// (channel pair, token lane): 256 threads cover C / 2 channel pairs x 512 / C token lanes, every lane walks its
-// tokens four at a time (all loads of a group in flight together), the lanes meet in LDS at the end.  Rows are read
-// coalesced (4 bytes of ds_0 and 8 bytes of x per thread); one partial row pair per workgroup.
+// (group of four channels, token lane): 256 threads cover C / 4 groups x 1024 / C token lanes, every lane walks its
+// tokens four at a time (all loads of a group in flight together: 16 bytes of x in fp32, 8 of ds_0), the lanes meet
+// in LDS at the end.  One partial row pair per workgroup.
 template <typename T>
 __global__ __launch_bounds__(256) void mlp_norm_grads_kernel(MlpBwdArgs a, int64_t tokens_per_wg)
 {
     using M_ = Mw<T>;
-    __shared__ float red[2][256][2];
-    const int pairs = a.C / 2, lanes = 256 / pairs;             // 16 x 16, 32 x 8 or 64 x 4
-    const int cp = threadIdx.x % pairs, tl = threadIdx.x / pairs;
+    __shared__ f32x4 red[2][256];
+    const int quads = a.C / 4, lanes = 256 / quads;             // 32 x 8, 16 x 16 or 8 x 32
+    const int cq = threadIdx.x % quads, tl = threadIdx.x / quads;
     const int64_t t0 = (int64_t)blockIdx.x * tokens_per_wg, t1 = t0 + tokens_per_wg < a.T ? t0 + tokens_per_wg : a.T;
-    float gs0 = 0.f, gs1 = 0.f, bs0 = 0.f, bs1 = 0.f;
-    auto xval = [&](int64_t t, float& x0, float& x1) {
-        const int64_t e = t * a.xs + 2 * cp;
-        if (a.x_dtype == 0) {
-            const float2 v = *reinterpret_cast<const float2*>(static_cast<const float*>(a.x) + e);
-            x0 = v.x; x1 = v.y;
-        } else {
-            const uint32_t v = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.x) + e);
-            if (a.x_dtype == 1) { x0 = __uint_as_float(v << 16); x1 = __uint_as_float(v & 0xffff0000u); }
-            else { x0 = Mw<f16_t>::lo(v); x1 = Mw<f16_t>::hi(v); }
-        }
-    };
+    f32x4 gs = {0.f, 0.f, 0.f, 0.f}, bs = {0.f, 0.f, 0.f, 0.f};
     for (int64_t t = t0 + tl; t < t1; t += 4 * lanes) {
-        float x0[4], x1[4];
+        f32x4 xv[4];
         float2 st[4];
-        uint32_t dv[4];
+        uint2 dv[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int64_t tt = t + u * lanes < t1 ? t + u * lanes : t1 - 1;
             st[u] = *reinterpret_cast<const float2*>(a.stats + 2 * tt);
-            xval(tt, x0[u], x1[u]);
-            dv[u] = *reinterpret_cast<const uint32_t*>(a.dn + (size_t)tt * a.C + 2 * cp);
+            xv[u] = ld4(a.x, tt * a.xs + 4 * cq, a.x_dtype);
+            dv[u] = *reinterpret_cast<const uint2*>(a.dn + (size_t)tt * a.C + 4 * cq);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             if (t + u * lanes >= t1) continue;
-            const float d0 = M_::lo(dv[u]), d1 = M_::hi(dv[u]);
-            gs0 = fmaf(d0, (x0[u] - st[u].x) * st[u].y, gs0);
-            gs1 = fmaf(d1, (x1[u] - st[u].x) * st[u].y, gs1);
-            bs0 += d0;
-            bs1 += d1;
+            const f32x4 d = {M_::lo(dv[u].x), M_::hi(dv[u].x), M_::lo(dv[u].y), M_::hi(dv[u].y)};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                gs[r] = fmaf(d[r], (xv[u][r] - st[u].x) * st[u].y, gs[r]);
+                bs[r] += d[r];
+            }
         }
     }
-    red[0][threadIdx.x][0] = gs0; red[0][threadIdx.x][1] = gs1;
-    red[1][threadIdx.x][0] = bs0; red[1][threadIdx.x][1] = bs1;
+    red[0][threadIdx.x] = gs;
+    red[1][threadIdx.x] = bs;
     __syncthreads();
-    if (threadIdx.x < pairs) {
-        float s[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
-        for (int l = 0; l < lanes; ++l)
-#pragma unroll
-            for (int k = 0; k < 2; ++k) {
-                s[k][0] += red[k][l * pairs + cp][0];
-                s[k][1] += red[k][l * pairs + cp][1];
-            }
-#pragma unroll
-        for (int k = 0; k < 2; ++k)
-            *reinterpret_cast<float2*>(a.gb_part + ((size_t)blockIdx.x * 2 + k) * a.C + 2 * cp) = make_float2(s[k][0], s[k][1]);
+    if ((int)threadIdx.x < 2 * quads) {
+        const int k = threadIdx.x / quads, q = threadIdx.x % quads;
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+        for (int l = 0; l < lanes; ++l) s += red[k][l * quads + q];
+        *reinterpret_cast<f32x4*>(a.gb_part + ((size_t)blockIdx.x * 2 + k) * a.C + 4 * q) = s;
     }
 }
 
-// db_l[c] = sum_t g_out[l,t,c] over the workgroup's token range (blockIdx.y = layer).  Thread = (piece of eight
-// channels, token lane): 256 threads cover C / 8 pieces x 2048 / C token lanes, 16 bytes per load, four tokens per
-// lane in flight; the lanes meet in LDS.  One partial row per workgroup and layer.
-template <typename T>
-__global__ __launch_bounds__(256) void mlp_bias_grads_kernel(MlpBwdArgs a, int64_t tokens_per_wg)
+// out[i] = sum over rows of part[row][i] (n = 2 C values per row).  A workgroup of 64 x 16 threads owns 64 values:
+// thread (x, y) adds the rows y, y + 16, ... with eight loads in flight, the 16 y meet in LDS.  Fixed order.
+__global__ __launch_bounds__(1024) void mlp_sum_rows_kernel(const float* part, int rows, int n, float* out)
 {
-    using M_ = Mw<T>;
-    __shared__ float red[256][8];
-    const int pieces = a.C / 8, lanes = 256 / pieces;           // 4 x 64, 8 x 32 or 16 x 16
-    const int pc = threadIdx.x % pieces, tl = threadIdx.x / pieces, l = blockIdx.y;
-    const int64_t t0 = (int64_t)blockIdx.x * tokens_per_wg, t1 = t0 + tokens_per_wg < a.T ? t0 + tokens_per_wg : a.T;
-    const uint16_t* g = a.g_out + (size_t)l * a.T * a.C + 8 * pc;
-    float s[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    for (int64_t t = t0 + tl; t < t1; t += 4 * lanes) {
-        u32x4 v[4];
+    __shared__ float red[16][64];
+    const int x = threadIdx.x & 63, y = threadIdx.x >> 6;
+    const int i = blockIdx.x * 64 + x;
+    float s = 0.f;
+    if (i < n) {
+        int r = y;
+        for (; r + 112 < rows; r += 128) {
+            float v[8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t tt = t + u * lanes < t1 ? t + u * lanes : t1 - 1;
-            v[u] = *reinterpret_cast<const u32x4*>(g + (size_t)tt * a.C);
+            for (int u = 0; u < 8; ++u) v[u] = part[(size_t)(r + 16 * u) * n + i];
+            s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
         }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            if (t + u * lanes >= t1) continue;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                s[2 * k] += M_::lo(v[u][k]);
-                s[2 * k + 1] += M_::hi(v[u][k]);
-            }
-        }
+        for (; r < rows; r += 16) s += part[(size_t)r * n + i];
     }
-#pragma unroll
-    for (int k = 0; k < 8; ++k) red[threadIdx.x][k] = s[k];
+    red[y][x] = s;
     __syncthreads();
-    if ((int)threadIdx.x < a.C) {
-        const int c = threadIdx.x;
-        float r = 0.f;
-        for (int q = 0; q < lanes; ++q) r += red[q * pieces + c / 8][c % 8];
-        a.db_part[((size_t)blockIdx.x * a.L + l) * a.C + c] = r;
+    if (y == 0 && i < n) {
+        float t = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) t += red[k][x];
+        out[i] = t;
     }
 }
 
@@ -528,15 +499,13 @@ hipError_t launch_l(const MlpBwdArgs& a, hipStream_t st)
     const int64_t cus = device_cus();
     hipLaunchKernelGGL(kern, dim3((unsigned)(nblk < cus ? nblk : cus)), dim3(64 * WAVES), lds, st, a, resident);
     e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess || a.norm == 0) return e;
     const int rows = mlp_bwd_partial_rows(a.T);
     const int64_t tpw = (a.T + rows - 1) / rows;
-    if (a.db_part) {
-        hipLaunchKernelGGL(mlp_bias_grads_kernel<T>, dim3(rows, a.L), dim3(256), 0, st, a, tpw);
-        e = hipGetLastError();
-    }
-    if (e != hipSuccess || a.norm == 0) return e;
     hipLaunchKernelGGL(mlp_norm_grads_kernel<T>, dim3(rows), dim3(256), 0, st, a, tpw);
+    e = hipGetLastError();
+    if (e != hipSuccess || !a.gb) return e;
+    hipLaunchKernelGGL(mlp_sum_rows_kernel, dim3((2 * C + 63) / 64), dim3(1024), 0, st, a.gb_part, rows, 2 * C, a.gb);
     return hipGetLastError();
 }
 

@@ -20,7 +20,7 @@ cached per module and rebuilt when a parameter changes.
 With gradients enabled the chain of C x C layers (the k/v projections, the feed-forward block and the output
 projection of a FLAREBlock at the reference's default ratios) runs through `_FusedMlpFn`: the same forward
 launch, and a backward that recomputes the chain per token tile in one launch (flare_mlp_bwd) and forms the
-parameter gradients from the rows it leaves with two batched library products.  The narrow-end, expanding and
+parameter gradients from the rows it leaves with one more launch (flare_mlp_wgrad).  The narrow-end, expanding and
 head-padded variants have no backward and stay with the torch layers while gradients are enabled.
 """
 from __future__ import annotations
@@ -345,24 +345,23 @@ def _packed_train(mod, layers, cd):
     return w, b, w_img, wt_img
 
 
-_DW_CHUNK = 4096      # tokens per partial product of the weight gradients
-
-
-def _weight_grads(g_out, a_in):
-    """dW[l] = g_out[l]^T a_in[l] over T tokens, [L, C, C] fp32.  The contraction is as long as the token axis and the
-    result is tiny, so it is split into chunks of _DW_CHUNK tokens that run as one batched product (the library then
-    has L * T / chunk independent problems instead of L with nothing to parallelise), and the partial results are
-    summed in fp32 in a fixed order."""
+def _weight_grads(d, g_out, a_in, want_bias):
+    """dW [L, C(out), C(in)] and db [L, C] (or None) in fp32 from the rows flare_mlp_bwd left: one pass of
+    flare_mlp_wgrad over both row arrays, partial results per token range summed in a fixed order."""
+    lib = _lib.load()
     L, T, Cdim = g_out.shape
-    n = T // _DW_CHUNK
-    parts = []
-    if n > 0:
-        gm = g_out[:, :n * _DW_CHUNK].reshape(L * n, _DW_CHUNK, Cdim)
-        am = a_in[:, :n * _DW_CHUNK].reshape(L * n, _DW_CHUNK, Cdim)
-        parts.append(torch.bmm(gm.transpose(1, 2), am).view(L, n, Cdim, Cdim).sum(dim=1, dtype=torch.float32))
-    if n * _DW_CHUNK < T:
-        parts.append(torch.bmm(g_out[:, n * _DW_CHUNK:].transpose(1, 2), a_in[:, n * _DW_CHUNK:]).float())
-    return parts[0] if len(parts) == 1 else parts[0] + parts[1]
+    parts = C.c_int32(0)
+    _lib.check(lib.flare_mlp_wgrad_partials(C.byref(d), C.byref(parts)), "flare_mlp_wgrad_partials")
+    dev = g_out.device
+    dwp = torch.empty(parts.value, L, Cdim, Cdim, dtype=torch.float32, device=dev)
+    dbp = torch.empty(parts.value, L, Cdim, dtype=torch.float32, device=dev) if want_bias else None
+    dw = torch.empty(L, Cdim, Cdim, dtype=torch.float32, device=dev)
+    db = torch.empty(L, Cdim, dtype=torch.float32, device=dev) if want_bias else None
+    with _on_device(dev):
+        rc = lib.flare_mlp_wgrad(C.byref(d), _ptr(a_in), _ptr(g_out), _ptr(dwp), _ptr(dbp), _ptr(dw), _ptr(db),
+                                 C.c_void_p(_stream_ptr(dev)))
+    _lib.check(rc, "flare_mlp_wgrad")
+    return dw, db
 
 
 class _FusedMlpFn(torch.autograd.Function):
@@ -409,32 +408,28 @@ class _FusedMlpFn(torch.autograd.Function):
         dx = torch.empty(T, Cdim, dtype=x2.dtype, device=dev)
         a_in = torch.empty(L, T, Cdim, dtype=cd, device=dev)
         g_out = torch.empty(L, T, Cdim, dtype=cd, device=dev)
-        dn = stats = gb = dbp = None
+        dn = stats = gb = gsum = None
         any_bias = any(l.bias is not None for l in layers)
-        rows = C.c_int32(0)
-        _lib.check(lib.flare_mlp_bwd_partial_rows(C.byref(d), C.byref(rows)), "flare_mlp_bwd_partial_rows")
-        if any_bias:
-            dbp = torch.empty(rows.value, L, Cdim, dtype=torch.float32, device=dev)
         if d.norm:
+            rows = C.c_int32(0)
+            _lib.check(lib.flare_mlp_bwd_partial_rows(C.byref(d), C.byref(rows)), "flare_mlp_bwd_partial_rows")
             dn = torch.empty(T, Cdim, dtype=cd, device=dev)
             stats = torch.empty(T, 2, dtype=torch.float32, device=dev)
             gb = torch.empty(rows.value, 2, Cdim, dtype=torch.float32, device=dev)
+            gsum = torch.empty(2, Cdim, dtype=torch.float32, device=dev)
         with _on_device(dev):
             rc = lib.flare_mlp_bwd(C.byref(d), _ptr(x2), _ptr(dy2), _ptr(w_img), _ptr(wt_img), _ptr(b), _ptr(gamma), _ptr(beta),
                                    1 if ctx.res_is_x else 0, _ptr(dx), _ptr(a_in), _ptr(g_out), _ptr(dn), _ptr(stats), _ptr(gb),
-                                   _ptr(dbp), C.c_void_p(_stream_ptr(dev)))
+                                   _ptr(gsum), C.c_void_p(_stream_ptr(dev)))
         _lib.check(rc, "flare_mlp_bwd")
-        # weight gradients: batched products over the rows the kernel left (16-bit products with fp32 accumulation,
-        # as torch runs a Linear's backward under autocast); bias and norm gradients: the kernels' partial rows,
-        # summed in a fixed order
-        dW = _weight_grads(g_out, a_in)                                  # [L, out, in] fp32
-        db = dbp.sum(0) if any_bias else None                            # [L, C]
+        # weight and bias gradients: one more launch over the rows the kernel left (16-bit products with fp32
+        # accumulation, as torch runs a Linear's backward under autocast); norm gradients: partial rows, summed here
+        dW, db = _weight_grads(d, g_out, a_in, any_bias)                 # [L, out, in], [L, C] fp32
         need = ctx.needs_input_grad            # (mod, cd, norm, out_dtype, x, res, gamma, beta, *wb)
         grads = [None, None, None, None]
         grads.append(dx.view(x.shape) if need[4] else None)
         grads.append(None if (not ctx.has_res or ctx.res_is_x or not need[5]) else dy)
         if d.norm:
-            gsum = gb.sum(0)
             grads.append(gsum[0].to(norm.weight.dtype) if need[6] else None)
             grads.append(gsum[1].to(norm.bias.dtype) if (need[7] and getattr(norm, "bias", None) is not None) else None)
         else:

@@ -316,25 +316,35 @@ int flare_mlp_io_fwd(const FlareMlpDesc* desc, int32_t in_dim, int32_t in_act, c
 /* Backward of flare_mlp_fwd for the chain of C x C layers (desc->flags == 0; at most 8 layers, 5 at C = 128): what
  * torch autograd computes for  y = res + ResidualMLP(norm(x))  (pdebench/models/flare.py:45-59, 204-215) when
  * the reference trains a block.  One token-parallel launch recomputes the forward and walks the chain back;
- * reductions over all tokens are left to the caller as library products:
+ * the reductions over all tokens that the weight and bias gradients need are a second call (flare_mlp_wgrad below):
  *   dx      [T,C]   contiguous, x's dtype: gradient of x (plus dy when add_dy != 0: the forward's res was x itself;
  *                   otherwise the gradient of res is dy)
  *   a_in    [L,T,C] the input of every layer and
  *   g_out   [L,T,C] the gradient at every layer's product, both in the weights' type:
- *                   dW_l = g_out[l]^T a_in[l],  db_l = column sums of g_out[l]
+ *                   dW_l = g_out[l]^T a_in[l],  db_l = column sums of g_out[l]  (flare_mlp_wgrad forms both)
  *   dn      [T,C]   (norm only) gradient at the norm's output, weights' type;  stats [T,2] fp32 mean and 1/std
  *   gb_part [rows,2,C] fp32 (norm only; rows from flare_mlp_bwd_partial_rows): dgamma = sum over rows of
  *                   gb_part[:,0,:], dbeta = sum of gb_part[:,1,:] (fixed order: no atomics)
- *   db_part [rows,L,C] fp32 or NULL (same rows): db_l = sum over rows of db_part[:,l,:]; NULL skips that launch
+ *   gb      [2,C]   fp32 or NULL (norm only): those two sums, formed by one more small launch in index order
  * dy has desc->y_dtype and row stride desc->y_stride.  w_img, wt_img [L,C,C]: the weights and their transposes as
  * the kernel's LDS images: element (row, col) of a tile sits at 16-bit position
  *   row * C + 8 * (((4 * (ch / 4) + 2 * (ch % 2) + (j / 4)) ^ key)) + 4 * ((ch % 4) / 2) + j % 4,
  *   ch = col / 8, j = col % 8, key = (row % 16) >> (C == 128 ? 0 : C == 64 ? 1 : 2)
  * (flare.py_amd/fused.py::mlp_weight_image builds them). */
 int flare_mlp_bwd_partial_rows(const FlareMlpDesc* desc, int32_t* rows);
+/* Weight and bias gradients from the rows flare_mlp_bwd leaves, in one pass over both (the reference gets them from
+ * torch's Linear backward: dW = dt^T s, db = column sums of dt; pdebench/models/flare.py:45-59 under autograd).
+ * Only T, C, L and w_dtype of the descriptor are read.  a_in, g_out [L,T,C] in the weights' type;
+ *   dw_part [parts,L,C,C] fp32: dW_l[out][in] = sum over parts of dw_part[:,l];
+ *   db_part [parts,L,C]   fp32 or NULL: db_l = sum over parts of db_part[:,l]
+ * with parts from flare_mlp_wgrad_partials;  dw [L,C,C], db [L,C] fp32 or NULL: those sums, formed by a second small
+ * launch in index order (no atomics, two runs give the same bits). */
+int flare_mlp_wgrad_partials(const FlareMlpDesc* desc, int32_t* parts);
+int flare_mlp_wgrad(const FlareMlpDesc* desc, const void* a_in, const void* g_out, float* dw_part, float* db_part,
+                    float* dw, float* db, void* stream);
 int flare_mlp_bwd(const FlareMlpDesc* desc, const void* x, const void* dy, const void* w_img, const void* wt_img,
                   const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* a_in,
-                  void* g_out, void* dn, float* stats, float* gb_part, float* db_part, void* stream);
+                  void* g_out, void* dn, float* stats, float* gb_part, float* gb, void* stream);
 
 int flare_triple_workspace_bytes(const FlareTripleDesc* desc, size_t* bytes);
 

@@ -265,3 +265,30 @@ def test_mlp_bwd_validation():
     assert call() == _lib.FLARE_EINVAL and "activation" in _lib.last_error()
     m.act, m.eps = 0, -1.0
     assert call() == _lib.FLARE_EINVAL and "eps" in _lib.last_error()
+
+
+def test_mlp_wgrad_validation():
+    lib = _lib.load()
+    m = _lib.FlareMlpDesc()
+    m.T, m.C, m.L = 262144, 128, 5
+    m.w_dtype = _lib.DT_BF16
+    fake, odd = C.c_void_p(4096), C.c_void_p(4100)
+    parts = C.c_int32(0)
+    assert lib.flare_mlp_wgrad_partials(m, C.byref(parts)) == _lib.FLARE_OK and 1 <= parts.value <= 1024
+    big = parts.value
+    m.T = 100
+    assert lib.flare_mlp_wgrad_partials(m, C.byref(parts)) == _lib.FLARE_OK and parts.value == 1
+    m.C = 32            # eight waves split a token tile: eight partials per token range
+    assert lib.flare_mlp_wgrad_partials(m, C.byref(parts)) == _lib.FLARE_OK and parts.value == 8
+    m.C, m.T = 128, 262144
+    assert lib.flare_mlp_wgrad_partials(m, None) == _lib.FLARE_EINVAL
+    assert lib.flare_mlp_wgrad(m, None, fake, fake, None, None, None, None) == _lib.FLARE_EINVAL and "must not be NULL" in _lib.last_error()
+    assert lib.flare_mlp_wgrad(m, fake, fake, odd, None, None, None, None) == _lib.FLARE_EINVAL and "16-byte" in _lib.last_error()
+    assert lib.flare_mlp_wgrad(m, fake, fake, fake, None, fake, fake, None) == _lib.FLARE_EINVAL and "db needs db_part" in _lib.last_error()
+    m.C = 96
+    assert lib.flare_mlp_wgrad(m, fake, fake, fake, None, None, None, None) == _lib.FLARE_EUNSUPPORTED
+    m.C, m.w_dtype = 128, _lib.DT_F32
+    assert lib.flare_mlp_wgrad(m, fake, fake, fake, None, None, None, None) == _lib.FLARE_EINVAL and "w_dtype" in _lib.last_error()
+    m.w_dtype, m.L = _lib.DT_BF16, 0
+    assert lib.flare_mlp_wgrad_partials(m, C.byref(parts)) == _lib.FLARE_EINVAL
+    assert big >= 64
