@@ -395,12 +395,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
             }
         }
         if (live) {
+            // every load of dy before the first store of dx (a load written after a store stays behind it: the two
+            // may be the same memory as far as the compiler knows)
+            if (a.add_dy) {
 #pragma unroll
-            for (int ft = 0; ft < FT; ++ft) {
-                f32x4 o = xs[ft];
-                if (a.add_dy) o += ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
-                st4(a.dx, tok * a.dxs + 16 * ft + 4 * g, a.dx_dtype, o);
+                for (int ft = 0; ft < FT; ++ft) xs[ft] += ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
             }
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) st4(a.dx, tok * a.dxs + 16 * ft + 4 * g, a.dx_dtype, xs[ft]);
         }
     }
 }

@@ -162,6 +162,17 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
         }
     };
 
+    // Parameter vectors are read without a branch (a branch per feature tile keeps the compiler from issuing the
+    // loads ahead of where they are used): a missing vector reads the weights instead, any mapped memory will do,
+    // and is replaced by zeros.
+    const bool has_bias = a.bias != nullptr, has_beta = a.beta != nullptr;
+    const float* bias0 = has_bias ? a.bias : reinterpret_cast<const float*>(a.w);
+    const float* beta0 = has_beta ? a.beta : reinterpret_cast<const float*>(a.w);
+    auto vec4 = [](const float* p, bool have) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(p);
+        return have ? v : f32x4{0.f, 0.f, 0.f, 0.f};
+    };
+
     int woff[KS];     // byte offset of this lane's chunk of k-step ks inside its weight row (swizzled)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) woff[ks] = ((4 * ks + g) ^ (c16 >> SWS)) << 4;
@@ -260,8 +271,7 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
 #pragma unroll
                 for (int ft = 0; ft < FT; ++ft) {
                     const f32x4 gm = *reinterpret_cast<const f32x4*>(a.gamma + 16 * ft + 4 * g);
-                    f32x4 bt = {0.f, 0.f, 0.f, 0.f};
-                    if (a.beta) bt = *reinterpret_cast<const f32x4*>(a.beta + 16 * ft + 4 * g);
+                    const f32x4 bt = vec4(beta0 + 16 * ft + 4 * g, has_beta);
 #pragma unroll
                     for (int r = 0; r < 4; ++r) xs[ft][tw][r] = (xs[ft][tw][r] - mean) * rstd * gm[r] + bt[r];
                 }
@@ -288,14 +298,14 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
                 const int slot = resident ? l : (lcount & 1);
                 if (!resident) fetch(l + 1 < a.L ? l + 1 : 0);
                 const uint8_t* wb = smem + slot * WBUF + c16 * RS;
-                const float* bl = a.bias ? a.bias + (size_t)l * C + 4 * g : nullptr;
+                const float* bl = bias0 + (size_t)l * C + 4 * g;
                 if (!(l & 1)) {
                     // h = act(W1[j] n + b1[j]): tile ft of h is half (ft & 1) of k-step ft / 2 of the next product
                     auto first = [&](auto act_c) {
                         constexpr int ACT = decltype(act_c)::value;
 #pragma unroll
                         for (int ft = 0; ft < FT; ++ft) {
-                            const f32x4 bias = bl ? *reinterpret_cast<const f32x4*>(bl + 16 * ft) : f32x4{0.f, 0.f, 0.f, 0.f};
+                            const f32x4 bias = vec4(bl + 16 * ft, has_bias);
                             f32x4 acc[TW];
 #pragma unroll
                             for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
@@ -326,7 +336,7 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
                         f32x4 acc[TW];
 #pragma unroll
                         for (int tw = 0; tw < TW; ++tw) acc[tw] = xs[ft][tw];
-                        if (bl && l == 1) {
+                        if (has_bias && l == 1) {
                             const f32x4 bias = *reinterpret_cast<const f32x4*>(bl + 16 * ft);
 #pragma unroll
                             for (int tw = 0; tw < TW; ++tw) acc[tw] += bias;
@@ -371,10 +381,16 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
             auto layer = [&](auto act_c, auto add_c) {
                 constexpr int ACT = decltype(act_c)::value;
                 constexpr bool ADD = decltype(add_c)::value;
+                // the bias of a feature tile is requested two tiles ahead: it initialises the accumulators, so a load
+                // issued where it is used would put a trip to the cache in front of every tile's first product
+                const float* bl = bias0 + (size_t)l * C + 4 * g;
+                f32x4 bias_q[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) bias_q[i] = vec4(bl + 16 * (i < FT ? i : 0), has_bias);
 #pragma unroll
                 for (int ft = 0; ft < FT; ++ft) {
-                    const f32x4 bias = a.bias ? *reinterpret_cast<const f32x4*>(a.bias + (size_t)l * C + 16 * ft + 4 * g)
-                                              : f32x4{0.f, 0.f, 0.f, 0.f};
+                    const f32x4 bias = bias_q[ft & 1];
+                    if (ft + 2 < FT) bias_q[ft & 1] = vec4(bl + 16 * (ft + 2), has_bias);
                     f32x4 acc[TW];
 #pragma unroll
                     for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
@@ -437,22 +453,26 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
                 const int cf = a.y_head == 8 ? 32 : 64, c0 = a.y_head == 8 ? 8 * g - 4 * (g & 1) : 16 * g;
                 const int nz = a.y_head == 8 ? ((g & 1) ? 2 : 0) : 3;        // groups of 4 zero columns behind this lane's channels
                 const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                if (a.res) {
+#pragma unroll
+                    for (int ft = 0; ft < FT; ++ft) xs[ft][tw] += load4(a.res, tok[tw] * a.rs + 16 * ft + 4 * g, a.res_dtype);
+                }
 #pragma unroll
                 for (int ft = 0; ft < FT; ++ft) {
-                    f32x4 o = xs[ft][tw];
-                    if (a.res) o += load4(a.res, tok[tw] * a.rs + 16 * ft + 4 * g, a.res_dtype);
                     const int64_t col = tok[tw] * a.ys + ft * cf + c0;
-                    store4(a.y, col, a.y_dtype, o);
+                    store4(a.y, col, a.y_dtype, xs[ft][tw]);
                     for (int z = 1; z <= nz; ++z) store4(a.y, col + 4 * z, a.y_dtype, zero);
                 }
                 continue;
             }
+            // all residual loads of the row before its first store: y may be the memory res points at, so a load
+            // written after a store also stays behind it, and the row would take one trip to memory per tile
+            if (a.res) {
 #pragma unroll
-            for (int ft = 0; ft < FT; ++ft) {
-                f32x4 o = xs[ft][tw];
-                if (a.res) o += load4(a.res, tok[tw] * a.rs + 16 * ft + 4 * g, a.res_dtype);
-                store4(a.y, tok[tw] * a.ys + 16 * ft + 4 * g, a.y_dtype, o);
+                for (int ft = 0; ft < FT; ++ft) xs[ft][tw] += load4(a.res, tok[tw] * a.rs + 16 * ft + 4 * g, a.res_dtype);
             }
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) store4(a.y, tok[tw] * a.ys + 16 * ft + 4 * g, a.y_dtype, xs[ft][tw]);
         }
     }
 }
