@@ -349,22 +349,25 @@ def bench_block(args, F, dev):
     xg = x.detach().clone().requires_grad_(True)
     gy = torch.randn_like(xg)
 
-    def train_step(layers_fused=True):
+    def train_step(layers_fused=True, block=None):
+        block = blk1 if block is None else block
         real = fused.compute_dtype
         if not layers_fused:
             fused.compute_dtype = lambda *a, **k: None
         try:
             with torch.autocast("cuda", dtype=torch.bfloat16):
-                y = blk1(xg)[0]
+                y = block(xg)[0]
             y.backward(gy)
         finally:
             fused.compute_dtype = real
-        blk1.zero_grad(set_to_none=True)
+        block.zero_grad(set_to_none=True)
         xg.grad = None
-    blk1.train()
+    blk1.train(); blk.train()
     ms_train = wall_ms(train_step, 20, 5)
     ms_train_torch = None if args.no_torch_sdpa else wall_ms(lambda: train_step(False), 10, 3)
-    blk1.eval()
+    ms_train4 = wall_ms(lambda: train_step(True, blk), 20, 5)
+    ms_train4_torch = None if args.no_torch_sdpa else wall_ms(lambda: train_step(False, blk), 10, 3)
+    blk1.eval(); blk.eval()
     kk = torch.randn(4, 65536, 128, device=dev).bfloat16().view(4, 65536, 8, 16).permute(0, 2, 1, 3)
     qq = (torch.randn(8, 128, 16, device=dev) * 0.25).bfloat16()
     ms_mixer = time_events(lambda: F.flare_multihead_mixer(qq, kk, kk), args.steps, 2)
@@ -401,6 +404,9 @@ def bench_block(args, F, dev):
     out["train_block_default_ffn"] = {"ms_fwd_bwd": round(ms_train, 3),
                                       "ms_fwd_bwd_torch_layers_hip_mixer": None if ms_train_torch is None else round(ms_train_torch, 3),
                                       "what": "forward + backward of the default block (3-layer C x C MLPs), bf16 autocast, gradients of x and of every parameter"}
+    out["train_block_4x_ffn"] = {"ms_fwd_bwd": round(ms_train4, 3),
+                                 "ms_fwd_bwd_torch_layers_hip_mixer": None if ms_train4_torch is None else round(ms_train4_torch, 3),
+                                 "what": "the same for the block with the 4x GELU MLP as its feed-forward (no lift)"}
     # the same modules the way the reference runs them on this device: torch Linear / LayerNorm layers under the
     # same autocast, the mixer as two torch scaled_dot_product_attention calls (pdebench/models/flare.py:122-156)
     try:

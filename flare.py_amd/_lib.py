@@ -101,7 +101,8 @@ SYMBOLS = {
     "flare_mlp_bwd_partial_rows": (C.c_int, [C.POINTER(FlareMlpDesc), C.POINTER(C.c_int32)]),
     "flare_mlp_bwd": (C.c_int, [C.POINTER(FlareMlpDesc), _P, _P, _P, _P, _P, _P, _P, C.c_int32, _P, _P, _P, _P, _P, _P, _P, _P]),
     "flare_mlp_wgrad_partials": (C.c_int, [C.POINTER(FlareMlpDesc), C.POINTER(C.c_int32)]),
-    "flare_mlp_wgrad": (C.c_int, [C.POINTER(FlareMlpDesc), _P, _P, _P, _P, _P, _P, _P]),
+    "flare_mlp_wgrad": (C.c_int, [C.POINTER(FlareMlpDesc), _P, C.c_int64, _P, C.c_int64, _P, _P, _P, _P, _P]),
+    "flare_mlp_expand_bwd": (C.c_int, [C.POINTER(FlareMlpDesc), _P, _P, _P, _P, _P, _P, _P, C.c_int32, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "flare_triple_workspace_bytes": (C.c_int, [C.POINTER(FlareTripleDesc), C.POINTER(_SZ)]),
     "flare_triple_state_fwd": (C.c_int, [C.POINTER(FlareTripleDesc), _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_triple_out_fwd": (C.c_int, [C.POINTER(FlareTripleDesc), _P, _P, _P, _P, _P, _P]),

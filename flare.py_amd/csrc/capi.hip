@@ -860,6 +860,46 @@ int flare_mlp_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const vo
     return hip_status(flare::launch_mlp_bwd(a, d->w_dtype, static_cast<hipStream_t>(stream)), "mlp backward launch");
 }
 
+int flare_mlp_expand_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const void* w_img, const void* wt_img,
+                         const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* n_row,
+                         void* dy_row, void* h, void* dt, void* dn, float* stats, float* gb_part, float* gb, void* stream)
+{
+    if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
+    if (d->T < 1) return fail(FLARE_EINVAL, "T >= 1 required");
+    if (d->flags != FLARE_MLP_EXPAND) return fail(FLARE_EINVAL, "flags must be FLARE_MLP_EXPAND");
+    if (d->L < 4 || d->L > 16 || (d->L & 1)) return fail(FLARE_EUNSUPPORTED, "L = 2 E tiles with 2 <= E <= 8 (got L = %d)", d->L);
+    if (d->w_dtype != FLARE_DT_BF16 && d->w_dtype != FLARE_DT_F16) return fail(FLARE_EINVAL, "w_dtype must be bf16 or f16");
+    if (d->x_dtype < FLARE_DT_F32 || d->x_dtype > FLARE_DT_F16 || d->y_dtype < FLARE_DT_F32 || d->y_dtype > FLARE_DT_F16)
+        return fail(FLARE_EINVAL, "unknown dtype");
+    if (d->norm < FLARE_NORM_NONE || d->norm > FLARE_NORM_RMS) return fail(FLARE_EINVAL, "unknown norm %d", d->norm);
+    if (d->act < FLARE_ACT_GELU_TANH || d->act > FLARE_ACT_SILU) return fail(FLARE_EINVAL, "unknown activation %d", d->act);
+    if (!flare::mlp_mfma_supported(d->w_dtype, d->C)) return fail(FLARE_EUNSUPPORTED, "C=%d: only 32, 64 and 128 are supported", d->C);
+    if (!x || !dy || !w_img || !wt_img || !dx || !n_row || !dy_row || !h || !dt)
+        return fail(FLARE_EINVAL, "x, dy, w_img, wt_img, dx, n_row, dy_row, h, dt must not be NULL");
+    if (d->norm != FLARE_NORM_NONE && (!gamma || !dn || !stats || !gb_part))
+        return fail(FLARE_EINVAL, "gamma, dn, stats and gb_part must not be NULL when a norm is requested");
+    if (d->norm != FLARE_NORM_NONE && !(d->eps >= 0.f)) return fail(FLARE_EINVAL, "eps must be >= 0");
+    if (d->x_stride < d->C || d->x_stride % 4 || !aligned16(x)) return fail(FLARE_EINVAL, "x: row stride >= C, a multiple of 4, base 16-byte aligned");
+    if (d->y_stride < d->C || d->y_stride % 4 || !aligned16(dy)) return fail(FLARE_EINVAL, "dy: row stride (y_stride) >= C, a multiple of 4, base 16-byte aligned");
+    const void* ptrs[] = {dx, n_row, dy_row, h, dt, w_img, wt_img, bias, gamma, beta, dn, stats, gb};
+    for (const void* p : ptrs)
+        if (p && !aligned16(p)) return fail(FLARE_EINVAL, "every buffer must be 16-byte aligned");
+    flare::MlpBwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.x = x; a.dy = dy; a.dx = dx;
+    a.w = static_cast<const uint16_t*>(w_img); a.wt = static_cast<const uint16_t*>(wt_img);
+    a.bias = bias; a.gamma = gamma; a.beta = beta;
+    a.a_in = static_cast<uint16_t*>(h); a.g_out = static_cast<uint16_t*>(dt);
+    a.n_row = static_cast<uint16_t*>(n_row); a.dy_row = static_cast<uint16_t*>(dy_row);
+    a.dn = static_cast<uint16_t*>(dn); a.stats = stats; a.gb_part = gb_part; a.gb = gb;
+    a.T = d->T; a.C = d->C; a.L = d->L; a.E = d->L / 2;
+    a.x_dtype = d->x_dtype; a.dy_dtype = d->y_dtype; a.dx_dtype = d->x_dtype;
+    a.norm = d->norm; a.eps = d->eps; a.act = d->act;
+    a.add_dy = add_dy ? 1 : 0;
+    a.xs = d->x_stride; a.dys = d->y_stride; a.dxs = d->C;
+    return hip_status(flare::launch_mlp_bwd(a, d->w_dtype, static_cast<hipStream_t>(stream)), "mlp expand backward launch");
+}
+
 static int check_wgrad_desc(const FlareMlpDesc* d)
 {
     if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
@@ -879,8 +919,8 @@ int flare_mlp_wgrad_partials(const FlareMlpDesc* d, int32_t* parts)
     return FLARE_OK;
 }
 
-int flare_mlp_wgrad(const FlareMlpDesc* d, const void* a_in, const void* g_out, float* dw_part, float* db_part,
-                    float* dw, float* db, void* stream)
+int flare_mlp_wgrad(const FlareMlpDesc* d, const void* a_in, int64_t a_layer_stride, const void* g_out, int64_t g_layer_stride,
+                    float* dw_part, float* db_part, float* dw, float* db, void* stream)
 {
     int rc = check_wgrad_desc(d);
     if (rc != FLARE_OK) return rc;
@@ -889,9 +929,12 @@ int flare_mlp_wgrad(const FlareMlpDesc* d, const void* a_in, const void* g_out, 
         (dw && !aligned16(dw)) || (db && !aligned16(db)))
         return fail(FLARE_EINVAL, "every buffer must be 16-byte aligned");
     if (db && !db_part) return fail(FLARE_EINVAL, "db needs db_part");
+    if (a_layer_stride < 0 || g_layer_stride < 0 || a_layer_stride % 8 || g_layer_stride % 8)
+        return fail(FLARE_EINVAL, "layer strides must be >= 0 and multiples of 8 elements");
     flare::MlpWgradArgs a;
     memset(&a, 0, sizeof(a));
     a.a_in = static_cast<const uint16_t*>(a_in); a.g_out = static_cast<const uint16_t*>(g_out);
+    a.a_lstride = a_layer_stride; a.g_lstride = g_layer_stride;
     a.dw_part = dw_part; a.db_part = db_part; a.dw = dw; a.db = db;
     a.T = d->T; a.C = d->C; a.L = d->L;
     return hip_status(flare::launch_mlp_wgrad(a, d->w_dtype, static_cast<hipStream_t>(stream)), "mlp weight-gradient launch");

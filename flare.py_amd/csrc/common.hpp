@@ -202,6 +202,8 @@ struct MlpBwdArgs {
     float* stats;                               // [T,2] out (norm != 0): mean and 1/std of every token
     float* gb_part;                             // [rows,2,C] out (norm != 0): partial sums of dgamma, dbeta over token ranges
     float* gb;                                  // [2,C] out or null (norm != 0): the partial rows summed in index order
+    int E;                                      // > 0: the expanding MLP C -> E C -> C (w, wt, bias hold 2 E tiles / rows;
+    uint16_t* n_row; uint16_t* dy_row;          // a_in = h_j, g_out = dt_j per chunk; n and dy as 16-bit rows [T,C])
     int64_t T;
     int C, L;
     int x_dtype, dy_dtype, dx_dtype;            // 0 f32, 1 bf16, 2 f16
@@ -217,6 +219,7 @@ struct MlpBwdArgs {
 struct MlpWgradArgs {
     const uint16_t* a_in;                       // [L,T,C] the input of every layer (16-bit)
     const uint16_t* g_out;                      // [L,T,C] the gradient at every layer's product (16-bit)
+    int64_t a_lstride, g_lstride;               // elements from one layer's rows to the next's (0: all layers share one array)
     float* dw_part;                             // [parts,L,C,C] out: partial dW_l[out][in] per token range
     float* db_part;                             // [parts,L,C] out or null: partial db_l
     float* dw; float* db;                       // [L,C,C], [L,C] out or null: the partials summed in index order

@@ -407,6 +407,258 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
     }
 }
 
+// Backward of the expanding two-layer MLP  y = res + W2 act(W1 norm(x) + b1) + b2  (the "4x" feed-forward block; the
+// forward is mode 1 of mlp_mfma.hip, hidden width E * C run as E chunks of C).  Per chunk j and 16-token tile:
+//   t_j = W1[j] n + b1[j],  h_j = act(t_j)                       (recomputed; tile 2 j of a.w)
+//   dh_j = W2[:,j]^T dy,    dt_j = dh_j * act'(t_j)              (tile 2 j + 1 of a.wt)
+//   dn  += W1[j]^T dt_j                                          (tile 2 j of a.wt)
+// three ring steps per chunk, nothing kept from one chunk to the next but dn.  Rows left for the weight gradients:
+// n and dy in 16 bits (one row array each, shared by all chunks), h_j (a.a_in) and dt_j (a.g_out) per chunk:
+//   dW1[j] = dt_j^T n,  db1[j] = column sums of dt_j,  dW2[:,j] = dy^T h_j,  db2 = column sums of dy.
+constexpr int kExpandMax = 8;
+template <typename T, int C, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArgs a)
+{
+    constexpr int NT = 64 * WAVES;
+    constexpr int NCH = (C * C / 8 + NT - 1) / NT;
+    constexpr int FT = C / 16, KS = C / 32, RS = C * 2, WBUF = C * RS, CPR = C / 8;
+    constexpr int SWS = CPR == 16 ? 0 : CPR == 8 ? 1 : 2;
+    constexpr int PG = kExpandMax, PB = kExpandMax + 1;          // rows of pvec: b1[0..E), gamma, beta
+    using M_ = Mw<T>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    __shared__ __attribute__((aligned(16))) float pvec[(kExpandMax + 2) * C];
+
+    const int tid = threadIdx.x, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int E = a.E, Q = 3 * E;
+    for (int i = tid; i < (kExpandMax + 2) * C; i += NT) {
+        const int row = i / C, c = i % C;
+        float v = 0.f;
+        if (row < kExpandMax) { if (a.bias && row < E) v = a.bias[(size_t)(2 * row) * C + c]; }
+        else if (row == PG) { if (a.norm != 0) v = a.gamma[c]; }
+        else if (a.norm != 0 && a.beta) v = a.beta[c];
+        pvec[i] = v;
+    }
+
+    auto stage = [&](int q, int slot) {
+        const int j = q / 3, r = q - 3 * j;
+        const uint16_t* tile = r == 0 ? a.w + (size_t)(2 * j) * C * C : a.wt + (size_t)(2 * j + (r == 1 ? 1 : 0)) * C * C;
+        const uint8_t* img = reinterpret_cast<const uint8_t*>(tile);
+        uint32_t loff = lane * 16;
+        asm volatile("" : "+v"(loff));      // the address of a chunk is formed here, not kept across the token loop
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c0 = i * NT + w * 64;
+            if ((C * C / 8) % NT == 0 || c0 < C * C / 8)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(img + (size_t)c0 * 16 + loff),
+                                                 (__attribute__((address_space(3))) void*)(smem + slot * WBUF + c0 * 16), 16, 0, 0);
+        }
+    };
+    auto staged = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    };
+    int woff[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) woff[ks] = ((4 * ks + g) ^ (c16 >> SWS)) << 4;
+
+    auto store_rows = [&](uint16_t* base, const u32x4* q, int64_t t, int64_t n_tok) {      // as in mlp_bwd_kernel
+        u32x4 piece[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) piece[ks] = row_piece(q[ks]);
+        const int rc = row_col(g);
+        if constexpr (KS == 1) {
+            if (t < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)t * C + rc) = piece[0];
+        } else {
+            const bool low = c16 < 8;
+#pragma unroll
+            for (int kp = 0; kp < KS; kp += 2) {
+                u32x4 send, recv, va, vb;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    send[r] = low ? piece[kp + 1][r] : piece[kp][r];
+                    recv[r] = __builtin_amdgcn_update_dpp(send[r], send[r], 0x128, 0xf, 0xf, false);     // row_ror:8
+                    va[r] = low ? piece[kp][r] : recv[r];
+                    vb[r] = low ? recv[r] : piece[kp + 1][r];
+                }
+                const int64_t ta = low ? t : t - 8, tb = low ? t + 8 : t;
+                const int col = 32 * (low ? kp : kp + 1) + rc;
+                if (ta < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)ta * C + col) = va;
+                if (tb < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)tb * C + col) = vb;
+            }
+        }
+    };
+    auto pack4 = [](const f32x4& lo, const f32x4& hi) {
+        return u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
+    };
+
+    int qcount = 0;
+    stage(0, 0);
+    staged();
+    auto step_begin = [&](int q) -> const uint8_t* {
+        const int slot = qcount & 1;
+        stage(q + 1 < Q ? q + 1 : 0, slot ^ 1);
+        return smem + slot * WBUF + c16 * RS;
+    };
+    auto step_end = [&]() {
+        staged();
+        ++qcount;
+    };
+
+    const int64_t nblk = ((int64_t)a.T + WAVES * 16 - 1) / (WAVES * 16);
+    for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
+        const int64_t t = blk * (WAVES * 16) + w * 16 + c16;
+        const bool live = t < a.T;
+        const int64_t tok = live ? t : a.T - 1;
+
+        // n = norm(x) and dy, both packed once as B operands and left as 16-bit rows
+        f32x4 xs[FT];
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft) xs[ft] = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+        float mean = 0.f, rstd = 1.f;
+        if (a.norm != 0) {
+            float s = 0.f;
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) s += xs[ft][0] + xs[ft][1] + xs[ft][2] + xs[ft][3];
+            const float rowmean = tok_sum(s) * (1.f / C);
+            mean = a.norm == 1 ? rowmean : 0.f;
+            float ss = 0.f;
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float d = xs[ft][r] - mean;
+                    ss = fmaf(d, d, ss);
+                }
+            rstd = rsqrtf(tok_sum(ss) * (1.f / C) + a.eps);
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                const f32x4 gm = *reinterpret_cast<const f32x4*>(pvec + PG * C + 16 * ft + 4 * g);
+                const f32x4 bt = *reinterpret_cast<const f32x4*>(pvec + PB * C + 16 * ft + 4 * g);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) xs[ft][r] = (xs[ft][r] - mean) * rstd * gm[r] + bt[r];
+            }
+        }
+        u32x4 nb[KS], dyb[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) nb[ks] = pack4(xs[2 * ks], xs[2 * ks + 1]);
+        store_rows(a.n_row, nb, t, a.T);
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft) {
+            xs[ft] = ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
+            if (!live) xs[ft] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) dyb[ks] = pack4(xs[2 * ks], xs[2 * ks + 1]);
+        store_rows(a.dy_row, dyb, t, a.T);
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft) xs[ft] = f32x4{0.f, 0.f, 0.f, 0.f};      // from here on: dn
+
+        for (int j = 0; j < E; ++j) {
+            u32x4 hb[KS], sl[KS], dtb[KS];
+            {   // t_j, h_j and the slopes
+                const uint8_t* wb = step_begin(3 * j);
+                auto first = [&](auto act_c) {
+                    constexpr int ACT = decltype(act_c)::value;
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        f32x4 hv[2], sv[2];
+#pragma unroll
+                        for (int half = 0; half < 2; ++half) {
+                            const int ft = 2 * ks + half;
+                            f32x4 acc = *reinterpret_cast<const f32x4*>(pvec + j * C + 16 * ft + 4 * g);
+#pragma unroll
+                            for (int k2 = 0; k2 < KS; ++k2)
+                                acc = M_::mma(*reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[k2]), nb[k2], acc);
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                float value, slope;
+                                act_and_slope<ACT>(acc[r], value, slope);
+                                hv[half][r] = value;
+                                sv[half][r] = slope;
+                            }
+                        }
+                        hb[ks] = pack4(hv[0], hv[1]);
+                        sl[ks] = pack4(sv[0], sv[1]);
+                    }
+                };
+                if (a.act == 0) first(std::integral_constant<int, 1>{}); else first(std::integral_constant<int, 2>{});
+                store_rows(a.a_in + (size_t)j * a.T * C, hb, t, a.T);
+                step_end();
+            }
+            {   // dh_j = W2[:,j]^T dy, dt_j = dh_j * act'(t_j)
+                const uint8_t* wb = step_begin(3 * j + 1);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    f32x4 dv[2];
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        const int ft = 2 * ks + half;
+                        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int k2 = 0; k2 < KS; ++k2)
+                            acc = M_::mma(*reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[k2]), dyb[k2], acc);
+                        const uint32_t s0 = sl[ks][2 * half], s1 = sl[ks][2 * half + 1];
+                        dv[half] = f32x4{acc[0] * M_::lo(s0), acc[1] * M_::hi(s0), acc[2] * M_::lo(s1), acc[3] * M_::hi(s1)};
+                    }
+                    dtb[ks] = pack4(dv[0], dv[1]);
+                }
+                store_rows(a.g_out + (size_t)j * a.T * C, dtb, t, a.T);
+                step_end();
+            }
+            {   // dn += W1[j]^T dt_j
+                const uint8_t* wb = step_begin(3 * j + 2);
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft) {
+                    f32x4 acc = xs[ft];
+#pragma unroll
+                    for (int k2 = 0; k2 < KS; ++k2)
+                        acc = M_::mma(*reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[k2]), dtb[k2], acc);
+                    xs[ft] = acc;
+                }
+                step_end();
+            }
+        }
+
+        // ---- the norm's backward, dx (as in mlp_bwd_kernel) ----
+        if (a.norm != 0) {
+            u32x4 dq[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) dq[ks] = pack4(xs[2 * ks], xs[2 * ks + 1]);
+            store_rows(a.dn, dq, t, a.T);
+            if (live && lane < 16) *reinterpret_cast<float2*>(a.stats + 2 * tok) = make_float2(mean, rstd);
+            float m1 = 0.f, m2 = 0.f;
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                const f32x4 xr = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+                const f32x4 gm = *reinterpret_cast<const f32x4*>(pvec + PG * C + 16 * ft + 4 * g);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    xs[ft][r] *= gm[r];
+                    m1 += xs[ft][r];
+                    m2 = fmaf(xs[ft][r], (xr[r] - mean) * rstd, m2);
+                }
+            }
+            m1 = a.norm == 1 ? tok_sum(m1) * (1.f / C) : 0.f;
+            m2 = tok_sum(m2) * (1.f / C);
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) {
+                const f32x4 xr = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) xs[ft][r] = rstd * (xs[ft][r] - m1 - (xr[r] - mean) * rstd * m2);
+            }
+        }
+        if (live) {
+            if (a.add_dy) {
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft) xs[ft] += ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
+            }
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) st4(a.dx, tok * a.dxs + 16 * ft + 4 * g, a.dx_dtype, xs[ft]);
+        }
+    }
+}
+
 // dgamma[c] = sum_t ds_0[t,c] xhat[t,c],  dbeta[c] = sum_t ds_0[t,c]  over the workgroup's token range.  Thread =
 // (group of four channels, token lane): 256 threads cover C / 4 groups x 1024 / C token lanes, every lane walks its
 // tokens four at a time (all loads of a group in flight together: 16 bytes of x in fp32, 8 of ds_0), the lanes meet
@@ -522,9 +774,39 @@ hipError_t launch_c(const MlpBwdArgs& a, hipStream_t st)
     return hipErrorInvalidValue;
 }
 
+template <typename T, int C, int WAVES>
+hipError_t launch_expand(const MlpBwdArgs& a, hipStream_t st)
+{
+    auto kern = mlp_bwd_expand_kernel<T, C, WAVES>;
+    const size_t lds = (size_t)2 * C * C * 2;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    const int64_t nblk = (a.T + WAVES * 16 - 1) / (WAVES * 16);
+    const int64_t cus = device_cus();
+    hipLaunchKernelGGL(kern, dim3((unsigned)(nblk < cus ? nblk : cus)), dim3(64 * WAVES), lds, st, a);
+    e = hipGetLastError();
+    if (e != hipSuccess || a.norm == 0) return e;
+    const int rows = mlp_bwd_partial_rows(a.T);
+    const int64_t tpw = (a.T + rows - 1) / rows;
+    hipLaunchKernelGGL(mlp_norm_grads_kernel<T>, dim3(rows), dim3(256), 0, st, a, tpw);
+    e = hipGetLastError();
+    if (e != hipSuccess || !a.gb) return e;
+    hipLaunchKernelGGL(mlp_sum_rows_kernel, dim3((2 * C + 63) / 64), dim3(1024), 0, st, a.gb_part, rows, 2 * C, a.gb);
+    return hipGetLastError();
+}
+
 template <typename T>
 hipError_t launch_t(const MlpBwdArgs& a, hipStream_t st)
 {
+    if (a.E > 0) {
+        if (a.E > kExpandMax) return hipErrorInvalidValue;
+        switch (a.C) {
+            case 32:  return launch_expand<T, 32, 16>(a, st);
+            case 64:  return launch_expand<T, 64, 16>(a, st);
+            case 128: return launch_expand<T, 128, 8>(a, st);
+            default:  return hipErrorInvalidValue;
+        }
+    }
     switch (a.C) {
         case 32:  return launch_c<T, 32>(a, st);
         case 64:  return launch_c<T, 64>(a, st);

@@ -85,8 +85,8 @@ __global__ __launch_bounds__(64 * WO * WI * WK) void mlp_wgrad_kernel(MlpWgradAr
     const int64_t t0 = (int64_t)blockIdx.x * a.tokens_per_wg;
     const int64_t t1 = t0 + a.tokens_per_wg < a.T ? t0 + a.tokens_per_wg : a.T;
     const int ns = (int)((t1 - t0 + KT - 1) / KT);
-    const uint16_t* gl = a.g_out + (size_t)l * a.T * C;
-    const uint16_t* al = a.a_in + (size_t)l * a.T * C;
+    const uint16_t* gl = a.g_out + (size_t)l * a.g_lstride;
+    const uint16_t* al = a.a_in + (size_t)l * a.a_lstride;
 
     // 16-byte chunk c of a row of token `tok` (tile-relative) sits at chunk c ^ swz(tok): the transposed reads of a
     // wave touch 16 consecutive rows, which without the key would all start in the same bank

@@ -100,7 +100,8 @@ _BWD_MAX_LAYERS = {32: 8, 64: 8, 128: 5}      # the backward keeps every layer's
 
 def compute_dtype(x, mod):
     """The 16-bit type the fused kernels may run this module in, or None (then torch runs it).  With gradients
-    enabled only the chain of C x C layers qualifies (the shapes flare_mlp_bwd differentiates)."""
+    enabled only the chain of C x C layers and the expanding two-layer MLP qualify (the shapes flare_mlp_bwd and
+    flare_mlp_expand_bwd differentiate)."""
     if x.device.type != "cuda":
         return None
     info = _layers_of(mod)
@@ -111,10 +112,11 @@ def compute_dtype(x, mod):
         return None
     if torch.is_grad_enabled():
         Cdim = x.shape[-1]
-        if Cdim not in _SUPPORTED_C or len(layers) > _BWD_MAX_LAYERS[Cdim]:
+        if Cdim not in _SUPPORTED_C:
             return None
-        if any(l.in_features != Cdim or l.out_features != Cdim for l in layers):
-            return None
+        if not _expand_factor(mod, Cdim):
+            if len(layers) > _BWD_MAX_LAYERS[Cdim] or any(l.in_features != Cdim or l.out_features != Cdim for l in layers):
+                return None
     io = _io_dims(mod, layers)
     if io is not None and (io[1] or io[2]):
         if io[0] not in _SUPPORTED_C or x.shape[-1] != layers[0].in_features:
@@ -345,11 +347,31 @@ def _packed_train(mod, layers, cd):
     return w, b, w_img, wt_img
 
 
-def _weight_grads(d, g_out, a_in, want_bias):
-    """dW [L, C(out), C(in)] and db [L, C] (or None) in fp32 from the rows flare_mlp_bwd left: one pass of
-    flare_mlp_wgrad over both row arrays, partial results per token range summed in a fixed order."""
+def _packed_train_expand(mod, E, cd):
+    """The same for the expanding two-layer MLP: its 2 E tiles (see _packed_expand) and their transposes as images."""
+    f1, f2 = mod.fc1, mod.fc2
+    key = ("train-expand", cd, tuple((l.weight.data_ptr(), l.weight._version, None if l.bias is None else l.bias._version)
+                                     for l in (f1, f2)))
+    cache = mod.__dict__.get("_flare_packed_train")
+    if cache is not None and cache[0] == key:
+        return cache[1:]
+    w, b = _packed_expand(mod, E, cd)
+    w_img = mlp_weight_image(w)
+    wt_img = mlp_weight_image(w.transpose(1, 2).contiguous())
+    mod.__dict__["_flare_packed_train"] = (key, w, b, w_img, wt_img)
+    return w, b, w_img, wt_img
+
+
+def _weight_grads(d, g_out, a_in, want_bias, L=None):
+    """dW [L, C(out), C(in)] and db [L, C] (or None) in fp32 from the rows the backward launch left: one pass of
+    flare_mlp_wgrad over both row arrays, partial results per token range summed in a fixed order.  g_out, a_in:
+    [L,T,C], or [T,C] for an array all L layers share."""
     lib = _lib.load()
-    L, T, Cdim = g_out.shape
+    T, Cdim = g_out.shape[-2:]
+    L = (g_out.shape[0] if g_out.dim() == 3 else a_in.shape[0]) if L is None else L
+    d2 = _lib.FlareMlpDesc()
+    d2.T, d2.C, d2.L, d2.w_dtype = T, Cdim, L, d.w_dtype
+    d = d2
     parts = C.c_int32(0)
     _lib.check(lib.flare_mlp_wgrad_partials(C.byref(d), C.byref(parts)), "flare_mlp_wgrad_partials")
     dev = g_out.device
@@ -358,8 +380,9 @@ def _weight_grads(d, g_out, a_in, want_bias):
     dw = torch.empty(L, Cdim, Cdim, dtype=torch.float32, device=dev)
     db = torch.empty(L, Cdim, dtype=torch.float32, device=dev) if want_bias else None
     with _on_device(dev):
-        rc = lib.flare_mlp_wgrad(C.byref(d), _ptr(a_in), _ptr(g_out), _ptr(dwp), _ptr(dbp), _ptr(dw), _ptr(db),
-                                 C.c_void_p(_stream_ptr(dev)))
+        rc = lib.flare_mlp_wgrad(C.byref(d), _ptr(a_in), T * Cdim if a_in.dim() == 3 else 0,
+                                 _ptr(g_out), T * Cdim if g_out.dim() == 3 else 0,
+                                 _ptr(dwp), _ptr(dbp), _ptr(dw), _ptr(db), C.c_void_p(_stream_ptr(dev)))
     _lib.check(rc, "flare_mlp_wgrad")
     return dw, db
 
@@ -388,6 +411,9 @@ class _FusedMlpFn(torch.autograd.Function):
         layers, act_mask, add_mask, act = _layers_of(mod)
         L = len(layers)
         Cdim = x.shape[-1]
+        E = _expand_factor(mod, Cdim)
+        if E:
+            return _FusedMlpFn._backward_expand(ctx, dy, x, E)
         _, b, w_img, wt_img = _packed_train(mod, layers, cd)
         x2 = x.reshape(-1, Cdim)
         if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 16:
@@ -439,6 +465,72 @@ class _FusedMlpFn(torch.autograd.Function):
         for i, l in enumerate(layers):
             grads.append(db[i].to(l.bias.dtype) if (l.bias is not None and need[8 + L + i]) else None)
         return tuple(grads)
+
+
+def _rows2d(t, Cdim):
+    t2 = t.reshape(-1, Cdim)
+    if t2.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        t2 = t2.float()
+    if t2.stride(-1) != 1 or t2.stride(0) % 4 or t2.data_ptr() % 16:
+        t2 = t2.contiguous()
+    return t2
+
+
+def _backward_expand(ctx, dy, x, E):
+    """Backward of y = res + fc2(act(fc1(norm(x)))) with hidden width E C: flare_mlp_expand_bwd, then two passes of
+    flare_mlp_wgrad (dW1, db1 from the rows dt against n; dW2, db2 from dy against the rows h)."""
+    mod, cd, norm = ctx.mod, ctx.cd, ctx.norm
+    lib = _lib.load()
+    _, _, _, act = _layers_of(mod)
+    f1, f2 = mod.fc1, mod.fc2
+    Cdim = x.shape[-1]
+    _, b, w_img, wt_img = _packed_train_expand(mod, E, cd)
+    x2, dy2 = _rows2d(x, Cdim), _rows2d(dy, Cdim)
+    T = x2.shape[0]
+    dev = x.device
+    d = _lib.FlareMlpDesc()
+    d.T, d.C, d.L, d.flags = T, Cdim, 2 * E, _lib.MLP_EXPAND
+    d.w_dtype, d.x_dtype, d.y_dtype = _dtype_code(w_img), _dtype_code(x2), _dtype_code(dy2)
+    d.act, d.act_mask, d.add_mask = act, 1, 0
+    d.x_stride, d.y_stride = x2.stride(0), dy2.stride(0)
+    gamma, beta = _norm_args(d, norm, x, Cdim)
+    dx = torch.empty(T, Cdim, dtype=x2.dtype, device=dev)
+    n_row = torch.empty(T, Cdim, dtype=cd, device=dev)
+    dy_row = torch.empty(T, Cdim, dtype=cd, device=dev)
+    h = torch.empty(E, T, Cdim, dtype=cd, device=dev)
+    dt = torch.empty(E, T, Cdim, dtype=cd, device=dev)
+    dn = stats = gb = gsum = None
+    if d.norm:
+        rows = C.c_int32(0)
+        _lib.check(lib.flare_mlp_bwd_partial_rows(C.byref(d), C.byref(rows)), "flare_mlp_bwd_partial_rows")
+        dn = torch.empty(T, Cdim, dtype=cd, device=dev)
+        stats = torch.empty(T, 2, dtype=torch.float32, device=dev)
+        gb = torch.empty(rows.value, 2, Cdim, dtype=torch.float32, device=dev)
+        gsum = torch.empty(2, Cdim, dtype=torch.float32, device=dev)
+    with _on_device(dev):
+        rc = lib.flare_mlp_expand_bwd(C.byref(d), _ptr(x2), _ptr(dy2), _ptr(w_img), _ptr(wt_img), _ptr(b), _ptr(gamma), _ptr(beta),
+                                      1 if ctx.res_is_x else 0, _ptr(dx), _ptr(n_row), _ptr(dy_row), _ptr(h), _ptr(dt),
+                                      _ptr(dn), _ptr(stats), _ptr(gb), _ptr(gsum), C.c_void_p(_stream_ptr(dev)))
+    _lib.check(rc, "flare_mlp_expand_bwd")
+    dW1, db1 = _weight_grads(d, dt, n_row, f1.bias is not None)          # [E, C(hidden chunk), C(in)], [E, C]
+    dW2, db2 = _weight_grads(d, dy_row, h, f2.bias is not None, L=E)     # [E, C(out), C(hidden chunk)], [E, C] (E equal rows)
+    need = ctx.needs_input_grad            # (mod, cd, norm, out_dtype, x, res, gamma, beta, w1, w2, b1, b2)
+    grads = [None, None, None, None]
+    grads.append(dx.view(x.shape) if need[4] else None)
+    grads.append(None if (not ctx.has_res or ctx.res_is_x or not need[5]) else dy)
+    if d.norm:
+        grads.append(gsum[0].to(norm.weight.dtype) if need[6] else None)
+        grads.append(gsum[1].to(norm.bias.dtype) if (need[7] and getattr(norm, "bias", None) is not None) else None)
+    else:
+        grads += [None, None]
+    grads.append(dW1.reshape(E * Cdim, Cdim).to(f1.weight.dtype) if need[8] else None)
+    grads.append(dW2.permute(1, 0, 2).reshape(Cdim, E * Cdim).to(f2.weight.dtype) if need[9] else None)
+    grads.append(db1.reshape(E * Cdim).to(f1.bias.dtype) if (f1.bias is not None and need[10]) else None)
+    grads.append(db2[0].to(f2.bias.dtype) if (f2.bias is not None and need[11]) else None)
+    return tuple(grads)
+
+
+_FusedMlpFn._backward_expand = staticmethod(_backward_expand)
 
 
 def _fused_mlp_train(x, mod, cd, norm, res, out_dtype):

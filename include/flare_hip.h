@@ -334,14 +334,26 @@ int flare_mlp_io_fwd(const FlareMlpDesc* desc, int32_t in_dim, int32_t in_act, c
 int flare_mlp_bwd_partial_rows(const FlareMlpDesc* desc, int32_t* rows);
 /* Weight and bias gradients from the rows flare_mlp_bwd leaves, in one pass over both (the reference gets them from
  * torch's Linear backward: dW = dt^T s, db = column sums of dt; pdebench/models/flare.py:45-59 under autograd).
- * Only T, C, L and w_dtype of the descriptor are read.  a_in, g_out [L,T,C] in the weights' type;
+ * Only T, C, L and w_dtype of the descriptor are read.  a_in, g_out: L arrays of [T,C] rows in the weights' type,
+ * a_layer_stride / g_layer_stride elements apart (T C when contiguous, 0 when all layers share one array);
  *   dw_part [parts,L,C,C] fp32: dW_l[out][in] = sum over parts of dw_part[:,l];
  *   db_part [parts,L,C]   fp32 or NULL: db_l = sum over parts of db_part[:,l]
  * with parts from flare_mlp_wgrad_partials;  dw [L,C,C], db [L,C] fp32 or NULL: those sums, formed by a second small
  * launch in index order (no atomics, two runs give the same bits). */
 int flare_mlp_wgrad_partials(const FlareMlpDesc* desc, int32_t* parts);
-int flare_mlp_wgrad(const FlareMlpDesc* desc, const void* a_in, const void* g_out, float* dw_part, float* db_part,
-                    float* dw, float* db, void* stream);
+int flare_mlp_wgrad(const FlareMlpDesc* desc, const void* a_in, int64_t a_layer_stride, const void* g_out, int64_t g_layer_stride,
+                    float* dw_part, float* db_part, float* dw, float* db, void* stream);
+/* Backward of flare_mlp_fwd with FLARE_MLP_EXPAND (y = res + W2 act(W1 norm(x) + b1) + b2, hidden width E C run as E
+ * chunks; desc as for the forward: L = 2 E tiles, flags = FLARE_MLP_EXPAND; w_img, wt_img: LDS images of the 2 E tiles
+ * and of their transposes, bias [2E,C] as for the forward).  Outputs as flare_mlp_bwd, with the rows for the weight
+ * gradients arranged per chunk:
+ *   n_row  [T,C]   norm(x) and  dy_row [T,C]  dy, both in the weights' type (shared by all chunks)
+ *   h      [E,T,C] the hidden activations of every chunk,  dt [E,T,C] the gradient at the first product
+ *   dW1[jC:(j+1)C, :] = dt[j]^T n_row,  db1[jC:(j+1)C] = column sums of dt[j]      (flare_mlp_wgrad, a stride 0)
+ *   dW2[:, jC:(j+1)C] = dy_row^T h[j],   db2 = column sums of dy_row               (flare_mlp_wgrad, g stride 0) */
+int flare_mlp_expand_bwd(const FlareMlpDesc* desc, const void* x, const void* dy, const void* w_img, const void* wt_img,
+                         const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* n_row,
+                         void* dy_row, void* h, void* dt, void* dn, float* stats, float* gb_part, float* gb, void* stream);
 int flare_mlp_bwd(const FlareMlpDesc* desc, const void* x, const void* dy, const void* w_img, const void* wt_img,
                   const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* a_in,
                   void* g_out, void* dn, float* stats, float* gb_part, float* gb, void* stream);

@@ -282,13 +282,40 @@ def test_mlp_wgrad_validation():
     assert lib.flare_mlp_wgrad_partials(m, C.byref(parts)) == _lib.FLARE_OK and parts.value == 8
     m.C, m.T = 128, 262144
     assert lib.flare_mlp_wgrad_partials(m, None) == _lib.FLARE_EINVAL
-    assert lib.flare_mlp_wgrad(m, None, fake, fake, None, None, None, None) == _lib.FLARE_EINVAL and "must not be NULL" in _lib.last_error()
-    assert lib.flare_mlp_wgrad(m, fake, fake, odd, None, None, None, None) == _lib.FLARE_EINVAL and "16-byte" in _lib.last_error()
-    assert lib.flare_mlp_wgrad(m, fake, fake, fake, None, fake, fake, None) == _lib.FLARE_EINVAL and "db needs db_part" in _lib.last_error()
+    assert lib.flare_mlp_wgrad(m, None, 0, fake, 0, fake, None, None, None, None) == _lib.FLARE_EINVAL and "must not be NULL" in _lib.last_error()
+    assert lib.flare_mlp_wgrad(m, fake, 0, fake, 0, odd, None, None, None, None) == _lib.FLARE_EINVAL and "16-byte" in _lib.last_error()
+    assert lib.flare_mlp_wgrad(m, fake, 0, fake, 0, fake, None, fake, fake, None) == _lib.FLARE_EINVAL and "db needs db_part" in _lib.last_error()
     m.C = 96
-    assert lib.flare_mlp_wgrad(m, fake, fake, fake, None, None, None, None) == _lib.FLARE_EUNSUPPORTED
+    assert lib.flare_mlp_wgrad(m, fake, 0, fake, 0, fake, None, None, None, None) == _lib.FLARE_EUNSUPPORTED
     m.C, m.w_dtype = 128, _lib.DT_F32
-    assert lib.flare_mlp_wgrad(m, fake, fake, fake, None, None, None, None) == _lib.FLARE_EINVAL and "w_dtype" in _lib.last_error()
-    m.w_dtype, m.L = _lib.DT_BF16, 0
+    assert lib.flare_mlp_wgrad(m, fake, 0, fake, 0, fake, None, None, None, None) == _lib.FLARE_EINVAL and "w_dtype" in _lib.last_error()
+    m.w_dtype = _lib.DT_BF16
+    assert lib.flare_mlp_wgrad(m, fake, 4, fake, 0, fake, None, None, None, None) == _lib.FLARE_EINVAL and "layer strides" in _lib.last_error()
+    m.L = 0
     assert lib.flare_mlp_wgrad_partials(m, C.byref(parts)) == _lib.FLARE_EINVAL
     assert big >= 64
+
+
+def test_mlp_expand_bwd_validation():
+    lib = _lib.load()
+    m = _lib.FlareMlpDesc()
+    m.T, m.C, m.L, m.flags = 64, 128, 8, _lib.MLP_EXPAND
+    m.x_dtype = m.y_dtype = m.w_dtype = _lib.DT_BF16
+    m.norm, m.act, m.eps = 1, 0, 1e-5
+    m.x_stride = m.y_stride = 128
+    fake, odd = C.c_void_p(4096), C.c_void_p(4100)
+
+    def call(x=fake, h=fake, gamma=fake, dn=fake):
+        return lib.flare_mlp_expand_bwd(m, x, fake, fake, fake, fake, gamma, fake, 0, fake, fake, fake, h, fake, dn, fake, fake, None, None)
+
+    assert call(x=None) == _lib.FLARE_EINVAL and "must not be NULL" in _lib.last_error()
+    assert call(h=odd) == _lib.FLARE_EINVAL and "16-byte" in _lib.last_error()
+    assert call(gamma=None) == _lib.FLARE_EINVAL and "norm" in _lib.last_error()
+    m.L = 7
+    assert call() == _lib.FLARE_EUNSUPPORTED and "2 E tiles" in _lib.last_error()
+    m.L = 18
+    assert call() == _lib.FLARE_EUNSUPPORTED
+    m.L, m.flags = 8, 0
+    assert call() == _lib.FLARE_EINVAL and "FLARE_MLP_EXPAND" in _lib.last_error()
+    m.flags, m.C = _lib.MLP_EXPAND, 96
+    assert call() == _lib.FLARE_EUNSUPPORTED

@@ -156,15 +156,102 @@ def test_block_trains_through_the_fused_launches(dev, C, H, M, N):
 
 
 def test_shapes_without_a_backward_keep_their_torch_layers(dev):
-    """With gradients enabled compute_dtype admits the C x C chain only."""
+    """With gradients enabled compute_dtype admits the C x C chain and the expanding two-layer MLP only."""
     x = torch.randn(10, 64, device=dev)
     with torch.autocast("cuda", torch.bfloat16):
         assert fused.compute_dtype(x, ResidualMLP(64, 64, 64, num_layers=3).to(dev)) == torch.bfloat16
-        assert fused.compute_dtype(x, ResidualMLP(64, 256, 64, num_layers=0, input_residual=False, output_residual=False).to(dev)) is None
+        assert fused.compute_dtype(x, ResidualMLP(64, 256, 64, num_layers=0, input_residual=False, output_residual=False).to(dev)) == torch.bfloat16
+        assert fused.compute_dtype(x, ResidualMLP(64, 256, 64, num_layers=1, input_residual=False, output_residual=False).to(dev)) is None   # wide hidden stream
+        assert fused.compute_dtype(torch.randn(10, 3, device=dev), ResidualMLP(3, 64, 64, num_layers=2, input_residual=False).to(dev)) is None   # narrow end
         assert fused.compute_dtype(x, ResidualMLP(64, 64, 64, num_layers=9).to(dev)) is None          # 11 layers: above the limit
         assert fused.compute_dtype(torch.randn(10, 128, device=dev), ResidualMLP(128, 128, 128, num_layers=4).to(dev)) is None
         with torch.no_grad():
-            assert fused.compute_dtype(x, ResidualMLP(64, 256, 64, num_layers=0, input_residual=False, output_residual=False).to(dev)) == torch.bfloat16
+            assert fused.compute_dtype(torch.randn(10, 3, device=dev), ResidualMLP(3, 64, 64, num_layers=2, input_residual=False).to(dev)) == torch.bfloat16
     with pytest.raises(ValueError):
         with torch.autocast("cuda", torch.bfloat16):
             fused.fused_mlp(torch.randn(10, 128, device=dev), ResidualMLP(64, 64, 64, num_layers=1).to(dev), torch.bfloat16, x_head=8)
+
+
+@pytest.mark.parametrize("C,E,T,norm_kind,dtype,act,res", [
+    (128, 4, 700, "ln", torch.bfloat16, "gelu", "x"), (64, 2, 1000, "rms", torch.bfloat16, "silu", "x"),
+    (32, 8, 333, "ln", torch.float16, "gelu", "other"), (128, 2, 33000, "ln", torch.bfloat16, "gelu", None),
+    (64, 4, 19, None, torch.bfloat16, "gelu", "x")])
+def test_expanding_mlp_gradients_against_fp32_torch_layers(dev, C, E, T, norm_kind, dtype, act, res):
+    """y = res + fc2(act(fc1(norm(x)))) with hidden width E C (ResidualMLP with num_layers=0, the "4x" feed-forward
+    block): flare_mlp_expand_bwd and two passes of flare_mlp_wgrad behind autograd."""
+    torch.manual_seed(C + E + T)
+    mod = ResidualMLP(C, E * C, C, num_layers=0, act=act, input_residual=False, output_residual=False).to(dev)
+    norm = None if norm_kind is None else (nn.LayerNorm(C) if norm_kind == "ln" else nn.RMSNorm(C)).to(dev)
+    with torch.no_grad():
+        if norm is not None:
+            norm.weight.uniform_(0.5, 1.5)
+            if getattr(norm, "bias", None) is not None:
+                norm.bias.uniform_(-0.3, 0.3)
+        for p in mod.parameters():
+            p.mul_(2.0) if p.dim() == 2 else p.uniform_(-0.5, 0.5)
+    x = torch.randn(2, T, C, device=dev, requires_grad=True)
+    other = torch.randn(2, T, C, device=dev, requires_grad=True)
+    gy = torch.randn(2, T, C, device=dev)
+    params = list(mod.parameters()) + ([] if norm is None else list(norm.parameters())) + ([other] if res == "other" else [])
+    r = lambda: x if res == "x" else other if res == "other" else None
+
+    def layers():
+        y = mod(norm(x) if norm is not None else x)
+        return y if r() is None else r() + y
+
+    def hip():
+        with torch.autocast("cuda", dtype):
+            cd = fused.compute_dtype(x, mod)
+            assert cd == dtype
+            return fused.fused_mlp(x, mod, cd, norm=norm, res=r())
+
+    def torch16():
+        with torch.autocast("cuda", dtype):
+            return layers()
+
+    ref, t16, got = _run(layers, x, params, gy), _run(torch16, x, params, gy), _run(hip, x, params, gy)
+    assert len(got) == len(ref) == 2 + len(params)
+    for i, (g, t, rr) in enumerate(zip(got, t16, ref)):
+        e = rel(g, rr)
+        assert torch.isfinite(g).all()
+        assert e <= 3e-2, f"tensor {i}: rel-L2 {e:.3e} (torch layers under autocast: {rel(t, rr):.3e})"
+    again = _run(hip, x, params, gy)
+    assert all(torch.equal(p, q) for p, q in zip(got, again))          # no atomics anywhere: same bits
+
+
+def test_block_with_expanding_ffn_trains_fused(dev):
+    """The block of BASELINE config 2 as worded (feed-forward = GELU MLP with 4x expansion): under autocast with
+    gradients enabled every MLP of the block runs through the fused launches; gradients against fp32 torch layers."""
+    from torch.profiler import ProfilerActivity, profile
+    torch.manual_seed(11)
+    blk = F.FLAREBlock(channel_dim=64, num_heads=4, num_latents=64, num_layers_ffn=0, ffn_mlp_ratio=4.0).to(dev)
+    x = torch.randn(2, 2000, 64, device=dev, requires_grad=True)
+    gy = torch.randn(2, 2000, 64, device=dev)
+    params = [p for p in blk.parameters()]
+
+    def run(kind):
+        for p in params + [x]:
+            p.grad = None
+        if kind == "fp32":
+            y = blk(x)[0]
+        else:
+            real = fused.compute_dtype
+            if kind == "torch16":
+                fused.compute_dtype = lambda *a, **k: None
+            try:
+                with torch.autocast("cuda", torch.bfloat16):
+                    y = blk(x)[0]
+            finally:
+                fused.compute_dtype = real
+        y.float().backward(gy)
+        return [y.detach().float(), x.grad.clone()] + [p.grad.clone() for p in params]
+
+    ref, t16 = run("fp32"), run("torch16")
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        got = run("hip")
+        torch.cuda.synchronize()
+    names = " ".join(e.key for e in prof.key_averages())
+    assert "mlp_bwd_expand_kernel" in names and "mlp_wgrad_kernel" in names and "mlp_bwd_kernel" in names
+    for i, (g, t, r) in enumerate(zip(got, t16, ref)):
+        e, et = rel(g, r), rel(t, r)
+        assert e <= min(6e-2, max(3e-2, 2 * et)), f"tensor {i}: rel-L2 {e:.3e} (torch layers under autocast: {et:.3e})"
