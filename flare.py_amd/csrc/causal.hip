@@ -109,12 +109,13 @@ __global__ __launch_bounds__(kThreads) void causal_generic_kernel(CausalArgs a)
     for (int idx = tid; idx < M * D; idx += kThreads) {
         const int m = idx / D, d = idx - m * D;
         qs[m * (D + 1) + d] = to_f32(q[(int64_t)m * a.qs[2] + d]) * sl2;
-        U[idx] = mu_g[m] <= kNegBig ? 0.f : num_g[idx];      // a fresh latent's sums are not read (they may be uninitialised)
+        const float mu = mu_g[m], un = num_g[idx];
+        U[idx] = mu <= kNegBig ? 0.f : un;                   // a fresh latent's sums are dropped (they may be uninitialised)
     }
     for (int m = tid; m < M; m += kThreads) {
-        const float mu = mu_g[m];
+        const float mu = mu_g[m], dn = den_g[m];
         mu_s[m] = mu <= kNegBig ? kNegBig : mu * kLog2e;
-        den_s[m] = mu <= kNegBig ? 0.f : den_g[m];
+        den_s[m] = mu <= kNegBig ? 0.f : dn;
     }
 
     for (int n0 = 0; n0 < N; n0 += TB) {

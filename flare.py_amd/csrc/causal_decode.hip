@@ -94,9 +94,12 @@ __global__ __launch_bounds__(64 * kDecWaves) void causal_decode_kernel(CausalArg
 
     // one shift for the softmax over latents: the largest per-latent shift of the incoming state
     float cref = kNegBig;
-    for (int m = lane; m < M; m += 64) {
-        const float mu = mu_g[m];
-        cref = fmaxf(cref, mu <= kNegBig ? 0.f : mu * kLog2e);
+    for (int m = lane; m < M; m += 256) {          // up to four loads in flight (M <= 256: one round trip)
+        float mu[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) mu[u] = mu_g[m + 64 * u < M ? m + 64 * u : m];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) cref = fmaxf(cref, mu[u] <= kNegBig ? 0.f : mu[u] * kLog2e);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) cref = fmaxf(cref, __shfl_xor(cref, o));
@@ -115,15 +118,22 @@ __global__ __launch_bounds__(64 * kDecWaves) void causal_decode_kernel(CausalArg
     const bool fresh = mu_in <= kNegBig;
     const float mu0 = fresh ? 0.f : mu_in * kLog2e;
     const float fw = fast_exp2(mu0 - cref);
-    float den = fresh ? 0.f : den_g[m_s];
+    const float den_in = den_g[m_s];       // read whether fresh or not: a load under the condition would wait for mu first
+    float den = fresh ? 0.f : den_in;
 
     // state stage: column d, latents w * MW + mp * ML + j
     const int d = lane % D, mp = lane / D;
     float U[ML];
+    {
+        float mu_j[ML];
 #pragma unroll
-    for (int j = 0; j < ML; ++j) {
-        const int m = w * MW + mp * ML + j;
-        U[j] = mu_g[m] <= kNegBig ? 0.f : num_g[(int64_t)m * D + d];
+        for (int j = 0; j < ML; ++j) {
+            const int m = w * MW + mp * ML + j;
+            mu_j[j] = mu_g[m];
+            U[j] = num_g[(int64_t)m * D + d];      // all loads in flight together; a fresh latent's sums are dropped below
+        }
+#pragma unroll
+        for (int j = 0; j < ML; ++j) U[j] = mu_j[j] <= kNegBig ? 0.f : U[j];
     }
 
     // k_t and v_t arrive kPF steps ahead of their use: a step is shorter than the latency of the loads

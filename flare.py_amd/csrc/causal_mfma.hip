@@ -95,9 +95,12 @@ __device__ __forceinline__ uint2 tr16(const void* lds_addr)
 __device__ __forceinline__ float common_shift(const float* mu_g, int M, int lane)
 {
     float mx = kNegBig;
-    for (int m = lane; m < M; m += 64) {
-        const float mu = mu_g[m];
-        mx = fmaxf(mx, mu <= kNegBig ? 0.f : mu * kLog2e);
+    for (int m = lane; m < M; m += 256) {          // up to four loads in flight (M <= 256: one round trip)
+        float mu[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) mu[u] = mu_g[m + 64 * u < M ? m + 64 * u : m];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) mx = fmaxf(mx, mu[u] <= kNegBig ? 0.f : mu[u] * kLog2e);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
@@ -168,7 +171,11 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
         const float mu = mu_g[m];
         mu0[ct] = mu <= kNegBig ? 0.f : mu * kLog2e;
         negmu[ct] = f32x4{-mu0[ct], -mu0[ct], -mu0[ct], -mu0[ct]};
-        float d0 = (STATE_ONLY || mu <= kNegBig) ? 0.f : den_g[m];
+        float d0 = 0.f;
+        if constexpr (!STATE_ONLY) {
+            const float dn_in = den_g[m];          // read whether the latent is fresh or not (no load behind a wait for mu)
+            d0 = mu <= kNegBig ? 0.f : dn_in;
+        }
         if (!STATE_ONLY)
             for (int s = 0; s < seg; ++s) d0 += a.seg_den[((int64_t)bh * a.n_segs + s) * M + m];
         den[ct] = f32x4{d0, d0, d0, d0};
@@ -182,7 +189,11 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = m0 + mt * 16 + 4 * g + r;
-                float u = (STATE_ONLY || mu_g[m] <= kNegBig) ? 0.f : num_g[(int64_t)m * D + dt * 16 + c16];
+                float u = 0.f;
+                if constexpr (!STATE_ONLY) {
+                    const float mu_m = mu_g[m], un = num_g[(int64_t)m * D + dt * 16 + c16];
+                    u = mu_m <= kNegBig ? 0.f : un;
+                }
                 if (!STATE_ONLY)
                     for (int s = 0; s < seg; ++s)
                         u += a.seg_num[(((int64_t)bh * a.n_segs + s) * M + m) * D + dt * 16 + c16];
@@ -590,23 +601,40 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     // running denominators of every latent (column c16 of tile ct), replicated in the waves
     // (the earlier segments' local states are added segment by segment, in segment order: every load of one
     // segment's contribution is issued before the first is consumed, instead of one round trip per element)
+    // (state of a fresh latent: its sums are read all the same and replaced by zeros.  A load under "if the
+    // latent is not fresh" waits for the latent's mu first: one trip to memory after the other, 8 + 16 of them here)
     float den0[CTA];
+    {
+        float mu_c[CTA], dn_c[CTA];
 #pragma unroll
-    for (int ct = 0; ct < CTA; ++ct) {
-        const int m = ct * 16 + c16;
-        den0[ct] = mu_g[m] <= kNegBig ? 0.f : den_g[m];
+        for (int ct = 0; ct < CTA; ++ct) {
+            mu_c[ct] = mu_g[ct * 16 + c16];
+            dn_c[ct] = den_g[ct * 16 + c16];
+        }
+#pragma unroll
+        for (int ct = 0; ct < CTA; ++ct) den0[ct] = mu_c[ct] <= kNegBig ? 0.f : dn_c[ct];
     }
     // state numerator of the wave's own latents: tile (mt, dt) holds rows m0 + 16 mt + 4g + r, column 16 dt + c16
     f32x4 U[MT][DT];
+    {
+        float mu_r[MT][4];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+            for (int r = 0; r < 4; ++r) mu_r[mt][r] = mu_g[m0 + mt * 16 + 4 * g + r];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int m = m0 + mt * 16 + 4 * g + r;
-                U[mt][dt][r] = mu_g[m] <= kNegBig ? 0.f : num_g[(int64_t)m * D + dt * 16 + c16];
-            }
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) U[mt][dt][r] = num_g[(int64_t)(m0 + mt * 16 + 4 * g + r) * D + dt * 16 + c16];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) U[mt][dt][r] = mu_r[mt][r] <= kNegBig ? 0.f : U[mt][dt][r];
+    }
     for (int s = 0; s < seg; ++s) {
         const float* sd = a.seg_den + ((int64_t)bh * a.n_segs + s) * M;
         const float* sn = a.seg_num + ((int64_t)bh * a.n_segs + s) * M * D;
