@@ -819,9 +819,10 @@ int flare_mlp_bwd_partial_rows(const FlareMlpDesc* d, int32_t* rows)
     return FLARE_OK;
 }
 
-int flare_mlp_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const void* w_img, const void* wt_img,
-                  const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* a_in,
-                  void* g_out, void* dn, float* stats, float* gb_part, float* gb, void* stream)
+// what flare_mlp_bwd and flare_mlp_expand_bwd ask of the descriptor and of the buffers they share
+static int check_mlp_bwd_common(const FlareMlpDesc* d, const void* x, const void* dy, const void* w_img, const void* wt_img,
+                                const float* bias, const float* gamma, const float* beta, const void* dx, const void* dn,
+                                const float* stats, const float* gb_part, const float* gb)
 {
     if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
     if (d->T < 1 || d->L < 1) return fail(FLARE_EINVAL, "T >= 1 and L >= 1 required (got %lld, %d)", (long long)d->T, d->L);
@@ -831,20 +832,30 @@ int flare_mlp_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const vo
     if (d->norm < FLARE_NORM_NONE || d->norm > FLARE_NORM_RMS) return fail(FLARE_EINVAL, "unknown norm %d", d->norm);
     if (d->act < FLARE_ACT_GELU_TANH || d->act > FLARE_ACT_SILU) return fail(FLARE_EINVAL, "unknown activation %d", d->act);
     if (!flare::mlp_mfma_supported(d->w_dtype, d->C)) return fail(FLARE_EUNSUPPORTED, "C=%d: only 32, 64 and 128 are supported", d->C);
-    if (d->L > flare::mlp_bwd_max_layers(d->C))
-        return fail(FLARE_EUNSUPPORTED, "the backward keeps every layer's slopes in registers: at most %d layers at C=%d (got %d)",
-                    flare::mlp_bwd_max_layers(d->C), d->C, d->L);
-    if (d->flags != 0) return fail(FLARE_EUNSUPPORTED, "the backward covers the chain of C x C layers only (flags must be 0)");
-    if (!x || !dy || !w_img || !wt_img || !dx || !a_in || !g_out) return fail(FLARE_EINVAL, "x, dy, w_img, wt_img, dx, a_in, g_out must not be NULL");
+    if (!x || !dy || !w_img || !wt_img || !dx) return fail(FLARE_EINVAL, "x, dy, w_img, wt_img and dx must not be NULL");
     if (d->norm != FLARE_NORM_NONE && (!gamma || !dn || !stats || !gb_part))
         return fail(FLARE_EINVAL, "gamma, dn, stats and gb_part must not be NULL when a norm is requested");
     if (d->norm != FLARE_NORM_NONE && !(d->eps >= 0.f)) return fail(FLARE_EINVAL, "eps must be >= 0");
     if (d->x_stride < d->C || d->x_stride % 4 || !aligned16(x)) return fail(FLARE_EINVAL, "x: row stride >= C, a multiple of 4, base 16-byte aligned");
     if (d->y_stride < d->C || d->y_stride % 4 || !aligned16(dy)) return fail(FLARE_EINVAL, "dy: row stride (y_stride) >= C, a multiple of 4, base 16-byte aligned");
-    if (!aligned16(dx) || !aligned16(a_in) || !aligned16(g_out) || !aligned16(w_img) || !aligned16(wt_img) ||
-        (bias && !aligned16(bias)) || (gamma && !aligned16(gamma)) || (beta && !aligned16(beta)) || (dn && !aligned16(dn)) ||
-        (stats && !aligned16(stats)))
-        return fail(FLARE_EINVAL, "every buffer must be 16-byte aligned");
+    const void* ptrs[] = {dx, w_img, wt_img, bias, gamma, beta, dn, stats, gb_part, gb};
+    for (const void* p : ptrs)
+        if (p && !aligned16(p)) return fail(FLARE_EINVAL, "every buffer must be 16-byte aligned");
+    return FLARE_OK;
+}
+
+int flare_mlp_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const void* w_img, const void* wt_img,
+                  const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* a_in,
+                  void* g_out, void* dn, float* stats, float* gb_part, float* gb, void* stream)
+{
+    int rc = check_mlp_bwd_common(d, x, dy, w_img, wt_img, bias, gamma, beta, dx, dn, stats, gb_part, gb);
+    if (rc != FLARE_OK) return rc;
+    if (d->flags != 0) return fail(FLARE_EUNSUPPORTED, "the backward covers the chain of C x C layers only (flags must be 0)");
+    if (d->L > flare::mlp_bwd_max_layers(d->C))
+        return fail(FLARE_EUNSUPPORTED, "the backward keeps every layer's slopes in registers: at most %d layers at C=%d (got %d)",
+                    flare::mlp_bwd_max_layers(d->C), d->C, d->L);
+    if (!a_in || !g_out) return fail(FLARE_EINVAL, "a_in and g_out must not be NULL");
+    if (!aligned16(a_in) || !aligned16(g_out)) return fail(FLARE_EINVAL, "every buffer must be 16-byte aligned");
     flare::MlpBwdArgs a;
     memset(&a, 0, sizeof(a));
     a.x = x; a.dy = dy; a.dx = dx;
@@ -864,26 +875,12 @@ int flare_mlp_expand_bwd(const FlareMlpDesc* d, const void* x, const void* dy, c
                          const float* bias, const float* gamma, const float* beta, int32_t add_dy, void* dx, void* n_row,
                          void* dy_row, void* h, void* dt, void* dn, float* stats, float* gb_part, float* gb, void* stream)
 {
-    if (!d) return fail(FLARE_EINVAL, "descriptor is NULL");
-    if (d->T < 1) return fail(FLARE_EINVAL, "T >= 1 required");
+    int rc = check_mlp_bwd_common(d, x, dy, w_img, wt_img, bias, gamma, beta, dx, dn, stats, gb_part, gb);
+    if (rc != FLARE_OK) return rc;
     if (d->flags != FLARE_MLP_EXPAND) return fail(FLARE_EINVAL, "flags must be FLARE_MLP_EXPAND");
     if (d->L < 4 || d->L > 16 || (d->L & 1)) return fail(FLARE_EUNSUPPORTED, "L = 2 E tiles with 2 <= E <= 8 (got L = %d)", d->L);
-    if (d->w_dtype != FLARE_DT_BF16 && d->w_dtype != FLARE_DT_F16) return fail(FLARE_EINVAL, "w_dtype must be bf16 or f16");
-    if (d->x_dtype < FLARE_DT_F32 || d->x_dtype > FLARE_DT_F16 || d->y_dtype < FLARE_DT_F32 || d->y_dtype > FLARE_DT_F16)
-        return fail(FLARE_EINVAL, "unknown dtype");
-    if (d->norm < FLARE_NORM_NONE || d->norm > FLARE_NORM_RMS) return fail(FLARE_EINVAL, "unknown norm %d", d->norm);
-    if (d->act < FLARE_ACT_GELU_TANH || d->act > FLARE_ACT_SILU) return fail(FLARE_EINVAL, "unknown activation %d", d->act);
-    if (!flare::mlp_mfma_supported(d->w_dtype, d->C)) return fail(FLARE_EUNSUPPORTED, "C=%d: only 32, 64 and 128 are supported", d->C);
-    if (!x || !dy || !w_img || !wt_img || !dx || !n_row || !dy_row || !h || !dt)
-        return fail(FLARE_EINVAL, "x, dy, w_img, wt_img, dx, n_row, dy_row, h, dt must not be NULL");
-    if (d->norm != FLARE_NORM_NONE && (!gamma || !dn || !stats || !gb_part))
-        return fail(FLARE_EINVAL, "gamma, dn, stats and gb_part must not be NULL when a norm is requested");
-    if (d->norm != FLARE_NORM_NONE && !(d->eps >= 0.f)) return fail(FLARE_EINVAL, "eps must be >= 0");
-    if (d->x_stride < d->C || d->x_stride % 4 || !aligned16(x)) return fail(FLARE_EINVAL, "x: row stride >= C, a multiple of 4, base 16-byte aligned");
-    if (d->y_stride < d->C || d->y_stride % 4 || !aligned16(dy)) return fail(FLARE_EINVAL, "dy: row stride (y_stride) >= C, a multiple of 4, base 16-byte aligned");
-    const void* ptrs[] = {dx, n_row, dy_row, h, dt, w_img, wt_img, bias, gamma, beta, dn, stats, gb};
-    for (const void* p : ptrs)
-        if (p && !aligned16(p)) return fail(FLARE_EINVAL, "every buffer must be 16-byte aligned");
+    if (!n_row || !dy_row || !h || !dt) return fail(FLARE_EINVAL, "n_row, dy_row, h and dt must not be NULL");
+    if (!aligned16(n_row) || !aligned16(dy_row) || !aligned16(h) || !aligned16(dt)) return fail(FLARE_EINVAL, "every buffer must be 16-byte aligned");
     flare::MlpBwdArgs a;
     memset(&a, 0, sizeof(a));
     a.x = x; a.dy = dy; a.dx = dx;

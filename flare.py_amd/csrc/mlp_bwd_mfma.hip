@@ -107,6 +107,41 @@ __device__ __forceinline__ u32x4 row_piece(u32x4 q)
 }
 __device__ __forceinline__ int row_col(int g) { return (g & 1) ? 12 + 4 * g : 4 * g; }
 
+// A [T,C] 16-bit row array receives a wave's 16 tokens from packed operand quads.  After row_piece a token's four
+// lanes hold 64 contiguous bytes per k-step; the two half-rows of 8 lanes then trade pieces of neighbouring k-steps
+// (one rotate by 8 within each 16 lanes), so that one store instruction completes 128-byte lines: the first for
+// tokens 0-7 of the tile, the second for tokens 8-15.  t: the lane's token, n_tok: tokens in the array.  All lanes
+// of the wave must be active.
+template <int C>
+__device__ __forceinline__ void store_rows(uint16_t* base, const u32x4* q, int64_t t, int64_t n_tok, int g, int c16)
+{
+    constexpr int KS = C / 32;
+    u32x4 piece[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) piece[ks] = row_piece(q[ks]);
+    const int rc = row_col(g);
+    if constexpr (KS == 1) {
+        if (t < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)t * C + rc) = piece[0];
+    } else {
+        const bool low = c16 < 8;
+#pragma unroll
+        for (int kp = 0; kp < KS; kp += 2) {
+            u32x4 send, recv, va, vb;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                send[r] = low ? piece[kp + 1][r] : piece[kp][r];
+                recv[r] = __builtin_amdgcn_update_dpp(send[r], send[r], 0x128, 0xf, 0xf, false);     // row_ror:8
+                va[r] = low ? piece[kp][r] : recv[r];
+                vb[r] = low ? recv[r] : piece[kp + 1][r];
+            }
+            const int64_t ta = low ? t : t - 8, tb = low ? t + 8 : t;
+            const int col = 32 * (low ? kp : kp + 1) + rc;
+            if (ta < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)ta * C + col) = va;
+            if (tb < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)tb * C + col) = vb;
+        }
+    }
+}
+
 // act(t) = t * gate and its derivative.  tanh-GELU: gate = sigmoid(2u), 2u = t (1.5957691 + 0.0713548 t^2), so
 // act' = gate (1 + t (1 - gate) (1.5957691 + 0.2140645 t^2));  SiLU: gate = sigmoid(t), act' = gate (1 + t (1 - gate)).
 template <int ACT>
@@ -183,41 +218,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) woff[ks] = ((4 * ks + g) ^ (c16 >> SWS)) << 4;
 
-    // A [T,C] 16-bit row array receives the wave's 16 tokens from packed operand quads.  After row_piece a token's
-    // four lanes hold 64 contiguous bytes per k-step; the two half-rows of 8 lanes then trade pieces of neighbouring
-    // k-steps (one rotate by 8 within each 16 lanes), so that one store instruction completes 128-byte lines: the
-    // first for tokens 0-7 of the tile, the second for tokens 8-15.
-    auto store_rows = [&](uint16_t* base, const u32x4* q, int64_t t, int64_t n_tok) {
-        u32x4 piece[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) piece[ks] = row_piece(q[ks]);
-        const int rc = row_col(g);
-        if constexpr (KS == 1) {
-            if (t < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)t * C + rc) = piece[0];
-        } else {
-            const bool low = c16 < 8;
-#pragma unroll
-            for (int kp = 0; kp < KS; kp += 2) {
-                u32x4 send, recv;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    send[r] = low ? piece[kp + 1][r] : piece[kp][r];
-                    recv[r] = __builtin_amdgcn_update_dpp(send[r], send[r], 0x128, 0xf, 0xf, false);     // row_ror:8
-                }
-                u32x4 va, vb;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    va[r] = low ? piece[kp][r] : recv[r];
-                    vb[r] = low ? recv[r] : piece[kp + 1][r];
-                }
-                const int64_t ta = low ? t : t - 8, tb = low ? t + 8 : t;
-                const int col = 32 * (low ? kp : kp + 1) + rc;
-                if (ta < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)ta * C + col) = va;
-                if (tb < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)tb * C + col) = vb;
-            }
-        }
-    };
-
     int qcount = 0;      // ring mode: steps done by this workgroup; its parity names the slot in use
     if (resident) {
         for (int q = 0; q < 2 * L; ++q) stage(q, q);
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
                 const f32x4 lo = xs[2 * ks], hi = xs[2 * ks + 1];
                 xb[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
             }
-            store_rows(a.a_in + (size_t)l * a.T * C, xb, t, a.T);      // s_l, the input of layer l, as a 16-bit row (for dW_l)
+            store_rows<C>(a.a_in + (size_t)l * a.T * C, xb, t, a.T, g, c16);      // s_l, the input of layer l, as a 16-bit row (for dW_l)
             const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
             auto layer = [&](auto act_c, auto add_c) {
                 constexpr int ACT = decltype(act_c)::value;
@@ -347,7 +347,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
                 }
                 db[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
             }
-            store_rows(a.g_out + (size_t)l * a.T * C, db, t, a.T);
+            store_rows<C>(a.g_out + (size_t)l * a.T * C, db, t, a.T, g, c16);
             // ds_l = (ds_{l+1} if the layer added to the stream) + W_l^T dt_l
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
@@ -371,7 +371,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
                 const f32x4 lo = xs[2 * ks], hi = xs[2 * ks + 1];
                 dq[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
             }
-            store_rows(a.dn, dq, t, a.T);
+            store_rows<C>(a.dn, dq, t, a.T, g, c16);
             if (live && lane < 16) *reinterpret_cast<float2*>(a.stats + 2 * tok) = make_float2(mean, rstd);
             float m1 = 0.f, m2 = 0.f;
 #pragma unroll
@@ -462,32 +462,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) woff[ks] = ((4 * ks + g) ^ (c16 >> SWS)) << 4;
 
-    auto store_rows = [&](uint16_t* base, const u32x4* q, int64_t t, int64_t n_tok) {      // as in mlp_bwd_kernel
-        u32x4 piece[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) piece[ks] = row_piece(q[ks]);
-        const int rc = row_col(g);
-        if constexpr (KS == 1) {
-            if (t < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)t * C + rc) = piece[0];
-        } else {
-            const bool low = c16 < 8;
-#pragma unroll
-            for (int kp = 0; kp < KS; kp += 2) {
-                u32x4 send, recv, va, vb;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    send[r] = low ? piece[kp + 1][r] : piece[kp][r];
-                    recv[r] = __builtin_amdgcn_update_dpp(send[r], send[r], 0x128, 0xf, 0xf, false);     // row_ror:8
-                    va[r] = low ? piece[kp][r] : recv[r];
-                    vb[r] = low ? recv[r] : piece[kp + 1][r];
-                }
-                const int64_t ta = low ? t : t - 8, tb = low ? t + 8 : t;
-                const int col = 32 * (low ? kp : kp + 1) + rc;
-                if (ta < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)ta * C + col) = va;
-                if (tb < n_tok) *reinterpret_cast<u32x4*>(base + (size_t)tb * C + col) = vb;
-            }
-        }
-    };
     auto pack4 = [](const f32x4& lo, const f32x4& hi) {
         return u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
     };
@@ -542,7 +516,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
         u32x4 nb[KS], dyb[KS];
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) nb[ks] = pack4(xs[2 * ks], xs[2 * ks + 1]);
-        store_rows(a.n_row, nb, t, a.T);
+        store_rows<C>(a.n_row, nb, t, a.T, g, c16);
 #pragma unroll
         for (int ft = 0; ft < FT; ++ft) {
             xs[ft] = ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
@@ -550,7 +524,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
         }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) dyb[ks] = pack4(xs[2 * ks], xs[2 * ks + 1]);
-        store_rows(a.dy_row, dyb, t, a.T);
+        store_rows<C>(a.dy_row, dyb, t, a.T, g, c16);
 #pragma unroll
         for (int ft = 0; ft < FT; ++ft) xs[ft] = f32x4{0.f, 0.f, 0.f, 0.f};      // from here on: dn
 
@@ -583,7 +557,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
                     }
                 };
                 if (a.act == 0) first(std::integral_constant<int, 1>{}); else first(std::integral_constant<int, 2>{});
-                store_rows(a.a_in + (size_t)j * a.T * C, hb, t, a.T);
+                store_rows<C>(a.a_in + (size_t)j * a.T * C, hb, t, a.T, g, c16);
                 step_end();
             }
             {   // dh_j = W2[:,j]^T dy, dt_j = dh_j * act'(t_j)
@@ -603,7 +577,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
                     }
                     dtb[ks] = pack4(dv[0], dv[1]);
                 }
-                store_rows(a.g_out + (size_t)j * a.T * C, dtb, t, a.T);
+                store_rows<C>(a.g_out + (size_t)j * a.T * C, dtb, t, a.T, g, c16);
                 step_end();
             }
             {   // dn += W1[j]^T dt_j
@@ -625,7 +599,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
             u32x4 dq[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) dq[ks] = pack4(xs[2 * ks], xs[2 * ks + 1]);
-            store_rows(a.dn, dq, t, a.T);
+            store_rows<C>(a.dn, dq, t, a.T, g, c16);
             if (live && lane < 16) *reinterpret_cast<float2*>(a.stats + 2 * tok) = make_float2(mean, rstd);
             float m1 = 0.f, m2 = 0.f;
 #pragma unroll

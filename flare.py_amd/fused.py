@@ -413,7 +413,7 @@ class _FusedMlpFn(torch.autograd.Function):
         Cdim = x.shape[-1]
         E = _expand_factor(mod, Cdim)
         if E:
-            return _FusedMlpFn._backward_expand(ctx, dy, x, E)
+            return _backward_expand(ctx, dy, x, E)
         _, b, w_img, wt_img = _packed_train(mod, layers, cd)
         x2 = x.reshape(-1, Cdim)
         if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 16:
@@ -528,9 +528,6 @@ def _backward_expand(ctx, dy, x, E):
     grads.append(db1.reshape(E * Cdim).to(f1.bias.dtype) if (f1.bias is not None and need[10]) else None)
     grads.append(db2[0].to(f2.bias.dtype) if (f2.bias is not None and need[11]) else None)
     return tuple(grads)
-
-
-_FusedMlpFn._backward_expand = staticmethod(_backward_expand)
 
 
 def _fused_mlp_train(x, mod, cd, norm, res, out_dtype):
