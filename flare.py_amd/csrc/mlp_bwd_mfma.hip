@@ -238,7 +238,22 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
         ++qcount;
     };
 
+    // The waves of a workgroup move in step (one barrier per layer), so a trip to memory that one of them waits for
+    // is a trip all of them wait for.  The rows of x are therefore requested where registers are free and nothing
+    // waits for them yet: the next tile's row while this tile's norm is walked back (x_next), and this tile's row
+    // again, for that walk, at the start of the last backward step (x_again), when the slopes of the later layers
+    // are dead.
     const int64_t nblk = ((int64_t)a.T + WAVES * 16 - 1) / (WAVES * 16);
+    auto row_of = [&](int64_t blk) {
+        const int64_t t = blk * (WAVES * 16) + w * 16 + c16;
+        return t < a.T ? t : a.T - 1;
+    };
+    f32x4 x_next[FT];
+    {
+        const int64_t r = row_of(blockIdx.x);           // blockIdx.x < nblk: the grid is never larger
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft) x_next[ft] = ld4(a.x, r * a.xs + 16 * ft + 4 * g, a.x_dtype);
+    }
     for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
         const int64_t t = blk * (WAVES * 16) + w * 16 + c16;
         const bool live = t < a.T;
@@ -247,7 +262,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
         // ---- forward, recomputed: the stream, the inputs of every layer, the slopes of every activation ----
         f32x4 xs[FT];
 #pragma unroll
-        for (int ft = 0; ft < FT; ++ft) xs[ft] = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+        for (int ft = 0; ft < FT; ++ft) xs[ft] = x_next[ft];
         float mean = 0.f, rstd = 1.f;
         if (a.norm != 0) {
             float s = 0.f;
@@ -277,7 +292,6 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
 #pragma unroll
         for (int l = 0; l < LMAX; ++l) {
             if (l >= L) break;
-            const uint8_t* wb = ring_step_begin(l);
             u32x4 xb[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -285,6 +299,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
                 xb[ks] = u32x4{M_::pack2(lo[0], lo[1]), M_::pack2(lo[2], lo[3]), M_::pack2(hi[0], hi[1]), M_::pack2(hi[2], hi[3])};
             }
             store_rows<C>(a.a_in + (size_t)l * a.T * C, xb, t, a.T, g, c16);      // s_l, the input of layer l, as a 16-bit row (for dW_l)
+            const uint8_t* wb = ring_step_begin(l);
             const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
             auto layer = [&](auto act_c, auto add_c) {
                 constexpr int ACT = decltype(act_c)::value;
@@ -324,6 +339,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
         }
 
         // ---- backward through the chain: xs becomes ds ----
+        f32x4 x_again[FT];
 #pragma unroll
         for (int ft = 0; ft < FT; ++ft) {
             xs[ft] = ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
@@ -332,6 +348,10 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
 #pragma unroll
         for (int l = LMAX - 1; l >= 0; --l) {
             if (l >= L) continue;
+            if (l == 0 && a.norm != 0) {
+#pragma unroll
+                for (int ft = 0; ft < FT; ++ft) x_again[ft] = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+            }
             const uint8_t* wb = ring_step_begin(2 * L - 1 - l);
             const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
             // dt_l = ds_{l+1} * act'(t_l), packed: the B operands of this product and the rows kept for dW_l, db_l
@@ -362,9 +382,15 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
         }
 
         // ---- the norm's backward, dx ----
+        {   // without a condition (the last tile reads its own row once more): under one, the registers of x_next
+            // would have to keep their old value through the whole tile
+            const int64_t r = row_of(blk + gridDim.x < nblk ? blk + gridDim.x : blk);
+#pragma unroll
+            for (int ft = 0; ft < FT; ++ft) x_next[ft] = ld4(a.x, r * a.xs + 16 * ft + 4 * g, a.x_dtype);
+        }
         if (a.norm != 0) {
-            // ds_0 and the token's statistics go out for dgamma, dbeta; xhat is taken again from x (the row is still
-            // in cache) rather than kept in registers;  g = ds_0 * gamma
+            // ds_0 and the token's statistics go out for dgamma, dbeta; xhat is taken again from x (x_again) rather
+            // than kept in registers through the chain;  g = ds_0 * gamma
             u32x4 dq[KS];
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -376,7 +402,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
             float m1 = 0.f, m2 = 0.f;
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
-                const f32x4 xr = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+                const f32x4 xr = x_again[ft];
                 const f32x4 gm = *reinterpret_cast<const f32x4*>(pvec + LMAX * C + 16 * ft + 4 * g);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -389,7 +415,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
             m2 = tok_sum(m2) * (1.f / C);
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
-                const f32x4 xr = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+                const f32x4 xr = x_again[ft];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) xs[ft][r] = rstd * (xs[ft][r] - m1 - (xr[r] - mean) * rstd * m2);
             }
