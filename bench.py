@@ -437,6 +437,23 @@ def bench_block(args, F, dev):
         pass
     except Exception as e:
         out["torch_layers_same_gpu"] = {"error": f"{type(e).__name__}: {str(e)[:160]}"}
+    if not args.no_cpu:
+        # the oracle's restatement of the lift MLP and the block (fp64, explicit score matrices) on batch element 0
+        from oracle import flare_oracle as O
+        n_cpu = pts.shape[1]   # the whole element: the block's mixer is a softmax over all of its tokens
+        sd_l = {k_: v_.detach().cpu() for k_, v_ in lift.state_dict().items()}
+        sd_b = {k_: v_.detach().cpu() for k_, v_ in blk.state_dict().items()}
+        p0 = pts[:1, :n_cpu].cpu()
+        t0 = time.perf_counter()
+        x0 = O._mlp(sd_l, "", p0.double(), "gelu", False, True)
+        y_cpu = O.flare_block(sd_b, "", x0, 8)
+        dt = time.perf_counter() - t0
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+            y_gpu = blk(fused.fused_mlp(pts[:1, :n_cpu].contiguous(), lift, fused.compute_dtype(pts, lift)))[0]
+        out["cpu_baseline"] = {"value": round(n_cpu / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(),
+                               "kind": "port", "sample": f"lift MLP + block of the oracle (torch, fp64, explicit score matrices) on batch element 0 of "
+                               f"{pts.shape[0]} ({n_cpu} tokens), {dt:.2f} s"}
+        out["rel_l2_vs_cpu_on_sample"] = O.rel_l2(y_gpu.float().cpu(), y_cpu.float())
     return out
 
 
