@@ -20,8 +20,10 @@ cached per module and rebuilt when a parameter changes.
 With gradients enabled the chain of C x C layers (the k/v projections, the feed-forward block and the output
 projection of a FLAREBlock at the reference's default ratios) runs through `_FusedMlpFn`: the same forward
 launch, and a backward that recomputes the chain per token tile in one launch (flare_mlp_bwd) and forms the
-parameter gradients from the rows it leaves with one more launch (flare_mlp_wgrad).  The narrow-end, expanding and
-head-padded variants have no backward and stay with the torch layers while gradients are enabled.
+parameter gradients from the rows it leaves with one more launch (flare_mlp_wgrad); the expanding two-layer MLP has a
+backward launch of its own (flare_mlp_expand_bwd).  A stack with a narrow first input or last output keeps that one
+layer as a torch layer while gradients are enabled and sends the C x C layers between through the same path; the
+head-padded variants have no backward.
 """
 from __future__ import annotations
 
@@ -98,10 +100,44 @@ def _io_dims(mod, layers):
 _BWD_MAX_LAYERS = {32: 8, 64: 8, 128: 5}      # the backward keeps every layer's slopes in registers
 
 
+class _SubChain:
+    """The C x C layers of a stack whose first input and/or last output is narrow, as a stack of their own: what the
+    fused launches and their backward see while gradients are enabled.  `first` / `last`: the narrow nn.Linear that
+    stays a torch layer on that side (or None); the packed-weight caches live on this object."""
+
+    num_layers = None
+
+    def __init__(self, layers, act_mask, add_mask, act, C, first, first_act, last, act_module):
+        self.__dict__["_flare_layers"] = ((layers, act_mask, add_mask, act),)
+        self.C, self.first, self.first_act, self.last, self.act_module = C, first, first_act, last, act_module
+
+
+def _train_subchain(mod):
+    """_SubChain of a stack with a narrow end (None for every other module); kept on the module."""
+    cached = mod.__dict__.get("_flare_subchain", 0)
+    if cached != 0:
+        return cached
+    sub = None
+    info = _layers_of(mod)
+    if info is not None:
+        layers, act_mask, add_mask, act = info
+        io = _io_dims(mod, layers)
+        if io is not None and (io[1] or io[2]):
+            Cdim, in_dim, out_dim = io
+            lo, hi = (1 if in_dim else 0), (len(layers) - 1 if out_dim else len(layers))
+            n = hi - lo
+            if n >= 1:
+                keep = (1 << n) - 1
+                sub = _SubChain(layers[lo:hi], (act_mask >> lo) & keep, (add_mask >> lo) & keep, act, Cdim,
+                                layers[0] if in_dim else None, bool(act_mask & 1), layers[-1] if out_dim else None, mod.act)
+    mod.__dict__["_flare_subchain"] = sub
+    return sub
+
+
 def compute_dtype(x, mod):
     """The 16-bit type the fused kernels may run this module in, or None (then torch runs it).  With gradients
-    enabled only the chain of C x C layers and the expanding two-layer MLP qualify (the shapes flare_mlp_bwd and
-    flare_mlp_expand_bwd differentiate)."""
+    enabled the chain of C x C layers and the expanding two-layer MLP qualify (the shapes flare_mlp_bwd and
+    flare_mlp_expand_bwd differentiate), and a stack with a narrow end for the chain between its narrow layers."""
     if x.device.type != "cuda":
         return None
     info = _layers_of(mod)
@@ -111,12 +147,18 @@ def compute_dtype(x, mod):
     if len(layers) > 16:
         return None
     if torch.is_grad_enabled():
-        Cdim = x.shape[-1]
-        if Cdim not in _SUPPORTED_C:
-            return None
-        if not _expand_factor(mod, Cdim):
-            if len(layers) > _BWD_MAX_LAYERS[Cdim] or any(l.in_features != Cdim or l.out_features != Cdim for l in layers):
+        sub = _train_subchain(mod)
+        if sub is not None:                 # narrow first input / last output: the C x C layers between them
+            n = len(_layers_of(sub)[0])
+            if sub.C not in _SUPPORTED_C or n > _BWD_MAX_LAYERS[sub.C] or x.shape[-1] != layers[0].in_features:
                 return None
+        else:
+            Cdim = x.shape[-1]
+            if Cdim not in _SUPPORTED_C:
+                return None
+            if not _expand_factor(mod, Cdim):
+                if len(layers) > _BWD_MAX_LAYERS[Cdim] or any(l.in_features != Cdim or l.out_features != Cdim for l in layers):
+                    return None
     io = _io_dims(mod, layers)
     if io is not None and (io[1] or io[2]):
         if io[0] not in _SUPPORTED_C or x.shape[-1] != layers[0].in_features:
@@ -253,6 +295,21 @@ def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None, x_head=0, y_head=
     if torch.is_grad_enabled():
         if x_head or y_head:
             raise ValueError("head-padded rows have no backward: call under torch.no_grad()")
+        sub = _train_subchain(mod)
+        if sub is not None:
+            # narrow ends: those layers run as torch layers (under the caller's autocast), the chain between them fused
+            out_dtype = x.dtype if out_dtype is None else out_dtype
+            h, hn = x, norm
+            if sub.first is not None:
+                if hn is not None and not isinstance(hn, nn.Identity):
+                    h, hn = hn(h), None
+                h = sub.first(h)
+                if sub.first_act:
+                    h = sub.act_module(h)
+            y = _fused_mlp_train(h, sub, cd, hn, None, cd if sub.last is not None else out_dtype)
+            if sub.last is not None:
+                y = sub.last(y).to(out_dtype)
+            return y if res is None else res + y
         return _fused_mlp_train(x, mod, cd, norm, res, out_dtype)
     return _fused_mlp_fwd(x, mod, cd, norm, res, out_dtype, x_head, y_head)
 

@@ -162,7 +162,8 @@ def test_shapes_without_a_backward_keep_their_torch_layers(dev):
         assert fused.compute_dtype(x, ResidualMLP(64, 64, 64, num_layers=3).to(dev)) == torch.bfloat16
         assert fused.compute_dtype(x, ResidualMLP(64, 256, 64, num_layers=0, input_residual=False, output_residual=False).to(dev)) == torch.bfloat16
         assert fused.compute_dtype(x, ResidualMLP(64, 256, 64, num_layers=1, input_residual=False, output_residual=False).to(dev)) is None   # wide hidden stream
-        assert fused.compute_dtype(torch.randn(10, 3, device=dev), ResidualMLP(3, 64, 64, num_layers=2, input_residual=False).to(dev)) is None   # narrow end
+        assert fused.compute_dtype(torch.randn(10, 3, device=dev), ResidualMLP(3, 64, 64, num_layers=2, input_residual=False).to(dev)) == torch.bfloat16   # narrow end: its chain
+        assert fused.compute_dtype(torch.randn(10, 3, device=dev), ResidualMLP(3, 128, 128, num_layers=6, input_residual=False).to(dev)) is None   # 7 C x C layers at C = 128
         assert fused.compute_dtype(x, ResidualMLP(64, 64, 64, num_layers=9).to(dev)) is None          # 11 layers: above the limit
         assert fused.compute_dtype(torch.randn(10, 128, device=dev), ResidualMLP(128, 128, 128, num_layers=4).to(dev)) is None
         with torch.no_grad():
@@ -255,3 +256,45 @@ def test_block_with_expanding_ffn_trains_fused(dev):
     for i, (g, t, r) in enumerate(zip(got, t16, ref)):
         e, et = rel(g, r), rel(t, r)
         assert e <= min(6e-2, max(3e-2, 2 * et)), f"tensor {i}: rel-L2 {e:.3e} (torch layers under autocast: {et:.3e})"
+
+
+@pytest.mark.parametrize("C,in_dim,out_dim,num_layers,T,norm_kind,dtype", [
+    (128, 3, 128, 2, 3000, None, torch.bfloat16), (64, 64, 1, 2, 2500, "ln", torch.bfloat16), (32, 2, 4, 3, 777, None, torch.float16),
+    (128, 128, 3, 3, 1100, "rms", torch.bfloat16)])
+def test_narrow_end_stacks_train_through_the_fused_chain(dev, C, in_dim, out_dim, num_layers, T, norm_kind, dtype):
+    """in_proj / out_proj of the models (pdebench/models/flare.py:137-147): the narrow Linear stays a torch layer, the
+    C x C layers between go through flare_mlp_bwd / flare_mlp_wgrad; gradients of every parameter against fp32."""
+    from torch.profiler import ProfilerActivity, profile
+    torch.manual_seed(C + T)
+    mod = ResidualMLP(in_dim, C, out_dim, num_layers=num_layers, input_residual=(in_dim == C), output_residual=(out_dim == C)).to(dev)
+    norm = None if norm_kind is None else (nn.LayerNorm(C) if norm_kind == "ln" else nn.RMSNorm(C)).to(dev)
+    with torch.no_grad():
+        for p in mod.parameters():
+            if p.dim() == 2:
+                p.mul_(2.0)
+    x = torch.randn(2, T, in_dim, device=dev, requires_grad=True)
+    gy = torch.randn(2, T, out_dim, device=dev)
+    params = list(mod.parameters()) + ([] if norm is None else list(norm.parameters()))
+    layers = lambda: mod(norm(x) if norm is not None else x)
+
+    def hip():
+        with torch.autocast("cuda", dtype):
+            cd = fused.compute_dtype(x, mod)
+            assert cd == dtype
+            return fused.fused_mlp(x, mod, cd, norm=norm)
+
+    def torch16():
+        with torch.autocast("cuda", dtype):
+            return layers()
+
+    ref, t16 = _run(layers, x, params, gy), _run(torch16, x, params, gy)
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        got = _run(hip, x, params, gy)
+        torch.cuda.synchronize()
+    names = " ".join(e.key for e in prof.key_averages())
+    assert "mlp_bwd_kernel" in names and "mlp_wgrad_kernel" in names
+    assert got[0].dtype == torch.float32 and got[0].shape == ref[0].shape
+    for i, (g, t, r) in enumerate(zip(got, t16, ref)):
+        e, et = rel(g, r), rel(t, r)
+        assert torch.isfinite(g).all()
+        assert e <= max(3e-2, 2 * et), f"tensor {i}: rel-L2 {e:.3e} (torch layers under autocast: {et:.3e})"
