@@ -112,6 +112,34 @@ class _SubChain:
         self.C, self.first, self.first_act, self.last, self.act_module = C, first, first_act, last, act_module
 
 
+class _NarrowLinearFn(torch.autograd.Function):
+    """t = x W^T + b for a Linear with a few input columns (the lift of the models' in_proj) under autocast.  Only the
+    weight gradient differs from torch's own: dW = g^T x contracts over all tokens into a [C, in_dim] result, which the
+    library runs as one long product with nothing to parallelise; here it is a batched product over chunks of 4096
+    tokens whose partial results are summed in fp32."""
+
+    @staticmethod
+    def forward(ctx, x2, w, b, cd):
+        ctx.save_for_backward(x2, w)
+        ctx.has_bias = b is not None
+        return torch.nn.functional.linear(x2.to(cd), w.to(cd), None if b is None else b.to(cd))
+
+    @staticmethod
+    def backward(ctx, g):
+        x2, w = ctx.saved_tensors
+        T, chunk = g.shape[0], 4096
+        n = T // chunk
+        xc = x2.to(g.dtype)
+        dw = torch.zeros(w.shape, dtype=torch.float32, device=g.device)
+        if n > 0:
+            dw += torch.bmm(g[:n * chunk].view(n, chunk, -1).transpose(1, 2), xc[:n * chunk].view(n, chunk, -1)).sum(0, dtype=torch.float32)
+        if n * chunk < T:
+            dw += (g[n * chunk:].t() @ xc[n * chunk:]).float()
+        db = g.sum(0, dtype=torch.float32).to(w.dtype) if ctx.has_bias else None
+        dx = (g @ w.to(g.dtype)).to(x2.dtype) if ctx.needs_input_grad[0] else None
+        return dx, dw.to(w.dtype), db, None
+
+
 def _train_subchain(mod):
     """_SubChain of a stack with a narrow end (None for every other module); kept on the module."""
     cached = mod.__dict__.get("_flare_subchain", 0)
@@ -303,7 +331,7 @@ def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None, x_head=0, y_head=
             if sub.first is not None:
                 if hn is not None and not isinstance(hn, nn.Identity):
                     h, hn = hn(h), None
-                h = sub.first(h)
+                h = _NarrowLinearFn.apply(h.reshape(-1, h.shape[-1]), sub.first.weight, sub.first.bias, cd).view(*h.shape[:-1], -1)
                 if sub.first_act:
                     h = sub.act_module(h)
             y = _fused_mlp_train(h, sub, cd, hn, None, cd if sub.last is not None else out_dtype)
