@@ -6,10 +6,11 @@ the reference loads with strict=True.  The projections, norms and MLPs are ordin
 layers (hipBLASLt GEMMs); the mixer is the HIP engine (`functional.flare_multihead_mixer`),
 which reads k and v as strided [B,N,H*D] views, so no head-split copy is made.
 
-Inference fast path: when no gradient is needed and the Linear layers may run in bf16/f16
-(autocast, or 16-bit weights) and channel_dim is 32, 64 or 128, FLAREBlock runs as four fused HIP
-launches around the mixer (norm1 + k_proj, norm1 + v_proj, out_proj + residual, norm2 + FFN +
-residual; see fused.py) instead of ~70 torch kernels.  Training and fp32 use the torch layers.
+Fast path: when the Linear layers may run in bf16/f16 (autocast, or 16-bit weights) and channel_dim
+is 32, 64 or 128, FLAREBlock runs as four fused HIP launches around the mixer (norm1 + k_proj,
+norm1 + v_proj, out_proj + residual, norm2 + FFN + residual; see fused.py) instead of ~70 torch
+kernels; with gradients enabled the same launches are differentiable (fused._FusedMlpFn).  fp32
+without autocast uses the torch layers.
 """
 from __future__ import annotations
 
