@@ -228,6 +228,15 @@ struct MlpWgradArgs {
     int64_t tokens_per_wg;                      // set by the launcher
 };
 
+// Workgroups of the backward's dq pass (bwd_lat_kernel, MODE 1) that fit a compute unit: its instances with 16 or
+// 32 latents per wave at head dim 16, and with 16 at head dim 32, need few enough registers for three or four (measured:
+// 143 -> 119 us at M = 128, D = 16; 86 -> 74 us at M = 64, D = 16; 133 -> 106 us at M = 64, D = 32); squeezing the
+// others spills.  CT = 16-latent tiles per wave.
+constexpr int bwd_dq_wgs_per_cu(int D, int CT)
+{
+    return D <= 16 ? (CT == 1 ? 4 : CT == 2 ? 3 : 2) : D <= 32 ? (CT == 1 ? 3 : 2) : 2;
+}
+
 // ---- launchers implemented in the .hip files -------------------------------------------
 hipError_t launch_gather_generic(const MixerArgs& a, int dtype, hipStream_t st);
 hipError_t launch_gather_merge(const MixerArgs& a, hipStream_t st);

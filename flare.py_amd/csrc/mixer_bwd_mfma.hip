@@ -167,7 +167,7 @@ constexpr int kBTile = 64;   // tokens per LDS tile
 
 // One workgroup = 4 waves x (16 CT latents) x one token range.  MODE 0: dz partial; MODE 1: dq partial.
 template <typename T, int D, int CT, int MODE>
-__global__ __launch_bounds__(256, 2) void bwd_lat_kernel(MixerBwdArgs a)
+__global__ __launch_bounds__(256, MODE == 1 ? bwd_dq_wgs_per_cu(D, CT) : 2) void bwd_lat_kernel(MixerBwdArgs a)
 {
     constexpr int KD = (D + 31) / 32, RT = D / 16, CH = D / 8, MB = 64 * CT, ROWB = D * 2, TILEB = kBTile * ROWB;
     constexpr int NT = MODE == 0 ? 2 : 4;          // staged tiles: K rows, dY^T | K rows, K^T, V rows, dY rows
