@@ -485,12 +485,18 @@ class _FusedMlpFn(torch.autograd.Function):
                         and res.stride() == x.stride() and res.dtype == x.dtype)
         ctx.has_res = res is not None
         ctx.n_wb = len(wb)
+        # the backward reads the parameters again (its packed copies are keyed by their versions) instead of saving
+        # them: as with a saved tensor, changing one in place between forward and backward is an error
+        ctx.versions = tuple(None if t is None else t._version for t in (gamma, beta, *wb))
+        ctx.params = (gamma, beta, *wb)
         ctx.save_for_backward(x)
         return y
 
     @staticmethod
     def backward(ctx, dy):
         (x,) = ctx.saved_tensors
+        if ctx.versions != tuple(None if t is None else t._version for t in ctx.params):
+            raise RuntimeError("a parameter of the fused MLP was modified in place between its forward and its backward")
         mod, cd, norm = ctx.mod, ctx.cd, ctx.norm
         lib = _lib.load()
         layers, act_mask, add_mask, act = _layers_of(mod)

@@ -298,3 +298,14 @@ def test_narrow_end_stacks_train_through_the_fused_chain(dev, C, in_dim, out_dim
         e, et = rel(g, r), rel(t, r)
         assert torch.isfinite(g).all()
         assert e <= max(3e-2, 2 * et), f"tensor {i}: rel-L2 {e:.3e} (torch layers under autocast: {et:.3e})"
+
+
+def test_parameter_changed_between_forward_and_backward_is_an_error(dev):
+    mod = nn.Linear(64, 64).to(dev)
+    x = torch.randn(100, 64, device=dev, requires_grad=True)
+    with torch.autocast("cuda", torch.bfloat16):
+        y = fused.fused_mlp(x, mod, fused.compute_dtype(x, mod))
+    with torch.no_grad():
+        mod.weight.mul_(2.0)
+    with pytest.raises(RuntimeError, match="modified in place"):
+        y.sum().backward()
