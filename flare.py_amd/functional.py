@@ -16,6 +16,7 @@ import math
 from typing import Optional, Tuple
 
 import torch
+from torch.autograd.function import once_differentiable
 
 from . import _lib
 from ._lib import FlareCausalDesc, FlareMixerDesc, FlareTripleDesc
@@ -404,6 +405,7 @@ class _MixerFn(torch.autograd.Function):
         return y, z
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, gy, _gz):
         if ctx.hip:
             q, k, v, y, z, lse_lat, lse_tok = ctx.saved_tensors
@@ -468,6 +470,7 @@ class _MixerDropoutFn(torch.autograd.Function):
         return y, z
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, gy, _gz):
         q, k, v = ctx.saved_tensors
         gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy, ctx.drop)
@@ -700,6 +703,7 @@ class _GatherFn(torch.autograd.Function):
         return z, lse
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, gz, _glse):
         q, k, v = ctx.saved_tensors
         return (*_half_torch_grad("gather", q, k, v, ctx.scale, ctx.key_mask, gz), None, None, None, None)
@@ -713,6 +717,7 @@ class _ScatterFn(torch.autograd.Function):
         return _scatter_forward(q, k, z, scale, key_mask, force_generic)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, gy):
         q, k, z = ctx.saved_tensors
         return (*_half_torch_grad("scatter", q, k, z, ctx.scale, ctx.key_mask, gy), None, None, None)
@@ -1020,6 +1025,7 @@ class _CausalLinearFn(torch.autograd.Function):
         return _causal_linear_forward(q, k, v)
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, gy):
         q, k, v = ctx.saved_tensors
         with torch.enable_grad():
@@ -1159,6 +1165,7 @@ class _TripleFn(torch.autograd.Function):
         return state, out
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, dstate, dout):
         q1, q2, k1, k2, v, state = ctx.saved_tensors
         N = q1.shape[2]

@@ -31,6 +31,7 @@ import ctypes as C
 
 import torch
 from torch import nn
+from torch.autograd.function import once_differentiable
 
 from . import _lib
 from .functional import _autocast_dtype, _dtype_code, _on_device, _ptr, _stream_ptr
@@ -125,6 +126,7 @@ class _NarrowLinearFn(torch.autograd.Function):
         return torch.nn.functional.linear(x2.to(cd), w.to(cd), None if b is None else b.to(cd))
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, g):
         x2, w = ctx.saved_tensors
         T, chunk = g.shape[0], 4096
@@ -481,8 +483,9 @@ class _FusedMlpFn(torch.autograd.Function):
         with torch.no_grad():
             y = _fused_mlp_fwd(x, mod, cd, norm=norm, res=res, out_dtype=out_dtype)
         ctx.mod, ctx.cd, ctx.norm = mod, cd, norm
-        ctx.res_is_x = (res is not None and res.data_ptr() == x.data_ptr() and res.shape == x.shape
-                        and res.stride() == x.stride() and res.dtype == x.dtype)
+        # res and x one tensor: dy is added to dx inside the kernel.  (Two tensors over the same memory are not
+        # enough: one of them may be detached, and then its path carries no gradient.)
+        ctx.res_is_x = res is x
         ctx.has_res = res is not None
         ctx.n_wb = len(wb)
         # the backward reads the parameters again (its packed copies are keyed by their versions) instead of saving
@@ -493,6 +496,7 @@ class _FusedMlpFn(torch.autograd.Function):
         return y
 
     @staticmethod
+    @once_differentiable
     def backward(ctx, dy):
         (x,) = ctx.saved_tensors
         if ctx.versions != tuple(None if t is None else t._version for t in ctx.params):

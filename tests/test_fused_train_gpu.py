@@ -94,6 +94,44 @@ def test_separate_residual_and_no_residual(dev):
     assert rel(x.grad, xr.grad) <= 1e-2
 
 
+def test_detached_residual_over_the_rows_of_x(dev):
+    """res = x.detach(): the same memory, but no gradient flows through the residual; dx must not contain dy.  With
+    res = x itself the sum is formed inside the backward launch."""
+    torch.manual_seed(8)
+    C, T = 64, 500
+    mod = nn.Linear(C, C).to(dev)
+    x = torch.randn(T, C, device=dev, requires_grad=True)
+    gy = torch.randn(T, C, device=dev)
+    with torch.autocast("cuda", torch.bfloat16):
+        y = fused.fused_mlp(x, mod, torch.bfloat16, res=x.detach())
+    assert not y.grad_fn.res_is_x
+    y.backward(gy)
+    g_detached = x.grad.clone()
+    x.grad = None
+    with torch.autocast("cuda", torch.bfloat16):
+        y = fused.fused_mlp(x, mod, torch.bfloat16, res=x)
+    assert y.grad_fn.res_is_x
+    y.backward(gy)
+    assert rel(x.grad - g_detached, gy) <= 1e-2
+    xr = x.detach().clone().requires_grad_(True)
+    (xr @ mod.weight.detach().t()).backward(gy)
+    assert rel(g_detached, xr.grad) <= 1e-2
+
+
+def test_second_order_gradients_are_refused(dev):
+    """The backward is a HIP launch with no graph of its own: differentiating it again raises instead of returning
+    zeros."""
+    torch.manual_seed(9)
+    C, T = 32, 100
+    mod = nn.Linear(C, C).to(dev)
+    x = torch.randn(T, C, device=dev, requires_grad=True)
+    with torch.autocast("cuda", torch.bfloat16):
+        y = fused.fused_mlp(x, mod, torch.bfloat16)
+    (gx,) = torch.autograd.grad(y.float().square().sum(), x, create_graph=True)
+    with pytest.raises(RuntimeError, match="once_differentiable"):
+        gx.sum().backward()
+
+
 def test_backward_is_deterministic(dev):
     torch.manual_seed(6)
     C, T = 128, 5000
