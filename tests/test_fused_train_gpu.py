@@ -347,3 +347,29 @@ def test_parameter_changed_between_forward_and_backward_is_an_error(dev):
         mod.weight.mul_(2.0)
     with pytest.raises(RuntimeError, match="modified in place"):
         y.sum().backward()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_block_with_16bit_parameters_trains_fused(dev, dtype):
+    """No autocast: a block cast to a 16-bit type trains through the same launches, every gradient in that type."""
+    from torch.profiler import ProfilerActivity, profile
+    torch.manual_seed(0)
+    ref = F.FLAREBlock(channel_dim=64, num_heads=4, num_latents=64).to(dev)
+    blk = F.FLAREBlock(channel_dim=64, num_heads=4, num_latents=64).to(dev)
+    blk.load_state_dict(ref.state_dict())
+    blk = blk.to(dtype)
+    x = torch.randn(2, 3000, 64, device=dev)
+    gy = torch.randn_like(x)
+    xr, xh = x.clone().requires_grad_(True), x.to(dtype).requires_grad_(True)
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        y = blk(xh)[0]
+        y.backward(gy.to(dtype))
+    names = {e.key for e in prof.key_averages()}
+    for kernel in ("mlp_bwd_kernel", "mlp_wgrad_kernel", "bwd_tok_kernel"):
+        assert any(kernel in n for n in names), kernel
+    yr = ref(xr)[0]
+    yr.backward(gy)
+    assert rel(y.detach(), yr.detach()) <= 2e-2 and rel(xh.grad, xr.grad) <= 3e-2
+    for (n, p), (_, q) in zip(blk.named_parameters(), ref.named_parameters()):
+        assert p.grad is not None and p.grad.dtype == dtype, n
+        assert rel(p.grad, q.grad) <= 8e-2, n
