@@ -98,8 +98,15 @@ __global__ __launch_bounds__(kThreads) void triple_merge_kernel(TripleArgs a)
     if (idx >= total) return;
     const size_t bh = idx / per, e = idx - bh * per;
     const float* p = a.part + bh * a.n_parts * per + e;
+    // eight partials requested at a time (a load per iteration would wait for the one before); summed in split order
     float s = 0.f;
-    for (int sp = 0; sp < a.n_parts; ++sp) s += p[(size_t)sp * per];
+    for (int sp = 0; sp < a.n_parts; sp += 8) {
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) t[u] = p[(size_t)min(sp + u, a.n_parts - 1) * per];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += sp + u < a.n_parts ? t[u] : 0.f;
+    }
     s *= 1.0f / (float)a.N;
     if (!a.diag_parts) {
         if (e < ns) a.state[bh * ns + e] = s;
