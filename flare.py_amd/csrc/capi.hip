@@ -219,7 +219,7 @@ bool causal_wants_mfma(const FlareCausalDesc* d)
 
 // Matrix-core prefill plan: the token axis is cut into segments that run in parallel (local
 // states first, then the recurrence of each segment from the summed states before it).
-struct CausalPlan { bool mfma; int n_segs, seg_len; size_t off_den, off_num, total; };
+struct CausalPlan { bool mfma; int n_segs, seg_len, n_pieces, piece_len, n_slots; size_t off_den, off_num, total; };
 
 CausalPlan plan_causal(const FlareCausalDesc* d)
 {
@@ -242,13 +242,30 @@ CausalPlan plan_causal(const FlareCausalDesc* d)
         seg_len = ((d->N + 63) / 64 + 15) / 16 * 16;
         n_segs = (d->N + seg_len - 1) / seg_len;
     }
+    p.n_pieces = 0;
+    p.piece_len = (int)seg_len;
+    p.n_slots = 1;
     if (n_segs > 1) {
         p.n_segs = (int)n_segs;
         p.seg_len = (int)seg_len;
+        // The first phase covers the tokens before the last segment.  With one workgroup per segment it would run
+        // n_segs - 1 workgroups per (b,h) where the device holds n_segs: some CUs with two, some with one.  It is cut
+        // into as many pieces as there are segments instead (whole 64-token tiles, at least 256 tokens); a piece that
+        // reaches across a segment boundary leaves one local state on either side.
+        const int64_t end = (n_segs - 1) * seg_len;
+        int64_t piece = seg_len, pieces = n_segs - 1;
+        if (d->chunk <= 0) {
+            piece = std::max<int64_t>(256, ((end + n_segs - 1) / n_segs + 63) / 64 * 64);
+            if (piece >= seg_len) piece = seg_len;
+            pieces = (end + piece - 1) / piece;
+        }
+        p.n_pieces = (int)pieces;
+        p.piece_len = (int)piece;
+        p.n_slots = (int)(pieces + n_segs);      // at most one more local state per boundary, and the staging slot
     }
     p.off_den = ((size_t)BH * sizeof(int) + 255) / 256 * 256;
-    p.off_num = p.off_den + (p.n_segs > 1 ? (size_t)BH * p.n_segs * d->M * sizeof(float) : 0);
-    p.total = p.off_num + (p.n_segs > 1 ? (size_t)BH * p.n_segs * d->M * d->D * sizeof(float) : 0);
+    p.off_num = p.off_den + (p.n_segs > 1 ? (size_t)BH * p.n_slots * d->M * sizeof(float) : 0);
+    p.total = p.off_num + (p.n_segs > 1 ? (size_t)BH * p.n_slots * d->M * d->D * sizeof(float) : 0);
     return p;
 }
 
@@ -648,6 +665,9 @@ int causal_run(const FlareCausalDesc* desc, bool decode, const void* q, const vo
         a.flags = static_cast<int*>(workspace);
         a.n_segs = decode ? 1 : p.n_segs;          // decode steps are sequential by nature
         a.seg_len = decode ? desc->N : p.seg_len;
+        a.n_pieces = decode ? 0 : p.n_pieces;
+        a.piece_len = decode ? std::max(desc->N, 1) : p.piece_len;
+        a.n_slots = decode ? 1 : p.n_slots;
         a.seg_den = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p.off_den);
         a.seg_num = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p.off_num);
         hipError_t e = flare::launch_causal_mfma(a, desc->dtype, decode ? 1 : 16, st);

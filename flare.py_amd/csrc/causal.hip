@@ -76,12 +76,12 @@ __global__ __launch_bounds__(kThreads) void causal_generic_kernel(CausalArgs a)
     const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H;
     if (a.flags != nullptr && a.flags[bh] == 0) {
         // Launched behind the matrix-core kernels: only marked (b,h) are redone.  For the others a prefill in several
-        // segments has staged its final state in the last segment's workspace slot; it becomes (mu, den, num) here,
+        // segments has staged its final state in the last workspace slot; it becomes (mu, den, num) here,
         // once every segment is known to have passed (a fresh state's shift becomes 0).
         if (a.n_segs > 1) {
             const int M = a.M, D = a.D;
-            const float* sd = a.seg_den + ((int64_t)bh * a.n_segs + a.n_segs - 1) * M;
-            const float* sn = a.seg_num + ((int64_t)bh * a.n_segs + a.n_segs - 1) * M * D;
+            const float* sd = a.seg_den + ((int64_t)bh * a.n_slots + a.n_slots - 1) * M;
+            const float* sn = a.seg_num + ((int64_t)bh * a.n_slots + a.n_slots - 1) * M * D;
             float* num = a.num + (int64_t)bh * M * D;
             for (int i = tid; i < M; i += kThreads) {
                 const float mu = a.mu[(int64_t)bh * M + i];

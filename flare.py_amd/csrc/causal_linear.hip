@@ -145,11 +145,20 @@ __global__ __launch_bounds__(256) void causal_linear_prefix_kernel(CausalLinearA
     const int sz = a.Dk * a.Dv;
     if (e >= sz) return;
     float* S = a.states + (int64_t)bh * a.n_segs * sz + e;
+    // eight slots read before the first of them is overwritten: one trip to memory per eight segments
     float run = 0.f;
-    for (int s = 0; s < a.n_segs; ++s) {
-        const float t = s + 1 < a.n_segs ? S[(int64_t)s * sz] : 0.f;
-        S[(int64_t)s * sz] = run;
-        run += t;
+    for (int s0 = 0; s0 < a.n_segs; s0 += 8) {
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) t[u] = S[(int64_t)min(s0 + u, a.n_segs - 1) * sz];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int s = s0 + u;
+            if (s < a.n_segs) {
+                S[(int64_t)s * sz] = run;
+                run += s + 1 < a.n_segs ? t[u] : 0.f;
+            }
+        }
     }
 }
 

@@ -136,10 +136,12 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
     const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H, seg = blockIdx.y;
-    const int n_lo = seg * a.seg_len, N = min(a.N, n_lo + a.seg_len);   // this segment: tokens n_lo .. N-1
+    // this segment: tokens n_lo .. N-1 (the first phase walks the parts of its piece instead, see below)
+    int n_lo = seg * a.seg_len, N = min(a.N, n_lo + a.seg_len);
     const bool single = a.n_segs == 1;
-    float* seg_den = a.seg_den + ((int64_t)bh * a.n_segs + seg) * M;
-    float* seg_num = a.seg_num + ((int64_t)bh * a.n_segs + seg) * M * D;
+    float* seg_den = a.seg_den + ((int64_t)bh * a.n_slots + a.n_slots - 1) * M;        // staging slot of the final state
+    float* seg_num = a.seg_num + ((int64_t)bh * a.n_slots + a.n_slots - 1) * M * D;
+    const int n_before = STATE_ONLY ? 0 : causal_slots_before(seg, a.seg_len, a.piece_len);
     const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
     const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
     const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
@@ -177,7 +179,7 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
             d0 = mu <= kNegBig ? 0.f : dn_in;
         }
         if (!STATE_ONLY)
-            for (int s = 0; s < seg; ++s) d0 += a.seg_den[((int64_t)bh * a.n_segs + s) * M + m];
+            for (int s = 0; s < n_before; ++s) d0 += a.seg_den[((int64_t)bh * a.n_slots + s) * M + m];
         den[ct] = f32x4{d0, d0, d0, d0};
     }
     // state numerator U[m, d]: tile (mt, dt) holds rows m0 + 16 mt + 4g + r, column 16 dt + c16
@@ -195,8 +197,8 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
                     u = mu_m <= kNegBig ? 0.f : un;
                 }
                 if (!STATE_ONLY)
-                    for (int s = 0; s < seg; ++s)
-                        u += a.seg_num[(((int64_t)bh * a.n_segs + s) * M + m) * D + dt * 16 + c16];
+                    for (int s = 0; s < n_before; ++s)
+                        u += a.seg_num[(((int64_t)bh * a.n_slots + s) * M + m) * D + dt * 16 + c16];
                 U[mt][dt][r] = u;
             }
 
@@ -253,9 +255,10 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
 
     if constexpr (STATE_ONLY) {
         // The first phase never raises a flag, and the recurrence phase starts after it has finished: its first
-        // segment clears the (b,h)'s redo flag (by a kernel, so that a caller may capture the call in a graph).
+        // workgroup clears the (b,h)'s redo flag (by a kernel, so that a caller may capture the call in a graph).
         if (seg == 0 && tid == 0) a.flags[bh] = 0;
-        // Local state of the segment.  A 16-token block is too little work here to cover the memory
+        // Local states of this workgroup's piece of the tokens: one per segment the piece reaches into (n_lo, N are
+        // set to each such part in turn).  A 16-token block is too little work here to cover the memory
         // latency of its own prefetch, so this phase walks 64-token tiles: K as four A operands per
         // lane, V through a 64-row LDS tile.  Three register sets take turns, each refilled with the tile
         // three ahead as soon as its own has been used: loads are unconditional (rows past the end of
@@ -293,68 +296,105 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
                 *reinterpret_cast<u32x4*>(&v64[buf][tok][ch * 8]) = o;
             }
         };
-        // the tile's contribution; the denominators count live tokens only (the A operand of their product
-        // holds ones in the k-slots of live tokens)
+        // the tile's contribution, two 16-token blocks per product (k-slots 8g + i: token 4g + i of the first block,
+        // 8g + 4 + i: of the second); the denominators count live tokens only (the A operand of their product holds
+        // ones in the k-slots of live tokens)
         auto work = [&](int n0, int buf, const Tile& t) {
 #pragma unroll
-            for (int sb = 0; sb < 4; ++sb) {
-                const int tb = N - (n0 + sb * 16);   // tokens >= tb of this block are beyond the segment
-                uint2 live4 = ones4;
-                if (tb < 16) {
+            for (int sp = 0; sp < 2; ++sp) {
+                const int tb = N - (n0 + sp * 32);   // tokens >= tb of this pair of blocks are beyond the part
+                u32x4 live8 = u32x4{ones4.x, ones4.y, ones4.x, ones4.y};
+                if (tb < 32) {
                     const uint32_t one = P_::kOnes2 & 0xffffu;
-                    live4 = make_uint2((4 * g + 0 < tb ? one : 0u) | (4 * g + 1 < tb ? one << 16 : 0u),
-                                       (4 * g + 2 < tb ? one : 0u) | (4 * g + 3 < tb ? one << 16 : 0u));
-                }
-                uint2 vop[DT];
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) vop[dt] = tr16(&v64[buf][sb * 16 + 4 * g + (c16 >> 2)][dt * 16 + (c16 & 3) * 4]);
+                    for (int hb = 0; hb < 2; ++hb) {
+                        const int t0 = hb * 16 + 4 * g;
+                        live8[2 * hb] = (t0 + 0 < tb ? one : 0u) | (t0 + 1 < tb ? one << 16 : 0u);
+                        live8[2 * hb + 1] = (t0 + 2 < tb ? one : 0u) | (t0 + 3 < tb ? one << 16 : 0u);
+                    }
+                }
+                u32x4 vop[DT];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    const uint2 lo = tr16(&v64[buf][sp * 32 + 4 * g + (c16 >> 2)][dt * 16 + (c16 & 3) * 4]);
+                    const uint2 hi = tr16(&v64[buf][sp * 32 + 16 + 4 * g + (c16 >> 2)][dt * 16 + (c16 & 3) * 4]);
+                    vop[dt] = u32x4{lo.x, lo.y, hi.x, hi.y};
+                }
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
-                    f32x4 s = negmu[ct];
+                    f32x4 s0 = negmu[ct], s1 = negmu[ct];
 #pragma unroll
-                    for (int kd = 0; kd < KD; ++kd) s = M_::mma32(t.k[sb][kd], qb[ct][kd], s);
-                    const uint2 ppk = make_uint2(P_::pack2(fast_exp2(s[0]), fast_exp2(s[1])), P_::pack2(fast_exp2(s[2]), fast_exp2(s[3])));
-                    den[ct] = P_::mma16(live4, ppk, den[ct]);
+                    for (int kd = 0; kd < KD; ++kd) {
+                        s0 = M_::mma32(t.k[2 * sp][kd], qb[ct][kd], s0);
+                        s1 = M_::mma32(t.k[2 * sp + 1][kd], qb[ct][kd], s1);
+                    }
+                    const u32x4 ppk = u32x4{P_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])), P_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
+                                            P_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])), P_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]))};
+                    den[ct] = P_::mma32(live8, ppk, den[ct]);
 #pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) U[ct][dt] = P_::mma16(ppk, vop[dt], U[ct][dt]);
+                    for (int dt = 0; dt < DT; ++dt) U[ct][dt] = P_::mma32(ppk, vop[dt], U[ct][dt]);
                 }
             }
         };
+        const int p_lo = seg * a.piece_len, p_hi = min(p_lo + a.piece_len, (a.n_segs - 1) * a.seg_len);
+        for (int s = p_lo / a.seg_len; s <= (p_hi - 1) / a.seg_len; ++s) {
+        n_lo = max(p_lo, s * a.seg_len);
+        N = min(p_hi, (s + 1) * a.seg_len);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            den[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) U[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        __syncthreads();   // the part before has read its last tile
         Tile ta, tb_, tc;
         fetch(n_lo, ta);
         fetch(n_lo + 64, tb_);
         fetch(n_lo + 128, tc);
         stage(n_lo, 0, ta);
         __syncthreads();
-        int buf = 0;
-        for (int n0 = n_lo;; n0 += 192) {
+        // Whole groups of three tiles in a loop with one exit at its bottom, the last one or two tiles behind it: an
+        // exit from the middle of the group would reach the loop's head again in the compiler's control flow, and
+        // with prefetches in flight on that path every pass through the head would wait for all of them.
+        const int tiles = (N - n_lo + 63) >> 6;
+        int buf = 0, n0 = n_lo;
+        for (int gi = 0; gi < tiles / 3; ++gi, n0 += 192) {
             // tile n0 (K in ta, V staged in v64[buf]); the next tile's V goes into the other buffer meanwhile
             work(n0, buf, ta);
             fetch(n0 + 192, ta);
-            if (n0 + 64 >= N) break;
             stage(n0 + 64, buf ^ 1, tb_);
             __syncthreads();
             work(n0 + 64, buf ^ 1, tb_);
             fetch(n0 + 256, tb_);
-            if (n0 + 128 >= N) break;
             stage(n0 + 128, buf, tc);
             __syncthreads();
             work(n0 + 128, buf, tc);
             fetch(n0 + 320, tc);
-            if (n0 + 192 >= N) break;
             stage(n0 + 192, buf ^ 1, ta);
             __syncthreads();
             buf ^= 1;
         }
-        // local state of the segment, relative to the shift of the incoming state; whatever
+        if (tiles % 3 >= 1) work(n0, buf, ta);
+        if (tiles % 3 == 2) {
+            stage(n0 + 64, buf ^ 1, tb_);
+            __syncthreads();
+            work(n0 + 64, buf ^ 1, tb_);
+        }
+        // nothing of this part stays in flight (the prefetches past its end were never used)
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        // local state of the part, relative to the shift of the incoming state; whatever
         // overflowed or vanished here is caught by the checks of the segments that use it
+        const int64_t slot = (int64_t)bh * a.n_slots + causal_slot(seg, s, a.seg_len, a.piece_len);
+        float* part_den = a.seg_den + slot * M;
+        float* part_num = a.seg_num + slot * M * D;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
-            if (g == 0) seg_den[m0 + ct * 16 + c16] = den[ct][0];
+            if (g == 0) part_den[m0 + ct * 16 + c16] = den[ct][0];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) seg_num[(int64_t)(m0 + ct * 16 + 4 * g + r) * D + dt * 16 + c16] = U[ct][dt][r];
+                for (int r = 0; r < 4; ++r) part_num[(int64_t)(m0 + ct * 16 + 4 * g + r) * D + dt * 16 + c16] = U[ct][dt][r];
+        }
         }
         return;
     }
@@ -551,8 +591,9 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H, seg = blockIdx.y;
     const int n_lo = seg * a.seg_len, N = min(a.N, n_lo + a.seg_len);
     const bool single = a.n_segs == 1;
-    float* seg_den = a.seg_den + ((int64_t)bh * a.n_segs + seg) * M;
-    float* seg_num = a.seg_num + ((int64_t)bh * a.n_segs + seg) * M * D;
+    float* seg_den = a.seg_den + ((int64_t)bh * a.n_slots + a.n_slots - 1) * M;        // staging slot of the final state
+    float* seg_num = a.seg_num + ((int64_t)bh * a.n_slots + a.n_slots - 1) * M * D;
+    const int n_before = causal_slots_before(seg, a.seg_len, a.piece_len);
     const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
     const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
     const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
@@ -635,9 +676,9 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) U[mt][dt][r] = mu_r[mt][r] <= kNegBig ? 0.f : U[mt][dt][r];
     }
-    for (int s = 0; s < seg; ++s) {
-        const float* sd = a.seg_den + ((int64_t)bh * a.n_segs + s) * M;
-        const float* sn = a.seg_num + ((int64_t)bh * a.n_segs + s) * M * D;
+    for (int s = 0; s < n_before; ++s) {
+        const float* sd = a.seg_den + ((int64_t)bh * a.n_slots + s) * M;
+        const float* sn = a.seg_num + ((int64_t)bh * a.n_slots + s) * M * D;
         float td[CTA];
         f32x4 tu[MT][DT];
 #pragma unroll
@@ -932,7 +973,7 @@ hipError_t launch_t(const CausalArgs& a, int step, hipStream_t st)
     const int BH = a.B * a.H;
     if (a.n_segs == 1) return launch_recurrence<T>(a, step, dim3(BH, 1), st);
     // the first phase also clears the redo flags and segment counters
-    hipError_t e = launch_phase<T, true>(a, step, dim3(BH, a.n_segs - 1), st);
+    hipError_t e = launch_phase<T, true>(a, step, dim3(BH, a.n_pieces), st);
     if (e != hipSuccess) return e;
     // The last segment has staged the final state in the workspace; the fp32 kernel launched behind this one copies
     // it into (mu, den, num) for every (b,h) whose flag stayed clear and redoes the others from their incoming state.

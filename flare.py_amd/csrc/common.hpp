@@ -101,13 +101,38 @@ struct CausalArgs {
     float* mu; float* den; float* num;   // state, natural-log units for mu
     float* lse;                          // [B,H,N] or null: natural log of each token's softmax sum over the latents
     int* flags;                          // [B*H] or null: per-(b,h) "redo with the fp32 kernel" marks
-    float* seg_den; float* seg_num;      // [B*H, n_segs, M] and [B*H, n_segs, M, D]: per-segment states (matrix-core prefill)
+    float* seg_den; float* seg_num;      // [B*H, n_slots, M] and [B*H, n_slots, M, D]: local states (matrix-core prefill)
     int n_segs, seg_len;                 // token segments processed in parallel; seg_len is a multiple of 16
+    // First phase: tokens [0, (n_segs - 1) seg_len) cut into n_pieces pieces of piece_len tokens, one workgroup each
+    // (so that this phase fills the device as evenly as the recurrence does, whatever n_segs - 1 is).  A piece writes
+    // one local state per segment it touches; the slots are numbered in token order (causal_slot), and the last of the
+    // n_slots slots stages the final state.
+    int n_pieces, piece_len, n_slots;
     int B, H, N, M, D;
     int chunk;
     float scale;
     int64_t qs[3], ks[3], vs[3], ys[3];
 };
+
+// Segment boundaries b seg_len, b = 1..s, that fall inside a piece (not on a piece boundary): each of them splits a
+// piece's tokens into two local states.
+__host__ __device__ inline int causal_split_bounds(int s, int seg_len, int piece_len)
+{
+    int c = 0;
+    for (int b = 1; b <= s; ++b) c += ((int64_t)b * seg_len) % piece_len != 0;
+    return c;
+}
+// Slot of the local state of piece j's tokens inside segment s (the pair must exist), and the number of slots that
+// hold tokens before segment `seg` (what its recurrence starts from, summed in slot order).
+__host__ __device__ inline int causal_slot(int j, int s, int seg_len, int piece_len)
+{
+    return j + causal_split_bounds(s, seg_len, piece_len);
+}
+__host__ __device__ inline int causal_slots_before(int seg, int seg_len, int piece_len)
+{
+    if (seg <= 0) return 0;
+    return (int)(((int64_t)seg * seg_len + piece_len - 1) / piece_len) + causal_split_bounds(seg - 1, seg_len, piece_len);
+}
 
 constexpr int kJoinMaxGroups = 16;
 struct CausalJoinArgs {

@@ -190,6 +190,25 @@ def test_mfma_prefill_segment_length_independence(dev):
         state_close(stc, str_, 2e-2)
 
 
+@pytest.mark.parametrize("shape", [(8, 16, 3000, 128, 64), (8, 16, 5000, 128, 32), (8, 16, 3000, 256, 32), (6, 16, 2611, 128, 64)])
+def test_mfma_prefill_first_phase_pieces(dev, shape):
+    """With as many (b,h) as config 4 the library's own plan has segments longer than 256 tokens, and its first phase
+    runs as pieces that reach across segment boundaries (one local state on either side).  Same results as one
+    segment, bit-stable, and the oracle's on the (b,h) checked."""
+    B, H, N, M, D = shape
+    q, k, v = make(B, H, N, M, D, torch.bfloat16, seed=21)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    y, st = F.flare_causal_prefill(qd, kd, vd)
+    y2, st2 = F.flare_causal_prefill(qd, kd, vd)
+    assert torch.equal(y, y2) and all(torch.equal(a, b) for a, b in zip(st, st2))
+    y1, st1 = F.flare_causal_prefill(qd, kd, vd, chunk=N)
+    assert O.rel_l2(y, y1) <= 1e-2
+    state_close(st, tuple(t.double().cpu() for t in st1), 1e-2)
+    for b, h in ((0, 0), (B - 1, H - 1)):
+        yr, _ = O.causal_recurrent(q[h:h + 1].float(), k[b:b + 1, h:h + 1].float(), v[b:b + 1, h:h + 1].float())
+        assert O.rel_l2(y[b:b + 1, h:h + 1], yr) <= 2e-2
+
+
 def test_mfma_prefill_fallback_from_a_middle_segment(dev):
     # only the tokens of one middle segment leave the window: the whole (b,h) must be redone by the
     # fp32 kernel FROM THE INCOMING STATE (which the matrix-core pass must not have touched)
