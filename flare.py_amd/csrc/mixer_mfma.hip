@@ -228,8 +228,8 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * 256;
-            if (c < TCH) {
-                const int nn = n0 + c / CH, n = min(nn, n_end - 1), ch = c % CH;
+            if (TCH % 256 == 0 || c < TCH) {
+                const int nn = n0 + c / CH, n = max(min(nn, n_end - 1), 0), ch = c % CH;
                 kr[S][i] = load16_stream(k + (int64_t)n * a.ks[2] + ch * 8);
                 vr[S][i] = load16_stream(v + (int64_t)n * a.vs[2] + ch * 8);
                 if constexpr (MASKED) live[S][i] = nn < n_end && mask[n] != 0;
@@ -242,7 +242,7 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
 #pragma unroll
         for (int i = 0; i < CPT; ++i) {
             const int c = tid + i * 256;
-            if (c < TCH) {
+            if (TCH % 256 == 0 || c < TCH) {
                 const int tok = c / CH, ch = c % CH;
                 *reinterpret_cast<u32x4*>(&kt[S][k_slot(tok, ch)]) = kr[S][i];
                 if constexpr (MASKED) {
@@ -404,24 +404,31 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
             if (ragged) tile(std::true_type{});
             else        tile(std::false_type{});
         };
+        // Loads and LDS stores of the staging are unconditional (rows past the range repeat its last row, a tile past
+        // it is staged and never read) and the loop over pairs of tiles has its one exit at the bottom: with a branch
+        // around a load, or a way from the middle of the pair back to the loop's head, the compiler cannot count the
+        // loads in flight and waits for all of them at every tile, the ones requested an iteration ago included.
         auto iter = [&](int n0, auto par) {
             constexpr int P = decltype(par)::value;
             using Other = std::integral_constant<int, 1 - P>;
             __syncthreads();
-            if (n0 + kGTile < n_end) store_tile(Other{}, masked_tag);
-            if (n0 + 3 * kGTile < n_end) load_tile(Other{}, n0 + 3 * kGTile, masked_tag);
+            store_tile(Other{}, masked_tag);
+            load_tile(Other{}, n0 + 3 * kGTile, masked_tag);
             process(n0, P);
         };
-        if (n_begin < n_end) {
+        const int tiles = n_begin < n_end ? (n_end - n_begin + kGTile - 1) / kGTile : 0;
+        if (tiles > 0) {
             load_tile(Set0{}, n_begin, masked_tag);
-            if (n_begin + kGTile < n_end) load_tile(Set1{}, n_begin + kGTile, masked_tag);
+            load_tile(Set1{}, n_begin + kGTile, masked_tag);
             store_tile(Set0{}, masked_tag);
-            if (n_begin + 2 * kGTile < n_end) load_tile(Set0{}, n_begin + 2 * kGTile, masked_tag);
+            load_tile(Set0{}, n_begin + 2 * kGTile, masked_tag);
         }
-        for (int n0 = n_begin; n0 < n_end; n0 += 2 * kGTile) {
+        int n0 = n_begin;
+        for (int i = 0; i < tiles / 2; ++i, n0 += 2 * kGTile) {
             iter(n0, Set0{});
-            if (n0 + kGTile < n_end) iter(n0 + kGTile, Set1{});
+            iter(n0 + kGTile, Set1{});
         }
+        if (tiles & 1) iter(n0, Set0{});
     };
 
     // validate: every denominator of this wave inside the safe range, numerators finite.  With a key mask a
