@@ -303,9 +303,14 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
                     // h = act(W1[j] n + b1[j]): tile ft of h is half (ft & 1) of k-step ft / 2 of the next product
                     auto first = [&](auto act_c) {
                         constexpr int ACT = decltype(act_c)::value;
+                        // bias rows requested two feature tiles ahead, as in the chain below
+                        f32x4 bias_q[2];
+#pragma unroll
+                        for (int i = 0; i < 2; ++i) bias_q[i] = vec4(bl + 16 * (i < FT ? i : 0), has_bias);
 #pragma unroll
                         for (int ft = 0; ft < FT; ++ft) {
-                            const f32x4 bias = vec4(bl + 16 * ft, has_bias);
+                            const f32x4 bias = bias_q[ft & 1];
+                            if (ft + 2 < FT) bias_q[ft & 1] = vec4(bl + 16 * (ft + 2), has_bias);
                             f32x4 acc[TW];
 #pragma unroll
                             for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
