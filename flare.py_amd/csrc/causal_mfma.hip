@@ -858,6 +858,10 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
                 yacc[dt] = P_::mma16(aop, vop, yacc[dt]);
             }
         }
+        // The next chunk's rows, requested at the top of this iteration, are waited for here, before the stores below
+        // are issued: loads and stores complete in order on one counter, the stores sit under per-lane conditions, and
+        // a wait placed at the hand-over after them could only wait for everything, store acknowledgements included.
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
         // y rows / softmax sums, transposed through the wave's (now free) G^T region: lane (g, c16) ends
         // up with y[token c16][16 dt + 4g .. 4g + 3]
         {
