@@ -760,6 +760,11 @@ int flare_causal_linear_fwd(const FlareCausalLinearDesc* desc, const void* q, co
     for (int i = 0; i < 3; ++i) {
         a.qs[i] = desc->q_stride[i]; a.ks[i] = desc->k_stride[i]; a.vs[i] = desc->v_stride[i]; a.ys[i] = desc->y_stride[i];
     }
+    // 16-bit inputs of the sizes the matrix-core kernels take go there when every row is 16-byte aligned
+    const bool mfma = !(desc->flags & FLARE_FLAG_FORCE_GENERIC) && flare::causal_linear_mfma_supported(desc->dtype, desc->Dk, desc->Dv) &&
+                      strides_mult8(desc->q_stride) && strides_mult8(desc->k_stride) && strides_mult8(desc->v_stride) &&
+                      strides_mult8(desc->y_stride) && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(y);
+    if (mfma) return hip_status(flare::launch_causal_linear_mfma(a, desc->dtype, static_cast<hipStream_t>(stream)), "causal linear launch");
     return hip_status(flare::launch_causal_linear(a, desc->dtype, static_cast<hipStream_t>(stream)), "causal linear launch");
 }
 

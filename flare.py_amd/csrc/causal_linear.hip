@@ -197,6 +197,12 @@ hipError_t launch_t(const CausalLinearArgs& a, hipStream_t st)
 
 int causal_linear_tile() { return kTile; }
 
+hipError_t launch_causal_linear_prefix(const CausalLinearArgs& a, hipStream_t st)
+{
+    hipLaunchKernelGGL(causal_linear_prefix_kernel, dim3((a.Dk * a.Dv + 255) / 256, a.B * a.H), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
 hipError_t launch_causal_linear(const CausalLinearArgs& a, int dtype, hipStream_t st)
 {
     if (a.Dk > 128 || a.Dv > 128) return hipErrorInvalidValue;

@@ -307,6 +307,10 @@ hipError_t launch_mlp_wgrad(const MlpWgradArgs& a, int w_dtype, hipStream_t st);
 
 int        causal_linear_tile();
 hipError_t launch_causal_linear(const CausalLinearArgs& a, int dtype, hipStream_t st);
+hipError_t launch_causal_linear_prefix(const CausalLinearArgs& a, hipStream_t st);   // exclusive prefix over the segment states
+// matrix-core kernels (causal_linear_mfma.hip): 16-bit inputs, Dk in {64, 128}, Dv in {32, 64, 128}
+bool       causal_linear_mfma_supported(int dtype, int Dk, int Dv);
+hipError_t launch_causal_linear_mfma(const CausalLinearArgs& a, int dtype, hipStream_t st);
 
 hipError_t launch_triple_state(const TripleArgs& a, int dtype, hipStream_t st);
 hipError_t launch_triple_merge(const TripleArgs& a, hipStream_t st);

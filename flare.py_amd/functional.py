@@ -974,7 +974,7 @@ def flare_causal_decode_step(q, k_t, v_t, state, scale: float = 1.0, inplace: bo
 # --------------------------------------------------------------------------------------
 # causal linear attention
 # --------------------------------------------------------------------------------------
-def _causal_linear_forward(q, k, v, n_segs: int = 0):
+def _causal_linear_forward(q, k, v, n_segs: int = 0, force_generic: bool = False):
     _require_cuda(q, k, v)
     lib = _lib.load()
     if q.dim() != 4 or q.shape != k.shape:
@@ -991,6 +991,7 @@ def _causal_linear_forward(q, k, v, n_segs: int = 0):
     d.B, d.H, d.N, d.Dk, d.Dv = B, H, N, Dk, Dv
     d.dtype = _dtype_code(q)
     d.n_segs = int(n_segs)
+    d.flags = _lib.FLAG_FORCE_GENERIC if force_generic else 0
     d.q_stride, d.k_stride, d.v_stride, d.y_stride = _s3(q), _s3(k), _s3(v), _s3(y)
     with _on_device(q.device):
         need = C.c_size_t(0)
@@ -1034,12 +1035,15 @@ class _CausalLinearFn(torch.autograd.Function):
             return torch.autograd.grad(y, (qq, kk, vv), gy)
 
 
-def causal_linear_attention(q, k, v, n_segs: int = 0):
+def causal_linear_attention(q, k, v, n_segs: int = 0, force_generic: bool = False):
     """y_t = (1/N) sum_{tau<=t} <q_t,k_tau> v_tau for q,k [B,H,N,Dk], v [B,H,N,Dv] -> [B,H,N,Dv]
-    (lra/models/triton/causal_linear.py:317-336).  n_segs = token segments run in parallel (0 = auto)."""
-    if n_segs == 0 and torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+    (lra/models/triton/causal_linear.py:317-336).  n_segs = token segments run in parallel (0 = auto).
+    bf16 / f16 inputs with Dk in {64, 128}, Dv in {32, 64, 128} and 16-byte aligned rows run on the matrix cores
+    (products in the input type, fp32 accumulation and state); everything else, and force_generic=True, in fp32
+    arithmetic."""
+    if n_segs == 0 and not force_generic and torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
         return _CausalLinearFn.apply(q, k, v)
-    return _causal_linear_forward(q, k, v, n_segs)
+    return _causal_linear_forward(q, k, v, n_segs, force_generic)
 
 
 class CausalLinear:

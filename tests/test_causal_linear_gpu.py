@@ -77,3 +77,49 @@ def test_errors_and_autograd_plumbing(dev):
     O.causal_linear_closed_form(qr, kr, vr).square().sum().backward()
     for a, b in ((qd, qr), (kd, kr), (vd, vr)):
         assert O.rel_l2(a.grad, b.grad) <= 1e-4
+
+
+# ---- matrix-core kernels (bf16 / f16, Dk in {64, 128}, Dv in {32, 64, 128}) ---------------------------------
+@pytest.mark.parametrize("shape", [(1, 2, 64, 64, 32), (1, 2, 65, 64, 32), (2, 2, 300, 64, 64), (1, 1, 513, 128, 32),
+                                   (1, 3, 1, 64, 128), (2, 1, 17, 128, 64), (1, 2, 4096, 64, 32), (1, 1, 2500, 128, 128)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_matrix_core_shapes(dev, shape, dtype):
+    """Every segment count gives the oracle's result (the state crosses tile and segment boundaries), twice the same
+    bits, and close to the fp32-arithmetic kernel on the same inputs."""
+    q, k, v = make(*shape, dtype, seed=shape[2])
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    yr = O.causal_linear_closed_form(q, k, v)
+    for s in (0, 1, 3):
+        y = F.causal_linear_attention(qd, kd, vd, n_segs=s)
+        assert y.dtype == dtype and torch.equal(y, F.causal_linear_attention(qd, kd, vd, n_segs=s))
+        assert O.rel_l2(y, yr) <= TOL[dtype], s
+    yg = F.causal_linear_attention(qd, kd, vd, force_generic=True)
+    assert O.rel_l2(y, yg.cpu()) <= TOL[dtype]
+
+
+def test_matrix_core_kernel_runs_and_takes_token_major_views(dev):
+    """The reference's own test shape in bf16, q, k, v as 'b n (h d) -> b h n d' views: the matrix-core kernels run
+    (profiler), no copy is made, and rows that are not 16-byte aligned fall back to the fp32-arithmetic kernel."""
+    from torch.profiler import ProfilerActivity, profile
+    B, H, N, Dk, Dv = 1, 8, 2048, 128, 32
+    g = torch.Generator().manual_seed(7)
+    xq = torch.randn(2, B, N, H * Dk, generator=g).bfloat16().to(dev)
+    xv = torch.randn(B, N, H * Dv, generator=g).bfloat16().to(dev)
+    q, k = (t.view(B, N, H, Dk).permute(0, 2, 1, 3) for t in xq)
+    v = xv.view(B, N, H, Dv).permute(0, 2, 1, 3)
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        y = F.causal_linear_attention(q, k, v)
+        torch.cuda.synchronize()
+    names = {e.key for e in prof.key_averages()}
+    assert any("causal_linear_mfma_kernel" in n for n in names), names
+    assert not any("copy" in n.lower() for n in names), names
+    yr = O.causal_linear_closed_form(q.cpu(), k.cpu(), v.cpu())
+    assert O.rel_l2(y, yr) <= 2e-2
+    # a view that starts 8 bytes into a row: the same values through the other kernel
+    pad = torch.zeros(B, H, N, Dk + 4, dtype=torch.bfloat16, device=dev)
+    pad[..., 4:] = q
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        y2 = F.causal_linear_attention(pad[..., 4:], k, v)
+        torch.cuda.synchronize()
+    assert not any("causal_linear_mfma_kernel" in e.key for e in prof.key_averages())
+    assert O.rel_l2(y2, yr) <= 2e-2
