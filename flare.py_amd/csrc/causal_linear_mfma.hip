@@ -1,4 +1,5 @@
-// Causal linear attention on the matrix cores (bf16 / f16, Dk in {64, 128}, Dv in {32, 64, 128}).
+// Causal linear attention on the matrix cores: bf16 / f16 (Dk in {64, 128}, Dv in {32, 64, 128}) and, further down,
+// fp32 (Dk in {64, 128}, Dv in {32, 64}).
 //
 //   y_t = (1/N) sum_{tau <= t} <q_t, k_tau> v_tau        (lra/models/triton/causal_linear.py:317-336)
 //
@@ -268,6 +269,214 @@ __global__ __launch_bounds__(256, 2) void causal_linear_mfma_kernel(CausalLinear
     }
 }
 
+// ---- fp32 inputs: the same scheme on v_mfma_f32_16x16x4_f32 ------------------------------------------------------
+// A: lane (row c16, k = g) one float, B: lane (column c16, k = g) one float, accumulators as above.  A product over Dk
+// takes Dk/4 instructions; the k-slot of lane group g in instruction j is feature g Dk/4 + j, so that a lane's share of a
+// Q or K row is contiguous (16-byte loads).  An accumulator tile of A^T (lane = token t, registers = tokens tau = 4g + r)
+// is the B operand of four instructions of the next product, register r for the instruction whose k-slots are 4g + r.
+template <int DK, int DV, bool STATE_ONLY>
+constexpr size_t lds_bytes_f32()
+{
+    return (size_t)kTile * (DK + 4 + DV + 4) * 4 + (STATE_ONLY ? 0 : (size_t)DV * DK * 4);
+}
+
+template <int DK, int DV, bool STATE_ONLY>
+__global__ __launch_bounds__(256, 2) void causal_linear_f32_kernel(CausalLinearArgs a)
+{
+    constexpr int QL = DK / 4;                       // features per lane group
+    constexpr int IT = DK / 16, DT = DV / 16, ITW = IT / 4;
+    constexpr int KS = DK + 4, VS = DV + 4;          // LDS row strides in floats
+    constexpr int KPT = kTile * (DK / 4) / 256, VPT = kTile * (DV / 4) / 256;
+    static_assert(IT % 4 == 0 && VPT >= 1, "Dk in {64, 128}, Dv a multiple of 16 from 16");
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    float* kt = reinterpret_cast<float*>(smem);      // [64][KS]
+    float* vt = kt + kTile * KS;                     // [64][VS]
+    float* sop = vt + kTile * VS;                    // [DT][QL][64]: S^T / N as A operands of the inter-tile product
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int seg = blockIdx.x, bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+    const float* q = (const float*)a.q + b * a.qs[0] + h * a.qs[1];
+    const float* k = (const float*)a.k + b * a.ks[0] + h * a.ks[1];
+    const float* v = (const float*)a.v + b * a.vs[0] + h * a.vs[1];
+    float* y = (float*)a.y + b * a.ys[0] + h * a.ys[1];
+    float* slot = a.states + ((int64_t)bh * a.n_segs + seg) * DK * DV;
+    const int n_lo = seg * a.seg_len, n_hi = min(a.N, n_lo + a.seg_len);
+    const int tiles = (n_hi - n_lo + kTile - 1) / kTile;
+
+    f32x4 U[ITW][DT];
+#pragma unroll
+    for (int itw = 0; itw < ITW; ++itw)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                U[itw][dt][r] = STATE_ONLY ? 0.f : slot[(int64_t)(16 * (w * ITW + itw) + 4 * g + r) * DV + 16 * dt + c16];
+
+    f32x4 kr[KPT], vr[VPT], qn[QL / 4], qc[QL / 4];
+    auto fetch = [&](int n0) {
+#pragma unroll
+        for (int i = 0; i < KPT; ++i) {
+            const int c = tid + i * 256, tok = c / (DK / 4), ch = c % (DK / 4);
+            kr[i] = *reinterpret_cast<const f32x4*>(k + (int64_t)min(n0 + tok, n_hi - 1) * a.ks[2] + ch * 4);
+        }
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int c = tid + i * 256, tok = c / (DV / 4), ch = c % (DV / 4);
+            vr[i] = *reinterpret_cast<const f32x4*>(v + (int64_t)min(n0 + tok, n_hi - 1) * a.vs[2] + ch * 4);
+        }
+        if constexpr (!STATE_ONLY) {
+            const int n = min(n0 + 16 * w + c16, n_hi - 1);
+#pragma unroll
+            for (int j = 0; j < QL / 4; ++j) qn[j] = *reinterpret_cast<const f32x4*>(q + (int64_t)n * a.qs[2] + g * QL + 4 * j);
+        }
+    };
+    auto stage = [&](int n0) {
+        const f32x4 z4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < KPT; ++i) {
+            const int c = tid + i * 256, tok = c / (DK / 4), ch = c % (DK / 4);
+            *reinterpret_cast<f32x4*>(kt + tok * KS + ch * 4) = n0 + tok < n_hi ? kr[i] : z4;
+        }
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int c = tid + i * 256, tok = c / (DV / 4), ch = c % (DV / 4);
+            *reinterpret_cast<f32x4*>(vt + tok * VS + ch * 4) = n0 + tok < n_hi ? vr[i] : z4;
+        }
+    };
+    // entry (dt, j, lane (gl, cl)) = S[gl QL + j][16 dt + cl] / N; the owner of S[i][16 dt + c16] writes it there
+    auto publish = [&]() {
+#pragma unroll
+        for (int itw = 0; itw < ITW; ++itw)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 16 * (w * ITW + itw) + 4 * g + r;
+                    sop[(dt * QL + i % QL) * 64 + (i / QL) * 16 + c16] = U[itw][dt][r] * a.inv_n;
+                }
+    };
+    auto update = [&]() {
+#pragma unroll
+        for (int m = 0; m < kTile / 4; ++m) {       // tokens 4m + g
+            float vop[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vop[dt] = vt[(4 * m + g) * VS + 16 * dt + c16];
+#pragma unroll
+            for (int itw = 0; itw < ITW; ++itw) {
+                const float kop = kt[(4 * m + g) * KS + 16 * (w * ITW + itw) + c16];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) U[itw][dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(kop, vop[dt], U[itw][dt], 0, 0, 0);
+            }
+        }
+    };
+
+    if (tiles > 0) {
+        fetch(n_lo);
+        stage(n_lo);
+        if constexpr (!STATE_ONLY) {
+#pragma unroll
+            for (int j = 0; j < QL / 4; ++j) qc[j] = qn[j];
+            publish();
+        }
+    }
+    __syncthreads();
+
+    const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
+    int n0 = n_lo;
+    for (int t = 0; t < tiles; ++t, n0 += kTile) {
+        fetch(n0 + kTile);
+
+        if constexpr (!STATE_ONLY) {
+            f32x4 yacc[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) yacc[dt] = zf;
+#pragma unroll
+            for (int bl = 0; bl < 4; ++bl) {
+                if (bl > w) break;      // uniform over the wave
+                f32x4 s = zf;
+#pragma unroll
+                for (int j4 = 0; j4 < QL / 4; ++j4) {
+                    const f32x4 ka = *reinterpret_cast<const f32x4*>(kt + (16 * bl + c16) * KS + g * QL + 4 * j4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) s = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[e], qc[j4][e], s, 0, 0, 0);
+                }
+                if (bl == w) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) s[r] = 4 * g + r <= c16 ? s[r] : 0.f;
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+                        yacc[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(vt[(16 * bl + 4 * g + r) * VS + 16 * dt + c16], s[r], yacc[dt], 0, 0, 0);
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) yacc[dt] *= a.inv_n;
+#pragma unroll
+            for (int j4 = 0; j4 < QL / 4; ++j4)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+                        yacc[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(sop[(dt * QL + 4 * j4 + e) * 64 + lane], qc[j4][e], yacc[dt], 0, 0, 0);
+            __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the next tile's rows, before the stores (see the 16-bit kernel)
+            const int n = n0 + 16 * w + c16;
+            if (n < n_hi) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f32x4*>(y + (int64_t)n * a.ys[2] + 16 * dt + 4 * g) = yacc[dt];
+            }
+        }
+
+        update();
+        __syncthreads();
+        stage(n0 + kTile);
+        if constexpr (!STATE_ONLY) {
+#pragma unroll
+            for (int j = 0; j < QL / 4; ++j) qc[j] = qn[j];
+            publish();
+        }
+        __syncthreads();
+    }
+
+    if constexpr (STATE_ONLY) {
+#pragma unroll
+        for (int itw = 0; itw < ITW; ++itw)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    slot[(int64_t)(16 * (w * ITW + itw) + 4 * g + r) * DV + 16 * dt + c16] = U[itw][dt][r];
+    }
+}
+
+template <int DK, int DV>
+hipError_t launch_f32_dd(const CausalLinearArgs& a, hipStream_t st)
+{
+    const int BH = a.B * a.H;
+    auto state_k = causal_linear_f32_kernel<DK, DV, true>;
+    auto out_k = causal_linear_f32_kernel<DK, DV, false>;
+    constexpr size_t lds_s = lds_bytes_f32<DK, DV, true>(), lds_o = lds_bytes_f32<DK, DV, false>();
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(state_k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_s);
+    if (e != hipSuccess) return e;
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(out_k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_o);
+    if (e != hipSuccess) return e;
+    if (a.n_segs > 1) hipLaunchKernelGGL(state_k, dim3(a.n_segs - 1, BH), dim3(256), lds_s, st, a);
+    e = launch_causal_linear_prefix(a, st);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(out_k, dim3(a.n_segs, BH), dim3(256), lds_o, st, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_f32(const CausalLinearArgs& a, hipStream_t st)
+{
+    if (a.Dk == 64 && a.Dv == 32) return launch_f32_dd<64, 32>(a, st);
+    if (a.Dk == 64 && a.Dv == 64) return launch_f32_dd<64, 64>(a, st);
+    if (a.Dk == 128 && a.Dv == 32) return launch_f32_dd<128, 32>(a, st);
+    if (a.Dk == 128 && a.Dv == 64) return launch_f32_dd<128, 64>(a, st);
+    return hipErrorInvalidValue;
+}
+
 template <typename T, int DK, int DV>
 hipError_t launch_dd(const CausalLinearArgs& a, hipStream_t st)
 {
@@ -309,11 +518,13 @@ hipError_t launch_t(const CausalLinearArgs& a, hipStream_t st)
 
 bool causal_linear_mfma_supported(int dtype, int Dk, int Dv)
 {
+    if (dtype == 0) return (Dk == 64 || Dk == 128) && (Dv == 32 || Dv == 64);
     return (dtype == 1 || dtype == 2) && (Dk == 64 || Dk == 128) && (Dv == 32 || Dv == 64 || Dv == 128);
 }
 
 hipError_t launch_causal_linear_mfma(const CausalLinearArgs& a, int dtype, hipStream_t st)
 {
+    if (dtype == 0) return launch_f32(a, st);
     return dtype == 1 ? launch_t<bf16_t>(a, st) : launch_t<f16_t>(a, st);
 }
 

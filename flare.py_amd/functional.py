@@ -1038,9 +1038,9 @@ class _CausalLinearFn(torch.autograd.Function):
 def causal_linear_attention(q, k, v, n_segs: int = 0, force_generic: bool = False):
     """y_t = (1/N) sum_{tau<=t} <q_t,k_tau> v_tau for q,k [B,H,N,Dk], v [B,H,N,Dv] -> [B,H,N,Dv]
     (lra/models/triton/causal_linear.py:317-336).  n_segs = token segments run in parallel (0 = auto).
-    bf16 / f16 inputs with Dk in {64, 128}, Dv in {32, 64, 128} and 16-byte aligned rows run on the matrix cores
-    (products in the input type, fp32 accumulation and state); everything else, and force_generic=True, in fp32
-    arithmetic."""
+    Dk in {64, 128} with 16-byte aligned rows runs on the matrix cores: bf16 / f16 with Dv in {32, 64, 128} (products
+    in the input type, fp32 accumulation and state), fp32 with Dv in {32, 64} (fp32 products); everything else, and
+    force_generic=True, as fp32 FMA loops."""
     if n_segs == 0 and not force_generic and torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
         return _CausalLinearFn.apply(q, k, v)
     return _causal_linear_forward(q, k, v, n_segs, force_generic)

@@ -285,9 +285,9 @@ int flare_causal_join(int32_t dtype, int32_t n_groups, int64_t rows, int32_t D, 
 int flare_causal_linear_workspace_bytes(const FlareCausalLinearDesc* desc, size_t* bytes);
 
 /* Segment states, exclusive prefix over the segments, then the outputs; sums in a fixed order.
- * bf16 / f16 problems with Dk in {64, 128}, Dv in {32, 64, 128}, strides that are multiples of 8 elements and
- * 16-byte aligned pointers run on the matrix cores (products in the input type, fp32 accumulation and state);
- * everything else, and FLARE_FLAG_FORCE_GENERIC, in fp32 arithmetic. */
+ * Problems with Dk in {64, 128}, strides that are multiples of 8 elements and 16-byte aligned pointers run on the
+ * matrix cores: bf16 / f16 with Dv in {32, 64, 128} (products in the input type, fp32 accumulation and state) and
+ * fp32 with Dv in {32, 64} (fp32 products).  Everything else, and FLARE_FLAG_FORCE_GENERIC, as fp32 FMA loops. */
 int flare_causal_linear_fwd(const FlareCausalLinearDesc* desc, const void* q, const void* k,
                             const void* v, void* y, void* workspace, size_t workspace_bytes,
                             void* stream);

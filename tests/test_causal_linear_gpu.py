@@ -79,13 +79,15 @@ def test_errors_and_autograd_plumbing(dev):
         assert O.rel_l2(a.grad, b.grad) <= 1e-4
 
 
-# ---- matrix-core kernels (bf16 / f16, Dk in {64, 128}, Dv in {32, 64, 128}) ---------------------------------
+# ---- matrix-core kernels (Dk in {64, 128}; bf16 / f16 with Dv in {32, 64, 128}, fp32 with Dv in {32, 64}) ------
 @pytest.mark.parametrize("shape", [(1, 2, 64, 64, 32), (1, 2, 65, 64, 32), (2, 2, 300, 64, 64), (1, 1, 513, 128, 32),
                                    (1, 3, 1, 64, 128), (2, 1, 17, 128, 64), (1, 2, 4096, 64, 32), (1, 1, 2500, 128, 128)])
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_matrix_core_shapes(dev, shape, dtype):
     """Every segment count gives the oracle's result (the state crosses tile and segment boundaries), twice the same
     bits, and close to the fp32-arithmetic kernel on the same inputs."""
+    if dtype == torch.float32 and shape[4] > 64:
+        shape = shape[:4] + (64,)             # the fp32 kernels (16x16x4 products) take Dv up to 64
     q, k, v = make(*shape, dtype, seed=shape[2])
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     yr = O.causal_linear_closed_form(q, k, v)
@@ -123,3 +125,18 @@ def test_matrix_core_kernel_runs_and_takes_token_major_views(dev):
         torch.cuda.synchronize()
     assert not any("causal_linear_mfma_kernel" in e.key for e in prof.key_averages())
     assert O.rel_l2(y2, yr) <= 2e-2
+
+
+def test_fp32_matrix_core_kernel_runs_at_the_reference_shape(dev):
+    """B=1, H=8, N=2048, Dk=128, Dv=32 in fp32 (causal_linear.py:650) goes through the 16x16x4 fp32 products."""
+    from torch.profiler import ProfilerActivity, profile
+    q, k, v = make(1, 8, 2048, 128, 32, torch.float32, seed=3)
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        y = F.causal_linear_attention(q.to(dev), k.to(dev), v.to(dev))
+        torch.cuda.synchronize()
+    assert any("causal_linear_f32_kernel" in e.key for e in prof.key_averages())
+    yr = O.causal_linear_closed_form(q, k, v)
+    assert O.rel_l2(y, yr) <= 1e-5
+    assert torch.allclose(y.cpu().double(), yr, atol=1e-5, rtol=1e-5)
+    yg = F.causal_linear_attention(q.to(dev), k.to(dev), v.to(dev), force_generic=True)
+    assert O.rel_l2(yg, yr) <= 1e-5
