@@ -12,9 +12,10 @@
 // One workgroup = 4 waves = one segment of one (b,h).  Wave w owns tokens 16 w .. 16 w + 15 of every tile for the
 // output and the state rows i = (Dk/4) w .. (Dk/4)(w+1) - 1 for the update.  All products are taken transposed,
 //   A^T[tau, t] = sum_i K[tau,i] Q[t,i]        (16x16x32; K rows from LDS, Q rows straight from global memory)
-//   Y^T[d, t]  += sum_tau V^T[d,tau] A^T[tau,t] (16x16x16; the accumulator tile of A^T, masked and packed, is the B operand)
+//   Y^T[d, t]  += sum_tau V^T[d,tau] A^T[tau,t] (16x16x32 over two token blocks; the accumulator tiles of A^T, masked and
+//                                                packed, are the B operand)
 //   Y^T[d, t]  += sum_i S^T[d,i] Q[t,i]         (16x16x32; S^T published in LDS in operand order by its owners)
-//   S[i, d]    += sum_tau K^T[i,tau] V[tau,d]   (16x16x16; both operands by transposed LDS reads)
+//   S[i, d]    += sum_tau K^T[i,tau] V[tau,d]   (16x16x32; both operands by transposed LDS reads)
 // so that a lane ends up with four consecutive channels of one token's output row.
 #include <type_traits>
 
@@ -170,18 +171,25 @@ __global__ __launch_bounds__(256, 2) void causal_linear_mfma_kernel(CausalLinear
             }
         }
     };
+    // two 16-token blocks as one operand of a 32-deep product: k-slots 8g + e = token 4g + e of block bl for e < 4,
+    // of block bl + 1 for e >= 4 (any order of the contraction index will do as long as both operands agree)
+    auto tr32 = [&](const uint16_t* tile, int stride, int bl, int col) {
+        const uint2 lo = tr16(tile + (16 * bl + 4 * g + (c16 >> 2)) * stride + col + 4 * (c16 & 3));
+        const uint2 hi = tr16(tile + (16 * bl + 16 + 4 * g + (c16 >> 2)) * stride + col + 4 * (c16 & 3));
+        return u32x4{lo.x, lo.y, hi.x, hi.y};
+    };
     // S += K^T V over the 64 tokens of the staged tile, for the wave's rows of S
     auto update = [&]() {
 #pragma unroll
-        for (int bl = 0; bl < 4; ++bl) {
-            uint2 vop[DT];
+        for (int bl = 0; bl < 4; bl += 2) {
+            u32x4 vop[DT];
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vop[dt] = tr16(vt + (16 * bl + 4 * g + (c16 >> 2)) * VS + 16 * dt + 4 * (c16 & 3));
+            for (int dt = 0; dt < DT; ++dt) vop[dt] = tr32(vt, VS, bl, 16 * dt);
 #pragma unroll
             for (int itw = 0; itw < ITW; ++itw) {
-                const uint2 kop = tr16(kt + (16 * bl + 4 * g + (c16 >> 2)) * KS + 16 * (w * ITW + itw) + 4 * (c16 & 3));
+                const u32x4 kop = tr32(kt, KS, bl, 16 * (w * ITW + itw));
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) U[itw][dt] = M_::mma16(kop, vop[dt], U[itw][dt]);
+                for (int dt = 0; dt < DT; ++dt) U[itw][dt] = M_::mma32(kop, vop[dt], U[itw][dt]);
             }
         }
     };
@@ -207,26 +215,29 @@ __global__ __launch_bounds__(256, 2) void causal_linear_mfma_kernel(CausalLinear
             f32x4 yacc[DT];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) yacc[dt] = zf;
-#pragma unroll
-            for (int bl = 0; bl < 4; ++bl) {
-                if (bl > w) break;      // uniform over the wave
+            // A^T of a block: lane = column t = c16, rows tau = 4g + r; the diagonal block keeps tau <= t
+            auto block_scores = [&](int bl) {
                 f32x4 s = zf;
 #pragma unroll
                 for (int kd = 0; kd < KD; ++kd) {
                     const u32x4 ka = *reinterpret_cast<const u32x4*>(kt + (16 * bl + c16) * KS + 32 * kd + 8 * g);
                     s = M_::mma32(ka, qc[kd], s);
                 }
-                // lane: column t = c16, rows tau = 4g + r of block bl
                 if (bl == w) {
 #pragma unroll
                     for (int r = 0; r < 4; ++r) s[r] = 4 * g + r <= c16 ? s[r] : 0.f;
                 }
-                const uint2 pb = make_uint2(M_::pack2(s[0], s[1]), M_::pack2(s[2], s[3]));
+                return make_uint2(M_::pack2(s[0], s[1]), M_::pack2(s[2], s[3]));
+            };
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    const uint2 vop = tr16(vt + (16 * bl + 4 * g + (c16 >> 2)) * VS + 16 * dt + 4 * (c16 & 3));
-                    yacc[dt] = M_::mma16(vop, pb, yacc[dt]);
-                }
+            for (int bl = 0; bl < 4; bl += 2) {
+                if (bl > w) break;      // uniform over the wave
+                const uint2 p0 = block_scores(bl);
+                uint2 p1 = make_uint2(0u, 0u);
+                if (bl + 1 <= w) p1 = block_scores(bl + 1);
+                const u32x4 pb = {p0.x, p0.y, p1.x, p1.y};
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) yacc[dt] = M_::mma32(tr32(vt, VS, bl, 16 * dt), pb, yacc[dt]);
             }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) yacc[dt] *= a.inv_n;
