@@ -144,6 +144,7 @@ void fill_mixer_args(flare::MixerArgs& a, const FlareMixerDesc* d, const MixerPl
     a.scale_log2 = d->scale * flare::kLog2e;
     a.no_mfma32 = (d->flags & FLARE_FLAG_MFMA16) ? 1 : 0;
     a.gather32 = (d->flags & FLARE_FLAG_GATHER32) ? 1 : 0;
+    a.force_fma = (d->flags & FLARE_FLAG_FORCE_GENERIC) ? 1 : 0;
     for (int i = 0; i < 3; ++i) {
         a.qs[i] = d->q_stride[i]; a.ks[i] = d->k_stride[i]; a.vs[i] = d->v_stride[i]; a.ys[i] = d->y_stride[i];
     }

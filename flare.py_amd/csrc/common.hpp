@@ -89,6 +89,7 @@ struct MixerArgs {
     float scale_log2;         // scale * log2(e)
     int no_mfma32;            // 1: keep the 16x16x32 kernels where the 32x32x16 ones would run
     int gather32;             // 1: the gather may take the 32x32x16 kernel too
+    int force_fma;            // 1: fp32 problems keep the FMA kernels (no fp32 matrix-core kernels)
     // attention dropout (fp32-FMA kernels only): an entry of the softmax weights is kept when its hash is >= drop_thr
     // (24-bit compare) and then scaled by drop_rs = 1 / (1 - p); drop_thr == 0 switches it off
     uint32_t drop_thr, seed_lo, seed_hi;
@@ -266,6 +267,10 @@ constexpr int bwd_dq_wgs_per_cu(int D, int CT)
 hipError_t launch_gather_generic(const MixerArgs& a, int dtype, hipStream_t st);
 hipError_t launch_gather_merge(const MixerArgs& a, hipStream_t st);
 hipError_t launch_scatter_generic(const MixerArgs& a, int dtype, hipStream_t st);
+// fp32 inputs on v_mfma_f32_16x16x4_f32 (mixer_f32_mfma.hip): taken by the two launchers above when the problem allows
+bool       f32_mfma_mixer_ok(const MixerArgs& a, bool scatter);
+hipError_t launch_gather_f32_mfma(const MixerArgs& a, hipStream_t st);
+hipError_t launch_scatter_f32_mfma(const MixerArgs& a, hipStream_t st);
 int        gather_generic_parts_per_wg();
 
 bool       mfma_mixer_supported(int dtype, int M, int D);

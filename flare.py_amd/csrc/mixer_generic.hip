@@ -244,6 +244,8 @@ int gather_generic_parts_per_wg() { return kGatherGroups; }
 
 hipError_t launch_gather_generic(const MixerArgs& a, int dtype, hipStream_t st)
 {
+    // fp32 problems the matrix-core kernels take (same grid, one partial per wave as here)
+    if (dtype == 0 && f32_mfma_mixer_ok(a, false)) return launch_gather_f32_mfma(a, st);
     const int mblocks = (a.M + kGatherLat - 1) / kGatherLat;
     dim3 grid(a.n_splits * mblocks, a.H, a.B);
     switch (dtype) {
@@ -263,6 +265,7 @@ hipError_t launch_gather_merge(const MixerArgs& a, hipStream_t st)
 
 hipError_t launch_scatter_generic(const MixerArgs& a, int dtype, hipStream_t st)
 {
+    if (dtype == 0 && f32_mfma_mixer_ok(a, true)) return launch_scatter_f32_mfma(a, st);
     dim3 grid((a.N + kScatterThreads - 1) / kScatterThreads, a.H, a.B);
     switch (dtype) {
         case 0: return scatter_dispatch_d<float>(a, grid, st);

@@ -574,3 +574,68 @@ def test_dead_latents_get_no_weight_at_any_scale(dev, dtype, scale):
     if dtype == torch.float16 and scale == 1e-4:
         assert bias is None and F.mixer_kernel_name(q.to(dev), k.to(dev), v.to(dev), scale=scale) == "generic"
     check(dev, q, k, v, scale=scale)
+
+
+# ---- fp32 inputs on the fp32 matrix instruction (taken by the generic launchers when the problem allows) -------------
+@pytest.mark.parametrize("shape", [(1, 8, 4096, 64, 16), (2, 3, 1000, 16, 16), (1, 2, 777, 48, 32), (1, 2, 5000, 256, 32),
+                                   (2, 1, 333, 80, 64), (1, 1, 1, 16, 16), (1, 2, 17, 128, 64), (3, 2, 2049, 32, 32)])
+def test_fp32_matrix_core_mixer_shapes(dev, shape):
+    """Parity at the fp32 bar, every split count the same result to rounding, two runs the same bits, the latents'
+    log-sum-exp against the oracle's."""
+    from torch.profiler import ProfilerActivity, profile
+    q, k, v = make(*shape, torch.float32, seed=shape[2])
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        y, z = check(dev, q, k, v, scale=0.8)
+    names = {e.key for e in prof.key_averages()}
+    assert any("gather_f32_mfma_kernel" in n for n in names) and any("scatter_f32_mfma_kernel" in n for n in names), names
+    y2, z2 = F.flare_multihead_mixer(qd, kd, vd, scale=0.8, return_z=True)
+    assert torch.equal(y, y2) and torch.equal(z, z2)
+    for s in (1, 3):
+        ys, zs = check(dev, q, k, v, scale=0.8, n_splits=s)
+    zg, lse = F.flare_gather(qd, kd, vd, scale=0.8)
+    sc = 0.8 * torch.einsum("hmd,bhnd->bhmn", q.double(), k.double())
+    assert float((lse.double().cpu() - torch.logsumexp(sc, -1)).abs().max()) <= 1e-4
+    assert O.rel_l2(F.flare_scatter(qd, kd, zg, scale=0.8), y) <= 1e-5
+
+
+def test_fp32_matrix_core_mixer_views_and_fallbacks(dev):
+    """Token-major 'b n (h d) -> b h n d' views go through without a copy; a key mask and a latent count that is not a
+    multiple of 16 keep the FMA kernels, and so does force_generic."""
+    from torch.profiler import ProfilerActivity, profile
+    B, H, N, M, D = 2, 4, 3000, 64, 32
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(2, B, N, H * D, generator=g)
+    q = torch.randn(H, M, D, generator=g) * D ** -0.5
+    k, v = (t.view(B, N, H, D).permute(0, 2, 1, 3) for t in x)
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        y = F.flare_multihead_mixer(q.to(dev), *(t.to(dev).view(B, N, H, D).permute(0, 2, 1, 3) for t in x))
+        torch.cuda.synchronize()
+    names = {e.key for e in prof.key_averages()}
+    assert any("scatter_f32_mfma_kernel" in n for n in names) and not any("copy" in n.lower() for n in names), names
+    yr, _ = O.mixer_explicit(q, k, v, 1.0, None)
+    assert O.rel_l2(y, yr) <= 1e-5
+    mask = torch.ones(B, N, dtype=torch.bool)
+    mask[1, 2000:] = False
+    # a head dim of 24 is zero-padded to 32 and takes the matrix-core kernels; the other two do not
+    for kw, qq, kk, vv, mfma in (({"key_mask": mask}, q, k, v, False), ({}, q[:, :, :24], k[..., :24], v[..., :24], True),
+                                 ({}, q[:, :40], k, v, False), ({"force_generic": True}, q, k, v, False)):
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            check(dev, qq.contiguous(), kk.contiguous(), vv.contiguous(), **kw)
+        assert any("f32_mfma" in e.key for e in prof.key_averages()) == mfma, kw
+
+
+def test_fp32_narrow_heads_are_padded_to_the_matrix_core_kernels(dev):
+    """D = 8 (the reference's default model: 64 channels, 8 heads) in fp32: q, k, v zero-padded to 16 columns run on
+    the fp32 matrix-core kernels; values and gradients as the oracle's."""
+    from torch.profiler import ProfilerActivity, profile
+    q, k, v = make(2, 8, 3000, 64, 8, torch.float32, seed=4)
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        check(dev, q, k, v, scale=1.3)
+    assert any("gather_f32_mfma_kernel" in e.key for e in prof.key_averages())
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    F.flare_multihead_mixer(qd, kd, vd, scale=1.3).square().sum().backward()
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    O.mixer_explicit(qr, kr, vr, 1.3, None)[0].square().sum().backward()
+    for a, b in ((qd, qr), (kd, kr), (vd, vr)):
+        assert a.grad.shape == b.grad.shape and O.rel_l2(a.grad, b.grad) <= 1e-4
