@@ -1,6 +1,6 @@
 // FLARE mixer for fp32 inputs on the fp32 matrix instruction v_mfma_f32_16x16x4_f32 (README.md:39-52 of the
 // reference: z = softmax_n(s q k^T) v, y = softmax_m(s k q^T) z).  Taken by the fp32 launchers of mixer_generic.hip for
-// problems without a key mask or dropout, D in {16, 32, 64}, M a multiple of 16 and 16-byte aligned rows; same
+// problems without dropout, D in {16, 32, 64}, M a multiple of 16 and 16-byte aligned rows; same
 // workspace layout, partial format and merge kernel as the FMA kernels there.
 //
 // Operands: A is one float per lane (row c16, k = lane group g), B one float per lane (column c16, k = g), the
@@ -48,6 +48,7 @@ __global__ __launch_bounds__(256) void gather_f32_mfma_kernel(MixerArgs a)
     const float* q = (const float*)a.q + b * a.qs[0] + h * a.qs[1];
     const float* k = (const float*)a.k + b * a.ks[0] + h * a.ks[1];
     const float* v = (const float*)a.v + b * a.vs[0] + h * a.vs[1];
+    const uint8_t* mask = a.mask ? a.mask + (int64_t)b * a.N : nullptr;
 
     // latent operands (B of the score product), log2-scaled; latent tiles past M hold zeros and are not stored
     f32x4 qb[CT][QL / 4];
@@ -78,14 +79,22 @@ __global__ __launch_bounds__(256) void gather_f32_mfma_kernel(MixerArgs a)
     // K rows as A operands straight from global memory, V rows through the wave's LDS tile; the next tile is requested
     // while this one is worked on (rows past the range repeat its last row: no branch around a load)
     f32x4 ka[QL / 4], vr[VPT];
+    uint8_t keep_n[4] = {1, 1, 1, 1};      // key mask of the lane's four tokens (rows 4g + r of the tile)
+    bool vkeep[VPT];                       // the V chunk's token takes part (else it is staged as zeros: 0 * NaN is NaN)
     auto fetch = [&](int n0) {
+        if (mask != nullptr) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) keep_n[r] = mask[max(min(n0 + 4 * g + r, n_end - 1), 0)];
+        }
         const int n = max(min(n0 + c16, n_end - 1), 0);
 #pragma unroll
         for (int j4 = 0; j4 < QL / 4; ++j4) ka[j4] = *reinterpret_cast<const f32x4*>(k + (int64_t)n * a.ks[2] + g * QL + 4 * j4);
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             const int c = lane + 64 * i, tok = c / (D / 4), ch = c % (D / 4);
-            vr[i] = *reinterpret_cast<const f32x4*>(v + (int64_t)max(min(n0 + tok, n_end - 1), 0) * a.vs[2] + 4 * ch);
+            const int nv = max(min(n0 + tok, n_end - 1), 0);
+            vr[i] = *reinterpret_cast<const f32x4*>(v + (int64_t)nv * a.vs[2] + 4 * ch);
+            vkeep[i] = n0 + tok < n_end && (mask == nullptr || mask[nv] != 0);
         }
     };
     int n0 = n_begin + 16 * w;
@@ -97,12 +106,12 @@ __global__ __launch_bounds__(256) void gather_f32_mfma_kernel(MixerArgs a)
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             const int c = lane + 64 * i, tok = c / (D / 4), ch = c % (D / 4);
-            *reinterpret_cast<f32x4*>(&vt[w][tok][4 * ch]) = vr[i];
+            *reinterpret_cast<f32x4*>(&vt[w][tok][4 * ch]) = vkeep[i] ? vr[i] : f32x4{0.f, 0.f, 0.f, 0.f};
         }
-        fetch(n0 + 64);
-        bool valid[4];
+        bool valid[4];      // a token past the range or padded by the key mask takes no part
 #pragma unroll
-        for (int r = 0; r < 4; ++r) valid[r] = n0 + 4 * g + r < n_end;
+        for (int r = 0; r < 4; ++r) valid[r] = n0 + 4 * g + r < n_end && keep_n[r] != 0;
+        fetch(n0 + 64);
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             // scores: lane = latent column c16, rows = tokens 4g + r
@@ -224,9 +233,12 @@ __global__ __launch_bounds__(256) void scatter_f32_mfma_kernel(MixerArgs a)
         // the next tile's rows are waited for before the stores are issued (one in-order counter for loads and stores)
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
         if (n < a.N) {
+            // a padded token's row is 0 whatever its key row held
+            const bool on = a.mask == nullptr || a.mask[(int64_t)b * a.N + n] != 0;
             const float inv = 1.f / l;
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) *reinterpret_cast<f32x4*>(y + (int64_t)n * a.ys[2] + 16 * rt + 4 * g) = yacc[rt] * inv;
+            for (int rt = 0; rt < RT; ++rt)
+                *reinterpret_cast<f32x4*>(y + (int64_t)n * a.ys[2] + 16 * rt + 4 * g) = on ? yacc[rt] * inv : f32x4{0.f, 0.f, 0.f, 0.f};
             if (a.lse_tok && g == 0) a.lse_tok[((int64_t)b * a.H + h) * a.N + n] = (mx + __log2f(l)) * kLn2;
         }
     }
@@ -243,7 +255,7 @@ constexpr size_t kF32ScatterLdsMax = 150 * 1024;
 
 bool f32_mfma_mixer_ok(const MixerArgs& a, bool scatter)
 {
-    if (a.mask != nullptr || a.drop_thr != 0 || a.force_fma) return false;
+    if (a.drop_thr != 0 || a.force_fma) return false;
     if (a.D != 16 && a.D != 32 && a.D != 64) return false;
     if (a.M < 16 || a.M % 16 != 0) return false;
     if (!rows16(a.q, a.qs) || !rows16(a.k, a.ks)) return false;

@@ -481,13 +481,13 @@ def _narrow_head_pad(q, k, force_generic, masked=False) -> int:
     """Columns of zeros to append to a head dim so that the matrix-core kernels (D in {16, 32, 64}) take the problem,
     or 0.  Zero columns change neither the scores q.k nor the first D output columns; the reference's default model
     has D = channel_dim / num_heads = 8, which the fp32-FMA kernels would serve 5-15x slower.  fp32 problems have
-    matrix-core kernels too (latent counts that are multiples of 16, no key mask or dropout: `masked`)."""
+    matrix-core kernels too (latent counts that are multiples of 16, no dropout: `masked`)."""
     D = k.shape[-1]
     if force_generic or D > 64 or k.device.type != "cuda":
         return 0
     target = 16 if D <= 16 else 32 if D <= 32 else 64
     if k.dtype == torch.float32:
-        return target - D if q.shape[-2] % 16 == 0 and not masked else 0
+        return target - D if q.shape[-2] % 16 == 0 and not masked else 0      # masked: dropout (FMA kernels only)
     if k.dtype not in (torch.bfloat16, torch.float16):
         return 0
     return target - D if q.shape[-2] % 32 == 0 else 0
@@ -539,7 +539,7 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
             and k.dtype in (torch.bfloat16, torch.float16) and k.device.type == "cuda"
             and _dead_latent_bias(float(scale), k.dtype) is not None):
         return _mixer_odd_latents(q, k, v, float(scale), key_mask, return_z, n_splits, token_major_out)
-    pad = _narrow_head_pad(q, k, force_generic, key_mask is not None or dropout_p > 0) if q.dtype == k.dtype == v.dtype else 0
+    pad = _narrow_head_pad(q, k, force_generic, dropout_p > 0) if q.dtype == k.dtype == v.dtype else 0
     if pad:
         q, k, v = _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad)
     needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))
@@ -734,7 +734,7 @@ def flare_gather(q, k, v, scale: float = 1.0, key_mask=None, n_splits: int = 0,
     Differentiable in q, k, v (the backward recomputes the scores with torch ops: for models that put
     layers between the two halves; the whole mixer has its own HIP backward)."""
     D = k.shape[-1]
-    pad = _narrow_head_pad(q, k, force_generic, key_mask is not None) if q.dtype == k.dtype == v.dtype else 0
+    pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype == v.dtype else 0
     if pad:
         q, k, v = _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad)
     if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
@@ -748,7 +748,7 @@ def flare_scatter(q, k, z, scale: float = 1.0, key_mask=None, force_generic: boo
     """y [B,H,N,D] = softmax_m(scale k q^T) z with z [B,H,M,D] (computed from its fp32 copy).
     Differentiable in q, k, z like flare_gather."""
     D = k.shape[-1]
-    pad = _narrow_head_pad(q, k, force_generic, key_mask is not None) if q.dtype == k.dtype else 0
+    pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype else 0
     if pad:
         q, k, z = _pad_last(q, pad), _pad_last(k, pad), _pad_last(z, pad)
     if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, z)):

@@ -105,7 +105,7 @@ def test_strided_views_no_copy(dev):
     assert O.rel_l2(y, yr) <= 2e-2
 
 
-@pytest.mark.parametrize("dtype,fg", [(torch.float32, True), (torch.bfloat16, False), (torch.bfloat16, True)])
+@pytest.mark.parametrize("dtype,fg", [(torch.float32, True), (torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
 def test_key_mask(dev, dtype, fg):
     q, k, v = make(3, 2, 333, 64, 32, dtype, seed=5)
     mask = torch.ones(3, 333, dtype=torch.bool)
@@ -600,8 +600,8 @@ def test_fp32_matrix_core_mixer_shapes(dev, shape):
 
 
 def test_fp32_matrix_core_mixer_views_and_fallbacks(dev):
-    """Token-major 'b n (h d) -> b h n d' views go through without a copy; a key mask and a latent count that is not a
-    multiple of 16 keep the FMA kernels, and so does force_generic."""
+    """Token-major 'b n (h d) -> b h n d' views go through without a copy, a key mask too; a latent count that is not a
+    multiple of 16 keeps the FMA kernels, and so does force_generic."""
     from torch.profiler import ProfilerActivity, profile
     B, H, N, M, D = 2, 4, 3000, 64, 32
     g = torch.Generator().manual_seed(11)
@@ -617,8 +617,8 @@ def test_fp32_matrix_core_mixer_views_and_fallbacks(dev):
     assert O.rel_l2(y, yr) <= 1e-5
     mask = torch.ones(B, N, dtype=torch.bool)
     mask[1, 2000:] = False
-    # a head dim of 24 is zero-padded to 32 and takes the matrix-core kernels; the other two do not
-    for kw, qq, kk, vv, mfma in (({"key_mask": mask}, q, k, v, False), ({}, q[:, :, :24], k[..., :24], v[..., :24], True),
+    # a key mask and a head dim of 24 (zero-padded to 32) take the matrix-core kernels; the other two do not
+    for kw, qq, kk, vv, mfma in (({"key_mask": mask}, q, k, v, True), ({}, q[:, :, :24], k[..., :24], v[..., :24], True),
                                  ({}, q[:, :40], k, v, False), ({"force_generic": True}, q, k, v, False)):
         with profile(activities=[ProfilerActivity.CUDA]) as prof:
             check(dev, qq.contiguous(), kk.contiguous(), vv.contiguous(), **kw)
@@ -639,3 +639,25 @@ def test_fp32_narrow_heads_are_padded_to_the_matrix_core_kernels(dev):
     O.mixer_explicit(qr, kr, vr, 1.3, None)[0].square().sum().backward()
     for a, b in ((qd, qr), (kd, kr), (vd, vr)):
         assert a.grad.shape == b.grad.shape and O.rel_l2(a.grad, b.grad) <= 1e-4
+
+
+@pytest.mark.parametrize("garbage", [0.0, 1.0e30, float("nan")])
+def test_fp32_key_mask_over_many_splits_and_padding_garbage(dev, garbage):
+    """The fp32 matrix-core kernels with a key mask: split ranges without a real token, a fully padded batch element,
+    holes, and padded rows that hold huge values or NaN never reach a result."""
+    q, k, v = make(4, 2, 8192, 128, 32, torch.float32, seed=12)
+    mask = torch.ones(4, 8192, dtype=torch.bool)
+    mask[1, 100:] = False
+    mask[2, 5000:] = False
+    mask[2, 17:4000:5] = False
+    mask[3] = False
+    kk, vv = k.clone(), v.clone()
+    if garbage != 0.0:
+        kk[~mask[:, None, :, None].expand_as(k)] = garbage
+        vv[~mask[:, None, :, None].expand_as(v)] = garbage
+    y, z = F.flare_multihead_mixer(q.to(dev), kk.to(dev), vv.to(dev), key_mask=mask.to(dev), return_z=True)
+    yr, zr = O.mixer_explicit(q, k, v, 1.0, mask)
+    keep = mask[:, None, :, None].expand_as(yr)
+    assert torch.isfinite(z).all() and O.rel_l2(z, zr) <= 1e-5
+    assert O.rel_l2(y.cpu()[keep], yr[keep]) <= 1e-5
+    assert (y.cpu()[~keep] == 0).all() and (z[3] == 0).all()
