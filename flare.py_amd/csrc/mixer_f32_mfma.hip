@@ -259,7 +259,8 @@ bool f32_mfma_mixer_ok(const MixerArgs& a, bool scatter)
     if (a.D != 16 && a.D != 32 && a.D != 64) return false;
     if (a.M < 16 || a.M % 16 != 0) return false;
     if (!rows16(a.q, a.qs) || !rows16(a.k, a.ks)) return false;
-    if (scatter) return rows16(a.y, a.ys) && (size_t)a.M * (a.D + 4) * 8 <= kF32ScatterLdsMax;
+    if (scatter)
+        return rows16(a.y, a.ys) && (reinterpret_cast<uintptr_t>(a.z) & 15) == 0 && (size_t)a.M * (a.D + 4) * 8 <= kF32ScatterLdsMax;
     return rows16(a.v, a.vs);
 }
 

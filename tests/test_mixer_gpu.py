@@ -661,3 +661,15 @@ def test_fp32_key_mask_over_many_splits_and_padding_garbage(dev, garbage):
     assert torch.isfinite(z).all() and O.rel_l2(z, zr) <= 1e-5
     assert O.rel_l2(y.cpu()[keep], yr[keep]) <= 1e-5
     assert (y.cpu()[~keep] == 0).all() and (z[3] == 0).all()
+
+
+def test_fp32_scatter_takes_a_misaligned_z(dev):
+    """z handed to flare_scatter four bytes off a 16-byte boundary: the FMA kernel takes it (same values)."""
+    q, k, v = make(1, 2, 500, 32, 16, torch.float32, seed=6)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    z, _ = F.flare_gather(qd, kd, vd)
+    buf = torch.zeros(z.numel() + 1, device=dev)
+    zo = buf[1:].view_as(z)
+    zo.copy_(z)
+    assert zo.data_ptr() % 16 != 0
+    assert O.rel_l2(F.flare_scatter(qd, kd, zo), F.flare_scatter(qd, kd, z)) <= 1e-6
