@@ -320,6 +320,11 @@ hipError_t launch_causal_linear_mfma(const CausalLinearArgs& a, int dtype, hipSt
 hipError_t launch_triple_state(const TripleArgs& a, int dtype, hipStream_t st);
 hipError_t launch_triple_merge(const TripleArgs& a, hipStream_t st);
 hipError_t launch_triple_out(const TripleArgs& a, int dtype, hipStream_t st);
+// fp32 inputs with head dims 16 on v_mfma_f32_16x16x4_f32 (triple_f32_mfma.hip): taken by the launchers above
+bool       triple_f32_mfma_state_ok(const TripleArgs& a);
+bool       triple_f32_mfma_out_ok(const TripleArgs& a);
+hipError_t launch_triple_state_f32_mfma(const TripleArgs& a, hipStream_t st);
+hipError_t launch_triple_out_f32_mfma(const TripleArgs& a, hipStream_t st);
 bool       triple_mfma_supported(int dtype, int Dq, int Dv);
 hipError_t launch_triple_state_mfma(const TripleArgs& a, int dtype, hipStream_t st);
 hipError_t launch_triple_out_mfma(const TripleArgs& a, int dtype, hipStream_t st);

@@ -237,6 +237,7 @@ hipError_t out_launch(const TripleArgs& a, hipStream_t st)
 
 hipError_t launch_triple_state(const TripleArgs& a, int dtype, hipStream_t st)
 {
+    if (dtype == 0 && triple_f32_mfma_state_ok(a)) return launch_triple_state_f32_mfma(a, st);     // fp32, head dims 16
     switch (dtype) {
         case 0: return state_launch<float>(a, st);
         case 1: return state_launch<bf16_t>(a, st);
@@ -254,6 +255,7 @@ hipError_t launch_triple_merge(const TripleArgs& a, hipStream_t st)
 
 hipError_t launch_triple_out(const TripleArgs& a, int dtype, hipStream_t st)
 {
+    if (dtype == 0 && triple_f32_mfma_out_ok(a)) return launch_triple_out_f32_mfma(a, st);
     switch (dtype) {
         case 0: return out_launch<float>(a, st);
         case 1: return out_launch<bf16_t>(a, st);

@@ -1,0 +1,212 @@
+// Triple (third-order) linear attention for fp32 inputs with head dims 16 on v_mfma_f32_16x16x4_f32
+// (lra/models/backends.py:1285-1292, lra/models/triton/triple.py:29-121 of the reference):
+//   state[i,j,k] = (1/N) sum_n f(k1)[n,i] v[n,j] f(k2)[n,k],   out[n,j] = sum_{i,k} f(q1)[n,i] state[i,j,k] f(q2)[n,k].
+// Taken by the fp32 launchers of triple.hip when Dq = Dv = 16 and the rows are 16-byte aligned; same split-N partials
+// ([i][j][k] and the normaliser's [i][k]), merge kernel and workspace layout as the FMA kernels there.
+//
+// The instruction takes one float per lane for A (row c16, k-slot = lane group g) and for B (column c16, k-slot g).
+// State: for every i a 16 x 16 tile over (k, j), contracted over four tokens at a time: A = f(k1)[n,i] f(k2)[n,k]
+// (one multiply per lane and instruction), B = v[n,j].  Output: out^T[j, n] contracted over the 256 pairs (i,k), four k
+// at a time: A = state[i][j][k] from LDS, B = f(q1)[n,i] f(q2)[n,k] (one multiply again).  The normaliser rides along
+// as plain sums of the same products.
+#include <algorithm>
+
+#include "common.hpp"
+
+namespace flare {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 mma4(float a, float b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+__device__ __forceinline__ float feat(float x, int fm)
+{
+    if (!fm) return x;
+    return x > 0.f ? x + 1.f : __expf(x);
+}
+__device__ __forceinline__ float groups_sum(float x)
+{
+    x += __shfl_xor(x, 16);
+    return x + __shfl_xor(x, 32);
+}
+
+constexpr int kD = 16;
+
+// grid = (n_splits, H, B).  Wave w takes the 16-token groups w, w + 4, ... of the split; the four waves' sums meet in
+// LDS in wave order (bit-stable) and wave 0 writes the split's partial.
+__global__ __launch_bounds__(256) void triple_state_f32_mfma_kernel(TripleArgs a)
+{
+    __shared__ __attribute__((aligned(16))) f32x4 red[3][kD][64];
+    __shared__ float redk[3][kD][64];
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int split = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const float* k1 = (const float*)a.k1 + b * a.k1s[0] + h * a.k1s[1];
+    const float* k2 = (const float*)a.k2 + b * a.k2s[0] + h * a.k2s[1];
+    const float* v = (const float*)a.v + b * a.vs[0] + h * a.vs[1];
+
+    f32x4 acc[kD];
+    float kkacc[kD];
+#pragma unroll
+    for (int i = 0; i < kD; ++i) {
+        acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        kkacc[i] = 0.f;
+    }
+    const int n_begin = split * a.tokens_per_split;
+    const int n_end = min(a.N, n_begin + a.tokens_per_split);
+    const int groups = n_begin < n_end ? (n_end - n_begin + 15) / 16 : 0;
+    const int mine = groups > w ? (groups - w + 3) / 4 : 0;
+
+    // the lane's four tokens of a group are 4c + g, c = 0..3: their 16 features of k1, feature c16 of k2 and of v.
+    // The next group is requested while this one is worked on (rows past the split repeat its last row, no branch).
+    f32x4 k1n[4][4];
+    float k2n[4], vn[4];
+    auto fetch = [&](int n0) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int n = max(min(n0 + 4 * c + g, n_end - 1), 0);
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) k1n[c][q4] = *reinterpret_cast<const f32x4*>(k1 + (int64_t)n * a.k1s[2] + 4 * q4);
+            k2n[c] = k2[(int64_t)n * a.k2s[2] + c16];
+            vn[c] = v[(int64_t)n * a.vs[2] + c16];
+        }
+    };
+    int n0 = n_begin + 16 * w;
+    if (mine > 0) fetch(n0);
+    for (int t = 0; t < mine; ++t, n0 += 64) {
+        f32x4 k1c[4][4];
+        float k2c[4], vc[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const bool valid = n0 + 4 * c + g < n_end;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) k1c[c][q4] = k1n[c][q4];
+            k2c[c] = valid ? feat(k2n[c], a.feature_map) : 0.f;       // a token past the split adds nothing
+            vc[c] = valid ? vn[c] : 0.f;
+        }
+        fetch(n0 + 64);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int i = 0; i < kD; ++i) {
+                const float p = feat(k1c[c][i >> 2][i & 3], a.feature_map) * k2c[c];
+                acc[i] = mma4(p, vc[c], acc[i]);        // rows k = 4g + r, column j = c16
+                kkacc[i] += p;                          // kk[i][k = c16], this lane group's tokens
+            }
+    }
+
+    if (w > 0) {
+#pragma unroll
+        for (int i = 0; i < kD; ++i) {
+            red[w - 1][i][lane] = acc[i];
+            redk[w - 1][i][lane] = kkacc[i];
+        }
+    }
+    __syncthreads();
+    if (w > 0) return;
+    constexpr size_t per = (size_t)kD * kD * kD + (size_t)kD * kD;
+    float* part = a.part + (((size_t)b * a.H + h) * a.n_parts + split) * per;
+#pragma unroll
+    for (int i = 0; i < kD; ++i) {
+        f32x4 s = acc[i];
+        float kk = kkacc[i];
+#pragma unroll
+        for (int ww = 0; ww < 3; ++ww) {
+            s += red[ww][i][lane];
+            kk += redk[ww][i][lane];
+        }
+        kk = groups_sum(kk);
+        *reinterpret_cast<f32x4*>(part + ((size_t)i * kD + c16) * kD + 4 * g) = s;      // [i][j = c16][k = 4g + r]
+        if (g == 0) part[(size_t)kD * kD * kD + (size_t)i * kD + c16] = kk;
+    }
+}
+
+// grid = (workgroups, H, B); a wave takes 16 tokens at a time.
+__global__ __launch_bounds__(256) void triple_out_f32_mfma_kernel(TripleArgs a)
+{
+    __shared__ float ss[kD * kD * 17];      // state[i][j][k] at (i 16 + j) 17 + k: the 16 rows j of a read fall into 16 banks
+    __shared__ float kks[kD * kD];
+
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const size_t bh = (size_t)b * a.H + h;
+    const float* q1 = (const float*)a.q1 + b * a.q1s[0] + h * a.q1s[1];
+    const float* q2 = (const float*)a.q2 + b * a.q2s[0] + h * a.q2s[1];
+    float* out = (float*)a.out + b * a.os[0] + h * a.os[1];
+    const float* state = a.state + bh * kD * kD * kD;
+
+    for (int idx = tid; idx < kD * kD * kD; idx += 256) ss[(idx >> 4) * 17 + (idx & 15)] = state[idx];
+    if (a.normalize) kks[tid] = a.kk[bh * kD * kD + tid];
+    __syncthreads();
+
+    const int tiles = (a.N + 15) / 16, stride = gridDim.x * 4;
+    int tile = blockIdx.x * 4 + w;
+    const int mine = tile < tiles ? (tiles - tile + stride - 1) / stride : 0;
+    f32x4 q1n[4];
+    float q2n[4];
+    auto fetch = [&](int tl) {
+        const int n = min(tl * 16 + c16, a.N - 1);
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) q1n[q4] = *reinterpret_cast<const f32x4*>(q1 + (int64_t)n * a.q1s[2] + 4 * q4);
+#pragma unroll
+        for (int kq = 0; kq < 4; ++kq) q2n[kq] = q2[(int64_t)n * a.q2s[2] + 4 * kq + g];
+    };
+    if (mine > 0) fetch(tile);
+    for (int t = 0; t < mine; ++t, tile += stride) {
+        float q1c[kD], q2c[4];
+#pragma unroll
+        for (int i = 0; i < kD; ++i) q1c[i] = feat(q1n[i >> 2][i & 3], a.feature_map);
+#pragma unroll
+        for (int kq = 0; kq < 4; ++kq) q2c[kq] = feat(q2n[kq], a.feature_map);
+        fetch(tile + stride);
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        float den = 0.f;
+#pragma unroll
+        for (int i = 0; i < kD; ++i)
+#pragma unroll
+            for (int kq = 0; kq < 4; ++kq) {
+                const float p = q1c[i] * q2c[kq];                                   // token c16, pair (i, k = 4 kq + g)
+                acc = mma4(ss[(i * kD + c16) * 17 + 4 * kq + g], p, acc);           // rows j = 4g + r, column n = c16
+                if (a.normalize) den = fmaf(p, kks[i * kD + 4 * kq + g], den);
+            }
+        den = a.normalize ? groups_sum(den) : 1.f;
+        const int n = tile * 16 + c16;
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the next tile's rows, before the stores
+        if (n < a.N) *reinterpret_cast<f32x4*>(out + (int64_t)n * a.os[2] + 4 * g) = acc * (1.f / den);
+    }
+}
+
+bool rows16(const void* p, const int64_t* s)
+{
+    return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && s[0] % 4 == 0 && s[1] % 4 == 0 && s[2] % 4 == 0;
+}
+
+}  // namespace
+
+bool triple_f32_mfma_state_ok(const TripleArgs& a)
+{
+    return a.Dq == kD && a.Dv == kD && !a.diag_parts && rows16(a.k1, a.k1s) && rows16(a.k2, a.k2s) && rows16(a.v, a.vs) &&
+           (reinterpret_cast<uintptr_t>(a.part) & 15) == 0;
+}
+
+bool triple_f32_mfma_out_ok(const TripleArgs& a)
+{
+    return a.Dq == kD && a.Dv == kD && rows16(a.q1, a.q1s) && rows16(a.q2, a.q2s) && rows16(a.out, a.os);
+}
+
+hipError_t launch_triple_state_f32_mfma(const TripleArgs& a, hipStream_t st)
+{
+    hipLaunchKernelGGL(triple_state_f32_mfma_kernel, dim3(a.n_splits, a.H, a.B), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_triple_out_f32_mfma(const TripleArgs& a, hipStream_t st)
+{
+    const int64_t groups = ((int64_t)a.N + 63) / 64;
+    const int64_t want = std::max<int64_t>(1, ((int64_t)8 * device_cus() + (int64_t)a.B * a.H - 1) / ((int64_t)a.B * a.H));
+    hipLaunchKernelGGL(triple_out_f32_mfma_kernel, dim3((unsigned)std::min<int64_t>(groups, want), a.H, a.B), dim3(256), 0, st, a);
+    return hipGetLastError();
+}
+
+}  // namespace flare
