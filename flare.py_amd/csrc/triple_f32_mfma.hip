@@ -6,7 +6,7 @@
 //
 // The instruction takes one float per lane for A (row c16, k-slot = lane group g) and for B (column c16, k-slot g).
 // State: for every i a 16 x 16 tile over (k, j), contracted over four tokens at a time: A = f(k1)[n,i] f(k2)[n,k]
-// (one multiply per lane and instruction), B = v[n,j].  Output: out^T[j, n] contracted over the 256 pairs (i,k), four k
+// (f(k1)[n,i] by a shuffle from the lane that holds it, one multiply per lane and instruction), B = v[n,j].  Output: out^T[j, n] contracted over the 256 pairs (i,k), four k
 // at a time: A = state[i][j][k] from LDS, B = f(q1)[n,i] f(q2)[n,k] (one multiply again).  The normaliser rides along
 // as plain sums of the same products.
 #include <algorithm>
@@ -35,7 +35,7 @@ constexpr int kD = 16;
 
 // grid = (n_splits, H, B).  Wave w takes the 16-token groups w, w + 4, ... of the split; the four waves' sums meet in
 // LDS in wave order (bit-stable) and wave 0 writes the split's partial.
-__global__ __launch_bounds__(256) void triple_state_f32_mfma_kernel(TripleArgs a)
+__global__ __launch_bounds__(256, 2) void triple_state_f32_mfma_kernel(TripleArgs a)
 {
     __shared__ __attribute__((aligned(16))) f32x4 red[3][kD][64];
     __shared__ float redk[3][kD][64];
@@ -58,16 +58,15 @@ __global__ __launch_bounds__(256) void triple_state_f32_mfma_kernel(TripleArgs a
     const int groups = n_begin < n_end ? (n_end - n_begin + 15) / 16 : 0;
     const int mine = groups > w ? (groups - w + 3) / 4 : 0;
 
-    // the lane's four tokens of a group are 4c + g, c = 0..3: their 16 features of k1, feature c16 of k2 and of v.
+    // the lane's four tokens of a group are 4c + g, c = 0..3: feature c16 of their k1, k2 and v rows.  f(k1)[n, i] for
+    // the other i comes from the lane (g, i) by a shuffle: one feature map per lane and token instead of sixteen.
     // The next group is requested while this one is worked on (rows past the split repeat its last row, no branch).
-    f32x4 k1n[4][4];
-    float k2n[4], vn[4];
+    float k1n[4], k2n[4], vn[4];
     auto fetch = [&](int n0) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const int n = max(min(n0 + 4 * c + g, n_end - 1), 0);
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) k1n[c][q4] = *reinterpret_cast<const f32x4*>(k1 + (int64_t)n * a.k1s[2] + 4 * q4);
+            k1n[c] = k1[(int64_t)n * a.k1s[2] + c16];
             k2n[c] = k2[(int64_t)n * a.k2s[2] + c16];
             vn[c] = v[(int64_t)n * a.vs[2] + c16];
         }
@@ -75,13 +74,11 @@ __global__ __launch_bounds__(256) void triple_state_f32_mfma_kernel(TripleArgs a
     int n0 = n_begin + 16 * w;
     if (mine > 0) fetch(n0);
     for (int t = 0; t < mine; ++t, n0 += 64) {
-        f32x4 k1c[4][4];
-        float k2c[4], vc[4];
+        float k1c[4], k2c[4], vc[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const bool valid = n0 + 4 * c + g < n_end;
-#pragma unroll
-            for (int q4 = 0; q4 < 4; ++q4) k1c[c][q4] = k1n[c][q4];
+            k1c[c] = feat(k1n[c], a.feature_map);
             k2c[c] = valid ? feat(k2n[c], a.feature_map) : 0.f;       // a token past the split adds nothing
             vc[c] = valid ? vn[c] : 0.f;
         }
@@ -90,7 +87,7 @@ __global__ __launch_bounds__(256) void triple_state_f32_mfma_kernel(TripleArgs a
         for (int c = 0; c < 4; ++c)
 #pragma unroll
             for (int i = 0; i < kD; ++i) {
-                const float p = feat(k1c[c][i >> 2][i & 3], a.feature_map) * k2c[c];
+                const float p = __shfl(k1c[c], (lane & 48) | i) * k2c[c];
                 acc[i] = mma4(p, vc[c], acc[i]);        // rows k = 4g + r, column j = c16
                 kkacc[i] += p;                          // kk[i][k = c16], this lane group's tokens
             }
@@ -186,8 +183,7 @@ bool rows16(const void* p, const int64_t* s)
 
 bool triple_f32_mfma_state_ok(const TripleArgs& a)
 {
-    return a.Dq == kD && a.Dv == kD && !a.diag_parts && rows16(a.k1, a.k1s) && rows16(a.k2, a.k2s) && rows16(a.v, a.vs) &&
-           (reinterpret_cast<uintptr_t>(a.part) & 15) == 0;
+    return a.Dq == kD && a.Dv == kD && !a.diag_parts && (reinterpret_cast<uintptr_t>(a.part) & 15) == 0;
 }
 
 bool triple_f32_mfma_out_ok(const TripleArgs& a)
