@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FLARE mixer forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block|train]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block|train|linear|fp32]
 
 One step = one forward of the mixer (split-N gather, merge, scatter) over the headline workload
 B=1, H=8, N=1,048,576, M=256, D=32, bf16 in / fp32 accumulate, inputs resident in HBM.
@@ -17,7 +17,9 @@ of GPU work about 7 % slower than the steady state.
 causal FLARE prefill of 8192 tokens + 256 decode steps at B=8,H=16,M=128,D=64; triple = triple
 attention at B=4,H=8,N=16384,D=16 (elu+1, normalised); block = lift MLP 3 -> 128 and one FLAREBlock forward with a
 4x GELU MLP at B=4,N=65536,C=128,H=8,M=128 under bf16 autocast (fused HIP launches around the HIP mixer); train =
-the headline configuration with the backward pass (HIP kernels both ways).
+the headline configuration with the backward pass (HIP kernels both ways); linear = causal linear attention at
+B=4,H=8,N=65536,Dk=Dv=64 (bf16, and fp32 beside it); fp32 = the mixer forward in fp32 at B=1,H=8,N=262144,M=256,D=32
+with BASELINE config 1 beside it.
 """
 from __future__ import annotations
 
@@ -266,6 +268,80 @@ def bench_triple(args, F, dev):
     return out
 
 
+def bench_linear(args, F, dev):
+    """Causal linear attention (lra/models/triton/causal_linear.py:23-145) at B=4, H=8, N=65,536, Dk=Dv=64: bf16 on the
+    16x16x32 kernels; the same shape in fp32 (16x16x4 fp32 products) and the fp32-FMA kernel beside it."""
+    from oracle import flare_oracle as O
+
+    B, H, N, Dk, Dv = 4, 8, 65536, 64, 64
+    g = torch.Generator(device=dev).manual_seed(0)
+    q, k, v = (torch.randn(B, H, N, D, generator=g, device=dev) for D in (Dk, Dk, Dv))
+    qb, kb, vb = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    step = lambda: F.causal_linear_attention(qb, kb, vb)
+    ms_step = wall_ms(step, args.steps, args.warmup)
+    ms_ev = time_events(step, args.steps, 2)
+    nbytes = B * H * N * (2 * Dk + 2 * Dv) * 2
+    achieved = nbytes / (ms_ev * 1e-3) / 1e9
+    out = base_record(args, "causal linear attention tokens/sec at B=4,H=8,N=65536,Dk=Dv=64 bf16", B * N / (ms_step * 1e-3),
+                      "tokens/s", ms_step, "causal linear attention B=4,H=8,N=65536,Dk=64,Dv=64 (the reference's CausalLinear; no BASELINE config)")
+    out["roofline"] = {"bound": "hbm", "kernel": "causal_linear_mfma_kernel (state phase + output phase)",
+                       "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                       "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "algorithmic_bytes": nbytes,
+                       "ms_events": round(ms_ev, 4)}
+    ms32 = time_events(lambda: F.causal_linear_attention(q, k, v), 20, 3)
+    out["roofline"]["ms_fp32_inputs"] = round(ms32, 4)
+    out["roofline"]["fp32_GBps"] = round(2 * nbytes / (ms32 * 1e-3) / 1e9, 1)
+    if not args.no_torch_sdpa:
+        out["roofline"]["ms_fp32_fma_kernel"] = round(time_events(lambda: F.causal_linear_attention(q, k, v, force_generic=True), 3, 1), 3)
+    if not args.no_cpu:
+        ns = 4096                                   # bounded sample: the first 4096 tokens of every (b,h), fp64 closed form
+        c = [t[:, :, :ns].float().cpu() for t in (qb, kb, vb)]
+        t0 = time.perf_counter()
+        ref = O.causal_linear_closed_form(*c)
+        dt = time.perf_counter() - t0
+        y = F.causal_linear_attention(qb[:, :, :ns], kb[:, :, :ns], vb[:, :, :ns])
+        out["cpu_baseline"] = {"value": round(B * ns / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(),
+                               "cpu": cpu_model(), "kind": "port",
+                               "sample": f"closed form tril(QK^T)V/N (torch, fp64) on the first {ns} tokens of every (b,h), {dt:.2f} s"}
+        out["rel_l2_vs_cpu_on_sample"] = O.rel_l2(y, ref)
+    return out
+
+
+def bench_fp32(args, F, dev):
+    """The mixer forward in fp32 (16x16x4 fp32 matrix products) at B=1, H=8, N=262,144, M=256, D=32, BASELINE config 1
+    (B=1, H=8, N=4096, M=64, D=16, fp32) beside it."""
+    from oracle import flare_oracle as O
+
+    B, H, N, M, D = 1, 8, 262144, 256, 32
+    q, k, v = make_inputs(B, H, N, M, D, torch.float32, dev)
+    step = lambda: F.flare_multihead_mixer(q, k, v)
+    ms_step = wall_ms(step, args.steps, args.warmup)
+    ms_ev = time_events(step, args.steps, 2)
+    flops = 8.0 * B * H * N * M * D
+    tf = flops / (ms_ev * 1e-3) / 1e12
+    out = base_record(args, "FLARE mixer tokens/sec at N=262144,M=256,D=32 fp32", B * N / (ms_step * 1e-3), "tokens/s", ms_step,
+                      "FLARE mixer forward in fp32, B=1,H=8,N=262144,M=256,D=32 (the headline geometry at a quarter of its length)")
+    out["dtype"] = "f32"
+    out["roofline"] = {"bound": "mfma", "kernel": "gather_f32_mfma_kernel + scatter_f32_mfma_kernel",
+                       "achieved": round(tf, 1), "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4),
+                       "traffic": None, "algorithmic_flops": flops, "ms_events": round(ms_ev, 4)}
+    q1, k1, v1 = make_inputs(1, 8, 4096, 64, 16, torch.float32, dev)
+    out["roofline"]["ms_config1"] = round(time_events(lambda: F.flare_multihead_mixer(q1, k1, v1), 50, 5), 4)
+    if not args.no_torch_sdpa:
+        out["roofline"]["ms_fma_kernels"] = round(time_events(lambda: F.flare_multihead_mixer(q, k, v, force_generic=True), 3, 1), 3)
+    if not args.no_cpu:
+        c = [t.cpu() for t in (q1, k1, v1)]
+        t0 = time.perf_counter()
+        for _ in range(5):
+            ref, _ = O.mixer_sdpa(*c, 1.0)
+        dt = (time.perf_counter() - t0) / 5
+        out["cpu_baseline"] = {"value": round(4096 / dt, 1), "unit": "tokens/s", "cores": torch.get_num_threads(),
+                               "cpu": cpu_model(), "kind": "port",
+                               "sample": f"BASELINE config 1 whole (torch SDPA MATH backend, fp32), {dt * 1e3:.1f} ms per forward"}
+        out["rel_l2_vs_cpu_on_sample"] = O.rel_l2(F.flare_multihead_mixer(q1, k1, v1), ref)
+    return out
+
+
 def bench_train(args, F, dev):
     """Headline configuration, forward + backward of the mixer (HIP kernels both ways)."""
     B, H, N, M, D = 1, 8, 1 << 20, 256, 32
@@ -465,7 +541,7 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=1048576, help="tokens of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-torch-sdpa", action="store_true", help="skip the legs that time torch's own formulation (fused SDPA, einsum, torch layers) on the GPU")
-    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train"], default="mixer",
+    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train", "linear", "fp32"], default="mixer",
                     help="mixer = the headline configuration (default); the others are BASELINE configs 4, 5, 2")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -480,7 +556,8 @@ def main():
 
     dev = torch.device("cuda:0")
     if args.workload != "mixer":
-        fn = {"causal": bench_causal, "triple": bench_triple, "block": bench_block, "train": bench_train}[args.workload]
+        fn = {"causal": bench_causal, "triple": bench_triple, "block": bench_block, "train": bench_train,
+              "linear": bench_linear, "fp32": bench_fp32}[args.workload]
         print(json.dumps(fn(args, F, dev)))
         return
     B, H, N, M, D = 1, 8, 1 << 20, 256, 32
