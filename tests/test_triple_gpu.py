@@ -129,24 +129,25 @@ def test_state_is_tight_for_any_number_of_tiles_per_wave(dev, dtype, tol, D):
 
 @pytest.mark.parametrize("shape", [(1, 2, 500), (2, 3, 1), (1, 1, 17), (2, 2, 4097)])
 @pytest.mark.parametrize("fm,nz", [(None, False), ("elu", True), ("elu", False)])
-def test_fp32_head_dim_16_on_the_matrix_cores(dev, shape, fm, nz):
-    """fp32 inputs with Dq = Dv = 16 run on the fp32 matrix instruction (profiler), at the fp32 bar, the same bits twice;
-    rows that are not 16-byte aligned keep the FMA kernels."""
+@pytest.mark.parametrize("D", [16, 32])
+def test_fp32_head_dims_16_and_32_on_the_matrix_cores(dev, shape, fm, nz, D):
+    """fp32 inputs with Dq = Dv = 16 or 32 run on the fp32 matrix instruction (profiler), at the fp32 bar, the same bits
+    twice; rows that are not 16-byte aligned keep the FMA kernels."""
     from torch.profiler import ProfilerActivity, profile
     B, H, N = shape
     g = torch.Generator().manual_seed(N)
-    a = [torch.randn(B, H, N, 16, generator=g) * 0.25 for _ in range(5)]
+    a = [torch.randn(B, H, N, D, generator=g) * 0.25 for _ in range(5)]
     ad = [t.to(dev) for t in a]
     with profile(activities=[ProfilerActivity.CUDA]) as prof:
         st, out = F.triple_attention(*ad, normalize=nz, feature_map=fm)
         torch.cuda.synchronize()
     names = {e.key for e in prof.key_averages()}
-    assert any("triple_state_f32_mfma_kernel" in n for n in names) and any("triple_out_f32_mfma_kernel" in n for n in names)
+    assert any("triple_state_f32_mfma" in n for n in names) and any("triple_out_f32_mfma" in n for n in names)
     sr, orf = O.triple_einsum(*a, feature_map=fm == "elu", normalize=nz)
     assert O.rel_l2(st, sr) <= 1e-5 and O.rel_l2(out, orf) <= 1e-5
     st2, out2 = F.triple_attention(*ad, normalize=nz, feature_map=fm)
     assert torch.equal(st, st2) and torch.equal(out, out2)
-    pad = [torch.zeros(B, H, N, 17, device=dev) for _ in range(5)]
+    pad = [torch.zeros(B, H, N, D + 1, device=dev) for _ in range(5)]
     for p, t in zip(pad, ad):
         p[..., 1:] = t
     with profile(activities=[ProfilerActivity.CUDA]) as prof:
