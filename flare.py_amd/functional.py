@@ -1009,21 +1009,6 @@ def _causal_linear_forward(q, k, v, n_segs: int = 0, force_generic: bool = False
     return y
 
 
-def _causal_linear_torch(q, k, v):
-    # differentiable restatement used for the backward pass only: tril(Q K^T) V / N per 128-token
-    # chunk plus the running state, in fp32
-    B, H, N, Dk = q.shape
-    qf, kf, vf = q.float(), k.float(), v.float()
-    S = qf.new_zeros(B, H, Dk, v.shape[-1])
-    out = []
-    for n0 in range(0, N, 128):
-        qc, kc, vc = qf[:, :, n0:n0 + 128], kf[:, :, n0:n0 + 128], vf[:, :, n0:n0 + 128]
-        a = torch.tril(qc @ kc.mT)
-        out.append(qc @ S + a @ vc)
-        S = S + kc.mT @ vc
-    return (torch.cat(out, 2) / N).to(q.dtype)
-
-
 class _CausalLinearFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v):
@@ -1033,11 +1018,22 @@ class _CausalLinearFn(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, gy):
+        # Every gradient is a causal linear attention again (the same kernels):
+        #   dq_t   = (1/N) sum_{tau <= t} <gy_t, v_tau> k_tau   = CL(gy, v, k)
+        #   dk_tau = (1/N) sum_{t >= tau} <v_tau, gy_t> q_t     = CL(v, gy, q) with the token axis reversed
+        #   dv_tau = (1/N) sum_{t >= tau} <k_tau, q_t> gy_t     = CL(k, q, gy) with the token axis reversed
         q, k, v = ctx.saved_tensors
-        with torch.enable_grad():
-            qq, kk, vv = (t.detach().requires_grad_(True) for t in (q, k, v))
-            y = _causal_linear_torch(qq, kk, vv)
-            return torch.autograd.grad(y, (qq, kk, vv), gy)
+        gy = gy.to(q.dtype)
+        need = ctx.needs_input_grad
+        gq = _causal_linear_forward(gy, v, k) if need[0] else None
+        gk = gv = None
+        if need[1] or need[2]:
+            qr, kr, vr, gr = (t.flip(2) for t in (q, k, v, gy))
+            if need[1]:
+                gk = _causal_linear_forward(vr, gr, qr).flip(2)
+            if need[2]:
+                gv = _causal_linear_forward(kr, qr, gr).flip(2)
+        return gq, gk, gv
 
 
 def causal_linear_attention(q, k, v, n_segs: int = 0, force_generic: bool = False):

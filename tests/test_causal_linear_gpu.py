@@ -140,3 +140,20 @@ def test_fp32_matrix_core_kernel_runs_at_the_reference_shape(dev):
     assert torch.allclose(y.cpu().double(), yr, atol=1e-5, rtol=1e-5)
     yg = F.causal_linear_attention(q.to(dev), k.to(dev), v.to(dev), force_generic=True)
     assert O.rel_l2(yg, yr) <= 1e-5
+
+
+@pytest.mark.parametrize("shape,dtype,tol", [((2, 2, 700, 64, 64), torch.bfloat16, 3e-2), ((1, 2, 1000, 128, 32), torch.float16, 3e-2),
+                                             ((1, 3, 333, 64, 32), torch.float32, 1e-4), ((2, 1, 100, 24, 40), torch.float32, 1e-4)])
+def test_gradients_through_the_same_kernels(dev, shape, dtype, tol):
+    """dq, dk, dv are causal linear attentions themselves (dk, dv on the reversed token axis): against fp64 autograd of
+    the closed form on the same rounded inputs."""
+    q, k, v = make(*shape, dtype, seed=9)
+    g = torch.Generator().manual_seed(10)
+    gy = torch.randn(shape[0], shape[1], shape[2], shape[4], generator=g).to(dtype)
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    F.CausalLinear.apply(qd, kd, vd).backward(gy.to(dev))
+    qr, kr, vr = (t.double().requires_grad_(True) for t in (q, k, v))
+    O.causal_linear_closed_form(qr, kr, vr).backward(gy.double())
+    for a, b in ((qd, qr), (kd, kr), (vd, vr)):
+        assert a.grad.dtype == dtype and a.grad.shape == b.grad.shape
+        assert O.rel_l2(a.grad, b.grad) <= tol
