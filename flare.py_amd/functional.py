@@ -352,7 +352,11 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None):
     keep = None if key_mask is None else key_mask.to(torch.bool)
     T = _grad_tile(B, H, M, N)
     gy = gy if keep is None else gy * keep[:, None, :, None].to(gy.dtype)
-    L, z = _gather_stats_tiled(qe, k, v, scale, keep, T, drop)
+    if (drop is None and keep is None and k.is_cuda and q.dtype == k.dtype == v.dtype == torch.float32 and D <= 128):
+        # the latents' log-sum-exp and z from the forward's own gather kernel (fp32: matrix cores) instead of a torch pass
+        z, L = _gather_forward(q, k, v, scale, None, 0, False)
+    else:
+        L, z = _gather_stats_tiled(qe, k, v, scale, keep, T, drop)
     rs = 1.0 if drop is None else 1.0 / (1.0 - drop[0])
     dz = torch.zeros_like(z)
     for n0 in range(0, N, T):
