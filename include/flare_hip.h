@@ -180,7 +180,10 @@ int         flare_abi_version(void);
 const char* flare_last_error_string(void);
 
 /* Name of the kernel family the dispatcher would pick for this problem
- * ("mfma_bf16", "mfma_f16", "generic"); NULL + error on an invalid descriptor. */
+ * ("mfma_bf16", "mfma_f16", "generic"); NULL + error on an invalid descriptor.  "generic" names the family that
+ * serves fp32 and the shapes the 16-bit matrix-core kernels do not take: inside it, fp32 problems with D in
+ * {16, 32, 64}, M a multiple of 16, no dropout and 16-byte aligned rows run on fp32 matrix-core kernels
+ * (v_mfma_f32_16x16x4_f32), everything else as fp32 FMA loops; the workspace layout is the same for both. */
 const char* flare_mixer_kernel_name(const FlareMixerDesc* desc);
 
 /* Bytes of device workspace flare_gather_fwd / flare_mixer_fwd need for this problem. */
