@@ -358,37 +358,39 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None):
     else:
         L, z = _gather_stats_tiled(qe, k, v, scale, keep, T, drop)
     rs = 1.0 if drop is None else 1.0 / (1.0 - drop[0])
+    # The score tiles are taken token-major, [B,H,T,M]: the softmax over the latents then runs along the last axis
+    # (torch's kernel for an inner axis is an order of magnitude slower), and the products take transposed views.
     dz = torch.zeros_like(z)
     for n0 in range(0, N, T):
-        s = scale * (qe @ k[:, :, n0:n0 + T].float().mT)
-        Bt = torch.softmax(s, dim=2)
+        sT = scale * (k[:, :, n0:n0 + T].float() @ qe.mT)
+        BT = torch.softmax(sT, dim=-1)
         if drop is not None:
-            Bt = Bt * _dropout_keep(drop[1], 1, B, H, M, n0, min(N, n0 + T), drop[0], k.device) * rs
-        dz += Bt @ gy[:, :, n0:n0 + T].float()
+            BT = BT * _dropout_keep(drop[1], 1, B, H, M, n0, min(N, n0 + T), drop[0], k.device).mT * rs
+        dz += BT.mT @ gy[:, :, n0:n0 + T].float()
     Delta = (dz * z).sum(-1)
     gq = torch.zeros((B, H, M, D), device=k.device)
     gk = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
     gv = torch.empty((B, H, N, D), dtype=v.dtype, device=k.device)
     for n0 in range(0, N, T):
         kt, vt, gyt = k[:, :, n0:n0 + T].float(), v[:, :, n0:n0 + T].float(), gy[:, :, n0:n0 + T].float()
-        s = scale * (qe @ kt.mT)
-        Bt = torch.softmax(s, dim=2)
+        sT = scale * (kt @ qe.mT)
+        BT = torch.softmax(sT, dim=-1)
         if keep is not None:
-            s = s.masked_fill(~keep[:, None, None, n0:n0 + T], float("-inf"))
-        A = torch.exp(s - L[..., None])
+            sT = sT.masked_fill(~keep[:, None, n0:n0 + T, None], float("-inf"))
+        AT = torch.exp(sT - L[:, :, None, :])
         if drop is None:
-            delta = (gyt * (Bt.mT @ z)).sum(-1)
-            dS = A * (dz @ vt.mT - Delta[..., None]) + Bt * (z @ gyt.mT - delta[:, :, None, :])
+            delta = (gyt * (BT @ z)).sum(-1)
+            dST = AT * (vt @ dz.mT - Delta[:, :, None, :]) + BT * (gyt @ z.mT - delta[..., None])
         else:
             n1 = min(N, n0 + T)
-            K1 = _dropout_keep(drop[1], 0, B, H, M, n0, n1, drop[0], k.device) * rs
-            K2 = _dropout_keep(drop[1], 1, B, H, M, n0, n1, drop[0], k.device) * rs
-            delta = (gyt * ((Bt * K2).mT @ z)).sum(-1)
-            dS = A * (K1 * (dz @ vt.mT) - Delta[..., None]) + Bt * (K2 * (z @ gyt.mT) - delta[:, :, None, :])
-            A = A * K1
-        gv[:, :, n0:n0 + T] = (A.mT @ dz).to(gv.dtype)
-        gk[:, :, n0:n0 + T] = (scale * (dS.mT @ qe)).to(gk.dtype)
-        gq += scale * (dS @ kt)
+            K1 = _dropout_keep(drop[1], 0, B, H, M, n0, n1, drop[0], k.device).mT * rs
+            K2 = _dropout_keep(drop[1], 1, B, H, M, n0, n1, drop[0], k.device).mT * rs
+            delta = (gyt * ((BT * K2) @ z)).sum(-1)
+            dST = AT * (K1 * (vt @ dz.mT) - Delta[:, :, None, :]) + BT * (K2 * (gyt @ z.mT) - delta[..., None])
+            AT = AT * K1
+        gv[:, :, n0:n0 + T] = (AT @ dz).to(gv.dtype)
+        gk[:, :, n0:n0 + T] = (scale * (dST @ qe)).to(gk.dtype)
+        gq += scale * (dST.mT @ kt)
     if q.dim() == 3:
         gq = gq.sum(0)
     return gq.to(q.dtype), gk, gv
@@ -690,12 +692,12 @@ def _half_torch_grad(which, q, k, x, scale, key_mask, g):
         gz = torch.zeros((B, H, M, D), device=k.device)
         for n0 in range(0, N, T):
             kt, gyt = k[:, :, n0:n0 + T].float(), gy[:, :, n0:n0 + T].float()
-            Bt = torch.softmax(scale * (qe @ kt.mT), dim=2)
-            delta = (gyt * (Bt.mT @ z)).sum(-1)
-            dS = Bt * (z @ gyt.mT - delta[:, :, None, :])
-            gz += Bt @ gyt
-            gk[:, :, n0:n0 + T] = (scale * (dS.mT @ qe)).to(gk.dtype)
-            gq += scale * (dS @ kt)
+            BT = torch.softmax(scale * (kt @ qe.mT), dim=-1)       # token-major tile: the softmax runs along the last axis
+            delta = (gyt * (BT @ z)).sum(-1)
+            dST = BT * (gyt @ z.mT - delta[..., None])
+            gz += BT.mT @ gyt
+            gk[:, :, n0:n0 + T] = (scale * (dST @ qe)).to(gk.dtype)
+            gq += scale * (dST.mT @ kt)
         gx = gz.to(x.dtype)
     if q.dim() == 3:
         gq = gq.sum(0)
