@@ -360,9 +360,10 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None):
     rs = 1.0 if drop is None else 1.0 / (1.0 - drop[0])
     # The score tiles are taken token-major, [B,H,T,M]: the softmax over the latents then runs along the last axis
     # (torch's kernel for an inner axis is an order of magnitude slower), and the products take transposed views.
+    qs = scale * qe  # the scale rides on the small operand instead of a pass over every score tile
     dz = torch.zeros_like(z)
     for n0 in range(0, N, T):
-        sT = scale * (k[:, :, n0:n0 + T].float() @ qe.mT)
+        sT = k[:, :, n0:n0 + T].float() @ qs.mT
         BT = torch.softmax(sT, dim=-1)
         if drop is not None:
             BT = BT * _dropout_keep(drop[1], 1, B, H, M, n0, min(N, n0 + T), drop[0], k.device).mT * rs
@@ -373,14 +374,15 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None):
     gv = torch.empty((B, H, N, D), dtype=v.dtype, device=k.device)
     for n0 in range(0, N, T):
         kt, vt, gyt = k[:, :, n0:n0 + T].float(), v[:, :, n0:n0 + T].float(), gy[:, :, n0:n0 + T].float()
-        sT = scale * (kt @ qe.mT)
+        sT = kt @ qs.mT
         BT = torch.softmax(sT, dim=-1)
         if keep is not None:
             sT = sT.masked_fill(~keep[:, None, n0:n0 + T, None], float("-inf"))
-        AT = torch.exp(sT - L[:, :, None, :])
+        AT = sT.sub_(L[:, :, None, :]).exp_()
         if drop is None:
             delta = (gyt * (BT @ z)).sum(-1)
-            dST = AT * (vt @ dz.mT - Delta[:, :, None, :]) + BT * (gyt @ z.mT - delta[..., None])
+            dST = (vt @ dz.mT).sub_(Delta[:, :, None, :]).mul_(AT)
+            dST.addcmul_(BT, (gyt @ z.mT).sub_(delta[..., None]))
         else:
             n1 = min(N, n0 + T)
             K1 = _dropout_keep(drop[1], 0, B, H, M, n0, n1, drop[0], k.device).mT * rs
@@ -389,8 +391,9 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None):
             dST = AT * (K1 * (vt @ dz.mT) - Delta[:, :, None, :]) + BT * (K2 * (gyt @ z.mT) - delta[..., None])
             AT = AT * K1
         gv[:, :, n0:n0 + T] = (AT @ dz).to(gv.dtype)
-        gk[:, :, n0:n0 + T] = (scale * (dST @ qe)).to(gk.dtype)
-        gq += scale * (dST.mT @ kt)
+        gk[:, :, n0:n0 + T] = (dST @ qs).to(gk.dtype)
+        gq += dST.mT @ kt
+    gq *= scale
     if q.dim() == 3:
         gq = gq.sum(0)
     return gq.to(q.dtype), gk, gv
