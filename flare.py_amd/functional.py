@@ -337,7 +337,7 @@ def _gather_stats_tiled(qe, k, v, scale, keep, T, drop=None):
     return L, z
 
 
-def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None):
+def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None, stats=None):
     """dq, dk, dv of the mixer by recomputation in plain torch ops on the device: used for what the HIP backward
     does not cover (fp32, unusual shapes); the forward never takes this path.  The scores are recomputed in token
     tiles of [B,H,M,T] (GRAD_TILE_ELEMS), never as the whole [B,H,M,N] matrix, with the formulas of the HIP
@@ -345,14 +345,17 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None):
     dS = A (dz v^T - Delta) + B (z dy^T - delta), dv = A^T dz, dk = s dS^T q, dq = s dS k.
     drop = (p, seed): attention dropout as the forward kernels applied it; with keep masks K1, K2 (recomputed from
     the seed) and r = 1 / (1 - p) the weights that met v and z were A K1 r and B K2 r, so
-    dz = (B K2 r) dy, dS = A (K1 r dz v^T - Delta) + B (K2 r z dy^T - delta), dv = (A K1 r)^T dz."""
+    dz = (B K2 r) dy, dS = A (K1 r dz v^T - Delta) + B (K2 r z dy^T - delta), dv = (A K1 r)^T dz.
+    stats = (L, z) as the forward's gather kernel left them (no mask, no dropout) spares their recomputation."""
     B, H, N, D = k.shape
     qe = (q if q.dim() == 4 else q.unsqueeze(0)).float()
     M = qe.shape[2]
     keep = None if key_mask is None else key_mask.to(torch.bool)
     T = _grad_tile(B, H, M, N)
     gy = gy if keep is None else gy * keep[:, None, :, None].to(gy.dtype)
-    if (drop is None and keep is None and k.is_cuda and q.dtype == k.dtype == v.dtype == torch.float32 and D <= 128):
+    if stats is not None:
+        L, z = stats
+    elif (drop is None and keep is None and k.is_cuda and q.dtype == k.dtype == v.dtype == torch.float32 and D <= 128):
         # the latents' log-sum-exp and z from the forward's own gather kernel (fp32: matrix cores) instead of a torch pass
         z, L = _gather_forward(q, k, v, scale, None, 0, False)
     else:
@@ -407,6 +410,11 @@ class _MixerFn(torch.autograd.Function):
         if ctx.hip:
             y, z, lse_lat, lse_tok = _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major, True)
             ctx.save_for_backward(q, k, v, y, z, lse_lat, lse_tok)
+        elif (key_mask is None and k.is_cuda and q.dtype == k.dtype == v.dtype == torch.float32
+              and any(t.requires_grad for t in (q, k, v))):
+            # the torch recomputation starts from the latents' log-sum-exp and z: keep the forward's own
+            y, z, lse_lat, _ = _mixer_forward(q, k, v, scale, None, n_splits, force_generic, token_major, True)
+            ctx.save_for_backward(q, k, v, z, lse_lat)
         else:
             y, z = _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major)
             ctx.save_for_backward(q, k, v)
@@ -434,8 +442,9 @@ class _MixerFn(torch.autograd.Function):
             if km is not None:
                 gk, gv = torch.where(m4, gk, zero), torch.where(m4, gv, zero)
         else:
-            q, k, v = ctx.saved_tensors
-            gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy)
+            q, k, v, *stats = ctx.saved_tensors
+            gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy,
+                                           stats=(stats[1], stats[0]) if stats else None)
         return gq, gk, gv, None, None, None, None, None
 
 
