@@ -346,15 +346,16 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None, stats=None):
     drop = (p, seed): attention dropout as the forward kernels applied it; with keep masks K1, K2 (recomputed from
     the seed) and r = 1 / (1 - p) the weights that met v and z were A K1 r and B K2 r, so
     dz = (B K2 r) dy, dS = A (K1 r dz v^T - Delta) + B (K2 r z dy^T - delta), dv = (A K1 r)^T dz.
-    stats = (L, z) as the forward's gather kernel left them (no mask, no dropout) spares their recomputation."""
+    stats = (L, z, y) as the forward's kernels left them (no mask, no dropout) spares their recomputation."""
     B, H, N, D = k.shape
     qe = (q if q.dim() == 4 else q.unsqueeze(0)).float()
     M = qe.shape[2]
     keep = None if key_mask is None else key_mask.to(torch.bool)
     T = _grad_tile(B, H, M, N)
     gy = gy if keep is None else gy * keep[:, None, :, None].to(gy.dtype)
+    y = None
     if stats is not None:
-        L, z = stats
+        L, z, y = stats
     elif (drop is None and keep is None and k.is_cuda and q.dtype == k.dtype == v.dtype == torch.float32 and D <= 128):
         # the latents' log-sum-exp and z from the forward's own gather kernel (fp32: matrix cores) instead of a torch pass
         z, L = _gather_forward(q, k, v, scale, None, 0, False)
@@ -383,7 +384,7 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None, stats=None):
             sT = sT.masked_fill(~keep[:, None, n0:n0 + T, None], float("-inf"))
         AT = sT.sub_(L[:, :, None, :]).exp_()
         if drop is None:
-            delta = (gyt * (BT @ z)).sum(-1)
+            delta = (gyt * (BT @ z if y is None else y[:, :, n0:n0 + T].float())).sum(-1)
             dST = (vt @ dz.mT).sub_(Delta[:, :, None, :]).mul_(AT)
             dST.addcmul_(BT, (gyt @ z.mT).sub_(delta[..., None]))
         else:
@@ -414,7 +415,7 @@ class _MixerFn(torch.autograd.Function):
               and any(t.requires_grad for t in (q, k, v))):
             # the torch recomputation starts from the latents' log-sum-exp and z: keep the forward's own
             y, z, lse_lat, _ = _mixer_forward(q, k, v, scale, None, n_splits, force_generic, token_major, True)
-            ctx.save_for_backward(q, k, v, z, lse_lat)
+            ctx.save_for_backward(q, k, v, z, lse_lat, y)
         else:
             y, z = _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major)
             ctx.save_for_backward(q, k, v)
@@ -444,7 +445,7 @@ class _MixerFn(torch.autograd.Function):
         else:
             q, k, v, *stats = ctx.saved_tensors
             gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy,
-                                           stats=(stats[1], stats[0]) if stats else None)
+                                           stats=(stats[1], stats[0], stats[2]) if stats else None)
         return gq, gk, gv, None, None, None, None, None
 
 
