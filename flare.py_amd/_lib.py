@@ -16,7 +16,6 @@ FLARE_OK, FLARE_EINVAL, FLARE_EUNSUPPORTED, FLARE_EWORKSPACE, FLARE_EHIP = 0, -1
 DT_F32, DT_BF16, DT_F16 = 0, 1, 2
 FLAG_FORCE_GENERIC = 1
 FLAG_MFMA16 = 2
-FLAG_GATHER32 = 4
 FLAG_GRAD_LIKE_KV = 8
 MLP_EXPAND = 1
 ABI_VERSION = 1

@@ -90,13 +90,14 @@ MixerPlan plan_mixer(const FlareMixerDesc* d, bool want_mfma)
 {
     MixerPlan p;
     p.mfma = want_mfma;
-    const int unit = p.mfma ? flare::mfma_gather_tokens_per_iter() : 32;
+    const bool allow32 = !(d->flags & FLARE_FLAG_MFMA16);
+    const int unit = p.mfma ? flare::mfma_gather_tokens_per_iter(d->dtype, d->M, d->D, allow32) : 32;
     const int mblk = p.mfma ? ((d->M % 256 == 0 && d->D <= 32) ? d->M / 256 : (d->M % 128 == 0) ? d->M / 128 : (d->M + 63) / 64)
                             : (d->M + 63) / 64;
     int s = d->n_splits;
     if (s <= 0) {
         // one full round of resident workgroups (MFMA kernels) or ~4 per CU (generic)
-        const int64_t target = p.mfma ? flare::mfma_gather_resident_slots(d->dtype, d->M, d->D) : 4 * flare::device_cus();
+        const int64_t target = p.mfma ? flare::mfma_gather_resident_slots(d->dtype, d->M, d->D, allow32) : 4 * flare::device_cus();
         int64_t per = (int64_t)d->B * d->H * mblk;
         s = (int)((target + per - 1) / per);
         if (s < 1) s = 1;
@@ -143,7 +144,6 @@ void fill_mixer_args(flare::MixerArgs& a, const FlareMixerDesc* d, const MixerPl
     a.n_splits = p.n_splits; a.n_parts = p.n_parts; a.tokens_per_split = p.tokens_per_split;
     a.scale_log2 = d->scale * flare::kLog2e;
     a.no_mfma32 = (d->flags & FLARE_FLAG_MFMA16) ? 1 : 0;
-    a.gather32 = (d->flags & FLARE_FLAG_GATHER32) ? 1 : 0;
     a.force_fma = (d->flags & FLARE_FLAG_FORCE_GENERIC) ? 1 : 0;
     for (int i = 0; i < 3; ++i) {
         a.qs[i] = d->q_stride[i]; a.ks[i] = d->k_stride[i]; a.vs[i] = d->v_stride[i]; a.ys[i] = d->y_stride[i];

@@ -88,7 +88,6 @@ struct MixerArgs {
     int tokens_per_split;
     float scale_log2;         // scale * log2(e)
     int no_mfma32;            // 1: keep the 16x16x32 kernels where the 32x32x16 ones would run
-    int gather32;             // 1: the gather may take the 32x32x16 kernel too
     int force_fma;            // 1: fp32 problems keep the FMA kernels (no fp32 matrix-core kernels)
     // attention dropout (fp32-FMA kernels only): an entry of the softmax weights is kept when its hash is >= drop_thr
     // (24-bit compare) and then scaled by drop_rs = 1 / (1 - p); drop_thr == 0 switches it off
@@ -274,8 +273,8 @@ hipError_t launch_scatter_f32_mfma(const MixerArgs& a, hipStream_t st);
 int        gather_generic_parts_per_wg();
 
 bool       mfma_mixer_supported(int dtype, int M, int D);
-int        mfma_gather_tokens_per_iter();
-int        mfma_gather_resident_slots(int dtype, int M, int D);
+int        mfma_gather_tokens_per_iter(int dtype, int M, int D, bool allow32);
+int        mfma_gather_resident_slots(int dtype, int M, int D, bool allow32);   // allow32: the 32x32x16 gather where it takes the shape
 // workgroups of `kern` resident on the current device at once (CUs x occupancy), cached per kernel, LDS size and device
 int        resident_slots(const void* kern, size_t dyn_lds, int block_threads = 256);
 int        device_cus();
@@ -284,7 +283,7 @@ hipError_t launch_scatter_mfma(const MixerArgs& a, int dtype, hipStream_t st);
 // 32x32x16 instances (bf16, D = 32), chosen inside the two launchers above
 bool       mfma32_gather_supported(int dtype, int M, int D, bool masked);
 bool       mfma32_scatter_supported(int dtype, int M, int D, bool masked);
-int        mfma32_gather_resident_slots();
+int        mfma32_gather_resident_slots(int M);
 hipError_t launch_gather_mfma32(const MixerArgs& a, hipStream_t st);
 hipError_t launch_scatter_mfma32(const MixerArgs& a, hipStream_t st);
 

@@ -919,17 +919,24 @@ bool mfma_mixer_supported(int dtype, int M, int D)
     return true;
 }
 
-int mfma_gather_tokens_per_iter() { return kGTile; }
-
-int mfma_gather_resident_slots(int dtype, int M, int D)
+// Token granularity of a gather split: the 64-token tile of the 16x16x32 kernel, or one 32-token pass of each of
+// the four waves of the 32x32x16 kernel.  The plan depends on the descriptor only; a launch that turns out to carry a
+// key mask runs the 16x16x32 kernel on the same split, which it takes as well.
+int mfma_gather_tokens_per_iter(int dtype, int M, int D, bool allow32)
 {
+    return allow32 && mfma32_gather_supported(dtype, M, D, false) ? 128 : kGTile;
+}
+
+int mfma_gather_resident_slots(int dtype, int M, int D, bool allow32)
+{
+    if (allow32 && mfma32_gather_supported(dtype, M, D, false)) return mfma32_gather_resident_slots(M);
     const void* k = dtype == 1 ? gather_kernel_ptr_d<bf16_t>(M, D) : gather_kernel_ptr_d<f16_t>(M, D);
     return resident_slots(k, 0);
 }
 
 hipError_t launch_gather_mfma(const MixerArgs& a, int dtype, hipStream_t st)
 {
-    if (!a.no_mfma32 && a.gather32 && mfma32_gather_supported(dtype, a.M, a.D, a.mask != nullptr)) return launch_gather_mfma32(a, st);
+    if (!a.no_mfma32 && mfma32_gather_supported(dtype, a.M, a.D, a.mask != nullptr)) return launch_gather_mfma32(a, st);
     return dtype == 1 ? gather_launch_d<bf16_t>(a, st) : gather_launch_d<f16_t>(a, st);
 }
 

@@ -8,7 +8,9 @@
 // accumulators of a score tile, exponentiated and packed in pairs, ARE the two B operands of the
 // value product (registers 0..7: rows 8 (e / 4) + 4 g2 + e % 4, registers 8..15: the same + 16);
 // the A operand of the value product is laid out to match, once, when it is written to LDS
-// (scatter) or by the addresses of the LDS transpose reads (gather).
+// (scatter) or by the addresses of the LDS transpose reads (gather).  Both kernels are token parallel: a wave
+// streams its own tokens' K rows straight from global memory into matrix operands and shares nothing but the
+// latent operands in LDS with the other waves, so there is no barrier in either token loop.
 //
 // Compared with the 16x16x32 kernels this halves the number of matrix instructions per score
 // (each one keeps the vector ALU from issuing for about ten cycles, which is what bounds these
@@ -101,6 +103,15 @@ template <int Q> __device__ __forceinline__ void pack_quarter(f32x4 e, u32x4 (&p
 // putting two matrix instructions next to each other, where the second one would stall its wave.
 #define FLARE_FENCE() __builtin_amdgcn_sched_barrier(0)
 
+// f(integral_constant<int, I>) for I = I0 .. N - 1, unrolled at compile time
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 // LDS transpose read: the 16 lanes of a group each name 8 bytes (4 elements) of a row-major tile; lane i of
 // the group receives element i of the four 16-element rows named by lane quads 0..3.
 __device__ __forceinline__ u32x2 lds_read_tr16(const void* lds_addr)
@@ -111,9 +122,6 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const void* lds_addr)
     asm volatile("" ::: "memory");
     return __builtin_bit_cast(u32x2, r);
 }
-
-// c ? x : y on values (both already in registers)
-__device__ __forceinline__ u32x4 pick(bool c, u32x4 x, u32x4 y) { return c ? x : y; }
 
 __device__ __forceinline__ float max16(const f32x16& s)
 {
@@ -378,156 +386,194 @@ __global__ __launch_bounds__(256, 2) void scatter32_kernel(MixerArgs a, int toke
 }
 
 // =====================================================================================
-// gather: z = softmax_n(s q k^T) v, split over N
+// gather: z = softmax_n(s q k^T) v, token parallel inside a workgroup
 // =====================================================================================
-constexpr int kG32Tile = 128;                 // tokens per LDS tile
-constexpr int kG32TileB = kG32Tile * 64;      // bytes per K or V tile (64 bytes per token row)
-
-// One workgroup = 4 waves, 256 latents (wave w owns two latent tiles of 32), one token range.  K and V tiles of
-// 128 tokens go from global memory straight into LDS (global_load_lds, 16 bytes per lane, no registers, no
-// ds_write), double buffered; K chunks are XOR-swizzled on the global-address side so that the A-operand reads
-// are conflict free.  Score tile: rows = tokens, columns = latents; V^T operands come from the LDS transpose
-// read.  The pipeline unit is a slot = (32-token sub-tile, latent tile); sub-tiles form one sequence across
-// tile boundaries, so the pipeline never drains: the single barrier per tile sits at the start of the tile's
-// last sub-tile, when every read of the tile has been issued, and is followed by the loads of the tile after
-// the next.
+// One workgroup = 4 waves that own the same 32 MT latents and different tokens: wave w takes the 32-token passes
+// w, w + 4, w + 8, ... of the workgroup's token range.  Score tile: rows = tokens (A = K rows, straight from global
+// memory, one lane per token), columns = latents (B = Q, read from LDS where it is written once in operand order).
+// The sixteen accumulators of a score tile, exponentiated and packed, are the two B operands of the value product;
+// its A operand V^T comes from a wave-private LDS tile through the transposing read.  Nothing in the token loop is
+// shared between waves: no barrier.  The pipeline unit is a slot = (pass, latent tile): the matrix pipe computes the
+// scores of slot s + 1 and the value product of slot s - 1 while the vector ALU exponentiates slot s; the slots of
+// consecutive passes form one sequence.  K and V rows of the next pass are requested at the start of a pass.
+// At the end the four waves' sums meet in LDS and the workgroup writes one partial.
+template <int MT>
 __global__ __launch_bounds__(256, 2) void gather32_kernel(MixerArgs a)
 {
-    constexpr int D = 32, CT = 2;
-    __shared__ __attribute__((aligned(16))) uint8_t kt[2][kG32TileB];
-    __shared__ __attribute__((aligned(16))) uint8_t vt[2][kG32TileB];
-    __shared__ int wg_flag[4];
+    constexpr int D = 32;
+    static_assert(MT >= 2, "at least two latent tiles per wave");
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem32g[];
+    u32x4* qb = reinterpret_cast<u32x4*>(smem32g);              // [MT][2][64]: B operands of the score product
 
-    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g2 = lane >> 5, c32 = lane & 31;
-    const int mblocks = a.M / 256;
+    const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, g2 = lane >> 5, c32 = lane & 31;
+    uint8_t* vb = smem32g + MT * 2048 + w * 2048;               // this wave's V tile: 32 rows of 64 bytes
+    const int mblocks = a.M / (32 * MT);
     const int split = blockIdx.x / mblocks, mb = blockIdx.x % mblocks;
     const int h = blockIdx.y, b = blockIdx.z;
 
     const uint16_t* q = (const uint16_t*)a.q + b * a.qs[0] + h * a.qs[1];
     const uint16_t* k = (const uint16_t*)a.k + b * a.ks[0] + h * a.ks[1];
     const uint16_t* v = (const uint16_t*)a.v + b * a.vs[0] + h * a.vs[1];
-    const int m_base = mb * 256 + w * 64;
+    const int m_base = mb * 32 * MT;
 
-    // latent operands (B of the score product), log2-scaled
-    u32x4 qb[CT][2];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-        for (int kd = 0; kd < 2; ++kd)
-            qb[ct][kd] = scale8(load16(q + (int64_t)(m_base + ct * 32 + c32) * a.qs[2] + (2 * kd + g2) * 8), a.scale_log2);
+    for (int idx = tid; idx < MT * 128; idx += 256) {
+        const int ln = idx & 63, kd = (idx >> 6) & 1, mt = idx >> 7;
+        const int m = m_base + 32 * mt + (ln & 31), ch = 2 * kd + (ln >> 5);
+        qb[idx] = scale8(load16(q + (int64_t)m * a.qs[2] + ch * 8), a.scale_log2);
+    }
+    __syncthreads();
 
     const int n_begin = split * a.tokens_per_split;
     const int n_end = min(a.N, n_begin + a.tokens_per_split);
-    const int range = max(n_end - n_begin, 0);
-    const int G = (range + 31) >> 5;                   // sub-tiles of 32 tokens
-    const int n_tiles = (range + kG32Tile - 1) / kG32Tile;
-    const int valid_last = range - 32 * (G - 1);       // tokens of the last sub-tile (1..32)
+    const int n_last = max(n_end - 1, 0);
+    const int first = n_begin + 32 * w;
+    const int n_full = first + 32 <= n_end ? (n_end - 32 - first) / 128 + 1 : 0;   // passes of this wave inside the range
+    const int tail0 = first + 128 * n_full;                                          // start of a last, shorter pass
+    const int tail_valid = tail0 < n_end ? n_end - tail0 : 0;                        // its tokens (0: none)
 
-    // tile t of the range -> LDS buffer buf.  16-byte slot p of a tile = (token p / 4, chunk position p % 4); K
-    // stores chunk ch at position ch ^ ((token / 4) % 4).  Rows past the range end repeat its last row (their
-    // probabilities are zeroed where they are used).
-    auto stage = [&](int t, int buf) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int sb = (2 * w + j) * 64, p = sb + lane, tok = p >> 2, cp = p & 3;
-            const int n = min(n_begin + t * kG32Tile + tok, n_end - 1);
-            const uint16_t* kp = k + (int64_t)n * a.ks[2] + (cp ^ ((tok >> 2) & 3)) * 8;
-            const uint16_t* vp = v + (int64_t)n * a.vs[2] + cp * 8;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kp,
-                                             (__attribute__((address_space(3))) void*)&kt[buf][sb * 16], 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vp,
-                                             (__attribute__((address_space(3))) void*)&vt[buf][sb * 16], 16, 0, 0);
-        }
+    // K rows of a pass as A operands: lane (token c32, g2) holds d = 16 kd + 8 g2 .. + 7.  V rows as they are
+    // written to the LDS tile: lane l holds the 16-byte chunk l % 4 of row 16 j + l / 4.
+    // Rows past the end of the range repeat its last row (their probabilities are set to zero where they are used).
+    auto load_k = [&](int n0, u32x4 (&dst)[2]) {
+        const uint16_t* kr = k + (int64_t)min(n0 + c32, n_last) * a.ks[2] + g2 * 8;
+        dst[0] = load16_stream(kr);
+        dst[1] = load16_stream(kr + 16);
     };
-    auto wait_stage = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
-
-    // operands of sub-tile g: K rows (A of the score product) and V^T (A of the value product)
-    auto read_k = [&](int g, u32x4 (&ka)[2]) {
-        const uint8_t* base = kt[(g >> 2) & 1];
-        const int tok = (g & 3) * 32 + c32;
+    auto load_v = [&](int n0, u32x4 (&dst)[2]) {
 #pragma unroll
-        for (int kd = 0; kd < 2; ++kd)
-            ka[kd] = *reinterpret_cast<const u32x4*>(base + tok * 64 + (((2 * kd + g2) ^ ((tok >> 2) & 3)) << 4));
+        for (int j = 0; j < 2; ++j)
+            dst[j] = load16_stream(v + (int64_t)min(n0 + 16 * j + (lane >> 2), n_last) * a.vs[2] + (lane & 3) * 8);
     };
-    auto read_v = [&](int g, u32x4 (&va)[2]) {
-        const uint8_t* base = vt[(g >> 2) & 1];
-        const int grp = lane >> 4, i = lane & 15;       // group: rows d = 16 (grp & 1) + i, tokens of half g2 = grp >> 1
+    auto put_v = [&](const u32x4 (&src)[2]) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) *reinterpret_cast<u32x4*>(vb + (j * 64 + lane) * 16) = src[j];
+    };
+    // A operands of the value product: row d = c32, k-slot e of half hf = token 16 hf + 8 (e / 4) + 4 g2 + e % 4
+    auto read_v = [&](u32x4 (&va)[2]) {
+        const int grp = lane >> 4, i = lane & 15;
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            const int t0 = (g & 3) * 32 + 16 * hf + 4 * (grp >> 1) + (i >> 2);
+            const int t0 = 16 * hf + 4 * (grp >> 1) + (i >> 2);
             const int col = (16 * (grp & 1) + 4 * (i & 3)) * 2;
-            const u32x2 lo = lds_read_tr16(base + t0 * 64 + col);
-            const u32x2 hi = lds_read_tr16(base + (t0 + 8) * 64 + col);
+            const u32x2 lo = lds_read_tr16(vb + t0 * 64 + col);
+            const u32x2 hi = lds_read_tr16(vb + (t0 + 8) * 64 + col);
             va[hf] = u32x4{lo[0], lo[1], hi[0], hi[1]};
         }
     };
 
-    float shift[CT];
-    f32x16 zacc[CT];
-    float lsum[CT];       // this lane's share of the denominators (its 16 tokens of every sub-tile)
+    float shift[MT];
+    f32x16 zacc[MT];
+    float lsum[MT];       // this lane's share of the denominators (its 16 tokens of every pass)
 
-    // ---- optimistic pass: no softmax shift -------------------------------------------------------------
+    // ---- optimistic passes: no softmax shift ---------------------------------------------------------------
     {
-        f32x4 dsum[CT];
+        // Denominators: v_mfma_f32_4x4x4_16B_bf16 with a row selector as A adds the four probabilities a lane holds in
+        // two registers into register r of the accumulator (A row r = ones, the other rows zeros), so one f32x4 serves
+        // four latent tiles.
+        constexpr int ND = (MT + 3) / 4;
+        f32x4 dsum4[ND];
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            shift[ct] = 0.f;
-            zacc[ct] = zero16();
-            dsum[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int mt = 0; mt < MT; ++mt) {
+            shift[mt] = 0.f;
+            zacc[mt] = zero16();
+            lsum[mt] = 0.f;
         }
-        if (G > 0) {
-            u32x4 ka[2][2], va[2][2];          // by parity of the sub-tile
-            u32x4 pb[2] = {zero4(), zero4()};  // probabilities of the previous slot (none yet: zeros, met by zero values)
-            va[1][0] = zero4();
-            va[1][1] = zero4();
-            stage(0, 0);
-            wait_stage();
-            __syncthreads();
-            if (n_tiles > 1) stage(1, 1);
-            read_k(0, ka[0]);
-            read_v(0, va[0]);
-            f32x16 sc = mma32(ka[0][0], qb[0][0], zero16());
-            sc = mma32(ka[0][1], qb[0][1], sc);
-
-            auto sums = [&](int ct) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) dsum[ct] = lane_sum4(u32x2{pb[e >> 1][2 * (e & 1)], pb[e >> 1][2 * (e & 1) + 1]}, dsum[ct]);
+        for (int i = 0; i < ND; ++i) dsum4[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (n_full > 0) {
+            u32x2 sel[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const uint32_t o = (lane & 3) == r ? 0x3f803f80u : 0u;
+                sel[r] = u32x2{o, o};
+            }
+            // uniform row bases that advance by a pass, per-lane byte offsets inside a pass (no clamps: full passes only)
+            const char* kbase = reinterpret_cast<const char*>(k + (int64_t)first * a.ks[2]);
+            const char* vbase0 = reinterpret_cast<const char*>(v + (int64_t)first * a.vs[2]);
+            const char* vbase1 = reinterpret_cast<const char*>(v + (int64_t)(first + 16) * a.vs[2]);
+            const uint32_t koff = (uint32_t)((c32 * a.ks[2] + g2 * 8) * 2);
+            const uint32_t voff = (uint32_t)(((lane >> 2) * a.vs[2] + (lane & 3) * 8) * 2);
+            const int64_t kstep = 256 * a.ks[2], vstep = 256 * a.vs[2];       // bytes per 128 rows
+            auto ld_k = [&](u32x4 (&dst)[2]) {
+                dst[0] = load16_stream(kbase + koff);
+                dst[1] = load16_stream(kbase + koff + 32);
             };
-            // One slot of the steady state: exponentials of the current scores; scores of the next slot from K operands
-            // kn and latent tile CTN; value product and denominators of the previous slot (latent tile CTP) from vp.
-            auto slot = [&](auto ctn_c, const u32x4 (&kn)[2], const u32x4 (&vp)[2]) {
-                constexpr int CTN = decltype(ctn_c)::value, CTP = CTN;     // two latent tiles: next and previous coincide
+            auto ld_v = [&](u32x4 (&dst)[2]) {
+                dst[0] = load16_stream(vbase0 + voff);
+                dst[1] = load16_stream(vbase1 + voff);
+            };
+            u32x4 kb[2], kn[2], vr[2];
+            u32x4 va[2] = {zero4(), zero4()};
+            u32x4 pb[2] = {zero4(), zero4()};      // probabilities of the previous slot (none yet: zeros, met by zero values)
+            u32x4 qreg[2];
+            ld_k(kb);
+            ld_v(vr);
+            qreg[0] = qb[lane];
+            qreg[1] = qb[64 + lane];
+            f32x16 sc = mma32(kb[0], qreg[0], zero16());
+            sc = mma32(kb[1], qreg[1], sc);
+            qreg[0] = qb[2 * 64 + lane];
+            qreg[1] = qb[3 * 64 + lane];
+
+            auto den = [&](auto prev_c, auto q_c) {
+                constexpr int PREV = decltype(prev_c)::value, QQ = decltype(q_c)::value;
+                dsum4[PREV >> 2] = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(
+                    __builtin_bit_cast(s16x4, sel[PREV & 3]),
+                    __builtin_bit_cast(s16x4, u32x2{pb[QQ >> 1][2 * (QQ & 1)], pb[QQ >> 1][2 * (QQ & 1) + 1]}), dsum4[PREV >> 2], 0, 0, 0);
+            };
+            using Q0 = std::integral_constant<int, 0>;
+            using Q1 = std::integral_constant<int, 1>;
+            using Q2 = std::integral_constant<int, 2>;
+            using Q3 = std::integral_constant<int, 3>;
+
+            // One slot: exponentials of the current scores (sc); scores of the next slot (latent tile (S + 1) % MT, of the
+            // next pass's rows in the last slot); value product and denominators of the previous slot.  The latent
+            // operands of the slot after the next one are requested as soon as a product has consumed its register.
+            auto slot = [&](auto s_c) {
+                constexpr int S = decltype(s_c)::value;
+                constexpr bool LAST = S + 1 == MT;
+                using PREV = std::integral_constant<int, (S + MT - 1) % MT>;
+                constexpr int QF = (S + 2) % MT;
+                const u32x4 kx0 = LAST ? kn[0] : kb[0], kx1 = LAST ? kn[1] : kb[1];
+                f32x16 sn;
                 u32x4 pc[2];
                 f32x4 ex;
-                f32x16 sn = mma32(kn[0], qb[CTN][0], zero16());
+                // quarter 0
+                sn = mma32(kx0, qreg[0], zero16());
                 FLARE_FENCE();
+                qreg[0] = qb[(2 * QF) * 64 + lane];
                 ex = exp_quarter<0>(sc);
                 FLARE_FENCE();
-                dsum[CTP] = lane_sum4(u32x2{pb[0][0], pb[0][1]}, dsum[CTP]);
+                den(PREV{}, Q0{});
                 FLARE_FENCE();
                 pack_quarter<0>(ex, pc);
                 FLARE_FENCE();
-                zacc[CTP] = mma32(vp[0], pb[0], zacc[CTP]);
+                // quarter 1
+                zacc[PREV::value] = mma32(va[0], pb[0], zacc[PREV::value]);
                 FLARE_FENCE();
                 ex = exp_quarter<1>(sc);
                 FLARE_FENCE();
-                dsum[CTP] = lane_sum4(u32x2{pb[0][2], pb[0][3]}, dsum[CTP]);
+                den(PREV{}, Q1{});
                 FLARE_FENCE();
                 pack_quarter<1>(ex, pc);
                 FLARE_FENCE();
-                sn = mma32(kn[1], qb[CTN][1], sn);
+                // quarter 2
+                sn = mma32(kx1, qreg[1], sn);
                 FLARE_FENCE();
+                qreg[1] = qb[(2 * QF + 1) * 64 + lane];
                 ex = exp_quarter<2>(sc);
                 FLARE_FENCE();
-                dsum[CTP] = lane_sum4(u32x2{pb[1][0], pb[1][1]}, dsum[CTP]);
+                den(PREV{}, Q2{});
                 FLARE_FENCE();
                 pack_quarter<2>(ex, pc);
                 FLARE_FENCE();
-                zacc[CTP] = mma32(vp[1], pb[1], zacc[CTP]);
+                // quarter 3
+                zacc[PREV::value] = mma32(va[1], pb[1], zacc[PREV::value]);
                 FLARE_FENCE();
+                if constexpr (S == 0) read_v(va);      // this pass's V^T, after the last product with the previous pass's
                 ex = exp_quarter<3>(sc);
                 FLARE_FENCE();
-                dsum[CTP] = lane_sum4(u32x2{pb[1][2], pb[1][3]}, dsum[CTP]);
+                den(PREV{}, Q3{});
                 FLARE_FENCE();
                 pack_quarter<3>(ex, pc);
                 FLARE_FENCE();
@@ -535,168 +581,206 @@ __global__ __launch_bounds__(256, 2) void gather32_kernel(MixerArgs a)
                 pb[1] = pc[1];
                 sc = sn;
             };
-            using I0 = std::integral_constant<int, 0>;
-            using I1 = std::integral_constant<int, 1>;
-            // both slots of sub-tile g, which is not the last one (PAR = g & 1)
-            auto subtile = [&](auto par_c, int g) {
-                constexpr int PAR = decltype(par_c)::value;
-                if (PAR == 1 && (g & 3) == 3 && (g >> 2) + 1 < n_tiles) {
-                    // every read of this tile has been issued (and, by the barrier's own wait, has completed):
-                    // the next tile must have landed before anyone reads it, and this tile's buffer is free
-                    wait_stage();
-                    __syncthreads();
-                    if ((g >> 2) + 2 < n_tiles) stage((g >> 2) + 2, (g >> 2) & 1);
-                }
-                read_k(g + 1, ka[1 - PAR]);
-                slot(I1{}, ka[PAR], va[1 - PAR]);        // slot (g, 0): next (g, 1), previous (g - 1, 1)
-                read_v(g + 1, va[1 - PAR]);
-                slot(I0{}, ka[1 - PAR], va[PAR]);        // slot (g, 1): next (g + 1, 0), previous (g, 0)
-            };
-            const int Gm = G - 1;
-            int g = 0;
-            for (; g + 1 < Gm; g += 2) {
-                subtile(I0{}, g);
-                subtile(I1{}, g + 1);
-            }
-            if (g < Gm) subtile(I0{}, g);
 
-            // last sub-tile (tokens past the end of the range get probability 0), then the pipeline drains
-            {
-                const bool odd = (Gm & 1) != 0;
-                u32x4 kl[2], vl[2], vq[2];      // K, V^T of the last sub-tile; V^T of the one before it
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    kl[i] = pick(odd, ka[1][i], ka[0][i]);
-                    vl[i] = pick(odd, va[1][i], va[0][i]);
-                    vq[i] = pick(odd, va[0][i], va[1][i]);
-                }
-                auto exps = [&](u32x4 (&pc)[2]) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int r0 = 2 * e, r1 = 2 * e + 1;
-                        const bool ok0 = 8 * (r0 >> 2) + 4 * g2 + (r0 & 3) < valid_last, ok1 = 8 * (r1 >> 2) + 4 * g2 + (r1 & 3) < valid_last;
-                        pc[e >> 2][e & 3] = pack2(ok0 ? fast_exp2(sc[r0]) : 0.f, ok1 ? fast_exp2(sc[r1]) : 0.f);
-                    }
-                };
-                u32x4 pc[2];
-                // slot (G - 1, 0)
-                f32x16 sn = mma32(kl[0], qb[1][0], zero16());
-                sn = mma32(kl[1], qb[1][1], sn);
-                exps(pc);
-                zacc[1] = mma32(vq[0], pb[0], zacc[1]);
-                zacc[1] = mma32(vq[1], pb[1], zacc[1]);
-                sums(1);
-                pb[0] = pc[0]; pb[1] = pc[1]; sc = sn;
-                // slot (G - 1, 1)
-                exps(pc);
-                zacc[0] = mma32(vl[0], pb[0], zacc[0]);
-                zacc[0] = mma32(vl[1], pb[1], zacc[0]);
-                sums(0);
-                pb[0] = pc[0]; pb[1] = pc[1];
-                // drain
-                zacc[1] = mma32(vl[0], pb[0], zacc[1]);
-                zacc[1] = mma32(vl[1], pb[1], zacc[1]);
-                sums(1);
+            asm volatile("" ::"v"(kb[0]), "v"(kb[1]));
+#pragma unroll 1
+            for (int p = 0; p < n_full; ++p) {
+                put_v(vr);
+                const bool more = p + 1 < n_full;       // the last pass requests its own rows again (unused)
+                kbase += more ? kstep : 0;
+                vbase0 += more ? vstep : 0;
+                vbase1 += more ? vstep : 0;
+                ld_k(kn);
+                ld_v(vr);
+                static_for<0, MT>(slot);
+                kb[0] = kn[0];
+                kb[1] = kn[1];
             }
+            // drain: the last slot's value product and denominators
+            zacc[MT - 1] = mma32(va[0], pb[0], zacc[MT - 1]);
+            zacc[MT - 1] = mma32(va[1], pb[1], zacc[MT - 1]);
+            using PL = std::integral_constant<int, MT - 1>;
+            den(PL{}, Q0{});
+            den(PL{}, Q1{});
+            den(PL{}, Q2{});
+            den(PL{}, Q3{});
         }
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) lsum[ct] = dsum[ct][0];
+        for (int mt = 0; mt < MT; ++mt) lsum[mt] = dsum4[mt >> 2][mt & 3];
     }
 
-    // validate: every denominator of this wave inside the safe range, numerators finite
-    bool exact;
+    // one pass without pipelining: the shorter last pass of a range (`valid` tokens), and every pass of a wave
+    // that repeats its range with a running maximum per latent (EXACT)
+    auto plain_pass = [&](auto exact_c, int n0, int valid) {
+        constexpr bool EXACT = decltype(exact_c)::value;
+        u32x4 kb[2], vr[2], va[2];
+        load_k(n0, kb);
+        load_v(n0, vr);
+        put_v(vr);
+        read_v(va);
+        bool ok[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ok[r] = 8 * (r >> 2) + 4 * g2 + (r & 3) < valid;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const u32x4 q0 = qb[(2 * mt) * 64 + lane], q1 = qb[(2 * mt + 1) * 64 + lane];
+            f32x16 s = mma32(kb[0], q0, zero16());
+            s = mma32(kb[1], q1, s);
+            float nc = 0.f;
+            if (EXACT) {
+                float mx = kNegBig;
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    if (ok[r]) mx = fmaxf(mx, s[r]);
+                mx = max_xor32(mx);
+                nc = fmaxf(shift[mt], mx);
+                const float al = fast_exp2(shift[mt] - nc);
+                zacc[mt] *= al;
+                lsum[mt] *= al;
+                shift[mt] = nc;
+            }
+            u32x4 p[2];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float p0 = ok[2 * e] ? fast_exp2(s[2 * e] - nc) : 0.f;
+                const float p1 = ok[2 * e + 1] ? fast_exp2(s[2 * e + 1] - nc) : 0.f;
+                p[e >> 2][e & 3] = pack2(p0, p1);
+            }
+            float tsum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) tsum = dot2_ones(p[e >> 2][e & 3], tsum);
+            lsum[mt] += tsum;
+            zacc[mt] = mma32(va[0], p[0], zacc[mt]);
+            zacc[mt] = mma32(va[1], p[1], zacc[mt]);
+        }
+    };
+    if (tail_valid > 0) plain_pass(std::false_type{}, tail0, tail_valid);
+
+    // validate: every denominator of this wave inside the safe range, numerators finite (and small enough for the
+    // sum of four waves); a wave that fails repeats its own passes with a running maximum
+    float lfull[MT];
     {
         bool bad = false;
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            const float l = sum_xor32(lsum[ct]);
-            bad = bad || !(l <= kLMax) || (G > 0 && !(l >= kLMin));
+        for (int mt = 0; mt < MT; ++mt) {
+            const float l = sum_xor32(lsum[mt]);
+            lfull[mt] = l;
+            bad = bad || !(l <= kLMax) || (first < n_end && !(l >= kLMin));
 #pragma unroll
-            for (int r = 0; r < 16; ++r) bad = bad || !(fabsf(zacc[ct][r]) <= 3.0e38f);
+            for (int r = 0; r < 16; ++r) bad = bad || !(fabsf(zacc[mt][r]) <= 8.0e37f);
         }
-        const int anybad = __any(bad);
-        __syncthreads();
-        if (lane == 0) wg_flag[w] = anybad;
-        __syncthreads();
-        exact = (wg_flag[0] | wg_flag[1] | wg_flag[2] | wg_flag[3]) != 0;
-    }
-    if (exact) {
-        // ---- exact pass: running maximum per latent, one tile at a time ---------------------------------
-        asm volatile("; exact pass" ::: "memory");
+        if (__any(bad)) {
+            asm volatile("; exact pass" ::: "memory");
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            shift[ct] = kNegBig;
-            zacc[ct] = zero16();
-            lsum[ct] = 0.f;
-        }
-#pragma unroll 1
-        for (int t = 0; t < n_tiles; ++t) {
-            __syncthreads();
-            stage(t, 0);
-            wait_stage();
-            __syncthreads();
-            const int g_end = min(G, 4 * t + 4);
-#pragma unroll 1
-            for (int g = 4 * t; g < g_end; ++g) {
-                u32x4 ka[2], va[2];
-                read_k(g & 3, ka);
-                read_v(g & 3, va);
-                const int valid = g == G - 1 ? valid_last : 32;
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct) {
-                    f32x16 s = mma32(ka[0], qb[ct][0], zero16());
-                    s = mma32(ka[1], qb[ct][1], s);
-                    bool ok[16];
-                    float mx = kNegBig;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        ok[r] = 8 * (r >> 2) + 4 * g2 + (r & 3) < valid;
-                        if (ok[r]) mx = fmaxf(mx, s[r]);
-                    }
-                    mx = max_xor32(mx);
-                    const float nc = fmaxf(shift[ct], mx);
-                    const float al = fast_exp2(shift[ct] - nc);
-                    zacc[ct] *= al;
-                    lsum[ct] *= al;
-                    shift[ct] = nc;
-                    u32x4 p[2];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float p0 = ok[2 * e] ? fast_exp2(s[2 * e] - nc) : 0.f;
-                        const float p1 = ok[2 * e + 1] ? fast_exp2(s[2 * e + 1] - nc) : 0.f;
-                        p[e >> 2][e & 3] = pack2(p0, p1);
-                    }
-                    float tsum = 0.f;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) tsum = dot2_ones(p[e >> 2][e & 3], tsum);
-                    lsum[ct] += tsum;
-                    zacc[ct] = mma32(va[0], p[0], zacc[ct]);
-                    zacc[ct] = mma32(va[1], p[1], zacc[ct]);
-                }
+            for (int mt = 0; mt < MT; ++mt) {
+                shift[mt] = kNegBig;
+                zacc[mt] = zero16();
+                lsum[mt] = 0.f;
             }
+#pragma unroll 1
+            for (int n0 = first; n0 < n_end; n0 += 128) plain_pass(std::true_type{}, n0, min(32, n_end - n0));
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) lfull[mt] = sum_xor32(lsum[mt]);
         }
     }
 
-    // partial for this split: shift (log2 units), sum, numerator, renormalised so that the sum has exponent 0
-    // (keeps the merge free of overflow whatever the pass left behind)
+    // ---- the four waves' sums meet in LDS: (w0 + w2) + (w1 + w3) --------------------------------------------
+    // slot layout: [MT * 4][64] f32x4 numerators, then [MT][64] shifts, [MT][64] sums
+    constexpr int kSlotB = MT * 4 * 64 * 16 + 2 * MT * 64 * 4;
+    auto publish = [&](int slot_i) {
+        uint8_t* base = smem32g + slot_i * kSlotB;
+        f32x4* z4 = reinterpret_cast<f32x4*>(base);
+        float* sh = reinterpret_cast<float*>(base + MT * 4 * 64 * 16);
+        float* ls = sh + MT * 64;
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        const float l = sum_xor32(lsum[ct]);
-        int e = 0;
-        if (l > 0.f) (void)frexpf(l, &e);
-        const float scl = l > 0.f ? ldexpf(1.f, -e) : 0.f;
-        const int m = m_base + ct * 32 + c32;
-        const int64_t row = (((int64_t)b * a.H + h) * a.n_parts + split) * a.M + m;
-        if (g2 == 0) {
-            a.part_m[row] = l > 0.f ? shift[ct] + (float)e : kNegBig;
-            a.part_l[row] = l * scl;
+        for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                z4[(mt * 4 + j) * 64 + lane] = f32x4{zacc[mt][4 * j], zacc[mt][4 * j + 1], zacc[mt][4 * j + 2], zacc[mt][4 * j + 3]};
+            sh[mt * 64 + lane] = shift[mt];
+            ls[mt * 64 + lane] = lfull[mt];
         }
+    };
+    auto absorb = [&](int slot_i) {
+        const uint8_t* base = smem32g + slot_i * kSlotB;
+        const f32x4* z4 = reinterpret_cast<const f32x4*>(base);
+        const float* sh = reinterpret_cast<const float*>(base + MT * 4 * 64 * 16);
+        const float* ls = sh + MT * 64;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const f32x4 o = {zacc[ct][4 * j] * scl, zacc[ct][4 * j + 1] * scl, zacc[ct][4 * j + 2] * scl, zacc[ct][4 * j + 3] * scl};
-            *reinterpret_cast<f32x4*>(a.part_acc + row * D + 8 * j + 4 * g2) = o;
+        for (int mt = 0; mt < MT; ++mt) {
+            const float so = sh[mt * 64 + lane], lo = ls[mt * 64 + lane];
+            const float ns = fmaxf(shift[mt], so);
+            const float fa = fast_exp2(shift[mt] - ns), fb = fast_exp2(so - ns);
+            lfull[mt] = lfull[mt] * fa + lo * fb;
+            shift[mt] = ns;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f32x4 o = z4[(mt * 4 + j) * 64 + lane];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) zacc[mt][4 * j + i] = zacc[mt][4 * j + i] * fa + o[i] * fb;
+            }
+        }
+    };
+    __syncthreads();
+    if (w >= 2) publish(w - 2);
+    __syncthreads();
+    if (w < 2) absorb(w);
+    __syncthreads();
+    if (w == 1) publish(0);
+    __syncthreads();
+    if (w == 0) {
+        absorb(0);
+        // partial for this split: shift (log2 units), sum, numerator, renormalised so that the sum has exponent 0
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const float l = lfull[mt];
+            int e = 0;
+            if (l > 0.f) (void)frexpf(l, &e);
+            const float scl = l > 0.f ? ldexpf(1.f, -e) : 0.f;
+            const int m = m_base + mt * 32 + c32;
+            const int64_t row = (((int64_t)b * a.H + h) * a.n_parts + split) * a.M + m;
+            if (g2 == 0) {
+                a.part_m[row] = l > 0.f ? shift[mt] + (float)e : kNegBig;
+                a.part_l[row] = l * scl;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f32x4 o = {zacc[mt][4 * j] * scl, zacc[mt][4 * j + 1] * scl, zacc[mt][4 * j + 2] * scl, zacc[mt][4 * j + 3] * scl};
+                *reinterpret_cast<f32x4*>(a.part_acc + row * D + 8 * j + 4 * g2) = o;
+            }
         }
     }
+}
+
+// LDS of a gather workgroup: the latent operands and four V tiles in the token loop, two publishing slots afterwards
+template <int MT>
+constexpr size_t gather32_lds()
+{
+    const size_t main_b = (size_t)MT * 2048 + 4 * 2048;
+    const size_t red_b = 2 * ((size_t)MT * 4 * 64 * 16 + 2 * MT * 64 * 4);
+    return main_b > red_b ? main_b : red_b;
+}
+
+template <int MT>
+hipError_t gather32_launch(const MixerArgs& a, hipStream_t st)
+{
+    auto kern = gather32_kernel<MT>;
+    constexpr size_t lds = gather32_lds<MT>();
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    dim3 grid(a.n_splits * (a.M / (32 * MT)), a.H, a.B);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, a);
+    return hipGetLastError();
+}
+
+template <int MT>
+int gather32_slots()
+{
+    auto kern = gather32_kernel<MT>;
+    constexpr size_t lds = gather32_lds<MT>();
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        (void)hipGetLastError();
+    return resident_slots(reinterpret_cast<const void*>(kern), lds);
 }
 
 template <int KS, bool LSE>
@@ -726,11 +810,11 @@ hipError_t scatter32_launch(const MixerArgs& a, hipStream_t st)
 
 }  // namespace
 
-// bf16, D = 32; the gather takes latent counts that are multiples of 256 and no key mask, the scatter the
-// latent counts its pipeline is unrolled for.
+// bf16, D = 32, no key mask; the gather takes latent counts that are multiples of 64 (256, 128 or 64 latents per
+// workgroup), the scatter the latent counts its pipeline is unrolled for.
 bool mfma32_gather_supported(int dtype, int M, int D, bool masked)
 {
-    return dtype == 1 && D == 32 && M >= 256 && M % 256 == 0 && !masked;
+    return dtype == 1 && D == 32 && M >= 64 && M % 64 == 0 && !masked;
 }
 
 bool mfma32_scatter_supported(int dtype, int M, int D, bool masked)
@@ -738,16 +822,14 @@ bool mfma32_scatter_supported(int dtype, int M, int D, bool masked)
     return dtype == 1 && D == 32 && (M == 64 || M == 128 || M == 256 || M == 512) && !masked;
 }
 
-int mfma32_gather_resident_slots()
+int mfma32_gather_resident_slots(int M)
 {
-    return resident_slots(reinterpret_cast<const void*>(gather32_kernel), 0);
+    return M % 256 == 0 ? gather32_slots<8>() : M % 128 == 0 ? gather32_slots<4>() : gather32_slots<2>();
 }
 
 hipError_t launch_gather_mfma32(const MixerArgs& a, hipStream_t st)
 {
-    dim3 grid(a.n_splits * (a.M / 256), a.H, a.B);
-    hipLaunchKernelGGL(gather32_kernel, grid, dim3(256), 0, st, a);
-    return hipGetLastError();
+    return a.M % 256 == 0 ? gather32_launch<8>(a, st) : a.M % 128 == 0 ? gather32_launch<4>(a, st) : gather32_launch<2>(a, st);
 }
 
 hipError_t launch_scatter_mfma32(const MixerArgs& a, hipStream_t st)

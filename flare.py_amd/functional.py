@@ -103,8 +103,7 @@ _extra_mixer_flags = 0
 
 class mixer_flags:
     """Context manager that ORs FLARE_FLAG_* bits into every mixer descriptor built inside it (e.g.
-    ``_lib.FLAG_MFMA16`` to time or test the 16x16x32 kernels where the 32x32x16 scatter would run,
-    ``_lib.FLAG_GATHER32`` to run the gather on 32x32x16 products as well)."""
+    ``_lib.FLAG_MFMA16`` to time or test the 16x16x32 kernels where the 32x32x16 gather and scatter would run)."""
 
     def __init__(self, flags: int):
         self.flags = int(flags)

@@ -62,9 +62,8 @@ extern "C" {
 
 /* FlareMixerDesc.flags */
 #define FLARE_FLAG_FORCE_GENERIC 1  /* skip every matrix-core kernel (16-bit and fp32), use the fp32-FMA kernels */
-#define FLARE_FLAG_MFMA16        2  /* keep the 16x16x32 MFMA kernels where the 32x32x16 scatter (bf16, D = 32, no key mask) would run */
+#define FLARE_FLAG_MFMA16        2  /* keep the 16x16x32 MFMA kernels where the 32x32x16 gather and scatter (bf16, D = 32, no key mask) would run */
 #define FLARE_FLAG_GRAD_LIKE_KV  8  /* flare_mixer_bwd: dk has k's strides and dv has v's (default: both [B,H,N,D] contiguous) */
-#define FLARE_FLAG_GATHER32      4  /* also run the gather on 32x32x16 products (bf16, D = 32, M % 256 == 0, no key mask); measured slower than the 16x16x32 gather at the headline shape, kept for comparison */
 
 /*
  * Mixer problem description.  Logical shapes:

@@ -462,21 +462,18 @@ def test_latent_counts_that_are_multiples_of_8(dev, shape, dtype):
         assert err <= 3e-2, f"{name} rel-L2 {err:.3e}"
 
 
-# ---- 32x32x16 kernels (bf16, D = 32, no key mask): scatter at M in {64, 128, 256, 512} (default), gather at
-# M % 256 == 0 (behind FLAG_GATHER32) ----
+# ---- 32x32x16 kernels (bf16, D = 32, no key mask): scatter at M in {64, 128, 256, 512}, gather at M % 64 == 0 ----
 @pytest.mark.parametrize("shape", [
     (1, 1, 1, 256, 32), (1, 2, 5, 256, 32), (1, 2, 31, 256, 32), (1, 2, 33, 256, 32), (2, 2, 127, 256, 32),
     (1, 2, 129, 256, 32), (1, 3, 1000, 256, 32), (2, 2, 4096 + 17, 256, 32), (1, 2, 3000, 512, 32),
     (1, 2, 20000, 256, 32), (1, 2, 777, 64, 32), (1, 2, 1999, 128, 32),
+    (1, 2, 2500, 192, 32), (1, 1, 1300, 320, 32), (1, 2, 2100, 384, 32), (1, 1, 5000, 768, 32),   # 3, 5, 3, 3 latent blocks
 ])
 def test_mfma32_shapes_and_ragged_ends(dev, shape):
     from flare_py_amd import _lib
     from flare_py_amd import functional as FN
     q, k, v = make(*shape, torch.bfloat16, seed=3)
-    y, z = check(dev, q, k, v)                  # default: 32x32x16 scatter
-    with FN.mixer_flags(_lib.FLAG_GATHER32):    # 32x32x16 gather as well
-        y32, z32 = check(dev, q, k, v)
-    assert O.rel_l2(y32, y) < 1e-2
+    y, z = check(dev, q, k, v)                  # default: 32x32x16 gather and scatter
     with FN.mixer_flags(_lib.FLAG_MFMA16):      # the 16x16x32 kernels on the same problem
         y16, z16 = check(dev, q, k, v)
     assert O.rel_l2(z, z16) < 5e-3 and O.rel_l2(y, y16) < 1e-2
@@ -488,9 +485,8 @@ def test_mfma32_split_invariance_and_determinism(dev, n_splits):
     from flare_py_amd import functional as FN
     q, k, v = make(1, 2, 9000, 256, 32, torch.bfloat16, seed=5)
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
-    with FN.mixer_flags(_lib.FLAG_GATHER32):
-        y, z = F.flare_multihead_mixer(qd, kd, vd, return_z=True, n_splits=n_splits)
-        y2, z2 = F.flare_multihead_mixer(qd, kd, vd, return_z=True, n_splits=n_splits)
+    y, z = F.flare_multihead_mixer(qd, kd, vd, return_z=True, n_splits=n_splits)
+    y2, z2 = F.flare_multihead_mixer(qd, kd, vd, return_z=True, n_splits=n_splits)
     assert torch.equal(y, y2) and torch.equal(z, z2)
     yr, zr = O.mixer_explicit(q.float(), k.float(), v.float(), 1.0)
     assert O.rel_l2(z, zr) <= 2e-2 and O.rel_l2(y, yr) <= 2e-2
@@ -509,9 +505,29 @@ def test_mfma32_large_scores_take_the_exact_paths(dev):
     from flare_py_amd import _lib
     from flare_py_amd import functional as FN
     check(dev, q, k, v, tol=3e-2)
-    with FN.mixer_flags(_lib.FLAG_GATHER32):
+    check(dev, q, k, v, n_splits=4, tol=3e-2)
+    with FN.mixer_flags(_lib.FLAG_MFMA16):
         check(dev, q, k, v, tol=3e-2)
-        check(dev, q, k, v, n_splits=4, tol=3e-2)
+
+
+@pytest.mark.parametrize("wave", [0, 2, 3])
+def test_gather32_one_wave_repeats_exactly_the_others_do_not(dev, wave):
+    # the gather's waves own the 32-token passes w, w + 4, ... of a range and decide each for itself whether its sums
+    # left the unshifted window: huge scores on one wave's tokens only make that wave repeat with a running maximum,
+    # and the workgroup then adds partial sums that carry different shifts
+    B, H, N, M, D = 1, 2, 4096, 256, 32
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn(H, M, D, generator=g) * D ** -0.5
+    k = torch.randn(B, H, N, D, generator=g)
+    v = torch.randn(B, H, N, D, generator=g)
+    n = torch.arange(N)
+    hot = ((n // 32) % 4 == wave) & (n >= 1024) & (n < 1536)
+    k[:, :, hot] *= 60.0
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    s = torch.einsum("hmd,bhnd->bhmn", q.float(), k.float()) * 1.4427
+    assert float(s.max()) > 130.0
+    for n_splits in (1, 2, 0):
+        check(dev, q, k, v, n_splits=n_splits, tol=3e-2)
 
 
 @pytest.mark.parametrize("offset", [-30.0, 60.0])
@@ -527,7 +543,7 @@ def test_mfma32_constant_score_offset_stays_on_the_fast_path(dev, offset):
     k0[..., 0] = 0.0
     from flare_py_amd import _lib
     from flare_py_amd import functional as FN
-    for flags in (0, _lib.FLAG_GATHER32):
+    for flags in (0, _lib.FLAG_MFMA16):
         with FN.mixer_flags(flags):
             y0, _ = check(dev, q0, k0, v)
             y1, _ = check(dev, q2, k2, v)
