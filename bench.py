@@ -597,9 +597,9 @@ def main():
     flops_phase = 4 * B * H * N * M * D             # per phase: two products of 2*N*M*D
     # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two passes, scaled by the
     # readings of a 1 GiB copy: x2.000 and x1.000); they cannot be collected from inside this process.
-    traffic_measured = {"gather_mfma_kernel": 1.0928e9, "scatter32_kernel": 1.1088e9}
+    traffic_measured = {"gather32_kernel": 1.1113e9, "scatter32_kernel": 1.1087e9}
     if ms_gather >= ms_scatter:
-        dom, ms_dom, bytes_dom = "gather_mfma_kernel", ms_gather, bytes_gather
+        dom, ms_dom, bytes_dom = "gather32_kernel", ms_gather, bytes_gather
     else:
         dom, ms_dom, bytes_dom = "scatter32_kernel", ms_scatter, bytes_scatter
     achieved = bytes_dom / (ms_dom * 1e-3) / 1e9
