@@ -36,6 +36,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0        # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16, published
 
 
 class _Skip(Exception):
@@ -393,6 +394,109 @@ def bench_train(args, F, dev):
     return out
 
 
+def bench_layer(args, F, dev):
+    """The reference's own published benchmark (ablation/time_memory_bwd.py:208-251, 460-478, 508-513): forward +
+    backward of ONE FLARE layer - channel_dim 128, 8 heads (D = 16), k/v projections = ResidualMLPs with 3 hidden
+    layers (5 Linear each), out_proj - with an MSE loss under fp16 autocast on x[1, N, 128] ~ N(0,1) (requires_grad), for
+    M in {128, 512, 2048} latents; median time of 10 steps after 5, peak allocated memory of one more step.  The
+    reference's figure was read off a plot on one H100; it is quoted as context, not as a baseline."""
+    import torch.nn.functional as TF
+    from torch import nn
+    C, H = 128, 8
+    lengths = [int(t) for t in args.lengths.split(",")]
+    latents = [int(t) for t in args.latents.split(",")]
+    h100 = {128: 70.0, 512: 80.0, 2048: 120.0}      # ms at N = 1,000,000, +-20 %: read off figs/time_memory_bwd_fp16.png
+
+    class TorchLayer(nn.Module):
+        """The same layer as the reference writes it: torch layers and two fused scaled_dot_product_attention calls."""
+        def __init__(self, src):
+            super().__init__()
+            self.latent_q, self.k_proj, self.v_proj, self.out_proj = src.latent_q, src.k_proj, src.v_proj, src.out_proj
+            self.M = src.num_latents
+        def forward(self, x):
+            B, N, _ = x.shape
+            q = self.latent_q.view(H, self.M, C // H).unsqueeze(0).expand(B, -1, -1, -1)
+            k = self.k_proj(x).view(B, N, H, C // H).permute(0, 2, 1, 3)
+            v = self.v_proj(x).view(B, N, H, C // H).permute(0, 2, 1, 3)
+            z = TF.scaled_dot_product_attention(q, k, v, scale=1.0)
+            y = TF.scaled_dot_product_attention(k, q, z, scale=1.0)
+            return self.out_proj(y.permute(0, 2, 1, 3).reshape(B, N, C))
+
+    def measure(fwd, model, x, target, steps=10, warmup=5):
+        def fb():
+            model.zero_grad(set_to_none=True)
+            x.grad = None
+            with torch.autocast("cuda", dtype=torch.float16):
+                loss = TF.mse_loss(fwd(x), target)
+            loss.backward()
+        for _ in range(warmup):
+            fb()
+        times = []
+        for _ in range(steps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(); fb(); e1.record(); e1.synchronize()
+            times.append(e0.elapsed_time(e1))
+        times.sort()
+        torch.cuda.synchronize(); torch.cuda.empty_cache(); torch.cuda.reset_peak_memory_stats()
+        fb(); torch.cuda.synchronize()
+        return times[len(times) // 2], torch.cuda.max_memory_allocated() / 2 ** 30
+
+    results = {}
+    for N in lengths:
+        for M in latents:
+            torch.manual_seed(42)
+            layer = F.FLARE(channel_dim=C, num_heads=H, num_latents=M, num_layers_k_proj=3, num_layers_v_proj=3).to(dev).train()
+            x = torch.randn(1, N, C, device=dev, requires_grad=True)
+            target = torch.randn(1, N, C, device=dev)
+            ms, gib = measure(lambda t: layer(t)[0], layer, x, target)
+            # per token (C = 128): what has to cross HBM at least once, and the flops of the Linear layers and of the
+            # mixer (forward 4 products of 2 N M D per head, backward 10 with the scores recomputed)
+            per_token = {
+                "forward: x (fp32) in, k, v out": 4 * C + 2 * 2 * C,
+                "forward: mixer (k twice, v in, y out)": 4 * 2 * C,
+                "forward: out_proj (y in, out out) and loss (out, target fp32 in)": 2 * C + 2 * C + 2 * C + 4 * C,
+                "backward: d out, out_proj (d out, y in, dy out)": 2 * C + 2 * C + 2 * C + 2 * C,
+                "backward: mixer (k, v, dy in, dk, dv out)": 5 * 2 * C,
+                "backward: k/v projections (dk, dv, x in, dx out)": 2 * 2 * C + 4 * C + 4 * C,
+            }
+            nbytes = N * sum(per_token.values())
+            flops = N * (3 * 11 * 2 * C * C + (8 + 20) * M * C)
+            t_hbm, t_mfma = nbytes / (HBM_PEAK_GBPS * 1e9), flops / (MFMA_F16_PEAK_TFLOPS * 1e12)
+            rec = {"ms_fwd_bwd": round(ms, 3), "peak_GiB": round(gib, 3), "tokens_per_s": round(N / (ms * 1e-3), 1),
+                   "algorithmic_bytes": nbytes, "algorithmic_flops": flops,
+                   "ms_at_hbm_peak": round(t_hbm * 1e3, 3), "ms_at_mfma_peak": round(t_mfma * 1e3, 3),
+                   "frac_of_roofline": round(max(t_hbm, t_mfma) * 1e3 / ms, 4), "step_tflops": round(flops / (ms * 1e-3) / 1e12, 1)}
+            if N == lengths[0]:
+                rec["bytes_per_token_by_stage"] = per_token
+                if N == 1_000_000 and M in h100:
+                    rec["reference_on_h100_ms_read_off_plot"] = h100[M]
+            if not args.no_torch_sdpa:
+                try:
+                    tl = TorchLayer(layer)
+                    ms_t, gib_t = measure(tl, tl, x, target, steps=3, warmup=1)
+                    rec["torch_layers_same_gpu"] = {"ms_fwd_bwd": round(ms_t, 2), "peak_GiB": round(gib_t, 3), "speedup": round(ms_t / ms, 1)}
+                except Exception as e:
+                    rec["torch_layers_same_gpu"] = {"error": f"{type(e).__name__}: {str(e)[:120]}"}
+            results[f"N={N},M={M}"] = rec
+            del layer, x, target
+            torch.cuda.empty_cache()
+    head = results[f"N={lengths[0]},M={latents[0]}"]
+    out = base_record(args, f"FLARE layer forward+backward tokens/sec at N={lengths[0]:,}, C=128, H=8, M={latents[0]}, fp16 autocast",
+                      head["tokens_per_s"], "tokens/s", head["ms_fwd_bwd"],
+                      "one FLARE layer (C=128, H=8, D=16, two 5-Linear ResidualMLP projections, out_proj), forward + backward with MSE "
+                      "loss under fp16 autocast, B=1: the reference's time_memory_bwd benchmark", {"latents": latents, "lengths": lengths})
+    out["dtype"] = "f16"
+    out["steps"], out["warmup"] = 10, 5
+    bound = "hbm" if head["ms_at_hbm_peak"] >= head["ms_at_mfma_peak"] else "mfma"
+    out["roofline"] = {"bound": bound, "kernel": f"whole training step (N={lengths[0]:,}, M={latents[0]})",
+                       "achieved": round(head["algorithmic_bytes"] / (head["ms_fwd_bwd"] * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS,
+                       "unit": "GB/s", "frac": head["frac_of_roofline"], "traffic": None}
+    out["layer"] = results
+    out["reference_context"] = ("vpuri3/FLARE.py publishes this step only as a plot on one H100 80 GB: about 70 / 80 / 120 ms at "
+                                "N = 1,000,000 for M = 128 / 512 / 2048 and about 9 GB peak (read off figs/time_memory_bwd_fp16.png, +-20 %)")
+    return out
+
+
 def bench_block(args, F, dev):
     """BASELINE config 2: lift MLP (2 coordinates + 1 field -> 128), then one FLAREBlock forward (LayerNorm, k/v
     ResidualMLPs, HIP mixer, out_proj, residual, LayerNorm, GELU MLP with 4x expansion, residual)."""
@@ -541,7 +645,9 @@ def main():
     ap.add_argument("--cpu-sample", type=int, default=1048576, help="tokens of the CPU baseline sample")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-torch-sdpa", action="store_true", help="skip the legs that time torch's own formulation (fused SDPA, einsum, torch layers) on the GPU")
-    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train", "linear", "fp32"], default="mixer",
+    ap.add_argument("--lengths", default="1000000,100000", help="layer workload: token counts (the first one is the headline of the line)")
+    ap.add_argument("--latents", default="128,512,2048", help="layer workload: latent counts")
+    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train", "linear", "fp32", "layer"], default="mixer",
                     help="mixer = the headline configuration (default); the others are BASELINE configs 4, 5, 2")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -557,7 +663,7 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload != "mixer":
         fn = {"causal": bench_causal, "triple": bench_triple, "block": bench_block, "train": bench_train,
-              "linear": bench_linear, "fp32": bench_fp32}[args.workload]
+              "linear": bench_linear, "fp32": bench_fp32, "layer": bench_layer}[args.workload]
         print(json.dumps(fn(args, F, dev)))
         return
     B, H, N, M, D = 1, 8, 1 << 20, 256, 32

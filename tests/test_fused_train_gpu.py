@@ -193,6 +193,53 @@ def test_block_trains_through_the_fused_launches(dev, C, H, M, N):
         assert e <= min(6e-2, max(3e-2, 2.0 * et)), f"{n}: rel-L2 {e:.3e} (torch layers under autocast: {et:.3e})"
 
 
+@pytest.mark.parametrize("M,N", [(128, 3000), (512, 2500), (2048, 1500)])
+def test_benchmark_layer_f16_gradients_against_the_fp64_oracle(dev, M, N):
+    """The layer of the reference's time/memory benchmark (ablation/time_memory_bwd.py:208-251: channel_dim 128, 8 heads,
+    two ResidualMLP projections with 3 hidden layers, out_proj; :460-478: MSE loss under fp16 autocast) at a length the
+    CPU oracle finishes in seconds: loss, dx and every parameter's gradient against fp64 autograd through the oracle's
+    restatement of the layer on the same weights.  M = 2048 (M D = 32,768) takes the token-side backward kernel in two
+    chunks of latents."""
+    import torch.nn.functional as TF
+    from oracle import flare_oracle as O
+    torch.manual_seed(M)
+    C, H = 128, 8
+    layer = F.FLARE(channel_dim=C, num_heads=H, num_latents=M, num_layers_k_proj=3, num_layers_v_proj=3).to(dev).train()
+    x = torch.randn(1, N, C, device=dev, requires_grad=True)
+    target = torch.randn(1, N, C, device=dev)
+    def step():
+        layer.zero_grad(set_to_none=True)
+        x.grad = None
+        with torch.autocast("cuda", dtype=torch.float16):
+            loss = TF.mse_loss(layer(x)[0], target)
+        loss.backward()
+        return loss.detach(), {"x": x.grad.cpu(), **{n: p.grad.cpu() for n, p in layer.named_parameters()}}
+
+    with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CUDA]) as prof:
+        loss, got = step()
+        torch.cuda.synchronize()
+    kernels = " ".join(e.key for e in prof.key_averages())
+    assert "mlp_bwd_kernel" in kernels and "bwd_tok_kernel" in kernels and "bwd_lat_kernel" in kernels
+    saved = fused.compute_dtype
+    fused.compute_dtype = lambda *a, **k: None      # the projections as torch layers under the same autocast
+    try:
+        _, t16 = step()
+    finally:
+        fused.compute_dtype = saved
+    # fp64 oracle on the CPU, same weights
+    sd = {k: v.detach().cpu().double().requires_grad_(True) for k, v in layer.state_dict().items()}
+    xr = x.detach().cpu().double().requires_grad_(True)
+    lr = ((O.flare_layer(sd, "", xr, H) - target.cpu().double()) ** 2).mean()
+    lr.backward()
+    assert abs(float(loss) - float(lr.detach())) <= 2e-2 * abs(float(lr.detach()))
+    want = {"x": xr.grad, **{n: sd[n].grad for n, _ in layer.named_parameters()}}
+    for name in got:
+        e, et = rel(got[name], want[name]), rel(t16[name], want[name])
+        # the projections' gradients pass through the mixer's 16-bit backward and up to five layers; torch's own layers
+        # under the same autocast are as far from fp64: the bar is twice that run's error where it exceeds 1.5e-2, 6e-2 at most
+        assert e <= min(6e-2, max(3e-2, 2.0 * et)), f"{name}: rel-L2 {e:.3e} (torch layers under autocast: {et:.3e})"
+
+
 def test_shapes_without_a_backward_keep_their_torch_layers(dev):
     """With gradients enabled compute_dtype admits the C x C chain and the expanding two-layer MLP only."""
     x = torch.randn(10, 64, device=dev)
