@@ -326,6 +326,19 @@ def bench_fp32(args, F, dev):
     out["roofline"] = {"bound": "mfma", "kernel": "gather_f32_mfma_kernel + scatter_f32_mfma_kernel",
                        "achieved": round(tf, 1), "peak": 157.3, "unit": "TFLOP/s", "frac": round(tf / 157.3, 4),
                        "traffic": None, "algorithmic_flops": flops, "ms_events": round(ms_ev, 4)}
+    # forward + backward (fp32 is the reference's default training precision): 4 products forward, 11 in the three
+    # backward passes (dz; dk and dv; dq), each of 2 B H N M D flops
+    qd, kd, vd = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    gy = torch.randn_like(kd)
+
+    def train_step():
+        F.flare_multihead_mixer(qd, kd, vd).backward(gy)
+        qd.grad = kd.grad = vd.grad = None
+    ms_fb = time_events(train_step, max(3, args.steps // 5), 2)
+    flops_fb = 15 * 2.0 * B * H * N * M * D
+    out["ms_fwd_bwd"] = round(ms_fb, 3)
+    out["fwd_bwd_tflops"] = round(flops_fb / (ms_fb * 1e-3) / 1e12, 1)
+    out["fwd_bwd_frac_of_fp32_mfma_peak"] = round(flops_fb / (ms_fb * 1e-3) / 1e12 / 157.3, 4)
     q1, k1, v1 = make_inputs(1, 8, 4096, 64, 16, torch.float32, dev)
     out["roofline"]["ms_config1"] = round(time_events(lambda: F.flare_multihead_mixer(q1, k1, v1), 50, 5), 4)
     if not args.no_torch_sdpa:

@@ -442,7 +442,8 @@ BwdPlan plan_bwd(const FlareMixerDesc* d)
 {
     BwdPlan p;
     const int64_t bh = (int64_t)d->B * d->H;
-    const int mblocks = d->M % 256 == 0 ? d->M / 256 : d->M % 128 == 0 ? d->M / 128 : (d->M + 63) / 64;
+    const bool f32 = d->dtype == FLARE_DT_F32;      // the fp32 kernels cover 64 latents per workgroup, two workgroups per CU
+    const int mblocks = f32 ? (d->M + 63) / 64 : d->M % 256 == 0 ? d->M / 256 : d->M % 128 == 0 ? d->M / 128 : (d->M + 63) / 64;
     // As many workgroups per compute unit over the latent-side grids as the registers of the dq pass allow (two at
     // the larger shapes, see bwd_dq_wgs_per_cu); the dz pass needs fewer and gets three at D = 32 with 64 latents per
     // wave, four below that (measured: 74 -> 66 us at M = 128, D = 16; 203 -> 193 us at M = 128, D = 32), with its
@@ -454,8 +455,8 @@ BwdPlan plan_bwd(const FlareMixerDesc* d)
         tokens_per_split = (int)tps;
         n_splits = (int)(((int64_t)d->N + tps - 1) / tps);
     };
-    split(flare::bwd_dq_wgs_per_cu(d->D, d->M % 256 == 0 ? 4 : d->M % 128 == 0 ? 2 : 1), p.n_splits, p.tokens_per_split);
-    split(d->D <= 16 ? 4 : d->D <= 32 ? (d->M % 256 ? 4 : 3) : 2, p.n_splits0, p.tokens_per_split0);
+    split(f32 ? 2 : flare::bwd_dq_wgs_per_cu(d->D, d->M % 256 == 0 ? 4 : d->M % 128 == 0 ? 2 : 1), p.n_splits, p.tokens_per_split);
+    split(f32 ? 2 : d->D <= 16 ? 4 : d->D <= 32 ? (d->M % 256 ? 4 : 3) : 2, p.n_splits0, p.tokens_per_split0);
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     p.off_dz = up((size_t)bh * d->N * 4);
     p.off_dl = p.off_dz + up((size_t)bh * d->M * d->D * 4);
@@ -469,8 +470,15 @@ int check_bwd(const FlareMixerDesc* d)
 {
     int rc = check_mixer_desc(d);
     if (rc != FLARE_OK) return rc;
+    if (d->dtype == FLARE_DT_F32) {
+        if (!flare::mixer_bwd_f32_supported(d->M, d->D))
+            return fail(FLARE_EUNSUPPORTED, "fp32 mixer backward covers D in {16,32,64}, M %% 16 == 0 (got M=%d, D=%d)", d->M, d->D);
+        if (!strides_mult4(d->q_stride) || !strides_mult4(d->k_stride) || !strides_mult4(d->v_stride) || !strides_mult4(d->y_stride))
+            return fail(FLARE_EUNSUPPORTED, "fp32 mixer backward needs strides that are multiples of 4 elements");
+        return FLARE_OK;
+    }
     if (!flare::mixer_bwd_supported(d->dtype, d->M, d->D))
-        return fail(FLARE_EUNSUPPORTED, "mixer backward covers bf16/f16, D in {16,32,64}, M %% 32 == 0, M*D <= 65536 "
+        return fail(FLARE_EUNSUPPORTED, "mixer backward covers bf16/f16, D in {16,32,64}, M %% 32 == 0, M*D <= 65536, and fp32 "
                                         "(got dtype %d, M=%d, D=%d)", d->dtype, d->M, d->D);
     if (!strides_mult8(d->q_stride) || !strides_mult8(d->k_stride) || !strides_mult8(d->v_stride) || !strides_mult8(d->y_stride))
         return fail(FLARE_EUNSUPPORTED, "mixer backward needs strides that are multiples of 8 elements");
@@ -496,7 +504,9 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
     if (rc != FLARE_OK) return rc;
     if (!q || !k || !v || !y || !z || !lse_lat || !lse_tok || !dy || !dy_stride || !dq || !dk || !dv)
         return fail(FLARE_EINVAL, "q, k, v, y, z, lse_lat, lse_tok, dy, dy_stride, dq, dk, dv must not be NULL");
-    if (!strides_mult8(dy_stride) || dy_stride[2] < desc->D) return fail(FLARE_EINVAL, "dy strides must be multiples of 8 and its rows >= D");
+    const bool f32 = desc->dtype == FLARE_DT_F32;
+    if (!(f32 ? strides_mult4(dy_stride) : strides_mult8(dy_stride)) || dy_stride[2] < desc->D)
+        return fail(FLARE_EINVAL, "dy strides must be multiples of 16 bytes and its rows >= D");
     const void* ptrs[7] = {q, k, v, y, dy, dk, dv};
     for (const void* p : ptrs)
         if (!aligned16(p)) return fail(FLARE_EINVAL, "q, k, v, y, dy, dk, dv must be 16-byte aligned");
@@ -526,6 +536,7 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
     a.dks[0] = a.dvs[0] = (int64_t)desc->H * nd; a.dks[1] = a.dvs[1] = nd; a.dks[2] = a.dvs[2] = desc->D;
     if (desc->flags & FLARE_FLAG_GRAD_LIKE_KV)
         for (int i = 0; i < 3; ++i) { a.dks[i] = desc->k_stride[i]; a.dvs[i] = desc->v_stride[i]; }
+    if (f32) return hip_status(flare::launch_mixer_bwd_f32(a, static_cast<hipStream_t>(stream)), "fp32 mixer backward launch");
     return hip_status(flare::launch_mixer_bwd(a, desc->dtype, static_cast<hipStream_t>(stream)), "mixer backward launch");
 }
 

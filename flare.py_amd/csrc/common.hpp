@@ -299,6 +299,9 @@ size_t     mixer_bwd_lds_bytes(int M, int D);
 int        mixer_bwd_tok_chunks(int M, int D);
 bool       mixer_bwd_supported(int dtype, int M, int D);
 hipError_t launch_mixer_bwd(const MixerBwdArgs& a, int dtype, hipStream_t st);
+// fp32 inputs on v_mfma_f32_16x16x4_f32 (mixer_bwd_f32_mfma.hip): D in {16, 32, 64}, M a multiple of 16
+bool       mixer_bwd_f32_supported(int M, int D);
+hipError_t launch_mixer_bwd_f32(const MixerBwdArgs& a, hipStream_t st);
 
 bool       mlp_mfma_supported(int w_dtype, int C);
 hipError_t launch_mlp_mfma(const MlpArgs& a, int w_dtype, hipStream_t st);

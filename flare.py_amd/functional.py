@@ -225,9 +225,9 @@ def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_majo
 
 
 def _hip_backward_ok(q, k, v, key_mask, force_generic) -> bool:
-    """True when flare_mixer_bwd covers this problem (16-bit types, supported M, D, strides; a key mask is
+    """True when flare_mixer_bwd covers this problem (bf16/f16 and fp32, supported M, D, strides; a key mask is
     handled around the kernels, see _MixerFn.backward)."""
-    if force_generic or k.dtype not in (torch.bfloat16, torch.float16):
+    if force_generic or k.dtype not in (torch.bfloat16, torch.float16, torch.float32):
         return False
     if q.dtype != k.dtype or v.dtype != k.dtype or k.device.type != "cuda":
         return False
@@ -248,7 +248,8 @@ def _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy):
     q4 = _q4(q, B)
     M = q4.shape[2]
     gy = gy.to(k.dtype)
-    if gy.stride(-1) != 1 or any(s % 8 for s in gy.stride()[:3]) or gy.data_ptr() % 16:
+    per16 = 16 // k.element_size()       # elements in 16 bytes
+    if gy.stride(-1) != 1 or any(s % per16 for s in gy.stride()[:3]) or gy.data_ptr() % 16:
         gy = gy.contiguous()
     d = _mixer_desc(q4, k, v, y, scale, 0, False)
     dq = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)

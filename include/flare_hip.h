@@ -204,7 +204,9 @@ int flare_scatter_fwd(const FlareMixerDesc* desc, const void* q, const void* k, 
 int flare_scatter_fwd_lse(const FlareMixerDesc* desc, const void* q, const void* k, const float* z,
                           const uint8_t* key_mask, void* y, float* lse_tok, void* stream);
 
-/* Backward of the mixer (bf16 / f16; the shapes flare_mixer_bwd_workspace_bytes accepts).  There is no key-mask
+/* Backward of the mixer (bf16 / f16: D in {16,32,64}, M % 32 == 0, M D <= 65536; fp32: D in {16,32,64}, M % 16 == 0 -
+ * the shapes flare_mixer_bwd_workspace_bytes accepts).  fp32 is the reference's default training precision
+ * (pdebench/__main__.py:1106).  There is no key-mask
  * argument because none is needed: zero the k, v and dy rows of padded tokens, pass 1e30 as their lse_tok (and as
  * lse_lat of a batch element without tokens), and clear their dk, dv rows afterwards.
  * Inputs: q, k, v as in the forward; y and z its outputs; lse_lat = lse of flare_gather_fwd;

@@ -74,8 +74,9 @@ def test_backward_is_deterministic_and_matches_torch_recompute(dev):
 
 
 def test_fallbacks_keep_working(dev):
-    # fp32 problems and shapes the kernels do not take differentiate through the torch recomputation
-    q, k, v, gy = make(1, 2, 200, 64, 16, torch.float32, seed=7)
+    # shapes the kernels do not take (fp32 with a latent count that is not a multiple of 16) differentiate through the
+    # torch recomputation
+    q, k, v, gy = make(1, 2, 200, 40, 16, torch.float32, seed=7)
     qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
     assert not FN._hip_backward_ok(qd, kd, vd, None, False)
     big = [t.to(dev).bfloat16() for t in make(1, 1, 64, 2048, 64, torch.float32)[:3]]
@@ -83,6 +84,72 @@ def test_fallbacks_keep_working(dev):
     F.flare_multihead_mixer(qd, kd, vd).backward(gy.to(dev))
     gq, gk, gv = oracle_grads(q, k, v, gy, 1.0)
     assert O.rel_l2(qd.grad, gq) <= 1e-4 and O.rel_l2(kd.grad, gk) <= 1e-4 and O.rel_l2(vd.grad, gv) <= 1e-4
+
+
+# ---- fp32 inputs: backward kernels on the fp32 matrix instruction ----
+@pytest.mark.parametrize("shape", [(1, 2, 777, 64, 32), (2, 2, 1000, 128, 16), (1, 1, 300, 256, 32), (1, 2, 500, 128, 64),
+                                   (1, 1, 1, 16, 16), (1, 2, 15, 48, 32), (1, 3, 4100, 80, 16), (1, 1, 2100, 512, 32),
+                                   (1, 1, 900, 272, 64), (1, 2, 70001, 256, 32), (1, 2, 333, 64, 8), (1, 2, 257, 32, 24)])
+def test_fp32_backward_vs_autograd_oracle(dev, shape):
+    """fp32 is the reference's default training precision (pdebench/__main__.py:1106): dq, dk, dv of the HIP kernels
+    against fp64 autograd through the explicit-softmax oracle at 1e-4, incl. latent counts that need the token pass in
+    chunks (512 x 32, 272 x 64), ragged token counts, a single token, and head dims that are zero-padded (8, 24)."""
+    q, k, v, gy = make(*shape, torch.float32, seed=sum(shape))
+    scale = 0.8
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    if shape[4] in (16, 32, 64):
+        assert FN._hip_backward_ok(qd, kd, vd, None, False)
+    with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CUDA]) as prof:
+        F.flare_multihead_mixer(qd, kd, vd, scale=scale).backward(gy.to(dev))
+        torch.cuda.synchronize()
+    kernels = " ".join(e.key for e in prof.key_averages())
+    assert "bwd_f32_tok_kernel" in kernels and "bwd_f32_lat_kernel" in kernels, kernels
+    gq, gk, gv = oracle_grads(q, k, v, gy, scale)
+    for name, got, ref in (("dq", qd.grad, gq), ("dk", kd.grad, gk), ("dv", vd.grad, gv)):
+        assert got.dtype == torch.float32 and got.shape == ref.shape
+        err = float((got.cpu().double() - ref).norm() / (ref.norm() + 1e-300))
+        tol = 1e-4 if float(ref.norm()) > 1e-6 else float("inf")      # N = 1: dq, dk are exactly 0 up to rounding
+        assert err <= tol, f"{name} rel-L2 {err:.3e}"
+        if tol == float("inf"):
+            assert float(got.abs().max()) <= 1e-5
+
+
+def test_fp32_backward_masks_per_batch_q_strided_views_and_determinism(dev):
+    B, H, N, M, D = 3, 2, 700, 64, 32
+    g = torch.Generator().manual_seed(17)
+    q = torch.randn(B, H, M, D, generator=g) * D ** -0.5                        # one latent set per batch element
+    kk = torch.randn(B, N, H * D, generator=g)
+    vv = torch.randn(B, N, H * D, generator=g)
+    gy = torch.randn(B, H, N, D, generator=g)
+    mask = torch.ones(B, N, dtype=torch.bool)
+    mask[0, 500:] = False
+    mask[1, ::3] = False
+    mask[2, :] = False                                                           # a batch element without a token
+    kk[0, 600] = float("nan")                                                    # padding may hold anything
+    outs = []
+    for _ in range(2):
+        qd = q.to(dev).requires_grad_(True)
+        kd = kk.to(dev).requires_grad_(True)
+        vd = vv.to(dev).requires_grad_(True)
+        k4 = kd.view(B, N, H, D).permute(0, 2, 1, 3)
+        v4 = vd.view(B, N, H, D).permute(0, 2, 1, 3)
+        with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CUDA]) as prof:
+            F.flare_multihead_mixer(qd, k4, v4, key_mask=mask.to(dev)).backward(gy.to(dev))
+            torch.cuda.synchronize()
+        assert "bwd_f32_tok_kernel" in " ".join(e.key for e in prof.key_averages())
+        outs.append((qd.grad.cpu(), kd.grad.cpu(), vd.grad.cpu()))
+    assert all(torch.equal(a, b) for a, b in zip(*outs))                         # bit-stable
+    kc = torch.nan_to_num(kk, nan=0.0)
+    qr = q.double().requires_grad_(True)
+    kr = kc.double().requires_grad_(True)
+    vr = vv.double().requires_grad_(True)
+    y, _ = O.mixer_explicit(qr, kr.view(B, N, H, D).permute(0, 2, 1, 3), vr.view(B, N, H, D).permute(0, 2, 1, 3), 1.0, mask)
+    y.backward(gy.double())
+    for name, got, ref in zip(("dq", "dk", "dv"), outs[0], (qr.grad, kr.grad, vr.grad)):
+        assert torch.isfinite(got).all(), name
+        err = float((got.double() - ref).norm() / ref.norm())
+        assert err <= 1e-4, f"{name} rel-L2 {err:.3e}"
+    assert (outs[0][1][0, 500:] == 0).all() and (outs[0][2][2] == 0).all()
 
 
 def test_lse_outputs(dev):
