@@ -82,6 +82,8 @@ SYMBOLS = {
     "flare_scatter_fwd_lse": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, _P]),
     "flare_mixer_bwd_workspace_bytes": (C.c_int, [C.POINTER(FlareMixerDesc), C.POINTER(_SZ)]),
     "flare_mixer_bwd": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, _P, _P, C.POINTER(C.c_int64), _P, _P, _P, _P, _SZ, _P]),
+    "flare_gather_bwd": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
+    "flare_scatter_bwd": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, C.POINTER(C.c_int64), _P, _P, _P, _P, _SZ, _P]),
     "flare_mixer_fwd": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P, _P, _SZ, _P]),
     "flare_mixer_fwd_dropout": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, C.c_float, C.c_uint64, _P, _P, _P, _SZ, _P]),
     "flare_mixer_fwd_static": (C.c_int, [C.POINTER(FlareMixerDesc), _P, _P, _P, _P, _P, _P]),

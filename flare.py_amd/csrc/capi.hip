@@ -540,6 +540,87 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
     return hip_status(flare::launch_mixer_bwd(a, desc->dtype, static_cast<hipStream_t>(stream)), "mixer backward launch");
 }
 
+namespace {
+// Argument block of the fp32 half backwards: the whole-mixer workspace layout, one term of dS switched off.
+int half_bwd_args(flare::MixerBwdArgs& a, const FlareMixerDesc* desc, void* workspace, size_t workspace_bytes)
+{
+    int rc = check_bwd(desc);
+    if (rc != FLARE_OK) return rc;
+    if (desc->dtype != FLARE_DT_F32) return fail(FLARE_EUNSUPPORTED, "the half backwards cover fp32 (got dtype %d)", desc->dtype);
+    const BwdPlan p = plan_bwd(desc);
+    if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
+    if (workspace_bytes < p.total) return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, p.total);
+    if (!aligned16(workspace)) return fail(FLARE_EINVAL, "workspace must be 16-byte aligned");
+    memset(&a, 0, sizeof(a));
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    a.delta_tok = reinterpret_cast<float*>(ws);
+    a.dz = reinterpret_cast<float*>(ws + p.off_dz);
+    a.delta_lat = reinterpret_cast<float*>(ws + p.off_dl);
+    a.rho_min = reinterpret_cast<float*>(ws + p.off_rm);
+    a.part = reinterpret_cast<float*>(ws + p.off_part);
+    a.B = desc->B; a.H = desc->H; a.N = desc->N; a.M = desc->M; a.D = desc->D;
+    a.n_splits = p.n_splits; a.tokens_per_split = p.tokens_per_split;
+    a.n_splits0 = p.n_splits0; a.tokens_per_split0 = p.tokens_per_split0;
+    a.scale = desc->scale; a.scale_log2 = desc->scale * 1.4426950408889634f;
+    const int64_t nd = (int64_t)desc->N * desc->D;
+    for (int i = 0; i < 3; ++i) {
+        a.qs[i] = desc->q_stride[i]; a.ks[i] = desc->k_stride[i]; a.vs[i] = desc->v_stride[i]; a.ys[i] = desc->y_stride[i];
+    }
+    a.dks[0] = a.dvs[0] = (int64_t)desc->H * nd; a.dks[1] = a.dvs[1] = nd; a.dks[2] = a.dvs[2] = desc->D;
+    if (desc->flags & FLARE_FLAG_GRAD_LIKE_KV)
+        for (int i = 0; i < 3; ++i) { a.dks[i] = desc->k_stride[i]; a.dvs[i] = desc->v_stride[i]; }
+    return FLARE_OK;
+}
+}  // namespace
+
+int flare_gather_bwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v, const float* z,
+                     const float* lse_lat, const float* dz, float* dq, void* dk, void* dv,
+                     void* workspace, size_t workspace_bytes, void* stream)
+{
+    flare::MixerBwdArgs a;
+    int rc = half_bwd_args(a, desc, workspace, workspace_bytes);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !v || !z || !lse_lat || !dz || !dq || !dk || !dv)
+        return fail(FLARE_EINVAL, "q, k, v, z, lse_lat, dz, dq, dk, dv must not be NULL");
+    const void* ptrs[7] = {q, k, v, z, dz, dk, dv};
+    for (const void* p : ptrs)
+        if (!aligned16(p)) return fail(FLARE_EINVAL, "q, k, v, z, dz, dk, dv must be 16-byte aligned");
+    a.half = 1;
+    a.q = q; a.k = k; a.v = v; a.z = z; a.lse_lat = lse_lat;
+    a.dz = const_cast<float*>(dz);                 // read only in this mode
+    // the scatter term is switched off: its operands only have to be readable
+    a.y = v; a.dy = v;
+    for (int i = 0; i < 3; ++i) a.ys[i] = a.dys[i] = a.vs[i];
+    a.lse_tok = a.delta_tok;
+    a.dq = dq; a.dk = dk; a.dv = dv;
+    return hip_status(flare::launch_mixer_bwd_f32(a, static_cast<hipStream_t>(stream)), "fp32 gather backward launch");
+}
+
+int flare_scatter_bwd(const FlareMixerDesc* desc, const void* q, const void* k, const float* z, const void* y,
+                      const float* lse_tok, const void* dy, const int64_t dy_stride[3], float* dq, void* dk, float* dz,
+                      void* workspace, size_t workspace_bytes, void* stream)
+{
+    flare::MixerBwdArgs a;
+    int rc = half_bwd_args(a, desc, workspace, workspace_bytes);
+    if (rc != FLARE_OK) return rc;
+    if (!q || !k || !z || !y || !lse_tok || !dy || !dy_stride || !dq || !dk || !dz)
+        return fail(FLARE_EINVAL, "q, k, z, y, lse_tok, dy, dy_stride, dq, dk, dz must not be NULL");
+    if (!strides_mult4(dy_stride) || dy_stride[2] < desc->D) return fail(FLARE_EINVAL, "dy strides must be multiples of 16 bytes and its rows >= D");
+    const void* ptrs[7] = {q, k, z, y, dy, dk, dz};
+    for (const void* p : ptrs)
+        if (!aligned16(p)) return fail(FLARE_EINVAL, "q, k, z, y, dy, dk, dz must be 16-byte aligned");
+    a.half = 2;
+    a.q = q; a.k = k; a.z = z; a.y = y; a.dy = dy; a.lse_tok = lse_tok;
+    for (int i = 0; i < 3; ++i) a.dys[i] = dy_stride[i];
+    a.dz = dz;                                     // written by the first pass's merge, read by the other two
+    // the gather term is switched off: its operands only have to be readable
+    a.v = k;
+    for (int i = 0; i < 3; ++i) a.vs[i] = a.ks[i];
+    a.lse_lat = a.delta_lat;
+    a.dq = dq; a.dk = dk; a.dv = nullptr;
+    return hip_status(flare::launch_mixer_bwd_f32(a, static_cast<hipStream_t>(stream)), "fp32 scatter backward launch");
+}
+
 int flare_mixer_fwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
                     const uint8_t* key_mask, void* y, float* z_out, void* workspace,
                     size_t workspace_bytes, void* stream)

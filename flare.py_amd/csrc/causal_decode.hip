@@ -172,7 +172,9 @@ __global__ __launch_bounds__(64 * kDecWaves) void causal_decode_kernel(CausalArg
             const float p = fast_exp2(s - mu0);
             den += p;
             const float wgt = p * fw;
+            asm volatile("" ::: "memory");      // the lanes' stores and their reads of each other's entries keep their order
             if (score_lane) *reinterpret_cast<f32x4*>(&pgw[w][ms][0]) = f32x4{p, wgt * __builtin_amdgcn_rcpf(den), wgt, 0.f};
+            asm volatile("" ::: "memory");
 
             // ---- state stage (the table is private to the wave: its reads follow its writes in program order) ----
             float acc4[4] = {0.f, 0.f, 0.f, 0.f}, rw4[4] = {0.f, 0.f, 0.f, 0.f};     // four short chains, not one long

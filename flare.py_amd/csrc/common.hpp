@@ -182,6 +182,8 @@ struct MixerBwdArgs {
     int64_t qs[3], ks[3], vs[3], ys[3], dys[3], dks[3], dvs[3];
     int m0, mc, accumulate;  // token-side kernel only: latents [m0, m0 + mc) of the M (mc = 0: all), added to dk, dv when accumulate
     int scal_lds;            // token-side kernel only: per-latent scalars are tabled in LDS behind the operand sets
+    int half;                // fp32 kernels: 0 = whole mixer, 1 = gather half only (dz given, no scatter term), 2 = scatter half only
+                             // (no gather term, dv not written; dz is an output)
 };
 
 struct CausalLinearArgs {

@@ -12,6 +12,8 @@
 //   dz pass   (latent side, split over N)  dz partials, delta_n             -> merge: dz, Delta_m
 //   token pass (token side)                dk, dv   (q, z, dz of the (b,h) in LDS)
 //   dq pass   (latent side, split over N)  dq partials                      -> merge: dq
+// The halves called separately (models with layers between them) run the same kernels with one term of dS dropped:
+// the gather half takes dz from the caller, the scatter half returns it.
 // Every sum has a fixed order: two runs give the same bits.  A key mask needs nothing here: the caller zeroes the
 // padded tokens' rows and raises their log-sum-exp, so that their weights vanish.
 #include <algorithm>
@@ -53,7 +55,7 @@ template <int Q4> __device__ __forceinline__ f32x4 dot_rows(const f32x4 (&a)[Q4]
 // waves' sums meet in LDS and the workgroup writes one partial [64][D].
 // MODE 0: dz_m += B[n,m] dy_n (values = dY), and delta_n = <dy_n, y_n> from the first latent block.
 // MODE 1: dq_m += dS[m,n] k_n (values = K), dS assembled from three score-like products.
-template <int D, int MODE>
+template <int D, int MODE, int HALF>
 __global__ __launch_bounds__(256, (D == 64 && MODE == 1) ? 1 : 2) void bwd_f32_lat_kernel(MixerBwdArgs a)
 {
     constexpr int QL = D / 4, Q4 = QL / 4, RT = D / 16, VS = D + 4, VPT = D / 16;
@@ -74,6 +76,7 @@ __global__ __launch_bounds__(256, (D == 64 && MODE == 1) ? 1 : 2) void bwd_f32_l
     float* delta_tok = a.delta_tok + bh * a.N;
     const int tps = MODE == 0 ? a.tokens_per_split0 : a.tokens_per_split;
     const int n_parts = MODE == 0 ? a.n_splits0 : a.n_splits;
+    constexpr bool use_a = HALF != 2, use_b = HALF != 1;      // gather term, scatter term of dS
 
     // latent operands (B of the score-like products): q log2-scaled; for the dq pass also dz and z with their scalars
     f32x4 qb[CT][Q4], dzb[MODE ? CT : 1][Q4], zb[MODE ? CT : 1][Q4];
@@ -150,11 +153,15 @@ __global__ __launch_bounds__(256, (D == 64 && MODE == 1) ? 1 : 2) void bwd_f32_l
             rh[r] = rho[r];
             de[r] = MODE ? dt[r] : 0.f;
         }
+        // The tile passes between the lanes of the wave through LDS.  To the compiler every lane is a thread of its own: it
+        // may move a lane's reads of other lanes' rows across that lane's own stores unless told not to.
+        asm volatile("" ::: "memory");
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             const int c = lane + 64 * i, tok = c / (D / 4), ch = c % (D / 4);
             *reinterpret_cast<f32x4*>(&vt[w][tok][4 * ch]) = vr[i];
         }
+        asm volatile("" ::: "memory");
         if constexpr (MODE == 0) if (mb == 0) {
             // delta_n = <dy_n, y_n>: the lane's share of the row, summed over the four lane groups
             float s = 0.f;
@@ -182,8 +189,11 @@ __global__ __launch_bounds__(256, (D == 64 && MODE == 1) ? 1 : 2) void bwd_f32_l
                 const f32x4 t2 = dot_rows<Q4>(dyc, zb[ct]);      // <dy_n, z_m>
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const float wa = fast_exp2(s[r] - l2[ct]), wb = fast_exp2(s[r] - rh[r]);
-                    p[r] = valid[r] ? wa * (t1[r] - dl[ct]) + wb * (t2[r] - de[r]) : 0.f;
+                    // a half's absent term is left out at compile time: its operands may be anything
+                    float ds = 0.f;
+                    if constexpr (use_a) ds = fast_exp2(s[r] - l2[ct]) * (t1[r] - dl[ct]);
+                    if constexpr (use_b) ds += fast_exp2(s[r] - rh[r]) * (t2[r] - de[r]);
+                    p[r] = valid[r] ? ds : 0.f;
                 }
             }
 #pragma unroll
@@ -242,11 +252,24 @@ __global__ __launch_bounds__(256) void bwd_f32_merge_kernel(MixerBwdArgs a)
     if (MODE == 0) a.delta_lat[r] = delta;
 }
 
+// Delta_m = <dz_m, z_m> of a dz that the caller hands in (gather half): one thread per (b, h, m).
+__global__ __launch_bounds__(256) void bwd_f32_delta_kernel(MixerBwdArgs a)
+{
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= (int64_t)a.B * a.H * a.M) return;
+    float delta = 0.f;
+    for (int d = 0; d < a.D; d += 4) {
+        const f32x4 s = *reinterpret_cast<const f32x4*>(a.dz + r * a.D + d), zz = *reinterpret_cast<const f32x4*>(a.z + r * a.D + d);
+        delta += s[0] * zz[0] + s[1] * zz[1] + s[2] * zz[2] + s[3] * zz[3];
+    }
+    a.delta_lat[r] = delta;
+}
+
 // ---- token pass: dk, dv ---------------------------------------------------------------------------------------------
 // q (log2-scaled), z and dz rows of latents [m0, m0 + mc) of one (b,h) in LDS with their scalars; a wave takes 16 tokens
 // at a time (lane = token column c16) and walks the latents 16 at a time (rows 4g + r).  8 waves per workgroup share
 // the operands.  dk comes out in units of the log2-scaled q: multiplied by ln 2 at the end.
-template <int D>
+template <int D, int HALF>
 __global__ __launch_bounds__(512) void bwd_f32_tok_kernel(MixerBwdArgs a)
 {
     constexpr int QL = D / 4, Q4 = QL / 4, RT = D / 16, LS = D + 4;
@@ -282,6 +305,7 @@ __global__ __launch_bounds__(512) void bwd_f32_tok_kernel(MixerBwdArgs a)
     }
     __syncthreads();
 
+    constexpr bool use_a = HALF != 2, use_b = HALF != 1;      // gather term, scatter term of dS
     const int tiles = (a.N + 15) / 16;
     const int stride = gridDim.x * 8;
     int tile = blockIdx.x * 8 + w;
@@ -332,8 +356,14 @@ __global__ __launch_bounds__(512) void bwd_f32_tok_kernel(MixerBwdArgs a)
             float wa[4], ds[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                wa[r] = fast_exp2(s[r] - l2[r]);
-                ds[r] = wa[r] * (t1[r] - dl[r]) + fast_exp2(s[r] - rho) * (t2[r] - dlt);
+                // a half's absent term is left out at compile time: its operands may be anything
+                wa[r] = 0.f;
+                ds[r] = 0.f;
+                if constexpr (use_a) {
+                    wa[r] = fast_exp2(s[r] - l2[r]);
+                    ds[r] = wa[r] * (t1[r] - dl[r]);
+                }
+                if constexpr (use_b) ds[r] += fast_exp2(s[r] - rho) * (t2[r] - dlt);
             }
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -357,10 +387,10 @@ __global__ __launch_bounds__(512) void bwd_f32_tok_kernel(MixerBwdArgs a)
                 f32x4 ok = dka[rt] * kLn2, ov = dva[rt];
                 if (a.accumulate) {
                     ok += *pk;
-                    ov += *pv;
+                    if constexpr (use_a) ov += *pv;
                 }
                 *pk = ok;
-                *pv = ov;
+                if constexpr (use_a) *pv = ov;
             }
         }
     }
@@ -379,17 +409,21 @@ int tok_chunk(int M, int D)
     return mc;
 }
 
-template <int D>
-hipError_t launch_d(const MixerBwdArgs& a0, hipStream_t st)
+template <int D, int HALF>
+hipError_t launch_dh(const MixerBwdArgs& a0, hipStream_t st)
 {
     MixerBwdArgs a = a0;
     const int mblocks = (a.M + 16 * lat_tiles(D, 0) - 1) / (16 * lat_tiles(D, 0)), mblocks1 = (a.M + 16 * lat_tiles(D, 1) - 1) / (16 * lat_tiles(D, 1));
     const int64_t rows = (int64_t)a.B * a.H * a.M;
-    hipLaunchKernelGGL((bwd_f32_lat_kernel<D, 0>), dim3(a.n_splits0 * mblocks, a.H, a.B), dim3(256), 0, st, a);
-    hipLaunchKernelGGL(bwd_f32_merge_kernel<0>, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a);
+    if (HALF == 1) {
+        hipLaunchKernelGGL(bwd_f32_delta_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL((bwd_f32_lat_kernel<D, 0, 0>), dim3(a.n_splits0 * mblocks, a.H, a.B), dim3(256), 0, st, a);
+        hipLaunchKernelGGL(bwd_f32_merge_kernel<0>, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a);
+    }
     // token pass, in chunks of latents when their operands do not fit the LDS
     const int mc = tok_chunk(a.M, D);
-    auto kern = bwd_f32_tok_kernel<D>;
+    auto kern = bwd_f32_tok_kernel<D, HALF>;
     const size_t lds = (size_t)mc * ((size_t)3 * (D + 4) * 4 + 8);
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
@@ -403,9 +437,15 @@ hipError_t launch_d(const MixerBwdArgs& a0, hipStream_t st)
         a.accumulate = m0 > 0;
         hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, a);
     }
-    hipLaunchKernelGGL((bwd_f32_lat_kernel<D, 1>), dim3(a.n_splits * mblocks1, a.H, a.B), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((bwd_f32_lat_kernel<D, 1, HALF>), dim3(a.n_splits * mblocks1, a.H, a.B), dim3(256), 0, st, a);
     hipLaunchKernelGGL(bwd_f32_merge_kernel<1>, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a);
     return hipGetLastError();
+}
+
+template <int D>
+hipError_t launch_d(const MixerBwdArgs& a, hipStream_t st)
+{
+    return a.half == 1 ? launch_dh<D, 1>(a, st) : a.half == 2 ? launch_dh<D, 2>(a, st) : launch_dh<D, 0>(a, st);
 }
 
 }  // namespace

@@ -103,11 +103,15 @@ __global__ __launch_bounds__(256) void gather_f32_mfma_kernel(MixerArgs a)
         f32x4 kc[QL / 4];
 #pragma unroll
         for (int j4 = 0; j4 < QL / 4; ++j4) kc[j4] = ka[j4];
+        // The tile passes between the lanes of the wave through LDS.  To the compiler every lane is a thread of its own: it
+        // may move a lane's reads of other lanes' rows across that lane's own stores unless told not to.
+        asm volatile("" ::: "memory");
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             const int c = lane + 64 * i, tok = c / (D / 4), ch = c % (D / 4);
             *reinterpret_cast<f32x4*>(&vt[w][tok][4 * ch]) = vkeep[i] ? vr[i] : f32x4{0.f, 0.f, 0.f, 0.f};
         }
+        asm volatile("" ::: "memory");
         bool valid[4];      // a token past the range or padded by the key mask takes no part
 #pragma unroll
         for (int r = 0; r < 4; ++r) valid[r] = n0 + 4 * g + r < n_end && keep_n[r] != 0;

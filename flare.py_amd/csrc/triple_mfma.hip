@@ -294,7 +294,11 @@ __global__ __launch_bounds__(256) void triple_out_mfma_kernel(TripleArgs a, int 
     };
     auto tile = [&](int n0, uint2 r1, uint2 r2) {
         const uint2 f2 = feat4_of<T>(r2, n0 + tok < wg_n1, a.feature_map);
+        // (to the compiler every lane is a thread of its own: without the two fences it may move a lane's reads of other
+        // lanes' rows across that lane's own store)
+        asm volatile("" ::: "memory");
         *reinterpret_cast<f32x4*>(&q2f[w][tok][piece]) = f32x4{M_::lo(f2.x), M_::hi(f2.x), M_::lo(f2.y), M_::hi(f2.y)};
+        asm volatile("" ::: "memory");
         const uint2 q1b = feat4_of<T>(r1, n0 + c16 < wg_n1, a.feature_map);
         // the sixteen f(q2) of the lane's token (the tile is private to the wave: reads follow its writes in program order)
         float r[kD];
@@ -398,12 +402,14 @@ __global__ __launch_bounds__(256) void triple_out_blocks_kernel(TripleArgs a, in
                 r1[i] = *reinterpret_cast<const uint2*>(q1r + 16 * i);
                 r2[i] = *reinterpret_cast<const uint2*>(q2r + 16 * i);
             }
+        asm volatile("" ::: "memory");      // the lanes' stores and their reads of each other's rows keep their order
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             if (i < nbq) {
                 const uint2 f2 = feat4_of<T>(r2[i], n0 + tok < wg_n1, a.feature_map);
                 *reinterpret_cast<f32x4*>(q2w + tok * QS + 16 * i + piece) = f32x4{M_::lo(f2.x), M_::hi(f2.x), M_::lo(f2.y), M_::hi(f2.y)};
             }
+        asm volatile("" ::: "memory");
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};   // out[n = c16][j = 16 jb + 4g + e]
         float den = 0.f;
         for (int ibb = 0; ibb < nbq; ++ibb) {

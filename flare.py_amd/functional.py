@@ -650,7 +650,8 @@ def _gather_forward(q, k, v, scale, key_mask, n_splits, force_generic):
     return z, lse
 
 
-def _scatter_forward(q, k, z, scale, key_mask, force_generic):
+def _scatter_forward(q, k, z, scale, key_mask, force_generic, want_lse=False):
+    """y (and with want_lse each token's log-sum-exp over the latents, which the HIP backward of the half needs)."""
     _require_cuda(q, k, z)
     lib = _lib.load()
     if q.dtype != k.dtype:
@@ -666,6 +667,13 @@ def _scatter_forward(q, k, z, scale, key_mask, force_generic):
     y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
     mask = _mask_u8(key_mask, B, N, k.device)
     d = _mixer_desc(q4, k, None, y, scale, 0, force_generic)
+    if want_lse:
+        lse_tok = torch.empty((B, H, N), dtype=torch.float32, device=k.device)
+        with _on_device(k.device):
+            rc = lib.flare_scatter_fwd_lse(C.byref(d), _ptr(q4), _ptr(k), _ptr(z), _ptr(mask), _ptr(y), _ptr(lse_tok),
+                                           C.c_void_p(_stream_ptr(k.device)))
+        _lib.check(rc, "flare_scatter_fwd_lse")
+        return y, lse_tok
     with _on_device(k.device):
         rc = lib.flare_scatter_fwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(z), _ptr(mask), _ptr(y),
                                    C.c_void_p(_stream_ptr(k.device)))
@@ -717,18 +725,96 @@ def _half_torch_grad(which, q, k, x, scale, key_mask, g):
     return gq.to(q.dtype), gk, gx
 
 
+def _half_hip_ok(q, k, other, key_mask, force_generic) -> bool:
+    """True when the fp32 HIP backward of a half (flare_gather_bwd / flare_scatter_bwd) covers the problem."""
+    if force_generic or k.dtype != torch.float32 or q.dtype != torch.float32 or other.dtype != torch.float32 or not k.is_cuda:
+        return False
+    k = _rows_last_contig(k)
+    q4 = _q4(q, k.shape[0])
+    if any(t.data_ptr() % 16 for t in (q4, k)):
+        return False
+    d = _mixer_desc(q4, k, k, None, 1.0, 0, False)
+    need = C.c_size_t(0)
+    return _lib.load().flare_mixer_bwd_workspace_bytes(C.byref(d), C.byref(need)) == _lib.FLARE_OK
+
+
+def _half_hip_grad(which, q, k, x, z, aux, scale, key_mask, g):
+    """Gradients of a half from the fp32 HIP kernels.  gather: x = v, aux = lse_lat, g = dz -> (dq, dk, dv);
+    scatter: x = y, aux = lse_tok, g = dy -> (dq, dk, dz).  A key mask is handled as in _MixerFn.backward."""
+    lib = _lib.load()
+    k = _rows_last_contig(k)
+    B, H, N, D = k.shape
+    q4 = _q4(q, B)
+    M = q4.shape[2]
+    keep = None
+    if key_mask is not None:
+        keep = key_mask.to(torch.bool)
+        m4 = keep[:, None, :, None]
+        k = torch.where(m4, k, k.new_zeros(()))
+    z = z.contiguous()
+    dq = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
+    dk = torch.empty((B, H, N, D), dtype=torch.float32, device=k.device)
+    if which == "gather":
+        v = _rows_last_contig(x)
+        aux = aux.contiguous()
+        if keep is not None:
+            v = torch.where(m4, v, v.new_zeros(()))
+            aux = torch.where(torch.isfinite(aux), aux, aux.new_tensor(1e30))
+        if v.data_ptr() % 16 or any(s % 4 for s in v.stride()[:3]):
+            v = v.contiguous()
+        gz = g.to(torch.float32).contiguous()
+        d = _mixer_desc(q4, k, v, None, scale, 0, False)
+        out = torch.empty((B, H, N, D), dtype=torch.float32, device=k.device)
+    else:
+        y = x.contiguous()
+        gy = g.to(torch.float32)
+        aux = aux.contiguous()
+        if keep is not None:
+            gy = torch.where(m4, gy, gy.new_zeros(()))
+            aux = torch.where(keep[:, None, :], aux, aux.new_tensor(1e30))
+        if gy.stride(-1) != 1 or any(s % 4 for s in gy.stride()[:3]) or gy.data_ptr() % 16:
+            gy = gy.contiguous()
+        d = _mixer_desc(q4, k, k, y, scale, 0, False)
+        out = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
+    need = C.c_size_t(0)
+    _lib.check(lib.flare_mixer_bwd_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_bwd_workspace_bytes")
+    ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
+    st = C.c_void_p(_stream_ptr(k.device))
+    with _on_device(k.device):
+        if which == "gather":
+            rc = lib.flare_gather_bwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(z), _ptr(aux), _ptr(gz), _ptr(dq), _ptr(dk),
+                                      _ptr(out), _ptr(ws), ws.numel(), st)
+        else:
+            rc = lib.flare_scatter_bwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(z), _ptr(y), _ptr(aux), _ptr(gy), _s3(gy), _ptr(dq),
+                                       _ptr(dk), _ptr(out), _ptr(ws), ws.numel(), st)
+    _lib.check(rc, "flare_gather_bwd" if which == "gather" else "flare_scatter_bwd")
+    if keep is not None:
+        dk = torch.where(m4, dk, dk.new_zeros(()))
+        if which == "gather":
+            out = torch.where(m4, out, out.new_zeros(()))
+    gq = dq.sum(0) if q.dim() == 3 else dq
+    return gq, dk, out
+
+
 class _GatherFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, scale, key_mask, n_splits, force_generic):
         ctx.scale, ctx.key_mask = scale, key_mask
-        ctx.save_for_backward(q, k, v)
         z, lse = _gather_forward(q, k, v, scale, key_mask, n_splits, force_generic)
+        ctx.hip = _half_hip_ok(q, k, v, key_mask, force_generic)
+        if ctx.hip:
+            ctx.save_for_backward(q, k, v, z, lse)
+        else:
+            ctx.save_for_backward(q, k, v)
         ctx.mark_non_differentiable(lse)
         return z, lse
 
     @staticmethod
     @once_differentiable
     def backward(ctx, gz, _glse):
+        if ctx.hip:
+            q, k, v, z, lse = ctx.saved_tensors
+            return (*_half_hip_grad("gather", q, k, v, z, lse, ctx.scale, ctx.key_mask, gz), None, None, None, None)
         q, k, v = ctx.saved_tensors
         return (*_half_torch_grad("gather", q, k, v, ctx.scale, ctx.key_mask, gz), None, None, None, None)
 
@@ -737,12 +823,20 @@ class _ScatterFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, z, scale, key_mask, force_generic):
         ctx.scale, ctx.key_mask = scale, key_mask
+        ctx.hip = _half_hip_ok(q, k, z, key_mask, force_generic)
+        if ctx.hip:
+            y, lse_tok = _scatter_forward(q, k, z, scale, key_mask, force_generic, want_lse=True)
+            ctx.save_for_backward(q, k, z, y, lse_tok)
+            return y
         ctx.save_for_backward(q, k, z)
         return _scatter_forward(q, k, z, scale, key_mask, force_generic)
 
     @staticmethod
     @once_differentiable
     def backward(ctx, gy):
+        if ctx.hip:
+            q, k, z, y, lse_tok = ctx.saved_tensors
+            return (*_half_hip_grad("scatter", q, k, y, z, lse_tok, ctx.scale, ctx.key_mask, gy), None, None, None)
         q, k, z = ctx.saved_tensors
         return (*_half_torch_grad("scatter", q, k, z, ctx.scale, ctx.key_mask, gy), None, None, None)
 

@@ -16,6 +16,7 @@
  *   flare_gather_fwd           first F.scaled_dot_product_attention(q, k, v) of the above
  *   flare_scatter_fwd          second F.scaled_dot_product_attention(k, q, z) of the above
  *   flare_scatter_fwd_lse      the same, also returning each token's log-sum-exp over the latents
+ *   flare_gather_bwd / flare_scatter_bwd   gradients of the two calls above taken one at a time
  *   flare_mixer_bwd            gradient of flare_multihead_mixer (torch autograd through the two SDPA
  *                              calls upstream; ablation/time_memory_bwd.py:460-478 times fwd+bwd)
  *   flare_mixer_fwd_dropout    the same two calls with dropout_p > 0 (lra/models/backends.py:592,605-606)
@@ -219,6 +220,20 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
                     const float* z, const float* lse_lat, const float* lse_tok, const void* dy,
                     const int64_t dy_stride[3], float* dq, void* dk, void* dv,
                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* Backward of the two halves called separately, fp32 only (same shapes and workspace as flare_mixer_bwd; models that
+ * put layers between the halves: pdebench/models/flare_ablations.py:19-311 of the reference).  A key mask is handled
+ * around them as for flare_mixer_bwd.
+ * flare_gather_bwd:  gradient of flare_gather_fwd (the first scaled_dot_product_attention(q, k, v)): from dz
+ *                    [B,H,M,D] fp32, with z and lse_lat of the forward, to dq [B,H,M,D] fp32, dk, dv [B,H,N,D].
+ * flare_scatter_bwd: gradient of flare_scatter_fwd (the second scaled_dot_product_attention(k, q, z)): from dy, with y
+ *                    and lse_tok of flare_scatter_fwd_lse, to dq, dk and dz [B,H,M,D] fp32 (the gradient of z). */
+int flare_gather_bwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v, const float* z,
+                     const float* lse_lat, const float* dz, float* dq, void* dk, void* dv,
+                     void* workspace, size_t workspace_bytes, void* stream);
+int flare_scatter_bwd(const FlareMixerDesc* desc, const void* q, const void* k, const float* z, const void* y,
+                      const float* lse_tok, const void* dy, const int64_t dy_stride[3], float* dq, void* dk, float* dz,
+                      void* workspace, size_t workspace_bytes, void* stream);
 
 /* gather + merge + scatter on one stream.  z_out (fp32 [B,H,M,D]) may be NULL, in which
  * case z lives in the workspace. */

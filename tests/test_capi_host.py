@@ -174,7 +174,14 @@ def test_new_struct_sizes_and_entry_point_validation():
     # mixer backward: supported shapes only, workspace checked
     d = _mixer_desc(M=128, D=32)
     assert lib.flare_mixer_bwd_workspace_bytes(d, C.byref(need)) == _lib.FLARE_OK and need.value > 0
-    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(dtype=_lib.DT_F32), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
+    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(dtype=_lib.DT_F32), C.byref(need)) == _lib.FLARE_OK     # fp32 kernels
+    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(dtype=_lib.DT_F32, M=40), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
+    assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(dtype=_lib.DT_F32, D=24), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
+    # the halves' backward: fp32 only, arguments checked before anything is launched
+    f = _mixer_desc(dtype=_lib.DT_F32)
+    assert lib.flare_gather_bwd(d, *([None] * 9), None, 0, None) == _lib.FLARE_EUNSUPPORTED
+    assert lib.flare_gather_bwd(f, *([None] * 9), None, 0, None) == _lib.FLARE_EWORKSPACE
+    assert lib.flare_scatter_bwd(f, *([None] * 6), None, None, None, None, None, 0, None) == _lib.FLARE_EWORKSPACE
     assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=256, D=64), C.byref(need)) == _lib.FLARE_OK      # one LDS-full exactly
     assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=1024, D=64), C.byref(need)) == _lib.FLARE_OK     # four chunks of latents
     assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=2048, D=64), C.byref(need)) == _lib.FLARE_EUNSUPPORTED

@@ -152,6 +152,39 @@ def test_fp32_backward_masks_per_batch_q_strided_views_and_determinism(dev):
     assert (outs[0][1][0, 500:] == 0).all() and (outs[0][2][2] == 0).all()
 
 
+@pytest.mark.parametrize("shape,masked", [((1, 2, 777, 64, 32), False), ((2, 2, 1000, 128, 16), True), ((1, 1, 300, 256, 64), False),
+                                          ((2, 3, 97, 48, 32), True), ((1, 1, 1300, 512, 32), False)])
+def test_fp32_halves_backward_vs_autograd_oracle(dev, shape, masked):
+    """flare_gather and flare_scatter called separately with a layer between them (what the ablation models do,
+    pdebench/models/flare_ablations.py): fp32 gradients of q, k, v from the HIP kernels of the two halves
+    (flare_gather_bwd, flare_scatter_bwd) against fp64 autograd through the explicit formulas."""
+    B, H, N, M, D = shape
+    q, k, v, gy = make(*shape, torch.float32, seed=3 + N)
+    w = torch.randn(D, D, generator=torch.Generator().manual_seed(1)) * D ** -0.5         # the layer between the halves
+    mask = None
+    if masked:
+        mask = torch.ones(B, N, dtype=torch.bool)
+        mask[0, N // 2:] = False
+        mask[-1, ::4] = False
+    qd, kd, vd, wd = (t.to(dev).requires_grad_(True) for t in (q, k, v, w))
+    md = None if mask is None else mask.to(dev)
+    with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CUDA]) as prof:
+        z, _ = F.flare_gather(qd, kd, vd, scale=0.9, key_mask=md)
+        y = F.flare_scatter(qd, kd, torch.tanh(z @ wd), scale=0.9, key_mask=md)
+        y.backward(gy.to(dev))
+        torch.cuda.synchronize()
+    kernels = " ".join(e.key for e in prof.key_averages())
+    assert "bwd_f32_tok_kernel" in kernels and "bwd_f32_delta_kernel" in kernels, kernels
+    qr, kr, vr, wr = (t.double().requires_grad_(True) for t in (q, k, v, w))
+    zr = O.gather_explicit(qr, kr, vr, 0.9, mask)
+    zr = zr[0] if isinstance(zr, tuple) else zr
+    yr = O.scatter_explicit(qr, kr, torch.tanh(zr @ wr), 0.9, mask)
+    yr.backward(gy.double())
+    for name, got, ref in (("dq", qd.grad, qr.grad), ("dk", kd.grad, kr.grad), ("dv", vd.grad, vr.grad), ("dw", wd.grad, wr.grad)):
+        err = float((got.cpu().double() - ref).norm() / ref.norm())
+        assert err <= 1e-4, f"{name} rel-L2 {err:.3e}"
+
+
 def test_lse_outputs(dev):
     q, k, v, _ = make(1, 2, 500, 64, 32, torch.bfloat16, seed=9)
     y, z, lse_lat, lse_tok = FN._mixer_forward(q.to(dev), k.to(dev), v.to(dev), 0.7, None, 0, False, False, True)
