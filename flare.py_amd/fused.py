@@ -40,14 +40,29 @@ _SUPPORTED_C = (32, 64, 128)
 _ACTS = {"gelu": 0, "silu": 1}
 
 
+def _structure_key(mod):
+    """Identity of everything the structural caches are built from: the layers, the activation module and the flags
+    that set the masks.  Assigning a new submodule (a LoRA wrap, a re-initialisation by assignment) changes it."""
+    if isinstance(mod, _SubChain):
+        return None
+    if isinstance(mod, nn.Linear) or getattr(mod, "num_layers", None) is None:
+        return (type(mod),)
+    if mod.num_layers == -1:
+        return (-1, id(mod.fc), bool(mod.residual))
+    return (mod.num_layers, id(mod.fc1), tuple(id(l) for l in mod.fcs), id(mod.fc2), id(mod.act),
+            getattr(mod.act, "approximate", None), bool(mod.input_residual), bool(mod.output_residual))
+
+
 def _layers_of(mod):
-    """(linear layers, act_mask, add_mask, act code) of a ResidualMLP or nn.Linear, or None.  The structure of a
-    module does not change after construction: the answer is kept on the module."""
+    """(linear layers, act_mask, add_mask, act code) of a ResidualMLP or nn.Linear, or None.  The answer is kept on
+    the module together with the identities of the submodules it was read from, and rebuilt when one of them is
+    replaced."""
+    key = _structure_key(mod)
     cached = mod.__dict__.get("_flare_layers")
-    if cached is not None:
+    if cached is not None and cached[1] == key:
         return cached[0]
     info = _layers_of_uncached(mod)
-    mod.__dict__["_flare_layers"] = (info,)
+    mod.__dict__["_flare_layers"] = (info, key)
     return info
 
 
@@ -109,7 +124,7 @@ class _SubChain:
     num_layers = None
 
     def __init__(self, layers, act_mask, add_mask, act, C, first, first_act, last, act_module):
-        self.__dict__["_flare_layers"] = ((layers, act_mask, add_mask, act),)
+        self.__dict__["_flare_layers"] = ((layers, act_mask, add_mask, act), None)
         self.C, self.first, self.first_act, self.last, self.act_module = C, first, first_act, last, act_module
 
 
@@ -144,9 +159,10 @@ class _NarrowLinearFn(torch.autograd.Function):
 
 def _train_subchain(mod):
     """_SubChain of a stack with a narrow end (None for every other module); kept on the module."""
-    cached = mod.__dict__.get("_flare_subchain", 0)
-    if cached != 0:
-        return cached
+    key = _structure_key(mod)
+    cached = mod.__dict__.get("_flare_subchain")
+    if cached is not None and cached[1] == key:
+        return cached[0]
     sub = None
     info = _layers_of(mod)
     if info is not None:
@@ -160,7 +176,7 @@ def _train_subchain(mod):
                 keep = (1 << n) - 1
                 sub = _SubChain(layers[lo:hi], (act_mask >> lo) & keep, (add_mask >> lo) & keep, act, Cdim,
                                 layers[0] if in_dim else None, bool(act_mask & 1), layers[-1] if out_dim else None, mod.act)
-    mod.__dict__["_flare_subchain"] = sub
+    mod.__dict__["_flare_subchain"] = (sub, key)
     return sub
 
 

@@ -2,10 +2,13 @@
  * flare_hip.h — C-ABI of libflare_hip.so, the MI355X (gfx950) FLARE attention engine.
  *
  * Plain pointers and sizes only; no torch types.  Every device pointer is owned by the
- * caller (inputs, outputs and the workspace).  The library allocates no device memory,
- * keeps no mutable global state beyond a mutex-guarded cache of occupancy queries,
- * launches asynchronously on the hipStream_t handed in (passed as void*) and never
- * synchronises the device.  All entry points return an int
+ * caller (inputs, outputs and the workspace), with one exception: flare_mixer_fwd_static
+ * works in a 64 MiB device array that is part of the library's code object, so every
+ * process that loads the library holds those 64 MiB on each GPU it uses, whether or not it
+ * calls that entry point.  The library calls no allocator (hipMalloc, hipFree), keeps no
+ * mutable host state beyond a mutex-guarded cache of occupancy queries and of that array's
+ * per-device address, launches asynchronously on the hipStream_t handed in (passed as
+ * void*) and never synchronises the device.  All entry points return an int
  * status (0 = OK, negative = error); the text of the last error on the calling thread is
  * available from flare_last_error_string().  Shapes, dtypes, strides, alignment and the
  * workspace size are validated on the host BEFORE anything is launched.
@@ -258,7 +261,12 @@ int flare_mixer_fwd_dropout(const FlareMixerDesc* desc, const void* q, const voi
  * (one copy per GPU, held until the process ends); the call allocates and frees nothing.  A problem whose
  * flare_mixer_workspace_bytes() exceeds that size is rejected with FLARE_EWORKSPACE before anything is
  * launched.  All calls on one GPU share the buffer: calls that overlap in time on the same GPU (different
- * streams or threads) race and must be serialised by the caller.  Results are those of flare_mixer_fwd. */
+ * streams or threads) race and must be serialised by the caller.  Results are those of flare_mixer_fwd.
+ * Cost: the array is device memory of every process that has loaded the library, on every GPU that process
+ * touches (16 processes sharing a GPU hold 1 GiB between them).  The first call on a device looks the
+ * array's address up (hipGetSymbolAddress, which may load the code object): make that first call, with any
+ * small problem, BEFORE a stream capture begins, since a lookup during capture can be refused; later calls
+ * only launch kernels and may be captured. */
 #define FLARE_STATIC_SCRATCH_BYTES (64u << 20)
 int flare_mixer_fwd_static(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
                            const uint8_t* key_mask, void* y, void* stream);

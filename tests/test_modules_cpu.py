@@ -162,3 +162,24 @@ def test_rotary_embedding_module_against_oracle():
     assert O.rel_l2(rope(k.bfloat16()).float(), O.rope_reference(k.bfloat16().float())) <= 2e-2
     with pytest.raises(AssertionError):
         rope(torch.randn(1, 1, 65, 16))
+
+
+def test_fused_structure_cache_follows_replaced_submodules():
+    """The layer list the fused path keeps on a module is rebuilt when a submodule or the activation is replaced
+    after the first look (a LoRA wrap, a re-initialisation by assignment)."""
+    from torch import nn
+    from flare_py_amd import fused
+    from flare_py_amd.modules import ResidualMLP
+    mlp = ResidualMLP(3, 32, 32, num_layers=2, act="gelu")
+    first = fused._layers_of(mlp)
+    assert first is fused._layers_of(mlp)                      # cached while nothing changes
+    sub = fused._train_subchain(mlp)
+    assert sub is not None and sub.first is mlp.fc1 and sub is fused._train_subchain(mlp)
+    mlp.fcs[0] = nn.Linear(32, 32)
+    again = fused._layers_of(mlp)
+    assert again is not first and again[0][1] is mlp.fcs[0]
+    assert fused._layers_of(fused._train_subchain(mlp))[0][0] is mlp.fcs[0]
+    mlp.fc1 = nn.Linear(3, 32)
+    assert fused._train_subchain(mlp).first is mlp.fc1
+    mlp.act = nn.ReLU()                                        # an activation the kernels do not have
+    assert fused._layers_of(mlp) is None and fused._train_subchain(mlp) is None

@@ -64,3 +64,49 @@ def test_static_scratch_equals_workspace_entry_point_twice(dev, dtype):
         want, _ = O.mixer_explicit(q.double().cpu(), k.double().cpu(), v.double().cpu(), 1.0)
         err = (y_new.double().cpu() - want).norm() / want.norm()
         assert err <= (1e-5 if dtype == _lib.DT_F32 else 2e-2), err
+
+
+@pytest.mark.gpu
+def test_static_scratch_with_key_mask_and_replayed_from_a_graph_on_dirty_scratch(dev):
+    """A masked problem through the static scratch, first eagerly, then replayed from a captured graph after other
+    problems have left their partials in the scratch: every replay equals the caller-workspace entry point."""
+    lib = _lib.load()
+    B, H, N, M, D = 2, 2, 3000, 64, 32
+    g = torch.Generator().manual_seed(5)
+    q = (torch.randn(H, M, D, generator=g) * D ** -0.5).bfloat16().to(dev)
+    k = torch.randn(B, H, N, D, generator=g).bfloat16().to(dev)
+    v = torch.randn(B, H, N, D, generator=g).bfloat16().to(dev)
+    mask = (torch.rand(B, N, generator=g) > 0.3).to(torch.uint8)
+    mask[1, 1000:] = 0
+    mask = mask.to(dev)
+    d = _desc(B, H, N, M, D)
+    n = C.c_size_t(0)
+    assert lib.flare_mixer_workspace_bytes(C.byref(d), C.byref(n)) == 0 and n.value <= _lib.STATIC_SCRATCH_BYTES
+    ws = torch.empty(n.value, dtype=torch.uint8, device=dev)
+    y_ref = torch.empty_like(k)
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.flare_mixer_fwd(C.byref(d), q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), y_ref.data_ptr(), None,
+                               ws.data_ptr(), n.value, st) == 0, _lib.last_error()
+    y = torch.full_like(k, float("nan"))
+    # the first call on the device (it resolves the scratch address) happens before any capture
+    assert lib.flare_mixer_fwd_static(C.byref(d), q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), y.data_ptr(), st) == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_ref)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = lib.flare_mixer_fwd_static(C.byref(d), q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), y.data_ptr(),
+                                            torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _lib.last_error()
+    torch.cuda.current_stream().wait_stream(side)
+    for i in range(3):
+        print(f"static scratch graph replay {i}", flush=True)
+        # another problem dirties the scratch between replays (eager work on the same scratch)
+        _both(lib, dev, 1, 2 + i, 5000 + 100 * i, 128, 32, _lib.DT_BF16, seed=30 + i)
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, y_ref), i
