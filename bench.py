@@ -183,6 +183,12 @@ def bench_causal(args, F, dev):
                                        out=y_steps[:, :, t:t + 1])
 
     ms_tok = time_events(token_steps, max(2, args.steps // 10), 2)
+    # host share of a separate call: the time the 256 calls take to return (argument checks, ctypes, one launch each)
+    torch.cuda.synchronize(dev)
+    t0 = time.perf_counter()
+    token_steps()
+    us_host = (time.perf_counter() - t0) / ND * 1e6
+    torch.cuda.synchronize(dev)
     side = torch.cuda.Stream(device=dev)
     side.wait_stream(torch.cuda.current_stream(dev))
     with torch.cuda.stream(side):
@@ -194,6 +200,22 @@ def bench_causal(args, F, dev):
     ms_tok_graph = time_events(graph.replay, max(2, args.steps // 5), 2)
     out["roofline"]["us_per_decode_step_separate_calls"] = round(ms_tok / ND * 1e3, 3)
     out["roofline"]["us_per_decode_step_graph_replay"] = round(ms_tok_graph / ND * 1e3, 3)
+    out["roofline"]["us_host_per_separate_call"] = round(us_host, 3)
+    # what a chain of 256 dependent graph nodes costs on this machine when each node does next to nothing
+    # (a one-element add): the floor under the per-step figure above
+    one = torch.zeros(1, device=dev)
+
+    def tiny_nodes():
+        for _ in range(ND):
+            one.add_(1.0)
+
+    with torch.cuda.stream(side):
+        tiny_nodes()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    tiny_graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(tiny_graph):
+        tiny_nodes()
+    out["roofline"]["us_per_graph_node_one_element_add"] = round(time_events(tiny_graph.replay, max(2, args.steps // 5), 2) / ND * 1e3, 3)
     # a latent count that runs as two groups of 128 joined by their softmax sums (256 latents with D = 64)
     q2 = torch.cat([q, q.flip(1)], dim=1)
     ms_prefill_256 = time_events(lambda: F.flare_causal_prefill(q2, kp, vp), max(2, args.steps // 5), 2)

@@ -765,6 +765,7 @@ int causal_run(const FlareCausalDesc* desc, bool decode, const void* q, const vo
         a.seg_num = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + p.off_num);
         hipError_t e = flare::launch_causal_mfma(a, desc->dtype, decode ? 1 : 16, st);
         if (e != hipSuccess) return hip_status(e, "causal (mfma) launch");
+        if (decode) return FLARE_OK;      // the decode kernel redoes what it cannot validate itself: one launch
     }
     hipError_t e = decode ? flare::launch_causal_decode(a, desc->dtype, st) : flare::launch_causal_prefill(a, desc->dtype, st);
     return hip_status(e, decode ? "causal decode launch" : "causal prefill launch");

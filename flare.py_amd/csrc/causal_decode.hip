@@ -12,7 +12,8 @@
 //                 lane's ML = MW * D / 64 latents, plus sum_m W_m.
 // The eight partial output rows and weight sums meet in LDS (double buffered: one barrier per step); the waves
 // take turns to divide, validate (sum of weights inside 2^-60..2^120, finite output) and stores the row.  A (b,h) that
-// fails validation leaves its state untouched and raises its flag for the fp32 kernel of causal.hip.
+// fails validation has left its state untouched: its workgroup repeats the steps on the spot with a running maximum
+// per latent (the exact path at the end of the kernel), so a call is one launch whatever the scores are.
 #include <type_traits>
 
 #include "common.hpp"
@@ -76,7 +77,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void causal_decode_kernel(CausalArg
 
     __shared__ __attribute__((aligned(16))) float pgw[NW][MW][4];   // P, G, W of the wave's latents (one 16-byte read each)
     __shared__ float ypart[2][NW][D];
-    __shared__ float rpart[2][NW];
+    __shared__ float rpart[4][NW];      // [2][NW] partial weight sums; the exact path keeps each step's largest score per wave behind them
     __shared__ int bad_flag;
 
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
@@ -214,10 +215,89 @@ __global__ __launch_bounds__(64 * kDecWaves) void causal_decode_kernel(CausalArg
     if (__any(bad) && lane == 0) bad_flag = 1;
     __syncthreads();
     if (bad_flag) {
-        if (tid == 0) a.flags[bh] = 1;
+        // Exact path, in the same launch: the workgroup repeats all N steps from the incoming state (nothing of it has
+        // been overwritten) with a running maximum per latent, scores in fp32 from the unrounded latents, and the
+        // softmax over the latents shifted by each step's own largest score.  Same two lane maps; the step's largest
+        // score crosses the waves through LDS, which costs a second barrier per step.
+        float* cmax = &rpart[0][0] + 2 * NW;      // [2][NW], behind rpart (declared below as one array of 4 NW floats)
+        float qf[DS];
+        {
+            const uint16_t* qr = q + (int64_t)m_s * a.qs[2] + dp * DS;
+#pragma unroll
+            for (int j = 0; j < DS; ++j) qf[j] = E::unpack(qr[j]);
+        }
+        float mu2 = fresh ? kNegBig : mu_in * kLog2e;
+        den = fresh ? 0.f : den_in;
+        {
+            float mu_j[ML];
+#pragma unroll
+            for (int j = 0; j < ML; ++j) {
+                const int m = w * MW + mp * ML + j;
+                mu_j[j] = mu_g[m];
+                U[j] = num_g[(int64_t)m * D + d];
+            }
+#pragma unroll
+            for (int j = 0; j < ML; ++j) U[j] = mu_j[j] <= kNegBig ? 0.f : U[j];
+        }
+        for (int n = 0; n < N; ++n) {
+            const int buf = n & 1;
+            const uint16_t* kr = k + (int64_t)n * a.ks[2] + dp * DS;
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < DS; ++j) s = fmaf(qf[j], E::unpack(kr[j]), s);
+            if constexpr (MW == 16) s = sum_xor16(s);
+            s = sum_xor32(s) * sl2;
+            const float mun = fmaxf(mu2, s);
+            const float al = fast_exp2(mu2 - mun), p = fast_exp2(s - mun);
+            den = fmaf(al, den, p);
+            mu2 = mun;
+            float cm = s;
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) cm = fmaxf(cm, __shfl_xor(cm, o));
+            if (lane == 0) cmax[buf * NW + w] = cm;
+            asm volatile("" ::: "memory");
+            if (score_lane) *reinterpret_cast<f32x4*>(&pgw[w][ms][0]) = f32x4{al, p, s, 1.f / den};
+            asm volatile("" ::: "memory");
+            __syncthreads();
+            float c = cmax[buf * NW];
+#pragma unroll
+            for (int i = 1; i < NW; ++i) c = fmaxf(c, cmax[buf * NW + i]);
+            const float vd = E::unpack(v[(int64_t)n * a.vs[2] + d]);
+            float acc = 0.f, rw = 0.f;
+#pragma unroll
+            for (int j = 0; j < ML; ++j) {
+                const f32x4 t = *reinterpret_cast<const f32x4*>(&pgw[w][mp * ML + j][0]);
+                U[j] = fmaf(t[1], vd, t[0] * U[j]);
+                const float wgt = fast_exp2(t[2] - c);
+                acc = fmaf(wgt * t[3], U[j], acc);
+                rw += wgt;
+            }
+            if constexpr (NP == 2) {
+                acc = sum_xor32(acc);
+                rw = sum_xor32(rw);
+            }
+            if (mp == 0) ypart[buf][w][d] = acc;
+            if (lane == 0) rpart[buf][w] = rw;
+            __syncthreads();
+            if (w == (n & (NW - 1)) && lane < D) {
+                float ys = 0.f, r = 0.f;
+#pragma unroll
+                for (int i = 0; i < NW; ++i) {
+                    ys += ypart[buf][i][lane];
+                    r += rpart[buf][i];
+                }
+                y[(int64_t)n * a.ys[2] + lane] = E::bits(ys / r);
+                if (a.lse && lane == 0) a.lse[(int64_t)bh * N + n] = (c + __log2f(r)) * kLn2;
+            }
+        }
+        if (score_lane) {
+            mu_g[m_s] = mu2 * kLn2;
+            den_g[m_s] = den;
+        }
+#pragma unroll
+        for (int j = 0; j < ML; ++j) num_g[(int64_t)(w * MW + mp * ML + j) * D + d] = U[j];
         return;
     }
-    if (tid == 0) a.flags[bh] = 0;
     if (score_lane) {
         mu_g[m_s] = mu0 * kLn2;
         den_g[m_s] = den;

@@ -483,3 +483,33 @@ def test_decode_steps_replay_from_a_hip_graph(dev):
         for a, b in zip(st, st_all):
             assert torch.equal(a, b)
         F.flare_causal_prefill(qd, kp, vp)               # eager work between replays
+
+
+@pytest.mark.parametrize("M,D", [(128, 64), (256, 32)])
+def test_decode_steps_outside_the_window_are_redone_in_the_same_launch(dev, M, D):
+    """Decode steps whose scores leave the window in which the kernel may skip the running maximum: the workgroup of
+    that (b,h) repeats the call's steps with a running maximum inside the same launch (fp32 scores, so what is left is
+    the rounding of the 16-bit output); the other head stays on the fast path.  Then both continue from the states
+    those calls left, back inside the window."""
+    q, k, v = make(1, 2, 90, M, D, torch.bfloat16, seed=9, std=1.0)
+    k[:, 0, :60] *= 8.0                   # head 0: |score| up to several hundred during the first call
+    k[:, 0, 60:] *= 0.05
+    k[:, 1] *= 0.05
+    s = torch.einsum("hmd,bhnd->bhmn", q.float(), k.float())
+    assert float(s[:, 0, :, :60].abs().max()) > 150 and float(s[:, 1].abs().max()) < 20
+    yr, str_ = O.causal_recurrent(q.float(), k.float(), v.float())
+    st = F.causal_fresh_state(1, 2, M, D, dev)
+    y1, st = F.flare_causal_decode(q.to(dev), k[:, :, :60].to(dev), v[:, :, :60].to(dev), st)
+    y2, st = F.flare_causal_decode(q.to(dev), k[:, :, 60:].to(dev), v[:, :, 60:].to(dev), st)
+    y = torch.cat([y1, y2], 2)
+    assert torch.isfinite(y.float()).all()
+    assert O.rel_l2(y[:, 0, :60], yr[:, 0, :60]) <= 1e-2 and O.rel_l2(y[:, 1], yr[:, 1]) <= 2e-2
+    assert O.rel_l2(y[:, 0, 60:], yr[:, 0, 60:]) <= 2e-2
+    state_close(st, str_, 2e-2)
+    # one step at a time through the same path gives the same rows to rounding
+    st1 = F.causal_fresh_state(1, 2, M, D, dev)
+    rows = []
+    for t in range(8):
+        yt, st1 = F.flare_causal_decode(q.to(dev), k[:, :, t:t + 1].to(dev), v[:, :, t:t + 1].to(dev), st1)
+        rows.append(yt)
+    assert O.rel_l2(torch.cat(rows, 2)[:, 0], yr[:, 0, :8]) <= 1e-2

@@ -154,3 +154,30 @@ def test_fp32_head_dims_16_and_32_on_the_matrix_cores(dev, shape, fm, nz, D):
         st3, out3 = F.triple_attention(*[p[..., 1:] for p in pad], normalize=nz, feature_map=fm)
         torch.cuda.synchronize()
     assert O.rel_l2(out3, orf) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype,eps", [(torch.bfloat16, 2.0 ** -8), (torch.float16, 2.0 ** -10)])
+@pytest.mark.parametrize("N", [1, 2])
+@pytest.mark.parametrize("Dq,Dv", [(32, 16), (16, 16), (32, 32), (64, 16)])
+def test_16bit_kernels_with_one_or_two_tokens_against_the_conditioning_bound(dev, dtype, eps, N, Dq, Dv):
+    """Signed features and one or two tokens: out[n,j] = sum_ik q1_i state_ijk q2_k is then (q1.k1)(q2.k2) v_j (a sum of
+    two such products for N = 2), a sum of Dq^2 signed terms that mostly cancel, so its error relative to |out| says
+    nothing about the kernel.  What the 16-bit kernels can promise is an error that is small against the sum of the
+    terms' magnitudes: each term carries a few roundings to the element type (the products k1 k2 and q1 q2, the state
+    as a matrix operand) and the output is rounded once.  Checked element by element."""
+    for seed in range(4):
+        a = make(1, 2, N, Dq, Dv, dtype, seed=100 * N + seed)
+        st, out = F.triple_attention(*[t.to(dev) for t in a])
+        q1, q2, k1, k2, v = (t.double() for t in a)
+        sr, orf = O.triple_einsum(q1, q2, k1, k2, v, dtype=torch.float64)
+        mag_state = torch.einsum("bhni,bhnj,bhnk->bhijk", k1.abs(), v.abs(), k2.abs()) / N
+        mag = torch.einsum("bhni,bhijk,bhnk->bhnj", q1.abs(), mag_state, q2.abs())
+        err = (out.double().cpu() - orf).abs()
+        worst = float((err / mag).max())
+        assert worst <= eps, (seed, worst, eps, float(mag.norm() / orf.norm()))
+        # the state itself has no cancellation with one token (one term per entry) and little with two.  The kernel
+        # rounds each product k1[n,i] k2[n,k] to the element type: in f16 a product below 2^-14 is subnormal and
+        # carries an absolute error of up to 2^-25, which then meets |v[n,j]|
+        sub = (2.0 ** -24 * v.abs().mean(2))[:, :, None, :, None] if dtype == torch.float16 else 0.0
+        excess = (st.double().cpu() - sr).abs() - 2 * eps * mag_state - sub
+        assert float(excess.max()) <= 0.0, float(excess.max())
