@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FLARE mixer forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block|train|linear|fp32]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block|train|linear|fp32|layer|lra]
 
 One step = one forward of the mixer (split-N gather, merge, scatter) over the headline workload
 B=1, H=8, N=1,048,576, M=256, D=32, bf16 in / fp32 accumulate, inputs resident in HBM.
@@ -378,6 +378,66 @@ def bench_fp32(args, F, dev):
     return out
 
 
+def bench_lra(args, F, dev):
+    """Training step of one sequence-benchmark FLARE block with and without attention dropout (out/lra/run.sh of the
+    reference: channel_dim 128, 8 heads, 128 latents, 3-layer k/v projections and feed-forward, batch 32, fp32
+    ("--mixed_precision false"), attn_drop 0.1 on pathfinder32 / listops / text)."""
+    from flare_py_amd import lra_modules
+
+    C_, H, M, B = 128, 8, 128, 32
+    rows = {}
+    for name, N, ragged in (("pathfinder32 (N=1024, no padding)", 1024, False), ("text (N=4096, padded)", 4096, True)):
+        torch.manual_seed(0)
+        x = torch.randn(B, N, C_, device=dev)
+        mask = None
+        if ragged:
+            lens = torch.randint(N // 4, N + 1, (B,), generator=torch.Generator().manual_seed(1))
+            mask = (torch.arange(N)[None, :] < lens[:, None]).to(dev)
+        row = {}
+        for dtype_name, ac in (("fp32", None), ("bf16_autocast", torch.bfloat16)):
+            for p_drop in (0.0, 0.1):
+                torch.manual_seed(0)
+                blk = lra_modules.FLAREBlock(channel_dim=C_, num_heads=H, num_latents=M, num_layers_kv_proj=3, num_layers_ffn=3,
+                                             kv_proj_hidden_dim=C_, ffn_hidden_dim=C_, attn_drop=p_drop).to(dev).train()
+                xg = x.clone().requires_grad_(True)
+
+                def step():
+                    if ac is None:
+                        y = blk(xg, mask)
+                    else:
+                        with torch.autocast("cuda", dtype=ac):
+                            y = blk(xg, mask)
+                    y.float().square().mean().backward()
+                    xg.grad = None
+                    for prm in blk.parameters():
+                        prm.grad = None
+
+                row[f"ms_fwd_bwd_{dtype_name}_attn_drop_{p_drop}"] = round(time_events(step, max(5, args.steps // 5), 3), 3)
+            row[f"ratio_{dtype_name}"] = round(row[f"ms_fwd_bwd_{dtype_name}_attn_drop_0.1"] / row[f"ms_fwd_bwd_{dtype_name}_attn_drop_0.0"], 3)
+        rows[name] = row
+    head = rows["pathfinder32 (N=1024, no padding)"]
+    ms = head["ms_fwd_bwd_fp32_attn_drop_0.1"]
+    out = base_record(args, "sequence-benchmark FLARE block training step tokens/sec, attn_drop=0.1, B=32,N=1024,C=128,H=8,M=128 fp32",
+                      B * 1024 / (ms * 1e-3), "tokens/s", ms,
+                      "one lra FLAREBlock (norm, 3-layer k/v projections, mixer with attention dropout 0.1, out_proj, 3-layer FFN), forward + backward, fp32")
+    out["dtype"] = "f32"
+    out["roofline"] = None
+    out["blocks"] = rows
+    # what the keep mask costs where the mixer is all there is: the headline shape, forward only
+    q, k, v = make_inputs(1, 8, 1 << 20, 256, 32, torch.bfloat16, dev)
+    out["headline_shape_forward_ms"] = {
+        "no_dropout": round(time_events(lambda: F.flare_multihead_mixer(q, k, v), 20, 3), 3),
+        "no_dropout_16x16x32_kernels": round(time_events(lambda: _mfma16(F, q, k, v), 20, 3), 3),
+        "dropout_0.1": round(time_events(lambda: F.flare_multihead_mixer(q, k, v, dropout_p=0.1, dropout_seed=1), 10, 2), 3)}
+    return out
+
+
+def _mfma16(F, q, k, v):
+    from flare_py_amd import _lib, functional
+    with functional.mixer_flags(_lib.FLAG_MFMA16):
+        return F.flare_multihead_mixer(q, k, v)
+
+
 def bench_train(args, F, dev):
     """Headline configuration, forward + backward of the mixer (HIP kernels both ways)."""
     B, H, N, M, D = 1, 8, 1 << 20, 256, 32
@@ -682,7 +742,7 @@ def main():
     ap.add_argument("--no-torch-sdpa", action="store_true", help="skip the legs that time torch's own formulation (fused SDPA, einsum, torch layers) on the GPU")
     ap.add_argument("--lengths", default="1000000,100000", help="layer workload: token counts (the first one is the headline of the line)")
     ap.add_argument("--latents", default="128,512,2048", help="layer workload: latent counts")
-    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train", "linear", "fp32", "layer"], default="mixer",
+    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train", "linear", "fp32", "layer", "lra"], default="mixer",
                     help="mixer = the headline configuration (default); the others are BASELINE configs 4, 5, 2")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -698,7 +758,7 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload != "mixer":
         fn = {"causal": bench_causal, "triple": bench_triple, "block": bench_block, "train": bench_train,
-              "linear": bench_linear, "fp32": bench_fp32, "layer": bench_layer}[args.workload]
+              "linear": bench_linear, "fp32": bench_fp32, "layer": bench_layer, "lra": bench_lra}[args.workload]
         print(json.dumps(fn(args, F, dev)))
         return
     B, H, N, M, D = 1, 8, 1 << 20, 256, 32

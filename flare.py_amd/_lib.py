@@ -18,7 +18,7 @@ FLAG_FORCE_GENERIC = 1
 FLAG_MFMA16 = 2
 FLAG_GRAD_LIKE_KV = 8
 MLP_EXPAND = 1
-ABI_VERSION = 1
+ABI_VERSION = 2
 STATIC_SCRATCH_BYTES = 64 << 20
 
 I3 = C.c_int64 * 3
@@ -30,6 +30,7 @@ class FlareMixerDesc(C.Structure):
         ("dtype", C.c_int32), ("scale", C.c_float), ("n_splits", C.c_int32), ("flags", C.c_int32),
         ("reserved", C.c_int32),
         ("q_stride", I3), ("k_stride", I3), ("v_stride", I3), ("y_stride", I3),
+        ("dropout_p", C.c_float), ("reserved2", C.c_int32), ("dropout_seed", C.c_uint64),
     ]
 
 

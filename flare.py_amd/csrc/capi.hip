@@ -64,6 +64,7 @@ int check_mixer_desc(const FlareMixerDesc* d)
     if (d->D > 128) return fail(FLARE_EUNSUPPORTED, "head dim D=%d > 128 is not supported", d->D);
     if (d->H > 65535 || d->B > 65535) return fail(FLARE_EUNSUPPORTED, "B and H must be <= 65535");
     if (d->n_splits < 0) return fail(FLARE_EINVAL, "n_splits must be >= 0");
+    if (!(d->dropout_p >= 0.f) || !(d->dropout_p < 1.f)) return fail(FLARE_EINVAL, "dropout_p must be in [0, 1) (got %g)", (double)d->dropout_p);
     const int64_t* ss[4] = {d->q_stride, d->k_stride, d->v_stride, d->y_stride};
     const char* nm[4] = {"q", "k", "v", "y"};
     for (int t = 0; t < 4; ++t) {
@@ -83,6 +84,10 @@ bool mixer_ptrs_ok_for_mfma(const FlareMixerDesc* d, const void* q, const void* 
            strides_mult8(d->y_stride);
 }
 
+// 24-bit threshold of the keep/drop hash: an entry is dropped when its hash is below it.  0 = no dropout (also for a
+// dropout_p below 2^-24, which keeps every weight and rescales nothing).
+uint32_t drop_threshold(const FlareMixerDesc* d) { return (uint32_t)((double)d->dropout_p * 16777216.0); }
+
 // The plan depends on the descriptor only (never on pointer values) so that the workspace
 // query and the launch always agree.  Misaligned pointers demote to the generic kernels,
 // whose partial count (4 per workgroup) is covered by sizing for the larger of the two.
@@ -90,7 +95,7 @@ MixerPlan plan_mixer(const FlareMixerDesc* d, bool want_mfma)
 {
     MixerPlan p;
     p.mfma = want_mfma;
-    const bool allow32 = !(d->flags & FLARE_FLAG_MFMA16);
+    const bool allow32 = !(d->flags & FLARE_FLAG_MFMA16) && drop_threshold(d) == 0;     // the 32x32x16 kernels carry no dropout
     const int unit = p.mfma ? flare::mfma_gather_tokens_per_iter(d->dtype, d->M, d->D, allow32) : 32;
     const int mblk = p.mfma ? ((d->M % 256 == 0 && d->D <= 32) ? d->M / 256 : (d->M % 128 == 0) ? d->M / 128 : (d->M + 63) / 64)
                             : (d->M + 63) / 64;
@@ -145,6 +150,14 @@ void fill_mixer_args(flare::MixerArgs& a, const FlareMixerDesc* d, const MixerPl
     a.scale_log2 = d->scale * flare::kLog2e;
     a.no_mfma32 = (d->flags & FLARE_FLAG_MFMA16) ? 1 : 0;
     a.force_fma = (d->flags & FLARE_FLAG_FORCE_GENERIC) ? 1 : 0;
+    a.drop_thr = drop_threshold(d);
+    a.drop_rs = 1.f;
+    if (a.drop_thr != 0) {
+        a.no_mfma32 = 1;
+        a.drop_rs = 1.0f / (1.0f - d->dropout_p);
+        a.seed_lo = (uint32_t)(d->dropout_seed & 0xffffffffu);
+        a.seed_hi = (uint32_t)(d->dropout_seed >> 32);
+    }
     for (int i = 0; i < 3; ++i) {
         a.qs[i] = d->q_stride[i]; a.ks[i] = d->k_stride[i]; a.vs[i] = d->v_stride[i]; a.ys[i] = d->y_stride[i];
     }
@@ -528,6 +541,13 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
     a.n_splits = p.n_splits; a.tokens_per_split = p.tokens_per_split;
     a.n_splits0 = p.n_splits0; a.tokens_per_split0 = p.tokens_per_split0;
     a.scale = desc->scale; a.scale_log2 = desc->scale * 1.4426950408889634f;
+    a.drop_thr = drop_threshold(desc);
+    a.drop_rs = 1.f;
+    if (a.drop_thr != 0) {
+        a.drop_rs = 1.0f / (1.0f - desc->dropout_p);
+        a.seed_lo = (uint32_t)(desc->dropout_seed & 0xffffffffu);
+        a.seed_hi = (uint32_t)(desc->dropout_seed >> 32);
+    }
     const int64_t nd = (int64_t)desc->N * desc->D;
     for (int i = 0; i < 3; ++i) {
         a.qs[i] = desc->q_stride[i]; a.ks[i] = desc->k_stride[i]; a.vs[i] = desc->v_stride[i];
@@ -562,6 +582,13 @@ int half_bwd_args(flare::MixerBwdArgs& a, const FlareMixerDesc* desc, void* work
     a.n_splits = p.n_splits; a.tokens_per_split = p.tokens_per_split;
     a.n_splits0 = p.n_splits0; a.tokens_per_split0 = p.tokens_per_split0;
     a.scale = desc->scale; a.scale_log2 = desc->scale * 1.4426950408889634f;
+    a.drop_thr = drop_threshold(desc);
+    a.drop_rs = 1.f;
+    if (a.drop_thr != 0) {
+        a.drop_rs = 1.0f / (1.0f - desc->dropout_p);
+        a.seed_lo = (uint32_t)(desc->dropout_seed & 0xffffffffu);
+        a.seed_hi = (uint32_t)(desc->dropout_seed >> 32);
+    }
     const int64_t nd = (int64_t)desc->N * desc->D;
     for (int i = 0; i < 3; ++i) {
         a.qs[i] = desc->q_stride[i]; a.ks[i] = desc->k_stride[i]; a.vs[i] = desc->v_stride[i]; a.ys[i] = desc->y_stride[i];
@@ -672,30 +699,11 @@ int flare_mixer_fwd_dropout(const FlareMixerDesc* desc, const void* q, const voi
                             const uint8_t* key_mask, float dropout_p, uint64_t seed, void* y, float* z_out,
                             void* workspace, size_t workspace_bytes, void* stream)
 {
-    int rc = check_mixer_desc(desc);
-    if (rc != FLARE_OK) return rc;
-    if (!q || !k || !v || !y) return fail(FLARE_EINVAL, "q, k, v, y must not be NULL");
-    if (!(dropout_p >= 0.f) || !(dropout_p < 1.f)) return fail(FLARE_EINVAL, "dropout_p must be in [0, 1) (got %g)", (double)dropout_p);
-    if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
-    if (!aligned16(workspace)) return fail(FLARE_EINVAL, "workspace must be 16-byte aligned");
-    const size_t need = mixer_ws_bytes(desc);
-    if (workspace_bytes < need) return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, need);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    // the fp32-FMA kernels carry the dropout; the plan is the generic one whatever the shape
-    const MixerPlan p = plan_mixer(desc, false);
-    flare::MixerArgs a;
-    fill_mixer_args(a, desc, p, workspace);
-    float* z = z_out ? z_out : reinterpret_cast<float*>(static_cast<char*>(workspace) + p.off_z);
-    a.q = q; a.k = k; a.v = v; a.y = y; a.mask = key_mask; a.z = z;
-    a.drop_thr = (uint32_t)((double)dropout_p * 16777216.0);
-    a.drop_rs = 1.0f / (1.0f - dropout_p);
-    a.seed_lo = (uint32_t)(seed & 0xffffffffu);
-    a.seed_hi = (uint32_t)(seed >> 32);
-    hipError_t e = flare::launch_gather_generic(a, desc->dtype, st);
-    if (e != hipSuccess) return hip_status(e, "gather launch");
-    e = flare::launch_gather_merge(a, st);
-    if (e != hipSuccess) return hip_status(e, "gather merge launch");
-    return hip_status(flare::launch_scatter_generic(a, desc->dtype, st), "scatter launch");
+    if (!desc) return fail(FLARE_EINVAL, "descriptor is NULL");
+    FlareMixerDesc d = *desc;
+    d.dropout_p = dropout_p;
+    d.dropout_seed = seed;
+    return flare_mixer_fwd(&d, q, k, v, key_mask, y, z_out, workspace, workspace_bytes, stream);
 }
 
 int flare_mixer_fwd_static(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,

@@ -72,6 +72,13 @@ __host__ __device__ __forceinline__ uint32_t dropout_hash24(uint32_t seed_lo, ui
     return lowbias32(lowbias32(x) ^ seed_hi) >> 8;
 }
 
+// Factor an entry of the softmax weights meets under attention dropout: 1 / (1 - p) if it is kept, 0 if not.
+__device__ __forceinline__ float dropout_factor(uint32_t thr, float rs, uint32_t seed_lo, uint32_t seed_hi, uint32_t phase,
+                                                uint32_t bh, uint32_t m, uint32_t n)
+{
+    return dropout_hash24(seed_lo, seed_hi, phase, bh, m, n) >= thr ? rs : 0.f;
+}
+
 // ---- kernel argument blocks (host fills them; passed by value) -------------------------
 struct MixerArgs {
     const void* q; const void* k; const void* v; void* y;
@@ -89,7 +96,7 @@ struct MixerArgs {
     float scale_log2;         // scale * log2(e)
     int no_mfma32;            // 1: keep the 16x16x32 kernels where the 32x32x16 ones would run
     int force_fma;            // 1: fp32 problems keep the FMA kernels (no fp32 matrix-core kernels)
-    // attention dropout (fp32-FMA kernels only): an entry of the softmax weights is kept when its hash is >= drop_thr
+    // attention dropout (not in the 32x32x16 kernels): an entry of the softmax weights is kept when its hash is >= drop_thr
     // (24-bit compare) and then scaled by drop_rs = 1 / (1 - p); drop_thr == 0 switches it off
     uint32_t drop_thr, seed_lo, seed_hi;
     float drop_rs;
@@ -184,6 +191,9 @@ struct MixerBwdArgs {
     int scal_lds;            // token-side kernel only: per-latent scalars are tabled in LDS behind the operand sets
     int half;                // fp32 kernels: 0 = whole mixer, 1 = gather half only (dz given, no scatter term), 2 = scatter half only
                              // (no gather term, dv not written; dz is an output)
+    // attention dropout of the forward this is the backward of (same fields as MixerArgs; drop_thr == 0: none)
+    uint32_t drop_thr, seed_lo, seed_hi;
+    float drop_rs;
 };
 
 struct CausalLinearArgs {

@@ -14,6 +14,9 @@
 //   dq pass   (latent side, split over N)  dq partials                      -> merge: dq
 // The halves called separately (models with layers between them) run the same kernels with one term of dS dropped:
 // the gather half takes dz from the caller, the scatter half returns it.
+// Attention dropout of the forward (MixerBwdArgs::drop_thr != 0): its keep masks are regenerated from the same hash; with
+// K the keep factors (0 or 1 / (1 - p)) the weights the forward used were K A and K B, so dz and dv meet K B and K A,
+// and dS = A (K <dz, v> - Delta) + B (K <dy, z> - delta) with the same Delta and delta (they are sums over kept weights).
 // Every sum has a fixed order: two runs give the same bits.  A key mask needs nothing here: the caller zeroes the
 // padded tokens' rows and raises their log-sum-exp, so that their weights vanish.
 #include <algorithm>
@@ -55,7 +58,7 @@ template <int Q4> __device__ __forceinline__ f32x4 dot_rows(const f32x4 (&a)[Q4]
 // waves' sums meet in LDS and the workgroup writes one partial [64][D].
 // MODE 0: dz_m += B[n,m] dy_n (values = dY), and delta_n = <dy_n, y_n> from the first latent block.
 // MODE 1: dq_m += dS[m,n] k_n (values = K), dS assembled from three score-like products.
-template <int D, int MODE, int HALF>
+template <int D, int MODE, int HALF, bool DROP>
 __global__ __launch_bounds__(256, (D == 64 && MODE == 1) ? 1 : 2) void bwd_f32_lat_kernel(MixerBwdArgs a)
 {
     constexpr int QL = D / 4, Q4 = QL / 4, RT = D / 16, VS = D + 4, VPT = D / 16;
@@ -77,6 +80,7 @@ __global__ __launch_bounds__(256, (D == 64 && MODE == 1) ? 1 : 2) void bwd_f32_l
     const int tps = MODE == 0 ? a.tokens_per_split0 : a.tokens_per_split;
     const int n_parts = MODE == 0 ? a.n_splits0 : a.n_splits;
     constexpr bool use_a = HALF != 2, use_b = HALF != 1;      // gather term, scatter term of dS
+    constexpr bool drop = DROP;                               // the forward dropped weights: the same masks are regenerated here
 
     // latent operands (B of the score-like products): q log2-scaled; for the dq pass also dz and z with their scalars
     f32x4 qb[CT][Q4], dzb[MODE ? CT : 1][Q4], zb[MODE ? CT : 1][Q4];
@@ -181,12 +185,29 @@ __global__ __launch_bounds__(256, (D == 64 && MODE == 1) ? 1 : 2) void bwd_f32_l
             // lane = latent column c16, rows = tokens 4g + r
             const f32x4 s = dot_rows<Q4>(kc, qb[ct]);
             float p[4];
+            const uint32_t m_lat = (uint32_t)(mb * MB + 16 * ct + c16);
             if constexpr (MODE == 0) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) p[r] = valid[r] ? fast_exp2(s[r] - rh[r]) : 0.f;
+                if constexpr (drop) {     // dz meets the scatter's weights as the forward applied them: kept ones, rescaled
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        p[r] *= dropout_factor(a.drop_thr, a.drop_rs, a.seed_lo, a.seed_hi, 1u, (uint32_t)bh, m_lat, (uint32_t)(n0 + 4 * g + r));
+                }
             } else {
-                const f32x4 t1 = dot_rows<Q4>(vc, dzb[ct]);      // <dz_m, v_n>
-                const f32x4 t2 = dot_rows<Q4>(dyc, zb[ct]);      // <dy_n, z_m>
+                f32x4 t1 = dot_rows<Q4>(vc, dzb[ct]);      // <dz_m, v_n>
+                f32x4 t2 = dot_rows<Q4>(dyc, zb[ct]);      // <dy_n, z_m>
+                if constexpr (drop) {
+                    // With W the weights and K the keep factors (0 or 1 / (1 - p)) the forward used K W, and the softmax
+                    // gradient becomes W (K t - Delta): the inner products meet the keep factor, the row sums do not
+                    // (Delta_m = <dz_m, z_m> and delta_n = <dy_n, y_n> already are the sums over the kept weights).
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const uint32_t n = (uint32_t)(n0 + 4 * g + r);
+                        if constexpr (use_a) t1[r] *= dropout_factor(a.drop_thr, a.drop_rs, a.seed_lo, a.seed_hi, 0u, (uint32_t)bh, m_lat, n);
+                        if constexpr (use_b) t2[r] *= dropout_factor(a.drop_thr, a.drop_rs, a.seed_lo, a.seed_hi, 1u, (uint32_t)bh, m_lat, n);
+                    }
+                }
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     // a half's absent term is left out at compile time: its operands may be anything
@@ -306,6 +327,7 @@ __global__ __launch_bounds__(512) void bwd_f32_tok_kernel(MixerBwdArgs a)
     __syncthreads();
 
     constexpr bool use_a = HALF != 2, use_b = HALF != 1;      // gather term, scatter term of dS
+    const bool drop = a.drop_thr != 0;
     const int tiles = (a.N + 15) / 16;
     const int stride = gridDim.x * 8;
     int tile = blockIdx.x * 8 + w;
@@ -349,10 +371,23 @@ __global__ __launch_bounds__(512) void bwd_f32_tok_kernel(MixerBwdArgs a)
                 dza[j4] = *reinterpret_cast<const f32x4*>(dzs + (16 * mt + c16) * LS + g * QL + 4 * j4);
             }
             const f32x4 s = dot_rows<Q4>(qa, kb);
-            const f32x4 t1 = dot_rows<Q4>(dza, vb);       // <dz_m, v_n>
-            const f32x4 t2 = dot_rows<Q4>(za, dyb);       // <z_m, dy_n>
+            f32x4 t1 = dot_rows<Q4>(dza, vb);       // <dz_m, v_n>
+            f32x4 t2 = dot_rows<Q4>(za, dyb);       // <z_m, dy_n>
             const f32x4 l2 = *reinterpret_cast<const f32x4*>(l2s + 16 * mt + 4 * g);
             const f32x4 dl = *reinterpret_cast<const f32x4*>(dls + 16 * mt + 4 * g);
+            float kf[4] = {1.f, 1.f, 1.f, 1.f};      // keep factors of the gather's weights (dv meets them too)
+            if (drop) {
+                const uint32_t n = (uint32_t)min(tile * 16 + c16, a.N - 1);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const uint32_t m = (uint32_t)(a.m0 + 16 * mt + 4 * g + r);
+                    if constexpr (use_a) {
+                        kf[r] = dropout_factor(a.drop_thr, a.drop_rs, a.seed_lo, a.seed_hi, 0u, (uint32_t)bh, m, n);
+                        t1[r] *= kf[r];
+                    }
+                    if constexpr (use_b) t2[r] *= dropout_factor(a.drop_thr, a.drop_rs, a.seed_lo, a.seed_hi, 1u, (uint32_t)bh, m, n);
+                }
+            }
             float wa[4], ds[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -360,8 +395,9 @@ __global__ __launch_bounds__(512) void bwd_f32_tok_kernel(MixerBwdArgs a)
                 wa[r] = 0.f;
                 ds[r] = 0.f;
                 if constexpr (use_a) {
-                    wa[r] = fast_exp2(s[r] - l2[r]);
-                    ds[r] = wa[r] * (t1[r] - dl[r]);
+                    const float wgt = fast_exp2(s[r] - l2[r]);
+                    ds[r] = wgt * (t1[r] - dl[r]);
+                    wa[r] = wgt * kf[r];
                 }
                 if constexpr (use_b) ds[r] += fast_exp2(s[r] - rho) * (t2[r] - dlt);
             }
@@ -418,7 +454,8 @@ hipError_t launch_dh(const MixerBwdArgs& a0, hipStream_t st)
     if (HALF == 1) {
         hipLaunchKernelGGL(bwd_f32_delta_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a);
     } else {
-        hipLaunchKernelGGL((bwd_f32_lat_kernel<D, 0, 0>), dim3(a.n_splits0 * mblocks, a.H, a.B), dim3(256), 0, st, a);
+        if (a.drop_thr != 0) hipLaunchKernelGGL((bwd_f32_lat_kernel<D, 0, 0, true>), dim3(a.n_splits0 * mblocks, a.H, a.B), dim3(256), 0, st, a);
+        else                 hipLaunchKernelGGL((bwd_f32_lat_kernel<D, 0, 0, false>), dim3(a.n_splits0 * mblocks, a.H, a.B), dim3(256), 0, st, a);
         hipLaunchKernelGGL(bwd_f32_merge_kernel<0>, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a);
     }
     // token pass, in chunks of latents when their operands do not fit the LDS
@@ -437,7 +474,8 @@ hipError_t launch_dh(const MixerBwdArgs& a0, hipStream_t st)
         a.accumulate = m0 > 0;
         hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, a);
     }
-    hipLaunchKernelGGL((bwd_f32_lat_kernel<D, 1, HALF>), dim3(a.n_splits * mblocks1, a.H, a.B), dim3(256), 0, st, a);
+    if (a.drop_thr != 0) hipLaunchKernelGGL((bwd_f32_lat_kernel<D, 1, HALF, true>), dim3(a.n_splits * mblocks1, a.H, a.B), dim3(256), 0, st, a);
+    else                 hipLaunchKernelGGL((bwd_f32_lat_kernel<D, 1, HALF, false>), dim3(a.n_splits * mblocks1, a.H, a.B), dim3(256), 0, st, a);
     hipLaunchKernelGGL(bwd_f32_merge_kernel<1>, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, st, a);
     return hipGetLastError();
 }

@@ -32,6 +32,12 @@
 // smallest rho2_n by more than kFactorSpan takes the two-exponential form for all its tiles.
 // (Padded tokens and empty batch elements carry log-sum-exps of 1e30: the former are ignored by the minimum and
 // get eR = 0, the latter send their (b,h) to the two-exponential form.)
+//
+// Attention dropout of the forward (MixerBwdArgs::drop_thr != 0): the keep masks are regenerated from the same hash.  With
+// K1, K2 the keep factors (0 or 1 / (1 - p)) of the two phases the forward used K1 A and K2 Bt, so
+//   dz_m = sum_n K2 Bt dy_n,  dv_n = sum_m K1 A dz_m,  dS = A (K1 <dz_m,v_n> - Delta_m) + Bt (K2 <dy_n,z_m> - delta_n)
+// with the same Delta_m = <dz_m, z_m> and delta_n = <dy_n, y_n> (sums over the kept weights already).  These problems
+// take the two-exponential form with every additive term applied element by element.
 #include <type_traits>
 
 #include "common.hpp"
@@ -166,7 +172,7 @@ __device__ __forceinline__ float dot8(u32x4 u, u32x4 w)
 constexpr int kBTile = 64;   // tokens per LDS tile
 
 // One workgroup = 4 waves x (16 CT latents) x one token range.  MODE 0: dz partial; MODE 1: dq partial.
-template <typename T, int D, int CT, int MODE>
+template <typename T, int D, int CT, int MODE, bool DROPK>
 __global__ __launch_bounds__(256, MODE == 1 ? bwd_dq_wgs_per_cu(D, CT) : 2) void bwd_lat_kernel(MixerBwdArgs a)
 {
     constexpr int KD = (D + 31) / 32, RT = D / 16, CH = D / 8, MB = 64 * CT, ROWB = D * 2, TILEB = kBTile * ROWB;
@@ -193,8 +199,10 @@ __global__ __launch_bounds__(256, MODE == 1 ? bwd_dq_wgs_per_cu(D, CT) : 2) void
     const bool make_delta = MODE == 0 && mb == 0;
 
     // the dq pass forms the token scatter's weights from the gather's where the (b,h) allows it
+    // (a forward with attention dropout: the two weights meet different keep masks, which the one-exponential form,
+    // one accumulator for both inner products, cannot apply)
     float lmax2 = 0.f;
-    const bool fast = MODE == 1 && factor_plan(a, bh, lane, lmax2);
+    const bool fast = MODE == 1 && !DROPK && factor_plan(a, bh, lane, lmax2);
 
     // latent operands (B of the score-like products) and per-latent scalars
     u32x4 qb[CT][KD], dzb[CT][KD], zb[CT][KD];
@@ -303,8 +311,13 @@ __global__ __launch_bounds__(256, MODE == 1 ? bwd_dq_wgs_per_cu(D, CT) : 2) void
         for (int rt = 0; rt < RT; ++rt) acc[rt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
     const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
 
-    auto process = [&](auto fast_c, int n0, int buf) {
+    auto process = [&](auto fast_c, auto drop_c, int n0, int buf) {
         constexpr bool FAST = decltype(fast_c)::value;      // one-exponential form (dq pass only)
+        // DROP: the forward dropped weights.  Every additive term is then applied element by element (accumulators start
+        // at zero), because the inner products meet their keep factors before the row sums are subtracted:
+        // dS = A (K1 <dz,v> - Delta) + B (K2 <dy,z> - delta), and dz = sum_n K2 B dy.
+        constexpr bool DROP = decltype(drop_c)::value;
+        constexpr bool FoldLat = kFoldLat && !DROP;
         const bool full = n0 + kBTile <= n_end;
 #pragma unroll
         for (int ks = 0; ks < kBTile / 32; ++ks) {
@@ -380,26 +393,42 @@ __global__ __launch_bounds__(256, MODE == 1 ? bwd_dq_wgs_per_cu(D, CT) : 2) void
                     continue;
                 }
                 // S - rho_n: the token scatter's exponent
-                constexpr bool kFoldTok = MODE == 0 || kFoldLat;
+                constexpr bool kFoldTok = (MODE == 0 || kFoldLat) && !DROP;
                 f32x4 b0 = kFoldTok ? ra : zf, b1 = kFoldTok ? rb : zf;
 #pragma unroll
                 for (int kd = 0; kd < KD; ++kd) {
                     b0 = M_::mma(ka0[kd], qb[ct][kd], b0);
                     b1 = M_::mma(ka1[kd], qb[ct][kd], b1);
                 }
+                // keep factors (0 or 1 / (1 - p)) of the lane's eight entries: gather's weights, scatter's weights
+                float k1[DROP ? 8 : 1], k2[DROP ? 8 : 1];
+                if constexpr (DROP) {
+                    const uint32_t m = (uint32_t)(m_base + ct * 16 + c16);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const uint32_t n = (uint32_t)(n0 + tb + (e >> 2) * 16 + (e & 3));
+                        if (MODE == 1) k1[e] = dropout_factor(a.drop_thr, a.drop_rs, a.seed_lo, a.seed_hi, 0u, (uint32_t)bh, m, n);
+                        k2[e] = dropout_factor(a.drop_thr, a.drop_rs, a.seed_lo, a.seed_hi, 1u, (uint32_t)bh, m, n);
+                    }
+                }
                 if (MODE == 0) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        o[e] = fast_exp2(b0[e]);
-                        o[e + 4] = fast_exp2(b1[e]);
+                        if constexpr (DROP) {
+                            o[e] = fast_exp2(b0[e] + ra[e]) * k2[e];
+                            o[e + 4] = fast_exp2(b1[e] + rb[e]) * k2[e + 4];
+                        } else {
+                            o[e] = fast_exp2(b0[e]);
+                            o[e + 4] = fast_exp2(b1[e]);
+                        }
                     }
                 } else {
                     // S - L_m (the latent gather's exponent), <dz_m, v_n> - Delta_m and <dy_n, z_m> - delta_n
-                    f32x4 a0 = kFoldLat ? nl4[kFoldLat ? ct : 0] : zf, a1 = a0;
-                    f32x4 g10 = kFoldLat ? nd4[kFoldLat ? ct : 0] : zf, g11 = g10, g20 = kFoldLat ? da : zf, g21 = kFoldLat ? db : zf;
+                    f32x4 a0 = FoldLat ? nl4[kFoldLat ? ct : 0] : zf, a1 = a0;
+                    f32x4 g10 = FoldLat ? nd4[kFoldLat ? ct : 0] : zf, g11 = g10, g20 = FoldLat ? da : zf, g21 = FoldLat ? db : zf;
 #pragma unroll
                     for (int kd = 0; kd < KD; ++kd) {
-                        if constexpr (kFoldLat) {
+                        if constexpr (FoldLat) {
                             a0 = M_::mma(ka0[kd], qb[ct][kd], a0);
                             a1 = M_::mma(ka1[kd], qb[ct][kd], a1);
                         }
@@ -410,7 +439,11 @@ __global__ __launch_bounds__(256, MODE == 1 ? bwd_dq_wgs_per_cu(D, CT) : 2) void
                     }
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        if constexpr (kFoldLat) {
+                        if constexpr (DROP) {
+                            o[e] = fast_exp2(b0[e] - l2m[ct]) * (k1[e] * g10[e] - dm[ct]) + fast_exp2(b0[e] + ra[e]) * (k2[e] * g20[e] + da[e]);
+                            o[e + 4] = fast_exp2(b1[e] - l2m[ct]) * (k1[e + 4] * g11[e] - dm[ct]) +
+                                       fast_exp2(b1[e] + rb[e]) * (k2[e + 4] * g21[e] + db[e]);
+                        } else if constexpr (kFoldLat) {
                             o[e] = fast_exp2(a0[e]) * g10[e] + fast_exp2(b0[e]) * g20[e];
                             o[e + 4] = fast_exp2(a1[e]) * g11[e] + fast_exp2(b1[e]) * g21[e];
                         } else {    // plain products; every term is applied element by element
@@ -438,21 +471,23 @@ __global__ __launch_bounds__(256, MODE == 1 ? bwd_dq_wgs_per_cu(D, CT) : 2) void
         store_tile(0);
     }
     __syncthreads();
-    auto walk = [&](auto fast_c) {
+    auto walk = [&](auto fast_c, auto drop_c) {
         int buf = 0;
         for (int n0 = n_begin; n0 < n_end; n0 += kBTile, buf ^= 1) {
             const bool more = n0 + kBTile < n_end;
             if (more) load_tile(n0 + kBTile);
-            process(fast_c, n0, buf);
+            process(fast_c, drop_c, n0, buf);
             if (more) store_tile(buf ^ 1);
             __syncthreads();
         }
     };
-    if constexpr (MODE == 1) {
-        if (fast) walk(std::true_type{});
-        else walk(std::false_type{});
+    if constexpr (DROPK) {
+        walk(std::false_type{}, std::true_type{});
+    } else if constexpr (MODE == 1) {
+        if (fast) walk(std::true_type{}, std::false_type{});
+        else walk(std::false_type{}, std::false_type{});
     } else {
-        walk(std::false_type{});
+        walk(std::false_type{}, std::false_type{});
     }
 
     if (make_delta) {
@@ -509,7 +544,7 @@ __global__ __launch_bounds__(256) void bwd_merge_kernel(MixerBwdArgs a)
 template <int D> constexpr int kTokWaves = D <= 32 ? 12 : 8;
 template <int D> constexpr int kTokTiles = 2;      // 16-token column tiles per wave iteration
 
-template <typename T, int D>
+template <typename T, int D, bool DROPK>
 __global__ __launch_bounds__(64 * kTokWaves<D>, 1) void bwd_tok_kernel(MixerBwdArgs a, int tokens_per_wg)
 {
     constexpr int NTH = 64 * kTokWaves<D>;
@@ -549,7 +584,7 @@ __global__ __launch_bounds__(64 * kTokWaves<D>, 1) void bwd_tok_kernel(MixerBwdA
     const float* dlt = a.delta_tok + bh * a.N;
 
     float lmax2 = 0.f;
-    const bool fast = factor_plan(a, (int64_t)blockIdx.z * a.H + blockIdx.y, threadIdx.x & 63, lmax2);
+    const bool fast = !DROPK && factor_plan(a, (int64_t)blockIdx.z * a.H + blockIdx.y, threadIdx.x & 63, lmax2);
     if (a.scal_lds) {
         for (int m = threadIdx.x; m < M; m += NTH) {
             const float l2 = lse_lat[m] * kLog2e;
@@ -589,8 +624,11 @@ __global__ __launch_bounds__(64 * kTokWaves<D>, 1) void bwd_tok_kernel(MixerBwdA
 
     // FAST = the one-exponential form (head of this file): the rows of dy and delta_n carry eR[n], the element-wise
     // part applies eL[m]; otherwise both exponentials are taken.
-    auto walk = [&](auto fast_c, const float lmax2) {
+    // DROP = the forward dropped weights: -Delta_m leaves the accumulator of <dz, v> and is applied after the keep factor,
+    // dS = A (K1 <dz,v> - Delta) + B (K2 <dy,z> - delta), and dv meets K1 A.
+    auto walk = [&](auto fast_c, auto drop_c, const float lmax2) {
     constexpr bool FAST = decltype(fast_c)::value;
+    constexpr bool DROP = decltype(drop_c)::value;
     for (int t0 = wg_n0 + w * 16 * kBTW; t0 < wg_n1; t0 += kTokWaves<D> * 16 * kBTW) {
         u32x4 kb[kBTW][KD], vb[kBTW][KD], yb[kBTW][KD];
         float r2[kBTW], de[kBTW];      // FAST: r2 is unused, de = eR delta_n
@@ -716,7 +754,7 @@ __global__ __launch_bounds__(64 * kTokWaves<D>, 1) void bwd_tok_kernel(MixerBwdA
             }
 #pragma unroll
             for (int tw = 0; tw < kBTW; ++tw) {
-                f32x4 a0 = la, a1 = lb, s0 = zf, s1 = zf, g10 = da, g11 = db, g20 = zf, g21 = zf;
+                f32x4 a0 = la, a1 = lb, s0 = zf, s1 = zf, g10 = DROP ? zf : da, g11 = DROP ? zf : db, g20 = zf, g21 = zf;
                 __builtin_amdgcn_s_setprio(1);      // matrix-product issue goes first, the other waves' vector work fills in behind
 #pragma unroll
                 for (int kd = 0; kd < KD; ++kd) {
@@ -731,12 +769,27 @@ __global__ __launch_bounds__(64 * kTokWaves<D>, 1) void bwd_tok_kernel(MixerBwdA
                 }
                 __builtin_amdgcn_s_setprio(0);
                 float av[8], ds[8];
+                if constexpr (DROP) {
+                    const uint32_t n = (uint32_t)min(t0 + tw * 16 + c16, wg_n1 - 1);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const uint32_t m = (uint32_t)(a.m0 + 32 * ks + (e >> 2) * 16 + 4 * g + (e & 3));
+                        const float k1 = dropout_factor(a.drop_thr, a.drop_rs, a.seed_lo, a.seed_hi, 0u, (uint32_t)bh, m, n);
+                        const float k2 = dropout_factor(a.drop_thr, a.drop_rs, a.seed_lo, a.seed_hi, 1u, (uint32_t)bh, m, n);
+                        const float wa = fast_exp2(e < 4 ? a0[e & 3] : a1[e & 3]);
+                        const float g1 = e < 4 ? g10[e & 3] : g11[e & 3], g2 = e < 4 ? g20[e & 3] : g21[e & 3];
+                        const float sc = e < 4 ? s0[e & 3] : s1[e & 3], dl = e < 4 ? da[e & 3] : db[e & 3];
+                        ds[e] = wa * fmaf(k1, g1, dl) + fast_exp2(sc - r2[tw]) * (k2 * g2 - de[tw]);
+                        av[e] = wa * k1;
+                    }
+                } else {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     av[e] = fast_exp2(a0[e]);
                     av[e + 4] = fast_exp2(a1[e]);
                     ds[e] = av[e] * g10[e] + fast_exp2(s0[e] - r2[tw]) * (g20[e] - de[tw]);
                     ds[e + 4] = av[e + 4] * g11[e] + fast_exp2(s1[e] - r2[tw]) * (g21[e] - de[tw]);
+                }
                 }
                 const u32x4 pa = pack8(av), pd = pack8(ds);
 #pragma unroll
@@ -781,36 +834,41 @@ __global__ __launch_bounds__(64 * kTokWaves<D>, 1) void bwd_tok_kernel(MixerBwdA
         }
     }
     };
-    if (fast) walk(std::true_type{}, lmax2);
-    else walk(std::false_type{}, 0.f);
+    if constexpr (DROPK) {
+        walk(std::false_type{}, std::true_type{}, 0.f);
+    } else {
+        if (fast) walk(std::true_type{}, std::false_type{}, lmax2);
+        else walk(std::false_type{}, std::false_type{}, 0.f);
+    }
 }
 
-template <typename T, int D, int MODE>
+template <typename T, int D, int MODE, bool DROPK>
 hipError_t lat_launch(const MixerBwdArgs& a, hipStream_t st)
 {
-    // 4 latent tiles per wave need too many registers at D = 64 in the dq pass
-    if (a.M % 256 == 0 && !(D == 64 && MODE == 1)) {
-        hipLaunchKernelGGL((bwd_lat_kernel<T, D, 4, MODE>), dim3(a.n_splits * (a.M / 256), a.H, a.B), dim3(256), 0, st, a);
-    } else if (a.M % 128 == 0) {
-        hipLaunchKernelGGL((bwd_lat_kernel<T, D, 2, MODE>), dim3(a.n_splits * (a.M / 128), a.H, a.B), dim3(256), 0, st, a);
+    // 4 latent tiles per wave need too many registers at D = 64 in the dq pass, and with the keep factors of a forward
+    // with dropout everywhere (then 2 tiles, 1 at D = 64 in the dq pass)
+    if (a.M % 256 == 0 && !(D == 64 && MODE == 1) && !DROPK) {
+        hipLaunchKernelGGL((bwd_lat_kernel<T, D, DROPK ? 2 : 4, MODE, DROPK>), dim3(a.n_splits * (a.M / 256), a.H, a.B), dim3(256), 0, st, a);
+    } else if (a.M % 128 == 0 && !(DROPK && D == 64 && MODE == 1)) {
+        hipLaunchKernelGGL((bwd_lat_kernel<T, D, 2, MODE, DROPK>), dim3(a.n_splits * (a.M / 128), a.H, a.B), dim3(256), 0, st, a);
     } else {
-        hipLaunchKernelGGL((bwd_lat_kernel<T, D, 1, MODE>), dim3(a.n_splits * ((a.M + 63) / 64), a.H, a.B), dim3(256), 0, st, a);
+        hipLaunchKernelGGL((bwd_lat_kernel<T, D, 1, MODE, DROPK>), dim3(a.n_splits * ((a.M + 63) / 64), a.H, a.B), dim3(256), 0, st, a);
     }
     return hipGetLastError();
 }
 
-template <typename T, int D>
+template <typename T, int D, bool DROPK>
 hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
 {
     const int64_t lat = (int64_t)a.B * a.H * a.M;
     MixerBwdArgs a0 = a;          // the dz pass and its merge work in the dz pass's own split of the token axis
     a0.n_splits = a.n_splits0;
     a0.tokens_per_split = a.tokens_per_split0;
-    hipError_t e = lat_launch<T, D, 0>(a0, st);
+    hipError_t e = lat_launch<T, D, 0, DROPK>(a0, st);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(bwd_merge_kernel<0>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a0);
     {
-        auto kern = bwd_tok_kernel<T, D>;
+        auto kern = bwd_tok_kernel<T, D, DROPK>;
         // the latents are covered in 1, 2 or 4 launches, each with the operand sets of its chunk in LDS
         const int chunks = mixer_bwd_tok_chunks(a.M, D);
         if (chunks == 0) return hipErrorInvalidValue;
@@ -834,7 +892,7 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
             hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(64 * kTokWaves<D>), lds, st, ac, (int)tpw);
         }
     }
-    e = lat_launch<T, D, 1>(a, st);
+    e = lat_launch<T, D, 1, DROPK>(a, st);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(bwd_merge_kernel<1>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a);
     return hipGetLastError();
@@ -843,10 +901,18 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
 template <typename T>
 hipError_t bwd_d(const MixerBwdArgs& a, hipStream_t st)
 {
+    if (a.drop_thr != 0) {      // the forward dropped weights: kernels that regenerate the keep masks
+        switch (a.D) {
+            case 16: return bwd_all<T, 16, true>(a, st);
+            case 32: return bwd_all<T, 32, true>(a, st);
+            case 64: return bwd_all<T, 64, true>(a, st);
+            default: return hipErrorInvalidValue;
+        }
+    }
     switch (a.D) {
-        case 16: return bwd_all<T, 16>(a, st);
-        case 32: return bwd_all<T, 32>(a, st);
-        case 64: return bwd_all<T, 64>(a, st);
+        case 16: return bwd_all<T, 16, false>(a, st);
+        case 32: return bwd_all<T, 32, false>(a, st);
+        case 64: return bwd_all<T, 64, false>(a, st);
         default: return hipErrorInvalidValue;
     }
 }

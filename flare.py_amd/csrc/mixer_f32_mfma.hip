@@ -1,6 +1,7 @@
 // FLARE mixer for fp32 inputs on the fp32 matrix instruction v_mfma_f32_16x16x4_f32 (README.md:39-52 of the
 // reference: z = softmax_n(s q k^T) v, y = softmax_m(s k q^T) z).  Taken by the fp32 launchers of mixer_generic.hip for
-// problems without dropout, D in {16, 32, 64}, M a multiple of 16 and 16-byte aligned rows; same
+// D in {16, 32, 64}, M a multiple of 16 and 16-byte aligned rows, with or without attention dropout (the keep mask is
+// applied to the exponentials in registers on their way into the value product; the denominators keep every weight); same
 // workspace layout, partial format and merge kernel as the FMA kernels there.
 //
 // Operands: A is one float per lane (row c16, k = lane group g), B one float per lane (column c16, k = g), the
@@ -35,7 +36,7 @@ __device__ __forceinline__ float groups_sum(float x)
 
 // ---- gather: one workgroup = 64 latents x one token range; wave w takes the 16-token tiles w, w + 4, ... of the range
 // and writes its own partial (the layout the FMA gather uses: one partial per wave).
-template <int D>
+template <int D, bool DROP>
 __global__ __launch_bounds__(256) void gather_f32_mfma_kernel(MixerArgs a)
 {
     constexpr int QL = D / 4, RT = D / 16, CT = 4, VS = D + 4, VPT = D / 16;
@@ -137,6 +138,13 @@ __global__ __launch_bounds__(256) void gather_f32_mfma_kernel(MixerArgs a)
             }
             lsum[ct] = lsum[ct] * al + ps;
             mx[ct] = mn;
+            if constexpr (DROP) {       // the denominator keeps every weight; the numerator meets the kept ones, rescaled
+                const uint32_t m = mb * 64 + 16 * ct + c16;
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    p[r] = dropout_hash24(a.seed_lo, a.seed_hi, 0u, (uint32_t)(b * a.H + h), m, (uint32_t)(n0 + 4 * g + r)) >= a.drop_thr
+                               ? p[r] * a.drop_rs : 0.f;
+            }
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 f32x4 z = zacc[ct][rt] * al;
@@ -164,7 +172,7 @@ __global__ __launch_bounds__(256) void gather_f32_mfma_kernel(MixerArgs a)
 }
 
 // ---- scatter: Q (log2-scaled) and Z of one (b,h) in LDS; a wave takes 16 tokens at a time and walks all latents.
-template <int D>
+template <int D, bool DROP>
 __global__ __launch_bounds__(256) void scatter_f32_mfma_kernel(MixerArgs a)
 {
     constexpr int QL = D / 4, RT = D / 16, LS = D + 4;
@@ -224,6 +232,13 @@ __global__ __launch_bounds__(256) void scatter_f32_mfma_kernel(MixerArgs a)
             for (int r = 0; r < 4; ++r) p[r] = fast_exp2(s[r] - mn);
             lsum = lsum * al + (p[0] + p[1]) + (p[2] + p[3]);
             mx = mn;
+            if constexpr (DROP) {
+                const uint32_t n = (uint32_t)min(tile * 16 + c16, a.N - 1);
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    p[r] = dropout_hash24(a.seed_lo, a.seed_hi, 1u, (uint32_t)(b * a.H + h), (uint32_t)(16 * mt + 4 * g + r), n) >= a.drop_thr
+                               ? p[r] * a.drop_rs : 0.f;
+            }
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
                 f32x4 o = yacc[rt] * al;
@@ -259,7 +274,7 @@ constexpr size_t kF32ScatterLdsMax = 150 * 1024;
 
 bool f32_mfma_mixer_ok(const MixerArgs& a, bool scatter)
 {
-    if (a.drop_thr != 0 || a.force_fma) return false;
+    if (a.force_fma) return false;
     if (a.D != 16 && a.D != 32 && a.D != 64) return false;
     if (a.M < 16 || a.M % 16 != 0) return false;
     if (!rows16(a.q, a.qs) || !rows16(a.k, a.ks)) return false;
@@ -272,16 +287,22 @@ hipError_t launch_gather_f32_mfma(const MixerArgs& a, hipStream_t st)
 {
     const int mblocks = (a.M + 63) / 64;
     dim3 grid(a.n_splits * mblocks, a.H, a.B);
-    if (a.D == 16)      hipLaunchKernelGGL(gather_f32_mfma_kernel<16>, grid, dim3(256), 0, st, a);
-    else if (a.D == 32) hipLaunchKernelGGL(gather_f32_mfma_kernel<32>, grid, dim3(256), 0, st, a);
-    else                hipLaunchKernelGGL(gather_f32_mfma_kernel<64>, grid, dim3(256), 0, st, a);
+    if (a.drop_thr != 0) {
+        if (a.D == 16)      hipLaunchKernelGGL((gather_f32_mfma_kernel<16, true>), grid, dim3(256), 0, st, a);
+        else if (a.D == 32) hipLaunchKernelGGL((gather_f32_mfma_kernel<32, true>), grid, dim3(256), 0, st, a);
+        else                hipLaunchKernelGGL((gather_f32_mfma_kernel<64, true>), grid, dim3(256), 0, st, a);
+    } else {
+        if (a.D == 16)      hipLaunchKernelGGL((gather_f32_mfma_kernel<16, false>), grid, dim3(256), 0, st, a);
+        else if (a.D == 32) hipLaunchKernelGGL((gather_f32_mfma_kernel<32, false>), grid, dim3(256), 0, st, a);
+        else                hipLaunchKernelGGL((gather_f32_mfma_kernel<64, false>), grid, dim3(256), 0, st, a);
+    }
     return hipGetLastError();
 }
 
-template <int D>
+template <int D, bool DROP>
 hipError_t scatter_launch_d(const MixerArgs& a, hipStream_t st)
 {
-    auto kern = scatter_f32_mfma_kernel<D>;
+    auto kern = scatter_f32_mfma_kernel<D, DROP>;
     const size_t lds = (size_t)a.M * (D + 4) * 8;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
@@ -295,9 +316,14 @@ hipError_t scatter_launch_d(const MixerArgs& a, hipStream_t st)
 
 hipError_t launch_scatter_f32_mfma(const MixerArgs& a, hipStream_t st)
 {
-    if (a.D == 16) return scatter_launch_d<16>(a, st);
-    if (a.D == 32) return scatter_launch_d<32>(a, st);
-    return scatter_launch_d<64>(a, st);
+    if (a.drop_thr != 0) {
+        if (a.D == 16) return scatter_launch_d<16, true>(a, st);
+        if (a.D == 32) return scatter_launch_d<32, true>(a, st);
+        return scatter_launch_d<64, true>(a, st);
+    }
+    if (a.D == 16) return scatter_launch_d<16, false>(a, st);
+    if (a.D == 32) return scatter_launch_d<32, false>(a, st);
+    return scatter_launch_d<64, false>(a, st);
 }
 
 }  // namespace flare

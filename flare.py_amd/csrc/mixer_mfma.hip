@@ -259,6 +259,8 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
 
     float shift[CT];
     f32x4 zacc[RT][CT], lacc[CT];
+    // With attention dropout the optimistic pass is skipped: the keep mask is applied element by element in the exact pass.
+    const bool drop = a.drop_thr != 0;
 
     // one pass over the token range; EXACT keeps a running maximum per latent
     // MASKED: the problem has a key mask (decided once per launch, so the unmasked instance carries none of it)
@@ -395,8 +397,20 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                         }
                         const u32x4 pb = {P_::pack2(p[0], p[1]), P_::pack2(p[2], p[3]),
                                           P_::pack2(p[4], p[5]), P_::pack2(p[6], p[7])};
+                        u32x4 pbv = pb;
+                        if (EXACT && drop) {
+                            // attention dropout: the denominator keeps every weight, the value product meets the kept
+                            // ones (their common factor 1 / (1 - p) is applied to the partial at the end)
+                            const uint32_t m = (uint32_t)(m_base + ct * 16 + c16), bh = (uint32_t)(b * a.H + h);
     #pragma unroll
-                        for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = P_::mma(va[rt], pb, zacc[rt][ct]);
+                            for (int e = 0; e < 8; ++e) {
+                                const uint32_t n = (uint32_t)(n0 + ks * 32 + (e >> 2) * 16 + 4 * g + (e & 3));
+                                p[e] = dropout_hash24(a.seed_lo, a.seed_hi, 0u, bh, m, n) >= a.drop_thr ? p[e] : 0.f;
+                            }
+                            pbv = u32x4{P_::pack2(p[0], p[1]), P_::pack2(p[2], p[3]), P_::pack2(p[4], p[5]), P_::pack2(p[6], p[7])};
+                        }
+    #pragma unroll
+                        for (int rt = 0; rt < RT; ++rt) zacc[rt][ct] = P_::mma(va[rt], pbv, zacc[rt][ct]);
                         lacc[ct] = P_::mma(ones8, pb, lacc[ct]);   // row of ones: the softmax denominator
                     }
                 }
@@ -434,8 +448,8 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
     // validate: every denominator of this wave inside the safe range, numerators finite.  With a key mask a
     // range without a single real token legitimately gives l = 0: the lower bound applies only when the
     // range holds one (counted here; the mask and the range are uniform over the workgroup).
-    bool exact;
-    {
+    bool exact = true;
+    if (!drop) {
         int has_valid = n_begin < n_end;
         if (mask != nullptr) {
             run(std::false_type{}, std::true_type{});
@@ -484,7 +498,7 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
         }
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
-            *reinterpret_cast<f32x4*>(a.part_acc + row * D + rt * 16 + 4 * g) = zacc[rt][ct] * sc;
+            *reinterpret_cast<f32x4*>(a.part_acc + row * D + rt * 16 + 4 * g) = zacc[rt][ct] * (drop ? sc * a.drop_rs : sc);
     }
 }
 
@@ -597,7 +611,10 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
         bool redo = false;
 #pragma unroll
         for (int tw = 0; tw < kSTW; ++tw) lshift[tw] = 0.f;
-        {
+        const bool drop = a.drop_thr != 0;      // attention dropout: straight to the element-wise exact path
+        if (drop) {
+            redo = true;
+        } else {
             // Optimistic pass: no softmax shift at all.  fp32 and bf16 share an 8-bit exponent, so
             // exp2(score) is exact enough whenever the scores of a token stay inside (-60, 120);
             // that is validated afterwards on the denominators, and only a token tile that
@@ -704,8 +721,20 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                     t = P_::sum2(pb[2], t);
                     t = P_::sum2(pb[3], t);
                     lsum[tw] += t;
+                    u32x4 pbv = pb;
+                    if (drop) {     // the denominator keeps every weight, the value product meets the kept ones
+                        const uint32_t n = (uint32_t)min(t0 + tw * 16 + c16, a.N - 1), bh = (uint32_t)(b * a.H + h);
+                        float pd[8];
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = P_::mma(za[rt], pb, yacc[tw][rt]);
+                        for (int e = 0; e < 8; ++e) {
+                            const uint32_t m = (uint32_t)(32 * ks + (e >> 2) * 16 + 4 * g + (e & 3));
+                            const float pe = fast_exp2((e < 4 ? s0[e & 3] : s1[e & 3]) - nc);
+                            pd[e] = dropout_hash24(a.seed_lo, a.seed_hi, 1u, bh, m, n) >= a.drop_thr ? pe : 0.f;
+                        }
+                        pbv = u32x4{P_::pack2(pd[0], pd[1]), P_::pack2(pd[2], pd[3]), P_::pack2(pd[4], pd[5]), P_::pack2(pd[6], pd[7])};
+                    }
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) yacc[tw][rt] = P_::mma(za[rt], pbv, yacc[tw][rt]);
                 }
             }
 #pragma unroll
@@ -725,7 +754,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
                 const int n = t0 + tw * 16 + c16;
                 const bool in = FULL || n < wg_n1;
                 const bool on = FULL || (in && (mask == nullptr || mask[n] != 0));
-                const float inv = on ? __builtin_amdgcn_rcpf(lrow[tw]) : 0.f;
+                const float inv = on ? __builtin_amdgcn_rcpf(lrow[tw]) * (drop ? a.drop_rs : 1.f) : 0.f;
                 if (in) {
                     uint16_t* yr = yr0 + (int64_t)tw * 16 * a.ys[2];
                     uint32_t o[2 * RT];

@@ -12,6 +12,7 @@ implementation behind these calls, and a missing library raises.
 from __future__ import annotations
 
 import ctypes as C
+import struct
 import math
 from typing import Optional, Tuple
 
@@ -120,9 +121,12 @@ class mixer_flags:
         return False
 
 
-def _mixer_desc(q4, k, v, y, scale, n_splits, force_generic) -> FlareMixerDesc:
+def _mixer_desc(q4, k, v, y, scale, n_splits, force_generic, drop=None) -> FlareMixerDesc:
+    """drop = (p, seed) of attention dropout, or None."""
     B, H, N, D = k.shape
     d = FlareMixerDesc()
+    if drop is not None:
+        d.dropout_p, d.dropout_seed = float(drop[0]), int(drop[1]) & 0xFFFFFFFFFFFFFFFF
     d.B, d.H, d.N, d.M, d.D = B, H, N, q4.shape[2], D
     d.dtype = _dtype_code(k)
     d.scale = float(scale)
@@ -183,8 +187,8 @@ def _autocast_dtype(t):
     return None
 
 
-def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major=False, want_lse=False):
-    """y, z (and with want_lse the two log-sum-exps the HIP backward needs)."""
+def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_major=False, want_lse=False, drop=None):
+    """y, z (and with want_lse the two log-sum-exps the HIP backward needs); drop = (p, seed): attention dropout."""
     _require_cuda(q, k, v)
     lib = _lib.load()
     if q.dtype != k.dtype:
@@ -202,7 +206,7 @@ def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_majo
         y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
     z = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
     mask = _mask_u8(key_mask, B, N, k.device)
-    d = _mixer_desc(q4, k, v, y, scale, n_splits, force_generic)
+    d = _mixer_desc(q4, k, v, y, scale, n_splits, force_generic, drop)
     need = C.c_size_t(0)
     _lib.check(lib.flare_mixer_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_workspace_bytes")
     ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
@@ -224,7 +228,7 @@ def _mixer_forward(q, k, v, scale, key_mask, n_splits, force_generic, token_majo
     return y, z
 
 
-def _hip_backward_ok(q, k, v, key_mask, force_generic) -> bool:
+def _hip_backward_ok(q, k, v, key_mask, force_generic, drop=None) -> bool:
     """True when flare_mixer_bwd covers this problem (bf16/f16 and fp32, supported M, D, strides; a key mask is
     handled around the kernels, see _MixerFn.backward)."""
     if force_generic or k.dtype not in (torch.bfloat16, torch.float16, torch.float32):
@@ -235,13 +239,13 @@ def _hip_backward_ok(q, k, v, key_mask, force_generic) -> bool:
     q4 = _q4(q, k.shape[0])
     if any(t.data_ptr() % 16 for t in (q4, k, v)):      # the kernels read 16-byte chunks: a view that starts off
         return False                                    # that grid differentiates through the torch recomputation
-    d = _mixer_desc(q4, k, v, None, 1.0, 0, False)
+    d = _mixer_desc(q4, k, v, None, 1.0, 0, False, drop)
     need = C.c_size_t(0)
     return _lib.load().flare_mixer_bwd_workspace_bytes(C.byref(d), C.byref(need)) == _lib.FLARE_OK
 
 
-def _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy):
-    """dq, dk, dv from the HIP backward kernels (flare_mixer_bwd)."""
+def _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy, drop=None):
+    """dq, dk, dv from the HIP backward kernels (flare_mixer_bwd); drop = (p, seed) of the forward's attention dropout."""
     lib = _lib.load()
     k, v = _rows_last_contig(k), _rows_last_contig(v)
     B, H, N, D = k.shape
@@ -251,7 +255,7 @@ def _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy):
     per16 = 16 // k.element_size()       # elements in 16 bytes
     if gy.stride(-1) != 1 or any(s % per16 for s in gy.stride()[:3]) or gy.data_ptr() % 16:
         gy = gy.contiguous()
-    d = _mixer_desc(q4, k, v, y, scale, 0, False)
+    d = _mixer_desc(q4, k, v, y, scale, 0, False, drop)
     dq = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
     # k and v that are token-major views ([B,N,H,D] storage, as a projection's output is) get their gradients in the
     # same layout: the projection's backward then reads them as [B*N, H*D] rows without a copy
@@ -295,10 +299,20 @@ def _lowbias32(x):
     return x ^ (x >> 16)
 
 
+def _p32(p: float) -> float:
+    """p as the library sees it: rounded to float32 on its way through the C ABI."""
+    return struct.unpack("f", struct.pack("f", p))[0]
+
+
+def _dropout_threshold(p: float) -> int:
+    """The 24-bit threshold the kernels compare the hash with (floor(p * 2^24) of the float32 p)."""
+    return int(_p32(p) * 16777216.0)
+
+
 def _dropout_keep(seed: int, phase: int, B, H, M, n0, n1, p: float, device):
     """The keep mask [B,H,M,n1-n0] of attention dropout, bit for bit the decision the kernels take
     (dropout_hash24 in csrc/common.hpp): 32-bit wrap-around arithmetic carried out in int64."""
-    thr = int(p * 16777216.0)
+    thr = _dropout_threshold(p)
     bh = torch.arange(B * H, device=device, dtype=torch.int64).view(B, H, 1, 1)
     m = torch.arange(M, device=device, dtype=torch.int64).view(1, 1, M, 1)
     n = torch.arange(n0, n1, device=device, dtype=torch.int64).view(1, 1, 1, -1)
@@ -403,6 +417,25 @@ def _mixer_torch_grad(q, k, v, scale, key_mask, gy, drop=None, stats=None):
     return gq.to(q.dtype), gk, gv
 
 
+def _masked_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, km, gy, drop=None):
+    """_mixer_hip_grad for a problem that may carry a key mask."""
+    if km is not None:
+        # A padded token takes no part in either softmax.  The kernels need no mask for that: with its k, v
+        # and dy rows zeroed it adds nothing to dq or dz, with its log-sum-exp set far above any score its
+        # scatter weights vanish, and its own dk, dv rows are cleared afterwards.  A batch element without
+        # a single real token has lse_lat = -inf; the same treatment turns its gather weights into 0.
+        keep = km.to(torch.bool)
+        m4 = keep[:, None, :, None]
+        zero = torch.zeros((), dtype=k.dtype, device=k.device)
+        k, v, gy = torch.where(m4, k, zero), torch.where(m4, v, zero), torch.where(m4, gy.to(k.dtype), zero)
+        lse_tok = torch.where(keep[:, None, :], lse_tok, lse_tok.new_tensor(1e30))
+        lse_lat = torch.where(torch.isfinite(lse_lat), lse_lat, lse_lat.new_tensor(1e30))
+    gq, gk, gv = _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy, drop)
+    if km is not None:
+        gk, gv = torch.where(m4, gk, zero), torch.where(m4, gv, zero)
+    return gq, gk, gv
+
+
 class _MixerFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, scale, key_mask, n_splits, force_generic, token_major):
@@ -427,21 +460,7 @@ class _MixerFn(torch.autograd.Function):
     def backward(ctx, gy, _gz):
         if ctx.hip:
             q, k, v, y, z, lse_lat, lse_tok = ctx.saved_tensors
-            km = ctx.key_mask
-            if km is not None:
-                # A padded token takes no part in either softmax.  The kernels need no mask for that: with its k, v
-                # and dy rows zeroed it adds nothing to dq or dz, with its log-sum-exp set far above any score its
-                # scatter weights vanish, and its own dk, dv rows are cleared afterwards.  A batch element without
-                # a single real token has lse_lat = -inf; the same treatment turns its gather weights into 0.
-                keep = km.to(torch.bool)
-                m4 = keep[:, None, :, None]
-                zero = torch.zeros((), dtype=k.dtype, device=k.device)
-                k, v, gy = torch.where(m4, k, zero), torch.where(m4, v, zero), torch.where(m4, gy.to(k.dtype), zero)
-                lse_tok = torch.where(keep[:, None, :], lse_tok, lse_tok.new_tensor(1e30))
-                lse_lat = torch.where(torch.isfinite(lse_lat), lse_lat, lse_lat.new_tensor(1e30))
-            gq, gk, gv = _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, ctx.scale, gy)
-            if km is not None:
-                gk, gv = torch.where(m4, gk, zero), torch.where(m4, gv, zero)
+            gq, gk, gv = _masked_hip_grad(q, k, v, y, z, lse_lat, lse_tok, ctx.scale, ctx.key_mask, gy)
         else:
             q, k, v, *stats = ctx.saved_tensors
             gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy,
@@ -449,64 +468,47 @@ class _MixerFn(torch.autograd.Function):
         return gq, gk, gv, None, None, None, None, None
 
 
-def _mixer_forward_dropout(q, k, v, scale, key_mask, p, seed, token_major):
-    """y, z of the mixer with attention dropout (flare_mixer_fwd_dropout: fp32-FMA kernels)."""
-    _require_cuda(q, k, v)
-    lib = _lib.load()
-    if q.dtype != k.dtype:
-        q = q.to(k.dtype)
-    if v.dtype != k.dtype:
-        raise TypeError("k and v must share a dtype")
-    k, v = _rows_last_contig(k), _rows_last_contig(v)
-    q4 = _q4(q, k.shape[0])
-    _check_mixer_shapes(q4, k, v)
-    B, H, N, D = k.shape
-    M = q4.shape[2]
-    if token_major:
-        y = torch.empty((B, N, H, D), dtype=k.dtype, device=k.device).permute(0, 2, 1, 3)
-    else:
-        y = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
-    z = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
-    mask = _mask_u8(key_mask, B, N, k.device)
-    d = _mixer_desc(q4, k, v, y, scale, 0, True)
-    need = C.c_size_t(0)
-    _lib.check(lib.flare_mixer_workspace_bytes(C.byref(d), C.byref(need)), "flare_mixer_workspace_bytes")
-    ws = torch.empty(max(int(need.value), 16), dtype=torch.uint8, device=k.device)
-    with _on_device(k.device):
-        rc = lib.flare_mixer_fwd_dropout(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(mask), float(p), int(seed), _ptr(y), _ptr(z),
-                                         _ptr(ws), ws.numel(), C.c_void_p(_stream_ptr(k.device)))
-    _lib.check(rc, "flare_mixer_fwd_dropout")
-    return y, z
-
-
 class _MixerDropoutFn(torch.autograd.Function):
+    """The mixer with attention dropout.  Where flare_mixer_bwd takes the problem (fp32 on the matrix cores) the backward
+    runs there and regenerates the keep masks from (p, seed); elsewhere it is the tiled torch recomputation with the
+    same masks (_dropout_keep)."""
+
     @staticmethod
     def forward(ctx, q, k, v, scale, key_mask, p, seed, token_major):
         ctx.scale, ctx.key_mask, ctx.drop = scale, key_mask, (p, seed)
-        ctx.save_for_backward(q, k, v)
-        y, z = _mixer_forward_dropout(q, k, v, scale, key_mask, p, seed, token_major)
+        ctx.hip = _hip_backward_ok(q, k, v, key_mask, False, ctx.drop)
+        if ctx.hip:
+            y, z, lse_lat, lse_tok = _mixer_forward(q, k, v, scale, key_mask, 0, False, token_major, True, ctx.drop)
+            ctx.save_for_backward(q, k, v, y, z, lse_lat, lse_tok)
+        else:
+            y, z = _mixer_forward(q, k, v, scale, key_mask, 0, False, token_major, False, ctx.drop)
+            ctx.save_for_backward(q, k, v)
         ctx.mark_non_differentiable(z)
         return y, z
 
     @staticmethod
     @once_differentiable
     def backward(ctx, gy, _gz):
-        q, k, v = ctx.saved_tensors
-        gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy, ctx.drop)
+        if ctx.hip:
+            q, k, v, y, z, lse_lat, lse_tok = ctx.saved_tensors
+            gq, gk, gv = _masked_hip_grad(q, k, v, y, z, lse_lat, lse_tok, ctx.scale, ctx.key_mask, gy, ctx.drop)
+        else:
+            q, k, v = ctx.saved_tensors
+            gq, gk, gv = _mixer_torch_grad(q, k, v, ctx.scale, ctx.key_mask, gy, ctx.drop)
         return gq, gk, gv, None, None, None, None, None
 
 
-def _narrow_head_pad(q, k, force_generic, masked=False) -> int:
+def _narrow_head_pad(q, k, force_generic) -> int:
     """Columns of zeros to append to a head dim so that the matrix-core kernels (D in {16, 32, 64}) take the problem,
     or 0.  Zero columns change neither the scores q.k nor the first D output columns; the reference's default model
     has D = channel_dim / num_heads = 8, which the fp32-FMA kernels would serve 5-15x slower.  fp32 problems have
-    matrix-core kernels too (latent counts that are multiples of 16, no dropout: `masked`)."""
+    matrix-core kernels too (latent counts that are multiples of 16)."""
     D = k.shape[-1]
     if force_generic or D > 64 or k.device.type != "cuda":
         return 0
     target = 16 if D <= 16 else 32 if D <= 32 else 64
     if k.dtype == torch.float32:
-        return target - D if q.shape[-2] % 16 == 0 and not masked else 0      # masked: dropout (FMA kernels only)
+        return target - D if q.shape[-2] % 16 == 0 else 0
     if k.dtype not in (torch.bfloat16, torch.float16):
         return 0
     return target - D if q.shape[-2] % 32 == 0 else 0
@@ -531,7 +533,9 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
     [B,N,H,D] in memory (returned as its [B,H,N,D] view) so that merging the heads is free.
     dropout_p > 0 drops entries of both softmaxes' weights the way torch's scaled_dot_product_attention does
     in training (lra/models/backends.py:592,605-606); the mask is a function of dropout_seed (drawn from torch's
-    default generator when None), so the backward recomputes it.  That path runs on the fp32-FMA kernels.
+    default generator when None), so the backward recomputes it.  The 32x32x16 kernels carry no dropout: 16-bit problems
+    run on the 16x16x32 kernels (element-wise exact passes) and differentiate through the torch recomputation, fp32
+    problems run forward and backward on the fp32 matrix-core kernels.
     """
     ac = _autocast_dtype(k)
     if ac is not None:
@@ -540,10 +544,18 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
         if not dropout_p < 1.0:
             raise ValueError("dropout_p must be in [0, 1)")
         seed = int(torch.randint(0, 2 ** 62, (), dtype=torch.int64)) if dropout_seed is None else int(dropout_seed)
+        D = k.shape[-1]
+        # zero columns change neither the scores nor the mask's indices: narrow heads reach the matrix-core kernels
+        pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype == v.dtype else 0
+        if pad:
+            q, k, v = _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad)
         if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
             y, z = _MixerDropoutFn.apply(q, k, v, float(scale), key_mask, float(dropout_p), seed, token_major_out)
         else:
-            y, z = _mixer_forward_dropout(q, k, v, float(scale), key_mask, float(dropout_p), seed, token_major_out)
+            y, z = _mixer_forward(q, k, v, float(scale), key_mask, 0, force_generic, token_major_out, False,
+                                  (float(dropout_p), seed))
+        if pad:
+            y, z = y[..., :D], z[..., :D]
         return (y, z) if return_z else y
     D = k.shape[-1]
     r = _latent_copies(q, k, force_generic)
@@ -558,7 +570,7 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
             and k.dtype in (torch.bfloat16, torch.float16) and k.device.type == "cuda"
             and _dead_latent_bias(float(scale), k.dtype) is not None):
         return _mixer_odd_latents(q, k, v, float(scale), key_mask, return_z, n_splits, token_major_out)
-    pad = _narrow_head_pad(q, k, force_generic, dropout_p > 0) if q.dtype == k.dtype == v.dtype else 0
+    pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype == v.dtype else 0
     if pad:
         q, k, v = _pad_last(q, pad), _pad_last(k, pad), _pad_last(v, pad)
     needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v))

@@ -50,7 +50,7 @@
 extern "C" {
 #endif
 
-#define FLARE_ABI_VERSION 1
+#define FLARE_ABI_VERSION 2
 
 /* status codes */
 #define FLARE_OK            0
@@ -89,6 +89,19 @@ typedef struct FlareMixerDesc {
     int64_t k_stride[3];
     int64_t v_stride[3];
     int64_t y_stride[3];
+    /* Attention dropout on both softmaxes, as torch's scaled_dot_product_attention applies it in training
+     * (lra/models/backends.py:592,605-606: dropout_p on both calls): every normalised weight is kept with
+     * probability 1 - dropout_p and then divided by it, independently in the gather and in the scatter.  The
+     * decision for the weight of (batch, head, latent, token) is a counter-based hash of those indices, the phase
+     * and dropout_seed compared with floor(dropout_p * 2^24) (no state, nothing stored): every entry point that
+     * is handed the same descriptor sees the same mask, so the backward entry points regenerate the forward's.
+     * 0 <= dropout_p < 1; 0 (and anything below 2^-24) switches dropout off.  Honoured by flare_gather_fwd,
+     * flare_scatter_fwd(_lse), flare_mixer_fwd(_static) and flare_mixer_bwd; the 32x32x16 kernels carry no mask,
+     * so a problem with dropout runs on the 16x16x32 (16-bit) or 16x16x4 (fp32) matrix-core kernels or on the
+     * fp32-FMA kernels, and its workspace is sized from the descriptor with these fields set. */
+    float    dropout_p;
+    int32_t  reserved2;
+    uint64_t dropout_seed;
 } FlareMixerDesc;
 
 /*
@@ -185,7 +198,7 @@ const char* flare_last_error_string(void);
 /* Name of the kernel family the dispatcher would pick for this problem
  * ("mfma_bf16", "mfma_f16", "generic"); NULL + error on an invalid descriptor.  "generic" names the family that
  * serves fp32 and the shapes the 16-bit matrix-core kernels do not take: inside it, fp32 problems with D in
- * {16, 32, 64}, M a multiple of 16, no dropout and 16-byte aligned rows run on fp32 matrix-core kernels
+ * {16, 32, 64}, M a multiple of 16 and 16-byte aligned rows run on fp32 matrix-core kernels
  * (v_mfma_f32_16x16x4_f32), everything else as fp32 FMA loops; the workspace layout is the same for both. */
 const char* flare_mixer_kernel_name(const FlareMixerDesc* desc);
 
@@ -217,7 +230,9 @@ int flare_scatter_fwd_lse(const FlareMixerDesc* desc, const void* q, const void*
  * lse_tok of flare_scatter_fwd_lse; dy [B,H,N,D] with strides dy_stride.
  * Outputs: dq fp32 [B,H,M,D] contiguous (per batch element: sum over b when q is shared);
  * dk, dv [B,H,N,D] in the element type: contiguous, or with FLARE_FLAG_GRAD_LIKE_KV laid out as k and v are (a
- * projection that produced k token-major then takes dk back without a copy). */
+ * projection that produced k token-major then takes dk back without a copy).
+ * A forward that ran with desc->dropout_p > 0 is differentiated by handing the same descriptor (dropout_p and
+ * dropout_seed) in here: the kernels regenerate its keep masks. */
 int flare_mixer_bwd_workspace_bytes(const FlareMixerDesc* desc, size_t* bytes);
 int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, const void* v, const void* y,
                     const float* z, const float* lse_lat, const float* lse_tok, const void* dy,
@@ -244,13 +259,9 @@ int flare_mixer_fwd(const FlareMixerDesc* desc, const void* q, const void* k, co
                     const uint8_t* key_mask, void* y, float* z_out,
                     void* workspace, size_t workspace_bytes, void* stream);
 
-/* The mixer with attention dropout on both softmaxes, as torch's scaled_dot_product_attention applies it in
- * training (lra/models/backends.py:592,605-606: dropout_p on both calls): every normalised weight is kept with
- * probability 1 - dropout_p and then divided by it, independently in the gather and in the scatter.  The decision
- * for the weight of (batch, head, latent, token) is a counter-based hash of those indices, the phase and `seed`
- * (no state, nothing stored): the same call repeats the same mask and a backward pass can recompute it.  Runs on
- * the fp32-FMA kernels for every element type; dropout_p = 0 gives flare_mixer_fwd's result on those kernels.
- * Workspace as flare_mixer_workspace_bytes(). */
+/* flare_mixer_fwd with the descriptor's dropout fields taken from the arguments instead (desc->dropout_p and
+ * desc->dropout_seed are ignored): the form lra/models/backends.py:592,605-606 calls, dropout_p on both softmaxes.
+ * The workspace must hold flare_mixer_workspace_bytes() of the descriptor with dropout_p set. */
 int flare_mixer_fwd_dropout(const FlareMixerDesc* desc, const void* q, const void* k, const void* v,
                             const uint8_t* key_mask, float dropout_p, uint64_t seed, void* y, float* z_out,
                             void* workspace, size_t workspace_bytes, void* stream);

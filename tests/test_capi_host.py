@@ -30,11 +30,11 @@ def test_header_symbols_all_exported():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in flare_hip.h but not exported"
     assert declared == set(_lib.SYMBOLS), "ctypes binding and header disagree"
-    assert lib.flare_abi_version() == 1
+    assert lib.flare_abi_version() == _lib.ABI_VERSION == 2
 
 
 def test_struct_sizes_match_header_layout():
-    assert C.sizeof(_lib.FlareMixerDesc) == 10 * 4 + 4 * 24
+    assert C.sizeof(_lib.FlareMixerDesc) == 10 * 4 + 4 * 24 + 16       # + dropout_p, reserved2, dropout_seed
     assert C.sizeof(_lib.FlareCausalDesc) == 10 * 4 + 4 * 24
     assert C.sizeof(_lib.FlareTripleDesc) == 10 * 4 + 6 * 24
 
