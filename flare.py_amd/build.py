@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libflare_hip.so")
-SOURCES = ["capi.hip", "mixer_generic.hip", "mixer_f32_mfma.hip", "mixer_mfma.hip", "mixer_mfma32.hip", "mixer_bwd_mfma.hip", "mixer_bwd_f32_mfma.hip", "causal.hip", "causal_mfma.hip", "causal_decode.hip", "causal_linear.hip", "causal_linear_mfma.hip", "mlp_mfma.hip", "mlp_bwd_mfma.hip", "mlp_wgrad_mfma.hip", "triple.hip", "triple_f32_mfma.hip", "triple_mfma.hip"]
+SOURCES = ["capi.hip", "mixer_generic.hip", "mixer_f32_mfma.hip", "mixer_mfma.hip", "mixer_mfma32.hip", "mixer_bwd_mfma.hip", "mixer_bwd_mfma32.hip", "mixer_bwd_f32_mfma.hip", "causal.hip", "causal_mfma.hip", "causal_decode.hip", "causal_linear.hip", "causal_linear_mfma.hip", "mlp_mfma.hip", "mlp_bwd_mfma.hip", "mlp_wgrad_mfma.hip", "triple.hip", "triple_f32_mfma.hip", "triple_mfma.hip"]
 # packed-fp32 instruction selection is switched off for every device translation unit
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-math-errno", "-ffp-contract=fast",

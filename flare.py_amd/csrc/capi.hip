@@ -451,6 +451,11 @@ int flare_scatter_fwd_lse(const FlareMixerDesc* desc, const void* q, const void*
 namespace {
 struct BwdPlan { int n_splits, tokens_per_split, n_splits0, tokens_per_split0; size_t off_dz, off_dl, off_rm, off_part, total; };
 
+bool bwd_wants_dz32(const FlareMixerDesc* d)
+{
+    return !(d->flags & FLARE_FLAG_MFMA16) && drop_threshold(d) == 0 && flare::bwd_dz32_supported(d->dtype, d->M, d->D);
+}
+
 BwdPlan plan_bwd(const FlareMixerDesc* d)
 {
     BwdPlan p;
@@ -468,8 +473,22 @@ BwdPlan plan_bwd(const FlareMixerDesc* d)
         tokens_per_split = (int)tps;
         n_splits = (int)(((int64_t)d->N + tps - 1) / tps);
     };
-    split(f32 ? 2 : flare::bwd_dq_wgs_per_cu(d->D, d->M % 256 == 0 ? 4 : d->M % 128 == 0 ? 2 : 1), p.n_splits, p.tokens_per_split);
-    split(f32 ? 2 : d->D <= 16 ? 4 : d->D <= 32 ? (d->M % 256 ? 4 : 3) : 2, p.n_splits0, p.tokens_per_split0);
+    if (bwd_wants_dz32(d)) {
+        // the 32x32x16 dz and dq passes: two workgroups per compute unit, ranges a multiple of their four waves' 32-token
+        // passes; 256 latents per workgroup in the dz pass, 128 in the dq pass
+        auto split32 = [&](int64_t blocks, int& n_splits, int& tokens_per_split) {
+            int64_t s = std::max<int64_t>(1, 2 * flare::device_cus() / (bh * blocks));
+            int64_t tps = (((int64_t)d->N + s - 1) / s + 127) / 128 * 128;
+            if (tps < 512) tps = 512;
+            tokens_per_split = (int)tps;
+            n_splits = (int)(((int64_t)d->N + tps - 1) / tps);
+        };
+        split32(mblocks, p.n_splits0, p.tokens_per_split0);
+        split32(flare::bwd_dq32_mblocks(d->M), p.n_splits, p.tokens_per_split);
+    } else {
+        split(f32 ? 2 : flare::bwd_dq_wgs_per_cu(d->D, d->M % 256 == 0 ? 4 : d->M % 128 == 0 ? 2 : 1), p.n_splits, p.tokens_per_split);
+        split(f32 ? 2 : d->D <= 16 ? 4 : d->D <= 32 ? (d->M % 256 ? 4 : 3) : 2, p.n_splits0, p.tokens_per_split0);
+    }
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     p.off_dz = up((size_t)bh * d->N * 4);
     p.off_dl = p.off_dz + up((size_t)bh * d->M * d->D * 4);
@@ -540,6 +559,7 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
     a.B = desc->B; a.H = desc->H; a.N = desc->N; a.M = desc->M; a.D = desc->D;
     a.n_splits = p.n_splits; a.tokens_per_split = p.tokens_per_split;
     a.n_splits0 = p.n_splits0; a.tokens_per_split0 = p.tokens_per_split0;
+    a.no_mfma32 = bwd_wants_dz32(desc) ? 0 : 1;
     a.scale = desc->scale; a.scale_log2 = desc->scale * 1.4426950408889634f;
     a.drop_thr = drop_threshold(desc);
     a.drop_rs = 1.f;
@@ -581,6 +601,7 @@ int half_bwd_args(flare::MixerBwdArgs& a, const FlareMixerDesc* desc, void* work
     a.B = desc->B; a.H = desc->H; a.N = desc->N; a.M = desc->M; a.D = desc->D;
     a.n_splits = p.n_splits; a.tokens_per_split = p.tokens_per_split;
     a.n_splits0 = p.n_splits0; a.tokens_per_split0 = p.tokens_per_split0;
+    a.no_mfma32 = bwd_wants_dz32(desc) ? 0 : 1;
     a.scale = desc->scale; a.scale_log2 = desc->scale * 1.4426950408889634f;
     a.drop_thr = drop_threshold(desc);
     a.drop_rs = 1.f;

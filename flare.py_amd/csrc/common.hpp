@@ -191,10 +191,36 @@ struct MixerBwdArgs {
     int scal_lds;            // token-side kernel only: per-latent scalars are tabled in LDS behind the operand sets
     int half;                // fp32 kernels: 0 = whole mixer, 1 = gather half only (dz given, no scatter term), 2 = scatter half only
                              // (no gather term, dv not written; dz is an output)
+    int no_mfma32;           // 1: keep the 16x16x32 kernels where the 32x32x16 passes would run
+    int only_form;           // token-side kernels: 0 = every (b,h); 1 = only those that take the unshifted one-exponential
+                             // form (bwd_unshifted_form), 2 = only the others (a workgroup of the other kind returns at once)
     // attention dropout of the forward this is the backward of (same fields as MixerArgs; drop_thr == 0: none)
     uint32_t drop_thr, seed_lo, seed_hi;
     float drop_rs;
 };
+
+// Whether a (b,h) takes the form of the backward in which both weights come from exp2(S) alone (kernels on the 32x32x16
+// product): the one-exponential form's own condition (the latents' largest log-sum-exp and the tokens' smallest one at
+// most 64 apart, log2 units) and every latent log-sum-exp within +-60, so that exp2(S) can stand in for exp2(S - L2_m)
+// with the constant exp2(-L2_m) applied elsewhere.  Every lane of a wave gets the same answer; lmax2 = largest L2_m.
+__device__ __forceinline__ bool bwd_unshifted_form(const MixerBwdArgs& a, int64_t bh, int lane, float& lmax2)
+{
+    float lm = -3.0e38f, ln = 3.0e38f, rm = -3.0e38f;
+    for (int m = lane; m < a.M; m += 64) {
+        const float l = a.lse_lat[bh * a.M + m];
+        lm = fmaxf(lm, l);
+        ln = fminf(ln, l);
+    }
+    for (int p = lane; p < a.n_splits0; p += 64) rm = fmaxf(rm, -a.rho_min[bh * a.n_splits0 + p]);
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        lm = fmaxf(lm, __shfl_xor(lm, o));
+        ln = fminf(ln, __shfl_xor(ln, o));
+        rm = fmaxf(rm, __shfl_xor(rm, o));
+    }
+    lmax2 = lm * kLog2e;
+    return lmax2 <= 60.f && ln * kLog2e >= -60.f && lmax2 + rm <= 64.f;
+}
 
 struct CausalLinearArgs {
     const void* q; const void* k; const void* v; void* y;
@@ -275,6 +301,13 @@ constexpr int bwd_dq_wgs_per_cu(int D, int CT)
 }
 
 // ---- launchers implemented in the .hip files -------------------------------------------
+// dz pass of the mixer backward on the 32x32x16 product (mixer_bwd_mfma32.hip): bf16, D = 32, M % 64 == 0
+bool       bwd_dz32_supported(int dtype, int M, int D);
+hipError_t launch_bwd_dz32(const MixerBwdArgs& a, hipStream_t st);
+int        bwd_dq32_mblocks(int M);
+bool       bwd_tok32_supported(int dtype, int M, int D);
+hipError_t launch_bwd_tok32(const MixerBwdArgs& a, hipStream_t st);      // only the (b,h) of the unshifted form
+hipError_t launch_bwd_dq32(const MixerBwdArgs& a, hipStream_t st);
 hipError_t launch_gather_generic(const MixerArgs& a, int dtype, hipStream_t st);
 hipError_t launch_gather_merge(const MixerArgs& a, hipStream_t st);
 hipError_t launch_scatter_generic(const MixerArgs& a, int dtype, hipStream_t st);

@@ -585,6 +585,10 @@ __global__ __launch_bounds__(64 * kTokWaves<D>, 1) void bwd_tok_kernel(MixerBwdA
 
     float lmax2 = 0.f;
     const bool fast = !DROPK && factor_plan(a, (int64_t)blockIdx.z * a.H + blockIdx.y, threadIdx.x & 63, lmax2);
+    if (a.only_form == 2) {     // the 32x32x16 token pass has taken the (b,h) of the unshifted form
+        float unused;
+        if (bwd_unshifted_form(a, (int64_t)blockIdx.z * a.H + blockIdx.y, threadIdx.x & 63, unused)) return;
+    }
     if (a.scal_lds) {
         for (int m = threadIdx.x; m < M; m += NTH) {
             const float l2 = lse_lat[m] * kLog2e;
@@ -864,9 +868,18 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
     MixerBwdArgs a0 = a;          // the dz pass and its merge work in the dz pass's own split of the token axis
     a0.n_splits = a.n_splits0;
     a0.tokens_per_split = a.tokens_per_split0;
-    hipError_t e = lat_launch<T, D, 0, DROPK>(a0, st);
+    // bf16 at D = 32 without dropout: the token-parallel dz pass on the 32x32x16 product
+    const bool dz32 = !DROPK && !a.no_mfma32 && std::is_same<T, bf16_t>::value && bwd_dz32_supported(1, a.M, D);
+    hipError_t e = dz32 ? launch_bwd_dz32(a0, st) : lat_launch<T, D, 0, DROPK>(a0, st);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(bwd_merge_kernel<0>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a0);
+    // the token pass on the 32x32x16 product takes the (b,h) of the unshifted one-exponential form; the kernel below
+    // then only works on the others (normally none: its workgroups return at once)
+    const bool tok32 = dz32 && bwd_tok32_supported(1, a.M, D);
+    if (tok32) {
+        e = launch_bwd_tok32(a, st);
+        if (e != hipSuccess) return e;
+    }
     {
         auto kern = bwd_tok_kernel<T, D, DROPK>;
         // the latents are covered in 1, 2 or 4 launches, each with the operand sets of its chunk in LDS
@@ -889,10 +902,11 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
             ac.mc = mc;
             ac.accumulate = c > 0;
             ac.scal_lds = scal_lds ? 1 : 0;
+            ac.only_form = tok32 ? 2 : 0;
             hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(64 * kTokWaves<D>), lds, st, ac, (int)tpw);
         }
     }
-    e = lat_launch<T, D, 1, DROPK>(a, st);
+    e = dz32 ? launch_bwd_dq32(a, st) : lat_launch<T, D, 1, DROPK>(a, st);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(bwd_merge_kernel<1>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a);
     return hipGetLastError();
