@@ -32,7 +32,8 @@ def oracle_grads(q, k, v, gy, scale):
 
 
 @pytest.mark.parametrize("shape", [(1, 2, 777, 64, 32), (2, 2, 1000, 128, 16), (1, 1, 300, 256, 32), (1, 2, 500, 128, 64),
-                                   (2, 1, 2500, 256, 32), (1, 8, 4100, 64, 16), (1, 2, 900, 512, 16), (1, 1, 70001, 256, 32)])
+                                   (2, 1, 2500, 256, 32), (1, 8, 4100, 64, 16), (1, 2, 900, 512, 16), (1, 1, 70001, 256, 32),
+                                   (1, 2, 1300, 512, 32), (2, 1, 1111, 192, 32), (1, 3, 5000, 128, 32), (1, 1, 33, 64, 32)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_backward_vs_autograd_oracle(dev, shape, dtype):
     q, k, v, gy = make(*shape, dtype)
@@ -220,6 +221,33 @@ def test_backward_with_log_sum_exps_far_apart(dev, a):
     # dominant tokens) and enter the matrix cores rounded to bf16, hence the wider bar.
     err = O.rel_l2(kd.grad[:, :, ::2], gk[:, :, ::2])
     assert err <= 6e-2, f"dk of the low-scoring tokens rel-L2 {err:.3e}"
+
+
+@pytest.mark.parametrize("a", [7.5, -7.5])
+@pytest.mark.parametrize("M", [64, 256, 512])
+def test_backward_with_large_log_sum_exps(dev, a, M):
+    """The bf16 kernels on the 32x32x16 product take exp2(S) for the gather's weights and apply exp2(-L2_m) elsewhere
+    while every latent log-sum-exp stays within +-60 (log2 units).  Every score near +56 or -56 puts all of them outside
+    (the span between the two families of log-sum-exps stays small): these (b,h) take the general form, the dq pass in
+    its plain passes and the token pass in the 16x16x32 kernel launched behind the 32x32x16 one; head 1 stays inside
+    and takes the fast kernels in the same launch."""
+    B, H, N, D = 1, 2, 700, 32
+    q, k, v, gy = make(B, H, N, M, D, torch.bfloat16, seed=37)
+    q[0, :, 0] = abs(a)
+    k[:, 0, :, 0] = a
+    s = torch.einsum("hmd,bhnd->bhmn", q.float(), k.float())
+    lse2 = torch.logsumexp(s, -1) * 1.4426950408889634
+    assert float(lse2[0, 0].abs().min()) > 60 and float(lse2[0, 1].abs().max()) < 60
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    assert FN._hip_backward_ok(qd, kd, vd, None, False)
+    F.flare_multihead_mixer(qd, kd, vd).backward(gy.to(dev))
+    gq, gk, gv = oracle_grads(q, k, v, gy, 1.0)
+    for name, got, ref in (("dq", qd.grad, gq), ("dk", kd.grad, gk), ("dv", vd.grad, gv)):
+        assert torch.isfinite(got).all()
+        for hd in range(H):
+            sl = (slice(None), hd) if name != "dq" else (hd,)
+            err = O.rel_l2(got[sl], ref[sl])
+            assert err <= 3e-2, f"{name} head {hd} rel-L2 {err:.3e}"
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
