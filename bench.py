@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FLARE mixer forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block|train|linear|fp32|layer|lra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block|train|linear|fp32|layer|lra|power]
 
 One step = one forward of the mixer (split-N gather, merge, scatter) over the headline workload
 B=1, H=8, N=1,048,576, M=256, D=32, bf16 in / fp32 accumulate, inputs resident in HBM.
@@ -438,6 +438,87 @@ def _mfma16(F, q, k, v):
         return F.flare_multihead_mixer(q, k, v)
 
 
+def _smi_sample():
+    """Socket power (W) and the XCDs' shader clocks (MHz) as amd-smi reports them right now, or None."""
+    import re
+    import subprocess
+    try:
+        txt = subprocess.run(["amd-smi", "metric", "-p", "-c"], capture_output=True, text=True, timeout=30).stdout
+    except Exception:
+        return None
+    pw = re.search(r"SOCKET_POWER:\s*([0-9.]+)\s*W", txt)
+    clks = [int(c) for c in re.findall(r"GFX_\d+:\s*\n\s*CLK:\s*(\d+)\s*MHz", txt)]
+    cap = re.search(r"MAX_CLK:\s*(\d+)\s*MHz", txt)
+    if pw is None or not clks:
+        return None
+    return {"socket_power_w": float(pw.group(1)), "gfx_clk_mhz_mean": round(sum(clks) / len(clks)), "gfx_clk_mhz_min": min(clks),
+            "gfx_clk_mhz_max": max(clks), "gfx_max_clk_mhz": int(cap.group(1)) if cap else None}
+
+
+def bench_power(args, F, dev):
+    """Socket power and shader clock (amd-smi) while each of a few loads runs for some seconds: the headline forward,
+    the headline forward + backward, a plain device-to-device copy, and the idle device.  The line's value is the
+    forward's throughput during its sustained run."""
+    import subprocess
+    import threading
+
+    B, H, N, M, D = 1, 8, 1 << 20, 256, 32
+    q, k, v = make_inputs(B, H, N, M, D, torch.bfloat16, dev)
+    gy = torch.randn_like(k)
+    qd, kd, vd = (t.detach().requires_grad_(True) for t in (q, k, v))
+    big1 = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    big2 = torch.empty_like(big1)
+
+    def train_step():
+        F.flare_multihead_mixer(qd, kd, vd).backward(gy)
+        qd.grad = kd.grad = vd.grad = None
+
+    loads = {"mixer forward (headline shape)": lambda: F.flare_multihead_mixer(q, k, v),
+             "mixer forward + backward (headline shape)": train_step,
+             "device-to-device copy of 1 GiB": lambda: big2.copy_(big1)}
+    rows = {"idle": _smi_sample()}
+    try:
+        cap = subprocess.run(["rocm-smi", "--showmaxpower"], capture_output=True, text=True, timeout=30).stdout
+        cap = [ln.split(":")[-1].strip() for ln in cap.splitlines() if "Max Graphics Package Power" in ln]
+        rows["max_package_power_w"] = float(cap[0]) if cap else None
+    except Exception:
+        rows["max_package_power_w"] = None
+    ms_fwd = None
+    for name, fn in loads.items():
+        stop = threading.Event()
+        count = [0]
+
+        def run():
+            with torch.cuda.device(dev):
+                while not stop.is_set():
+                    for _ in range(100):
+                        fn()
+                    torch.cuda.synchronize(dev)
+                    count[0] += 100
+
+        th = threading.Thread(target=run)
+        th.start()
+        time.sleep(3.0)                   # let the clock settle under the load
+        c0, t0 = count[0], time.perf_counter()
+        samples = []
+        for _ in range(4):
+            samples.append(_smi_sample())
+            time.sleep(1.0)
+        c1, t1 = count[0], time.perf_counter()
+        stop.set()
+        th.join()
+        ms = (t1 - t0) * 1e3 / max(c1 - c0, 1)
+        good = [x for x in samples if x]
+        rows[name] = {"ms_per_call_sustained": round(ms, 4), "samples": good}
+        if name.startswith("mixer forward (") :
+            ms_fwd = ms
+    out = base_record(args, "FLARE mixer tokens/sec at N=1M,M=256,D=32 bf16 (sustained for seconds, power sampled)", B * N / (ms_fwd * 1e-3), "tokens/s",
+                      ms_fwd, "FLARE mixer forward B=1,H=8,N=1048576,M=256,D=32 (BASELINE config 3), run back to back while amd-smi is read")
+    out["roofline"] = None
+    out["power"] = rows
+    return out
+
+
 def bench_train(args, F, dev):
     """Headline configuration, forward + backward of the mixer (HIP kernels both ways)."""
     B, H, N, M, D = 1, 8, 1 << 20, 256, 32
@@ -742,7 +823,7 @@ def main():
     ap.add_argument("--no-torch-sdpa", action="store_true", help="skip the legs that time torch's own formulation (fused SDPA, einsum, torch layers) on the GPU")
     ap.add_argument("--lengths", default="1000000,100000", help="layer workload: token counts (the first one is the headline of the line)")
     ap.add_argument("--latents", default="128,512,2048", help="layer workload: latent counts")
-    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train", "linear", "fp32", "layer", "lra"], default="mixer",
+    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train", "linear", "fp32", "layer", "lra", "power"], default="mixer",
                     help="mixer = the headline configuration (default); the others are BASELINE configs 4, 5, 2")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -758,7 +839,7 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload != "mixer":
         fn = {"causal": bench_causal, "triple": bench_triple, "block": bench_block, "train": bench_train,
-              "linear": bench_linear, "fp32": bench_fp32, "layer": bench_layer, "lra": bench_lra}[args.workload]
+              "linear": bench_linear, "fp32": bench_fp32, "layer": bench_layer, "lra": bench_lra, "power": bench_power}[args.workload]
         print(json.dumps(fn(args, F, dev)))
         return
     B, H, N, M, D = 1, 8, 1 << 20, 256, 32
