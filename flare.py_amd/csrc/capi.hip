@@ -581,12 +581,14 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
 }
 
 namespace {
-// Argument block of the fp32 half backwards: the whole-mixer workspace layout, one term of dS switched off.
+// Argument block of the half backwards: the whole-mixer workspace layout, one term of dS switched off (fp32: compiled
+// out; bf16 / f16: its softmax weights forced to zero through a log-sum-exp of 1e30, see bwd_half_prep_kernel).
 int half_bwd_args(flare::MixerBwdArgs& a, const FlareMixerDesc* desc, void* workspace, size_t workspace_bytes)
 {
     int rc = check_bwd(desc);
     if (rc != FLARE_OK) return rc;
-    if (desc->dtype != FLARE_DT_F32) return fail(FLARE_EUNSUPPORTED, "the half backwards cover fp32 (got dtype %d)", desc->dtype);
+    if (desc->dtype != FLARE_DT_F32 && drop_threshold(desc) != 0)
+        return fail(FLARE_EUNSUPPORTED, "the bf16 / f16 half backwards do not take attention dropout");
     const BwdPlan p = plan_bwd(desc);
     if (!workspace) return fail(FLARE_EWORKSPACE, "workspace is NULL");
     if (workspace_bytes < p.total) return fail(FLARE_EWORKSPACE, "workspace has %zu bytes, %zu needed", workspace_bytes, p.total);
@@ -630,9 +632,9 @@ int flare_gather_bwd(const FlareMixerDesc* desc, const void* q, const void* k, c
     if (rc != FLARE_OK) return rc;
     if (!q || !k || !v || !z || !lse_lat || !dz || !dq || !dk || !dv)
         return fail(FLARE_EINVAL, "q, k, v, z, lse_lat, dz, dq, dk, dv must not be NULL");
-    const void* ptrs[7] = {q, k, v, z, dz, dk, dv};
+    const void* ptrs[8] = {q, k, v, z, dz, dq, dk, dv};
     for (const void* p : ptrs)
-        if (!aligned16(p)) return fail(FLARE_EINVAL, "q, k, v, z, dz, dk, dv must be 16-byte aligned");
+        if (!aligned16(p)) return fail(FLARE_EINVAL, "q, k, v, z, dz, dq, dk, dv must be 16-byte aligned");
     a.half = 1;
     a.q = q; a.k = k; a.v = v; a.z = z; a.lse_lat = lse_lat;
     a.dz = const_cast<float*>(dz);                 // read only in this mode
@@ -641,6 +643,8 @@ int flare_gather_bwd(const FlareMixerDesc* desc, const void* q, const void* k, c
     for (int i = 0; i < 3; ++i) a.ys[i] = a.dys[i] = a.vs[i];
     a.lse_tok = a.delta_tok;
     a.dq = dq; a.dk = dk; a.dv = dv;
+    if (desc->dtype != FLARE_DT_F32)
+        return hip_status(flare::launch_mixer_bwd(a, desc->dtype, static_cast<hipStream_t>(stream)), "gather backward launch");
     return hip_status(flare::launch_mixer_bwd_f32(a, static_cast<hipStream_t>(stream)), "fp32 gather backward launch");
 }
 
@@ -654,9 +658,11 @@ int flare_scatter_bwd(const FlareMixerDesc* desc, const void* q, const void* k, 
     if (!q || !k || !z || !y || !lse_tok || !dy || !dy_stride || !dq || !dk || !dz)
         return fail(FLARE_EINVAL, "q, k, z, y, lse_tok, dy, dy_stride, dq, dk, dz must not be NULL");
     if (!strides_mult4(dy_stride) || dy_stride[2] < desc->D) return fail(FLARE_EINVAL, "dy strides must be multiples of 16 bytes and its rows >= D");
-    const void* ptrs[7] = {q, k, z, y, dy, dk, dz};
+    const void* ptrs[8] = {q, k, z, y, dy, dq, dk, dz};
     for (const void* p : ptrs)
-        if (!aligned16(p)) return fail(FLARE_EINVAL, "q, k, z, y, dy, dk, dz must be 16-byte aligned");
+        if (!aligned16(p)) return fail(FLARE_EINVAL, "q, k, z, y, dy, dq, dk, dz must be 16-byte aligned");
+    if (desc->dtype != FLARE_DT_F32 && !strides_mult8(dy_stride))
+        return fail(FLARE_EINVAL, "dy strides must be multiples of 8 elements");
     a.half = 2;
     a.q = q; a.k = k; a.z = z; a.y = y; a.dy = dy; a.lse_tok = lse_tok;
     for (int i = 0; i < 3; ++i) a.dys[i] = dy_stride[i];
@@ -666,6 +672,8 @@ int flare_scatter_bwd(const FlareMixerDesc* desc, const void* q, const void* k, 
     for (int i = 0; i < 3; ++i) a.vs[i] = a.ks[i];
     a.lse_lat = a.delta_lat;
     a.dq = dq; a.dk = dk; a.dv = nullptr;
+    if (desc->dtype != FLARE_DT_F32)
+        return hip_status(flare::launch_mixer_bwd(a, desc->dtype, static_cast<hipStream_t>(stream)), "scatter backward launch");
     return hip_status(flare::launch_mixer_bwd_f32(a, static_cast<hipStream_t>(stream)), "fp32 scatter backward launch");
 }
 

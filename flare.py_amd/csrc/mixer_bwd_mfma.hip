@@ -38,6 +38,7 @@
 //   dz_m = sum_n K2 Bt dy_n,  dv_n = sum_m K1 A dz_m,  dS = A (K1 <dz_m,v_n> - Delta_m) + Bt (K2 <dy_n,z_m> - delta_n)
 // with the same Delta_m = <dz_m, z_m> and delta_n = <dy_n, y_n> (sums over the kept weights already).  These problems
 // take the two-exponential form with every additive term applied element by element.
+#include <algorithm>
 #include <type_traits>
 
 #include "common.hpp"
@@ -530,10 +531,36 @@ __global__ __launch_bounds__(256) void bwd_merge_kernel(MixerBwdArgs a)
         for (int o = 1; o < dq4; o <<= 1) delta += __shfl_xor(delta, o);   // the threads of a row are neighbours
         if (live) {
             *reinterpret_cast<f32x4*>(a.dz + r * a.D + d) = s;
-            if (d == 0) a.delta_lat[r] = delta;
+            // scatter half alone: the array stands in for lse_lat there and keeps the value that switches the gather term off
+            if (d == 0 && a.half != 2) a.delta_lat[r] = delta;
         }
     } else if (live) {
         *reinterpret_cast<f32x4*>(a.dq + r * a.D + d) = s * a.scale;
+    }
+}
+
+// The halves of the mixer differentiated alone run the whole mixer's kernels with the other half's softmax weights
+// forced to zero: a log-sum-exp of 1e30 makes exp2(S - 1.44e30) vanish, and every term that multiplies it stays
+// finite.  Gather half (a.half == 1, dz given): lse_tok, delta_tok (one array) and rho_min are filled with 1e30 and
+// Delta_m = <dz_m, z_m> is formed here instead of in the dz pass's merge.  Scatter half (a.half == 2): delta_lat, which
+// stands in for lse_lat, is filled with 1e30 (that batch element then takes the two-exponential form).
+__global__ __launch_bounds__(256) void bwd_half_prep_kernel(MixerBwdArgs a)
+{
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x, step = (int64_t)gridDim.x * 256;
+    const int64_t lat = (int64_t)a.B * a.H * a.M;
+    if (a.half == 2) {
+        for (int64_t i = t; i < lat; i += step) a.delta_lat[i] = 1.0e30f;
+        return;
+    }
+    for (int64_t i = t; i < (int64_t)a.B * a.H * a.N; i += step) a.delta_tok[i] = 1.0e30f;
+    for (int64_t i = t; i < (int64_t)a.B * a.H * a.n_splits0; i += step) a.rho_min[i] = 1.0e30f;
+    for (int64_t r = t; r < lat; r += step) {
+        float s = 0.f;
+        for (int d = 0; d < a.D; d += 4) {
+            const f32x4 x = *reinterpret_cast<const f32x4*>(a.dz + r * a.D + d), y = *reinterpret_cast<const f32x4*>(a.z + r * a.D + d);
+            s += x[0] * y[0] + x[1] * y[1] + x[2] * y[2] + x[3] * y[3];
+        }
+        a.delta_lat[r] = s;
     }
 }
 
@@ -834,7 +861,7 @@ __global__ __launch_bounds__(64 * kTokWaves<D>, 1) void bwd_tok_kernel(MixerBwdA
                 }
             };
             put(dk, a.dks[2], adk[tw]);
-            put(dv, a.dvs[2], adv[tw]);
+            if (a.dv) put(dv, a.dvs[2], adv[tw]);
         }
     }
     };
@@ -868,14 +895,24 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
     MixerBwdArgs a0 = a;          // the dz pass and its merge work in the dz pass's own split of the token axis
     a0.n_splits = a.n_splits0;
     a0.tokens_per_split = a.tokens_per_split0;
-    // bf16 at D = 32 without dropout: the token-parallel dz pass on the 32x32x16 product
-    const bool dz32 = !DROPK && !a.no_mfma32 && std::is_same<T, bf16_t>::value && bwd_dz32_supported(1, a.M, D);
-    hipError_t e = dz32 ? launch_bwd_dz32(a0, st) : lat_launch<T, D, 0, DROPK>(a0, st);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(bwd_merge_kernel<0>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a0);
+    // bf16 at D = 32 without dropout: the token-parallel passes on the 32x32x16 product.  The scatter half alone stays on
+    // the two-exponential form, which only the 16x16x32 token and dq passes run at full speed.
+    const bool mfma32 = !DROPK && !a.no_mfma32 && std::is_same<T, bf16_t>::value && bwd_dz32_supported(1, a.M, D);
+    const bool dz32 = mfma32, dq32 = mfma32 && a.half != 2;
+    hipError_t e = hipSuccess;
+    if (a.half != 0) {
+        if (DROPK) return hipErrorInvalidValue;
+        const int64_t items = std::max<int64_t>((int64_t)a.B * a.H * (a.half == 1 ? a.N : a.M), lat);
+        hipLaunchKernelGGL(bwd_half_prep_kernel, dim3((unsigned)std::min<int64_t>((items + 255) / 256, 4096)), dim3(256), 0, st, a);
+    }
+    if (a.half != 1) {      // the gather half is handed dz
+        e = dz32 ? launch_bwd_dz32(a0, st) : lat_launch<T, D, 0, DROPK>(a0, st);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(bwd_merge_kernel<0>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a0);
+    }
     // the token pass on the 32x32x16 product takes the (b,h) of the unshifted one-exponential form; the kernel below
     // then only works on the others (normally none: its workgroups return at once)
-    const bool tok32 = dz32 && bwd_tok32_supported(1, a.M, D);
+    const bool tok32 = dq32 && bwd_tok32_supported(1, a.M, D);
     if (tok32) {
         e = launch_bwd_tok32(a, st);
         if (e != hipSuccess) return e;
@@ -906,7 +943,7 @@ hipError_t bwd_all(const MixerBwdArgs& a, hipStream_t st)
             hipLaunchKernelGGL(kern, dim3((unsigned)((a.N + tpw - 1) / tpw), a.H, a.B), dim3(64 * kTokWaves<D>), lds, st, ac, (int)tpw);
         }
     }
-    e = dz32 ? launch_bwd_dq32(a, st) : lat_launch<T, D, 1, DROPK>(a, st);
+    e = dq32 ? launch_bwd_dq32(a, st) : lat_launch<T, D, 1, DROPK>(a, st);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(bwd_merge_kernel<1>, dim3((unsigned)((lat * (D / 4) + 255) / 256)), dim3(256), 0, st, a);
     return hipGetLastError();

@@ -534,8 +534,7 @@ def flare_multihead_mixer(q, k, v, scale: float = 1.0, key_mask=None, return_z: 
     dropout_p > 0 drops entries of both softmaxes' weights the way torch's scaled_dot_product_attention does
     in training (lra/models/backends.py:592,605-606); the mask is a function of dropout_seed (drawn from torch's
     default generator when None), so the backward recomputes it.  The 32x32x16 kernels carry no dropout: 16-bit problems
-    run on the 16x16x32 kernels (element-wise exact passes) and differentiate through the torch recomputation, fp32
-    problems run forward and backward on the fp32 matrix-core kernels.
+    run forward and backward on the 16x16x32 kernels, fp32 problems on the fp32 matrix-core kernels.
     """
     ac = _autocast_dtype(k)
     if ac is not None:
@@ -617,7 +616,7 @@ def _mixer_odd_latents(q, k, v, scale, key_mask, return_z, n_splits, token_major
     weight: k receives one extra column of ones and the dead queries hold a large negative number there (the real
     ones 0; -16384, or -256 / scale when the scale is small, so that scale * bias stays below -200), which takes
     their scores out of every token's softmax.  The extra column rides in the zero padding of the head dim (D grows to
-    the next of 16, 32, 64 that leaves room for it).  Gradients come from the two halves' torch recomputation."""
+    the next of 16, 32, 64 that leaves room for it).  Gradients come from the two halves' own backward."""
     M, D = q.shape[-2], k.shape[-1]
     Mp = -(-M // 32) * 32
     Dp = 16 if D < 16 else 32 if D < 32 else 64
@@ -738,8 +737,11 @@ def _half_torch_grad(which, q, k, x, scale, key_mask, g):
 
 
 def _half_hip_ok(q, k, other, key_mask, force_generic) -> bool:
-    """True when the fp32 HIP backward of a half (flare_gather_bwd / flare_scatter_bwd) covers the problem."""
-    if force_generic or k.dtype != torch.float32 or q.dtype != torch.float32 or other.dtype != torch.float32 or not k.is_cuda:
+    """True when the HIP backward of a half (flare_gather_bwd / flare_scatter_bwd) covers the problem: q and k of one
+    dtype, `other` (v of the gather, z of the scatter) of that dtype or, for z, fp32."""
+    if force_generic or q.dtype != k.dtype or other.dtype not in (k.dtype, torch.float32) or not k.is_cuda:
+        return False
+    if k.dtype not in (torch.float32, torch.bfloat16, torch.float16):
         return False
     k = _rows_last_contig(k)
     q4 = _q4(q, k.shape[0])
@@ -751,40 +753,41 @@ def _half_hip_ok(q, k, other, key_mask, force_generic) -> bool:
 
 
 def _half_hip_grad(which, q, k, x, z, aux, scale, key_mask, g):
-    """Gradients of a half from the fp32 HIP kernels.  gather: x = v, aux = lse_lat, g = dz -> (dq, dk, dv);
+    """Gradients of a half from the HIP kernels.  gather: x = v, aux = lse_lat, g = dz -> (dq, dk, dv);
     scatter: x = y, aux = lse_tok, g = dy -> (dq, dk, dz).  A key mask is handled as in _MixerFn.backward."""
     lib = _lib.load()
     k = _rows_last_contig(k)
     B, H, N, D = k.shape
     q4 = _q4(q, B)
     M = q4.shape[2]
+    al = 4 if k.dtype == torch.float32 else 8          # strides in elements that keep rows 16-byte aligned
     keep = None
     if key_mask is not None:
         keep = key_mask.to(torch.bool)
         m4 = keep[:, None, :, None]
         k = torch.where(m4, k, k.new_zeros(()))
-    z = z.contiguous()
+    z32 = z.to(torch.float32).contiguous()
     dq = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
-    dk = torch.empty((B, H, N, D), dtype=torch.float32, device=k.device)
+    dk = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
     if which == "gather":
         v = _rows_last_contig(x)
         aux = aux.contiguous()
         if keep is not None:
             v = torch.where(m4, v, v.new_zeros(()))
             aux = torch.where(torch.isfinite(aux), aux, aux.new_tensor(1e30))
-        if v.data_ptr() % 16 or any(s % 4 for s in v.stride()[:3]):
+        if v.data_ptr() % 16 or any(s % al for s in v.stride()[:3]):
             v = v.contiguous()
         gz = g.to(torch.float32).contiguous()
         d = _mixer_desc(q4, k, v, None, scale, 0, False)
-        out = torch.empty((B, H, N, D), dtype=torch.float32, device=k.device)
+        out = torch.empty((B, H, N, D), dtype=k.dtype, device=k.device)
     else:
         y = x.contiguous()
-        gy = g.to(torch.float32)
+        gy = g.to(k.dtype)
         aux = aux.contiguous()
         if keep is not None:
             gy = torch.where(m4, gy, gy.new_zeros(()))
             aux = torch.where(keep[:, None, :], aux, aux.new_tensor(1e30))
-        if gy.stride(-1) != 1 or any(s % 4 for s in gy.stride()[:3]) or gy.data_ptr() % 16:
+        if gy.stride(-1) != 1 or any(s % al for s in gy.stride()[:3]) or gy.data_ptr() % 16:
             gy = gy.contiguous()
         d = _mixer_desc(q4, k, k, y, scale, 0, False)
         out = torch.empty((B, H, M, D), dtype=torch.float32, device=k.device)
@@ -794,18 +797,20 @@ def _half_hip_grad(which, q, k, x, z, aux, scale, key_mask, g):
     st = C.c_void_p(_stream_ptr(k.device))
     with _on_device(k.device):
         if which == "gather":
-            rc = lib.flare_gather_bwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(z), _ptr(aux), _ptr(gz), _ptr(dq), _ptr(dk),
+            rc = lib.flare_gather_bwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(v), _ptr(z32), _ptr(aux), _ptr(gz), _ptr(dq), _ptr(dk),
                                       _ptr(out), _ptr(ws), ws.numel(), st)
         else:
-            rc = lib.flare_scatter_bwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(z), _ptr(y), _ptr(aux), _ptr(gy), _s3(gy), _ptr(dq),
+            rc = lib.flare_scatter_bwd(C.byref(d), _ptr(q4), _ptr(k), _ptr(z32), _ptr(y), _ptr(aux), _ptr(gy), _s3(gy), _ptr(dq),
                                        _ptr(dk), _ptr(out), _ptr(ws), ws.numel(), st)
     _lib.check(rc, "flare_gather_bwd" if which == "gather" else "flare_scatter_bwd")
     if keep is not None:
         dk = torch.where(m4, dk, dk.new_zeros(()))
         if which == "gather":
             out = torch.where(m4, out, out.new_zeros(()))
+    if which == "scatter":
+        out = out.to(z.dtype)
     gq = dq.sum(0) if q.dim() == 3 else dq
-    return gq, dk, out
+    return gq.to(q.dtype), dk, out
 
 
 class _GatherFn(torch.autograd.Function):
@@ -856,8 +861,8 @@ class _ScatterFn(torch.autograd.Function):
 def flare_gather(q, k, v, scale: float = 1.0, key_mask=None, n_splits: int = 0,
                  force_generic: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
     """z [B,H,M,D] fp32 = softmax_n(scale q k^T) v and lse [B,H,M] (natural log).
-    Differentiable in q, k, v (the backward recomputes the scores with torch ops: for models that put
-    layers between the two halves; the whole mixer has its own HIP backward)."""
+    Differentiable in q, k, v (flare_gather_bwd where the HIP backward covers the shape, otherwise a recomputation of the
+    scores with torch ops): for models that put layers between the two halves; the whole mixer has its own backward."""
     D = k.shape[-1]
     pad = _narrow_head_pad(q, k, force_generic) if q.dtype == k.dtype == v.dtype else 0
     if pad:

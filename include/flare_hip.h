@@ -239,7 +239,8 @@ int flare_mixer_bwd(const FlareMixerDesc* desc, const void* q, const void* k, co
                     const int64_t dy_stride[3], float* dq, void* dk, void* dv,
                     void* workspace, size_t workspace_bytes, void* stream);
 
-/* Backward of the two halves called separately, fp32 only (same shapes and workspace as flare_mixer_bwd; models that
+/* Backward of the two halves called separately (same dtypes, shapes and workspace as flare_mixer_bwd, no dropout in
+ * bf16 / f16; dk, dv in the element type, dy in the element type with strides that keep rows 16-byte aligned; models that
  * put layers between the halves: pdebench/models/flare_ablations.py:19-311 of the reference).  A key mask is handled
  * around them as for flare_mixer_bwd.
  * flare_gather_bwd:  gradient of flare_gather_fwd (the first scaled_dot_product_attention(q, k, v)): from dz

@@ -177,9 +177,12 @@ def test_new_struct_sizes_and_entry_point_validation():
     assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(dtype=_lib.DT_F32), C.byref(need)) == _lib.FLARE_OK     # fp32 kernels
     assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(dtype=_lib.DT_F32, M=40), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
     assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(dtype=_lib.DT_F32, D=24), C.byref(need)) == _lib.FLARE_EUNSUPPORTED
-    # the halves' backward: fp32 only, arguments checked before anything is launched
+    # the halves' backward: every dtype (16-bit without dropout), arguments checked before anything is launched
     f = _mixer_desc(dtype=_lib.DT_F32)
-    assert lib.flare_gather_bwd(d, *([None] * 9), None, 0, None) == _lib.FLARE_EUNSUPPORTED
+    assert lib.flare_gather_bwd(d, *([None] * 9), None, 0, None) == _lib.FLARE_EWORKSPACE
+    d.dropout_p = 0.25
+    assert lib.flare_gather_bwd(d, *([None] * 9), None, 0, None) == _lib.FLARE_EUNSUPPORTED and "dropout" in _lib.last_error()
+    d.dropout_p = 0.0
     assert lib.flare_gather_bwd(f, *([None] * 9), None, 0, None) == _lib.FLARE_EWORKSPACE
     assert lib.flare_scatter_bwd(f, *([None] * 6), None, None, None, None, None, 0, None) == _lib.FLARE_EWORKSPACE
     assert lib.flare_mixer_bwd_workspace_bytes(_mixer_desc(M=256, D=64), C.byref(need)) == _lib.FLARE_OK      # one LDS-full exactly

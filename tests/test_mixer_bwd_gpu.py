@@ -186,6 +186,49 @@ def test_fp32_halves_backward_vs_autograd_oracle(dev, shape, masked):
         assert err <= 1e-4, f"{name} rel-L2 {err:.3e}"
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,masked", [((1, 2, 777, 64, 32), False), ((2, 2, 1000, 128, 16), True), ((1, 1, 300, 256, 64), False),
+                                          ((2, 3, 97, 96, 32), True), ((1, 1, 1300, 512, 32), False), ((2, 2, 4000, 256, 32), False),
+                                          ((3, 1, 2100, 128, 32), True)])
+def test_16bit_halves_backward_vs_autograd_oracle(dev, dtype, shape, masked):
+    """The two halves with a layer between them in bf16 / f16 (pdebench/models/flare_ablations.py under autocast): gradients
+    from flare_gather_bwd / flare_scatter_bwd, which run the whole mixer's kernels with the other half's softmax weights
+    switched off, against fp64 autograd through the explicit formulas on the same 16-bit inputs.  Bars: bf16 3e-2, f16 1e-2
+    relative L2; z passes through the layer in fp32 here, so the only rounding is the kernels' own."""
+    B, H, N, M, D = shape
+    q, k, v, gy = make(*shape, dtype, seed=5 + N)
+    w = torch.randn(D, D, generator=torch.Generator().manual_seed(1)) * D ** -0.5
+    mask = None
+    if masked:
+        mask = torch.ones(B, N, dtype=torch.bool)
+        mask[0, N // 2:] = False
+        mask[-1, ::4] = False
+        if B > 2:
+            mask[1] = False          # a batch element without tokens
+    qd, kd, vd, wd = (t.to(dev).requires_grad_(True) for t in (q, k, v, w))
+    md = None if mask is None else mask.to(dev)
+    assert FN._half_hip_ok(qd, kd, vd, md, False)
+    with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CUDA]) as prof:
+        z, _ = F.flare_gather(qd, kd, vd, scale=0.9, key_mask=md)
+        y = F.flare_scatter(qd, kd, torch.tanh(z @ wd), scale=0.9, key_mask=md)
+        y.backward(gy.to(dev))
+        torch.cuda.synchronize()
+    kernels = " ".join(e.key for e in prof.key_averages())
+    assert "bwd_half_prep_kernel" in kernels and "bwd_tok" in kernels, kernels
+    qr, kr, vr, wr = (t.double().requires_grad_(True) for t in (q, k, v, w))
+    zr = O.gather_explicit(qr, kr, vr, 0.9, mask)
+    zr = zr[0] if isinstance(zr, tuple) else zr
+    yr = O.scatter_explicit(qr, kr, torch.tanh(zr @ wr), 0.9, mask)
+    yr.backward(gy.double())
+    tol = 3e-2 if dtype == torch.bfloat16 else 1e-2
+    for name, got, ref in (("dq", qd.grad, qr.grad), ("dk", kd.grad, kr.grad), ("dv", vd.grad, vr.grad), ("dw", wd.grad, wr.grad)):
+        assert torch.isfinite(got).all(), name
+        err = float((got.cpu().double() - ref).norm() / ref.norm())
+        assert err <= tol, f"{name} rel-L2 {err:.3e}"
+    if masked:
+        assert (kd.grad[0, :, N // 2:] == 0).all() and (vd.grad[0, :, N // 2:] == 0).all()
+
+
 def test_lse_outputs(dev):
     q, k, v, _ = make(1, 2, 500, 64, 32, torch.bfloat16, seed=9)
     y, z, lse_lat, lse_tok = FN._mixer_forward(q.to(dev), k.to(dev), v.to(dev), 0.7, None, 0, False, False, True)
