@@ -87,6 +87,43 @@ __device__ __forceinline__ uint2 tr16(const void* lds_addr)
     return __builtin_bit_cast(uint2, r);
 }
 
+// The same read at a byte address in LDS plus a compile-time offset: the offset goes into the instruction's offset
+// field, so the many reads of one step share a few address registers (as pointers each would occupy its own).
+template <int OFF>
+__device__ __forceinline__ uint2 tr16_at(uint32_t lds_byte_addr)
+{
+    typedef s16x4 __attribute__((address_space(3))) * lds_ptr_t;
+    asm volatile("" ::: "memory");
+    const s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr_t)(uintptr_t)(lds_byte_addr + OFF));
+    asm volatile("" ::: "memory");
+    return __builtin_bit_cast(uint2, r);
+}
+
+// f(integral_constant<int, I>) for I = 0 .. N - 1, unrolled at compile time
+template <int N, int I = 0, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<N, I + 1>(f);
+    }
+}
+
+typedef uint32_t u32v2 __attribute__((ext_vector_type(2)));
+// An ordinary LDS read of a V (a scalar or a compiler vector type) at a byte address plus a compile-time offset (same reason).
+template <typename V, int OFF>
+__device__ __forceinline__ V lds_at(uint32_t lds_byte_addr)
+{
+    typedef const V __attribute__((address_space(3))) * ptr_t;
+    return *(ptr_t)(uintptr_t)(lds_byte_addr + OFF);
+}
+// Keeps the compiler from folding an address into the expressions that use it (it would re-derive one register per use).
+__device__ __forceinline__ uint32_t opaque(uint32_t x)
+{
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
 // The state's numerators and denominators are relative to a shift mu0[m] per latent, which cancels in
 // z = U/den.  The softmax over the latents of one token's scores needs ONE shift for all latents
 // instead: its weights are exp2(score - cref) = P[t,m] * exp2(mu0[m] - cref) with
@@ -559,6 +596,7 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
 //   U[own m] += sum_w' P_w'[:, m]^T V_w';   den += sum_w' cs_w'
 // U0 = the state at the start of the chunk, published by its owners as bf16 B operands in LDS.
 constexpr int kChunk = 64;
+#define FLARE_CHUNK_FENCE() __builtin_amdgcn_sched_barrier(0)
 
 template <int D> constexpr size_t causal_chunk_lds()
 {
@@ -581,14 +619,15 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     uint16_t* pt = vs + kChunk * VS;                                              // [4][M][16]
     uint16_t* gt = pt + 4 * M * 16;                                               // [4][M][16]
     u32x4* u0s = reinterpret_cast<u32x4*>(gt + 4 * M * 16);                       // [KS][DT][64]
-    float* cs = reinterpret_cast<float*>(u0s + KS * DT * 64);                     // [4][M]
+    float* cs = reinterpret_cast<float*>(u0s + KS * DT * 64);                     // [M][4]: column sums of the four waves' P
     u32x4* fops = reinterpret_cast<u32x4*>(cs + 4 * M);                           // [KS][4]: weight factors as B operands
     float* mu0s = reinterpret_cast<float*>(fops + KS * 4);                        // [M] shift of each latent (log2 units)
     float* fws = mu0s + M;                                                        // [M] weight factor exp2(mu0 - cref)
     __shared__ int bad_flag;
 
-    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
+    const int tid = threadIdx.x, lane = tid & 63, g = lane >> 4, c16 = lane & 15;
     const int bh = blockIdx.x, b = bh / a.H, h = bh % a.H, seg = blockIdx.y;
+    const int w = __builtin_amdgcn_readfirstlane(2 * seg >= a.n_segs ? 3 - (tid >> 6) : tid >> 6);
     const int n_lo = seg * a.seg_len, N = min(a.N, n_lo + a.seg_len);
     const bool single = a.n_segs == 1;
     float* seg_den = a.seg_den + ((int64_t)bh * a.n_slots + a.n_slots - 1) * M;        // staging slot of the final state
@@ -743,11 +782,62 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
                                                    P_::pack2(u1[0], u1[1]), P_::pack2(u1[2], u1[3])};
         }
     };
-    // operand with tokens in lanes and latents in k-slots from a [latent][token] tile (k-step ks = 32 latents)
-    auto tr_op = [&](const uint16_t* tile, int ks) {
-        const int r0 = ks * 32 + 4 * g + (c16 >> 2), piece = (c16 & 3) * 4;
-        const uint2 lo = tr16(tile + r0 * 16 + piece), hi = tr16(tile + (r0 + 16) * 16 + piece);
-        return u32x4{lo.x, lo.y, hi.x, hi.y};
+    // Transposing reads: byte addresses in LDS of the lane's piece in a [latent][16 tokens] tile and in the V chunk; every
+    // read adds a compile-time offset to one of these.
+    const uint32_t lane_t = (4 * g + (c16 >> 2)) * 32 + (c16 & 3) * 8;
+    const uint32_t pt_b = opaque((uint32_t)(uintptr_t)pt + lane_t);                  // P^T of wave 0
+    const uint32_t ptw_b = opaque(pt_b + w * (M * 32)), gtw_b = opaque((uint32_t)(uintptr_t)gt + w * (M * 32) + lane_t);
+    const uint32_t vs_b = opaque((uint32_t)(uintptr_t)vs + (4 * g + (c16 >> 2)) * (VS * 2) + (c16 & 3) * 8);    // V rows of wave 0's tokens
+    const uint32_t vsw_b = opaque(vs_b + w * (16 * VS * 2));
+    // ordinary reads: operand sets by lane, per-latent tables by column c16, P^T rows of the wave's own latents
+    const uint32_t qs_b = opaque((uint32_t)(uintptr_t)qs + lane * 16), u0_b = opaque((uint32_t)(uintptr_t)u0s + lane * 16);
+    const uint32_t cs_b = opaque((uint32_t)(uintptr_t)cs + c16 * 16), fo_b = opaque((uint32_t)(uintptr_t)fops + g * 16);
+    const uint32_t mu_b = opaque((uint32_t)(uintptr_t)mu0s + c16 * 4);        // fws follows mu0s
+    const uint32_t up_b = opaque((uint32_t)(uintptr_t)pt + (m0 + c16) * 32 + g * 8);
+    // operands with tokens in lanes and latents in k-slots from a [latent][token] tile (k-step ks = 32 latents)
+    auto tr_ops = [&](uint32_t tile_b, auto off_c, u32x4 (&o)[KS]) {
+        constexpr int OFF = decltype(off_c)::value;
+        static_assert(KS == 4, "four k-steps of 32 latents");
+        const uint2 l0 = tr16_at<OFF>(tile_b), h0 = tr16_at<OFF + 512>(tile_b);
+        const uint2 l1 = tr16_at<OFF + 1024>(tile_b), h1 = tr16_at<OFF + 1536>(tile_b);
+        const uint2 l2 = tr16_at<OFF + 2048>(tile_b), h2 = tr16_at<OFF + 2560>(tile_b);
+        const uint2 l3 = tr16_at<OFF + 3072>(tile_b), h3 = tr16_at<OFF + 3584>(tile_b);
+        o[0] = u32x4{l0.x, l0.y, h0.x, h0.y};
+        o[1] = u32x4{l1.x, l1.y, h1.x, h1.y};
+        o[2] = u32x4{l2.x, l2.y, h2.x, h2.y};
+        o[3] = u32x4{l3.x, l3.y, h3.x, h3.y};
+    };
+    // V rows of one wave's 16 tokens as B operands (token k-slots, lane = column d), DT column tiles
+    auto v_ops = [&](uint32_t v_b, auto off_c, uint2 (&o)[DT]) {
+        constexpr int OFF = decltype(off_c)::value;
+        o[0] = tr16_at<OFF>(v_b);
+        o[1] = tr16_at<OFF + 32>(v_b);
+        if constexpr (DT == 4) {
+            o[2] = tr16_at<OFF + 64>(v_b);
+            o[3] = tr16_at<OFF + 96>(v_b);
+        }
+    };
+
+    // Everything a step reads from LDS is requested in one batch ahead of the step and held in registers, with the
+    // compiler kept from moving the requests next to their uses (it otherwise issues them one by one, each followed by a
+    // wait: the chunk is a dependent chain, and with two waves per SIMD nothing else covers an LDS round trip).
+    u32x4 qo[CTA][KD];      // q operands of the score product: constant, re-read per chunk (64 registers held all chunk long cost more)
+    float mu0[CTA];
+    auto load_q = [&]() {
+        static_for<CTA>([&](auto ct_c) {
+            constexpr int ct = decltype(ct_c)::value;
+            mu0[ct] = lds_at<float, ct * 64>(mu_b);
+            static_for<KD>([&](auto kd_c) {
+                constexpr int kd = decltype(kd_c)::value;
+                qo[ct][kd] = lds_at<u32x4, (ct * KD + kd) * 1024>(qs_b);
+            });
+        });
+    };
+    // operands of one 16-token tile of another wave against this wave's G: its P^T (A operands) and its V rows
+    auto load_pair = [&](auto wp_c, u32x4 (&po)[KS], uint2 (&vo)[DT]) {
+        constexpr int WP = decltype(wp_c)::value;
+        tr_ops(pt_b, std::integral_constant<int, WP * M * 32>{}, po);
+        v_ops(vs_b, std::integral_constant<int, WP * 16 * VS * 2>{}, vo);
     };
 
     bool bad = false;
@@ -757,6 +847,7 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
     __syncthreads();                                        // q operands
 
     for (int n0 = n_lo; n0 < N; n0 += kChunk) {
+        load_q();
         const int tbase = n0 + 16 * w;
         const int tbw = min(16, max(0, N - tbase));        // valid tokens of this wave in the chunk
         // Tokens past the end of the segment (only its last chunk can have any) get probability 0 through the initial
@@ -771,8 +862,6 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
         load_chunk(n0 + kChunk, kn);
 
         // ---- token side, part 1: scores, P, column sums; publish P^T ----
-        // (staged over the eight latent tiles: every LDS read before the first LDS write, so that the reads
-        // can be issued together instead of one tile's round trip after the other)
         float p[CTA][4];
         uint2 ppk[CTA];
         {
@@ -781,14 +870,13 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
             for (int ct = 0; ct < CTA; ++ct) {
                 f32x4 s = absent;
 #pragma unroll
-                for (int kd = 0; kd < KD; ++kd) s = M_::mma32(ka[kd], qs[(ct * KD + kd) * 64 + lane], s);
+                for (int kd = 0; kd < KD; ++kd) s = M_::mma32(ka[kd], qo[ct][kd], s);
                 sc[ct] = s;
             }
 #pragma unroll
             for (int ct = 0; ct < CTA; ++ct) {
-                const float mu0 = mu0s[ct * 16 + c16];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) p[ct][r] = fast_exp2(sc[ct][r] - mu0);
+                for (int r = 0; r < 4; ++r) p[ct][r] = fast_exp2(sc[ct][r] - mu0[ct]);
                 ppk[ct] = make_uint2(P_::pack2(p[ct][0], p[ct][1]), P_::pack2(p[ct][2], p[ct][3]));
             }
             f32x4 csv[CTA];
@@ -796,68 +884,127 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
             for (int ct = 0; ct < CTA; ++ct) csv[ct] = P_::mma16(ones4, ppk[ct], zf);
 #pragma unroll
             for (int ct = 0; ct < CTA; ++ct) {
-                if (g == 0) cs[w * M + ct * 16 + c16] = csv[ct][0];
+                if (g == 0) cs[(ct * 16 + c16) * 4 + w] = csv[ct][0];
                 *reinterpret_cast<uint2*>(ptw + (ct * 16 + c16) * 16 + 4 * g) = ppk[ct];
             }
         }
         __syncthreads();                                    // P^T, cs, V chunk, U0 operands visible
 
         // ---- token side, part 2: running denominators, G ----
+        {
+            f32x4 c4[CTA];
+            float fw[CTA];      // the token's softmax weight over the latents is P * exp2(mu0 - cref)
+            static_for<CTA>([&](auto ct_c) {
+                constexpr int ct = decltype(ct_c)::value;
+                c4[ct] = lds_at<f32x4, ct * 256>(cs_b);
+                fw[ct] = lds_at<float, M * 4 + ct * 64>(mu_b);
+            });
+            FLARE_CHUNK_FENCE();
+            f32x4 dc[CTA];
 #pragma unroll
-        for (int ct = 0; ct < CTA; ++ct) {
-            const int m = ct * 16 + c16;
-            const float c0 = cs[m], c1 = cs[M + m], c2 = cs[2 * M + m], c3 = cs[3 * M + m];
-            float base = den0[ct];
-            if (w > 0) base += c0;
-            if (w > 1) base += c1;
-            if (w > 2) base += c2;
-            den0[ct] = den0[ct] + c0 + c1 + c2 + c3;        // same order in every wave
-            const f32x4 dc = P_::mma16(ltri, ppk[ct], zf);
-            float gv[4];
-            const float fw = fws[m];      // the token's softmax weight over the latents is P * exp2(mu0 - cref)
+            for (int ct = 0; ct < CTA; ++ct) dc[ct] = P_::mma16(ltri, ppk[ct], zf);
 #pragma unroll
-            for (int r = 0; r < 4; ++r)      // dcum >= the element's own P: clamped away from 0 it gives G = 0 where P = 0
-                gv[r] = p[ct][r] * fw * __builtin_amdgcn_rcpf(fmaxf(dc[r] + base, 1.17549435e-38f));
-            *reinterpret_cast<uint2*>(gtw + (ct * 16 + c16) * 16 + 4 * g) = make_uint2(P_::pack2(gv[0], gv[1]), P_::pack2(gv[2], gv[3]));
+            for (int ct = 0; ct < CTA; ++ct) {
+                float base = den0[ct];
+                if (w > 0) base += c4[ct][0];
+                if (w > 1) base += c4[ct][1];
+                if (w > 2) base += c4[ct][2];
+                den0[ct] = den0[ct] + c4[ct][0] + c4[ct][1] + c4[ct][2] + c4[ct][3];        // same order in every wave
+                float gv[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r)      // dcum >= the element's own P: clamped away from 0 it gives G = 0 where P = 0
+                    gv[r] = p[ct][r] * fw[ct] * __builtin_amdgcn_rcpf(fmaxf(dc[ct][r] + base, 1.17549435e-38f));
+                *reinterpret_cast<uint2*>(gtw + (ct * 16 + c16) * 16 + 4 * g) = make_uint2(P_::pack2(gv[0], gv[1]), P_::pack2(gv[2], gv[3]));
+            }
         }
-        u32x4 gop[KS], pop[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            gop[ks] = tr_op(gtw, ks);
-            pop[ks] = tr_op(ptw, ks);
-        }
+        // operands of the outputs: G and P of the wave's tokens, the weight factors, U0 (two column tiles at a time), the
+        // wave's own V rows, and the first of the earlier waves' tiles (w is uniform over the wave)
+        u32x4 gop[KS], pop[KS], fo[KS], uo[2][KS];
+        uint2 vd[DT];
+        u32x4 pa[KS], pb[KS];
+        uint2 va[DT], vb[DT];
+        auto load_u0 = [&](auto half_c) {
+            constexpr int h0 = decltype(half_c)::value * 2;
+            static_for<KS>([&](auto ks_c) {
+                constexpr int ks = decltype(ks_c)::value;
+                uo[0][ks] = lds_at<u32x4, (ks * DT + h0) * 1024>(u0_b);
+                uo[1][ks] = lds_at<u32x4, (ks * DT + h0 + 1) * 1024>(u0_b);
+            });
+        };
+        tr_ops(gtw_b, std::integral_constant<int, 0>{}, gop);
+        tr_ops(ptw_b, std::integral_constant<int, 0>{}, pop);
+        static_for<KS>([&](auto ks_c) {
+            constexpr int ks = decltype(ks_c)::value;
+            fo[ks] = lds_at<u32x4, ks * 64>(fo_b);
+        });
+        load_u0(std::integral_constant<int, 0>{});
+        FLARE_CHUNK_FENCE();
         // softmax sums over the latents of the wave's tokens (rows t = 4g + r, equal in every column)
         f32x4 rsum = zf;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) rsum = P_::mma32(pop[ks], fops[ks * 4 + g], rsum);
+        for (int ks = 0; ks < KS; ++ks) rsum = P_::mma32(pop[ks], fo[ks], rsum);
 
         // ---- outputs: G U0, then the chunk's own tokens up to and including this wave's ----
         f32x4 yacc[DT];
+        auto g_u0 = [&](int d0) {
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            f32x4 acc = zf;
+            for (int j = 0; j < 2; ++j) {
+                f32x4 acc = zf;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) acc = P_::mma32(gop[ks], u0s[(ks * DT + dt) * 64 + lane], acc);
-            yacc[dt] = acc;
-        }
-        for (int wp = 0; wp <= w; ++wp) {
-            f32x4 acct = zf;      // [tau of wave wp, t of this wave] = sum_m P[tau,m] G[t,m]
-            if (wp == w) {
+                for (int ks = 0; ks < KS; ++ks) acc = P_::mma32(gop[ks], uo[j][ks], acc);
+                yacc[d0 + j] = acc;
+            }
+        };
+        g_u0(0);
+        FLARE_CHUNK_FENCE();
+        if constexpr (DT == 4) load_u0(std::integral_constant<int, 1>{});
+        v_ops(vsw_b, std::integral_constant<int, 0>{}, vd);
+        if (w > 0) load_pair(std::integral_constant<int, 0>{}, pa, va);
+        FLARE_CHUNK_FENCE();
+        if constexpr (DT == 4) g_u0(2);
+        // [tau of wave wp, t of this wave] = sum_m P[tau,m] G[t,m], then times V of wave wp
+        auto pair = [&](const u32x4 (&po)[KS], const uint2 (&vo)[DT], bool diag) {
+            f32x4 acct = zf;
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) acct = P_::mma32(pop[ks], gop[ks], acct);
+            for (int ks = 0; ks < KS; ++ks) acct = P_::mma32(po[ks], gop[ks], acct);
+            if (diag) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acct[r] = (4 * g + r <= c16) ? acct[r] : 0.f;
-            } else {
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) acct = P_::mma32(tr_op(pt + wp * M * 16, ks), gop[ks], acct);
             }
             const uint2 aop = make_uint2(P_::pack2(acct[0], acct[1]), P_::pack2(acct[2], acct[3]));
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const uint2 vop = tr16(vs + (wp * 16 + 4 * g + (c16 >> 2)) * VS + dt * 16 + (c16 & 3) * 4);
-                yacc[dt] = P_::mma16(aop, vop, yacc[dt]);
+            for (int dt = 0; dt < DT; ++dt) yacc[dt] = P_::mma16(aop, vo[dt], yacc[dt]);
+        };
+        {
+            if (w > 1) load_pair(std::integral_constant<int, 1>{}, pb, vb);
+            FLARE_CHUNK_FENCE();
+            if (w > 0) {
+                pair(pa, va, false);
+                if (w > 2) load_pair(std::integral_constant<int, 2>{}, pa, va);
+                FLARE_CHUNK_FENCE();
+                if (w > 1) {
+                    pair(pb, vb, false);
+                    if (w > 2) pair(pa, va, false);
+                }
             }
+            pair(pop, vd, true);
         }
+        // operands of the state update (P^T of all four waves at this wave's latents, V of the whole chunk): requested ahead
+        // of the output's trip through LDS
+        uint2 uv[4][DT], up[4][MT];
+        v_ops(vs_b, std::integral_constant<int, 0>{}, uv[0]);
+        v_ops(vs_b, std::integral_constant<int, 16 * VS * 2>{}, uv[1]);
+        v_ops(vs_b, std::integral_constant<int, 32 * VS * 2>{}, uv[2]);
+        v_ops(vs_b, std::integral_constant<int, 48 * VS * 2>{}, uv[3]);
+        static_for<4>([&](auto wp_c) {
+            constexpr int wp = decltype(wp_c)::value;
+            static_for<MT>([&](auto mt_c) {
+                constexpr int mt = decltype(mt_c)::value;
+                const u32v2 t = lds_at<u32v2, wp * M * 32 + mt * 512>(up_b);
+                up[wp][mt] = make_uint2(t[0], t[1]);
+            });
+        });
+        FLARE_CHUNK_FENCE();
         // The next chunk's rows, requested at the top of this iteration, are waited for here, before the stores below
         // are issued: loads and stores complete in order on one counter, the stores sit under per-lane conditions, and
         // a wait placed at the hand-over after them could only wait for everything, store acknowledgements included.
@@ -884,26 +1031,26 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
                 }
                 *reinterpret_cast<uint2*>(gtw + (dt * 16 + c16) * 16 + 4 * g) = make_uint2(M_::pack2(o[0], o[1]), M_::pack2(o[2], o[3]));
             }
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                const uint2 o = tr16(gtw + (dt * 16 + 4 * g + (c16 >> 2)) * 16 + (c16 & 3) * 4);
-                if (c16 < tbw) *reinterpret_cast<uint2*>(y + (int64_t)(tbase + c16) * a.ys[2] + dt * 16 + 4 * g) = o;
-            }
         }
+        uint2 yo[DT];
+        yo[0] = tr16_at<0>(gtw_b);
+        yo[1] = tr16_at<512>(gtw_b);
+        if constexpr (DT == 4) {
+            yo[2] = tr16_at<1024>(gtw_b);
+            yo[3] = tr16_at<1536>(gtw_b);
+        }
+        FLARE_CHUNK_FENCE();
 
-        // ---- state update of the wave's own latents over all 64 tokens ----
+        // ---- state update of the wave's own latents over all 64 tokens (covers the transposition's round trip) ----
 #pragma unroll
-        for (int wp = 0; wp < 4; ++wp) {
-            uint2 vop[DT];
+        for (int wp = 0; wp < 4; ++wp)
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vop[dt] = tr16(vs + (wp * 16 + 4 * g + (c16 >> 2)) * VS + dt * 16 + (c16 & 3) * 4);
+            for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const uint2 pa = *reinterpret_cast<const uint2*>(pt + wp * M * 16 + (m0 + mt * 16 + c16) * 16 + 4 * g);
+                for (int dt = 0; dt < DT; ++dt) U[mt][dt] = P_::mma16(up[wp][mt], uv[wp][dt], U[mt][dt]);
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) U[mt][dt] = P_::mma16(pa, vop[dt], U[mt][dt]);
-            }
-        }
+        for (int dt = 0; dt < DT; ++dt)
+            if (c16 < tbw) *reinterpret_cast<uint2*>(y + (int64_t)(tbase + c16) * a.ys[2] + dt * 16 + 4 * g) = yo[dt];
 
         __syncthreads();                                    // everyone is done with V, U0, P^T of this chunk
         if (n0 + kChunk < N) {
