@@ -1042,12 +1042,17 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
         FLARE_CHUNK_FENCE();
 
         // ---- state update of the wave's own latents over all 64 tokens (covers the transposition's round trip) ----
+        // Two waves' tokens share one product over 32 tokens: k-slot 8g + j of the 16x16x32 instruction holds token 4g + j of
+        // the first wave for j < 4 and token 4g + j - 4 of the second otherwise, on both operands.
 #pragma unroll
-        for (int wp = 0; wp < 4; ++wp)
+        for (int h2 = 0; h2 < 4; h2 += 2)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
+            for (int mt = 0; mt < MT; ++mt) {
+                const u32x4 pa2 = u32x4{up[h2][mt].x, up[h2][mt].y, up[h2 + 1][mt].x, up[h2 + 1][mt].y};
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) U[mt][dt] = P_::mma16(up[wp][mt], uv[wp][dt], U[mt][dt]);
+                for (int dt = 0; dt < DT; ++dt)
+                    U[mt][dt] = P_::mma32(pa2, u32x4{uv[h2][dt].x, uv[h2][dt].y, uv[h2 + 1][dt].x, uv[h2 + 1][dt].y}, U[mt][dt]);
+            }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
             if (c16 < tbw) *reinterpret_cast<uint2*>(y + (int64_t)(tbase + c16) * a.ys[2] + dt * 16 + 4 * g) = yo[dt];
