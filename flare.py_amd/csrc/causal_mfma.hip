@@ -301,25 +301,25 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
         // three ahead as soon as its own has been used: loads are unconditional (rows past the end of
         // the segment repeat its last row) and never copied between registers, so that every wait counts
         // exactly what is in flight.
-        __shared__ __attribute__((aligned(16))) uint16_t v64[2][64][D + kVPad];
-        constexpr int VPT = 64 * (D / 8) / 256;     // 16-byte V chunks per thread and tile
-        static_assert(64 * (D / 8) == VPT * 256, "every thread stages the same number of V chunks");
-        struct Tile { u32x4 k[4][KD]; u32x4 v[VPT]; };
-        auto fetch = [&](int n0, Tile& t) {
-#pragma unroll
-            for (int sb = 0; sb < 4; ++sb) {
-                const int n = min(n0 + sb * 16 + c16, N - 1);
-#pragma unroll
-                for (int kd = 0; kd < KD; ++kd) t.k[sb][kd] = *reinterpret_cast<const u32x4*>(k + (int64_t)n * a.ks[2] + kd * 32 + g * 8);
-            }
+        // K and V tiles in LDS (K rows padded by 8 elements: the 16 rows a wave reads as one operand then start in 16
+        // different bank groups; V rows by kVPad for the transposing reads)
+        constexpr int KROW = (D + 8) * 2, VROW = (D + kVPad) * 2;       // row strides in bytes
+        __shared__ __attribute__((aligned(16))) uint8_t k64[2][64 * KROW];
+        __shared__ __attribute__((aligned(16))) uint8_t v64[2][64 * VROW];
+        constexpr int VPT = 64 * (D / 8) / 256;     // 16-byte K and V chunks per thread and tile
+        static_assert(64 * (D / 8) == VPT * 256, "every thread stages the same number of chunks");
+        struct Tile { u32x4 k[VPT]; u32x4 v[VPT]; };
+        auto fetch = [&](int n0, Tile& t) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
                 const int c = tid + i * 256, tok = c / (D / 8), ch = c % (D / 8);
-                t.v[i] = *reinterpret_cast<const u32x4*>(v + (int64_t)min(n0 + tok, N - 1) * a.vs[2] + ch * 8);
+                const int64_t row = min(n0 + tok, N - 1);
+                t.k[i] = *reinterpret_cast<const u32x4*>(k + row * a.ks[2] + ch * 8);
+                t.v[i] = *reinterpret_cast<const u32x4*>(v + row * a.vs[2] + ch * 8);
             }
         };
         // V rows of absent tokens are staged as zeros (their probabilities then add nothing to the numerators)
-        auto stage = [&](int n0, int buf, const Tile& t) {
+        auto stage = [&](int n0, int buf, const Tile& t) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < VPT; ++i) {
                 const int c = tid + i * 256, tok = c / (D / 8), ch = c % (D / 8);
@@ -330,15 +330,20 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
                         o[j] = P_::pack2(M_::unpack(uint16_t(t.v[i][j] & 0xffffu)), M_::unpack(uint16_t(t.v[i][j] >> 16)));
                 }
                 if (n0 + tok >= N) o = u32x4{0u, 0u, 0u, 0u};
-                *reinterpret_cast<u32x4*>(&v64[buf][tok][ch * 8]) = o;
+                *reinterpret_cast<u32x4*>(&k64[buf][tok * KROW + ch * 16]) = t.k[i];
+                *reinterpret_cast<u32x4*>(&v64[buf][tok * VROW + ch * 16]) = o;
             }
         };
+        // byte addresses in LDS of the lane's pieces: K row c16, 16 bytes at 8g elements; V row 4g + (c16 >> 2), piece c16 & 3
+        const uint32_t k_b = opaque((uint32_t)(uintptr_t)&k64[0][0] + c16 * KROW + g * 16);
+        const uint32_t v_b = opaque((uint32_t)(uintptr_t)&v64[0][0] + (4 * g + (c16 >> 2)) * VROW + (c16 & 3) * 8);
         // the tile's contribution, two 16-token blocks per product (k-slots 8g + i: token 4g + i of the first block,
         // 8g + 4 + i: of the second); the denominators count live tokens only (the A operand of their product holds
         // ones in the k-slots of live tokens)
-        auto work = [&](int n0, int buf, const Tile& t) {
-#pragma unroll
-            for (int sp = 0; sp < 2; ++sp) {
+        auto work = [&](int n0, auto buf_c) __attribute__((always_inline)) {
+            constexpr int KB = decltype(buf_c)::value * 64 * KROW, VB = decltype(buf_c)::value * 64 * VROW;
+            static_for<2>([&](auto sp_c) {
+                constexpr int sp = decltype(sp_c)::value;
                 const int tb = N - (n0 + sp * 32);   // tokens >= tb of this pair of blocks are beyond the part
                 u32x4 live8 = u32x4{ones4.x, ones4.y, ones4.x, ones4.y};
                 if (tb < 32) {
@@ -350,20 +355,26 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
                         live8[2 * hb + 1] = (t0 + 2 < tb ? one : 0u) | (t0 + 3 < tb ? one << 16 : 0u);
                     }
                 }
-                u32x4 vop[DT];
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    const uint2 lo = tr16(&v64[buf][sp * 32 + 4 * g + (c16 >> 2)][dt * 16 + (c16 & 3) * 4]);
-                    const uint2 hi = tr16(&v64[buf][sp * 32 + 16 + 4 * g + (c16 >> 2)][dt * 16 + (c16 & 3) * 4]);
+                // all operands of the pair of blocks requested at once
+                u32x4 ka[2][KD], vop[DT];
+                static_for<KD>([&](auto kd_c) {
+                    constexpr int kd = decltype(kd_c)::value;
+                    ka[0][kd] = lds_at<u32x4, KB + (2 * sp) * 16 * KROW + kd * 64>(k_b);
+                    ka[1][kd] = lds_at<u32x4, KB + (2 * sp + 1) * 16 * KROW + kd * 64>(k_b);
+                });
+                static_for<DT>([&](auto dt_c) {
+                    constexpr int dt = decltype(dt_c)::value;
+                    const uint2 lo = tr16_at<VB + sp * 32 * VROW + dt * 32>(v_b);
+                    const uint2 hi = tr16_at<VB + (sp * 32 + 16) * VROW + dt * 32>(v_b);
                     vop[dt] = u32x4{lo.x, lo.y, hi.x, hi.y};
-                }
+                });
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
                     f32x4 s0 = negmu[ct], s1 = negmu[ct];
 #pragma unroll
                     for (int kd = 0; kd < KD; ++kd) {
-                        s0 = M_::mma32(t.k[2 * sp][kd], qb[ct][kd], s0);
-                        s1 = M_::mma32(t.k[2 * sp + 1][kd], qb[ct][kd], s1);
+                        s0 = M_::mma32(ka[0][kd], qb[ct][kd], s0);
+                        s1 = M_::mma32(ka[1][kd], qb[ct][kd], s1);
                     }
                     const u32x4 ppk = u32x4{P_::pack2(fast_exp2(s0[0]), fast_exp2(s0[1])), P_::pack2(fast_exp2(s0[2]), fast_exp2(s0[3])),
                                             P_::pack2(fast_exp2(s1[0]), fast_exp2(s1[1])), P_::pack2(fast_exp2(s1[2]), fast_exp2(s1[3]))};
@@ -371,7 +382,7 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
 #pragma unroll
                     for (int dt = 0; dt < DT; ++dt) U[ct][dt] = P_::mma32(ppk, vop[dt], U[ct][dt]);
                 }
-            }
+            });
         };
         const int p_lo = seg * a.piece_len, p_hi = min(p_lo + a.piece_len, (a.n_segs - 1) * a.seg_len);
         for (int s = p_lo / a.seg_len; s <= (p_hi - 1) / a.seg_len; ++s) {
@@ -384,39 +395,32 @@ __global__ __launch_bounds__(256, 2) void causal_mfma_kernel(CausalArgs a, int s
             for (int dt = 0; dt < DT; ++dt) U[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
         __syncthreads();   // the part before has read its last tile
-        Tile ta, tb_, tc;
+        // Two register sets take turns: each is staged into LDS one tile ahead of its use and refilled at once with the
+        // tile two further on.  Loads are unconditional (rows past the end of the part repeat its last row) and never
+        // copied between registers, so that every wait counts exactly what is in flight.
+        Tile ta, tb_;
         fetch(n_lo, ta);
         fetch(n_lo + 64, tb_);
-        fetch(n_lo + 128, tc);
         stage(n_lo, 0, ta);
+        fetch(n_lo + 128, ta);
         __syncthreads();
-        // Whole groups of three tiles in a loop with one exit at its bottom, the last one or two tiles behind it: an
-        // exit from the middle of the group would reach the loop's head again in the compiler's control flow, and
-        // with prefetches in flight on that path every pass through the head would wait for all of them.
+        // Whole pairs of tiles in a loop with one exit at its bottom, a last odd tile behind it: an exit from the middle
+        // of the pair would reach the loop's head again in the compiler's control flow, and with prefetches in flight on
+        // that path every pass through the head would wait for all of them.
         const int tiles = (N - n_lo + 63) >> 6;
-        int buf = 0, n0 = n_lo;
-        for (int gi = 0; gi < tiles / 3; ++gi, n0 += 192) {
-            // tile n0 (K in ta, V staged in v64[buf]); the next tile's V goes into the other buffer meanwhile
-            work(n0, buf, ta);
-            fetch(n0 + 192, ta);
-            stage(n0 + 64, buf ^ 1, tb_);
+        int n0 = n_lo;
+        for (int gi = 0; gi < tiles / 2; ++gi, n0 += 128) {
+            // tile n0 (in buffer 0); the next tile goes into buffer 1 meanwhile
+            work(n0, std::integral_constant<int, 0>{});
+            stage(n0 + 64, 1, tb_);
+            fetch(n0 + 192, tb_);
             __syncthreads();
-            work(n0 + 64, buf ^ 1, tb_);
-            fetch(n0 + 256, tb_);
-            stage(n0 + 128, buf, tc);
+            work(n0 + 64, std::integral_constant<int, 1>{});
+            stage(n0 + 128, 0, ta);
+            fetch(n0 + 256, ta);
             __syncthreads();
-            work(n0 + 128, buf, tc);
-            fetch(n0 + 320, tc);
-            stage(n0 + 192, buf ^ 1, ta);
-            __syncthreads();
-            buf ^= 1;
         }
-        if (tiles % 3 >= 1) work(n0, buf, ta);
-        if (tiles % 3 == 2) {
-            stage(n0 + 64, buf ^ 1, tb_);
-            __syncthreads();
-            work(n0 + 64, buf ^ 1, tb_);
-        }
+        if (tiles & 1) work(n0, std::integral_constant<int, 0>{});
         // nothing of this part stays in flight (the prefetches past its end were never used)
         __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
         // local state of the part, relative to the shift of the incoming state; whatever
