@@ -740,7 +740,7 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
             for (int dt = 0; dt < DT; ++dt) U[mt][dt] += tu[mt][dt];
     }
 
-    uint2 ltri, ones4 = make_uint2(P_::kOnes2, P_::kOnes2);
+    uint2 ltri;
     {
         const uint32_t one = P_::kOnes2 & 0xffffu;
         uint32_t e[4];
@@ -868,6 +868,7 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
         // ---- token side, part 1: scores, P, column sums; publish P^T ----
         float p[CTA][4];
         uint2 ppk[CTA];
+        f32x4 dc[CTA];
         {
             f32x4 sc[CTA];
 #pragma unroll
@@ -883,12 +884,12 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
                 for (int r = 0; r < 4; ++r) p[ct][r] = fast_exp2(sc[ct][r] - mu0[ct]);
                 ppk[ct] = make_uint2(P_::pack2(p[ct][0], p[ct][1]), P_::pack2(p[ct][2], p[ct][3]));
             }
-            f32x4 csv[CTA];
+            // running sums over the wave's tokens (row t = 4g + r: tokens 0..t); the last row is the column sum
 #pragma unroll
-            for (int ct = 0; ct < CTA; ++ct) csv[ct] = P_::mma16(ones4, ppk[ct], zf);
+            for (int ct = 0; ct < CTA; ++ct) dc[ct] = P_::mma16(ltri, ppk[ct], zf);
 #pragma unroll
             for (int ct = 0; ct < CTA; ++ct) {
-                if (g == 0) cs[(ct * 16 + c16) * 4 + w] = csv[ct][0];
+                if (g == 3) cs[(ct * 16 + c16) * 4 + w] = dc[ct][3];
                 *reinterpret_cast<uint2*>(ptw + (ct * 16 + c16) * 16 + 4 * g) = ppk[ct];
             }
         }
@@ -904,9 +905,6 @@ __global__ __launch_bounds__(256, 2) void causal_chunk_kernel(CausalArgs a)
                 fw[ct] = lds_at<float, M * 4 + ct * 64>(mu_b);
             });
             FLARE_CHUNK_FENCE();
-            f32x4 dc[CTA];
-#pragma unroll
-            for (int ct = 0; ct < CTA; ++ct) dc[ct] = P_::mma16(ltri, ppk[ct], zf);
 #pragma unroll
             for (int ct = 0; ct < CTA; ++ct) {
                 float base = den0[ct];
