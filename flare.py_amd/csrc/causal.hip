@@ -244,8 +244,45 @@ hipError_t launch_dt(const CausalArgs& a, int dtype, hipStream_t st)
 }
 
 // Joins latent groups that ran as causal problems of their own: y[r,:] = sum_g w_g y_g[r,:] with
-// w_g = exp(lse_g[r]) / sum_g' exp(lse_g'[r]).  One thread per 8 consecutive elements of a row (16 bytes of a
-// 16-bit type), fp32 arithmetic, groups visited in order (bit-stable).
+// w_g = exp(lse_g[r]) / sum_g' exp(lse_g'[r]).  One thread per 8 consecutive elements of a row, moved as 16-byte
+// pieces (one for a 16-bit type, two for fp32); fp32 arithmetic, groups visited in order (bit-stable).
+template <typename T> __device__ __forceinline__ void join_load8(const T* p, float (&x)[8])
+{
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    if constexpr (sizeof(T) == 4) {
+        const u4 lo = *reinterpret_cast<const u4*>(p), hi = *reinterpret_cast<const u4*>(p + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            x[e] = __uint_as_float(lo[e]);
+            x[4 + e] = __uint_as_float(hi[e]);
+        }
+    } else {
+        const u4 raw = *reinterpret_cast<const u4*>(p);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint16_t b0 = uint16_t(raw[e] & 0xffffu), b1 = uint16_t(raw[e] >> 16);
+            x[2 * e] = to_f32(__builtin_bit_cast(T, b0));
+            x[2 * e + 1] = to_f32(__builtin_bit_cast(T, b1));
+        }
+    }
+}
+template <typename T> __device__ __forceinline__ void join_store8(T* p, const float (&x)[8])
+{
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    if constexpr (sizeof(T) == 4) {
+        *reinterpret_cast<u4*>(p) = u4{__float_as_uint(x[0]), __float_as_uint(x[1]), __float_as_uint(x[2]), __float_as_uint(x[3])};
+        *reinterpret_cast<u4*>(p + 4) = u4{__float_as_uint(x[4]), __float_as_uint(x[5]), __float_as_uint(x[6]), __float_as_uint(x[7])};
+    } else {
+        u4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const T lo = from_f32<T>(x[2 * e]), hi = from_f32<T>(x[2 * e + 1]);
+            o[e] = uint32_t(__builtin_bit_cast(uint16_t, lo)) | (uint32_t(__builtin_bit_cast(uint16_t, hi)) << 16);
+        }
+        *reinterpret_cast<u4*>(p) = o;
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void causal_join_kernel(CausalJoinArgs a)
 {
@@ -261,14 +298,15 @@ __global__ __launch_bounds__(256) void causal_join_kernel(CausalJoinArgs a)
     for (int g = 0; g < a.n_groups; ++g) {
         const float w = __expf(a.lse[g][r] - mx);
         sum += w;
-        const T* src = (const T*)a.yg[g] + r * a.D + c;
+        float x[8];
+        join_load8((const T*)a.yg[g] + r * a.D + c, x);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] = fmaf(w, to_f32(src[e]), acc[e]);
+        for (int e = 0; e < 8; ++e) acc[e] = fmaf(w, x[e], acc[e]);
     }
     const float inv = 1.f / sum;
-    T* dst = (T*)a.y + r * a.D + c;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) dst[e] = from_f32<T>(acc[e] * inv);
+    for (int e = 0; e < 8; ++e) acc[e] *= inv;
+    join_store8((T*)a.y + r * a.D + c, acc);
 }
 
 }  // namespace
