@@ -1340,15 +1340,23 @@ def triple_attention(q1, q2, k1, k2, v, normalize: bool = False, feature_map: Op
     already went through the kernel map (as TripleAttention.forward does at backends.py:1258);
     feature_map='elu' applies elu(x)+1 to q1,q2,k1,k2 inside the kernels.
     normalize=True divides out by the matching normaliser (same contraction with v == 1).
+    Differentiable in all five inputs in every mode.
     """
     if feature_map not in (None, "identity", "elu"):
         raise ValueError("feature_map must be None, 'identity' or 'elu'")
     needs_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (q1, q2, k1, k2, v))
     if needs_grad:
-        if normalize or feature_map == "elu":
-            raise NotImplementedError("gradients of triple_attention are available for feature_map=None, "
-                                      "normalize=False (apply the feature map in torch, as the reference does)")
-        return _TripleFn.apply(q1, q2, k1, k2, v)
+        # Under autograd the feature map is applied with torch ops in front of the kernels (where the reference applies it,
+        # backends.py:1258) and the normaliser is formed with two small einsums behind them, so that both differentiate
+        # through torch while the two contractions and their gradients stay on the HIP kernels.
+        if feature_map == "elu":
+            q1, q2, k1, k2 = (torch.nn.functional.elu(t) + 1 for t in (q1, q2, k1, k2))
+        state, out = _TripleFn.apply(q1, q2, k1, k2, v)
+        if normalize:
+            kk = torch.einsum("bhni,bhnk->bhik", k1.float(), k2.float()) / k1.shape[-2]
+            den = torch.einsum("bhni,bhik,bhnk->bhn", q1.float(), kk, q2.float())
+            out = (out.float() / den.unsqueeze(-1)).to(out.dtype)
+        return state, out
     return _triple_forward(q1, q2, k1, k2, v, feature_map == "elu", normalize, n_splits)
 
 

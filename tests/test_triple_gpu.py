@@ -96,6 +96,31 @@ def test_backward_matches_autograd_of_the_einsum_oracle(dev, dtype, D, Dv, tol):
         assert err <= tol, f"{name}: {err:.3e}"
 
 
+@pytest.mark.parametrize("dtype,D,Dv,tol", [(torch.float32, 16, 16, 1e-4), (torch.bfloat16, 16, 16, 3e-2), (torch.float32, 8, 12, 1e-4)])
+@pytest.mark.parametrize("fm,norm", [("elu", True), ("elu", False), (None, True)])
+def test_backward_with_feature_map_and_normaliser(dev, dtype, D, Dv, tol, fm, norm):
+    """Gradients with the elu + 1 feature map and / or the normaliser (the module's training mode, backends.py:1258,
+    1285-1292): the map and the division differentiate through torch around the HIP contractions; checked against fp64
+    autograd through the einsum definition."""
+    g = torch.Generator().manual_seed(13)
+    B, H, N = 1, 2, 260
+    ins = [(torch.randn(B, H, N, D, generator=g) * 0.5).to(dtype) for _ in range(4)] + [torch.randn(B, H, N, Dv, generator=g).to(dtype)]
+    if fm is None:
+        ins[:4] = [t.abs() + 0.1 for t in ins[:4]]           # positive features, as a kernel map leaves them: the normaliser stays away from 0
+    gs = torch.randn(B, H, D, Dv, D, generator=g)
+    go = torch.randn(B, H, N, Dv, generator=g).to(dtype)
+    dins = [t.to(dev).requires_grad_(True) for t in ins]
+    st, out = F.triple_attention(*dins, normalize=norm, feature_map=fm)
+    (st * gs.to(dev)).sum().add((out.float() * go.to(dev).float()).sum()).backward()
+    rins = [t.double().requires_grad_(True) for t in ins]
+    sr, orf = O.triple_einsum(*rins, feature_map=fm == "elu", normalize=norm, dtype=torch.float64)
+    ((sr * gs.double()).sum() + (orf * go.double()).sum()).backward()
+    assert O.rel_l2(out, orf) <= (1e-5 if dtype == torch.float32 else 2e-2)
+    for name, a, b in zip(("dq1", "dq2", "dk1", "dk2", "dv"), dins, rins):
+        err = O.rel_l2(a.grad, b.grad)
+        assert err <= tol, f"{name}: {err:.3e}"
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("Dq,Dv", [(32, 32), (16, 32), (32, 16), (64, 64), (48, 32), (8, 8), (20, 24), (4, 40)])
 def test_head_dims_in_blocks_of_16(dev, Dq, Dv, dtype):
