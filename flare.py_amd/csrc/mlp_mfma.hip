@@ -396,14 +396,22 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
                 for (int ft = 0; ft < FT; ++ft) {
                     const f32x4 bias = bias_q[ft & 1];
                     if (ft + 2 < FT) bias_q[ft & 1] = vec4(bl + 16 * (ft + 2), has_bias);
+                    // The weight operands of a feature tile (one LDS read per k-step) are requested together at the head of
+                    // the tile: left to itself the compiler, short of registers, issues each read where it is used, and
+                    // every pair of products then starts with a round trip to LDS.  The fence keeps LDS reads from sinking
+                    // below it and lets everything else cross (the epilogue of the tile before runs under this tile's
+                    // reads).  Measured on the chain and the narrow-input modes; the expanding mode above is no faster for it.
+                    u32x4 wq[KS];
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) wq[ks] = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]);
+                    __builtin_amdgcn_sched_barrier(0x7F);
                     f32x4 acc[TW];
 #pragma unroll
                     for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
 #pragma unroll
                     for (int ks = 0; ks < KS; ++ks) {
-                        const u32x4 wa = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]);
 #pragma unroll
-                        for (int tw = 0; tw < TW; ++tw) acc[tw] = M_::mma(wa, xb[ks][tw], acc[tw]);
+                        for (int tw = 0; tw < TW; ++tw) acc[tw] = M_::mma(wq[ks], xb[ks][tw], acc[tw]);
                     }
                     // tile ft of the stream is not an input of this layer any more once xb is packed
 #pragma unroll
