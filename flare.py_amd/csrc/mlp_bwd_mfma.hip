@@ -307,9 +307,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
 #pragma unroll
                 for (int ft = 0; ft < FT; ++ft) {
                     f32x4 acc = *reinterpret_cast<const f32x4*>(pvec + l * C + 16 * ft + 4 * g);
+                    // the tile's weight operands requested together: read where they are used, every product starts with
+                    // a round trip to LDS (the fence holds LDS reads in place and lets everything else cross)
+                    u32x4 wq[KS];
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks)
-                        acc = M_::mma(*reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]), xb[ks], acc);
+                    for (int ks = 0; ks < KS; ++ks) wq[ks] = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]);
+                    __builtin_amdgcn_sched_barrier(0x7F);
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) acc = M_::mma(wq[ks], xb[ks], acc);
                     float sl[4];
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
@@ -372,9 +377,12 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
                 f32x4 acc = add ? xs[ft] : f32x4{0.f, 0.f, 0.f, 0.f};
+                u32x4 wq[KS];      // requested together, as above (two tiles at a time, their chains alternating, is no faster)
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks)
-                    acc = M_::mma(*reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]), db[ks], acc);
+                for (int ks = 0; ks < KS; ++ks) wq[ks] = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]);
+                __builtin_amdgcn_sched_barrier(0x7F);
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) acc = M_::mma(wq[ks], db[ks], acc);
                 xs[ft] = acc;
                 if (C == 128 && (ft & 1)) __builtin_amdgcn_sched_barrier(0);
             }
