@@ -20,6 +20,7 @@ from torch import nn
 from torch.nn import functional as F
 
 from .functional import flare_multihead_mixer, triple_attention
+from . import fused
 from .modules import ResidualMLP, _norm
 
 __all__ = ["FLARE", "FLAREBlock", "TripleAttention", "TripleBlock", "make_kernel", "RotaryPositionalEmbeddings"]
@@ -76,18 +77,36 @@ class FLARE(nn.Module):
                                   act=act, input_residual=True, output_residual=True)
         self.out_proj = nn.Linear(channel_dim, channel_dim)
 
-    def forward(self, x, attention_mask=None):
+    def _fusable(self, x):
+        """The 16-bit dtype the fused token-wise launches may run the three projections in, or None (torch layers)."""
+        cds = {fused.compute_dtype(x, m) for m in (self.k_proj, self.v_proj, self.out_proj)}
+        return cds.pop() if len(cds) == 1 else None
+
+    def forward(self, x, attention_mask=None, _norm=None, _res=None):
+        """_norm / _res are FLAREBlock's pre-norm and residual: under autocast (or with 16-bit weights) they are folded
+        into the fused launches of the projections, and the result is _res + att(_norm(x))."""
         B, N, C = x.shape
         drop = self.attn_drop_p if self.training else 0.0       # on both softmaxes, as backends.py:592,605-606
+        pdrop = self.proj_drop_p if self.training else 0.0
         q = self.latent_q.view(self.num_heads, self.num_latents, self.head_dim)
-        k = self.k_proj(x).view(B, N, self.num_heads, self.head_dim).permute(0, 2, 1, 3)
-        v = self.v_proj(x).view(B, N, self.num_heads, self.head_dim).permute(0, 2, 1, 3)
+        cd = self._fusable(x)
+        if cd is not None:
+            k = fused.fused_mlp(x, self.k_proj, cd, norm=_norm, out_dtype=cd)
+            v = fused.fused_mlp(x, self.v_proj, cd, norm=_norm, out_dtype=cd)
+        else:
+            xn = x if _norm is None else _norm(x)
+            k, v = self.k_proj(xn), self.v_proj(xn)
+        k = k.view(B, N, self.num_heads, self.head_dim).permute(0, 2, 1, 3)
+        v = v.view(B, N, self.num_heads, self.head_dim).permute(0, 2, 1, 3)
         if self.rope is not None:
             k = self.rope(k)
         y = flare_multihead_mixer(q, k, v, scale=self.attn_scale, key_mask=attention_mask, token_major_out=True,
                                   dropout_p=drop)
-        y = self.out_proj(y.permute(0, 2, 1, 3).reshape(B, N, C))
-        return F.dropout(y, p=self.proj_drop_p if self.training else 0.0)
+        y = y.permute(0, 2, 1, 3).reshape(B, N, C)
+        if cd is not None and pdrop == 0.0:
+            return fused.fused_mlp(y, self.out_proj, cd, res=_res, out_dtype=(x if _res is None else _res).dtype)
+        y = F.dropout(self.out_proj(y), p=pdrop)
+        return y if _res is None else _res + y
 
 
 class FLAREBlock(nn.Module):
@@ -106,7 +125,10 @@ class FLAREBlock(nn.Module):
                                input_residual=True, output_residual=True)
 
     def forward(self, x, attention_mask=None):
-        x = x + self.att(self.norm1(x), attention_mask=attention_mask)
+        x = self.att(x, attention_mask=attention_mask, _norm=self.norm1, _res=x)
+        cd = fused.compute_dtype(x, self.mlp)
+        if cd is not None:
+            return fused.fused_mlp(x, self.mlp, cd, norm=self.norm2, res=x)
         return x + self.mlp(self.norm2(x))
 
 

@@ -313,6 +313,51 @@ def test_lra_block_with_rope_and_mask_against_oracle(dev):
     assert O.rel_l2(y_nomask, O.flare_block(sd, "", x.cpu(), 4)) > 1e-3             # the rotation matters
 
 
+@pytest.mark.parametrize("masked,pdrop", [(False, 0.0), (True, 0.0), (False, 0.2)])
+def test_lra_block_under_autocast_runs_the_fused_launches(dev, masked, pdrop):
+    """The sequence block under bf16 autocast: norm1 + k/v projections, out_proj + residual and norm2 + feed-forward + residual
+    run as the fused token-wise launches (lra/models/backends.py:541-672 names the same torch layers), forward and backward.
+    Forward and gradients against the fp64 state-dict oracle (autograd through its torch ops).  Tolerances: bf16 arithmetic
+    through one block.  With projection dropout the
+    output projection keeps its torch layer (only shapes and finiteness are checked there: the mask is torch's)."""
+    torch.manual_seed(21)
+    blk = lra_modules.FLAREBlock(channel_dim=64, num_heads=4, num_latents=32, kv_proj_hidden_dim=64, ffn_hidden_dim=64,
+                                 proj_drop=pdrop).to(dev)
+    for p_ in blk.parameters():
+        torch.nn.init.normal_(p_, 0.0, 0.2) if p_.dim() > 1 else torch.nn.init.normal_(p_, 0.2, 0.2)
+    x = torch.randn(3, 333, 64, device=dev)
+    mask = None
+    if masked:
+        mask = torch.ones(3, 333, dtype=torch.bool, device=dev)
+        mask[1, 200:] = False
+    gy = torch.randn(3, 333, 64, device=dev)
+    if mask is not None:
+        gy = gy * mask[..., None]
+    blk.train()
+    with torch.profiler.profile(activities=[torch.profiler.ProfilerActivity.CUDA]) as prof:
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            y = blk(x, attention_mask=mask)
+        y.float().backward(gy)
+        torch.cuda.synchronize()
+    kernels = " ".join(e.key for e in prof.key_averages())
+    assert "mlp_mfma_kernel" in kernels and "mlp_bwd_kernel" in kernels, kernels
+    assert y.shape == x.shape and torch.isfinite(y).all()
+    grads = {n: p_.grad.clone() for n, p_ in blk.named_parameters()}
+    assert all(torch.isfinite(g_).all() for g_ in grads.values())
+    if pdrop > 0.0:
+        return
+    keep = torch.ones(3, 333, dtype=torch.bool) if mask is None else mask.cpu()
+    sd = {k_: v_.detach().cpu().double().requires_grad_(True) for k_, v_ in blk.state_dict().items()}
+    yo = O.flare_block(sd, "", x.cpu().double(), 4, key_mask=None if mask is None else mask.cpu())
+    assert O.rel_l2(y.detach().cpu()[keep], yo.detach()[keep]) <= 2e-2
+    (yo * gy.cpu().double()).sum().backward()
+    for n, g_ in grads.items():
+        err = O.rel_l2(g_, sd[n].grad)
+        # (the gradients of the latents and of the key projection are sums of cancelling terms over all tokens, formed from
+        # 16-bit operands: the same step through the torch layers under autocast sits as far from fp64 on those tensors)
+        assert err <= (1e-1 if n == "att.latent_q" or n.startswith("att.k_proj") else 5e-2), f"{n}: {err:.3e}"
+
+
 def test_default_model_geometry_uses_matrix_core_mixer(dev, monkeypatch):
     """The reference's default model (channel_dim 64, 8 heads: head dim 8; pdebench/__main__.py:1122-1143 with 64
     latents) under bf16 autocast: the mixer runs on the matrix-core kernels and the model matches the oracle."""
