@@ -21,7 +21,7 @@ from torch.nn import functional as F
 
 from .functional import flare_multihead_mixer, triple_attention
 from . import fused
-from .modules import ResidualMLP, _norm
+from .modules import ResidualMLP, _lin, _norm
 
 __all__ = ["FLARE", "FLAREBlock", "TripleAttention", "TripleBlock", "make_kernel", "RotaryPositionalEmbeddings"]
 
@@ -105,7 +105,7 @@ class FLARE(nn.Module):
         y = y.permute(0, 2, 1, 3).reshape(B, N, C)
         if cd is not None and pdrop == 0.0:
             return fused.fused_mlp(y, self.out_proj, cd, res=_res, out_dtype=(x if _res is None else _res).dtype)
-        y = F.dropout(self.out_proj(y), p=pdrop)
+        y = F.dropout(_lin(self.out_proj, y), p=pdrop)
         return y if _res is None else _res + y
 
 
@@ -266,7 +266,7 @@ class TripleAttention(nn.Module):
                 q1, q2, k1, k2, v = (t * mask for t in (q1, q2, k1, k2, v))
         _, out = self.attn(q1, q2, k1, k2, v, feature_map="elu" if in_kernel_map else None)
         out = out.permute(0, 2, 1, 3).reshape(B, N, C)
-        return self.proj_drop(self.out_proj(self.norm(out)))
+        return self.proj_drop(_lin(self.out_proj, self.norm(out)))
 
     def attn(self, q1, q2, k1, k2, v, feature_map=None):
         """(state, out) of backends.py:1285-1292 on the HIP kernels."""

@@ -183,3 +183,28 @@ def test_fused_structure_cache_follows_replaced_submodules():
     assert fused._train_subchain(mlp).first is mlp.fc1
     mlp.act = nn.ReLU()                                        # an activation the kernels do not have
     assert fused._layers_of(mlp) is None and fused._train_subchain(mlp) is None
+
+
+def test_linear_with_sliced_weight_gradient_equals_linear():
+    """modules._LinearLongRows (the Linear layers of a token-wise model in training: dW as a batched product over slices of
+    the rows) against autograd through F.linear, for row counts with and without a power-of-two factor, with and without bias."""
+    from flare_py_amd import modules
+    torch.manual_seed(3)
+    for rows, cin, cout, bias in ((4096, 24, 16, True), (4100, 8, 8, False), (777, 5, 7, True), (2, 3 * 640, 4, True)):
+        x = torch.randn(2, rows // 2, cin, dtype=torch.float64, requires_grad=True)
+        w = torch.randn(cout, cin, dtype=torch.float64, requires_grad=True)
+        b = torch.randn(cout, dtype=torch.float64, requires_grad=True) if bias else None
+        g = torch.randn(2, rows // 2, cout, dtype=torch.float64)
+        y = modules._LinearLongRows.apply(x, w, b)
+        y.backward(g)
+        got = [t.grad.clone() for t in (x, w) + ((b,) if bias else ())]
+        for t in (x, w) + ((b,) if bias else ()):
+            t.grad = None
+        yr = torch.nn.functional.linear(x, w, b)
+        yr.backward(g)
+        assert torch.equal(y, yr)
+        for a_, t in zip(got, (x, w) + ((b,) if bias else ())):
+            assert torch.allclose(a_, t.grad, rtol=1e-12, atol=1e-12)
+    # the dispatcher only takes it in training, on a GPU, outside autocast, over many rows
+    lin = torch.nn.Linear(8, 8)
+    assert modules._lin(lin, torch.randn(5000, 8)).grad_fn.name() != "_LinearLongRowsBackward"

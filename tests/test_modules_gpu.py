@@ -358,6 +358,36 @@ def test_lra_block_under_autocast_runs_the_fused_launches(dev, masked, pdrop):
         assert err <= (1e-1 if n == "att.latent_q" or n.startswith("att.k_proj") else 5e-2), f"{n}: {err:.3e}"
 
 
+def test_fp32_training_uses_the_sliced_weight_gradient(dev, monkeypatch):
+    """A ResidualMLP over many rows in fp32 training: its Linear layers go through modules._LinearLongRows; outputs equal and
+    gradients within fp32 summation-order noise of the same module with the dispatcher switched off."""
+    torch.manual_seed(4)
+    mlp = modules.ResidualMLP(64, 64, 64, num_layers=2, input_residual=True, output_residual=True).to(dev)
+    x = torch.randn(4, 4096, 64, device=dev, requires_grad=True)
+    g = torch.randn(4, 4096, 64, device=dev)
+    y = mlp(x)
+    seen, todo = set(), [y.grad_fn]
+    while todo:
+        f = todo.pop()
+        if f is None or f in seen:
+            continue
+        seen.add(f)
+        todo.extend(n for n, _ in f.next_functions)
+    assert sum("LinearLongRows" in f.name() for f in seen) == 4           # fc1, two hidden layers, fc2
+    y.backward(g)
+    got = {n: p_.grad.clone() for n, p_ in mlp.named_parameters()}
+    gx = x.grad.clone()
+    for p_ in mlp.parameters():
+        p_.grad = None
+    x.grad = None
+    monkeypatch.setattr(modules, "_LONG_ROWS", 1 << 40)
+    y2 = mlp(x)
+    y2.backward(g)
+    assert torch.equal(y, y2) and O.rel_l2(gx, x.grad) <= 1e-6
+    for n, p_ in mlp.named_parameters():
+        assert O.rel_l2(got[n], p_.grad) <= 1e-5, n
+
+
 def test_default_model_geometry_uses_matrix_core_mixer(dev, monkeypatch):
     """The reference's default model (channel_dim 64, 8 heads: head dim 8; pdebench/__main__.py:1122-1143 with 64
     latents) under bf16 autocast: the mixer runs on the matrix-core kernels and the model matches the oracle."""
