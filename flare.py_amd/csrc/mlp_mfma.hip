@@ -49,6 +49,26 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// Four stream values of a lane as separate registers.  As a 4-vector every single-element update copies the
+// other three (the vector is one value to the compiler, and one register tuple), which the activation of a tile,
+// element by element, would pay for with three moves per element.
+struct Row4 {
+    float e[4];
+    __device__ __forceinline__ float& operator[](int i) { return e[i]; }
+    __device__ __forceinline__ float operator[](int i) const { return e[i]; }
+    __device__ __forceinline__ Row4& operator=(f32x4 v)
+    {
+        e[0] = v[0]; e[1] = v[1]; e[2] = v[2]; e[3] = v[3];
+        return *this;
+    }
+    __device__ __forceinline__ Row4& operator+=(f32x4 v)
+    {
+        e[0] += v[0]; e[1] += v[1]; e[2] += v[2]; e[3] += v[3];
+        return *this;
+    }
+    __device__ __forceinline__ operator f32x4() const { return f32x4{e[0], e[1], e[2], e[3]}; }
+};
+
 template <typename T> struct Mm;
 template <> struct Mm<bf16_t> {
     static __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c)
@@ -73,23 +93,44 @@ template <> struct Mm<f16_t> {
     }
 };
 
-// four consecutive elements of a row of element type dt (0 f32, 1 bf16, 2 f16) as fp32
-__device__ __forceinline__ f32x4 load4(const void* base, int64_t elem, int dt)
+// Element type of a row (0 f32, 1 bf16, 2 f16) as a compile-time constant of the code that moves the row: the type is
+// a launch argument, and a branch on it around every single load would put each load into a basic block of its own,
+// where the 16-bit ones are followed by a wait for the data they convert -- one trip to memory per tile of a row.
+// with_dtype branches once (uniformly) and runs a body in which all loads of a pass are issued back to back.
+template <int DT> using Dt = std::integral_constant<int, DT>;
+template <typename F> __device__ __forceinline__ void with_dtype(int dt, F&& f)
 {
-    if (dt == 0) return *reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + elem);
-    const uint2 r = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + elem);
-    if (dt == 1)
-        return f32x4{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
-                     __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u)};
-    const f16x2 lo = __builtin_bit_cast(f16x2, r.x), hi = __builtin_bit_cast(f16x2, r.y);
-    return f32x4{(float)lo[0], (float)lo[1], (float)hi[0], (float)hi[1]};
+    if (dt == 0) f(Dt<0>{});
+    else if (dt == 1) f(Dt<1>{});
+    else f(Dt<2>{});
 }
 
-__device__ __forceinline__ void store4(void* base, int64_t elem, int dt, f32x4 v)
+// four consecutive elements of a row as they lie in memory, and as fp32
+template <int DT> struct Raw4 { using type = uint2; };
+template <> struct Raw4<0> { using type = f32x4; };
+template <int DT> __device__ __forceinline__ typename Raw4<DT>::type load4_raw(const void* base, int64_t elem)
 {
-    if (dt == 0) {
+    if constexpr (DT == 0) return *reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + elem);
+    else return *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + elem);
+}
+template <int DT> __device__ __forceinline__ f32x4 unpack4(typename Raw4<DT>::type r)
+{
+    if constexpr (DT == 0) {
+        return r;
+    } else if constexpr (DT == 1) {
+        return f32x4{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
+                     __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u)};
+    } else {
+        const f16x2 lo = __builtin_bit_cast(f16x2, r.x), hi = __builtin_bit_cast(f16x2, r.y);
+        return f32x4{(float)lo[0], (float)lo[1], (float)hi[0], (float)hi[1]};
+    }
+}
+
+template <int DT> __device__ __forceinline__ void store4(void* base, int64_t elem, f32x4 v)
+{
+    if constexpr (DT == 0) {
         *reinterpret_cast<f32x4*>(static_cast<float*>(base) + elem) = v;
-    } else if (dt == 1) {
+    } else if constexpr (DT == 1) {
         *reinterpret_cast<uint2*>(static_cast<uint16_t*>(base) + elem) =
             make_uint2(Mm<bf16_t>::pack2(v[0], v[1]), Mm<bf16_t>::pack2(v[2], v[3]));
     } else {
@@ -117,10 +158,23 @@ __device__ __forceinline__ float silu_gate(float x)
 }
 
 // MODE: 0 the C x C chain, 1 the expanding two-layer MLP, 2 the chain with a narrow first input and/or last output,
-// 3 the chain with head-padded rows on either end
-template <typename T, int C, int TW, int WAVES, int MODE>
+// 3 the chain with head-padded rows on either end.
+// PF: 1 = the bias vectors of all layers stay in registers for the whole launch, element e in lane e % 64 of register
+// e / 64, and reach the lanes that need them by ds_bpermute, which moves data through the LDS crossbar without touching
+// LDS memory (all 160 KB hold weights).  No instruction of a layer then waits on the vector-memory counter, which retires
+// in order: a bias load inside a layer waits for every older request, the row loads of the pass and the stores of the
+// pass before included.  Resident weights only, PF_MAXL layers at most.
+constexpr size_t kMlpLdsMax = 160 * 1024;   // all of a CU's LDS: five layers of 128 channels stay resident
+
+template <int C> constexpr int pf_max_layers() { return 160 * 1024 / (C * C * 2) < 8 ? 160 * 1024 / (C * C * 2) : 8; }
+
+template <typename T, int C, int TW, int WAVES, int MODE, int PF>
 __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * WAVES) : 1)) void mlp_mfma_kernel(MlpArgs a, int resident)
 {
+    static_assert(PF == 0 || MODE != 1, "the expanding mode streams its tiles through a ring");
+    if constexpr (PF != 0) resident = 1;
+    constexpr int PF_MAXL = pf_max_layers<C>();
+    constexpr int NV = (C + 63) / 64;   // registers per parameter vector
     constexpr int NT = 64 * WAVES;
     constexpr int NCH = (C * C / 8 + NT - 1) / NT;   // 16-byte weight chunks per thread and layer
     constexpr int FT = C / 16;        // feature tiles of the stream
@@ -173,9 +227,48 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
         return have ? v : f32x4{0.f, 0.f, 0.f, 0.f};
     };
 
+    // PF: parameter vectors in registers; vec_at(v, ft) = elements 16 ft + 4 g .. + 3 of the vector
+    uint32_t bv[PF ? PF_MAXL : 1][NV];
+    if constexpr (PF != 0) {
+        auto elem = [&](const float* p, bool have, int j) {
+            const int e = 64 * j + lane;
+            const float v = p[e < C ? e : 0];
+            return have ? __float_as_uint(v) : 0u;
+        };
+#pragma unroll
+        for (int l = 0; l < PF_MAXL; ++l)
+#pragma unroll
+            for (int j = 0; j < NV; ++j) bv[l][j] = elem(bias0 + (size_t)(l < a.L ? l : 0) * C, has_bias, j);
+    }
+    // The layer number is a run-time value and registers cannot be indexed by one (an indexed array would be placed in
+    // scratch memory, whose loads count on the vector-memory counter as well): the bias vectors form a ring that
+    // turns by one position per layer, so that the current layer's vector is always bv[0].
+    auto rotate_bias = [&]() {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const uint32_t first = bv[0][j];
+#pragma unroll
+            for (int i = 0; i + 1 < (PF ? PF_MAXL : 1); ++i) bv[i][j] = bv[i + 1][j];
+            bv[(PF ? PF_MAXL : 1) - 1][j] = first;
+        }
+    };
+    int perm0 = 16 * g;     // byte address of lane 4 g in ds_bpermute's terms
+    auto vec_at = [&](const uint32_t (&v)[NV], int ft) {
+        const uint32_t src = v[(16 * ft) >> 6];
+        f32x4 o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            o[r] = __int_as_float(__builtin_amdgcn_ds_bpermute(perm0 + 4 * ((16 * ft) & 63) + 4 * r, (int)src));
+        return o;
+    };
+
     int woff[KS];     // byte offset of this lane's chunk of k-step ks inside its weight row (swizzled)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) woff[ks] = ((4 * ks + g) ^ (c16 >> SWS)) << 4;
+    // the same as LDS byte addresses of this lane's chunk in row c16 of slot 0 (the chain reads through these)
+    uint32_t wa[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) wa[ks] = (uint32_t)(uintptr_t)smem + c16 * RS + woff[ks];
 
     int lcount = 0;   // ring mode: layers done by this workgroup; its parity names the slot in use
     if (resident) {
@@ -190,6 +283,7 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
     __syncthreads();
 
     const int64_t nblk = ((int64_t)a.T + WAVES * TOKW - 1) / (WAVES * TOKW);
+
     for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
         int64_t tok[TW];
         bool live[TW];
@@ -200,8 +294,25 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
             tok[tw] = live[tw] ? t : a.T - 1;
         }
 
+        // All loads of a pass's rows (both token tiles, every feature tile) are issued before the first is unpacked.
+        // Rows of absent tokens are the last row's (tok is clamped), so nothing here depends on `live`.
+        auto load_rows = [&](const void* base, int dt, int64_t stride, int cf, int c0, auto&& sink) {
+            with_dtype(dt, [&](auto dc) {
+                constexpr int DT = decltype(dc)::value;
+                typename Raw4<DT>::type raw[FT][TW];
+#pragma unroll
+                for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+                    for (int ft = 0; ft < FT; ++ft) raw[ft][tw] = load4_raw<DT>(base, tok[tw] * stride + ft * cf + c0);
+#pragma unroll
+                for (int tw = 0; tw < TW; ++tw)
+#pragma unroll
+                    for (int ft = 0; ft < FT; ++ft) sink(ft, tw, unpack4<DT>(raw[ft][tw]));
+            });
+        };
+
         // the stream: lane (c16, g) holds features 16 ft + 4 g + r of token c16 of each tile
-        f32x4 xs[FT][TW];
+        Row4 xs[FT][TW];
         if (MODE == 2 && a.in_dim > 0) {
             // lifting layer: s[f] = act(b_in[f] + sum_i w_in[f][i] x[i]) from the token's few input features
             float xin[TW][4];
@@ -238,15 +349,9 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
             // head-padded rows: channel f = 16 ft + 4 g of the row sits at column 16 (f / x_head) + f % x_head,
             // which is ft * 32 + 8 g - 4 (g & 1) for heads of 8 and ft * 64 + 16 g for heads of 4
             const int cf = a.x_head == 8 ? 32 : 64, c0 = a.x_head == 8 ? 8 * g - 4 * (g & 1) : 16 * g;
-#pragma unroll
-            for (int tw = 0; tw < TW; ++tw)
-#pragma unroll
-                for (int ft = 0; ft < FT; ++ft) xs[ft][tw] = load4(a.x, tok[tw] * a.xs + ft * cf + c0, a.x_dtype);
+            load_rows(a.x, a.x_dtype, a.xs, cf, c0, [&](int ft, int tw, f32x4 v) { xs[ft][tw] = v; });
         } else {
-#pragma unroll
-            for (int tw = 0; tw < TW; ++tw)
-#pragma unroll
-                for (int ft = 0; ft < FT; ++ft) xs[ft][tw] = load4(a.x, tok[tw] * a.xs + 16 * ft + 4 * g, a.x_dtype);
+            load_rows(a.x, a.x_dtype, a.xs, 16, 4 * g, [&](int ft, int tw, f32x4 v) { xs[ft][tw] = v; });
         }
 
         if (a.norm != 0) {
@@ -379,7 +484,7 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
                 }
 
             const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
-            const uint8_t* wb = smem + slot * WBUF + c16 * RS;
+            const uint32_t so = slot * WBUF;
             // One layer for the wave's tokens.  ACT: 0 none, 1 tanh-GELU, 2 SiLU; ADD: the result is added to
             // the stream.  Both are compile-time here (the caller branches once per layer, uniformly), so the
             // epilogue has no selects and the last multiply of the activation fuses with the residual add.
@@ -389,44 +494,69 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
                 // the bias of a feature tile is requested two tiles ahead: it initialises the accumulators, so a load
                 // issued where it is used would put a trip to the cache in front of every tile's first product
                 const float* bl = bias0 + (size_t)l * C + 4 * g;
-                f32x4 bias_q[2];
+                auto bias_at = [&](int ft) {
+                    if constexpr (PF != 0) return vec_at(bv[0], ft);    // the ring of bias vectors has this layer's in front
+                    else return vec4(bl + 16 * ft, has_bias);
+                };
+                // Software pipeline over the feature tiles, written out: step ft issues the products of tile ft in between
+                // the activations of tile ft - 1, group by group, and requests the weight operands of tile ft + 1 (one
+                // LDS read per k-step, together) and the bias of tile ft + 2 first, so that no product waits for LDS and
+                // no activation for a product issued just before it.  Left to the compiler the tile ran in source order:
+                // reads, a wait, the products, a wait, the activations, with nothing of the next tile under any of it.
+                // The fences pin the interleaving (everything may move inside a group, nothing across).
+                auto rd = [&](int ft, int ks) {
+                    typedef const u32x4 __attribute__((address_space(3))) * lds_ptr;
+                    return *(lds_ptr)(uintptr_t)(wa[ks] + so + (16 * ft) * RS);
+                };
+                constexpr int NP = KS * TW, NE = TW * 4;      // products and activations per tile
+                constexpr int GS = 2;                           // per group: GS activations and their share of the products
+                constexpr int NG = NE / GS;
+                // one set of weight operands: the operand of k-step ks is requested for the next tile right behind the
+                // last product that reads it for this one
+                u32x4 wq[KS];
+                f32x4 bias_q[2], accp[TW];
 #pragma unroll
-                for (int i = 0; i < 2; ++i) bias_q[i] = vec4(bl + 16 * (i < FT ? i : 0), has_bias);
+                for (int ks = 0; ks < KS; ++ks) wq[ks] = rd(0, ks);
 #pragma unroll
-                for (int ft = 0; ft < FT; ++ft) {
-                    const f32x4 bias = bias_q[ft & 1];
-                    if (ft + 2 < FT) bias_q[ft & 1] = vec4(bl + 16 * (ft + 2), has_bias);
-                    // The weight operands of a feature tile (one LDS read per k-step) are requested together at the head of
-                    // the tile: left to itself the compiler, short of registers, issues each read where it is used, and
-                    // every pair of products then starts with a round trip to LDS.  The fence keeps LDS reads from sinking
-                    // below it and lets everything else cross (the epilogue of the tile before runs under this tile's
-                    // reads).  Measured on the chain and the narrow-input modes; the expanding mode above is no faster for it.
-                    u32x4 wq[KS];
+                for (int i = 0; i < 2; ++i) bias_q[i] = bias_at(i < FT ? i : 0);
 #pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) wq[ks] = *reinterpret_cast<const u32x4*>(wb + (16 * ft) * RS + woff[ks]);
-                    __builtin_amdgcn_sched_barrier(0x7F);
+                for (int ft = 0; ft <= FT; ++ft) {
                     f32x4 acc[TW];
+                    if (ft < FT) {
 #pragma unroll
-                    for (int tw = 0; tw < TW; ++tw) acc[tw] = bias;
-#pragma unroll
-                    for (int ks = 0; ks < KS; ++ks) {
-#pragma unroll
-                        for (int tw = 0; tw < TW; ++tw) acc[tw] = M_::mma(wq[ks], xb[ks][tw], acc[tw]);
+                        for (int tw = 0; tw < TW; ++tw) acc[tw] = bias_q[ft & 1];
+                        if (ft + 2 < FT) bias_q[ft & 1] = bias_at(ft + 2);
                     }
-                    // tile ft of the stream is not an input of this layer any more once xb is packed
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int tw = 0; tw < TW; ++tw) {
+                    for (int gi = 0; gi < NG; ++gi) {
+                        if (ft < FT) {
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            const float t = acc[tw][r];
-                            if constexpr (ACT == 0) {
-                                xs[ft][tw][r] = ADD ? xs[ft][tw][r] + t : t;
-                            } else {
-                                const float gate = ACT == 1 ? gelu_gate(t) : silu_gate(t);     // act(t) = t * gate
-                                xs[ft][tw][r] = ADD ? fmaf(t, gate, xs[ft][tw][r]) : t * gate;
+                            for (int i = gi * NP / NG; i < (gi + 1) * NP / NG; ++i) {
+                                const int ks = i / TW, tw = i % TW;
+                                acc[tw] = M_::mma(wq[ks], xb[ks][tw], acc[tw]);
+                                if (tw == TW - 1 && ft + 1 < FT) wq[ks] = rd(ft + 1, ks);
                             }
                         }
+                        if (ft > 0) {
+                            // tile ft - 1 of the stream is not an input of this layer any more once xb is packed
+#pragma unroll
+                            for (int i = gi * GS; i < (gi + 1) * GS; ++i) {
+                                const int tw = i % TW, r = i / TW;
+                                const float t = accp[tw][r];
+                                const float o = xs[ft - 1][tw][r];
+                                if constexpr (ACT == 0) {
+                                    xs[ft - 1][tw][r] = ADD ? o + t : t;
+                                } else {
+                                    const float gate = ACT == 1 ? gelu_gate(t) : silu_gate(t);     // act(t) = t * gate
+                                    xs[ft - 1][tw][r] = ADD ? fmaf(t, gate, o) : t * gate;
+                                }
+                            }
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
                     }
+#pragma unroll
+                    for (int tw = 0; tw < TW; ++tw) accp[tw] = acc[tw];
                 }
             };
             using I0 = std::integral_constant<int, 0>;
@@ -443,59 +573,66 @@ __global__ __launch_bounds__(64 * WAVES, (512 / (64 * WAVES) > 0 ? 512 / (64 * W
                 put(slot ^ 1);      // nobody reads that slot during this layer
                 __syncthreads();
             }
+            if constexpr (PF != 0) rotate_bias();
         }
+        if constexpr (PF != 0)
+            for (int l = a.L; l < PF_MAXL; ++l) rotate_bias();     // back to layer 0 in front for the next pass
 
+        if (MODE == 2 && a.out_dim > 0) {
+            // projecting last layer: only its first out_dim <= 4 rows are real, lane g == 0 holds them
 #pragma unroll
-        for (int tw = 0; tw < TW; ++tw) {
-            if (!live[tw]) continue;
-            if (MODE == 2 && a.out_dim > 0) {
-                // projecting last layer: only its first out_dim <= 4 rows are real, lane g == 0 holds them
-                if (g == 0)
-                    for (int r = 0; r < a.out_dim; ++r) {
-                        const int64_t e = tok[tw] * a.ys + r;
-                        const float o = xs[0][tw][r];
-                        if (a.y_dtype == 0) static_cast<float*>(a.y)[e] = o;
-                        else if (a.y_dtype == 1) static_cast<uint16_t*>(a.y)[e] = (uint16_t)Mm<bf16_t>::pack2(o, 0.f);
-                        else static_cast<_Float16*>(a.y)[e] = (_Float16)o;
-                    }
-                continue;
+            for (int tw = 0; tw < TW; ++tw) {
+                if (!live[tw] || g != 0) continue;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {       // r is a constant of each copy: a run-time index would move the stream to scratch
+                    if (r >= a.out_dim) continue;
+                    const int64_t e = tok[tw] * a.ys + r;
+                    const float o = xs[0][tw][r];
+                    if (a.y_dtype == 0) static_cast<float*>(a.y)[e] = o;
+                    else if (a.y_dtype == 1) static_cast<uint16_t*>(a.y)[e] = (uint16_t)Mm<bf16_t>::pack2(o, 0.f);
+                    else static_cast<_Float16*>(a.y)[e] = (_Float16)o;
+                }
             }
+            continue;
+        }
+        // all residual loads of a pass before its first store: y may be the memory res points at, so a load written
+        // after a store also stays behind it, and the rows would take one trip to memory per tile
+        if (a.res) load_rows(a.res, a.res_dtype, a.rs, 16, 4 * g, [&](int ft, int tw, f32x4 v) { xs[ft][tw] += v; });
+        with_dtype(a.y_dtype, [&](auto dc) {
+            constexpr int DT = decltype(dc)::value;
             if (MODE == 3 && a.y_head > 0) {
                 // head-padded rows (columns as for x above): each head's channels, then zeros up to 16 columns,
                 // written by the lane that holds the head's last four channels
                 const int cf = a.y_head == 8 ? 32 : 64, c0 = a.y_head == 8 ? 8 * g - 4 * (g & 1) : 16 * g;
                 const int nz = a.y_head == 8 ? ((g & 1) ? 2 : 0) : 3;        // groups of 4 zero columns behind this lane's channels
                 const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-                if (a.res) {
 #pragma unroll
-                    for (int ft = 0; ft < FT; ++ft) xs[ft][tw] += load4(a.res, tok[tw] * a.rs + 16 * ft + 4 * g, a.res_dtype);
+                for (int tw = 0; tw < TW; ++tw) {
+                    if (!live[tw]) continue;
+#pragma unroll
+                    for (int ft = 0; ft < FT; ++ft) {
+                        const int64_t col = tok[tw] * a.ys + ft * cf + c0;
+                        store4<DT>(a.y, col, xs[ft][tw]);
+                        for (int z = 1; z <= nz; ++z) store4<DT>(a.y, col + 4 * z, zero);
+                    }
                 }
+            } else {
 #pragma unroll
-                for (int ft = 0; ft < FT; ++ft) {
-                    const int64_t col = tok[tw] * a.ys + ft * cf + c0;
-                    store4(a.y, col, a.y_dtype, xs[ft][tw]);
-                    for (int z = 1; z <= nz; ++z) store4(a.y, col + 4 * z, a.y_dtype, zero);
+                for (int tw = 0; tw < TW; ++tw) {
+                    if (!live[tw]) continue;
+#pragma unroll
+                    for (int ft = 0; ft < FT; ++ft) store4<DT>(a.y, tok[tw] * a.ys + 16 * ft + 4 * g, xs[ft][tw]);
                 }
-                continue;
             }
-            // all residual loads of the row before its first store: y may be the memory res points at, so a load
-            // written after a store also stays behind it, and the row would take one trip to memory per tile
-            if (a.res) {
-#pragma unroll
-                for (int ft = 0; ft < FT; ++ft) xs[ft][tw] += load4(a.res, tok[tw] * a.rs + 16 * ft + 4 * g, a.res_dtype);
-            }
-#pragma unroll
-            for (int ft = 0; ft < FT; ++ft) store4(a.y, tok[tw] * a.ys + 16 * ft + 4 * g, a.y_dtype, xs[ft][tw]);
-        }
+        });
     }
 }
 
-constexpr size_t kMlpLdsMax = 160 * 1024;   // all of a CU's LDS: five layers of 128 channels stay resident
 
-template <typename T, int C, int TW, int WAVES, int MODE>
-hipError_t launch_cte(const MlpArgs& a, hipStream_t st)
+template <typename T, int C, int TW, int WAVES, int MODE, int PF>
+hipError_t launch_pf(const MlpArgs& a, hipStream_t st)
 {
-    auto kern = mlp_mfma_kernel<T, C, TW, WAVES, MODE>;
+    auto kern = mlp_mfma_kernel<T, C, TW, WAVES, MODE, PF>;
     const size_t wbuf = (size_t)C * C * 2;
     int resident = (size_t)a.L * wbuf <= kMlpLdsMax ? 1 : 0;
     size_t lds = (resident ? (size_t)a.L : 2) * wbuf;
@@ -511,8 +648,24 @@ hipError_t launch_cte(const MlpArgs& a, hipStream_t st)
     const int64_t per = 16 * TW * WAVES;
     const int64_t nblk = ((int64_t)a.T + per - 1) / per;
     const unsigned grid = (unsigned)(nblk < slots ? nblk : slots);
+    if (PF != 0 && !resident) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES), lds, st, a, resident);
     return hipGetLastError();
+}
+
+// Picks the instance with the bias vectors in registers where it applies: many tokens per workgroup (TW > 1 marks
+// those launches) and weights that stay resident.
+template <typename T, int C, int TW, int WAVES, int MODE>
+hipError_t launch_cte(const MlpArgs& a, hipStream_t st)
+{
+    if constexpr (MODE != 1 && TW > 1) {
+        if ((size_t)a.L * C * C * 2 <= kMlpLdsMax && a.L <= pf_max_layers<C>()) {
+            const hipError_t e = launch_pf<T, C, TW, WAVES, MODE, 1>(a, st);
+            if (e != hipErrorInvalidValue) return e;
+            (void)hipGetLastError();
+        }
+    }
+    return launch_pf<T, C, TW, WAVES, MODE, 0>(a, st);
 }
 
 template <typename T, int C, int TW, int WAVES>
