@@ -455,6 +455,33 @@ def test_many_token_instances_of_every_mode(dev, C):
         assert torch.equal(fused.fused_mlp(yp, lin, torch.bfloat16, x_head=8), fused.fused_mlp(y, lin, torch.bfloat16))
 
 
+@pytest.mark.parametrize("C,n", [(128, -1), (128, 0), (128, 1), (128, 2), (128, 3), (64, 0), (64, 4), (64, 6), (64, 7), (32, 2)])
+def test_bias_vectors_in_registers_over_several_passes(dev, C, n):
+    """The many-token chain keeps the bias of every layer in registers as a ring that turns by one per layer and has
+    to be back at layer 0 when the workgroup's next pass begins, whatever the number of layers: enough tokens for
+    three to four passes per workgroup, every chain length the ring takes at this width and one beyond it (C = 64,
+    9 layers: bias from memory), a norm in front (its gamma and beta) and a residual behind."""
+    T = 200000
+    torch.manual_seed(C + n)
+    x = torch.randn(T, C, device=dev) * 1.2 - 0.2
+    m = make_mlp(C, n, True, True, "gelu", dev, seed=7 * C + n) if n >= 0 else nn.Linear(C, C).to(dev)
+    if n < 0:
+        nn.init.normal_(m.bias, 0.0, 0.5)
+    norm = nn.LayerNorm(C).to(dev)
+    nn.init.normal_(norm.weight, 1.0, 0.3)
+    nn.init.normal_(norm.bias, 0.0, 0.3)
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        y = fused.fused_mlp(x, m, torch.bfloat16, norm=norm, res=x)
+        y2 = fused.fused_mlp(x, m, torch.bfloat16, norm=norm, res=x)
+    assert torch.equal(y, y2)
+    ref = oracle_of(m, x, torch.bfloat16, norm, x)
+    assert O.rel_l2(y, ref) <= 2e-2
+    # the last pass of the last workgroup as well as the first: a ring out of step shows as a wrong bias, i.e. an error of
+    # the order of the bias itself in every row of the later passes
+    for lo in (0, T - 4096):
+        assert O.rel_l2(y[lo:lo + 4096], ref[lo:lo + 4096]) <= 2e-2
+
+
 @pytest.mark.parametrize("C,H", [(64, 8), (64, 4)])
 def test_cached_operands_follow_parameter_updates(dev, C, H):
     """The fast path caches 16-bit copies of the weights and of latent_q on the modules; an in-place update of a
