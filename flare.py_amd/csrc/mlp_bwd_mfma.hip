@@ -63,16 +63,45 @@ template <> struct Mw<f16_t> {
     static __device__ __forceinline__ float hi(uint32_t p) { return (float)__builtin_bit_cast(f16x2, p)[1]; }
 };
 
-// four consecutive elements of a row of element type dt (0 f32, 1 bf16, 2 f16) as fp32
-__device__ __forceinline__ f32x4 ld4(const void* base, int64_t elem, int dt)
+// Element type of a row (0 f32, 1 bf16, 2 f16) as a compile-time constant of the code that moves the row: the type is
+// a launch argument, and a branch on it around every single load puts each load into a basic block of its own, where a
+// wait for everything in flight precedes the next -- one trip to memory per feature tile of a row instead of one per
+// row.  with_dtype branches once (uniformly); load_row issues all loads of a row back to back and unpacks afterwards.
+template <typename F> __device__ __forceinline__ void with_dtype(int dt, F&& f)
 {
-    if (dt == 0) return *reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + elem);
-    const uint2 r = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + elem);
-    if (dt == 1)
+    if (dt == 0) f(std::integral_constant<int, 0>{});
+    else if (dt == 1) f(std::integral_constant<int, 1>{});
+    else f(std::integral_constant<int, 2>{});
+}
+template <int DT> struct Raw4 { using type = uint2; };
+template <> struct Raw4<0> { using type = f32x4; };
+template <int DT> __device__ __forceinline__ f32x4 unpack4(typename Raw4<DT>::type r)
+{
+    if constexpr (DT == 0) {
+        return r;
+    } else if constexpr (DT == 1) {
         return f32x4{__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
                      __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u)};
-    const f16x2 lo = __builtin_bit_cast(f16x2, r.x), hi = __builtin_bit_cast(f16x2, r.y);
-    return f32x4{(float)lo[0], (float)lo[1], (float)hi[0], (float)hi[1]};
+    } else {
+        const f16x2 lo = __builtin_bit_cast(f16x2, r.x), hi = __builtin_bit_cast(f16x2, r.y);
+        return f32x4{(float)lo[0], (float)lo[1], (float)hi[0], (float)hi[1]};
+    }
+}
+// tiles ft = 0 .. FT-1 of a row: four elements each, 16 apart, from element elem0 on; sink(ft, values)
+template <int FT, typename F>
+__device__ __forceinline__ void load_row(const void* base, int dt, int64_t elem0, F&& sink)
+{
+    with_dtype(dt, [&](auto dc) {
+        constexpr int DT = decltype(dc)::value;
+        typename Raw4<DT>::type raw[FT];
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft) {
+            if constexpr (DT == 0) raw[ft] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + elem0 + 16 * ft);
+            else raw[ft] = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(base) + elem0 + 16 * ft);
+        }
+#pragma unroll
+        for (int ft = 0; ft < FT; ++ft) sink(ft, unpack4<DT>(raw[ft]));
+    });
 }
 
 __device__ __forceinline__ void st4(void* base, int64_t elem, int dt, f32x4 v)
@@ -251,8 +280,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
     f32x4 x_next[FT];
     {
         const int64_t r = row_of(blockIdx.x);           // blockIdx.x < nblk: the grid is never larger
-#pragma unroll
-        for (int ft = 0; ft < FT; ++ft) x_next[ft] = ld4(a.x, r * a.xs + 16 * ft + 4 * g, a.x_dtype);
+        load_row<FT>(a.x, a.x_dtype, r * a.xs + 4 * g, [&](int ft, f32x4 v) { x_next[ft] = v; });
     }
     for (int64_t blk = blockIdx.x; blk < nblk; blk += gridDim.x) {
         const int64_t t = blk * (WAVES * 16) + w * 16 + c16;
@@ -345,17 +373,12 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
 
         // ---- backward through the chain: xs becomes ds ----
         f32x4 x_again[FT];
-#pragma unroll
-        for (int ft = 0; ft < FT; ++ft) {
-            xs[ft] = ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
-            if (!live) xs[ft] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
+        load_row<FT>(a.dy, a.dy_dtype, tok * a.dys + 4 * g, [&](int ft, f32x4 v) { xs[ft] = live ? v : f32x4{0.f, 0.f, 0.f, 0.f}; });
 #pragma unroll
         for (int l = LMAX - 1; l >= 0; --l) {
             if (l >= L) continue;
             if (l == 0 && a.norm != 0) {
-#pragma unroll
-                for (int ft = 0; ft < FT; ++ft) x_again[ft] = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+                load_row<FT>(a.x, a.x_dtype, tok * a.xs + 4 * g, [&](int ft, f32x4 v) { x_again[ft] = v; });
             }
             const uint8_t* wb = ring_step_begin(2 * L - 1 - l);
             const bool act = (a.act_mask >> l) & 1u, add = (a.add_mask >> l) & 1u;
@@ -393,8 +416,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
         {   // without a condition (the last tile reads its own row once more): under one, the registers of x_next
             // would have to keep their old value through the whole tile
             const int64_t r = row_of(blk + gridDim.x < nblk ? blk + gridDim.x : blk);
-#pragma unroll
-            for (int ft = 0; ft < FT; ++ft) x_next[ft] = ld4(a.x, r * a.xs + 16 * ft + 4 * g, a.x_dtype);
+            load_row<FT>(a.x, a.x_dtype, r * a.xs + 4 * g, [&](int ft, f32x4 v) { x_next[ft] = v; });
         }
         if (a.norm != 0) {
             // ds_0 and the token's statistics go out for dgamma, dbeta; xhat is taken again from x (x_again) rather
@@ -432,11 +454,12 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
             // every load of dy before the first store of dx (a load written after a store stays behind it: the two
             // may be the same memory as far as the compiler knows)
             if (a.add_dy) {
-#pragma unroll
-                for (int ft = 0; ft < FT; ++ft) xs[ft] += ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
+                load_row<FT>(a.dy, a.dy_dtype, tok * a.dys + 4 * g, [&](int ft, f32x4 v) { xs[ft] += v; });
             }
+            with_dtype(a.dx_dtype, [&](auto dc) {
 #pragma unroll
-            for (int ft = 0; ft < FT; ++ft) st4(a.dx, tok * a.dxs + 16 * ft + 4 * g, a.dx_dtype, xs[ft]);
+                for (int ft = 0; ft < FT; ++ft) st4(a.dx, tok * a.dxs + 16 * ft + 4 * g, decltype(dc)::value, xs[ft]);
+            });
         }
     }
 }
@@ -521,8 +544,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
 
         // n = norm(x) and dy, both packed once as B operands and left as 16-bit rows
         f32x4 xs[FT];
-#pragma unroll
-        for (int ft = 0; ft < FT; ++ft) xs[ft] = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+        load_row<FT>(a.x, a.x_dtype, tok * a.xs + 4 * g, [&](int ft, f32x4 v) { xs[ft] = v; });
         float mean = 0.f, rstd = 1.f;
         if (a.norm != 0) {
             float s = 0.f;
@@ -551,11 +573,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) nb[ks] = pack4(xs[2 * ks], xs[2 * ks + 1]);
         store_rows<C>(a.n_row, nb, t, a.T, g, c16);
-#pragma unroll
-        for (int ft = 0; ft < FT; ++ft) {
-            xs[ft] = ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
-            if (!live) xs[ft] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
+        load_row<FT>(a.dy, a.dy_dtype, tok * a.dys + 4 * g, [&](int ft, f32x4 v) { xs[ft] = live ? v : f32x4{0.f, 0.f, 0.f, 0.f}; });
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) dyb[ks] = pack4(xs[2 * ks], xs[2 * ks + 1]);
         store_rows<C>(a.dy_row, dyb, t, a.T, g, c16);
@@ -636,9 +654,11 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
             store_rows<C>(a.dn, dq, t, a.T, g, c16);
             if (live && lane < 16) *reinterpret_cast<float2*>(a.stats + 2 * tok) = make_float2(mean, rstd);
             float m1 = 0.f, m2 = 0.f;
+            f32x4 xrow[FT];
+            load_row<FT>(a.x, a.x_dtype, tok * a.xs + 4 * g, [&](int ft, f32x4 v) { xrow[ft] = v; });
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
-                const f32x4 xr = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+                const f32x4 xr = xrow[ft];
                 const f32x4 gm = *reinterpret_cast<const f32x4*>(pvec + PG * C + 16 * ft + 4 * g);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -651,18 +671,19 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
             m2 = tok_sum(m2) * (1.f / C);
 #pragma unroll
             for (int ft = 0; ft < FT; ++ft) {
-                const f32x4 xr = ld4(a.x, tok * a.xs + 16 * ft + 4 * g, a.x_dtype);
+                const f32x4 xr = xrow[ft];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) xs[ft][r] = rstd * (xs[ft][r] - m1 - (xr[r] - mean) * rstd * m2);
             }
         }
         if (live) {
             if (a.add_dy) {
-#pragma unroll
-                for (int ft = 0; ft < FT; ++ft) xs[ft] += ld4(a.dy, tok * a.dys + 16 * ft + 4 * g, a.dy_dtype);
+                load_row<FT>(a.dy, a.dy_dtype, tok * a.dys + 4 * g, [&](int ft, f32x4 v) { xs[ft] += v; });
             }
+            with_dtype(a.dx_dtype, [&](auto dc) {
 #pragma unroll
-            for (int ft = 0; ft < FT; ++ft) st4(a.dx, tok * a.dxs + 16 * ft + 4 * g, a.dx_dtype, xs[ft]);
+                for (int ft = 0; ft < FT; ++ft) st4(a.dx, tok * a.dxs + 16 * ft + 4 * g, decltype(dc)::value, xs[ft]);
+            });
         }
     }
 }
@@ -684,13 +705,24 @@ __global__ __launch_bounds__(256) void mlp_norm_grads_kernel(MlpBwdArgs a, int64
         f32x4 xv[4];
         float2 st[4];
         uint2 dv[4];
+        int64_t tt[4];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int64_t tt = t + u * lanes < t1 ? t + u * lanes : t1 - 1;
-            st[u] = *reinterpret_cast<const float2*>(a.stats + 2 * tt);
-            xv[u] = ld4(a.x, tt * a.xs + 4 * cq, a.x_dtype);
-            dv[u] = *reinterpret_cast<const uint2*>(a.dn + (size_t)tt * a.C + 4 * cq);
+            tt[u] = t + u * lanes < t1 ? t + u * lanes : t1 - 1;
+            st[u] = *reinterpret_cast<const float2*>(a.stats + 2 * tt[u]);
+            dv[u] = *reinterpret_cast<const uint2*>(a.dn + (size_t)tt[u] * a.C + 4 * cq);
         }
+        with_dtype(a.x_dtype, [&](auto dc) {        // one branch on the element type, the four loads back to back
+            constexpr int DT = decltype(dc)::value;
+            typename Raw4<DT>::type raw[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if constexpr (DT == 0) raw[u] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(a.x) + tt[u] * a.xs + 4 * cq);
+                else raw[u] = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(a.x) + tt[u] * a.xs + 4 * cq);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) xv[u] = unpack4<DT>(raw[u]);
+        });
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             if (t + u * lanes >= t1) continue;
