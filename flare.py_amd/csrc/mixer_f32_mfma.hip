@@ -81,7 +81,11 @@ __global__ __launch_bounds__(256) void gather_f32_mfma_kernel(MixerArgs a)
     // while this one is worked on (rows past the range repeat its last row: no branch around a load)
     f32x4 ka[QL / 4], vr[VPT];
     uint8_t keep_n[4] = {1, 1, 1, 1};      // key mask of the lane's four tokens (rows 4g + r of the tile)
-    bool vkeep[VPT];                       // the V chunk's token takes part (else it is staged as zeros: 0 * NaN is NaN)
+    // the V chunk's token takes part (else it is staged as zeros: 0 * NaN is NaN): inside the range, and its mask byte,
+    // kept as loaded until the chunk is staged -- a flag computed from the byte here would wait for it, and with it,
+    // in order, for the K and V rows requested around it
+    bool vin[VPT];
+    uint32_t vmb[VPT];
     auto fetch = [&](int n0) {
         if (mask != nullptr) {
 #pragma unroll
@@ -95,7 +99,8 @@ __global__ __launch_bounds__(256) void gather_f32_mfma_kernel(MixerArgs a)
             const int c = lane + 64 * i, tok = c / (D / 4), ch = c % (D / 4);
             const int nv = max(min(n0 + tok, n_end - 1), 0);
             vr[i] = *reinterpret_cast<const f32x4*>(v + (int64_t)nv * a.vs[2] + 4 * ch);
-            vkeep[i] = n0 + tok < n_end && (mask == nullptr || mask[nv] != 0);
+            vin[i] = n0 + tok < n_end;
+            vmb[i] = mask != nullptr ? (uint32_t)mask[nv] : 1u;
         }
     };
     int n0 = n_begin + 16 * w;
@@ -110,7 +115,7 @@ __global__ __launch_bounds__(256) void gather_f32_mfma_kernel(MixerArgs a)
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
             const int c = lane + 64 * i, tok = c / (D / 4), ch = c % (D / 4);
-            *reinterpret_cast<f32x4*>(&vt[w][tok][4 * ch]) = vkeep[i] ? vr[i] : f32x4{0.f, 0.f, 0.f, 0.f};
+            *reinterpret_cast<f32x4*>(&vt[w][tok][4 * ch]) = (vin[i] && vmb[i] != 0) ? vr[i] : f32x4{0.f, 0.f, 0.f, 0.f};
         }
         asm volatile("" ::: "memory");
         bool valid[4];      // a token past the range or padded by the key mask takes no part

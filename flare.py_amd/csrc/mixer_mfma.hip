@@ -221,7 +221,10 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
     // token that is padded or lies past the range keeps a (finite) K row but gets a zero V row and a zero in the
     // tile's row of "ones": whatever its probability, it adds nothing to the numerators or the denominators.
     u32x4 kr[2][CPT], vr[2][CPT];
-    bool live[2][CPT];
+    // the token's mask byte as loaded and "inside the range": combined only where the tile is stored -- a flag computed
+    // from the byte at the load would wait for it there, and with it, in order, for the K and V rows requested just before
+    uint32_t mbyte[2][CPT];
+    bool inr[2][CPT];
     auto load_tile = [&](auto set_tag, int n0, auto masked_tag) {
         constexpr int S = decltype(set_tag)::value;
         constexpr bool MASKED = decltype(masked_tag)::value;
@@ -232,7 +235,10 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                 const int nn = n0 + c / CH, n = max(min(nn, n_end - 1), 0), ch = c % CH;
                 kr[S][i] = load16_stream(k + (int64_t)n * a.ks[2] + ch * 8);
                 vr[S][i] = load16_stream(v + (int64_t)n * a.vs[2] + ch * 8);
-                if constexpr (MASKED) live[S][i] = nn < n_end && mask[n] != 0;
+                if constexpr (MASKED) {
+                    mbyte[S][i] = mask[n];
+                    inr[S][i] = nn < n_end;
+                }
             }
         }
     };
@@ -246,8 +252,9 @@ __global__ __launch_bounds__(256, 2) void gather_mfma_kernel(MixerArgs a)
                 const int tok = c / CH, ch = c % CH;
                 *reinterpret_cast<u32x4*>(&kt[S][k_slot(tok, ch)]) = kr[S][i];
                 if constexpr (MASKED) {
-                    *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = live[S][i] ? to_bf16x8<T>(vr[S][i]) : zero4();
-                    if (ch == 0) mt[S][tok] = live[S][i] ? uint16_t(P_::kOnes2 & 0xffffu) : uint16_t(0);
+                    const bool live = inr[S][i] && mbyte[S][i] != 0;
+                    *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = live ? to_bf16x8<T>(vr[S][i]) : zero4();
+                    if (ch == 0) mt[S][tok] = live ? uint16_t(P_::kOnes2 & 0xffffu) : uint16_t(0);
                 } else {
                     *reinterpret_cast<u32x4*>(&vt[S][v_slot(tok, ch)]) = to_bf16x8<T>(vr[S][i]);
                 }
@@ -569,7 +576,14 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
     const u32x4 ones8 = {P_::kOnes2, P_::kOnes2, P_::kOnes2, P_::kOnes2};
     const f32x4 zf = {0.f, 0.f, 0.f, 0.f};
 
-    auto load_k = [&](int t0, u32x4 (&dst)[kSTW][KD]) {
+    // (the tokens' mask bytes travel with their K rows: loaded where a tile's rows are stored, the byte would be waited for
+    // on the spot, and with it, in order, the K rows of the next tile requested before)
+    auto load_k = [&](int t0, u32x4 (&dst)[kSTW][KD], uint32_t (&mdst)[kSTW]) {
+#pragma unroll
+        for (int tw = 0; tw < kSTW; ++tw) {
+            const int n = t0 + tw * 16 + c16;
+            mdst[tw] = mask != nullptr ? (uint32_t)mask[n < wg_n1 ? n : wg_n1 - 1] : 1u;
+        }
         if (CH == 4 * KD && t0 + kSTokWave <= wg_n1) {      // wave-uniform: whole tile in range, no per-lane tests
             const uint16_t* kr = k + (int64_t)(t0 + c16) * a.ks[2] + g * 8;
 #pragma unroll
@@ -604,7 +618,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
     };
 
     // one 64-token tile of this wave: kb = its K rows as B operands
-    auto tile64 = [&](const u32x4 (&kb)[kSTW][KD], int t0) {
+    auto tile64 = [&](const u32x4 (&kb)[kSTW][KD], const uint32_t (&mb)[kSTW], int t0) {
         f32x4 yacc[kSTW][RT];
         float lrow[kSTW];       // softmax denominators, complete for the lane's token
         float lshift[kSTW];     // log2 shift the denominators are relative to (0 in the optimistic pass)
@@ -753,7 +767,7 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
             for (int tw = 0; tw < kSTW; ++tw) {
                 const int n = t0 + tw * 16 + c16;
                 const bool in = FULL || n < wg_n1;
-                const bool on = FULL || (in && (mask == nullptr || mask[n] != 0));
+                const bool on = FULL || (in && mb[tw] != 0);
                 const float inv = on ? __builtin_amdgcn_rcpf(lrow[tw]) * (drop ? a.drop_rs : 1.f) : 0.f;
                 if (in) {
                     uint16_t* yr = yr0 + (int64_t)tw * 16 * a.ys[2];
@@ -788,15 +802,16 @@ __global__ __launch_bounds__(256, 2) void scatter_mfma_kernel(MixerArgs a, int t
 
     // two K register sets alternate, each fetched one tile before its use
     u32x4 ka[kSTW][KD], kc[kSTW][KD];
+    uint32_t ma[kSTW], mc[kSTW];
     constexpr int kStride = 4 * kSTokWave;
     int t0 = wg_n0 + w * kSTokWave;
-    if (t0 < wg_n1) load_k(t0, ka);
+    if (t0 < wg_n1) load_k(t0, ka, ma);
     for (; t0 < wg_n1; t0 += 2 * kStride) {
-        if (t0 + kStride < wg_n1) load_k(t0 + kStride, kc);
-        tile64(ka, t0);
+        if (t0 + kStride < wg_n1) load_k(t0 + kStride, kc, mc);
+        tile64(ka, ma, t0);
         if (t0 + kStride < wg_n1) {
-            if (t0 + 2 * kStride < wg_n1) load_k(t0 + 2 * kStride, ka);
-            tile64(kc, t0 + kStride);
+            if (t0 + 2 * kStride < wg_n1) load_k(t0 + 2 * kStride, ka, ma);
+            tile64(kc, mc, t0 + kStride);
         }
     }
 }
