@@ -455,8 +455,9 @@ def test_many_token_instances_of_every_mode(dev, C):
         assert torch.equal(fused.fused_mlp(yp, lin, torch.bfloat16, x_head=8), fused.fused_mlp(y, lin, torch.bfloat16))
 
 
+@pytest.mark.parametrize("cd", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("C,n", [(128, -1), (128, 0), (128, 1), (128, 2), (128, 3), (64, 0), (64, 4), (64, 6), (64, 7), (32, 2)])
-def test_bias_vectors_in_registers_over_several_passes(dev, C, n):
+def test_bias_vectors_in_registers_over_several_passes(dev, C, n, cd):
     """The many-token chain keeps the bias of every layer in registers as a ring that turns by one per layer and has
     to be back at layer 0 when the workgroup's next pass begins, whatever the number of layers: enough tokens for
     three to four passes per workgroup, every chain length the ring takes at this width and one beyond it (C = 64,
@@ -470,11 +471,11 @@ def test_bias_vectors_in_registers_over_several_passes(dev, C, n):
     norm = nn.LayerNorm(C).to(dev)
     nn.init.normal_(norm.weight, 1.0, 0.3)
     nn.init.normal_(norm.bias, 0.0, 0.3)
-    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
-        y = fused.fused_mlp(x, m, torch.bfloat16, norm=norm, res=x)
-        y2 = fused.fused_mlp(x, m, torch.bfloat16, norm=norm, res=x)
+    with torch.no_grad(), torch.autocast("cuda", dtype=cd):
+        y = fused.fused_mlp(x, m, cd, norm=norm, res=x)
+        y2 = fused.fused_mlp(x, m, cd, norm=norm, res=x)
     assert torch.equal(y, y2)
-    ref = oracle_of(m, x, torch.bfloat16, norm, x)
+    ref = oracle_of(m, x, cd, norm, x)
     assert O.rel_l2(y, ref) <= 2e-2
     # the last pass of the last workgroup as well as the first: a ring out of step shows as a wrong bias, i.e. an error of
     # the order of the bias itself in every row of the later passes
