@@ -18,6 +18,8 @@ FLAG_FORCE_GENERIC = 1
 FLAG_MFMA16 = 2
 FLAG_GRAD_LIKE_KV = 8
 MLP_EXPAND = 1
+MLP_BWD_ADD_DY = 1           # bits of flare_mlp_bwd's add_dy argument
+MLP_BWD_ACCUMULATE = 2
 ABI_VERSION = 2
 STATIC_SCRATCH_BYTES = 64 << 20
 

@@ -1024,7 +1024,8 @@ int flare_mlp_bwd(const FlareMlpDesc* d, const void* x, const void* dy, const vo
     a.T = d->T; a.C = d->C; a.L = d->L;
     a.x_dtype = d->x_dtype; a.dy_dtype = d->y_dtype; a.dx_dtype = d->x_dtype;
     a.norm = d->norm; a.eps = d->eps; a.act = d->act; a.act_mask = d->act_mask; a.add_mask = d->add_mask;
-    a.add_dy = add_dy ? 1 : 0;
+    if (add_dy & ~(FLARE_MLP_BWD_ADD_DY | FLARE_MLP_BWD_ACCUMULATE)) return fail(FLARE_EINVAL, "add_dy holds unknown bits (got %d)", add_dy);
+    a.add_dy = add_dy;
     a.xs = d->x_stride; a.dys = d->y_stride; a.dxs = d->C;
     return hip_status(flare::launch_mlp_bwd(a, d->w_dtype, static_cast<hipStream_t>(stream)), "mlp backward launch");
 }

@@ -274,7 +274,7 @@ struct MlpBwdArgs {
     float eps;
     int act;                                    // 0 tanh-GELU, 1 SiLU
     uint32_t act_mask, add_mask;
-    int add_dy;                                 // the forward's residual input was x itself: dx also receives dy
+    int add_dy;                                 // bit 0: the forward's residual input was x itself, dx also receives dy; bit 1 (chain only): dx holds a gradient already and receives the sum
     int64_t xs, dys, dxs;                       // row strides in elements
 };
 

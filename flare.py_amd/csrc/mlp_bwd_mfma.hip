@@ -453,8 +453,11 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_kernel(MlpBwdArgs a, in
         if (live) {
             // every load of dy before the first store of dx (a load written after a store stays behind it: the two
             // may be the same memory as far as the compiler knows)
-            if (a.add_dy) {
+            if (a.add_dy & 1) {
                 load_row<FT>(a.dy, a.dy_dtype, tok * a.dys + 4 * g, [&](int ft, f32x4 v) { xs[ft] += v; });
+            }
+            if (a.add_dy & 2) {     // dx holds another path's gradient of the same x: the sum goes back
+                load_row<FT>(a.dx, a.dx_dtype, tok * a.dxs + 4 * g, [&](int ft, f32x4 v) { xs[ft] += v; });
             }
             with_dtype(a.dx_dtype, [&](auto dc) {
 #pragma unroll
@@ -677,7 +680,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void mlp_bwd_expand_kernel(MlpBwdArg
             }
         }
         if (live) {
-            if (a.add_dy) {
+            if (a.add_dy & 1) {
                 load_row<FT>(a.dy, a.dy_dtype, tok * a.dys + 4 * g, [&](int ft, f32x4 v) { xs[ft] += v; });
             }
             with_dtype(a.dx_dtype, [&](auto dc) {

@@ -360,6 +360,22 @@ def fused_mlp(x, mod, cd, norm=None, res=None, out_dtype=None, x_head=0, y_head=
     return _fused_mlp_fwd(x, mod, cd, norm, res, out_dtype, x_head, y_head)
 
 
+def fused_mlp_pair(x, mod_a, mod_b, cd, norm=None, out_dtype=None):
+    """(mod_a(norm(x)), mod_b(norm(x))) as fused_mlp computes them, for two stacks that read the same rows through the
+    same norm (a block's k and v projections).  With gradients enabled and both stacks plain chains of C x C layers the
+    pair is one autograd node whose backward sums the two gradients of x inside the second launch."""
+    if torch.is_grad_enabled() and all(_train_subchain(m) is None and not _expand_factor(m, x.shape[-1]) for m in (mod_a, mod_b)):
+        has_norm = norm is not None and not isinstance(norm, nn.Identity)
+        gamma = getattr(norm, "weight", None) if has_norm else None
+        beta = getattr(norm, "bias", None) if has_norm else None
+        wb = []
+        for m in (mod_a, mod_b):
+            layers = _layers_of(m)[0]
+            wb += [l.weight for l in layers] + [l.bias for l in layers]
+        return _FusedPairFn.apply(mod_a, mod_b, cd, norm if has_norm else None, out_dtype, x, gamma, beta, *wb)
+    return fused_mlp(x, mod_a, cd, norm=norm, out_dtype=out_dtype), fused_mlp(x, mod_b, cd, norm=norm, out_dtype=out_dtype)
+
+
 def _fused_mlp_fwd(x, mod, cd, norm=None, res=None, out_dtype=None, x_head=0, y_head=0):
     lib = _lib.load()
     info = _layers_of(mod)
@@ -518,63 +534,113 @@ class _FusedMlpFn(torch.autograd.Function):
         if ctx.versions != tuple(None if t is None else t._version for t in ctx.params):
             raise RuntimeError("a parameter of the fused MLP was modified in place between its forward and its backward")
         mod, cd, norm = ctx.mod, ctx.cd, ctx.norm
-        lib = _lib.load()
-        layers, act_mask, add_mask, act = _layers_of(mod)
+        if _expand_factor(mod, x.shape[-1]):
+            return _backward_expand(ctx, dy, x, _expand_factor(mod, x.shape[-1]))
+        dx, gsum, dW, db, layers = _chain_backward(mod, cd, norm, x, dy, ctx.res_is_x)
         L = len(layers)
-        Cdim = x.shape[-1]
-        E = _expand_factor(mod, Cdim)
-        if E:
-            return _backward_expand(ctx, dy, x, E)
-        _, b, w_img, wt_img = _packed_train(mod, layers, cd)
-        x2 = x.reshape(-1, Cdim)
-        if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 16:
-            x2 = x2.contiguous()
-        dy2 = dy.reshape(-1, Cdim)
-        if dy2.dtype not in (torch.float32, torch.bfloat16, torch.float16):
-            dy2 = dy2.float()
-        if dy2.stride(-1) != 1 or dy2.stride(0) % 4 or dy2.data_ptr() % 16:
-            dy2 = dy2.contiguous()
-        T = x2.shape[0]
-        dev = x.device
-        d = _lib.FlareMlpDesc()
-        d.T, d.C, d.L = T, Cdim, L
-        d.w_dtype, d.x_dtype, d.y_dtype = _dtype_code(w_img), _dtype_code(x2), _dtype_code(dy2)
-        d.act, d.act_mask, d.add_mask = act, act_mask, add_mask
-        d.x_stride, d.y_stride = x2.stride(0), dy2.stride(0)
-        gamma, beta = _norm_args(d, norm, x, Cdim)
-        dx = torch.empty(T, Cdim, dtype=x2.dtype, device=dev)
-        a_in = torch.empty(L, T, Cdim, dtype=cd, device=dev)
-        g_out = torch.empty(L, T, Cdim, dtype=cd, device=dev)
-        dn = stats = gb = gsum = None
-        any_bias = any(l.bias is not None for l in layers)
-        if d.norm:
-            rows = C.c_int32(0)
-            _lib.check(lib.flare_mlp_bwd_partial_rows(C.byref(d), C.byref(rows)), "flare_mlp_bwd_partial_rows")
-            dn = torch.empty(T, Cdim, dtype=cd, device=dev)
-            stats = torch.empty(T, 2, dtype=torch.float32, device=dev)
-            gb = torch.empty(rows.value, 2, Cdim, dtype=torch.float32, device=dev)
-            gsum = torch.empty(2, Cdim, dtype=torch.float32, device=dev)
-        with _on_device(dev):
-            rc = lib.flare_mlp_bwd(C.byref(d), _ptr(x2), _ptr(dy2), _ptr(w_img), _ptr(wt_img), _ptr(b), _ptr(gamma), _ptr(beta),
-                                   1 if ctx.res_is_x else 0, _ptr(dx), _ptr(a_in), _ptr(g_out), _ptr(dn), _ptr(stats), _ptr(gb),
-                                   _ptr(gsum), C.c_void_p(_stream_ptr(dev)))
-        _lib.check(rc, "flare_mlp_bwd")
-        # weight and bias gradients: one more launch over the rows the kernel left (16-bit products with fp32
-        # accumulation, as torch runs a Linear's backward under autocast); norm gradients: partial rows, summed here
-        dW, db = _weight_grads(d, g_out, a_in, any_bias)                 # [L, out, in], [L, C] fp32
         need = ctx.needs_input_grad            # (mod, cd, norm, out_dtype, x, res, gamma, beta, *wb)
         grads = [None, None, None, None]
         grads.append(dx.view(x.shape) if need[4] else None)
         grads.append(None if (not ctx.has_res or ctx.res_is_x or not need[5]) else dy)
-        if d.norm:
-            grads.append(gsum[0].to(norm.weight.dtype) if need[6] else None)
-            grads.append(gsum[1].to(norm.bias.dtype) if (need[7] and getattr(norm, "bias", None) is not None) else None)
-        else:
-            grads += [None, None]
+        grads += _norm_grads(norm, gsum, need[6], need[7])
         for i, l in enumerate(layers):
             grads.append(dW[i].to(l.weight.dtype) if need[8 + i] else None)
         for i, l in enumerate(layers):
             grads.append(db[i].to(l.bias.dtype) if (l.bias is not None and need[8 + L + i]) else None)
+        return tuple(grads)
+
+
+def _norm_grads(norm, gsum, need_gamma, need_beta):
+    if gsum is None:
+        return [None, None]
+    return [gsum[0].to(norm.weight.dtype) if need_gamma else None,
+            gsum[1].to(norm.bias.dtype) if (need_beta and getattr(norm, "bias", None) is not None) else None]
+
+
+def _chain_backward(mod, cd, norm, x, dy, res_is_x, dx_acc=None):
+    """Backward of y = [x +] chain(norm(x)) for the chain of C x C layers: (dx [T,C], the norm's [2,C] sums or None,
+    dW [L,out,in], db [L,C] or None, the layers).  dx_acc: a [T,C] gradient of the same x that another chain left
+    (x's dtype, contiguous); the kernel adds its result into it and it is returned as dx."""
+    lib = _lib.load()
+    layers, act_mask, add_mask, act = _layers_of(mod)
+    L = len(layers)
+    Cdim = x.shape[-1]
+    _, b, w_img, wt_img = _packed_train(mod, layers, cd)
+    x2 = x.reshape(-1, Cdim)
+    if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    dy2 = _rows2d(dy, Cdim)
+    T = x2.shape[0]
+    dev = x.device
+    d = _lib.FlareMlpDesc()
+    d.T, d.C, d.L = T, Cdim, L
+    d.w_dtype, d.x_dtype, d.y_dtype = _dtype_code(w_img), _dtype_code(x2), _dtype_code(dy2)
+    d.act, d.act_mask, d.add_mask = act, act_mask, add_mask
+    d.x_stride, d.y_stride = x2.stride(0), dy2.stride(0)
+    gamma, beta = _norm_args(d, norm, x, Cdim)
+    if dx_acc is not None and (dx_acc.shape != (T, Cdim) or dx_acc.dtype != x2.dtype or not dx_acc.is_contiguous()):
+        raise ValueError("dx_acc must be a contiguous [T, C] tensor of x's dtype")
+    dx = dx_acc if dx_acc is not None else torch.empty(T, Cdim, dtype=x2.dtype, device=dev)
+    a_in = torch.empty(L, T, Cdim, dtype=cd, device=dev)
+    g_out = torch.empty(L, T, Cdim, dtype=cd, device=dev)
+    dn = stats = gb = gsum = None
+    any_bias = any(l.bias is not None for l in layers)
+    if d.norm:
+        rows = C.c_int32(0)
+        _lib.check(lib.flare_mlp_bwd_partial_rows(C.byref(d), C.byref(rows)), "flare_mlp_bwd_partial_rows")
+        dn = torch.empty(T, Cdim, dtype=cd, device=dev)
+        stats = torch.empty(T, 2, dtype=torch.float32, device=dev)
+        gb = torch.empty(rows.value, 2, Cdim, dtype=torch.float32, device=dev)
+        gsum = torch.empty(2, Cdim, dtype=torch.float32, device=dev)
+    bits = (_lib.MLP_BWD_ADD_DY if res_is_x else 0) | (_lib.MLP_BWD_ACCUMULATE if dx_acc is not None else 0)
+    with _on_device(dev):
+        rc = lib.flare_mlp_bwd(C.byref(d), _ptr(x2), _ptr(dy2), _ptr(w_img), _ptr(wt_img), _ptr(b), _ptr(gamma), _ptr(beta),
+                               bits, _ptr(dx), _ptr(a_in), _ptr(g_out), _ptr(dn), _ptr(stats), _ptr(gb),
+                               _ptr(gsum), C.c_void_p(_stream_ptr(dev)))
+    _lib.check(rc, "flare_mlp_bwd")
+    # weight and bias gradients: one more launch over the rows the kernel left (16-bit products with fp32
+    # accumulation, as torch runs a Linear's backward under autocast); norm gradients: partial rows, summed by the launch
+    dW, db = _weight_grads(d, g_out, a_in, any_bias)                 # [L, out, in], [L, C] fp32
+    return dx, gsum, dW, db, layers
+
+
+class _FusedPairFn(torch.autograd.Function):
+    """(ya, yb) = (chain_a(norm(x)), chain_b(norm(x))): two chains that read the same rows through the same norm (the k
+    and v projections of a block).  Forward: the two launches of _FusedMlpFn.  Backward: the second chain's launch adds
+    its gradient of x into the first one's, which autograd would otherwise do with a launch of its own over three
+    [T, C] arrays.  Inputs: (x, gamma, beta, weights and biases of a, weights and biases of b)."""
+
+    @staticmethod
+    def forward(ctx, mod_a, mod_b, cd, norm, out_dtype, x, gamma, beta, *wb):
+        with torch.no_grad():
+            ya = _fused_mlp_fwd(x, mod_a, cd, norm=norm, out_dtype=out_dtype)
+            yb = _fused_mlp_fwd(x, mod_b, cd, norm=norm, out_dtype=out_dtype)
+        ctx.mods, ctx.cd, ctx.norm = (mod_a, mod_b), cd, norm
+        ctx.versions = tuple(None if t is None else t._version for t in (gamma, beta, *wb))
+        ctx.params = (gamma, beta, *wb)
+        ctx.save_for_backward(x)
+        return ya, yb
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dya, dyb):
+        (x,) = ctx.saved_tensors
+        if ctx.versions != tuple(None if t is None else t._version for t in ctx.params):
+            raise RuntimeError("a parameter of the fused MLP was modified in place between its forward and its backward")
+        mod_a, mod_b = ctx.mods
+        dx, gs_a, dWa, dba, la = _chain_backward(mod_a, ctx.cd, ctx.norm, x, dya, False)
+        dx, gs_b, dWb, dbb, lb = _chain_backward(mod_b, ctx.cd, ctx.norm, x, dyb, False, dx_acc=dx)
+        need = ctx.needs_input_grad            # (mod_a, mod_b, cd, norm, out_dtype, x, gamma, beta, *wb)
+        grads = [None, None, None, None, None, dx.view(x.shape) if need[5] else None]
+        grads += _norm_grads(ctx.norm, None if gs_a is None else gs_a + gs_b, need[6], need[7])
+        at = 8
+        for layers, dW, db in ((la, dWa, dba), (lb, dWb, dbb)):
+            n = len(layers)
+            for i, l in enumerate(layers):
+                grads.append(dW[i].to(l.weight.dtype) if need[at + i] else None)
+            for i, l in enumerate(layers):
+                grads.append(db[i].to(l.bias.dtype) if (l.bias is not None and need[at + n + i]) else None)
+            at += 2 * n
         return tuple(grads)
 
 

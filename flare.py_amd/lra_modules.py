@@ -91,8 +91,7 @@ class FLARE(nn.Module):
         q = self.latent_q.view(self.num_heads, self.num_latents, self.head_dim)
         cd = self._fusable(x)
         if cd is not None:
-            k = fused.fused_mlp(x, self.k_proj, cd, norm=_norm, out_dtype=cd)
-            v = fused.fused_mlp(x, self.v_proj, cd, norm=_norm, out_dtype=cd)
+            k, v = fused.fused_mlp_pair(x, self.k_proj, self.v_proj, cd, norm=_norm, out_dtype=cd)
         else:
             xn = x if _norm is None else _norm(x)
             k, v = self.k_proj(xn), self.v_proj(xn)

@@ -190,8 +190,8 @@ class FLARE(nn.Module):
             out_dtype = _res.dtype if _res is not None else x.dtype
             return fused.fused_mlp(y, self.out_proj, cd, res=_res, out_dtype=out_dtype, x_head=D), None
         if cd is not None:
-            k = self._heads(fused.fused_mlp(x, self.k_proj, cd, norm=_norm, out_dtype=cd))
-            v = self._heads(fused.fused_mlp(x, self.v_proj, cd, norm=_norm, out_dtype=cd))
+            k, v = fused.fused_mlp_pair(x, self.k_proj, self.v_proj, cd, norm=_norm, out_dtype=cd)
+            k, v = self._heads(k), self._heads(v)
             if self.qk_norm:
                 q = self.q_norm(q)
                 k = self.k_norm(k)

@@ -355,12 +355,18 @@ int flare_mlp_io_fwd(const FlareMlpDesc* desc, int32_t in_dim, int32_t in_act, c
                      const float* b_in, int32_t out_dim, const void* x, const void* w, const float* bias,
                      const float* gamma, const float* beta, const void* res, void* y, void* stream);
 
+#define FLARE_MLP_BWD_ADD_DY 1
+#define FLARE_MLP_BWD_ACCUMULATE 2
+
 /* Backward of flare_mlp_fwd for the chain of C x C layers (desc->flags == 0; at most 8 layers, 5 at C = 128): what
  * torch autograd computes for  y = res + ResidualMLP(norm(x))  (pdebench/models/flare.py:45-59, 204-215) when
  * the reference trains a block.  One token-parallel launch recomputes the forward and walks the chain back;
  * the reductions over all tokens that the weight and bias gradients need are a second call (flare_mlp_wgrad below):
- *   dx      [T,C]   contiguous, x's dtype: gradient of x (plus dy when add_dy != 0: the forward's res was x itself;
- *                   otherwise the gradient of res is dy)
+ *   dx      [T,C]   contiguous, x's dtype: gradient of x.  add_dy is a set of bits: FLARE_MLP_BWD_ADD_DY = dy is
+ *                   added (the forward's res was x itself; otherwise the gradient of res is dy);
+ *                   FLARE_MLP_BWD_ACCUMULATE (this entry point only) = dx already holds a gradient of the same x, from
+ *                   another chain that read it (the k and v projections of one block), and receives the sum -- what
+ *                   autograd would otherwise add with a launch of its own
  *   a_in    [L,T,C] the input of every layer and
  *   g_out   [L,T,C] the gradient at every layer's product, both in the weights' type:
  *                   dW_l = g_out[l]^T a_in[l],  db_l = column sums of g_out[l]  (flare_mlp_wgrad forms both)

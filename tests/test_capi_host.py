@@ -244,6 +244,9 @@ def test_mlp_bwd_validation():
         return lib.flare_mlp_bwd(m, x, dy, fake, fake, ff, gamma, ff, 0, fake, fake, fake, dn, stats, gb, None, None)
 
     assert lib.flare_mlp_bwd(None, *([None] * 7), 0, *([None] * 8)) == _lib.FLARE_EINVAL
+    # add_dy is a set of two bits (add dy, accumulate into dx); anything else is refused before a launch
+    assert lib.flare_mlp_bwd(m, fake, fake, fake, fake, ff, ff, ff, 4, fake, fake, fake, fake, ff, ff, None, None) == _lib.FLARE_EINVAL
+    assert "unknown bits" in _lib.last_error()
     assert call(x=None) == _lib.FLARE_EINVAL and "must not be NULL" in _lib.last_error()
     assert call(gamma=None) == _lib.FLARE_EINVAL and "norm" in _lib.last_error()
     assert call(gb=None) == _lib.FLARE_EINVAL and "norm" in _lib.last_error()

@@ -149,6 +149,45 @@ def test_backward_is_deterministic(dev):
     assert all(torch.equal(u, v) for u, v in zip(a, b))
 
 
+@pytest.mark.parametrize("C,T,xdt", [(128, 70000, torch.float32), (64, 5000, torch.float32), (128, 3000, torch.bfloat16)])
+def test_pair_of_chains_sums_its_input_gradients_in_the_second_launch(dev, C, T, xdt):
+    """fused_mlp_pair (a block's k and v projections over the same normalised rows) against the two stacks called one by
+    one: same outputs; with fp32 rows the gradient of x is bit-equal (one fp32 addition either way), with 16-bit rows it
+    differs by the rounding the separate sum takes twice; every parameter gradient bit-equal."""
+    torch.manual_seed(11)
+    ma = ResidualMLP(C, C, C, num_layers=3, act="gelu", input_residual=True, output_residual=True).to(dev)
+    mb = ResidualMLP(C, C, C, num_layers=1, act="gelu", input_residual=True, output_residual=True).to(dev)
+    norm = nn.LayerNorm(C).to(dev)
+    nn.init.normal_(norm.weight, 1.0, 0.2)
+    x = torch.randn(T, C, device=dev).to(xdt).requires_grad_(True)
+    ga, gb = torch.randn(T, C, device=dev), torch.randn(T, C, device=dev)
+    params = list(ma.parameters()) + list(mb.parameters()) + list(norm.parameters())
+
+    def run(pair):
+        for p in [x] + params:
+            p.grad = None
+        with torch.autocast("cuda", torch.bfloat16):
+            if pair:
+                ya, yb = fused.fused_mlp_pair(x, ma, mb, torch.bfloat16, norm=norm, out_dtype=torch.bfloat16)
+            else:
+                ya = fused.fused_mlp(x, ma, torch.bfloat16, norm=norm, out_dtype=torch.bfloat16)
+                yb = fused.fused_mlp(x, mb, torch.bfloat16, norm=norm, out_dtype=torch.bfloat16)
+        ((ya.float() * ga).sum() + (yb.float() * gb).sum()).backward()
+        return ya.detach(), yb.detach(), x.grad.clone(), [p.grad.clone() for p in params]
+
+    ya1, yb1, gx1, gp1 = run(True)
+    ya0, yb0, gx0, gp0 = run(False)
+    assert torch.equal(ya1, ya0) and torch.equal(yb1, yb0)
+    if xdt == torch.float32:
+        assert torch.equal(gx1, gx0)
+    else:
+        assert (gx1.float() - gx0.float()).norm() <= 1e-2 * gx0.float().norm()
+    for u, v in zip(gp1[:-2], gp0[:-2]):
+        assert torch.equal(u, v)
+    for u, v in zip(gp1[-2:], gp0[-2:]):        # the norm's parameters: the two chains' sums added in another order
+        assert (u - v).norm() <= 1e-5 * v.norm()
+
+
 @pytest.mark.parametrize("C,H,M,N", [(64, 8, 64, 3000), (128, 8, 128, 2000), (32, 2, 32, 1000)])
 def test_block_trains_through_the_fused_launches(dev, C, H, M, N):
     """A whole FLAREBlock under bf16 autocast with gradients enabled: fused projections and feed-forward (forward and
