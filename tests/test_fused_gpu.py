@@ -419,7 +419,7 @@ def test_graphed_forward_helper(dev):
 
 @pytest.mark.parametrize("C", [32, 64, 128])
 def test_many_token_instances_of_every_mode(dev, C):
-    """Launches of fewer than 32768 tokens take kernel instances with one 16-token tile per wave; this test feeds the
+    """Launches of up to 32768 tokens take kernel instances with one 16-token tile per wave; this test feeds the
     many-token instances (4 tiles per wave, 2 at C = 128) of every mode: chain with both norms, expanding MLP,
     narrow ends, head-padded rows."""
     T = 40000
