@@ -42,15 +42,21 @@ _ACTS = {"gelu": 0, "silu": 1}
 
 def _structure_key(mod):
     """Identity of everything the structural caches are built from: the layers, the activation module and the flags
-    that set the masks.  Assigning a new submodule (a LoRA wrap, a re-initialisation by assignment) changes it."""
+    that set the masks.  Assigning a new submodule (a LoRA wrap, a re-initialisation by assignment) changes it.
+    Read from the module's own tables: every fused call asks several times, and attribute access on a Module goes
+    through its __getattr__ for submodules."""
     if isinstance(mod, _SubChain):
         return None
-    if isinstance(mod, nn.Linear) or getattr(mod, "num_layers", None) is None:
+    d = mod.__dict__
+    nl = d.get("num_layers")
+    if isinstance(mod, nn.Linear) or nl is None:
         return (type(mod),)
-    if mod.num_layers == -1:
-        return (-1, id(mod.fc), bool(mod.residual))
-    return (mod.num_layers, id(mod.fc1), tuple(id(l) for l in mod.fcs), id(mod.fc2), id(mod.act),
-            getattr(mod.act, "approximate", None), bool(mod.input_residual), bool(mod.output_residual))
+    m = d["_modules"]
+    if nl == -1:
+        return (-1, id(m["fc"]), bool(d["residual"]))
+    act = m["act"] if "act" in m else d.get("act")
+    return (nl, id(m["fc1"]), tuple(map(id, m["fcs"]._modules.values())), id(m["fc2"]), id(act),
+            getattr(act, "approximate", None), bool(d["input_residual"]), bool(d["output_residual"]))
 
 
 def _layers_of(mod):
@@ -186,35 +192,16 @@ def compute_dtype(x, mod):
     flare_mlp_expand_bwd differentiate), and a stack with a narrow end for the chain between its narrow layers."""
     if x.device.type != "cuda":
         return None
-    info = _layers_of(mod)
-    if info is None:
+    # what depends on the module's structure and the row width only is decided once per (structure, width, grad mode)
+    grad = torch.is_grad_enabled()
+    key = (_structure_key(mod), x.shape[-1], grad)
+    cached = mod.__dict__.get("_flare_shape_ok")
+    if cached is None or cached[0] != key:
+        cached = (key, _shape_ok(x.shape[-1], mod, grad))
+        mod.__dict__["_flare_shape_ok"] = cached
+    if not cached[1]:
         return None
-    layers = info[0]
-    if len(layers) > 16:
-        return None
-    if torch.is_grad_enabled():
-        sub = _train_subchain(mod)
-        if sub is not None:                 # narrow first input / last output: the C x C layers between them
-            n = len(_layers_of(sub)[0])
-            if sub.C not in _SUPPORTED_C or n > _BWD_MAX_LAYERS[sub.C] or x.shape[-1] != layers[0].in_features:
-                return None
-        else:
-            Cdim = x.shape[-1]
-            if Cdim not in _SUPPORTED_C:
-                return None
-            if not _expand_factor(mod, Cdim):
-                if len(layers) > _BWD_MAX_LAYERS[Cdim] or any(l.in_features != Cdim or l.out_features != Cdim for l in layers):
-                    return None
-    io = _io_dims(mod, layers)
-    if io is not None and (io[1] or io[2]):
-        if io[0] not in _SUPPORTED_C or x.shape[-1] != layers[0].in_features:
-            return None
-    else:
-        Cdim = x.shape[-1]
-        if Cdim not in _SUPPORTED_C:
-            return None
-        if not _expand_factor(mod, Cdim) and any(l.in_features != Cdim or l.out_features != Cdim for l in layers):
-            return None
+    layers = _layers_of(mod)[0]
     if x.dtype not in (torch.float32, torch.bfloat16, torch.float16) or x.stride(-1) != 1:
         return None
     ac = _autocast_dtype(x)
@@ -224,6 +211,37 @@ def compute_dtype(x, mod):
     if ac is None and wd in (torch.bfloat16, torch.float16) and all(l.weight.dtype == wd for l in layers):
         return wd
     return None
+
+
+def _shape_ok(width, mod, grad):
+    info = _layers_of(mod)
+    if info is None:
+        return False
+    layers = info[0]
+    if len(layers) > 16:
+        return False
+    if grad:
+        sub = _train_subchain(mod)
+        if sub is not None:                 # narrow first input / last output: the C x C layers between them
+            n = len(_layers_of(sub)[0])
+            if sub.C not in _SUPPORTED_C or n > _BWD_MAX_LAYERS[sub.C] or width != layers[0].in_features:
+                return False
+        else:
+            if width not in _SUPPORTED_C:
+                return False
+            if not _expand_factor(mod, width):
+                if len(layers) > _BWD_MAX_LAYERS[width] or any(l.in_features != width or l.out_features != width for l in layers):
+                    return False
+    io = _io_dims(mod, layers)
+    if io is not None and (io[1] or io[2]):
+        if io[0] not in _SUPPORTED_C or width != layers[0].in_features:
+            return False
+    else:
+        if width not in _SUPPORTED_C:
+            return False
+        if not _expand_factor(mod, width) and any(l.in_features != width or l.out_features != width for l in layers):
+            return False
+    return True
 
 
 def _packed(mod, layers, cd):
