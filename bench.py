@@ -413,6 +413,14 @@ def bench_lra(args, F, dev):
                         prm.grad = None
 
                 row[f"ms_fwd_bwd_{dtype_name}_attn_drop_{p_drop}"] = round(time_events(step, max(5, args.steps // 5), 3), 3)
+                if ac is not None and p_drop == 0.0:
+                    # the same step (input gradient included) recorded once in a HIP graph and replayed: what is left
+                    # when the host's share of the launches is gone; the copies of x into the graph's buffer are inside
+                    from flare_py_amd import GraphedTrainStep
+                    zero = torch.zeros((), device=dev)
+                    graphed = GraphedTrainStep(blk, lambda y, t: y.float().square().mean(), autocast_dtype=ac)
+                    row[f"ms_fwd_bwd_{dtype_name}_attn_drop_0.0_graph_replay"] = round(
+                        time_events(lambda: graphed(xg, mask, zero), max(5, args.steps // 5), 3), 3)
             row[f"ratio_{dtype_name}"] = round(row[f"ms_fwd_bwd_{dtype_name}_attn_drop_0.1"] / row[f"ms_fwd_bwd_{dtype_name}_attn_drop_0.0"], 3)
         rows[name] = row
     head = rows["pathfinder32 (N=1024, no padding)"]
@@ -763,6 +771,40 @@ def bench_block(args, F, dev):
     out["train_block_4x_ffn"] = {"ms_fwd_bwd": round(ms_train4, 3),
                                  "ms_fwd_bwd_torch_layers_hip_mixer": None if ms_train4_torch is None else round(ms_train4_torch, 3),
                                  "what": "the same for the block with the 4x GELU MLP as its feed-forward (no lift)"}
+    # a whole model's training step where the launches, not the kernels, set the pace: 8 blocks (C=128, H=8, M=128,
+    # pdebench/models/flare.py:236-301) with fused AdamW on small meshes, enqueued eagerly and with forward + loss +
+    # backward replayed from one HIP graph (GraphedTrainStep; the optimizer step stays eager in both)
+    from flare_py_amd import GraphedTrainStep
+    from flare_py_amd import modules as Mod8
+    rows8 = {}
+    for n_pts in (4096, 16384, 65536):
+        torch.manual_seed(0)
+        model = Mod8.FLAREModel(in_dim=3, out_dim=1, channel_dim=128, num_blocks=8, num_heads=8, num_latents=128).to(dev).train()
+        prm = list(model.parameters())
+        opt = torch.optim.AdamW(prm, lr=1e-4, fused=True)
+        xm, tm = torch.randn(1, n_pts, 3, device=dev), torch.randn(1, n_pts, 1, device=dev)
+
+        def mse(o, t):
+            return ((o[0] if isinstance(o, tuple) else o).float() - t).square().mean()
+
+        def eager_step():
+            for p_ in prm:
+                p_.grad = None
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                o = model(xm)
+            mse(o, tm).backward()
+            opt.step()
+
+        graphed = GraphedTrainStep(model, mse, autocast_dtype=torch.bfloat16)
+
+        def graph_step():
+            graphed(xm, tm)
+            opt.step()
+
+        rows8[f"N={n_pts}"] = {"ms_eager": round(wall_ms(eager_step, 20, 5), 3), "ms_graph_replay": round(wall_ms(graph_step, 20, 5), 3),
+                               "ms_graph_replay_without_optimizer": round(wall_ms(lambda: graphed(xm, tm), 20, 5), 3)}
+        del graphed, model, opt
+    out["train_model_8_blocks_adamw"] = dict(rows8, what="forward + MSE + backward + fused AdamW of an 8-block model, B=1, bf16 autocast, wall clock per step")
     # the same modules the way the reference runs them on this device: torch Linear / LayerNorm layers under the
     # same autocast, the mixer as two torch scaled_dot_product_attention calls (pdebench/models/flare.py:122-156)
     try:

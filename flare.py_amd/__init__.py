@@ -22,9 +22,10 @@ from .functional import (
 )
 from .modules import FLARE, FLAREBlock, FLAREModel, FinalLayer, ResidualMLP
 from .serving import GraphedForward
+from .train_graph import GraphedTrainStep
 
 __all__ = [
     "CausalLinear", "causal_linear_attention", "FLARE", "FLAREBlock", "FLAREModel", "FinalLayer", "ResidualMLP", "TripleAttentionFunction",
     "causal_fresh_state", "causal_workspace", "flare_causal_decode", "flare_causal_decode_step", "flare_causal_prefill",
-    "flare_gather", "flare_multihead_mixer", "flare_scatter", "mixer_kernel_name", "triple_attention", "GraphedForward",
+    "flare_gather", "flare_multihead_mixer", "flare_scatter", "mixer_kernel_name", "triple_attention", "GraphedForward", "GraphedTrainStep",
 ]

@@ -428,8 +428,8 @@ def _masked_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, km, gy, drop=None):
         m4 = keep[:, None, :, None]
         zero = torch.zeros((), dtype=k.dtype, device=k.device)
         k, v, gy = torch.where(m4, k, zero), torch.where(m4, v, zero), torch.where(m4, gy.to(k.dtype), zero)
-        lse_tok = torch.where(keep[:, None, :], lse_tok, lse_tok.new_tensor(1e30))
-        lse_lat = torch.where(torch.isfinite(lse_lat), lse_lat, lse_lat.new_tensor(1e30))
+        lse_tok = torch.where(keep[:, None, :], lse_tok, 1e30)
+        lse_lat = torch.where(torch.isfinite(lse_lat), lse_lat, 1e30)
     gq, gk, gv = _mixer_hip_grad(q, k, v, y, z, lse_lat, lse_tok, scale, gy, drop)
     if km is not None:
         gk, gv = torch.where(m4, gk, zero), torch.where(m4, gv, zero)
@@ -774,7 +774,7 @@ def _half_hip_grad(which, q, k, x, z, aux, scale, key_mask, g):
         aux = aux.contiguous()
         if keep is not None:
             v = torch.where(m4, v, v.new_zeros(()))
-            aux = torch.where(torch.isfinite(aux), aux, aux.new_tensor(1e30))
+            aux = torch.where(torch.isfinite(aux), aux, 1e30)
         if v.data_ptr() % 16 or any(s % al for s in v.stride()[:3]):
             v = v.contiguous()
         gz = g.to(torch.float32).contiguous()
@@ -786,7 +786,7 @@ def _half_hip_grad(which, q, k, x, z, aux, scale, key_mask, g):
         aux = aux.contiguous()
         if keep is not None:
             gy = torch.where(m4, gy, gy.new_zeros(()))
-            aux = torch.where(keep[:, None, :], aux, aux.new_tensor(1e30))
+            aux = torch.where(keep[:, None, :], aux, 1e30)
         if gy.stride(-1) != 1 or any(s % al for s in gy.stride()[:3]) or gy.data_ptr() % 16:
             gy = gy.contiguous()
         d = _mixer_desc(q4, k, k, y, scale, 0, False)
