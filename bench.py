@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the FLARE mixer forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block|train|linear|fp32|layer|lra|power]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mixer|causal|triple|block|train|linear|fp32|layer|lra|model|power]
 
 One step = one forward of the mixer (split-N gather, merge, scatter) over the headline workload
 B=1, H=8, N=1,048,576, M=256, D=32, bf16 in / fp32 accumulate, inputs resident in HBM.
@@ -19,7 +19,8 @@ attention at B=4,H=8,N=16384,D=16 (elu+1, normalised); block = lift MLP 3 -> 128
 4x GELU MLP at B=4,N=65536,C=128,H=8,M=128 under bf16 autocast (fused HIP launches around the HIP mixer); train =
 the headline configuration with the backward pass (HIP kernels both ways); linear = causal linear attention at
 B=4,H=8,N=65536,Dk=Dv=64 (bf16, and fp32 beside it); fp32 = the mixer forward in fp32 at B=1,H=8,N=262144,M=256,D=32
-with BASELINE config 1 beside it.
+with BASELINE config 1 beside it; model = the training step of an 8-block model (C=128,H=8,M=128, fused AdamW) on small
+meshes (--lengths, default 4096,16384,65536 points), enqueued eagerly and replayed from a HIP graph.
 """
 from __future__ import annotations
 
@@ -440,6 +441,61 @@ def bench_lra(args, F, dev):
     return out
 
 
+def _model_train_rows(dev, lengths, graph_only=False):
+    """A whole model's training step where the launches, not the kernels, set the pace: 8 blocks (C=128, H=8, M=128,
+    pdebench/models/flare.py:236-301) with fused AdamW on small meshes, enqueued eagerly and with forward + loss +
+    backward replayed from one HIP graph (GraphedTrainStep; the optimizer step stays eager in both)."""
+    from flare_py_amd import GraphedTrainStep
+    from flare_py_amd import modules as Mod8
+    rows8 = {}
+    for n_pts in lengths:
+        torch.manual_seed(0)
+        model = Mod8.FLAREModel(in_dim=3, out_dim=1, channel_dim=128, num_blocks=8, num_heads=8, num_latents=128).to(dev).train()
+        prm = list(model.parameters())
+        opt = torch.optim.AdamW(prm, lr=1e-4, fused=True)
+        xm, tm = torch.randn(1, n_pts, 3, device=dev), torch.randn(1, n_pts, 1, device=dev)
+
+        def mse(o, t):
+            return ((o[0] if isinstance(o, tuple) else o).float() - t).square().mean()
+
+        def eager_step():
+            for p_ in prm:
+                p_.grad = None
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                o = model(xm)
+            mse(o, tm).backward()
+            opt.step()
+
+        graphed = GraphedTrainStep(model, mse, autocast_dtype=torch.bfloat16)
+
+        def graph_step():
+            graphed(xm, tm)
+            opt.step()
+
+        row = {} if graph_only else {"ms_eager": round(wall_ms(eager_step, 20, 5), 3)}
+        row["ms_graph_replay"] = round(wall_ms(graph_step, 20, 5), 3)
+        row["ms_graph_replay_without_optimizer"] = round(wall_ms(lambda: graphed(xm, tm), 20, 5), 3)
+        rows8[f"N={n_pts}"] = row
+        del graphed, model, opt
+    return dict(rows8, what="forward + MSE + backward + fused AdamW of an 8-block model, B=1, bf16 autocast, wall clock per step")
+
+
+def bench_model(args, F, dev):
+    """The 8-block model's training step on small meshes (--lengths; default 4096, 16384, 65536 points), eager and
+    replayed from a HIP graph."""
+    lengths = tuple(int(v) for v in args.lengths.split(",")) if args.lengths != "1000000,100000" else (4096, 16384, 65536)
+    rows = _model_train_rows(dev, lengths)
+    head = rows[f"N={lengths[0]}"]
+    ms = head["ms_graph_replay"]
+    out = base_record(args, f"8-block FLARE model training step points/sec, N={lengths[0]},C=128,H=8,M=128 bf16, HIP graph replay",
+                      lengths[0] / (ms * 1e-3), "points/s", ms,
+                      "FLAREModel (in_proj, 8 blocks, out_proj), forward + MSE + backward replayed from a HIP graph, fused AdamW eager, B=1")
+    out["dtype"] = "bf16"
+    out["roofline"] = None
+    out["meshes"] = rows
+    return out
+
+
 def _mfma16(F, q, k, v):
     from flare_py_amd import _lib, functional
     with functional.mixer_flags(_lib.FLAG_MFMA16):
@@ -771,40 +827,7 @@ def bench_block(args, F, dev):
     out["train_block_4x_ffn"] = {"ms_fwd_bwd": round(ms_train4, 3),
                                  "ms_fwd_bwd_torch_layers_hip_mixer": None if ms_train4_torch is None else round(ms_train4_torch, 3),
                                  "what": "the same for the block with the 4x GELU MLP as its feed-forward (no lift)"}
-    # a whole model's training step where the launches, not the kernels, set the pace: 8 blocks (C=128, H=8, M=128,
-    # pdebench/models/flare.py:236-301) with fused AdamW on small meshes, enqueued eagerly and with forward + loss +
-    # backward replayed from one HIP graph (GraphedTrainStep; the optimizer step stays eager in both)
-    from flare_py_amd import GraphedTrainStep
-    from flare_py_amd import modules as Mod8
-    rows8 = {}
-    for n_pts in (4096, 16384, 65536):
-        torch.manual_seed(0)
-        model = Mod8.FLAREModel(in_dim=3, out_dim=1, channel_dim=128, num_blocks=8, num_heads=8, num_latents=128).to(dev).train()
-        prm = list(model.parameters())
-        opt = torch.optim.AdamW(prm, lr=1e-4, fused=True)
-        xm, tm = torch.randn(1, n_pts, 3, device=dev), torch.randn(1, n_pts, 1, device=dev)
-
-        def mse(o, t):
-            return ((o[0] if isinstance(o, tuple) else o).float() - t).square().mean()
-
-        def eager_step():
-            for p_ in prm:
-                p_.grad = None
-            with torch.autocast("cuda", dtype=torch.bfloat16):
-                o = model(xm)
-            mse(o, tm).backward()
-            opt.step()
-
-        graphed = GraphedTrainStep(model, mse, autocast_dtype=torch.bfloat16)
-
-        def graph_step():
-            graphed(xm, tm)
-            opt.step()
-
-        rows8[f"N={n_pts}"] = {"ms_eager": round(wall_ms(eager_step, 20, 5), 3), "ms_graph_replay": round(wall_ms(graph_step, 20, 5), 3),
-                               "ms_graph_replay_without_optimizer": round(wall_ms(lambda: graphed(xm, tm), 20, 5), 3)}
-        del graphed, model, opt
-    out["train_model_8_blocks_adamw"] = dict(rows8, what="forward + MSE + backward + fused AdamW of an 8-block model, B=1, bf16 autocast, wall clock per step")
+    out["train_model_8_blocks_adamw"] = _model_train_rows(dev, (4096, 16384, 65536))
     # the same modules the way the reference runs them on this device: torch Linear / LayerNorm layers under the
     # same autocast, the mixer as two torch scaled_dot_product_attention calls (pdebench/models/flare.py:122-156)
     try:
@@ -865,7 +888,7 @@ def main():
     ap.add_argument("--no-torch-sdpa", action="store_true", help="skip the legs that time torch's own formulation (fused SDPA, einsum, torch layers) on the GPU")
     ap.add_argument("--lengths", default="1000000,100000", help="layer workload: token counts (the first one is the headline of the line)")
     ap.add_argument("--latents", default="128,512,2048", help="layer workload: latent counts")
-    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train", "linear", "fp32", "layer", "lra", "power"], default="mixer",
+    ap.add_argument("--workload", choices=["mixer", "causal", "triple", "block", "train", "linear", "fp32", "layer", "lra", "model", "power"], default="mixer",
                     help="mixer = the headline configuration (default); the others are BASELINE configs 4, 5, 2")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -881,7 +904,7 @@ def main():
     dev = torch.device("cuda:0")
     if args.workload != "mixer":
         fn = {"causal": bench_causal, "triple": bench_triple, "block": bench_block, "train": bench_train,
-              "linear": bench_linear, "fp32": bench_fp32, "layer": bench_layer, "lra": bench_lra, "power": bench_power}[args.workload]
+              "linear": bench_linear, "fp32": bench_fp32, "layer": bench_layer, "lra": bench_lra, "model": bench_model, "power": bench_power}[args.workload]
         print(json.dumps(fn(args, F, dev)))
         return
     B, H, N, M, D = 1, 8, 1 << 20, 256, 32
