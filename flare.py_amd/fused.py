@@ -470,6 +470,24 @@ def mlp_weight_image(w):
     return w.reshape(L, Cdim * Cdim)[:, _image_index(Cdim, w.device)].contiguous()
 
 
+_IMG_INDEX2 = {}
+
+
+def mlp_weight_images(w):
+    """(image of w, image of its transposes) as one gather: the transposed tile's element (row, col) is w[col][row], so
+    its image reads w through the same index with row and column swapped.  A training step packs after every
+    optimizer update, and on small meshes each saved launch counts."""
+    L, Cdim, _ = w.shape
+    key = (Cdim, L, str(w.device))
+    ix = _IMG_INDEX2.get(key)
+    if ix is None:
+        idx = _image_index(Cdim, w.device)
+        both = torch.stack([idx, (idx % Cdim) * Cdim + idx // Cdim])                     # [2, C*C]
+        ix = _IMG_INDEX2[key] = (torch.arange(L, device=w.device).view(1, L, 1), both.view(2, 1, Cdim * Cdim))
+    imgs = w.reshape(L, Cdim * Cdim)[ix[0], ix[1]]                                          # [2, L, C*C], contiguous
+    return imgs[0], imgs[1]
+
+
 def _packed_train(mod, layers, cd):
     """(w [L,C,C] for the forward launch, images of the weights and of their transposes for the backward, fp32 biases
     [L,C]), cached on the module until a parameter changes."""
@@ -478,8 +496,7 @@ def _packed_train(mod, layers, cd):
     if cache is not None and cache[0] == key:
         return cache[1:]
     w, b = _packed(mod, layers, cd)
-    w_img = mlp_weight_image(w)
-    wt_img = mlp_weight_image(w.transpose(1, 2).contiguous())
+    w_img, wt_img = mlp_weight_images(w)
     mod.__dict__["_flare_packed_train"] = (key, w, b, w_img, wt_img)
     return w, b, w_img, wt_img
 
@@ -493,8 +510,7 @@ def _packed_train_expand(mod, E, cd):
     if cache is not None and cache[0] == key:
         return cache[1:]
     w, b = _packed_expand(mod, E, cd)
-    w_img = mlp_weight_image(w)
-    wt_img = mlp_weight_image(w.transpose(1, 2).contiguous())
+    w_img, wt_img = mlp_weight_images(w)
     mod.__dict__["_flare_packed_train"] = (key, w, b, w_img, wt_img)
     return w, b, w_img, wt_img
 

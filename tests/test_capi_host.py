@@ -193,6 +193,18 @@ def test_new_struct_sizes_and_entry_point_validation():
     assert lib.flare_scatter_fwd_lse(d, None, None, None, None, None, None, None) == _lib.FLARE_EINVAL
 
 
+@pytest.mark.parametrize("Cdim,L", [(32, 1), (64, 3), (128, 8)])
+def test_both_weight_images_from_one_gather_equal_the_two_single_ones(Cdim, L):
+    """A training step builds the image of the weights and of their transposes in one indexed read; each has to be what
+    mlp_weight_image (checked against the header's formula below) gives for the matrix and for its transpose."""
+    from flare_py_amd import fused
+    w = torch.randn(L, Cdim, Cdim, generator=torch.Generator().manual_seed(Cdim + L)).to(torch.bfloat16)
+    img, img_t = fused.mlp_weight_images(w)
+    assert img.is_contiguous() and img_t.is_contiguous() and img.shape == img_t.shape == (L, Cdim * Cdim)
+    assert torch.equal(img, fused.mlp_weight_image(w))
+    assert torch.equal(img_t, fused.mlp_weight_image(w.transpose(1, 2).contiguous()))
+
+
 @pytest.mark.parametrize("Cdim", [32, 64, 128])
 def test_mlp_weight_image_follows_the_header_formula(Cdim):
     """fused.mlp_weight_image against include/flare_hip.h's position formula, element by element in plain loops:
